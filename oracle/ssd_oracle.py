@@ -1,0 +1,214 @@
+"""CPU oracle for the state-space-duality (Mamba-2) operator family.
+
+TEST INFRASTRUCTURE ONLY.
+
+The reference repository has no code for this family (its ``ssd_chunk_scan``
+is an element-wise diagonal recurrence, see ``ops_oracle.ssd_chunk_scan``).
+Its semantics are fixed by vectors the reference ships, captured from the
+third-party ``mamba_ssm`` Triton kernels (state-spaces/mamba, commit
+10b5d6358f27966f6a40e4bf0baa17a460688128; recorded in the ``meta`` block of
+tests/mamba_reference_cases.json) through the call sites in
+scripts/refresh_mamba_goldens.py:405-486 (components), :568-632 (combined)
+and :677-705 (bmm).  That dependency's source is not part of the reference
+tree, so its published algorithm is restated here:
+
+    dt'  = clamp(softplus(dt + dt_bias), dt_min, dt_max)
+    h_t  = exp(dt'_t A_h) h_{t-1} + dt'_t x_t (outer) B_t          (P x N per head)
+    y_t  = h_t C_t + D x_t ;  y_t *= silu(z_t)
+
+and decomposed over chunks of Q tokens as
+
+    chunk_cumsum   dA_cs[c,l]   = sum_{j<=l} dt'_j A_h
+    bmm_chunk      CB[c,l,s]    = <C_l, B_s>
+    chunk_state    S_c[p,n]     = sum_l B_l[n] exp(dA_cs[last]-dA_cs[l]) dt'_l x_l[p]
+    state_passing  H_{c+1}      = exp(dA_cs[c,last]) H_c + S_c
+    chunk_scan     y_l          = exp(dA_cs[l]) C_l.H_c
+                                  + sum_{s<=l} CB[l,s] exp(dA_cs[l]-dA_cs[s]) dt'_s x_s + D x_l
+
+Pinned by tests/test_oracle_golden.py against the fixture sections
+``ssd_components`` (chunk_cumsum, chunk_cumsum_clamped, chunk_state,
+state_passing, chunk_scan_*), ``ssd_bmm`` and ``ssd_combined.combined_full``
+and by the identity "chunked == sequential" in float64.  The upstream kernels
+evaluate ``exp(min(x, 0))`` for the intra-chunk decay factors; with A < 0 (the
+only regime used by models) the clamp is inactive, but the fixtures use
+random-sign A, so ``clamp_decay=True`` reproduces them.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+
+def prepare_dt(dt, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf")), acc=torch.float64):
+    """(B,L,H) raw step -> effective step."""
+    v = dt.to(acc)
+    if dt_bias is not None:
+        v = v + dt_bias.to(acc)[None, None, :]
+    if dt_softplus:
+        v = F.softplus(v)
+    lo, hi = dt_limit
+    if lo != 0.0 or hi != float("inf"):
+        v = v.clamp(min=lo, max=hi)
+    return v
+
+
+def ssd_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=False,
+                   dt_limit=(0.0, float("inf")), initial_states=None, acc=torch.float64):
+    """Token-by-token recurrence; returns ``(y (B,L,H,P), final_states (B,H,P,N))``.
+
+    Shapes: x (B,L,H,P); dt (B,L,H); A (H,); B,C (B,L,G,N); D (H,)|(H,P);
+    z (B,L,H,P); initial_states (B,H,P,N)."""
+    batch, seqlen, heads, hdim = x.shape
+    groups, nstate = B.shape[2], B.shape[3]
+    per = heads // groups
+    dtv = prepare_dt(dt, dt_bias, dt_softplus, dt_limit, acc)
+    xx = x.to(acc)
+    Bh = B.to(acc).repeat_interleave(per, dim=2)     # (B,L,H,N)
+    Ch = C.to(acc).repeat_interleave(per, dim=2)
+    AA = A.to(acc)
+    h = (initial_states.to(acc) if initial_states is not None
+         else torch.zeros(batch, heads, hdim, nstate, dtype=acc))
+    ys = []
+    for t in range(seqlen):
+        step = dtv[:, t]                                           # (B,H)
+        decay = torch.exp(step * AA[None])                         # (B,H)
+        h = decay[:, :, None, None] * h \
+            + (step[:, :, None] * xx[:, t])[:, :, :, None] * Bh[:, t][:, :, None, :]
+        y = (h * Ch[:, t][:, :, None, :]).sum(-1)                  # (B,H,P)
+        if D is not None:
+            Dv = D.to(acc)
+            y = y + (Dv[None, :, None] if Dv.ndim == 1 else Dv[None]) * xx[:, t]
+        if z is not None:
+            y = y * F.silu(z[:, t].to(acc))
+        ys.append(y)
+    return torch.stack(ys, dim=1), h
+
+
+def _pad_to_chunks(t, Q, dim=1):
+    L = t.shape[dim]
+    pad = (-L) % Q
+    if pad == 0:
+        return t
+    shape = list(t.shape)
+    shape[dim] = pad
+    return torch.cat([t, torch.zeros(shape, dtype=t.dtype)], dim=dim)
+
+
+def chunk_cumsum(dt, A, chunk_size, dt_bias=None, dt_softplus=False,
+                 dt_limit=(0.0, float("inf")), acc=torch.float64):
+    """-> ``(dA_cumsum, dt_out)`` each (B,H,nc,Q); the tail of a ragged last
+    chunk has dt'=0."""
+    Q = int(chunk_size)
+    dtv = prepare_dt(dt, dt_bias, dt_softplus, dt_limit, acc)
+    dtv = _pad_to_chunks(dtv, Q, dim=1)
+    batch, Lp, heads = dtv.shape
+    nc = Lp // Q
+    dtc = dtv.view(batch, nc, Q, heads).permute(0, 3, 1, 2)          # (B,H,nc,Q)
+    dA = dtc * A.to(acc)[None, :, None, None]
+    return dA.cumsum(dim=-1), dtc.contiguous()
+
+
+def bmm_chunk(a, b, chunk_size, seq_idx=None, causal=False, acc=torch.float64):
+    """``out[b,c,(g,)l,s] = <a[b,cQ+l,(g,)], b[b,cQ+s,(g,)]>``; entries whose
+    ``l`` and ``s`` lie in different sequences (``seq_idx``) are 0; with
+    ``causal`` the strict upper triangle is returned as 0 (unspecified by the
+    fixtures)."""
+    Q = int(chunk_size)
+    grouped = a.dim() == 4
+    aa = a.to(acc) if grouped else a.to(acc)[:, :, None, :]
+    bb = b.to(acc) if grouped else b.to(acc)[:, :, None, :]
+    aa = _pad_to_chunks(aa, Q)
+    bb = _pad_to_chunks(bb, Q)
+    batch, Lp, G, K = aa.shape
+    nc = Lp // Q
+    ac = aa.view(batch, nc, Q, G, K)
+    bc = bb.view(batch, nc, Q, G, K)
+    out = torch.einsum("bclgk,bcsgk->bcgls", ac, bc)
+    if seq_idx is not None:
+        si = _pad_to_chunks(seq_idx.to(torch.long) + 1, Q).view(batch, nc, Q) - 1
+        same = si[:, :, :, None] == si[:, :, None, :]
+        out = out * same[:, :, None].to(acc)
+    if causal:
+        out = out * torch.tril(torch.ones(Q, Q, dtype=acc))
+    return out if grouped else out[:, :, 0]
+
+
+def _seg_exp(delta, clamp_decay):
+    return torch.exp(delta.clamp(max=0.0)) if clamp_decay else torch.exp(delta)
+
+
+def chunk_state(B, x, dt_c, dA_cumsum, clamp_decay=True, acc=torch.float64):
+    """-> states (B,nc,H,P,N): contribution of each chunk to the state at its end."""
+    batch, H, nc, Q = dt_c.shape
+    G, N = B.shape[2], B.shape[3]
+    per = H // G
+    xx = _pad_to_chunks(x.to(acc), Q).view(batch, nc, Q, H, -1)
+    Bh = _pad_to_chunks(B.to(acc), Q).view(batch, nc, Q, G, N).repeat_interleave(per, dim=3)
+    dA = dA_cumsum.to(acc)
+    w = _seg_exp(dA[..., -1:] - dA, clamp_decay) * dt_c.to(acc)      # (B,H,nc,Q)
+    return torch.einsum("bclhn,bhcl,bclhp->bchpn", Bh, w, xx)
+
+
+def state_passing(states, dA_chunk_last, initial_states=None, acc=torch.float64):
+    """states (B,nc,H,...); dA_chunk_last (B,H,nc).  Returns ``(entering, final)``
+    where ``entering[:,c]`` is the state at the START of chunk c."""
+    st = states.to(acc)
+    batch, nc, H = st.shape[:3]
+    cur = (initial_states.to(acc).reshape(st[:, 0].shape) if initial_states is not None
+           else torch.zeros_like(st[:, 0]))
+    outs = []
+    extra = (1,) * (st.dim() - 3)
+    for c in range(nc):
+        outs.append(cur)
+        g = torch.exp(dA_chunk_last.to(acc)[:, :, c]).view(batch, H, *extra)
+        cur = g * cur + st[:, c]
+    return torch.stack(outs, dim=1), cur
+
+
+def chunk_scan(B, C, x, dt_c, dA_cumsum, prev_states, D=None, z=None,
+               clamp_decay=True, acc=torch.float64):
+    """-> y (B,L,H,P) from entering states ``prev_states`` (B,nc,H,P,N)."""
+    batch, H, nc, Q = dt_c.shape
+    L = x.shape[1]
+    G, N = B.shape[2], B.shape[3]
+    per = H // G
+    P = x.shape[3]
+    xx = _pad_to_chunks(x.to(acc), Q).view(batch, nc, Q, H, P)
+    Bh = _pad_to_chunks(B.to(acc), Q).view(batch, nc, Q, G, N).repeat_interleave(per, dim=3)
+    Ch = _pad_to_chunks(C.to(acc), Q).view(batch, nc, Q, G, N).repeat_interleave(per, dim=3)
+    dA = dA_cumsum.to(acc)                                            # (B,H,nc,Q)
+    # inter-chunk: exp(dA_cs[l]) * C_l . H_c
+    y_off = torch.einsum("bclhn,bchpn->bclhp", Ch, prev_states.to(acc)) \
+        * torch.exp(dA).permute(0, 2, 3, 1)[..., None]
+    # intra-chunk: sum_{s<=l} CB[l,s] * exp(dA_cs[l]-dA_cs[s]) * dt_s * x_s
+    CB = torch.einsum("bclhn,bcshn->bchls", Ch, Bh)
+    seg = dA.permute(0, 2, 1, 3)                                     # (B,nc,H,Q)
+    decay = _seg_exp(seg[..., :, None] - seg[..., None, :], clamp_decay)
+    mask = torch.tril(torch.ones(Q, Q, dtype=torch.bool))
+    M = torch.where(mask, CB * decay, torch.zeros((), dtype=acc))
+    M = M * dt_c.to(acc).permute(0, 2, 1, 3)[..., None, :]
+    y_diag = torch.einsum("bchls,bcshp->bclhp", M, xx)
+    y = y_off + y_diag
+    if D is not None:
+        Dv = D.to(acc)
+        y = y + (Dv[None, None, None, :, None] if Dv.ndim == 1 else Dv[None, None, None]) * xx
+    y = y.reshape(batch, nc * Q, H, P)[:, :L]
+    if z is not None:
+        y = y * F.silu(z.to(acc))
+    return y
+
+
+def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
+                 initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
+                 clamp_decay=True, acc=torch.float64):
+    """cumsum -> chunk_state -> state_passing -> chunk_scan; returns
+    ``(y, final_states (B,H,P,N))``."""
+    dA_cs, dt_c = chunk_cumsum(dt, A, chunk_size, dt_bias, dt_softplus, dt_limit, acc)
+    st = chunk_state(B, x, dt_c, dA_cs, clamp_decay, acc)
+    entering, final = state_passing(st, dA_cs[..., -1], initial_states, acc)
+    y = chunk_scan(B, C, x, dt_c, dA_cs, entering, D=D, z=z, clamp_decay=clamp_decay, acc=acc)
+    return y, final
