@@ -1,0 +1,124 @@
+"""ctypes binding of ``libssm_amd.so`` (the C ABI declared in include/ssm_amd.h).
+
+The shared library is built ahead of time by ``python -m ssm_amd.build`` and is
+loaded from ``ssm_amd/lib``.  There is no fallback: if the library is missing
+or a call returns a non-zero status, an exception is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from pathlib import Path
+from typing import Optional
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libssm_amd.so"
+ABI_VERSION = 1
+
+SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
+PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
+
+_DTYPE_ENUM = {torch.float32: SSM_F32, torch.bfloat16: SSM_BF16, torch.float16: SSM_F16}
+
+_vp, _i32, _f32, _i64 = C.c_void_p, C.c_int32, C.c_float, C.c_int64
+
+
+class BackendUnavailable(RuntimeError):
+    """The HIP library could not be loaded."""
+
+
+class KernelError(RuntimeError):
+    """A C-ABI entry point returned a failure status."""
+
+
+class ScanFwdArgs(C.Structure):
+    _fields_ = [
+        ("u", _vp), ("delta", _vp), ("z", _vp), ("A", _vp), ("Bproj", _vp), ("Cproj", _vp),
+        ("Dskip", _vp), ("dt_bias", _vp), ("out", _vp), ("last_state", _vp),
+        ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32),
+        ("io_dtype", _i32), ("bc_dtype", _i32), ("b_kind", _i32), ("c_kind", _i32),
+        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("tune_items", _i32),
+    ]
+
+
+# name -> argument struct (every entry point is ``int f(const args*, void* stream)``)
+ENTRY_POINTS = {
+    "ssm_scan_fwd": ScanFwdArgs,
+}
+PLAIN_SYMBOLS = ["ssm_amd_abi_version", "ssm_amd_status_string", "ssm_amd_last_error"]
+
+_lock = threading.Lock()
+_lib: Optional[C.CDLL] = None
+_load_error: Optional[Exception] = None
+
+
+def load() -> C.CDLL:
+    """Load the library once; raise :class:`BackendUnavailable` if impossible."""
+    global _lib, _load_error
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if _load_error is not None:
+            raise BackendUnavailable(str(_load_error))
+        try:
+            if not LIB_PATH.exists():
+                raise FileNotFoundError(
+                    f"{LIB_PATH} not found: build it with `python -m ssm_amd.build`")
+            lib = C.CDLL(str(LIB_PATH))
+            lib.ssm_amd_abi_version.restype = C.c_int
+            lib.ssm_amd_status_string.restype = C.c_char_p
+            lib.ssm_amd_status_string.argtypes = [C.c_int]
+            lib.ssm_amd_last_error.restype = C.c_char_p
+            got = lib.ssm_amd_abi_version()
+            if got != ABI_VERSION:
+                raise RuntimeError(f"libssm_amd ABI {got}, binding expects {ABI_VERSION}")
+            for name, struct in ENTRY_POINTS.items():
+                fn = getattr(lib, name)
+                fn.restype = C.c_int
+                fn.argtypes = [C.POINTER(struct), _vp]
+            _lib = lib
+        except Exception as exc:  # remembered: a broken install stays broken
+            _load_error = exc
+            raise BackendUnavailable(str(exc)) from exc
+    return _lib
+
+
+def available() -> bool:
+    try:
+        load()
+        return True
+    except BackendUnavailable:
+        return False
+
+
+def dtype_enum(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_ENUM[dt]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dt}: the HIP backend handles float32, bfloat16 and float16")
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def stream_handle(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def call(name: str, args: C.Structure, device: torch.device) -> None:
+    """Invoke an entry point on the current stream of ``device``; a contract
+    violation reported by the library surfaces as ``ValueError`` (as the
+    reference's compiled backends do, src/ssm/ops/__init__.py:1244-1252)."""
+    lib = load()
+    with torch.cuda.device(device):
+        status = getattr(lib, name)(C.byref(args), stream_handle(device))
+    if status != 0:
+        detail = lib.ssm_amd_last_error().decode() or lib.ssm_amd_status_string(status).decode()
+        if status == -7:
+            raise KernelError(f"{name}: {detail}")
+        raise ValueError(f"{name}: {detail}")

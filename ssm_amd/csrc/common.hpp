@@ -1,0 +1,205 @@
+// Shared device/host helpers for the gfx950 kernels: dtype conversion, vector
+// loads, fp32 transcendental helpers, wave64 DPP scans, error reporting.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/ssm_amd.h"
+
+namespace ssm {
+
+// ---------------------------------------------------------------- host side
+
+void set_error(const char *fmt, ...);   // defined in status.hip
+
+#define SSM_REQUIRE(cond, code, ...)        \
+  do {                                      \
+    if (!(cond)) {                          \
+      ::ssm::set_error(__VA_ARGS__);        \
+      return (code);                        \
+    }                                       \
+  } while (0)
+
+#define SSM_CHECK_LAUNCH(what)                                                  \
+  do {                                                                          \
+    hipError_t e_ = hipGetLastError();                                          \
+    if (e_ != hipSuccess) {                                                     \
+      ::ssm::set_error("%s: %s", (what), hipGetErrorString(e_));                \
+      return SSM_ERR_LAUNCH;                                                    \
+    }                                                                           \
+  } while (0)
+
+inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
+inline bool valid_dtype(int d) { return d == SSM_F32 || d == SSM_BF16 || d == SSM_F16; }
+inline int dtype_size(int d) { return d == SSM_F32 ? 4 : 2; }
+
+// Raise the dynamic-LDS ceiling of a kernel once (needed above 64 KiB).
+template <typename KernelT>
+inline hipError_t allow_dynamic_lds(KernelT kernel, size_t bytes) {
+  if (bytes <= 48 * 1024) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+// -------------------------------------------------------------- device side
+
+constexpr int WAVE = 64;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+__device__ __forceinline__ float to_f32(f16_t v) { return (float)v.v; }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t x = __float_as_uint(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);  // quiet NaN
+  x += 0x7fffu + ((x >> 16) & 1u);                                              // round to nearest even
+  return (uint16_t)(x >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_f32(float f);
+template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) { return bf16_t{f32_to_bf16_bits(f)}; }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float f) { return f16_t{(_Float16)f}; }
+
+// Read element i of a buffer whose dtype is only known at run time (uniform branch).
+__device__ __forceinline__ float load_as_f32(const void *p, int dtype, size_t i) {
+  if (dtype == SSM_F32) return reinterpret_cast<const float *>(p)[i];
+  if (dtype == SSM_BF16) return to_f32(reinterpret_cast<const bf16_t *>(p)[i]);
+  return to_f32(reinterpret_cast<const f16_t *>(p)[i]);
+}
+
+// A run of K consecutive elements owned by one lane, moved with the widest
+// aligned vector access available (16 bytes), or element-wise with bounds.
+template <typename T, int K>
+struct alignas(sizeof(T) * K >= 16 ? 16 : sizeof(T) * K) Pack { T v[K]; };
+
+template <typename T, int K>
+__device__ __forceinline__ void load_run(const T *base, int t, int len, bool vec_ok, float (&out)[K]) {
+  constexpr int PIECE = (sizeof(T) * K >= 16) ? (16 / sizeof(T)) : K;   // elements per vector access
+  if (vec_ok && t + K <= len) {
+#pragma unroll
+    for (int j = 0; j < K / PIECE; ++j) {
+      Pack<T, PIECE> p = *reinterpret_cast<const Pack<T, PIECE> *>(base + t + j * PIECE);
+#pragma unroll
+      for (int i = 0; i < PIECE; ++i) out[j * PIECE + i] = to_f32(p.v[i]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < K; ++i) out[i] = (t + i < len) ? to_f32(base[t + i]) : 0.0f;
+  }
+}
+
+template <typename T, int K>
+__device__ __forceinline__ void store_run(T *base, int t, int len, bool vec_ok, const float (&in)[K]) {
+  constexpr int PIECE = (sizeof(T) * K >= 16) ? (16 / sizeof(T)) : K;
+  if (vec_ok && t + K <= len) {
+#pragma unroll
+    for (int j = 0; j < K / PIECE; ++j) {
+      Pack<T, PIECE> p;
+#pragma unroll
+      for (int i = 0; i < PIECE; ++i) p.v[i] = from_f32<T>(in[j * PIECE + i]);
+      *reinterpret_cast<Pack<T, PIECE> *>(base + t + j * PIECE) = p;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+      if (t + i < len) base[t + i] = from_f32<T>(in[i]);
+  }
+}
+
+// 2^x on the transcendental unit (v_exp_f32, 1 ulp; results below 2^-126 flush to 0).
+__device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float log2_hw(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float rcp_hw(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// e^x with the argument split so that the rounding of x*log2(e) does not
+// cost relative accuracy for |x| up to ~100.
+__device__ __forceinline__ float exp_f32(float x) {
+  const float hi = x * LOG2E;
+  const float lo = __builtin_fmaf(x, LOG2E, -hi) + x * 1.925963033500864e-08f;  // log2(e) - (float)log2(e)
+  return exp2_hw(hi) * __builtin_fmaf(lo, LN2, 1.0f);
+}
+
+// log(1 + e) for e >= 0 without cancellation (Kahan): log(w) * e / (w - 1), w = fl(1 + e).
+__device__ __forceinline__ float log1p_pos(float e) {
+  const float w = 1.0f + e;
+  const float d = w - 1.0f;
+  const float r = log2_hw(w) * LN2 * (e * rcp_hw(d));
+  return d == 0.0f ? e : r;
+}
+
+// torch.nn.functional.softplus with its default threshold of 20.
+__device__ __forceinline__ float softplus_f32(float x) {
+  return x > 20.0f ? x : log1p_pos(exp_f32(x));
+}
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return rcp_hw(1.0f + exp_f32(-x)); }
+__device__ __forceinline__ float silu_f32(float x) { return x * sigmoid_f32(x); }
+
+// ---- wave64 cross-lane helpers (DPP; rows are 16 lanes) --------------------
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float keep, float src) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(keep), __float_as_int(src), CTRL,
+                                                    ROW_MASK, 0xf, false));
+}
+
+constexpr int DPP_ROW_SHR1 = 0x111, DPP_ROW_SHR2 = 0x112, DPP_ROW_SHR4 = 0x114, DPP_ROW_SHR8 = 0x118;
+constexpr int DPP_ROW_BCAST15 = 0x142, DPP_ROW_BCAST31 = 0x143, DPP_WAVE_SHR1 = 0x138;
+constexpr int DPP_ROW_SHL1 = 0x101, DPP_ROW_SHL2 = 0x102, DPP_ROW_SHL4 = 0x104, DPP_ROW_SHL8 = 0x108;
+constexpr int DPP_WAVE_SHL1 = 0x130;
+
+// Inclusive scan across the 64 lanes of the pair (a, b) under
+//   (a1, b1) then (a2, b2)  ->  (a1 a2, a2 b1 + b2)
+// i.e. the composition of the affine maps h -> a h + b, earlier lanes first.
+__device__ __forceinline__ void wave_scan_affine(float &a, float &b) {
+#define SSM_SCAN_STEP(CTRL, RM)                      \
+  {                                                  \
+    const float ap = dpp_move<CTRL, RM>(1.0f, a);    \
+    const float bp = dpp_move<CTRL, RM>(0.0f, b);    \
+    b = __builtin_fmaf(a, bp, b);                    \
+    a = a * ap;                                      \
+  }
+  SSM_SCAN_STEP(DPP_ROW_SHR1, 0xf)
+  SSM_SCAN_STEP(DPP_ROW_SHR2, 0xf)
+  SSM_SCAN_STEP(DPP_ROW_SHR4, 0xf)
+  SSM_SCAN_STEP(DPP_ROW_SHR8, 0xf)
+  SSM_SCAN_STEP(DPP_ROW_BCAST15, 0xa)
+  SSM_SCAN_STEP(DPP_ROW_BCAST31, 0xc)
+#undef SSM_SCAN_STEP
+}
+
+// Value of the previous lane (lane 0 receives `first`).
+__device__ __forceinline__ float wave_prev(float v, float first) {
+  return dpp_move<DPP_WAVE_SHR1, 0xf>(first, v);
+}
+// Value of the next lane (lane 63 receives `last`).
+__device__ __forceinline__ float wave_next(float v, float last) {
+  return dpp_move<DPP_WAVE_SHL1, 0xf>(last, v);
+}
+
+__device__ __forceinline__ float wave_read_lane(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// Sum over the 64 lanes, result valid in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, WAVE);
+  return v;
+}
+
+__device__ __forceinline__ int wave_id_uniform() {
+  return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+}
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63); }
+
+}  // namespace ssm

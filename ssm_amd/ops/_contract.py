@@ -1,0 +1,123 @@
+"""Host-side argument contract shared by the operator façade.
+
+The checks and their ``ValueError`` behaviour follow the reference's Python
+path (src/ssm/ops/python/reference.py; each function cites its lines) so that
+code written against ``ssm.ops`` sees the same failures here.  Nothing in this
+module touches a device.
+"""
+
+from __future__ import annotations
+
+from typing import Iterable, Optional
+
+import torch
+
+SUPPORTED = (torch.float32, torch.bfloat16, torch.float16)
+
+
+class DeviceError(RuntimeError):
+    """Inputs are not all on one ROCm device (this backend has no CPU path)."""
+
+
+def require_gpu(*tensors: Optional[torch.Tensor]) -> torch.device:
+    """All tensor arguments must live on the same ``cuda`` (ROCm) device.
+
+    The reference dispatches on the same predicate
+    (src/ssm/ops/__init__.py:116-122) but falls back to Python loops otherwise;
+    this backend refuses instead of silently computing on the CPU."""
+    devs = {t.device for t in tensors if isinstance(t, torch.Tensor)}
+    if not devs:
+        raise DeviceError("no tensor arguments")
+    if len(devs) != 1:
+        raise DeviceError(f"tensors live on different devices: {sorted(map(str, devs))}")
+    dev = next(iter(devs))
+    if dev.type != "cuda":
+        raise DeviceError(
+            f"ssm_amd runs on ROCm devices only; got tensors on '{dev}'. "
+            "There is deliberately no CPU fallback.")
+    return dev
+
+
+def check_float(name: str, t: torch.Tensor) -> None:
+    if t.dtype not in SUPPORTED:
+        raise ValueError(
+            f"{name} has dtype {t.dtype}; the HIP backend supports float32, bfloat16 and float16 "
+            "(accumulation is always float32).")
+
+
+def common_io_dtype(tensors: Iterable[Optional[torch.Tensor]]) -> torch.dtype:
+    """Activation dtype the kernel reads: the shared dtype, or fp32 if mixed
+    (widening is exact, so mixed inputs keep the reference's fp32 arithmetic)."""
+    dts = {t.dtype for t in tensors if t is not None}
+    return next(iter(dts)) if len(dts) == 1 else torch.float32
+
+
+def as_f32_vec(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    return t.detach().to(torch.float32).contiguous()
+
+
+def cast_c(t: Optional[torch.Tensor], dt: torch.dtype) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    t = t.detach()
+    if t.dtype != dt:
+        t = t.to(dt)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+# ----------------------------------------------------------- selective scan
+
+def scan_projection_kind(name: str, p: torch.Tensor, batch: int, dim: int, nstate: int,
+                         length: int) -> tuple[int, int]:
+    """-> (kind, groups) for a B/C argument (reference.py:22-56)."""
+    from .._lib import PROJ_BDN, PROJ_BGNL, PROJ_DN
+
+    if p.dim() == 2:
+        if tuple(p.shape) != (dim, nstate):
+            raise ValueError(f"{name} must have shape (D, N).")
+        return PROJ_DN, 1
+    if p.dim() == 3:
+        if tuple(p.shape) != (batch, dim, nstate):
+            raise ValueError(f"{name} must have shape (B, D, N) when 3-D.")
+        return PROJ_BDN, 1
+    if p.dim() == 4:
+        if p.shape[0] != batch or p.shape[-1] != length:
+            raise ValueError(f"{name} must have shape (B, G, N, L) when 4-D.")
+        groups = int(p.shape[1])
+        if groups == 0 or dim % groups != 0:
+            raise ValueError("Group dimension must divide D.")
+        if p.shape[2] != nstate:
+            raise ValueError(f"{name} has mismatched state dimension.")
+        return PROJ_BGNL, groups
+    raise ValueError(f"Unsupported rank for {name}.")
+
+
+def check_selective_scan(u, delta, A, B, C, D, z, dt_bias):
+    """Shape contract of ``selective_scan`` (reference.py:124-165)."""
+    if u.ndim != 3 or delta.ndim != 3:
+        raise ValueError("u and delta must have shape (B, D, L).")
+    batch, dim, length = (int(s) for s in u.shape)
+    if tuple(delta.shape) != (batch, dim, length):
+        raise ValueError("delta must match the shape of u.")
+    if A.ndim < 1:
+        raise ValueError("A must have shape (D, N).")
+    nstate = int(A.shape[-1])
+    if tuple(A.shape) != (dim, nstate):
+        raise ValueError("A must have shape (D, N).")
+    bk = scan_projection_kind("B", B, batch, dim, nstate, length)
+    ck = scan_projection_kind("C", C, batch, dim, nstate, length)
+    if D is not None and tuple(D.shape) != (dim,):
+        raise ValueError("D must have shape (D,).")
+    if z is not None and tuple(z.shape) != (batch, dim, length):
+        raise ValueError("z must have shape (B, D, L).")
+    if dt_bias is not None and tuple(dt_bias.shape) != (dim,):
+        raise ValueError("dt_bias must have shape (D,).")
+    for name, t in (("u", u), ("delta", delta), ("A", A), ("B", B), ("C", C), ("D", D), ("z", z),
+                    ("dt_bias", dt_bias)):
+        if t is not None:
+            check_float(name, t)
+    if batch == 0 or dim == 0 or length == 0 or nstate == 0:
+        raise ValueError("selective_scan needs non-empty B, D, L and N.")
+    return batch, dim, length, nstate, bk, ck

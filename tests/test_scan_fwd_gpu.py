@@ -1,0 +1,252 @@
+"""GPU parity of ``selective_scan`` forward: HIP kernels (through the C ABI)
+against the CPU oracle, the reference's JSON vectors and size-independent
+properties at the benchmark shapes."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import ops_oracle as O
+from tests import fixtures as fx
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = dict(rtol=1e-5, atol=1e-5)          # north-star tolerance for fp32
+HALF_TOL = dict(rtol=2e-2, atol=2e-3)          # bf16/fp16 inputs, fp32 accumulation
+
+
+def _ops():
+    from ssm_amd import ops
+    return ops
+
+
+def dev(t):
+    return None if t is None else t.cuda()
+
+
+def make_inputs(seed, batch, dim, length, nstate, dtype=torch.float32, bkind="bgnl", ckind="bgnl",
+                groups=1, use_D=True, use_z=True, use_bias=True, bc_dtype=None):
+    """Synthetic inputs with the value distributions of the benchmark configs:
+    u, delta_raw, z ~ N(0,1); A[d,n] = -(n+1); B, C ~ N(0,1); dt_bias = softplus^-1(dt),
+    dt log-uniform in [1e-3, 0.1]."""
+    g = torch.Generator().manual_seed(seed)
+    bc_dtype = bc_dtype or dtype
+    u = torch.randn(batch, dim, length, generator=g).to(dtype)
+    delta = torch.randn(batch, dim, length, generator=g).to(dtype)
+    z = torch.randn(batch, dim, length, generator=g).to(dtype) if use_z else None
+    A = -torch.arange(1, nstate + 1, dtype=torch.float32).repeat(dim, 1)
+    A = A * (1.0 + 0.05 * torch.rand(dim, nstate, generator=g))
+
+    def proj(kind):
+        if kind == "dn":
+            return torch.randn(dim, nstate, generator=g).to(bc_dtype)
+        if kind == "bdn":
+            return torch.randn(batch, dim, nstate, generator=g).to(bc_dtype)
+        return torch.randn(batch, groups, nstate, length, generator=g).to(bc_dtype)
+
+    Bm, Cm = proj(bkind), proj(ckind)
+    D = torch.ones(dim) + 0.1 * torch.randn(dim, generator=g) if use_D else None
+    if use_bias:
+        dt = torch.exp(torch.rand(dim, generator=g) * (math.log(0.1) - math.log(1e-3)) + math.log(1e-3))
+        bias = dt + torch.log(-torch.expm1(-dt))
+    else:
+        bias = None
+    return dict(u=u, delta=delta, A=A, B=Bm, C=Cm, D=D, z=z, dt_bias=bias)
+
+
+def run_both(inp, softplus=True, **kw):
+    ops = _ops()
+    y_ref, h_ref = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"],
+                                    z=inp["z"], dt_bias=inp["dt_bias"], softplus=softplus,
+                                    return_last_state=True)
+    y, h = ops.selective_scan(dev(inp["u"]), dev(inp["delta"]), dev(inp["A"]), dev(inp["B"]),
+                              dev(inp["C"]), D=dev(inp["D"]), z=dev(inp["z"]),
+                              dt_bias=dev(inp["dt_bias"]), softplus=softplus, return_last_state=True, **kw)
+    torch.cuda.synchronize()
+    return (y.cpu(), h.cpu()), (y_ref, h_ref)
+
+
+# ------------------------------------------------------------------ fixtures
+
+@pytest.mark.parametrize("name", ["selective_scan_case1", "selective_scan_grouped"])
+def test_reference_nested_goldens(name):
+    i, o, _ = fx.nested_case(name)
+    y, h = _ops().selective_scan(dev(i["u"]), dev(i["delta"]), dev(i["A"]), dev(i["B"]), dev(i["C"]),
+                                 D=dev(i["D"]), z=dev(i["z"]), dt_bias=dev(i["dt_bias"]),
+                                 softplus=bool(i["softplus"]), return_last_state=True)
+    torch.testing.assert_close(y.cpu(), o["out"], **FP32_TOL)
+    torch.testing.assert_close(h.cpu(), o["last_state"], **FP32_TOL)
+
+
+@pytest.mark.parametrize("case", fx.flat_cases(), ids=lambda c: c[0])
+def test_reference_flat_goldens(case):
+    _, i, o = case
+    y, h = _ops().selective_scan(dev(i["u"]), dev(i["delta"]), dev(i["A"]), dev(i["B"]), dev(i["C"]),
+                                 D=dev(i["D"]), z=dev(i["z"]), dt_bias=dev(i["dt_bias"]),
+                                 softplus=True, return_last_state=True)
+    torch.testing.assert_close(y.cpu(), o["y"], **FP32_TOL)
+    torch.testing.assert_close(h.cpu(), o["state"], **FP32_TOL)
+
+
+@pytest.mark.parametrize("case,softplus", [("full", True), ("minimal", False), ("minimal_fp16", False),
+                                           ("minimal_bf16", False), ("time_varying_3d", True)])
+def test_upstream_vectors(case, softplus):
+    rec = fx.upstream("selective_scan", case)
+    i = rec["inputs"]
+    Bm, Cm = i["B"], i["C"]
+    if case == "time_varying_3d":
+        Bm, Cm = Bm[:, None].contiguous(), Cm[:, None].contiguous()
+    y = _ops().selective_scan(dev(i["u"]), dev(i["delta"]), dev(i["A"]), dev(Bm), dev(Cm),
+                              D=dev(i.get("D")), z=dev(i.get("z")), dt_bias=dev(i.get("delta_bias")),
+                              softplus=softplus)
+    want = rec["outputs"]["y"]
+    half = want.dtype != torch.float32
+    tol = dict(rtol=2e-2, atol=2e-2) if half else dict(rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(y.cpu(), want, **tol)
+
+
+# ------------------------------------------------------- oracle, option matrix
+
+SHAPES = [
+    # batch, dim, length, nstate
+    (1, 1, 1, 1), (2, 3, 5, 4), (2, 8, 64, 16), (1, 4, 65, 3), (3, 6, 257, 16), (2, 16, 512, 16),
+    (1, 8, 1000, 17), (2, 8, 2048, 16), (1, 2, 3000, 40),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("kinds", [("bgnl", "bgnl"), ("dn", "dn"), ("bdn", "bgnl"), ("bgnl", "dn")])
+def test_fp32_matches_oracle(shape, kinds):
+    b, d, l, n = shape
+    inp = make_inputs(hash(shape) % 1000, b, d, l, n, bkind=kinds[0], ckind=kinds[1])
+    (y, h), (yr, hr) = run_both(inp)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+    torch.testing.assert_close(h, hr, **FP32_TOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 8, 64, 16), (2, 16, 777, 16), (1, 8, 2048, 16)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_half_matches_oracle(dtype, shape):
+    b, d, l, n = shape
+    inp = make_inputs(7, b, d, l, n, dtype=dtype)
+    (y, h), (yr, hr) = run_both(inp)
+    assert y.dtype == dtype and h.dtype == dtype
+    torch.testing.assert_close(y.float(), yr.float(), **HALF_TOL)
+    torch.testing.assert_close(h.float(), hr.float(), **HALF_TOL)
+
+
+@pytest.mark.parametrize("groups,dim", [(1, 8), (2, 8), (4, 8), (8, 8), (3, 6), (2, 24)])
+def test_groups(groups, dim):
+    inp = make_inputs(11, 2, dim, 300, 16, groups=groups)
+    (y, h), (yr, hr) = run_both(inp)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+    torch.testing.assert_close(h, hr, **FP32_TOL)
+
+
+@pytest.mark.parametrize("use_D,use_z,use_bias,softplus", [
+    (False, False, False, False), (True, False, False, True), (False, True, True, False),
+    (False, False, True, True), (True, True, False, False)])
+def test_optional_arguments(use_D, use_z, use_bias, softplus):
+    inp = make_inputs(3, 2, 4, 130, 8, use_D=use_D, use_z=use_z, use_bias=use_bias)
+    if not softplus:   # raw deltas must stay positive and small for a decaying system
+        inp["delta"] = inp["delta"].abs() * 0.1
+        if inp["dt_bias"] is not None:
+            inp["dt_bias"] = inp["dt_bias"].abs() * 0.01
+    (y, h), (yr, hr) = run_both(inp, softplus=softplus)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+    torch.testing.assert_close(h, hr, **FP32_TOL)
+
+
+def test_mixed_dtypes_and_fp32_projections_with_bf16_activations():
+    inp = make_inputs(5, 2, 8, 200, 16, dtype=torch.bfloat16, bc_dtype=torch.float32)
+    (y, h), (yr, hr) = run_both(inp)
+    torch.testing.assert_close(y.float(), yr.float(), **HALF_TOL)
+    inp["delta"] = inp["delta"].float()        # mixed activation dtypes widen to fp32
+    (y, h), (yr, hr) = run_both(inp)
+    assert y.dtype == torch.bfloat16
+    torch.testing.assert_close(y.float(), yr.float(), **HALF_TOL)
+
+
+def test_large_state_dimension():
+    inp = make_inputs(9, 1, 4, 96, 256)
+    inp["A"] = inp["A"] / 16.0
+    (y, h), (yr, hr) = run_both(inp)
+    torch.testing.assert_close(y, yr, rtol=1e-5, atol=3e-5)
+    torch.testing.assert_close(h, hr, **FP32_TOL)
+
+
+def test_non_contiguous_inputs_and_unaligned_lengths():
+    inp = make_inputs(13, 2, 6, 101, 16)
+    big = torch.randn(2, 6, 202)
+    big[:, :, ::2] = inp["u"]
+    inp_nc = dict(inp)
+    ops = _ops()
+    y = ops.selective_scan(big.cuda()[:, :, ::2], dev(inp["delta"]), dev(inp["A"]), dev(inp["B"]),
+                           dev(inp["C"]), D=dev(inp["D"]), z=dev(inp["z"]), dt_bias=dev(inp["dt_bias"]),
+                           softplus=True)
+    yr = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                          dt_bias=inp["dt_bias"], softplus=True)
+    torch.testing.assert_close(y.cpu(), yr, **FP32_TOL)
+
+
+@pytest.mark.parametrize("items", [4, 8, 16])
+def test_every_tile_width_matches_oracle(items):
+    from ssm_amd.ops import _scan_forward
+    inp = make_inputs(17, 2, 8, 1500, 16)
+    yr, hr = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"],
+                              z=inp["z"], dt_bias=inp["dt_bias"], softplus=True, return_last_state=True)
+    y, h = _scan_forward(dev(inp["u"]), dev(inp["delta"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]),
+                         dev(inp["D"]), dev(inp["z"]), dev(inp["dt_bias"]), True, True, tune_items=items)
+    torch.testing.assert_close(y.cpu(), yr, **FP32_TOL)
+    torch.testing.assert_close(h.cpu(), hr, **FP32_TOL)
+
+
+# ---------------------------------------------- benchmark shapes and properties
+
+def test_config0_fp32_full_size_against_oracle():
+    """BASELINE config 0: B=1, D=512, L=2048, N=16, fp32, one group."""
+    inp = make_inputs(0, 1, 512, 2048, 16)
+    inp["A"] = -torch.arange(1, 17, dtype=torch.float32).repeat(512, 1)
+    inp["D"] = torch.ones(512)
+    (y, h), (yr, hr) = run_both(inp)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+    torch.testing.assert_close(h, hr, **FP32_TOL)
+    y64, h64 = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"],
+                                z=inp["z"], dt_bias=inp["dt_bias"], softplus=True,
+                                return_last_state=True, acc=torch.float64)
+    ours = (y.double() - y64.double()).abs().max().item()
+    theirs = (yr.double() - y64.double()).abs().max().item()
+    print(f"config0 max |err| vs fp64: hip {ours:.3e}, fp32 oracle {theirs:.3e}")
+    assert ours < 5e-5
+
+
+def test_config1_shape_bf16_properties():
+    """B=8, D=1536, L=2048, N=16 in bf16: too large for the CPU oracle in a test,
+    so check (a) a slice of channels against the oracle, (b) causality: the
+    first half of the output is bit-identical when the input is truncated, and
+    (c) last_state equals the state reached by continuing from the half-way
+    state (composition of the two halves through a second scan is not
+    available, so compare the half-way last_state of the truncated run with an
+    oracle run on the slice)."""
+    ops = _ops()
+    inp = make_inputs(1, 8, 1536, 2048, 16, dtype=torch.bfloat16)
+    gpu = {k: dev(v) for k, v in inp.items()}
+    y, h = ops.selective_scan(gpu["u"], gpu["delta"], gpu["A"], gpu["B"], gpu["C"], D=gpu["D"],
+                              z=gpu["z"], dt_bias=gpu["dt_bias"], softplus=True, return_last_state=True)
+    assert torch.isfinite(y.float()).all()
+    # (a) channel slice vs oracle (whole batch, 16 channels spread over D)
+    idx = torch.arange(0, 1536, 96)
+    sl = dict(u=inp["u"][:, idx], delta=inp["delta"][:, idx], A=inp["A"][idx], B=inp["B"], C=inp["C"],
+              D=inp["D"][idx], z=inp["z"][:, idx], dt_bias=inp["dt_bias"][idx])
+    yr, hr = O.selective_scan(sl["u"], sl["delta"], sl["A"], sl["B"], sl["C"], D=sl["D"], z=sl["z"],
+                              dt_bias=sl["dt_bias"], softplus=True, return_last_state=True)
+    torch.testing.assert_close(y[:, idx.cuda()].float().cpu(), yr.float(), **HALF_TOL)
+    torch.testing.assert_close(h[:, idx.cuda()].float().cpu(), hr.float(), **HALF_TOL)
+    # (b) causality
+    half = 1024
+    y2 = ops.selective_scan(gpu["u"][:, :, :half], gpu["delta"][:, :, :half], gpu["A"],
+                            gpu["B"][..., :half], gpu["C"][..., :half], D=gpu["D"],
+                            z=gpu["z"][:, :, :half], dt_bias=gpu["dt_bias"], softplus=True)
+    assert torch.equal(y2, y[:, :, :half])
