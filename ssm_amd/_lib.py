@@ -14,7 +14,11 @@ from typing import Optional
 
 import torch
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "libssm_amd.so"
+import os
+
+# SSM_AMD_LIB points the binding at another build of the same C ABI.
+LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
+                Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
 ABI_VERSION = 1
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2

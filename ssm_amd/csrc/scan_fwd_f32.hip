@@ -1,0 +1,6 @@
+// Instantiates the forward selective-scan kernels for f32 activations.
+#include "scan_fwd_kernel.hpp"
+
+namespace ssm {
+template int scan_fwd_dispatch<float>(const ScanFwdParams &, int, int, hipStream_t);
+}

@@ -46,30 +46,48 @@ def _cpu_backend_status() -> _BackendCandidate:
 # selective scan
 # ---------------------------------------------------------------------------
 
+class ScanPlan:
+    """A fully prepared ``ssm_scan_fwd`` call: argument struct, the tensors it
+    points into (kept alive here) and the output buffers.  ``run()`` may be
+    called repeatedly; it enqueues one launch on the current stream."""
+
+    def __init__(self, u, delta, A, B, C, D, z, dt_bias, softplus, want_state, tune_items=0,
+                 out=None, last=None):
+        batch, dim, length, nstate, (bkind, bgroups), (ckind, cgroups) = \
+            K.check_selective_scan(u, delta, A, B, C, D, z, dt_bias)
+        self.device = K.require_gpu(u, delta, A, B, C, D, z, dt_bias)
+        io = K.common_io_dtype([u, delta, z])
+        bc = K.common_io_dtype([B, C])
+        self.result_dtype = u.dtype
+        self.keep = dict(u=K.cast_c(u, io), delta=K.cast_c(delta, io), z=K.cast_c(z, io),
+                         B=K.cast_c(B, bc), C=K.cast_c(C, bc), A=K.as_f32_vec(A),
+                         D=K.as_f32_vec(D), bias=K.as_f32_vec(dt_bias))
+        k = self.keep
+        self.out = out if out is not None else torch.empty_like(k["u"])
+        self.last = last
+        if want_state and last is None:
+            self.last = torch.empty(batch, dim, nstate, dtype=io, device=self.device)
+        self.args = _lib.ScanFwdArgs(
+            u=_lib.ptr(k["u"]), delta=_lib.ptr(k["delta"]), z=_lib.ptr(k["z"]), A=_lib.ptr(k["A"]),
+            Bproj=_lib.ptr(k["B"]), Cproj=_lib.ptr(k["C"]), Dskip=_lib.ptr(k["D"]),
+            dt_bias=_lib.ptr(k["bias"]), out=_lib.ptr(self.out), last_state=_lib.ptr(self.last),
+            batch=batch, dim=dim, seqlen=length, nstate=nstate,
+            io_dtype=_lib.dtype_enum(io), bc_dtype=_lib.dtype_enum(bc),
+            b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
+            delta_softplus=int(bool(softplus)), tune_items=int(tune_items))
+
+    def run(self):
+        _lib.call("ssm_scan_fwd", self.args, self.device)
+        return self.out, self.last
+
+
 def _scan_forward(u, delta, A, B, C, D, z, dt_bias, softplus, want_state, tune_items=0):
     """Validate, normalise dtypes/layout, and run ``ssm_scan_fwd``."""
-    batch, dim, length, nstate, (bkind, bgroups), (ckind, cgroups) = \
-        K.check_selective_scan(u, delta, A, B, C, D, z, dt_bias)
-    dev = K.require_gpu(u, delta, A, B, C, D, z, dt_bias)
-    io = K.common_io_dtype([u, delta, z])
-    bc = K.common_io_dtype([B, C])
-    u_c, dl_c, z_c = K.cast_c(u, io), K.cast_c(delta, io), K.cast_c(z, io)
-    B_c, C_c = K.cast_c(B, bc), K.cast_c(C, bc)
-    A_c, D_c, bias_c = K.as_f32_vec(A), K.as_f32_vec(D), K.as_f32_vec(dt_bias)
-    out = torch.empty_like(u_c)
-    last = torch.empty(batch, dim, nstate, dtype=io, device=dev) if want_state else None
-    args = _lib.ScanFwdArgs(
-        u=_lib.ptr(u_c), delta=_lib.ptr(dl_c), z=_lib.ptr(z_c), A=_lib.ptr(A_c),
-        Bproj=_lib.ptr(B_c), Cproj=_lib.ptr(C_c), Dskip=_lib.ptr(D_c), dt_bias=_lib.ptr(bias_c),
-        out=_lib.ptr(out), last_state=_lib.ptr(last),
-        batch=batch, dim=dim, seqlen=length, nstate=nstate,
-        io_dtype=_lib.dtype_enum(io), bc_dtype=_lib.dtype_enum(bc),
-        b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
-        delta_softplus=int(bool(softplus)), tune_items=int(tune_items))
-    _lib.call("ssm_scan_fwd", args, dev)
-    if out.dtype != u.dtype:
-        out = out.to(u.dtype)
-        last = last.to(u.dtype) if last is not None else None
+    plan = ScanPlan(u, delta, A, B, C, D, z, dt_bias, softplus, want_state, tune_items)
+    out, last = plan.run()
+    if out.dtype != plan.result_dtype:
+        out = out.to(plan.result_dtype)
+        last = last.to(plan.result_dtype) if last is not None else None
     return out, last
 
 
