@@ -74,16 +74,165 @@ typedef struct ssm_scan_fwd_args {
   const float *dt_bias;   /* (D,) fp32, or NULL */
   void *out;              /* (B, D, L) io dtype */
   void *last_state;       /* (B, D, N) io dtype, or NULL */
+  float *chunk_states;    /* (B, D, ceil(L / ssm_scan_chunk_len()), N) fp32, or NULL: the state
+                             entering each chunk, which ssm_scan_bwd restarts from */
   int32_t batch, dim, seqlen, nstate;
   int32_t io_dtype;       /* ssm_dtype of u, delta, z, out, last_state */
   int32_t bc_dtype;       /* ssm_dtype of Bproj and Cproj */
   int32_t b_kind, c_kind; /* ssm_proj_kind */
   int32_t b_groups, c_groups; /* G for SSM_PROJ_BGNL (must divide D), else ignored */
   int32_t delta_softplus; /* 0 / 1 */
-  int32_t tune_items;     /* 0 = automatic; else time steps per lane (4, 8 or 16) */
+  int32_t tune_items;     /* 0 = automatic; else 100 * steps-per-lane + states-per-LDS-pass (408, 808, 816) */
 } ssm_scan_fwd_args;
 
 int ssm_scan_fwd(const ssm_scan_fwd_args *args, void *hip_stream);
+/* Time steps per checkpointed chunk (the granularity of chunk_states). */
+int ssm_scan_chunk_len(void);
+
+/* ------------------------------------------------------------------------
+ * selective scan, backward.  Recomputes the states from `chunk_states` (as
+ * written by ssm_scan_fwd with the same inputs) and returns the gradients of
+ * every input for an upstream gradient `dout` (and optionally one for the
+ * last state).  Stands behind `selective_scan_backward(grad_out,
+ * grad_last_state, u, delta, A, B, C, D, z, dt_bias, softplus, ...)` as
+ * invoked at src/ssm/ops/__init__.py:351-471 (formulas:
+ * src/ssm/ops/cpu/selective_scan.cpp:393-532).  nstate <= 16 per call.
+ * dB / dC have the shape of Bproj / Cproj and are fp32; results are
+ * bit-reproducible (no atomics).
+ * ---------------------------------------------------------------------- */
+typedef struct ssm_scan_bwd_args {
+  const void *u, *delta, *z;      /* (B, D, L) io dtype; z may be NULL */
+  const void *dout;               /* (B, D, L) io dtype */
+  const float *A;                 /* (D, N) */
+  const void *Bproj, *Cproj;      /* as in the forward call, bc dtype */
+  const float *Dskip, *dt_bias;   /* (D,) or NULL */
+  const float *dlast_state;       /* (B, D, N) fp32 gradient of last_state, or NULL */
+  const float *chunk_states;      /* from ssm_scan_fwd */
+  void *du, *ddelta, *dz;         /* (B, D, L) io dtype; dz NULL iff z NULL */
+  float *dA;                      /* (D, N) */
+  float *dB, *dC;                 /* fp32, shape of Bproj / Cproj */
+  float *dD, *ddt_bias;           /* (D,) or NULL */
+  void *workspace;                /* ssm_scan_bwd_workspace_bytes(), 256-byte aligned */
+  size_t workspace_bytes;
+  int32_t batch, dim, seqlen, nstate;
+  int32_t io_dtype, bc_dtype;
+  int32_t b_kind, c_kind, b_groups, c_groups;
+  int32_t delta_softplus;
+} ssm_scan_bwd_args;
+
+size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, int nstate, int b_kind, int c_kind,
+                                    int b_groups, int c_groups);
+int ssm_scan_bwd(const ssm_scan_bwd_args *args, void *hip_stream);
+
+/* ------------------------------------------------------------------------
+ * selective state update for one token (decode step); `state` is updated in
+ * place.  Stands behind `selective_state_step(state, x, dt, A, B, C, D, z,
+ * dt_bias, softplus)` as invoked at src/ssm/ops/__init__.py:1395-1409
+ * (semantics: src/ssm/ops/python/reference.py:197-309).  The grouped
+ * projection form (B, G, N) is passed as SSM_PROJ_BGNL with L = 1.
+ * ---------------------------------------------------------------------- */
+typedef struct ssm_state_step_args {
+  void *state;            /* (B, D, N) state dtype, read and written */
+  const void *x;          /* (B, D) io dtype */
+  const void *dt;         /* (B, D) io dtype */
+  const void *z;          /* (B, D) io dtype, or NULL */
+  const float *A;         /* (D, N) fp32 */
+  const void *Bproj;      /* (D,N) | (B,D,N) | (B,G,N), bc dtype */
+  const void *Cproj;
+  const float *Dskip;     /* (D,) fp32 or NULL */
+  const float *dt_bias;   /* (D,) fp32 or NULL */
+  void *out;              /* (B, D) io dtype */
+  int32_t batch, dim, nstate;
+  int32_t state_dtype, io_dtype, bc_dtype;
+  int32_t b_kind, c_kind, b_groups, c_groups;
+  int32_t dt_softplus;
+} ssm_state_step_args;
+
+int ssm_state_step(const ssm_state_step_args *args, void *hip_stream);
+
+/* ------------------------------------------------------------------------
+ * depthwise causal conv1d (+ optional SiLU).
+ * Forward stands behind `dw_causal_conv(x, weight, bias, activation)`
+ * (src/ssm/ops/__init__.py:1594-1600; semantics reference.py:466-537);
+ * backward behind `dw_causal_conv_backward(grad_out, x, weight, bias,
+ * activation)` (formulas: src/ssm/ops/cpu/dw_causal_conv.cpp:161-204).
+ * ---------------------------------------------------------------------- */
+typedef enum ssm_layout { SSM_LAYOUT_BCL = 0, SSM_LAYOUT_BLC = 1 } ssm_layout;
+typedef enum ssm_activation { SSM_ACT_IDENTITY = 0, SSM_ACT_SILU = 1 } ssm_activation;
+
+typedef struct ssm_conv1d_fwd_args {
+  const void *x;          /* (B,C,L) or (B,L,C), io dtype */
+  const float *weight;    /* (C, K) fp32 */
+  const float *bias;      /* (C,) fp32 or NULL */
+  void *y;                /* same layout and dtype as x */
+  int32_t batch, channels, seqlen, width;
+  int32_t io_dtype, layout, activation;
+} ssm_conv1d_fwd_args;
+
+int ssm_conv1d_fwd(const ssm_conv1d_fwd_args *args, void *hip_stream);
+
+typedef struct ssm_conv1d_bwd_args {
+  const void *x;          /* forward input */
+  const void *dout;       /* gradient of y, same layout/dtype as x */
+  const float *weight;
+  const float *bias;      /* or NULL (needed to rebuild the pre-activation) */
+  void *dx;               /* same layout/dtype as x */
+  float *dweight;         /* (C, K) fp32 */
+  float *dbias;           /* (C,) fp32 or NULL */
+  void *workspace;        /* ssm_conv1d_bwd_workspace_bytes() bytes of device memory */
+  size_t workspace_bytes;
+  int32_t batch, channels, seqlen, width;
+  int32_t io_dtype, layout, activation;
+} ssm_conv1d_bwd_args;
+
+size_t ssm_conv1d_bwd_workspace_bytes(int batch, int channels, int width);
+int ssm_conv1d_bwd(const ssm_conv1d_bwd_args *args, void *hip_stream);
+
+/* ------------------------------------------------------------------------
+ * residual-add + LayerNorm / RMSNorm over the last axis of (rows, hidden).
+ * Forward stands behind `fused_layer_norm(x, weight, bias, residual, is_rms,
+ * eps, prenorm, residual_in_fp32)` (src/ssm/ops/__init__.py:1640-1652;
+ * semantics reference.py:540-609) and can additionally emit the pre-norm sum
+ * (`residual_out`) and the row statistics; backward stands behind
+ * `fused_layer_norm_backward` (formulas: src/ssm/ops/cpu/layer_norm.cpp:277-336).
+ * ---------------------------------------------------------------------- */
+typedef struct ssm_norm_fwd_args {
+  const void *x;            /* (rows, hidden) x dtype */
+  const void *residual;     /* (rows, hidden) residual dtype, or NULL */
+  const float *weight;      /* (hidden,) fp32 */
+  const float *bias;        /* (hidden,) fp32 or NULL */
+  void *y;                  /* (rows, hidden) x dtype */
+  void *residual_out;       /* (rows, hidden) residual_out dtype, or NULL: x (+ residual if prenorm) */
+  float *mean;              /* (rows,) or NULL (written as 0 for RMSNorm) */
+  float *rstd;              /* (rows,) or NULL */
+  int32_t rows, hidden;
+  int32_t x_dtype, residual_dtype, residual_out_dtype;
+  int32_t is_rms, prenorm;
+  float eps;
+} ssm_norm_fwd_args;
+
+int ssm_norm_fwd(const ssm_norm_fwd_args *args, void *hip_stream);
+
+typedef struct ssm_norm_bwd_args {
+  const void *x;
+  const void *residual;     /* or NULL */
+  const void *dy;           /* (rows, hidden) x dtype */
+  const float *weight;
+  const float *mean;        /* (rows,) from the forward pass (ignored for RMSNorm) */
+  const float *rstd;        /* (rows,) from the forward pass */
+  void *dx;                 /* (rows, hidden) x dtype */
+  void *dresidual;          /* (rows, hidden) residual dtype, or NULL */
+  float *dweight;           /* (hidden,) fp32 */
+  float *dbias;             /* (hidden,) fp32 or NULL */
+  void *workspace;          /* ssm_norm_bwd_workspace_bytes() bytes of device memory */
+  size_t workspace_bytes;
+  int32_t rows, hidden;
+  int32_t x_dtype, residual_dtype;
+  int32_t is_rms, prenorm;
+} ssm_norm_bwd_args;
+
+size_t ssm_norm_bwd_workspace_bytes(int rows, int hidden);
+int ssm_norm_bwd(const ssm_norm_bwd_args *args, void *hip_stream);
 
 #ifdef __cplusplus
 }

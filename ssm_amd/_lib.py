@@ -40,18 +40,97 @@ class KernelError(RuntimeError):
 class ScanFwdArgs(C.Structure):
     _fields_ = [
         ("u", _vp), ("delta", _vp), ("z", _vp), ("A", _vp), ("Bproj", _vp), ("Cproj", _vp),
-        ("Dskip", _vp), ("dt_bias", _vp), ("out", _vp), ("last_state", _vp),
+        ("Dskip", _vp), ("dt_bias", _vp), ("out", _vp), ("last_state", _vp), ("chunk_states", _vp),
         ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32),
         ("io_dtype", _i32), ("bc_dtype", _i32), ("b_kind", _i32), ("c_kind", _i32),
         ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("tune_items", _i32),
     ]
 
 
+class ScanBwdArgs(C.Structure):
+    _fields_ = [
+        ("u", _vp), ("delta", _vp), ("z", _vp), ("dout", _vp), ("A", _vp), ("Bproj", _vp), ("Cproj", _vp),
+        ("Dskip", _vp), ("dt_bias", _vp), ("dlast_state", _vp), ("chunk_states", _vp),
+        ("du", _vp), ("ddelta", _vp), ("dz", _vp), ("dA", _vp), ("dB", _vp), ("dC", _vp), ("dD", _vp),
+        ("ddt_bias", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
+        ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32),
+        ("io_dtype", _i32), ("bc_dtype", _i32), ("b_kind", _i32), ("c_kind", _i32),
+        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32),
+    ]
+
+
+class StateStepArgs(C.Structure):
+    _fields_ = [
+        ("state", _vp), ("x", _vp), ("dt", _vp), ("z", _vp), ("A", _vp), ("Bproj", _vp), ("Cproj", _vp),
+        ("Dskip", _vp), ("dt_bias", _vp), ("out", _vp),
+        ("batch", _i32), ("dim", _i32), ("nstate", _i32),
+        ("state_dtype", _i32), ("io_dtype", _i32), ("bc_dtype", _i32),
+        ("b_kind", _i32), ("c_kind", _i32), ("b_groups", _i32), ("c_groups", _i32),
+        ("dt_softplus", _i32),
+    ]
+
+
+LAYOUT_BCL, LAYOUT_BLC = 0, 1
+ACT_IDENTITY, ACT_SILU = 0, 1
+
+
+class Conv1dFwdArgs(C.Structure):
+    _fields_ = [
+        ("x", _vp), ("weight", _vp), ("bias", _vp), ("y", _vp),
+        ("batch", _i32), ("channels", _i32), ("seqlen", _i32), ("width", _i32),
+        ("io_dtype", _i32), ("layout", _i32), ("activation", _i32),
+    ]
+
+
+class Conv1dBwdArgs(C.Structure):
+    _fields_ = [
+        ("x", _vp), ("dout", _vp), ("weight", _vp), ("bias", _vp), ("dx", _vp), ("dweight", _vp),
+        ("dbias", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
+        ("batch", _i32), ("channels", _i32), ("seqlen", _i32), ("width", _i32),
+        ("io_dtype", _i32), ("layout", _i32), ("activation", _i32),
+    ]
+
+
+class NormFwdArgs(C.Structure):
+    _fields_ = [
+        ("x", _vp), ("residual", _vp), ("weight", _vp), ("bias", _vp), ("y", _vp), ("residual_out", _vp),
+        ("mean", _vp), ("rstd", _vp),
+        ("rows", _i32), ("hidden", _i32),
+        ("x_dtype", _i32), ("residual_dtype", _i32), ("residual_out_dtype", _i32),
+        ("is_rms", _i32), ("prenorm", _i32), ("eps", _f32),
+    ]
+
+
+class NormBwdArgs(C.Structure):
+    _fields_ = [
+        ("x", _vp), ("residual", _vp), ("dy", _vp), ("weight", _vp), ("mean", _vp), ("rstd", _vp),
+        ("dx", _vp), ("dresidual", _vp), ("dweight", _vp), ("dbias", _vp),
+        ("workspace", _vp), ("workspace_bytes", C.c_size_t),
+        ("rows", _i32), ("hidden", _i32), ("x_dtype", _i32), ("residual_dtype", _i32),
+        ("is_rms", _i32), ("prenorm", _i32),
+    ]
+
+
 # name -> argument struct (every entry point is ``int f(const args*, void* stream)``)
 ENTRY_POINTS = {
     "ssm_scan_fwd": ScanFwdArgs,
+    "ssm_scan_bwd": ScanBwdArgs,
+    "ssm_state_step": StateStepArgs,
+    "ssm_conv1d_fwd": Conv1dFwdArgs,
+    "ssm_conv1d_bwd": Conv1dBwdArgs,
+    "ssm_norm_fwd": NormFwdArgs,
+    "ssm_norm_bwd": NormBwdArgs,
 }
-PLAIN_SYMBOLS = ["ssm_amd_abi_version", "ssm_amd_status_string", "ssm_amd_last_error"]
+# name -> (restype, argtypes) of the remaining exported functions
+PLAIN_SYMBOLS = {
+    "ssm_amd_abi_version": (C.c_int, []),
+    "ssm_amd_status_string": (C.c_char_p, [C.c_int]),
+    "ssm_amd_last_error": (C.c_char_p, []),
+    "ssm_scan_chunk_len": (C.c_int, []),
+    "ssm_scan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 8),
+    "ssm_conv1d_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
+    "ssm_norm_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+}
 
 _lock = threading.Lock()
 _lib: Optional[C.CDLL] = None
@@ -73,10 +152,10 @@ def load() -> C.CDLL:
                 raise FileNotFoundError(
                     f"{LIB_PATH} not found: build it with `python -m ssm_amd.build`")
             lib = C.CDLL(str(LIB_PATH))
-            lib.ssm_amd_abi_version.restype = C.c_int
-            lib.ssm_amd_status_string.restype = C.c_char_p
-            lib.ssm_amd_status_string.argtypes = [C.c_int]
-            lib.ssm_amd_last_error.restype = C.c_char_p
+            for name, (res, argt) in PLAIN_SYMBOLS.items():
+                fn = getattr(lib, name)
+                fn.restype = res
+                fn.argtypes = argt
             got = lib.ssm_amd_abi_version()
             if got != ABI_VERSION:
                 raise RuntimeError(f"libssm_amd ABI {got}, binding expects {ABI_VERSION}")

@@ -1,0 +1,420 @@
+// Depthwise causal 1-D convolution (+ optional SiLU), forward and backward.
+//
+//   pre[b,c,t] = bias[c] + sum_k w[c,k] x[b,c,t-(K-1)+k]      (x = 0 for t < 0)
+//   y          = silu(pre) or pre
+//
+// Pure streaming kernels: every thread owns one 16-byte run of the output
+// (VEC elements) and rebuilds its input window from the 16-byte runs around
+// it, so HBM sees each byte once and the overlap is served by L1/L2.
+//   channels-first (B,C,L): runs are along time; one workgroup per (b,c) row.
+//   channels-last  (B,L,C): runs are along channels; a thread slides over a
+//                           strip of time steps keeping K rows in registers.
+// Shapes the vector path cannot take (misaligned rows, K-1 > VEC) go through
+// an element-wise kernel with explicit bounds.
+//
+// Backward recomputes pre (no activation is saved), forms g = dout*silu'(pre),
+// emits dx = sum_k g[t+(K-1)-k] w[k] and per-row partial sums of dw/dbias that
+// a second kernel folds over the batch in a fixed order (no atomics).
+#include "common.hpp"
+
+namespace ssm {
+
+constexpr int CONV_TAPS = 5;           // widest kernel the vector paths take (K <= 5)
+constexpr int CONV_THREADS = 256;
+
+// Taps in reverse order: wrev[m] multiplies x[t - m]; zero beyond the kernel width.
+__device__ __forceinline__ void load_taps(const float *w, int c, int K, float (&wrev)[CONV_TAPS]) {
+#pragma unroll
+  for (int m = 0; m < CONV_TAPS; ++m) wrev[m] = m < K ? w[(size_t)c * K + (K - 1 - m)] : 0.0f;
+}
+
+struct ConvParams {
+  const void *x, *dout;
+  const float *w, *bias;     // (C,K) fp32, (C,) fp32 or null
+  void *y;                   // fwd: y ; bwd: dx
+  float *partial;            // bwd: [B][C][K+1] partial sums (dw..., dbias)
+  int batch, chans, len, K;
+  int silu;
+};
+
+__device__ __forceinline__ float silu_grad(float pre) {
+  const float s = sigmoid_f32(pre);
+  return s * __builtin_fmaf(pre, 1.0f - s, 1.0f);
+}
+
+// ---------------------------------------------------------------- forward, (B,C,L)
+
+template <typename T>
+__global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvParams p) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int row = blockIdx.x;                       // b * C + c
+  const int c = row % p.chans;
+  const T *xr = reinterpret_cast<const T *>(p.x) + (size_t)row * p.len;
+  T *yr = reinterpret_cast<T *>(p.y) + (size_t)row * p.len;
+  float wrev[CONV_TAPS];
+  load_taps(p.w, c, p.K, wrev);
+  const float bias = p.bias ? p.bias[c] : 0.0f;
+  for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
+    float win[2 * VEC];
+    if (t0 > 0) {
+      float prev[VEC];
+      load_run<T, VEC>(xr, t0 - VEC, p.len, true, prev);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) win[i] = prev[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) win[i] = 0.0f;
+    }
+    {
+      float cur[VEC];
+      load_run<T, VEC>(xr, t0, p.len, true, cur);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) win[VEC + i] = cur[i];
+    }
+    float out[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float acc = bias;
+#pragma unroll
+      for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[m], win[VEC + i - m], acc);
+      out[i] = p.silu ? silu_f32(acc) : acc;
+    }
+    store_run<T, VEC>(yr, t0, p.len, true, out);
+  }
+}
+
+// Element-wise forward for any K / alignment, either layout.
+template <typename T>
+__global__ __launch_bounds__(CONV_THREADS) void conv_fwd_generic_kernel(const ConvParams p, int channels_last) {
+  const size_t total = (size_t)p.batch * p.chans * p.len;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+    int b, c, t;
+    if (channels_last) { c = (int)(e % p.chans); t = (int)((e / p.chans) % p.len); b = (int)(e / ((size_t)p.chans * p.len)); }
+    else { t = (int)(e % p.len); c = (int)((e / p.len) % p.chans); b = (int)(e / ((size_t)p.chans * p.len)); }
+    float acc = p.bias ? p.bias[c] : 0.0f;
+    for (int k = 0; k < p.K; ++k) {
+      const int ts = t - (p.K - 1) + k;
+      if (ts < 0) continue;
+      const size_t idx = channels_last ? ((size_t)b * p.len + ts) * p.chans + c : ((size_t)b * p.chans + c) * p.len + ts;
+      acc = __builtin_fmaf(p.w[(size_t)c * p.K + k], to_f32(reinterpret_cast<const T *>(p.x)[idx]), acc);
+    }
+    reinterpret_cast<T *>(p.y)[e] = from_f32<T>(p.silu ? silu_f32(acc) : acc);
+  }
+}
+
+// ---------------------------------------------------------------- forward, (B,L,C)
+
+constexpr int CONV_CL_STRIP = 16;   // time steps per thread
+
+template <typename T>
+__global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvParams p) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int cvecs = p.chans / VEC;
+  const int strips = (p.len + CONV_CL_STRIP - 1) / CONV_CL_STRIP;
+  const size_t total = (size_t)p.batch * strips * cvecs;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int cv = (int)(gid % cvecs);
+  const int strip = (int)((gid / cvecs) % strips);
+  const int b = (int)(gid / ((size_t)cvecs * strips));
+  const int c0 = cv * VEC;
+  const int K = p.K;
+  constexpr int HIST = CONV_TAPS - 1;
+  float wrev[VEC][CONV_TAPS], bias[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    bias[i] = p.bias ? p.bias[c0 + i] : 0.0f;
+    load_taps(p.w, c0 + i, K, wrev[i]);
+  }
+  const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
+  T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
+  const int t_begin = strip * CONV_CL_STRIP;
+  const int t_end = min(p.len, t_begin + CONV_CL_STRIP);
+  // hist[j] holds x at time (t - 1 - j); filled with the K-1 rows before the strip
+  float hist[HIST][VEC];
+#pragma unroll
+  for (int j = 0; j < HIST; ++j) {
+    const int ts = t_begin - 1 - j;
+    float v[VEC];
+    if (j < K - 1 && ts >= 0) load_run<T, VEC>(xb + (size_t)ts * p.chans, 0, VEC, true, v);
+    else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) hist[j][i] = v[i];
+  }
+  for (int t = t_begin; t < t_end; ++t) {
+    float cur[VEC], out[VEC];
+    load_run<T, VEC>(xb + (size_t)t * p.chans, 0, VEC, true, cur);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float acc = __builtin_fmaf(wrev[i][0], cur[i], bias[i]);
+#pragma unroll
+      for (int j = 0; j < HIST; ++j) acc = __builtin_fmaf(wrev[i][j + 1], hist[j][i], acc);
+      out[i] = p.silu ? silu_f32(acc) : acc;
+    }
+    store_run<T, VEC>(yb + (size_t)t * p.chans, 0, VEC, true, out);
+#pragma unroll
+    for (int j = HIST - 1; j > 0; --j)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) hist[j][i] = hist[j - 1][i];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) hist[0][i] = cur[i];
+  }
+}
+
+// --------------------------------------------------------------- backward, (B,C,L)
+
+template <typename T>
+__global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvParams p) {
+  constexpr int VEC = 16 / sizeof(T);
+  __shared__ float red[CONV_THREADS / WAVE][CONV_TAPS + 1];
+  const int row = blockIdx.x;
+  const int c = row % p.chans;
+  const int K = p.K;
+  const T *xr = reinterpret_cast<const T *>(p.x) + (size_t)row * p.len;
+  const T *gr = reinterpret_cast<const T *>(p.dout) + (size_t)row * p.len;
+  T *dxr = reinterpret_cast<T *>(p.y) + (size_t)row * p.len;
+  float wrev[CONV_TAPS];
+  load_taps(p.w, c, K, wrev);
+  const float bias = p.bias ? p.bias[c] : 0.0f;
+  float dwrev[CONV_TAPS], db = 0.0f;
+#pragma unroll
+  for (int m = 0; m < CONV_TAPS; ++m) dwrev[m] = 0.0f;
+
+  for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
+    // x over [t0-VEC, t0+2*VEC), dout over [t0, t0+2*VEC)
+    float xw[3 * VEC], g[2 * VEC];
+    {
+      float v[VEC];
+      if (t0 > 0) load_run<T, VEC>(xr, t0 - VEC, p.len, true, v);
+      else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = 0.0f;
+      }
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) xw[i] = v[i];
+      load_run<T, VEC>(xr, t0, p.len, true, v);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) xw[VEC + i] = v[i];
+      load_run<T, VEC>(xr, t0 + VEC, p.len, true, v);       // zero past the end
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) xw[2 * VEC + i] = v[i];
+      load_run<T, VEC>(gr, t0, p.len, true, v);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) g[i] = v[i];
+      load_run<T, VEC>(gr, t0 + VEC, p.len, true, v);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) g[VEC + i] = v[i];
+    }
+    if (p.silu) {
+      // g <- dout * silu'(pre) on [t0, t0 + VEC + K - 1)
+#pragma unroll
+      for (int i = 0; i < 2 * VEC; ++i) {
+        if (i < VEC + K - 1) {
+          float pre = bias;
+#pragma unroll
+          for (int m = 0; m < CONV_TAPS; ++m) pre = __builtin_fmaf(wrev[m], xw[VEC + i - m], pre);
+          g[i] *= silu_grad(pre);
+        }
+      }
+    }
+    float dx[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(g[i + m], wrev[m], acc);
+      dx[i] = acc;
+      db += g[i];
+#pragma unroll
+      for (int m = 0; m < CONV_TAPS; ++m) dwrev[m] = __builtin_fmaf(g[i], xw[VEC + i - m], dwrev[m]);
+    }
+    store_run<T, VEC>(dxr, t0, p.len, true, dx);
+  }
+  // block reduction of dw[0..K) and db
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int m = 0; m < CONV_TAPS; ++m) {
+    const float s = wave_sum(dwrev[m]);
+    if (lane == 0) red[wave][m] = s;
+  }
+  {
+    const float s = wave_sum(db);
+    if (lane == 0) red[wave][CONV_TAPS] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x <= K) {
+    // slot k < K holds dw[k] = dwrev[K-1-k]; slot K holds dbias
+    const int src = threadIdx.x < K ? (K - 1 - (int)threadIdx.x) : CONV_TAPS;
+    float s = 0.0f;
+    for (int wv = 0; wv < CONV_THREADS / WAVE; ++wv) s += red[wv][src];
+    p.partial[(size_t)row * (K + 1) + threadIdx.x] = s;
+  }
+}
+
+// Element-wise backward (any K / alignment, either layout): one thread per
+// (b, c) row walks the row sequentially.  Slow path, correctness only.
+template <typename T>
+__global__ __launch_bounds__(CONV_THREADS) void conv_bwd_generic_kernel(const ConvParams p, int channels_last) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= p.batch * p.chans) return;
+  const int b = row / p.chans, c = row % p.chans;
+  const int K = p.K;
+  auto at = [&](int t) -> size_t {
+    return channels_last ? ((size_t)b * p.len + t) * p.chans + c : ((size_t)b * p.chans + c) * p.len + t;
+  };
+  const T *x = reinterpret_cast<const T *>(p.x);
+  const T *go = reinterpret_cast<const T *>(p.dout);
+  T *dx = reinterpret_cast<T *>(p.y);
+  const float bias = p.bias ? p.bias[c] : 0.0f;
+  auto gval = [&](int t) -> float {
+    float g = to_f32(go[at(t)]);
+    if (p.silu) {
+      float pre = bias;
+      for (int k = 0; k < K; ++k) {
+        const int ts = t - (K - 1) + k;
+        if (ts >= 0) pre = __builtin_fmaf(p.w[(size_t)c * K + k], to_f32(x[at(ts)]), pre);
+      }
+      g *= silu_grad(pre);
+    }
+    return g;
+  };
+  float *part = p.partial + (size_t)row * (K + 1);
+  for (int k = 0; k <= K; ++k) part[k] = 0.0f;
+  for (int t = 0; t < p.len; ++t) {
+    const float g = gval(t);
+    part[K] += g;
+    for (int k = 0; k < K; ++k) {
+      const int ts = t - (K - 1) + k;
+      if (ts >= 0) part[k] = __builtin_fmaf(g, to_f32(x[at(ts)]), part[k]);
+    }
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) {
+      const int tg = t + (K - 1) - k;
+      if (tg < p.len) acc = __builtin_fmaf(gval(tg), p.w[(size_t)c * K + k], acc);
+    }
+    dx[at(t)] = from_f32<T>(acc);
+  }
+}
+
+// dw[c,k] = sum_b partial[b][c][k], dbias[c] = sum_b partial[b][c][K]; fixed order.
+__global__ __launch_bounds__(CONV_THREADS) void conv_bwd_fold_kernel(const float *partial, float *dw, float *dbias,
+                                                                      int batch, int chans, int K) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= chans * (K + 1)) return;
+  const int c = e / (K + 1), k = e % (K + 1);
+  float s = 0.0f;
+  for (int b = 0; b < batch; ++b) s += partial[((size_t)b * chans + c) * (K + 1) + k];
+  if (k < K) dw[(size_t)c * K + k] = s;
+  else if (dbias) dbias[c] = s;
+}
+
+template <typename T>
+static int conv_fwd_typed(const ConvParams &p, int channels_last, bool vec_ok, hipStream_t s) {
+  constexpr int VEC = 16 / sizeof(T);
+  const size_t total = (size_t)p.batch * p.chans * p.len;
+  if (vec_ok && p.K <= CONV_TAPS && !channels_last && p.len % VEC == 0) {
+    hipLaunchKernelGGL(conv_fwd_cf_kernel<T>, dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+  } else if (vec_ok && p.K <= CONV_TAPS && channels_last && p.chans % VEC == 0) {
+    const int strips = (p.len + CONV_CL_STRIP - 1) / CONV_CL_STRIP;
+    const size_t threads = (size_t)p.batch * strips * (p.chans / VEC);
+    hipLaunchKernelGGL(conv_fwd_cl_kernel<T>, dim3((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS)),
+                       dim3(CONV_THREADS), 0, s, p);
+  } else {
+    const unsigned grid = (unsigned)min((size_t)65535 * 16, (total + CONV_THREADS - 1) / CONV_THREADS);
+    hipLaunchKernelGGL(conv_fwd_generic_kernel<T>, dim3(grid), dim3(CONV_THREADS), 0, s, p, channels_last);
+  }
+  SSM_CHECK_LAUNCH("ssm_conv1d_fwd");
+  return SSM_OK;
+}
+
+template <typename T>
+static int conv_bwd_typed(const ConvParams &p, int channels_last, bool vec_ok, float *dw, float *dbias,
+                          hipStream_t s) {
+  constexpr int VEC = 16 / sizeof(T);
+  if (vec_ok && p.K <= CONV_TAPS && !channels_last && p.len % VEC == 0) {
+    hipLaunchKernelGGL(conv_bwd_cf_kernel<T>, dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+  } else {
+    const int rows = p.batch * p.chans;
+    hipLaunchKernelGGL(conv_bwd_generic_kernel<T>, dim3((rows + CONV_THREADS - 1) / CONV_THREADS),
+                       dim3(CONV_THREADS), 0, s, p, channels_last);
+  }
+  SSM_CHECK_LAUNCH("ssm_conv1d_bwd");
+  const int n = p.chans * (p.K + 1);
+  hipLaunchKernelGGL(conv_bwd_fold_kernel, dim3((n + CONV_THREADS - 1) / CONV_THREADS), dim3(CONV_THREADS), 0, s,
+                     p.partial, dw, dbias, p.batch, p.chans, p.K);
+  SSM_CHECK_LAUNCH("ssm_conv1d_bwd(fold)");
+  return SSM_OK;
+}
+
+static int conv_check(const char *who, const void *x, const void *w, const void *y, int batch, int chans, int len,
+                      int K, int dtype, int layout, int act) {
+  SSM_REQUIRE(x && w && y, SSM_ERR_NULL_POINTER, "%s: x, weight and output are required", who);
+  SSM_REQUIRE(batch > 0 && chans > 0 && len > 0 && K > 0, SSM_ERR_BAD_SHAPE,
+              "%s: batch=%d channels=%d seqlen=%d width=%d must all be positive", who, batch, chans, len, K);
+  SSM_REQUIRE(valid_dtype(dtype), SSM_ERR_BAD_DTYPE, "%s: dtype=%d", who, dtype);
+  SSM_REQUIRE(layout == SSM_LAYOUT_BCL || layout == SSM_LAYOUT_BLC, SSM_ERR_BAD_KIND, "%s: layout=%d", who, layout);
+  SSM_REQUIRE(act == SSM_ACT_IDENTITY || act == SSM_ACT_SILU, SSM_ERR_BAD_KIND, "%s: activation=%d", who, act);
+  SSM_REQUIRE((size_t)batch * chans < ((size_t)1 << 31) && (size_t)batch * chans * len < ((size_t)1 << 40),
+              SSM_ERR_TOO_LARGE, "%s: tensor too large", who);
+  const int es = dtype_size(dtype);
+  SSM_REQUIRE(aligned_to(x, es) && aligned_to(y, es) && aligned_to(w, 4), SSM_ERR_ALIGNMENT,
+              "%s: a pointer is not aligned to its element size", who);
+  return SSM_OK;
+}
+
+}  // namespace ssm
+
+extern "C" int ssm_conv1d_fwd(const ssm_conv1d_fwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_conv1d_fwd: args is NULL");
+  int rc = conv_check("ssm_conv1d_fwd", a->x, a->weight, a->y, a->batch, a->channels, a->seqlen, a->width,
+                      a->io_dtype, a->layout, a->activation);
+  if (rc != SSM_OK) return rc;
+  ConvParams p{};
+  p.x = a->x; p.w = a->weight; p.bias = a->bias; p.y = a->y;
+  p.batch = a->batch; p.chans = a->channels; p.len = a->seqlen; p.K = a->width;
+  p.silu = a->activation == SSM_ACT_SILU;
+  const bool vec_ok = aligned_to(a->x, 16) && aligned_to(a->y, 16);
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  const int cl = a->layout == SSM_LAYOUT_BLC;
+  switch (a->io_dtype) {
+    case SSM_F32: return conv_fwd_typed<float>(p, cl, vec_ok, s);
+    case SSM_BF16: return conv_fwd_typed<bf16_t>(p, cl, vec_ok, s);
+    default: return conv_fwd_typed<f16_t>(p, cl, vec_ok, s);
+  }
+}
+
+extern "C" size_t ssm_conv1d_bwd_workspace_bytes(int batch, int channels, int width) {
+  if (batch <= 0 || channels <= 0 || width <= 0) return 0;
+  return (size_t)batch * channels * (width + 1) * sizeof(float);
+}
+
+extern "C" int ssm_conv1d_bwd(const ssm_conv1d_bwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_conv1d_bwd: args is NULL");
+  int rc = conv_check("ssm_conv1d_bwd", a->x, a->weight, a->dx, a->batch, a->channels, a->seqlen, a->width,
+                      a->io_dtype, a->layout, a->activation);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(a->dout && a->dweight, SSM_ERR_NULL_POINTER, "ssm_conv1d_bwd: dout and dweight are required");
+  SSM_REQUIRE(a->workspace && a->workspace_bytes >= ssm_conv1d_bwd_workspace_bytes(a->batch, a->channels, a->width),
+              SSM_ERR_WORKSPACE, "ssm_conv1d_bwd: workspace of %zu bytes required",
+              ssm_conv1d_bwd_workspace_bytes(a->batch, a->channels, a->width));
+  SSM_REQUIRE(aligned_to(a->dout, dtype_size(a->io_dtype)) && aligned_to(a->dweight, 4) && aligned_to(a->workspace, 4),
+              SSM_ERR_ALIGNMENT, "ssm_conv1d_bwd: a pointer is not aligned to its element size");
+  ConvParams p{};
+  p.x = a->x; p.dout = a->dout; p.w = a->weight; p.bias = a->bias; p.y = a->dx;
+  p.partial = reinterpret_cast<float *>(a->workspace);
+  p.batch = a->batch; p.chans = a->channels; p.len = a->seqlen; p.K = a->width;
+  p.silu = a->activation == SSM_ACT_SILU;
+  const bool vec_ok = aligned_to(a->x, 16) && aligned_to(a->dx, 16) && aligned_to(a->dout, 16);
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  const int cl = a->layout == SSM_LAYOUT_BLC;
+  switch (a->io_dtype) {
+    case SSM_F32: return conv_bwd_typed<float>(p, cl, vec_ok, a->dweight, a->dbias, s);
+    case SSM_BF16: return conv_bwd_typed<bf16_t>(p, cl, vec_ok, a->dweight, a->dbias, s);
+    default: return conv_bwd_typed<f16_t>(p, cl, vec_ok, a->dweight, a->dbias, s);
+  }
+}

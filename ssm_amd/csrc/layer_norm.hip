@@ -1,0 +1,414 @@
+// Residual-add + LayerNorm / RMSNorm, forward and backward, for gfx950.
+//
+//   v = x (+ residual when prenorm)           accumulated in fp32
+//   LayerNorm: y = (v - mean) * rsqrt(var + eps) * w + b     (two-pass biased variance)
+//   RMSNorm:   y = v * rsqrt(mean(v^2) + eps) * w + b
+//   post-norm: y += residual
+//
+// One wavefront normalises one row and keeps the row in registers, so x and
+// the residual are read from HBM exactly once and y / residual_out are written
+// once; row statistics (mean, rstd) can be saved for the backward pass.
+// Rows longer than the register budget (64 lanes * 32 values) fall back to a
+// re-reading variant.
+//
+// Backward: a persistent grid walks rows; each wavefront produces dx (and
+// dresidual) for its rows and accumulates dw/db columns in registers; per-wave
+// partials are written once and folded by a second kernel in a fixed order.
+#include "common.hpp"
+
+namespace ssm {
+
+constexpr int LN_THREADS = 256;
+constexpr int LN_WAVES = LN_THREADS / WAVE;
+constexpr int LN_MAX_PER_LANE = 32;          // cached values per lane -> hidden <= 2048
+
+struct NormParams {
+  const void *x, *res, *dy;
+  const float *w, *b;
+  void *y, *res_out, *dx, *dres;
+  float *mean, *rstd;       // per row; fwd: optional outputs, bwd: required inputs (mean unused for RMS)
+  float *partial;           // bwd: [nwaves_total][2][hidden]
+  int rows, hidden;
+  int x_dtype, res_dtype, res_out_dtype;
+  int is_rms, prenorm;
+  float eps;
+};
+
+__device__ __forceinline__ void store_f32_as(void *p, int dtype, size_t i, float v) {
+  if (dtype == SSM_F32) reinterpret_cast<float *>(p)[i] = v;
+  else if (dtype == SSM_BF16) reinterpret_cast<bf16_t *>(p)[i] = from_f32<bf16_t>(v);
+  else reinterpret_cast<f16_t *>(p)[i] = from_f32<f16_t>(v);
+}
+
+// Row element j of lane `lane`, trip `k`: column = (k * 64 + lane) * VEC + i.
+template <int VEC>
+__device__ __forceinline__ void load_cols(const void *p, int dtype, size_t base, int col, int hidden, bool vec_ok,
+                                          float (&v)[VEC]) {
+  if (vec_ok && col + VEC <= hidden) {
+    if (dtype == SSM_F32) {
+      Pack<float, VEC> r = *reinterpret_cast<const Pack<float, VEC> *>(reinterpret_cast<const float *>(p) + base + col);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = r.v[i];
+    } else if (dtype == SSM_BF16) {
+      Pack<bf16_t, VEC> r = *reinterpret_cast<const Pack<bf16_t, VEC> *>(reinterpret_cast<const bf16_t *>(p) + base + col);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = to_f32(r.v[i]);
+    } else {
+      Pack<f16_t, VEC> r = *reinterpret_cast<const Pack<f16_t, VEC> *>(reinterpret_cast<const f16_t *>(p) + base + col);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = to_f32(r.v[i]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = (col + i < hidden) ? load_as_f32(p, dtype, base + col + i) : 0.0f;
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_cols(void *p, int dtype, size_t base, int col, int hidden, bool vec_ok,
+                                           const float (&v)[VEC]) {
+  if (vec_ok && col + VEC <= hidden) {
+    if (dtype == SSM_F32) {
+      Pack<float, VEC> r;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) r.v[i] = v[i];
+      *reinterpret_cast<Pack<float, VEC> *>(reinterpret_cast<float *>(p) + base + col) = r;
+    } else if (dtype == SSM_BF16) {
+      Pack<bf16_t, VEC> r;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) r.v[i] = from_f32<bf16_t>(v[i]);
+      *reinterpret_cast<Pack<bf16_t, VEC> *>(reinterpret_cast<bf16_t *>(p) + base + col) = r;
+    } else {
+      Pack<f16_t, VEC> r;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) r.v[i] = from_f32<f16_t>(v[i]);
+      *reinterpret_cast<Pack<f16_t, VEC> *>(reinterpret_cast<f16_t *>(p) + base + col) = r;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+      if (col + i < hidden) store_f32_as(p, dtype, base + col + i, v[i]);
+  }
+}
+
+// ------------------------------------------------------------------ forward
+
+// TRIPS * 64 * VEC >= hidden; VEC = 4 keeps every access <= 16 bytes for all dtypes.
+template <int TRIPS>
+__global__ __launch_bounds__(LN_THREADS) void norm_fwd_kernel(const NormParams p, int vec_ok) {
+  constexpr int VEC = 4;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row = blockIdx.x * LN_WAVES + wave;
+  if (row >= p.rows) return;
+  const int H = p.hidden;
+  const size_t base = (size_t)row * H;
+  const bool vok = vec_ok != 0;
+  float v[TRIPS][VEC], r[TRIPS][VEC];
+  float sum = 0.0f;
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int col = (k * WAVE + lane) * VEC;
+    load_cols<VEC>(p.x, p.x_dtype, base, col, H, vok, v[k]);
+    if (p.res) {
+      load_cols<VEC>(p.res, p.res_dtype, base, col, H, vok, r[k]);
+      if (p.prenorm) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[k][i] += r[k][i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) sum += v[k][i];
+    if (p.res_out) store_cols<VEC>(p.res_out, p.res_out_dtype, base, col, H, vok, v[k]);
+  }
+  const float inv_h = 1.0f / (float)H;
+  float mean = 0.0f;
+  if (!p.is_rms) mean = wave_sum(sum) * inv_h;
+  float sq = 0.0f;
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int col = (k * WAVE + lane) * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float c = (col + i < H) ? v[k][i] - mean : 0.0f;
+      sq = __builtin_fmaf(c, c, sq);
+    }
+  }
+  const float rstd = 1.0f / sqrtf(wave_sum(sq) * inv_h + p.eps);
+  if (lane == 0) {
+    if (p.mean) p.mean[row] = mean;
+    if (p.rstd) p.rstd[row] = rstd;
+  }
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int col = (k * WAVE + lane) * VEC;
+    if (col >= H) continue;
+    float wv[VEC], bv[VEC], out[VEC];
+    load_cols<VEC>(p.w, SSM_F32, 0, col, H, vok, wv);
+    if (p.b) load_cols<VEC>(p.b, SSM_F32, 0, col, H, vok, bv);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float o = (v[k][i] - mean) * rstd * wv[i];
+      if (p.b) o += bv[i];
+      if (p.res && !p.prenorm) o += r[k][i];
+      out[i] = o;
+    }
+    store_cols<VEC>(p.y, p.x_dtype, base, col, H, vok, out);
+  }
+}
+
+// Any hidden size: three sweeps over the row from memory.
+__global__ __launch_bounds__(LN_THREADS) void norm_fwd_long_kernel(const NormParams p) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row = blockIdx.x * LN_WAVES + wave;
+  if (row >= p.rows) return;
+  const int H = p.hidden;
+  const size_t base = (size_t)row * H;
+  auto val = [&](int c) -> float {
+    float v = load_as_f32(p.x, p.x_dtype, base + c);
+    if (p.res && p.prenorm) v += load_as_f32(p.res, p.res_dtype, base + c);
+    return v;
+  };
+  float sum = 0.0f;
+  for (int c = lane; c < H; c += WAVE) sum += val(c);
+  const float inv_h = 1.0f / (float)H;
+  const float mean = p.is_rms ? 0.0f : wave_sum(sum) * inv_h;
+  float sq = 0.0f;
+  for (int c = lane; c < H; c += WAVE) {
+    const float d = val(c) - mean;
+    sq = __builtin_fmaf(d, d, sq);
+  }
+  const float rstd = 1.0f / sqrtf(wave_sum(sq) * inv_h + p.eps);
+  if (lane == 0) {
+    if (p.mean) p.mean[row] = mean;
+    if (p.rstd) p.rstd[row] = rstd;
+  }
+  for (int c = lane; c < H; c += WAVE) {
+    const float v = val(c);
+    if (p.res_out) store_f32_as(p.res_out, p.res_out_dtype, base + c, v);
+    float o = (v - mean) * rstd * p.w[c];
+    if (p.b) o += p.b[c];
+    if (p.res && !p.prenorm) o += load_as_f32(p.res, p.res_dtype, base + c);
+    store_f32_as(p.y, p.x_dtype, base + c, o);
+  }
+}
+
+// ----------------------------------------------------------------- backward
+
+// Each wave handles rows wave_global, wave_global + nwaves, ...; columns are
+// owned by (lane, trip) exactly as in the forward kernel.
+template <int TRIPS>
+__global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p, int vec_ok) {
+  constexpr int VEC = 4;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int nwaves = gridDim.x * LN_WAVES;
+  const int gw = blockIdx.x * LN_WAVES + wave;
+  const int H = p.hidden;
+  const bool vok = vec_ok != 0;
+  const float inv_h = 1.0f / (float)H;
+  float dw[TRIPS][VEC], db[TRIPS][VEC], wv[TRIPS][VEC];
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int col = (k * WAVE + lane) * VEC;
+    load_cols<VEC>(p.w, SSM_F32, 0, col, H, vok, wv[k]);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) dw[k][i] = db[k][i] = 0.0f;
+  }
+  for (int row = gw; row < p.rows; row += nwaves) {
+    const size_t base = (size_t)row * H;
+    const float mean = p.is_rms ? 0.0f : p.mean[row];
+    const float rstd = p.rstd[row];
+    float xh[TRIPS][VEC], g[TRIPS][VEC], dyv[TRIPS][VEC];
+    float s1 = 0.0f, s2 = 0.0f;     // sum g*xhat, sum g
+#pragma unroll
+    for (int k = 0; k < TRIPS; ++k) {
+      const int col = (k * WAVE + lane) * VEC;
+      float v[VEC];
+      load_cols<VEC>(p.x, p.x_dtype, base, col, H, vok, v);
+      if (p.res && p.prenorm) {
+        float r[VEC];
+        load_cols<VEC>(p.res, p.res_dtype, base, col, H, vok, r);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] += r[i];
+      }
+      load_cols<VEC>(p.dy, p.x_dtype, base, col, H, vok, dyv[k]);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const bool in = col + i < H;
+        xh[k][i] = in ? (v[i] - mean) * rstd : 0.0f;
+        g[k][i] = in ? dyv[k][i] * wv[k][i] : 0.0f;
+        s1 = __builtin_fmaf(g[k][i], xh[k][i], s1);
+        s2 += g[k][i];
+        dw[k][i] = __builtin_fmaf(dyv[k][i], xh[k][i], dw[k][i]);
+        db[k][i] += dyv[k][i];
+      }
+    }
+    const float c1 = wave_sum(s1) * inv_h;
+    const float c2 = p.is_rms ? 0.0f : wave_sum(s2) * inv_h;
+#pragma unroll
+    for (int k = 0; k < TRIPS; ++k) {
+      const int col = (k * WAVE + lane) * VEC;
+      if (col >= H) continue;
+      float dxv[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) dxv[i] = (g[k][i] - c2 - xh[k][i] * c1) * rstd;
+      store_cols<VEC>(p.dx, p.x_dtype, base, col, H, vok, dxv);
+      if (p.dres) store_cols<VEC>(p.dres, p.res_dtype, base, col, H, vok, p.prenorm ? dxv : dyv[k]);
+    }
+  }
+  float *pw = p.partial + (size_t)gw * 2 * H;
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int col = (k * WAVE + lane) * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+      if (col + i < H) {
+        pw[col + i] = dw[k][i];
+        pw[H + col + i] = db[k][i];
+      }
+  }
+}
+
+__global__ __launch_bounds__(LN_THREADS) void norm_bwd_long_kernel(const NormParams p) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int nwaves = gridDim.x * LN_WAVES;
+  const int gw = blockIdx.x * LN_WAVES + wave;
+  const int H = p.hidden;
+  const float inv_h = 1.0f / (float)H;
+  float *pw = p.partial + (size_t)gw * 2 * H;
+  for (int c = lane; c < 2 * H; c += WAVE) pw[c] = 0.0f;
+  for (int row = gw; row < p.rows; row += nwaves) {
+    const size_t base = (size_t)row * H;
+    const float mean = p.is_rms ? 0.0f : p.mean[row];
+    const float rstd = p.rstd[row];
+    auto xhat = [&](int c) -> float {
+      float v = load_as_f32(p.x, p.x_dtype, base + c);
+      if (p.res && p.prenorm) v += load_as_f32(p.res, p.res_dtype, base + c);
+      return (v - mean) * rstd;
+    };
+    float s1 = 0.0f, s2 = 0.0f;
+    for (int c = lane; c < H; c += WAVE) {
+      const float dy = load_as_f32(p.dy, p.x_dtype, base + c);
+      const float gg = dy * p.w[c];
+      const float xh = xhat(c);
+      s1 = __builtin_fmaf(gg, xh, s1);
+      s2 += gg;
+      pw[c] = __builtin_fmaf(dy, xh, pw[c]);
+      pw[H + c] += dy;
+    }
+    const float c1 = wave_sum(s1) * inv_h;
+    const float c2 = p.is_rms ? 0.0f : wave_sum(s2) * inv_h;
+    for (int c = lane; c < H; c += WAVE) {
+      const float dy = load_as_f32(p.dy, p.x_dtype, base + c);
+      const float dxv = (dy * p.w[c] - c2 - xhat(c) * c1) * rstd;
+      store_f32_as(p.dx, p.x_dtype, base + c, dxv);
+      if (p.dres) store_f32_as(p.dres, p.res_dtype, base + c, p.prenorm ? dxv : dy);
+    }
+  }
+}
+
+// dw[c] = sum_w partial[w][0][c], db[c] = sum_w partial[w][1][c]
+__global__ __launch_bounds__(LN_THREADS) void norm_bwd_fold_kernel(const float *partial, float *dw, float *db,
+                                                                    int nwaves, int hidden) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= hidden) return;
+  float sw = 0.0f, sb = 0.0f;
+  for (int w = 0; w < nwaves; ++w) {
+    sw += partial[(size_t)w * 2 * hidden + c];
+    sb += partial[(size_t)w * 2 * hidden + hidden + c];
+  }
+  dw[c] = sw;
+  if (db) db[c] = sb;
+}
+
+static int norm_bwd_grid(int rows) {
+  // persistent: at most 4 workgroups per CU on a 256-CU part, never more waves than rows
+  const int want = (rows + LN_WAVES - 1) / LN_WAVES;
+  return want < 1024 ? (want < 1 ? 1 : want) : 1024;
+}
+
+static int norm_check(const char *who, const void *x, const float *w, const void *y, int rows, int hidden,
+                      int x_dtype, const void *res, int res_dtype) {
+  SSM_REQUIRE(x && w && y, SSM_ERR_NULL_POINTER, "%s: x, weight and output are required", who);
+  SSM_REQUIRE(rows > 0 && hidden > 0, SSM_ERR_BAD_SHAPE, "%s: rows=%d hidden=%d must be positive", who, rows, hidden);
+  SSM_REQUIRE(valid_dtype(x_dtype) && (!res || valid_dtype(res_dtype)), SSM_ERR_BAD_DTYPE,
+              "%s: x_dtype=%d residual_dtype=%d", who, x_dtype, res_dtype);
+  SSM_REQUIRE((size_t)rows * hidden < ((size_t)1 << 40), SSM_ERR_TOO_LARGE, "%s: tensor too large", who);
+  return SSM_OK;
+}
+
+}  // namespace ssm
+
+extern "C" int ssm_norm_fwd(const ssm_norm_fwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_norm_fwd: args is NULL");
+  int rc = norm_check("ssm_norm_fwd", a->x, a->weight, a->y, a->rows, a->hidden, a->x_dtype, a->residual,
+                      a->residual_dtype);
+  if (rc != SSM_OK) return rc;
+  if (a->residual_out)
+    SSM_REQUIRE(valid_dtype(a->residual_out_dtype), SSM_ERR_BAD_DTYPE, "ssm_norm_fwd: residual_out_dtype=%d",
+                a->residual_out_dtype);
+  NormParams p{};
+  p.x = a->x; p.res = a->residual; p.w = a->weight; p.b = a->bias; p.y = a->y; p.res_out = a->residual_out;
+  p.mean = a->mean; p.rstd = a->rstd;
+  p.rows = a->rows; p.hidden = a->hidden;
+  p.x_dtype = a->x_dtype; p.res_dtype = a->residual_dtype; p.res_out_dtype = a->residual_out_dtype;
+  p.is_rms = a->is_rms ? 1 : 0; p.prenorm = a->prenorm ? 1 : 0; p.eps = a->eps;
+  const int vec_ok = a->hidden % 4 == 0 && aligned_to(a->x, 16) && aligned_to(a->y, 16) &&
+                     aligned_to(a->weight, 16) && (!a->bias || aligned_to(a->bias, 16)) &&
+                     (!a->residual || aligned_to(a->residual, 16)) &&
+                     (!a->residual_out || aligned_to(a->residual_out, 16));
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  const unsigned grid = (unsigned)((a->rows + LN_WAVES - 1) / LN_WAVES);
+  const int per_lane = (a->hidden + WAVE - 1) / WAVE;
+  if (per_lane <= 4) hipLaunchKernelGGL(norm_fwd_kernel<1>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 8) hipLaunchKernelGGL(norm_fwd_kernel<2>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 12) hipLaunchKernelGGL(norm_fwd_kernel<3>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 16) hipLaunchKernelGGL(norm_fwd_kernel<4>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 32) hipLaunchKernelGGL(norm_fwd_kernel<8>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else hipLaunchKernelGGL(norm_fwd_long_kernel, dim3(grid), dim3(LN_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_norm_fwd");
+  return SSM_OK;
+}
+
+extern "C" size_t ssm_norm_bwd_workspace_bytes(int rows, int hidden) {
+  if (rows <= 0 || hidden <= 0) return 0;
+  return (size_t)ssm::norm_bwd_grid(rows) * ssm::LN_WAVES * 2 * (size_t)hidden * sizeof(float);
+}
+
+extern "C" int ssm_norm_bwd(const ssm_norm_bwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_norm_bwd: args is NULL");
+  int rc = norm_check("ssm_norm_bwd", a->x, a->weight, a->dx, a->rows, a->hidden, a->x_dtype, a->residual,
+                      a->residual_dtype);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(a->dy && a->rstd && a->dweight && (a->is_rms || a->mean), SSM_ERR_NULL_POINTER,
+              "ssm_norm_bwd: dy, rstd, dweight (and mean for LayerNorm) are required");
+  SSM_REQUIRE(!a->dresidual || a->residual, SSM_ERR_NULL_POINTER, "ssm_norm_bwd: dresidual needs residual");
+  SSM_REQUIRE(a->workspace && a->workspace_bytes >= ssm_norm_bwd_workspace_bytes(a->rows, a->hidden),
+              SSM_ERR_WORKSPACE, "ssm_norm_bwd: workspace of %zu bytes required",
+              ssm_norm_bwd_workspace_bytes(a->rows, a->hidden));
+  NormParams p{};
+  p.x = a->x; p.res = a->residual; p.dy = a->dy; p.w = a->weight; p.dx = a->dx; p.dres = a->dresidual;
+  p.mean = const_cast<float *>(a->mean); p.rstd = const_cast<float *>(a->rstd);
+  p.partial = reinterpret_cast<float *>(a->workspace);
+  p.rows = a->rows; p.hidden = a->hidden;
+  p.x_dtype = a->x_dtype; p.res_dtype = a->residual_dtype;
+  p.is_rms = a->is_rms ? 1 : 0; p.prenorm = a->prenorm ? 1 : 0;
+  const int vec_ok = a->hidden % 4 == 0 && aligned_to(a->x, 16) && aligned_to(a->dy, 16) && aligned_to(a->dx, 16) &&
+                     aligned_to(a->weight, 16) && (!a->residual || aligned_to(a->residual, 16)) &&
+                     (!a->dresidual || aligned_to(a->dresidual, 16));
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  const int grid = norm_bwd_grid(a->rows);
+  const int per_lane = (a->hidden + WAVE - 1) / WAVE;
+  if (per_lane <= 4) hipLaunchKernelGGL(norm_bwd_kernel<1>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 8) hipLaunchKernelGGL(norm_bwd_kernel<2>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 12) hipLaunchKernelGGL(norm_bwd_kernel<3>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 16) hipLaunchKernelGGL(norm_bwd_kernel<4>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else hipLaunchKernelGGL(norm_bwd_long_kernel, dim3(grid), dim3(LN_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_norm_bwd");
+  const int nwaves = grid * LN_WAVES;
+  hipLaunchKernelGGL(norm_bwd_fold_kernel, dim3((a->hidden + LN_THREADS - 1) / LN_THREADS), dim3(LN_THREADS), 0, s,
+                     p.partial, a->dweight, a->dbias, nwaves, a->hidden);
+  SSM_CHECK_LAUNCH("ssm_norm_bwd(fold)");
+  return SSM_OK;
+}

@@ -1,0 +1,611 @@
+// Selective scan, backward, for gfx950.
+//
+// Per (batch, channel) row, with a_t = exp(delta_t A), b_t = delta_t u_t B_t:
+//   forward    h_t  = a_t h_{t-1} + b_t ,   pre_t = <h_t, C_t> + D u_t ,  y_t = pre_t silu(z_t)
+//   adjoint    gh_t = g_t C_t + q_{t+1} ,   q_t = a_t gh_t                (g_t = dout_t silu(z_t))
+//   dC_t += g_t h_t             dB_t += gh_t delta_t u_t      du_t = delta_t <gh_t, B_t> + g_t D
+//   ddelta_t = u_t <gh_t, B_t> + sum_n q_t h_{t-1} A_n        dA_n += q_t h_{t-1} delta_t
+// Nothing but the inputs and the state entering each 512-step chunk (written by
+// the forward kernel) is saved: h is recomputed chunk by chunk, chunks being
+// visited last to first so that q can be carried backwards.
+//
+// Work split.  A workgroup of 8 wavefronts walks a block of channels that share
+// one B/C group.  For one (row, chunk) the 8 wavefronts split the STATE axis
+// (wave w owns states 2w and 2w+1), lanes split time (8 consecutive steps per
+// lane) and both directions are DPP scans (the reverse one on lane-reversed
+// operands).  That way dB/dC - which sum over all channels of a group - simply
+// accumulate in registers while the workgroup moves from channel to channel,
+// and are written once per chunk as one partial per workgroup; a fold kernel
+// adds the partials in a fixed order.  Quantities that sum over states (pre,
+// <gh,B>, the A-term of ddelta) are exchanged through LDS once per row.
+// There are no atomics: results are bit-reproducible.
+#include "common.hpp"
+
+namespace ssm {
+
+constexpr int BW_K = 8;                  // steps per lane
+constexpr int BW_T = WAVE * BW_K;        // 512 steps per chunk
+constexpr int BW_WAVES = 8;
+constexpr int BW_THREADS = WAVE * BW_WAVES;
+constexpr int BW_MAX_N = 2 * BW_WAVES;   // 16 states per pass
+
+struct ScanBwdParams {
+  const void *u, *delta, *z, *dout, *Bp, *Cp;
+  const float *A, *Dk, *bias, *dlast, *chunk_states;
+  void *du, *ddelta, *dz;
+  float *dA_rows;        // (B, D, N)  per-row sums, folded over batch afterwards
+  float *dD_rows;        // (B, D)
+  float *dbias_rows;     // (B, D)
+  float *dB_part;        // BVARY: (B, nblk, N, L) partials ; else (B, D, N) per-row sums
+  float *dC_part;
+  int batch, dim, len, nstate;
+  int bc_dtype;
+  int b_kind, c_kind, b_groups, c_groups;
+  int softplus;
+  int rows_per_wg;       // channels walked by one workgroup (all in one B group and one C group)
+  int nblk;              // workgroups per batch row = dim / rows_per_wg
+  int bc_vec_ok;
+};
+
+// Stage one [BW_MAX_N][BW_T] slab of a time-varying projection (fp32, transposed
+// so that lane l finds steps 8l..8l+7 of state n at n*T + {l*4, 256 + l*4}).
+__device__ __forceinline__ void bw_stage_tile(float *dst, const void *src, int dtype, size_t src_off, int len,
+                                              int t0, int nn, bool vec_ok) {
+  constexpr int QT = BW_T / 4;
+  for (int e = threadIdx.x; e < BW_MAX_N * QT; e += BW_THREADS) {
+    const int nl = e / QT;
+    const int tl = (e % QT) * 4;
+    const int t = t0 + tl;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (nl < nn) {
+      const size_t off = src_off + (size_t)nl * len + t;
+      if (vec_ok && t + 4 <= len) {
+        if (dtype == SSM_F32) {
+          v = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(src) + off);
+        } else {
+          const uint2 raw = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(src) + off);
+          if (dtype == SSM_BF16) {
+            v.x = __uint_as_float(raw.x << 16);
+            v.y = __uint_as_float(raw.x & 0xffff0000u);
+            v.z = __uint_as_float(raw.y << 16);
+            v.w = __uint_as_float(raw.y & 0xffff0000u);
+          } else {
+            union { uint32_t u; _Float16 h[2]; } a, b;
+            a.u = raw.x;
+            b.u = raw.y;
+            v.x = (float)a.h[0];
+            v.y = (float)a.h[1];
+            v.z = (float)b.h[0];
+            v.w = (float)b.h[1];
+          }
+        }
+      } else {
+        v.x = (t + 0 < len) ? load_as_f32(src, dtype, off + 0) : 0.0f;
+        v.y = (t + 1 < len) ? load_as_f32(src, dtype, off + 1) : 0.0f;
+        v.z = (t + 2 < len) ? load_as_f32(src, dtype, off + 2) : 0.0f;
+        v.w = (t + 3 < len) ? load_as_f32(src, dtype, off + 3) : 0.0f;
+      }
+    }
+    const int owner = tl / BW_K, item = tl % BW_K;
+    *reinterpret_cast<float4 *>(dst + nl * BW_T + (item >> 2) * (WAVE * 4) + owner * 4) = v;
+  }
+}
+
+#define SSM_BW_STEP2(CTRL)                                \
+  "v_fmac_f32_dpp %1, %1, %0 " CTRL "\n\t"                \
+  "v_fmac_f32_dpp %3, %3, %2 " CTRL "\n\t"                \
+  "v_mul_f32_dpp %0, %0, %0 " CTRL "\n\t"                 \
+  "v_mul_f32_dpp %2, %2, %2 " CTRL "\n\t"
+
+// Two independent inclusive scans of affine maps (see wave_scan_affine); only the
+// offsets b0/b1 are complete in every lane afterwards.
+__device__ __forceinline__ void bw_scan_x2(float &a0, float &b0, float &a1, float &b1) {
+  asm volatile(
+      "s_nop 4\n\t"
+      SSM_BW_STEP2("row_shr:1 row_mask:0xf bank_mask:0xf")
+      SSM_BW_STEP2("row_shr:2 row_mask:0xf bank_mask:0xf")
+      SSM_BW_STEP2("row_shr:4 row_mask:0xf bank_mask:0xf")
+      SSM_BW_STEP2("row_shr:8 row_mask:0xf bank_mask:0xf")
+      SSM_BW_STEP2("row_bcast:15 row_mask:0xa bank_mask:0xf")
+      "v_fmac_f32_dpp %1, %1, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %3, %3, %2 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1\n\t"
+      : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
+}
+
+__device__ __forceinline__ float lane_gather(float v, int src_lane) {
+  return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
+}
+
+template <typename io_t, bool BVARY, bool CVARY>
+__global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParams p) {
+  constexpr int K = BW_K, T = BW_T;
+  extern __shared__ __align__(16) float lds[];
+  // layout: [B tile][C tile][elem: delta,u,g][partials: 8 x 3 x T][qcarry rows x 16][red 2 x 8 x 2]
+  float *Bs = lds;
+  float *Cs = Bs + (BVARY ? BW_MAX_N * T : 0);
+  float *e_dl = Cs + (CVARY ? BW_MAX_N * T : 0);
+  float *e_u = e_dl + T;
+  float *e_g = e_u + T;
+  float *part = e_g + T;                          // [wave][3][T]
+  float *qcarry = part + BW_WAVES * 3 * T;        // [rows_per_wg][16]
+  float *red = qcarry + p.rows_per_wg * BW_MAX_N; // [2][BW_WAVES][2]
+
+  const int wave = wave_id_uniform();
+  const int lane = lane_id();
+  const int tid = threadIdx.x;
+  const int b = (int)blockIdx.x / p.nblk;
+  const int blk = (int)blockIdx.x % p.nblk;
+  const int d_first = blk * p.rows_per_wg;
+  const int L = p.len, N = p.nstate;
+  const int nchunks = (L + T - 1) / T;
+  const int n0 = 2 * wave, n1 = 2 * wave + 1;
+  const bool v0 = n0 < N, v1 = n1 < N;
+
+  size_t b_tile_off = 0, c_tile_off = 0;
+  if (BVARY) b_tile_off = ((size_t)b * p.b_groups + d_first / (p.dim / p.b_groups)) * (size_t)N * L;
+  if (CVARY) c_tile_off = ((size_t)b * p.c_groups + d_first / (p.dim / p.c_groups)) * (size_t)N * L;
+
+  // adjoint entering from beyond the end of the sequence
+  for (int e = tid; e < p.rows_per_wg * BW_MAX_N; e += BW_THREADS) {
+    const int r = e / BW_MAX_N, n = e % BW_MAX_N;
+    const size_t row = (size_t)b * p.dim + d_first + r;
+    qcarry[e] = (p.dlast && n < N) ? p.dlast[row * N + n] : 0.0f;
+  }
+
+  const int rev_lane = WAVE - 1 - lane;
+
+  for (int c = nchunks - 1; c >= 0; --c) {
+    const int t0 = c * T;
+    __syncthreads();     // tiles and qcarry free / visible
+    if (BVARY) bw_stage_tile(Bs, p.Bp, p.bc_dtype, b_tile_off, L, t0, N, p.bc_vec_ok != 0);
+    if (CVARY) bw_stage_tile(Cs, p.Cp, p.bc_dtype, c_tile_off, L, t0, N, p.bc_vec_ok != 0);
+
+    float accB[2][K], accC[2][K];
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int i = 0; i < K; ++i) accB[w][i] = accC[w][i] = 0.0f;
+
+    for (int r = 0; r < p.rows_per_wg; ++r) {
+      const int d = d_first + r;
+      const size_t row = (size_t)b * p.dim + d;
+      const float Dk = p.Dk ? p.Dk[d] : 0.0f;
+
+      // ---- element-wise stage: thread tid owns step t0 + tid of this row
+      const int te = t0 + tid;
+      float el_u = 0.0f, el_dl = 0.0f, el_g = 0.0f, el_sig = 1.0f, el_dz = 0.0f;
+      if (te < L) {
+        const size_t idx = row * L + te;
+        el_u = to_f32(reinterpret_cast<const io_t *>(p.u)[idx]);
+        float draw = to_f32(reinterpret_cast<const io_t *>(p.delta)[idx]);
+        if (p.bias) draw += p.bias[d];
+        if (p.softplus) {
+          el_dl = softplus_f32(draw);
+          el_sig = draw > 20.0f ? 1.0f : sigmoid_f32(draw);
+        } else {
+          el_dl = draw;
+        }
+        const float go = to_f32(reinterpret_cast<const io_t *>(p.dout)[idx]);
+        if (p.z) {
+          const float zv = to_f32(reinterpret_cast<const io_t *>(p.z)[idx]);
+          const float sg = sigmoid_f32(zv);
+          el_g = go * zv * sg;
+          el_dz = go * sg * __builtin_fmaf(zv, 1.0f - sg, 1.0f);      // dout * silu'(z)
+        } else {
+          el_g = go;
+        }
+      }
+      e_dl[tid] = el_dl;
+      e_u[tid] = el_u;
+      e_g[tid] = el_g;
+      __syncthreads();                                                  // (1) staged row visible
+
+      // ---- per-state work: this wave owns states n0, n1
+      float dl[K], uu[K], g[K];
+      {
+        const float4 a0 = *reinterpret_cast<const float4 *>(e_dl + lane * K);
+        const float4 a1 = *reinterpret_cast<const float4 *>(e_dl + lane * K + 4);
+        const float4 b0 = *reinterpret_cast<const float4 *>(e_u + lane * K);
+        const float4 b1 = *reinterpret_cast<const float4 *>(e_u + lane * K + 4);
+        const float4 c0 = *reinterpret_cast<const float4 *>(e_g + lane * K);
+        const float4 c1 = *reinterpret_cast<const float4 *>(e_g + lane * K + 4);
+        dl[0] = a0.x; dl[1] = a0.y; dl[2] = a0.z; dl[3] = a0.w; dl[4] = a1.x; dl[5] = a1.y; dl[6] = a1.z; dl[7] = a1.w;
+        uu[0] = b0.x; uu[1] = b0.y; uu[2] = b0.z; uu[3] = b0.w; uu[4] = b1.x; uu[5] = b1.y; uu[6] = b1.z; uu[7] = b1.w;
+        g[0] = c0.x; g[1] = c0.y; g[2] = c0.z; g[3] = c0.w; g[4] = c1.x; g[5] = c1.y; g[6] = c1.z; g[7] = c1.w;
+      }
+      float dsum = 0.0f;
+#pragma unroll
+      for (int i = 0; i < K; ++i) dsum += dl[i];
+
+      float a[2][K], hp[2][K], cc[2][K], bq[2][K];   // decay, state before step, g*C, B values
+      float P[2], h[2], Hin[2], A2[2], Qa[2], Pr[2], qin_carry[2];
+      float pre[K], sgb[K], dda[K];                   // partial sums over this wave's states
+#pragma unroll
+      for (int i = 0; i < K; ++i) pre[i] = sgb[i] = dda[i] = 0.0f;
+
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const int n = w == 0 ? n0 : n1;
+        const bool valid = w == 0 ? v0 : v1;
+        A2[w] = valid ? p.A[(size_t)d * N + n] * LOG2E : 0.0f;
+        Hin[w] = valid ? p.chunk_states[(row * nchunks + c) * (size_t)N + n] : 0.0f;
+        qin_carry[w] = qcarry[r * BW_MAX_N + (valid ? n : 0)];
+        if (!valid) qin_carry[w] = 0.0f;
+        float bconst = 0.0f, cconst = 0.0f;
+        if (!BVARY && valid) {
+          const size_t off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N + n;
+          bconst = load_as_f32(p.Bp, p.bc_dtype, off);
+        }
+        if (!CVARY && valid) {
+          const size_t off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N + n;
+          cconst = load_as_f32(p.Cp, p.bc_dtype, off);
+        }
+        const int nrow = valid ? n : 0;
+#pragma unroll
+        for (int q4 = 0; q4 < K / 4; ++q4) {
+          float4 bv, cv;
+          if (BVARY) bv = *reinterpret_cast<const float4 *>(Bs + nrow * T + q4 * (WAVE * 4) + lane * 4);
+          else bv = make_float4(bconst, bconst, bconst, bconst);
+          if (CVARY) cv = *reinterpret_cast<const float4 *>(Cs + nrow * T + q4 * (WAVE * 4) + lane * 4);
+          else cv = make_float4(cconst, cconst, cconst, cconst);
+          if (!valid) { bv = make_float4(0.f, 0.f, 0.f, 0.f); cv = bv; }
+          bq[w][q4 * 4 + 0] = bv.x; bq[w][q4 * 4 + 1] = bv.y; bq[w][q4 * 4 + 2] = bv.z; bq[w][q4 * 4 + 3] = bv.w;
+          cc[w][q4 * 4 + 0] = cv.x; cc[w][q4 * 4 + 1] = cv.y; cc[w][q4 * 4 + 2] = cv.z; cc[w][q4 * 4 + 3] = cv.w;
+        }
+        // forward fold of the lane's 8 steps
+        float hh = 0.0f;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+          a[w][i] = exp2_hw(dl[i] * A2[w]);
+          hh = __builtin_fmaf(a[w][i], hh, dl[i] * uu[i] * bq[w][i]);
+        }
+        P[w] = exp2_hw(dsum * A2[w]);
+        Pr[w] = P[w];
+        h[w] = __builtin_fmaf(P[w], lane == 0 ? Hin[w] : 0.0f, hh);
+      }
+      bw_scan_x2(P[0], h[0], P[1], h[1]);
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        // replay forward: hp[i] = state before step i, hcur = state after it
+        float hcur = wave_prev(h[w], Hin[w]);
+        float Q = 0.0f;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+          hp[w][i] = hcur;
+          hcur = __builtin_fmaf(a[w][i], hcur, dl[i] * uu[i] * bq[w][i]);
+          pre[i] = __builtin_fmaf(hcur, cc[w][i], pre[i]);
+          const float gc = g[i] * cc[w][i];
+          accC[w][i] = __builtin_fmaf(g[i], hcur, accC[w][i]);
+          cc[w][i] = gc;                        // from here on cc holds g_t * C_t
+        }
+        // reverse fold: q_first = Pr * q_in + Qa
+#pragma unroll
+        for (int i = K - 1; i >= 0; --i) Q = a[w][i] * (cc[w][i] + Q);
+        Qa[w] = Q;
+      }
+      // reverse scan: run the forward scan on lane-reversed operands
+      float rP0 = lane_gather(Pr[0], rev_lane), rQ0 = lane_gather(Qa[0], rev_lane);
+      float rP1 = lane_gather(Pr[1], rev_lane), rQ1 = lane_gather(Qa[1], rev_lane);
+      rQ0 = __builtin_fmaf(rP0, lane == 0 ? qin_carry[0] : 0.0f, rQ0);
+      rQ1 = __builtin_fmaf(rP1, lane == 0 ? qin_carry[1] : 0.0f, rQ1);
+      bw_scan_x2(rP0, rQ0, rP1, rQ1);
+      // reversed lane j now holds q at the first step of original lane 63-j
+      const float qn0 = wave_read_lane(rQ0, WAVE - 1), qn1 = wave_read_lane(rQ1, WAVE - 1);
+      float qin[2];
+      {
+        const int src = (WAVE - 2 - lane) & (WAVE - 1);        // original lane + 1, in the reversed domain
+        const float t0v = lane_gather(rQ0, src), t1v = lane_gather(rQ1, src);
+        qin[0] = lane == WAVE - 1 ? qin_carry[0] : t0v;
+        qin[1] = lane == WAVE - 1 ? qin_carry[1] : t1v;
+      }
+      float dA_acc[2] = {0.0f, 0.0f}, dBc_acc[2] = {0.0f, 0.0f};
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        float q = qin[w];
+#pragma unroll
+        for (int i = K - 1; i >= 0; --i) {
+          const float gh = cc[w][i] + q;
+          const float du_i = dl[i] * uu[i];
+          if (BVARY) accB[w][i] = __builtin_fmaf(gh, du_i, accB[w][i]);
+          else dBc_acc[w] = __builtin_fmaf(gh, du_i, dBc_acc[w]);
+          sgb[i] = __builtin_fmaf(gh, bq[w][i], sgb[i]);
+          q = a[w][i] * gh;
+          const float wv = q * hp[w][i];
+          dda[i] = __builtin_fmaf(wv, A2[w], dda[i]);
+          dA_acc[w] = __builtin_fmaf(wv, dl[i], dA_acc[w]);
+        }
+      }
+      // partial sums over this wave's two states -> LDS
+      {
+        float *pw = part + (size_t)wave * 3 * T + lane * K;
+        *reinterpret_cast<float4 *>(pw) = make_float4(pre[0], pre[1], pre[2], pre[3]);
+        *reinterpret_cast<float4 *>(pw + 4) = make_float4(pre[4], pre[5], pre[6], pre[7]);
+        *reinterpret_cast<float4 *>(pw + T) = make_float4(sgb[0], sgb[1], sgb[2], sgb[3]);
+        *reinterpret_cast<float4 *>(pw + T + 4) = make_float4(sgb[4], sgb[5], sgb[6], sgb[7]);
+        *reinterpret_cast<float4 *>(pw + 2 * T) = make_float4(dda[0], dda[1], dda[2], dda[3]);
+        *reinterpret_cast<float4 *>(pw + 2 * T + 4) = make_float4(dda[4], dda[5], dda[6], dda[7]);
+      }
+      // per-row, per-state sums (this wave is the only writer of these addresses)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const int n = w == 0 ? n0 : n1;
+        const bool valid = w == 0 ? v0 : v1;
+        const float sA = wave_sum(dA_acc[w]);
+        float sB = 0.0f, sC = 0.0f;
+        if (!BVARY) sB = wave_sum(dBc_acc[w]);
+        if (!CVARY) {
+          float t = 0.0f;
+#pragma unroll
+          for (int i = 0; i < K; ++i) t += accC[w][i];
+          sC = wave_sum(t);
+#pragma unroll
+          for (int i = 0; i < K; ++i) accC[w][i] = 0.0f;
+        }
+        if (valid && lane == 0) {
+          const size_t o = row * N + n;
+          const bool first = c == nchunks - 1;
+          p.dA_rows[o] = (first ? 0.0f : p.dA_rows[o]) + sA;
+          if (!BVARY) p.dB_part[o] = (first ? 0.0f : p.dB_part[o]) + sB;
+          if (!CVARY) p.dC_part[o] = (first ? 0.0f : p.dC_part[o]) + sC;
+          qcarry[r * BW_MAX_N + n] = w == 0 ? qn0 : qn1;
+        }
+      }
+      __syncthreads();                                                  // (2) partials visible
+
+      // ---- finish element tid of this row
+      float s_pre = 0.0f, s_gb = 0.0f, s_da = 0.0f;
+#pragma unroll
+      for (int wv = 0; wv < BW_WAVES; ++wv) {
+        s_pre += part[(size_t)wv * 3 * T + tid];
+        s_gb += part[(size_t)wv * 3 * T + T + tid];
+        s_da += part[(size_t)wv * 3 * T + 2 * T + tid];
+      }
+      float dD_c = 0.0f, dbias_c = 0.0f;
+      if (te < L) {
+        const size_t idx = row * L + te;
+        const float du = __builtin_fmaf(s_gb, el_dl, el_g * Dk);
+        const float ddl = __builtin_fmaf(s_gb, el_u, s_da * LN2) * el_sig;
+        reinterpret_cast<io_t *>(p.du)[idx] = from_f32<io_t>(du);
+        reinterpret_cast<io_t *>(p.ddelta)[idx] = from_f32<io_t>(ddl);
+        if (p.z) reinterpret_cast<io_t *>(p.dz)[idx] = from_f32<io_t>(el_dz * __builtin_fmaf(Dk, el_u, s_pre));
+        dD_c = el_g * el_u;
+        dbias_c = ddl;
+      }
+      {
+        const float sD = wave_sum(dD_c), sb = wave_sum(dbias_c);
+        float *rr = red + (size_t)(r & 1) * BW_WAVES * 2;
+        if (lane == 0) {
+          rr[wave * 2] = sD;
+          rr[wave * 2 + 1] = sb;
+        }
+      }
+      __syncthreads();                                                  // (3) e_*, part reusable; red visible
+      if (tid == 0) {
+        const float *rr = red + (size_t)(r & 1) * BW_WAVES * 2;
+        float sD = 0.0f, sb = 0.0f;
+        for (int wv = 0; wv < BW_WAVES; ++wv) {
+          sD += rr[wv * 2];
+          sb += rr[wv * 2 + 1];
+        }
+        const bool first = c == nchunks - 1;
+        p.dD_rows[row] = (first ? 0.0f : p.dD_rows[row]) + sD;
+        p.dbias_rows[row] = (first ? 0.0f : p.dbias_rows[row]) + sb;
+      }
+    }
+
+    // ---- flush this chunk's dB / dC partials (sum over the workgroup's channels)
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const int n = w == 0 ? n0 : n1;
+      const bool valid = w == 0 ? v0 : v1;
+      if (!valid) continue;
+      const size_t base = (((size_t)b * p.nblk + blk) * N + n) * (size_t)L + t0 + lane * K;
+      const bool full = t0 + lane * K + K <= L && L % 4 == 0;
+      if (BVARY) {
+        if (full) {
+          *reinterpret_cast<float4 *>(p.dB_part + base) = make_float4(accB[w][0], accB[w][1], accB[w][2], accB[w][3]);
+          *reinterpret_cast<float4 *>(p.dB_part + base + 4) = make_float4(accB[w][4], accB[w][5], accB[w][6], accB[w][7]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < K; ++i)
+            if (t0 + lane * K + i < L) p.dB_part[base + i] = accB[w][i];
+        }
+      }
+      if (CVARY) {
+        if (full) {
+          *reinterpret_cast<float4 *>(p.dC_part + base) = make_float4(accC[w][0], accC[w][1], accC[w][2], accC[w][3]);
+          *reinterpret_cast<float4 *>(p.dC_part + base + 4) = make_float4(accC[w][4], accC[w][5], accC[w][6], accC[w][7]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < K; ++i)
+            if (t0 + lane * K + i < L) p.dC_part[base + i] = accC[w][i];
+        }
+      }
+    }
+  }
+}
+
+// out[o][i] = sum_{j < count} in[(o * count + j) * inner + i], fixed order.
+__global__ __launch_bounds__(256) void fold_sum_kernel(const float *in, float *out, size_t outer, int count,
+                                                       size_t inner) {
+  const size_t total = outer * inner;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t o = e / inner, i = e % inner;
+    float s = 0.0f;
+    for (int j = 0; j < count; ++j) s += in[(o * count + j) * inner + i];
+    out[e] = s;
+  }
+}
+
+// out[i] = sum_{j < count} in[j * inner + i]
+__global__ __launch_bounds__(256) void fold_rows_kernel(const float *in, float *out, int count, size_t inner) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < inner; i += (size_t)gridDim.x * blockDim.x) {
+    float s = 0.0f;
+    for (int j = 0; j < count; ++j) s += in[(size_t)j * inner + i];
+    out[i] = s;
+  }
+}
+
+static unsigned fold_grid(size_t n) {
+  const size_t g = (n + 255) / 256;
+  return (unsigned)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
+}
+
+struct BwdPlan {
+  int rows_per_wg, nblk;
+  size_t off_dA, off_dD, off_dbias, off_dB, off_dC, total;   // byte offsets into the workspace
+};
+
+static BwdPlan plan_bwd(int batch, int dim, int len, int nstate, int b_kind, int c_kind, int b_groups,
+                        int c_groups) {
+  const bool bv = b_kind == SSM_PROJ_BGNL, cv = c_kind == SSM_PROJ_BGNL;
+  const int per_b = bv ? dim / b_groups : dim, per_c = cv ? dim / c_groups : dim;
+  // Block of channels (<= 32) that stays inside one B group and one C group; among
+  // the divisors >= 8 prefer one whose grid is a whole number of 256-CU rounds.
+  int rows = 1;
+  for (int r = 32; r >= 1; --r)
+    if (per_b % r == 0 && per_c % r == 0) { rows = r; break; }
+  for (int r = 32; r >= 8; --r)
+    if (per_b % r == 0 && per_c % r == 0 && ((size_t)batch * (dim / r)) % 256 == 0) { rows = r; break; }
+  BwdPlan pl;
+  pl.rows_per_wg = rows;
+  pl.nblk = dim / rows;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) / 256 * 256; return o; };
+  pl.off_dA = take((size_t)batch * dim * nstate * 4);
+  pl.off_dD = take((size_t)batch * dim * 4);
+  pl.off_dbias = take((size_t)batch * dim * 4);
+  pl.off_dB = take(bv ? (size_t)batch * pl.nblk * nstate * len * 4 : (size_t)batch * dim * nstate * 4);
+  pl.off_dC = take(cv ? (size_t)batch * pl.nblk * nstate * len * 4 : (size_t)batch * dim * nstate * 4);
+  pl.total = off;
+  return pl;
+}
+
+template <typename io_t>
+static int launch_bwd(const ScanBwdParams &p, hipStream_t s) {
+  const bool bv = p.b_kind == SSM_PROJ_BGNL, cv = p.c_kind == SSM_PROJ_BGNL;
+  const size_t lds = ((size_t)((int)bv + (int)cv) * BW_MAX_N * BW_T + 3 * BW_T + BW_WAVES * 3 * BW_T +
+                      (size_t)p.rows_per_wg * BW_MAX_N + 2 * BW_WAVES * 2) * sizeof(float);
+  const unsigned grid = (unsigned)((size_t)p.batch * p.nblk);
+#define SSM_BW_LAUNCH(BV, CV)                                                              \
+  {                                                                                        \
+    auto kernel = scan_bwd_kernel<io_t, BV, CV>;                                           \
+    if (allow_dynamic_lds(kernel, lds) != hipSuccess) {                                    \
+      (void)hipGetLastError();                                                             \
+      set_error("ssm_scan_bwd: cannot reserve %zu bytes of LDS", lds);                     \
+      return SSM_ERR_LAUNCH;                                                               \
+    }                                                                                      \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(BW_THREADS), lds, s, p);                   \
+  }
+  if (bv && cv) SSM_BW_LAUNCH(true, true)
+  else if (bv) SSM_BW_LAUNCH(true, false)
+  else if (cv) SSM_BW_LAUNCH(false, true)
+  else SSM_BW_LAUNCH(false, false)
+#undef SSM_BW_LAUNCH
+  SSM_CHECK_LAUNCH("ssm_scan_bwd");
+  return SSM_OK;
+}
+
+}  // namespace ssm
+
+extern "C" size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, int nstate, int b_kind, int c_kind,
+                                               int b_groups, int c_groups) {
+  using namespace ssm;
+  if (batch <= 0 || dim <= 0 || seqlen <= 0 || nstate <= 0) return 0;
+  if (b_kind == SSM_PROJ_BGNL && (b_groups <= 0 || dim % b_groups)) return 0;
+  if (c_kind == SSM_PROJ_BGNL && (c_groups <= 0 || dim % c_groups)) return 0;
+  return plan_bwd(batch, dim, seqlen, nstate, b_kind, c_kind, b_groups, c_groups).total;
+}
+
+extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_scan_bwd: args is NULL");
+  SSM_REQUIRE(a->u && a->delta && a->A && a->Bproj && a->Cproj && a->dout && a->chunk_states &&
+                  a->du && a->ddelta && a->dA && a->dB && a->dC,
+              SSM_ERR_NULL_POINTER,
+              "ssm_scan_bwd: u, delta, A, Bproj, Cproj, dout, chunk_states, du, ddelta, dA, dB and dC are required");
+  SSM_REQUIRE(!a->z == !a->dz, SSM_ERR_NULL_POINTER, "ssm_scan_bwd: z and dz must be given together");
+  SSM_REQUIRE(!a->Dskip || a->dD, SSM_ERR_NULL_POINTER, "ssm_scan_bwd: dD is required when Dskip is given");
+  SSM_REQUIRE(a->batch > 0 && a->dim > 0 && a->seqlen > 0 && a->nstate > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_scan_bwd: batch=%d dim=%d seqlen=%d nstate=%d must all be positive", a->batch, a->dim, a->seqlen,
+              a->nstate);
+  SSM_REQUIRE(a->nstate <= BW_MAX_N, SSM_ERR_TOO_LARGE,
+              "ssm_scan_bwd: nstate=%d exceeds %d per call (split the state axis)", a->nstate, BW_MAX_N);
+  SSM_REQUIRE(valid_dtype(a->io_dtype) && valid_dtype(a->bc_dtype), SSM_ERR_BAD_DTYPE,
+              "ssm_scan_bwd: io_dtype=%d bc_dtype=%d", a->io_dtype, a->bc_dtype);
+  auto kind_ok = [](int k) { return k == SSM_PROJ_DN || k == SSM_PROJ_BDN || k == SSM_PROJ_BGNL; };
+  SSM_REQUIRE(kind_ok(a->b_kind) && kind_ok(a->c_kind), SSM_ERR_BAD_KIND, "ssm_scan_bwd: b_kind=%d c_kind=%d",
+              a->b_kind, a->c_kind);
+  const bool bv = a->b_kind == SSM_PROJ_BGNL, cv = a->c_kind == SSM_PROJ_BGNL;
+  if (bv) SSM_REQUIRE(a->b_groups > 0 && a->dim % a->b_groups == 0, SSM_ERR_BAD_SHAPE,
+                      "ssm_scan_bwd: b_groups=%d must divide dim=%d", a->b_groups, a->dim);
+  if (cv) SSM_REQUIRE(a->c_groups > 0 && a->dim % a->c_groups == 0, SSM_ERR_BAD_SHAPE,
+                      "ssm_scan_bwd: c_groups=%d must divide dim=%d", a->c_groups, a->dim);
+  SSM_REQUIRE((size_t)a->batch * a->dim < ((size_t)1 << 31) &&
+                  (size_t)a->batch * a->dim * a->seqlen < ((size_t)1 << 40),
+              SSM_ERR_TOO_LARGE, "ssm_scan_bwd: tensor too large");
+  const BwdPlan pl = plan_bwd(a->batch, a->dim, a->seqlen, a->nstate, a->b_kind, a->c_kind,
+                              bv ? a->b_groups : 1, cv ? a->c_groups : 1);
+  SSM_REQUIRE(a->workspace && a->workspace_bytes >= pl.total && aligned_to(a->workspace, 256), SSM_ERR_WORKSPACE,
+              "ssm_scan_bwd: a 256-byte aligned workspace of %zu bytes is required", pl.total);
+  const int es = dtype_size(a->io_dtype), bs = dtype_size(a->bc_dtype);
+  SSM_REQUIRE(aligned_to(a->u, es) && aligned_to(a->delta, es) && aligned_to(a->dout, es) && aligned_to(a->du, es) &&
+                  aligned_to(a->ddelta, es) && (!a->z || (aligned_to(a->z, es) && aligned_to(a->dz, es))) &&
+                  aligned_to(a->Bproj, bs) && aligned_to(a->Cproj, bs) && aligned_to(a->dB, 16) &&
+                  aligned_to(a->dC, 16),
+              SSM_ERR_ALIGNMENT, "ssm_scan_bwd: a pointer is not sufficiently aligned");
+
+  char *ws = reinterpret_cast<char *>(a->workspace);
+  ScanBwdParams p{};
+  p.u = a->u; p.delta = a->delta; p.z = a->z; p.dout = a->dout; p.Bp = a->Bproj; p.Cp = a->Cproj;
+  p.A = a->A; p.Dk = a->Dskip; p.bias = a->dt_bias; p.dlast = a->dlast_state; p.chunk_states = a->chunk_states;
+  p.du = a->du; p.ddelta = a->ddelta; p.dz = a->dz;
+  p.dA_rows = reinterpret_cast<float *>(ws + pl.off_dA);
+  p.dD_rows = reinterpret_cast<float *>(ws + pl.off_dD);
+  p.dbias_rows = reinterpret_cast<float *>(ws + pl.off_dbias);
+  p.dB_part = reinterpret_cast<float *>(ws + pl.off_dB);
+  p.dC_part = reinterpret_cast<float *>(ws + pl.off_dC);
+  p.batch = a->batch; p.dim = a->dim; p.len = a->seqlen; p.nstate = a->nstate;
+  p.bc_dtype = a->bc_dtype; p.b_kind = a->b_kind; p.c_kind = a->c_kind;
+  p.b_groups = bv ? a->b_groups : 1; p.c_groups = cv ? a->c_groups : 1;
+  p.softplus = a->delta_softplus ? 1 : 0;
+  p.rows_per_wg = pl.rows_per_wg; p.nblk = pl.nblk;
+  p.bc_vec_ok = a->seqlen % 4 == 0 && aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs);
+
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  int rc;
+  switch (a->io_dtype) {
+    case SSM_F32: rc = launch_bwd<float>(p, s); break;
+    case SSM_BF16: rc = launch_bwd<bf16_t>(p, s); break;
+    default: rc = launch_bwd<f16_t>(p, s); break;
+  }
+  if (rc != SSM_OK) return rc;
+
+  const int Bn = a->batch, D = a->dim, N = a->nstate, L = a->seqlen;
+  // dA (D,N), dD (D,), dbias (D,): fold over batch
+  hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)D * N)), dim3(256), 0, s, p.dA_rows, a->dA, Bn,
+                     (size_t)D * N);
+  if (a->dD) hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid(D)), dim3(256), 0, s, p.dD_rows, a->dD, Bn, (size_t)D);
+  if (a->ddt_bias)
+    hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid(D)), dim3(256), 0, s, p.dbias_rows, a->ddt_bias, Bn, (size_t)D);
+  // dB / dC in the shape of the given projection
+  auto fold_proj = [&](int kind, int groups, const float *partial, float *out) {
+    if (kind == SSM_PROJ_BGNL) {
+      // (B, G, nblk/G, N*L) -> (B, G, N*L)
+      const int per_group = pl.nblk / groups;
+      hipLaunchKernelGGL(fold_sum_kernel, dim3(fold_grid((size_t)Bn * groups * N * L)), dim3(256), 0, s, partial,
+                         out, (size_t)Bn * groups, per_group, (size_t)N * L);
+    } else if (kind == SSM_PROJ_BDN) {
+      hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)Bn * D * N)), dim3(256), 0, s, partial, out, 1,
+                         (size_t)Bn * D * N);
+    } else {
+      hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)D * N)), dim3(256), 0, s, partial, out, Bn,
+                         (size_t)D * N);
+    }
+  };
+  fold_proj(a->b_kind, p.b_groups, p.dB_part, a->dB);
+  fold_proj(a->c_kind, p.c_groups, p.dC_part, a->dC);
+  SSM_CHECK_LAUNCH("ssm_scan_bwd(fold)");
+  return SSM_OK;
+}

@@ -13,6 +13,8 @@ static bool valid_kind(int k) { return k == SSM_PROJ_DN || k == SSM_PROJ_BDN || 
 
 }  // namespace ssm
 
+extern "C" int ssm_scan_chunk_len(void) { return 512; }
+
 extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   using namespace ssm;
   SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_scan_fwd: args is NULL");
@@ -47,6 +49,7 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   ScanFwdParams p;
   p.u = a->u; p.delta = a->delta; p.z = a->z; p.Bp = a->Bproj; p.Cp = a->Cproj;
   p.A = a->A; p.Dk = a->Dskip; p.bias = a->dt_bias; p.out = a->out; p.last = a->last_state;
+  p.chunk_states = a->chunk_states;
   p.batch = a->batch; p.dim = a->dim; p.len = a->seqlen; p.nstate = a->nstate;
   p.bc_dtype = a->bc_dtype;
   p.b_kind = a->b_kind; p.c_kind = a->c_kind;
@@ -63,7 +66,11 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   while (rows > 1 && (per_b % rows != 0 || per_c % rows != 0)) rows >>= 1;
 
   int tune = a->tune_items;
-  if (tune == 0) tune = a->seqlen <= 256 ? 408 : 808;
+  if (tune == 0) tune = (a->seqlen <= 256 && !a->chunk_states) ? 408 : 808;
+  if (a->chunk_states)
+    SSM_REQUIRE(tune / 100 * WAVE == ssm_scan_chunk_len(), SSM_ERR_BAD_KIND,
+                "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (tune_items 808 or 816)",
+                ssm_scan_chunk_len());
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   switch (a->io_dtype) {
     case SSM_F32: return scan_fwd_dispatch<float>(p, tune, rows, stream);

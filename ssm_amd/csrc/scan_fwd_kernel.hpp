@@ -31,6 +31,7 @@ struct ScanFwdParams {
   const void *u, *delta, *z, *Bp, *Cp;
   const float *A, *Dk, *bias;
   void *out, *last;
+  float *chunk_states;   // optional (B, D, nchunks, N): row state entering each chunk
   int batch, dim, len, nstate;
   int bc_dtype;
   int b_kind, c_kind, b_groups, c_groups;
@@ -177,6 +178,12 @@ __global__ __launch_bounds__(WAVE *SCAN_MAX_WAVES) void scan_fwd_kernel(const Sc
   for (int c = 0; c < nchunks; ++c) {
     const int t0 = c * T;
     const int t = t0 + lane * K;
+    if (p.chunk_states) {
+      float *cs = p.chunk_states + (row * nchunks + c) * (size_t)N;
+      if (lane < N) cs[lane] = carry_lanes;
+      if (!SMALLN)
+        for (int n = SCAN_LANE_STATES + lane; n < N; n += WAVE) cs[n] = carry_hi[wave][n - SCAN_LANE_STATES];
+    }
 
     float dl[K], du[K], y[K];
     {

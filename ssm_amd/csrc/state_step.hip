@@ -1,0 +1,161 @@
+// Single-token selective state update (decode step) for gfx950.
+//
+//   dt'   = softplus(dt + dt_bias)
+//   h'    = exp(dt' A) h + dt' x B          (state overwritten in place)
+//   y     = <h', C> + D x ;  y *= silu(z)
+//
+// The op moves 2 * B*D*N state elements and little else, so it is laid out
+// for HBM streaming: TPR lanes share one (batch, channel) row, each lane owns
+// VEC consecutive state entries per trip (128-bit accesses when VEC = 4), and
+// the partial dot products are combined with a butterfly inside the wave.
+#include "common.hpp"
+
+namespace ssm {
+
+struct StepParams {
+  void *state;
+  const void *x, *dt, *z, *Bp, *Cp;
+  const float *A, *Dk, *bias;
+  void *out;
+  int batch, dim, nstate;
+  int io_dtype, bc_dtype;
+  int b_kind, c_kind, b_groups, c_groups;
+  int softplus;
+  int tpr_log2;   // lanes per row = 1 << tpr_log2
+};
+
+__device__ __forceinline__ void store_from_f32(void *p, int dtype, size_t i, float v) {
+  if (dtype == SSM_F32) reinterpret_cast<float *>(p)[i] = v;
+  else if (dtype == SSM_BF16) reinterpret_cast<bf16_t *>(p)[i] = from_f32<bf16_t>(v);
+  else reinterpret_cast<f16_t *>(p)[i] = from_f32<f16_t>(v);
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec(const T *p, float (&v)[VEC]) {
+  Pack<T, VEC> raw = *reinterpret_cast<const Pack<T, VEC> *>(p);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) v[i] = to_f32(raw.v[i]);
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_vec_rt(const void *p, int dtype, size_t off, float (&v)[VEC]) {
+  if (dtype == SSM_F32) load_vec<float, VEC>(reinterpret_cast<const float *>(p) + off, v);
+  else if (dtype == SSM_BF16) load_vec<bf16_t, VEC>(reinterpret_cast<const bf16_t *>(p) + off, v);
+  else load_vec<f16_t, VEC>(reinterpret_cast<const f16_t *>(p) + off, v);
+}
+
+template <typename state_t, int VEC>
+__global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
+  const int tpr = 1 << p.tpr_log2;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t row = gid >> p.tpr_log2;
+  const int sub = (int)(gid & (tpr - 1));
+  const size_t nrows = (size_t)p.batch * p.dim;
+  const bool live = row < nrows;
+  const size_t r = live ? row : 0;          // dead lanes shadow row 0 but never store
+  const int b = (int)(r / p.dim), d = (int)(r % p.dim);
+  const int N = p.nstate;
+
+  float dtv = load_as_f32(p.dt, p.io_dtype, r);
+  if (p.bias) dtv += p.bias[d];
+  if (p.softplus) dtv = softplus_f32(dtv);
+  const float xv = load_as_f32(p.x, p.io_dtype, r);
+  const float dx = dtv * xv;
+  const float dt2 = dtv * LOG2E;
+
+  size_t b_off, c_off;
+  if (p.b_kind == SSM_PROJ_BGNL) b_off = ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * N;
+  else b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+  if (p.c_kind == SSM_PROJ_BGNL) c_off = ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * N;
+  else c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+
+  state_t *srow = reinterpret_cast<state_t *>(p.state) + r * N;
+  const float *arow = p.A + (size_t)d * N;
+  float acc = 0.0f;
+  for (int n0 = sub * VEC; n0 < N; n0 += tpr * VEC) {
+    float h[VEC], a[VEC], bv[VEC], cv[VEC];
+    load_vec<state_t, VEC>(srow + n0, h);
+    load_vec<float, VEC>(arow + n0, a);
+    load_vec_rt<VEC>(p.Bp, p.bc_dtype, b_off + n0, bv);
+    load_vec_rt<VEC>(p.Cp, p.bc_dtype, c_off + n0, cv);
+    Pack<state_t, VEC> outv;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float hn = __builtin_fmaf(exp2_hw(dt2 * a[i]), h[i], dx * bv[i]);
+      acc = __builtin_fmaf(hn, cv[i], acc);
+      outv.v[i] = from_f32<state_t>(hn);
+    }
+    if (live) *reinterpret_cast<Pack<state_t, VEC> *>(srow + n0) = outv;
+  }
+  for (int m = tpr >> 1; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, WAVE);
+  if (live && sub == 0) {
+    float y = acc;
+    if (p.Dk) y = __builtin_fmaf(p.Dk[d], xv, y);
+    if (p.z) y *= silu_f32(load_as_f32(p.z, p.io_dtype, r));
+    store_from_f32(p.out, p.io_dtype, r, y);
+  }
+}
+
+template <typename state_t>
+static int launch_step(const StepParams &p0, bool vec4, hipStream_t stream) {
+  StepParams p = p0;
+  const int vec = vec4 ? 4 : 1;
+  const int per_row = (p.nstate + vec - 1) / vec;
+  int lg = 0;
+  while ((1 << lg) < per_row && lg < 4) ++lg;    // at most 16 lanes per row
+  p.tpr_log2 = lg;
+  const size_t threads = ((size_t)p.batch * p.dim) << lg;
+  const unsigned grid = (unsigned)((threads + 255) / 256);
+  if (vec4) hipLaunchKernelGGL((state_step_kernel<state_t, 4>), dim3(grid), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((state_step_kernel<state_t, 1>), dim3(grid), dim3(256), 0, stream, p);
+  SSM_CHECK_LAUNCH("ssm_state_step");
+  return SSM_OK;
+}
+
+}  // namespace ssm
+
+extern "C" int ssm_state_step(const ssm_state_step_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_state_step: args is NULL");
+  SSM_REQUIRE(a->state && a->x && a->dt && a->A && a->Bproj && a->Cproj && a->out, SSM_ERR_NULL_POINTER,
+              "ssm_state_step: state, x, dt, A, Bproj, Cproj and out are required");
+  SSM_REQUIRE(a->batch > 0 && a->dim > 0 && a->nstate > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_state_step: batch=%d dim=%d nstate=%d must all be positive", a->batch, a->dim, a->nstate);
+  SSM_REQUIRE(valid_dtype(a->state_dtype) && valid_dtype(a->io_dtype) && valid_dtype(a->bc_dtype),
+              SSM_ERR_BAD_DTYPE, "ssm_state_step: state_dtype=%d io_dtype=%d bc_dtype=%d", a->state_dtype,
+              a->io_dtype, a->bc_dtype);
+  auto kind_ok = [](int k) { return k == SSM_PROJ_DN || k == SSM_PROJ_BDN || k == SSM_PROJ_BGNL; };
+  SSM_REQUIRE(kind_ok(a->b_kind) && kind_ok(a->c_kind), SSM_ERR_BAD_KIND, "ssm_state_step: b_kind=%d c_kind=%d",
+              a->b_kind, a->c_kind);
+  if (a->b_kind == SSM_PROJ_BGNL)
+    SSM_REQUIRE(a->b_groups > 0 && a->dim % a->b_groups == 0, SSM_ERR_BAD_SHAPE,
+                "ssm_state_step: b_groups=%d must divide dim=%d", a->b_groups, a->dim);
+  if (a->c_kind == SSM_PROJ_BGNL)
+    SSM_REQUIRE(a->c_groups > 0 && a->dim % a->c_groups == 0, SSM_ERR_BAD_SHAPE,
+                "ssm_state_step: c_groups=%d must divide dim=%d", a->c_groups, a->dim);
+  SSM_REQUIRE((size_t)a->batch * a->dim < ((size_t)1 << 27), SSM_ERR_TOO_LARGE, "ssm_state_step: too many rows");
+  const int ss = dtype_size(a->state_dtype), es = dtype_size(a->io_dtype), bs = dtype_size(a->bc_dtype);
+  SSM_REQUIRE(aligned_to(a->state, ss) && aligned_to(a->x, es) && aligned_to(a->dt, es) &&
+                  aligned_to(a->out, es) && (!a->z || aligned_to(a->z, es)) && aligned_to(a->A, 4) &&
+                  aligned_to(a->Bproj, bs) && aligned_to(a->Cproj, bs),
+              SSM_ERR_ALIGNMENT, "ssm_state_step: a pointer is not aligned to its element size");
+
+  StepParams p;
+  p.state = a->state; p.x = a->x; p.dt = a->dt; p.z = a->z; p.Bp = a->Bproj; p.Cp = a->Cproj;
+  p.A = a->A; p.Dk = a->Dskip; p.bias = a->dt_bias; p.out = a->out;
+  p.batch = a->batch; p.dim = a->dim; p.nstate = a->nstate;
+  p.io_dtype = a->io_dtype; p.bc_dtype = a->bc_dtype;
+  p.b_kind = a->b_kind; p.c_kind = a->c_kind;
+  p.b_groups = a->b_kind == SSM_PROJ_BGNL ? a->b_groups : 1;
+  p.c_groups = a->c_kind == SSM_PROJ_BGNL ? a->c_groups : 1;
+  p.softplus = a->dt_softplus ? 1 : 0;
+  p.tpr_log2 = 0;
+  const bool vec4 = a->nstate % 4 == 0 && aligned_to(a->state, 4 * ss) && aligned_to(a->A, 16) &&
+                    aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs);
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  switch (a->state_dtype) {
+    case SSM_F32: return launch_step<float>(p, vec4, stream);
+    case SSM_BF16: return launch_step<bf16_t>(p, vec4, stream);
+    default: return launch_step<f16_t>(p, vec4, stream);
+  }
+}

@@ -52,7 +52,7 @@ class ScanPlan:
     called repeatedly; it enqueues one launch on the current stream."""
 
     def __init__(self, u, delta, A, B, C, D, z, dt_bias, softplus, want_state, tune_items=0,
-                 out=None, last=None):
+                 out=None, last=None, want_chunk_states=False):
         batch, dim, length, nstate, (bkind, bgroups), (ckind, cgroups) = \
             K.check_selective_scan(u, delta, A, B, C, D, z, dt_bias)
         self.device = K.require_gpu(u, delta, A, B, C, D, z, dt_bias)
@@ -67,10 +67,18 @@ class ScanPlan:
         self.last = last
         if want_state and last is None:
             self.last = torch.empty(batch, dim, nstate, dtype=io, device=self.device)
+        self.chunk_states = None
+        if want_chunk_states:
+            chunk = _lib.load().ssm_scan_chunk_len()
+            nchunks = (length + chunk - 1) // chunk
+            self.chunk_states = torch.empty(batch, dim, nchunks, nstate, dtype=torch.float32,
+                                            device=self.device)
+            tune_items = tune_items or 808
         self.args = _lib.ScanFwdArgs(
             u=_lib.ptr(k["u"]), delta=_lib.ptr(k["delta"]), z=_lib.ptr(k["z"]), A=_lib.ptr(k["A"]),
             Bproj=_lib.ptr(k["B"]), Cproj=_lib.ptr(k["C"]), Dskip=_lib.ptr(k["D"]),
             dt_bias=_lib.ptr(k["bias"]), out=_lib.ptr(self.out), last_state=_lib.ptr(self.last),
+            chunk_states=_lib.ptr(self.chunk_states),
             batch=batch, dim=dim, seqlen=length, nstate=nstate,
             io_dtype=_lib.dtype_enum(io), bc_dtype=_lib.dtype_enum(bc),
             b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
@@ -89,6 +97,100 @@ def _scan_forward(u, delta, A, B, C, D, z, dt_bias, softplus, want_state, tune_i
         out = out.to(plan.result_dtype)
         last = last.to(plan.result_dtype) if last is not None else None
     return out, last
+
+
+_BWD_MAX_STATES = 16     # states handled by one ssm_scan_bwd call
+
+
+def _slice_states(p, kind, lo, hi):
+    if kind == _lib.PROJ_DN:
+        return p[:, lo:hi]
+    if kind == _lib.PROJ_BDN:
+        return p[:, :, lo:hi]
+    return p[:, :, lo:hi, :]
+
+
+def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softplus, chunk_states=None):
+    """Run ``ssm_scan_bwd``; returns fp32/io-dtype gradients in input order
+    ``(du, ddelta, dA, dB, dC, dD, dz, ddt_bias)``.  State sizes above 16 are
+    processed in blocks of 16 states (the recurrence is independent per state and
+    every gradient is additive over states)."""
+    batch, dim, length, nstate, (bkind, bgroups), (ckind, cgroups) = \
+        K.check_selective_scan(u, delta, A, B, C, D, z, dt_bias)
+    dev = K.require_gpu(u, delta, A, B, C, D, z, dt_bias, grad_out)
+    io = K.common_io_dtype([u, delta, z])
+    bc = K.common_io_dtype([B, C])
+    u_c, dl_c, z_c = K.cast_c(u, io), K.cast_c(delta, io), K.cast_c(z, io)
+    go_c = K.cast_c(grad_out, io)
+    A_f, D_f, bias_f = K.as_f32_vec(A), K.as_f32_vec(D), K.as_f32_vec(dt_bias)
+    B_c, C_c = K.cast_c(B, bc), K.cast_c(C, bc)
+    glast = K.as_f32_vec(grad_last) if grad_last is not None else None
+    lib = _lib.load()
+
+    dA = torch.empty(dim, nstate, dtype=torch.float32, device=dev)
+    dB = torch.empty(B_c.shape, dtype=torch.float32, device=dev)
+    dC = torch.empty(C_c.shape, dtype=torch.float32, device=dev)
+    dD = torch.empty(dim, dtype=torch.float32, device=dev) if D is not None else None
+    dbias = torch.empty(dim, dtype=torch.float32, device=dev) if dt_bias is not None else None
+    blocks = [(lo, min(nstate, lo + _BWD_MAX_STATES)) for lo in range(0, nstate, _BWD_MAX_STATES)]
+    single = len(blocks) == 1
+    du = ddl = dz = None
+    for bi, (lo, hi) in enumerate(blocks):
+        n_blk = hi - lo
+        if single:
+            A_b, B_b, C_b, gl_b = A_f, B_c, C_c, glast
+            cs = chunk_states
+        else:
+            A_b = A_f[:, lo:hi].contiguous()
+            B_b = _slice_states(B_c, bkind, lo, hi).contiguous()
+            C_b = _slice_states(C_c, ckind, lo, hi).contiguous()
+            gl_b = glast[:, :, lo:hi].contiguous() if glast is not None else None
+            cs = None
+        D_b = D_f if bi == 0 else None
+        if cs is None:      # regenerate the chunk checkpoints for this block of states
+            fwd = ScanPlan(u_c, dl_c, A_b, B_b, C_b, D_b, z_c, bias_f, softplus, False,
+                           want_chunk_states=True)
+            fwd.run()
+            cs = fwd.chunk_states
+        du_b, ddl_b = torch.empty_like(u_c), torch.empty_like(u_c)
+        dz_b = torch.empty_like(u_c) if z_c is not None else None
+        dA_b = dA if single else torch.empty(dim, n_blk, dtype=torch.float32, device=dev)
+        dB_b = dB if single else torch.empty(B_b.shape, dtype=torch.float32, device=dev)
+        dC_b = dC if single else torch.empty(C_b.shape, dtype=torch.float32, device=dev)
+        dD_b = dD if bi == 0 else None
+        dbias_b = torch.empty(dim, dtype=torch.float32, device=dev) if dt_bias is not None else None
+        nbytes = lib.ssm_scan_bwd_workspace_bytes(batch, dim, length, n_blk, bkind, ckind, bgroups, cgroups)
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
+        ws_ptr = (ws.data_ptr() + 255) // 256 * 256
+        args = _lib.ScanBwdArgs(
+            u=_lib.ptr(u_c), delta=_lib.ptr(dl_c), z=_lib.ptr(z_c), dout=_lib.ptr(go_c), A=_lib.ptr(A_b),
+            Bproj=_lib.ptr(B_b), Cproj=_lib.ptr(C_b), Dskip=_lib.ptr(D_b), dt_bias=_lib.ptr(bias_f),
+            dlast_state=_lib.ptr(gl_b), chunk_states=_lib.ptr(cs), du=_lib.ptr(du_b), ddelta=_lib.ptr(ddl_b),
+            dz=_lib.ptr(dz_b), dA=_lib.ptr(dA_b), dB=_lib.ptr(dB_b), dC=_lib.ptr(dC_b), dD=_lib.ptr(dD_b),
+            ddt_bias=_lib.ptr(dbias_b), workspace=ws_ptr, workspace_bytes=nbytes,
+            batch=batch, dim=dim, seqlen=length, nstate=n_blk, io_dtype=_lib.dtype_enum(io),
+            bc_dtype=_lib.dtype_enum(bc), b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
+            delta_softplus=int(bool(softplus)))
+        _lib.call("ssm_scan_bwd", args, dev)
+        if single:
+            du, ddl, dz, dbias = du_b, ddl_b, dz_b, dbias_b
+        else:
+            dA[:, lo:hi] = dA_b
+            _slice_states(dB, bkind, lo, hi).copy_(dB_b)
+            _slice_states(dC, ckind, lo, hi).copy_(dC_b)
+            if bi == 0:
+                du, ddl = du_b.float(), ddl_b.float()
+                dz = dz_b.float() if dz_b is not None else None
+                if dbias is not None:
+                    dbias.copy_(dbias_b)
+            else:
+                du += du_b
+                ddl += ddl_b
+                if dz is not None:
+                    dz += dz_b
+                if dbias is not None:
+                    dbias += dbias_b
+    return du, ddl, dA, dB, dC, dD, dz, dbias
 
 
 def selective_scan(u, delta, A, B, C, D=None, z=None, dt_bias=None, softplus=False,
@@ -127,8 +229,255 @@ def selective_scan(u, delta, A, B, C, D=None, z=None, dt_bias=None, softplus=Fal
     return out
 
 
+# ---------------------------------------------------------------------------
+# selective state step (decode)
+# ---------------------------------------------------------------------------
+
+class StepPlan:
+    """A prepared ``ssm_state_step`` call that updates ``state`` in place."""
+
+    def __init__(self, state, x, dt, A, B, C, D, z, dt_bias, softplus, out=None):
+        batch, dim, nstate, (bkind, bgroups), (ckind, cgroups) = \
+            K.check_state_step(state, x, dt, A, B, C, D, z, dt_bias)
+        self.device = K.require_gpu(state, x, dt, A, B, C, D, z, dt_bias)
+        if not state.is_contiguous():
+            raise ValueError("state must be contiguous to be updated in place")
+        io = K.common_io_dtype([x, dt, z])
+        bc = K.common_io_dtype([B, C])
+        self.result_dtype = x.dtype
+        self.keep = dict(x=K.cast_c(x, io), dt=K.cast_c(dt, io), z=K.cast_c(z, io), B=K.cast_c(B, bc),
+                         C=K.cast_c(C, bc), A=K.as_f32_vec(A), D=K.as_f32_vec(D), bias=K.as_f32_vec(dt_bias))
+        k = self.keep
+        self.state = state.detach()
+        self.out = out if out is not None else torch.empty(batch, dim, dtype=io, device=self.device)
+        self.args = _lib.StateStepArgs(
+            state=_lib.ptr(self.state), x=_lib.ptr(k["x"]), dt=_lib.ptr(k["dt"]), z=_lib.ptr(k["z"]),
+            A=_lib.ptr(k["A"]), Bproj=_lib.ptr(k["B"]), Cproj=_lib.ptr(k["C"]), Dskip=_lib.ptr(k["D"]),
+            dt_bias=_lib.ptr(k["bias"]), out=_lib.ptr(self.out),
+            batch=batch, dim=dim, nstate=nstate,
+            state_dtype=_lib.dtype_enum(state.dtype), io_dtype=_lib.dtype_enum(io),
+            bc_dtype=_lib.dtype_enum(bc), b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
+            dt_softplus=int(bool(softplus)))
+
+    def run(self):
+        _lib.call("ssm_state_step", self.args, self.device)
+        return self.out
+
+
+def selective_state_step(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, softplus=True):
+    """Advance the selective state by one token on the GPU; ``state`` is updated in place.
+
+    Args:
+        state: Recurrent state ``(B, D, N)`` (float32, bfloat16 or float16), overwritten.
+        x: Input drive ``(B, D)``.
+        dt: Time-step ``(B, D)``.
+        A: State matrix ``(D, N)``.
+        B: Input projection ``(D, N)``, ``(B, D, N)`` or grouped ``(B, G, N)`` with ``G | D``.
+        C: Output projection, same accepted shapes as ``B``.
+        D: Optional skip ``(D,)``.
+        z: Optional gate ``(B, D)``; ``silu`` is applied.
+        dt_bias: Optional bias ``(D,)`` added before ``softplus``.
+        softplus: Apply ``softplus`` to the biased ``dt`` (default ``True``).
+
+    Returns:
+        Output ``(B, D)`` in ``x.dtype``.
+    """
+    tensors = (state, x, dt, A, B, C, D, z, dt_bias)
+    if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
+        from ._autograd import state_step_with_grad
+        return state_step_with_grad(state, x, dt, A, B, C, D, z, dt_bias, bool(softplus))
+    if state.is_contiguous():
+        plan = StepPlan(state, x, dt, A, B, C, D, z, dt_bias, softplus)
+        out = plan.run()
+    else:
+        work = state.contiguous()
+        plan = StepPlan(work, x, dt, A, B, C, D, z, dt_bias, softplus)
+        out = plan.run()
+        state.copy_(work)
+    return out if out.dtype == x.dtype else out.to(x.dtype)
+
+
+# ---------------------------------------------------------------------------
+# depthwise causal convolution
+# ---------------------------------------------------------------------------
+
+def _conv_weight_f32(weight):
+    w = weight.detach()
+    if w.ndim == 3:
+        w = w[:, 0, :]
+    return w.to(torch.float32).contiguous()
+
+
+def _conv_forward(x, weight, bias, activation):
+    batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation)
+    dev = K.require_gpu(x, weight, bias)
+    xc = K.cast_c(x, x.dtype)
+    wf, bf = _conv_weight_f32(weight), K.as_f32_vec(bias)
+    y = torch.empty_like(xc)
+    args = _lib.Conv1dFwdArgs(
+        x=_lib.ptr(xc), weight=_lib.ptr(wf), bias=_lib.ptr(bf), y=_lib.ptr(y),
+        batch=batch, channels=chans, seqlen=length, width=width, io_dtype=_lib.dtype_enum(xc.dtype),
+        layout=_lib.LAYOUT_BCL if channels_first else _lib.LAYOUT_BLC,
+        activation=_lib.ACT_SILU if silu else _lib.ACT_IDENTITY)
+    _lib.call("ssm_conv1d_fwd", args, dev)
+    return y
+
+
+def _conv_backward(grad_out, x, weight, bias, activation):
+    """-> (dx, dweight (C,K) fp32, dbias (C,) fp32 or None)."""
+    batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation)
+    dev = K.require_gpu(x, weight, bias, grad_out)
+    xc, gc = K.cast_c(x, x.dtype), K.cast_c(grad_out, x.dtype)
+    wf, bf = _conv_weight_f32(weight), K.as_f32_vec(bias)
+    dx = torch.empty_like(xc)
+    dw = torch.empty(chans, width, dtype=torch.float32, device=dev)
+    db = torch.empty(chans, dtype=torch.float32, device=dev) if bias is not None else None
+    nbytes = _lib.load().ssm_conv1d_bwd_workspace_bytes(batch, chans, width)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    args = _lib.Conv1dBwdArgs(
+        x=_lib.ptr(xc), dout=_lib.ptr(gc), weight=_lib.ptr(wf), bias=_lib.ptr(bf), dx=_lib.ptr(dx),
+        dweight=_lib.ptr(dw), dbias=_lib.ptr(db), workspace=_lib.ptr(ws), workspace_bytes=nbytes,
+        batch=batch, channels=chans, seqlen=length, width=width, io_dtype=_lib.dtype_enum(xc.dtype),
+        layout=_lib.LAYOUT_BCL if channels_first else _lib.LAYOUT_BLC,
+        activation=_lib.ACT_SILU if silu else _lib.ACT_IDENTITY)
+    _lib.call("ssm_conv1d_bwd", args, dev)
+    return dx, dw, db
+
+
+def dw_causal_conv(x, weight, bias=None, activation="silu"):
+    """Depthwise causal 1-D convolution with optional SiLU on the GPU.
+
+    Args:
+        x: Input ``(B, C, L)`` or ``(B, L, C)``; the layout is channels-first when
+            ``x.shape[1] == C`` (tested first), else channels-last.
+        weight: Depthwise kernel ``(C, K)`` or ``(C, 1, K)``.
+        bias: Optional bias ``(C,)``.
+        activation: ``"silu"``/``"swish"`` or ``"identity"``/``"none"``.
+
+    Returns:
+        Tensor with the layout and dtype of ``x``.
+    """
+    tensors = (x, weight, bias)
+    if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
+        from ._autograd import CausalConvFn
+        return CausalConvFn.apply(x, weight, bias, activation)
+    return _conv_forward(x, weight, bias, activation)
+
+
+# ---------------------------------------------------------------------------
+# residual-add + LayerNorm / RMSNorm
+# ---------------------------------------------------------------------------
+
+def _norm_forward(x, weight, bias, residual, is_rms, eps, prenorm, residual_in_fp32,
+                  want_residual_out=False, want_stats=False):
+    rows, hidden = K.check_norm(x, weight, bias, residual)
+    dev = K.require_gpu(x, weight, bias, residual)
+    xc = K.cast_c(x, x.dtype)
+    rc = K.cast_c(residual, residual.dtype) if residual is not None else None
+    wf, bf = K.as_f32_vec(weight), K.as_f32_vec(bias)
+    y = torch.empty_like(xc)
+    res_out = None
+    if want_residual_out:
+        # what the next block should carry: fp32 when a fp32 residual stream is requested,
+        # otherwise the residual's (or x's) own dtype
+        if residual is not None:
+            ro_dtype = torch.float32 if residual_in_fp32 else residual.dtype
+        else:
+            ro_dtype = torch.float32 if residual_in_fp32 else x.dtype
+        res_out = torch.empty(x.shape, dtype=ro_dtype, device=dev)
+    mean = torch.empty(rows, dtype=torch.float32, device=dev) if want_stats else None
+    rstd = torch.empty(rows, dtype=torch.float32, device=dev) if want_stats else None
+    args = _lib.NormFwdArgs(
+        x=_lib.ptr(xc), residual=_lib.ptr(rc), weight=_lib.ptr(wf), bias=_lib.ptr(bf), y=_lib.ptr(y),
+        residual_out=_lib.ptr(res_out), mean=_lib.ptr(mean), rstd=_lib.ptr(rstd),
+        rows=rows, hidden=hidden, x_dtype=_lib.dtype_enum(xc.dtype),
+        residual_dtype=_lib.dtype_enum(rc.dtype) if rc is not None else 0,
+        residual_out_dtype=_lib.dtype_enum(res_out.dtype) if res_out is not None else 0,
+        is_rms=int(bool(is_rms)), prenorm=int(bool(prenorm)), eps=float(eps))
+    _lib.call("ssm_norm_fwd", args, dev)
+    return y, res_out, mean, rstd
+
+
+def _norm_backward(grad_out, x, weight, residual, mean, rstd, is_rms, prenorm, want_dbias, want_dres):
+    rows, hidden = K.check_norm(x, weight, None, residual)
+    dev = K.require_gpu(x, weight, residual, grad_out)
+    xc, gc = K.cast_c(x, x.dtype), K.cast_c(grad_out, x.dtype)
+    rc = K.cast_c(residual, residual.dtype) if residual is not None else None
+    wf = K.as_f32_vec(weight)
+    dx = torch.empty_like(xc)
+    dres = torch.empty_like(rc) if (want_dres and rc is not None) else None
+    dw = torch.empty(hidden, dtype=torch.float32, device=dev)
+    db = torch.empty(hidden, dtype=torch.float32, device=dev) if want_dbias else None
+    nbytes = _lib.load().ssm_norm_bwd_workspace_bytes(rows, hidden)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    args = _lib.NormBwdArgs(
+        x=_lib.ptr(xc), residual=_lib.ptr(rc), dy=_lib.ptr(gc), weight=_lib.ptr(wf), mean=_lib.ptr(mean),
+        rstd=_lib.ptr(rstd), dx=_lib.ptr(dx), dresidual=_lib.ptr(dres), dweight=_lib.ptr(dw),
+        dbias=_lib.ptr(db), workspace=_lib.ptr(ws), workspace_bytes=nbytes, rows=rows, hidden=hidden,
+        x_dtype=_lib.dtype_enum(xc.dtype),
+        residual_dtype=_lib.dtype_enum(rc.dtype) if rc is not None else 0,
+        is_rms=int(bool(is_rms)), prenorm=int(bool(prenorm)))
+    _lib.call("ssm_norm_bwd", args, dev)
+    return dx, dres, dw, db
+
+
+def fused_layer_norm(x, weight, bias, residual=None, is_rms=False, eps=1e-5, prenorm=True,
+                     residual_in_fp32=True):
+    """Residual addition fused with LayerNorm or RMSNorm on the GPU.
+
+    Args:
+        x: Input ``(B, L, D)``.
+        weight: Scale ``(D,)``.
+        bias: Optional shift ``(D,)``.
+        residual: Optional residual, same shape as ``x`` (any supported dtype).
+        is_rms: RMSNorm when ``True``, LayerNorm otherwise.
+        eps: Numerical stabiliser.
+        prenorm: Add the residual before normalising (``True``) or after (``False``).
+        residual_in_fp32: Kept for signature parity; sums are always formed in float32.
+
+    Returns:
+        Normalised tensor with the shape and dtype of ``x``.
+    """
+    tensors = (x, weight, bias, residual)
+    if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
+        from ._autograd import FusedNormFn
+        return FusedNormFn.apply(x, weight, bias, residual, bool(is_rms), float(eps), bool(prenorm),
+                                 bool(residual_in_fp32), False)[0]
+    return _norm_forward(x, weight, bias, residual, is_rms, eps, prenorm, residual_in_fp32)[0]
+
+
+def fused_layer_norm_with_residual(x, weight, bias, residual=None, is_rms=False, eps=1e-5,
+                                   prenorm=True, residual_in_fp32=True):
+    """Like :func:`fused_layer_norm` but also returns the pre-normalisation sum.
+
+    The reference's operator returns only the normalised tensor
+    (src/ssm/ops/python/reference.py:609), so a block has to redo ``x + residual``
+    to carry the residual stream; this entry returns both from one pass.
+
+    Args:
+        x, weight, bias, residual, is_rms, eps, prenorm, residual_in_fp32: as in
+            :func:`fused_layer_norm`.
+
+    Returns:
+        ``(y, residual_out)`` where ``residual_out = x (+ residual if prenorm)`` in
+        float32 when ``residual_in_fp32`` else in the residual's (or ``x``'s) dtype.
+    """
+    tensors = (x, weight, bias, residual)
+    if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
+        from ._autograd import FusedNormFn
+        return FusedNormFn.apply(x, weight, bias, residual, bool(is_rms), float(eps), bool(prenorm),
+                                 bool(residual_in_fp32), True)
+    y, res_out, _, _ = _norm_forward(x, weight, bias, residual, is_rms, eps, prenorm, residual_in_fp32,
+                                     want_residual_out=True)
+    return y, res_out
+
+
 __all__ = [
     "selective_scan",
+    "selective_state_step",
+    "dw_causal_conv",
+    "fused_layer_norm",
+    "fused_layer_norm_with_residual",
     "_cpu_backend_status",
     "_cuda_backend_status",
     "_hip_backend_status",

@@ -1,0 +1,125 @@
+"""``torch.autograd.Function`` wrappers that route backward passes to the HIP
+kernels.
+
+They play the role of the reference's ``_SelectiveScanCudaFunction`` ...
+``_FusedLayerNormCudaFunction`` (src/ssm/ops/__init__.py:198-1224): what is
+saved for backward, which inputs get gradients, and the rule that an input
+which did not require a gradient receives ``None`` (``:284-291``).  Gradients
+are returned in the dtype of the corresponding input.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _contract as K
+
+
+def _like(grad, ref):
+    """Cast/reshape a kernel gradient to what autograd expects for ``ref``."""
+    if grad is None or ref is None:
+        return None
+    if grad.shape != ref.shape:
+        grad = grad.reshape(ref.shape)
+    return grad if grad.dtype == ref.dtype else grad.to(ref.dtype)
+
+
+class CausalConvFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, activation):
+        from . import _conv_forward
+
+        y = _conv_forward(x, weight, bias, activation)
+        ctx.save_for_backward(x, weight, bias)
+        ctx.activation = activation
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from . import _conv_backward
+
+        x, weight, bias = ctx.saved_tensors
+        dx, dw, db = _conv_backward(grad_out, x, weight, bias, ctx.activation)
+        need = ctx.needs_input_grad
+        return (_like(dx, x) if need[0] else None,
+                _like(dw, weight) if need[1] else None,
+                _like(db, bias) if (bias is not None and need[2]) else None,
+                None)
+
+
+class FusedNormFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, residual, is_rms, eps, prenorm, residual_in_fp32, want_res_out):
+        from . import _norm_forward
+
+        y, res_out, mean, rstd = _norm_forward(x, weight, bias, residual, is_rms, eps, prenorm,
+                                               residual_in_fp32, want_residual_out=want_res_out,
+                                               want_stats=True)
+        ctx.save_for_backward(x, weight, bias, residual, mean, rstd)
+        ctx.cfg = (is_rms, prenorm)
+        if res_out is None:
+            res_out = x.new_empty(0)
+            ctx.mark_non_differentiable(res_out)
+        ctx.has_res_out = want_res_out
+        return y, res_out
+
+    @staticmethod
+    def backward(ctx, grad_y, grad_res_out):
+        from . import _norm_backward
+
+        x, weight, bias, residual, mean, rstd = ctx.saved_tensors
+        is_rms, prenorm = ctx.cfg
+        need = ctx.needs_input_grad
+        want_dres = residual is not None and need[3]
+        dx, dres, dw, db = _norm_backward(grad_y.contiguous(), x, weight, residual, mean, rstd, is_rms,
+                                          prenorm, bias is not None, want_dres)
+        if ctx.has_res_out and grad_res_out is not None and grad_res_out.numel() == x.numel():
+            # residual_out = x (+ residual when prenorm): its gradient flows straight through
+            dx = dx + grad_res_out.to(dx.dtype)
+            if dres is not None and prenorm:
+                dres = dres + grad_res_out.to(dres.dtype)
+        return (_like(dx, x) if need[0] else None,
+                _like(dw, weight) if need[1] else None,
+                _like(db, bias) if (bias is not None and need[2]) else None,
+                _like(dres, residual) if want_dres else None,
+                None, None, None, None, None)
+
+
+class SelectiveScanFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, u, delta, A, B, C, D, z, dt_bias, softplus, want_state):
+        from . import ScanPlan, _BWD_MAX_STATES
+
+        keep_cs = A.shape[-1] <= _BWD_MAX_STATES
+        plan = ScanPlan(u, delta, A, B, C, D, z, dt_bias, softplus, want_state, want_chunk_states=keep_cs)
+        out, last = plan.run()
+        if out.dtype != u.dtype:
+            out = out.to(u.dtype)
+            last = last.to(u.dtype) if last is not None else None
+        ctx.save_for_backward(u, delta, A, B, C, D, z, dt_bias, plan.chunk_states)
+        ctx.softplus = softplus
+        if last is None:
+            last = u.new_empty(0)
+            ctx.mark_non_differentiable(last)
+        return out, last
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_last):
+        from . import _scan_backward
+
+        u, delta, A, B, C, D, z, dt_bias, chunk_states = ctx.saved_tensors
+        if grad_last is not None and grad_last.numel() == 0:
+            grad_last = None
+        grads = _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, ctx.softplus,
+                               chunk_states=chunk_states)
+        need = ctx.needs_input_grad
+        refs = (u, delta, A, B, C, D, z, dt_bias)
+        out = tuple(_like(g, r) if (r is not None and need[i]) else None
+                    for i, (g, r) in enumerate(zip(grads, refs)))
+        return out + (None, None)
+
+
+def state_step_with_grad(state, x, dt, A, B, C, D, z, dt_bias, softplus):
+    raise NotImplementedError(
+        "selective_state_step has no backward kernel in this backend yet; call it under "
+        "torch.no_grad() (decode) or differentiate through selective_scan instead.")

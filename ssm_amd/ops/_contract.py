@@ -121,3 +121,131 @@ def check_selective_scan(u, delta, A, B, C, D, z, dt_bias):
     if batch == 0 or dim == 0 or length == 0 or nstate == 0:
         raise ValueError("selective_scan needs non-empty B, D, L and N.")
     return batch, dim, length, nstate, bk, ck
+
+
+# ------------------------------------------------------ selective state step
+
+def step_projection_kind(name: str, p: torch.Tensor, batch: int, dim: int, nstate: int) -> tuple[int, int]:
+    """-> (kind, groups).  A 3-D tensor whose second axis is not ``D`` is the
+    grouped ``(B, G, N)`` form (reference.py:252-272)."""
+    from .._lib import PROJ_BDN, PROJ_BGNL, PROJ_DN
+
+    if p.dim() == 3 and p.shape[0] == batch and p.shape[1] != dim:
+        groups = int(p.shape[1])
+        if groups == 0 or dim % groups != 0:
+            raise ValueError(f"{name} group dimension must divide D.")
+        if p.shape[2] != nstate:
+            raise ValueError(f"{name} must have matching state dimension.")
+        return PROJ_BGNL, groups
+    if p.dim() == 2:
+        if tuple(p.shape) != (dim, nstate):
+            raise ValueError(f"{name} must have shape (D, N).")
+        return PROJ_DN, 1
+    if p.dim() == 3:
+        if tuple(p.shape) != (batch, dim, nstate):
+            raise ValueError(f"{name} must have shape (B, D, N) when 3-D.")
+        return PROJ_BDN, 1
+    if p.dim() == 4:
+        # the reference broadcasts through its scan helper with L == 1
+        if p.shape[0] != batch or p.shape[-1] != 1:
+            raise ValueError(f"{name} must have shape (B, G, N, L) when 4-D.")
+        groups = int(p.shape[1])
+        if groups == 0 or dim % groups != 0:
+            raise ValueError("Group dimension must divide D.")
+        if p.shape[2] != nstate:
+            raise ValueError(f"{name} has mismatched state dimension.")
+        return PROJ_BGNL, groups
+    raise ValueError(f"Unsupported rank for {name}.")
+
+
+def check_state_step(state, x, dt, A, B, C, D, z, dt_bias):
+    """Shape contract of ``selective_state_step`` (reference.py:231-291)."""
+    if state.ndim != 3:
+        raise ValueError("state must have shape (B, D, N).")
+    if x.ndim != 2 or dt.ndim != 2:
+        raise ValueError("x and dt must have shape (B, D).")
+    batch, dim, nstate = (int(s) for s in state.shape)
+    if tuple(x.shape) != (batch, dim) or tuple(dt.shape) != (batch, dim):
+        raise ValueError("x and dt must match the first two dimensions of state.")
+    if tuple(A.shape) != (dim, nstate):
+        raise ValueError("A must have shape (D, N).")
+    bk = step_projection_kind("B", B, batch, dim, nstate)
+    ck = step_projection_kind("C", C, batch, dim, nstate)
+    if D is not None and tuple(D.shape) != (dim,):
+        raise ValueError("D must have shape (D,).")
+    if z is not None and tuple(z.shape) != (batch, dim):
+        raise ValueError("z must have shape (B, D).")
+    if dt_bias is not None and tuple(dt_bias.shape) != (dim,):
+        raise ValueError("dt_bias must have shape (D,).")
+    for name, t in (("state", state), ("x", x), ("dt", dt), ("A", A), ("B", B), ("C", C), ("D", D),
+                    ("z", z), ("dt_bias", dt_bias)):
+        if t is not None:
+            check_float(name, t)
+    if batch == 0 or dim == 0 or nstate == 0:
+        raise ValueError("selective_state_step needs non-empty B, D and N.")
+    return batch, dim, nstate, bk, ck
+
+
+# ------------------------------------------------------------ depthwise conv
+
+def check_conv(x, weight, bias, activation):
+    """Layout detection and shape contract of ``dw_causal_conv``
+    (reference.py:483-533): channels-first is tested first."""
+    if x.ndim != 3:
+        raise ValueError("x must have shape (B, C, L) or (B, L, C).")
+    chans = int(weight.shape[0]) if weight.ndim >= 1 else -1
+    if x.shape[1] == chans:
+        channels_first = True
+    elif x.shape[2] == chans:
+        channels_first = False
+    else:
+        raise ValueError("weight channel dimension must match x.")
+    if weight.ndim == 2:
+        width = int(weight.shape[1])
+    elif weight.ndim == 3:
+        if weight.shape[1] != 1:
+            raise ValueError("Expected depthwise weights with shape (C, 1, K).")
+        width = int(weight.shape[2])
+    else:
+        raise ValueError("weight must have 2 or 3 dimensions.")
+    if bias is not None and tuple(bias.shape) != (chans,):
+        raise ValueError("bias must have shape (C,).")
+    act = str(activation).lower()
+    if act in ("silu", "swish"):
+        silu = True
+    elif act in ("identity", "none"):
+        silu = False
+    else:
+        raise ValueError(f"Unsupported activation '{activation}'.")
+    for name, t in (("x", x), ("weight", weight), ("bias", bias)):
+        if t is not None:
+            check_float(name, t)
+    if channels_first:
+        batch, _, length = (int(s) for s in x.shape)
+    else:
+        batch, length, _ = (int(s) for s in x.shape)
+    if batch == 0 or chans == 0 or length == 0 or width == 0:
+        raise ValueError("dw_causal_conv needs non-empty B, C, L and K.")
+    return batch, chans, length, width, channels_first, silu
+
+
+# ----------------------------------------------------------------- layer norm
+
+def check_norm(x, weight, bias, residual):
+    """Shape contract of ``fused_layer_norm`` (reference.py:565-572)."""
+    if x.ndim != 3:
+        raise ValueError("x must have shape (B, L, D).")
+    hidden = int(x.shape[-1])
+    if tuple(weight.shape) != (hidden,):
+        raise ValueError("weight must match the last dimension of x.")
+    if bias is not None and tuple(bias.shape) != (hidden,):
+        raise ValueError("bias must match the last dimension of x.")
+    if residual is not None and tuple(residual.shape) != tuple(x.shape):
+        raise ValueError("residual must match the shape of x.")
+    for name, t in (("x", x), ("weight", weight), ("bias", bias), ("residual", residual)):
+        if t is not None:
+            check_float(name, t)
+    rows = int(x.shape[0]) * int(x.shape[1])
+    if rows == 0 or hidden == 0:
+        raise ValueError("fused_layer_norm needs a non-empty input.")
+    return rows, hidden

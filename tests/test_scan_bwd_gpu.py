@@ -1,0 +1,201 @@
+"""GPU parity of the selective-scan backward pass: gradients from the HIP
+kernels against autograd through the CPU oracle (fp32 and fp64) and against
+the upstream-CUDA gradient vectors."""
+
+import pytest
+import torch
+
+from oracle import ops_oracle as O
+from tests import fixtures as fx
+from tests.test_scan_fwd_gpu import make_inputs
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("u", "delta", "A", "B", "C", "D", "z", "dt_bias")
+
+
+def _ops():
+    from ssm_amd import ops
+    return ops
+
+
+def grads_both(inp, softplus=True, with_last=False, acc=None, seed=5):
+    g = torch.Generator().manual_seed(seed)
+    go = torch.randn(inp["u"].shape, generator=g).to(inp["u"].dtype)
+    gl = torch.randn(inp["u"].shape[0], inp["u"].shape[1], inp["A"].shape[1], generator=g).to(inp["u"].dtype)
+    res = []
+    for where in ("gpu", "cpu"):
+        leaves = {}
+        for k in NAMES:
+            v = inp[k]
+            if v is None:
+                leaves[k] = None
+                continue
+            v = v.clone()
+            if where == "gpu":
+                v = v.cuda()
+            leaves[k] = v.requires_grad_(True)
+        kw = dict(D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"], softplus=softplus,
+                  return_last_state=with_last)
+        if where == "gpu":
+            out = _ops().selective_scan(leaves["u"], leaves["delta"], leaves["A"], leaves["B"], leaves["C"], **kw)
+        else:
+            out = O.selective_scan(leaves["u"], leaves["delta"], leaves["A"], leaves["B"], leaves["C"], acc=acc, **kw)
+        dev = "cuda" if where == "gpu" else "cpu"
+        if with_last:
+            y, last = out
+            loss = (y.float() * go.to(dev).float()).sum() + (last.float() * gl.to(dev).float()).sum()
+        else:
+            loss = (out.float() * go.to(dev).float()).sum()
+        loss.backward()
+        res.append({k: (leaves[k].grad.detach().cpu() if leaves[k] is not None else None) for k in NAMES})
+    return res
+
+
+def compare(got, want, rtol, atol, scale_atol=True):
+    for k in NAMES:
+        if want[k] is None:
+            assert got[k] is None
+            continue
+        w = want[k].float()
+        a = atol * max(1.0, float(w.abs().max())) if scale_atol else atol
+        torch.testing.assert_close(got[k].float(), w, rtol=rtol, atol=a, msg=lambda m, k=k: f"grad {k}: {m}")
+
+
+@pytest.mark.parametrize("case,softplus", [("full", True), ("minimal", False), ("time_varying_3d", True)])
+def test_upstream_gradient_vectors(case, softplus):
+    rec = fx.upstream("selective_scan", case)
+    i = rec["inputs"]
+    Bm, Cm = i["B"], i["C"]
+    if case == "time_varying_3d":
+        Bm, Cm = Bm[:, None].contiguous(), Cm[:, None].contiguous()
+    leaves = dict(u=i["u"], delta=i["delta"], A=i["A"], B=Bm, C=Cm, D=i.get("D"), z=i.get("z"),
+                  dt_bias=i.get("delta_bias"))
+    leaves = {k: (v.clone().cuda().requires_grad_(True) if v is not None else None) for k, v in leaves.items()}
+    y = _ops().selective_scan(leaves["u"], leaves["delta"], leaves["A"], leaves["B"], leaves["C"], D=leaves["D"],
+                              z=leaves["z"], dt_bias=leaves["dt_bias"], softplus=softplus)
+    y.sum().backward()
+    for name, gref in rec["gradients"].items():
+        if gref is None:
+            continue
+        key = "dt_bias" if name == "delta_bias" else name
+        got = leaves[key].grad.cpu()
+        if case == "time_varying_3d" and name in ("B", "C"):
+            got = got[:, 0]
+        ok = torch.isfinite(gref)
+        if ok.any():
+            torch.testing.assert_close(got[ok], gref[ok], rtol=2e-4, atol=2e-5)
+
+
+SHAPES = [(1, 1, 1, 1), (2, 3, 5, 4), (2, 8, 64, 16), (1, 4, 65, 3), (3, 6, 513, 16), (2, 32, 1024, 16),
+          (1, 8, 1500, 7), (2, 4, 300, 40)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("kinds", [("bgnl", "bgnl"), ("dn", "dn"), ("bdn", "bgnl"), ("bgnl", "dn")])
+def test_fp32_gradients_match_oracle(shape, kinds):
+    b, d, l, n = shape
+    inp = make_inputs(sum(shape), b, d, l, n, bkind=kinds[0], ckind=kinds[1])
+    got, want = grads_both(inp)
+    compare(got, want, rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("groups,dim", [(1, 8), (2, 8), (8, 8), (3, 6), (2, 96)])
+def test_groups(groups, dim):
+    inp = make_inputs(4, 2, dim, 200, 16, groups=groups)
+    got, want = grads_both(inp)
+    compare(got, want, rtol=1e-4, atol=2e-5)
+
+
+def test_gradient_of_last_state():
+    inp = make_inputs(6, 2, 8, 700, 16)
+    got, want = grads_both(inp, with_last=True)
+    compare(got, want, rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("use_D,use_z,use_bias,softplus", [(False, False, False, False), (True, False, True, True),
+                                                           (False, True, False, True)])
+def test_optional_arguments(use_D, use_z, use_bias, softplus):
+    inp = make_inputs(3, 2, 4, 130, 8, use_D=use_D, use_z=use_z, use_bias=use_bias)
+    if not softplus:
+        inp["delta"] = inp["delta"].abs() * 0.1
+    got, want = grads_both(inp, softplus=softplus)
+    compare(got, want, rtol=1e-4, atol=2e-5)
+
+
+def test_only_requested_inputs_get_gradients():
+    inp = make_inputs(2, 1, 4, 40, 4)
+    g = {k: (v.cuda() if v is not None else None) for k, v in inp.items()}
+    g["u"].requires_grad_(True); g["A"].requires_grad_(True)
+    y = _ops().selective_scan(g["u"], g["delta"], g["A"], g["B"], g["C"], D=g["D"], z=g["z"],
+                              dt_bias=g["dt_bias"], softplus=True)
+    y.sum().backward()
+    assert g["u"].grad is not None and g["A"].grad is not None
+    assert g["delta"].grad is None and g["B"].grad is None and g["z"].grad is None
+
+
+def test_against_float64_oracle_and_bitwise_determinism():
+    inp = make_inputs(9, 2, 16, 1024, 16)
+    got, want64 = grads_both(inp, acc=torch.float64)
+    compare(got, want64, rtol=2e-4, atol=2e-5)
+    again, _ = grads_both(inp, acc=torch.float64)
+    for k in NAMES:
+        assert torch.equal(got[k], again[k]), k
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_half_inputs(dtype):
+    inp = make_inputs(8, 2, 16, 600, 16, dtype=dtype)
+    got, want = grads_both(inp)
+    for k in ("u", "delta", "z", "B", "C"):
+        assert got[k].dtype == dtype
+    for k in ("A", "D", "dt_bias"):
+        assert got[k].dtype == torch.float32
+    # the oracle differentiates the same bf16-rounded inputs in fp32; outputs are rounded once
+    compare(got, want, rtol=3e-2, atol=3e-2)
+
+
+def test_config1_shape_bf16_slice():
+    """B=8, D=1536, L=2048, N=16, bf16, G=1: full-size backward on the GPU.  du, ddelta
+    and the parameter gradients of a channel slice are compared with the oracle run on
+    that slice; dB/dC (sums over all 1536 channels) are checked through linearity: the
+    gradient of the full problem equals the sum of the gradients of two channel halves."""
+    ops = _ops()
+    inp = make_inputs(1, 8, 1536, 2048, 16, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(11)
+    go = torch.randn(8, 1536, 2048, generator=g).to(torch.bfloat16)
+
+    def run(sl):
+        lv = {}
+        for k in NAMES:
+            v = inp[k]
+            if k in ("u", "delta", "z"):
+                v = v[:, sl]
+            elif k in ("A", "D", "dt_bias"):
+                v = v[sl]
+            lv[k] = v.contiguous().cuda().requires_grad_(True)
+        y = ops.selective_scan(lv["u"], lv["delta"], lv["A"], lv["B"], lv["C"], D=lv["D"], z=lv["z"],
+                               dt_bias=lv["dt_bias"], softplus=True)
+        y.backward(go[:, sl].contiguous().cuda())
+        return {k: lv[k].grad for k in NAMES}
+
+    full = run(slice(0, 1536))
+    lo, hi = run(slice(0, 768)), run(slice(768, 1536))
+    for k in ("B", "C"):
+        s = lo[k].float() + hi[k].float()
+        torch.testing.assert_close(full[k].float(), s, rtol=2e-2, atol=2e-2 * float(s.abs().max()))
+    torch.testing.assert_close(full["u"][:, :768].float(), lo["u"].float(), rtol=0, atol=0)
+    # slice of 8 channels against the oracle
+    idx = torch.arange(0, 1536, 192)
+    sub = {k: (inp[k][:, idx] if k in ("u", "delta", "z") else inp[k][idx] if k in ("A", "D", "dt_bias") else inp[k])
+           for k in NAMES}
+    lv = {k: v.clone().requires_grad_(True) for k, v in sub.items()}
+    y = O.selective_scan(lv["u"], lv["delta"], lv["A"], lv["B"], lv["C"], D=lv["D"], z=lv["z"],
+                         dt_bias=lv["dt_bias"], softplus=True)
+    y.backward(go[:, idx])
+    for k in ("u", "delta", "z"):
+        w = lv[k].grad.float()
+        torch.testing.assert_close(full[k][:, idx.cuda()].float().cpu(), w, rtol=3e-2, atol=3e-2 * float(w.abs().max()))
+    for k in ("A", "D", "dt_bias"):
+        w = lv[k].grad.float()
+        torch.testing.assert_close(full[k][idx.cuda()].float().cpu(), w, rtol=3e-2, atol=3e-2 * float(w.abs().max()))

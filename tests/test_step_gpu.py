@@ -1,0 +1,168 @@
+"""GPU parity of ``selective_state_step`` against the CPU oracle and the
+upstream ``selective_state_update`` vectors."""
+
+import pytest
+import torch
+
+from oracle import ops_oracle as O
+from tests import fixtures as fx
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = dict(rtol=1e-5, atol=1e-5)
+HALF_TOL = dict(rtol=2e-2, atol=2e-3)
+
+
+def dev(t):
+    return None if t is None else t.cuda()
+
+
+def _ops():
+    from ssm_amd import ops
+    return ops
+
+
+def make(seed, batch, dim, nstate, io=torch.float32, st=torch.float32, bkind="bgn", ckind="bgn", groups=1,
+         use_D=True, use_z=True, use_bias=True):
+    g = torch.Generator().manual_seed(seed)
+    state = torch.randn(batch, dim, nstate, generator=g).to(st)
+    x = torch.randn(batch, dim, generator=g).to(io)
+    dt = torch.randn(batch, dim, generator=g).to(io)
+    z = torch.randn(batch, dim, generator=g).to(io) if use_z else None
+    A = -torch.arange(1, nstate + 1, dtype=torch.float32).repeat(dim, 1) * (1 + 0.1 * torch.rand(dim, nstate, generator=g))
+
+    def proj(kind):
+        if kind == "dn":
+            return torch.randn(dim, nstate, generator=g).to(io)
+        if kind == "bdn":
+            return torch.randn(batch, dim, nstate, generator=g).to(io)
+        return torch.randn(batch, groups, nstate, generator=g).to(io)
+
+    Bm, Cm = proj(bkind), proj(ckind)
+    D = torch.randn(dim, generator=g) if use_D else None
+    bias = torch.randn(dim, generator=g) - 3.0 if use_bias else None
+    return dict(state=state, x=x, dt=dt, A=A, B=Bm, C=Cm, D=D, z=z, dt_bias=bias)
+
+
+def run_both(inp, softplus=True):
+    st_ref = inp["state"].clone()
+    y_ref = O.selective_state_step(st_ref, inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"],
+                                   z=inp["z"], dt_bias=inp["dt_bias"], softplus=softplus)
+    st = dev(inp["state"].clone())
+    y = _ops().selective_state_step(st, dev(inp["x"]), dev(inp["dt"]), dev(inp["A"]), dev(inp["B"]),
+                                    dev(inp["C"]), D=dev(inp["D"]), z=dev(inp["z"]),
+                                    dt_bias=dev(inp["dt_bias"]), softplus=softplus)
+    return (y.cpu(), st.cpu()), (y_ref, st_ref)
+
+
+def test_upstream_baseline_vector():
+    rec = fx.upstream("selective_state_update", "baseline_full")
+    i = rec["inputs"]
+    st = dev(i["state"].clone())
+    y = _ops().selective_state_step(st, dev(i["x"]), dev(i["dt"]), dev(i["A"]), dev(i["B"][:, None].contiguous()),
+                                    dev(i["C"][:, None].contiguous()), D=dev(i["D"]), z=dev(i["z"]),
+                                    dt_bias=dev(i["dt_bias"]), softplus=True)
+    torch.testing.assert_close(y.cpu(), rec["outputs"]["y"], rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(st.cpu(), rec["outputs"]["updated_state"], rtol=1e-4, atol=1e-5)
+
+
+def test_upstream_grouped_heads_vector():
+    rec = fx.upstream("selective_state_update", "grouped")
+    i = rec["inputs"]
+    b, h, d, n = i["state"].shape
+    st = dev(i["state"].reshape(b, h * d, n).clone())
+    y = _ops().selective_state_step(st, dev(i["x"].reshape(b, h * d)), dev(i["dt"].reshape(b, h * d)),
+                                    dev(i["A"].reshape(h * d, n)), dev(i["B"]), dev(i["C"]),
+                                    dt_bias=dev(i["dt_bias"].reshape(h * d)), softplus=False)
+    torch.testing.assert_close(y.cpu().reshape(b, h, d), rec["outputs"]["y"], rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(st.cpu().reshape(b, h, d, n), rec["outputs"]["updated_state"], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (2, 3, 4), (4, 512, 16), (3, 40, 17), (2, 64, 64), (2, 8, 256), (5, 7, 6)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("kinds", [("bgn", "bgn"), ("dn", "dn"), ("bdn", "bgn"), ("bgn", "dn")])
+def test_fp32_matches_oracle(shape, kinds):
+    b, d, n = shape
+    inp = make(sum(shape), b, d, n, bkind=kinds[0], ckind=kinds[1])
+    (y, st), (yr, sr) = run_both(inp)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+    torch.testing.assert_close(st, sr, **FP32_TOL)
+
+
+@pytest.mark.parametrize("groups,dim", [(1, 8), (2, 8), (4, 8), (3, 6)])
+def test_groups(groups, dim):
+    inp = make(3, 3, dim, 16, groups=groups)
+    (y, st), (yr, sr) = run_both(inp)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+    torch.testing.assert_close(st, sr, **FP32_TOL)
+
+
+@pytest.mark.parametrize("io,st", [(torch.bfloat16, torch.float32), (torch.float16, torch.float32),
+                                   (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16)])
+def test_half_activations(io, st):
+    inp = make(5, 4, 96, 16, io=io, st=st)
+    (y, s), (yr, sr) = run_both(inp)
+    assert y.dtype == io and s.dtype == st
+    torch.testing.assert_close(y.float(), yr.float(), **HALF_TOL)
+    tol = FP32_TOL if st == torch.float32 else HALF_TOL
+    torch.testing.assert_close(s.float(), sr.float(), **tol)
+
+
+@pytest.mark.parametrize("use_D,use_z,use_bias,softplus", [(False, False, False, False), (True, False, True, True),
+                                                           (False, True, False, True)])
+def test_optional_arguments(use_D, use_z, use_bias, softplus):
+    inp = make(8, 2, 24, 8, use_D=use_D, use_z=use_z, use_bias=use_bias)
+    if not softplus:
+        inp["dt"] = inp["dt"].abs() * 0.1
+    (y, st), (yr, sr) = run_both(inp, softplus=softplus)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+    torch.testing.assert_close(st, sr, **FP32_TOL)
+
+
+def test_repeated_steps_equal_scan_last_state():
+    """L steps from a zero state reproduce selective_scan and its last_state."""
+    from tests.test_scan_fwd_gpu import make_inputs
+    ops = _ops()
+    inp = make_inputs(21, 2, 16, 33, 16)
+    g = {k: dev(v) for k, v in inp.items()}
+    y, h = ops.selective_scan(g["u"], g["delta"], g["A"], g["B"], g["C"], D=g["D"], z=g["z"],
+                              dt_bias=g["dt_bias"], softplus=True, return_last_state=True)
+    st = torch.zeros(2, 16, 16, device="cuda")
+    for t in range(33):
+        yt = ops.selective_state_step(st, g["u"][:, :, t].contiguous(), g["delta"][:, :, t].contiguous(), g["A"],
+                                      g["B"][..., t].contiguous(), g["C"][..., t].contiguous(), D=g["D"],
+                                      z=g["z"][:, :, t].contiguous(), dt_bias=g["dt_bias"], softplus=True)
+        torch.testing.assert_close(yt, y[:, :, t], **FP32_TOL)
+    torch.testing.assert_close(st, h, **FP32_TOL)
+
+
+def test_config2_shape_512_steps():
+    """BASELINE config 2: B=64, D=5120, N=16, bf16 activations, fp32 state, grouped
+    B/C (64,1,16).  512 in-place steps on the GPU; a channel slice is replayed on the
+    CPU oracle (a linear slice is exact because channels are independent)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(2)
+    Bsz, D, N, steps = 64, 5120, 16, 512
+    state = torch.randn(Bsz, D, N, generator=g)
+    A = -torch.arange(1, N + 1, dtype=torch.float32).repeat(D, 1)
+    Dk = torch.ones(D)
+    from ssm_amd.configs import inverse_softplus_dt
+    bias = inverse_softplus_dt(D, g)
+    idx = torch.arange(0, D, 640)
+    st_gpu = state.cuda()
+    st_ref = state[:, idx].clone()
+    A_g, D_g, b_g = A.cuda(), Dk.cuda(), bias.cuda()
+    check_at = {0, 1, 17, 255, 511}
+    for s in range(steps):
+        x = torch.randn(Bsz, D, generator=g).to(torch.bfloat16)
+        z = torch.randn(Bsz, D, generator=g).to(torch.bfloat16)
+        dt = torch.randn(Bsz, D, generator=g).to(torch.bfloat16)
+        Bm = torch.randn(Bsz, 1, N, generator=g).to(torch.bfloat16)
+        Cm = torch.randn(Bsz, 1, N, generator=g).to(torch.bfloat16)
+        y = ops.selective_state_step(st_gpu, x.cuda(), dt.cuda(), A_g, Bm.cuda(), Cm.cuda(), D=D_g, z=z.cuda(),
+                                     dt_bias=b_g, softplus=True)
+        yr = O.selective_state_step(st_ref, x[:, idx], dt[:, idx], A[idx], Bm, Cm, D=Dk[idx], z=z[:, idx],
+                                    dt_bias=bias[idx], softplus=True)
+        if s in check_at:
+            torch.testing.assert_close(y[:, idx.cuda()].float().cpu(), yr.float(), **HALF_TOL)
+    torch.testing.assert_close(st_gpu[:, idx.cuda()].cpu(), st_ref, rtol=1e-4, atol=1e-4)
