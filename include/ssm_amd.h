@@ -151,6 +151,40 @@ typedef struct ssm_state_step_args {
 int ssm_state_step(const ssm_state_step_args *args, void *hip_stream);
 
 /* ------------------------------------------------------------------------
+ * diagonal chunk scan: the operator the reference calls `ssd_chunk_scan`
+ * (an element-wise recurrence per (batch, head, p); chunking does not change
+ * the result).  Stands behind `ssd_chunk_scan(X, dt, A, B, C, chunk_size, D,
+ * z, seq_lens, cu_seqlens, initial_states)` as invoked at
+ * src/ssm/ops/__init__.py:1516-1531 (semantics: reference.py:312-463).
+ * ---------------------------------------------------------------------- */
+typedef enum ssm_chunk_kind {
+  SSM_CHUNK_HP = 0,    /* (H, P) */
+  SSM_CHUNK_BHP = 1,   /* (B, H, P) */
+  SSM_CHUNK_BLHP = 2   /* (B, L, H, P) */
+} ssm_chunk_kind;
+
+typedef struct ssm_dscan_fwd_args {
+  const void *X;              /* (B, L, H, P) x dtype */
+  const void *dt;             /* (B, L, H) dt dtype; used as given */
+  const float *A;             /* (H, P) if a_per_p else (H,) */
+  const void *Bproj, *Cproj;  /* see b_kind / c_kind, bc dtype */
+  const float *Dskip;         /* (H, P) if d_per_p else (H,), or NULL */
+  const void *z;              /* (B, L, H, P) if z_per_p else (B, L, H), z dtype, or NULL */
+  const void *initial_states; /* (B, H, P) init dtype, or NULL */
+  const int32_t *seq_lens;    /* (B,) valid steps per batch row (device memory), or NULL */
+  void *Y;                    /* (B, L, H, P) x dtype; rows at or beyond seq_lens[b] are zero */
+  void *workspace;            /* ssm_dscan_fwd_workspace_bytes() bytes */
+  size_t workspace_bytes;
+  int32_t batch, seqlen, heads, proj;
+  int32_t x_dtype, dt_dtype, bc_dtype, z_dtype, init_dtype;
+  int32_t b_kind, c_kind;     /* ssm_chunk_kind */
+  int32_t a_per_p, d_per_p, z_per_p;
+} ssm_dscan_fwd_args;
+
+size_t ssm_dscan_fwd_workspace_bytes(int batch, int seqlen, int heads, int proj);
+int ssm_dscan_fwd(const ssm_dscan_fwd_args *args, void *hip_stream);
+
+/* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).
  * Forward stands behind `dw_causal_conv(x, weight, bias, activation)`
  * (src/ssm/ops/__init__.py:1594-1600; semantics reference.py:466-537);

@@ -70,6 +70,20 @@ class StateStepArgs(C.Structure):
     ]
 
 
+CHUNK_HP, CHUNK_BHP, CHUNK_BLHP = 0, 1, 2
+
+
+class DscanFwdArgs(C.Structure):
+    _fields_ = [
+        ("X", _vp), ("dt", _vp), ("A", _vp), ("Bproj", _vp), ("Cproj", _vp), ("Dskip", _vp), ("z", _vp),
+        ("initial_states", _vp), ("seq_lens", _vp), ("Y", _vp), ("workspace", _vp),
+        ("workspace_bytes", C.c_size_t),
+        ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("proj", _i32),
+        ("x_dtype", _i32), ("dt_dtype", _i32), ("bc_dtype", _i32), ("z_dtype", _i32), ("init_dtype", _i32),
+        ("b_kind", _i32), ("c_kind", _i32), ("a_per_p", _i32), ("d_per_p", _i32), ("z_per_p", _i32),
+    ]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -116,6 +130,7 @@ ENTRY_POINTS = {
     "ssm_scan_fwd": ScanFwdArgs,
     "ssm_scan_bwd": ScanBwdArgs,
     "ssm_state_step": StateStepArgs,
+    "ssm_dscan_fwd": DscanFwdArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_norm_fwd": NormFwdArgs,
@@ -128,6 +143,7 @@ PLAIN_SYMBOLS = {
     "ssm_amd_last_error": (C.c_char_p, []),
     "ssm_scan_chunk_len": (C.c_int, []),
     "ssm_scan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 8),
+    "ssm_dscan_fwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ssm_conv1d_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "ssm_norm_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
 }

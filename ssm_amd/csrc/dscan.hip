@@ -1,0 +1,163 @@
+// Diagonal chunked scan: the operator the reference exposes as `ssd_chunk_scan`.
+//
+//   s_t = exp(dt_t A) s_{t-1} + dt_t B_t X_t        per (batch, head, p) channel
+//   y_t = s_t C_t + D X_t ;  y_t *= silu(z_t) ;  y_t = 0 for t >= len(batch)
+//
+// Tensors are channels-last, (B, L, H, P): consecutive lanes take consecutive
+// channels so every time step is one coalesced access.  Time is cut into
+// segments that run in parallel:
+//   pass 1  every (segment, channel) folds its steps into (decay product, local state)
+//   pass 2  every (segment, channel) rebuilds the state entering it from the folds of
+//           the segments before it, then replays its steps and emits y
+// which costs one extra read of X/dt/B but fills the device even when B*H*P is
+// small.  dt is used as given (no bias, no softplus), as in the reference.
+#include "common.hpp"
+
+namespace ssm {
+
+constexpr int DS_THREADS = 256;
+
+struct DscanParams {
+  const void *X, *dt, *Bp, *Cp, *z, *init;
+  const float *A, *Dk;
+  const int *lengths;           // (B,) valid steps per batch row, or null
+  void *Y;
+  float *fold;                  // (B, nseg, H*P, 2): decay product, local state
+  int batch, len, heads, proj;
+  int x_dtype, dt_dtype, bc_dtype, z_dtype, init_dtype;
+  int a_stride_p;               // 1 for A (H,P), 0 for A (H,)
+  int d_stride_p;               // 1 for D (H,P), 0 for D (H,)
+  long long b_stride_b, b_stride_t, c_stride_b, c_stride_t;   // element strides of B / C (0 = broadcast)
+  int z_per_p;                  // 1 for z (B,L,H,P), 0 for z (B,L,H)
+  int seg_len, nseg;
+};
+
+__device__ __forceinline__ void ds_store(void *p, int dtype, size_t i, float v) {
+  if (dtype == SSM_F32) reinterpret_cast<float *>(p)[i] = v;
+  else if (dtype == SSM_BF16) reinterpret_cast<bf16_t *>(p)[i] = from_f32<bf16_t>(v);
+  else reinterpret_cast<f16_t *>(p)[i] = from_f32<f16_t>(v);
+}
+
+template <int PASS>
+__global__ __launch_bounds__(DS_THREADS) void dscan_kernel(const DscanParams p) {
+  const int HP = p.heads * p.proj;
+  const int hp = blockIdx.x * DS_THREADS + threadIdx.x;
+  if (hp >= HP) return;
+  const int seg = blockIdx.y, b = blockIdx.z;
+  const int h = hp / p.proj, pp = hp % p.proj;
+  const int valid = p.lengths ? min(max(p.lengths[b], 0), p.len) : p.len;
+  const int t_begin = seg * p.seg_len;
+  const int t_end = min(p.len, t_begin + p.seg_len);
+  const float A2 = p.A[(size_t)h * (p.a_stride_p ? p.proj : 1) + (p.a_stride_p ? pp : 0)] * LOG2E;
+  const size_t x_row = (size_t)b * p.len;            // + t, then * HP + hp
+  const size_t fold_at = (((size_t)b * p.nseg + seg) * HP + hp) * 2;
+
+  if (PASS == 1) {
+    float prod = 1.0f, s = 0.0f;
+    const int stop = min(t_end, valid);
+    for (int t = t_begin; t < stop; ++t) {
+      const float dtv = load_as_f32(p.dt, p.dt_dtype, (x_row + t) * p.heads + h);
+      const float xv = load_as_f32(p.X, p.x_dtype, (x_row + t) * HP + hp);
+      const float bv = load_as_f32(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
+      const float a = exp2_hw(dtv * A2);
+      s = __builtin_fmaf(a, s, dtv * bv * xv);
+      prod *= a;
+    }
+    p.fold[fold_at] = prod;
+    p.fold[fold_at + 1] = s;
+    return;
+  }
+
+  // PASS 2: state entering this segment
+  float s = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + hp) : 0.0f;
+  for (int j = 0; j < seg; ++j) {
+    const size_t f = (((size_t)b * p.nseg + j) * HP + hp) * 2;
+    s = __builtin_fmaf(p.fold[f], s, p.fold[f + 1]);
+  }
+  const float Dk = p.Dk ? p.Dk[(size_t)h * (p.d_stride_p ? p.proj : 1) + (p.d_stride_p ? pp : 0)] : 0.0f;
+  for (int t = t_begin; t < t_end; ++t) {
+    const size_t xi = (x_row + t) * HP + hp;
+    float y = 0.0f;
+    if (t < valid) {
+      const float dtv = load_as_f32(p.dt, p.dt_dtype, (x_row + t) * p.heads + h);
+      const float xv = load_as_f32(p.X, p.x_dtype, xi);
+      const float bv = load_as_f32(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
+      const float cv = load_as_f32(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
+      s = __builtin_fmaf(exp2_hw(dtv * A2), s, dtv * bv * xv);
+      y = __builtin_fmaf(s, cv, Dk * xv);
+      if (p.z) {
+        const size_t zi = p.z_per_p ? xi : (x_row + t) * p.heads + h;
+        y *= silu_f32(load_as_f32(p.z, p.z_dtype, zi));
+      }
+    }
+    ds_store(p.Y, p.x_dtype, xi, y);
+  }
+}
+
+static int dscan_segments(int batch, int len, int hp) {
+  // enough (segment, channel-block) workgroups to cover ~4 per CU, segments of >= 32 steps
+  const int blocks = (hp + DS_THREADS - 1) / DS_THREADS;
+  int want = (1024 + batch * blocks - 1) / (batch * blocks);
+  const int max_seg = (len + 31) / 32;
+  if (want > max_seg) want = max_seg;
+  if (want < 1) want = 1;
+  return want;
+}
+
+}  // namespace ssm
+
+extern "C" size_t ssm_dscan_fwd_workspace_bytes(int batch, int seqlen, int heads, int proj) {
+  if (batch <= 0 || seqlen <= 0 || heads <= 0 || proj <= 0) return 0;
+  const int nseg = ssm::dscan_segments(batch, seqlen, heads * proj);
+  return (size_t)batch * nseg * heads * proj * 2 * sizeof(float);
+}
+
+extern "C" int ssm_dscan_fwd(const ssm_dscan_fwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_dscan_fwd: args is NULL");
+  SSM_REQUIRE(a->X && a->dt && a->A && a->Bproj && a->Cproj && a->Y, SSM_ERR_NULL_POINTER,
+              "ssm_dscan_fwd: X, dt, A, Bproj, Cproj and Y are required");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->proj > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_dscan_fwd: batch=%d seqlen=%d heads=%d proj=%d must all be positive", a->batch, a->seqlen,
+              a->heads, a->proj);
+  SSM_REQUIRE(valid_dtype(a->x_dtype) && valid_dtype(a->dt_dtype) && valid_dtype(a->bc_dtype) &&
+                  (!a->z || valid_dtype(a->z_dtype)) && (!a->initial_states || valid_dtype(a->init_dtype)),
+              SSM_ERR_BAD_DTYPE, "ssm_dscan_fwd: unsupported dtype");
+  SSM_REQUIRE(a->batch < 65536, SSM_ERR_TOO_LARGE, "ssm_dscan_fwd: batch too large");
+  SSM_REQUIRE((size_t)a->batch * a->seqlen * a->heads * a->proj < ((size_t)1 << 40), SSM_ERR_TOO_LARGE,
+              "ssm_dscan_fwd: tensor too large");
+  auto kind_ok = [](int k) { return k == SSM_CHUNK_HP || k == SSM_CHUNK_BHP || k == SSM_CHUNK_BLHP; };
+  SSM_REQUIRE(kind_ok(a->b_kind) && kind_ok(a->c_kind), SSM_ERR_BAD_KIND, "ssm_dscan_fwd: b_kind=%d c_kind=%d",
+              a->b_kind, a->c_kind);
+  const size_t need = ssm_dscan_fwd_workspace_bytes(a->batch, a->seqlen, a->heads, a->proj);
+  SSM_REQUIRE(a->workspace && a->workspace_bytes >= need, SSM_ERR_WORKSPACE,
+              "ssm_dscan_fwd: workspace of %zu bytes required", need);
+
+  DscanParams p{};
+  p.X = a->X; p.dt = a->dt; p.Bp = a->Bproj; p.Cp = a->Cproj; p.z = a->z; p.init = a->initial_states;
+  p.A = a->A; p.Dk = a->Dskip; p.lengths = a->seq_lens; p.Y = a->Y;
+  p.fold = reinterpret_cast<float *>(a->workspace);
+  p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.proj = a->proj;
+  p.x_dtype = a->x_dtype; p.dt_dtype = a->dt_dtype; p.bc_dtype = a->bc_dtype; p.z_dtype = a->z_dtype;
+  p.init_dtype = a->init_dtype;
+  p.a_stride_p = a->a_per_p ? 1 : 0;
+  p.d_stride_p = a->d_per_p ? 1 : 0;
+  const long long HP = (long long)a->heads * a->proj;
+  auto strides = [&](int kind, long long &sb, long long &st) {
+    sb = kind == SSM_CHUNK_HP ? 0 : (kind == SSM_CHUNK_BHP ? HP : HP * a->seqlen);
+    st = kind == SSM_CHUNK_BLHP ? HP : 0;
+  };
+  strides(a->b_kind, p.b_stride_b, p.b_stride_t);
+  strides(a->c_kind, p.c_stride_b, p.c_stride_t);
+  p.z_per_p = a->z_per_p ? 1 : 0;
+  p.nseg = dscan_segments(a->batch, a->seqlen, (int)HP);
+  p.seg_len = (a->seqlen + p.nseg - 1) / p.nseg;
+  p.nseg = (a->seqlen + p.seg_len - 1) / p.seg_len;
+
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  const dim3 grid((unsigned)((HP + DS_THREADS - 1) / DS_THREADS), (unsigned)p.nseg, (unsigned)a->batch);
+  if (p.nseg > 1) hipLaunchKernelGGL(dscan_kernel<1>, grid, dim3(DS_THREADS), 0, s, p);
+  hipLaunchKernelGGL(dscan_kernel<2>, grid, dim3(DS_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_dscan_fwd");
+  return SSM_OK;
+}

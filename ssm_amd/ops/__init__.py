@@ -298,6 +298,63 @@ def selective_state_step(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, so
 
 
 # ---------------------------------------------------------------------------
+# diagonal chunk scan (the reference's ``ssd_chunk_scan``)
+# ---------------------------------------------------------------------------
+
+def ssd_chunk_scan(X, dt, A, B, C, chunk_size, D=None, z=None, seq_meta=None, initial_states=None):
+    """Chunked diagonal state-space scan on the GPU (the reference's "SSD chunk scan").
+
+    ``s_t = exp(dt_t A) s_{t-1} + dt_t B_t X_t``, ``y_t = s_t C_t + D X_t`` per
+    ``(batch, head, p)`` channel, optionally gated by ``silu(z_t)``; ``dt`` is used
+    as given.  ``chunk_size`` is validated but does not affect the result.
+
+    Args:
+        X: Activations ``(B, L, H, P)``.
+        dt: Per-head time-steps ``(B, L, H)``.
+        A: ``(H, P)`` or ``(H,)``.
+        B: ``(H, P)``, ``(B, H, P)`` or time-varying ``(B, L, H, P)``.
+        C: Same accepted shapes as ``B``.
+        chunk_size: Positive integer.
+        D: Optional skip ``(H,)`` or ``(H, P)``.
+        z: Optional gate ``(B, L, H)`` or ``(B, L, H, P)``.
+        seq_meta: Optional dict with ``cu_seqlens`` (length ``B + 1``) or ``seq_lens``
+            (length ``B``); steps at or beyond a row's length produce zeros.
+        initial_states: Optional initial state ``(B, H, P)``.
+
+    Returns:
+        Tensor ``(B, L, H, P)`` in ``X.dtype``.
+    """
+    tensors = (X, dt, A, B, C, D, z, initial_states)
+    if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
+        raise NotImplementedError(
+            "ssd_chunk_scan has no backward kernel in this backend yet; run it under torch.no_grad().")
+    batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p = \
+        K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
+    dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states)
+    lengths = K.sequence_lengths(seq_meta, batch, dev)
+    bc = K.common_io_dtype([B, C])
+    Xc, dtc = K.cast_c(X, X.dtype), K.cast_c(dt, dt.dtype)
+    Bc, Cc = K.cast_c(B, bc), K.cast_c(C, bc)
+    zc = K.cast_c(z, z.dtype) if z is not None else None
+    ic = K.cast_c(initial_states, initial_states.dtype) if initial_states is not None else None
+    Af, Df = K.as_f32_vec(A), K.as_f32_vec(D)
+    Y = torch.empty_like(Xc)
+    nbytes = _lib.load().ssm_dscan_fwd_workspace_bytes(batch, seqlen, heads, proj)
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
+    args = _lib.DscanFwdArgs(
+        X=_lib.ptr(Xc), dt=_lib.ptr(dtc), A=_lib.ptr(Af), Bproj=_lib.ptr(Bc), Cproj=_lib.ptr(Cc),
+        Dskip=_lib.ptr(Df), z=_lib.ptr(zc), initial_states=_lib.ptr(ic), seq_lens=_lib.ptr(lengths),
+        Y=_lib.ptr(Y), workspace=_lib.ptr(ws), workspace_bytes=nbytes,
+        batch=batch, seqlen=seqlen, heads=heads, proj=proj,
+        x_dtype=_lib.dtype_enum(Xc.dtype), dt_dtype=_lib.dtype_enum(dtc.dtype), bc_dtype=_lib.dtype_enum(bc),
+        z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
+        init_dtype=_lib.dtype_enum(ic.dtype) if ic is not None else 0,
+        b_kind=bk, c_kind=ck, a_per_p=int(a_per_p), d_per_p=int(d_per_p), z_per_p=int(z_per_p))
+    _lib.call("ssm_dscan_fwd", args, dev)
+    return Y
+
+
+# ---------------------------------------------------------------------------
 # depthwise causal convolution
 # ---------------------------------------------------------------------------
 
@@ -475,6 +532,7 @@ def fused_layer_norm_with_residual(x, weight, bias, residual=None, is_rms=False,
 __all__ = [
     "selective_scan",
     "selective_state_step",
+    "ssd_chunk_scan",
     "dw_causal_conv",
     "fused_layer_norm",
     "fused_layer_norm_with_residual",

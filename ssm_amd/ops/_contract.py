@@ -249,3 +249,99 @@ def check_norm(x, weight, bias, residual):
     if rows == 0 or hidden == 0:
         raise ValueError("fused_layer_norm needs a non-empty input.")
     return rows, hidden
+
+
+# -------------------------------------------- diagonal chunk scan (ssd_chunk_scan)
+
+def chunk_projection_kind(name, p, batch, seqlen, heads, proj) -> int:
+    """-> kind of a B/C argument of ``ssd_chunk_scan`` (reference.py:59-84)."""
+    from .._lib import CHUNK_BHP, CHUNK_BLHP, CHUNK_HP
+
+    if p.dim() == 2:
+        if tuple(p.shape) != (heads, proj):
+            raise ValueError(f"{name} must have shape (H, P).")
+        return CHUNK_HP
+    if p.dim() == 3:
+        if tuple(p.shape) != (batch, heads, proj):
+            raise ValueError(f"{name} must be (B, H, P) when 3-D.")
+        return CHUNK_BHP
+    if p.dim() == 4:
+        if tuple(p.shape) != (batch, seqlen, heads, proj):
+            raise ValueError(f"{name} must have shape (B, L, H, P) when 4-D.")
+        return CHUNK_BLHP
+    raise ValueError(f"Unsupported rank for {name}.")
+
+
+def check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states):
+    """Shape contract of ``ssd_chunk_scan`` (reference.py:346-411)."""
+    if X.ndim != 4:
+        raise ValueError("X must have shape (B, L, H, P).")
+    if dt.ndim != 3:
+        raise ValueError("dt must have shape (B, L, H).")
+    batch, seqlen, heads, proj = (int(s) for s in X.shape)
+    if tuple(dt.shape) != (batch, seqlen, heads):
+        raise ValueError("dt must align with (B, L, H).")
+    if A.ndim == 1:
+        if A.shape[0] != heads:
+            raise ValueError("A must have shape (H,) when 1-D.")
+        a_per_p = False
+    elif A.ndim == 2:
+        if tuple(A.shape) != (heads, proj):
+            raise ValueError("A must have shape (H, P) when 2-D.")
+        a_per_p = True
+    else:
+        raise ValueError("A must be 1-D or 2-D.")
+    bk = chunk_projection_kind("B", B, batch, seqlen, heads, proj)
+    ck = chunk_projection_kind("C", C, batch, seqlen, heads, proj)
+    d_per_p = False
+    if D is not None:
+        if D.ndim == 1:
+            if D.shape[0] != heads:
+                raise ValueError("D must have shape (H,).")
+        elif D.ndim == 2:
+            if tuple(D.shape) != (heads, proj):
+                raise ValueError("D must have shape (H, P) when 2-D.")
+            d_per_p = True
+        else:
+            raise ValueError("Unsupported rank for D.")
+    z_per_p = False
+    if z is not None:
+        if z.ndim == 3:
+            if tuple(z.shape) != (batch, seqlen, heads):
+                raise ValueError("z must have shape (B, L, H) when 3-D.")
+        elif z.ndim == 4:
+            if tuple(z.shape) != (batch, seqlen, heads, proj):
+                raise ValueError("z must have shape (B, L, H, P) when 4-D.")
+            z_per_p = True
+        else:
+            raise ValueError("Unsupported rank for z.")
+    if initial_states is not None and tuple(initial_states.shape) != (batch, heads, proj):
+        raise ValueError("initial_states must have shape (B, H, P).")
+    if int(chunk_size) <= 0:
+        raise ValueError("chunk_size must be positive.")
+    for name, t in (("X", X), ("dt", dt), ("A", A), ("B", B), ("C", C), ("D", D), ("z", z),
+                    ("initial_states", initial_states)):
+        if t is not None:
+            check_float(name, t)
+    if batch == 0 or seqlen == 0 or heads == 0 or proj == 0:
+        raise ValueError("ssd_chunk_scan needs non-empty B, L, H and P.")
+    return batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p
+
+
+def sequence_lengths(seq_meta, batch: int, device) -> Optional[torch.Tensor]:
+    """``seq_meta`` -> int32 device tensor of valid lengths, or ``None``.
+    ``cu_seqlens`` (B+1) wins over ``seq_lens`` (B) (reference.py:413-428;
+    list/tensor handling as src/ssm/ops/__init__.py:1460-1481).  No host sync."""
+    if not seq_meta:
+        return None
+    if seq_meta.get("cu_seqlens") is not None:
+        cu = torch.as_tensor(seq_meta["cu_seqlens"]).to(device=device, dtype=torch.long).flatten()
+        if cu.numel() != batch + 1:
+            raise ValueError("cu_seqlens must have length B + 1.")
+        return (cu[1:] - cu[:-1]).to(torch.int32).contiguous()
+    if seq_meta.get("seq_lens") is not None:
+        sl = torch.as_tensor(seq_meta["seq_lens"]).to(device=device, dtype=torch.int32).flatten()
+        if sl.numel() != batch:
+            raise ValueError("seq_lens must have length B.")
+        return sl.contiguous()
+    raise ValueError("seq_meta must provide cu_seqlens or seq_lens.")

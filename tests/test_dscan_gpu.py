@@ -1,0 +1,113 @@
+"""GPU parity of the reference-semantics ``ssd_chunk_scan`` (diagonal chunk
+scan) against the CPU oracle and the reference's two JSON goldens."""
+
+import pytest
+import torch
+
+from oracle import ops_oracle as O
+from tests import fixtures as fx
+
+pytestmark = pytest.mark.gpu
+FP32_TOL = dict(rtol=1e-5, atol=1e-5)
+HALF_TOL = dict(rtol=2e-2, atol=2e-3)
+
+
+def _ops():
+    from ssm_amd import ops
+    return ops
+
+
+def dev(t):
+    return None if t is None else t.cuda()
+
+
+@pytest.mark.parametrize("name", ["ssd_chunk_scan_case1", "ssd_chunk_scan_varlen"])
+def test_reference_goldens(name):
+    i, o, _ = fx.nested_case(name)
+    raw = i.get("seq_meta") or {}
+    meta = {}
+    if raw.get("seq_lens") is not None:
+        meta["seq_lens"] = [int(v) for v in raw["seq_lens"]]
+    if raw.get("cu_seqlens") is not None:
+        meta["cu_seqlens"] = torch.tensor(raw["cu_seqlens"], dtype=torch.long)
+    y = _ops().ssd_chunk_scan(dev(i["X"]), dev(i["dt"]), dev(i["A"]), dev(i["B"]), dev(i["C"]),
+                              int(i["chunk_size"]), D=dev(i.get("D")), z=dev(i.get("z")), seq_meta=meta or None,
+                              initial_states=dev(i.get("initial_states")))
+    torch.testing.assert_close(y.cpu(), o["Y"], **FP32_TOL)
+
+
+def make(seed, b, l, h, p, dtype=torch.float32, bkind=4, ckind=4, a_vec=False, d_mode="vec", z_mode=4, init=True):
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(b, l, h, p, generator=g).to(dtype)
+    dt = (torch.rand(b, l, h, generator=g) * 0.2).to(dtype)
+    A = -(torch.rand(h, generator=g) * 4 + 0.1) if a_vec else -(torch.rand(h, p, generator=g) * 4 + 0.1)
+
+    def proj(k):
+        shape = {2: (h, p), 3: (b, h, p), 4: (b, l, h, p)}[k]
+        return torch.randn(*shape, generator=g).to(dtype)
+
+    D = {"none": None, "vec": torch.randn(h, generator=g), "mat": torch.randn(h, p, generator=g)}[d_mode]
+    z = {0: None, 3: torch.randn(b, l, h, generator=g).to(dtype), 4: torch.randn(b, l, h, p, generator=g).to(dtype)}[z_mode]
+    init_s = torch.randn(b, h, p, generator=g) if init else None
+    return dict(X=X, dt=dt, A=A, B=proj(bkind), C=proj(ckind), D=D, z=z, init=init_s)
+
+
+def both(inp, chunk=64, meta=None):
+    yr = O.ssd_chunk_scan(inp["X"], inp["dt"], inp["A"], inp["B"], inp["C"], chunk, D=inp["D"], z=inp["z"],
+                          seq_meta=meta, initial_states=inp["init"])
+    y = _ops().ssd_chunk_scan(dev(inp["X"]), dev(inp["dt"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]), chunk,
+                              D=dev(inp["D"]), z=dev(inp["z"]), seq_meta=meta, initial_states=dev(inp["init"]))
+    return y.cpu(), yr
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (2, 6, 2, 3), (2, 37, 3, 5), (1, 384, 4, 64), (2, 1000, 2, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("kinds", [(4, 4), (2, 2), (3, 4), (4, 2)])
+def test_fp32_matches_oracle(shape, kinds):
+    inp = make(sum(shape), *shape, bkind=kinds[0], ckind=kinds[1])
+    y, yr = both(inp)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+
+
+@pytest.mark.parametrize("a_vec,d_mode,z_mode,init", [(True, "none", 0, False), (True, "mat", 3, True),
+                                                      (False, "vec", 4, False), (False, "none", 3, True)])
+def test_option_matrix(a_vec, d_mode, z_mode, init):
+    inp = make(7, 2, 130, 3, 6, a_vec=a_vec, d_mode=d_mode, z_mode=z_mode, init=init)
+    y, yr = both(inp)
+    torch.testing.assert_close(y, yr, **FP32_TOL)
+
+
+def test_ragged_lengths_and_chunk_invariance():
+    inp = make(3, 3, 200, 2, 4)
+    for meta in ({"seq_lens": [200, 77, 0]}, {"cu_seqlens": torch.tensor([0, 5, 205, 300])}):
+        y, yr = both(inp, chunk=16, meta=meta)
+        torch.testing.assert_close(y, yr, **FP32_TOL)
+    y2, _ = both(inp, chunk=7, meta={"seq_lens": [200, 77, 0]})
+    y3, _ = both(inp, chunk=512, meta={"seq_lens": [200, 77, 0]})
+    assert torch.equal(y2, y3)
+    assert torch.count_nonzero(y2[1, 77:]) == 0 and torch.count_nonzero(y2[2]) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_half(dtype):
+    inp = make(5, 2, 384, 4, 64, dtype=dtype)
+    y, yr = both(inp)
+    assert y.dtype == dtype
+    torch.testing.assert_close(y.float(), yr.float(), **HALF_TOL)
+
+
+def test_config3_outer_shape_bf16_slice():
+    """(B, L, H, P) = (4, 4096, 80, 64) in bf16 with A (80,), B, C (80, 64): full size on the
+    GPU; two heads are replayed on the oracle (heads are independent)."""
+    g = torch.Generator().manual_seed(3)
+    X = torch.randn(4, 4096, 80, 64, generator=g).to(torch.bfloat16)
+    dt = torch.nn.functional.softplus(torch.randn(4, 4096, 80, generator=g) - 3).to(torch.bfloat16)
+    A = -(torch.rand(80, generator=g) * 15 + 1)
+    Bm = torch.randn(80, 64, generator=g).to(torch.bfloat16)
+    Cm = torch.randn(80, 64, generator=g).to(torch.bfloat16)
+    D = torch.ones(80)
+    z = torch.randn(4, 4096, 80, 64, generator=g).to(torch.bfloat16)
+    y = _ops().ssd_chunk_scan(X.cuda(), dt.cuda(), A.cuda(), Bm.cuda(), Cm.cuda(), 256, D=D.cuda(), z=z.cuda())
+    hs = [3, 77]
+    yr = O.ssd_chunk_scan(X[:, :, hs], dt[:, :, hs], A[hs], Bm[hs], Cm[hs], 256, D=D[hs], z=z[:, :, hs])
+    torch.testing.assert_close(y[:, :, hs].float().cpu(), yr.float(), **HALF_TOL)
