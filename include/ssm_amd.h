@@ -185,6 +185,78 @@ size_t ssm_dscan_fwd_workspace_bytes(int batch, int seqlen, int heads, int proj)
 int ssm_dscan_fwd(const ssm_dscan_fwd_args *args, void *hip_stream);
 
 /* ------------------------------------------------------------------------
+ * state-space duality (Mamba-2) operator family.  The reference has no code
+ * for these; their semantics are fixed by the vectors it ships in
+ * tests/mamba_reference_cases.json, recorded through the call sites in
+ * scripts/refresh_mamba_goldens.py:430-486 (chunk_cumsum, chunk_state,
+ * state_passing, chunk_scan), :591-604 (combined) and :680-705 (bmm_chunk).
+ * Layouts: x, z, y (B,L,H,P); dt (B,L,H); A (H,); Bm, Cm (B,L,G,N);
+ * dt_out, dA_cumsum (B,H,nc,Q) fp32; CB (B,nc,G,Q,Q); states (B,nc,H,P,N);
+ * final_states (B,H,P,N) fp32; nc = ceil(L/Q).  `force_generic` skips the
+ * bf16 MFMA kernels (used by the tests to cross-check them).
+ * ---------------------------------------------------------------------- */
+typedef struct ssm_ssd_dims {
+  int32_t batch, seqlen, heads, headdim, groups, nstate, chunk;
+} ssm_ssd_dims;
+
+typedef struct ssm_ssd_cumsum_args {
+  const void *dt;           /* (B,L,H) dt dtype */
+  const float *A;           /* (H,) */
+  const float *dt_bias;     /* (H,) or NULL */
+  float *dA_cumsum;         /* (B,H,nc,Q) */
+  float *dt_out;            /* (B,H,nc,Q) */
+  ssm_ssd_dims dims;        /* headdim, groups, nstate unused */
+  int32_t dt_dtype, dt_softplus;
+  float dt_min, dt_max;     /* clamp applied after softplus; use 0 and +inf for none */
+} ssm_ssd_cumsum_args;
+int ssm_ssd_chunk_cumsum(const ssm_ssd_cumsum_args *args, void *hip_stream);
+
+typedef struct ssm_ssd_bmm_args {
+  const void *a, *b;        /* (B,L,G,K) in dtype */
+  const int32_t *seq_idx;   /* (B,L) or NULL: entries across sequences are zeroed */
+  void *out;                /* (B,nc,G,Q,Q) out dtype: out[l][s] = <a_l, b_s> */
+  int32_t batch, seqlen, groups, kdim, chunk;
+  int32_t in_dtype, out_dtype, causal, force_generic;
+} ssm_ssd_bmm_args;
+int ssm_ssd_bmm_chunk(const ssm_ssd_bmm_args *args, void *hip_stream);
+
+typedef struct ssm_ssd_chunk_state_args {
+  const void *Bm;           /* (B,L,G,N) b dtype */
+  const void *x;            /* (B,L,H,P) x dtype */
+  const float *dt;          /* (B,H,nc,Q) */
+  const float *dA_cumsum;   /* (B,H,nc,Q) */
+  void *states;             /* (B,nc,H,P,N) states dtype */
+  ssm_ssd_dims dims;
+  int32_t x_dtype, b_dtype, states_dtype, force_generic;
+} ssm_ssd_chunk_state_args;
+int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *args, void *hip_stream);
+
+typedef struct ssm_ssd_state_passing_args {
+  const void *states;        /* (B,nc,H,dim) states dtype: per-chunk contributions */
+  const float *dA_chunk_last;/* (B,H,nc): dA_cumsum at the last step of each chunk */
+  const float *initial_states; /* (B,H,dim) fp32 or NULL */
+  void *states_out;          /* (B,nc,H,dim) states dtype: state entering each chunk */
+  float *final_states;       /* (B,H,dim) */
+  int32_t batch, nchunks, heads, dim;
+  int32_t states_dtype;
+} ssm_ssd_state_passing_args;
+int ssm_ssd_state_passing(const ssm_ssd_state_passing_args *args, void *hip_stream);
+
+typedef struct ssm_ssd_chunk_scan_args {
+  const void *CB;           /* (B,nc,G,Q,Q) cb dtype, lower triangle used */
+  const void *Cm;           /* (B,L,G,N) c dtype */
+  const void *x;            /* (B,L,H,P) x dtype */
+  const void *z;            /* (B,L,H,P) z dtype or NULL */
+  const void *prev_states;  /* (B,nc,H,P,N) states dtype: state entering each chunk */
+  const float *dt, *dA_cumsum; /* (B,H,nc,Q) */
+  const float *Dskip;       /* (H,P) if d_per_p else (H,), or NULL */
+  void *y;                  /* (B,L,H,P) x dtype */
+  ssm_ssd_dims dims;
+  int32_t x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype, d_per_p, force_generic;
+} ssm_ssd_chunk_scan_args;
+int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
+
+/* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).
  * Forward stands behind `dw_causal_conv(x, weight, bias, activation)`
  * (src/ssm/ops/__init__.py:1594-1600; semantics reference.py:466-537);

@@ -84,6 +84,40 @@ class DscanFwdArgs(C.Structure):
     ]
 
 
+class SsdDims(C.Structure):
+    _fields_ = [("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("headdim", _i32), ("groups", _i32),
+                ("nstate", _i32), ("chunk", _i32)]
+
+
+class SsdCumsumArgs(C.Structure):
+    _fields_ = [("dt", _vp), ("A", _vp), ("dt_bias", _vp), ("dA_cumsum", _vp), ("dt_out", _vp),
+                ("dims", SsdDims), ("dt_dtype", _i32), ("dt_softplus", _i32), ("dt_min", _f32), ("dt_max", _f32)]
+
+
+class SsdBmmArgs(C.Structure):
+    _fields_ = [("a", _vp), ("b", _vp), ("seq_idx", _vp), ("out", _vp),
+                ("batch", _i32), ("seqlen", _i32), ("groups", _i32), ("kdim", _i32), ("chunk", _i32),
+                ("in_dtype", _i32), ("out_dtype", _i32), ("causal", _i32), ("force_generic", _i32)]
+
+
+class SsdChunkStateArgs(C.Structure):
+    _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("states", _vp), ("dims", SsdDims),
+                ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("force_generic", _i32)]
+
+
+class SsdStatePassingArgs(C.Structure):
+    _fields_ = [("states", _vp), ("dA_chunk_last", _vp), ("initial_states", _vp), ("states_out", _vp),
+                ("final_states", _vp), ("batch", _i32), ("nchunks", _i32), ("heads", _i32), ("dim", _i32),
+                ("states_dtype", _i32)]
+
+
+class SsdChunkScanArgs(C.Structure):
+    _fields_ = [("CB", _vp), ("Cm", _vp), ("x", _vp), ("z", _vp), ("prev_states", _vp), ("dt", _vp),
+                ("dA_cumsum", _vp), ("Dskip", _vp), ("y", _vp), ("dims", SsdDims),
+                ("x_dtype", _i32), ("c_dtype", _i32), ("cb_dtype", _i32), ("states_dtype", _i32),
+                ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32)]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -131,6 +165,11 @@ ENTRY_POINTS = {
     "ssm_scan_bwd": ScanBwdArgs,
     "ssm_state_step": StateStepArgs,
     "ssm_dscan_fwd": DscanFwdArgs,
+    "ssm_ssd_chunk_cumsum": SsdCumsumArgs,
+    "ssm_ssd_bmm_chunk": SsdBmmArgs,
+    "ssm_ssd_chunk_state": SsdChunkStateArgs,
+    "ssm_ssd_state_passing": SsdStatePassingArgs,
+    "ssm_ssd_chunk_scan": SsdChunkScanArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_norm_fwd": NormFwdArgs,

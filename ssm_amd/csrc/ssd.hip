@@ -1,0 +1,276 @@
+// State-space-duality (Mamba-2) operator family: C-ABI entry points and the
+// shape-generic kernels.
+//
+//   chunk_cumsum   dt' = clamp(softplus(dt + bias)); dA_cs[c,l] = sum_{j<=l} dt'_j A_h
+//   bmm_chunk      CB[c,l,s] = <a_l, b_s>                       (C B^T per chunk and group)
+//   chunk_state    S_c[p,n]  = sum_l B_l[n] exp(dA_cs[last]-dA_cs[l]) dt'_l x_l[p]
+//   state_passing  H_{c+1}   = exp(dA_cs[c,last]) H_c + S_c      (H_0 = initial state)
+//   chunk_scan     y_l = exp(dA_cs[l]) C_l.H_c + sum_{s<=l} CB[l,s] exp(dA_cs[l]-dA_cs[s]) dt'_s x_s
+//                        + D x_l ;  y_l *= silu(z_l)
+//
+// The three contractions have bf16 MFMA implementations (ssd_mfma.hip) that are
+// taken whenever the shape allows; the kernels here accept every shape and
+// dtype, accumulate in fp32 and serve as their fallback.
+#include "ssd_common.hpp"
+
+namespace ssm {
+
+constexpr int SSD_THREADS = 256;
+
+static unsigned grid_for(size_t n) {
+  const size_t g = (n + SSD_THREADS - 1) / SSD_THREADS;
+  return (unsigned)(g < 1 ? 1 : g);
+}
+
+// One thread per (b, h, c): sequential running sum over the chunk.
+__global__ __launch_bounds__(SSD_THREADS) void ssd_cumsum_kernel(const SsdCumsumParams p) {
+  const SsdDims &d = p.d;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t total = (size_t)d.batch * d.heads * d.nchunks;
+  if (gid >= total) return;
+  const int c = (int)(gid % d.nchunks);
+  const int h = (int)((gid / d.nchunks) % d.heads);
+  const int b = (int)(gid / ((size_t)d.nchunks * d.heads));
+  const float A = p.A[h];
+  const float bias = p.bias ? p.bias[h] : 0.0f;
+  float run = 0.0f;
+  const size_t out = (((size_t)b * d.heads + h) * d.nchunks + c) * d.chunk;
+  for (int l = 0; l < d.chunk; ++l) {
+    const int t = c * d.chunk + l;
+    float v = 0.0f;
+    if (t < d.len) {
+      v = load_as_f32(p.dt, p.dt_dtype, ((size_t)b * d.len + t) * d.heads + h) + bias;
+      if (p.softplus) v = softplus_f32(v);
+      v = fminf(fmaxf(v, p.dt_min), p.dt_max);
+    }
+    run = __builtin_fmaf(v, A, run);
+    p.dt_out[out + l] = v;
+    p.dA_cs[out + l] = run;
+  }
+}
+
+// One thread per output element.
+__global__ __launch_bounds__(SSD_THREADS) void ssd_bmm_kernel(const SsdBmmParams p) {
+  const int Q = p.chunk;
+  const size_t total = (size_t)p.batch * p.nchunks * p.groups * Q * Q;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int s = (int)(gid % Q), l = (int)((gid / Q) % Q);
+  const int g = (int)((gid / ((size_t)Q * Q)) % p.groups);
+  const int c = (int)((gid / ((size_t)Q * Q * p.groups)) % p.nchunks);
+  const int b = (int)(gid / ((size_t)Q * Q * p.groups * p.nchunks));
+  const int tl = c * Q + l, ts = c * Q + s;
+  float acc = 0.0f;
+  if (tl < p.len && ts < p.len && !(p.causal && s > l)) {
+    const size_t ra = (((size_t)b * p.len + tl) * p.groups + g) * p.kdim;
+    const size_t rb = (((size_t)b * p.len + ts) * p.groups + g) * p.kdim;
+    for (int k = 0; k < p.kdim; ++k)
+      acc = __builtin_fmaf(load_as_f32(p.a, p.in_dtype, ra + k), load_as_f32(p.b, p.in_dtype, rb + k), acc);
+    if (p.seq_idx && p.seq_idx[(size_t)b * p.len + tl] != p.seq_idx[(size_t)b * p.len + ts]) acc = 0.0f;
+  }
+  store_any(p.out, p.out_dtype, gid, acc);
+}
+
+// One thread per (b, c, h, p, n).
+__global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_state_kernel(const SsdStateParams p) {
+  const SsdDims &d = p.d;
+  const size_t total = (size_t)d.batch * d.nchunks * d.heads * d.hdim * d.nstate;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int n = (int)(gid % d.nstate);
+  const int pp = (int)((gid / d.nstate) % d.hdim);
+  const int h = (int)((gid / ((size_t)d.nstate * d.hdim)) % d.heads);
+  const int c = (int)((gid / ((size_t)d.nstate * d.hdim * d.heads)) % d.nchunks);
+  const int b = (int)(gid / ((size_t)d.nstate * d.hdim * d.heads * d.nchunks));
+  const int g = h / (d.heads / d.groups);
+  const size_t cs = (((size_t)b * d.heads + h) * d.nchunks + c) * d.chunk;
+  const float last = p.dA_cs[cs + d.chunk - 1];
+  float acc = 0.0f;
+  for (int l = 0; l < d.chunk; ++l) {
+    const int t = c * d.chunk + l;
+    if (t >= d.len) break;
+    const float w = decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
+    const float bv = load_as_f32(p.Bm, p.b_dtype, (((size_t)b * d.len + t) * d.groups + g) * d.nstate + n);
+    const float xv = load_as_f32(p.x, p.x_dtype, (((size_t)b * d.len + t) * d.heads + h) * d.hdim + pp);
+    acc = __builtin_fmaf(bv * w, xv, acc);
+  }
+  store_any(p.states, p.states_dtype, gid, acc);
+}
+
+// One thread per (b, h, i): sequential over chunks.
+__global__ __launch_bounds__(SSD_THREADS) void ssd_state_passing_kernel(const SsdPassParams p) {
+  const size_t total = (size_t)p.batch * p.heads * p.dim;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int i = (int)(gid % p.dim);
+  const int h = (int)((gid / p.dim) % p.heads);
+  const int b = (int)(gid / ((size_t)p.dim * p.heads));
+  float cur = p.init ? p.init[gid] : 0.0f;
+  for (int c = 0; c < p.nchunks; ++c) {
+    const size_t at = (((size_t)b * p.nchunks + c) * p.heads + h) * p.dim + i;
+    const float contrib = load_as_f32(p.states, p.states_dtype, at);
+    store_any(p.out, p.states_dtype, at, cur);
+    cur = __builtin_fmaf(exp2_hw(p.dA_last[((size_t)b * p.heads + h) * p.nchunks + c] * LOG2E), cur, contrib);
+  }
+  p.final_states[gid] = cur;
+}
+
+// One thread per (b, t, h, p).
+__global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_scan_kernel(const SsdScanParams p) {
+  const SsdDims &d = p.d;
+  const size_t total = (size_t)d.batch * d.len * d.heads * d.hdim;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int pp = (int)(gid % d.hdim);
+  const int h = (int)((gid / d.hdim) % d.heads);
+  const int t = (int)((gid / ((size_t)d.hdim * d.heads)) % d.len);
+  const int b = (int)(gid / ((size_t)d.hdim * d.heads * d.len));
+  const int c = t / d.chunk, l = t % d.chunk;
+  const int g = h / (d.heads / d.groups);
+  const size_t cs = (((size_t)b * d.heads + h) * d.nchunks + c) * d.chunk;
+  const float dal = p.dA_cs[cs + l];
+  // carried-in state
+  float acc = 0.0f;
+  const size_t crow = (((size_t)b * d.len + t) * d.groups + g) * d.nstate;
+  const size_t srow = ((((size_t)b * d.nchunks + c) * d.heads + h) * d.hdim + pp) * d.nstate;
+  for (int n = 0; n < d.nstate; ++n)
+    acc = __builtin_fmaf(load_as_f32(p.Cm, p.c_dtype, crow + n), load_as_f32(p.prev, p.states_dtype, srow + n), acc);
+  acc *= exp2_hw(dal * LOG2E);
+  // within the chunk
+  const size_t cbrow = ((((size_t)b * d.nchunks + c) * d.groups + g) * d.chunk + l) * d.chunk;
+  for (int s = 0; s <= l; ++s) {
+    const float m = load_as_f32(p.CB, p.cb_dtype, cbrow + s) * decay_exp(dal - p.dA_cs[cs + s]) * p.dt[cs + s];
+    const float xv = load_as_f32(p.x, p.x_dtype, (((size_t)b * d.len + c * d.chunk + s) * d.heads + h) * d.hdim + pp);
+    acc = __builtin_fmaf(m, xv, acc);
+  }
+  const float xl = load_as_f32(p.x, p.x_dtype, gid);
+  if (p.Dk) acc = __builtin_fmaf(p.Dk[p.d_per_p ? (size_t)h * d.hdim + pp : (size_t)h], xl, acc);
+  if (p.z) acc *= silu_f32(load_as_f32(p.z, p.z_dtype, gid));
+  store_any(p.y, p.x_dtype, gid, acc);
+}
+
+static int dims_check(const char *who, const ssm_ssd_dims &s, SsdDims &d) {
+  SSM_REQUIRE(s.batch > 0 && s.seqlen > 0 && s.heads > 0 && s.headdim > 0 && s.groups > 0 && s.nstate > 0 &&
+                  s.chunk > 0,
+              SSM_ERR_BAD_SHAPE, "%s: all of batch, seqlen, heads, headdim, groups, nstate, chunk must be positive", who);
+  SSM_REQUIRE(s.heads % s.groups == 0, SSM_ERR_BAD_SHAPE, "%s: groups=%d must divide heads=%d", who, s.groups, s.heads);
+  d.batch = s.batch; d.len = s.seqlen; d.heads = s.heads; d.hdim = s.headdim; d.groups = s.groups;
+  d.nstate = s.nstate; d.chunk = s.chunk; d.nchunks = (s.seqlen + s.chunk - 1) / s.chunk;
+  SSM_REQUIRE((size_t)d.batch * d.nchunks * d.heads * d.hdim * d.nstate < ((size_t)1 << 40) &&
+                  (size_t)d.batch * d.len * d.heads * d.hdim < ((size_t)1 << 40),
+              SSM_ERR_TOO_LARGE, "%s: tensor too large", who);
+  return SSM_OK;
+}
+
+}  // namespace ssm
+
+extern "C" int ssm_ssd_chunk_cumsum(const ssm_ssd_cumsum_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a && a->dt && a->A && a->dA_cumsum && a->dt_out, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_chunk_cumsum: dt, A, dA_cumsum and dt_out are required");
+  SsdCumsumParams p{};
+  ssm_ssd_dims dd = a->dims;
+  if (dd.headdim <= 0) dd.headdim = 1;
+  if (dd.groups <= 0) dd.groups = 1;
+  if (dd.nstate <= 0) dd.nstate = 1;
+  int rc = dims_check("ssm_ssd_chunk_cumsum", dd, p.d);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(valid_dtype(a->dt_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_chunk_cumsum: dt_dtype=%d", a->dt_dtype);
+  p.dt = a->dt; p.A = a->A; p.bias = a->dt_bias; p.dA_cs = a->dA_cumsum; p.dt_out = a->dt_out;
+  p.dt_dtype = a->dt_dtype; p.softplus = a->dt_softplus ? 1 : 0; p.dt_min = a->dt_min; p.dt_max = a->dt_max;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(grid_for((size_t)p.d.batch * p.d.heads * p.d.nchunks)),
+                     dim3(SSD_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_chunk_cumsum");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_bmm_chunk(const ssm_ssd_bmm_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a && a->a && a->b && a->out, SSM_ERR_NULL_POINTER, "ssm_ssd_bmm_chunk: a, b and out are required");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->groups > 0 && a->kdim > 0 && a->chunk > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bmm_chunk: batch, seqlen, groups, kdim and chunk must be positive");
+  SSM_REQUIRE(valid_dtype(a->in_dtype) && valid_dtype(a->out_dtype), SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_bmm_chunk: in_dtype=%d out_dtype=%d", a->in_dtype, a->out_dtype);
+  SsdBmmParams p{};
+  p.a = a->a; p.b = a->b; p.seq_idx = a->seq_idx; p.out = a->out;
+  p.batch = a->batch; p.len = a->seqlen; p.groups = a->groups; p.kdim = a->kdim; p.chunk = a->chunk;
+  p.nchunks = (a->seqlen + a->chunk - 1) / a->chunk;
+  p.in_dtype = a->in_dtype; p.out_dtype = a->out_dtype; p.causal = a->causal ? 1 : 0;
+  const size_t total = (size_t)p.batch * p.nchunks * p.groups * p.chunk * p.chunk;
+  SSM_REQUIRE(total < ((size_t)1 << 40), SSM_ERR_TOO_LARGE, "ssm_ssd_bmm_chunk: tensor too large");
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  if (!a->force_generic && ssd_bmm_mfma(p, s)) {
+    SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk(mfma)");
+    return SSM_OK;
+  }
+  hipLaunchKernelGGL(ssd_bmm_kernel, dim3(grid_for(total)), dim3(SSD_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a && a->Bm && a->x && a->dt && a->dA_cumsum && a->states, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_chunk_state: Bm, x, dt, dA_cumsum and states are required");
+  SsdStateParams p{};
+  int rc = dims_check("ssm_ssd_chunk_state", a->dims, p.d);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(valid_dtype(a->x_dtype) && valid_dtype(a->b_dtype) && valid_dtype(a->states_dtype), SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_chunk_state: unsupported dtype");
+  p.Bm = a->Bm; p.x = a->x; p.dt = a->dt; p.dA_cs = a->dA_cumsum; p.states = a->states;
+  p.x_dtype = a->x_dtype; p.b_dtype = a->b_dtype; p.states_dtype = a->states_dtype;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  if (!a->force_generic && ssd_chunk_state_mfma(p, s)) {
+    SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
+    return SSM_OK;
+  }
+  const size_t total = (size_t)p.d.batch * p.d.nchunks * p.d.heads * p.d.hdim * p.d.nstate;
+  hipLaunchKernelGGL(ssd_chunk_state_kernel, dim3(grid_for(total)), dim3(SSD_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_chunk_state");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_state_passing(const ssm_ssd_state_passing_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a && a->states && a->dA_chunk_last && a->states_out && a->final_states, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_state_passing: states, dA_chunk_last, states_out and final_states are required");
+  SSM_REQUIRE(a->batch > 0 && a->nchunks > 0 && a->heads > 0 && a->dim > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_state_passing: batch, nchunks, heads and dim must be positive");
+  SSM_REQUIRE(valid_dtype(a->states_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_state_passing: states_dtype=%d",
+              a->states_dtype);
+  SsdPassParams p{};
+  p.states = a->states; p.dA_last = a->dA_chunk_last; p.init = a->initial_states; p.out = a->states_out;
+  p.final_states = a->final_states;
+  p.batch = a->batch; p.nchunks = a->nchunks; p.heads = a->heads; p.dim = a->dim; p.states_dtype = a->states_dtype;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(ssd_state_passing_kernel, dim3(grid_for((size_t)p.batch * p.heads * p.dim)), dim3(SSD_THREADS),
+                     0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_state_passing");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a && a->CB && a->Cm && a->x && a->dt && a->dA_cumsum && a->prev_states && a->y, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_chunk_scan: CB, Cm, x, dt, dA_cumsum, prev_states and y are required");
+  SsdScanParams p{};
+  int rc = dims_check("ssm_ssd_chunk_scan", a->dims, p.d);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(valid_dtype(a->x_dtype) && valid_dtype(a->c_dtype) && valid_dtype(a->cb_dtype) &&
+                  valid_dtype(a->states_dtype) && (!a->z || valid_dtype(a->z_dtype)),
+              SSM_ERR_BAD_DTYPE, "ssm_ssd_chunk_scan: unsupported dtype");
+  p.CB = a->CB; p.Cm = a->Cm; p.x = a->x; p.z = a->z; p.prev = a->prev_states; p.dt = a->dt; p.dA_cs = a->dA_cumsum;
+  p.Dk = a->Dskip; p.y = a->y;
+  p.x_dtype = a->x_dtype; p.c_dtype = a->c_dtype; p.cb_dtype = a->cb_dtype; p.states_dtype = a->states_dtype;
+  p.z_dtype = a->z_dtype; p.d_per_p = a->d_per_p ? 1 : 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
+    SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
+    return SSM_OK;
+  }
+  const size_t total = (size_t)p.d.batch * p.d.len * p.d.heads * p.d.hdim;
+  hipLaunchKernelGGL(ssd_chunk_scan_kernel, dim3(grid_for(total)), dim3(SSD_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan");
+  return SSM_OK;
+}

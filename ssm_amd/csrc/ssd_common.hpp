@@ -1,0 +1,78 @@
+// Parameter blocks shared by the state-space-duality (Mamba-2) kernels.
+//
+// Tensor layouts (row-major):
+//   x, z, y        (B, L, H, P)        dt (B, L, H)       A (H,)
+//   Bm, Cm         (B, L, G, N)        head h reads group h / (H/G)
+//   dt_out, dA_cs  (B, H, nc, Q) fp32  (chunked step and its running sum times A)
+//   CB             (B, nc, G, Q, Q)    CB[l][s] = <C_l, B_s>
+//   states         (B, nc, H, P, N)    per-chunk contribution / state entering a chunk
+//   final_states   (B, H, P, N) fp32
+#pragma once
+#include "common.hpp"
+
+namespace ssm {
+
+struct SsdDims {
+  int batch, len, heads, hdim, groups, nstate, chunk, nchunks;
+};
+
+struct SsdCumsumParams {
+  const void *dt;
+  const float *A, *bias;
+  float *dA_cs, *dt_out;
+  SsdDims d;
+  int dt_dtype, softplus;
+  float dt_min, dt_max;
+};
+
+struct SsdBmmParams {
+  const void *a, *b;          // (B, L, G, K)
+  const int *seq_idx;         // (B, L) or null
+  void *out;                  // (B, nc, G, Q, Q)
+  int batch, len, groups, kdim, chunk, nchunks;
+  int in_dtype, out_dtype, causal;
+};
+
+struct SsdStateParams {
+  const void *Bm, *x;
+  const float *dt, *dA_cs;
+  void *states;
+  SsdDims d;
+  int x_dtype, b_dtype, states_dtype;
+};
+
+struct SsdPassParams {
+  const void *states;         // (B, nc, H, dim)
+  const float *dA_last;       // (B, H, nc)
+  const float *init;          // (B, H, dim) or null
+  void *out;                  // (B, nc, H, dim): state entering each chunk
+  float *final_states;        // (B, H, dim)
+  int batch, nchunks, heads, dim;
+  int states_dtype;
+};
+
+struct SsdScanParams {
+  const void *CB, *Cm, *x, *z, *prev;
+  const float *dt, *dA_cs, *Dk;
+  void *y;
+  SsdDims d;
+  int x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype;
+  int d_per_p;                // D is (H, P) instead of (H,)
+};
+
+__device__ __forceinline__ void store_any(void *p, int dtype, size_t i, float v) {
+  if (dtype == SSM_F32) reinterpret_cast<float *>(p)[i] = v;
+  else if (dtype == SSM_BF16) reinterpret_cast<bf16_t *>(p)[i] = from_f32<bf16_t>(v);
+  else reinterpret_cast<f16_t *>(p)[i] = from_f32<f16_t>(v);
+}
+
+// exp(min(v, 0)): decay factors inside a chunk never exceed 1 when A <= 0; the
+// clamp only matters for (unphysical) positive A and mirrors the published kernels.
+__device__ __forceinline__ float decay_exp(float v) { return exp2_hw(fminf(v, 0.0f) * LOG2E); }
+
+// MFMA variants, defined in ssd_mfma.hip; return false when the shape is not covered.
+bool ssd_bmm_mfma(const SsdBmmParams &p, hipStream_t s);
+bool ssd_chunk_state_mfma(const SsdStateParams &p, hipStream_t s);
+bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s);
+
+}  // namespace ssm

@@ -1,0 +1,281 @@
+"""State-space-duality (Mamba-2) operators on the GPU.
+
+The reference repository ships no implementation of these (its
+``ssd_chunk_scan`` is a diagonal recurrence, see :func:`ssm_amd.ops.ssd_chunk_scan`);
+it only records their behaviour as vectors in ``tests/mamba_reference_cases.json``.
+The functions below take the argument order of the calls that produced those
+vectors (scripts/refresh_mamba_goldens.py:430-486, :591-604, :680-705) so that the
+vectors can be replayed one to one.
+
+Shapes: ``x, z, y (B, L, H, P)``; ``dt (B, L, H)``; ``A (H,)``; ``B, C (B, L, G, N)``;
+``dt_out, dA_cumsum (B, H, nc, Q)`` float32; ``states (B, nc, H, P, N)``;
+``final_states (B, H, P, N)`` float32, with ``nc = ceil(L / Q)``.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from . import _contract as K
+
+
+def _dims(batch, seqlen, heads, headdim, groups, nstate, chunk) -> _lib.SsdDims:
+    return _lib.SsdDims(batch=batch, seqlen=seqlen, heads=heads, headdim=headdim, groups=groups,
+                        nstate=nstate, chunk=chunk)
+
+
+def _need(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def chunk_cumsum(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
+    """Effective step and its chunk-wise running sum times ``A``.
+
+    Args:
+        dt: ``(B, L, H)`` raw steps.
+        A: ``(H,)``.
+        chunk_size: ``Q``.
+        dt_bias: Optional ``(H,)`` added before ``softplus``.
+        dt_softplus: Apply ``softplus`` to ``dt + dt_bias``.
+        dt_limit: ``(min, max)`` clamp applied last.
+
+    Returns:
+        ``(dA_cumsum, dt_out)``, both ``(B, H, nc, Q)`` float32; steps past ``L`` in
+        the last chunk have ``dt_out = 0``.
+    """
+    _need(dt.ndim == 3, "dt must have shape (B, L, H).")
+    batch, seqlen, heads = (int(s) for s in dt.shape)
+    _need(tuple(A.shape) == (heads,), "A must have shape (H,).")
+    _need(dt_bias is None or tuple(dt_bias.shape) == (heads,), "dt_bias must have shape (H,).")
+    Q = int(chunk_size)
+    _need(Q > 0, "chunk_size must be positive.")
+    K.check_float("dt", dt)
+    dev = K.require_gpu(dt, A, dt_bias)
+    nc = (seqlen + Q - 1) // Q
+    dtc = K.cast_c(dt, dt.dtype)
+    Af, bf = K.as_f32_vec(A), K.as_f32_vec(dt_bias)
+    dA = torch.empty(batch, heads, nc, Q, dtype=torch.float32, device=dev)
+    dto = torch.empty_like(dA)
+    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    args = _lib.SsdCumsumArgs(
+        dt=_lib.ptr(dtc), A=_lib.ptr(Af), dt_bias=_lib.ptr(bf), dA_cumsum=_lib.ptr(dA), dt_out=_lib.ptr(dto),
+        dims=_dims(batch, seqlen, heads, 1, 1, 1, Q), dt_dtype=_lib.dtype_enum(dtc.dtype),
+        dt_softplus=int(bool(dt_softplus)), dt_min=lo if lo > -math.inf else -3.0e38,
+        dt_max=hi if hi < math.inf else 3.0e38)
+    _lib.call("ssm_ssd_chunk_cumsum", args, dev)
+    return dA, dto
+
+
+def bmm_chunk(a, b, chunk_size, seq_idx=None, causal=False, output_dtype=None, force_generic=False):
+    """Per-chunk ``a b^T``: ``out[b, c, (g,) l, s] = <a[b, cQ+l, (g,)], b[b, cQ+s, (g,)]>``.
+
+    Args:
+        a, b: ``(B, L, K)`` or grouped ``(B, L, G, K)``.
+        chunk_size: ``Q``.
+        seq_idx: Optional ``(B, L)`` int sequence ids; products across sequences are 0.
+        causal: Only ``s <= l`` is computed (the rest is returned as 0).
+        output_dtype: dtype of the result (default: dtype of ``a``).
+
+    Returns:
+        ``(B, nc, Q, Q)`` or ``(B, nc, G, Q, Q)``.
+    """
+    _need(a.ndim in (3, 4) and a.shape == b.shape, "a and b must both be (B, L, K) or (B, L, G, K).")
+    grouped = a.ndim == 4
+    batch, seqlen = int(a.shape[0]), int(a.shape[1])
+    groups = int(a.shape[2]) if grouped else 1
+    kdim = int(a.shape[-1])
+    Q = int(chunk_size)
+    _need(Q > 0, "chunk_size must be positive.")
+    K.check_float("a", a)
+    K.check_float("b", b)
+    dev = K.require_gpu(a, b, seq_idx)
+    io = K.common_io_dtype([a, b])
+    ac, bc = K.cast_c(a, io), K.cast_c(b, io)
+    out_dt = output_dtype or a.dtype
+    nc = (seqlen + Q - 1) // Q
+    out = torch.empty((batch, nc, groups, Q, Q), dtype=out_dt, device=dev)
+    si = None
+    if seq_idx is not None:
+        _need(tuple(seq_idx.shape) == (batch, seqlen), "seq_idx must have shape (B, L).")
+        si = seq_idx.to(torch.int32).contiguous()
+    args = _lib.SsdBmmArgs(a=_lib.ptr(ac), b=_lib.ptr(bc), seq_idx=_lib.ptr(si), out=_lib.ptr(out),
+                           batch=batch, seqlen=seqlen, groups=groups, kdim=kdim, chunk=Q,
+                           in_dtype=_lib.dtype_enum(io), out_dtype=_lib.dtype_enum(out_dt),
+                           causal=int(bool(causal)), force_generic=int(bool(force_generic)))
+    _lib.call("ssm_ssd_bmm_chunk", args, dev)
+    return out if grouped else out[:, :, 0]
+
+
+def _ssd_shapes(x, B):
+    _need(x.ndim == 4, "x must have shape (B, L, H, P).")
+    _need(B.ndim == 4 and B.shape[0] == x.shape[0] and B.shape[1] == x.shape[1],
+          "B and C must have shape (B, L, G, N).")
+    batch, seqlen, heads, hdim = (int(s) for s in x.shape)
+    groups, nstate = int(B.shape[2]), int(B.shape[3])
+    _need(groups > 0 and heads % groups == 0, "ngroups must divide nheads.")
+    return batch, seqlen, heads, hdim, groups, nstate
+
+
+def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=False):
+    """Contribution of each chunk to the state at its end.
+
+    Args:
+        B: ``(B, L, G, N)``.
+        x: ``(B, L, H, P)``.
+        dt: ``(B, H, nc, Q)`` float32 (``dt_out`` of :func:`chunk_cumsum`).
+        dA_cumsum: ``(B, H, nc, Q)`` float32.
+        states_dtype: dtype of the result.
+
+    Returns:
+        ``states (B, nc, H, P, N)``.
+    """
+    batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
+    _need(dt.ndim == 4 and dt.shape == dA_cumsum.shape and dt.shape[0] == batch and dt.shape[1] == heads,
+          "dt and dA_cumsum must have shape (B, H, nc, Q).")
+    nc, Q = int(dt.shape[2]), int(dt.shape[3])
+    _need(nc == (seqlen + Q - 1) // Q, "dt has the wrong number of chunks for this sequence length.")
+    dev = K.require_gpu(B, x, dt, dA_cumsum)
+    xc, Bc = K.cast_c(x, x.dtype), K.cast_c(B, B.dtype)
+    K.check_float("x", xc)
+    K.check_float("B", Bc)
+    dtf, daf = K.as_f32_vec(dt), K.as_f32_vec(dA_cumsum)
+    states = torch.empty(batch, nc, heads, hdim, nstate, dtype=states_dtype, device=dev)
+    args = _lib.SsdChunkStateArgs(
+        Bm=_lib.ptr(Bc), x=_lib.ptr(xc), dt=_lib.ptr(dtf), dA_cumsum=_lib.ptr(daf), states=_lib.ptr(states),
+        dims=_dims(batch, seqlen, heads, hdim, groups, nstate, Q), x_dtype=_lib.dtype_enum(xc.dtype),
+        b_dtype=_lib.dtype_enum(Bc.dtype), states_dtype=_lib.dtype_enum(states_dtype),
+        force_generic=int(bool(force_generic)))
+    _lib.call("ssm_ssd_chunk_state", args, dev)
+    return states
+
+
+def state_passing(states, dA_chunk_cumsum, initial_states=None):
+    """Carry states across chunks: ``H_{c+1} = exp(dA_c) H_c + states_c``.
+
+    Args:
+        states: ``(B, nc, H, ...)`` per-chunk contributions (any trailing shape).
+        dA_chunk_cumsum: ``(B, H, nc)``: ``dA_cumsum[..., -1]``.
+        initial_states: Optional ``(B, H, ...)``.
+
+    Returns:
+        ``(states_passed, final_states)``: the state entering each chunk (shape and dtype
+        of ``states``) and the state after the last chunk ``(B, H, ...)`` in float32.
+    """
+    _need(states.ndim >= 4, "states must have shape (B, nc, H, ...).")
+    batch, nc, heads = (int(s) for s in states.shape[:3])
+    trailing = tuple(int(s) for s in states.shape[3:])
+    dim = 1
+    for s_ in trailing:
+        dim *= s_
+    _need(tuple(dA_chunk_cumsum.shape) == (batch, heads, nc), "dA_chunk_cumsum must have shape (B, H, nc).")
+    dev = K.require_gpu(states, dA_chunk_cumsum, initial_states)
+    sc = K.cast_c(states, states.dtype)
+    K.check_float("states", sc)
+    daf = K.as_f32_vec(dA_chunk_cumsum)
+    init = None
+    if initial_states is not None:
+        _need(tuple(initial_states.shape) == (batch, heads) + trailing, "initial_states must have shape (B, H, ...).")
+        init = K.as_f32_vec(initial_states)
+    out = torch.empty_like(sc)
+    final = torch.empty((batch, heads) + trailing, dtype=torch.float32, device=dev)
+    args = _lib.SsdStatePassingArgs(
+        states=_lib.ptr(sc), dA_chunk_last=_lib.ptr(daf), initial_states=_lib.ptr(init),
+        states_out=_lib.ptr(out), final_states=_lib.ptr(final), batch=batch, nchunks=nc, heads=heads, dim=dim,
+        states_dtype=_lib.dtype_enum(sc.dtype))
+    _lib.call("ssm_ssd_state_passing", args, dev)
+    return out, final
+
+
+def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False):
+    """Outputs of every chunk from the state entering it.
+
+    Args:
+        B, C: ``(B, L, G, N)``.
+        x: ``(B, L, H, P)``.
+        dt, dA_cumsum: ``(B, H, nc, Q)`` float32.
+        prev_states: ``(B, nc, H, P, N)`` state entering each chunk.
+        D: Optional skip ``(H,)`` or ``(H, P)``.
+        z: Optional gate ``(B, L, H, P)``.
+        CB: Optional precomputed ``bmm_chunk(C, B, Q)``.
+
+    Returns:
+        ``y (B, L, H, P)`` in ``x.dtype``.
+    """
+    batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
+    _need(C.shape == B.shape, "B and C must have the same shape.")
+    _need(dt.ndim == 4 and dt.shape == dA_cumsum.shape and dt.shape[0] == batch and dt.shape[1] == heads,
+          "dt and dA_cumsum must have shape (B, H, nc, Q).")
+    nc, Q = int(dt.shape[2]), int(dt.shape[3])
+    _need(tuple(prev_states.shape) == (batch, nc, heads, hdim, nstate),
+          "prev_states must have shape (B, nc, H, P, N).")
+    d_per_p = False
+    if D is not None:
+        _need(tuple(D.shape) in ((heads,), (heads, hdim)), "D must have shape (H,) or (H, P).")
+        d_per_p = D.ndim == 2
+    _need(z is None or z.shape == x.shape, "z must have the shape of x.")
+    dev = K.require_gpu(B, C, x, dt, dA_cumsum, prev_states, D, z)
+    if CB is None:
+        CB = bmm_chunk(C, B, Q, causal=True, output_dtype=x.dtype if x.dtype != torch.float32 else torch.float32,
+                       force_generic=force_generic)
+    _need(tuple(CB.shape) == (batch, nc, groups, Q, Q), "CB must have shape (B, nc, G, Q, Q).")
+    xc, Cc, zc = K.cast_c(x, x.dtype), K.cast_c(C, C.dtype), (K.cast_c(z, z.dtype) if z is not None else None)
+    for name, t in (("x", xc), ("C", Cc), ("z", zc), ("CB", CB), ("prev_states", prev_states)):
+        if t is not None:
+            K.check_float(name, t)
+    ps, cb = K.cast_c(prev_states, prev_states.dtype), K.cast_c(CB, CB.dtype)
+    dtf, daf, Df = K.as_f32_vec(dt), K.as_f32_vec(dA_cumsum), K.as_f32_vec(D)
+    y = torch.empty_like(xc)
+    args = _lib.SsdChunkScanArgs(
+        CB=_lib.ptr(cb), Cm=_lib.ptr(Cc), x=_lib.ptr(xc), z=_lib.ptr(zc), prev_states=_lib.ptr(ps),
+        dt=_lib.ptr(dtf), dA_cumsum=_lib.ptr(daf), Dskip=_lib.ptr(Df), y=_lib.ptr(y),
+        dims=_dims(batch, seqlen, heads, hdim, groups, nstate, Q), x_dtype=_lib.dtype_enum(xc.dtype),
+        c_dtype=_lib.dtype_enum(Cc.dtype), cb_dtype=_lib.dtype_enum(cb.dtype),
+        states_dtype=_lib.dtype_enum(ps.dtype), z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
+        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)))
+    _lib.call("ssm_ssd_chunk_scan", args, dev)
+    return y
+
+
+def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
+                 dt_softplus=False, dt_limit=(0.0, float("inf")), return_final_states=False,
+                 states_dtype=None, force_generic=False):
+    """Mamba-2 SSD forward: ``chunk_cumsum -> bmm_chunk, chunk_state -> state_passing -> chunk_scan``.
+
+    Args:
+        x: ``(B, L, H, P)``.
+        dt: ``(B, L, H)``.
+        A: ``(H,)`` (negative for a decaying system).
+        B, C: ``(B, L, G, N)``.
+        chunk_size: ``Q``.
+        D: Optional skip ``(H,)`` or ``(H, P)``.
+        z: Optional gate ``(B, L, H, P)``.
+        dt_bias: Optional ``(H,)``.
+        initial_states: Optional ``(B, H, P, N)``.
+        dt_softplus: Apply ``softplus`` to ``dt + dt_bias``.
+        dt_limit: ``(min, max)`` clamp of the effective step.
+        return_final_states: Also return the state after the last token.
+        states_dtype: dtype of the per-chunk states kept in HBM between the kernels
+            (default: ``x.dtype``; the recurrence itself accumulates in float32).
+
+    Returns:
+        ``y (B, L, H, P)`` in ``x.dtype``, or ``(y, final_states (B, H, P, N) float32)``.
+    """
+    batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
+    _need(C.shape == B.shape, "B and C must have the same shape.")
+    _need(tuple(dt.shape) == (batch, seqlen, heads), "dt must have shape (B, L, H).")
+    _need(initial_states is None or tuple(initial_states.shape) == (batch, heads, hdim, nstate),
+          "initial_states must have shape (B, H, P, N).")
+    Q = int(chunk_size)
+    sdt = states_dtype or x.dtype
+    dA, dtc = chunk_cumsum(dt, A, Q, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit)
+    states = chunk_state(B, x, dtc, dA, states_dtype=sdt, force_generic=force_generic)
+    entering, final = state_passing(states, dA[:, :, :, -1].contiguous(), initial_states=initial_states)
+    y = chunk_scan(B, C, x, dtc, dA, entering, D=D, z=z, force_generic=force_generic)
+    if return_final_states:
+        return y, final
+    return y

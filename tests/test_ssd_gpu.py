@@ -1,0 +1,157 @@
+"""GPU parity of the state-space-duality (Mamba-2) operators: component vectors
+shipped by the reference, the float64 sequential recurrence, and the bf16 MFMA
+kernels against the shape-generic kernels at the benchmark shape."""
+
+import pytest
+import torch
+
+from oracle import ssd_oracle as S
+from tests import fixtures as fx
+
+pytestmark = pytest.mark.gpu
+TF32 = dict(rtol=2e-2, atol=2e-2)          # the shipped vectors were produced with TF32 dots
+FP32_TOL = dict(rtol=1e-4, atol=1e-4)
+
+
+def ssd():
+    from ssm_amd.ops import ssd as m
+    return m
+
+
+def cu(t):
+    return None if t is None else t.cuda()
+
+
+def test_chunk_cumsum_vectors():
+    rec = fx.upstream("ssd_components", "chunk_cumsum"); i = rec["inputs"]
+    dA, dt_c = ssd().chunk_cumsum(cu(i["dt"]), cu(i["A"]), 3, dt_bias=cu(i["dt_bias"]), dt_softplus=True)
+    torch.testing.assert_close(dA.cpu(), rec["outputs"]["dA_cumsum"], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(dt_c.cpu(), rec["outputs"]["dt_out"], rtol=1e-5, atol=1e-6)
+    rec = fx.upstream("ssd_components", "chunk_cumsum_clamped"); i = rec["inputs"]
+    dA, dt_c = ssd().chunk_cumsum(cu(i["dt"]), cu(i["A"]), 3, dt_limit=(0.01, 1.0))
+    torch.testing.assert_close(dA.cpu(), rec["outputs"]["dA_cumsum"], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(dt_c.cpu(), rec["outputs"]["dt_out"], rtol=1e-5, atol=1e-6)
+
+
+def test_bmm_vectors():
+    rec = fx.upstream("ssd_bmm", "basic"); i = rec["inputs"]
+    torch.testing.assert_close(ssd().bmm_chunk(cu(i["a"]), cu(i["b"]), 3).cpu(), rec["outputs"]["out"], **TF32)
+    rec = fx.upstream("ssd_bmm", "grouped"); i = rec["inputs"]
+    torch.testing.assert_close(ssd().bmm_chunk(cu(i["a"]), cu(i["b"]), 3).cpu(), rec["outputs"]["out"], **TF32)
+    rec = fx.upstream("ssd_bmm", "causal_seq"); i = rec["inputs"]
+    got = ssd().bmm_chunk(cu(i["a"]), cu(i["b"]), 3, seq_idx=cu(i["seq_idx"]), causal=True).cpu()
+    tri = torch.tril(torch.ones(3, 3, dtype=torch.bool))
+    torch.testing.assert_close(got[..., tri], rec["outputs"]["out"][..., tri], **TF32)
+
+
+def test_chunk_state_vector():
+    rec = fx.upstream("ssd_components", "chunk_state"); i = rec["inputs"]
+    st = ssd().chunk_state(cu(i["B"]), cu(i["x"]), cu(i["dt"]), cu(i["dA_cumsum"]))
+    torch.testing.assert_close(st.cpu(), rec["outputs"]["states"], **TF32)
+
+
+def test_state_passing_vector():
+    rec = fx.upstream("ssd_components", "state_passing"); i = rec["inputs"]
+    entering, final = ssd().state_passing(cu(i["states"]), cu(i["dA_last"]))
+    torch.testing.assert_close(entering.cpu(), rec["outputs"]["states_passed"], rtol=1e-5, atol=1e-6)
+    b, nc, h, p, n = i["states"].shape
+    torch.testing.assert_close(final.cpu().reshape(b, h, p * n), rec["outputs"]["final_states"], rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("case", ["chunk_scan_matrix_D_z", "chunk_scan_vector_D"])
+def test_chunk_scan_vectors(case):
+    rec = fx.upstream("ssd_components", case); i = rec["inputs"]
+    y = ssd().chunk_scan(cu(i["B"]), cu(i["C"]), cu(i["x"]), cu(i["dt"]), cu(i["dA_cumsum"]), cu(i["states"]),
+                         D=cu(i["D"]), z=cu(i.get("z")))
+    torch.testing.assert_close(y.cpu(), rec["outputs"]["y"], **TF32)
+
+
+def test_combined_vector():
+    rec = fx.upstream("ssd_combined", "combined_full"); i = rec["inputs"]
+    y, fin = ssd().ssd_combined(cu(i["X"]), cu(i["dt"]), cu(i["A"]), cu(i["B"]), cu(i["C"]), int(i["chunk_size"]),
+                                D=cu(i["D"]), z=cu(i["z"]), dt_bias=cu(i["dt_bias"]),
+                                initial_states=cu(i["initial_states"]), dt_softplus=True, return_final_states=True)
+    torch.testing.assert_close(y.cpu(), rec["outputs"]["y"], **TF32)
+    torch.testing.assert_close(fin.cpu(), rec["outputs"]["final_states"], **TF32)
+
+
+def make(seed, b, l, h, p, g, n, dtype=torch.float32, d_mat=False, use_z=True, use_init=True):
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(b, l, h, p, generator=gen).to(dtype)
+    dt = torch.nn.functional.softplus(torch.randn(b, l, h, generator=gen) - 3.0)
+    A = -(torch.rand(h, generator=gen) * 15 + 1)
+    Bm = torch.randn(b, l, g, n, generator=gen).to(dtype)
+    Cm = torch.randn(b, l, g, n, generator=gen).to(dtype)
+    D = torch.randn(h, p, generator=gen) if d_mat else torch.ones(h)
+    z = torch.randn(b, l, h, p, generator=gen).to(dtype) if use_z else None
+    init = torch.randn(b, h, p, n, generator=gen) if use_init else None
+    return dict(x=x, dt=dt, A=A, B=Bm, C=Cm, D=D, z=z, init=init)
+
+
+@pytest.mark.parametrize("shape,Q", [((1, 1, 1, 1, 1, 1), 1), ((2, 19, 4, 5, 2, 6), 8), ((2, 64, 4, 16, 1, 32), 16),
+                                     ((1, 300, 2, 64, 2, 128), 64), ((2, 130, 3, 7, 3, 9), 256)],
+                         ids=lambda v: str(v).replace(" ", ""))
+def test_fp32_combined_matches_float64_recurrence(shape, Q):
+    b, l, h, p, g, n = shape
+    inp = make(sum(shape), b, l, h, p, g, n, d_mat=(l % 2 == 1))
+    y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                                initial_states=inp["init"])
+    y, fin = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q,
+                                D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]),
+                                return_final_states=True)
+    torch.testing.assert_close(y.cpu().double(), y64, **FP32_TOL)
+    torch.testing.assert_close(fin.cpu().double(), f64, **FP32_TOL)
+
+
+def test_components_match_oracle_fp32():
+    inp = make(3, 2, 96, 4, 8, 2, 16)
+    Q = 32
+    dA, dtc = ssd().chunk_cumsum(cu(inp["dt"]), cu(inp["A"]), Q)
+    dA_o, dtc_o = S.chunk_cumsum(inp["dt"], inp["A"], Q)
+    torch.testing.assert_close(dA.cpu().double(), dA_o, rtol=1e-5, atol=1e-5)
+    st = ssd().chunk_state(cu(inp["B"]), cu(inp["x"]), dtc, dA)
+    st_o = S.chunk_state(inp["B"], inp["x"], dtc_o, dA_o)
+    torch.testing.assert_close(st.cpu().double(), st_o, **FP32_TOL)
+    ent, fin = ssd().state_passing(st, dA[..., -1].contiguous(), initial_states=cu(inp["init"]))
+    ent_o, fin_o = S.state_passing(st_o, dA_o[..., -1], inp["init"])
+    torch.testing.assert_close(ent.cpu().double(), ent_o, **FP32_TOL)
+    torch.testing.assert_close(fin.cpu().double(), fin_o, **FP32_TOL)
+    CB = ssd().bmm_chunk(cu(inp["C"]), cu(inp["B"]), Q)
+    torch.testing.assert_close(CB.cpu().double(), S.bmm_chunk(inp["C"], inp["B"], Q), **FP32_TOL)
+    y = ssd().chunk_scan(cu(inp["B"]), cu(inp["C"]), cu(inp["x"]), dtc, dA, ent, D=cu(inp["D"]), z=cu(inp["z"]))
+    y_o = S.chunk_scan(inp["B"], inp["C"], inp["x"], dtc_o, dA_o, ent_o, D=inp["D"], z=inp["z"])
+    torch.testing.assert_close(y.cpu().double(), y_o, **FP32_TOL)
+
+
+@pytest.mark.parametrize("shape,Q", [((2, 512, 4, 64, 1, 128), 256), ((1, 256, 2, 64, 2, 64), 64),
+                                     ((2, 384, 8, 32, 1, 128), 128), ((1, 700, 2, 64, 1, 128), 256)],
+                         ids=lambda v: str(v).replace(" ", ""))
+def test_bf16_mfma_matches_generic_and_oracle(shape, Q):
+    b, l, h, p, g, n = shape
+    inp = make(11, b, l, h, p, g, n, dtype=torch.bfloat16)
+    args = (cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
+    kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
+    y, fin = ssd().ssd_combined(*args, **kw)
+    yg, fing = ssd().ssd_combined(*args, force_generic=True, states_dtype=torch.float32, **kw)
+    y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                                initial_states=inp["init"])
+    scale = float(y64.abs().max())
+    torch.testing.assert_close(yg.float().cpu().double(), y64, rtol=2e-2, atol=2e-2 * scale)
+    torch.testing.assert_close(y.float().cpu().double(), y64, rtol=2e-2, atol=2e-2 * scale)
+    fs = float(f64.abs().max())
+    torch.testing.assert_close(fin.cpu().double(), f64, rtol=2e-2, atol=2e-2 * fs)
+
+
+def test_config3_shape_bf16():
+    """BASELINE config 3: B=4, L=4096, H=80, P=64, N=128, G=1, Q=256, bf16.  Full size on the
+    GPU; two heads of one batch row are replayed by the float64 sequential recurrence."""
+    inp = make(3, 4, 4096, 80, 64, 1, 128, dtype=torch.bfloat16, use_init=False)
+    y, fin = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), 256,
+                                D=cu(inp["D"]), z=cu(inp["z"]), return_final_states=True)
+    assert y.dtype == torch.bfloat16 and fin.dtype == torch.float32 and tuple(fin.shape) == (4, 80, 64, 128)
+    hs = [5, 71]
+    y64, f64 = S.ssd_sequential(inp["x"][1:2, :, hs], inp["dt"][1:2, :, hs], inp["A"][hs], inp["B"][1:2],
+                                inp["C"][1:2], D=inp["D"][hs], z=inp["z"][1:2, :, hs])
+    scale = float(y64.abs().max())
+    torch.testing.assert_close(y[1:2, :, hs].float().cpu().double(), y64, rtol=2e-2, atol=2e-2 * scale)
+    torch.testing.assert_close(fin[1:2, hs].cpu().double(), f64, rtol=2e-2, atol=2e-2 * float(f64.abs().max()))
