@@ -195,6 +195,10 @@ int ssm_dscan_fwd(const ssm_dscan_fwd_args *args, void *hip_stream);
  * final_states (B,H,P,N) fp32; nc = ceil(L/Q).  `force_generic` skips the
  * bf16 MFMA kernels (used by the tests to cross-check them).
  * ---------------------------------------------------------------------- */
+/* Which of the calls made by this thread since the last query ran a bf16 MFMA
+ * kernel: bit 0 bmm_chunk, bit 1 chunk_state, bit 2 chunk_scan.  Resets on read. */
+int ssm_ssd_mfma_launches(void);
+
 typedef struct ssm_ssd_dims {
   int32_t batch, seqlen, heads, headdim, groups, nstate, chunk;
 } ssm_ssd_dims;
@@ -226,9 +230,13 @@ typedef struct ssm_ssd_chunk_state_args {
   const float *dt;          /* (B,H,nc,Q) */
   const float *dA_cumsum;   /* (B,H,nc,Q) */
   void *states;             /* (B,nc,H,P,N) states dtype */
+  void *workspace;          /* optional: ssm_ssd_chunk_state_workspace_bytes() bytes of device memory;
+                               without it the MFMA kernel is not used */
+  size_t workspace_bytes;
   ssm_ssd_dims dims;
   int32_t x_dtype, b_dtype, states_dtype, force_generic;
 } ssm_ssd_chunk_state_args;
+size_t ssm_ssd_chunk_state_workspace_bytes(const ssm_ssd_dims *dims);
 int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *args, void *hip_stream);
 
 typedef struct ssm_ssd_state_passing_args {

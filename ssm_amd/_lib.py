@@ -101,7 +101,8 @@ class SsdBmmArgs(C.Structure):
 
 
 class SsdChunkStateArgs(C.Structure):
-    _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("states", _vp), ("dims", SsdDims),
+    _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("states", _vp),
+                ("workspace", _vp), ("workspace_bytes", C.c_size_t), ("dims", SsdDims),
                 ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("force_generic", _i32)]
 
 
@@ -183,6 +184,8 @@ PLAIN_SYMBOLS = {
     "ssm_scan_chunk_len": (C.c_int, []),
     "ssm_scan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 8),
     "ssm_dscan_fwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
+    "ssm_ssd_chunk_state_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
+    "ssm_ssd_mfma_launches": (C.c_int, []),
     "ssm_conv1d_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "ssm_norm_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
 }

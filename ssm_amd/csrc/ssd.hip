@@ -17,6 +17,8 @@ namespace ssm {
 
 constexpr int SSD_THREADS = 256;
 
+static thread_local int g_mfma_launches = 0;   // bit0 bmm_chunk, bit1 chunk_state, bit2 chunk_scan
+
 static unsigned grid_for(size_t n) {
   const size_t g = (n + SSD_THREADS - 1) / SSD_THREADS;
   return (unsigned)(g < 1 ? 1 : g);
@@ -164,6 +166,12 @@ static int dims_check(const char *who, const ssm_ssd_dims &s, SsdDims &d) {
 
 }  // namespace ssm
 
+extern "C" int ssm_ssd_mfma_launches(void) {
+  const int v = ssm::g_mfma_launches;
+  ssm::g_mfma_launches = 0;
+  return v;
+}
+
 extern "C" int ssm_ssd_chunk_cumsum(const ssm_ssd_cumsum_args *a, void *hip_stream) {
   using namespace ssm;
   SSM_REQUIRE(a && a->dt && a->A && a->dA_cumsum && a->dt_out, SSM_ERR_NULL_POINTER,
@@ -201,12 +209,20 @@ extern "C" int ssm_ssd_bmm_chunk(const ssm_ssd_bmm_args *a, void *hip_stream) {
   SSM_REQUIRE(total < ((size_t)1 << 40), SSM_ERR_TOO_LARGE, "ssm_ssd_bmm_chunk: tensor too large");
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   if (!a->force_generic && ssd_bmm_mfma(p, s)) {
+    g_mfma_launches |= 1;
     SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk(mfma)");
     return SSM_OK;
   }
   hipLaunchKernelGGL(ssd_bmm_kernel, dim3(grid_for(total)), dim3(SSD_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk");
   return SSM_OK;
+}
+
+extern "C" size_t ssm_ssd_chunk_state_workspace_bytes(const ssm_ssd_dims *dims) {
+  using namespace ssm;
+  SsdDims d;
+  if (!dims || dims_check("ssm_ssd_chunk_state_workspace_bytes", *dims, d) != SSM_OK) return 0;
+  return ssd_chunk_state_scratch_bytes(d);
 }
 
 extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_stream) {
@@ -219,9 +235,11 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   SSM_REQUIRE(valid_dtype(a->x_dtype) && valid_dtype(a->b_dtype) && valid_dtype(a->states_dtype), SSM_ERR_BAD_DTYPE,
               "ssm_ssd_chunk_state: unsupported dtype");
   p.Bm = a->Bm; p.x = a->x; p.dt = a->dt; p.dA_cs = a->dA_cumsum; p.states = a->states;
+  p.scratch = a->workspace; p.scratch_bytes = a->workspace_bytes;
   p.x_dtype = a->x_dtype; p.b_dtype = a->b_dtype; p.states_dtype = a->states_dtype;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   if (!a->force_generic && ssd_chunk_state_mfma(p, s)) {
+    g_mfma_launches |= 2;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
     return SSM_OK;
   }
@@ -266,6 +284,7 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   p.z_dtype = a->z_dtype; p.d_per_p = a->d_per_p ? 1 : 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
+    g_mfma_launches |= 4;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
     return SSM_OK;
   }

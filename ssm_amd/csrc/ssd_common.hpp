@@ -37,6 +37,8 @@ struct SsdStateParams {
   const void *Bm, *x;
   const float *dt, *dA_cs;
   void *states;
+  void *scratch;              // optional device scratch for the MFMA path (transposed B)
+  size_t scratch_bytes;
   SsdDims d;
   int x_dtype, b_dtype, states_dtype;
 };
@@ -73,6 +75,7 @@ __device__ __forceinline__ float decay_exp(float v) { return exp2_hw(fminf(v, 0.
 // MFMA variants, defined in ssd_mfma.hip; return false when the shape is not covered.
 bool ssd_bmm_mfma(const SsdBmmParams &p, hipStream_t s);
 bool ssd_chunk_state_mfma(const SsdStateParams &p, hipStream_t s);
+size_t ssd_chunk_state_scratch_bytes(const SsdDims &d);
 bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s);
 
 }  // namespace ssm

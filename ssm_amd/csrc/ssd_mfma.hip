@@ -1,8 +1,368 @@
-// bf16 MFMA kernels of the state-space-duality family (placeholder: shapes not yet covered).
+// bf16 MFMA kernels of the state-space-duality family for gfx950
+// (v_mfma_f32_32x32x16_bf16: 32x32 fp32 tile += 32x16 (A) * 16x32 (B)).
+//
+// Register layout of one instruction, lane l of 64:
+//   A operand  8 bf16: row  m = l % 32, k = 8 * (l / 32) + j
+//   B operand  8 bf16: col  n = l % 32, k = 8 * (l / 32) + j
+//   C / D     16 fp32: col  n = l % 32, row m = 8 * (r / 4) + 4 * (l / 32) + r % 4
+// Both operands want the reduction index contiguous per lane.  C B^T and C.S
+// have it contiguous in memory already; contractions over time (chunk_state and
+// the x operand of chunk_scan) read x through an LDS tile transposed on the way
+// in, and chunk_state reads B through a once-per-call transposed copy.
+//
+// Taken for bf16 inputs when L % Q == 0, Q % 32 == 0, Q <= 256, N % 16 == 0 and
+// P is 32 or 64; every other case runs the shape-generic kernels.
 #include "ssd_common.hpp"
 
 namespace ssm {
-bool ssd_bmm_mfma(const SsdBmmParams &, hipStream_t) { return false; }
-bool ssd_chunk_state_mfma(const SsdStateParams &, hipStream_t) { return false; }
-bool ssd_chunk_scan_mfma(const SsdScanParams &, hipStream_t) { return false; }
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+__device__ __forceinline__ f32x16_t mma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ bf16x8_t load_frag(const void *p) { return *reinterpret_cast<const bf16x8_t *>(p); }
+
+__device__ __forceinline__ bf16x8_t pack8(const float (&v)[8]) {
+  bf16x8_t r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = (__bf16)v[j];
+  return r;
+}
+
+__device__ __forceinline__ void unpack8(bf16x8_t r, float (&v)[8]) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (float)r[j];
+}
+
+// Row of C-layout register r for a lane in half g = lane / 32.
+__device__ __forceinline__ int crow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+
+constexpr int MF_THREADS = 256;
+constexpr int MF_WAVES = 4;
+constexpr int XT_PAD = 8;      // bf16 elements of padding per transposed row
+
+// Offset (in bf16 elements) of (p, l) inside the transposed, XOR-swizzled x tile.
+__device__ __forceinline__ int xt_off(int p, int l, int stride) {
+  return p * stride + ((((l >> 3) ^ ((p >> 3) & 7))) << 3) + (l & 7);
+}
+
+// Transpose the [Q][P] bf16 slab x[b, t0.., h, :] into LDS as [P][Q] (optionally
+// scaling row l by w[l]).  A thread moves 8x8 blocks: eight 16-byte global reads
+// along p, eight 16-byte LDS writes along l.
+template <bool WEIGHTED>
+__device__ __forceinline__ void stage_xT(__bf16 *xT, const __bf16 *x, size_t row_stride, int Q, int P,
+                                         const float *w_lds, int stride) {
+  const int pblocks = P >> 3;
+  const int nblocks = (Q >> 3) * pblocks;
+  for (int blk = threadIdx.x; blk < nblocks; blk += MF_THREADS) {
+    const int pb = blk % pblocks, lb = blk / pblocks;
+    float v[8][8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const bf16x8_t raw = load_frag(x + (size_t)(lb * 8 + r) * row_stride + pb * 8);
+      const float w = WEIGHTED ? w_lds[lb * 8 + r] : 1.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[r][i] = WEIGHTED ? (float)raw[i] * w : (float)raw[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      bf16x8_t col;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) col[r] = (__bf16)v[r][i];
+      *reinterpret_cast<bf16x8_t *>(xT + xt_off(pb * 8 + i, lb * 8, stride)) = col;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ bmm_chunk
+// out[b,c,g,l,s] = <a[b,cQ+l,g,:], b[b,cQ+s,g,:]>; one workgroup per 64x64 tile.
+template <typename out_t>
+__global__ __launch_bounds__(MF_THREADS) void ssd_bmm_mfma_kernel(const SsdBmmParams p) {
+  const int Q = p.chunk, K = p.kdim;
+  const int tiles = Q / 64 + (Q % 64 ? 1 : 0);          // 64-wide tiles per side (Q % 32 == 0)
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int unit = blockIdx.x / (tiles * tiles);
+  const int tile = blockIdx.x % (tiles * tiles);
+  const int g = unit % p.groups;
+  const int c = (unit / p.groups) % p.nchunks;
+  const int b = unit / (p.groups * p.nchunks);
+  const int l0 = (tile / tiles) * 64 + (wave >> 1) * 32;
+  const int s0 = (tile % tiles) * 64 + (wave & 1) * 32;
+  if (l0 >= Q || s0 >= Q) return;
+  out_t *out = reinterpret_cast<out_t *>(p.out) + (((size_t)b * p.nchunks + c) * p.groups + g) * (size_t)Q * Q;
+  const int g2 = lane >> 5, m = lane & 31;
+  f32x16_t acc = {0};
+  const bool skip = p.causal && s0 > l0 + 31;
+  if (!skip) {
+    const __bf16 *arow = reinterpret_cast<const __bf16 *>(p.a) + (((size_t)b * p.len + c * Q + l0 + m) * p.groups + g) * K + 8 * g2;
+    const __bf16 *brow = reinterpret_cast<const __bf16 *>(p.b) + (((size_t)b * p.len + c * Q + s0 + m) * p.groups + g) * K + 8 * g2;
+    for (int k0 = 0; k0 < K; k0 += 16) acc = mma(load_frag(arow + k0), load_frag(brow + k0), acc);
+  }
+  const int *sid = p.seq_idx ? p.seq_idx + (size_t)b * p.len + c * Q : nullptr;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int l = l0 + crow(r, g2), s = s0 + m;
+    float v = acc[r];
+    if (p.causal && s > l) v = 0.0f;
+    if (sid && sid[l] != sid[s]) v = 0.0f;
+    out[(size_t)l * Q + s] = from_f32<out_t>(v);
+  }
+}
+
+// ---------------------------------------------------------------- transpose B
+// Bt[b,g,n,t] = Bm[b,t,g,n]   (bf16), tiles of 64 x 64 through LDS.
+__global__ __launch_bounds__(MF_THREADS) void ssd_transpose_kernel(const uint16_t *src, uint16_t *dst, int len, int groups,
+                                                                    int nstate) {
+  __shared__ uint16_t tile[64][66];
+  const int tb = blockIdx.x, nb = blockIdx.y;
+  const int bg = blockIdx.z;
+  const int b = bg / groups, g = bg % groups;
+  for (int e = threadIdx.x; e < 64 * 64; e += MF_THREADS) {
+    const int tl = e / 64, nl = e % 64;
+    const int t = tb * 64 + tl, n = nb * 64 + nl;
+    tile[tl][nl] = (t < len && n < nstate) ? src[(((size_t)b * len + t) * groups + g) * nstate + n] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 64 * 64; e += MF_THREADS) {
+    const int nl = e / 64, tl = e % 64;
+    const int t = tb * 64 + tl, n = nb * 64 + nl;
+    if (t < len && n < nstate) dst[(((size_t)b * groups + g) * nstate + n) * len + t] = tile[tl][nl];
+  }
+}
+
+// ---------------------------------------------------------------- chunk_state
+// states[b,c,h,p,n] = sum_l xw[l][p] * B[l][n];  one workgroup per (b, c, h).
+template <typename st_t, int PT>
+__global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const SsdStateParams p, const __bf16 *Bt) {
+  const SsdDims &d = p.d;
+  const int Q = d.chunk, P = 32 * PT, N = d.nstate;
+  const int stride = Q + XT_PAD;
+  extern __shared__ __align__(16) unsigned char smem[];
+  __bf16 *xT = reinterpret_cast<__bf16 *>(smem);                         // [P][Q + pad]
+  float *w = reinterpret_cast<float *>(smem + (size_t)P * stride * 2);   // [Q]
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int h = blockIdx.x % d.heads;
+  const int c = (blockIdx.x / d.heads) % d.nchunks;
+  const int b = blockIdx.x / (d.heads * d.nchunks);
+  const int g = h / (d.heads / d.groups);
+  const size_t cs = (((size_t)b * d.heads + h) * d.nchunks + c) * Q;
+  const float last = p.dA_cs[cs + Q - 1];
+  for (int l = threadIdx.x; l < Q; l += MF_THREADS) w[l] = decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
+  __syncthreads();
+  const __bf16 *xg = reinterpret_cast<const __bf16 *>(p.x) + (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
+  stage_xT<true>(xT, xg, (size_t)d.heads * P, Q, P, w, stride);
+  __syncthreads();
+
+  const int g2 = lane >> 5, m = lane & 31;
+  st_t *out = reinterpret_cast<st_t *>(p.states) + ((((size_t)b * d.nchunks + c) * d.heads + h) * P) * (size_t)N;
+  for (int n0 = wave * 32; n0 < N; n0 += MF_WAVES * 32) {
+    f32x16_t acc[PT];
+#pragma unroll
+    for (int i = 0; i < PT; ++i) acc[i] = (f32x16_t){0};
+    const bool ncol_ok = n0 + m < N;
+    const __bf16 *bt = Bt + (((size_t)b * d.groups + g) * N + (ncol_ok ? n0 + m : 0)) * (size_t)d.len + (size_t)c * Q + 8 * g2;
+    for (int k0 = 0; k0 < Q; k0 += 16) {
+      bf16x8_t bf = load_frag(bt + k0);
+      if (!ncol_ok) bf = (bf16x8_t){0};
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
+        const bf16x8_t af = load_frag(xT + xt_off(32 * i + m, k0 + 8 * g2, stride));
+        acc[i] = mma(af, bf, acc[i]);
+      }
+    }
+    if (ncol_ok) {
+#pragma unroll
+      for (int i = 0; i < PT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[(size_t)(32 * i + crow(r, g2)) * N + n0 + m] = from_f32<st_t>(acc[i][r]);
+    }
+  }
+}
+
+// ----------------------------------------------------------------- chunk_scan
+// One workgroup per (b, c, h); wave w owns row blocks w, nlb-1-w, w+4, ... of 32 rows.
+template <typename st_t, int PT>
+__global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const SsdScanParams p) {
+  const SsdDims &d = p.d;
+  const int Q = d.chunk, P = 32 * PT, N = d.nstate;
+  const int stride = Q + XT_PAD;
+  extern __shared__ __align__(16) unsigned char smem[];
+  __bf16 *xT = reinterpret_cast<__bf16 *>(smem);                          // [P][Q + pad], unweighted
+  float *dAs = reinterpret_cast<float *>(smem + (size_t)P * stride * 2);  // [Q]
+  float *dts = dAs + Q;                                                   // [Q]
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int h = blockIdx.x % d.heads;
+  const int c = (blockIdx.x / d.heads) % d.nchunks;
+  const int b = blockIdx.x / (d.heads * d.nchunks);
+  const int g = h / (d.heads / d.groups);
+  const size_t cs = (((size_t)b * d.heads + h) * d.nchunks + c) * Q;
+  for (int l = threadIdx.x; l < Q; l += MF_THREADS) {
+    dAs[l] = p.dA_cs[cs + l];
+    dts[l] = p.dt[cs + l];
+  }
+  const size_t xrow = (size_t)d.heads * P;                                 // elements between time steps
+  const size_t xbase = (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
+  const __bf16 *xg = reinterpret_cast<const __bf16 *>(p.x) + xbase;
+  stage_xT<false>(xT, xg, xrow, Q, P, nullptr, stride);
+  __syncthreads();
+
+  const int g2 = lane >> 5, m = lane & 31;
+  const int nlb = Q / 32;
+  const __bf16 *Cg = reinterpret_cast<const __bf16 *>(p.Cm) + (((size_t)b * d.len + (size_t)c * Q) * d.groups + g) * N;
+  const size_t c_stride = (size_t)d.groups * N;
+  const st_t *Sg = reinterpret_cast<const st_t *>(p.prev) + ((((size_t)b * d.nchunks + c) * d.heads + h) * P) * (size_t)N;
+  const __bf16 *CBg = reinterpret_cast<const __bf16 *>(p.CB) + (((size_t)b * d.nchunks + c) * d.groups + g) * (size_t)Q * Q;
+  const __bf16 *zg = p.z ? reinterpret_cast<const __bf16 *>(p.z) + xbase : nullptr;
+  __bf16 *yg = reinterpret_cast<__bf16 *>(p.y) + xbase;
+
+  for (int pair = wave; pair < (nlb + 1) / 2; pair += MF_WAVES) {
+    for (int side = 0; side < 2; ++side) {
+      const int lb = side == 0 ? pair : nlb - 1 - pair;
+      if (side == 1 && lb == pair) break;             // odd count: middle block once
+      const int l0 = 32 * lb;
+      f32x16_t acc[PT];
+#pragma unroll
+      for (int i = 0; i < PT; ++i) acc[i] = (f32x16_t){0};
+
+      // carried-in state: C[l][:] . S[p][:]
+      const __bf16 *crow_p = Cg + (size_t)(l0 + m) * c_stride + 8 * g2;
+      for (int n0 = 0; n0 < N; n0 += 16) {
+        const bf16x8_t af = load_frag(crow_p + n0);
+#pragma unroll
+        for (int i = 0; i < PT; ++i) {
+          bf16x8_t bf;
+          const st_t *sp = Sg + (size_t)(32 * i + m) * N + n0 + 8 * g2;
+          if constexpr (sizeof(st_t) == 2) {
+            bf = load_frag(sp);
+          } else {
+            float t8[8];
+            const float4 lo = *reinterpret_cast<const float4 *>(sp), hi = *reinterpret_cast<const float4 *>(sp + 4);
+            t8[0] = lo.x; t8[1] = lo.y; t8[2] = lo.z; t8[3] = lo.w; t8[4] = hi.x; t8[5] = hi.y; t8[6] = hi.z; t8[7] = hi.w;
+            bf = pack8(t8);
+          }
+          acc[i] = mma(af, bf, acc[i]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float sc = exp2_hw(dAs[l0 + crow(r, g2)] * LOG2E);
+#pragma unroll
+        for (int i = 0; i < PT; ++i) acc[i][r] *= sc;
+      }
+
+      // within the chunk: M[l][s] = CB[l][s] exp(dA_l - dA_s) dt_s for s <= l
+      const int lrow = l0 + m;                       // this lane's row as an A operand
+      const float dal = dAs[lrow];
+      const __bf16 *cbrow = CBg + (size_t)lrow * Q + 8 * g2;
+      for (int s0 = 0; s0 < l0 + 32; s0 += 16) {
+        float cb[8];
+        unpack8(load_frag(cbrow + s0), cb);
+        const int sbase = s0 + 8 * g2;
+        const float4 a0 = *reinterpret_cast<const float4 *>(dAs + sbase), a1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
+        const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
+        const float das[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+        float mv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float v = cb[j] * decay_exp(dal - das[j]) * dtv[j];
+          mv[j] = (sbase + j <= lrow) ? v : 0.0f;
+        }
+        const bf16x8_t af = pack8(mv);
+#pragma unroll
+        for (int i = 0; i < PT; ++i) {
+          const bf16x8_t bf = load_frag(xT + xt_off(32 * i + m, sbase, stride));
+          acc[i] = mma(af, bf, acc[i]);
+        }
+      }
+      // epilogue: + D x, gate, store
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
+        const int pcol = 32 * i + m;
+        const float Dv = p.Dk ? p.Dk[p.d_per_p ? (size_t)h * P + pcol : (size_t)h] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int l = l0 + crow(r, g2);
+          const size_t at = (size_t)l * xrow + pcol;
+          float v = acc[i][r];
+          if (p.Dk) v = __builtin_fmaf(Dv, (float)xg[at], v);
+          if (zg) v *= silu_f32((float)zg[at]);
+          yg[at] = (__bf16)v;
+        }
+      }
+    }
+  }
+}
+
+static bool mfma_shape_ok(const SsdDims &d) {
+  return d.len % d.chunk == 0 && d.chunk % 32 == 0 && d.chunk <= 256 && d.nstate % 16 == 0 &&
+         (d.hdim == 32 || d.hdim == 64);
+}
+
+bool ssd_bmm_mfma(const SsdBmmParams &p, hipStream_t s) {
+  if (p.in_dtype != SSM_BF16 || p.out_dtype == SSM_F16) return false;
+  if (p.len % p.chunk != 0 || p.chunk % 32 != 0 || p.kdim % 16 != 0) return false;
+  if (!aligned_to(p.a, 16) || !aligned_to(p.b, 16)) return false;
+  const int tiles = (p.chunk + 63) / 64;
+  const unsigned grid = (unsigned)((size_t)p.batch * p.nchunks * p.groups * tiles * tiles);
+  if (p.out_dtype == SSM_F32) hipLaunchKernelGGL(ssd_bmm_mfma_kernel<float>, dim3(grid), dim3(MF_THREADS), 0, s, p);
+  else hipLaunchKernelGGL(ssd_bmm_mfma_kernel<bf16_t>, dim3(grid), dim3(MF_THREADS), 0, s, p);
+  return true;
+}
+
+size_t ssd_chunk_state_scratch_bytes(const SsdDims &d) {
+  return (size_t)d.batch * d.groups * d.nstate * d.len * 2;
+}
+
+bool ssd_chunk_state_mfma(const SsdStateParams &p, hipStream_t s) {
+  const SsdDims &d = p.d;
+  if (!mfma_shape_ok(d) || p.x_dtype != SSM_BF16 || p.b_dtype != SSM_BF16 || p.states_dtype == SSM_F16) return false;
+  if (!p.scratch || p.scratch_bytes < ssd_chunk_state_scratch_bytes(d)) return false;
+  if (!aligned_to(p.x, 16) || !aligned_to(p.scratch, 16) || d.len % 8 != 0) return false;
+  __bf16 *Bt = reinterpret_cast<__bf16 *>(p.scratch);
+  hipLaunchKernelGGL(ssd_transpose_kernel, dim3((d.len + 63) / 64, (d.nstate + 63) / 64, d.batch * d.groups),
+                     dim3(MF_THREADS), 0, s, reinterpret_cast<const uint16_t *>(p.Bm), reinterpret_cast<uint16_t *>(Bt),
+                     d.len, d.groups, d.nstate);
+  const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 4;
+  const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);
+#define SSM_LAUNCH_CS(ST, PT)                                                                              \
+  {                                                                                                        \
+    auto kernel = ssd_chunk_state_mfma_kernel<ST, PT>;                                                     \
+    if (allow_dynamic_lds(kernel, lds) != hipSuccess) { (void)hipGetLastError(); return false; }           \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(MF_THREADS), lds, s, p, Bt);                               \
+  }
+  if (p.states_dtype == SSM_F32) {
+    if (d.hdim == 64) SSM_LAUNCH_CS(float, 2) else SSM_LAUNCH_CS(float, 1)
+  } else {
+    if (d.hdim == 64) SSM_LAUNCH_CS(bf16_t, 2) else SSM_LAUNCH_CS(bf16_t, 1)
+  }
+#undef SSM_LAUNCH_CS
+  return true;
+}
+
+bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s) {
+  const SsdDims &d = p.d;
+  if (!mfma_shape_ok(d) || p.x_dtype != SSM_BF16 || p.c_dtype != SSM_BF16 || p.cb_dtype != SSM_BF16) return false;
+  if (p.states_dtype == SSM_F16 || (p.z && p.z_dtype != SSM_BF16)) return false;
+  if (!aligned_to(p.x, 16) || !aligned_to(p.Cm, 16) || !aligned_to(p.CB, 16) || !aligned_to(p.prev, 16)) return false;
+  const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 8;
+  const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);
+#define SSM_LAUNCH_SC(ST, PT)                                                                              \
+  {                                                                                                        \
+    auto kernel = ssd_chunk_scan_mfma_kernel<ST, PT>;                                                      \
+    if (allow_dynamic_lds(kernel, lds) != hipSuccess) { (void)hipGetLastError(); return false; }           \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(MF_THREADS), lds, s, p);                                   \
+  }
+  if (p.states_dtype == SSM_F32) {
+    if (d.hdim == 64) SSM_LAUNCH_SC(float, 2) else SSM_LAUNCH_SC(float, 1)
+  } else {
+    if (d.hdim == 64) SSM_LAUNCH_SC(bf16_t, 2) else SSM_LAUNCH_SC(bf16_t, 1)
+  }
+#undef SSM_LAUNCH_SC
+  return true;
+}
+
 }  // namespace ssm

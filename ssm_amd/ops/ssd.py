@@ -145,9 +145,14 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
     K.check_float("B", Bc)
     dtf, daf = K.as_f32_vec(dt), K.as_f32_vec(dA_cumsum)
     states = torch.empty(batch, nc, heads, hdim, nstate, dtype=states_dtype, device=dev)
+    dims = _dims(batch, seqlen, heads, hdim, groups, nstate, Q)
+    import ctypes
+    nbytes = _lib.load().ssm_ssd_chunk_state_workspace_bytes(ctypes.byref(dims))
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
     args = _lib.SsdChunkStateArgs(
         Bm=_lib.ptr(Bc), x=_lib.ptr(xc), dt=_lib.ptr(dtf), dA_cumsum=_lib.ptr(daf), states=_lib.ptr(states),
-        dims=_dims(batch, seqlen, heads, hdim, groups, nstate, Q), x_dtype=_lib.dtype_enum(xc.dtype),
+        workspace=_lib.ptr(ws), workspace_bytes=nbytes,
+        dims=dims, x_dtype=_lib.dtype_enum(xc.dtype),
         b_dtype=_lib.dtype_enum(Bc.dtype), states_dtype=_lib.dtype_enum(states_dtype),
         force_generic=int(bool(force_generic)))
     _lib.call("ssm_ssd_chunk_state", args, dev)

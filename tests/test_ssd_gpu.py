@@ -131,8 +131,13 @@ def test_bf16_mfma_matches_generic_and_oracle(shape, Q):
     inp = make(11, b, l, h, p, g, n, dtype=torch.bfloat16)
     args = (cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
     kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
+    from ssm_amd import _lib
+    _lib.load().ssm_ssd_mfma_launches()
     y, fin = ssd().ssd_combined(*args, **kw)
+    used = _lib.load().ssm_ssd_mfma_launches()
+    assert used == (7 if l % Q == 0 else 0), f"MFMA kernels used: {used:03b}"
     yg, fing = ssd().ssd_combined(*args, force_generic=True, states_dtype=torch.float32, **kw)
+    assert _lib.load().ssm_ssd_mfma_launches() == 0
     y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
                                 initial_states=inp["init"])
     scale = float(y64.abs().max())
@@ -148,6 +153,8 @@ def test_config3_shape_bf16():
     inp = make(3, 4, 4096, 80, 64, 1, 128, dtype=torch.bfloat16, use_init=False)
     y, fin = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), 256,
                                 D=cu(inp["D"]), z=cu(inp["z"]), return_final_states=True)
+    from ssm_amd import _lib
+    assert _lib.load().ssm_ssd_mfma_launches() & 7 == 7
     assert y.dtype == torch.bfloat16 and fin.dtype == torch.float32 and tuple(fin.shape) == (4, 80, 64, 128)
     hs = [5, 71]
     y64, f64 = S.ssd_sequential(inp["x"][1:2, :, hs], inp["dt"][1:2, :, hs], inp["A"][hs], inp["B"][1:2],
