@@ -48,6 +48,9 @@ typedef enum ssm_proj_kind {
   SSM_PROJ_BGNL = 2   /* (B, G, N, L) grouped and time-varying; channel d reads group d / (D/G) */
 } ssm_proj_kind;
 
+typedef enum ssm_layout { SSM_LAYOUT_BCL = 0, SSM_LAYOUT_BLC = 1 } ssm_layout;
+typedef enum ssm_activation { SSM_ACT_IDENTITY = 0, SSM_ACT_SILU = 1 } ssm_activation;
+
 int ssm_amd_abi_version(void);
 /* Static, human-readable text for a status code. */
 const char *ssm_amd_status_string(int status);
@@ -149,6 +152,27 @@ typedef struct ssm_state_step_args {
 } ssm_state_step_args;
 
 int ssm_state_step(const ssm_state_step_args *args, void *hip_stream);
+
+/* ------------------------------------------------------------------------
+ * fused decode step: roll the causal-conv window, apply the depthwise conv and
+ * its activation to the new input, then run the selective state update on the
+ * result - one launch per token.  It covers what `Mamba1.step` does with
+ * separate tensor ops at src/ssm/modules/mamba1.py:345-353 (window roll, tap
+ * sum, SiLU) followed by `selective_state_step` (:370-381) for callers whose
+ * dt, B and C do not depend on the conv output of the same step.
+ * `step.x` is the raw (pre-conv) input; `step.state` is the SSM state.
+ * ---------------------------------------------------------------------- */
+typedef struct ssm_decode_step_args {
+  ssm_state_step_args step;
+  void *conv_state;          /* (B, D, K) io dtype, rolled in place: [..., 1:] moves left, x appended */
+  const float *conv_weight;  /* (D, K) fp32 */
+  const float *conv_bias;    /* (D,) fp32 or NULL */
+  void *conv_out;            /* (B, D) io dtype or NULL: activated conv output */
+  int32_t conv_width;        /* K */
+  int32_t conv_activation;   /* ssm_activation */
+} ssm_decode_step_args;
+
+int ssm_decode_step(const ssm_decode_step_args *args, void *hip_stream);
 
 /* ------------------------------------------------------------------------
  * diagonal chunk scan: the operator the reference calls `ssd_chunk_scan`
@@ -271,8 +295,6 @@ int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
  * backward behind `dw_causal_conv_backward(grad_out, x, weight, bias,
  * activation)` (formulas: src/ssm/ops/cpu/dw_causal_conv.cpp:161-204).
  * ---------------------------------------------------------------------- */
-typedef enum ssm_layout { SSM_LAYOUT_BCL = 0, SSM_LAYOUT_BLC = 1 } ssm_layout;
-typedef enum ssm_activation { SSM_ACT_IDENTITY = 0, SSM_ACT_SILU = 1 } ssm_activation;
 
 typedef struct ssm_conv1d_fwd_args {
   const void *x;          /* (B,C,L) or (B,L,C), io dtype */

@@ -70,6 +70,11 @@ class StateStepArgs(C.Structure):
     ]
 
 
+class DecodeStepArgs(C.Structure):
+    _fields_ = [("step", StateStepArgs), ("conv_state", _vp), ("conv_weight", _vp), ("conv_bias", _vp),
+                ("conv_out", _vp), ("conv_width", _i32), ("conv_activation", _i32)]
+
+
 CHUNK_HP, CHUNK_BHP, CHUNK_BLHP = 0, 1, 2
 
 
@@ -165,6 +170,7 @@ ENTRY_POINTS = {
     "ssm_scan_fwd": ScanFwdArgs,
     "ssm_scan_bwd": ScanBwdArgs,
     "ssm_state_step": StateStepArgs,
+    "ssm_decode_step": DecodeStepArgs,
     "ssm_dscan_fwd": DscanFwdArgs,
     "ssm_ssd_chunk_cumsum": SsdCumsumArgs,
     "ssm_ssd_bmm_chunk": SsdBmmArgs,

@@ -22,6 +22,12 @@ struct StepParams {
   int b_kind, c_kind, b_groups, c_groups;
   int softplus;
   int tpr_log2;   // lanes per row = 1 << tpr_log2
+  // fused causal-conv front end (decode): x is the raw input, the conv window is rolled in place
+  void *conv_state;          // (B, D, K) io dtype or null
+  const float *conv_w;       // (D, K)
+  const float *conv_b;       // (D,) or null
+  void *conv_out;            // (B, D) io dtype or null: the activated conv output fed to the step
+  int conv_k, conv_silu;
 };
 
 __device__ __forceinline__ void store_from_f32(void *p, int dtype, size_t i, float v) {
@@ -59,7 +65,29 @@ __global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
   float dtv = load_as_f32(p.dt, p.io_dtype, r);
   if (p.bias) dtv += p.bias[d];
   if (p.softplus) dtv = softplus_f32(dtv);
-  const float xv = load_as_f32(p.x, p.io_dtype, r);
+  float xv = load_as_f32(p.x, p.io_dtype, r);
+  if (p.conv_state) {
+    // window <- (window[1:], x); x <- act(bias + sum_k w[k] window[k]).  The row's lanes
+    // share the taps; every lane loads before any lane of the row stores.
+    const int K = p.conv_k;
+    float part = 0.0f;
+    for (int k0 = 0; k0 < K; k0 += tpr) {
+      const int k = k0 + sub;
+      float v = 0.0f;
+      if (k < K) {
+        v = (k < K - 1) ? load_as_f32(p.conv_state, p.io_dtype, r * K + k + 1) : xv;
+        part = __builtin_fmaf(v, p.conv_w[(size_t)d * K + k], part);
+      }
+      if (live && k < K) store_from_f32(p.conv_state, p.io_dtype, r * K + k, v);
+    }
+    for (int m = tpr >> 1; m >= 1; m >>= 1) part += __shfl_xor(part, m, WAVE);
+    if (p.conv_b) part += p.conv_b[d];
+    xv = p.conv_silu ? silu_f32(part) : part;
+    // the step consumes what a separate conv kernel would have written in the io dtype
+    if (p.io_dtype == SSM_BF16) xv = to_f32(from_f32<bf16_t>(xv));
+    else if (p.io_dtype == SSM_F16) xv = to_f32(from_f32<f16_t>(xv));
+    if (p.conv_out && live && sub == 0) store_from_f32(p.conv_out, p.io_dtype, r, xv);
+  }
   const float dx = dtv * xv;
   const float dt2 = dtv * LOG2E;
 
@@ -114,9 +142,27 @@ static int launch_step(const StepParams &p0, bool vec4, hipStream_t stream) {
 
 }  // namespace ssm
 
+static int run_state_step(const ssm_state_step_args *a, const ssm_decode_step_args *dec, void *hip_stream);
+
 extern "C" int ssm_state_step(const ssm_state_step_args *a, void *hip_stream) {
-  using namespace ssm;
   SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_state_step: args is NULL");
+  return run_state_step(a, nullptr, hip_stream);
+}
+
+extern "C" int ssm_decode_step(const ssm_decode_step_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_decode_step: args is NULL");
+  SSM_REQUIRE(a->conv_state && a->conv_weight, SSM_ERR_NULL_POINTER,
+              "ssm_decode_step: conv_state and conv_weight are required");
+  SSM_REQUIRE(a->conv_width > 0 && a->conv_width <= 64, SSM_ERR_BAD_SHAPE, "ssm_decode_step: conv_width=%d",
+              a->conv_width);
+  SSM_REQUIRE(a->conv_activation == SSM_ACT_IDENTITY || a->conv_activation == SSM_ACT_SILU, SSM_ERR_BAD_KIND,
+              "ssm_decode_step: conv_activation=%d", a->conv_activation);
+  return run_state_step(&a->step, a, hip_stream);
+}
+
+static int run_state_step(const ssm_state_step_args *a, const ssm_decode_step_args *dec, void *hip_stream) {
+  using namespace ssm;
   SSM_REQUIRE(a->state && a->x && a->dt && a->A && a->Bproj && a->Cproj && a->out, SSM_ERR_NULL_POINTER,
               "ssm_state_step: state, x, dt, A, Bproj, Cproj and out are required");
   SSM_REQUIRE(a->batch > 0 && a->dim > 0 && a->nstate > 0, SSM_ERR_BAD_SHAPE,
@@ -150,6 +196,13 @@ extern "C" int ssm_state_step(const ssm_state_step_args *a, void *hip_stream) {
   p.c_groups = a->c_kind == SSM_PROJ_BGNL ? a->c_groups : 1;
   p.softplus = a->dt_softplus ? 1 : 0;
   p.tpr_log2 = 0;
+  p.conv_state = nullptr; p.conv_w = nullptr; p.conv_b = nullptr; p.conv_out = nullptr; p.conv_k = 0; p.conv_silu = 0;
+  if (dec) {
+    SSM_REQUIRE(aligned_to(dec->conv_state, es) && (!dec->conv_out || aligned_to(dec->conv_out, es)),
+                SSM_ERR_ALIGNMENT, "ssm_decode_step: a pointer is not aligned to its element size");
+    p.conv_state = dec->conv_state; p.conv_w = dec->conv_weight; p.conv_b = dec->conv_bias;
+    p.conv_out = dec->conv_out; p.conv_k = dec->conv_width; p.conv_silu = dec->conv_activation == SSM_ACT_SILU;
+  }
   const bool vec4 = a->nstate % 4 == 0 && aligned_to(a->state, 4 * ss) && aligned_to(a->A, 16) &&
                     aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs);
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);

@@ -297,6 +297,74 @@ def selective_state_step(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, so
     return out if out.dtype == x.dtype else out.to(x.dtype)
 
 
+class DecodePlan:
+    """A prepared fused decode step (``ssm_decode_step``): rolls ``conv_state`` and
+    updates ``ssm_state`` in place on every :meth:`run`."""
+
+    def __init__(self, conv_state, ssm_state, x, dt, A, B, C, conv_weight, conv_bias=None, D=None, z=None,
+                 dt_bias=None, softplus=True, activation="silu", want_conv_out=False):
+        step = StepPlan(ssm_state, x, dt, A, B, C, D, z, dt_bias, softplus)
+        batch, dim = int(x.shape[0]), int(x.shape[1])
+        if conv_state.ndim != 3 or tuple(conv_state.shape[:2]) != (batch, dim):
+            raise ValueError("conv_state must have shape (B, D, K).")
+        width = int(conv_state.shape[2])
+        w = conv_weight[:, 0, :] if conv_weight.ndim == 3 else conv_weight
+        if tuple(w.shape) != (dim, width):
+            raise ValueError("conv_weight must have shape (D, K) matching conv_state.")
+        if conv_bias is not None and tuple(conv_bias.shape) != (dim,):
+            raise ValueError("conv_bias must have shape (D,).")
+        act = str(activation).lower()
+        if act not in ("silu", "swish", "identity", "none"):
+            raise ValueError(f"Unsupported activation '{activation}'.")
+        K.require_gpu(conv_state, conv_weight, conv_bias, x)
+        io = step.keep["x"].dtype
+        if conv_state.dtype != io or not conv_state.is_contiguous():
+            raise ValueError("conv_state must be contiguous and share the dtype of x, dt and z")
+        self.step = step
+        self.device = step.device
+        self.out = step.out
+        self.keep = dict(w=K.as_f32_vec(w), b=K.as_f32_vec(conv_bias), conv_state=conv_state.detach())
+        self.conv_out = torch.empty(batch, dim, dtype=io, device=self.device) if want_conv_out else None
+        self.args = _lib.DecodeStepArgs(
+            step=step.args, conv_state=_lib.ptr(self.keep["conv_state"]), conv_weight=_lib.ptr(self.keep["w"]),
+            conv_bias=_lib.ptr(self.keep["b"]), conv_out=_lib.ptr(self.conv_out), conv_width=width,
+            conv_activation=_lib.ACT_SILU if act in ("silu", "swish") else _lib.ACT_IDENTITY)
+
+    def run(self):
+        _lib.call("ssm_decode_step", self.args, self.device)
+        return self.out
+
+
+def decode_step(conv_state, ssm_state, x, dt, A, B, C, conv_weight, conv_bias=None, D=None, z=None,
+                dt_bias=None, softplus=True, activation="silu", return_conv_out=False):
+    """One fused decode step: causal-conv window update + activation + selective state update.
+
+    Equivalent to rolling ``conv_state`` left by one, writing ``x`` into its last slot,
+    ``xc = act(bias + sum_k conv_state[..., k] * conv_weight[:, k])`` (rounded to the dtype of
+    ``x``) and ``selective_state_step(ssm_state, xc, dt, A, B, C, D, z, dt_bias, softplus)``;
+    both states are updated in place.
+
+    Args:
+        conv_state: ``(B, D, K)`` window of the last ``K`` inputs, same dtype as ``x``.
+        ssm_state: ``(B, D, N)`` recurrent state.
+        x: New (pre-convolution) input ``(B, D)``.
+        dt, A, B, C, D, z, dt_bias, softplus: as in :func:`selective_state_step`.
+        conv_weight: ``(D, K)`` or ``(D, 1, K)``.
+        conv_bias: Optional ``(D,)``.
+        activation: ``"silu"``/``"swish"`` or ``"identity"``/``"none"``.
+        return_conv_out: Also return the activated convolution output ``(B, D)``.
+
+    Returns:
+        ``y (B, D)`` in ``x.dtype``, or ``(y, conv_out)``.
+    """
+    plan = DecodePlan(conv_state, ssm_state, x, dt, A, B, C, conv_weight, conv_bias, D, z, dt_bias, softplus,
+                      activation, want_conv_out=return_conv_out)
+    y = plan.run()
+    if return_conv_out:
+        return y, plan.conv_out
+    return y
+
+
 # ---------------------------------------------------------------------------
 # diagonal chunk scan (the reference's ``ssd_chunk_scan``)
 # ---------------------------------------------------------------------------
@@ -532,6 +600,7 @@ def fused_layer_norm_with_residual(x, weight, bias, residual=None, is_rms=False,
 __all__ = [
     "selective_scan",
     "selective_state_step",
+    "decode_step",
     "ssd_chunk_scan",
     "dw_causal_conv",
     "fused_layer_norm",

@@ -166,3 +166,34 @@ def test_config2_shape_512_steps():
         if s in check_at:
             torch.testing.assert_close(y[:, idx.cuda()].float().cpu(), yr.float(), **HALF_TOL)
     torch.testing.assert_close(st_gpu[:, idx.cuda()].cpu(), st_ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("io", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("K", [2, 4, 7])
+def test_fused_decode_step_equals_conv_window_then_state_step(io, K):
+    """decode_step == (roll window, tap sum, SiLU) followed by selective_state_step,
+    the sequence of tensor ops in the reference's Mamba1.step."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(K)
+    Bsz, D, N = 3, 40, 16
+    inp = make(K, Bsz, D, N, io=io)
+    conv_state = torch.randn(Bsz, D, K, generator=g).to(io)
+    w = torch.rand(D, K, generator=g) - 0.5
+    cb = torch.randn(D, generator=g) * 0.02
+    # oracle: explicit window update on the CPU, then the oracle step
+    cs_ref = torch.roll(conv_state.float(), -1, dims=-1)
+    cs_ref[..., -1] = inp["x"].float()
+    xc = torch.nn.functional.silu((cs_ref * w).sum(-1) + cb).to(io)
+    st_ref = inp["state"].clone()
+    y_ref = O.selective_state_step(st_ref, xc, inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                                   dt_bias=inp["dt_bias"], softplus=True)
+    cs = conv_state.clone().cuda()
+    st = inp["state"].clone().cuda()
+    y, xc_gpu = ops.decode_step(cs, st, dev(inp["x"]), dev(inp["dt"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]),
+                                w.cuda(), conv_bias=cb.cuda(), D=dev(inp["D"]), z=dev(inp["z"]),
+                                dt_bias=dev(inp["dt_bias"]), softplus=True, return_conv_out=True)
+    tol = FP32_TOL if io == torch.float32 else HALF_TOL
+    torch.testing.assert_close(cs.float().cpu(), cs_ref.to(io).float(), rtol=0, atol=0)
+    torch.testing.assert_close(xc_gpu.float().cpu(), xc.float(), **tol)
+    torch.testing.assert_close(y.float().cpu(), y_ref.float(), **tol)
+    torch.testing.assert_close(st.cpu(), st_ref, **(FP32_TOL if io == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
