@@ -77,6 +77,145 @@ def bench_scan_fwd(steps, warmup, dtype=torch.bfloat16, batch=8, dim=1536, lengt
                 tokens=batch * length)
 
 
+def _time_us(fn, iters=20, warmup=3):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    avg_ms, med_ms = _event_ms(fn, iters)
+    return avg_ms * 1e3
+
+
+def bench_scan_bwd(dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nstate=16):
+    """Forward (with chunk checkpoints) + backward of the config-1 scan, all gradients."""
+    from ssm_amd import configs, ops
+
+    inp = configs.to_device(configs.scan_inputs(batch, dim, length, nstate, dtype=dtype, seed=0))
+    g = torch.Generator().manual_seed(1)
+    go = torch.randn(batch, dim, length, generator=g).to(dtype).cuda()
+    plan = ops.ScanPlan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], inp["D"], inp["z"], inp["dt_bias"],
+                        True, False, want_chunk_states=True)
+    plan.run()
+
+    def bwd(i):
+        ops._scan_backward(go, None, inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], inp["D"], inp["z"],
+                           inp["dt_bias"], True, chunk_states=plan.chunk_states)
+    us = _time_us(bwd, iters=10)
+    elt = 2 if dtype != torch.float32 else 4
+    nbytes = 7 * elt * batch * dim * length + 2 * elt * batch * nstate * length + 2 * 4 * batch * nstate * length
+    return {"kernel_us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
+            "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes}
+
+
+def bench_conv(dtype=torch.bfloat16, batch=8, chans=1536, length=2048, width=4):
+    from ssm_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    xs = [torch.randn(batch, chans, length, generator=g).to(dtype).cuda() for _ in range(3)]
+    w = (torch.rand(chans, width, generator=g) - 0.5).cuda()
+    b = (torch.randn(chans, generator=g) * 0.02).cuda()
+    go = torch.randn(batch, chans, length, generator=g).to(dtype).cuda()
+    elt = 2 if dtype != torch.float32 else 4
+    fwd_us = _time_us(lambda i: ops._conv_forward(xs[i % 3], w, b, "silu"))
+    bwd_us = _time_us(lambda i: ops._conv_backward(go, xs[i % 3], w, b, "silu"))
+    fb, bb = 2 * elt * batch * chans * length, 3 * elt * batch * chans * length
+    return {"fwd_us": round(fwd_us, 1), "fwd_GBps": round(fb / fwd_us / 1e3, 1),
+            "fwd_frac_hbm": round(fb / fwd_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bwd_us": round(bwd_us, 1), "bwd_GBps": round(bb / bwd_us / 1e3, 1),
+            "bwd_frac_hbm": round(bb / bwd_us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+
+def bench_norm(batch=16, length=2048, hidden=768):
+    from ssm_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    xs = [torch.randn(batch, length, hidden, generator=g).to(torch.bfloat16).cuda() for _ in range(3)]
+    rs = [torch.randn(batch, length, hidden, generator=g).cuda() for _ in range(3)]
+    w = torch.randn(hidden, generator=g).cuda()
+    us = _time_us(lambda i: ops._norm_forward(xs[i % 3], w, None, rs[i % 3], True, 1e-5, True, True,
+                                              want_residual_out=True))
+    nbytes = batch * length * hidden * (2 + 4 + 2 + 4)
+    return {"fwd_us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
+            "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes,
+            "shape": "x bf16 (16,2048,768) + fp32 residual -> y bf16 + fp32 residual_out, RMSNorm"}
+
+
+def bench_decode(batch=64, dim=5120, nstate=16, width=4, steps=512):
+    """Config 2: 512 consecutive in-place decode steps (fused conv window + state update),
+    bf16 activations, fp32 SSM state, grouped B/C (64,1,16)."""
+    from ssm_amd import configs, ops
+
+    g = torch.Generator().manual_seed(2)
+    ssm_state = torch.randn(batch, dim, nstate, generator=g).cuda()
+    conv_state = torch.randn(batch, dim, width, generator=g).to(torch.bfloat16).cuda()
+    A = -torch.arange(1, nstate + 1, dtype=torch.float32).repeat(dim, 1).cuda()
+    D = torch.ones(dim).cuda()
+    bias = configs.inverse_softplus_dt(dim, g).cuda()
+    w = (torch.rand(dim, width, generator=g) - 0.5).cuda()
+    cb = (torch.randn(dim, generator=g) * 0.02).cuda()
+    nset = 8
+    plans = []
+    for _ in range(nset):
+        x = torch.randn(batch, dim, generator=g).to(torch.bfloat16).cuda()
+        z = torch.randn(batch, dim, generator=g).to(torch.bfloat16).cuda()
+        dt = torch.randn(batch, dim, generator=g).to(torch.bfloat16).cuda()
+        Bm = torch.randn(batch, 1, nstate, generator=g).to(torch.bfloat16).cuda()
+        Cm = torch.randn(batch, 1, nstate, generator=g).to(torch.bfloat16).cuda()
+        plans.append(ops.DecodePlan(conv_state, ssm_state, x, dt, A, Bm, Cm, w, cb, D, z, bias, True))
+    for i in range(16):
+        plans[i % nset].run()
+    torch.cuda.synchronize()
+    # eager launches from Python
+    t0 = time.perf_counter()
+    for i in range(steps):
+        plans[i % nset].run()
+    torch.cuda.synchronize()
+    eager_us = (time.perf_counter() - t0) / steps * 1e6
+    # the same 512 launches captured once in a HIP graph and replayed
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(steps):
+                plans[i % nset].run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph.replay()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(3):
+        graph.replay()
+    e.record()
+    torch.cuda.synchronize()
+    graph_us = s.elapsed_time(e) / 3 / steps * 1e3
+    nbytes = 2 * 4 * batch * dim * nstate + 4 * 2 * batch * dim + 2 * 2 * batch * dim * width + 4 * dim * (nstate + 2 + width + 1)
+    return {"us_per_step_graph": round(graph_us, 2), "us_per_step_eager": round(eager_us, 2), "steps": steps,
+            "GBps_graph": round(nbytes / graph_us / 1e3, 1),
+            "frac_hbm_graph": round(nbytes / graph_us / 1e3 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes}
+
+
+def bench_ssd(batch=4, length=4096, heads=80, hdim=64, nstate=128, chunk=256):
+    """Config 3: Mamba-2 SSD forward, bf16, returns y and final states."""
+    from ssm_amd.ops import ssd
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(batch, length, heads, hdim, generator=g).to(torch.bfloat16).cuda()
+    from ssm_amd import configs
+    dt_bias = configs.inverse_softplus_dt(heads, g)
+    dt = torch.nn.functional.softplus(torch.randn(batch, length, heads, generator=g) + dt_bias).cuda()
+    A = -(torch.rand(heads, generator=g) * 15 + 1).cuda()
+    Bm = torch.randn(batch, length, 1, nstate, generator=g).to(torch.bfloat16).cuda()
+    Cm = torch.randn(batch, length, 1, nstate, generator=g).to(torch.bfloat16).cuda()
+    D = torch.ones(heads).cuda()
+    z = torch.randn(batch, length, heads, hdim, generator=g).to(torch.bfloat16).cuda()
+    us = _time_us(lambda i: ssd.ssd_combined(x, dt, A, Bm, Cm, chunk, D=D, z=z, return_final_states=True), iters=10)
+    nc = length // chunk
+    flops = (2 * chunk * chunk * nstate * batch * nc + 2 * chunk * chunk * hdim * batch * nc * heads
+             + 2 * 2 * chunk * nstate * hdim * batch * nc * heads)
+    return {"us": round(us, 1), "TFLOPs": round(flops / us / 1e6, 1),
+            "frac_mfma_bf16_peak": round(flops / us / 1e6 / 2500.0, 4), "dense_tile_flops": flops}
+
+
 def cpu_baseline_scan(dtype=torch.bfloat16, dim=1536, length=2048, nstate=16, budget_s=15.0):
     """Time the CPU restatement of the reference's Python loop on a batch slice
     of the headline workload; returns GB/s of the same algorithmic bytes."""
@@ -157,6 +296,11 @@ def main():
         extra["selective_scan_fwd_fp32_io"] = {
             "kernel_us": round(r32["kernel_ms"] * 1e3, 2), "GBps": round(a32, 1),
             "frac_hbm": round(a32 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": r32["bytes"]}
+        extra["selective_scan_bwd_bf16"] = bench_scan_bwd()
+        extra["dw_causal_conv_bf16"] = bench_conv()
+        extra["fused_add_rmsnorm"] = bench_norm()
+        extra["decode_step_config2"] = bench_decode()
+        extra["ssd_combined_config3"] = bench_ssd()
         line["extra"] = extra
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_scan()
