@@ -67,6 +67,11 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
 
   int tune = a->tune_items;
   if (tune == 0) tune = (a->seqlen <= 256 && !a->chunk_states) ? 408 : 808;
+  // tune 1616: slab of 16 states shared by 16 channels (two per wave)
+  if (tune == 1616) {
+    if (bvary && cvary && a->nstate <= 16 && per_b % 16 == 0 && per_c % 16 == 0) rows = 2 * SCAN_MAX_WAVES;
+    else tune = 816;
+  }
   if (a->chunk_states)
     SSM_REQUIRE(tune / 100 * WAVE == ssm_scan_chunk_len(), SSM_ERR_BAD_KIND,
                 "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (tune_items 808 or 816)",

@@ -131,46 +131,43 @@ __device__ __forceinline__ void wave_scan_affine_x1(float &a0, float &b0) {
 // Note: after the last step only b (the composed offset) is complete in every
 // lane; a is complete in rows 0-1 only and is not used afterwards.
 
-template <typename io_t, int K, int NB, bool BVARY, bool CVARY, bool SMALLN>
+// RPW rows per wave share one staged B/C slab (only used when all N states fit one
+// slab, so that nothing has to persist per row across slabs).
+template <typename io_t, int K, int NB, bool BVARY, bool CVARY, bool SMALLN, int RPW>
 __global__ __launch_bounds__(WAVE *SCAN_MAX_WAVES) void scan_fwd_kernel(const ScanFwdParams p) {
   constexpr int T = WAVE * K;
   extern __shared__ __align__(16) float tiles[];           // B tile [NB][T] then C tile [NB][T]
   __shared__ float carry_hi[SMALLN ? 1 : SCAN_MAX_WAVES][SMALLN ? 1 : SCAN_MAX_N - SCAN_LANE_STATES];
 
-  const int rows = (int)(blockDim.x >> 6);
+  const int waves = (int)(blockDim.x >> 6);
+  const int rows = waves * RPW;                            // channels per workgroup
   const int wave = wave_id_uniform();
   const int lane = lane_id();
   const int blocks_per_batch = p.dim / rows;
   const int b = (int)blockIdx.x / blocks_per_batch;
   const int d0 = ((int)blockIdx.x % blocks_per_batch) * rows;
-  const int d = d0 + wave;
   const int L = p.len, N = p.nstate;
-
-  const size_t row = (size_t)b * p.dim + d;
-  const io_t *u_row = reinterpret_cast<const io_t *>(p.u) + row * L;
-  const io_t *dl_row = reinterpret_cast<const io_t *>(p.delta) + row * L;
-  const io_t *z_row = p.z ? reinterpret_cast<const io_t *>(p.z) + row * L : nullptr;
-  io_t *out_row = reinterpret_cast<io_t *>(p.out) + row * L;
-  const float *A_row = p.A + (size_t)d * N;
-  const float Dk = p.Dk ? p.Dk[d] : 0.0f;
-  const float bias = p.bias ? p.bias[d] : 0.0f;
   const bool vec_ok = p.vec_ok != 0;
 
   constexpr bool bvary = BVARY, cvary = CVARY;
   float *Bs = tiles;
   float *Cs = tiles + (bvary ? NB * T : 0);
-  // element offset of this row's (or this group's) projection at n = 0, t = 0
-  size_t b_off, c_off;
-  if (bvary) b_off = ((size_t)b * p.b_groups + d0 / (p.dim / p.b_groups)) * (size_t)N * L;
-  else b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
-  if (cvary) c_off = ((size_t)b * p.c_groups + d0 / (p.dim / p.c_groups)) * (size_t)N * L;
-  else c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+  size_t b_tile = 0, c_tile = 0;     // element offset of the group's projection at n = 0, t = 0
+  if (bvary) b_tile = ((size_t)b * p.b_groups + d0 / (p.dim / p.b_groups)) * (size_t)N * L;
+  if (cvary) c_tile = ((size_t)b * p.c_groups + d0 / (p.dim / p.c_groups)) * (size_t)N * L;
 
   // per-row constants spread over lanes: lane n holds the value for state n (n < 64)
-  const float A2_lanes = lane < N ? A_row[lane] * LOG2E : 0.0f;
-  const float Bc_lanes = (!bvary && lane < N) ? load_as_f32(p.Bp, p.bc_dtype, b_off + lane) : 0.0f;
-  const float Cc_lanes = (!cvary && lane < N) ? load_as_f32(p.Cp, p.bc_dtype, c_off + lane) : 0.0f;
-  float carry_lanes = 0.0f;
+  float A2_lanes[RPW], Bc_lanes[RPW], Cc_lanes[RPW], carry_lanes[RPW];
+#pragma unroll
+  for (int rr = 0; rr < RPW; ++rr) {
+    const int d = d0 + wave * RPW + rr;
+    A2_lanes[rr] = lane < N ? p.A[(size_t)d * N + lane] * LOG2E : 0.0f;
+    const size_t bo = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+    const size_t co = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+    Bc_lanes[rr] = (!bvary && lane < N) ? load_as_f32(p.Bp, p.bc_dtype, bo + lane) : 0.0f;
+    Cc_lanes[rr] = (!cvary && lane < N) ? load_as_f32(p.Cp, p.bc_dtype, co + lane) : 0.0f;
+    carry_lanes[rr] = 0.0f;
+  }
   if (!SMALLN)
     for (int n = SCAN_LANE_STATES + lane; n < N; n += WAVE) carry_hi[wave][n - SCAN_LANE_STATES] = 0.0f;
 
@@ -178,151 +175,159 @@ __global__ __launch_bounds__(WAVE *SCAN_MAX_WAVES) void scan_fwd_kernel(const Sc
   for (int c = 0; c < nchunks; ++c) {
     const int t0 = c * T;
     const int t = t0 + lane * K;
-    if (p.chunk_states) {
-      float *cs = p.chunk_states + (row * nchunks + c) * (size_t)N;
-      if (lane < N) cs[lane] = carry_lanes;
-      if (!SMALLN)
-        for (int n = SCAN_LANE_STATES + lane; n < N; n += WAVE) cs[n] = carry_hi[wave][n - SCAN_LANE_STATES];
-    }
-
     float dl[K], du[K], y[K];
-    {
-      float uu[K];
-      load_run<io_t, K>(u_row, t, L, vec_ok, uu);
-      load_run<io_t, K>(dl_row, t, L, vec_ok, dl);
-#pragma unroll
-      for (int i = 0; i < K; ++i) {
-        float dv = dl[i] + bias;
-        if (p.softplus) dv = softplus_f32(dv);
-        dv = (t + i < L) ? dv : 0.0f;      // steps past the end are the identity map
-        dl[i] = dv;
-        du[i] = dv * uu[i];
-        y[i] = Dk * uu[i];
-      }
-    }
     float dsum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < K; ++i) dsum += dl[i];
 
     for (int nb = 0; nb < N; nb += NB) {
       const int nn = min(NB, N - nb);
       if constexpr (bvary || cvary) {
         __syncthreads();   // every wave is done with the previous slab
-        if constexpr (bvary) stage_tile<K>(Bs, p.Bp, p.bc_dtype, b_off + (size_t)nb * L, L, t0, nn, p.bc_vec_ok != 0);
-        if constexpr (cvary) stage_tile<K>(Cs, p.Cp, p.bc_dtype, c_off + (size_t)nb * L, L, t0, nn, p.bc_vec_ok != 0);
+        if constexpr (bvary) stage_tile<K>(Bs, p.Bp, p.bc_dtype, b_tile + (size_t)nb * L, L, t0, nn, p.bc_vec_ok != 0);
+        if constexpr (cvary) stage_tile<K>(Cs, p.Cp, p.bc_dtype, c_tile + (size_t)nb * L, L, t0, nn, p.bc_vec_ok != 0);
         __syncthreads();
       }
 
-      // One or two state indices at a time.  W is a compile-time width so that
-      // the per-state arrays stay in registers.
-      auto process = [&](auto width_tag, int nl) {
-        constexpr int W = decltype(width_tag)::value;
-        float a[W][K], bx[W][K], P[W], h[W], A2[W], H[W], cconst[W];
 #pragma unroll
-        for (int w = 0; w < W; ++w) {
-          const int n = nb + nl + w;
-          A2[w] = (SMALLN || n < SCAN_LANE_STATES) ? wave_read_lane(A2_lanes, n) : A_row[n] * LOG2E;
-          const float bconst = bvary ? 0.0f
-                                     : ((SMALLN || n < SCAN_LANE_STATES) ? wave_read_lane(Bc_lanes, n)
-                                                             : load_as_f32(p.Bp, p.bc_dtype, b_off + n));
-          cconst[w] = cvary ? 0.0f
-                            : ((SMALLN || n < SCAN_LANE_STATES) ? wave_read_lane(Cc_lanes, n)
-                                                    : load_as_f32(p.Cp, p.bc_dtype, c_off + n));
-          H[w] = (SMALLN || n < SCAN_LANE_STATES) ? wave_read_lane(carry_lanes, n) : carry_hi[wave][n - SCAN_LANE_STATES];
-          // fold the lane's K steps into (P, h): state_out = P * state_in + h
-#pragma unroll
-          for (int q = 0; q < K / 4; ++q) {
-            float4 bv;
-            if constexpr (bvary) bv = *reinterpret_cast<const float4 *>(Bs + (nl + w) * T + q * (WAVE * 4) + lane * 4);
-            else bv = make_float4(bconst, bconst, bconst, bconst);
-            const float bq[4] = {bv.x, bv.y, bv.z, bv.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int i = q * 4 + j;
-#if defined(SSM_ABLATE_EXP)
-              a[w][i] = dl[i] * A2[w] + 0.9f;
-#else
-              a[w][i] = exp2_hw(dl[i] * A2[w]);
-#endif
-              bx[w][i] = du[i] * bq[j];
-              h[w] = i == 0 ? bx[w][0] : __builtin_fmaf(a[w][i], h[w], bx[w][i]);
-            }
+      for (int rr = 0; rr < RPW; ++rr) {
+        const int d = d0 + wave * RPW + rr;
+        const size_t row = (size_t)b * p.dim + d;
+        const float *A_row = p.A + (size_t)d * N;
+        const size_t b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+        const size_t c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+
+        if (nb == 0) {
+          // load this row's K steps per lane: delta' and delta' * u, y starts at D * u
+          const float Dk = p.Dk ? p.Dk[d] : 0.0f;
+          const float bias = p.bias ? p.bias[d] : 0.0f;
+          float uu[K];
+          load_run<io_t, K>(reinterpret_cast<const io_t *>(p.u) + row * L, t, L, vec_ok, uu);
+          load_run<io_t, K>(reinterpret_cast<const io_t *>(p.delta) + row * L, t, L, vec_ok, dl);
+          if (p.chunk_states) {
+            float *cs = p.chunk_states + (row * nchunks + c) * (size_t)N;
+            if (lane < N) cs[lane] = carry_lanes[rr];
+            if (!SMALLN)
+              for (int n = SCAN_LANE_STATES + lane; n < N; n += WAVE) cs[n] = carry_hi[wave][n - SCAN_LANE_STATES];
           }
-          P[w] = exp2_hw(dsum * A2[w]);
-          // lane 0 absorbs the state carried in from the previous chunk
-          h[w] = __builtin_fmaf(P[w], lane == 0 ? H[w] : 0.0f, h[w]);
-        }
-#if !defined(SSM_ABLATE_SCAN)
-        if constexpr (W == 2) wave_scan_affine_x2(P[0], h[0], P[1], h[1]);
-        else wave_scan_affine_x1(P[0], h[0]);
-#endif
+          dsum = 0.0f;
 #pragma unroll
-        for (int w = 0; w < W; ++w) {
-          const int n = nb + nl + w;
-          // h[w] is now the row state at the END of each lane's run
-          float hs = wave_prev(h[w], H[w]);                       // state entering this lane
-          const float hend = wave_read_lane(h[w], WAVE - 1);      // state leaving the chunk
-          if (SMALLN || n < SCAN_LANE_STATES) {
-            carry_lanes = lane == n ? hend : carry_lanes;
-          } else if (lane == 0) {
-            carry_hi[wave][n - SCAN_LANE_STATES] = hend;
-          }
-          // replay the K steps from the true entering state
-#pragma unroll
-          for (int q = 0; q < K / 4; ++q) {
-            float4 cv;
-            if constexpr (cvary) cv = *reinterpret_cast<const float4 *>(Cs + (nl + w) * T + q * (WAVE * 4) + lane * 4);
-            else cv = make_float4(cconst[w], cconst[w], cconst[w], cconst[w]);
-            const float cq[4] = {cv.x, cv.y, cv.z, cv.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int i = q * 4 + j;
-#if defined(SSM_ABLATE_PASS2)
-              if (i == 0) y[i] = __builtin_fmaf(hs + a[w][K - 1] + bx[w][K - 1], cq[j], y[i]);
-#else
-              hs = __builtin_fmaf(a[w][i], hs, bx[w][i]);
-              y[i] = __builtin_fmaf(hs, cq[j], y[i]);
-#endif
-            }
+          for (int i = 0; i < K; ++i) {
+            float dv = dl[i] + bias;
+            if (p.softplus) dv = softplus_f32(dv);
+            dv = (t + i < L) ? dv : 0.0f;      // steps past the end are the identity map
+            dl[i] = dv;
+            du[i] = dv * uu[i];
+            y[i] = Dk * uu[i];
+            dsum += dv;
           }
         }
-      };
 
-      int nl = 0;
-      for (; nl + 2 <= nn; nl += 2) process(std::integral_constant<int, 2>{}, nl);
-      if (nl < nn) process(std::integral_constant<int, 1>{}, nl);
-    }
-
-    if (z_row) {
-      float zz[K];
-      load_run<io_t, K>(z_row, t, L, vec_ok, zz);
+        // One or two state indices at a time.  W is a compile-time width so that
+        // the per-state arrays stay in registers.
+        auto process = [&](auto width_tag, int nl) {
+          constexpr int W = decltype(width_tag)::value;
+          float a[W][K], bx[W][K], P[W], h[W], A2[W], H[W], cconst[W];
 #pragma unroll
-      for (int i = 0; i < K; ++i) y[i] *= silu_f32(zz[i]);
+          for (int w = 0; w < W; ++w) {
+            const int n = nb + nl + w;
+            const bool in_lanes = SMALLN || n < SCAN_LANE_STATES;
+            A2[w] = in_lanes ? wave_read_lane(A2_lanes[rr], n) : A_row[n] * LOG2E;
+            const float bconst = bvary ? 0.0f
+                                       : (in_lanes ? wave_read_lane(Bc_lanes[rr], n)
+                                                   : load_as_f32(p.Bp, p.bc_dtype, b_off + n));
+            cconst[w] = cvary ? 0.0f
+                              : (in_lanes ? wave_read_lane(Cc_lanes[rr], n) : load_as_f32(p.Cp, p.bc_dtype, c_off + n));
+            H[w] = in_lanes ? wave_read_lane(carry_lanes[rr], n) : carry_hi[wave][n - SCAN_LANE_STATES];
+            // fold the lane's K steps into (P, h): state_out = P * state_in + h
+#pragma unroll
+            for (int q = 0; q < K / 4; ++q) {
+              float4 bv;
+              if constexpr (bvary) bv = *reinterpret_cast<const float4 *>(Bs + (nl + w) * T + q * (WAVE * 4) + lane * 4);
+              else bv = make_float4(bconst, bconst, bconst, bconst);
+              const float bq[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int i = q * 4 + j;
+                a[w][i] = exp2_hw(dl[i] * A2[w]);
+                bx[w][i] = du[i] * bq[j];
+                h[w] = i == 0 ? bx[w][0] : __builtin_fmaf(a[w][i], h[w], bx[w][i]);
+              }
+            }
+            P[w] = exp2_hw(dsum * A2[w]);
+            // lane 0 absorbs the state carried in from the previous chunk
+            h[w] = __builtin_fmaf(P[w], lane == 0 ? H[w] : 0.0f, h[w]);
+          }
+          if constexpr (W == 2) wave_scan_affine_x2(P[0], h[0], P[1], h[1]);
+          else wave_scan_affine_x1(P[0], h[0]);
+#pragma unroll
+          for (int w = 0; w < W; ++w) {
+            const int n = nb + nl + w;
+            // h[w] is now the row state at the END of each lane's run
+            float hs = wave_prev(h[w], H[w]);                       // state entering this lane
+            const float hend = wave_read_lane(h[w], WAVE - 1);      // state leaving the chunk
+            if (SMALLN || n < SCAN_LANE_STATES) {
+              carry_lanes[rr] = lane == n ? hend : carry_lanes[rr];
+            } else if (lane == 0) {
+              carry_hi[wave][n - SCAN_LANE_STATES] = hend;
+            }
+            // replay the K steps from the true entering state
+#pragma unroll
+            for (int q = 0; q < K / 4; ++q) {
+              float4 cv;
+              if constexpr (cvary) cv = *reinterpret_cast<const float4 *>(Cs + (nl + w) * T + q * (WAVE * 4) + lane * 4);
+              else cv = make_float4(cconst[w], cconst[w], cconst[w], cconst[w]);
+              const float cq[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int i = q * 4 + j;
+                hs = __builtin_fmaf(a[w][i], hs, bx[w][i]);
+                y[i] = __builtin_fmaf(hs, cq[j], y[i]);
+              }
+            }
+          }
+        };
+
+        int nl = 0;
+        for (; nl + 2 <= nn; nl += 2) process(std::integral_constant<int, 2>{}, nl);
+        if (nl < nn) process(std::integral_constant<int, 1>{}, nl);
+
+        if (nb + NB >= N) {
+          if (p.z) {
+            float zz[K];
+            load_run<io_t, K>(reinterpret_cast<const io_t *>(p.z) + row * L, t, L, vec_ok, zz);
+#pragma unroll
+            for (int i = 0; i < K; ++i) y[i] *= silu_f32(zz[i]);
+          }
+          store_run<io_t, K>(reinterpret_cast<io_t *>(p.out) + row * L, t, L, vec_ok, y);
+        }
+      }
     }
-    store_run<io_t, K>(out_row, t, L, vec_ok, y);
   }
 
   if (p.last) {
-    io_t *last_row = reinterpret_cast<io_t *>(p.last) + row * N;
-    if (lane < N) last_row[lane] = from_f32<io_t>(carry_lanes);
-    if (!SMALLN)
-      for (int n = SCAN_LANE_STATES + lane; n < N; n += WAVE)
-        last_row[n] = from_f32<io_t>(carry_hi[wave][n - SCAN_LANE_STATES]);
+#pragma unroll
+    for (int rr = 0; rr < RPW; ++rr) {
+      const size_t row = (size_t)b * p.dim + d0 + wave * RPW + rr;
+      io_t *last_row = reinterpret_cast<io_t *>(p.last) + row * N;
+      if (lane < N) last_row[lane] = from_f32<io_t>(carry_lanes[rr]);
+      if (!SMALLN)
+        for (int n = SCAN_LANE_STATES + lane; n < N; n += WAVE)
+          last_row[n] = from_f32<io_t>(carry_hi[wave][n - SCAN_LANE_STATES]);
+    }
   }
 }
 
-
-template <typename io_t, int K, int NB, bool BV, bool CV, bool SN>
+template <typename io_t, int K, int NB, bool BV, bool CV, bool SN, int RPW>
 static int launch_scan_fwd(const ScanFwdParams &p, int rows, hipStream_t stream) {
   const size_t lds = (size_t)((int)BV + (int)CV) * NB * WAVE * K * sizeof(float);
-  auto kernel = scan_fwd_kernel<io_t, K, NB, BV, CV, SN>;
+  auto kernel = scan_fwd_kernel<io_t, K, NB, BV, CV, SN, RPW>;
   if (allow_dynamic_lds(kernel, lds) != hipSuccess) {
     (void)hipGetLastError();
     set_error("ssm_scan_fwd: cannot reserve %zu bytes of LDS", lds);
     return SSM_ERR_LAUNCH;
   }
+  // `rows` channels per workgroup = waves * RPW
   const unsigned grid = (unsigned)((size_t)p.batch * (p.dim / rows));
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(WAVE * rows), lds, stream, p);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(WAVE * (rows / RPW)), lds, stream, p);
   SSM_CHECK_LAUNCH("ssm_scan_fwd");
   return SSM_OK;
 }
@@ -331,16 +336,18 @@ template <typename io_t, int K, int NB>
 static int dispatch_flags(const ScanFwdParams &p, int rows, hipStream_t s) {
   const bool bv = p.b_kind == SSM_PROJ_BGNL, cv = p.c_kind == SSM_PROJ_BGNL;
   const bool sn = p.nstate <= SCAN_LANE_STATES;
+  // two rows per wave when a workgroup of 16 channels fits one group and all states fit one slab
+  if (bv && cv && sn && rows == 2 * SCAN_MAX_WAVES) return launch_scan_fwd<io_t, K, NB, true, true, true, 2>(p, rows, s);
   const int key = (bv ? 4 : 0) | (cv ? 2 : 0) | (sn ? 1 : 0);
   switch (key) {
-    case 0: return launch_scan_fwd<io_t, K, NB, false, false, false>(p, rows, s);
-    case 1: return launch_scan_fwd<io_t, K, NB, false, false, true>(p, rows, s);
-    case 2: return launch_scan_fwd<io_t, K, NB, false, true, false>(p, rows, s);
-    case 3: return launch_scan_fwd<io_t, K, NB, false, true, true>(p, rows, s);
-    case 4: return launch_scan_fwd<io_t, K, NB, true, false, false>(p, rows, s);
-    case 5: return launch_scan_fwd<io_t, K, NB, true, false, true>(p, rows, s);
-    case 6: return launch_scan_fwd<io_t, K, NB, true, true, false>(p, rows, s);
-    default: return launch_scan_fwd<io_t, K, NB, true, true, true>(p, rows, s);
+    case 0: return launch_scan_fwd<io_t, K, NB, false, false, false, 1>(p, rows, s);
+    case 1: return launch_scan_fwd<io_t, K, NB, false, false, true, 1>(p, rows, s);
+    case 2: return launch_scan_fwd<io_t, K, NB, false, true, false, 1>(p, rows, s);
+    case 3: return launch_scan_fwd<io_t, K, NB, false, true, true, 1>(p, rows, s);
+    case 4: return launch_scan_fwd<io_t, K, NB, true, false, false, 1>(p, rows, s);
+    case 5: return launch_scan_fwd<io_t, K, NB, true, false, true, 1>(p, rows, s);
+    case 6: return launch_scan_fwd<io_t, K, NB, true, true, false, 1>(p, rows, s);
+    default: return launch_scan_fwd<io_t, K, NB, true, true, true, 1>(p, rows, s);
   }
 }
 
@@ -351,8 +358,9 @@ int scan_fwd_dispatch(const ScanFwdParams &p, int tune, int rows, hipStream_t s)
     case 408: return dispatch_flags<io_t, 4, 8>(p, rows, s);
     case 808: return dispatch_flags<io_t, 8, 8>(p, rows, s);
     case 816: return dispatch_flags<io_t, 8, 16>(p, rows, s);
+    case 1616: return dispatch_flags<io_t, 8, 16>(p, rows, s);      // 816 with two rows per wave (see entry point)
     default:
-      set_error("ssm_scan_fwd: unsupported tune_items %d (408, 808, 816)", tune);
+      set_error("ssm_scan_fwd: unsupported tune_items %d (408, 808, 816, 1616)", tune);
       return SSM_ERR_BAD_KIND;
   }
 }
