@@ -85,7 +85,8 @@ typedef struct ssm_scan_fwd_args {
   int32_t b_kind, c_kind; /* ssm_proj_kind */
   int32_t b_groups, c_groups; /* G for SSM_PROJ_BGNL (must divide D), else ignored */
   int32_t delta_softplus; /* 0 / 1 */
-  int32_t tune_items;     /* 0 = automatic; else 100 * steps-per-lane + states-per-LDS-pass (408, 808, 816) */
+  int32_t tune_items;     /* 0 = automatic; else 100 * steps-per-lane + states-per-LDS-pass (408, 808, 816);
+                             1616 = 816 with two channels per wave */
 } ssm_scan_fwd_args;
 
 int ssm_scan_fwd(const ssm_scan_fwd_args *args, void *hip_stream);
@@ -220,7 +221,8 @@ int ssm_dscan_fwd(const ssm_dscan_fwd_args *args, void *hip_stream);
  * bf16 MFMA kernels (used by the tests to cross-check them).
  * ---------------------------------------------------------------------- */
 /* Which of the calls made by this thread since the last query ran a bf16 MFMA
- * kernel: bit 0 bmm_chunk, bit 1 chunk_state, bit 2 chunk_scan.  Resets on read. */
+ * kernel: bit 0 bmm_chunk, bit 1 chunk_state, bit 2 chunk_scan, bit 3 the one-pass
+ * ssm_ssd_combined_fwd.  Resets on read. */
 int ssm_ssd_mfma_launches(void);
 
 typedef struct ssm_ssd_dims {
@@ -287,6 +289,35 @@ typedef struct ssm_ssd_chunk_scan_args {
   int32_t x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype, d_per_p, force_generic;
 } ssm_ssd_chunk_scan_args;
 int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
+
+/* The whole forward (chunk_cumsum, bmm_chunk, chunk_state, state_passing,
+ * chunk_scan; combined call recorded at scripts/refresh_mamba_goldens.py:591-604)
+ * as one pass over the sequence that keeps the running state on chip: the
+ * per-chunk states never reach device memory.  Covers bf16 tensors with
+ * headdim 64, chunk in {32, 64, 128, 256}, nstate in {32, 64, 128},
+ * seqlen % chunk == 0 and A <= 0; ssm_ssd_combined_supported() tells, other
+ * shapes go through the five calls above. */
+typedef struct ssm_ssd_combined_args {
+  const void *x;              /* (B,L,H,P) io dtype */
+  const void *dt;             /* (B,L,H) dt dtype, before bias / softplus / clamp */
+  const float *A;             /* (H,) */
+  const float *dt_bias;       /* (H,) or NULL */
+  const void *Bm, *Cm;        /* (B,L,G,N) io dtype */
+  const float *Dskip;         /* (H,P) if d_per_p else (H,), or NULL */
+  const void *z;              /* (B,L,H,P) io dtype or NULL */
+  const float *initial_states;/* (B,H,P,N) fp32 or NULL */
+  void *y;                    /* (B,L,H,P) io dtype */
+  float *final_states;        /* (B,H,P,N) fp32 or NULL */
+  void *workspace;            /* ssm_ssd_combined_workspace_bytes() bytes, 256-byte aligned */
+  size_t workspace_bytes;
+  ssm_ssd_dims dims;
+  int32_t io_dtype;           /* must be SSM_BF16 */
+  int32_t dt_dtype, dt_softplus, d_per_p;
+  float dt_min, dt_max;       /* clamp applied after softplus; use 0 and +inf for none */
+} ssm_ssd_combined_args;
+int ssm_ssd_combined_supported(const ssm_ssd_dims *dims, int io_dtype);   /* 1 / 0 */
+size_t ssm_ssd_combined_workspace_bytes(const ssm_ssd_dims *dims);
+int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *args, void *hip_stream);
 
 /* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).

@@ -124,6 +124,13 @@ class SsdChunkScanArgs(C.Structure):
                 ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32)]
 
 
+class SsdCombinedArgs(C.Structure):
+    _fields_ = [("x", _vp), ("dt", _vp), ("A", _vp), ("dt_bias", _vp), ("Bm", _vp), ("Cm", _vp), ("Dskip", _vp),
+                ("z", _vp), ("initial_states", _vp), ("y", _vp), ("final_states", _vp), ("workspace", _vp),
+                ("workspace_bytes", C.c_size_t), ("dims", SsdDims), ("io_dtype", _i32), ("dt_dtype", _i32),
+                ("dt_softplus", _i32), ("d_per_p", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float)]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -177,6 +184,7 @@ ENTRY_POINTS = {
     "ssm_ssd_chunk_state": SsdChunkStateArgs,
     "ssm_ssd_state_passing": SsdStatePassingArgs,
     "ssm_ssd_chunk_scan": SsdChunkScanArgs,
+    "ssm_ssd_combined_fwd": SsdCombinedArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_norm_fwd": NormFwdArgs,
@@ -192,6 +200,8 @@ PLAIN_SYMBOLS = {
     "ssm_dscan_fwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ssm_ssd_chunk_state_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
     "ssm_ssd_mfma_launches": (C.c_int, []),
+    "ssm_ssd_combined_supported": (C.c_int, [C.POINTER(SsdDims), C.c_int]),
+    "ssm_ssd_combined_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
     "ssm_conv1d_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "ssm_norm_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
 }

@@ -66,7 +66,11 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 
 template <typename T> __device__ __forceinline__ T from_f32(float f);
 template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
-template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) { return bf16_t{f32_to_bf16_bits(f)}; }
+// gfx950 converts with round-to-nearest-even in hardware (v_cvt_pk_bf16_f32)
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
+  const __bf16 h = (__bf16)f;
+  return bf16_t{__builtin_bit_cast(uint16_t, h)};
+}
 template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float f) { return f16_t{(_Float16)f}; }
 
 // Read element i of a buffer whose dtype is only known at run time (uniform branch).
@@ -128,10 +132,13 @@ __device__ __forceinline__ float exp_f32(float x) { return exp2_hw(x * LOG2E); }
 // log(1 + e) = log(w) + (e - (w - 1)) / w with w = fl(1 + e): the second term
 // restores what the rounding of 1 + e lost, so small results keep full relative
 // accuracy (softplus of a very negative number is e itself).
+// Above w = 2 the restored term is below half an ulp of the result and is dropped;
+// below it, dividing it by w (< 2) would change the result by less than 4e-8 relative.
 __device__ __forceinline__ float softplus_f32(float x) {
   const float e = exp_f32(x);
   const float w = 1.0f + e;
-  const float r = __builtin_fmaf(e - (w - 1.0f), rcp_hw(w), log2_hw(w) * LN2);
+  const float lost = w < 2.0f ? e - (w - 1.0f) : 0.0f;
+  const float r = __builtin_fmaf(log2_hw(w), LN2, lost);
   return x > 20.0f ? x : r;
 }
 

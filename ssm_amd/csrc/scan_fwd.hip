@@ -65,16 +65,22 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   int rows = SCAN_MAX_WAVES;
   while (rows > 1 && (per_b % rows != 0 || per_c % rows != 0)) rows >>= 1;
 
+  // Two channels per wave (tune 1616) pay off once the grid still fills every CU twice.
+  const bool pair_ok = bvary && cvary && a->nstate <= 16 && per_b % 16 == 0 && per_c % 16 == 0;
   int tune = a->tune_items;
-  if (tune == 0) tune = (a->seqlen <= 256 && !a->chunk_states) ? 408 : 808;
-  // tune 1616: slab of 16 states shared by 16 channels (two per wave)
+  if (tune == 0) {
+    if (a->seqlen <= 256 && !a->chunk_states) tune = 408;
+    else if (pair_ok && (size_t)a->batch * a->dim / 16 >= 512) tune = 1616;
+    else tune = a->nstate > 8 ? 816 : 808;
+  }
   if (tune == 1616) {
-    if (bvary && cvary && a->nstate <= 16 && per_b % 16 == 0 && per_c % 16 == 0) rows = 2 * SCAN_MAX_WAVES;
+    if (pair_ok) rows = 2 * SCAN_MAX_WAVES;
     else tune = 816;
   }
+  const int steps_per_lane = tune == 1616 ? 8 : tune / 100;
   if (a->chunk_states)
-    SSM_REQUIRE(tune / 100 * WAVE == ssm_scan_chunk_len(), SSM_ERR_BAD_KIND,
-                "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (tune_items 808 or 816)",
+    SSM_REQUIRE(steps_per_lane * WAVE == ssm_scan_chunk_len(), SSM_ERR_BAD_KIND,
+                "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (tune_items 808, 816 or 1616)",
                 ssm_scan_chunk_len());
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   switch (a->io_dtype) {

@@ -209,15 +209,22 @@ __global__ __launch_bounds__(WAVE *SCAN_MAX_WAVES) void scan_fwd_kernel(const Sc
               for (int n = SCAN_LANE_STATES + lane; n < N; n += WAVE) cs[n] = carry_hi[wave][n - SCAN_LANE_STATES];
           }
           dsum = 0.0f;
+          if (p.softplus) {
+#pragma unroll
+            for (int i = 0; i < K; ++i) dl[i] = softplus_f32(dl[i] + bias);
+          } else {
+#pragma unroll
+            for (int i = 0; i < K; ++i) dl[i] += bias;
+          }
+          if (t + K > L) {                      // steps past the end are the identity map
+#pragma unroll
+            for (int i = 0; i < K; ++i) dl[i] = (t + i < L) ? dl[i] : 0.0f;
+          }
 #pragma unroll
           for (int i = 0; i < K; ++i) {
-            float dv = dl[i] + bias;
-            if (p.softplus) dv = softplus_f32(dv);
-            dv = (t + i < L) ? dv : 0.0f;      // steps past the end are the identity map
-            dl[i] = dv;
-            du[i] = dv * uu[i];
+            du[i] = dl[i] * uu[i];
             y[i] = Dk * uu[i];
-            dsum += dv;
+            dsum += dl[i];
           }
         }
 

@@ -17,7 +17,9 @@ namespace ssm {
 
 constexpr int SSD_THREADS = 256;
 
-static thread_local int g_mfma_launches = 0;   // bit0 bmm_chunk, bit1 chunk_state, bit2 chunk_scan
+static thread_local int g_mfma_launches = 0;   // bit0 bmm_chunk, bit1 chunk_state, bit2 chunk_scan, bit3 one-pass forward
+
+void note_mfma_launch(int bits) { g_mfma_launches |= bits; }
 
 static unsigned grid_for(size_t n) {
   const size_t g = (n + SSD_THREADS - 1) / SSD_THREADS;

@@ -72,10 +72,36 @@ __device__ __forceinline__ void store_any(void *p, int dtype, size_t i, float v)
 // clamp only matters for (unphysical) positive A and mirrors the published kernels.
 __device__ __forceinline__ float decay_exp(float v) { return exp2_hw(fminf(v, 0.0f) * LOG2E); }
 
+// ---- bf16 MFMA helpers (v_mfma_f32_32x32x16_bf16) ----
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+__device__ __forceinline__ f32x16_t mma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ bf16x8_t load_frag(const void *p) { return *reinterpret_cast<const bf16x8_t *>(p); }
+
+__device__ __forceinline__ bf16x8_t pack8(const float (&v)[8]) {
+  bf16x8_t r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = (__bf16)v[j];
+  return r;
+}
+
+__device__ __forceinline__ void unpack8(bf16x8_t r, float (&v)[8]) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (float)r[j];
+}
+
+// Row of C-layout register r for a lane in half g = lane / 32.
+__device__ __forceinline__ int crow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+
 // MFMA variants, defined in ssd_mfma.hip; return false when the shape is not covered.
 bool ssd_bmm_mfma(const SsdBmmParams &p, hipStream_t s);
 bool ssd_chunk_state_mfma(const SsdStateParams &p, hipStream_t s);
 size_t ssd_chunk_state_scratch_bytes(const SsdDims &d);
 bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s);
+void note_mfma_launch(int bits);   // recorded for ssm_ssd_mfma_launches()
 
 }  // namespace ssm

@@ -1,0 +1,548 @@
+// Mamba-2 SSD forward as one pass over the sequence: a workgroup owns one
+// (batch, head), walks its chunks in order and keeps the running state
+// S (P x N, fp32) in MFMA accumulators, so neither the per-chunk states nor
+// the state entering each chunk ever travel through HBM.
+//
+// Per chunk (Q steps, 32-step blocks lb = 0 .. Q/32-1, e_k = last step of block k,
+// cs[l] = running sum of dt A inside the chunk, cs[e_-1] := 0):
+//
+//   y_l = exp(cs_l) C_l.S  +  sum_{s<=l} CB[l,s] exp(cs_l - cs_s) dt_s x_s  (+ D x_l, gate)
+//
+// Only the 32x32 blocks on the diagonal need a decay factor per element.  For a
+// block of earlier steps the factor splits into three pieces that are all <= 1,
+//   exp(cs_l - cs_s) = exp(cs_l - cs[e_{lb-1}]) . exp(cs[e_{lb-1}] - cs[e_sb]) . exp(cs[e_sb] - cs_s),
+// a per-row factor applied once to the accumulator, a per-block scalar applied
+// as the accumulator moves from one block of s to the next (acc = acc * g_sb + CB_blk x~_blk
+// with g_k = exp(cs[e_k] - cs[e_{k-1}])), and a per-step weight folded with dt
+// into the staged operand x~_s = x_s dt_s exp(cs[e_sb] - cs_s).  The carried state
+// enters the same recurrence as its first term.  The state update
+//   S <- S * g_k + x~_blk^T B_blk          for k = 0 .. Q/32-1
+// uses the same x~ tile and ends each chunk with S decayed by exp(cs[Q-1]).
+//
+// B, C and CB are re-laid once per call so that every MFMA operand fragment is
+// one contiguous KiB (64 lanes x 8 bf16).
+//
+// Requires bf16 tensors, P = 64, Q in {32, 64, 128, 256}, N in {32, 64, 128},
+// L % Q == 0 and A <= 0 (the factors above are clamped to 1 individually).
+#include "ssd_common.hpp"
+
+namespace ssm {
+
+constexpr int FU_THREADS = 512;
+constexpr int FU_P = 64;
+constexpr int FU_TILE_BYTES = 32768;                       // [64][256] bf16
+constexpr int FU_LDS_BYTES = 2 * FU_TILE_BYTES + 3 * 256 * 4;
+constexpr int FRAG = 512;                                  // bf16 elements per operand fragment
+
+struct SsdFusedParams {
+  const __bf16 *x, *z;
+  __bf16 *y;
+  const float *dA2, *dtv, *ws;          // (B,H,nc,Q): log2-scaled running sum, step, staged weight
+  const __bf16 *Cblk, *Btblk, *CBblk;   // fragment-blocked copies
+  const float *Dk, *init;
+  float *final_states;
+  int batch, len, heads, groups, nstate, chunk, nchunks, d_per_p;
+};
+
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+
+__device__ __forceinline__ void wave_lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// ------------------------------------------------------------------ prep: dt
+// One wave per (b, h, c): step, running sums and the staged weight
+//   ws[l] = dt_l exp(cs[l | 31] - cs[l]).
+__global__ __launch_bounds__(256) void ssd_fused_prep_dt_kernel(const SsdCumsumParams p, float *dA2, float *ws) {
+  __shared__ float cs[4][256];
+  const SsdDims &d = p.d;
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const size_t unit = (size_t)blockIdx.x * 4 + wave;
+  if (unit >= (size_t)d.batch * d.heads * d.nchunks) return;
+  const int c = (int)(unit % d.nchunks);
+  const int h = (int)((unit / d.nchunks) % d.heads);
+  const int b = (int)(unit / ((size_t)d.nchunks * d.heads));
+  const int Q = d.chunk, per = (Q + 63) >> 6;
+  const float A = p.A[h];
+  const float bias = p.bias ? p.bias[h] : 0.0f;
+  float v[4], run[4];
+  float tot = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int l = lane * per + i;
+    v[i] = 0.0f;
+    if (i < per && l < Q) {
+      float x = load_as_f32(p.dt, p.dt_dtype, ((size_t)b * d.len + (size_t)c * Q + l) * d.heads + h) + bias;
+      if (p.softplus) x = softplus_f32(x);
+      v[i] = fminf(fmaxf(x, p.dt_min), p.dt_max);
+    }
+    tot = __builtin_fmaf(v[i], A, tot);
+    run[i] = tot;
+  }
+  float incl = tot;
+#pragma unroll
+  for (int off = 1; off < WAVE; off <<= 1) {
+    const float t = __shfl_up(incl, off, WAVE);
+    if (lane >= off) incl += t;
+  }
+  const float excl = incl - tot;
+  const size_t out = unit * (size_t)Q;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int l = lane * per + i;
+    if (i < per && l < Q) {
+      const float a = excl + run[i];
+      cs[wave][l] = a;
+      p.dA_cs[out + l] = a;
+      p.dt_out[out + l] = v[i];
+      dA2[out + l] = a * LOG2E;
+    }
+  }
+  wave_lds_sync();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int l = lane * per + i;
+    if (i < per && l < Q) ws[out + l] = v[i] * decay_exp(cs[wave][l | 31] - cs[wave][l]);
+  }
+}
+
+// ---------------------------------------------------------------- prep: pack
+// Fragment (lane, j) of a 32 x 16 operand block: row 32 rb + lane % 32,
+// column 16 kb + 8 (lane / 32) + j.  One wave per fragment.
+//   which = 0: Cblk [(b,c,g)][lb][kn]  from C  (rows = time, columns = state)
+//   which = 1: CBblk[(b,c,g)][lb][ks]  from CB (rows = l, columns = s), lower blocks only
+//   which = 2: Btblk[(b,c,g)][ks][nt]  from B  (rows = state, columns = time)
+__global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *src, __bf16 *dst, int which, int batch, int len,
+                                                             int groups, int nstate, int chunk) {
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int Q = chunk, N = nstate, nc = len / Q;
+  const int NLB = Q >> 5, KS = Q >> 4, KN = N >> 4, NT = N >> 5;
+  const int per_unit = which == 0 ? NLB * KN : (which == 1 ? NLB * KS : KS * NT);
+  const size_t f = (size_t)blockIdx.x * 4 + wave;
+  if (f >= (size_t)batch * nc * groups * per_unit) return;
+  const int inner = (int)(f % per_unit);
+  const size_t unit = f / per_unit;
+  const int g = (int)(unit % groups);
+  const int c = (int)((unit / groups) % nc);
+  const int b = (int)(unit / ((size_t)groups * nc));
+  const int m = lane & 31, g2 = lane >> 5;
+  bf16x8_t v;
+  if (which == 0) {
+    const int lb = inner / KN, kn = inner % KN;
+    v = load_frag(src + (((size_t)b * len + (size_t)c * Q + 32 * lb + m) * groups + g) * N + 16 * kn + 8 * g2);
+  } else if (which == 1) {
+    const int lb = inner / KS, ks = inner % KS;
+    if (ks > 2 * lb + 1) return;
+    v = load_frag(src + (unit * Q + 32 * lb + m) * (size_t)Q + 16 * ks + 8 * g2);
+  } else {
+    const int ks = inner / NT, nt = inner % NT;
+    const __bf16 *col = src + (((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * groups + g) * N + 32 * nt + m;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = col[(size_t)j * groups * N];
+  }
+  *reinterpret_cast<bf16x8_t *>(dst + f * FRAG + lane * 8) = v;
+}
+
+// --------------------------------------------------------------- fused kernel
+// Waves 0..7.  For the output phases wave w owns the 32 rows of block
+// lb = w (w < 4) or 11 - w, both 32-wide halves of P, so that the two waves
+// sharing a SIMD carry equal numbers of blocks below the diagonal.  For the state
+// phases wave w owns the 32 x 32 tile (n-tile w / 2, p-tile w % 2) of S^T.
+// Accumulators hold transposed tiles: lane = column (l for y, p for S^T),
+// registers = rows (p for y, n for S^T).
+__global__ __launch_bounds__(FU_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void ssd_fused_kernel(const SsdFusedParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  __bf16 *xw = reinterpret_cast<__bf16 *>(smem);                       // x~ [64][Q]; between chunks S as bf16 [64][N]
+  __bf16 *xr = reinterpret_cast<__bf16 *>(smem + FU_TILE_BYTES);       // x  [64][Q]; later the output staging
+  float *dAs = reinterpret_cast<float *>(smem + 2 * FU_TILE_BYTES);    // [Q] log2-scaled running sum
+  float *dts = dAs + 256;                                              // [Q]
+  float *wss = dts + 256;                                              // [Q] staged weight
+
+  const int Q = p.chunk, N = p.nstate, H = p.heads, G = p.groups, nc = p.nchunks;
+  const int NLB = Q >> 5, NT = N >> 5, KS = Q >> 4, KN = N >> 4;
+  const int qmask = min(15, (Q >> 3) - 1), nmask = min(15, (N >> 3) - 1);
+  const int tid = (int)threadIdx.x;
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int g2 = lane >> 5, m = lane & 31;
+  const int h = (int)blockIdx.x % H, b = (int)blockIdx.x / H;
+  const int g = h / (H / G);
+  const int lb = wave < 4 ? wave : 11 - wave;
+  const bool yact = lb < NLB;
+  const int pt_s = wave & 1, nt_s = wave >> 1;
+  const bool sact = nt_s < NT;
+  const bool has_init = p.init != nullptr;
+  const size_t xrow = (size_t)H * FU_P;                                // elements between time steps
+
+  f32x16_t S = {0};
+  if (sact && has_init) {
+    const float *ip = p.init + (((size_t)b * H + h) * FU_P + 32 * pt_s + m) * N + 32 * nt_s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[r] = ip[crow(r, g2)];
+  }
+  f32x16_t acc[2];
+
+  // staging role: a thread transposes 8 time steps x 4 head channels into both tiles
+
+  for (int c = 0; c < nc; ++c) {
+    // Lane-derived addresses are recomputed per chunk (the opaque copy keeps them from
+    // being hoisted out of the loop and held in registers across all of it).
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int lane = ln, g2 = ln >> 5, m = ln & 31, tid = wave * WAVE + ln;
+    const bool s_on = tid < 2 * Q;
+    const int spb = tid & 15, slb8 = tid >> 4;
+    const size_t cs = (((size_t)b * H + h) * nc + c) * Q;
+    const size_t unit = ((size_t)b * nc + c) * G + g;
+    const __bf16 *xg = p.x + (((size_t)b * p.len + (size_t)c * Q) * H + h) * FU_P;
+    const bool carry = c > 0 || has_init;
+
+    __syncthreads();                       // previous chunk: output staging and x~ reads are over
+    if (sact && carry) {
+      const int prow = 32 * pt_s + m;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        bf16x4_t v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = (__bf16)S[4 * q + j];
+        const int chunk16 = 4 * nt_s + q;
+        *reinterpret_cast<bf16x4_t *>(xw + prow * N + ((chunk16 ^ (prow & nmask)) << 3) + 4 * g2) = v;
+      }
+    }
+    if (tid < Q) {
+      dAs[tid] = p.dA2[cs + tid];
+      dts[tid] = p.dtv[cs + tid];
+      wss[tid] = p.ws[cs + tid];
+    }
+    // global reads for the staging that follows the carried-state product
+    bf16x4_t raw[8];
+    if (s_on) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r)
+        raw[r] = *reinterpret_cast<const bf16x4_t *>(xg + (size_t)(slb8 * 8 + r) * xrow + spb * 4);
+    }
+    __syncthreads();
+
+    // ---- carried state: acc[p][l] = sum_n S[p][n] C[l][n]
+    acc[0] = (f32x16_t){0};
+    acc[1] = (f32x16_t){0};
+    if (yact && carry) {
+      const __bf16 *cf = p.Cblk + ((unit * NLB + lb) * KN) * FRAG + lane * 8;
+      bf16x8_t fnext = load_frag(cf);
+      for (int kn = 0; kn < KN; ++kn) {
+        const bf16x8_t f = fnext;
+        if (kn + 1 < KN) fnext = load_frag(cf + (size_t)(kn + 1) * FRAG);
+#pragma unroll
+        for (int pt = 0; pt < 2; ++pt) {
+          const int prow = 32 * pt + m;
+          const bf16x8_t a = load_frag(xw + prow * N + (((2 * kn + g2) ^ (prow & nmask)) << 3));
+          acc[pt] = mma(a, f, acc[pt]);
+        }
+      }
+    }
+    __syncthreads();                       // S (bf16) consumed: the x~ tile may be written
+
+    // ---- stage x~ and x, transposed to [p][s]
+    if (s_on) {
+      const float4 a0 = *reinterpret_cast<const float4 *>(wss + slb8 * 8), a1 = *reinterpret_cast<const float4 *>(wss + slb8 * 8 + 4);
+      const float w8[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        bf16x8_t colw, colr;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          colr[r] = raw[r][i];
+          colw[r] = (__bf16)((float)raw[r][i] * w8[r]);
+        }
+        const int prow = spb * 4 + i;
+        const int at = prow * Q + ((slb8 ^ (prow & qmask)) << 3);
+        *reinterpret_cast<bf16x8_t *>(xw + at) = colw;
+        *reinterpret_cast<bf16x8_t *>(xr + at) = colr;
+      }
+    }
+    // gate and skip operands of this wave's rows, in the row-major order of the output pass
+    bf16x8_t zreg[2], xreg[2];            // p-half 0 now, p-half 1 while half 0 is written out
+    const size_t row_at = (size_t)(32 * lb + (lane >> 2)) * xrow + 8 * (lane & 3);
+    if (yact) {
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+        xreg[pass] = load_frag(xg + row_at + (size_t)(16 * pass) * xrow);
+        if (p.z) zreg[pass] = load_frag(p.z + (xg - p.x) + row_at + (size_t)(16 * pass) * xrow);
+      }
+    }
+    __syncthreads();
+
+    // ---- blocks below the diagonal, then the diagonal block
+    if (yact) {
+      const __bf16 *cbf = p.CBblk + ((unit * NLB + lb) * KS) * FRAG + lane * 8;
+      bf16x8_t fnext = load_frag(cbf);
+      float prev_end = 0.0f;
+      for (int sb = 0; sb < lb; ++sb) {
+        const float endv = dAs[32 * sb + 31];
+        const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));
+        prev_end = endv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          acc[0][r] *= gs;
+          acc[1][r] *= gs;
+        }
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const int ks = 2 * sb + kk;
+          const bf16x8_t f = fnext;
+          fnext = load_frag(cbf + (size_t)(ks + 1) * FRAG);
+#pragma unroll
+          for (int pt = 0; pt < 2; ++pt) {
+            const int prow = 32 * pt + m;
+            const bf16x8_t a = load_frag(xw + prow * Q + (((2 * ks + g2) ^ (prow & qmask)) << 3));
+            acc[pt] = mma(a, f, acc[pt]);
+          }
+        }
+      }
+      const int lrow = 32 * lb + m;
+      const float dal = dAs[lrow];
+      const float rf = exp2_hw(fminf(dal - prev_end, 0.0f));
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[0][r] *= rf;
+        acc[1][r] *= rf;
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const int ks = 2 * lb + kk;
+        const bf16x8_t f = fnext;
+        if (kk == 0) fnext = load_frag(cbf + (size_t)(ks + 1) * FRAG);
+        const int sbase = 16 * ks + 8 * g2;
+        const float4 a0 = *reinterpret_cast<const float4 *>(dAs + sbase), a1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
+        const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
+        const float das[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+        float mv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float v = (float)f[j] * exp2_hw(dal - das[j]) * dtv[j];
+          mv[j] = (sbase + j <= lrow) ? v : 0.0f;
+        }
+        const bf16x8_t bf = pack8(mv);
+#pragma unroll
+        for (int pt = 0; pt < 2; ++pt) {
+          const int prow = 32 * pt + m;
+          const bf16x8_t a = load_frag(xr + prow * Q + (((2 * ks + g2) ^ (prow & qmask)) << 3));
+          acc[pt] = mma(a, bf, acc[pt]);
+        }
+      }
+    }
+    __syncthreads();                       // the plain tile is free: it becomes the output staging
+
+    // ---- output: through a wave-private 32 x 32 fp32 tile to row-major 16-byte accesses
+    if (yact) {
+      float *stg = reinterpret_cast<float *>(smem + FU_TILE_BYTES) + wave * 1024;
+      __bf16 *yg = p.y + (xg - p.x);
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float4 v = make_float4(acc[pt][4 * q], acc[pt][4 * q + 1], acc[pt][4 * q + 2], acc[pt][4 * q + 3]);
+          *reinterpret_cast<float4 *>(stg + m * 32 + (((2 * q + g2) ^ (m & 7)) << 2)) = v;
+        }
+        wave_lds_sync();
+        bf16x8_t zcur[2] = {zreg[0], zreg[1]}, xcur[2] = {xreg[0], xreg[1]};
+        if (pt == 0) {
+#pragma unroll
+          for (int pass = 0; pass < 2; ++pass) {
+            xreg[pass] = load_frag(xg + row_at + (size_t)(16 * pass) * xrow + 32);
+            if (p.z) zreg[pass] = load_frag(p.z + (xg - p.x) + row_at + (size_t)(16 * pass) * xrow + 32);
+          }
+        }
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+          const int l = (lane >> 2) + 16 * pass, c4 = lane & 3;
+          const float4 v0 = *reinterpret_cast<const float4 *>(stg + l * 32 + (((2 * c4) ^ (l & 7)) << 2));
+          const float4 v1 = *reinterpret_cast<const float4 *>(stg + l * 32 + (((2 * c4 + 1) ^ (l & 7)) << 2));
+          float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+          const int pcol = 32 * pt + 8 * c4;
+          if (p.Dk) {
+            float dk[8];
+            if (p.d_per_p) {
+              const float4 d0 = *reinterpret_cast<const float4 *>(p.Dk + (size_t)h * FU_P + pcol);
+              const float4 d1 = *reinterpret_cast<const float4 *>(p.Dk + (size_t)h * FU_P + pcol + 4);
+              dk[0] = d0.x; dk[1] = d0.y; dk[2] = d0.z; dk[3] = d0.w; dk[4] = d1.x; dk[5] = d1.y; dk[6] = d1.z; dk[7] = d1.w;
+            } else {
+              const float dh = p.Dk[h];
+#pragma unroll
+              for (int j = 0; j < 8; ++j) dk[j] = dh;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = __builtin_fmaf(dk[j], (float)xcur[pass][j], v[j]);
+          }
+          if (p.z) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] *= silu_f32((float)zcur[pass][j]);
+          }
+          *reinterpret_cast<bf16x8_t *>(yg + (size_t)(32 * lb + l) * xrow + pcol) = pack8(v);
+        }
+        wave_lds_sync();
+      }
+    }
+
+    // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p]
+    if (sact) {
+      const __bf16 *btf = p.Btblk + ((unit * KS) * NT + nt_s) * FRAG + lane * 8;
+      bf16x8_t fnext = load_frag(btf);
+      float prev_end = 0.0f;
+      const int prow = 32 * pt_s + m;
+      for (int sb = 0; sb < NLB; ++sb) {
+        const float endv = dAs[32 * sb + 31];
+        const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));
+        prev_end = endv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) S[r] *= gs;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const int ks = 2 * sb + kk;
+          const bf16x8_t f = fnext;
+          if (ks + 1 < KS) fnext = load_frag(btf + (size_t)(ks + 1) * NT * FRAG);
+          const bf16x8_t xf = load_frag(xw + prow * Q + (((2 * ks + g2) ^ (prow & qmask)) << 3));
+          S = mma(f, xf, S);
+        }
+      }
+    }
+  }
+
+  if (p.final_states && sact) {
+    float *fp = p.final_states + (((size_t)b * H + h) * FU_P + 32 * pt_s + m) * N + 32 * nt_s;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<float4 *>(fp + 8 * q + 4 * g2) = make_float4(S[4 * q], S[4 * q + 1], S[4 * q + 2], S[4 * q + 3]);
+  }
+}
+
+static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct FusedLayout {
+  size_t dA_cs, dt_out, dA2, ws, Cblk, Btblk, CB, CBblk, total;
+};
+
+static FusedLayout fused_layout(const SsdDims &d) {
+  FusedLayout f;
+  const size_t per_step = align_up((size_t)d.batch * d.heads * d.len * sizeof(float));
+  const size_t bc = align_up((size_t)d.batch * d.len * d.groups * d.nstate * 2);
+  const size_t cb = align_up((size_t)d.batch * d.nchunks * d.groups * d.chunk * d.chunk * 2);
+  size_t at = 0;
+  f.dA_cs = at; at += per_step;
+  f.dt_out = at; at += per_step;
+  f.dA2 = at; at += per_step;
+  f.ws = at; at += per_step;
+  f.Cblk = at; at += bc;
+  f.Btblk = at; at += bc;
+  f.CB = at; at += cb;
+  f.CBblk = at; at += cb;
+  f.total = at;
+  return f;
+}
+
+static bool fused_shape_ok(const SsdDims &d) {
+  const bool q_ok = d.chunk == 32 || d.chunk == 64 || d.chunk == 128 || d.chunk == 256;
+  const bool n_ok = d.nstate == 32 || d.nstate == 64 || d.nstate == 128;
+  return q_ok && n_ok && d.hdim == FU_P && d.len % d.chunk == 0 && d.heads % d.groups == 0;
+}
+
+}  // namespace ssm
+
+static int fused_dims(const char *who, const ssm_ssd_dims *s, ssm::SsdDims &d) {
+  using namespace ssm;
+  SSM_REQUIRE(s, SSM_ERR_NULL_POINTER, "%s: dims is required", who);
+  SSM_REQUIRE(s->batch > 0 && s->seqlen > 0 && s->heads > 0 && s->headdim > 0 && s->groups > 0 && s->nstate > 0 &&
+                  s->chunk > 0,
+              SSM_ERR_BAD_SHAPE, "%s: all of batch, seqlen, heads, headdim, groups, nstate, chunk must be positive", who);
+  SSM_REQUIRE(s->heads % s->groups == 0, SSM_ERR_BAD_SHAPE, "%s: groups=%d must divide heads=%d", who, s->groups,
+              s->heads);
+  d.batch = s->batch; d.len = s->seqlen; d.heads = s->heads; d.hdim = s->headdim; d.groups = s->groups;
+  d.nstate = s->nstate; d.chunk = s->chunk; d.nchunks = (s->seqlen + s->chunk - 1) / s->chunk;
+  SSM_REQUIRE((size_t)d.batch * d.len * d.heads * d.hdim < ((size_t)1 << 40), SSM_ERR_TOO_LARGE, "%s: tensor too large",
+              who);
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_combined_supported(const ssm_ssd_dims *dims, int io_dtype) {
+  ssm::SsdDims d;
+  if (fused_dims("ssm_ssd_combined_supported", dims, d) != SSM_OK) return 0;
+  return io_dtype == SSM_BF16 && ssm::fused_shape_ok(d) ? 1 : 0;
+}
+
+extern "C" size_t ssm_ssd_combined_workspace_bytes(const ssm_ssd_dims *dims) {
+  ssm::SsdDims d;
+  if (fused_dims("ssm_ssd_combined_workspace_bytes", dims, d) != SSM_OK) return 0;
+  return ssm::fused_layout(d).total;
+}
+
+extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a && a->x && a->dt && a->A && a->Bm && a->Cm && a->y, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_combined_fwd: x, dt, A, Bm, Cm and y are required");
+  SsdDims d;
+  int rc = fused_dims("ssm_ssd_combined_fwd", &a->dims, d);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(a->io_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE, "ssm_ssd_combined_fwd: x, z, y, Bm and Cm must be bf16");
+  SSM_REQUIRE(valid_dtype(a->dt_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_combined_fwd: dt_dtype=%d", a->dt_dtype);
+  SSM_REQUIRE(fused_shape_ok(d), SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_combined_fwd: needs headdim 64, chunk in {32,64,128,256}, nstate in {32,64,128} and "
+              "seqlen %% chunk == 0 (got headdim=%d chunk=%d nstate=%d seqlen=%d)",
+              d.hdim, d.chunk, d.nstate, d.len);
+  const FusedLayout lay = fused_layout(d);
+  SSM_REQUIRE(a->workspace && a->workspace_bytes >= lay.total, SSM_ERR_WORKSPACE,
+              "ssm_ssd_combined_fwd: workspace of %zu bytes required", lay.total);
+  SSM_REQUIRE(aligned_to(a->x, 16) && aligned_to(a->y, 16) && (!a->z || aligned_to(a->z, 16)) && aligned_to(a->Bm, 16) &&
+                  aligned_to(a->Cm, 16) && aligned_to(a->workspace, 256) &&
+                  (!a->Dskip || aligned_to(a->Dskip, 16)) && (!a->final_states || aligned_to(a->final_states, 16)) &&
+                  (!a->initial_states || aligned_to(a->initial_states, 4)),
+              SSM_ERR_ALIGNMENT, "ssm_ssd_combined_fwd: tensors must be 16-byte aligned (workspace 256)");
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  unsigned char *ws = reinterpret_cast<unsigned char *>(a->workspace);
+
+  SsdCumsumParams cp{};
+  cp.dt = a->dt; cp.A = a->A; cp.bias = a->dt_bias;
+  cp.dA_cs = reinterpret_cast<float *>(ws + lay.dA_cs);
+  cp.dt_out = reinterpret_cast<float *>(ws + lay.dt_out);
+  cp.d = d; cp.dt_dtype = a->dt_dtype; cp.softplus = a->dt_softplus ? 1 : 0; cp.dt_min = a->dt_min; cp.dt_max = a->dt_max;
+  const size_t units = (size_t)d.batch * d.heads * d.nchunks;
+  hipLaunchKernelGGL(ssd_fused_prep_dt_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, cp,
+                     reinterpret_cast<float *>(ws + lay.dA2), reinterpret_cast<float *>(ws + lay.ws));
+  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(prep dt)");
+
+  SsdBmmParams bp{};
+  bp.a = a->Cm; bp.b = a->Bm; bp.seq_idx = nullptr; bp.out = ws + lay.CB;
+  bp.batch = d.batch; bp.len = d.len; bp.groups = d.groups; bp.kdim = d.nstate; bp.chunk = d.chunk; bp.nchunks = d.nchunks;
+  bp.in_dtype = SSM_BF16; bp.out_dtype = SSM_BF16; bp.causal = 1;
+  SSM_REQUIRE(ssd_bmm_mfma(bp, s), SSM_ERR_BAD_SHAPE, "ssm_ssd_combined_fwd: C B^T kernel rejected the shape");
+  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(bmm)");
+
+  const size_t bcg = (size_t)d.batch * d.nchunks * d.groups;
+  const int NLB = d.chunk >> 5, KS = d.chunk >> 4, KN = d.nstate >> 4, NT = d.nstate >> 5;
+  const __bf16 *srcs[3] = {reinterpret_cast<const __bf16 *>(a->Cm), reinterpret_cast<const __bf16 *>(ws + lay.CB),
+                           reinterpret_cast<const __bf16 *>(a->Bm)};
+  __bf16 *dsts[3] = {reinterpret_cast<__bf16 *>(ws + lay.Cblk), reinterpret_cast<__bf16 *>(ws + lay.CBblk),
+                     reinterpret_cast<__bf16 *>(ws + lay.Btblk)};
+  const size_t frags[3] = {bcg * NLB * KN, bcg * NLB * KS, bcg * KS * NT};
+  for (int which = 0; which < 3; ++which) {
+    hipLaunchKernelGGL(ssd_fused_pack_kernel, dim3((unsigned)((frags[which] + 3) / 4)), dim3(256), 0, s, srcs[which],
+                       dsts[which], which, d.batch, d.len, d.groups, d.nstate, d.chunk);
+    SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(pack)");
+  }
+
+  SsdFusedParams fp{};
+  fp.x = reinterpret_cast<const __bf16 *>(a->x); fp.z = reinterpret_cast<const __bf16 *>(a->z);
+  fp.y = reinterpret_cast<__bf16 *>(a->y);
+  fp.dA2 = reinterpret_cast<const float *>(ws + lay.dA2); fp.dtv = cp.dt_out; fp.ws = reinterpret_cast<const float *>(ws + lay.ws);
+  fp.Cblk = dsts[0]; fp.CBblk = dsts[1]; fp.Btblk = dsts[2];
+  fp.Dk = a->Dskip; fp.init = a->initial_states; fp.final_states = a->final_states;
+  fp.batch = d.batch; fp.len = d.len; fp.heads = d.heads; fp.groups = d.groups; fp.nstate = d.nstate; fp.chunk = d.chunk;
+  fp.nchunks = d.nchunks; fp.d_per_p = a->d_per_p ? 1 : 0;
+  if (allow_dynamic_lds(ssd_fused_kernel, FU_LDS_BYTES) != hipSuccess) {
+    (void)hipGetLastError();
+    set_error("ssm_ssd_combined_fwd: cannot reserve %d bytes of LDS", FU_LDS_BYTES);
+    return SSM_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(ssd_fused_kernel, dim3((unsigned)(d.batch * d.heads)), dim3(FU_THREADS), FU_LDS_BYTES, s, fp);
+  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd");
+  note_mfma_launch(8);
+  return SSM_OK;
+}

@@ -16,37 +16,17 @@
 
 namespace ssm {
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
-
-__device__ __forceinline__ f32x16_t mma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-
-__device__ __forceinline__ bf16x8_t load_frag(const void *p) { return *reinterpret_cast<const bf16x8_t *>(p); }
-
-__device__ __forceinline__ bf16x8_t pack8(const float (&v)[8]) {
-  bf16x8_t r;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) r[j] = (__bf16)v[j];
-  return r;
-}
-
-__device__ __forceinline__ void unpack8(bf16x8_t r, float (&v)[8]) {
-#pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = (float)r[j];
-}
-
-// Row of C-layout register r for a lane in half g = lane / 32.
-__device__ __forceinline__ int crow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
-
 constexpr int MF_THREADS = 256;
 constexpr int MF_WAVES = 4;
 constexpr int XT_PAD = 8;      // bf16 elements of padding per transposed row
 
 // Offset (in bf16 elements) of (p, l) inside the transposed, XOR-swizzled x tile.
+// The swizzle permutes 16-byte pieces inside aligned groups of (lowest set bit of Q / 8)
+// pieces, at most 8, so that it never leaves the row.
 __device__ __forceinline__ int xt_off(int p, int l, int stride) {
-  return p * stride + ((((l >> 3) ^ ((p >> 3) & 7))) << 3) + (l & 7);
+  const int pieces = (stride - XT_PAD) >> 3;
+  const int mask = min(8, pieces & -pieces) - 1;
+  return p * stride + ((((l >> 3) ^ ((p >> 3) & mask))) << 3) + (l & 7);
 }
 
 // Transpose the [Q][P] bf16 slab x[b, t0.., h, :] into LDS as [P][Q] (optionally

@@ -73,7 +73,6 @@ class ScanPlan:
             nchunks = (length + chunk - 1) // chunk
             self.chunk_states = torch.empty(batch, dim, nchunks, nstate, dtype=torch.float32,
                                             device=self.device)
-            tune_items = tune_items or 808
         self.args = _lib.ScanFwdArgs(
             u=_lib.ptr(k["u"]), delta=_lib.ptr(k["delta"]), z=_lib.ptr(k["z"]), A=_lib.ptr(k["A"]),
             Bproj=_lib.ptr(k["B"]), Cproj=_lib.ptr(k["C"]), Dskip=_lib.ptr(k["D"]),

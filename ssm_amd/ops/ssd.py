@@ -246,10 +246,58 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
     return y
 
 
+def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
+    """Whether the one-pass kernel covers this call (bf16 tensors on the GPU and a
+    shape ``ssm_ssd_combined_supported`` accepts)."""
+    if Q <= 0 or seqlen % Q != 0:
+        return False
+    tensors = [x, B, C] + ([z] if z is not None else [])
+    if any(t.dtype != torch.bfloat16 for t in tensors) or not x.is_cuda:
+        return False
+    dims = _dims(batch, seqlen, heads, hdim, groups, nstate, Q)
+    return bool(_lib.load().ssm_ssd_combined_supported(dims, _lib.dtype_enum(torch.bfloat16)))
+
+
+def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit, return_final_states, shape):
+    batch, seqlen, heads, hdim, groups, nstate = shape
+    d_per_p = False
+    if D is not None:
+        _need(tuple(D.shape) in ((heads,), (heads, hdim)), "D must have shape (H,) or (H, P).")
+        d_per_p = D.ndim == 2
+    _need(z is None or z.shape == x.shape, "z must have the shape of x.")
+    _need(tuple(A.shape) == (heads,), "A must have shape (H,).")
+    _need(dt_bias is None or tuple(dt_bias.shape) == (heads,), "dt_bias must have shape (H,).")
+    dev = K.require_gpu(x, dt, A, B, C, D, z, dt_bias, initial_states)
+    xc, Bc, Cc = K.cast_c(x, x.dtype), K.cast_c(B, B.dtype), K.cast_c(C, C.dtype)
+    zc = K.cast_c(z, z.dtype) if z is not None else None
+    dtc = K.cast_c(dt, dt.dtype)
+    K.check_float("dt", dtc)
+    Af, Df, bf, init = K.as_f32_vec(A), K.as_f32_vec(D), K.as_f32_vec(dt_bias), K.as_f32_vec(initial_states)
+    dims = _dims(batch, seqlen, heads, hdim, groups, nstate, Q)
+    nbytes = int(_lib.load().ssm_ssd_combined_workspace_bytes(dims))
+    work = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
+    off = (-work.data_ptr()) % 256
+    y = torch.empty_like(xc)
+    final = torch.empty(batch, heads, hdim, nstate, dtype=torch.float32, device=dev) if return_final_states else None
+    args = _lib.SsdCombinedArgs(
+        x=_lib.ptr(xc), dt=_lib.ptr(dtc), A=_lib.ptr(Af), dt_bias=_lib.ptr(bf), Bm=_lib.ptr(Bc), Cm=_lib.ptr(Cc),
+        Dskip=_lib.ptr(Df), z=_lib.ptr(zc), initial_states=_lib.ptr(init), y=_lib.ptr(y),
+        final_states=_lib.ptr(final), workspace=work.data_ptr() + off, workspace_bytes=nbytes, dims=dims,
+        io_dtype=_lib.dtype_enum(torch.bfloat16), dt_dtype=_lib.dtype_enum(dtc.dtype),
+        dt_softplus=int(bool(dt_softplus)), d_per_p=int(d_per_p),
+        dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]))
+    _lib.call("ssm_ssd_combined_fwd", args, dev)
+    if return_final_states:
+        return y, final
+    return y
+
+
 def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
                  dt_softplus=False, dt_limit=(0.0, float("inf")), return_final_states=False,
-                 states_dtype=None, force_generic=False):
-    """Mamba-2 SSD forward: ``chunk_cumsum -> bmm_chunk, chunk_state -> state_passing -> chunk_scan``.
+                 states_dtype=None, force_generic=False, fused=None):
+    """Mamba-2 SSD forward.  bf16 calls whose shape the one-pass kernel covers run
+    ``ssm_ssd_combined_fwd``; everything else runs
+    ``chunk_cumsum -> bmm_chunk, chunk_state -> state_passing -> chunk_scan``.
 
     Args:
         x: ``(B, L, H, P)``.
@@ -266,6 +314,8 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         return_final_states: Also return the state after the last token.
         states_dtype: dtype of the per-chunk states kept in HBM between the kernels
             (default: ``x.dtype``; the recurrence itself accumulates in float32).
+        fused: ``None`` picks the one-pass kernel when it applies, ``False`` never
+            uses it, ``True`` requires it (``ValueError`` if the call is not covered).
 
     Returns:
         ``y (B, L, H, P)`` in ``x.dtype``, or ``(y, final_states (B, H, P, N) float32)``.
@@ -276,6 +326,13 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
     _need(initial_states is None or tuple(initial_states.shape) == (batch, heads, hdim, nstate),
           "initial_states must have shape (B, H, P, N).")
     Q = int(chunk_size)
+    can_fuse = not force_generic and fused is not False and \
+        _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
+    _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "
+          "chunk in {32,64,128,256}, nstate in {32,64,128} and seqlen % chunk == 0.")
+    if can_fuse:
+        return _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit,
+                          return_final_states, (batch, seqlen, heads, hdim, groups, nstate))
     sdt = states_dtype or x.dtype
     dA, dtc = chunk_cumsum(dt, A, Q, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit)
     states = chunk_state(B, x, dtc, dA, states_dtype=sdt, force_generic=force_generic)

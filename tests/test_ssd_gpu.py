@@ -133,7 +133,7 @@ def test_bf16_mfma_matches_generic_and_oracle(shape, Q):
     kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
     from ssm_amd import _lib
     _lib.load().ssm_ssd_mfma_launches()
-    y, fin = ssd().ssd_combined(*args, **kw)
+    y, fin = ssd().ssd_combined(*args, fused=False, **kw)
     used = _lib.load().ssm_ssd_mfma_launches()
     assert used == (7 if l % Q == 0 else 0), f"MFMA kernels used: {used:03b}"
     yg, fing = ssd().ssd_combined(*args, force_generic=True, states_dtype=torch.float32, **kw)
@@ -147,14 +147,71 @@ def test_bf16_mfma_matches_generic_and_oracle(shape, Q):
     torch.testing.assert_close(fin.cpu().double(), f64, rtol=2e-2, atol=2e-2 * fs)
 
 
+FUSED_CASES = [
+    # (B, L, H, P, G, N), Q, d_mat, use_z, use_init
+    ((2, 512, 4, 64, 1, 128), 256, False, True, True),
+    ((1, 1024, 3, 64, 1, 128), 256, True, True, False),
+    ((2, 384, 4, 64, 2, 64), 128, False, False, True),
+    ((1, 256, 2, 64, 2, 32), 64, True, True, True),
+    ((3, 96, 2, 64, 1, 64), 32, False, True, False),
+    ((1, 256, 1, 64, 1, 128), 256, False, False, False),
+]
+
+
+@pytest.mark.parametrize("shape,Q,d_mat,use_z,use_init", FUSED_CASES, ids=lambda v: str(v).replace(" ", ""))
+def test_bf16_one_pass_matches_oracle_and_five_kernel_path(shape, Q, d_mat, use_z, use_init):
+    b, l, h, p, g, n = shape
+    inp = make(17 + l + Q, b, l, h, p, g, n, dtype=torch.bfloat16, d_mat=d_mat, use_z=use_z, use_init=use_init)
+    args = (cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
+    kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
+    from ssm_amd import _lib
+    _lib.load().ssm_ssd_mfma_launches()
+    y, fin = ssd().ssd_combined(*args, fused=True, **kw)
+    assert _lib.load().ssm_ssd_mfma_launches() == 8
+    y5, fin5 = ssd().ssd_combined(*args, fused=False, **kw)
+    y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                                initial_states=inp["init"])
+    scale, fs = float(y64.abs().max()), float(f64.abs().max())
+    torch.testing.assert_close(y.float().cpu().double(), y64, rtol=2e-2, atol=2e-2 * scale)
+    torch.testing.assert_close(fin.cpu().double(), f64, rtol=2e-2, atol=2e-2 * fs)
+    # the two GPU paths round at different places; they agree to bf16 resolution of the output scale
+    torch.testing.assert_close(y.float(), y5.float(), rtol=2e-2, atol=2e-2 * scale)
+    torch.testing.assert_close(fin, fin5, rtol=2e-2, atol=2e-2 * fs)
+    # mean error against the float64 recurrence: far below a bf16 ulp of the output scale
+    assert float((y.float().cpu().double() - y64).abs().mean()) < 2e-3 * scale
+
+
+def test_one_pass_dt_bias_softplus_and_clamp():
+    b, l, h, p, g, n, Q = 2, 256, 4, 64, 1, 64, 128
+    inp = make(5, b, l, h, p, g, n, dtype=torch.bfloat16, use_init=False)
+    gen = torch.Generator().manual_seed(1)
+    raw = torch.randn(b, l, h, generator=gen)
+    bias = torch.randn(h, generator=gen) - 2.0
+    kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), dt_bias=cu(bias), dt_softplus=True, dt_limit=(0.01, 0.5),
+              return_final_states=True)
+    y, fin = ssd().ssd_combined(cu(inp["x"]), cu(raw), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q, fused=True, **kw)
+    dt_eff = torch.nn.functional.softplus(raw + bias).clamp(0.01, 0.5)
+    y64, f64 = S.ssd_sequential(inp["x"], dt_eff, inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"])
+    scale, fs = float(y64.abs().max()), float(f64.abs().max())
+    torch.testing.assert_close(y.float().cpu().double(), y64, rtol=2e-2, atol=2e-2 * scale)
+    torch.testing.assert_close(fin.cpu().double(), f64, rtol=2e-2, atol=2e-2 * fs)
+
+
+def test_one_pass_rejects_uncovered_calls():
+    inp = make(1, 1, 64, 2, 32, 1, 64, dtype=torch.bfloat16, use_init=False)
+    with pytest.raises(ValueError):
+        ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), 32, fused=True)
+
+
 def test_config3_shape_bf16():
     """BASELINE config 3: B=4, L=4096, H=80, P=64, N=128, G=1, Q=256, bf16.  Full size on the
     GPU; two heads of one batch row are replayed by the float64 sequential recurrence."""
     inp = make(3, 4, 4096, 80, 64, 1, 128, dtype=torch.bfloat16, use_init=False)
+    from ssm_amd import _lib
+    _lib.load().ssm_ssd_mfma_launches()
     y, fin = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), 256,
                                 D=cu(inp["D"]), z=cu(inp["z"]), return_final_states=True)
-    from ssm_amd import _lib
-    assert _lib.load().ssm_ssd_mfma_launches() & 7 == 7
+    assert _lib.load().ssm_ssd_mfma_launches() == 8
     assert y.dtype == torch.bfloat16 and fin.dtype == torch.float32 and tuple(fin.shape) == (4, 80, 64, 128)
     hs = [5, 71]
     y64, f64 = S.ssd_sequential(inp["x"][1:2, :, hs], inp["dt"][1:2, :, hs], inp["A"][hs], inp["B"][1:2],
