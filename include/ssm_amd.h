@@ -294,7 +294,7 @@ int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
  * chunk_scan; combined call recorded at scripts/refresh_mamba_goldens.py:591-604)
  * as one pass over the sequence that keeps the running state on chip: the
  * per-chunk states never reach device memory.  Covers bf16 tensors with
- * headdim 64, chunk in {32, 64, 128, 256}, nstate in {32, 64, 128},
+ * headdim 64, chunk in {64, 128, 256}, nstate in {64, 128},
  * seqlen % chunk == 0 and A <= 0; ssm_ssd_combined_supported() tells, other
  * shapes go through the five calls above. */
 typedef struct ssm_ssd_combined_args {

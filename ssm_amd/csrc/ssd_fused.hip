@@ -22,7 +22,7 @@
 // B, C and CB are re-laid once per call so that every MFMA operand fragment is
 // one contiguous KiB (64 lanes x 8 bf16).
 //
-// Requires bf16 tensors, P = 64, Q in {32, 64, 128, 256}, N in {32, 64, 128},
+// Requires bf16 tensors, P = 64, Q in {64, 128, 256}, N in {64, 128},
 // L % Q == 0 and A <= 0 (the factors above are clamped to 1 individually).
 #include "ssd_common.hpp"
 
@@ -148,7 +148,9 @@ __global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *src, 
 // phases wave w owns the 32 x 32 tile (n-tile w / 2, p-tile w % 2) of S^T.
 // Accumulators hold transposed tiles: lane = column (l for y, p for S^T),
 // registers = rows (p for y, n for S^T).
-__global__ __launch_bounds__(FU_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
+// DMODE: 0 no skip term, 1 D per head, 2 D per (head, channel).
+template <int DMODE, bool HAS_Z>
+__global__ __launch_bounds__(FU_THREADS)
 void ssd_fused_kernel(const SsdFusedParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   __bf16 *xw = reinterpret_cast<__bf16 *>(smem);                       // x~ [64][Q]; between chunks S as bf16 [64][N]
@@ -194,6 +196,18 @@ void ssd_fused_kernel(const SsdFusedParams p) {
     const size_t unit = ((size_t)b * nc + c) * G + g;
     const __bf16 *xg = p.x + (((size_t)b * p.len + (size_t)c * Q) * H + h) * FU_P;
     const bool carry = c > 0 || has_init;
+    // Operand fragments stream through four registers sets: f0 is consumed, f1..f3 are in
+    // flight, a new read (clamped to the last fragment) enters at f3.
+    bf16x8_t f0, f1, f2, f3;
+
+    // fragments of C for the carried-state product: in flight across the barriers below
+    const __bf16 *cf = p.Cblk + ((unit * NLB + lb) * KN) * FRAG + lane * 8;
+    if (yact && carry) {
+      f0 = load_frag(cf);
+      f1 = load_frag(cf + (size_t)min(1, KN - 1) * FRAG);
+      f2 = load_frag(cf + (size_t)min(2, KN - 1) * FRAG);
+      f3 = load_frag(cf + (size_t)min(3, KN - 1) * FRAG);
+    }
 
     __syncthreads();                       // previous chunk: output staging and x~ reads are over
     if (sact && carry) {
@@ -213,11 +227,12 @@ void ssd_fused_kernel(const SsdFusedParams p) {
       wss[tid] = p.ws[cs + tid];
     }
     // global reads for the staging that follows the carried-state product
-    bf16x4_t raw[8];
-    if (s_on) {
+    bf16x4_t raw[8];                       // read by every thread (clamped rows) so that the values
+    {                                      // are not defined under a divergent branch
+      const int srow = min(slb8, (Q >> 3) - 1) * 8;
 #pragma unroll
       for (int r = 0; r < 8; ++r)
-        raw[r] = *reinterpret_cast<const bf16x4_t *>(xg + (size_t)(slb8 * 8 + r) * xrow + spb * 4);
+        raw[r] = *reinterpret_cast<const bf16x4_t *>(xg + (size_t)(srow + r) * xrow + spb * 4);
     }
     __syncthreads();
 
@@ -225,18 +240,34 @@ void ssd_fused_kernel(const SsdFusedParams p) {
     acc[0] = (f32x16_t){0};
     acc[1] = (f32x16_t){0};
     if (yact && carry) {
-      const __bf16 *cf = p.Cblk + ((unit * NLB + lb) * KN) * FRAG + lane * 8;
-      bf16x8_t fnext = load_frag(cf);
-      for (int kn = 0; kn < KN; ++kn) {
-        const bf16x8_t f = fnext;
-        if (kn + 1 < KN) fnext = load_frag(cf + (size_t)(kn + 1) * FRAG);
-#pragma unroll
-        for (int pt = 0; pt < 2; ++pt) {
-          const int prow = 32 * pt + m;
-          const bf16x8_t a = load_frag(xw + prow * N + (((2 * kn + g2) ^ (prow & nmask)) << 3));
-          acc[pt] = mma(a, f, acc[pt]);
-        }
+      // four steps per trip, one register set each: a set is refilled as soon as it is consumed
+      // (no copies between sets: a copy would wait for the read it moves)
+#define FU_STEP_A(F, KK)                                                                        \
+      {                                                                                         \
+        const bf16x8_t f = F;                                                                   \
+        F = load_frag(cf + (size_t)min((KK) + 4, KN - 1) * FRAG);                               \
+        _Pragma("unroll") for (int pt = 0; pt < 2; ++pt) {                                      \
+          const int prow = 32 * pt + m;                                                         \
+          const bf16x8_t a = load_frag(xw + prow * N + (((2 * (KK) + g2) ^ (prow & nmask)) << 3)); \
+          acc[pt] = mma(a, f, acc[pt]);                                                         \
+        }                                                                                       \
       }
+      for (int k0 = 0; k0 < KN; k0 += 4) {
+        FU_STEP_A(f0, k0)
+        FU_STEP_A(f1, k0 + 1)
+        FU_STEP_A(f2, k0 + 2)
+        FU_STEP_A(f3, k0 + 3)
+      }
+#undef FU_STEP_A
+    }
+    // fragments of CB for this wave's rows: in flight while the tiles are staged
+    const __bf16 *cbf = p.CBblk + ((unit * NLB + lb) * KS) * FRAG + lane * 8;
+    const int nkb = 2 * lb + 2;            // 16-step fragments up to and including the diagonal block
+    if (yact) {
+      f0 = load_frag(cbf);
+      f1 = load_frag(cbf + (size_t)FRAG);
+      f2 = load_frag(cbf + (size_t)min(2, nkb - 1) * FRAG);
+      f3 = load_frag(cbf + (size_t)min(3, nkb - 1) * FRAG);
     }
     __syncthreads();                       // S (bf16) consumed: the x~ tile may be written
 
@@ -258,47 +289,52 @@ void ssd_fused_kernel(const SsdFusedParams p) {
         *reinterpret_cast<bf16x8_t *>(xr + at) = colr;
       }
     }
-    // gate and skip operands of this wave's rows, in the row-major order of the output pass
-    bf16x8_t zreg[2], xreg[2];            // p-half 0 now, p-half 1 while half 0 is written out
-    const size_t row_at = (size_t)(32 * lb + (lane >> 2)) * xrow + 8 * (lane & 3);
-    if (yact) {
-#pragma unroll
-      for (int pass = 0; pass < 2; ++pass) {
-        xreg[pass] = load_frag(xg + row_at + (size_t)(16 * pass) * xrow);
-        if (p.z) zreg[pass] = load_frag(p.z + (xg - p.x) + row_at + (size_t)(16 * pass) * xrow);
-      }
-    }
     __syncthreads();
-
     // ---- blocks below the diagonal, then the diagonal block
     if (yact) {
-      const __bf16 *cbf = p.CBblk + ((unit * NLB + lb) * KS) * FRAG + lane * 8;
-      bf16x8_t fnext = load_frag(cbf);
       float prev_end = 0.0f;
-      for (int sb = 0; sb < lb; ++sb) {
-        const float endv = dAs[32 * sb + 31];
-        const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));
-        prev_end = endv;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          acc[0][r] *= gs;
-          acc[1][r] *= gs;
-        }
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          const int ks = 2 * sb + kk;
-          const bf16x8_t f = fnext;
-          fnext = load_frag(cbf + (size_t)(ks + 1) * FRAG);
-#pragma unroll
-          for (int pt = 0; pt < 2; ++pt) {
-            const int prow = 32 * pt + m;
-            const bf16x8_t a = load_frag(xw + prow * Q + (((2 * ks + g2) ^ (prow & qmask)) << 3));
-            acc[pt] = mma(a, f, acc[pt]);
-          }
-        }
-      }
       const int lrow = 32 * lb + m;
       const float dal = dAs[lrow];
+      // two 32-step blocks per trip: block sb0 streams through (f0, f1), block sb0 + 1 through (f2, f3)
+#define FU_BLOCK_B(FA, FB, SB)                                                                  \
+      {                                                                                         \
+        const float endv = dAs[32 * (SB) + 31];                                                 \
+        const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));                                 \
+        prev_end = endv;                                                                        \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) {                                        \
+          acc[0][r] *= gs;                                                                      \
+          acc[1][r] *= gs;                                                                      \
+        }                                                                                       \
+        const bf16x8_t fa = FA, fb = FB;                                                        \
+        FA = load_frag(cbf + (size_t)min(2 * (SB) + 4, nkb - 1) * FRAG);                        \
+        FB = load_frag(cbf + (size_t)min(2 * (SB) + 5, nkb - 1) * FRAG);                        \
+        _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {                                      \
+          _Pragma("unroll") for (int pt = 0; pt < 2; ++pt) {                                    \
+            const int prow = 32 * pt + m;                                                       \
+            const bf16x8_t a = load_frag(xw + prow * Q + (((4 * (SB) + 2 * kk + g2) ^ (prow & qmask)) << 3)); \
+            acc[pt] = mma(a, kk == 0 ? fa : fb, acc[pt]);                                       \
+          }                                                                                     \
+        }                                                                                       \
+      }
+      // Block sb streams through (f0, f1) when sb is even and (f2, f3) when it is odd; the loop
+      // takes two blocks per trip without a guard between them, so an odd count starts with
+      // block 0 on its own.
+      if (lb & 1) {
+        FU_BLOCK_B(f0, f1, 0)
+        for (int sb0 = 1; sb0 < lb; sb0 += 2) {
+          FU_BLOCK_B(f2, f3, sb0)
+          FU_BLOCK_B(f0, f1, sb0 + 1)
+        }
+        f0 = f2;                            // the diagonal block's fragments
+        f1 = f3;
+      } else {
+        for (int sb0 = 0; sb0 < lb; sb0 += 2) {
+          FU_BLOCK_B(f0, f1, sb0)
+          FU_BLOCK_B(f2, f3, sb0 + 1)
+        }
+      }
+#undef FU_BLOCK_B
+      // diagonal block: the per-row factor once, then the factor of every element
       const float rf = exp2_hw(fminf(dal - prev_end, 0.0f));
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -308,8 +344,7 @@ void ssd_fused_kernel(const SsdFusedParams p) {
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
         const int ks = 2 * lb + kk;
-        const bf16x8_t f = fnext;
-        if (kk == 0) fnext = load_frag(cbf + (size_t)(ks + 1) * FRAG);
+        const bf16x8_t f = kk == 0 ? f0 : f1;
         const int sbase = 16 * ks + 8 * g2;
         const float4 a0 = *reinterpret_cast<const float4 *>(dAs + sbase), a1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
         const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
@@ -317,9 +352,9 @@ void ssd_fused_kernel(const SsdFusedParams p) {
         const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
         float mv[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float v = (float)f[j] * exp2_hw(dal - das[j]) * dtv[j];
-          mv[j] = (sbase + j <= lrow) ? v : 0.0f;
+        for (int jj = 0; jj < 8; ++jj) {
+          const float v = (float)f[jj] * exp2_hw(dal - das[jj]) * dtv[jj];
+          mv[jj] = (sbase + jj <= lrow) ? v : 0.0f;
         }
         const bf16x8_t bf = pack8(mv);
 #pragma unroll
@@ -329,9 +364,78 @@ void ssd_fused_kernel(const SsdFusedParams p) {
           acc[pt] = mma(a, bf, acc[pt]);
         }
       }
+      // skip term D x_l from the plain tile (this lane's column l, the 16 rows p of each half)
+      if constexpr (DMODE != 0) {
+        const int xcol = lrow & 7, xchunk = lrow >> 3;
+        const float dh = DMODE == 1 ? p.Dk[h] : 0.0f;
+#pragma unroll
+        for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float dv[4] = {dh, dh, dh, dh};
+            if constexpr (DMODE == 2) {
+              const float4 d4 = *reinterpret_cast<const float4 *>(p.Dk + (size_t)h * FU_P + 32 * pt + 8 * q + 4 * g2);
+              dv[0] = d4.x; dv[1] = d4.y; dv[2] = d4.z; dv[3] = d4.w;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int prow = 32 * pt + 8 * q + 4 * g2 + j;
+              const float xv = (float)xr[prow * Q + ((xchunk ^ (prow & qmask)) << 3) + xcol];
+              acc[pt][4 * q + j] = __builtin_fmaf(dv[j], xv, acc[pt][4 * q + j]);
+            }
+          }
+      }
+    }
+
+    // gate operands of this wave's rows, in the row-major order of the output pass
+    bf16x8_t zreg[2], znext[2];
+    const __bf16 *zg = p.z + (xg - p.x) + (size_t)(32 * lb + (lane >> 2)) * xrow + 8 * (lane & 3);
+    if (yact && HAS_Z) {                   // requested now, used after the state update
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+        zreg[pass] = load_frag(zg + (size_t)(16 * pass) * xrow);
+        znext[pass] = load_frag(zg + (size_t)(16 * pass) * xrow + 32);
+      }
+    }
+    // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p]
+    if (sact) {
+      const __bf16 *btf = p.Btblk + ((unit * KS) * NT + nt_s) * FRAG + lane * 8;
+      const size_t kstep = (size_t)NT * FRAG;
+      f0 = load_frag(btf);
+      f1 = load_frag(btf + kstep);
+      f2 = load_frag(btf + (size_t)min(2, KS - 1) * kstep);
+      f3 = load_frag(btf + (size_t)min(3, KS - 1) * kstep);
+      float prev_end = 0.0f;
+      const int prow = 32 * pt_s + m;
+#define FU_STEP_C(F, KK)                                                                        \
+      {                                                                                         \
+        const bf16x8_t f = F;                                                                   \
+        F = load_frag(btf + (size_t)min((KK) + 4, KS - 1) * kstep);                             \
+        const bf16x8_t xf = load_frag(xw + prow * Q + (((2 * (KK) + g2) ^ (prow & qmask)) << 3)); \
+        S = mma(f, xf, S);                                                                      \
+      }
+      for (int k0 = 0; k0 < KS; k0 += 4) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          {
+            const float endv = dAs[16 * (k0 + 2 * half) + 31];
+            const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));
+            prev_end = endv;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) S[r] *= gs;
+          }
+          if (half == 0) {
+            FU_STEP_C(f0, k0)
+            FU_STEP_C(f1, k0 + 1)
+          } else {
+            FU_STEP_C(f2, k0 + 2)
+            FU_STEP_C(f3, k0 + 3)
+          }
+        }
+      }
+#undef FU_STEP_C
     }
     __syncthreads();                       // the plain tile is free: it becomes the output staging
-
     // ---- output: through a wave-private 32 x 32 fp32 tile to row-major 16-byte accesses
     if (yact) {
       float *stg = reinterpret_cast<float *>(smem + FU_TILE_BYTES) + wave * 1024;
@@ -344,65 +448,19 @@ void ssd_fused_kernel(const SsdFusedParams p) {
           *reinterpret_cast<float4 *>(stg + m * 32 + (((2 * q + g2) ^ (m & 7)) << 2)) = v;
         }
         wave_lds_sync();
-        bf16x8_t zcur[2] = {zreg[0], zreg[1]}, xcur[2] = {xreg[0], xreg[1]};
-        if (pt == 0) {
-#pragma unroll
-          for (int pass = 0; pass < 2; ++pass) {
-            xreg[pass] = load_frag(xg + row_at + (size_t)(16 * pass) * xrow + 32);
-            if (p.z) zreg[pass] = load_frag(p.z + (xg - p.x) + row_at + (size_t)(16 * pass) * xrow + 32);
-          }
-        }
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
           const int l = (lane >> 2) + 16 * pass, c4 = lane & 3;
           const float4 v0 = *reinterpret_cast<const float4 *>(stg + l * 32 + (((2 * c4) ^ (l & 7)) << 2));
           const float4 v1 = *reinterpret_cast<const float4 *>(stg + l * 32 + (((2 * c4 + 1) ^ (l & 7)) << 2));
           float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-          const int pcol = 32 * pt + 8 * c4;
-          if (p.Dk) {
-            float dk[8];
-            if (p.d_per_p) {
-              const float4 d0 = *reinterpret_cast<const float4 *>(p.Dk + (size_t)h * FU_P + pcol);
-              const float4 d1 = *reinterpret_cast<const float4 *>(p.Dk + (size_t)h * FU_P + pcol + 4);
-              dk[0] = d0.x; dk[1] = d0.y; dk[2] = d0.z; dk[3] = d0.w; dk[4] = d1.x; dk[5] = d1.y; dk[6] = d1.z; dk[7] = d1.w;
-            } else {
-              const float dh = p.Dk[h];
+          if (HAS_Z) {
 #pragma unroll
-              for (int j = 0; j < 8; ++j) dk[j] = dh;
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = __builtin_fmaf(dk[j], (float)xcur[pass][j], v[j]);
+            for (int j = 0; j < 8; ++j) v[j] *= silu_f32((float)(pt == 0 ? zreg[pass][j] : znext[pass][j]));
           }
-          if (p.z) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] *= silu_f32((float)zcur[pass][j]);
-          }
-          *reinterpret_cast<bf16x8_t *>(yg + (size_t)(32 * lb + l) * xrow + pcol) = pack8(v);
+          *reinterpret_cast<bf16x8_t *>(yg + (size_t)(32 * lb + l) * xrow + 32 * pt + 8 * c4) = pack8(v);
         }
         wave_lds_sync();
-      }
-    }
-
-    // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p]
-    if (sact) {
-      const __bf16 *btf = p.Btblk + ((unit * KS) * NT + nt_s) * FRAG + lane * 8;
-      bf16x8_t fnext = load_frag(btf);
-      float prev_end = 0.0f;
-      const int prow = 32 * pt_s + m;
-      for (int sb = 0; sb < NLB; ++sb) {
-        const float endv = dAs[32 * sb + 31];
-        const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));
-        prev_end = endv;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) S[r] *= gs;
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          const int ks = 2 * sb + kk;
-          const bf16x8_t f = fnext;
-          if (ks + 1 < KS) fnext = load_frag(btf + (size_t)(ks + 1) * NT * FRAG);
-          const bf16x8_t xf = load_frag(xw + prow * Q + (((2 * ks + g2) ^ (prow & qmask)) << 3));
-          S = mma(f, xf, S);
-        }
       }
     }
   }
@@ -440,8 +498,8 @@ static FusedLayout fused_layout(const SsdDims &d) {
 }
 
 static bool fused_shape_ok(const SsdDims &d) {
-  const bool q_ok = d.chunk == 32 || d.chunk == 64 || d.chunk == 128 || d.chunk == 256;
-  const bool n_ok = d.nstate == 32 || d.nstate == 64 || d.nstate == 128;
+  const bool q_ok = d.chunk == 64 || d.chunk == 128 || d.chunk == 256;
+  const bool n_ok = d.nstate == 64 || d.nstate == 128;
   return q_ok && n_ok && d.hdim == FU_P && d.len % d.chunk == 0 && d.heads % d.groups == 0;
 }
 
@@ -484,7 +542,7 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   SSM_REQUIRE(a->io_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE, "ssm_ssd_combined_fwd: x, z, y, Bm and Cm must be bf16");
   SSM_REQUIRE(valid_dtype(a->dt_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_combined_fwd: dt_dtype=%d", a->dt_dtype);
   SSM_REQUIRE(fused_shape_ok(d), SSM_ERR_BAD_SHAPE,
-              "ssm_ssd_combined_fwd: needs headdim 64, chunk in {32,64,128,256}, nstate in {32,64,128} and "
+              "ssm_ssd_combined_fwd: needs headdim 64, chunk in {64,128,256}, nstate in {64,128} and "
               "seqlen %% chunk == 0 (got headdim=%d chunk=%d nstate=%d seqlen=%d)",
               d.hdim, d.chunk, d.nstate, d.len);
   const FusedLayout lay = fused_layout(d);
@@ -536,12 +594,24 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   fp.Dk = a->Dskip; fp.init = a->initial_states; fp.final_states = a->final_states;
   fp.batch = d.batch; fp.len = d.len; fp.heads = d.heads; fp.groups = d.groups; fp.nstate = d.nstate; fp.chunk = d.chunk;
   fp.nchunks = d.nchunks; fp.d_per_p = a->d_per_p ? 1 : 0;
-  if (allow_dynamic_lds(ssd_fused_kernel, FU_LDS_BYTES) != hipSuccess) {
-    (void)hipGetLastError();
-    set_error("ssm_ssd_combined_fwd: cannot reserve %d bytes of LDS", FU_LDS_BYTES);
-    return SSM_ERR_LAUNCH;
+  const int dmode = !a->Dskip ? 0 : (a->d_per_p ? 2 : 1);
+  const unsigned grid = (unsigned)(d.batch * d.heads);
+#define SSM_LAUNCH_FUSED(DM, HZ)                                                                   \
+  {                                                                                                \
+    auto kernel = ssd_fused_kernel<DM, HZ>;                                                        \
+    if (allow_dynamic_lds(kernel, FU_LDS_BYTES) != hipSuccess) {                                   \
+      (void)hipGetLastError();                                                                     \
+      set_error("ssm_ssd_combined_fwd: cannot reserve %d bytes of LDS", FU_LDS_BYTES);             \
+      return SSM_ERR_LAUNCH;                                                                       \
+    }                                                                                              \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(FU_THREADS), FU_LDS_BYTES, s, fp);                 \
   }
-  hipLaunchKernelGGL(ssd_fused_kernel, dim3((unsigned)(d.batch * d.heads)), dim3(FU_THREADS), FU_LDS_BYTES, s, fp);
+  if (a->z) {
+    if (dmode == 0) SSM_LAUNCH_FUSED(0, true) else if (dmode == 1) SSM_LAUNCH_FUSED(1, true) else SSM_LAUNCH_FUSED(2, true)
+  } else {
+    if (dmode == 0) SSM_LAUNCH_FUSED(0, false) else if (dmode == 1) SSM_LAUNCH_FUSED(1, false) else SSM_LAUNCH_FUSED(2, false)
+  }
+#undef SSM_LAUNCH_FUSED
   SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd");
   note_mfma_launch(8);
   return SSM_OK;

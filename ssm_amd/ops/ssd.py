@@ -246,6 +246,9 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
     return y
 
 
+_KEEP_WORKSPACE = []      # debugging aid: when non-empty, receives [workspace tensor, offset] of the last one-pass call
+
+
 def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
     """Whether the one-pass kernel covers this call (bf16 tensors on the GPU and a
     shape ``ssm_ssd_combined_supported`` accepts)."""
@@ -287,6 +290,8 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
         dt_softplus=int(bool(dt_softplus)), d_per_p=int(d_per_p),
         dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]))
     _lib.call("ssm_ssd_combined_fwd", args, dev)
+    if _KEEP_WORKSPACE:
+        _KEEP_WORKSPACE[:] = [work, off]
     if return_final_states:
         return y, final
     return y
@@ -329,7 +334,7 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
     can_fuse = not force_generic and fused is not False and \
         _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
     _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "
-          "chunk in {32,64,128,256}, nstate in {32,64,128} and seqlen % chunk == 0.")
+          "chunk in {64,128,256}, nstate in {64,128} and seqlen % chunk == 0.")
     if can_fuse:
         return _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit,
                           return_final_states, (batch, seqlen, heads, hdim, groups, nstate))

@@ -152,8 +152,8 @@ FUSED_CASES = [
     ((2, 512, 4, 64, 1, 128), 256, False, True, True),
     ((1, 1024, 3, 64, 1, 128), 256, True, True, False),
     ((2, 384, 4, 64, 2, 64), 128, False, False, True),
-    ((1, 256, 2, 64, 2, 32), 64, True, True, True),
-    ((3, 96, 2, 64, 1, 64), 32, False, True, False),
+    ((1, 256, 2, 64, 2, 64), 64, True, True, True),
+    ((3, 192, 2, 64, 1, 64), 64, False, True, False),
     ((1, 256, 1, 64, 1, 128), 256, False, False, False),
 ]
 
