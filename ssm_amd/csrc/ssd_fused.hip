@@ -49,75 +49,96 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 __device__ __forceinline__ void wave_lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 // ------------------------------------------------------------------ prep: dt
-// One wave per (b, h, c): step, running sums and the staged weight
-//   ws[l] = dt_l exp(cs[l | 31] - cs[l]).
+// One workgroup per (b, c, 4 heads): the (Q x 4) slab of dt is read row by row
+// (16 contiguous bytes per step) into LDS transposed to [head][step]; then one
+// wave per head forms dt' = clamp(softplus(dt + bias)), the running sum of dt' A
+// and the staged weight  ws[l] = dt'_l exp(cs[l | 31] - cs[l]).
+constexpr int PD_HEADS = 4;
 __global__ __launch_bounds__(256) void ssd_fused_prep_dt_kernel(const SsdCumsumParams p, float *dA2, float *ws) {
-  __shared__ float cs[4][256];
+  __shared__ float tile[PD_HEADS][256 + 1];
   const SsdDims &d = p.d;
+  const int Q = d.chunk;
+  const int hgroups = (d.heads + PD_HEADS - 1) / PD_HEADS;
+  const int hg = (int)blockIdx.x % hgroups;
+  const int c = ((int)blockIdx.x / hgroups) % d.nchunks;
+  const int b = (int)blockIdx.x / (hgroups * d.nchunks);
+  const int h0 = hg * PD_HEADS;
+  for (int e = threadIdx.x; e < Q * PD_HEADS; e += 256) {
+    const int l = e / PD_HEADS, hh = e % PD_HEADS;
+    float v = 0.0f;
+    if (h0 + hh < d.heads) v = load_as_f32(p.dt, p.dt_dtype, ((size_t)b * d.len + (size_t)c * Q + l) * d.heads + h0 + hh);
+    tile[hh][l] = v;
+  }
+  __syncthreads();
   const int wave = wave_id_uniform(), lane = lane_id();
-  const size_t unit = (size_t)blockIdx.x * 4 + wave;
-  if (unit >= (size_t)d.batch * d.heads * d.nchunks) return;
-  const int c = (int)(unit % d.nchunks);
-  const int h = (int)((unit / d.nchunks) % d.heads);
-  const int b = (int)(unit / ((size_t)d.nchunks * d.heads));
-  const int Q = d.chunk, per = (Q + 63) >> 6;
-  const float A = p.A[h];
-  const float bias = p.bias ? p.bias[h] : 0.0f;
-  float v[4], run[4];
-  float tot = 0.0f;
+  const int per = (Q + 63) >> 6;
+  for (int hh = wave; hh < PD_HEADS; hh += 4) {
+    const int h = h0 + hh;
+    if (h >= d.heads) break;
+    const float A = p.A[h];
+    const float bias = p.bias ? p.bias[h] : 0.0f;
+    float v[4], run[4];
+    float tot = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int l = lane * per + i;
-    v[i] = 0.0f;
-    if (i < per && l < Q) {
-      float x = load_as_f32(p.dt, p.dt_dtype, ((size_t)b * d.len + (size_t)c * Q + l) * d.heads + h) + bias;
-      if (p.softplus) x = softplus_f32(x);
-      v[i] = fminf(fmaxf(x, p.dt_min), p.dt_max);
+    for (int i = 0; i < 4; ++i) {
+      const int l = lane * per + i;
+      v[i] = 0.0f;
+      if (i < per && l < Q) {
+        float x = tile[hh][l] + bias;
+        if (p.softplus) x = softplus_f32(x);
+        v[i] = fminf(fmaxf(x, p.dt_min), p.dt_max);
+      }
+      tot = __builtin_fmaf(v[i], A, tot);
+      run[i] = tot;
     }
-    tot = __builtin_fmaf(v[i], A, tot);
-    run[i] = tot;
-  }
-  float incl = tot;
+    float incl = tot;
 #pragma unroll
-  for (int off = 1; off < WAVE; off <<= 1) {
-    const float t = __shfl_up(incl, off, WAVE);
-    if (lane >= off) incl += t;
-  }
-  const float excl = incl - tot;
-  const size_t out = unit * (size_t)Q;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int l = lane * per + i;
-    if (i < per && l < Q) {
-      const float a = excl + run[i];
-      cs[wave][l] = a;
-      p.dA_cs[out + l] = a;
-      p.dt_out[out + l] = v[i];
-      dA2[out + l] = a * LOG2E;
+    for (int off = 1; off < WAVE; off <<= 1) {
+      const float t = __shfl_up(incl, off, WAVE);
+      if (lane >= off) incl += t;
     }
-  }
-  wave_lds_sync();
+    const float excl = incl - tot;
+    const size_t out = (((size_t)b * d.heads + h) * d.nchunks + c) * (size_t)Q;
+    wave_lds_sync();                       // the row is re-used for the running sums
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int l = lane * per + i;
-    if (i < per && l < Q) ws[out + l] = v[i] * decay_exp(cs[wave][l | 31] - cs[wave][l]);
+    for (int i = 0; i < 4; ++i) {
+      const int l = lane * per + i;
+      if (i < per && l < Q) {
+        const float a = excl + run[i];
+        tile[hh][l] = a;
+        p.dA_cs[out + l] = a;
+        p.dt_out[out + l] = v[i];
+        dA2[out + l] = a * LOG2E;
+      }
+    }
+    wave_lds_sync();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int l = lane * per + i;
+      if (i < per && l < Q) ws[out + l] = v[i] * decay_exp(tile[hh][l | 31] - tile[hh][l]);
+    }
   }
 }
 
 // ---------------------------------------------------------------- prep: pack
 // Fragment (lane, j) of a 32 x 16 operand block: row 32 rb + lane % 32,
-// column 16 kb + 8 (lane / 32) + j.  One wave per fragment.
-//   which = 0: Cblk [(b,c,g)][lb][kn]  from C  (rows = time, columns = state)
-//   which = 1: CBblk[(b,c,g)][lb][ks]  from CB (rows = l, columns = s), lower blocks only
-//   which = 2: Btblk[(b,c,g)][ks][nt]  from B  (rows = state, columns = time)
-__global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *src, __bf16 *dst, int which, int batch, int len,
-                                                             int groups, int nstate, int chunk) {
+// column 16 kb + 8 (lane / 32) + j.  One wave per fragment; the first
+// B nc G (NLB KN) fragments are those of C, the rest those of B^T:
+//   Cblk [(b,c,g)][lb][kn]  from C  (rows = time, columns = state)
+//   Btblk[(b,c,g)][ks][nt]  from B  (rows = state, columns = time)
+// (CBblk[(b,c,g)][lb][ks], rows = l, columns = s, is written by the C B^T kernel.)
+__global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *Cm, const __bf16 *Bm, __bf16 *Cblk, __bf16 *Btblk,
+                                                             int batch, int len, int groups, int nstate, int chunk) {
   const int wave = wave_id_uniform(), lane = lane_id();
   const int Q = chunk, N = nstate, nc = len / Q;
   const int NLB = Q >> 5, KS = Q >> 4, KN = N >> 4, NT = N >> 5;
-  const int per_unit = which == 0 ? NLB * KN : (which == 1 ? NLB * KS : KS * NT);
-  const size_t f = (size_t)blockIdx.x * 4 + wave;
-  if (f >= (size_t)batch * nc * groups * per_unit) return;
+  const size_t units = (size_t)batch * nc * groups;
+  const size_t nC = units * NLB * KN, nB = units * KS * NT;
+  size_t f = (size_t)blockIdx.x * 4 + wave;
+  if (f >= nC + nB) return;
+  const bool is_c = f < nC;
+  if (!is_c) f -= nC;
+  const int per_unit = is_c ? NLB * KN : KS * NT;
   const int inner = (int)(f % per_unit);
   const size_t unit = f / per_unit;
   const int g = (int)(unit % groups);
@@ -125,20 +146,16 @@ __global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *src, 
   const int b = (int)(unit / ((size_t)groups * nc));
   const int m = lane & 31, g2 = lane >> 5;
   bf16x8_t v;
-  if (which == 0) {
+  if (is_c) {
     const int lb = inner / KN, kn = inner % KN;
-    v = load_frag(src + (((size_t)b * len + (size_t)c * Q + 32 * lb + m) * groups + g) * N + 16 * kn + 8 * g2);
-  } else if (which == 1) {
-    const int lb = inner / KS, ks = inner % KS;
-    if (ks > 2 * lb + 1) return;
-    v = load_frag(src + (unit * Q + 32 * lb + m) * (size_t)Q + 16 * ks + 8 * g2);
+    v = load_frag(Cm + (((size_t)b * len + (size_t)c * Q + 32 * lb + m) * groups + g) * N + 16 * kn + 8 * g2);
   } else {
     const int ks = inner / NT, nt = inner % NT;
-    const __bf16 *col = src + (((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * groups + g) * N + 32 * nt + m;
+    const __bf16 *col = Bm + (((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * groups + g) * N + 32 * nt + m;
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = col[(size_t)j * groups * N];
   }
-  *reinterpret_cast<bf16x8_t *>(dst + f * FRAG + lane * 8) = v;
+  *reinterpret_cast<bf16x8_t *>((is_c ? Cblk : Btblk) + f * FRAG + lane * 8) = v;
 }
 
 // --------------------------------------------------------------- fused kernel
@@ -476,7 +493,7 @@ void ssd_fused_kernel(const SsdFusedParams p) {
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct FusedLayout {
-  size_t dA_cs, dt_out, dA2, ws, Cblk, Btblk, CB, CBblk, total;
+  size_t dA_cs, dt_out, dA2, ws, Cblk, Btblk, CBblk, total;
 };
 
 static FusedLayout fused_layout(const SsdDims &d) {
@@ -491,7 +508,6 @@ static FusedLayout fused_layout(const SsdDims &d) {
   f.ws = at; at += per_step;
   f.Cblk = at; at += bc;
   f.Btblk = at; at += bc;
-  f.CB = at; at += cb;
   f.CBblk = at; at += cb;
   f.total = at;
   return f;
@@ -561,36 +577,32 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   cp.dA_cs = reinterpret_cast<float *>(ws + lay.dA_cs);
   cp.dt_out = reinterpret_cast<float *>(ws + lay.dt_out);
   cp.d = d; cp.dt_dtype = a->dt_dtype; cp.softplus = a->dt_softplus ? 1 : 0; cp.dt_min = a->dt_min; cp.dt_max = a->dt_max;
-  const size_t units = (size_t)d.batch * d.heads * d.nchunks;
-  hipLaunchKernelGGL(ssd_fused_prep_dt_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, cp,
+  const size_t units = (size_t)d.batch * d.nchunks * ((d.heads + PD_HEADS - 1) / PD_HEADS);
+  hipLaunchKernelGGL(ssd_fused_prep_dt_kernel, dim3((unsigned)units), dim3(256), 0, s, cp,
                      reinterpret_cast<float *>(ws + lay.dA2), reinterpret_cast<float *>(ws + lay.ws));
   SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(prep dt)");
 
   SsdBmmParams bp{};
-  bp.a = a->Cm; bp.b = a->Bm; bp.seq_idx = nullptr; bp.out = ws + lay.CB;
+  bp.a = a->Cm; bp.b = a->Bm; bp.seq_idx = nullptr; bp.out = ws + lay.CBblk;
   bp.batch = d.batch; bp.len = d.len; bp.groups = d.groups; bp.kdim = d.nstate; bp.chunk = d.chunk; bp.nchunks = d.nchunks;
-  bp.in_dtype = SSM_BF16; bp.out_dtype = SSM_BF16; bp.causal = 1;
+  bp.in_dtype = SSM_BF16; bp.out_dtype = SSM_BF16; bp.causal = 1; bp.blocked = 1;
   SSM_REQUIRE(ssd_bmm_mfma(bp, s), SSM_ERR_BAD_SHAPE, "ssm_ssd_combined_fwd: C B^T kernel rejected the shape");
   SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(bmm)");
 
   const size_t bcg = (size_t)d.batch * d.nchunks * d.groups;
   const int NLB = d.chunk >> 5, KS = d.chunk >> 4, KN = d.nstate >> 4, NT = d.nstate >> 5;
-  const __bf16 *srcs[3] = {reinterpret_cast<const __bf16 *>(a->Cm), reinterpret_cast<const __bf16 *>(ws + lay.CB),
-                           reinterpret_cast<const __bf16 *>(a->Bm)};
-  __bf16 *dsts[3] = {reinterpret_cast<__bf16 *>(ws + lay.Cblk), reinterpret_cast<__bf16 *>(ws + lay.CBblk),
-                     reinterpret_cast<__bf16 *>(ws + lay.Btblk)};
-  const size_t frags[3] = {bcg * NLB * KN, bcg * NLB * KS, bcg * KS * NT};
-  for (int which = 0; which < 3; ++which) {
-    hipLaunchKernelGGL(ssd_fused_pack_kernel, dim3((unsigned)((frags[which] + 3) / 4)), dim3(256), 0, s, srcs[which],
-                       dsts[which], which, d.batch, d.len, d.groups, d.nstate, d.chunk);
-    SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(pack)");
-  }
+  __bf16 *Cblk = reinterpret_cast<__bf16 *>(ws + lay.Cblk), *Btblk = reinterpret_cast<__bf16 *>(ws + lay.Btblk);
+  const size_t frags = bcg * NLB * KN + bcg * KS * NT;
+  hipLaunchKernelGGL(ssd_fused_pack_kernel, dim3((unsigned)((frags + 3) / 4)), dim3(256), 0, s,
+                     reinterpret_cast<const __bf16 *>(a->Cm), reinterpret_cast<const __bf16 *>(a->Bm), Cblk, Btblk,
+                     d.batch, d.len, d.groups, d.nstate, d.chunk);
+  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(pack)");
 
   SsdFusedParams fp{};
   fp.x = reinterpret_cast<const __bf16 *>(a->x); fp.z = reinterpret_cast<const __bf16 *>(a->z);
   fp.y = reinterpret_cast<__bf16 *>(a->y);
   fp.dA2 = reinterpret_cast<const float *>(ws + lay.dA2); fp.dtv = cp.dt_out; fp.ws = reinterpret_cast<const float *>(ws + lay.ws);
-  fp.Cblk = dsts[0]; fp.CBblk = dsts[1]; fp.Btblk = dsts[2];
+  fp.Cblk = Cblk; fp.CBblk = reinterpret_cast<const __bf16 *>(ws + lay.CBblk); fp.Btblk = Btblk;
   fp.Dk = a->Dskip; fp.init = a->initial_states; fp.final_states = a->final_states;
   fp.batch = d.batch; fp.len = d.len; fp.heads = d.heads; fp.groups = d.groups; fp.nstate = d.nstate; fp.chunk = d.chunk;
   fp.nchunks = d.nchunks; fp.d_per_p = a->d_per_p ? 1 : 0;
