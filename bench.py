@@ -253,6 +253,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="only the headline kernel")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
+                         "the reference for hardware byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every operator on this path is independent per "
@@ -262,6 +265,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm device", file=sys.stderr)
         sys.exit(1)
+
+    if args.copy_calibration:
+        src = torch.full((64 * 1024 * 1024,), 1.0, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 0.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
+    from ssm_amd import configs
 
     r = bench_scan_fwd(args.steps, args.warmup)
     value = r["bytes"] / r["wall_s"] / 1e9
@@ -285,7 +298,8 @@ def main():
                    "tokens_per_s": round(r["tokens"] / r["wall_s"], 1),
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": configs.scan_fwd_headline_traffic_bytes(),
                      "kernel": "scan_fwd_kernel<bf16, 8>", "kernel_us": round(r["kernel_ms"] * 1e3, 2),
                      "algorithmic_bytes": r["bytes"]},
     }

@@ -1,7 +1,11 @@
-"""Turn the CSV that ``rocprofv3 --kernel-trace --stats`` writes into the short
-text summary kept under ``profiles/``.
+"""Turn the CSV files that ``rocprofv3`` writes into the short text summaries kept
+under ``profiles/``.
 
     python -m ssm_amd.profile_summary <dir-with-*_kernel_stats.csv> "<command that was profiled>"
+    python -m ssm_amd.profile_summary --pmc <dir-with-*_counter_collection.csv> "<command>"
+
+The second form averages every hardware counter per kernel over its dispatches
+(``rocprofv3 --pmc`` output).
 """
 
 from __future__ import annotations
@@ -27,5 +31,23 @@ def summarise(folder: str, command: str, top: int = 25) -> str:
     return "\n".join(out) + "\n"
 
 
+def summarise_pmc(folder: str, command: str) -> str:
+    files = glob.glob(f"{folder}/**/*counter_collection.csv", recursive=True)
+    if not files:
+        raise SystemExit(f"no *counter_collection.csv under {folder}")
+    acc = {}
+    for r in csv.DictReader(open(files[0])):
+        acc.setdefault((r["Kernel_Name"], r["Counter_Name"]), []).append(float(r["Counter_Value"]))
+    out = [f"command: {command}", f"source:  {files[0].split('/')[-1]} (rocprofv3 --pmc)", "",
+           f"{'kernel':<96} {'counter':<24} {'dispatches':>10} {'mean per dispatch':>20}"]
+    for (name, counter), vals in sorted(acc.items(), key=lambda kv: (-sum(kv[1]), kv[0])):
+        name = name if len(name) <= 95 else name[:92] + "..."
+        out.append(f"{name:<96} {counter:<24} {len(vals):>10} {sum(vals) / len(vals):>20.1f}")
+    return "\n".join(out) + "\n"
+
+
 if __name__ == "__main__":
-    sys.stdout.write(summarise(sys.argv[1], sys.argv[2] if len(sys.argv) > 2 else "?"))
+    if len(sys.argv) > 1 and sys.argv[1] == "--pmc":
+        sys.stdout.write(summarise_pmc(sys.argv[2], sys.argv[3] if len(sys.argv) > 3 else "?"))
+    else:
+        sys.stdout.write(summarise(sys.argv[1], sys.argv[2] if len(sys.argv) > 2 else "?"))
