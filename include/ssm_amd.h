@@ -154,6 +154,39 @@ typedef struct ssm_state_step_args {
 
 int ssm_state_step(const ssm_state_step_args *args, void *hip_stream);
 
+/* Backward of the state update.  Stands behind the backend call
+ * `selective_state_step_backward(grad_out, grad_state, state, x, dt, A, B, C, D,
+ * z, dt_bias, softplus)` made at src/ssm/ops/__init__.py:654-668 (nine
+ * gradients; formulas follow src/ssm/ops/cpu/state_step.cpp's backward).
+ * `state` is the state BEFORE the step; `grad_state` is the gradient with
+ * respect to the updated state. */
+typedef struct ssm_state_step_bwd_args {
+  const void *grad_out;    /* (B, D) io dtype, or NULL (zero) */
+  const void *grad_state;  /* (B, D, N) state dtype, or NULL (zero) */
+  const void *state;       /* (B, D, N) state dtype */
+  const void *x, *dt;      /* (B, D) io dtype */
+  const void *z;           /* (B, D) io dtype, or NULL */
+  const float *A;          /* (D, N) fp32 */
+  const void *Bproj, *Cproj; /* as in ssm_state_step_args */
+  const float *Dskip;      /* (D,) fp32 or NULL */
+  const float *dt_bias;    /* (D,) fp32 or NULL */
+  void *dstate;            /* (B, D, N) state dtype */
+  void *dx, *ddt;          /* (B, D) io dtype */
+  void *dz;                /* (B, D) io dtype; given exactly when z is */
+  float *dA;               /* (D, N) */
+  float *dB, *dC;          /* fp32, shaped like Bproj / Cproj */
+  float *dD, *ddt_bias;    /* (D,) or NULL */
+  void *workspace;         /* ssm_state_step_bwd_workspace_bytes() bytes */
+  size_t workspace_bytes;
+  int32_t batch, dim, nstate;
+  int32_t state_dtype, io_dtype, bc_dtype;
+  int32_t b_kind, c_kind, b_groups, c_groups;
+  int32_t dt_softplus;
+} ssm_state_step_bwd_args;
+
+size_t ssm_state_step_bwd_workspace_bytes(int batch, int dim, int nstate);
+int ssm_state_step_bwd(const ssm_state_step_bwd_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * fused decode step: roll the causal-conv window, apply the depthwise conv and
  * its activation to the new input, then run the selective state update on the

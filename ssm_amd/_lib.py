@@ -70,6 +70,19 @@ class StateStepArgs(C.Structure):
     ]
 
 
+class StateStepBwdArgs(C.Structure):
+    _fields_ = [
+        ("grad_out", _vp), ("grad_state", _vp), ("state", _vp), ("x", _vp), ("dt", _vp), ("z", _vp), ("A", _vp),
+        ("Bproj", _vp), ("Cproj", _vp), ("Dskip", _vp), ("dt_bias", _vp),
+        ("dstate", _vp), ("dx", _vp), ("ddt", _vp), ("dz", _vp), ("dA", _vp), ("dB", _vp), ("dC", _vp),
+        ("dD", _vp), ("ddt_bias", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
+        ("batch", _i32), ("dim", _i32), ("nstate", _i32),
+        ("state_dtype", _i32), ("io_dtype", _i32), ("bc_dtype", _i32),
+        ("b_kind", _i32), ("c_kind", _i32), ("b_groups", _i32), ("c_groups", _i32),
+        ("dt_softplus", _i32),
+    ]
+
+
 class DecodeStepArgs(C.Structure):
     _fields_ = [("step", StateStepArgs), ("conv_state", _vp), ("conv_weight", _vp), ("conv_bias", _vp),
                 ("conv_out", _vp), ("conv_width", _i32), ("conv_activation", _i32)]
@@ -177,6 +190,7 @@ ENTRY_POINTS = {
     "ssm_scan_fwd": ScanFwdArgs,
     "ssm_scan_bwd": ScanBwdArgs,
     "ssm_state_step": StateStepArgs,
+    "ssm_state_step_bwd": StateStepBwdArgs,
     "ssm_decode_step": DecodeStepArgs,
     "ssm_dscan_fwd": DscanFwdArgs,
     "ssm_ssd_chunk_cumsum": SsdCumsumArgs,
@@ -197,6 +211,7 @@ PLAIN_SYMBOLS = {
     "ssm_amd_last_error": (C.c_char_p, []),
     "ssm_scan_chunk_len": (C.c_int, []),
     "ssm_scan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 8),
+    "ssm_state_step_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 3),
     "ssm_dscan_fwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ssm_ssd_chunk_state_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
     "ssm_ssd_mfma_launches": (C.c_int, []),

@@ -44,6 +44,12 @@ inline hipError_t allow_dynamic_lds(KernelT kernel, size_t bytes) {
                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
+// Deterministic sums of per-block partials (defined in scan_bwd.hip):
+//   rows: out[i]    = sum_{j < count} in[j * inner + i]
+//   sum:  out[o][i] = sum_{j < count} in[(o * count + j) * inner + i]
+void launch_fold_rows(const float *in, float *out, int count, size_t inner, hipStream_t s);
+void launch_fold_sum(const float *in, float *out, size_t outer, int count, size_t inner, hipStream_t s);
+
 // -------------------------------------------------------------- device side
 
 constexpr int WAVE = 64;

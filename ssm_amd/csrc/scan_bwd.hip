@@ -452,6 +452,14 @@ static unsigned fold_grid(size_t n) {
   return (unsigned)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
 }
 
+void launch_fold_rows(const float *in, float *out, int count, size_t inner, hipStream_t s) {
+  hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid(inner)), dim3(256), 0, s, in, out, count, inner);
+}
+
+void launch_fold_sum(const float *in, float *out, size_t outer, int count, size_t inner, hipStream_t s) {
+  hipLaunchKernelGGL(fold_sum_kernel, dim3(fold_grid(outer * inner)), dim3(256), 0, s, in, out, outer, count, inner);
+}
+
 struct BwdPlan {
   int rows_per_wg, nblk;
   size_t off_dA, off_dD, off_dbias, off_dB, off_dC, total;   // byte offsets into the workspace

@@ -263,6 +263,44 @@ class StepPlan:
         return self.out
 
 
+def _state_step_backward(grad_out, grad_state, state, x, dt, A, B, C, D, z, dt_bias, softplus):
+    """Run ``ssm_state_step_bwd``: the nine gradients of one state update, in the order
+    ``(state, x, dt, A, B, C, D, z, dt_bias)``.  ``state`` is the state before the step;
+    ``grad_out`` / ``grad_state`` (gradient of the updated state) may be ``None``.
+    Parameter gradients come back in float32, the others in the dtype of their tensor."""
+    batch, dim, nstate, (bkind, bgroups), (ckind, cgroups) = \
+        K.check_state_step(state, x, dt, A, B, C, D, z, dt_bias)
+    dev = K.require_gpu(state, x, dt, A, B, C, D, z, dt_bias, grad_out, grad_state)
+    io = K.common_io_dtype([x, dt, z])
+    bc = K.common_io_dtype([B, C])
+    sc = K.cast_c(state, state.dtype)
+    xc, dtc, zc = K.cast_c(x, io), K.cast_c(dt, io), K.cast_c(z, io)
+    Bc, Cc = K.cast_c(B, bc), K.cast_c(C, bc)
+    Af, Df, bf = K.as_f32_vec(A), K.as_f32_vec(D), K.as_f32_vec(dt_bias)
+    go = K.cast_c(grad_out, io) if grad_out is not None else None
+    gs = K.cast_c(grad_state, state.dtype) if grad_state is not None else None
+    dstate = torch.empty_like(sc)
+    dx, ddt = torch.empty_like(xc), torch.empty_like(dtc)
+    dz = torch.empty_like(zc) if zc is not None else None
+    dA = torch.empty(dim, nstate, dtype=torch.float32, device=dev)
+    dB = torch.empty(Bc.shape, dtype=torch.float32, device=dev)
+    dC = torch.empty(Cc.shape, dtype=torch.float32, device=dev)
+    dD = torch.empty(dim, dtype=torch.float32, device=dev) if D is not None else None
+    dbias = torch.empty(dim, dtype=torch.float32, device=dev) if dt_bias is not None else None
+    nbytes = int(_lib.load().ssm_state_step_bwd_workspace_bytes(batch, dim, nstate))
+    work = torch.empty(nbytes // 4, dtype=torch.float32, device=dev)
+    args = _lib.StateStepBwdArgs(
+        grad_out=_lib.ptr(go), grad_state=_lib.ptr(gs), state=_lib.ptr(sc), x=_lib.ptr(xc), dt=_lib.ptr(dtc),
+        z=_lib.ptr(zc), A=_lib.ptr(Af), Bproj=_lib.ptr(Bc), Cproj=_lib.ptr(Cc), Dskip=_lib.ptr(Df),
+        dt_bias=_lib.ptr(bf), dstate=_lib.ptr(dstate), dx=_lib.ptr(dx), ddt=_lib.ptr(ddt), dz=_lib.ptr(dz),
+        dA=_lib.ptr(dA), dB=_lib.ptr(dB), dC=_lib.ptr(dC), dD=_lib.ptr(dD), ddt_bias=_lib.ptr(dbias),
+        workspace=_lib.ptr(work), workspace_bytes=nbytes, batch=batch, dim=dim, nstate=nstate,
+        state_dtype=_lib.dtype_enum(sc.dtype), io_dtype=_lib.dtype_enum(io), bc_dtype=_lib.dtype_enum(bc),
+        b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups, dt_softplus=int(bool(softplus)))
+    _lib.call("ssm_state_step_bwd", args, dev)
+    return dstate, dx, ddt, dA, dB, dC, dD, dz, dbias
+
+
 def selective_state_step(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, softplus=True):
     """Advance the selective state by one token on the GPU; ``state`` is updated in place.
 

@@ -119,7 +119,42 @@ class SelectiveScanFn(torch.autograd.Function):
         return out + (None, None)
 
 
+class StateStepFn(torch.autograd.Function):
+    """One state update as a function ``(state, ...) -> (y, new_state)``; the role of the
+    reference's ``_SelectiveStateStepCudaFunction`` (src/ssm/ops/__init__.py:570-668)."""
+
+    @staticmethod
+    def forward(ctx, state, x, dt, A, B, C, D, z, dt_bias, softplus):
+        from . import StepPlan
+
+        work = state.detach().clone().contiguous()
+        plan = StepPlan(work, x.detach(), dt.detach(), A.detach(), B.detach(), C.detach(),
+                        None if D is None else D.detach(), None if z is None else z.detach(),
+                        None if dt_bias is None else dt_bias.detach(), softplus)
+        out = plan.run()
+        if out.dtype != plan.result_dtype:
+            out = out.to(plan.result_dtype)
+        # the caller overwrites `state` afterwards: keep the values the step started from
+        ctx.save_for_backward(state.detach().clone(), x, dt, A, B, C, D, z, dt_bias)
+        ctx.softplus = softplus
+        return out, work
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_state):
+        from . import _state_step_backward
+
+        state, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors
+        grads = _state_step_backward(grad_out, grad_state, state, x, dt, A, B, C, D, z, dt_bias, ctx.softplus)
+        refs = (state, x, dt, A, B, C, D, z, dt_bias)
+        need = ctx.needs_input_grad
+        return tuple(_like(g, r) if (r is not None and need[i]) else None
+                     for i, (g, r) in enumerate(zip(grads, refs))) + (None,)
+
+
 def state_step_with_grad(state, x, dt, A, B, C, D, z, dt_bias, softplus):
-    raise NotImplementedError(
-        "selective_state_step has no backward kernel in this backend yet; call it under "
-        "torch.no_grad() (decode) or differentiate through selective_scan instead.")
+    """Differentiable state update: runs the kernels through ``StateStepFn`` and then
+    overwrites ``state`` with the new state, as the reference does
+    (src/ssm/ops/__init__.py:1376-1393)."""
+    out, new_state = StateStepFn.apply(state, x, dt, A, B, C, D, z, dt_bias, softplus)
+    state.copy_(new_state)
+    return out

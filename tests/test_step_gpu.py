@@ -197,3 +197,85 @@ def test_fused_decode_step_equals_conv_window_then_state_step(io, K):
     torch.testing.assert_close(xc_gpu.float().cpu(), xc.float(), **tol)
     torch.testing.assert_close(y.float().cpu(), y_ref.float(), **tol)
     torch.testing.assert_close(st.cpu(), st_ref, **(FP32_TOL if io == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
+
+
+# ---------------------------------------------------------------------------
+# backward: gradients of (y, new_state) against float64 autograd through the
+# CPU restatement of the step
+# ---------------------------------------------------------------------------
+
+def _oracle_grads(inp, softplus, gy, gs):
+    names = ["state", "x", "dt", "A", "B", "C", "D", "z", "dt_bias"]
+    leaves = {k: (inp[k].double().clone().requires_grad_(True) if inp.get(k) is not None else None) for k in names}
+    y, new_state = O.selective_state_step_functional(
+        leaves["state"], leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], D=leaves["D"],
+        z=leaves["z"], dt_bias=leaves["dt_bias"], softplus=softplus, acc=torch.float64)
+    loss = (y.double() * gy.double()).sum() + (new_state.double() * gs.double()).sum()
+    loss.backward()
+    return {k: (v.grad if v is not None else None) for k, v in leaves.items()}
+
+
+@pytest.mark.parametrize("kinds", [("dn", "dn"), ("bdn", "bgn"), ("bgn", "bdn"), ("bgn", "bgn")])
+@pytest.mark.parametrize("softplus", [True, False])
+def test_backward_matches_float64_autograd(kinds, softplus):
+    batch, dim, nstate, groups = 3, 8, 6, 2
+    inp = make(23, batch, dim, nstate, bkind=kinds[0], ckind=kinds[1], groups=groups)
+    if not softplus:
+        inp["dt"] = inp["dt"].abs() * 0.1
+        inp["dt_bias"] = inp["dt_bias"].abs() * 0.01
+    g = torch.Generator().manual_seed(5)
+    gy = torch.randn(batch, dim, generator=g)
+    gs = torch.randn(batch, dim, nstate, generator=g)
+    want = _oracle_grads(inp, softplus, gy, gs)
+    got = _ops()._state_step_backward(dev(gy), dev(gs), dev(inp["state"]), dev(inp["x"]), dev(inp["dt"]), dev(inp["A"]),
+                                      dev(inp["B"]), dev(inp["C"]), dev(inp["D"]), dev(inp["z"]), dev(inp["dt_bias"]),
+                                      softplus)
+    for name, gval in zip(["state", "x", "dt", "A", "B", "C", "D", "z", "dt_bias"], got):
+        torch.testing.assert_close(gval.cpu().double().reshape(want[name].shape), want[name], rtol=1e-4, atol=1e-5,
+                                   msg=lambda m, n=name: f"grad {n}: {m}")
+
+
+def test_backward_without_optional_inputs_and_with_missing_upstream_grads():
+    inp = make(29, 2, 5, 4, bkind="dn", ckind="bdn", use_D=False, use_z=False, use_bias=False)
+    g = torch.Generator().manual_seed(6)
+    gy = torch.randn(2, 5, generator=g)
+    want = _oracle_grads(inp, True, gy, torch.zeros(2, 5, 4))
+    got = _ops()._state_step_backward(dev(gy), None, dev(inp["state"]), dev(inp["x"]), dev(inp["dt"]), dev(inp["A"]),
+                                      dev(inp["B"]), dev(inp["C"]), None, None, None, True)
+    assert got[6] is None and got[7] is None and got[8] is None
+    for name, gval in zip(["state", "x", "dt", "A", "B", "C"], got[:6]):
+        torch.testing.assert_close(gval.cpu().double(), want[name], rtol=1e-4, atol=1e-5)
+
+
+def test_autograd_through_two_steps_matches_oracle():
+    """Back-propagation through time: two updates of the same state tensor."""
+    batch, dim, nstate = 2, 6, 4
+    a = make(31, batch, dim, nstate, bkind="bgn", ckind="bgn", groups=2)
+    b = make(32, batch, dim, nstate, bkind="bgn", ckind="bgn", groups=2)
+    ops = _ops()
+
+    def leaves_of(to, dtype):
+        return {k: to(a[k]).to(dtype).requires_grad_(True) for k in ["x", "dt", "A", "B", "C", "D", "z", "dt_bias"]}
+
+    # float64 oracle, functional chaining of the state
+    lw = leaves_of(lambda t: t, torch.float64)
+    y1, s1 = O.selective_state_step_functional(a["state"].double(), lw["x"], lw["dt"], lw["A"], lw["B"], lw["C"],
+                                               D=lw["D"], z=lw["z"], dt_bias=lw["dt_bias"], softplus=True,
+                                               acc=torch.float64)
+    y2, s2 = O.selective_state_step_functional(s1, b["x"].double(), b["dt"].double(), lw["A"], b["B"].double(),
+                                               b["C"].double(), D=lw["D"], z=b["z"].double(), dt_bias=lw["dt_bias"],
+                                               softplus=True, acc=torch.float64)
+    (y1.sum() + 2.0 * y2.sum() + s2.sum()).backward()
+
+    # GPU, the in-place API
+    lg = leaves_of(dev, torch.float32)
+    state = dev(a["state"]).clone()
+    z1 = ops.selective_state_step(state, lg["x"], lg["dt"], lg["A"], lg["B"], lg["C"], D=lg["D"], z=lg["z"],
+                                  dt_bias=lg["dt_bias"], softplus=True)
+    z2 = ops.selective_state_step(state, dev(b["x"]), dev(b["dt"]), lg["A"], dev(b["B"]), dev(b["C"]), D=lg["D"],
+                                  z=dev(b["z"]), dt_bias=lg["dt_bias"], softplus=True)
+    (z1.sum() + 2.0 * z2.sum() + state.sum()).backward()
+    torch.testing.assert_close(state.detach().cpu().double(), s2.detach(), rtol=1e-5, atol=1e-5)
+    for k in lw:
+        torch.testing.assert_close(lg[k].grad.cpu().double(), lw[k].grad, rtol=1e-4, atol=1e-5,
+                                   msg=lambda m, n=k: f"grad {n}: {m}")
