@@ -242,6 +242,38 @@ typedef struct ssm_dscan_fwd_args {
 size_t ssm_dscan_fwd_workspace_bytes(int batch, int seqlen, int heads, int proj);
 int ssm_dscan_fwd(const ssm_dscan_fwd_args *args, void *hip_stream);
 
+/* Backward of the diagonal chunk scan.  Stands behind the backend call
+ * `ssd_chunk_scan_backward(grad_out, X, dt, A, B, C, D, z, seq_lens, cu_seqlens,
+ * initial_states)` made at src/ssm/ops/__init__.py:869-884 (eight gradients:
+ * X, dt, A, B, C, D, z, initial_states).  Parameter gradients are fp32 and have
+ * the shape of the parameter; dX and dz have the dtype of X and z. */
+typedef struct ssm_dscan_bwd_args {
+  const void *grad_y;         /* (B, L, H, P) x dtype */
+  const void *X, *dt;         /* as in ssm_dscan_fwd_args */
+  const float *A;
+  const void *Bproj, *Cproj;
+  const float *Dskip;
+  const void *z;
+  const void *initial_states;
+  const int32_t *seq_lens;
+  void *dX;                   /* (B, L, H, P) x dtype */
+  float *ddt;                 /* (B, L, H) */
+  float *dA;                  /* (H, P) if a_per_p else (H,) */
+  float *dB, *dC;             /* fp32, shaped like Bproj / Cproj */
+  float *dD;                  /* (H, P) if d_per_p else (H,), or NULL */
+  float *dz;                  /* fp32, shaped like z; given exactly when z is */
+  float *dinitial_states;     /* (B, H, P) fp32 or NULL */
+  void *workspace;            /* ssm_dscan_bwd_workspace_bytes() bytes */
+  size_t workspace_bytes;
+  int32_t batch, seqlen, heads, proj;
+  int32_t x_dtype, dt_dtype, bc_dtype, z_dtype, init_dtype;
+  int32_t b_kind, c_kind;
+  int32_t a_per_p, d_per_p, z_per_p;
+} ssm_dscan_bwd_args;
+
+size_t ssm_dscan_bwd_workspace_bytes(int batch, int seqlen, int heads, int proj);
+int ssm_dscan_bwd(const ssm_dscan_bwd_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * state-space duality (Mamba-2) operator family.  The reference has no code
  * for these; their semantics are fixed by the vectors it ships in

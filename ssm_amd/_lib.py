@@ -102,6 +102,18 @@ class DscanFwdArgs(C.Structure):
     ]
 
 
+class DscanBwdArgs(C.Structure):
+    _fields_ = [
+        ("grad_y", _vp), ("X", _vp), ("dt", _vp), ("A", _vp), ("Bproj", _vp), ("Cproj", _vp), ("Dskip", _vp),
+        ("z", _vp), ("initial_states", _vp), ("seq_lens", _vp),
+        ("dX", _vp), ("ddt", _vp), ("dA", _vp), ("dB", _vp), ("dC", _vp), ("dD", _vp), ("dz", _vp),
+        ("dinitial_states", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
+        ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("proj", _i32),
+        ("x_dtype", _i32), ("dt_dtype", _i32), ("bc_dtype", _i32), ("z_dtype", _i32), ("init_dtype", _i32),
+        ("b_kind", _i32), ("c_kind", _i32), ("a_per_p", _i32), ("d_per_p", _i32), ("z_per_p", _i32),
+    ]
+
+
 class SsdDims(C.Structure):
     _fields_ = [("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("headdim", _i32), ("groups", _i32),
                 ("nstate", _i32), ("chunk", _i32)]
@@ -193,6 +205,7 @@ ENTRY_POINTS = {
     "ssm_state_step_bwd": StateStepBwdArgs,
     "ssm_decode_step": DecodeStepArgs,
     "ssm_dscan_fwd": DscanFwdArgs,
+    "ssm_dscan_bwd": DscanBwdArgs,
     "ssm_ssd_chunk_cumsum": SsdCumsumArgs,
     "ssm_ssd_bmm_chunk": SsdBmmArgs,
     "ssm_ssd_chunk_state": SsdChunkStateArgs,
@@ -213,6 +226,7 @@ PLAIN_SYMBOLS = {
     "ssm_scan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 8),
     "ssm_state_step_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 3),
     "ssm_dscan_fwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
+    "ssm_dscan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ssm_ssd_chunk_state_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
     "ssm_ssd_mfma_launches": (C.c_int, []),
     "ssm_ssd_combined_supported": (C.c_int, [C.POINTER(SsdDims), C.c_int]),

@@ -406,37 +406,12 @@ def decode_step(conv_state, ssm_state, x, dt, A, B, C, conv_weight, conv_bias=No
 # diagonal chunk scan (the reference's ``ssd_chunk_scan``)
 # ---------------------------------------------------------------------------
 
-def ssd_chunk_scan(X, dt, A, B, C, chunk_size, D=None, z=None, seq_meta=None, initial_states=None):
-    """Chunked diagonal state-space scan on the GPU (the reference's "SSD chunk scan").
-
-    ``s_t = exp(dt_t A) s_{t-1} + dt_t B_t X_t``, ``y_t = s_t C_t + D X_t`` per
-    ``(batch, head, p)`` channel, optionally gated by ``silu(z_t)``; ``dt`` is used
-    as given.  ``chunk_size`` is validated but does not affect the result.
-
-    Args:
-        X: Activations ``(B, L, H, P)``.
-        dt: Per-head time-steps ``(B, L, H)``.
-        A: ``(H, P)`` or ``(H,)``.
-        B: ``(H, P)``, ``(B, H, P)`` or time-varying ``(B, L, H, P)``.
-        C: Same accepted shapes as ``B``.
-        chunk_size: Positive integer.
-        D: Optional skip ``(H,)`` or ``(H, P)``.
-        z: Optional gate ``(B, L, H)`` or ``(B, L, H, P)``.
-        seq_meta: Optional dict with ``cu_seqlens`` (length ``B + 1``) or ``seq_lens``
-            (length ``B``); steps at or beyond a row's length produce zeros.
-        initial_states: Optional initial state ``(B, H, P)``.
-
-    Returns:
-        Tensor ``(B, L, H, P)`` in ``X.dtype``.
-    """
-    tensors = (X, dt, A, B, C, D, z, initial_states)
-    if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
-        raise NotImplementedError(
-            "ssd_chunk_scan has no backward kernel in this backend yet; run it under torch.no_grad().")
+def _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states):
+    """Validate, normalise dtypes/layout, and run ``ssm_dscan_fwd``; ``lengths`` is the
+    int32 device tensor of valid steps per batch row (or ``None``)."""
     batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p = \
         K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
     dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states)
-    lengths = K.sequence_lengths(seq_meta, batch, dev)
     bc = K.common_io_dtype([B, C])
     Xc, dtc = K.cast_c(X, X.dtype), K.cast_c(dt, dt.dtype)
     Bc, Cc = K.cast_c(B, bc), K.cast_c(C, bc)
@@ -457,6 +432,77 @@ def ssd_chunk_scan(X, dt, A, B, C, chunk_size, D=None, z=None, seq_meta=None, in
         b_kind=bk, c_kind=ck, a_per_p=int(a_per_p), d_per_p=int(d_per_p), z_per_p=int(z_per_p))
     _lib.call("ssm_dscan_fwd", args, dev)
     return Y
+
+
+def _dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_states):
+    """Run ``ssm_dscan_bwd``: gradients ``(dX, ddt, dA, dB, dC, dD, dz, dinitial_states)``.
+    ``dX`` comes back in ``X.dtype``, the rest in float32 with the shape of its tensor."""
+    batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p = \
+        K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
+    dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states, grad_y)
+    bc = K.common_io_dtype([B, C])
+    Xc, dtc = K.cast_c(X, X.dtype), K.cast_c(dt, dt.dtype)
+    gy = K.cast_c(grad_y, X.dtype)
+    Bc, Cc = K.cast_c(B, bc), K.cast_c(C, bc)
+    zc = K.cast_c(z, z.dtype) if z is not None else None
+    ic = K.cast_c(initial_states, initial_states.dtype) if initial_states is not None else None
+    Af, Df = K.as_f32_vec(A), K.as_f32_vec(D)
+    f32 = dict(dtype=torch.float32, device=dev)
+    dX = torch.empty_like(Xc)
+    ddt = torch.empty(batch, seqlen, heads, **f32)
+    dA = torch.empty(A.shape, **f32)
+    dB, dC = torch.empty(Bc.shape, **f32), torch.empty(Cc.shape, **f32)
+    dD = torch.empty(D.shape, **f32) if D is not None else None
+    dz = torch.empty(zc.shape, **f32) if zc is not None else None
+    dinit = torch.empty(batch, heads, proj, **f32) if ic is not None else None
+    nbytes = int(_lib.load().ssm_dscan_bwd_workspace_bytes(batch, seqlen, heads, proj))
+    ws = torch.empty(nbytes // 4, **f32)
+    args = _lib.DscanBwdArgs(
+        grad_y=_lib.ptr(gy), X=_lib.ptr(Xc), dt=_lib.ptr(dtc), A=_lib.ptr(Af), Bproj=_lib.ptr(Bc),
+        Cproj=_lib.ptr(Cc), Dskip=_lib.ptr(Df), z=_lib.ptr(zc), initial_states=_lib.ptr(ic),
+        seq_lens=_lib.ptr(lengths), dX=_lib.ptr(dX), ddt=_lib.ptr(ddt), dA=_lib.ptr(dA), dB=_lib.ptr(dB),
+        dC=_lib.ptr(dC), dD=_lib.ptr(dD), dz=_lib.ptr(dz), dinitial_states=_lib.ptr(dinit),
+        workspace=_lib.ptr(ws), workspace_bytes=nbytes, batch=batch, seqlen=seqlen, heads=heads, proj=proj,
+        x_dtype=_lib.dtype_enum(Xc.dtype), dt_dtype=_lib.dtype_enum(dtc.dtype), bc_dtype=_lib.dtype_enum(bc),
+        z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
+        init_dtype=_lib.dtype_enum(ic.dtype) if ic is not None else 0,
+        b_kind=bk, c_kind=ck, a_per_p=int(a_per_p), d_per_p=int(d_per_p), z_per_p=int(z_per_p))
+    _lib.call("ssm_dscan_bwd", args, dev)
+    return dX, ddt, dA, dB, dC, dD, dz, dinit
+
+
+def ssd_chunk_scan(X, dt, A, B, C, chunk_size, D=None, z=None, seq_meta=None, initial_states=None):
+    """Chunked diagonal state-space scan on the GPU (the reference's "SSD chunk scan").
+
+    ``s_t = exp(dt_t A) s_{t-1} + dt_t B_t X_t``, ``y_t = s_t C_t + D X_t`` per
+    ``(batch, head, p)`` channel, optionally gated by ``silu(z_t)``; ``dt`` is used
+    as given.  ``chunk_size`` is validated but does not affect the result.
+    Differentiable in every tensor argument.
+
+    Args:
+        X: Activations ``(B, L, H, P)``.
+        dt: Per-head time-steps ``(B, L, H)``.
+        A: ``(H, P)`` or ``(H,)``.
+        B: ``(H, P)``, ``(B, H, P)`` or time-varying ``(B, L, H, P)``.
+        C: Same accepted shapes as ``B``.
+        chunk_size: Positive integer.
+        D: Optional skip ``(H,)`` or ``(H, P)``.
+        z: Optional gate ``(B, L, H)`` or ``(B, L, H, P)``.
+        seq_meta: Optional dict with ``cu_seqlens`` (length ``B + 1``) or ``seq_lens``
+            (length ``B``); steps at or beyond a row's length produce zeros.
+        initial_states: Optional initial state ``(B, H, P)``.
+
+    Returns:
+        Tensor ``(B, L, H, P)`` in ``X.dtype``.
+    """
+    tensors = (X, dt, A, B, C, D, z, initial_states)
+    K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
+    dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states)
+    lengths = K.sequence_lengths(seq_meta, int(X.shape[0]), dev)
+    if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
+        from ._autograd import DiagScanFn
+        return DiagScanFn.apply(X, dt, A, B, C, int(chunk_size), D, z, lengths, initial_states)
+    return _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states)
 
 
 # ---------------------------------------------------------------------------

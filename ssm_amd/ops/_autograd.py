@@ -119,6 +119,32 @@ class SelectiveScanFn(torch.autograd.Function):
         return out + (None, None)
 
 
+class DiagScanFn(torch.autograd.Function):
+    """The diagonal chunk scan; the role of the reference's ``_SsdChunkScanCudaFunction``
+    (src/ssm/ops/__init__.py:780-905)."""
+
+    @staticmethod
+    def forward(ctx, X, dt, A, B, C, chunk_size, D, z, lengths, initial_states):
+        from . import _dscan_forward
+
+        Y = _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states)
+        ctx.save_for_backward(X, dt, A, B, C, D, z, lengths, initial_states)
+        ctx.chunk_size = chunk_size
+        return Y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        from . import _dscan_backward
+
+        X, dt, A, B, C, D, z, lengths, init = ctx.saved_tensors
+        dX, ddt, dA, dB, dC, dD, dz, dinit = _dscan_backward(grad_y, X, dt, A, B, C, ctx.chunk_size, D, z, lengths,
+                                                             init)
+        need = ctx.needs_input_grad
+        pick = lambda i, g, r: _like(g, r) if (r is not None and need[i]) else None
+        return (pick(0, dX, X), pick(1, ddt, dt), pick(2, dA, A), pick(3, dB, B), pick(4, dC, C), None,
+                pick(6, dD, D), pick(7, dz, z), None, pick(9, dinit, init))
+
+
 class StateStepFn(torch.autograd.Function):
     """One state update as a function ``(state, ...) -> (y, new_state)``; the role of the
     reference's ``_SelectiveStateStepCudaFunction`` (src/ssm/ops/__init__.py:570-668)."""
