@@ -62,10 +62,31 @@ __global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
   const int b = (int)(r / p.dim), d = (int)(r % p.dim);
   const int N = p.nstate;
 
+  size_t b_off, c_off;
+  if (p.b_kind == SSM_PROJ_BGNL) b_off = ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * N;
+  else b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+  if (p.c_kind == SSM_PROJ_BGNL) c_off = ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * N;
+  else c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+  state_t *srow = reinterpret_cast<state_t *>(p.state) + r * N;
+  const float *arow = p.A + (size_t)d * N;
+
+  // The first trip's operands are requested before anything else: they do not depend on the
+  // conv front end, and the compiler cannot move these reads above the window stores by itself.
+  const int n_first = sub * VEC;
+  const bool first_ok = n_first < N;
+  float h0[VEC], a0[VEC], bv0[VEC], cv0[VEC];
+  if (first_ok) {
+    load_vec<state_t, VEC>(srow + n_first, h0);
+    load_vec<float, VEC>(arow + n_first, a0);
+    load_vec_rt<VEC>(p.Bp, p.bc_dtype, b_off + n_first, bv0);
+    load_vec_rt<VEC>(p.Cp, p.bc_dtype, c_off + n_first, cv0);
+  }
+
   float dtv = load_as_f32(p.dt, p.io_dtype, r);
   if (p.bias) dtv += p.bias[d];
-  if (p.softplus) dtv = softplus_f32(dtv);
   float xv = load_as_f32(p.x, p.io_dtype, r);
+  const float zv = p.z ? load_as_f32(p.z, p.io_dtype, r) : 0.0f;
+  if (p.softplus) dtv = softplus_f32(dtv);
   if (p.conv_state) {
     // window <- (window[1:], x); x <- act(bias + sum_k w[k] window[k]).  The row's lanes
     // share the taps; every lane loads before any lane of the row stores.
@@ -91,21 +112,20 @@ __global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
   const float dx = dtv * xv;
   const float dt2 = dtv * LOG2E;
 
-  size_t b_off, c_off;
-  if (p.b_kind == SSM_PROJ_BGNL) b_off = ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * N;
-  else b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
-  if (p.c_kind == SSM_PROJ_BGNL) c_off = ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * N;
-  else c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
-
-  state_t *srow = reinterpret_cast<state_t *>(p.state) + r * N;
-  const float *arow = p.A + (size_t)d * N;
   float acc = 0.0f;
-  for (int n0 = sub * VEC; n0 < N; n0 += tpr * VEC) {
+  for (int n0 = n_first; n0 < N; n0 += tpr * VEC) {
     float h[VEC], a[VEC], bv[VEC], cv[VEC];
-    load_vec<state_t, VEC>(srow + n0, h);
-    load_vec<float, VEC>(arow + n0, a);
-    load_vec_rt<VEC>(p.Bp, p.bc_dtype, b_off + n0, bv);
-    load_vec_rt<VEC>(p.Cp, p.bc_dtype, c_off + n0, cv);
+    if (n0 == n_first) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        h[i] = h0[i]; a[i] = a0[i]; bv[i] = bv0[i]; cv[i] = cv0[i];
+      }
+    } else {
+      load_vec<state_t, VEC>(srow + n0, h);
+      load_vec<float, VEC>(arow + n0, a);
+      load_vec_rt<VEC>(p.Bp, p.bc_dtype, b_off + n0, bv);
+      load_vec_rt<VEC>(p.Cp, p.bc_dtype, c_off + n0, cv);
+    }
     Pack<state_t, VEC> outv;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -119,8 +139,93 @@ __global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
   if (live && sub == 0) {
     float y = acc;
     if (p.Dk) y = __builtin_fmaf(p.Dk[d], xv, y);
-    if (p.z) y *= silu_f32(load_as_f32(p.z, p.io_dtype, r));
+    if (p.z) y *= silu_f32(zv);
     store_from_f32(p.out, p.io_dtype, r, y);
+  }
+}
+
+// Variant for the common decode shapes (N = 4 * lanes-per-row, lanes-per-row in {4, 8, 16},
+// batch divisible by RB): a thread keeps what depends only on the channel (its four entries of
+// A, dt_bias, D, its conv tap) in registers and walks RB batch rows with them, which removes a
+// third of the cache traffic (A is as large as the state) and most of the small reads.  The three
+// per-row scalars x, dt, z are fetched by lanes 0, 1, 2 of the row with one instruction and
+// shared through the wave.
+template <typename state_t, int RB>
+__global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) {
+  constexpr int VEC = 4;
+  const int tpr = 1 << p.tpr_log2;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t col = gid >> p.tpr_log2;
+  const int sub = (int)(gid & (tpr - 1));
+  const size_t ncols = (size_t)p.dim * (p.batch / RB);
+  const bool live = col < ncols;
+  const size_t cc = live ? col : 0;
+  const int d = (int)(cc % p.dim), bg = (int)(cc / p.dim);
+  const int N = p.nstate, n0 = sub * VEC;
+  const int lane = lane_id(), base = lane & ~(tpr - 1);
+
+  float a[VEC];
+  load_vec<float, VEC>(p.A + (size_t)d * N + n0, a);
+  const float bias = p.bias ? p.bias[d] : 0.0f;
+  const float Dk = p.Dk ? p.Dk[d] : 0.0f;
+  const int K = p.conv_k;
+  const float tap = (p.conv_state && sub < K) ? p.conv_w[(size_t)d * K + sub] : 0.0f;
+  const float cbias = (p.conv_state && p.conv_b) ? p.conv_b[d] : 0.0f;
+  const void *scal_ptr = sub == 0 ? p.x : (sub == 1 ? p.dt : p.z);
+  const bool scal_on = sub < 2 || (sub == 2 && p.z);
+
+  float h[RB][VEC], bv[RB][VEC], cv[RB][VEC], scal[RB], win[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int b = bg * RB + rb;
+    const size_t r = (size_t)b * p.dim + d;
+    size_t b_off, c_off;
+    if (p.b_kind == SSM_PROJ_BGNL) b_off = ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * N;
+    else b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+    if (p.c_kind == SSM_PROJ_BGNL) c_off = ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * N;
+    else c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+    load_vec<state_t, VEC>(reinterpret_cast<const state_t *>(p.state) + r * N + n0, h[rb]);
+    load_vec_rt<VEC>(p.Bp, p.bc_dtype, b_off + n0, bv[rb]);
+    load_vec_rt<VEC>(p.Cp, p.bc_dtype, c_off + n0, cv[rb]);
+    scal[rb] = scal_on ? load_as_f32(scal_ptr, p.io_dtype, r) : 0.0f;
+    win[rb] = (p.conv_state && sub + 1 < K) ? load_as_f32(p.conv_state, p.io_dtype, r * K + sub + 1) : 0.0f;
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int b = bg * RB + rb;
+    const size_t r = (size_t)b * p.dim + d;
+    float xv = __shfl(scal[rb], base, WAVE);
+    float dtv = __shfl(scal[rb], base + 1, WAVE) + bias;
+    const float zv = __shfl(scal[rb], base + 2, WAVE);
+    if (p.softplus) dtv = softplus_f32(dtv);
+    if (p.conv_state) {
+      // window <- (window[1:], x); x <- act(bias + sum_k w[k] window[k]); lane k of the row owns tap k
+      const float v = sub + 1 < K ? win[rb] : xv;
+      float part = sub < K ? v * tap : 0.0f;
+      if (live && sub < K) store_from_f32(p.conv_state, p.io_dtype, r * K + sub, v);
+      for (int m = tpr >> 1; m >= 1; m >>= 1) part += __shfl_xor(part, m, WAVE);
+      part += cbias;
+      xv = p.conv_silu ? silu_f32(part) : part;
+      if (p.io_dtype == SSM_BF16) xv = to_f32(from_f32<bf16_t>(xv));
+      else if (p.io_dtype == SSM_F16) xv = to_f32(from_f32<f16_t>(xv));
+      if (p.conv_out && live && sub == 0) store_from_f32(p.conv_out, p.io_dtype, r, xv);
+    }
+    const float dx = dtv * xv, dt2 = dtv * LOG2E;
+    float acc = 0.0f;
+    Pack<state_t, VEC> outv;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float hn = __builtin_fmaf(exp2_hw(dt2 * a[i]), h[rb][i], dx * bv[rb][i]);
+      acc = __builtin_fmaf(hn, cv[rb][i], acc);
+      outv.v[i] = from_f32<state_t>(hn);
+    }
+    if (live) *reinterpret_cast<Pack<state_t, VEC> *>(reinterpret_cast<state_t *>(p.state) + r * N + n0) = outv;
+    for (int m = tpr >> 1; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, WAVE);
+    if (live && sub == 0) {
+      float y = __builtin_fmaf(Dk, xv, acc);
+      if (p.z) y *= silu_f32(zv);
+      store_from_f32(p.out, p.io_dtype, r, y);
+    }
   }
 }
 
@@ -132,6 +237,14 @@ static int launch_step(const StepParams &p0, bool vec4, hipStream_t stream) {
   int lg = 0;
   while ((1 << lg) < per_row && lg < 4) ++lg;    // at most 16 lanes per row
   p.tpr_log2 = lg;
+  constexpr int RB = 4;
+  if (vec4 && p.nstate == (4 << lg) && lg >= 2 && p.batch % RB == 0 && (!p.conv_state || p.conv_k <= (1 << lg))) {
+    const size_t threads_rb = ((size_t)p.dim * (p.batch / RB)) << lg;
+    hipLaunchKernelGGL((state_step_rb_kernel<state_t, RB>), dim3((unsigned)((threads_rb + 255) / 256)), dim3(256), 0,
+                       stream, p);
+    SSM_CHECK_LAUNCH("ssm_state_step");
+    return SSM_OK;
+  }
   const size_t threads = ((size_t)p.batch * p.dim) << lg;
   const unsigned grid = (unsigned)((threads + 255) / 256);
   if (vec4) hipLaunchKernelGGL((state_step_kernel<state_t, 4>), dim3(grid), dim3(256), 0, stream, p);
