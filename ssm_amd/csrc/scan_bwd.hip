@@ -167,18 +167,38 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
 #pragma unroll
       for (int i = 0; i < K; ++i) accB[w][i] = accC[w][i] = 0.0f;
 
+    // The four inputs of element (row, t0 + tid) are requested one row ahead: the reads of
+    // row r + 1 are in flight while the wave works on the states of row r.
+    const int te = t0 + tid;
+    const int te_c = min(te, L - 1);
+    io_t nx_u, nx_dl, nx_go, nx_z;
+    {
+      const size_t idx = ((size_t)b * p.dim + d_first) * L + te_c;
+      nx_u = reinterpret_cast<const io_t *>(p.u)[idx];
+      nx_dl = reinterpret_cast<const io_t *>(p.delta)[idx];
+      nx_go = reinterpret_cast<const io_t *>(p.dout)[idx];
+      nx_z = p.z ? reinterpret_cast<const io_t *>(p.z)[idx] : nx_u;
+    }
+
     for (int r = 0; r < p.rows_per_wg; ++r) {
       const int d = d_first + r;
       const size_t row = (size_t)b * p.dim + d;
       const float Dk = p.Dk ? p.Dk[d] : 0.0f;
 
       // ---- element-wise stage: thread tid owns step t0 + tid of this row
-      const int te = t0 + tid;
       float el_u = 0.0f, el_dl = 0.0f, el_g = 0.0f, el_sig = 1.0f, el_dz = 0.0f;
+      const io_t cur_u = nx_u, cur_dl = nx_dl, cur_go = nx_go, cur_z = nx_z;
+      {
+        const int rn = min(r + 1, p.rows_per_wg - 1);
+        const size_t idx = ((size_t)b * p.dim + d_first + rn) * L + te_c;
+        nx_u = reinterpret_cast<const io_t *>(p.u)[idx];
+        nx_dl = reinterpret_cast<const io_t *>(p.delta)[idx];
+        nx_go = reinterpret_cast<const io_t *>(p.dout)[idx];
+        nx_z = p.z ? reinterpret_cast<const io_t *>(p.z)[idx] : nx_u;
+      }
       if (te < L) {
-        const size_t idx = row * L + te;
-        el_u = to_f32(reinterpret_cast<const io_t *>(p.u)[idx]);
-        float draw = to_f32(reinterpret_cast<const io_t *>(p.delta)[idx]);
+        el_u = to_f32(cur_u);
+        float draw = to_f32(cur_dl);
         if (p.bias) draw += p.bias[d];
         if (p.softplus) {
           el_dl = softplus_f32(draw);
@@ -186,9 +206,9 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
         } else {
           el_dl = draw;
         }
-        const float go = to_f32(reinterpret_cast<const io_t *>(p.dout)[idx]);
+        const float go = to_f32(cur_go);
         if (p.z) {
-          const float zv = to_f32(reinterpret_cast<const io_t *>(p.z)[idx]);
+          const float zv = to_f32(cur_z);
           const float sg = sigmoid_f32(zv);
           el_g = go * zv * sg;
           el_dz = go * sg * __builtin_fmaf(zv, 1.0f - sg, 1.0f);      // dout * silu'(z)
