@@ -1,6 +1,6 @@
-// Mamba-2 SSD forward as one pass over the sequence: a workgroup owns one
-// (batch, head), walks its chunks in order and keeps the running state
-// S (P x N, fp32) in MFMA accumulators, so neither the per-chunk states nor
+// Mamba-2 SSD forward as one pass over the sequence: a workgroup owns 32 channels
+// (half a head) of one (batch, head), walks its chunks in order and keeps the running
+// state S (32 x N, fp32) in MFMA accumulators, so neither the per-chunk states nor
 // the state entering each chunk ever travel through HBM.
 //
 // Per chunk (Q steps, 32-step blocks lb = 0 .. Q/32-1, e_k = last step of block k,
@@ -28,20 +28,20 @@
 
 namespace ssm {
 
-constexpr int FU_THREADS = 512;
 constexpr int FU_P = 64;
-constexpr int FU_TILE_BYTES = 32768;                       // [64][256] bf16
-constexpr int FU_LDS_BYTES = 2 * FU_TILE_BYTES + 3 * 256 * 4;
 constexpr int FRAG = 512;                                  // bf16 elements per operand fragment
 
 struct SsdFusedParams {
   const __bf16 *x, *z;
   __bf16 *y;
-  const float *dA2, *dtv, *ws;          // (B,H,nc,Q): log2-scaled running sum, step, staged weight
+  const float *dA2, *dtv;               // (B,H,nc,Q): log2-scaled running sum, step
   const __bf16 *Cblk, *Btblk, *CBblk;   // fragment-blocked copies
   const float *Dk, *init;
   float *final_states;
   int batch, len, heads, groups, nstate, chunk, nchunks, d_per_p;
+#ifdef FH_TIMING
+  long long *times;
+#endif
 };
 
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
@@ -51,10 +51,10 @@ __device__ __forceinline__ void wave_lds_sync() { asm volatile("s_waitcnt lgkmcn
 // ------------------------------------------------------------------ prep: dt
 // One workgroup per (b, c, 4 heads): the (Q x 4) slab of dt is read row by row
 // (16 contiguous bytes per step) into LDS transposed to [head][step]; then one
-// wave per head forms dt' = clamp(softplus(dt + bias)), the running sum of dt' A
-// and the staged weight  ws[l] = dt'_l exp(cs[l | 31] - cs[l]).
+// wave per head forms dt' = clamp(softplus(dt + bias)) and the running sum of dt' A
+// (stored scaled by log2 e, the unit of the fused kernel's exponentials).
 constexpr int PD_HEADS = 4;
-__global__ __launch_bounds__(256) void ssd_fused_prep_dt_kernel(const SsdCumsumParams p, float *dA2, float *ws) {
+__global__ __launch_bounds__(256) void ssd_fused_prep_dt_kernel(const SsdCumsumParams p, float *dA2) {
   __shared__ float tile[PD_HEADS][256 + 1];
   const SsdDims &d = p.d;
   const int Q = d.chunk;
@@ -99,23 +99,13 @@ __global__ __launch_bounds__(256) void ssd_fused_prep_dt_kernel(const SsdCumsumP
     }
     const float excl = incl - tot;
     const size_t out = (((size_t)b * d.heads + h) * d.nchunks + c) * (size_t)Q;
-    wave_lds_sync();                       // the row is re-used for the running sums
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int l = lane * per + i;
       if (i < per && l < Q) {
-        const float a = excl + run[i];
-        tile[hh][l] = a;
-        p.dA_cs[out + l] = a;
         p.dt_out[out + l] = v[i];
-        dA2[out + l] = a * LOG2E;
+        dA2[out + l] = (excl + run[i]) * LOG2E;
       }
-    }
-    wave_lds_sync();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int l = lane * per + i;
-      if (i < per && l < Q) ws[out + l] = v[i] * decay_exp(tile[hh][l | 31] - tile[hh][l]);
     }
   }
 }
@@ -158,140 +148,280 @@ __global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *Cm, c
   *reinterpret_cast<bf16x8_t *>((is_c ? Cblk : Btblk) + f * FRAG + lane * 8) = v;
 }
 
-// --------------------------------------------------------------- fused kernel
-// Waves 0..7.  For the output phases wave w owns the 32 rows of block
-// lb = w (w < 4) or 11 - w, both 32-wide halves of P, so that the two waves
-// sharing a SIMD carry equal numbers of blocks below the diagonal.  For the state
-// phases wave w owns the 32 x 32 tile (n-tile w / 2, p-tile w % 2) of S^T.
-// Accumulators hold transposed tiles: lane = column (l for y, p for S^T),
-// registers = rows (p for y, n for S^T).
-// DMODE: 0 no skip term, 1 D per head, 2 D per (head, channel).
+// ------------------------------------------------- fused kernel, half a head
+// One workgroup of 4 waves walks the chunks of 32 channels (half a head): blockIdx ->
+// (b, h, half).  Per chunk:
+//   barrier; the carried state S goes to LDS as bf16 and the chunk's x, already in
+//     registers, is staged twice, plain and weighted, transposed to [p][s];
+//   barrier; Y = C S (carried state), then the blocks of (CB o decay) X below and on the
+//     diagonal for this wave's two row blocks;
+//   barrier; requests for z, and for the next chunk's x, dt and running sums, go out (the
+//     only reads that come from HBM: they are grouped so that the wave meets their
+//     latency once); S <- S g + B^T X~; skip term, gate and the store of Y.
+// Wave w owns the row blocks NLB - 1 - w and w (every wave the same number of blocks
+// below the diagonal) and the n-tile w of S^T.  Its fragments of C, CB and B^T form one
+// stream (C for both row blocks, CB of the first row block, CB of the second, B^T) that
+// runs through a ring of four registers; a register is refilled right after its use with
+// the fragment four places on, across the phases and into the next chunk.
+// All global accesses are buffer accesses: the lane's part of the address is a 32-bit
+// offset that does not change, the rest is scalar.
+constexpr int FH_THREADS = 256;
+constexpr int FH_TILE_BYTES = 16384;                       // [32][256] bf16
+constexpr int FH_LDS_BYTES = 3 * FH_TILE_BYTES + 3 * 256 * 4;
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2_t;
+
+// 2 GiB window from p on; accesses carry byte offsets below that.
+__device__ __forceinline__ rsrc_t make_rsrc(const void *p) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ bf16x8_t buf_load16(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ bf16x4_t buf_load8(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(bf16x4_t, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+}
+__device__ __forceinline__ float4 buf_load_f4(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ float buf_load_f1(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+
+// Where the part of a wave's fragment stream after the fragments of C lies: byte offsets from Cblk.
+struct HalfStream {
+  rsrc_t r;
+  int vf;                    // lane * 16
+  int n_first, n_both;       // fragments of CB of the first row block, of both
+  int off_first, off_second, off_bt, bt_step;
+};
+// Places i (even) and i + 1 of the stream; both lie in the same part of it.
+__device__ __forceinline__ void stream_pair(const HalfStream &st, int i, bf16x8_t &fa, bf16x8_t &fb) {
+  const int o1 = st.off_first + (i << 10);
+  const int o2 = st.off_second + ((i - st.n_first) << 10);
+  const int o3 = st.off_bt + (i - st.n_both) * st.bt_step;
+  const bool in1 = i < st.n_first, in2 = i < st.n_both;
+  const int o12 = in1 ? o1 : o2;
+  const int off = in2 ? o12 : o3;
+  const int step = in2 ? 1024 : st.bt_step;
+  fa = buf_load16(st.r, st.vf, off);
+  fb = buf_load16(st.r, st.vf, off + step);
+}
+
+// Blocks below the diagonal and the diagonal block of row block `lb` into `acc` (one 32 x 32
+// tile: lane = column l, registers = rows p).  Block sb takes its two fragments from (a0, a1)
+// if sb is even, from (b0, b1) if odd; they are the stream's places pos0 + 2 sb, + 1.
+// With SKIP, the per-head skip factor dskip joins the diagonal of the last operand (CB dt + D at
+// s = l, rounded to bf16 as one number), so that the product with the plain x adds D x.
+template <bool SKIP>
+__device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16x8_t &a1, bf16x8_t &b0, bf16x8_t &b1,
+                                               int lb, int pos0, const HalfStream &st, const __bf16 *xw, const __bf16 *xr,
+                                               const float *dAs, const float *dts, int Q, int qmask, int m, int g2,
+                                               float dskip) {
+  float prev_end = 0.0f;
+  const int lrow = 32 * lb + m;
+  const float dal = dAs[lrow];
+#define FH_BLOCK(FA, FB, SB)                                                                    \
+  {                                                                                             \
+    const float endv = dAs[32 * (SB) + 31];                                                     \
+    const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));                                     \
+    prev_end = endv;                                                                            \
+    _Pragma("unroll") for (int r = 0; r < 16; ++r) acc[r] *= gs;                                \
+    const bf16x8_t x0 = load_frag(xw + m * Q + (((4 * (SB) + g2) ^ (m & qmask)) << 3));         \
+    const bf16x8_t x1 = load_frag(xw + m * Q + (((4 * (SB) + 2 + g2) ^ (m & qmask)) << 3));     \
+    acc = mma(x0, FA, acc);                                                                     \
+    acc = mma(x1, FB, acc);                                                                     \
+    stream_pair(st, pos0 + 2 * (SB) + 4, FA, FB);                                               \
+  }
+  bf16x8_t d0, d1;
+  if (lb & 1) {
+    for (int sb0 = 0; sb0 < lb - 1; sb0 += 2) {
+      FH_BLOCK(a0, a1, sb0)
+      FH_BLOCK(b0, b1, sb0 + 1)
+    }
+    FH_BLOCK(a0, a1, lb - 1)
+    d0 = b0;
+    d1 = b1;
+    stream_pair(st, pos0 + 2 * lb + 4, b0, b1);
+  } else {
+    for (int sb0 = 0; sb0 < lb; sb0 += 2) {
+      FH_BLOCK(a0, a1, sb0)
+      FH_BLOCK(b0, b1, sb0 + 1)
+    }
+    d0 = a0;
+    d1 = a1;
+    stream_pair(st, pos0 + 2 * lb + 4, a0, a1);
+  }
+#undef FH_BLOCK
+  const float rf = exp2_hw(fminf(dal - prev_end, 0.0f));
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] *= rf;
+  // the diagonal block: its fragments of CB hold zeros above the diagonal, so that the decay
+  // only needs a bound there
+  int jdiag = m - 8 * g2;                  // the lane's diagonal element is number jdiag - 16 kk of fragment kk, if in 0..7
+  asm volatile("" : "+v"(jdiag));          // (rebuilt here for each row block rather than kept in registers)
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    const bf16x8_t f = kk == 0 ? d0 : d1;
+    const int sbase = 32 * lb + 16 * kk + 8 * g2;
+    const float4 q0 = *reinterpret_cast<const float4 *>(dAs + sbase), q1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
+    const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
+    const float das[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+    float mv[8];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+      mv[jj] = (float)f[jj] * dtv[jj] * exp2_hw(fminf(dal - das[jj], 0.0f));
+      if (SKIP) mv[jj] += (16 * kk + jj == jdiag) ? dskip : 0.0f;
+    }
+    const bf16x8_t a = load_frag(xr + m * Q + (((4 * lb + 2 * kk + g2) ^ (m & qmask)) << 3));
+    acc = mma(a, pack8(mv), acc);
+  }
+}
+
+// acc[p][l] += D[p] x[l][p] for row block lb, x read from the plain tile (per-channel skip factors).
+__device__ __forceinline__ void half_skip_term(f32x16_t &acc, int lb, const __bf16 *xr, int Q, int qmask, int m, int g2,
+                                               const float *Dp) {
+  const int lrow = 32 * lb + m;
+  const int xcol = lrow & 7, xchunk = lrow >> 3;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float4 d4 = *reinterpret_cast<const float4 *>(Dp + 8 * q + 4 * g2);
+    const float dv[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int prow = 8 * q + 4 * g2 + j;
+      const float xv = (float)xr[prow * Q + ((xchunk ^ (prow & qmask)) << 3) + xcol];
+      acc[4 * q + j] = __builtin_fmaf(dv[j], xv, acc[4 * q + j]);
+    }
+  }
+}
+
 template <int DMODE, bool HAS_Z>
-__global__ __launch_bounds__(FU_THREADS)
-void ssd_fused_kernel(const SsdFusedParams p) {
+__global__ __launch_bounds__(FH_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3)))
+void ssd_fused_half_kernel(const SsdFusedParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  __bf16 *xw = reinterpret_cast<__bf16 *>(smem);                       // x~ [64][Q]; between chunks S as bf16 [64][N]
-  __bf16 *xr = reinterpret_cast<__bf16 *>(smem + FU_TILE_BYTES);       // x  [64][Q]; later the output staging
-  float *dAs = reinterpret_cast<float *>(smem + 2 * FU_TILE_BYTES);    // [Q] log2-scaled running sum
-  float *dts = dAs + 256;                                              // [Q]
-  float *wss = dts + 256;                                              // [Q] staged weight
+  __bf16 *xw = reinterpret_cast<__bf16 *>(smem);                        // x~ [32][Q]
+  __bf16 *xr = reinterpret_cast<__bf16 *>(smem + FH_TILE_BYTES);        // x  [32][Q]
+  __bf16 *sbf = reinterpret_cast<__bf16 *>(smem + 2 * FH_TILE_BYTES);   // S as bf16 [32][N]; later the output staging
+  float *dAs = reinterpret_cast<float *>(smem + 3 * FH_TILE_BYTES);     // [Q] log2-scaled running sum
+  float *dts = dAs + 256;                                               // [Q] dt
+  float *wss = dts + 256;                                               // [Q] staging weight dt exp(cs[l | 31] - cs[l])
 
   const int Q = p.chunk, N = p.nstate, H = p.heads, G = p.groups, nc = p.nchunks;
   const int NLB = Q >> 5, NT = N >> 5, KS = Q >> 4, KN = N >> 4;
   const int qmask = min(15, (Q >> 3) - 1), nmask = min(15, (N >> 3) - 1);
-  const int tid = (int)threadIdx.x;
   const int wave = wave_id_uniform(), lane = lane_id();
   const int g2 = lane >> 5, m = lane & 31;
-  const int h = (int)blockIdx.x % H, b = (int)blockIdx.x / H;
+  // Workgroups go to the 8 XCDs round-robin by blockIdx: renumber them so that each XCD (own L2)
+  // works on neighbouring heads of one batch row, which stream the same fragments of C, B and CB.
+  int vid = (int)blockIdx.x;
+  if ((gridDim.x & 7) == 0) vid = (vid & 7) * (int)(gridDim.x >> 3) + (vid >> 3);
+  const int half = vid & 1;
+  const int h = (vid >> 1) % H, b = (vid >> 1) / H;
   const int g = h / (H / G);
-  const int lb = wave < 4 ? wave : 11 - wave;
-  const bool yact = lb < NLB;
-  const int pt_s = wave & 1, nt_s = wave >> 1;
+  const int p0 = 32 * half;
+  const bool yact = wave < (NLB >> 1);
+  const int lbF = NLB - 1 - wave, lbS = wave;          // first: many blocks below the diagonal, second: few
+  const int nt_s = wave;
   const bool sact = nt_s < NT;
   const bool has_init = p.init != nullptr;
-  const size_t xrow = (size_t)H * FU_P;                                // elements between time steps
+  const int xrow_b = H * FU_P * 2;                     // bytes between rows of x, z and y
+  const float dhead = DMODE == 1 ? p.Dk[h] : 0.0f;
+  const int tid = wave * WAVE + lane;
+
+  // ---- buffers and the lanes' constant offsets
+  const size_t xbase = ((size_t)b * p.len * H + h) * FU_P + p0;
+  const rsrc_t rx = make_rsrc(p.x + xbase), ry = make_rsrc(p.y + xbase);
+  const rsrc_t rz = make_rsrc(HAS_Z ? p.z + xbase : p.x + xbase);
+  const size_t tbase = ((size_t)b * H + h) * nc * Q;   // dA2 and dtv are laid out alike
+  const rsrc_t rt = make_rsrc(p.dtv + tbase);
+  const int t_dA = (int)((const char *)p.dA2 - (const char *)p.dtv);
+  const rsrc_t rf = make_rsrc(p.Cblk);
+  const int f_cb = (int)((const char *)p.CBblk - (const char *)p.Cblk), f_bt = (int)((const char *)p.Btblk - (const char *)p.Cblk);
+  const int srow = min(tid >> 3, (Q >> 3) - 1) * 8, spb = tid & 7, slb8 = tid >> 3;
+  const int v_raw = srow * xrow_b + spb * 8;                       // x for staging: rows srow.., 4 channels
+  const int v_row = (lane >> 2) * xrow_b + (lane & 3) * 16;        // row-major passes: row lane / 4, 8 channels
+  const int v_t = min(tid, Q - 1) * 4;
+  HalfStream st;
+  st.r = rf;
+  st.vf = lane * 16;
+  st.bt_step = NT << 10;
+  // waves without row blocks start two places on, so that the state update finds the ring alike
+  st.n_first = yact ? 2 * lbF + 2 : 0;
+  st.n_both = yact ? 2 * NLB + 2 : 2;
 
   f32x16_t S = {0};
   if (sact && has_init) {
-    const float *ip = p.init + (((size_t)b * H + h) * FU_P + 32 * pt_s + m) * N + 32 * nt_s;
+    const float *ip = p.init + (((size_t)b * H + h) * FU_P + p0 + m) * N + 32 * nt_s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) S[r] = ip[crow(r, g2)];
   }
-  f32x16_t acc[2];
-
-  // staging role: a thread transposes 8 time steps x 4 head channels into both tiles
+  f32x16_t accF, accS;
+  bf16x8_t f0, f1, f2, f3;
+  // what a chunk reads from HBM, requested one chunk ahead: x, dt and the running sums
+  bf16x4_t raw[8];
+  float dA_t, dt_t;
+#define FH_REQUEST_CHUNK(CC)                                                                              \
+  {                                                                                                       \
+    const int xo_ = (CC) * Q * xrow_b, to_ = (CC) * Q * 4;                                                \
+    _Pragma("unroll") for (int r = 0; r < 8; ++r) raw[r] = buf_load8(rx, v_raw, xo_ + r * xrow_b);        \
+    dA_t = buf_load_f1(rt, v_t, t_dA + to_);                                                              \
+    dt_t = buf_load_f1(rt, v_t, to_);                                                                     \
+  }
+  // fragments of C of chunk CC: (f0, f1) = (first, second row block) at kn = 0, (f2, f3) at kn = 1
+#define FH_C_OFF(CC, LB, KNI) ((((((b * nc + (CC)) * G + g) * NLB + (LB)) * KN + (KNI))) << 10)
+  FH_REQUEST_CHUNK(0)
+  if (yact && has_init) {
+    f0 = buf_load16(rf, st.vf, FH_C_OFF(0, lbF, 0));
+    f1 = buf_load16(rf, st.vf, FH_C_OFF(0, lbS, 0));
+    f2 = buf_load16(rf, st.vf, FH_C_OFF(0, lbF, 1));
+    f3 = buf_load16(rf, st.vf, FH_C_OFF(0, lbS, 1));
+  }
+#ifdef FH_TIMING
+  long long tacc[10] = {0}; long long tprev = __builtin_amdgcn_s_memtime();
+#define FH_T(i) { const long long tn = __builtin_amdgcn_s_memtime(); tacc[i] += tn - tprev; tprev = tn; }
+#else
+#define FH_T(i)
+#endif
 
   for (int c = 0; c < nc; ++c) {
-    // Lane-derived addresses are recomputed per chunk (the opaque copy keeps them from
-    // being hoisted out of the loop and held in registers across all of it).
+    // LDS addresses are rebuilt from the lane number in every chunk: kept across chunks they would
+    // occupy more registers than they cost to recompute
     int ln = lane;
     asm volatile("" : "+v"(ln));
     const int lane = ln, g2 = ln >> 5, m = ln & 31, tid = wave * WAVE + ln;
-    const bool s_on = tid < 2 * Q;
-    const int spb = tid & 15, slb8 = tid >> 4;
-    const size_t cs = (((size_t)b * H + h) * nc + c) * Q;
-    const size_t unit = ((size_t)b * nc + c) * G + g;
-    const __bf16 *xg = p.x + (((size_t)b * p.len + (size_t)c * Q) * H + h) * FU_P;
+    const int spb = tid & 7, slb8 = tid >> 3;
+    const int unit = (b * nc + c) * G + g;
     const bool carry = c > 0 || has_init;
-    // Operand fragments stream through four registers sets: f0 is consumed, f1..f3 are in
-    // flight, a new read (clamped to the last fragment) enters at f3.
-    bf16x8_t f0, f1, f2, f3;
+    st.off_first = f_cb + (((unit * NLB + lbF) * KS) << 10);
+    st.off_second = yact ? f_cb + (((unit * NLB + lbS) * KS) << 10) : f_bt + (((unit * KS) * NT + min(nt_s, NT - 1)) << 10);
+    st.off_bt = f_bt + (((unit * KS) * NT + min(nt_s, NT - 1)) << 10);
 
-    // fragments of C for the carried-state product: in flight across the barriers below
-    const __bf16 *cf = p.Cblk + ((unit * NLB + lb) * KN) * FRAG + lane * 8;
-    if (yact && carry) {
-      f0 = load_frag(cf);
-      f1 = load_frag(cf + (size_t)min(1, KN - 1) * FRAG);
-      f2 = load_frag(cf + (size_t)min(2, KN - 1) * FRAG);
-      f3 = load_frag(cf + (size_t)min(3, KN - 1) * FRAG);
-    }
-
-    __syncthreads();                       // previous chunk: output staging and x~ reads are over
+    __syncthreads();                       // previous chunk: every read of the tiles and the output staging are over
+    FH_T(0)
     if (sact && carry) {
-      const int prow = 32 * pt_s + m;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         bf16x4_t v;
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = (__bf16)S[4 * q + j];
         const int chunk16 = 4 * nt_s + q;
-        *reinterpret_cast<bf16x4_t *>(xw + prow * N + ((chunk16 ^ (prow & nmask)) << 3) + 4 * g2) = v;
+        *reinterpret_cast<bf16x4_t *>(sbf + m * N + ((chunk16 ^ (m & nmask)) << 3) + 4 * g2) = v;
       }
     }
-    if (tid < Q) {
-      dAs[tid] = p.dA2[cs + tid];
-      dts[tid] = p.dtv[cs + tid];
-      wss[tid] = p.ws[cs + tid];
-    }
-    // global reads for the staging that follows the carried-state product
-    bf16x4_t raw[8];                       // read by every thread (clamped rows) so that the values
-    {                                      // are not defined under a divergent branch
-      const int srow = min(slb8, (Q >> 3) - 1) * 8;
-#pragma unroll
-      for (int r = 0; r < 8; ++r)
-        raw[r] = *reinterpret_cast<const bf16x4_t *>(xg + (size_t)(srow + r) * xrow + spb * 4);
-    }
-    __syncthreads();
-
-    // ---- carried state: acc[p][l] = sum_n S[p][n] C[l][n]
-    acc[0] = (f32x16_t){0};
-    acc[1] = (f32x16_t){0};
-    if (yact && carry) {
-      // four steps per trip, one register set each: a set is refilled as soon as it is consumed
-      // (no copies between sets: a copy would wait for the read it moves)
-#define FU_STEP_A(F, KK)                                                                        \
-      {                                                                                         \
-        const bf16x8_t f = F;                                                                   \
-        F = load_frag(cf + (size_t)min((KK) + 4, KN - 1) * FRAG);                               \
-        _Pragma("unroll") for (int pt = 0; pt < 2; ++pt) {                                      \
-          const int prow = 32 * pt + m;                                                         \
-          const bf16x8_t a = load_frag(xw + prow * N + (((2 * (KK) + g2) ^ (prow & nmask)) << 3)); \
-          acc[pt] = mma(a, f, acc[pt]);                                                         \
-        }                                                                                       \
-      }
-      for (int k0 = 0; k0 < KN; k0 += 4) {
-        FU_STEP_A(f0, k0)
-        FU_STEP_A(f1, k0 + 1)
-        FU_STEP_A(f2, k0 + 2)
-        FU_STEP_A(f3, k0 + 3)
-      }
-#undef FU_STEP_A
-    }
-    // fragments of CB for this wave's rows: in flight while the tiles are staged
-    const __bf16 *cbf = p.CBblk + ((unit * NLB + lb) * KS) * FRAG + lane * 8;
-    const int nkb = 2 * lb + 2;            // 16-step fragments up to and including the diagonal block
-    if (yact) {
-      f0 = load_frag(cbf);
-      f1 = load_frag(cbf + (size_t)FRAG);
-      f2 = load_frag(cbf + (size_t)min(2, nkb - 1) * FRAG);
-      f3 = load_frag(cbf + (size_t)min(3, nkb - 1) * FRAG);
-    }
-    __syncthreads();                       // S (bf16) consumed: the x~ tile may be written
-
-    // ---- stage x~ and x, transposed to [p][s]
-    if (s_on) {
-      const float4 a0 = *reinterpret_cast<const float4 *>(wss + slb8 * 8), a1 = *reinterpret_cast<const float4 *>(wss + slb8 * 8 + 4);
-      const float w8[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    if (tid < Q) {                         // whole waves: Q is a multiple of 64
+      // weight of a step towards the end of its block of 32: the running sum there is in lane | 31
+      const float w_t = dt_t * exp2_hw(fminf(__shfl(dA_t, lane | 31, WAVE) - dA_t, 0.0f));
+      dAs[tid] = dA_t;
+      dts[tid] = dt_t;
+      wss[tid] = w_t;
+      wave_lds_sync();                     // the eight weights this thread needs come from its own wave
+      const float4 wa = *reinterpret_cast<const float4 *>(wss + slb8 * 8), wb = *reinterpret_cast<const float4 *>(wss + slb8 * 8 + 4);
+      const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+      // ---- stage x~ and x, transposed to [p][s]
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         bf16x8_t colw, colr;
@@ -306,162 +436,133 @@ void ssd_fused_kernel(const SsdFusedParams p) {
         *reinterpret_cast<bf16x8_t *>(xr + at) = colr;
       }
     }
+    FH_T(1)
     __syncthreads();
-    // ---- blocks below the diagonal, then the diagonal block
+    FH_T(2)
+
+    // ---- carried state: acc[p][l] = sum_n S[p][n] C[l][n] for both row blocks
+    accF = (f32x16_t){0};
+    accS = (f32x16_t){0};
+    if (yact && carry) {
+      const int cF = FH_C_OFF(c, lbF, 0), cS = FH_C_OFF(c, lbS, 0);
+#define FH_STEP_A(FF, FS, KK)                                                                     \
+      {                                                                                           \
+        const bf16x8_t a = load_frag(sbf + m * N + (((2 * (KK) + g2) ^ (m & nmask)) << 3));       \
+        accF = mma(a, FF, accF);                                                                  \
+        accS = mma(a, FS, accS);                                                                  \
+      }
+      for (int kn0 = 0; kn0 < KN - 2; kn0 += 2) {
+        FH_STEP_A(f0, f1, kn0)
+        f0 = buf_load16(rf, st.vf, cF + ((kn0 + 2) << 10));
+        f1 = buf_load16(rf, st.vf, cS + ((kn0 + 2) << 10));
+        FH_STEP_A(f2, f3, kn0 + 1)
+        f2 = buf_load16(rf, st.vf, cF + ((kn0 + 3) << 10));
+        f3 = buf_load16(rf, st.vf, cS + ((kn0 + 3) << 10));
+      }
+      FH_STEP_A(f0, f1, KN - 2)
+      stream_pair(st, 0, f0, f1);
+      FH_STEP_A(f2, f3, KN - 1)
+      stream_pair(st, 2, f2, f3);
+#undef FH_STEP_A
+    } else if (yact) {
+      stream_pair(st, 0, f0, f1);
+      stream_pair(st, 2, f2, f3);
+    } else {                               // no row blocks: straight to where the state update expects the ring
+      stream_pair(st, 2, f2, f3);
+      stream_pair(st, 4, f0, f1);
+    }
+    FH_T(3)
+
+    // ---- the two row blocks: the second one finds the ring one pair on when the first has an odd
+    // number of pairs (lbF even)
     if (yact) {
-      float prev_end = 0.0f;
-      const int lrow = 32 * lb + m;
-      const float dal = dAs[lrow];
-      // two 32-step blocks per trip: block sb0 streams through (f0, f1), block sb0 + 1 through (f2, f3)
-#define FU_BLOCK_B(FA, FB, SB)                                                                  \
-      {                                                                                         \
-        const float endv = dAs[32 * (SB) + 31];                                                 \
-        const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));                                 \
-        prev_end = endv;                                                                        \
-        _Pragma("unroll") for (int r = 0; r < 16; ++r) {                                        \
-          acc[0][r] *= gs;                                                                      \
-          acc[1][r] *= gs;                                                                      \
-        }                                                                                       \
-        const bf16x8_t fa = FA, fb = FB;                                                        \
-        FA = load_frag(cbf + (size_t)min(2 * (SB) + 4, nkb - 1) * FRAG);                        \
-        FB = load_frag(cbf + (size_t)min(2 * (SB) + 5, nkb - 1) * FRAG);                        \
-        _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {                                      \
-          _Pragma("unroll") for (int pt = 0; pt < 2; ++pt) {                                    \
-            const int prow = 32 * pt + m;                                                       \
-            const bf16x8_t a = load_frag(xw + prow * Q + (((4 * (SB) + 2 * kk + g2) ^ (prow & qmask)) << 3)); \
-            acc[pt] = mma(a, kk == 0 ? fa : fb, acc[pt]);                                       \
-          }                                                                                     \
-        }                                                                                       \
-      }
-      // Block sb streams through (f0, f1) when sb is even and (f2, f3) when it is odd; the loop
-      // takes two blocks per trip without a guard between them, so an odd count starts with
-      // block 0 on its own.
-      if (lb & 1) {
-        FU_BLOCK_B(f0, f1, 0)
-        for (int sb0 = 1; sb0 < lb; sb0 += 2) {
-          FU_BLOCK_B(f2, f3, sb0)
-          FU_BLOCK_B(f0, f1, sb0 + 1)
-        }
-        f0 = f2;                            // the diagonal block's fragments
-        f1 = f3;
-      } else {
-        for (int sb0 = 0; sb0 < lb; sb0 += 2) {
-          FU_BLOCK_B(f0, f1, sb0)
-          FU_BLOCK_B(f2, f3, sb0 + 1)
-        }
-      }
-#undef FU_BLOCK_B
-      // diagonal block: the per-row factor once, then the factor of every element
-      const float rf = exp2_hw(fminf(dal - prev_end, 0.0f));
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc[0][r] *= rf;
-        acc[1][r] *= rf;
-      }
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const int ks = 2 * lb + kk;
-        const bf16x8_t f = kk == 0 ? f0 : f1;
-        const int sbase = 16 * ks + 8 * g2;
-        const float4 a0 = *reinterpret_cast<const float4 *>(dAs + sbase), a1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
-        const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
-        const float das[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
-        float mv[8];
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-          const float v = (float)f[jj] * exp2_hw(dal - das[jj]) * dtv[jj];
-          mv[jj] = (sbase + jj <= lrow) ? v : 0.0f;
-        }
-        const bf16x8_t bf = pack8(mv);
-#pragma unroll
-        for (int pt = 0; pt < 2; ++pt) {
-          const int prow = 32 * pt + m;
-          const bf16x8_t a = load_frag(xr + prow * Q + (((2 * ks + g2) ^ (prow & qmask)) << 3));
-          acc[pt] = mma(a, bf, acc[pt]);
-        }
-      }
-      // skip term D x_l from the plain tile (this lane's column l, the 16 rows p of each half)
-      if constexpr (DMODE != 0) {
-        const int xcol = lrow & 7, xchunk = lrow >> 3;
-        const float dh = DMODE == 1 ? p.Dk[h] : 0.0f;
-#pragma unroll
-        for (int pt = 0; pt < 2; ++pt)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            float dv[4] = {dh, dh, dh, dh};
-            if constexpr (DMODE == 2) {
-              const float4 d4 = *reinterpret_cast<const float4 *>(p.Dk + (size_t)h * FU_P + 32 * pt + 8 * q + 4 * g2);
-              dv[0] = d4.x; dv[1] = d4.y; dv[2] = d4.z; dv[3] = d4.w;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int prow = 32 * pt + 8 * q + 4 * g2 + j;
-              const float xv = (float)xr[prow * Q + ((xchunk ^ (prow & qmask)) << 3) + xcol];
-              acc[pt][4 * q + j] = __builtin_fmaf(dv[j], xv, acc[pt][4 * q + j]);
-            }
-          }
+      half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
+      if (lbF & 1) half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
+      else half_row_block<DMODE == 1>(accS, f2, f3, f0, f1, lbS, st.n_first, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
+      if constexpr (DMODE == 2) {
+        half_skip_term(accF, lbF, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
+        half_skip_term(accS, lbS, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
       }
     }
+    FH_T(4)
+    __syncthreads();                       // every wave is past the carried state: its tile becomes the output staging
+    FH_T(5)
 
-    // gate operands of this wave's rows, in the row-major order of the output pass
-    bf16x8_t zreg[2], znext[2];
-    const __bf16 *zg = p.z + (xg - p.x) + (size_t)(32 * lb + (lane >> 2)) * xrow + 8 * (lane & 3);
-    if (yact && HAS_Z) {                   // requested now, used after the state update
+    // ---- requests to HBM: the gate operands of this wave's rows (in the row-major order of the
+    // output pass) and the next chunk's inputs
+    bf16x8_t zF[2], zS[2];
+    const int row_o = c * Q * xrow_b;
+    if (yact && HAS_Z) {
 #pragma unroll
       for (int pass = 0; pass < 2; ++pass) {
-        zreg[pass] = load_frag(zg + (size_t)(16 * pass) * xrow);
-        znext[pass] = load_frag(zg + (size_t)(16 * pass) * xrow + 32);
+        zF[pass] = buf_load16(rz, v_row, row_o + (32 * lbF + 16 * pass) * xrow_b);
+        zS[pass] = buf_load16(rz, v_row, row_o + (32 * lbS + 16 * pass) * xrow_b);
       }
     }
-    // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p]
+    const int cn = min(c + 1, nc - 1);
+    FH_REQUEST_CHUNK(cn)
+#ifdef FH_TIMING_WAIT
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    FH_T(8)
+#endif
+
+    // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p].  The ring stands one
+    // pair on; the last steps request the next chunk's first fragments of C.
     if (sact) {
-      const __bf16 *btf = p.Btblk + ((unit * KS) * NT + nt_s) * FRAG + lane * 8;
-      const size_t kstep = (size_t)NT * FRAG;
-      f0 = load_frag(btf);
-      f1 = load_frag(btf + kstep);
-      f2 = load_frag(btf + (size_t)min(2, KS - 1) * kstep);
-      f3 = load_frag(btf + (size_t)min(3, KS - 1) * kstep);
       float prev_end = 0.0f;
-      const int prow = 32 * pt_s + m;
-#define FU_STEP_C(F, KK)                                                                        \
+#define FH_STEP_C(F, KK)                                                                        \
       {                                                                                         \
-        const bf16x8_t f = F;                                                                   \
-        F = load_frag(btf + (size_t)min((KK) + 4, KS - 1) * kstep);                             \
-        const bf16x8_t xf = load_frag(xw + prow * Q + (((2 * (KK) + g2) ^ (prow & qmask)) << 3)); \
-        S = mma(f, xf, S);                                                                      \
+        const bf16x8_t xf = load_frag(xw + m * Q + (((2 * (KK) + g2) ^ (m & qmask)) << 3));     \
+        S = mma(F, xf, S);                                                                      \
       }
-      for (int k0 = 0; k0 < KS; k0 += 4) {
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          {
-            const float endv = dAs[16 * (k0 + 2 * half) + 31];
-            const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));
-            prev_end = endv;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) S[r] *= gs;
-          }
-          if (half == 0) {
-            FU_STEP_C(f0, k0)
-            FU_STEP_C(f1, k0 + 1)
-          } else {
-            FU_STEP_C(f2, k0 + 2)
-            FU_STEP_C(f3, k0 + 3)
-          }
-        }
+#define FH_SCALE_C(KK)                                                                          \
+      {                                                                                         \
+        const float endv = dAs[16 * (KK) + 31];                                                 \
+        const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));                                 \
+        prev_end = endv;                                                                        \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) S[r] *= gs;                              \
       }
-#undef FU_STEP_C
+      for (int k0 = 0; k0 < KS - 4; k0 += 4) {
+        FH_SCALE_C(k0)
+        FH_STEP_C(f2, k0)
+        f2 = buf_load16(rf, st.vf, st.off_bt + (k0 + 4) * st.bt_step);
+        FH_STEP_C(f3, k0 + 1)
+        f3 = buf_load16(rf, st.vf, st.off_bt + (k0 + 5) * st.bt_step);
+        FH_SCALE_C(k0 + 2)
+        FH_STEP_C(f0, k0 + 2)
+        f0 = buf_load16(rf, st.vf, st.off_bt + (k0 + 6) * st.bt_step);
+        FH_STEP_C(f1, k0 + 3)
+        f1 = buf_load16(rf, st.vf, st.off_bt + (k0 + 7) * st.bt_step);
+      }
+      FH_SCALE_C(KS - 4)
+      FH_STEP_C(f2, KS - 4)
+      if (yact) f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
+      FH_STEP_C(f3, KS - 3)
+      if (yact) f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
+      FH_SCALE_C(KS - 2)
+      FH_STEP_C(f0, KS - 2)
+      if (yact) f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
+      FH_STEP_C(f1, KS - 1)
+      if (yact) f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
+#undef FH_STEP_C
+#undef FH_SCALE_C
+    } else if (yact) {
+      f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
+      f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
+      f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
+      f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
     }
-    __syncthreads();                       // the plain tile is free: it becomes the output staging
-    // ---- output: through a wave-private 32 x 32 fp32 tile to row-major 16-byte accesses
+    FH_T(6)
+    // ---- the output through a wave-private 32 x 32 fp32 tile to row-major 16-byte accesses: gate, store
     if (yact) {
-      float *stg = reinterpret_cast<float *>(smem + FU_TILE_BYTES) + wave * 1024;
-      __bf16 *yg = p.y + (xg - p.x);
+      float *stg = reinterpret_cast<float *>(smem + 2 * FH_TILE_BYTES) + wave * 1024;
 #pragma unroll
-      for (int pt = 0; pt < 2; ++pt) {
+      for (int which = 0; which < 2; ++which) {
+        const int lb = which == 0 ? lbF : lbS;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float4 v = make_float4(acc[pt][4 * q], acc[pt][4 * q + 1], acc[pt][4 * q + 2], acc[pt][4 * q + 3]);
+          const float4 v = which == 0 ? make_float4(accF[4 * q], accF[4 * q + 1], accF[4 * q + 2], accF[4 * q + 3])
+                                      : make_float4(accS[4 * q], accS[4 * q + 1], accS[4 * q + 2], accS[4 * q + 3]);
           *reinterpret_cast<float4 *>(stg + m * 32 + (((2 * q + g2) ^ (m & 7)) << 2)) = v;
         }
         wave_lds_sync();
@@ -473,27 +574,36 @@ void ssd_fused_kernel(const SsdFusedParams p) {
           float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
           if (HAS_Z) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] *= silu_f32((float)(pt == 0 ? zreg[pass][j] : znext[pass][j]));
+            for (int j = 0; j < 8; ++j) v[j] *= silu_f32((float)(which == 0 ? zF[pass][j] : zS[pass][j]));
           }
-          *reinterpret_cast<bf16x8_t *>(yg + (size_t)(32 * lb + l) * xrow + 32 * pt + 8 * c4) = pack8(v);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, pack8(v)), ry, v_row,
+                                                 row_o + (32 * lb + 16 * pass) * xrow_b, 0);
         }
         wave_lds_sync();
       }
     }
+    FH_T(7)
   }
+#undef FH_REQUEST_CHUNK
+#undef FH_C_OFF
 
   if (p.final_states && sact) {
-    float *fp = p.final_states + (((size_t)b * H + h) * FU_P + 32 * pt_s + m) * N + 32 * nt_s;
+    float *fp = p.final_states + (((size_t)b * H + h) * FU_P + p0 + m) * N + 32 * nt_s;
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       *reinterpret_cast<float4 *>(fp + 8 * q + 4 * g2) = make_float4(S[4 * q], S[4 * q + 1], S[4 * q + 2], S[4 * q + 3]);
   }
+#ifdef FH_TIMING
+  if (lane == 0)
+    for (int i = 0; i < 10; ++i) p.times[((size_t)vid * 4 + wave) * 10 + i] = tacc[i];
+#endif
+#undef FH_T
 }
 
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct FusedLayout {
-  size_t dA_cs, dt_out, dA2, ws, Cblk, Btblk, CBblk, total;
+  size_t dt_out, dA2, Cblk, Btblk, CBblk, total;
 };
 
 static FusedLayout fused_layout(const SsdDims &d) {
@@ -502,13 +612,14 @@ static FusedLayout fused_layout(const SsdDims &d) {
   const size_t bc = align_up((size_t)d.batch * d.len * d.groups * d.nstate * 2);
   const size_t cb = align_up((size_t)d.batch * d.nchunks * d.groups * d.chunk * d.chunk * 2);
   size_t at = 0;
-  f.dA_cs = at; at += per_step;
   f.dt_out = at; at += per_step;
   f.dA2 = at; at += per_step;
-  f.ws = at; at += per_step;
   f.Cblk = at; at += bc;
   f.Btblk = at; at += bc;
   f.CBblk = at; at += cb;
+#ifdef FH_TIMING
+  at += (size_t)d.batch * d.heads * 2 * 4 * 10 * sizeof(long long);   // per-wave phase clocks behind everything else
+#endif
   f.total = at;
   return f;
 }
@@ -516,7 +627,12 @@ static FusedLayout fused_layout(const SsdDims &d) {
 static bool fused_shape_ok(const SsdDims &d) {
   const bool q_ok = d.chunk == 64 || d.chunk == 128 || d.chunk == 256;
   const bool n_ok = d.nstate == 64 || d.nstate == 128;
-  return q_ok && n_ok && d.hdim == FU_P && d.len % d.chunk == 0 && d.heads % d.groups == 0;
+  if (!(q_ok && n_ok && d.hdim == FU_P && d.len % d.chunk == 0 && d.heads % d.groups == 0)) return false;
+  // the kernel addresses with 32-bit byte offsets: inside one batch row of x, z and y, inside the
+  // per-step arrays and inside the fragment copies
+  const size_t lim = (size_t)1 << 31;
+  const FusedLayout f = fused_layout(d);
+  return (size_t)d.len * d.heads * FU_P * 2 < lim && f.Cblk - f.dt_out + (size_t)d.len * 4 < lim && f.total - f.Cblk < lim;
 }
 
 }  // namespace ssm
@@ -574,12 +690,12 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
 
   SsdCumsumParams cp{};
   cp.dt = a->dt; cp.A = a->A; cp.bias = a->dt_bias;
-  cp.dA_cs = reinterpret_cast<float *>(ws + lay.dA_cs);
+  cp.dA_cs = nullptr;
   cp.dt_out = reinterpret_cast<float *>(ws + lay.dt_out);
   cp.d = d; cp.dt_dtype = a->dt_dtype; cp.softplus = a->dt_softplus ? 1 : 0; cp.dt_min = a->dt_min; cp.dt_max = a->dt_max;
   const size_t units = (size_t)d.batch * d.nchunks * ((d.heads + PD_HEADS - 1) / PD_HEADS);
   hipLaunchKernelGGL(ssd_fused_prep_dt_kernel, dim3((unsigned)units), dim3(256), 0, s, cp,
-                     reinterpret_cast<float *>(ws + lay.dA2), reinterpret_cast<float *>(ws + lay.ws));
+                     reinterpret_cast<float *>(ws + lay.dA2));
   SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(prep dt)");
 
   SsdBmmParams bp{};
@@ -601,22 +717,24 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   SsdFusedParams fp{};
   fp.x = reinterpret_cast<const __bf16 *>(a->x); fp.z = reinterpret_cast<const __bf16 *>(a->z);
   fp.y = reinterpret_cast<__bf16 *>(a->y);
-  fp.dA2 = reinterpret_cast<const float *>(ws + lay.dA2); fp.dtv = cp.dt_out; fp.ws = reinterpret_cast<const float *>(ws + lay.ws);
+  fp.dA2 = reinterpret_cast<const float *>(ws + lay.dA2); fp.dtv = cp.dt_out;
   fp.Cblk = Cblk; fp.CBblk = reinterpret_cast<const __bf16 *>(ws + lay.CBblk); fp.Btblk = Btblk;
   fp.Dk = a->Dskip; fp.init = a->initial_states; fp.final_states = a->final_states;
   fp.batch = d.batch; fp.len = d.len; fp.heads = d.heads; fp.groups = d.groups; fp.nstate = d.nstate; fp.chunk = d.chunk;
   fp.nchunks = d.nchunks; fp.d_per_p = a->d_per_p ? 1 : 0;
+#ifdef FH_TIMING
+  fp.times = reinterpret_cast<long long *>(ws + lay.CBblk + align_up((size_t)d.batch * d.nchunks * d.groups * d.chunk * d.chunk * 2));
+#endif
   const int dmode = !a->Dskip ? 0 : (a->d_per_p ? 2 : 1);
-  const unsigned grid = (unsigned)(d.batch * d.heads);
+  const unsigned grid = (unsigned)(d.batch * d.heads) * 2;
 #define SSM_LAUNCH_FUSED(DM, HZ)                                                                   \
   {                                                                                                \
-    auto kernel = ssd_fused_kernel<DM, HZ>;                                                        \
-    if (allow_dynamic_lds(kernel, FU_LDS_BYTES) != hipSuccess) {                                   \
-      (void)hipGetLastError();                                                                     \
-      set_error("ssm_ssd_combined_fwd: cannot reserve %d bytes of LDS", FU_LDS_BYTES);             \
+    auto kernel = ssd_fused_half_kernel<DM, HZ>;                                                   \
+    if (allow_dynamic_lds(kernel, FH_LDS_BYTES) != hipSuccess) {                                   \
+      set_error("ssm_ssd_combined_fwd: cannot reserve %d bytes of LDS", FH_LDS_BYTES);             \
       return SSM_ERR_LAUNCH;                                                                       \
     }                                                                                              \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(FU_THREADS), FU_LDS_BYTES, s, fp);                 \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(FH_THREADS), FH_LDS_BYTES, s, fp);                 \
   }
   if (a->z) {
     if (dmode == 0) SSM_LAUNCH_FUSED(0, true) else if (dmode == 1) SSM_LAUNCH_FUSED(1, true) else SSM_LAUNCH_FUSED(2, true)
