@@ -211,8 +211,9 @@ __device__ __forceinline__ void stream_pair(const HalfStream &st, int i, bf16x8_
 }
 
 // Blocks below the diagonal and the diagonal block of row block `lb` into `acc` (one 32 x 32
-// tile: lane = column l, registers = rows p).  Block sb takes its two fragments from (a0, a1)
-// if sb is even, from (b0, b1) if odd; they are the stream's places pos0 + 2 sb, + 1.
+// tile: lane = column l, registers = rows p).  The fragments of block sb are the stream's places
+// pos0 + 2 sb, + 1; (a0, a1) is the register pair that holds those of the diagonal block and of
+// every second block before it, (b0, b1) the other pair.
 // With SKIP, the per-head skip factor dskip joins the diagonal of the last operand (CB dt + D at
 // s = l, rounded to bf16 as one number), so that the product with the plain x adds D x.
 template <bool SKIP>
@@ -235,24 +236,11 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
     acc = mma(x1, FB, acc);                                                                     \
     stream_pair(st, pos0 + 2 * (SB) + 4, FA, FB);                                               \
   }
-  bf16x8_t d0, d1;
-  if (lb & 1) {
-    for (int sb0 = 0; sb0 < lb - 1; sb0 += 2) {
-      FH_BLOCK(a0, a1, sb0)
-      FH_BLOCK(b0, b1, sb0 + 1)
-    }
-    FH_BLOCK(a0, a1, lb - 1)
-    d0 = b0;
-    d1 = b1;
-    stream_pair(st, pos0 + 2 * lb + 4, b0, b1);
-  } else {
-    for (int sb0 = 0; sb0 < lb; sb0 += 2) {
-      FH_BLOCK(a0, a1, sb0)
-      FH_BLOCK(b0, b1, sb0 + 1)
-    }
-    d0 = a0;
-    d1 = a1;
-    stream_pair(st, pos0 + 2 * lb + 4, a0, a1);
+  const int odd = lb & 1;
+  if (odd) FH_BLOCK(b0, b1, 0)
+  for (int sb0 = odd; sb0 < lb; sb0 += 2) {
+    FH_BLOCK(a0, a1, sb0)
+    FH_BLOCK(b0, b1, sb0 + 1)
   }
 #undef FH_BLOCK
   const float rf = exp2_hw(fminf(dal - prev_end, 0.0f));
@@ -260,11 +248,9 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
   for (int r = 0; r < 16; ++r) acc[r] *= rf;
   // the diagonal block: its fragments of CB hold zeros above the diagonal, so that the decay
   // only needs a bound there
-  int jdiag = m - 8 * g2;                  // the lane's diagonal element is number jdiag - 16 kk of fragment kk, if in 0..7
-  asm volatile("" : "+v"(jdiag));          // (rebuilt here for each row block rather than kept in registers)
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) {
-    const bf16x8_t f = kk == 0 ? d0 : d1;
+    const bf16x8_t f = kk == 0 ? a0 : a1;
     const int sbase = 32 * lb + 16 * kk + 8 * g2;
     const float4 q0 = *reinterpret_cast<const float4 *>(dAs + sbase), q1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
     const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
@@ -273,12 +259,21 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
     float mv[8];
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
-      mv[jj] = (float)f[jj] * dtv[jj] * exp2_hw(fminf(dal - das[jj], 0.0f));
-      if (SKIP) mv[jj] += (16 * kk + jj == jdiag) ? dskip : 0.0f;
+      const float cbdt = (float)f[jj] * dtv[jj], e = exp2_hw(fminf(dal - das[jj], 0.0f));
+      if (SKIP) {
+        // element jj of fragment kk lies on the diagonal in lane 16 kk + jj (g2 = 0) and lane 32 + 16 kk + 8 + jj (g2 = 1)
+        const unsigned long long on_diag = (1ull << (16 * kk + jj)) | (1ull << (40 + 16 * kk + jj));
+        float sel;
+        asm volatile("v_cndmask_b32_e64 %0, 0, %1, %2" : "=v"(sel) : "v"(dskip), "s"(on_diag));   // volatile: rebuilt at each use, not kept
+        mv[jj] = __builtin_fmaf(cbdt, e, sel);
+      } else {
+        mv[jj] = cbdt * e;
+      }
     }
     const bf16x8_t a = load_frag(xr + m * Q + (((4 * lb + 2 * kk + g2) ^ (m & qmask)) << 3));
     acc = mma(a, pack8(mv), acc);
   }
+  stream_pair(st, pos0 + 2 * lb + 4, a0, a1);
 }
 
 // acc[p][l] += D[p] x[l][p] for row block lb, x read from the plain tile (per-channel skip factors).
@@ -299,7 +294,7 @@ __device__ __forceinline__ void half_skip_term(f32x16_t &acc, int lb, const __bf
   }
 }
 
-template <int DMODE, bool HAS_Z>
+template <int Q, int N, int DMODE, bool HAS_Z>
 __global__ __launch_bounds__(FH_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void ssd_fused_half_kernel(const SsdFusedParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -310,9 +305,9 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
   float *dts = dAs + 256;                                               // [Q] dt
   float *wss = dts + 256;                                               // [Q] staging weight dt exp(cs[l | 31] - cs[l])
 
-  const int Q = p.chunk, N = p.nstate, H = p.heads, G = p.groups, nc = p.nchunks;
-  const int NLB = Q >> 5, NT = N >> 5, KS = Q >> 4, KN = N >> 4;
-  const int qmask = min(15, (Q >> 3) - 1), nmask = min(15, (N >> 3) - 1);
+  const int H = p.heads, G = p.groups, nc = p.nchunks;
+  constexpr int NLB = Q >> 5, NT = N >> 5, KS = Q >> 4, KN = N >> 4;
+  constexpr int qmask = Q >= 128 ? 15 : (Q >> 3) - 1, nmask = N >= 128 ? 15 : (N >> 3) - 1;
   const int wave = wave_id_uniform(), lane = lane_id();
   const int g2 = lane >> 5, m = lane & 31;
   // Workgroups go to the 8 XCDs round-robin by blockIdx: renumber them so that each XCD (own L2)
@@ -390,6 +385,15 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
   for (int c = 0; c < nc; ++c) {
     // LDS addresses are rebuilt from the lane number in every chunk: kept across chunks they would
     // occupy more registers than they cost to recompute
+    // The SIMD serves its oldest wave first: left alone, the workgroup that came to a CU last would run
+    // at the lowest rate throughout and finish long after the others.  Rotating the priority with the
+    // chunk number shares the CU evenly (slot = presumably the n-th workgroup on its CU).
+    {
+      const int pr = (c + ((int)blockIdx.x >> 3) / 32) % 3;
+      if (pr == 0) __builtin_amdgcn_s_setprio(0);
+      else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+      else __builtin_amdgcn_s_setprio(2);
+    }
     int ln = lane;
     asm volatile("" : "+v"(ln));
     const int lane = ln, g2 = ln >> 5, m = ln & 31, tid = wave * WAVE + ln;
@@ -441,8 +445,6 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     FH_T(2)
 
     // ---- carried state: acc[p][l] = sum_n S[p][n] C[l][n] for both row blocks
-    accF = (f32x16_t){0};
-    accS = (f32x16_t){0};
     if (yact && carry) {
       const int cF = FH_C_OFF(c, lbF, 0), cS = FH_C_OFF(c, lbS, 0);
 #define FH_STEP_A(FF, FS, KK)                                                                     \
@@ -451,7 +453,17 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
         accF = mma(a, FF, accF);                                                                  \
         accS = mma(a, FS, accS);                                                                  \
       }
-      for (int kn0 = 0; kn0 < KN - 2; kn0 += 2) {
+      {                                    // the first step starts the accumulators
+        const bf16x8_t a = load_frag(sbf + m * N + ((g2 ^ (m & nmask)) << 3));
+        accF = mma(a, f0, (f32x16_t){0});
+        accS = mma(a, f1, (f32x16_t){0});
+        f0 = buf_load16(rf, st.vf, cF + (2 << 10));
+        f1 = buf_load16(rf, st.vf, cS + (2 << 10));
+        FH_STEP_A(f2, f3, 1)
+        f2 = buf_load16(rf, st.vf, cF + (3 << 10));
+        f3 = buf_load16(rf, st.vf, cS + (3 << 10));
+      }
+      for (int kn0 = 2; kn0 < KN - 2; kn0 += 2) {
         FH_STEP_A(f0, f1, kn0)
         f0 = buf_load16(rf, st.vf, cF + ((kn0 + 2) << 10));
         f1 = buf_load16(rf, st.vf, cS + ((kn0 + 2) << 10));
@@ -464,7 +476,9 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
       FH_STEP_A(f2, f3, KN - 1)
       stream_pair(st, 2, f2, f3);
 #undef FH_STEP_A
-    } else if (yact) {
+    } else if (yact) {                     // first chunk without an initial state
+      accF = (f32x16_t){0};
+      accS = (f32x16_t){0};
       stream_pair(st, 0, f0, f1);
       stream_pair(st, 2, f2, f3);
     } else {                               // no row blocks: straight to where the state update expects the ring
@@ -473,12 +487,12 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     }
     FH_T(3)
 
-    // ---- the two row blocks: the second one finds the ring one pair on when the first has an odd
-    // number of pairs (lbF even)
+    // ---- the two row blocks.  Pair q of the stream lives in (f0, f1) if q is even, in (f2, f3) if odd:
+    // the diagonal block of the first row block is pair lbF, that of the second pair NLB.
     if (yact) {
-      half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
-      if (lbF & 1) half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
-      else half_row_block<DMODE == 1>(accS, f2, f3, f0, f1, lbS, st.n_first, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
+      if (lbF & 1) half_row_block<DMODE == 1>(accF, f2, f3, f0, f1, lbF, 0, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
+      else half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
+      half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
       if constexpr (DMODE == 2) {
         half_skip_term(accF, lbF, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
         half_skip_term(accS, lbS, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
@@ -727,20 +741,37 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
 #endif
   const int dmode = !a->Dskip ? 0 : (a->d_per_p ? 2 : 1);
   const unsigned grid = (unsigned)(d.batch * d.heads) * 2;
-#define SSM_LAUNCH_FUSED(DM, HZ)                                                                   \
+#define SSM_LAUNCH_FUSED(QQ, NN, DM, HZ)                                                           \
   {                                                                                                \
-    auto kernel = ssd_fused_half_kernel<DM, HZ>;                                                   \
+    auto kernel = ssd_fused_half_kernel<QQ, NN, DM, HZ>;                                           \
     if (allow_dynamic_lds(kernel, FH_LDS_BYTES) != hipSuccess) {                                   \
       set_error("ssm_ssd_combined_fwd: cannot reserve %d bytes of LDS", FH_LDS_BYTES);             \
       return SSM_ERR_LAUNCH;                                                                       \
     }                                                                                              \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(FH_THREADS), FH_LDS_BYTES, s, fp);                 \
   }
-  if (a->z) {
-    if (dmode == 0) SSM_LAUNCH_FUSED(0, true) else if (dmode == 1) SSM_LAUNCH_FUSED(1, true) else SSM_LAUNCH_FUSED(2, true)
-  } else {
-    if (dmode == 0) SSM_LAUNCH_FUSED(0, false) else if (dmode == 1) SSM_LAUNCH_FUSED(1, false) else SSM_LAUNCH_FUSED(2, false)
+#define SSM_LAUNCH_FUSED_DZ(QQ, NN)                                                                \
+  {                                                                                                \
+    if (a->z) {                                                                                    \
+      if (dmode == 0) SSM_LAUNCH_FUSED(QQ, NN, 0, true)                                            \
+      else if (dmode == 1) SSM_LAUNCH_FUSED(QQ, NN, 1, true)                                       \
+      else SSM_LAUNCH_FUSED(QQ, NN, 2, true)                                                       \
+    } else {                                                                                       \
+      if (dmode == 0) SSM_LAUNCH_FUSED(QQ, NN, 0, false)                                           \
+      else if (dmode == 1) SSM_LAUNCH_FUSED(QQ, NN, 1, false)                                      \
+      else SSM_LAUNCH_FUSED(QQ, NN, 2, false)                                                      \
+    }                                                                                              \
   }
+  if (d.nstate == 128) {
+    if (d.chunk == 256) SSM_LAUNCH_FUSED_DZ(256, 128)
+    else if (d.chunk == 128) SSM_LAUNCH_FUSED_DZ(128, 128)
+    else SSM_LAUNCH_FUSED_DZ(64, 128)
+  } else {
+    if (d.chunk == 256) SSM_LAUNCH_FUSED_DZ(256, 64)
+    else if (d.chunk == 128) SSM_LAUNCH_FUSED_DZ(128, 64)
+    else SSM_LAUNCH_FUSED_DZ(64, 64)
+  }
+#undef SSM_LAUNCH_FUSED_DZ
 #undef SSM_LAUNCH_FUSED
   SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd");
   note_mfma_launch(8);
