@@ -20,7 +20,6 @@ namespace ssm {
 
 constexpr int LN_THREADS = 256;
 constexpr int LN_WAVES = LN_THREADS / WAVE;
-constexpr int LN_MAX_PER_LANE = 32;          // cached values per lane -> hidden <= 2048
 
 struct NormParams {
   const void *x, *res, *dy;

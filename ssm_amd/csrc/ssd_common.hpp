@@ -31,7 +31,6 @@ struct SsdBmmParams {
   void *out;                  // (B, nc, G, Q, Q)
   int batch, len, groups, kdim, chunk, nchunks;
   int in_dtype, out_dtype, causal;
-  int blocked;                // MFMA kernel only: write 32 x 16 operand fragments [unit][l/32][s/16][lane][8] (bf16)
 };
 
 struct SsdStateParams {

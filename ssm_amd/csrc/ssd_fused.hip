@@ -48,20 +48,40 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 
 __device__ __forceinline__ void wave_lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-// ------------------------------------------------------------------ prep: dt
-// One workgroup per (b, c, 4 heads): the (Q x 4) slab of dt is read row by row
-// (16 contiguous bytes per step) into LDS transposed to [head][step]; then one
-// wave per head forms dt' = clamp(softplus(dt + bias)) and the running sum of dt' A
-// (stored scaled by log2 e, the unit of the fused kernel's exponentials).
+// ---------------------------------------------------------------------- prep
+// One launch prepares everything the fused kernel reads besides x and z; the
+// workgroups (256 threads) take one of three roles by their index:
+//
+//  dt:   one workgroup per (b, c, 4 heads).  The (Q x 4) slab of dt is read row by
+//        row (16 contiguous bytes per step) into LDS transposed to [head][step];
+//        then one wave per head forms dt' = clamp(softplus(dt + bias)) and the
+//        running sum of dt' A (stored scaled by log2 e, the unit of the fused
+//        kernel's exponentials).
+//  pack: one wave per operand fragment of C and B^T.  Fragment (lane, j) of a
+//        32 x 16 block: row 32 rb + lane % 32, column 16 kb + 8 (lane / 32) + j.
+//          Cblk [(b,c,g)][lb][kn]  from C  (rows = time, columns = state)
+//          Btblk[(b,c,g)][ks][nt]  from B  (rows = state, columns = time)
+//  CB:   one wave per 32 x 32 block on or below the diagonal of C B^T of a chunk:
+//        MFMA over the state dimension, then through a wave-private LDS tile into
+//          CBblk[(b,c,g)][lb][ks]  (rows = l, columns = s),
+//        with zeros above the diagonal inside the diagonal blocks.
 constexpr int PD_HEADS = 4;
-__global__ __launch_bounds__(256) void ssd_fused_prep_dt_kernel(const SsdCumsumParams p, float *dA2) {
-  __shared__ float tile[PD_HEADS][256 + 1];
+struct SsdPrepParams {
+  SsdCumsumParams cs;
+  float *dA2;
+  const __bf16 *Cm, *Bm;
+  __bf16 *Cblk, *Btblk, *CBblk;
+  unsigned n_dt, n_pack;                 // workgroups of the first two roles
+};
+
+__device__ __forceinline__ void prep_dt_role(const SsdCumsumParams &p, float *dA2, int wg, float *lds) {
+  float (*tile)[256 + 1] = reinterpret_cast<float (*)[256 + 1]>(lds);
   const SsdDims &d = p.d;
   const int Q = d.chunk;
   const int hgroups = (d.heads + PD_HEADS - 1) / PD_HEADS;
-  const int hg = (int)blockIdx.x % hgroups;
-  const int c = ((int)blockIdx.x / hgroups) % d.nchunks;
-  const int b = (int)blockIdx.x / (hgroups * d.nchunks);
+  const int hg = wg % hgroups;
+  const int c = (wg / hgroups) % d.nchunks;
+  const int b = wg / (hgroups * d.nchunks);
   const int h0 = hg * PD_HEADS;
   for (int e = threadIdx.x; e < Q * PD_HEADS; e += 256) {
     const int l = e / PD_HEADS, hh = e % PD_HEADS;
@@ -110,21 +130,14 @@ __global__ __launch_bounds__(256) void ssd_fused_prep_dt_kernel(const SsdCumsumP
   }
 }
 
-// ---------------------------------------------------------------- prep: pack
-// Fragment (lane, j) of a 32 x 16 operand block: row 32 rb + lane % 32,
-// column 16 kb + 8 (lane / 32) + j.  One wave per fragment; the first
-// B nc G (NLB KN) fragments are those of C, the rest those of B^T:
-//   Cblk [(b,c,g)][lb][kn]  from C  (rows = time, columns = state)
-//   Btblk[(b,c,g)][ks][nt]  from B  (rows = state, columns = time)
-// (CBblk[(b,c,g)][lb][ks], rows = l, columns = s, is written by the C B^T kernel.)
-__global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *Cm, const __bf16 *Bm, __bf16 *Cblk, __bf16 *Btblk,
-                                                             int batch, int len, int groups, int nstate, int chunk) {
+__device__ __forceinline__ void prep_pack_role(const SsdPrepParams &pp, unsigned wg) {
+  const SsdDims &d = pp.cs.d;
   const int wave = wave_id_uniform(), lane = lane_id();
-  const int Q = chunk, N = nstate, nc = len / Q;
+  const int Q = d.chunk, N = d.nstate, nc = d.nchunks, groups = d.groups, len = d.len;
   const int NLB = Q >> 5, KS = Q >> 4, KN = N >> 4, NT = N >> 5;
-  const size_t units = (size_t)batch * nc * groups;
+  const size_t units = (size_t)d.batch * nc * groups;
   const size_t nC = units * NLB * KN, nB = units * KS * NT;
-  size_t f = (size_t)blockIdx.x * 4 + wave;
+  size_t f = (size_t)wg * 4 + wave;
   if (f >= nC + nB) return;
   const bool is_c = f < nC;
   if (!is_c) f -= nC;
@@ -138,14 +151,60 @@ __global__ __launch_bounds__(256) void ssd_fused_pack_kernel(const __bf16 *Cm, c
   bf16x8_t v;
   if (is_c) {
     const int lb = inner / KN, kn = inner % KN;
-    v = load_frag(Cm + (((size_t)b * len + (size_t)c * Q + 32 * lb + m) * groups + g) * N + 16 * kn + 8 * g2);
+    v = load_frag(pp.Cm + (((size_t)b * len + (size_t)c * Q + 32 * lb + m) * groups + g) * N + 16 * kn + 8 * g2);
   } else {
     const int ks = inner / NT, nt = inner % NT;
-    const __bf16 *col = Bm + (((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * groups + g) * N + 32 * nt + m;
+    const __bf16 *col = pp.Bm + (((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * groups + g) * N + 32 * nt + m;
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = col[(size_t)j * groups * N];
   }
-  *reinterpret_cast<bf16x8_t *>((is_c ? Cblk : Btblk) + f * FRAG + lane * 8) = v;
+  *reinterpret_cast<bf16x8_t *>((is_c ? pp.Cblk : pp.Btblk) + f * FRAG + lane * 8) = v;
+}
+
+__device__ __forceinline__ void prep_cb_role(const SsdPrepParams &pp, unsigned wg, float *lds) {
+  const SsdDims &d = pp.cs.d;
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int Q = d.chunk, N = d.nstate, groups = d.groups;
+  const int NLB = Q >> 5, KS = Q >> 4;
+  const int per_unit = NLB * (NLB + 1) / 2;
+  const size_t units = (size_t)d.batch * d.nchunks * groups;
+  const size_t blk = (size_t)wg * 4 + wave;
+  if (blk >= units * per_unit) return;
+  const size_t unit = blk / per_unit;
+  const int idx = (int)(blk % per_unit);
+  int lb = 0;
+  while ((lb + 1) * (lb + 2) / 2 <= idx) ++lb;
+  const int sb = idx - lb * (lb + 1) / 2;
+  const int g = (int)(unit % groups);
+  const size_t bc = unit / groups;                        // b * nchunks + c: the chunk's first row is bc * Q
+  const int m = lane & 31, g2 = lane >> 5;
+  const __bf16 *crow_p = pp.Cm + ((bc * Q + 32 * lb + m) * groups + g) * N + 8 * g2;
+  const __bf16 *brow_p = pp.Bm + ((bc * Q + 32 * sb + m) * groups + g) * N + 8 * g2;
+  f32x16_t acc = {0};
+  for (int k0 = 0; k0 < N; k0 += 16) acc = mma(load_frag(crow_p + k0), load_frag(brow_p + k0), acc);
+  float (*tile)[33] = reinterpret_cast<float (*)[33]>(lds + wave * 32 * 33);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) tile[crow(r, g2)][m] = acc[r];
+  wave_lds_sync();
+  __bf16 *out = pp.CBblk + ((unit * NLB + lb) * KS + 2 * sb) * FRAG + lane * 8;
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int sl = 16 * kk + 8 * g2 + j;
+      v[j] = (sb < lb || sl <= m) ? tile[m][sl] : 0.0f;
+    }
+    *reinterpret_cast<bf16x8_t *>(out + kk * FRAG) = pack8(v);
+  }
+}
+
+__global__ __launch_bounds__(256) void ssd_fused_prep_kernel(const SsdPrepParams pp) {
+  __shared__ float lds[4 * 32 * 33];
+  const unsigned wg = blockIdx.x;
+  if (wg < pp.n_dt) prep_dt_role(pp.cs, pp.dA2, (int)wg, lds);
+  else if (wg < pp.n_dt + pp.n_pack) prep_pack_role(pp, wg - pp.n_dt);
+  else prep_cb_role(pp, wg - pp.n_dt - pp.n_pack, lds);
 }
 
 // ------------------------------------------------- fused kernel, half a head
@@ -219,7 +278,7 @@ __device__ __forceinline__ void stream_pair(const HalfStream &st, int i, bf16x8_
 template <bool SKIP>
 __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16x8_t &a1, bf16x8_t &b0, bf16x8_t &b1,
                                                int lb, int pos0, const HalfStream &st, const __bf16 *xw, const __bf16 *xr,
-                                               const float *dAs, const float *dts, int Q, int qmask, int m, int g2,
+                                               const float *dAs, const float *dqs, int Q, int qmask, int m, int g2,
                                                float dskip) {
   float prev_end = 0.0f;
   const int lrow = 32 * lb + m;
@@ -252,22 +311,21 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
   for (int kk = 0; kk < 2; ++kk) {
     const bf16x8_t f = kk == 0 ? a0 : a1;
     const int sbase = 32 * lb + 16 * kk + 8 * g2;
-    const float4 q0 = *reinterpret_cast<const float4 *>(dAs + sbase), q1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
-    const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
-    const float das[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-    const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+    const float4 q0 = *reinterpret_cast<const float4 *>(dqs + sbase), q1 = *reinterpret_cast<const float4 *>(dqs + sbase + 4);
+    const float dq[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
     float mv[8];
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
-      const float cbdt = (float)f[jj] * dtv[jj], e = exp2_hw(fminf(dal - das[jj], 0.0f));
+      // dt_s exp(cs_l - cs_s) as one exponential; the bound keeps the (zeroed) places above the diagonal finite
+      const float e = exp2_hw(fminf(dal + dq[jj], 126.0f));
       if (SKIP) {
         // element jj of fragment kk lies on the diagonal in lane 16 kk + jj (g2 = 0) and lane 32 + 16 kk + 8 + jj (g2 = 1)
         const unsigned long long on_diag = (1ull << (16 * kk + jj)) | (1ull << (40 + 16 * kk + jj));
         float sel;
         asm volatile("v_cndmask_b32_e64 %0, 0, %1, %2" : "=v"(sel) : "v"(dskip), "s"(on_diag));   // volatile: rebuilt at each use, not kept
-        mv[jj] = __builtin_fmaf(cbdt, e, sel);
+        mv[jj] = __builtin_fmaf((float)f[jj], e, sel);
       } else {
-        mv[jj] = cbdt * e;
+        mv[jj] = (float)f[jj] * e;
       }
     }
     const bf16x8_t a = load_frag(xr + m * Q + (((4 * lb + 2 * kk + g2) ^ (m & qmask)) << 3));
@@ -302,8 +360,8 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
   __bf16 *xr = reinterpret_cast<__bf16 *>(smem + FH_TILE_BYTES);        // x  [32][Q]
   __bf16 *sbf = reinterpret_cast<__bf16 *>(smem + 2 * FH_TILE_BYTES);   // S as bf16 [32][N]; later the output staging
   float *dAs = reinterpret_cast<float *>(smem + 3 * FH_TILE_BYTES);     // [Q] log2-scaled running sum
-  float *dts = dAs + 256;                                               // [Q] dt
-  float *wss = dts + 256;                                               // [Q] staging weight dt exp(cs[l | 31] - cs[l])
+  float *dqs = dAs + 256;                                               // [Q] log2(dt) - running sum: exponent offset of a step as a source
+  float *wss = dqs + 256;                                               // [Q] staging weight dt exp(cs[l | 31] - cs[l])
 
   const int H = p.heads, G = p.groups, nc = p.nchunks;
   constexpr int NLB = Q >> 5, NT = N >> 5, KS = Q >> 4, KN = N >> 4;
@@ -336,7 +394,7 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
   const int t_dA = (int)((const char *)p.dA2 - (const char *)p.dtv);
   const rsrc_t rf = make_rsrc(p.Cblk);
   const int f_cb = (int)((const char *)p.CBblk - (const char *)p.Cblk), f_bt = (int)((const char *)p.Btblk - (const char *)p.Cblk);
-  const int srow = min(tid >> 3, (Q >> 3) - 1) * 8, spb = tid & 7, slb8 = tid >> 3;
+  const int srow = min(tid >> 3, (Q >> 3) - 1) * 8, spb = tid & 7;
   const int v_raw = srow * xrow_b + spb * 8;                       // x for staging: rows srow.., 4 channels
   const int v_row = (lane >> 2) * xrow_b + (lane & 3) * 16;        // row-major passes: row lane / 4, 8 channels
   const int v_t = min(tid, Q - 1) * 4;
@@ -420,7 +478,7 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
       // weight of a step towards the end of its block of 32: the running sum there is in lane | 31
       const float w_t = dt_t * exp2_hw(fminf(__shfl(dA_t, lane | 31, WAVE) - dA_t, 0.0f));
       dAs[tid] = dA_t;
-      dts[tid] = dt_t;
+      dqs[tid] = log2_hw(dt_t) - dA_t;     // dt = 0: -inf, a weight of zero
       wss[tid] = w_t;
       wave_lds_sync();                     // the eight weights this thread needs come from its own wave
       const float4 wa = *reinterpret_cast<const float4 *>(wss + slb8 * 8), wb = *reinterpret_cast<const float4 *>(wss + slb8 * 8 + 4);
@@ -490,9 +548,9 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     // ---- the two row blocks.  Pair q of the stream lives in (f0, f1) if q is even, in (f2, f3) if odd:
     // the diagonal block of the first row block is pair lbF, that of the second pair NLB.
     if (yact) {
-      if (lbF & 1) half_row_block<DMODE == 1>(accF, f2, f3, f0, f1, lbF, 0, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
-      else half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
-      half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dts, Q, qmask, m, g2, dhead);
+      if (lbF & 1) half_row_block<DMODE == 1>(accF, f2, f3, f0, f1, lbF, 0, st, xw, xr, dAs, dqs, Q, qmask, m, g2, dhead);
+      else half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dqs, Q, qmask, m, g2, dhead);
+      half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dqs, Q, qmask, m, g2, dhead);
       if constexpr (DMODE == 2) {
         half_skip_term(accF, lbF, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
         half_skip_term(accS, lbS, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
@@ -702,31 +760,25 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   unsigned char *ws = reinterpret_cast<unsigned char *>(a->workspace);
 
-  SsdCumsumParams cp{};
+  const size_t bcg = (size_t)d.batch * d.nchunks * d.groups;
+  const int NLB = d.chunk >> 5, KS = d.chunk >> 4, KN = d.nstate >> 4, NT = d.nstate >> 5;
+  SsdPrepParams pp{};
+  SsdCumsumParams &cp = pp.cs;
   cp.dt = a->dt; cp.A = a->A; cp.bias = a->dt_bias;
   cp.dA_cs = nullptr;
   cp.dt_out = reinterpret_cast<float *>(ws + lay.dt_out);
   cp.d = d; cp.dt_dtype = a->dt_dtype; cp.softplus = a->dt_softplus ? 1 : 0; cp.dt_min = a->dt_min; cp.dt_max = a->dt_max;
-  const size_t units = (size_t)d.batch * d.nchunks * ((d.heads + PD_HEADS - 1) / PD_HEADS);
-  hipLaunchKernelGGL(ssd_fused_prep_dt_kernel, dim3((unsigned)units), dim3(256), 0, s, cp,
-                     reinterpret_cast<float *>(ws + lay.dA2));
-  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(prep dt)");
-
-  SsdBmmParams bp{};
-  bp.a = a->Cm; bp.b = a->Bm; bp.seq_idx = nullptr; bp.out = ws + lay.CBblk;
-  bp.batch = d.batch; bp.len = d.len; bp.groups = d.groups; bp.kdim = d.nstate; bp.chunk = d.chunk; bp.nchunks = d.nchunks;
-  bp.in_dtype = SSM_BF16; bp.out_dtype = SSM_BF16; bp.causal = 1; bp.blocked = 1;
-  SSM_REQUIRE(ssd_bmm_mfma(bp, s), SSM_ERR_BAD_SHAPE, "ssm_ssd_combined_fwd: C B^T kernel rejected the shape");
-  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(bmm)");
-
-  const size_t bcg = (size_t)d.batch * d.nchunks * d.groups;
-  const int NLB = d.chunk >> 5, KS = d.chunk >> 4, KN = d.nstate >> 4, NT = d.nstate >> 5;
+  pp.dA2 = reinterpret_cast<float *>(ws + lay.dA2);
+  pp.Cm = reinterpret_cast<const __bf16 *>(a->Cm); pp.Bm = reinterpret_cast<const __bf16 *>(a->Bm);
   __bf16 *Cblk = reinterpret_cast<__bf16 *>(ws + lay.Cblk), *Btblk = reinterpret_cast<__bf16 *>(ws + lay.Btblk);
-  const size_t frags = bcg * NLB * KN + bcg * KS * NT;
-  hipLaunchKernelGGL(ssd_fused_pack_kernel, dim3((unsigned)((frags + 3) / 4)), dim3(256), 0, s,
-                     reinterpret_cast<const __bf16 *>(a->Cm), reinterpret_cast<const __bf16 *>(a->Bm), Cblk, Btblk,
-                     d.batch, d.len, d.groups, d.nstate, d.chunk);
-  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(pack)");
+  pp.Cblk = Cblk; pp.Btblk = Btblk; pp.CBblk = reinterpret_cast<__bf16 *>(ws + lay.CBblk);
+  const size_t n_dt = (size_t)d.batch * d.nchunks * ((d.heads + PD_HEADS - 1) / PD_HEADS);
+  const size_t n_pack = (bcg * NLB * KN + bcg * KS * NT + 3) / 4;
+  const size_t n_cb = (bcg * (NLB * (NLB + 1) / 2) + 3) / 4;
+  SSM_REQUIRE(n_dt + n_pack + n_cb < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_combined_fwd: too many workgroups");
+  pp.n_dt = (unsigned)n_dt; pp.n_pack = (unsigned)n_pack;
+  hipLaunchKernelGGL(ssd_fused_prep_kernel, dim3((unsigned)(n_dt + n_pack + n_cb)), dim3(256), 0, s, pp);
+  SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(prep)");
 
   SsdFusedParams fp{};
   fp.x = reinterpret_cast<const __bf16 *>(a->x); fp.z = reinterpret_cast<const __bf16 *>(a->z);

@@ -81,28 +81,6 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_bmm_mfma_kernel(const SsdBmmPa
     const __bf16 *brow = reinterpret_cast<const __bf16 *>(p.b) + (((size_t)b * p.len + c * Q + s0 + m) * p.groups + g) * K + 8 * g2;
     for (int k0 = 0; k0 < K; k0 += 16) acc = mma(load_frag(arow + k0), load_frag(brow + k0), acc);
   }
-  if (p.blocked) {
-    // Through a wave-private LDS tile into the operand layout of later products: lane (m, g2)
-    // of fragment (l0 / 32, ks) holds CB[l0 + m][16 ks + 8 g2 .. + 7].  Blocks above the
-    // diagonal are never read and are not written.
-    __shared__ float tile[MF_WAVES][32][33];
-    if (s0 > l0) return;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) tile[wave][crow(r, g2)][m] = acc[r];
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    const size_t unit_frag = ((size_t)unit * (Q >> 5) + (l0 >> 5)) * (Q >> 4);
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      float v[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int sl = 16 * kk + 8 * g2 + j;
-        v[j] = (s0 + sl <= l0 + m) ? tile[wave][m][sl] : 0.0f;
-      }
-      *reinterpret_cast<bf16x8_t *>(reinterpret_cast<__bf16 *>(p.out) + (unit_frag + (s0 >> 4) + kk) * 512 + lane * 8) = pack8(v);
-    }
-    return;
-  }
   const int *sid = p.seq_idx ? p.seq_idx + (size_t)b * p.len + c * Q : nullptr;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -306,7 +284,6 @@ static bool mfma_shape_ok(const SsdDims &d) {
 
 bool ssd_bmm_mfma(const SsdBmmParams &p, hipStream_t s) {
   if (p.in_dtype != SSM_BF16 || p.out_dtype == SSM_F16) return false;
-  if (p.blocked && (p.out_dtype != SSM_BF16 || p.seq_idx || !p.causal)) return false;
   if (p.len % p.chunk != 0 || p.chunk % 32 != 0 || p.kdim % 16 != 0) return false;
   if (!aligned_to(p.a, 16) || !aligned_to(p.b, 16)) return false;
   const int tiles = (p.chunk + 63) / 64;
