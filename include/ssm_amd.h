@@ -326,6 +326,7 @@ typedef struct ssm_ssd_chunk_state_args {
   size_t workspace_bytes;
   ssm_ssd_dims dims;
   int32_t x_dtype, b_dtype, states_dtype, force_generic;
+  const int32_t *seq_idx;   /* (B,L) or NULL: steps of another sequence than the chunk's last step add nothing */
 } ssm_ssd_chunk_state_args;
 size_t ssm_ssd_chunk_state_workspace_bytes(const ssm_ssd_dims *dims);
 int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *args, void *hip_stream);
@@ -338,6 +339,9 @@ typedef struct ssm_ssd_state_passing_args {
   float *final_states;       /* (B,H,dim) */
   int32_t batch, nchunks, heads, dim;
   int32_t states_dtype;
+  int32_t seqlen, chunk;     /* only read with seq_idx */
+  const int32_t *seq_idx;    /* (B,L) or NULL: the carried state is dropped where the sequence id of a chunk's
+                                last step differs from that of the chunk before (the initial state belongs to id 0) */
 } ssm_ssd_state_passing_args;
 int ssm_ssd_state_passing(const ssm_ssd_state_passing_args *args, void *hip_stream);
 
@@ -352,8 +356,32 @@ typedef struct ssm_ssd_chunk_scan_args {
   void *y;                  /* (B,L,H,P) x dtype */
   ssm_ssd_dims dims;
   int32_t x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype, d_per_p, force_generic;
+  const int32_t *seq_idx;   /* (B,L) or NULL: the entering state only reaches steps whose sequence id equals that of
+                               the last step of the chunk before (id 0 for the first chunk); CB must have been
+                               formed with the same seq_idx */
 } ssm_ssd_chunk_scan_args;
 int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
+
+/* State at the last step of each sequence of a packed batch row (batch = 1): sequence i covers steps
+ * cu_seqlens[i] .. cu_seqlens[i+1]-1.  Takes the entering states of the chunks (formed with seq_idx, or from
+ * anywhere if every sequence starts on a chunk boundary) and adds the steps of the last chunk that belong to the
+ * sequence.  The entering state of the first chunk (the row's initial state) counts for the sequence that starts
+ * at step 0.  Replaces the upstream routine the reference's vectors were made with
+ * (`chunk_state_varlen`, reached through `mamba_chunk_scan_combined(..., cu_seqlens=, return_varlen_states=True)`
+ * at /root/reference/scripts/refresh_mamba_goldens.py:618-632; vectors `ssd_combined.combined_varlen`). */
+typedef struct ssm_ssd_chunk_state_varlen_args {
+  const void *Bm;           /* (1,L,G,N) b dtype */
+  const void *x;            /* (1,L,H,P) x dtype */
+  const float *dt;          /* (1,H,nc,Q) */
+  const float *dA_cumsum;   /* (1,H,nc,Q) */
+  const void *chunk_states; /* (1,nc,H,P,N) states dtype: state entering each chunk */
+  const int32_t *cu_seqlens;/* (nseq+1) on the device, increasing, first 0, last <= L */
+  float *states;            /* (nseq,H,P,N) */
+  ssm_ssd_dims dims;        /* batch must be 1 */
+  int32_t nseq;
+  int32_t x_dtype, b_dtype, states_dtype;
+} ssm_ssd_chunk_state_varlen_args;
+int ssm_ssd_chunk_state_varlen(const ssm_ssd_chunk_state_varlen_args *args, void *hip_stream);
 
 /* The whole forward (chunk_cumsum, bmm_chunk, chunk_state, state_passing,
  * chunk_scan; combined call recorded at scripts/refresh_mamba_goldens.py:591-604)

@@ -51,9 +51,9 @@ def prepare_dt(dt, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf"))
     if dt_softplus:
         v = F.softplus(v)
     lo, hi = dt_limit
-    if lo != 0.0 or hi != float("inf"):
-        v = v.clamp(min=lo, max=hi)
-    return v
+    # always applied, also with the default limits: a negative raw step (no softplus) becomes 0,
+    # as the vectors of `ssd_combined.combined_varlen` show (y = 0 at their first token)
+    return v.clamp(min=lo, max=hi)
 
 
 def ssd_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=False,
@@ -141,8 +141,18 @@ def _seg_exp(delta, clamp_decay):
     return torch.exp(delta.clamp(max=0.0)) if clamp_decay else torch.exp(delta)
 
 
-def chunk_state(B, x, dt_c, dA_cumsum, clamp_decay=True, acc=torch.float64):
-    """-> states (B,nc,H,P,N): contribution of each chunk to the state at its end."""
+def _chunk_last_ids(seq_idx, Q):
+    """Sequence id of the last real step of every chunk: (B, nc)."""
+    L = seq_idx.shape[1]
+    nc = (L + Q - 1) // Q
+    last = torch.tensor([min((c + 1) * Q, L) - 1 for c in range(nc)])
+    return seq_idx.to(torch.long)[:, last]
+
+
+def chunk_state(B, x, dt_c, dA_cumsum, clamp_decay=True, acc=torch.float64, seq_idx=None):
+    """-> states (B,nc,H,P,N): contribution of each chunk to the state at its end.
+    With ``seq_idx`` (B,L) only the steps that share the sequence id of the chunk's
+    last step contribute."""
     batch, H, nc, Q = dt_c.shape
     G, N = B.shape[2], B.shape[3]
     per = H // G
@@ -150,28 +160,43 @@ def chunk_state(B, x, dt_c, dA_cumsum, clamp_decay=True, acc=torch.float64):
     Bh = _pad_to_chunks(B.to(acc), Q).view(batch, nc, Q, G, N).repeat_interleave(per, dim=3)
     dA = dA_cumsum.to(acc)
     w = _seg_exp(dA[..., -1:] - dA, clamp_decay) * dt_c.to(acc)      # (B,H,nc,Q)
+    if seq_idx is not None:
+        ids = _pad_to_chunks(seq_idx.to(torch.long) + 1, Q).view(batch, nc, Q) - 1      # padding: id -1
+        same = ids == _chunk_last_ids(seq_idx, Q)[:, :, None]                           # (B,nc,Q)
+        w = w * same[:, None].to(acc)
     return torch.einsum("bclhn,bhcl,bclhp->bchpn", Bh, w, xx)
 
 
-def state_passing(states, dA_chunk_last, initial_states=None, acc=torch.float64):
+def state_passing(states, dA_chunk_last, initial_states=None, acc=torch.float64, seq_idx=None, chunk_size=None):
     """states (B,nc,H,...); dA_chunk_last (B,H,nc).  Returns ``(entering, final)``
-    where ``entering[:,c]`` is the state at the START of chunk c."""
+    where ``entering[:,c]`` is the state at the START of chunk c.  With ``seq_idx`` the
+    carried state is dropped where the id of a chunk's last step differs from that of
+    the chunk before; the initial state belongs to id 0."""
     st = states.to(acc)
     batch, nc, H = st.shape[:3]
     cur = (initial_states.to(acc).reshape(st[:, 0].shape) if initial_states is not None
            else torch.zeros_like(st[:, 0]))
     outs = []
     extra = (1,) * (st.dim() - 3)
+    last_ids = _chunk_last_ids(seq_idx, int(chunk_size)) if seq_idx is not None else None
+    prev_id = torch.zeros(batch, dtype=torch.long)
     for c in range(nc):
         outs.append(cur)
         g = torch.exp(dA_chunk_last.to(acc)[:, :, c]).view(batch, H, *extra)
+        if last_ids is not None:
+            keep = (last_ids[:, c] == prev_id).to(acc).view(batch, 1, *extra)
+            g = g * keep
+            prev_id = last_ids[:, c]
         cur = g * cur + st[:, c]
     return torch.stack(outs, dim=1), cur
 
 
 def chunk_scan(B, C, x, dt_c, dA_cumsum, prev_states, D=None, z=None,
-               clamp_decay=True, acc=torch.float64):
-    """-> y (B,L,H,P) from entering states ``prev_states`` (B,nc,H,P,N)."""
+               clamp_decay=True, acc=torch.float64, seq_idx=None):
+    """-> y (B,L,H,P) from entering states ``prev_states`` (B,nc,H,P,N).  With
+    ``seq_idx`` the entering state only reaches steps whose id equals that of the last
+    step of the chunk before (0 for the first chunk) and products across sequences
+    inside a chunk are dropped."""
     batch, H, nc, Q = dt_c.shape
     L = x.shape[1]
     G, N = B.shape[2], B.shape[3]
@@ -184,12 +209,20 @@ def chunk_scan(B, C, x, dt_c, dA_cumsum, prev_states, D=None, z=None,
     # inter-chunk: exp(dA_cs[l]) * C_l . H_c
     y_off = torch.einsum("bclhn,bchpn->bclhp", Ch, prev_states.to(acc)) \
         * torch.exp(dA).permute(0, 2, 3, 1)[..., None]
+    ids = None
+    if seq_idx is not None:
+        ids = _pad_to_chunks(seq_idx.to(torch.long) + 1, Q).view(batch, nc, Q) - 1
+        last_ids = _chunk_last_ids(seq_idx, Q)
+        prev_ids = torch.cat([torch.zeros(batch, 1, dtype=torch.long), last_ids[:, :-1]], dim=1)   # (B,nc)
+        y_off = y_off * (ids == prev_ids[:, :, None]).to(acc)[..., None, None]
     # intra-chunk: sum_{s<=l} CB[l,s] * exp(dA_cs[l]-dA_cs[s]) * dt_s * x_s
     CB = torch.einsum("bclhn,bcshn->bchls", Ch, Bh)
     seg = dA.permute(0, 2, 1, 3)                                     # (B,nc,H,Q)
     decay = _seg_exp(seg[..., :, None] - seg[..., None, :], clamp_decay)
     mask = torch.tril(torch.ones(Q, Q, dtype=torch.bool))
     M = torch.where(mask, CB * decay, torch.zeros((), dtype=acc))
+    if ids is not None:
+        M = M * (ids[:, :, :, None] == ids[:, :, None, :]).to(acc)[:, :, None]
     M = M * dt_c.to(acc).permute(0, 2, 1, 3)[..., None, :]
     y_diag = torch.einsum("bchls,bcshp->bclhp", M, xx)
     y = y_off + y_diag
@@ -202,13 +235,49 @@ def chunk_scan(B, C, x, dt_c, dA_cumsum, prev_states, D=None, z=None,
     return y
 
 
+def chunk_state_varlen(B, x, dt_c, dA_cumsum, cu_seqlens, chunk_states, clamp_decay=True, acc=torch.float64):
+    """State at the last step of every sequence of a packed batch row (batch 1):
+    -> (nseq,H,P,N).  ``chunk_states`` (1,nc,H,P,N) are the states entering the chunks;
+    the one entering the chunk of a sequence's last step counts only if the sequence
+    began before that chunk (or at step 0: the row's initial state belongs to the first
+    sequence).  Follows the routine behind
+    ``mamba_chunk_scan_combined(..., cu_seqlens=, return_varlen_states=True)``
+    (/root/reference/scripts/refresh_mamba_goldens.py:618-632)."""
+    _, H, nc, Q = dt_c.shape
+    G, N = B.shape[2], B.shape[3]
+    per = H // G
+    L = x.shape[1]
+    xx = x.to(acc)[0]                                  # (L,H,P)
+    Bh = B.to(acc)[0].repeat_interleave(per, dim=1)    # (L,H,N)
+    dA = dA_cumsum.to(acc)[0]                          # (H,nc,Q)
+    dtc = dt_c.to(acc)[0]
+    cu = [int(v) for v in cu_seqlens]
+    outs = []
+    for i in range(len(cu) - 1):
+        start, end = cu[i], min(cu[i + 1], L)
+        st = torch.zeros(H, xx.shape[2], N, dtype=acc)
+        if end > start:
+            c = (end - 1) // Q
+            last = dA[:, c, end - 1 - c * Q]           # (H,)
+            if start < c * Q or start == 0:            # start == 0: the row's initial state belongs to the first sequence
+                st = chunk_states.to(acc)[0, c] * torch.exp(last)[:, None, None]
+            for t in range(max(start, c * Q), end):
+                w = _seg_exp(last - dA[:, c, t - c * Q], clamp_decay) * dtc[:, c, t - c * Q]
+                st = st + w[:, None, None] * xx[t][:, :, None] * Bh[t][:, None, :]
+        outs.append(st)
+    return torch.stack(outs, dim=0)
+
+
 def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
                  initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
-                 clamp_decay=True, acc=torch.float64):
+                 clamp_decay=True, acc=torch.float64, seq_idx=None, cu_seqlens=None):
     """cumsum -> chunk_state -> state_passing -> chunk_scan; returns
-    ``(y, final_states (B,H,P,N))``."""
+    ``(y, final_states (B,H,P,N))``, and with ``cu_seqlens`` also the state at the end
+    of every packed sequence."""
     dA_cs, dt_c = chunk_cumsum(dt, A, chunk_size, dt_bias, dt_softplus, dt_limit, acc)
-    st = chunk_state(B, x, dt_c, dA_cs, clamp_decay, acc)
-    entering, final = state_passing(st, dA_cs[..., -1], initial_states, acc)
-    y = chunk_scan(B, C, x, dt_c, dA_cs, entering, D=D, z=z, clamp_decay=clamp_decay, acc=acc)
+    st = chunk_state(B, x, dt_c, dA_cs, clamp_decay, acc, seq_idx=seq_idx)
+    entering, final = state_passing(st, dA_cs[..., -1], initial_states, acc, seq_idx=seq_idx, chunk_size=chunk_size)
+    y = chunk_scan(B, C, x, dt_c, dA_cs, entering, D=D, z=z, clamp_decay=clamp_decay, acc=acc, seq_idx=seq_idx)
+    if cu_seqlens is not None:
+        return y, final, chunk_state_varlen(B, x, dt_c, dA_cs, cu_seqlens, entering, clamp_decay, acc)
     return y, final

@@ -133,20 +133,27 @@ class SsdBmmArgs(C.Structure):
 class SsdChunkStateArgs(C.Structure):
     _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("states", _vp),
                 ("workspace", _vp), ("workspace_bytes", C.c_size_t), ("dims", SsdDims),
-                ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("force_generic", _i32)]
+                ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("force_generic", _i32),
+                ("seq_idx", _vp)]
 
 
 class SsdStatePassingArgs(C.Structure):
     _fields_ = [("states", _vp), ("dA_chunk_last", _vp), ("initial_states", _vp), ("states_out", _vp),
                 ("final_states", _vp), ("batch", _i32), ("nchunks", _i32), ("heads", _i32), ("dim", _i32),
-                ("states_dtype", _i32)]
+                ("states_dtype", _i32), ("seqlen", _i32), ("chunk", _i32), ("seq_idx", _vp)]
 
 
 class SsdChunkScanArgs(C.Structure):
     _fields_ = [("CB", _vp), ("Cm", _vp), ("x", _vp), ("z", _vp), ("prev_states", _vp), ("dt", _vp),
                 ("dA_cumsum", _vp), ("Dskip", _vp), ("y", _vp), ("dims", SsdDims),
                 ("x_dtype", _i32), ("c_dtype", _i32), ("cb_dtype", _i32), ("states_dtype", _i32),
-                ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32)]
+                ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32), ("seq_idx", _vp)]
+
+
+class SsdChunkStateVarlenArgs(C.Structure):
+    _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("chunk_states", _vp),
+                ("cu_seqlens", _vp), ("states", _vp), ("dims", SsdDims), ("nseq", _i32),
+                ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32)]
 
 
 class SsdCombinedArgs(C.Structure):
@@ -211,6 +218,7 @@ ENTRY_POINTS = {
     "ssm_ssd_chunk_state": SsdChunkStateArgs,
     "ssm_ssd_state_passing": SsdStatePassingArgs,
     "ssm_ssd_chunk_scan": SsdChunkScanArgs,
+    "ssm_ssd_chunk_state_varlen": SsdChunkStateVarlenArgs,
     "ssm_ssd_combined_fwd": SsdCombinedArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,

@@ -89,10 +89,13 @@ __global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_state_kernel(const SsdS
   const int g = h / (d.heads / d.groups);
   const size_t cs = (((size_t)b * d.heads + h) * d.nchunks + c) * d.chunk;
   const float last = p.dA_cs[cs + d.chunk - 1];
+  const int *sid = p.seq_idx ? p.seq_idx + (size_t)b * d.len : nullptr;
+  const int sid_last = sid ? sid[min((c + 1) * d.chunk, d.len) - 1] : 0;
   float acc = 0.0f;
   for (int l = 0; l < d.chunk; ++l) {
     const int t = c * d.chunk + l;
     if (t >= d.len) break;
+    if (sid && sid[t] != sid_last) continue;
     const float w = decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
     const float bv = load_as_f32(p.Bm, p.b_dtype, (((size_t)b * d.len + t) * d.groups + g) * d.nstate + n);
     const float xv = load_as_f32(p.x, p.x_dtype, (((size_t)b * d.len + t) * d.heads + h) * d.hdim + pp);
@@ -110,11 +113,18 @@ __global__ __launch_bounds__(SSD_THREADS) void ssd_state_passing_kernel(const Ss
   const int h = (int)((gid / p.dim) % p.heads);
   const int b = (int)(gid / ((size_t)p.dim * p.heads));
   float cur = p.init ? p.init[gid] : 0.0f;
+  int sid_prev = 0;
   for (int c = 0; c < p.nchunks; ++c) {
     const size_t at = (((size_t)b * p.nchunks + c) * p.heads + h) * p.dim + i;
     const float contrib = load_as_f32(p.states, p.states_dtype, at);
     store_any(p.out, p.states_dtype, at, cur);
-    cur = __builtin_fmaf(exp2_hw(p.dA_last[((size_t)b * p.heads + h) * p.nchunks + c] * LOG2E), cur, contrib);
+    float scale = exp2_hw(p.dA_last[((size_t)b * p.heads + h) * p.nchunks + c] * LOG2E);
+    if (p.seq_idx) {
+      const int sid_new = p.seq_idx[(size_t)b * p.len + min((c + 1) * p.chunk, p.len) - 1];
+      if (sid_new != sid_prev) scale = 0.0f;
+      sid_prev = sid_new;
+    }
+    cur = __builtin_fmaf(scale, cur, contrib);
   }
   p.final_states[gid] = cur;
 }
@@ -140,6 +150,11 @@ __global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_scan_kernel(const SsdSc
   for (int n = 0; n < d.nstate; ++n)
     acc = __builtin_fmaf(load_as_f32(p.Cm, p.c_dtype, crow + n), load_as_f32(p.prev, p.states_dtype, srow + n), acc);
   acc *= exp2_hw(dal * LOG2E);
+  if (p.seq_idx) {
+    const int *sid = p.seq_idx + (size_t)b * d.len;
+    const int sid_prev = c > 0 ? sid[c * d.chunk - 1] : 0;
+    if (sid[t] != sid_prev) acc = 0.0f;
+  }
   // within the chunk
   const size_t cbrow = ((((size_t)b * d.nchunks + c) * d.groups + g) * d.chunk + l) * d.chunk;
   for (int s = 0; s <= l; ++s) {
@@ -151,6 +166,50 @@ __global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_scan_kernel(const SsdSc
   if (p.Dk) acc = __builtin_fmaf(p.Dk[p.d_per_p ? (size_t)h * d.hdim + pp : (size_t)h], xl, acc);
   if (p.z) acc *= silu_f32(load_as_f32(p.z, p.z_dtype, gid));
   store_any(p.y, p.x_dtype, gid, acc);
+}
+
+struct SsdVarlenParams {
+  const void *Bm, *x, *chunk_states;
+  const float *dt, *dA_cs;
+  const int *cu_seqlens;
+  float *states;
+  SsdDims d;
+  int nseq;
+  int x_dtype, b_dtype, states_dtype;
+};
+
+// One thread per (sequence, h, p, n): the state at the sequence's last step is the state entering the
+// chunk of that step, decayed, if the sequence began before that chunk (or at step 0), plus the steps of
+// the chunk that belong to the sequence.
+__global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_state_varlen_kernel(const SsdVarlenParams p) {
+  const SsdDims &d = p.d;
+  const size_t total = (size_t)p.nseq * d.heads * d.hdim * d.nstate;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int n = (int)(gid % d.nstate);
+  const int pp = (int)((gid / d.nstate) % d.hdim);
+  const int h = (int)((gid / ((size_t)d.nstate * d.hdim)) % d.heads);
+  const int q = (int)(gid / ((size_t)d.nstate * d.hdim * d.heads));
+  const int g = h / (d.heads / d.groups);
+  const int start = p.cu_seqlens[q], end = min(p.cu_seqlens[q + 1], d.len);
+  float acc = 0.0f;
+  if (end > start && start >= 0) {
+    const int c = (end - 1) / d.chunk;
+    const size_t cs = ((size_t)h * d.nchunks + c) * d.chunk;
+    const float last = p.dA_cs[cs + (end - 1 - c * d.chunk)];
+    if (start < c * d.chunk || start == 0) {   // start == 0: the row's initial state belongs to the first sequence
+      const size_t at = (((size_t)c * d.heads + h) * d.hdim + pp) * d.nstate + n;
+      acc = load_as_f32(p.chunk_states, p.states_dtype, at) * exp2_hw(last * LOG2E);
+    }
+    for (int t = max(start, c * d.chunk); t < end; ++t) {
+      const int l = t - c * d.chunk;
+      const float w = decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
+      const float bv = load_as_f32(p.Bm, p.b_dtype, ((size_t)t * d.groups + g) * d.nstate + n);
+      const float xv = load_as_f32(p.x, p.x_dtype, ((size_t)t * d.heads + h) * d.hdim + pp);
+      acc = __builtin_fmaf(bv * w, xv, acc);
+    }
+  }
+  p.states[gid] = acc;
 }
 
 static int dims_check(const char *who, const ssm_ssd_dims &s, SsdDims &d) {
@@ -239,8 +298,9 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   p.Bm = a->Bm; p.x = a->x; p.dt = a->dt; p.dA_cs = a->dA_cumsum; p.states = a->states;
   p.scratch = a->workspace; p.scratch_bytes = a->workspace_bytes;
   p.x_dtype = a->x_dtype; p.b_dtype = a->b_dtype; p.states_dtype = a->states_dtype;
+  p.seq_idx = a->seq_idx;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  if (!a->force_generic && ssd_chunk_state_mfma(p, s)) {
+  if (!a->force_generic && !a->seq_idx && ssd_chunk_state_mfma(p, s)) {
     g_mfma_launches |= 2;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
     return SSM_OK;
@@ -263,6 +323,11 @@ extern "C" int ssm_ssd_state_passing(const ssm_ssd_state_passing_args *a, void *
   p.states = a->states; p.dA_last = a->dA_chunk_last; p.init = a->initial_states; p.out = a->states_out;
   p.final_states = a->final_states;
   p.batch = a->batch; p.nchunks = a->nchunks; p.heads = a->heads; p.dim = a->dim; p.states_dtype = a->states_dtype;
+  p.seq_idx = a->seq_idx; p.len = a->seqlen; p.chunk = a->chunk;
+  if (a->seq_idx)
+    SSM_REQUIRE(a->chunk > 0 && a->seqlen > 0 && (a->seqlen + a->chunk - 1) / a->chunk == a->nchunks, SSM_ERR_BAD_SHAPE,
+                "ssm_ssd_state_passing: with seq_idx, seqlen=%d and chunk=%d must give nchunks=%d", a->seqlen, a->chunk,
+                a->nchunks);
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   hipLaunchKernelGGL(ssd_state_passing_kernel, dim3(grid_for((size_t)p.batch * p.heads * p.dim)), dim3(SSD_THREADS),
                      0, s, p);
@@ -284,8 +349,9 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   p.Dk = a->Dskip; p.y = a->y;
   p.x_dtype = a->x_dtype; p.c_dtype = a->c_dtype; p.cb_dtype = a->cb_dtype; p.states_dtype = a->states_dtype;
   p.z_dtype = a->z_dtype; p.d_per_p = a->d_per_p ? 1 : 0;
+  p.seq_idx = a->seq_idx;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
+  if (!a->force_generic && !a->seq_idx && ssd_chunk_scan_mfma(p, s)) {
     g_mfma_launches |= 4;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
     return SSM_OK;
@@ -293,5 +359,29 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   const size_t total = (size_t)p.d.batch * p.d.len * p.d.heads * p.d.hdim;
   hipLaunchKernelGGL(ssd_chunk_scan_kernel, dim3(grid_for(total)), dim3(SSD_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_chunk_state_varlen(const ssm_ssd_chunk_state_varlen_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a && a->Bm && a->x && a->dt && a->dA_cumsum && a->chunk_states && a->cu_seqlens && a->states,
+              SSM_ERR_NULL_POINTER,
+              "ssm_ssd_chunk_state_varlen: Bm, x, dt, dA_cumsum, chunk_states, cu_seqlens and states are required");
+  SsdVarlenParams p{};
+  int rc = dims_check("ssm_ssd_chunk_state_varlen", a->dims, p.d);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(p.d.batch == 1, SSM_ERR_BAD_SHAPE, "ssm_ssd_chunk_state_varlen: packed sequences need batch=1 (got %d)",
+              p.d.batch);
+  SSM_REQUIRE(a->nseq > 0, SSM_ERR_BAD_SHAPE, "ssm_ssd_chunk_state_varlen: nseq=%d", a->nseq);
+  SSM_REQUIRE(valid_dtype(a->x_dtype) && valid_dtype(a->b_dtype) && valid_dtype(a->states_dtype), SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_chunk_state_varlen: unsupported dtype");
+  p.Bm = a->Bm; p.x = a->x; p.chunk_states = a->chunk_states; p.dt = a->dt; p.dA_cs = a->dA_cumsum;
+  p.cu_seqlens = a->cu_seqlens; p.states = a->states; p.nseq = a->nseq;
+  p.x_dtype = a->x_dtype; p.b_dtype = a->b_dtype; p.states_dtype = a->states_dtype;
+  const size_t total = (size_t)p.nseq * p.d.heads * p.d.hdim * p.d.nstate;
+  SSM_REQUIRE(total < ((size_t)1 << 40), SSM_ERR_TOO_LARGE, "ssm_ssd_chunk_state_varlen: tensor too large");
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(ssd_chunk_state_varlen_kernel, dim3(grid_for(total)), dim3(SSD_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_chunk_state_varlen");
   return SSM_OK;
 }

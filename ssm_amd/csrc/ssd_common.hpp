@@ -41,6 +41,7 @@ struct SsdStateParams {
   size_t scratch_bytes;
   SsdDims d;
   int x_dtype, b_dtype, states_dtype;
+  const int *seq_idx;         // (B, L) or null
 };
 
 struct SsdPassParams {
@@ -51,6 +52,8 @@ struct SsdPassParams {
   float *final_states;        // (B, H, dim)
   int batch, nchunks, heads, dim;
   int states_dtype;
+  int len, chunk;             // only read with seq_idx
+  const int *seq_idx;         // (B, L) or null
 };
 
 struct SsdScanParams {
@@ -60,6 +63,7 @@ struct SsdScanParams {
   SsdDims d;
   int x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype;
   int d_per_p;                // D is (H, P) instead of (H,)
+  const int *seq_idx;         // (B, L) or null
 };
 
 __device__ __forceinline__ void store_any(void *p, int dtype, size_t i, float v) {

@@ -121,7 +121,16 @@ def _ssd_shapes(x, B):
     return batch, seqlen, heads, hdim, groups, nstate
 
 
-def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=False):
+def _seq_idx_i32(seq_idx, batch, seqlen):
+    """``seq_idx (B, L)`` as a contiguous int32 tensor (``None`` passes through)."""
+    if seq_idx is None:
+        return None
+    _need(tuple(seq_idx.shape) == (batch, seqlen), "seq_idx must have shape (B, L).")
+    _need(not seq_idx.dtype.is_floating_point, "seq_idx must hold integers.")
+    return seq_idx.to(torch.int32).contiguous()
+
+
+def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=False, seq_idx=None):
     """Contribution of each chunk to the state at its end.
 
     Args:
@@ -130,6 +139,8 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
         dt: ``(B, H, nc, Q)`` float32 (``dt_out`` of :func:`chunk_cumsum`).
         dA_cumsum: ``(B, H, nc, Q)`` float32.
         states_dtype: dtype of the result.
+        seq_idx: Optional ``(B, L)`` int sequence ids of a packed batch: steps of another
+            sequence than the chunk's last step add nothing.
 
     Returns:
         ``states (B, nc, H, P, N)``.
@@ -139,11 +150,12 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
           "dt and dA_cumsum must have shape (B, H, nc, Q).")
     nc, Q = int(dt.shape[2]), int(dt.shape[3])
     _need(nc == (seqlen + Q - 1) // Q, "dt has the wrong number of chunks for this sequence length.")
-    dev = K.require_gpu(B, x, dt, dA_cumsum)
+    dev = K.require_gpu(B, x, dt, dA_cumsum, seq_idx)
     xc, Bc = K.cast_c(x, x.dtype), K.cast_c(B, B.dtype)
     K.check_float("x", xc)
     K.check_float("B", Bc)
     dtf, daf = K.as_f32_vec(dt), K.as_f32_vec(dA_cumsum)
+    si = _seq_idx_i32(seq_idx, batch, seqlen)
     states = torch.empty(batch, nc, heads, hdim, nstate, dtype=states_dtype, device=dev)
     dims = _dims(batch, seqlen, heads, hdim, groups, nstate, Q)
     import ctypes
@@ -154,18 +166,22 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
         workspace=_lib.ptr(ws), workspace_bytes=nbytes,
         dims=dims, x_dtype=_lib.dtype_enum(xc.dtype),
         b_dtype=_lib.dtype_enum(Bc.dtype), states_dtype=_lib.dtype_enum(states_dtype),
-        force_generic=int(bool(force_generic)))
+        force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si))
     _lib.call("ssm_ssd_chunk_state", args, dev)
     return states
 
 
-def state_passing(states, dA_chunk_cumsum, initial_states=None):
+def state_passing(states, dA_chunk_cumsum, initial_states=None, seq_idx=None, chunk_size=None):
     """Carry states across chunks: ``H_{c+1} = exp(dA_c) H_c + states_c``.
 
     Args:
         states: ``(B, nc, H, ...)`` per-chunk contributions (any trailing shape).
         dA_chunk_cumsum: ``(B, H, nc)``: ``dA_cumsum[..., -1]``.
         initial_states: Optional ``(B, H, ...)``.
+        seq_idx: Optional ``(B, L)`` int sequence ids: the carried state is dropped where the
+            id of a chunk's last step differs from that of the chunk before (the initial
+            state belongs to id 0).  Needs ``chunk_size``.
+        chunk_size: ``Q`` (only with ``seq_idx``).
 
     Returns:
         ``(states_passed, final_states)``: the state entering each chunk (shape and dtype
@@ -178,7 +194,15 @@ def state_passing(states, dA_chunk_cumsum, initial_states=None):
     for s_ in trailing:
         dim *= s_
     _need(tuple(dA_chunk_cumsum.shape) == (batch, heads, nc), "dA_chunk_cumsum must have shape (B, H, nc).")
-    dev = K.require_gpu(states, dA_chunk_cumsum, initial_states)
+    dev = K.require_gpu(states, dA_chunk_cumsum, initial_states, seq_idx)
+    si, seqlen, Q = None, 0, 0
+    if seq_idx is not None:
+        _need(chunk_size is not None and int(chunk_size) > 0, "seq_idx needs chunk_size.")
+        Q = int(chunk_size)
+        _need(seq_idx.ndim == 2 and seq_idx.shape[0] == batch and (int(seq_idx.shape[1]) + Q - 1) // Q == nc,
+              "seq_idx must have shape (B, L) with ceil(L / chunk_size) == nc.")
+        seqlen = int(seq_idx.shape[1])
+        si = _seq_idx_i32(seq_idx, batch, seqlen)
     sc = K.cast_c(states, states.dtype)
     K.check_float("states", sc)
     daf = K.as_f32_vec(dA_chunk_cumsum)
@@ -191,12 +215,12 @@ def state_passing(states, dA_chunk_cumsum, initial_states=None):
     args = _lib.SsdStatePassingArgs(
         states=_lib.ptr(sc), dA_chunk_last=_lib.ptr(daf), initial_states=_lib.ptr(init),
         states_out=_lib.ptr(out), final_states=_lib.ptr(final), batch=batch, nchunks=nc, heads=heads, dim=dim,
-        states_dtype=_lib.dtype_enum(sc.dtype))
+        states_dtype=_lib.dtype_enum(sc.dtype), seqlen=seqlen, chunk=Q, seq_idx=_lib.ptr(si))
     _lib.call("ssm_ssd_state_passing", args, dev)
     return out, final
 
 
-def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False):
+def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False, seq_idx=None):
     """Outputs of every chunk from the state entering it.
 
     Args:
@@ -206,7 +230,10 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         prev_states: ``(B, nc, H, P, N)`` state entering each chunk.
         D: Optional skip ``(H,)`` or ``(H, P)``.
         z: Optional gate ``(B, L, H, P)``.
-        CB: Optional precomputed ``bmm_chunk(C, B, Q)``.
+        CB: Optional precomputed ``bmm_chunk(C, B, Q)`` (with the same ``seq_idx``).
+        seq_idx: Optional ``(B, L)`` int sequence ids: the entering state only reaches steps
+            whose id equals that of the last step of the chunk before (id 0 for the first
+            chunk), and products across sequences inside a chunk are dropped.
 
     Returns:
         ``y (B, L, H, P)`` in ``x.dtype``.
@@ -223,10 +250,11 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         _need(tuple(D.shape) in ((heads,), (heads, hdim)), "D must have shape (H,) or (H, P).")
         d_per_p = D.ndim == 2
     _need(z is None or z.shape == x.shape, "z must have the shape of x.")
-    dev = K.require_gpu(B, C, x, dt, dA_cumsum, prev_states, D, z)
+    dev = K.require_gpu(B, C, x, dt, dA_cumsum, prev_states, D, z, seq_idx)
+    si = _seq_idx_i32(seq_idx, batch, seqlen)
     if CB is None:
-        CB = bmm_chunk(C, B, Q, causal=True, output_dtype=x.dtype if x.dtype != torch.float32 else torch.float32,
-                       force_generic=force_generic)
+        CB = bmm_chunk(C, B, Q, seq_idx=si, causal=True,
+                       output_dtype=x.dtype if x.dtype != torch.float32 else torch.float32, force_generic=force_generic)
     _need(tuple(CB.shape) == (batch, nc, groups, Q, Q), "CB must have shape (B, nc, G, Q, Q).")
     xc, Cc, zc = K.cast_c(x, x.dtype), K.cast_c(C, C.dtype), (K.cast_c(z, z.dtype) if z is not None else None)
     for name, t in (("x", xc), ("C", Cc), ("z", zc), ("CB", CB), ("prev_states", prev_states)):
@@ -241,9 +269,50 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         dims=_dims(batch, seqlen, heads, hdim, groups, nstate, Q), x_dtype=_lib.dtype_enum(xc.dtype),
         c_dtype=_lib.dtype_enum(Cc.dtype), cb_dtype=_lib.dtype_enum(cb.dtype),
         states_dtype=_lib.dtype_enum(ps.dtype), z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
-        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)))
+        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si))
     _lib.call("ssm_ssd_chunk_scan", args, dev)
     return y
+
+
+def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
+    """State at the last step of every sequence of a packed batch row.
+
+    Args:
+        B: ``(1, L, G, N)``.
+        x: ``(1, L, H, P)``.
+        dt, dA_cumsum: ``(1, H, nc, Q)`` float32.
+        cu_seqlens: ``(nseq + 1,)`` ints, increasing from 0: sequence ``i`` covers steps
+            ``cu_seqlens[i] .. cu_seqlens[i+1] - 1``.
+        chunk_states: ``(1, nc, H, P, N)`` state entering each chunk (from :func:`state_passing`
+            with the matching ``seq_idx`` unless every sequence starts on a chunk boundary).
+
+    Returns:
+        ``states (nseq, H, P, N)`` float32.
+    """
+    batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
+    _need(batch == 1, "packed sequences need batch size 1.")
+    _need(dt.ndim == 4 and dt.shape == dA_cumsum.shape and dt.shape[0] == 1 and dt.shape[1] == heads,
+          "dt and dA_cumsum must have shape (1, H, nc, Q).")
+    nc, Q = int(dt.shape[2]), int(dt.shape[3])
+    _need(nc == (seqlen + Q - 1) // Q, "dt has the wrong number of chunks for this sequence length.")
+    _need(tuple(chunk_states.shape) == (1, nc, heads, hdim, nstate), "chunk_states must have shape (1, nc, H, P, N).")
+    _need(cu_seqlens.ndim == 1 and cu_seqlens.numel() >= 2 and not cu_seqlens.dtype.is_floating_point,
+          "cu_seqlens must be a 1-D integer tensor of length nseq + 1.")
+    dev = K.require_gpu(B, x, dt, dA_cumsum, cu_seqlens, chunk_states)
+    nseq = int(cu_seqlens.numel()) - 1
+    xc, Bc, cs = K.cast_c(x, x.dtype), K.cast_c(B, B.dtype), K.cast_c(chunk_states, chunk_states.dtype)
+    for name, t in (("x", xc), ("B", Bc), ("chunk_states", cs)):
+        K.check_float(name, t)
+    dtf, daf = K.as_f32_vec(dt), K.as_f32_vec(dA_cumsum)
+    cu = cu_seqlens.to(torch.int32).contiguous()
+    out = torch.empty(nseq, heads, hdim, nstate, dtype=torch.float32, device=dev)
+    args = _lib.SsdChunkStateVarlenArgs(
+        Bm=_lib.ptr(Bc), x=_lib.ptr(xc), dt=_lib.ptr(dtf), dA_cumsum=_lib.ptr(daf), chunk_states=_lib.ptr(cs),
+        cu_seqlens=_lib.ptr(cu), states=_lib.ptr(out), dims=_dims(1, seqlen, heads, hdim, groups, nstate, Q),
+        nseq=nseq, x_dtype=_lib.dtype_enum(xc.dtype), b_dtype=_lib.dtype_enum(Bc.dtype),
+        states_dtype=_lib.dtype_enum(cs.dtype))
+    _lib.call("ssm_ssd_chunk_state_varlen", args, dev)
+    return out
 
 
 _KEEP_WORKSPACE = []      # debugging aid: when non-empty, receives [workspace tensor, offset] of the last one-pass call
@@ -299,7 +368,8 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
 
 def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
                  dt_softplus=False, dt_limit=(0.0, float("inf")), return_final_states=False,
-                 states_dtype=None, force_generic=False, fused=None):
+                 states_dtype=None, force_generic=False, fused=None, seq_idx=None, cu_seqlens=None,
+                 return_varlen_states=False):
     """Mamba-2 SSD forward.  bf16 calls whose shape the one-pass kernel covers run
     ``ssm_ssd_combined_fwd``; everything else runs
     ``chunk_cumsum -> bmm_chunk, chunk_state -> state_passing -> chunk_scan``.
@@ -321,9 +391,16 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
             (default: ``x.dtype``; the recurrence itself accumulates in float32).
         fused: ``None`` picks the one-pass kernel when it applies, ``False`` never
             uses it, ``True`` requires it (``ValueError`` if the call is not covered).
+        seq_idx: Optional ``(B, L)`` int sequence ids of a packed batch (ids start at 0):
+            no state and no product crosses from one sequence into the next.
+        cu_seqlens: Optional ``(nseq + 1,)`` sequence boundaries of a packed batch row
+            (batch size 1), only used for ``return_varlen_states``.
+        return_varlen_states: Also return the state at the last step of every sequence,
+            ``(nseq, H, P, N)`` float32 (needs ``cu_seqlens``).
 
     Returns:
-        ``y (B, L, H, P)`` in ``x.dtype``, or ``(y, final_states (B, H, P, N) float32)``.
+        ``y (B, L, H, P)`` in ``x.dtype``; with ``return_final_states`` and / or
+        ``return_varlen_states`` a tuple ``(y[, final_states (B, H, P, N)][, varlen_states])``.
     """
     batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
     _need(C.shape == B.shape, "B and C must have the same shape.")
@@ -331,7 +408,10 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
     _need(initial_states is None or tuple(initial_states.shape) == (batch, heads, hdim, nstate),
           "initial_states must have shape (B, H, P, N).")
     Q = int(chunk_size)
-    can_fuse = not force_generic and fused is not False and \
+    _need(not return_varlen_states or cu_seqlens is not None, "return_varlen_states needs cu_seqlens.")
+    _need(cu_seqlens is None or batch == 1, "cu_seqlens describes one packed batch row: batch size must be 1.")
+    packed = seq_idx is not None or return_varlen_states
+    can_fuse = not force_generic and fused is not False and not packed and \
         _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
     _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "
           "chunk in {64,128,256}, nstate in {64,128} and seqlen % chunk == 0.")
@@ -340,9 +420,13 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
                           return_final_states, (batch, seqlen, heads, hdim, groups, nstate))
     sdt = states_dtype or x.dtype
     dA, dtc = chunk_cumsum(dt, A, Q, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit)
-    states = chunk_state(B, x, dtc, dA, states_dtype=sdt, force_generic=force_generic)
-    entering, final = state_passing(states, dA[:, :, :, -1].contiguous(), initial_states=initial_states)
-    y = chunk_scan(B, C, x, dtc, dA, entering, D=D, z=z, force_generic=force_generic)
+    states = chunk_state(B, x, dtc, dA, states_dtype=sdt, force_generic=force_generic, seq_idx=seq_idx)
+    entering, final = state_passing(states, dA[:, :, :, -1].contiguous(), initial_states=initial_states,
+                                    seq_idx=seq_idx, chunk_size=Q)
+    y = chunk_scan(B, C, x, dtc, dA, entering, D=D, z=z, force_generic=force_generic, seq_idx=seq_idx)
+    outs = [y]
     if return_final_states:
-        return y, final
-    return y
+        outs.append(final)
+    if return_varlen_states:
+        outs.append(chunk_state_varlen(B, x, dtc, dA, cu_seqlens, entering))
+    return outs[0] if len(outs) == 1 else tuple(outs)

@@ -57,7 +57,8 @@ def test_ctypes_struct_sizes_match_the_header(tmp_path):
              "SsdChunkScanArgs": "ssm_ssd_chunk_scan_args", "DecodeStepArgs": "ssm_decode_step_args",
              "SsdCombinedArgs": "ssm_ssd_combined_args",
              "StateStepBwdArgs": "ssm_state_step_bwd_args",
-             "DscanBwdArgs": "ssm_dscan_bwd_args"}
+             "DscanBwdArgs": "ssm_dscan_bwd_args",
+             "SsdChunkStateVarlenArgs": "ssm_ssd_chunk_state_varlen_args"}
     assert set(structs) <= set(cname), set(structs) - set(cname)
     src = tmp_path / "sizes.c"
     lines = ['#include <stdio.h>', f'#include "{HEADER}"', "int main(void) {"]

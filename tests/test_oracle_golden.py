@@ -343,6 +343,48 @@ def test_ssd_combined_fixture_and_grads():
         torch.testing.assert_close(leaves[k].grad.float(), g, rtol=5e-2, atol=5e-2)
 
 
+def test_ssd_combined_varlen_fixture():
+    """Packed row of two sequences (cu_seqlens 0, 3, 6; chunk 3): y is the plain result (the
+    upstream call passes no seq_idx), the per-sequence end states do not mix."""
+    rec = fx.upstream("ssd_combined", "combined_varlen"); i = rec["inputs"]
+    A = fx.upstream("ssd_combined", "combined_full")["inputs"]["A"]
+    y, _, vs = S.ssd_combined(i["X"], i["dt"], i["A"] if "A" in i else A, i["B"], i["C"], int(i["chunk_size"]),
+                              clamp_decay=True, cu_seqlens=[0, 3, 6])
+    torch.testing.assert_close(y.float(), rec["outputs"]["y"], **TF32)
+    torch.testing.assert_close(vs.float(), rec["outputs"]["varlen_states"], **TF32)
+
+
+@pytest.mark.parametrize("Q,lens", [(4, [5, 9, 1, 6]), (8, [3, 3, 10]), (3, [3, 3]), (16, [7, 2, 11])])
+def test_ssd_packed_with_seq_idx_equals_separate_sequences(Q, lens):
+    """A packed row with seq_idx (and cu_seqlens for the end states) gives, sequence by
+    sequence, what the token-by-token recurrence gives on each sequence alone; the initial
+    state goes to the first sequence (id 0) only."""
+    g = torch.Generator().manual_seed(11)
+    H, P, G, N = 4, 3, 2, 5
+    L = sum(lens)
+    x = torch.randn(1, L, H, P, generator=g, dtype=torch.float64)
+    dt = torch.rand(1, L, H, generator=g, dtype=torch.float64)
+    A = -torch.rand(H, generator=g, dtype=torch.float64) * 2
+    Bm = torch.randn(1, L, G, N, generator=g, dtype=torch.float64)
+    Cm = torch.randn(1, L, G, N, generator=g, dtype=torch.float64)
+    D = torch.randn(H, P, generator=g, dtype=torch.float64)
+    z = torch.randn(1, L, H, P, generator=g, dtype=torch.float64)
+    init = torch.randn(1, H, P, N, generator=g, dtype=torch.float64)
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    seq_idx = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])[None]
+    y, fin, vs = S.ssd_combined(x, dt, A, Bm, Cm, Q, D=D, z=z, initial_states=init, clamp_decay=False,
+                                seq_idx=seq_idx, cu_seqlens=cu)
+    for k in range(len(lens)):
+        sl = slice(cu[k], cu[k + 1])
+        yk, fk = S.ssd_sequential(x[:, sl], dt[:, sl], A, Bm[:, sl], Cm[:, sl], D=D, z=z[:, sl],
+                                  initial_states=init if k == 0 else None)
+        torch.testing.assert_close(y[:, sl], yk, rtol=1e-10, atol=1e-10)
+        torch.testing.assert_close(vs[k], fk[0], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(fin[0], vs[-1], rtol=1e-10, atol=1e-10)
+
+
 @pytest.mark.parametrize("Q", [1, 4, 8, 32])
 def test_ssd_chunked_equals_sequential(Q):
     g = torch.Generator().manual_seed(5)

@@ -88,6 +88,71 @@ def make(seed, b, l, h, p, g, n, dtype=torch.float32, d_mat=False, use_z=True, u
     return dict(x=x, dt=dt, A=A, B=Bm, C=Cm, D=D, z=z, init=init)
 
 
+def test_combined_varlen_vector():
+    """Packed row of two sequences (cu_seqlens 0, 3, 6; chunk 3), no seq_idx: y of the plain
+    scan, per-sequence end states that do not mix.  Negative raw steps are clamped to 0."""
+    rec = fx.upstream("ssd_combined", "combined_varlen"); i = rec["inputs"]
+    cu_seqlens = torch.tensor([0, 3, 6], dtype=torch.int32).cuda()
+    y, vs = ssd().ssd_combined(cu(i["X"]), cu(i["dt"]), cu(i["A"]), cu(i["B"]), cu(i["C"]), int(i["chunk_size"]),
+                               cu_seqlens=cu_seqlens, return_varlen_states=True)
+    torch.testing.assert_close(y.cpu(), rec["outputs"]["y"], **TF32)
+    torch.testing.assert_close(vs.cpu(), rec["outputs"]["varlen_states"], **TF32)
+
+
+@pytest.mark.parametrize("Q,lens,dtype", [(4, [5, 9, 1, 6], torch.float32), (8, [3, 3, 10], torch.float32),
+                                          (64, [100, 28, 200, 56], torch.float32),
+                                          (64, [100, 28, 200, 56], torch.bfloat16)])
+def test_packed_sequences_match_the_oracle_and_separate_runs(Q, lens, dtype):
+    """seq_idx + cu_seqlens: against the float64 oracle, and sequence by sequence against
+    separate calls of the same kernels (the first sequence takes the initial state)."""
+    g = torch.Generator().manual_seed(13)
+    H, P, G, N = 4, 16, 2, 32
+    L = sum(lens)
+    x = torch.randn(1, L, H, P, generator=g).to(dtype)
+    dt = torch.rand(1, L, H, generator=g) * 0.5
+    A = -torch.rand(H, generator=g) * 2
+    Bm = torch.randn(1, L, G, N, generator=g).to(dtype)
+    Cm = torch.randn(1, L, G, N, generator=g).to(dtype)
+    D = torch.randn(H, generator=g)
+    z = torch.randn(1, L, H, P, generator=g).to(dtype)
+    init = torch.randn(1, H, P, N, generator=g)
+    cu_l = [0]
+    for n in lens:
+        cu_l.append(cu_l[-1] + n)
+    seq_idx = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])[None]
+    y, fin, vs = ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
+                                    return_final_states=True, seq_idx=cu(seq_idx),
+                                    cu_seqlens=torch.tensor(cu_l, dtype=torch.int32).cuda(),
+                                    return_varlen_states=True, states_dtype=torch.float32)
+    wy, wf, wv = S.ssd_combined(x, dt, A, Bm, Cm, Q, D=D, z=z, initial_states=init, clamp_decay=False,
+                                seq_idx=seq_idx, cu_seqlens=cu_l)
+    tol = FP32_TOL if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2 * float(wy.abs().max()))
+    torch.testing.assert_close(y.float().cpu(), wy.float(), **tol)
+    stol = FP32_TOL if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2 * float(wv.abs().max()))
+    torch.testing.assert_close(vs.cpu(), wv.float(), **stol)
+    torch.testing.assert_close(fin.cpu(), wf.float(), **stol)
+    for k in range(len(lens)):
+        sl = slice(cu_l[k], cu_l[k + 1])
+        yk, fk = ssd().ssd_combined(cu(x[:, sl]), cu(dt[:, sl]), cu(A), cu(Bm[:, sl]), cu(Cm[:, sl]), Q, D=cu(D),
+                                    z=cu(z[:, sl]), initial_states=cu(init) if k == 0 else None,
+                                    return_final_states=True, states_dtype=torch.float32, fused=False)
+        torch.testing.assert_close(y[:, sl].float().cpu(), yk.float().cpu(), **tol)
+        torch.testing.assert_close(vs[k].cpu(), fk[0].cpu(), **stol)
+
+
+def test_packed_arguments_are_checked():
+    x = torch.zeros(2, 8, 2, 4).cuda()
+    dt = torch.zeros(2, 8, 2).cuda()
+    A = -torch.ones(2).cuda()
+    Bm = torch.zeros(2, 8, 1, 4).cuda()
+    with pytest.raises(ValueError):
+        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, return_varlen_states=True)                       # no cu_seqlens
+    with pytest.raises(ValueError):
+        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, cu_seqlens=torch.tensor([0, 8]).cuda(), return_varlen_states=True)
+    with pytest.raises(ValueError):
+        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, seq_idx=torch.zeros(2, 7, dtype=torch.int32).cuda())
+
+
 @pytest.mark.parametrize("shape,Q", [((1, 1, 1, 1, 1, 1), 1), ((2, 19, 4, 5, 2, 6), 8), ((2, 64, 4, 16, 1, 32), 16),
                                      ((1, 300, 2, 64, 2, 128), 64), ((2, 130, 3, 7, 3, 9), 256)],
                          ids=lambda v: str(v).replace(" ", ""))
