@@ -256,6 +256,10 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
                          "the reference for hardware byte counters")
+    ap.add_argument("--only", default=None,
+                    choices=["scan_bwd", "conv", "norm", "decode", "ssd"],
+                    help="run one of the secondary workloads alone and print its figures "
+                         "(for profiling that kernel; not the benchmark line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every operator on this path is independent per "
@@ -275,6 +279,12 @@ def main():
         del src, dst
 
     from ssm_amd import configs
+
+    if args.only:
+        fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
+              "ssd": bench_ssd}[args.only]
+        print(json.dumps({args.only: fn()}))
+        return
 
     r = bench_scan_fwd(args.steps, args.warmup)
     value = r["bytes"] / r["wall_s"] / 1e9
