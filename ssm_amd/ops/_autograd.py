@@ -184,3 +184,42 @@ def state_step_with_grad(state, x, dt, A, B, C, D, z, dt_bias, softplus):
     out, new_state = StateStepFn.apply(state, x, dt, A, B, C, D, z, dt_bias, softplus)
     state.copy_(new_state)
     return out
+
+
+class SsdCombinedFn(torch.autograd.Function):
+    """Mamba-2 SSD ``(x, dt, A, B, C, ...) -> (y, final_states)``.  The reference has no code for
+    this operator; the gradients it ships (``ssd_combined.combined_full`` in
+    tests/mamba_reference_cases.json, made by the call at scripts/refresh_mamba_goldens.py:588-606)
+    pin the backward."""
+
+    @staticmethod
+    def forward(ctx, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, dt_softplus, dt_limit,
+                states_dtype, force_generic, fused):
+        from .ssd import _ssd_combined_forward
+
+        y, final = _ssd_combined_forward(x.detach(), dt.detach(), A.detach(), B.detach(), C.detach(), chunk_size,
+                                         D=None if D is None else D.detach(), z=None if z is None else z.detach(),
+                                         dt_bias=None if dt_bias is None else dt_bias.detach(),
+                                         initial_states=None if initial_states is None else initial_states.detach(),
+                                         dt_softplus=dt_softplus, dt_limit=dt_limit, return_final_states=True,
+                                         states_dtype=states_dtype, force_generic=force_generic, fused=fused)
+        ctx.save_for_backward(x, dt, A, B, C, D, z, dt_bias, initial_states)
+        ctx.conf = (chunk_size, dt_softplus, dt_limit)
+        return y, final
+
+    @staticmethod
+    def backward(ctx, grad_y, grad_final):
+        from .ssd import ssd_combined_backward
+
+        x, dt, A, B, C, D, z, dt_bias, init = ctx.saved_tensors
+        Q, softplus, limit = ctx.conf
+        if grad_y is None:
+            grad_y = torch.zeros_like(x)
+        dx, ddt, dA, dB, dC, dD, dz, dbias, dinit = ssd_combined_backward(
+            grad_y, grad_final, x, dt, A, B, C, Q, D=D, z=z, dt_bias=dt_bias, initial_states=init,
+            dt_softplus=softplus, dt_limit=limit)
+        need = ctx.needs_input_grad
+        pick = lambda i, g, r: _like(g, r) if (r is not None and g is not None and need[i]) else None
+        return (pick(0, dx, x), pick(1, ddt, dt), pick(2, dA, A), pick(3, dB, B), pick(4, dC, C), None,
+                pick(6, dD, D), pick(7, dz, z), pick(8, dbias, dt_bias), pick(9, dinit, init),
+                None, None, None, None, None)

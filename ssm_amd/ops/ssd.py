@@ -370,7 +370,8 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
                  dt_softplus=False, dt_limit=(0.0, float("inf")), return_final_states=False,
                  states_dtype=None, force_generic=False, fused=None, seq_idx=None, cu_seqlens=None,
                  return_varlen_states=False):
-    """Mamba-2 SSD forward.  bf16 calls whose shape the one-pass kernel covers run
+    """Mamba-2 SSD, differentiable in ``x, dt, A, B, C, D, z, dt_bias, initial_states`` (gradients:
+    :func:`ssd_combined_backward`).  bf16 calls whose shape the one-pass kernel covers run
     ``ssm_ssd_combined_fwd``; everything else runs
     ``chunk_cumsum -> bmm_chunk, chunk_state -> state_passing -> chunk_scan``.
 
@@ -402,6 +403,27 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         ``y (B, L, H, P)`` in ``x.dtype``; with ``return_final_states`` and / or
         ``return_varlen_states`` a tuple ``(y[, final_states (B, H, P, N)][, varlen_states])``.
     """
+    tensors = (x, dt, A, B, C, D, z, dt_bias, initial_states)
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        _need(seq_idx is None and cu_seqlens is None and not return_varlen_states,
+              "gradients of packed sequences (seq_idx / cu_seqlens) are not implemented.")
+        from ._autograd import SsdCombinedFn
+        y, final = SsdCombinedFn.apply(x, dt, A, B, C, int(chunk_size), D, z, dt_bias, initial_states,
+                                       bool(dt_softplus), (float(dt_limit[0]), float(dt_limit[1])),
+                                       states_dtype, bool(force_generic), fused)
+        return (y, final) if return_final_states else y
+    return _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias,
+                                 initial_states=initial_states, dt_softplus=dt_softplus, dt_limit=dt_limit,
+                                 return_final_states=return_final_states, states_dtype=states_dtype,
+                                 force_generic=force_generic, fused=fused, seq_idx=seq_idx, cu_seqlens=cu_seqlens,
+                                 return_varlen_states=return_varlen_states)
+
+
+def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
+                          dt_softplus=False, dt_limit=(0.0, float("inf")), return_final_states=False,
+                          states_dtype=None, force_generic=False, fused=None, seq_idx=None, cu_seqlens=None,
+                          return_varlen_states=False):
+    """The forward of :func:`ssd_combined` (same arguments); runs no autograd bookkeeping."""
     batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
     _need(C.shape == B.shape, "B and C must have the same shape.")
     _need(tuple(dt.shape) == (batch, seqlen, heads), "dt must have shape (B, L, H).")
@@ -430,3 +452,100 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
     if return_varlen_states:
         outs.append(chunk_state_varlen(B, x, dtc, dA, cu_seqlens, entering))
     return outs[0] if len(outs) == 1 else tuple(outs)
+
+
+def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None):
+    """``y_t = sum_{s<=t} exp(cs_t - cs_s) <C_t, B_s> w_s x_s + exp(cs_t) C_t . init`` and the state
+    after the last step, through chunk_state -> state_passing -> chunk_scan (float32)."""
+    states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32)
+    entering, final = state_passing(states, dA_cs[:, :, :, -1].contiguous(), initial_states=init)
+    return chunk_scan(Bm, Cm, x, w_c, dA_cs, entering), final
+
+
+def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
+                          initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
+    """Gradients of :func:`ssd_combined` (outputs ``y`` and ``final_states``).
+
+    With ``a_t = exp(dt_t A)``, ``H_t = a_t H_{t-1} + dt_t x_t (x) B_t`` and the adjoint state
+    ``G_t = dy_t (x) C_t + a_{t+1} G_{t+1}``, every contraction is again a chunked scan of the forward
+    kind and runs through the same three kernels with the operands in other roles:
+
+    * ``u_t = G_t B_t`` (then ``dx = dt u + D dy``): time reversed, ``x <- dy``, ``B <- C``, ``C <- B``;
+    * ``dB_t = dt_t G_t^T x_t``: time reversed, ``x <- C``, ``B <- dy``, ``C <- x`` (state and channel
+      axes trade places);
+    * ``dC_t = H_t^T dy_t``: forward in time, ``x <- dt B``, ``B <- x``, ``C <- dy``;
+    * ``y`` before skip and gate (for ``dz`` and the scalar below): the forward itself.
+
+    The decay of the reversed passes is that of the following step (``a_{t+1}``).  The per-step
+    scalar ``q_t = a_t <G_t, H_{t-1}>`` that ``ddt`` and ``dA`` need follows from
+    ``<G_t, H_t> = <G_{t-1}, H_{t-1}> - <dy_{t-1}, H_{t-1} C_{t-1}> + dt_t <x_t, u_t>``, a running sum of
+    quantities the passes have already produced.  The element-wise steps between the passes are
+    ordinary tensor operations.
+
+    Args:
+        dout: ``(B, L, H, P)`` gradient of ``y``.
+        dfinal: ``(B, H, P, N)`` gradient of ``final_states`` or ``None``.
+        (others): the arguments of the forward.
+
+    Returns:
+        ``(dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)`` in float32 (``None`` for absent inputs).
+    """
+    batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
+    Q = int(chunk_size)
+    per = heads // groups
+    f32 = torch.float32
+    xf, Bf, Cf, Af = x.detach().to(f32), B.detach().to(f32), C.detach().to(f32), A.detach().to(f32)
+    dof = dout.detach().to(f32)
+    Df = None if D is None else D.detach().to(f32)
+    Dx = 0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * xf
+    init = None if initial_states is None else initial_states.detach().to(f32)
+    dfin = None if dfinal is None else dfinal.detach().to(f32).contiguous()
+
+    def blh(t_c):                         # (B, H, nc, Q) -> (B, L, H)
+        return t_c.permute(0, 2, 3, 1).reshape(batch, -1, heads)[:, :seqlen]
+
+    dA_cs, dt_c = chunk_cumsum(dt.detach(), Af, Q, dt_bias=None if dt_bias is None else dt_bias.detach(),
+                               dt_softplus=dt_softplus, dt_limit=dt_limit)
+    dte = blh(dt_c)                                                   # effective step
+    ypre, _ = _lin_pass(xf, dt_c, dA_cs, Bf, Cf, init)                # before skip and gate
+    if z is not None:
+        zf = z.detach().to(f32)
+        sg = torch.sigmoid(zf)
+        dy = dof * zf * sg
+        dz = dof * (ypre + Dx) * (sg * (1.0 + zf * (1.0 - sg)))
+    else:
+        dy, dz = dof, None
+    dD = None
+    if Df is not None:
+        dD = (dy * xf).sum(dim=(0, 1, 3)) if Df.ndim == 1 else (dy * xf).sum(dim=(0, 1))
+    # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
+    dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
+    dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
+    _, ones_c = chunk_cumsum(torch.ones_like(dte), torch.zeros_like(Af), Q)
+    dyr = dy.flip(1).contiguous()
+    u_r, Gfin = _lin_pass(dyr, ones_c, dA_r, Cf.flip(1).contiguous(), Bf.flip(1).contiguous(), dfin)
+    u = u_r.flip(1)
+    dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin
+    dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
+    Bh = Bf.repeat_interleave(per, dim=2) if per > 1 else Bf
+    Ch = Cf.repeat_interleave(per, dim=2) if per > 1 else Cf
+    v_r, _ = _lin_pass(Ch.flip(1).contiguous(), ones_c, dA_r, dyr, xf.flip(1).contiguous(),
+                       None if dfin is None else dfin.transpose(2, 3).contiguous())
+    dB = (dte[..., None] * v_r.flip(1)).view(batch, seqlen, groups, per, nstate).sum(3)
+    dCh, _ = _lin_pass(Bh.contiguous(), dt_c, dA_cs, xf, dy.contiguous(),
+                       None if init is None else init.transpose(2, 3).contiguous())
+    dC = dCh.view(batch, seqlen, groups, per, nstate).sum(3)
+    xu = (xf * u).sum(-1)                                             # (B, L, H)
+    s1 = dte * xu
+    s2 = (dy * ypre).sum(-1)
+    W0 = (dinit * init).sum(dim=(2, 3)) if init is not None else torch.zeros(batch, heads, dtype=f32, device=x.device)
+    left = torch.cat([torch.zeros_like(s2[:, :1]), s2[:, :-1]], dim=1)
+    q = W0[:, None] + (s1 - left).cumsum(1) - s1
+    ddte = Af[None, None] * q + xu
+    dA = (dte * q).sum(dim=(0, 1))
+    raw = dt.detach().to(f32) + (0.0 if dt_bias is None else dt_bias.detach().to(f32)[None, None])
+    v = torch.nn.functional.softplus(raw) if dt_softplus else raw
+    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    ddt = ddte * (torch.sigmoid(raw) if dt_softplus else 1.0) * ((v >= lo) & (v <= hi)).to(f32)
+    dbias = ddt.sum(dim=(0, 1)) if dt_bias is not None else None
+    return dx, ddt, dA, dB, dC, dD, dz, dbias, (dinit if init is not None else None)

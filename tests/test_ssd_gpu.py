@@ -88,6 +88,86 @@ def make(seed, b, l, h, p, g, n, dtype=torch.float32, d_mat=False, use_z=True, u
     return dict(x=x, dt=dt, A=A, B=Bm, C=Cm, D=D, z=z, init=init)
 
 
+def _leaves(inp, names, dtype=None):
+    out = {}
+    for k in names:
+        v = inp.get(k)
+        out[k] = None if v is None else v.clone().requires_grad_(True)
+    return out
+
+
+@pytest.mark.parametrize("shape,Q,dtype,d_mat,use_z,use_init,softplus", [
+    ((2, 19, 4, 5, 2, 6), 8, torch.float32, False, True, True, True),
+    ((1, 12, 2, 3, 1, 4), 4, torch.float32, True, False, False, False),
+    ((2, 64, 4, 16, 4, 32), 16, torch.float32, False, True, True, True),
+    ((2, 256, 4, 64, 1, 64), 64, torch.bfloat16, False, True, True, True),
+    ((1, 512, 2, 64, 2, 128), 256, torch.bfloat16, True, True, False, True),
+], ids=lambda v: str(v).replace(" ", ""))
+def test_combined_gradients_match_float64_autograd(shape, Q, dtype, d_mat, use_z, use_init, softplus):
+    """All nine gradients of (y, final_states) against float64 autograd through the token-by-token
+    recurrence, for random upstream gradients of both outputs."""
+    b, l, h, p, g, n = shape
+    gen = torch.Generator().manual_seed(23 + l)
+    x = torch.randn(b, l, h, p, generator=gen).to(dtype)
+    dt = torch.randn(b, l, h, generator=gen) * 0.5 if softplus else torch.rand(b, l, h, generator=gen) * 0.3
+    A = -(torch.rand(h, generator=gen) + 0.2)
+    Bm = (torch.randn(b, l, g, n, generator=gen) * 0.5).to(dtype)
+    Cm = (torch.randn(b, l, g, n, generator=gen) * 0.5).to(dtype)
+    D = torch.randn(h, p, generator=gen) if d_mat else torch.randn(h, generator=gen)
+    z = torch.randn(b, l, h, p, generator=gen).to(dtype) if use_z else None
+    bias = torch.randn(h, generator=gen) * 0.3 if softplus else None
+    init = torch.randn(b, h, p, n, generator=gen) if use_init else None
+    dout = torch.randn(b, l, h, p, generator=gen)
+    dfin = torch.randn(b, h, p, n, generator=gen)
+    names = ["x", "dt", "A", "B", "C", "D", "z", "dt_bias", "init"]
+    vals = dict(x=x, dt=dt, A=A, B=Bm, C=Cm, D=D, z=z, dt_bias=bias, init=init)
+    # float64 reference
+    w = {k: (None if v is None else v.double().clone().requires_grad_(True)) for k, v in vals.items()}
+    y64, f64 = S.ssd_sequential(w["x"], w["dt"], w["A"], w["B"], w["C"], D=w["D"], z=w["z"], dt_bias=w["dt_bias"],
+                                dt_softplus=softplus, initial_states=w["init"])
+    ((y64 * dout.double()).sum() + (f64 * dfin.double()).sum()).backward()
+    # device
+    d = {k: (None if v is None else v.cuda().clone().requires_grad_(True)) for k, v in vals.items()}
+    y, fin = ssd().ssd_combined(d["x"], d["dt"], d["A"], d["B"], d["C"], Q, D=d["D"], z=d["z"], dt_bias=d["dt_bias"],
+                                initial_states=d["init"], dt_softplus=softplus, return_final_states=True)
+    ((y.float() * dout.cuda()).sum() + (fin * dfin.cuda()).sum()).backward()
+    for k in names:
+        if vals[k] is None:
+            continue
+        want = w[k].grad
+        got = d[k].grad.float().cpu().double()
+        assert got.shape == want.shape and d[k].grad.dtype == vals[k].dtype
+        scale = float(want.abs().max())
+        if dtype == torch.float32:
+            torch.testing.assert_close(got, want, rtol=2e-3, atol=2e-4 * scale, msg=lambda m: f"{k}: {m}")
+        else:
+            torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2 * scale, msg=lambda m: f"{k}: {m}")
+
+
+def test_combined_gradient_vector_on_the_decaying_head():
+    """Gradients shipped by the reference for loss = y.sum() (dt_softplus, D matrix, z, initial
+    state).  Head 1 of that case has A > 0, where the upstream kernels clamp the decay inside
+    chunks; the comparison is made on head 0 (A < 0), for the inputs that belong to one head."""
+    rec = fx.upstream("ssd_combined", "combined_full"); i = rec["inputs"]; gr = rec["gradients"]
+    d = {k: cu(i[k]).clone().requires_grad_(True) for k in ("X", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states")}
+    y = ssd().ssd_combined(d["X"], d["dt"], d["A"], d["B"], d["C"], int(i["chunk_size"]), D=d["D"], z=d["z"],
+                           dt_bias=d["dt_bias"], initial_states=d["initial_states"], dt_softplus=True)
+    y.sum().backward()
+    pick = {"X": lambda t: t[:, :, 0], "dt": lambda t: t[:, :, 0], "A": lambda t: t[0], "D": lambda t: t[0],
+            "z": lambda t: t[:, :, 0], "dt_bias": lambda t: t[0], "initial_states": lambda t: t[:, 0]}
+    for k, f in pick.items():
+        torch.testing.assert_close(f(d[k].grad.cpu()), f(gr[k]), rtol=5e-2, atol=5e-2, msg=lambda m: f"{k}: {m}")
+
+
+def test_gradients_of_packed_sequences_are_refused():
+    x = torch.zeros(1, 8, 2, 4).cuda().requires_grad_(True)
+    dt = torch.zeros(1, 8, 2).cuda()
+    A = -torch.ones(2).cuda()
+    Bm = torch.zeros(1, 8, 1, 4).cuda()
+    with pytest.raises(ValueError):
+        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, seq_idx=torch.zeros(1, 8, dtype=torch.int32).cuda())
+
+
 def test_combined_varlen_vector():
     """Packed row of two sequences (cu_seqlens 0, 3, 6; chunk 3), no seq_idx: y of the plain
     scan, per-sequence end states that do not mix.  Negative raw steps are clamped to 0."""
