@@ -1,0 +1,214 @@
+"""A Mamba-2 language-model stack built on the operators of this package: the
+measurement harness for whole-model prefill and greedy decoding.
+
+It is not a port of the reference's modules.  The reference's ``Mamba2`` block
+(/root/reference/src/ssm/modules/mamba2.py:20-140) is a simplified block around
+its diagonal ``ssd_chunk_scan``; this harness is the state-space-duality block the
+benchmark configuration describes (``d_state = 128``, one B/C group, gated
+RMSNorm before the output projection), as published with Mamba-2:
+
+    residual, h = add + RMSNorm                        fused_layer_norm_with_residual
+    z | xBC | dt = in_proj(h)                          GEMM (torch)
+    xBC = silu(conv1d(xBC))                            dw_causal_conv (channels last)
+    y = SSD(x, dt, A, B, C, D, gate z)                 ssm_amd.ops.ssd.ssd_combined
+    out = out_proj(RMSNorm(y))                         fused_layer_norm, GEMM (torch)
+
+and, per generated token, the same block on cached states:
+
+    conv window roll + taps + silu                     dw_causal_conv on the K-step window
+    h <- exp(dt A) h + dt x (x) B ;  y = h C + D x     selective_state_step (in place)
+
+Weights are random (N(0, 0.02), tied embeddings) as the benchmark prescribes.
+What pins it: every operator has its own parity tests; the stack itself is
+checked for self-consistency (prefill + cached decoding reproduces the logits of
+one full forward).  Parity with a particular trained checkpoint or with the
+reference's simplified block is not claimed.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import ops
+from .ops import ssd as ssd_ops
+
+
+@dataclass
+class Mamba2Config:
+    d_model: int = 768
+    n_layer: int = 24
+    expand: int = 2
+    headdim: int = 64
+    d_state: int = 128
+    ngroups: int = 1
+    d_conv: int = 4
+    chunk_size: int = 256
+    vocab_size: int = 50280
+    eps: float = 1e-5
+    dtype: torch.dtype = torch.bfloat16
+
+    @property
+    def d_inner(self) -> int:
+        return self.expand * self.d_model
+
+    @property
+    def nheads(self) -> int:
+        return self.d_inner // self.headdim
+
+    @property
+    def conv_dim(self) -> int:
+        return self.d_inner + 2 * self.ngroups * self.d_state
+
+
+class _Layer:
+    def __init__(self, cfg: Mamba2Config, gen: torch.Generator, device):
+        d, di, H = cfg.d_model, cfg.d_inner, cfg.nheads
+        proj = di + cfg.conv_dim + H
+
+        def rnd(*shape, std=0.02):
+            return (torch.randn(*shape, generator=gen) * std).to(cfg.dtype).to(device)
+
+        self.norm_w = torch.ones(d, dtype=torch.float32, device=device)
+        self.in_proj = rnd(proj, d)
+        self.conv_w = (torch.rand(cfg.conv_dim, cfg.d_conv, generator=gen) - 0.5).to(cfg.dtype).to(device)
+        self.conv_b = rnd(cfg.conv_dim)
+        dt = torch.exp(torch.rand(H, generator=gen) * (math.log(0.1) - math.log(1e-3)) + math.log(1e-3))
+        self.dt_bias = (dt + torch.log(-torch.expm1(-dt))).float().to(device)      # inverse softplus
+        self.A = (-(torch.rand(H, generator=gen) * 15.0 + 1.0)).float().to(device)
+        self.D = torch.ones(H, dtype=torch.float32, device=device)
+        self.gate_norm_w = torch.ones(di, dtype=torch.float32, device=device)
+        self.out_proj = rnd(d, di)
+        # per-channel views of the per-head parameters for the single-token update
+        self.A_dn = self.A.repeat_interleave(cfg.headdim)[:, None].expand(di, cfg.d_state).contiguous()
+        self.D_d = self.D.repeat_interleave(cfg.headdim).contiguous()
+        self.dt_bias_d = self.dt_bias.repeat_interleave(cfg.headdim).contiguous()
+
+
+@dataclass
+class DecodeCache:
+    conv: List[torch.Tensor]       # per layer (B, K, conv_dim): the last K inputs of the convolution
+    ssm: List[torch.Tensor]        # per layer (B, d_inner, N) float32
+    residual: Optional[torch.Tensor] = None
+
+
+class Mamba2LM:
+    """Embedding -> n_layer blocks -> final norm -> tied output projection."""
+
+    def __init__(self, cfg: Mamba2Config, device="cuda", seed: int = 0):
+        self.cfg = cfg
+        self.device = torch.device(device)
+        gen = torch.Generator().manual_seed(seed)
+        self.embedding = (torch.randn(cfg.vocab_size, cfg.d_model, generator=gen) * 0.02).to(cfg.dtype).to(self.device)
+        self.layers = [_Layer(cfg, gen, self.device) for _ in range(cfg.n_layer)]
+        self.final_norm_w = torch.ones(cfg.d_model, dtype=torch.float32, device=self.device)
+
+    # ------------------------------------------------------------------ full sequence
+    def _mixer(self, layer: _Layer, h: torch.Tensor, want_state: bool):
+        cfg = self.cfg
+        Bsz, L, _ = h.shape
+        di, H, P, G, N = cfg.d_inner, cfg.nheads, cfg.headdim, cfg.ngroups, cfg.d_state
+        zxbcdt = h @ layer.in_proj.t()
+        z, xBC, dt = torch.split(zxbcdt, [di, cfg.conv_dim, H], dim=-1)
+        xBC_in = xBC.contiguous()
+        xBC = ops.dw_causal_conv(xBC_in, layer.conv_w, layer.conv_b, activation="silu")      # (B, L, C) channels last
+        x, Bm, Cm = torch.split(xBC, [di, G * N, G * N], dim=-1)
+        out = ssd_ops.ssd_combined(x.reshape(Bsz, L, H, P), dt.contiguous(), layer.A, Bm.reshape(Bsz, L, G, N),
+                                   Cm.reshape(Bsz, L, G, N), cfg.chunk_size, D=layer.D,
+                                   z=z.reshape(Bsz, L, H, P), dt_bias=layer.dt_bias, dt_softplus=True,
+                                   return_final_states=want_state)
+        y, final = out if want_state else (out, None)
+        y = ops.fused_layer_norm(y.reshape(Bsz, L, di), layer.gate_norm_w, None, is_rms=True, eps=cfg.eps)
+        res = y @ layer.out_proj.t()
+        if not want_state:
+            return res, None, None
+        K = cfg.d_conv
+        window = xBC_in[:, -K:] if L >= K else torch.cat(
+            [torch.zeros(Bsz, K - L, cfg.conv_dim, dtype=xBC_in.dtype, device=h.device), xBC_in], dim=1)
+        return res, window.contiguous(), final.reshape(Bsz, di, N).contiguous()
+
+    def forward(self, tokens: torch.Tensor, return_cache: bool = False, last_only: bool = False):
+        """tokens (B, L) -> logits (B, L, vocab) in the model dtype, or (B, 1, vocab) for the last
+        position only (and the decoding cache)."""
+        cfg = self.cfg
+        hidden = self.embedding[tokens]
+        residual = None
+        conv, ssm = [], []
+        for layer in self.layers:
+            hidden, residual = ops.fused_layer_norm_with_residual(hidden, layer.norm_w, None, residual=residual,
+                                                                  is_rms=True, eps=cfg.eps)
+            hidden, cw, st = self._mixer(layer, hidden, return_cache)
+            if return_cache:
+                conv.append(cw)
+                ssm.append(st)
+        hidden, residual = ops.fused_layer_norm_with_residual(hidden, self.final_norm_w, None, residual=residual,
+                                                              is_rms=True, eps=cfg.eps)
+        logits = (hidden[:, -1:] if last_only else hidden) @ self.embedding.t()
+        if return_cache:
+            return logits, DecodeCache(conv, ssm)
+        return logits
+
+    # ------------------------------------------------------------------ one token
+    def step(self, tokens: torch.Tensor, cache: DecodeCache) -> torch.Tensor:
+        """tokens (B,) -> logits (B, vocab); the cache is updated in place."""
+        cfg = self.cfg
+        di, H, P, G, N, K = cfg.d_inner, cfg.nheads, cfg.headdim, cfg.ngroups, cfg.d_state, cfg.d_conv
+        hidden = self.embedding[tokens][:, None]                      # (B, 1, d)
+        Bsz = hidden.shape[0]
+        residual = None
+        for layer, cw, st in zip(self.layers, cache.conv, cache.ssm):
+            hidden, residual = ops.fused_layer_norm_with_residual(hidden, layer.norm_w, None, residual=residual,
+                                                                  is_rms=True, eps=cfg.eps)
+            zxbcdt = hidden[:, 0] @ layer.in_proj.t()
+            z, xBC, dt = torch.split(zxbcdt, [di, cfg.conv_dim, H], dim=-1)
+            cw.copy_(torch.cat([cw[:, 1:], xBC[:, None]], dim=1))
+            xBC = ops.dw_causal_conv(cw, layer.conv_w, layer.conv_b, activation="silu")[:, -1]
+            x, Bm, Cm = torch.split(xBC, [di, G * N, G * N], dim=-1)
+            y = ops.selective_state_step(st, x.contiguous(), dt.repeat_interleave(P, dim=-1), layer.A_dn,
+                                         Bm.reshape(Bsz, G, N), Cm.reshape(Bsz, G, N), D=layer.D_d,
+                                         z=z.contiguous(), dt_bias=layer.dt_bias_d, softplus=True)
+            y = ops.fused_layer_norm(y[:, None], layer.gate_norm_w, None, is_rms=True, eps=cfg.eps)
+            hidden = y @ layer.out_proj.t()
+        hidden, residual = ops.fused_layer_norm_with_residual(hidden, self.final_norm_w, None, residual=residual,
+                                                              is_rms=True, eps=cfg.eps)
+        return hidden[:, 0] @ self.embedding.t()
+
+    # ------------------------------------------------------------------ generation
+    @torch.no_grad()
+    def generate(self, tokens: torch.Tensor, new_tokens: int, use_graph: bool = True) -> Tuple[torch.Tensor, dict]:
+        """Greedy decoding: prefill on ``tokens (B, L)``, then ``new_tokens`` single-token steps on
+        cached states.  With ``use_graph`` the step is captured once as a HIP graph and replayed.
+        Returns ``(generated (B, new_tokens), timings in seconds)``."""
+        start, mid, end = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        start.record()
+        logits, cache = self.forward(tokens, return_cache=True, last_only=True)
+        nxt = logits[:, -1].float().argmax(-1)
+        mid.record()
+        out = [nxt]
+        if use_graph and new_tokens > 1:
+            static_tok = nxt.clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):                              # warm-up outside capture, on a scratch cache
+                scratch = DecodeCache([c.clone() for c in cache.conv], [s.clone() for s in cache.ssm])
+                self.step(static_tok, scratch)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_next = self.step(static_tok, cache).float().argmax(-1)
+            # the capture run did not execute: the cache is still the prefill's
+            for _ in range(new_tokens - 1):
+                graph.replay()
+                static_tok.copy_(static_next)
+                out.append(static_next.clone())
+        else:
+            for _ in range(new_tokens - 1):
+                nxt = self.step(nxt, cache).float().argmax(-1)
+                out.append(nxt)
+        end.record()
+        torch.cuda.synchronize()
+        return torch.stack(out, dim=1), {"prefill_s": start.elapsed_time(mid) * 1e-3,
+                                          "decode_s": mid.elapsed_time(end) * 1e-3}
