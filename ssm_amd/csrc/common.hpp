@@ -197,11 +197,17 @@ __device__ __forceinline__ float wave_read_lane(float v, int lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
-// Sum over the 64 lanes, result valid in every lane.
+// Sum over the 64 lanes, result valid in every lane (uniform).  Six DPP additions (a running
+// sum inside each row of 16, then the row totals passed on: lane 63 ends with everything) and
+// one read of lane 63: no trip through the LDS crossbar as with shuffles.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, WAVE);
-  return v;
+  v += dpp_move<DPP_ROW_SHR1, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR2, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR4, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR8, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.0f, v);
+  v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.0f, v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), WAVE - 1));
 }
 
 __device__ __forceinline__ int wave_id_uniform() {
