@@ -376,10 +376,12 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
   const int h = (vid >> 1) % H, b = (vid >> 1) / H;
   const int g = h / (H / G);
   const int p0 = 32 * half;
-  const bool yact = wave < (NLB >> 1);
+  // with four or more pairs of row blocks (state tiles) every wave has some: say so at compile time, the
+  // waits for loads are exact only on straight-line code
+  const bool yact = (NLB >> 1) >= 4 ? true : wave < (NLB >> 1);
   const int lbF = NLB - 1 - wave, lbS = wave;          // first: many blocks below the diagonal, second: few
   const int nt_s = wave;
-  const bool sact = nt_s < NT;
+  const bool sact = NT >= 4 ? true : nt_s < NT;
   const bool has_init = p.init != nullptr;
   const int xrow_b = H * FU_P * 2;                     // bytes between rows of x, z and y
   const float dhead = DMODE == 1 ? p.Dk[h] : 0.0f;
@@ -560,28 +562,15 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     __syncthreads();                       // every wave is past the carried state: its tile becomes the output staging
     FH_T(5)
 
-    // ---- requests to HBM: the gate operands of this wave's rows (in the row-major order of the
-    // output pass) and the next chunk's inputs
+    // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p], and the chunk's reads from
+    // HBM: the gate operands of this wave's rows (in the row-major order of the output pass) and the next
+    // chunk's inputs.  Vector memory reads of a wave return in order, so whatever is requested after a
+    // read from HBM waits for it: the requests go out after the first four steps, behind the ring's first
+    // refills.  The ring stands one pair on; its last refills are the next chunk's first fragments of C.
+    const int cn = min(c + 1, nc - 1);
     bf16x8_t zF[2], zS[2];
     const int row_o = c * Q * xrow_b;
-    if (yact && HAS_Z) {
-#pragma unroll
-      for (int pass = 0; pass < 2; ++pass) {
-        zF[pass] = buf_load16(rz, v_row, row_o + (32 * lbF + 16 * pass) * xrow_b);
-        zS[pass] = buf_load16(rz, v_row, row_o + (32 * lbS + 16 * pass) * xrow_b);
-      }
-    }
-    const int cn = min(c + 1, nc - 1);
-    FH_REQUEST_CHUNK(cn)
-#ifdef FH_TIMING_WAIT
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    FH_T(8)
-#endif
-
-    // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p].  The ring stands one
-    // pair on; the last steps request the next chunk's first fragments of C.
-    if (sact) {
-      float prev_end = 0.0f;
+    float prev_end = 0.0f;
 #define FH_STEP_C(F, KK)                                                                        \
       {                                                                                         \
         const bf16x8_t xf = load_frag(xw + m * Q + (((2 * (KK) + g2) ^ (m & qmask)) << 3));     \
@@ -594,37 +583,54 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
         prev_end = endv;                                                                        \
         _Pragma("unroll") for (int r = 0; r < 16; ++r) S[r] *= gs;                              \
       }
-      for (int k0 = 0; k0 < KS - 4; k0 += 4) {
+#define FH_REQUEST_HBM                                                                          \
+      {                                                                                         \
+        if (yact && HAS_Z) {                                                                    \
+          _Pragma("unroll") for (int pass = 0; pass < 2; ++pass) {                              \
+            zF[pass] = buf_load16(rz, v_row, row_o + (32 * lbF + 16 * pass) * xrow_b);          \
+            zS[pass] = buf_load16(rz, v_row, row_o + (32 * lbS + 16 * pass) * xrow_b);          \
+          }                                                                                     \
+        }                                                                                       \
+        FH_REQUEST_CHUNK(cn)                                                                    \
+        /* the requests go out here: the scheduler must not sink them into the update */        \
+        asm volatile("" ::: "memory");                                                          \
+      }
+    if (sact) {
+#pragma unroll
+      for (int k0 = 0; k0 < KS; k0 += 4) {
+        const bool more = k0 + 4 < KS;
         FH_SCALE_C(k0)
         FH_STEP_C(f2, k0)
-        f2 = buf_load16(rf, st.vf, st.off_bt + (k0 + 4) * st.bt_step);
+        if (more) f2 = buf_load16(rf, st.vf, st.off_bt + (k0 + 4) * st.bt_step);
+        else if (yact) f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
         FH_STEP_C(f3, k0 + 1)
-        f3 = buf_load16(rf, st.vf, st.off_bt + (k0 + 5) * st.bt_step);
+        if (more) f3 = buf_load16(rf, st.vf, st.off_bt + (k0 + 5) * st.bt_step);
+        else if (yact) f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
         FH_SCALE_C(k0 + 2)
         FH_STEP_C(f0, k0 + 2)
-        f0 = buf_load16(rf, st.vf, st.off_bt + (k0 + 6) * st.bt_step);
+        if (more) f0 = buf_load16(rf, st.vf, st.off_bt + (k0 + 6) * st.bt_step);
+        else if (yact) f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
         FH_STEP_C(f1, k0 + 3)
-        f1 = buf_load16(rf, st.vf, st.off_bt + (k0 + 7) * st.bt_step);
+        if (more) f1 = buf_load16(rf, st.vf, st.off_bt + (k0 + 7) * st.bt_step);
+        else if (yact) f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
+        if (k0 == 0) FH_REQUEST_HBM
       }
-      FH_SCALE_C(KS - 4)
-      FH_STEP_C(f2, KS - 4)
-      if (yact) f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
-      FH_STEP_C(f3, KS - 3)
-      if (yact) f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
-      FH_SCALE_C(KS - 2)
-      FH_STEP_C(f0, KS - 2)
-      if (yact) f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
-      FH_STEP_C(f1, KS - 1)
-      if (yact) f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
+    } else {
+      FH_REQUEST_HBM
+      if (yact) {
+        f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
+        f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
+        f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
+        f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
+      }
+    }
+#undef FH_REQUEST_HBM
 #undef FH_STEP_C
 #undef FH_SCALE_C
-    } else if (yact) {
-      f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
-      f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
-      f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
-      f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
-    }
     FH_T(6)
+    // the gate operands are first looked at here: without this the scheduler starts converting them in
+    // the middle of the state update, which then waits for the reads from HBM after all
+    if (HAS_Z) asm volatile("" : "+v"(zF[0]), "+v"(zF[1]), "+v"(zS[0]), "+v"(zS[1]) : : "memory");
     // ---- the output through a wave-private 32 x 32 fp32 tile to row-major 16-byte accesses: gate, store
     if (yact) {
       float *stg = reinterpret_cast<float *>(smem + 2 * FH_TILE_BYTES) + wave * 1024;
@@ -648,8 +654,14 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] *= silu_f32((float)(which == 0 ? zF[pass][j] : zS[pass][j]));
           }
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, pack8(v)), ry, v_row,
-                                                 row_o + (32 * lb + 16 * pass) * xrow_b, 0);
+          // A 16-byte buffer store reads its data registers a few cycles after it issues.  The compiler's
+          // hazard model holds that a scalar-register offset covers that delay; on this chip an arithmetic
+          // instruction that rewrites the registers in the next two slots has been seen to get ahead of the
+          // read under load (wrong dwords in the last quarter of each 16 lanes).  So the data stays live, and
+          // idle slots follow the store.
+          const u32x4_t packed = __builtin_bit_cast(u32x4_t, pack8(v));
+          __builtin_amdgcn_raw_buffer_store_b128(packed, ry, v_row, row_o + (32 * lb + 16 * pass) * xrow_b, 0);
+          asm volatile("s_nop 3" : : "v"(packed) : "memory");
         }
         wave_lds_sync();
       }
