@@ -21,6 +21,13 @@
 // There are no atomics: results are bit-reproducible.
 #include "common.hpp"
 
+#include <type_traits>
+#include <utility>
+#ifdef BW_TIMING
+#include <cstdio>
+#include <vector>
+#endif
+
 namespace ssm {
 
 constexpr int BW_K = 8;                  // steps per lane
@@ -45,13 +52,70 @@ struct ScanBwdParams {
   int rows_per_wg;       // channels walked by one workgroup (all in one B group and one C group)
   int nblk;              // workgroups per batch row = dim / rows_per_wg
   int bc_vec_ok;
+#ifdef BW_TIMING
+  long long *times;      // [workgroup][wave][12] clock counts per phase (debug builds)
+#endif
 };
 
 // Stage one [BW_MAX_N][BW_T] slab of a time-varying projection (fp32, transposed
 // so that lane l finds steps 8l..8l+7 of state n at n*T + {l*4, 256 + l*4}).
+__device__ __forceinline__ float4 bw_tile_quad_slow(const void *src, int dtype, size_t off, int t, int len) {
+  float4 v;
+  v.x = (t + 0 < len) ? load_as_f32(src, dtype, off + 0) : 0.0f;
+  v.y = (t + 1 < len) ? load_as_f32(src, dtype, off + 1) : 0.0f;
+  v.z = (t + 2 < len) ? load_as_f32(src, dtype, off + 2) : 0.0f;
+  v.w = (t + 3 < len) ? load_as_f32(src, dtype, off + 3) : 0.0f;
+  return v;
+}
+
+__device__ __forceinline__ float4 bw_quad_from16(uint2 raw, int dtype) {
+  float4 v;
+  if (dtype == SSM_BF16) {
+    v.x = __uint_as_float(raw.x << 16);
+    v.y = __uint_as_float(raw.x & 0xffff0000u);
+    v.z = __uint_as_float(raw.y << 16);
+    v.w = __uint_as_float(raw.y & 0xffff0000u);
+  } else {
+    union { uint32_t u; _Float16 h[2]; } a, b;
+    a.u = raw.x;
+    b.u = raw.y;
+    v.x = (float)a.h[0];
+    v.y = (float)a.h[1];
+    v.z = (float)b.h[0];
+    v.w = (float)b.h[1];
+  }
+  return v;
+}
+
 __device__ __forceinline__ void bw_stage_tile(float *dst, const void *src, int dtype, size_t src_off, int len,
                                               int t0, int nn, bool vec_ok) {
   constexpr int QT = BW_T / 4;
+  constexpr int PER = BW_MAX_N * QT / BW_THREADS;          // quads per thread: 4
+  auto place = [&](int e) { const int nl = e / QT, tl = (e % QT) * 4; return dst + nl * BW_T + ((tl % BW_K) >> 2) * (WAVE * 4) + (tl / BW_K) * 4; };
+  if (vec_ok && t0 + BW_T <= len && nn == BW_MAX_N) {
+    // whole slab inside the sequence: every read of the thread is requested before the first is used
+    static_assert(PER == 4, "four quads per thread");
+    const int e0 = threadIdx.x, e1 = e0 + BW_THREADS, e2 = e1 + BW_THREADS, e3 = e2 + BW_THREADS;
+    auto at = [&](int e) { return src_off + (size_t)(e / QT) * len + t0 + (e % QT) * 4; };
+    if (dtype == SSM_F32) {
+      const float *f = reinterpret_cast<const float *>(src);
+      const float4 v0 = *reinterpret_cast<const float4 *>(f + at(e0)), v1 = *reinterpret_cast<const float4 *>(f + at(e1));
+      const float4 v2 = *reinterpret_cast<const float4 *>(f + at(e2)), v3 = *reinterpret_cast<const float4 *>(f + at(e3));
+      *reinterpret_cast<float4 *>(place(e0)) = v0;
+      *reinterpret_cast<float4 *>(place(e1)) = v1;
+      *reinterpret_cast<float4 *>(place(e2)) = v2;
+      *reinterpret_cast<float4 *>(place(e3)) = v3;
+    } else {
+      const uint16_t *h = reinterpret_cast<const uint16_t *>(src);
+      const uint2 r0 = *reinterpret_cast<const uint2 *>(h + at(e0)), r1 = *reinterpret_cast<const uint2 *>(h + at(e1));
+      const uint2 r2 = *reinterpret_cast<const uint2 *>(h + at(e2)), r3 = *reinterpret_cast<const uint2 *>(h + at(e3));
+      *reinterpret_cast<float4 *>(place(e0)) = bw_quad_from16(r0, dtype);
+      *reinterpret_cast<float4 *>(place(e1)) = bw_quad_from16(r1, dtype);
+      *reinterpret_cast<float4 *>(place(e2)) = bw_quad_from16(r2, dtype);
+      *reinterpret_cast<float4 *>(place(e3)) = bw_quad_from16(r3, dtype);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < BW_MAX_N * QT; e += BW_THREADS) {
     const int nl = e / QT;
     const int tl = (e % QT) * 4;
@@ -60,34 +124,13 @@ __device__ __forceinline__ void bw_stage_tile(float *dst, const void *src, int d
     if (nl < nn) {
       const size_t off = src_off + (size_t)nl * len + t;
       if (vec_ok && t + 4 <= len) {
-        if (dtype == SSM_F32) {
-          v = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(src) + off);
-        } else {
-          const uint2 raw = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(src) + off);
-          if (dtype == SSM_BF16) {
-            v.x = __uint_as_float(raw.x << 16);
-            v.y = __uint_as_float(raw.x & 0xffff0000u);
-            v.z = __uint_as_float(raw.y << 16);
-            v.w = __uint_as_float(raw.y & 0xffff0000u);
-          } else {
-            union { uint32_t u; _Float16 h[2]; } a, b;
-            a.u = raw.x;
-            b.u = raw.y;
-            v.x = (float)a.h[0];
-            v.y = (float)a.h[1];
-            v.z = (float)b.h[0];
-            v.w = (float)b.h[1];
-          }
-        }
+        if (dtype == SSM_F32) v = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(src) + off);
+        else v = bw_quad_from16(*reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(src) + off), dtype);
       } else {
-        v.x = (t + 0 < len) ? load_as_f32(src, dtype, off + 0) : 0.0f;
-        v.y = (t + 1 < len) ? load_as_f32(src, dtype, off + 1) : 0.0f;
-        v.z = (t + 2 < len) ? load_as_f32(src, dtype, off + 2) : 0.0f;
-        v.w = (t + 3 < len) ? load_as_f32(src, dtype, off + 3) : 0.0f;
+        v = bw_tile_quad_slow(src, dtype, off, t, len);
       }
     }
-    const int owner = tl / BW_K, item = tl % BW_K;
-    *reinterpret_cast<float4 *>(dst + nl * BW_T + (item >> 2) * (WAVE * 4) + owner * 4) = v;
+    *reinterpret_cast<float4 *>(place(e)) = v;
   }
 }
 
@@ -113,23 +156,52 @@ __device__ __forceinline__ void bw_scan_x2(float &a0, float &b0, float &a1, floa
       : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
 }
 
+// The 24 partial sums of one step (8 waves x {pre, <gh,B>, A-term}), all requested before the first
+// is used.  Written out because the compiler, short of registers at this point, otherwise reads them
+// one by one and waits for each (24 LDS latencies per row).
+template <int OFF>
+__device__ __forceinline__ float bw_lds_read(unsigned addr) {
+  float v;
+  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int... J>
+__device__ __forceinline__ void bw_read_parts(const float *p, float (&pv)[3 * BW_WAVES], std::integer_sequence<int, J...>) {
+  const unsigned addr = (unsigned)(uintptr_t)p;            // low half of a generic LDS address = LDS offset
+  ((pv[J] = bw_lds_read<((J / 3) * 3 * BW_T + (J % 3) * BW_T) * 4>(addr)), ...);
+  // the values exist only after this wait: it takes them as operands so that no use can move above it
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(pv[0]), "+v"(pv[1]), "+v"(pv[2]), "+v"(pv[3]), "+v"(pv[4]), "+v"(pv[5]), "+v"(pv[6]), "+v"(pv[7]),
+                 "+v"(pv[8]), "+v"(pv[9]), "+v"(pv[10]), "+v"(pv[11]), "+v"(pv[12]), "+v"(pv[13]), "+v"(pv[14]),
+                 "+v"(pv[15]), "+v"(pv[16]), "+v"(pv[17]), "+v"(pv[18]), "+v"(pv[19]), "+v"(pv[20]), "+v"(pv[21]),
+                 "+v"(pv[22]), "+v"(pv[23]));
+}
+
 __device__ __forceinline__ float lane_gather(float v, int src_lane) {
   return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
 }
 
-template <typename io_t, bool BVARY, bool CVARY>
-__global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParams p) {
+// LDS admits one workgroup per CU, i.e. two waves per SIMD: telling the compiler so lets its scheduler spend
+// registers on keeping several LDS reads in flight instead of waiting for each in turn.
+template <typename io_t, bool BVARY, bool CVARY, bool HAS_Z>
+__global__ __launch_bounds__(BW_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void scan_bwd_kernel(const ScanBwdParams p) {
   constexpr int K = BW_K, T = BW_T;
   extern __shared__ __align__(16) float lds[];
-  // layout: [B tile][C tile][elem: delta,u,g][partials: 8 x 3 x T][qcarry rows x 16][red 2 x 8 x 2]
+  // layout: [B tile][C tile][elem: delta,u,g][partials: 8 x 3 x T][red 2 x 8 x 2], then per (row, state):
+  // qcarry, A log2(e), chunk-entering state, constant B and C, sums for dA / dB / dC; per row: D, bias, sums
   float *Bs = lds;
   float *Cs = Bs + (BVARY ? BW_MAX_N * T : 0);
   float *e_dl = Cs + (CVARY ? BW_MAX_N * T : 0);
   float *e_u = e_dl + T;
   float *e_g = e_u + T;
   float *part = e_g + T;                          // [wave][3][T]
-  float *qcarry = part + BW_WAVES * 3 * T;        // [rows_per_wg][16]
-  float *red = qcarry + p.rows_per_wg * BW_MAX_N; // [2][BW_WAVES][2]
+  float *red = part + BW_WAVES * 3 * T;           // [2][BW_WAVES][2]
+  const int RN = p.rows_per_wg * BW_MAX_N;
+  float *qcarry = red + 2 * BW_WAVES * 2;         // [rows_per_wg][16] each from here on
+  float *A2s = qcarry + RN, *Hins = A2s + RN, *Bcs = Hins + RN, *Ccs = Bcs + RN;
+  float *sumA = Ccs + RN, *sumB = sumA + RN, *sumC = sumB + RN;
+  float *Dks = sumC + RN;                         // [rows_per_wg] each
+  float *biass = Dks + p.rows_per_wg, *sumD = biass + p.rows_per_wg, *sumb = sumD + p.rows_per_wg;
 
   const int wave = wave_id_uniform();
   const int lane = lane_id();
@@ -146,20 +218,50 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
   if (BVARY) b_tile_off = ((size_t)b * p.b_groups + d_first / (p.dim / p.b_groups)) * (size_t)N * L;
   if (CVARY) c_tile_off = ((size_t)b * p.c_groups + d_first / (p.dim / p.c_groups)) * (size_t)N * L;
 
-  // adjoint entering from beyond the end of the sequence
-  for (int e = tid; e < p.rows_per_wg * BW_MAX_N; e += BW_THREADS) {
+  // Everything a row needs besides its four streams is fetched here, once: inside the row loop a read
+  // from global memory that the next instruction depends on costs more than the row's arithmetic.
+  // Per-row sums are kept in LDS and written at the end.
+  for (int e = tid; e < RN; e += BW_THREADS) {
     const int r = e / BW_MAX_N, n = e % BW_MAX_N;
-    const size_t row = (size_t)b * p.dim + d_first + r;
-    qcarry[e] = (p.dlast && n < N) ? p.dlast[row * N + n] : 0.0f;
+    const int d = d_first + r;
+    const size_t row = (size_t)b * p.dim + d;
+    const bool valid = n < N;
+    qcarry[e] = (p.dlast && valid) ? p.dlast[row * N + n] : 0.0f;      // adjoint from beyond the end
+    A2s[e] = valid ? p.A[(size_t)d * N + n] * LOG2E : 0.0f;
+    float bc = 0.0f, cc = 0.0f;
+    if (!BVARY && valid) bc = load_as_f32(p.Bp, p.bc_dtype, ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N + n);
+    if (!CVARY && valid) cc = load_as_f32(p.Cp, p.bc_dtype, ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N + n);
+    Bcs[e] = bc;
+    Ccs[e] = cc;
+    sumA[e] = sumB[e] = sumC[e] = 0.0f;
   }
+  for (int r = tid; r < p.rows_per_wg; r += BW_THREADS) {
+    Dks[r] = p.Dk ? p.Dk[d_first + r] : 0.0f;
+    biass[r] = p.bias ? p.bias[d_first + r] : 0.0f;
+    sumD[r] = sumb[r] = 0.0f;
+  }
+  const io_t *zsrc = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.u);
 
   const int rev_lane = WAVE - 1 - lane;
+#ifdef BW_TIMING
+  long long tacc[12] = {0}; long long tprev = __builtin_amdgcn_s_memtime();
+#define BT(i) { const long long tn = __builtin_amdgcn_s_memtime(); tacc[i] += tn - tprev; tprev = tn; }
+#else
+#define BT(i)
+#endif
 
   for (int c = nchunks - 1; c >= 0; --c) {
     const int t0 = c * T;
+    BT(0)
     __syncthreads();     // tiles and qcarry free / visible
+    BT(1)
     if (BVARY) bw_stage_tile(Bs, p.Bp, p.bc_dtype, b_tile_off, L, t0, N, p.bc_vec_ok != 0);
     if (CVARY) bw_stage_tile(Cs, p.Cp, p.bc_dtype, c_tile_off, L, t0, N, p.bc_vec_ok != 0);
+    for (int e = tid; e < RN; e += BW_THREADS) {           // the rows' states entering this chunk
+      const int r = e / BW_MAX_N, n = e % BW_MAX_N;
+      const size_t row = (size_t)b * p.dim + d_first + r;
+      Hins[e] = n < N ? p.chunk_states[(row * nchunks + c) * (size_t)N + n] : 0.0f;
+    }
 
     float accB[2][K], accC[2][K];
 #pragma unroll
@@ -177,13 +279,30 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
       nx_u = reinterpret_cast<const io_t *>(p.u)[idx];
       nx_dl = reinterpret_cast<const io_t *>(p.delta)[idx];
       nx_go = reinterpret_cast<const io_t *>(p.dout)[idx];
-      nx_z = p.z ? reinterpret_cast<const io_t *>(p.z)[idx] : nx_u;
+      nx_z = zsrc[idx];
     }
 
-    for (int r = 0; r < p.rows_per_wg; ++r) {
+    // per-row sums of dD and dbias: the waves' partial sums of row r lie in red[r & 1]
+    auto fold_red = [&](int r) {
+      const float *rr = red + (size_t)(r & 1) * BW_WAVES * 2;
+      float sD = 0.0f, sb = 0.0f;
+      for (int wv = 0; wv < BW_WAVES; ++wv) {
+        sD += rr[wv * 2];
+        sb += rr[wv * 2 + 1];
+      }
+      sumD[r] += sD;
+      sumb[r] += sb;
+    };
+
+    BT(2)
+    // One row.  FULL: the chunk lies wholly inside the sequence, so nothing in the row is conditional on
+    // the step index; the compiler then knows exactly how many memory operations are in flight at each
+    // wait and the reads requested a row ahead are not held up by the previous row's stores.
+    auto do_row = [&](auto full_tag, int r) {
+      constexpr bool FULL = decltype(full_tag)::value;
       const int d = d_first + r;
       const size_t row = (size_t)b * p.dim + d;
-      const float Dk = p.Dk ? p.Dk[d] : 0.0f;
+      const float Dk = Dks[r];
 
       // ---- element-wise stage: thread tid owns step t0 + tid of this row
       float el_u = 0.0f, el_dl = 0.0f, el_g = 0.0f, el_sig = 1.0f, el_dz = 0.0f;
@@ -194,12 +313,12 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
         nx_u = reinterpret_cast<const io_t *>(p.u)[idx];
         nx_dl = reinterpret_cast<const io_t *>(p.delta)[idx];
         nx_go = reinterpret_cast<const io_t *>(p.dout)[idx];
-        nx_z = p.z ? reinterpret_cast<const io_t *>(p.z)[idx] : nx_u;
+        nx_z = zsrc[idx];
       }
-      if (te < L) {
+      if (FULL || te < L) {
         el_u = to_f32(cur_u);
         float draw = to_f32(cur_dl);
-        if (p.bias) draw += p.bias[d];
+        draw += biass[r];
         if (p.softplus) {
           el_dl = softplus_f32(draw);
           el_sig = draw > 20.0f ? 1.0f : sigmoid_f32(draw);
@@ -207,7 +326,7 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
           el_dl = draw;
         }
         const float go = to_f32(cur_go);
-        if (p.z) {
+        if (HAS_Z) {
           const float zv = to_f32(cur_z);
           const float sg = sigmoid_f32(zv);
           el_g = go * zv * sg;
@@ -219,7 +338,10 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
       e_dl[tid] = el_dl;
       e_u[tid] = el_u;
       e_g[tid] = el_g;
+      BT(3)
       __syncthreads();                                                  // (1) staged row visible
+      BT(4)
+      if (tid == 0 && r > 0) fold_red(r - 1);
 
       // ---- per-state work: this wave owns states n0, n1
       float dl[K], uu[K], g[K];
@@ -248,19 +370,11 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
       for (int w = 0; w < 2; ++w) {
         const int n = w == 0 ? n0 : n1;
         const bool valid = w == 0 ? v0 : v1;
-        A2[w] = valid ? p.A[(size_t)d * N + n] * LOG2E : 0.0f;
-        Hin[w] = valid ? p.chunk_states[(row * nchunks + c) * (size_t)N + n] : 0.0f;
-        qin_carry[w] = qcarry[r * BW_MAX_N + (valid ? n : 0)];
-        if (!valid) qin_carry[w] = 0.0f;
-        float bconst = 0.0f, cconst = 0.0f;
-        if (!BVARY && valid) {
-          const size_t off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N + n;
-          bconst = load_as_f32(p.Bp, p.bc_dtype, off);
-        }
-        if (!CVARY && valid) {
-          const size_t off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N + n;
-          cconst = load_as_f32(p.Cp, p.bc_dtype, off);
-        }
+        const int rn_ = r * BW_MAX_N + n;              // n < 16 always: invalid states hold zeros
+        A2[w] = A2s[rn_];
+        Hin[w] = Hins[rn_];
+        qin_carry[w] = qcarry[rn_];
+        const float bconst = Bcs[rn_], cconst = Ccs[rn_];
         const int nrow = valid ? n : 0;
 #pragma unroll
         for (int q4 = 0; q4 < K / 4; ++q4) {
@@ -284,7 +398,9 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
         Pr[w] = P[w];
         h[w] = __builtin_fmaf(P[w], lane == 0 ? Hin[w] : 0.0f, hh);
       }
+      BT(5)
       bw_scan_x2(P[0], h[0], P[1], h[1]);
+      BT(6)
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
         // replay forward: hp[i] = state before step i, hcur = state after it
@@ -319,6 +435,7 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
         qin[0] = lane == WAVE - 1 ? qin_carry[0] : t0v;
         qin[1] = lane == WAVE - 1 ? qin_carry[1] : t1v;
       }
+      BT(8)
       float dA_acc[2] = {0.0f, 0.0f}, dBc_acc[2] = {0.0f, 0.0f};
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
@@ -363,35 +480,40 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
           for (int i = 0; i < K; ++i) accC[w][i] = 0.0f;
         }
         if (valid && lane == 0) {
-          const size_t o = row * N + n;
-          const bool first = c == nchunks - 1;
-          p.dA_rows[o] = (first ? 0.0f : p.dA_rows[o]) + sA;
-          if (!BVARY) p.dB_part[o] = (first ? 0.0f : p.dB_part[o]) + sB;
-          if (!CVARY) p.dC_part[o] = (first ? 0.0f : p.dC_part[o]) + sC;
-          qcarry[r * BW_MAX_N + n] = w == 0 ? qn0 : qn1;
+          const int o = r * BW_MAX_N + n;
+          sumA[o] += sA;
+          if (!BVARY) sumB[o] += sB;
+          if (!CVARY) sumC[o] += sC;
+          qcarry[o] = w == 0 ? qn0 : qn1;
         }
       }
+      BT(10)
       __syncthreads();                                                  // (2) partials visible
+      BT(11)
 
       // ---- finish element tid of this row
+      float pv[3 * BW_WAVES];
+      bw_read_parts(part + tid, pv, std::make_integer_sequence<int, 3 * BW_WAVES>{});
       float s_pre = 0.0f, s_gb = 0.0f, s_da = 0.0f;
 #pragma unroll
       for (int wv = 0; wv < BW_WAVES; ++wv) {
-        s_pre += part[(size_t)wv * 3 * T + tid];
-        s_gb += part[(size_t)wv * 3 * T + T + tid];
-        s_da += part[(size_t)wv * 3 * T + 2 * T + tid];
+        s_pre += pv[3 * wv];
+        s_gb += pv[3 * wv + 1];
+        s_da += pv[3 * wv + 2];
       }
+      BT(7)
       float dD_c = 0.0f, dbias_c = 0.0f;
-      if (te < L) {
+      if (FULL || te < L) {
         const size_t idx = row * L + te;
         const float du = __builtin_fmaf(s_gb, el_dl, el_g * Dk);
         const float ddl = __builtin_fmaf(s_gb, el_u, s_da * LN2) * el_sig;
         reinterpret_cast<io_t *>(p.du)[idx] = from_f32<io_t>(du);
         reinterpret_cast<io_t *>(p.ddelta)[idx] = from_f32<io_t>(ddl);
-        if (p.z) reinterpret_cast<io_t *>(p.dz)[idx] = from_f32<io_t>(el_dz * __builtin_fmaf(Dk, el_u, s_pre));
+        if (HAS_Z) reinterpret_cast<io_t *>(p.dz)[idx] = from_f32<io_t>(el_dz * __builtin_fmaf(Dk, el_u, s_pre));
         dD_c = el_g * el_u;
         dbias_c = ddl;
       }
+      BT(9)
       {
         const float sD = wave_sum(dD_c), sb = wave_sum(dbias_c);
         float *rr = red + (size_t)(r & 1) * BW_WAVES * 2;
@@ -400,19 +522,18 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
           rr[wave * 2 + 1] = sb;
         }
       }
-      __syncthreads();                                                  // (3) e_*, part reusable; red visible
-      if (tid == 0) {
-        const float *rr = red + (size_t)(r & 1) * BW_WAVES * 2;
-        float sD = 0.0f, sb = 0.0f;
-        for (int wv = 0; wv < BW_WAVES; ++wv) {
-          sD += rr[wv * 2];
-          sb += rr[wv * 2 + 1];
-        }
-        const bool first = c == nchunks - 1;
-        p.dD_rows[row] = (first ? 0.0f : p.dD_rows[row]) + sD;
-        p.dbias_rows[row] = (first ? 0.0f : p.dbias_rows[row]) + sb;
-      }
-    }
+      BT(2)
+      // No barrier here: the next row's element-wise stage writes e_* (last read before barrier 2),
+      // its per-state work writes `part` only after barrier 1 of that row, which every wave reaches
+      // after it has finished the sums above; `red` alternates between two buffers and is folded
+      // after that same barrier.
+    };
+    if (t0 + T <= L)
+      for (int r = 0; r < p.rows_per_wg; ++r) do_row(std::true_type{}, r);
+    else
+      for (int r = 0; r < p.rows_per_wg; ++r) do_row(std::false_type{}, r);
+    __syncthreads();
+    if (tid == 0) fold_red(p.rows_per_wg - 1);
 
     // ---- flush this chunk's dB / dC partials (sum over the workgroup's channels)
 #pragma unroll
@@ -444,6 +565,27 @@ __global__ __launch_bounds__(BW_THREADS) void scan_bwd_kernel(const ScanBwdParam
       }
     }
   }
+  // ---- the per-row sums
+  __syncthreads();
+  for (int e = tid; e < RN; e += BW_THREADS) {
+    const int r = e / BW_MAX_N, n = e % BW_MAX_N;
+    if (n < N) {
+      const size_t o = ((size_t)b * p.dim + d_first + r) * N + n;
+      p.dA_rows[o] = sumA[e];
+      if (!BVARY) p.dB_part[o] = sumB[e];
+      if (!CVARY) p.dC_part[o] = sumC[e];
+    }
+  }
+  for (int r = tid; r < p.rows_per_wg; r += BW_THREADS) {
+    const size_t row = (size_t)b * p.dim + d_first + r;
+    p.dD_rows[row] = sumD[r];
+    p.dbias_rows[row] = sumb[r];
+  }
+#ifdef BW_TIMING
+  if (lane == 0)
+    for (int i = 0; i < 12; ++i) p.times[((size_t)blockIdx.x * BW_WAVES + wave) * 12 + i] = tacc[i];
+#endif
+#undef BT
 }
 
 // out[o][i] = sum_{j < count} in[(o * count + j) * inner + i], fixed order.
@@ -514,11 +656,11 @@ template <typename io_t>
 static int launch_bwd(const ScanBwdParams &p, hipStream_t s) {
   const bool bv = p.b_kind == SSM_PROJ_BGNL, cv = p.c_kind == SSM_PROJ_BGNL;
   const size_t lds = ((size_t)((int)bv + (int)cv) * BW_MAX_N * BW_T + 3 * BW_T + BW_WAVES * 3 * BW_T +
-                      (size_t)p.rows_per_wg * BW_MAX_N + 2 * BW_WAVES * 2) * sizeof(float);
+                      2 * BW_WAVES * 2 + (size_t)p.rows_per_wg * (8 * BW_MAX_N + 4)) * sizeof(float);
   const unsigned grid = (unsigned)((size_t)p.batch * p.nblk);
 #define SSM_BW_LAUNCH(BV, CV)                                                              \
   {                                                                                        \
-    auto kernel = scan_bwd_kernel<io_t, BV, CV>;                                           \
+    auto kernel = p.z ? scan_bwd_kernel<io_t, BV, CV, true> : scan_bwd_kernel<io_t, BV, CV, false>; \
     if (allow_dynamic_lds(kernel, lds) != hipSuccess) {                                    \
       (void)hipGetLastError();                                                             \
       set_error("ssm_scan_bwd: cannot reserve %zu bytes of LDS", lds);                     \
@@ -601,6 +743,12 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
   p.rows_per_wg = pl.rows_per_wg; p.nblk = pl.nblk;
   p.bc_vec_ok = a->seqlen % 4 == 0 && aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs);
 
+#ifdef BW_TIMING
+  static long long *tbuf = nullptr;
+  const size_t tcount = (size_t)a->batch * pl.nblk * BW_WAVES * 12;
+  if (!tbuf) (void)hipMalloc(&tbuf, (size_t)1 << 26);
+  p.times = tbuf;
+#endif
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   int rc;
   switch (a->io_dtype) {
@@ -609,6 +757,19 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
     default: rc = launch_bwd<f16_t>(p, s); break;
   }
   if (rc != SSM_OK) return rc;
+#ifdef BW_TIMING
+  {
+    (void)hipDeviceSynchronize();
+    std::vector<long long> host(tcount);
+    (void)hipMemcpy(host.data(), tbuf, tcount * 8, hipMemcpyDeviceToHost);
+    const char *names[12] = {"chunk tail", "chunk barrier", "tiles+finish prev", "elementwise", "barrier 1", "load+fold", "scan fwd", "F: LDS sums", "replay..gathers", "F: stores", "final+part+sums", "barrier 2"};
+    double tot = 0; double ph[12] = {0};
+    for (size_t i = 0; i < tcount; ++i) { ph[i % 12] += (double)host[i]; tot += (double)host[i]; }
+    const double nw = (double)tcount / 12;
+    fprintf(stderr, "scan_bwd timing: %.0f counts per wave\n", tot / nw);
+    for (int i = 0; i < 12; ++i) fprintf(stderr, "  %-18s %9.0f  %5.1f%%\n", names[i], ph[i] / nw, 100.0 * ph[i] / tot);
+  }
+#endif
 
   const int Bn = a->batch, D = a->dim, N = a->nstate, L = a->seqlen;
   // dA (D,N), dD (D,), dbias (D,): fold over batch
