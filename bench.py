@@ -216,6 +216,43 @@ def bench_ssd(batch=4, length=4096, heads=80, hdim=64, nstate=128, chunk=256):
             "frac_mfma_bf16_peak": round(flops / us / 1e6 / 2500.0, 4), "dense_tile_flops": flops}
 
 
+def bench_ssd_train(batch=4, length=4096, heads=80, hdim=64, nstate=128, chunk=256):
+    """Config 3 shape through the parts of the SSD path that are not the one-pass forward: forward +
+    backward through autograd (the backward is four passes of the five-kernel pipeline with operands in
+    other roles) and the forward over packed sequences (`seq_idx`, generic kernels)."""
+    from ssm_amd.ops import ssd
+    from ssm_amd import configs
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(batch, length, heads, hdim, generator=g).to(torch.bfloat16).cuda().requires_grad_()
+    dt_bias = configs.inverse_softplus_dt(heads, g)
+    dt = torch.nn.functional.softplus(torch.randn(batch, length, heads, generator=g) + dt_bias).cuda().requires_grad_()
+    A = (-(torch.rand(heads, generator=g) * 15 + 1)).cuda().requires_grad_()
+    Bm = torch.randn(batch, length, 1, nstate, generator=g).to(torch.bfloat16).cuda().requires_grad_()
+    Cm = torch.randn(batch, length, 1, nstate, generator=g).to(torch.bfloat16).cuda().requires_grad_()
+    D = torch.ones(heads).cuda().requires_grad_()
+    z = torch.randn(batch, length, heads, hdim, generator=g).to(torch.bfloat16).cuda().requires_grad_()
+    dy = torch.randn(batch, length, heads, hdim, generator=g).to(torch.bfloat16).cuda()
+
+    def step(_):
+        y = ssd.ssd_combined(x, dt, A, Bm, Cm, chunk, D=D, z=z)
+        y.backward(dy)
+        for t in (x, dt, A, Bm, Cm, D, z):
+            t.grad = None
+
+    fb_us = _time_us(step, iters=5, warmup=2)
+    # four sequences of unequal length packed into every batch row
+    cuts = [0, length // 8, length // 2, length // 2 + 300, length]
+    seq_idx = torch.zeros(batch, length, dtype=torch.int32)
+    for i in range(len(cuts) - 1):
+        seq_idx[:, cuts[i]:cuts[i + 1]] = i
+    seq_idx = seq_idx.cuda()
+    with torch.no_grad():
+        pk_us = _time_us(lambda i: ssd.ssd_combined(x, dt, A, Bm, Cm, chunk, D=D, z=z, seq_idx=seq_idx), iters=5, warmup=2)
+    return {"fwd_bwd_us": round(fb_us, 1), "packed_fwd_us": round(pk_us, 1),
+            "shape": f"B={batch} L={length} H={heads} P={hdim} N={nstate} Q={chunk} bf16; packed: 4 sequences per row"}
+
+
 def bench_model(batch=16, prompt=2048, new_tokens=256):
     """BASELINE config 4: Mamba-2-130M-style stack (24 layers, d_model 768, d_state 128, tied embeddings,
     random weights, bf16): prefill of batch x prompt tokens, then greedy decoding on cached states with
@@ -279,7 +316,7 @@ def main():
                     help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
-                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "model"],
+                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "model"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
     args = ap.parse_args()
@@ -304,7 +341,7 @@ def main():
 
     if args.only:
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
-              "ssd": bench_ssd, "model": bench_model}[args.only]
+              "ssd": bench_ssd, "ssd_train": bench_ssd_train, "model": bench_model}[args.only]
         print(json.dumps({args.only: fn()}))
         return
 
@@ -347,6 +384,7 @@ def main():
         extra["fused_add_rmsnorm"] = bench_norm()
         extra["decode_step_config2"] = bench_decode()
         extra["ssd_combined_config3"] = bench_ssd()
+        extra["ssd_config3_backward_and_packed"] = bench_ssd_train()
         extra["mamba2_130m_style_model_config4"] = bench_model()
         line["extra"] = extra
     if not args.no_cpu_baseline:

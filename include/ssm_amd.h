@@ -353,12 +353,14 @@ typedef struct ssm_ssd_chunk_scan_args {
   const void *prev_states;  /* (B,nc,H,P,N) states dtype: state entering each chunk */
   const float *dt, *dA_cumsum; /* (B,H,nc,Q) */
   const float *Dskip;       /* (H,P) if d_per_p else (H,), or NULL */
-  void *y;                  /* (B,L,H,P) x dtype */
+  void *y;                  /* (B,L,H,P) x dtype (float32 if y_f32) */
   ssm_ssd_dims dims;
   int32_t x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype, d_per_p, force_generic;
   const int32_t *seq_idx;   /* (B,L) or NULL: the entering state only reaches steps whose sequence id equals that of
                                the last step of the chunk before (id 0 for the first chunk); CB must have been
                                formed with the same seq_idx */
+  int32_t y_f32;            /* nonzero: y is float32 whatever x's dtype is (the backward's running sums need the
+                               passes' results unrounded); 0: y has x's dtype */
 } ssm_ssd_chunk_scan_args;
 int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
 

@@ -147,7 +147,8 @@ class SsdChunkScanArgs(C.Structure):
     _fields_ = [("CB", _vp), ("Cm", _vp), ("x", _vp), ("z", _vp), ("prev_states", _vp), ("dt", _vp),
                 ("dA_cumsum", _vp), ("Dskip", _vp), ("y", _vp), ("dims", SsdDims),
                 ("x_dtype", _i32), ("c_dtype", _i32), ("cb_dtype", _i32), ("states_dtype", _i32),
-                ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32), ("seq_idx", _vp)]
+                ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32), ("seq_idx", _vp),
+                ("y_f32", _i32)]
 
 
 class SsdChunkStateVarlenArgs(C.Structure):

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_scan_kernel(const SsdSc
   const float xl = load_as_f32(p.x, p.x_dtype, gid);
   if (p.Dk) acc = __builtin_fmaf(p.Dk[p.d_per_p ? (size_t)h * d.hdim + pp : (size_t)h], xl, acc);
   if (p.z) acc *= silu_f32(load_as_f32(p.z, p.z_dtype, gid));
-  store_any(p.y, p.x_dtype, gid, acc);
+  store_any(p.y, p.y_dtype, gid, acc);
 }
 
 struct SsdVarlenParams {
@@ -300,7 +300,7 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   p.x_dtype = a->x_dtype; p.b_dtype = a->b_dtype; p.states_dtype = a->states_dtype;
   p.seq_idx = a->seq_idx;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  if (!a->force_generic && !a->seq_idx && ssd_chunk_state_mfma(p, s)) {
+  if (!a->force_generic && ssd_chunk_state_mfma(p, s)) {
     g_mfma_launches |= 2;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
     return SSM_OK;
@@ -350,8 +350,9 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   p.x_dtype = a->x_dtype; p.c_dtype = a->c_dtype; p.cb_dtype = a->cb_dtype; p.states_dtype = a->states_dtype;
   p.z_dtype = a->z_dtype; p.d_per_p = a->d_per_p ? 1 : 0;
   p.seq_idx = a->seq_idx;
+  p.y_dtype = a->y_f32 ? SSM_F32 : a->x_dtype;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  if (!a->force_generic && !a->seq_idx && ssd_chunk_scan_mfma(p, s)) {
+  if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
     g_mfma_launches |= 4;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
     return SSM_OK;

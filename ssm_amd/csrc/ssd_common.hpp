@@ -64,6 +64,7 @@ struct SsdScanParams {
   int x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype;
   int d_per_p;                // D is (H, P) instead of (H,)
   const int *seq_idx;         // (B, L) or null
+  int y_dtype;                // x_dtype, or SSM_F32 on request
 };
 
 __device__ __forceinline__ void store_any(void *p, int dtype, size_t i, float v) {

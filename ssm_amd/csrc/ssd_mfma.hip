@@ -130,7 +130,11 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const 
   const int g = h / (d.heads / d.groups);
   const size_t cs = (((size_t)b * d.heads + h) * d.nchunks + c) * Q;
   const float last = p.dA_cs[cs + Q - 1];
-  for (int l = threadIdx.x; l < Q; l += MF_THREADS) w[l] = decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
+  // packed sequences: steps of another sequence than the chunk's last step add nothing
+  const int *sid = p.seq_idx ? p.seq_idx + (size_t)b * d.len + (size_t)c * Q : nullptr;
+  const int sid_last = sid ? sid[Q - 1] : 0;
+  for (int l = threadIdx.x; l < Q; l += MF_THREADS)
+    w[l] = (sid && sid[l] != sid_last) ? 0.0f : decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
   __syncthreads();
   const __bf16 *xg = reinterpret_cast<const __bf16 *>(p.x) + (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
   stage_xT<true>(xT, xg, (size_t)d.heads * P, Q, P, w, stride);
@@ -173,15 +177,21 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   __bf16 *xT = reinterpret_cast<__bf16 *>(smem);                          // [P][Q + pad], unweighted
   float *dAs = reinterpret_cast<float *>(smem + (size_t)P * stride * 2);  // [Q]
   float *dts = dAs + Q;                                                   // [Q]
+  float *ent = dts + Q;                                                   // [Q] 1 where the entering state reaches the step
   const int wave = wave_id_uniform(), lane = lane_id();
   const int h = blockIdx.x % d.heads;
   const int c = (blockIdx.x / d.heads) % d.nchunks;
   const int b = blockIdx.x / (d.heads * d.nchunks);
   const int g = h / (d.heads / d.groups);
   const size_t cs = (((size_t)b * d.heads + h) * d.nchunks + c) * Q;
+  // packed sequences: the entering state belongs to the sequence of the last step before this chunk (id 0 at the
+  // start of the row); products across sequences inside the chunk are zero in CB already
+  const int *sid = p.seq_idx ? p.seq_idx + (size_t)b * d.len : nullptr;
+  const int sid_prev = (sid && c > 0) ? sid[(size_t)c * Q - 1] : 0;
   for (int l = threadIdx.x; l < Q; l += MF_THREADS) {
     dAs[l] = p.dA_cs[cs + l];
     dts[l] = p.dt[cs + l];
+    ent[l] = (sid && sid[(size_t)c * Q + l] != sid_prev) ? 0.0f : 1.0f;
   }
   const size_t xrow = (size_t)d.heads * P;                                 // elements between time steps
   const size_t xbase = (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
@@ -197,6 +207,8 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   const __bf16 *CBg = reinterpret_cast<const __bf16 *>(p.CB) + (((size_t)b * d.nchunks + c) * d.groups + g) * (size_t)Q * Q;
   const __bf16 *zg = p.z ? reinterpret_cast<const __bf16 *>(p.z) + xbase : nullptr;
   __bf16 *yg = reinterpret_cast<__bf16 *>(p.y) + xbase;
+  float *yf = reinterpret_cast<float *>(p.y) + xbase;
+  const bool y_f32 = p.y_dtype == SSM_F32;
 
   for (int pair = wave; pair < (nlb + 1) / 2; pair += MF_WAVES) {
     for (int side = 0; side < 2; ++side) {
@@ -228,7 +240,7 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float sc = exp2_hw(dAs[l0 + crow(r, g2)] * LOG2E);
+        const float sc = exp2_hw(dAs[l0 + crow(r, g2)] * LOG2E) * ent[l0 + crow(r, g2)];
 #pragma unroll
         for (int i = 0; i < PT; ++i) acc[i][r] *= sc;
       }
@@ -270,7 +282,8 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
           float v = acc[i][r];
           if (p.Dk) v = __builtin_fmaf(Dv, (float)xg[at], v);
           if (zg) v *= silu_f32((float)zg[at]);
-          yg[at] = (__bf16)v;
+          if (y_f32) yf[at] = v;
+          else yg[at] = (__bf16)v;
         }
       }
     }
@@ -328,7 +341,7 @@ bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s) {
   if (!mfma_shape_ok(d) || p.x_dtype != SSM_BF16 || p.c_dtype != SSM_BF16 || p.cb_dtype != SSM_BF16) return false;
   if (p.states_dtype == SSM_F16 || (p.z && p.z_dtype != SSM_BF16)) return false;
   if (!aligned_to(p.x, 16) || !aligned_to(p.Cm, 16) || !aligned_to(p.CB, 16) || !aligned_to(p.prev, 16)) return false;
-  const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 8;
+  const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 12;
   const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);
 #define SSM_LAUNCH_SC(ST, PT)                                                                              \
   {                                                                                                        \

@@ -220,7 +220,8 @@ def state_passing(states, dA_chunk_cumsum, initial_states=None, seq_idx=None, ch
     return out, final
 
 
-def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False, seq_idx=None):
+def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False, seq_idx=None,
+               out_f32=False):
     """Outputs of every chunk from the state entering it.
 
     Args:
@@ -234,9 +235,10 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         seq_idx: Optional ``(B, L)`` int sequence ids: the entering state only reaches steps
             whose id equals that of the last step of the chunk before (id 0 for the first
             chunk), and products across sequences inside a chunk are dropped.
+        out_f32: Return ``y`` in float32 (the accumulators as they are) instead of ``x.dtype``.
 
     Returns:
-        ``y (B, L, H, P)`` in ``x.dtype``.
+        ``y (B, L, H, P)`` in ``x.dtype`` (float32 with ``out_f32``).
     """
     batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
     _need(C.shape == B.shape, "B and C must have the same shape.")
@@ -262,14 +264,14 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
             K.check_float(name, t)
     ps, cb = K.cast_c(prev_states, prev_states.dtype), K.cast_c(CB, CB.dtype)
     dtf, daf, Df = K.as_f32_vec(dt), K.as_f32_vec(dA_cumsum), K.as_f32_vec(D)
-    y = torch.empty_like(xc)
+    y = torch.empty_like(xc, dtype=torch.float32) if out_f32 else torch.empty_like(xc)
     args = _lib.SsdChunkScanArgs(
         CB=_lib.ptr(cb), Cm=_lib.ptr(Cc), x=_lib.ptr(xc), z=_lib.ptr(zc), prev_states=_lib.ptr(ps),
         dt=_lib.ptr(dtf), dA_cumsum=_lib.ptr(daf), Dskip=_lib.ptr(Df), y=_lib.ptr(y),
         dims=_dims(batch, seqlen, heads, hdim, groups, nstate, Q), x_dtype=_lib.dtype_enum(xc.dtype),
         c_dtype=_lib.dtype_enum(Cc.dtype), cb_dtype=_lib.dtype_enum(cb.dtype),
         states_dtype=_lib.dtype_enum(ps.dtype), z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
-        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si))
+        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), y_f32=int(bool(out_f32)))
     _lib.call("ssm_ssd_chunk_scan", args, dev)
     return y
 
@@ -454,12 +456,25 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
     return outs[0] if len(outs) == 1 else tuple(outs)
 
 
-def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None):
+def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False):
     """``y_t = sum_{s<=t} exp(cs_t - cs_s) <C_t, B_s> w_s x_s + exp(cs_t) C_t . init`` and the state
-    after the last step, through chunk_state -> state_passing -> chunk_scan (float32)."""
+    after the last step, through chunk_state -> state_passing -> chunk_scan (states in float32).
+
+    Channels are independent of each other, so with bfloat16 operands a head dimension beyond 64 (the
+    backward's passes that put the state axis in the channel role) is cut into pieces of 64, the width
+    the matrix-core kernels are built for.  With ``want_entering`` the states entering the chunks
+    ``(B, nc, H, P, N)`` come back as a third result."""
+    hd = int(x.shape[-1])
+    if x.dtype == torch.bfloat16 and hd > 64 and hd % 64 == 0:
+        parts = [_lin_pass(x[..., k:k + 64].contiguous(), w_c, dA_cs, Bm, Cm,
+                           None if init is None else init[:, :, k:k + 64].contiguous(), want_entering)
+                 for k in range(0, hd, 64)]
+        out = (torch.cat([q[0] for q in parts], dim=-1), torch.cat([q[1] for q in parts], dim=2))
+        return out + (torch.cat([q[2] for q in parts], dim=3),) if want_entering else out
     states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32)
     entering, final = state_passing(states, dA_cs[:, :, :, -1].contiguous(), initial_states=init)
-    return chunk_scan(Bm, Cm, x, w_c, dA_cs, entering), final
+    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, out_f32=True)
+    return (y, final, entering) if want_entering else (y, final)
 
 
 def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
@@ -496,6 +511,10 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     f32 = torch.float32
     xf, Bf, Cf, Af = x.detach().to(f32), B.detach().to(f32), C.detach().to(f32), A.detach().to(f32)
     dof = dout.detach().to(f32)
+    # The passes take their operands in the inputs' precision when that is bfloat16 (matrix-core kernels,
+    # float32 accumulation and states); everything between the passes is float32 either way.
+    cd = torch.bfloat16 if (x.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and C.dtype == torch.bfloat16) else f32
+    xc, Bc, Cc = (x.detach(), B.detach(), C.detach()) if cd != f32 else (xf, Bf, Cf)
     Df = None if D is None else D.detach().to(f32)
     Dx = 0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * xf
     init = None if initial_states is None else initial_states.detach().to(f32)
@@ -507,7 +526,13 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     dA_cs, dt_c = chunk_cumsum(dt.detach(), Af, Q, dt_bias=None if dt_bias is None else dt_bias.detach(),
                                dt_softplus=dt_softplus, dt_limit=dt_limit)
     dte = blh(dt_c)                                                   # effective step
-    ypre, _ = _lin_pass(xf, dt_c, dA_cs, Bf, Cf, init)                # before skip and gate
+    # y before skip and gate.  The step enters through the operand (x~ = dt x, rounded once) rather than as a
+    # weight inside the kernels: then this pass and the reversed one below multiply the same rounded
+    # C.B-times-decay blocks, and the running sum that gives q (a difference of their row and column sums)
+    # sees each product twice with the same value instead of collecting the two passes' rounding noise.
+    _, ones_c = chunk_cumsum(torch.ones_like(dte), torch.zeros_like(Af), Q)
+    xt = (dte[..., None] * xf).to(cd)
+    ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
     if z is not None:
         zf = z.detach().to(f32)
         sg = torch.sigmoid(zf)
@@ -521,26 +546,38 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
     dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
     dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
-    _, ones_c = chunk_cumsum(torch.ones_like(dte), torch.zeros_like(Af), Q)
-    dyr = dy.flip(1).contiguous()
-    u_r, Gfin = _lin_pass(dyr, ones_c, dA_r, Cf.flip(1).contiguous(), Bf.flip(1).contiguous(), dfin)
+    dyc = dy.to(cd)
+    dyr = dyc.flip(1).contiguous()
+    u_r, Gfin, ent_r = _lin_pass(dyr, ones_c, dA_r, Cc.flip(1).contiguous(), Bc.flip(1).contiguous(), dfin,
+                                 want_entering=True)
     u = u_r.flip(1)
     dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin
     dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
-    Bh = Bf.repeat_interleave(per, dim=2) if per > 1 else Bf
-    Ch = Cf.repeat_interleave(per, dim=2) if per > 1 else Cf
-    v_r, _ = _lin_pass(Ch.flip(1).contiguous(), ones_c, dA_r, dyr, xf.flip(1).contiguous(),
+    Bh = Bc.repeat_interleave(per, dim=2) if per > 1 else Bc
+    Ch = Cc.repeat_interleave(per, dim=2) if per > 1 else Cc
+    v_r, _ = _lin_pass(Ch.flip(1).contiguous(), ones_c, dA_r, dyr, xc.flip(1).contiguous(),
                        None if dfin is None else dfin.transpose(2, 3).contiguous())
     dB = (dte[..., None] * v_r.flip(1)).view(batch, seqlen, groups, per, nstate).sum(3)
-    dCh, _ = _lin_pass(Bh.contiguous(), dt_c, dA_cs, xf, dy.contiguous(),
+    dCh, _ = _lin_pass(Bh.contiguous(), dt_c, dA_cs, xc, dyc.contiguous(),
                        None if init is None else init.transpose(2, 3).contiguous())
     dC = dCh.view(batch, seqlen, groups, per, nstate).sum(3)
     xu = (xf * u).sum(-1)                                             # (B, L, H)
-    s1 = dte * xu
-    s2 = (dy * ypre).sum(-1)
+    s1 = (xt.to(f32) * u).sum(-1)                  # with the rounded operand of the pass for y
+    s2 = (dyc.to(f32) * ypre).sum(-1)              # the same rounded dy that the pass for u saw
     W0 = (dinit * init).sum(dim=(2, 3)) if init is not None else torch.zeros(batch, heads, dtype=f32, device=x.device)
-    left = torch.cat([torch.zeros_like(s2[:, :1]), s2[:, :-1]], dim=1)
-    q = W0[:, None] + (s1 - left).cumsum(1) - s1
+    nc = (seqlen + Q - 1) // Q
+    if seqlen % Q == 0 and nc > 1:
+        # q at the first step of every chunk straight from the two passes' states at the chunk boundary
+        # (a_t <G_t, H_{t-1}>, float32), and from there the running sum inside the chunk only: what the
+        # two passes round differently then adds up over one chunk instead of the whole sequence.
+        a_first = torch.exp(dte[:, ::Q] * Af[None, None])                           # (B, nc, H)
+        anchor = (ent_r.flip(1)[:, :-1] * ent_f[:, 1:]).sum(dim=(3, 4))             # (B, nc-1, H): chunks 1..
+        anchor = torch.cat([W0[:, None], a_first[:, 1:] * anchor], dim=1)
+        dq = (s1 - s2).view(batch, nc, Q, heads)
+        q = (anchor[:, :, None] + dq.cumsum(2) - dq).reshape(batch, seqlen, heads)
+    else:
+        left = torch.cat([torch.zeros_like(s2[:, :1]), s2[:, :-1]], dim=1)
+        q = W0[:, None] + (s1 - left).cumsum(1) - s1
     ddte = Af[None, None] * q + xu
     dA = (dte * q).sum(dim=(0, 1))
     raw = dt.detach().to(f32) + (0.0 if dt_bias is None else dt_bias.detach().to(f32)[None, None])

@@ -179,14 +179,17 @@ def test_combined_varlen_vector():
     torch.testing.assert_close(vs.cpu(), rec["outputs"]["varlen_states"], **TF32)
 
 
-@pytest.mark.parametrize("Q,lens,dtype", [(4, [5, 9, 1, 6], torch.float32), (8, [3, 3, 10], torch.float32),
-                                          (64, [100, 28, 200, 56], torch.float32),
-                                          (64, [100, 28, 200, 56], torch.bfloat16)])
-def test_packed_sequences_match_the_oracle_and_separate_runs(Q, lens, dtype):
+@pytest.mark.parametrize("Q,lens,dtype,P", [(4, [5, 9, 1, 6], torch.float32, 16), (8, [3, 3, 10], torch.float32, 16),
+                                            (64, [100, 28, 200, 56], torch.float32, 16),
+                                            (64, [100, 28, 200, 56], torch.bfloat16, 16),
+                                            (64, [100, 28, 200, 56], torch.bfloat16, 64),
+                                            (128, [300, 1, 83, 128], torch.bfloat16, 32)])
+def test_packed_sequences_match_the_oracle_and_separate_runs(Q, lens, dtype, P):
     """seq_idx + cu_seqlens: against the float64 oracle, and sequence by sequence against
-    separate calls of the same kernels (the first sequence takes the initial state)."""
+    separate calls of the same kernels (the first sequence takes the initial state).  The cases
+    with 32 or 64 channels per head run the matrix-core kernels."""
     g = torch.Generator().manual_seed(13)
-    H, P, G, N = 4, 16, 2, 32
+    H, G, N = 4, 2, 32
     L = sum(lens)
     x = torch.randn(1, L, H, P, generator=g).to(dtype)
     dt = torch.rand(1, L, H, generator=g) * 0.5
@@ -200,10 +203,14 @@ def test_packed_sequences_match_the_oracle_and_separate_runs(Q, lens, dtype):
     for n in lens:
         cu_l.append(cu_l[-1] + n)
     seq_idx = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])[None]
+    from ssm_amd import _lib
+    _lib.load().ssm_ssd_mfma_launches()
     y, fin, vs = ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
                                     return_final_states=True, seq_idx=cu(seq_idx),
                                     cu_seqlens=torch.tensor(cu_l, dtype=torch.int32).cuda(),
                                     return_varlen_states=True, states_dtype=torch.float32)
+    used = _lib.load().ssm_ssd_mfma_launches()
+    assert (used & 6) == (6 if (dtype == torch.bfloat16 and P in (32, 64)) else 0)
     wy, wf, wv = S.ssd_combined(x, dt, A, Bm, Cm, Q, D=D, z=z, initial_states=init, clamp_decay=False,
                                 seq_idx=seq_idx, cu_seqlens=cu_l)
     tol = FP32_TOL if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2 * float(wy.abs().max()))
