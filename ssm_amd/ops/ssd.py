@@ -435,6 +435,25 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
     _need(not return_varlen_states or cu_seqlens is not None, "return_varlen_states needs cu_seqlens.")
     _need(cu_seqlens is None or batch == 1, "cu_seqlens describes one packed batch row: batch size must be 1.")
     packed = seq_idx is not None or return_varlen_states
+    if x.dtype == torch.bfloat16 and hdim > 64 and hdim % 64 == 0 and not force_generic:
+        # Channels of a head do not interact: a head of 64k channels is k heads of 64 with the same step,
+        # decay and group, which is the width the one-pass and matrix-core kernels are built for.  The
+        # channel axis is innermost, so this is a view of x, z and the states.
+        k = hdim // 64
+        rep = lambda t: None if t is None else t.repeat_interleave(k, dim=-1)
+        D2 = None if D is None else (D.repeat_interleave(k) if D.ndim == 1 else D.reshape(heads * k, 64))
+        out = _ssd_combined_forward(
+            x.reshape(batch, seqlen, heads * k, 64), rep(dt), rep(A), B, C, Q, D=D2,
+            z=None if z is None else z.reshape(batch, seqlen, heads * k, 64), dt_bias=rep(dt_bias),
+            initial_states=None if initial_states is None else initial_states.reshape(batch, heads * k, 64, nstate),
+            dt_softplus=dt_softplus, dt_limit=dt_limit, return_final_states=return_final_states,
+            states_dtype=states_dtype, fused=fused, seq_idx=seq_idx, cu_seqlens=cu_seqlens,
+            return_varlen_states=return_varlen_states)
+        outs = list(out) if isinstance(out, tuple) else [out]
+        outs[0] = outs[0].reshape(batch, seqlen, heads, hdim)
+        for i in range(1, len(outs)):                 # final states, per-sequence states: (.., H k, 64, N)
+            outs[i] = outs[i].reshape(outs[i].shape[0], heads, hdim, nstate)
+        return outs[0] if len(outs) == 1 else tuple(outs)
     can_fuse = not force_generic and fused is not False and not packed and \
         _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
     _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "

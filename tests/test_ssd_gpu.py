@@ -102,6 +102,7 @@ def _leaves(inp, names, dtype=None):
     ((2, 64, 4, 16, 4, 32), 16, torch.float32, False, True, True, True),
     ((2, 256, 4, 64, 1, 64), 64, torch.bfloat16, False, True, True, True),
     ((1, 512, 2, 64, 2, 128), 256, torch.bfloat16, True, True, False, True),
+    ((1, 256, 2, 128, 1, 64), 64, torch.bfloat16, False, True, True, True),
 ], ids=lambda v: str(v).replace(" ", ""))
 def test_combined_gradients_match_float64_autograd(shape, Q, dtype, d_mat, use_z, use_init, softplus):
     """All nine gradients of (y, final_states) against float64 autograd through the token-by-token
@@ -347,6 +348,33 @@ def test_one_pass_dt_bias_softplus_and_clamp():
     scale, fs = float(y64.abs().max()), float(f64.abs().max())
     torch.testing.assert_close(y.float().cpu().double(), y64, rtol=2e-2, atol=2e-2 * scale)
     torch.testing.assert_close(fin.cpu().double(), f64, rtol=2e-2, atol=2e-2 * fs)
+
+
+@pytest.mark.parametrize("shape,Q,d_mat", [((2, 512, 3, 128, 1, 128), 256, False), ((1, 256, 2, 192, 2, 64), 64, True)],
+                         ids=lambda v: str(v).replace(" ", ""))
+def test_wide_heads_run_as_heads_of_64_channels(shape, Q, d_mat):
+    """headdim 128 / 192 in bf16: the same result as the float64 recurrence, through the one-pass
+    kernel (a head of 64k channels is k heads of 64); packed sequences through the five kernels."""
+    b, l, h, p, g, n = shape
+    inp = make(5 + p, b, l, h, p, g, n, dtype=torch.bfloat16, d_mat=d_mat, use_z=True, use_init=True)
+    from ssm_amd import _lib
+    _lib.load().ssm_ssd_mfma_launches()
+    y, fin = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]),
+                                z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
+    assert _lib.load().ssm_ssd_mfma_launches() == 8
+    y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                                initial_states=inp["init"])
+    assert tuple(y.shape) == (b, l, h, p) and tuple(fin.shape) == (b, h, p, n)
+    torch.testing.assert_close(y.float().cpu().double(), y64, rtol=2e-2, atol=2e-2 * float(y64.abs().max()))
+    torch.testing.assert_close(fin.cpu().double(), f64, rtol=2e-2, atol=2e-2 * float(f64.abs().max()))
+    seq_idx = torch.zeros(b, l, dtype=torch.int32)
+    seq_idx[:, l // 3:] = 1
+    yp = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]),
+                            z=cu(inp["z"]), initial_states=cu(inp["init"]), seq_idx=cu(seq_idx))
+    wy = S.ssd_combined(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], Q, D=inp["D"], z=inp["z"],
+                        initial_states=inp["init"], clamp_decay=False, seq_idx=seq_idx)
+    wy = wy[0] if isinstance(wy, tuple) else wy
+    torch.testing.assert_close(yp.float().cpu(), wy.float(), rtol=2e-2, atol=2e-2 * float(wy.abs().max()))
 
 
 def test_one_pass_rejects_uncovered_calls():
