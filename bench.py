@@ -134,9 +134,42 @@ def bench_norm(batch=16, length=2048, hidden=768):
     us = _time_us(lambda i: ops._norm_forward(xs[i % 3], w, None, rs[i % 3], True, 1e-5, True, True,
                                               want_residual_out=True))
     nbytes = batch * length * hidden * (2 + 4 + 2 + 4)
+    # backward: reads x, residual, dy and the row statistics, writes dx and dresidual (+ dw)
+    _, _, mean, rstd = ops._norm_forward(xs[0], w, None, rs[0], True, 1e-5, True, True, want_stats=True)
+    gs = [torch.randn(batch, length, hidden, generator=g).to(torch.bfloat16).cuda() for _ in range(3)]
+    bus = _time_us(lambda i: ops._norm_backward(gs[i % 3], xs[0], w, rs[0], mean, rstd, True, True, False, True))
+    bbytes = batch * length * hidden * (2 + 4 + 2 + 2 + 4)
     return {"fwd_us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
             "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes,
+            "bwd_us": round(bus, 1), "bwd_GBps": round(bbytes / bus / 1e3, 1),
+            "bwd_frac_hbm": round(bbytes / bus / 1e3 / HBM_PEAK_GBPS, 4),
             "shape": "x bf16 (16,2048,768) + fp32 residual -> y bf16 + fp32 residual_out, RMSNorm"}
+
+
+def bench_dscan(batch=4, length=4096, heads=80, proj=64, chunk=256):
+    """The reference's own "SSD chunk scan" (an element-wise recurrence per (b, h, p)) at the outer
+    dimensions of config 3: bf16 X/z, per-token B/C of X's shape, per-head A and D."""
+    from ssm_amd import ops
+
+    g = torch.Generator().manual_seed(4)
+    X = torch.randn(batch, length, heads, proj, generator=g).to(torch.bfloat16).cuda()
+    dt = (torch.rand(batch, length, heads, generator=g) * 0.1).cuda()
+    A = -(torch.rand(heads, generator=g) * 15 + 1).cuda()
+    Bm = torch.randn(batch, length, heads, proj, generator=g).to(torch.bfloat16).cuda()
+    Cm = torch.randn(batch, length, heads, proj, generator=g).to(torch.bfloat16).cuda()
+    D = torch.ones(heads).cuda()
+    z = torch.randn(batch, length, heads, proj, generator=g).to(torch.bfloat16).cuda()
+    gy = torch.randn(batch, length, heads, proj, generator=g).to(torch.bfloat16).cuda()
+    fus = _time_us(lambda i: ops._dscan_forward(X, dt, A, Bm, Cm, chunk, D, z, None, None), iters=10)
+    bus = _time_us(lambda i: ops._dscan_backward(gy, X, dt, A, Bm, Cm, chunk, D, z, None, None), iters=10)
+    el = batch * length * heads * proj
+    fbytes = el * 2 * 5 + batch * length * heads * 4               # X, B, C, z in; Y out; dt
+    bbytes = el * 2 * 5 + el * 2 + el * 4 * 3 + batch * length * heads * 8   # + grad_y in; dX out; dB, dC, dz fp32 out
+    return {"fwd_us": round(fus, 1), "fwd_GBps": round(fbytes / fus / 1e3, 1),
+            "fwd_frac_hbm": round(fbytes / fus / 1e3 / HBM_PEAK_GBPS, 4),
+            "bwd_us": round(bus, 1), "bwd_GBps": round(bbytes / bus / 1e3, 1),
+            "bwd_frac_hbm": round(bbytes / bus / 1e3 / HBM_PEAK_GBPS, 4),
+            "shape": f"X (B={batch}, L={length}, H={heads}, P={proj}) bf16, chunk {chunk}"}
 
 
 def bench_decode(batch=64, dim=5120, nstate=16, width=4, steps=512):
@@ -316,7 +349,7 @@ def main():
                     help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
-                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "model"],
+                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
     args = ap.parse_args()
@@ -341,7 +374,7 @@ def main():
 
     if args.only:
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
-              "ssd": bench_ssd, "ssd_train": bench_ssd_train, "model": bench_model}[args.only]
+              "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model}[args.only]
         print(json.dumps({args.only: fn()}))
         return
 
@@ -383,6 +416,7 @@ def main():
         extra["dw_causal_conv_bf16"] = bench_conv()
         extra["fused_add_rmsnorm"] = bench_norm()
         extra["decode_step_config2"] = bench_decode()
+        extra["ssd_chunk_scan_diagonal"] = bench_dscan()
         extra["ssd_combined_config3"] = bench_ssd()
         extra["ssd_config3_backward_and_packed"] = bench_ssd_train()
         extra["mamba2_130m_style_model_config4"] = bench_model()

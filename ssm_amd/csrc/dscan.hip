@@ -13,9 +13,12 @@
 // small.  dt is used as given (no bias, no softplus), as in the reference.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace ssm {
 
 constexpr int DS_THREADS = 256;
+constexpr int DS_UNROLL = 8;         // time steps whose reads are in flight together
 
 struct DscanParams {
   const void *X, *dt, *Bp, *Cp, *z, *init;
@@ -38,7 +41,26 @@ __device__ __forceinline__ void ds_store(void *p, int dtype, size_t i, float v) 
   else reinterpret_cast<f16_t *>(p)[i] = from_f32<f16_t>(v);
 }
 
-template <int PASS>
+// Loads of the streamed tensors.  io_t = void: the element type is looked up at run time (any mix of
+// dtypes); otherwise X, B, C, z and Y all have type io_t and dt is float32, and the loads of a group of
+// steps are straight-line code that the compiler can issue together.
+template <typename io_t>
+__device__ __forceinline__ float ds_load(const void *p, int dtype, size_t i) {
+  if constexpr (std::is_void<io_t>::value) return load_as_f32(p, dtype, i);
+  else return to_f32(reinterpret_cast<const io_t *>(p)[i]);
+}
+template <typename io_t>
+__device__ __forceinline__ float ds_load_dt(const void *p, int dtype, size_t i) {
+  if constexpr (std::is_void<io_t>::value) return load_as_f32(p, dtype, i);
+  else return reinterpret_cast<const float *>(p)[i];
+}
+template <typename io_t>
+__device__ __forceinline__ void ds_store_y(void *p, int dtype, size_t i, float v) {
+  if constexpr (std::is_void<io_t>::value) ds_store(p, dtype, i, v);
+  else reinterpret_cast<io_t *>(p)[i] = from_f32<io_t>(v);
+}
+
+template <int PASS, typename io_t>
 __global__ __launch_bounds__(DS_THREADS) void dscan_kernel(const DscanParams p) {
   const int HP = p.heads * p.proj;
   const int hp = blockIdx.x * DS_THREADS + threadIdx.x;
@@ -52,16 +74,28 @@ __global__ __launch_bounds__(DS_THREADS) void dscan_kernel(const DscanParams p) 
   const size_t x_row = (size_t)b * p.len;            // + t, then * HP + hp
   const size_t fold_at = (((size_t)b * p.nseg + seg) * HP + hp) * 2;
 
+  // Time is walked DS_UNROLL steps at a time with all of a group's reads requested before the first is
+  // used: one step per trip leaves a wave waiting for memory at every step.
   if (PASS == 1) {
     float prod = 1.0f, s = 0.0f;
     const int stop = min(t_end, valid);
-    for (int t = t_begin; t < stop; ++t) {
-      const float dtv = load_as_f32(p.dt, p.dt_dtype, (x_row + t) * p.heads + h);
-      const float xv = load_as_f32(p.X, p.x_dtype, (x_row + t) * HP + hp);
-      const float bv = load_as_f32(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
-      const float a = exp2_hw(dtv * A2);
-      s = __builtin_fmaf(a, s, dtv * bv * xv);
-      prod *= a;
+    for (int t0 = t_begin; t0 < stop; t0 += DS_UNROLL) {
+      float dtv[DS_UNROLL], xv[DS_UNROLL], bv[DS_UNROLL];
+#pragma unroll
+      for (int j = 0; j < DS_UNROLL; ++j) {
+        const int t = min(t0 + j, stop - 1);
+        dtv[j] = ds_load_dt<io_t>(p.dt, p.dt_dtype, (x_row + t) * p.heads + h);
+        xv[j] = ds_load<io_t>(p.X, p.x_dtype, (x_row + t) * HP + hp);
+        bv[j] = ds_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
+      }
+#pragma unroll
+      for (int j = 0; j < DS_UNROLL; ++j) {
+        if (t0 + j < stop) {
+          const float a = exp2_hw(dtv[j] * A2);
+          s = __builtin_fmaf(a, s, dtv[j] * bv[j] * xv[j]);
+          prod *= a;
+        }
+      }
     }
     p.fold[fold_at] = prod;
     p.fold[fold_at + 1] = s;
@@ -75,26 +109,35 @@ __global__ __launch_bounds__(DS_THREADS) void dscan_kernel(const DscanParams p) 
     s = __builtin_fmaf(p.fold[f], s, p.fold[f + 1]);
   }
   const float Dk = p.Dk ? p.Dk[(size_t)h * (p.d_stride_p ? p.proj : 1) + (p.d_stride_p ? pp : 0)] : 0.0f;
-  for (int t = t_begin; t < t_end; ++t) {
-    const size_t xi = (x_row + t) * HP + hp;
-    float y = 0.0f;
-    if (t < valid) {
-      const float dtv = load_as_f32(p.dt, p.dt_dtype, (x_row + t) * p.heads + h);
-      const float xv = load_as_f32(p.X, p.x_dtype, xi);
-      const float bv = load_as_f32(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
-      const float cv = load_as_f32(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
-      s = __builtin_fmaf(exp2_hw(dtv * A2), s, dtv * bv * xv);
-      y = __builtin_fmaf(s, cv, Dk * xv);
-      if (p.z) {
-        const size_t zi = p.z_per_p ? xi : (x_row + t) * p.heads + h;
-        y *= silu_f32(load_as_f32(p.z, p.z_dtype, zi));
+  for (int t0 = t_begin; t0 < t_end; t0 += DS_UNROLL) {
+    float dtv[DS_UNROLL], xv[DS_UNROLL], bv[DS_UNROLL], cv[DS_UNROLL], zv[DS_UNROLL];
+#pragma unroll
+    for (int j = 0; j < DS_UNROLL; ++j) {
+      const int t = min(t0 + j, t_end - 1);
+      const size_t xi = (x_row + t) * HP + hp;
+      dtv[j] = ds_load_dt<io_t>(p.dt, p.dt_dtype, (x_row + t) * p.heads + h);
+      xv[j] = ds_load<io_t>(p.X, p.x_dtype, xi);
+      bv[j] = ds_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
+      cv[j] = ds_load<io_t>(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
+      zv[j] = p.z ? ds_load<io_t>(p.z, p.z_dtype, p.z_per_p ? xi : (x_row + t) * p.heads + h) : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < DS_UNROLL; ++j) {
+      const int t = t0 + j;
+      if (t < t_end) {
+        float y = 0.0f;
+        if (t < valid) {
+          s = __builtin_fmaf(exp2_hw(dtv[j] * A2), s, dtv[j] * bv[j] * xv[j]);
+          y = __builtin_fmaf(s, cv[j], Dk * xv[j]);
+          if (p.z) y *= silu_f32(zv[j]);
+        }
+        ds_store_y<io_t>(p.Y, p.x_dtype, (x_row + t) * HP + hp, y);
       }
     }
-    ds_store(p.Y, p.x_dtype, xi, y);
   }
 }
 
-static int dscan_segments(int batch, int len, int hp) {
+int dscan_segments(int batch, int len, int hp) {
   // enough (segment, channel-block) workgroups to cover ~4 per CU, segments of >= 32 steps
   const int blocks = (hp + DS_THREADS - 1) / DS_THREADS;
   int want = (1024 + batch * blocks - 1) / (batch * blocks);
@@ -156,8 +199,17 @@ extern "C" int ssm_dscan_fwd(const ssm_dscan_fwd_args *a, void *hip_stream) {
 
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid((unsigned)((HP + DS_THREADS - 1) / DS_THREADS), (unsigned)p.nseg, (unsigned)a->batch);
-  if (p.nseg > 1) hipLaunchKernelGGL(dscan_kernel<1>, grid, dim3(DS_THREADS), 0, s, p);
-  hipLaunchKernelGGL(dscan_kernel<2>, grid, dim3(DS_THREADS), 0, s, p);
+  const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
+#define SSM_DS_LAUNCH(T)                                                                   \
+  {                                                                                        \
+    if (p.nseg > 1) hipLaunchKernelGGL((dscan_kernel<1, T>), grid, dim3(DS_THREADS), 0, s, p); \
+    hipLaunchKernelGGL((dscan_kernel<2, T>), grid, dim3(DS_THREADS), 0, s, p);             \
+  }
+  if (typed && a->x_dtype == SSM_BF16) SSM_DS_LAUNCH(bf16_t)
+  else if (typed && a->x_dtype == SSM_F16) SSM_DS_LAUNCH(f16_t)
+  else if (typed && a->x_dtype == SSM_F32) SSM_DS_LAUNCH(float)
+  else SSM_DS_LAUNCH(void)
+#undef SSM_DS_LAUNCH
   SSM_CHECK_LAUNCH("ssm_dscan_fwd");
   return SSM_OK;
 }

@@ -8,14 +8,23 @@
 //   dC_t = g0_t s_t       dD += g0_t X_t      dX_t = g0_t D + lambda_t dt_t B_t      dB_t = lambda_t dt_t X_t
 //   ddt_t += lambda_t (s_{t-1} a_t A + B_t X_t)                 dA += lambda_t s_{t-1} a_t dt_t
 //   dinit = lambda_0 a_0
-// One thread per channel: a forward sweep stores the states, a reverse sweep
-// consumes them.  Everything that is a sum over channels, batch or time beyond
-// the thread's own loop is written as a partial and folded in a fixed order.
+// Time is cut into segments that run in parallel (as in the forward).  A first kernel folds every
+// (segment, channel) into three numbers: the product of its decays, the state it would reach from zero,
+// and the adjoint it would hand to the segment before it if nothing came in from the one after it
+// (mu_t = lambda_t a_t obeys mu_t = a_t mu_{t+1} + a_t g0_t C_t, the same decays).  The main kernel
+// rebuilds what enters a segment from both sides out of those folds, sweeps forward storing the
+// states, then sweeps backward producing every gradient.  Sums over channels, batch, segments or time
+// beyond a thread's own loop are written as partials and folded in a fixed order.
 #include "common.hpp"
+
+#include <type_traits>
 
 namespace ssm {
 
 constexpr int DB_THREADS = 256;
+constexpr int DB_UNROLL = 8;          // time steps whose reads are in flight together
+
+int dscan_segments(int batch, int len, int hp);   // dscan.hip: the forward's choice, reused here
 
 struct DscanBwdParams {
   const void *gy, *X, *dt, *Bp, *Cp, *z, *init;
@@ -23,16 +32,20 @@ struct DscanBwdParams {
   const int *lengths;
   void *dX;                       // (B,L,H,P) x dtype
   float *states;                  // (B,L,HP) scratch
-  float *ddt_p;                   // (B,L,HP) partial of ddt (summed over p afterwards)
+  float *ddt_p;                   // (B,L,HP) partial of ddt (summed over p afterwards); unused with ddt_direct
+  float *ddt_direct;              // (B,L,H): written by the kernel when a head is exactly one wavefront
   float *dz_p;                    // (B,L,HP): dz itself when z is per channel, else a partial
+  float *dz_direct;               // (B,L,H): per-head gate and a head is one wavefront
   float *dB_t, *dC_t;             // (B,L,HP) when the projection is time-varying, else null
-  float *pA, *pD, *pB, *pC;       // (B,HP) sums over time
+  float *fold;                    // (B, nseg, HP, 3): decay product, local state, local adjoint
+  float *pA, *pD, *pB, *pC;       // (B, nseg, HP) sums over the segment's steps
   float *dinit;                   // (B,HP) or null
   int batch, len, heads, proj;
   int x_dtype, dt_dtype, bc_dtype, z_dtype, init_dtype;
   int a_stride_p, d_stride_p;
   long long b_stride_b, b_stride_t, c_stride_b, c_stride_t;
   int z_per_p;
+  int seg_len, nseg;
 };
 
 __device__ __forceinline__ void db_store(void *p, int dtype, size_t i, float v) {
@@ -41,84 +54,210 @@ __device__ __forceinline__ void db_store(void *p, int dtype, size_t i, float v) 
   else reinterpret_cast<f16_t *>(p)[i] = from_f32<f16_t>(v);
 }
 
-__global__ __launch_bounds__(DB_THREADS) void dscan_bwd_kernel(const DscanBwdParams p) {
+// io_t = void: element types looked up at run time; otherwise gy, X, B, C, z and dX are io_t and dt is
+// float32, and the reads of a group of steps are straight-line code.
+template <typename io_t>
+__device__ __forceinline__ float db_load(const void *p, int dtype, size_t i) {
+  if constexpr (std::is_void<io_t>::value) return load_as_f32(p, dtype, i);
+  else return to_f32(reinterpret_cast<const io_t *>(p)[i]);
+}
+template <typename io_t>
+__device__ __forceinline__ float db_load_dt(const void *p, int dtype, size_t i) {
+  if constexpr (std::is_void<io_t>::value) return load_as_f32(p, dtype, i);
+  else return reinterpret_cast<const float *>(p)[i];
+}
+template <typename io_t>
+__device__ __forceinline__ void db_store_x(void *p, int dtype, size_t i, float v) {
+  if constexpr (std::is_void<io_t>::value) db_store(p, dtype, i, v);
+  else reinterpret_cast<io_t *>(p)[i] = from_f32<io_t>(v);
+}
+
+template <typename io_t>
+__global__ __launch_bounds__(DB_THREADS) void dscan_bwd_fold_kernel(const DscanBwdParams p) {
   const int HP = p.heads * p.proj;
   const int hp = blockIdx.x * DB_THREADS + threadIdx.x;
   if (hp >= HP) return;
-  const int b = blockIdx.y;
+  const int seg = blockIdx.y, b = blockIdx.z;
   const int h = hp / p.proj, pp = hp % p.proj;
   const int valid = p.lengths ? min(max(p.lengths[b], 0), p.len) : p.len;
+  const int t_begin = seg * p.seg_len;
+  const int stop = min(min(p.len, t_begin + p.seg_len), valid);
+  const float A2 = p.A[(size_t)h * (p.a_stride_p ? p.proj : 1) + (p.a_stride_p ? pp : 0)] * LOG2E;
+  const size_t row0 = (size_t)b * p.len;
+  float prod = 1.0f, s = 0.0f, M = 0.0f;
+  for (int t0 = t_begin; t0 < stop; t0 += DB_UNROLL) {
+    float dtv[DB_UNROLL], xv[DB_UNROLL], bv[DB_UNROLL], cv[DB_UNROLL], gv[DB_UNROLL], zv[DB_UNROLL];
+#pragma unroll
+    for (int j = 0; j < DB_UNROLL; ++j) {
+      const int t = min(t0 + j, stop - 1);
+      const size_t xi = (row0 + t) * HP + hp;
+      dtv[j] = db_load_dt<io_t>(p.dt, p.dt_dtype, (row0 + t) * p.heads + h);
+      xv[j] = db_load<io_t>(p.X, p.x_dtype, xi);
+      bv[j] = db_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
+      cv[j] = db_load<io_t>(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
+      gv[j] = db_load<io_t>(p.gy, p.x_dtype, xi);
+      zv[j] = p.z ? db_load<io_t>(p.z, p.z_dtype, p.z_per_p ? xi : (row0 + t) * p.heads + h) : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < DB_UNROLL; ++j) {
+      if (t0 + j < stop) {
+        const float a = exp2_hw(dtv[j] * A2);
+        s = __builtin_fmaf(a, s, dtv[j] * bv[j] * xv[j]);
+        prod *= a;                                          // product of the decays up to and including this step
+        const float g0 = p.z ? gv[j] * zv[j] * sigmoid_f32(zv[j]) : gv[j];
+        M = __builtin_fmaf(prod, g0 * cv[j], M);
+      }
+    }
+  }
+  float *f = p.fold + (((size_t)b * p.nseg + seg) * HP + hp) * 3;
+  f[0] = prod;
+  f[1] = s;
+  f[2] = M;
+}
+
+template <typename io_t>
+__global__ __launch_bounds__(DB_THREADS) void dscan_bwd_kernel(const DscanBwdParams p) {
+  const int HP = p.heads * p.proj;
+  const int hp = blockIdx.x * DB_THREADS + threadIdx.x;
+  // whole wavefronts leave together (the sums over a head below use every lane of a wavefront)
+  if (hp >= HP) return;
+  const int seg = blockIdx.y, b = blockIdx.z;
+  const int h = hp / p.proj, pp = hp % p.proj;
+  const int valid = p.lengths ? min(max(p.lengths[b], 0), p.len) : p.len;
+  const int t_begin = seg * p.seg_len;
+  const int t_end = min(p.len, t_begin + p.seg_len);
+  const int stop = min(t_end, valid);
   const float A = p.A[(size_t)h * (p.a_stride_p ? p.proj : 1) + (p.a_stride_p ? pp : 0)];
+  const float A2 = A * LOG2E;
   const float Dk = p.Dk ? p.Dk[(size_t)h * (p.d_stride_p ? p.proj : 1) + (p.d_stride_p ? pp : 0)] : 0.0f;
   const size_t row0 = (size_t)b * p.len;
-  const float s_init = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + hp) : 0.0f;
+  const int lane = threadIdx.x & 63;
+
+  // what enters the segment: the state from the left, the adjoint (times its decay) from the right
+  float s_in = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + hp) : 0.0f;
+  for (int j = 0; j < seg; ++j) {
+    const float *f = p.fold + (((size_t)b * p.nseg + j) * HP + hp) * 3;
+    s_in = __builtin_fmaf(f[0], s_in, f[1]);
+  }
+  float mu_in = 0.0f;
+  for (int j = p.nseg - 1; j > seg; --j) {
+    const float *f = p.fold + (((size_t)b * p.nseg + j) * HP + hp) * 3;
+    mu_in = __builtin_fmaf(f[0], mu_in, f[2]);
+  }
 
   // forward sweep: states[t] = s_t
-  float s = s_init;
-  for (int t = 0; t < valid; ++t) {
-    const float dtv = load_as_f32(p.dt, p.dt_dtype, (row0 + t) * p.heads + h);
-    const float xv = load_as_f32(p.X, p.x_dtype, (row0 + t) * HP + hp);
-    const float bv = load_as_f32(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
-    s = __builtin_fmaf(exp2_hw(dtv * A * LOG2E), s, dtv * bv * xv);
-    p.states[(row0 + t) * HP + hp] = s;
+  float s = s_in;
+  for (int t0 = t_begin; t0 < stop; t0 += DB_UNROLL) {
+    float dtv[DB_UNROLL], xv[DB_UNROLL], bv[DB_UNROLL];
+#pragma unroll
+    for (int j = 0; j < DB_UNROLL; ++j) {
+      const int t = min(t0 + j, stop - 1);
+      dtv[j] = db_load_dt<io_t>(p.dt, p.dt_dtype, (row0 + t) * p.heads + h);
+      xv[j] = db_load<io_t>(p.X, p.x_dtype, (row0 + t) * HP + hp);
+      bv[j] = db_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
+    }
+#pragma unroll
+    for (int j = 0; j < DB_UNROLL; ++j) {
+      if (t0 + j < stop) {
+        s = __builtin_fmaf(exp2_hw(dtv[j] * A2), s, dtv[j] * bv[j] * xv[j]);
+        p.states[(row0 + t0 + j) * HP + hp] = s;
+      }
+    }
   }
   // steps past the end contribute nothing
-  for (int t = valid; t < p.len; ++t) {
+  for (int t = max(stop, t_begin); t < t_end; ++t) {
     const size_t xi = (row0 + t) * HP + hp;
-    db_store(p.dX, p.x_dtype, xi, 0.0f);
-    p.ddt_p[xi] = 0.0f;
-    if (p.dz_p) p.dz_p[xi] = 0.0f;
+    db_store_x<io_t>(p.dX, p.x_dtype, xi, 0.0f);
+    if (p.ddt_direct) { if (pp == 0) p.ddt_direct[(row0 + t) * p.heads + h] = 0.0f; }
+    else p.ddt_p[xi] = 0.0f;
+    if (p.dz_direct) { if (pp == 0) p.dz_direct[(row0 + t) * p.heads + h] = 0.0f; }
+    else if (p.dz_p) p.dz_p[xi] = 0.0f;
     if (p.dB_t) p.dB_t[xi] = 0.0f;
     if (p.dC_t) p.dC_t[xi] = 0.0f;
   }
 
   // reverse sweep
-  float lam_next_a = 0.0f;          // lambda_{t+1} a_{t+1}
+  float lam_next_a = mu_in;         // lambda_{t+1} a_{t+1}
   float accA = 0.0f, accD = 0.0f, accB = 0.0f, accC = 0.0f;
-  for (int t = valid - 1; t >= 0; --t) {
-    const size_t xi = (row0 + t) * HP + hp;
-    const float dtv = load_as_f32(p.dt, p.dt_dtype, (row0 + t) * p.heads + h);
-    const float xv = load_as_f32(p.X, p.x_dtype, xi);
-    const float bv = load_as_f32(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
-    const float cv = load_as_f32(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
-    const float st = p.states[xi];
-    const float sprev = t > 0 ? p.states[xi - HP] : s_init;
-    const float a = exp2_hw(dtv * A * LOG2E);
-    const float gy = load_as_f32(p.gy, p.x_dtype, xi);
-    float g0 = gy;
-    if (p.z) {
-      const size_t zi = p.z_per_p ? xi : (row0 + t) * p.heads + h;
-      const float zv = load_as_f32(p.z, p.z_dtype, zi);
-      const float sg = sigmoid_f32(zv);
-      const float y0 = __builtin_fmaf(st, cv, Dk * xv);
-      p.dz_p[xi] = gy * y0 * sg * (1.0f + zv * (1.0f - sg));
-      g0 = gy * zv * sg;
+  for (int t1 = stop - 1; t1 >= t_begin; t1 -= DB_UNROLL) {
+    float dtv[DB_UNROLL], xv[DB_UNROLL], bv[DB_UNROLL], cv[DB_UNROLL], gv[DB_UNROLL], zv[DB_UNROLL];
+    float st[DB_UNROLL + 1];        // st[j] = s_{t1 - j}, st[UNROLL] = the state before the group's first step
+#pragma unroll
+    for (int j = 0; j < DB_UNROLL; ++j) {
+      const int t = max(t1 - j, t_begin);
+      const size_t xi = (row0 + t) * HP + hp;
+      dtv[j] = db_load_dt<io_t>(p.dt, p.dt_dtype, (row0 + t) * p.heads + h);
+      xv[j] = db_load<io_t>(p.X, p.x_dtype, xi);
+      bv[j] = db_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
+      cv[j] = db_load<io_t>(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
+      gv[j] = db_load<io_t>(p.gy, p.x_dtype, xi);
+      zv[j] = p.z ? db_load<io_t>(p.z, p.z_dtype, p.z_per_p ? xi : (row0 + t) * p.heads + h) : 0.0f;
+      st[j] = p.states[xi];
     }
-    const float lam = __builtin_fmaf(g0, cv, lam_next_a);
-    db_store(p.dX, p.x_dtype, xi, __builtin_fmaf(g0, Dk, lam * dtv * bv));
-    p.ddt_p[xi] = lam * __builtin_fmaf(sprev * a, A, bv * xv);
-    const float gB = lam * dtv * xv, gC = g0 * st;
-    if (p.dB_t) p.dB_t[xi] = gB; else accB += gB;
-    if (p.dC_t) p.dC_t[xi] = gC; else accC += gC;
-    accA = __builtin_fmaf(lam * sprev, a * dtv, accA);
-    accD = __builtin_fmaf(g0, xv, accD);
-    lam_next_a = lam * a;
+    {
+      const int t = t1 - DB_UNROLL;
+      st[DB_UNROLL] = t >= t_begin ? p.states[(row0 + t) * HP + hp] : s_in;
+    }
+#pragma unroll
+    for (int j = 0; j < DB_UNROLL; ++j) {
+      const int t = t1 - j;
+      if (t >= t_begin) {                       // uniform over the workgroup
+        const size_t xi = (row0 + t) * HP + hp;
+        const float sprev = t > t_begin ? st[j + 1] : s_in;
+        const float a = exp2_hw(dtv[j] * A2);
+        float g0 = gv[j];
+        if (p.z) {
+          const float sg = sigmoid_f32(zv[j]);
+          const float y0 = __builtin_fmaf(st[j], cv[j], Dk * xv[j]);
+          const float dzv = gv[j] * y0 * sg * (1.0f + zv[j] * (1.0f - sg));
+          if (p.dz_direct) {
+            const float tot = wave_sum(dzv);
+            if (lane == 0) p.dz_direct[(row0 + t) * p.heads + h] = tot;
+          } else {
+            p.dz_p[xi] = dzv;
+          }
+          g0 = gv[j] * zv[j] * sg;
+        }
+        const float lam = __builtin_fmaf(g0, cv[j], lam_next_a);
+        db_store_x<io_t>(p.dX, p.x_dtype, xi, __builtin_fmaf(g0, Dk, lam * dtv[j] * bv[j]));
+        const float ddtv = lam * __builtin_fmaf(sprev * a, A, bv[j] * xv[j]);
+        if (p.ddt_direct) {
+          const float tot = wave_sum(ddtv);
+          if (lane == 0) p.ddt_direct[(row0 + t) * p.heads + h] = tot;
+        } else {
+          p.ddt_p[xi] = ddtv;
+        }
+        const float gB = lam * dtv[j] * xv[j], gC = g0 * st[j];
+        if (p.dB_t) p.dB_t[xi] = gB; else accB += gB;
+        if (p.dC_t) p.dC_t[xi] = gC; else accC += gC;
+        accA = __builtin_fmaf(lam * sprev, a * dtv[j], accA);
+        accD = __builtin_fmaf(g0, xv[j], accD);
+        lam_next_a = lam * a;
+      }
+    }
   }
-  const size_t bi = (size_t)b * HP + hp;
+  const size_t bi = ((size_t)b * p.nseg + seg) * HP + hp;
   p.pA[bi] = accA;
   p.pD[bi] = accD;
   p.pB[bi] = accB;
   p.pC[bi] = accC;
-  if (p.dinit) p.dinit[bi] = lam_next_a;
+  if (p.dinit && seg == 0) p.dinit[(size_t)b * HP + hp] = lam_next_a;
 }
 
 }  // namespace ssm
 
-// Workspace (floats): states, ddt partial, dz partial, dB/dC time-varying copies are outputs
-// themselves; then four (B,HP) partials.
+// Workspace (floats): states, ddt partial, dz partial (dB/dC time-varying copies are outputs
+// themselves); then per (batch, segment, channel) the three folds and four partial sums.
+static void dscan_bwd_segments(int batch, int seqlen, int heads, int proj, int &seg_len, int &nseg) {
+  nseg = ssm::dscan_segments(batch, seqlen, heads * proj);
+  seg_len = (seqlen + nseg - 1) / nseg;
+  nseg = (seqlen + seg_len - 1) / seg_len;
+}
 static size_t dscan_bwd_floats(int batch, int seqlen, int heads, int proj) {
-  const size_t blhp = (size_t)batch * seqlen * heads * proj, bhp = (size_t)batch * heads * proj;
-  return 3 * blhp + 4 * bhp;
+  int seg_len, nseg;
+  dscan_bwd_segments(batch, seqlen, heads, proj, seg_len, nseg);
+  const size_t blhp = (size_t)batch * seqlen * heads * proj, bshp = (size_t)batch * nseg * heads * proj;
+  return 3 * blhp + 7 * bshp;
 }
 
 extern "C" size_t ssm_dscan_bwd_workspace_bytes(int batch, int seqlen, int heads, int proj) {
@@ -152,7 +291,9 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
 
   const int Bn = a->batch, L = a->seqlen, H = a->heads, P = a->proj;
   const long long HP = (long long)H * P;
-  const size_t blhp = (size_t)Bn * L * HP, bhp = (size_t)Bn * HP;
+  int seg_len, nseg;
+  dscan_bwd_segments(Bn, L, H, P, seg_len, nseg);
+  const size_t blhp = (size_t)Bn * L * HP, bhp = (size_t)Bn * HP, bshp = bhp * nseg;
   float *ws = reinterpret_cast<float *>(a->workspace);
   DscanBwdParams p{};
   p.gy = a->grad_y; p.X = a->X; p.dt = a->dt; p.Bp = a->Bproj; p.Cp = a->Cproj; p.z = a->z; p.init = a->initial_states;
@@ -162,8 +303,14 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   p.dz_p = !a->z ? nullptr : (dz_direct ? a->dz : ws + 2 * blhp);
   p.dB_t = a->b_kind == SSM_CHUNK_BLHP ? a->dB : nullptr;
   p.dC_t = a->c_kind == SSM_CHUNK_BLHP ? a->dC : nullptr;
-  p.pA = ws + 3 * blhp; p.pD = p.pA + bhp; p.pB = p.pD + bhp; p.pC = p.pB + bhp;
+  p.fold = ws + 3 * blhp;
+  p.pA = p.fold + 3 * bshp; p.pD = p.pA + bshp; p.pB = p.pD + bshp; p.pC = p.pB + bshp;
   p.dinit = a->dinitial_states;
+  p.seg_len = seg_len; p.nseg = nseg;
+  // a head of 64 channels is one wavefront: the sums over p are taken in the kernel
+  const bool wave_heads = P == WAVE;
+  p.ddt_direct = wave_heads ? a->ddt : nullptr;
+  p.dz_direct = (wave_heads && a->z && !a->z_per_p) ? a->dz : nullptr;
   p.batch = Bn; p.len = L; p.heads = H; p.proj = P;
   p.x_dtype = a->x_dtype; p.dt_dtype = a->dt_dtype; p.bc_dtype = a->bc_dtype; p.z_dtype = a->z_dtype;
   p.init_dtype = a->init_dtype;
@@ -178,28 +325,38 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   p.z_per_p = a->z_per_p ? 1 : 0;
 
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  const dim3 grid((unsigned)((HP + DB_THREADS - 1) / DB_THREADS), (unsigned)Bn);
-  hipLaunchKernelGGL(dscan_bwd_kernel, grid, dim3(DB_THREADS), 0, s, p);
+  const dim3 grid((unsigned)((HP + DB_THREADS - 1) / DB_THREADS), (unsigned)nseg, (unsigned)Bn);
+  const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
+#define SSM_DB_LAUNCH(T)                                                                       \
+  {                                                                                            \
+    if (nseg > 1) hipLaunchKernelGGL(dscan_bwd_fold_kernel<T>, grid, dim3(DB_THREADS), 0, s, p); \
+    hipLaunchKernelGGL(dscan_bwd_kernel<T>, grid, dim3(DB_THREADS), 0, s, p);                  \
+  }
+  if (typed && a->x_dtype == SSM_BF16) SSM_DB_LAUNCH(bf16_t)
+  else if (typed && a->x_dtype == SSM_F16) SSM_DB_LAUNCH(f16_t)
+  else if (typed && a->x_dtype == SSM_F32) SSM_DB_LAUNCH(float)
+  else SSM_DB_LAUNCH(void)
+#undef SSM_DB_LAUNCH
   SSM_CHECK_LAUNCH("ssm_dscan_bwd");
 
-  // ddt (B,L,H) and, for a per-head gate, dz (B,L,H): sums over p
-  launch_fold_sum(p.ddt_p, a->ddt, (size_t)Bn * L * H, P, 1, s);
-  if (a->z && !dz_direct) launch_fold_sum(p.dz_p, a->dz, (size_t)Bn * L * H, P, 1, s);
-  // sums over batch, then over p when the parameter is per head; `states` is free again and
-  // serves as the (H,P) intermediate
+  // ddt (B,L,H) and, for a per-head gate, dz (B,L,H): sums over p, unless the kernel took them itself
+  if (!p.ddt_direct) launch_fold_sum(p.ddt_p, a->ddt, (size_t)Bn * L * H, P, 1, s);
+  if (a->z && !dz_direct && !p.dz_direct) launch_fold_sum(p.dz_p, a->dz, (size_t)Bn * L * H, P, 1, s);
+  // sums over batch and segments, then over p when the parameter is per head; `states` is free again
+  // and serves as the (H,P) intermediate
   float *tmp = p.states;
   auto fold_param = [&](const float *partial, float *out, bool per_p) {
-    if (per_p) launch_fold_rows(partial, out, Bn, (size_t)HP, s);
+    if (per_p) launch_fold_rows(partial, out, Bn * nseg, (size_t)HP, s);
     else {
-      launch_fold_rows(partial, tmp, Bn, (size_t)HP, s);
+      launch_fold_rows(partial, tmp, Bn * nseg, (size_t)HP, s);
       launch_fold_sum(tmp, out, (size_t)H, P, 1, s);
     }
   };
   fold_param(p.pA, a->dA, a->a_per_p != 0);
   if (a->dD) fold_param(p.pD, a->dD, a->d_per_p != 0);
   auto fold_proj = [&](int kind, const float *partial, float *out) {
-    if (kind == SSM_CHUNK_HP) launch_fold_rows(partial, out, Bn, (size_t)HP, s);
-    else if (kind == SSM_CHUNK_BHP) launch_fold_rows(partial, out, 1, bhp, s);
+    if (kind == SSM_CHUNK_HP) launch_fold_rows(partial, out, Bn * nseg, (size_t)HP, s);
+    else if (kind == SSM_CHUNK_BHP) launch_fold_sum(partial, out, (size_t)Bn, nseg, (size_t)HP, s);
   };
   fold_proj(a->b_kind, p.pB, a->dB);
   fold_proj(a->c_kind, p.pC, a->dC);

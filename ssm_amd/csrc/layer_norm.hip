@@ -254,16 +254,36 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
       if (p.dres) store_cols<VEC>(p.dres, p.res_dtype, base, col, H, vok, p.prenorm ? dxv : dyv[k]);
     }
   }
-  float *pw = p.partial + (size_t)gw * 2 * H;
+  // one partial per workgroup: waves 1.. hand their column sums to wave 0 through LDS (fixed order)
+  __shared__ float wsum[LN_WAVES - 1][2][TRIPS * WAVE * VEC];
+  if (wave > 0) {
 #pragma unroll
-  for (int k = 0; k < TRIPS; ++k) {
-    const int col = (k * WAVE + lane) * VEC;
+    for (int k = 0; k < TRIPS; ++k) {
+      const int col = (k * WAVE + lane) * VEC;
+      *reinterpret_cast<float4 *>(&wsum[wave - 1][0][col]) = make_float4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
+      *reinterpret_cast<float4 *>(&wsum[wave - 1][1][col]) = make_float4(db[k][0], db[k][1], db[k][2], db[k][3]);
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float *pw = p.partial + (size_t)blockIdx.x * 2 * H;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i)
-      if (col + i < H) {
-        pw[col + i] = dw[k][i];
-        pw[H + col + i] = db[k][i];
+    for (int k = 0; k < TRIPS; ++k) {
+      const int col = (k * WAVE + lane) * VEC;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float a = dw[k][i], b = db[k][i];
+#pragma unroll
+        for (int w = 0; w < LN_WAVES - 1; ++w) {
+          a += wsum[w][0][col + i];
+          b += wsum[w][1][col + i];
+        }
+        if (col + i < H) {
+          pw[col + i] = a;
+          pw[H + col + i] = b;
+        }
       }
+    }
   }
 }
 
@@ -305,18 +325,33 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_long_kernel(const NormPar
   }
 }
 
-// dw[c] = sum_w partial[w][0][c], db[c] = sum_w partial[w][1][c]
+// dw[c] = sum_w partial[w][0][c], db[c] = sum_w partial[w][1][c].  A workgroup takes 16 columns; its 256
+// threads are 16 columns x 16 slices of the partials, summed in a fixed order (slice by slice, then over slices).
+constexpr int FOLD_COLS = 16, FOLD_SLICES = LN_THREADS / FOLD_COLS;
 __global__ __launch_bounds__(LN_THREADS) void norm_bwd_fold_kernel(const float *partial, float *dw, float *db,
-                                                                    int nwaves, int hidden) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= hidden) return;
+                                                                    int nparts, int hidden) {
+  __shared__ float sw_s[FOLD_SLICES][FOLD_COLS], sb_s[FOLD_SLICES][FOLD_COLS];
+  const int cl = threadIdx.x % FOLD_COLS, sl = threadIdx.x / FOLD_COLS;
+  const int c = blockIdx.x * FOLD_COLS + cl;
   float sw = 0.0f, sb = 0.0f;
-  for (int w = 0; w < nwaves; ++w) {
-    sw += partial[(size_t)w * 2 * hidden + c];
-    sb += partial[(size_t)w * 2 * hidden + hidden + c];
+  if (c < hidden) {
+    for (int w = sl; w < nparts; w += FOLD_SLICES) {
+      sw += partial[(size_t)w * 2 * hidden + c];
+      sb += partial[(size_t)w * 2 * hidden + hidden + c];
+    }
   }
-  dw[c] = sw;
-  if (db) db[c] = sb;
+  sw_s[sl][cl] = sw;
+  sb_s[sl][cl] = sb;
+  __syncthreads();
+  if (sl == 0 && c < hidden) {
+    float a = 0.0f, b = 0.0f;
+    for (int j = 0; j < FOLD_SLICES; ++j) {
+      a += sw_s[j][cl];
+      b += sb_s[j][cl];
+    }
+    dw[c] = a;
+    if (db) db[c] = b;
+  }
 }
 
 static int norm_bwd_grid(int rows) {
@@ -405,9 +440,9 @@ extern "C" int ssm_norm_bwd(const ssm_norm_bwd_args *a, void *hip_stream) {
   else if (per_lane <= 16) hipLaunchKernelGGL(norm_bwd_kernel<4>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
   else hipLaunchKernelGGL(norm_bwd_long_kernel, dim3(grid), dim3(LN_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_norm_bwd");
-  const int nwaves = grid * LN_WAVES;
-  hipLaunchKernelGGL(norm_bwd_fold_kernel, dim3((a->hidden + LN_THREADS - 1) / LN_THREADS), dim3(LN_THREADS), 0, s,
-                     p.partial, a->dweight, a->dbias, nwaves, a->hidden);
+  const int nparts = per_lane <= 16 ? grid : grid * LN_WAVES;      // the long-row kernel writes one per wave
+  hipLaunchKernelGGL(norm_bwd_fold_kernel, dim3((a->hidden + FOLD_COLS - 1) / FOLD_COLS), dim3(LN_THREADS), 0, s,
+                     p.partial, a->dweight, a->dbias, nparts, a->hidden);
   SSM_CHECK_LAUNCH("ssm_norm_bwd(fold)");
   return SSM_OK;
 }
