@@ -210,6 +210,17 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), WAVE - 1));
 }
 
+// Running sum over the lanes: lane l ends with the sum of lanes 0..l (the same steps as wave_sum).
+__device__ __forceinline__ float wave_inclusive_sum(float v) {
+  v += dpp_move<DPP_ROW_SHR1, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR2, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR4, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR8, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.0f, v);
+  v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.0f, v);
+  return v;
+}
+
 __device__ __forceinline__ int wave_id_uniform() {
   return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 }

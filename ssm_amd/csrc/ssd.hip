@@ -26,30 +26,36 @@ static unsigned grid_for(size_t n) {
   return (unsigned)(g < 1 ? 1 : g);
 }
 
-// One thread per (b, h, c): sequential running sum over the chunk.
+// One wavefront per (b, h, c): 64 steps at a time, running sum by a DPP scan across the lanes plus the
+// carry of the blocks before; reads and writes are contiguous runs.
 __global__ __launch_bounds__(SSD_THREADS) void ssd_cumsum_kernel(const SsdCumsumParams p) {
   const SsdDims &d = p.d;
-  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t gw = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int lane = lane_id();
   const size_t total = (size_t)d.batch * d.heads * d.nchunks;
-  if (gid >= total) return;
-  const int c = (int)(gid % d.nchunks);
-  const int h = (int)((gid / d.nchunks) % d.heads);
-  const int b = (int)(gid / ((size_t)d.nchunks * d.heads));
+  if (gw >= total) return;                          // whole wavefronts
+  const int c = (int)(gw % d.nchunks);
+  const int h = (int)((gw / d.nchunks) % d.heads);
+  const int b = (int)(gw / ((size_t)d.nchunks * d.heads));
   const float A = p.A[h];
   const float bias = p.bias ? p.bias[h] : 0.0f;
-  float run = 0.0f;
+  float carry = 0.0f;
   const size_t out = (((size_t)b * d.heads + h) * d.nchunks + c) * d.chunk;
-  for (int l = 0; l < d.chunk; ++l) {
+  for (int l0 = 0; l0 < d.chunk; l0 += WAVE) {
+    const int l = l0 + lane;
     const int t = c * d.chunk + l;
     float v = 0.0f;
-    if (t < d.len) {
+    if (l < d.chunk && t < d.len) {
       v = load_as_f32(p.dt, p.dt_dtype, ((size_t)b * d.len + t) * d.heads + h) + bias;
       if (p.softplus) v = softplus_f32(v);
       v = fminf(fmaxf(v, p.dt_min), p.dt_max);
     }
-    run = __builtin_fmaf(v, A, run);
-    p.dt_out[out + l] = v;
-    p.dA_cs[out + l] = run;
+    const float run = carry + wave_inclusive_sum(v * A);
+    if (l < d.chunk) {
+      p.dt_out[out + l] = v;
+      p.dA_cs[out + l] = run;
+    }
+    carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(run), WAVE - 1));
   }
 }
 
@@ -248,7 +254,7 @@ extern "C" int ssm_ssd_chunk_cumsum(const ssm_ssd_cumsum_args *a, void *hip_stre
   p.dt = a->dt; p.A = a->A; p.bias = a->dt_bias; p.dA_cs = a->dA_cumsum; p.dt_out = a->dt_out;
   p.dt_dtype = a->dt_dtype; p.softplus = a->dt_softplus ? 1 : 0; p.dt_min = a->dt_min; p.dt_max = a->dt_max;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(grid_for((size_t)p.d.batch * p.d.heads * p.d.nchunks)),
+  hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(grid_for((size_t)p.d.batch * p.d.heads * p.d.nchunks * WAVE)),
                      dim3(SSD_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_chunk_cumsum");
   return SSM_OK;

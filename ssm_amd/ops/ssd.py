@@ -475,7 +475,7 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
     return outs[0] if len(outs) == 1 else tuple(outs)
 
 
-def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False):
+def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None):
     """``y_t = sum_{s<=t} exp(cs_t - cs_s) <C_t, B_s> w_s x_s + exp(cs_t) C_t . init`` and the state
     after the last step, through chunk_state -> state_passing -> chunk_scan (states in float32).
 
@@ -485,14 +485,16 @@ def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False):
     ``(B, nc, H, P, N)`` come back as a third result."""
     hd = int(x.shape[-1])
     if x.dtype == torch.bfloat16 and hd > 64 and hd % 64 == 0:
+        Q = int(dA_cs.shape[3])
+        CB = bmm_chunk(Cm, Bm, Q, causal=True, output_dtype=x.dtype)          # the same for every piece
         parts = [_lin_pass(x[..., k:k + 64].contiguous(), w_c, dA_cs, Bm, Cm,
-                           None if init is None else init[:, :, k:k + 64].contiguous(), want_entering)
+                           None if init is None else init[:, :, k:k + 64].contiguous(), want_entering, CB=CB)
                  for k in range(0, hd, 64)]
         out = (torch.cat([q[0] for q in parts], dim=-1), torch.cat([q[1] for q in parts], dim=2))
         return out + (torch.cat([q[2] for q in parts], dim=3),) if want_entering else out
     states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32)
     entering, final = state_passing(states, dA_cs[:, :, :, -1].contiguous(), initial_states=init)
-    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, out_f32=True)
+    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, CB=CB, out_f32=True)
     return (y, final, entering) if want_entering else (y, final)
 
 
