@@ -254,6 +254,134 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
   }
 }
 
+// ---------------------------------------------------------------- backward, (B,L,C)
+// A thread owns 16 bytes of channels over one time segment and walks it once: x and dout of a step are
+// read, the pre-activation rebuilt from the last steps of x, the gradient g_t at the pre-activation kept
+// for the next steps, and dx of three steps back (which needs g up to three steps ahead) written.  Sums
+// for dw and dbias over the thread's own steps go out as one partial per (batch, segment).
+constexpr int CONV_CL_SEGS = 32;    // time segments per batch row at most (the workspace is sized for it)
+
+__host__ __device__ inline int conv_cl_seg_len(int len) {
+  const int per = (len + CONV_CL_SEGS - 1) / CONV_CL_SEGS;
+  return per < 16 ? 16 : per;
+}
+
+template <typename T>
+__global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvParams p) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int HIST = CONV_TAPS - 1;
+  const int cvecs = p.chans / VEC;
+  const int seg_len = conv_cl_seg_len(p.len);
+  const int nseg = (p.len + seg_len - 1) / seg_len;
+  const size_t total = (size_t)p.batch * nseg * cvecs;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int cv = (int)(gid % cvecs);
+  const int seg = (int)((gid / cvecs) % nseg);
+  const int b = (int)(gid / ((size_t)cvecs * nseg));
+  const int c0 = cv * VEC;
+  const int K = p.K;
+  float wrev[VEC][CONV_TAPS], bias[VEC], dwr[VEC][CONV_TAPS], db[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    bias[i] = p.bias ? p.bias[c0 + i] : 0.0f;
+    load_taps(p.w, c0 + i, K, wrev[i]);
+    db[i] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = 0.0f;
+  }
+  const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
+  const T *gb = reinterpret_cast<const T *>(p.dout) + (size_t)b * p.len * p.chans + c0;
+  T *dxb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
+  const int t_begin = seg * seg_len;
+  const int t_end = min(p.len, t_begin + seg_len);
+  // xh[j] = x at time (t - 1 - j), gh[m] = g at time (t - 1 - m) once the step's own values are pushed
+  float xh[HIST][VEC], gh[CONV_TAPS][VEC];
+#pragma unroll
+  for (int j = 0; j < HIST; ++j) {
+    const int ts = t_begin - 1 - j;
+    float v[VEC];
+    if (ts >= 0) load_run<T, VEC>(xb + (size_t)ts * p.chans, 0, VEC, true, v);
+    else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) xh[j][i] = v[i];
+  }
+#pragma unroll
+  for (int m = 0; m < CONV_TAPS; ++m)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) gh[m][i] = 0.0f;
+
+  const int t_last = t_end + HIST;                    // exclusive: dx of the last own step needs g three steps on
+  for (int t = t_begin; t < t_last; ++t) {
+    float cur[VEC], g[VEC];
+    if (t < p.len) {
+      float go[VEC];
+      load_run<T, VEC>(xb + (size_t)t * p.chans, 0, VEC, true, cur);
+      load_run<T, VEC>(gb + (size_t)t * p.chans, 0, VEC, true, go);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        g[i] = go[i];
+        if (p.silu) {
+          float pre = __builtin_fmaf(wrev[i][0], cur[i], bias[i]);
+#pragma unroll
+          for (int j = 0; j < HIST; ++j) pre = __builtin_fmaf(wrev[i][j + 1], xh[j][i], pre);
+          g[i] *= silu_grad(pre);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) cur[i] = g[i] = 0.0f;
+    }
+    if (t < t_end) {                                  // own step: sums for dw (reversed taps) and dbias
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        db[i] += g[i];
+        dwr[i][0] = __builtin_fmaf(g[i], cur[i], dwr[i][0]);
+#pragma unroll
+        for (int j = 0; j < HIST; ++j) dwr[i][j + 1] = __builtin_fmaf(g[i], xh[j][i], dwr[i][j + 1]);
+      }
+    }
+    // push: gh[0] = g_t ... gh[3] = g_{t-3};  xh[0] = x_t ...
+#pragma unroll
+    for (int m = CONV_TAPS - 1; m > 0; --m)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) gh[m][i] = gh[m - 1][i];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) gh[0][i] = g[i];
+#pragma unroll
+    for (int j = HIST - 1; j > 0; --j)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) xh[j][i] = xh[j - 1][i];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) xh[0][i] = cur[i];
+    // dx of the step three back: sum_j g_{t'+j} wrev[j] with t' = t - 3, i.e. g_{t'+j} = gh[3 - j]
+    const int td = t - HIST;
+    if (td >= t_begin) {
+      float out[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < CONV_TAPS; ++j) acc = __builtin_fmaf(gh[HIST - j][i], wrev[i][j], acc);
+        out[i] = acc;
+      }
+      store_run<T, VEC>(dxb + (size_t)td * p.chans, 0, VEC, true, out);
+    }
+  }
+  // partial[(b * nseg + seg)][c][K + 1]: taps in the order of w, then the bias sum
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    float *part = p.partial + (((size_t)b * nseg + seg) * p.chans + c0 + i) * (K + 1);
+#pragma unroll
+    for (int m = 0; m < CONV_TAPS; ++m)
+      if (m < K) part[K - 1 - m] = dwr[i][m];
+    part[K] = db[i];
+  }
+}
+
 // Element-wise backward (any K / alignment, either layout): one thread per
 // (b, c) row walks the row sequentially.  Slow path, correctness only.
 template <typename T>
@@ -334,8 +462,16 @@ template <typename T>
 static int conv_bwd_typed(const ConvParams &p, int channels_last, bool vec_ok, float *dw, float *dbias,
                           hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
+  int fold_count = p.batch;
   if (vec_ok && p.K <= CONV_TAPS && !channels_last && p.len % VEC == 0) {
     hipLaunchKernelGGL(conv_bwd_cf_kernel<T>, dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+  } else if (vec_ok && p.K <= CONV_TAPS && channels_last && p.chans % VEC == 0) {
+    const int seg_len = conv_cl_seg_len(p.len);
+    const int nseg = (p.len + seg_len - 1) / seg_len;
+    const size_t threads = (size_t)p.batch * nseg * (p.chans / VEC);
+    hipLaunchKernelGGL(conv_bwd_cl_kernel<T>, dim3((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS)),
+                       dim3(CONV_THREADS), 0, s, p);
+    fold_count = p.batch * nseg;
   } else {
     const int rows = p.batch * p.chans;
     hipLaunchKernelGGL(conv_bwd_generic_kernel<T>, dim3((rows + CONV_THREADS - 1) / CONV_THREADS),
@@ -344,7 +480,7 @@ static int conv_bwd_typed(const ConvParams &p, int channels_last, bool vec_ok, f
   SSM_CHECK_LAUNCH("ssm_conv1d_bwd");
   const int n = p.chans * (p.K + 1);
   hipLaunchKernelGGL(conv_bwd_fold_kernel, dim3((n + CONV_THREADS - 1) / CONV_THREADS), dim3(CONV_THREADS), 0, s,
-                     p.partial, dw, dbias, p.batch, p.chans, p.K);
+                     p.partial, dw, dbias, fold_count, p.chans, p.K);
   SSM_CHECK_LAUNCH("ssm_conv1d_bwd(fold)");
   return SSM_OK;
 }
@@ -389,7 +525,8 @@ extern "C" int ssm_conv1d_fwd(const ssm_conv1d_fwd_args *a, void *hip_stream) {
 
 extern "C" size_t ssm_conv1d_bwd_workspace_bytes(int batch, int channels, int width) {
   if (batch <= 0 || channels <= 0 || width <= 0) return 0;
-  return (size_t)batch * channels * (width + 1) * sizeof(float);
+  // one partial per batch row, or per (batch row, time segment) in the channels-last kernel
+  return (size_t)batch * ssm::CONV_CL_SEGS * channels * (width + 1) * sizeof(float);
 }
 
 extern "C" int ssm_conv1d_bwd(const ssm_conv1d_bwd_args *a, void *hip_stream) {
