@@ -127,7 +127,7 @@ def test_shape_and_dtype_errors_come_back_as_status_codes():
     a.b_groups = 1
     a.u = p + 2
     assert lib.ssm_scan_fwd(ctypes.byref(a), None) == -5            # misaligned pointer
-    assert lib.ssm_conv1d_bwd_workspace_bytes(8, 1536, 4) == 8 * 1536 * 5 * 4
+    assert lib.ssm_conv1d_bwd_workspace_bytes(8, 1536, 4) == 8 * 32 * 1536 * 5 * 4    # per (batch row, time segment)
     assert lib.ssm_conv1d_bwd_workspace_bytes(0, 1, 1) == 0
     assert lib.ssm_scan_bwd_workspace_bytes(8, 1536, 2048, 16, 2, 2, 1, 1) > 0
     assert lib.ssm_scan_bwd_workspace_bytes(8, 1536, 2048, 16, 2, 2, 7, 1) == 0
