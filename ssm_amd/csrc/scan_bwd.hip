@@ -618,7 +618,36 @@ void launch_fold_rows(const float *in, float *out, int count, size_t inner, hipS
   hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid(inner)), dim3(256), 0, s, in, out, count, inner);
 }
 
+// The same sum when there are few outputs and many terms each: a workgroup takes up to 16 neighbouring
+// outputs of one `o`; its 256 threads are those outputs x slices of the terms, added in a fixed order
+// (slice by slice, then over the slices).
+__global__ __launch_bounds__(256) void fold_sum_wide_kernel(const float *in, float *out, int count, size_t inner,
+                                                            int cols, int blocks_per_outer) {
+  __shared__ float part[256];
+  const int slices = 256 / cols;
+  const int cl = threadIdx.x % cols, sl = threadIdx.x / cols;
+  const size_t o = blockIdx.x / blocks_per_outer;
+  const size_t i = (size_t)(blockIdx.x % blocks_per_outer) * cols + cl;
+  float sum = 0.0f;
+  if (i < inner && sl < slices)
+    for (int j = sl; j < count; j += slices) sum += in[(o * count + j) * inner + i];
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  if (sl == 0 && i < inner) {
+    float t = 0.0f;
+    for (int k = 0; k < slices; ++k) t += part[k * cols + cl];
+    out[o * inner + i] = t;
+  }
+}
+
 void launch_fold_sum(const float *in, float *out, size_t outer, int count, size_t inner, hipStream_t s) {
+  if (outer * inner < 65536 && count >= 64) {
+    const int cols = inner >= 16 ? 16 : (inner >= 8 ? 8 : (inner >= 4 ? 4 : (inner >= 2 ? 2 : 1)));
+    const int bpo = (int)((inner + cols - 1) / cols);
+    hipLaunchKernelGGL(fold_sum_wide_kernel, dim3((unsigned)(outer * bpo)), dim3(256), 0, s, in, out, count, inner, cols,
+                       bpo);
+    return;
+  }
   hipLaunchKernelGGL(fold_sum_kernel, dim3(fold_grid(outer * inner)), dim3(256), 0, s, in, out, outer, count, inner);
 }
 
