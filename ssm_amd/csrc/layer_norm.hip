@@ -92,13 +92,32 @@ __device__ __forceinline__ void store_cols(void *p, int dtype, size_t base, int 
 
 // ------------------------------------------------------------------ forward
 
-// TRIPS * 64 * VEC >= hidden; VEC = 4 keeps every access <= 16 bytes for all dtypes.
-template <int TRIPS>
+// A row is held in registers by one wavefront (WG = false: TRIPS * 64 * VEC >= hidden) or, for long rows, by
+// the whole workgroup (WG = true: TRIPS * 256 * VEC >= hidden; sums over the row go through LDS).  VEC = 4
+// keeps every access <= 16 bytes for all dtypes.
+template <bool WG>
+__device__ __forceinline__ float row_sum(float v, float *red) {
+  v = wave_sum(v);
+  if constexpr (WG) {
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();                                   // the slots may still be read from the sum before
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < LN_WAVES; ++w) v += red[w];
+  }
+  return v;
+}
+
+template <int TRIPS, bool WG>
 __global__ __launch_bounds__(LN_THREADS) void norm_fwd_kernel(const NormParams p, int vec_ok) {
   constexpr int VEC = 4;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int row = blockIdx.x * LN_WAVES + wave;
-  if (row >= p.rows) return;
+  constexpr int OWNERS = WG ? LN_THREADS : WAVE;       // threads that share a row
+  __shared__ float red[LN_WAVES];
+  const int wave = threadIdx.x >> 6, lane = WG ? (int)threadIdx.x : (int)(threadIdx.x & 63);
+  const int row = WG ? (int)blockIdx.x : (int)(blockIdx.x * LN_WAVES + wave);
+  if (row >= p.rows) return;                           // whole workgroups in WG mode
   const int H = p.hidden;
   const size_t base = (size_t)row * H;
   const bool vok = vec_ok != 0;
@@ -106,7 +125,7 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_kernel(const NormParams p
   float sum = 0.0f;
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int col = (k * WAVE + lane) * VEC;
+    const int col = (k * OWNERS + lane) * VEC;
     load_cols<VEC>(p.x, p.x_dtype, base, col, H, vok, v[k]);
     if (p.res) {
       load_cols<VEC>(p.res, p.res_dtype, base, col, H, vok, r[k]);
@@ -121,25 +140,25 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_kernel(const NormParams p
   }
   const float inv_h = 1.0f / (float)H;
   float mean = 0.0f;
-  if (!p.is_rms) mean = wave_sum(sum) * inv_h;
+  if (!p.is_rms) mean = row_sum<WG>(sum, red) * inv_h;
   float sq = 0.0f;
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int col = (k * WAVE + lane) * VEC;
+    const int col = (k * OWNERS + lane) * VEC;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       const float c = (col + i < H) ? v[k][i] - mean : 0.0f;
       sq = __builtin_fmaf(c, c, sq);
     }
   }
-  const float rstd = 1.0f / sqrtf(wave_sum(sq) * inv_h + p.eps);
+  const float rstd = 1.0f / sqrtf(row_sum<WG>(sq, red) * inv_h + p.eps);
   if (lane == 0) {
     if (p.mean) p.mean[row] = mean;
     if (p.rstd) p.rstd[row] = rstd;
   }
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int col = (k * WAVE + lane) * VEC;
+    const int col = (k * OWNERS + lane) * VEC;
     if (col >= H) continue;
     float wv[VEC], bv[VEC], out[VEC];
     load_cols<VEC>(p.w, SSM_F32, 0, col, H, vok, wv);
@@ -195,19 +214,21 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_long_kernel(const NormPar
 
 // Each wave handles rows wave_global, wave_global + nwaves, ...; columns are
 // owned by (lane, trip) exactly as in the forward kernel.
-template <int TRIPS>
+template <int TRIPS, bool WG>
 __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p, int vec_ok) {
   constexpr int VEC = 4;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int nwaves = gridDim.x * LN_WAVES;
-  const int gw = blockIdx.x * LN_WAVES + wave;
+  constexpr int OWNERS = WG ? LN_THREADS : WAVE;       // threads that share a row
+  __shared__ float red[LN_WAVES];
+  const int wave = threadIdx.x >> 6, lane = WG ? (int)threadIdx.x : (int)(threadIdx.x & 63);
+  const int nwaves = WG ? (int)gridDim.x : (int)(gridDim.x * LN_WAVES);      // row owners in the grid
+  const int gw = WG ? (int)blockIdx.x : (int)(blockIdx.x * LN_WAVES + wave);
   const int H = p.hidden;
   const bool vok = vec_ok != 0;
   const float inv_h = 1.0f / (float)H;
   float dw[TRIPS][VEC], db[TRIPS][VEC], wv[TRIPS][VEC];
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int col = (k * WAVE + lane) * VEC;
+    const int col = (k * OWNERS + lane) * VEC;
     load_cols<VEC>(p.w, SSM_F32, 0, col, H, vok, wv[k]);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) dw[k][i] = db[k][i] = 0.0f;
@@ -220,7 +241,7 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
     float s1 = 0.0f, s2 = 0.0f;     // sum g*xhat, sum g
 #pragma unroll
     for (int k = 0; k < TRIPS; ++k) {
-      const int col = (k * WAVE + lane) * VEC;
+      const int col = (k * OWNERS + lane) * VEC;
       float v[VEC];
       load_cols<VEC>(p.x, p.x_dtype, base, col, H, vok, v);
       if (p.res && p.prenorm) {
@@ -241,11 +262,11 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
         db[k][i] += dyv[k][i];
       }
     }
-    const float c1 = wave_sum(s1) * inv_h;
-    const float c2 = p.is_rms ? 0.0f : wave_sum(s2) * inv_h;
+    const float c1 = row_sum<WG>(s1, red) * inv_h;
+    const float c2 = p.is_rms ? 0.0f : row_sum<WG>(s2, red) * inv_h;
 #pragma unroll
     for (int k = 0; k < TRIPS; ++k) {
-      const int col = (k * WAVE + lane) * VEC;
+      const int col = (k * OWNERS + lane) * VEC;
       if (col >= H) continue;
       float dxv[VEC];
 #pragma unroll
@@ -254,12 +275,26 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
       if (p.dres) store_cols<VEC>(p.dres, p.res_dtype, base, col, H, vok, p.prenorm ? dxv : dyv[k]);
     }
   }
+  if constexpr (WG) {                                  // every thread owns its columns: the partial is complete
+    float *pw = p.partial + (size_t)blockIdx.x * 2 * H;
+#pragma unroll
+    for (int k = 0; k < TRIPS; ++k) {
+      const int col = (k * OWNERS + lane) * VEC;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i)
+        if (col + i < H) {
+          pw[col + i] = dw[k][i];
+          pw[H + col + i] = db[k][i];
+        }
+    }
+    return;
+  }
   // one partial per workgroup: waves 1.. hand their column sums to wave 0 through LDS (fixed order)
-  __shared__ float wsum[LN_WAVES - 1][2][TRIPS * WAVE * VEC];
+  __shared__ float wsum[LN_WAVES - 1][2][WG ? 1 : TRIPS * WAVE * VEC];
   if (wave > 0) {
 #pragma unroll
     for (int k = 0; k < TRIPS; ++k) {
-      const int col = (k * WAVE + lane) * VEC;
+      const int col = (k * OWNERS + lane) * VEC;
       *reinterpret_cast<float4 *>(&wsum[wave - 1][0][col]) = make_float4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
       *reinterpret_cast<float4 *>(&wsum[wave - 1][1][col]) = make_float4(db[k][0], db[k][1], db[k][2], db[k][3]);
     }
@@ -269,7 +304,7 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
     float *pw = p.partial + (size_t)blockIdx.x * 2 * H;
 #pragma unroll
     for (int k = 0; k < TRIPS; ++k) {
-      const int col = (k * WAVE + lane) * VEC;
+      const int col = (k * OWNERS + lane) * VEC;
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         float a = dw[k][i], b = db[k][i];
@@ -394,11 +429,14 @@ extern "C" int ssm_norm_fwd(const ssm_norm_fwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const unsigned grid = (unsigned)((a->rows + LN_WAVES - 1) / LN_WAVES);
   const int per_lane = (a->hidden + WAVE - 1) / WAVE;
-  if (per_lane <= 4) hipLaunchKernelGGL(norm_fwd_kernel<1>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
-  else if (per_lane <= 8) hipLaunchKernelGGL(norm_fwd_kernel<2>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
-  else if (per_lane <= 12) hipLaunchKernelGGL(norm_fwd_kernel<3>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
-  else if (per_lane <= 16) hipLaunchKernelGGL(norm_fwd_kernel<4>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
-  else if (per_lane <= 32) hipLaunchKernelGGL(norm_fwd_kernel<8>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  if (per_lane <= 4) hipLaunchKernelGGL((norm_fwd_kernel<1, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 8) hipLaunchKernelGGL((norm_fwd_kernel<2, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 12) hipLaunchKernelGGL((norm_fwd_kernel<3, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 16) hipLaunchKernelGGL((norm_fwd_kernel<4, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 32) hipLaunchKernelGGL((norm_fwd_kernel<8, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (a->hidden <= 4096) hipLaunchKernelGGL((norm_fwd_kernel<4, true>), dim3(a->rows), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (a->hidden <= 8192) hipLaunchKernelGGL((norm_fwd_kernel<8, true>), dim3(a->rows), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (a->hidden <= 16384) hipLaunchKernelGGL((norm_fwd_kernel<16, true>), dim3(a->rows), dim3(LN_THREADS), 0, s, p, vec_ok);
   else hipLaunchKernelGGL(norm_fwd_long_kernel, dim3(grid), dim3(LN_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_norm_fwd");
   return SSM_OK;
@@ -434,13 +472,16 @@ extern "C" int ssm_norm_bwd(const ssm_norm_bwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const int grid = norm_bwd_grid(a->rows);
   const int per_lane = (a->hidden + WAVE - 1) / WAVE;
-  if (per_lane <= 4) hipLaunchKernelGGL(norm_bwd_kernel<1>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
-  else if (per_lane <= 8) hipLaunchKernelGGL(norm_bwd_kernel<2>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
-  else if (per_lane <= 12) hipLaunchKernelGGL(norm_bwd_kernel<3>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
-  else if (per_lane <= 16) hipLaunchKernelGGL(norm_bwd_kernel<4>, dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  if (per_lane <= 4) hipLaunchKernelGGL((norm_bwd_kernel<1, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 8) hipLaunchKernelGGL((norm_bwd_kernel<2, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (per_lane <= 12) hipLaunchKernelGGL((norm_bwd_kernel<3, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (a->hidden <= 1024) hipLaunchKernelGGL((norm_bwd_kernel<1, true>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (a->hidden <= 2048) hipLaunchKernelGGL((norm_bwd_kernel<2, true>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (a->hidden <= 4096) hipLaunchKernelGGL((norm_bwd_kernel<4, true>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  else if (a->hidden <= 8192) hipLaunchKernelGGL((norm_bwd_kernel<8, true>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
   else hipLaunchKernelGGL(norm_bwd_long_kernel, dim3(grid), dim3(LN_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_norm_bwd");
-  const int nparts = per_lane <= 16 ? grid : grid * LN_WAVES;      // the long-row kernel writes one per wave
+  const int nparts = a->hidden <= 8192 ? grid : grid * LN_WAVES;   // the long-row kernel writes one per wave
   hipLaunchKernelGGL(norm_bwd_fold_kernel, dim3((a->hidden + FOLD_COLS - 1) / FOLD_COLS), dim3(LN_THREADS), 0, s,
                      p.partial, a->dweight, a->dbias, nparts, a->hidden);
   SSM_CHECK_LAUNCH("ssm_norm_bwd(fold)");

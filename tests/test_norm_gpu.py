@@ -81,7 +81,7 @@ def test_upstream_rms_norm():
     torch.testing.assert_close(w.grad.cpu(), rec["gradients"]["w"], rtol=1e-3, atol=2e-5)
 
 
-@pytest.mark.parametrize("hidden", [1, 6, 64, 768, 770, 1024, 2048, 2500, 5120])
+@pytest.mark.parametrize("hidden", [1, 6, 64, 768, 770, 1024, 1536, 2048, 2500, 4096, 5120, 8192, 8200, 20000])
 @pytest.mark.parametrize("is_rms", [False, True])
 @pytest.mark.parametrize("prenorm", [True, False])
 def test_fp32_matches_oracle(hidden, is_rms, prenorm):
