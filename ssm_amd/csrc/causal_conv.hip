@@ -44,7 +44,9 @@ __device__ __forceinline__ float silu_grad(float pre) {
 
 // ---------------------------------------------------------------- forward, (B,C,L)
 
-template <typename T>
+// AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
+// number of vectors; otherwise the same kernel reads and writes element by element.
+template <typename T, bool AL>
 __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvParams p) {
   constexpr int VEC = 16 / sizeof(T);
   const int row = blockIdx.x;                       // b * C + c
@@ -58,7 +60,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvPar
     float win[2 * VEC];
     if (t0 > 0) {
       float prev[VEC];
-      load_run<T, VEC>(xr, t0 - VEC, p.len, true, prev);
+      load_run<T, VEC>(xr, t0 - VEC, p.len, AL, prev);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) win[i] = prev[i];
     } else {
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvPar
     }
     {
       float cur[VEC];
-      load_run<T, VEC>(xr, t0, p.len, true, cur);
+      load_run<T, VEC>(xr, t0, p.len, AL, cur);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) win[VEC + i] = cur[i];
     }
@@ -79,7 +81,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvPar
       for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[m], win[VEC + i - m], acc);
       out[i] = p.silu ? silu_f32(acc) : acc;
     }
-    store_run<T, VEC>(yr, t0, p.len, true, out);
+    store_run<T, VEC>(yr, t0, p.len, AL, out);
   }
 }
 
@@ -106,10 +108,12 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_generic_kernel(const Co
 
 constexpr int CONV_CL_STRIP = 16;   // time steps per thread
 
-template <typename T>
+// AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
+// number of vectors; otherwise the same kernel reads and writes element by element.
+template <typename T, bool AL>
 __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvParams p) {
   constexpr int VEC = 16 / sizeof(T);
-  const int cvecs = p.chans / VEC;
+  const int cvecs = (p.chans + VEC - 1) / VEC;
   const int strips = (p.len + CONV_CL_STRIP - 1) / CONV_CL_STRIP;
   const size_t total = (size_t)p.batch * strips * cvecs;
   const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -118,13 +122,14 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
   const int strip = (int)((gid / cvecs) % strips);
   const int b = (int)(gid / ((size_t)cvecs * strips));
   const int c0 = cv * VEC;
+  const int cw = min(VEC, p.chans - c0);          // channels of this vector that exist
   const int K = p.K;
   constexpr int HIST = CONV_TAPS - 1;
   float wrev[VEC][CONV_TAPS], bias[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
-    bias[i] = p.bias ? p.bias[c0 + i] : 0.0f;
-    load_taps(p.w, c0 + i, K, wrev[i]);
+    bias[i] = (p.bias && i < cw) ? p.bias[c0 + i] : 0.0f;
+    load_taps(p.w, i < cw ? c0 + i : c0, K, wrev[i]);
   }
   const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
   T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
@@ -136,7 +141,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
   for (int j = 0; j < HIST; ++j) {
     const int ts = t_begin - 1 - j;
     float v[VEC];
-    if (j < K - 1 && ts >= 0) load_run<T, VEC>(xb + (size_t)ts * p.chans, 0, VEC, true, v);
+    if (j < K - 1 && ts >= 0) load_run<T, VEC>(xb + (size_t)ts * p.chans, 0, cw, AL, v);
     else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) v[i] = 0.0f;
@@ -146,7 +151,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
   }
   for (int t = t_begin; t < t_end; ++t) {
     float cur[VEC], out[VEC];
-    load_run<T, VEC>(xb + (size_t)t * p.chans, 0, VEC, true, cur);
+    load_run<T, VEC>(xb + (size_t)t * p.chans, 0, cw, AL, cur);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       float acc = __builtin_fmaf(wrev[i][0], cur[i], bias[i]);
@@ -154,7 +159,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
       for (int j = 0; j < HIST; ++j) acc = __builtin_fmaf(wrev[i][j + 1], hist[j][i], acc);
       out[i] = p.silu ? silu_f32(acc) : acc;
     }
-    store_run<T, VEC>(yb + (size_t)t * p.chans, 0, VEC, true, out);
+    store_run<T, VEC>(yb + (size_t)t * p.chans, 0, cw, AL, out);
 #pragma unroll
     for (int j = HIST - 1; j > 0; --j)
 #pragma unroll
@@ -166,7 +171,9 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
 
 // --------------------------------------------------------------- backward, (B,C,L)
 
-template <typename T>
+// AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
+// number of vectors; otherwise the same kernel reads and writes element by element.
+template <typename T, bool AL>
 __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvParams p) {
   constexpr int VEC = 16 / sizeof(T);
   __shared__ float red[CONV_THREADS / WAVE][CONV_TAPS + 1];
@@ -188,23 +195,23 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
     float xw[3 * VEC], g[2 * VEC];
     {
       float v[VEC];
-      if (t0 > 0) load_run<T, VEC>(xr, t0 - VEC, p.len, true, v);
+      if (t0 > 0) load_run<T, VEC>(xr, t0 - VEC, p.len, AL, v);
       else {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) v[i] = 0.0f;
       }
 #pragma unroll
       for (int i = 0; i < VEC; ++i) xw[i] = v[i];
-      load_run<T, VEC>(xr, t0, p.len, true, v);
+      load_run<T, VEC>(xr, t0, p.len, AL, v);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) xw[VEC + i] = v[i];
-      load_run<T, VEC>(xr, t0 + VEC, p.len, true, v);       // zero past the end
+      load_run<T, VEC>(xr, t0 + VEC, p.len, AL, v);       // zero past the end
 #pragma unroll
       for (int i = 0; i < VEC; ++i) xw[2 * VEC + i] = v[i];
-      load_run<T, VEC>(gr, t0, p.len, true, v);
+      load_run<T, VEC>(gr, t0, p.len, AL, v);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) g[i] = v[i];
-      load_run<T, VEC>(gr, t0 + VEC, p.len, true, v);
+      load_run<T, VEC>(gr, t0 + VEC, p.len, AL, v);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) g[VEC + i] = v[i];
     }
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
 #pragma unroll
       for (int m = 0; m < CONV_TAPS; ++m) dwrev[m] = __builtin_fmaf(g[i], xw[VEC + i - m], dwrev[m]);
     }
-    store_run<T, VEC>(dxr, t0, p.len, true, dx);
+    store_run<T, VEC>(dxr, t0, p.len, AL, dx);
   }
   // block reduction of dw[0..K) and db
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -266,11 +273,13 @@ __host__ __device__ inline int conv_cl_seg_len(int len) {
   return per < 16 ? 16 : per;
 }
 
-template <typename T>
+// AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
+// number of vectors; otherwise the same kernel reads and writes element by element.
+template <typename T, bool AL>
 __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvParams p) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int HIST = CONV_TAPS - 1;
-  const int cvecs = p.chans / VEC;
+  const int cvecs = (p.chans + VEC - 1) / VEC;
   const int seg_len = conv_cl_seg_len(p.len);
   const int nseg = (p.len + seg_len - 1) / seg_len;
   const size_t total = (size_t)p.batch * nseg * cvecs;
@@ -280,12 +289,13 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
   const int seg = (int)((gid / cvecs) % nseg);
   const int b = (int)(gid / ((size_t)cvecs * nseg));
   const int c0 = cv * VEC;
+  const int cw = min(VEC, p.chans - c0);          // channels of this vector that exist
   const int K = p.K;
   float wrev[VEC][CONV_TAPS], bias[VEC], dwr[VEC][CONV_TAPS], db[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
-    bias[i] = p.bias ? p.bias[c0 + i] : 0.0f;
-    load_taps(p.w, c0 + i, K, wrev[i]);
+    bias[i] = (p.bias && i < cw) ? p.bias[c0 + i] : 0.0f;
+    load_taps(p.w, i < cw ? c0 + i : c0, K, wrev[i]);
     db[i] = 0.0f;
 #pragma unroll
     for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = 0.0f;
@@ -301,7 +311,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
   for (int j = 0; j < HIST; ++j) {
     const int ts = t_begin - 1 - j;
     float v[VEC];
-    if (ts >= 0) load_run<T, VEC>(xb + (size_t)ts * p.chans, 0, VEC, true, v);
+    if (ts >= 0) load_run<T, VEC>(xb + (size_t)ts * p.chans, 0, cw, AL, v);
     else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) v[i] = 0.0f;
@@ -319,8 +329,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
     float cur[VEC], g[VEC];
     if (t < p.len) {
       float go[VEC];
-      load_run<T, VEC>(xb + (size_t)t * p.chans, 0, VEC, true, cur);
-      load_run<T, VEC>(gb + (size_t)t * p.chans, 0, VEC, true, go);
+      load_run<T, VEC>(xb + (size_t)t * p.chans, 0, cw, AL, cur);
+      load_run<T, VEC>(gb + (size_t)t * p.chans, 0, cw, AL, go);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         g[i] = go[i];
@@ -368,12 +378,13 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
         for (int j = 0; j < CONV_TAPS; ++j) acc = __builtin_fmaf(gh[HIST - j][i], wrev[i][j], acc);
         out[i] = acc;
       }
-      store_run<T, VEC>(dxb + (size_t)td * p.chans, 0, VEC, true, out);
+      store_run<T, VEC>(dxb + (size_t)td * p.chans, 0, cw, AL, out);
     }
   }
   // partial[(b * nseg + seg)][c][K + 1]: taps in the order of w, then the bias sum
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
+    if (i >= cw) break;
     float *part = p.partial + (((size_t)b * nseg + seg) * p.chans + c0 + i) * (K + 1);
 #pragma unroll
     for (int m = 0; m < CONV_TAPS; ++m)
@@ -443,13 +454,15 @@ template <typename T>
 static int conv_fwd_typed(const ConvParams &p, int channels_last, bool vec_ok, hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
   const size_t total = (size_t)p.batch * p.chans * p.len;
-  if (vec_ok && p.K <= CONV_TAPS && !channels_last && p.len % VEC == 0) {
-    hipLaunchKernelGGL(conv_fwd_cf_kernel<T>, dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
-  } else if (vec_ok && p.K <= CONV_TAPS && channels_last && p.chans % VEC == 0) {
+  if (p.K <= CONV_TAPS && !channels_last) {
+    if (vec_ok && p.len % VEC == 0) hipLaunchKernelGGL((conv_fwd_cf_kernel<T, true>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((conv_fwd_cf_kernel<T, false>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+  } else if (p.K <= CONV_TAPS && channels_last) {
     const int strips = (p.len + CONV_CL_STRIP - 1) / CONV_CL_STRIP;
-    const size_t threads = (size_t)p.batch * strips * (p.chans / VEC);
-    hipLaunchKernelGGL(conv_fwd_cl_kernel<T>, dim3((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS)),
-                       dim3(CONV_THREADS), 0, s, p);
+    const size_t threads = (size_t)p.batch * strips * ((p.chans + VEC - 1) / VEC);
+    const dim3 grid((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS));
+    if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_fwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((conv_fwd_cl_kernel<T, false>), grid, dim3(CONV_THREADS), 0, s, p);
   } else {
     const unsigned grid = (unsigned)min((size_t)65535 * 16, (total + CONV_THREADS - 1) / CONV_THREADS);
     hipLaunchKernelGGL(conv_fwd_generic_kernel<T>, dim3(grid), dim3(CONV_THREADS), 0, s, p, channels_last);
@@ -463,14 +476,16 @@ static int conv_bwd_typed(const ConvParams &p, int channels_last, bool vec_ok, f
                           hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
   int fold_count = p.batch;
-  if (vec_ok && p.K <= CONV_TAPS && !channels_last && p.len % VEC == 0) {
-    hipLaunchKernelGGL(conv_bwd_cf_kernel<T>, dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
-  } else if (vec_ok && p.K <= CONV_TAPS && channels_last && p.chans % VEC == 0) {
+  if (p.K <= CONV_TAPS && !channels_last) {
+    if (vec_ok && p.len % VEC == 0) hipLaunchKernelGGL((conv_bwd_cf_kernel<T, true>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((conv_bwd_cf_kernel<T, false>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+  } else if (p.K <= CONV_TAPS && channels_last) {
     const int seg_len = conv_cl_seg_len(p.len);
     const int nseg = (p.len + seg_len - 1) / seg_len;
-    const size_t threads = (size_t)p.batch * nseg * (p.chans / VEC);
-    hipLaunchKernelGGL(conv_bwd_cl_kernel<T>, dim3((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS)),
-                       dim3(CONV_THREADS), 0, s, p);
+    const size_t threads = (size_t)p.batch * nseg * ((p.chans + VEC - 1) / VEC);
+    const dim3 grid((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS));
+    if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_bwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((conv_bwd_cl_kernel<T, false>), grid, dim3(CONV_THREADS), 0, s, p);
     fold_count = p.batch * nseg;
   } else {
     const int rows = p.batch * p.chans;
