@@ -405,6 +405,32 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         ``y (B, L, H, P)`` in ``x.dtype``; with ``return_final_states`` and / or
         ``return_varlen_states`` a tuple ``(y[, final_states (B, H, P, N)][, varlen_states])``.
     """
+    Q = int(chunk_size)
+    seqlen = int(x.shape[1]) if x.ndim == 4 else 0
+    if (x.ndim == 4 and x.dtype == torch.bfloat16 and Q > 0 and seqlen % Q != 0 and not force_generic
+            and float(dt_limit[0]) <= 0.0 and dt.ndim == 3):
+        # The matrix-core kernels take whole chunks.  Steps of size zero neither decay the state nor add to
+        # it, so a ragged end is filled up with them (zeros for x, B, C, z) and the extra rows of y dropped;
+        # gradients flow through the padding and the slice.
+        pad = (Q - seqlen % Q) % Q
+        tpad = lambda t: None if t is None else torch.nn.functional.pad(t, (0, 0) * (t.ndim - 2) + (0, pad))
+        if dt_softplus:
+            dt_fill = torch.full_like(dt[:, :1], float("-inf")).expand(-1, pad, -1)     # softplus(-inf) = 0
+        elif dt_bias is not None:
+            dt_fill = (-dt_bias.detach().to(dt.dtype))[None, None].expand(dt.shape[0], pad, -1)
+        else:
+            dt_fill = torch.zeros_like(dt[:, :1]).expand(-1, pad, -1)
+        sp = None
+        if seq_idx is not None:
+            sp = torch.cat([seq_idx, seq_idx[:, -1:].expand(-1, pad)], dim=1)
+        out = ssd_combined(tpad(x), torch.cat([dt, dt_fill], dim=1), A, tpad(B), tpad(C), Q, D=D, z=tpad(z),
+                           dt_bias=dt_bias, initial_states=initial_states, dt_softplus=dt_softplus,
+                           dt_limit=dt_limit, return_final_states=return_final_states, states_dtype=states_dtype,
+                           force_generic=force_generic, fused=fused, seq_idx=sp, cu_seqlens=cu_seqlens,
+                           return_varlen_states=return_varlen_states)
+        if isinstance(out, tuple):
+            return (out[0][:, :seqlen],) + tuple(out[1:])
+        return out[:, :seqlen]
     tensors = (x, dt, A, B, C, D, z, dt_bias, initial_states)
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         _need(seq_idx is None and cu_seqlens is None and not return_varlen_states,
