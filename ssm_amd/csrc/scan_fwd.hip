@@ -63,7 +63,7 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   const int per_b = bvary ? a->dim / a->b_groups : a->dim;
   const int per_c = cvary ? a->dim / a->c_groups : a->dim;
   int rows = SCAN_MAX_WAVES;
-  while (rows > 1 && (per_b % rows != 0 || per_c % rows != 0)) rows >>= 1;
+  while (rows > 1 && (per_b % rows != 0 || per_c % rows != 0)) --rows;      // any divisor, not only powers of two
 
   // Two channels per wave (tune 1616) pay off once the grid still fills every CU twice.
   const bool pair_ok = bvary && cvary && a->nstate <= 16 && per_b % 16 == 0 && per_c % 16 == 0;
