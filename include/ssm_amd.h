@@ -208,6 +208,30 @@ typedef struct ssm_decode_step_args {
 
 int ssm_decode_step(const ssm_decode_step_args *args, void *hip_stream);
 
+/* One decoding step of a Mamba-2 (SSD) block on cached states.  No counterpart in the reference (its
+ * `Mamba2` module, /root/reference/src/ssm/modules/mamba2.py:20-140, has no cached step): this is the
+ * single-token selective_state_step above (reference.py:197-309) with per-head step, decay and skip, preceded
+ * by the depthwise convolution of the x | B | C columns on their cached windows, for the block that
+ * configuration 4 describes.  The row of the input projection is consumed in place: z | xBC | dt with
+ * d_inner = heads * headdim, 2 * groups * nstate and heads columns.
+ *   xBC <- silu(conv(window rolled by one, xBC) + bias)          (window updated in place)
+ *   dt = softplus(dt + dt_bias) if dt_softplus;  S <- exp(dt A) S + dt x (x) B;  y = S C + D x;  y *= silu(z) if gate */
+typedef struct ssm_mamba2_decode_args {
+  const void *zxbcdt;        /* (B, 2*d_inner + 2*G*N + H) io dtype */
+  void *conv_state;          /* (B, d_inner + 2*G*N, K) io dtype: last K inputs per channel, oldest first; in place */
+  const float *conv_weight;  /* (d_inner + 2*G*N, K) fp32 */
+  const float *conv_bias;    /* (d_inner + 2*G*N,) fp32 or NULL */
+  float *xbc;                /* (B, d_inner + 2*G*N) fp32: activated conv output (needed as workspace) */
+  float *ssm_state;          /* (B, H, P, N) fp32, in place */
+  const float *A;            /* (H,) */
+  const float *Dskip;        /* (H,) or (H, P) if d_per_p, or NULL */
+  const float *dt_bias;      /* (H,) or NULL */
+  void *y;                   /* (B, d_inner) io dtype */
+  int32_t batch, heads, headdim, groups, nstate, conv_width;
+  int32_t io_dtype, d_per_p, dt_softplus, gate;
+} ssm_mamba2_decode_args;
+int ssm_mamba2_decode_step(const ssm_mamba2_decode_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * diagonal chunk scan: the operator the reference calls `ssd_chunk_scan`
  * (an element-wise recurrence per (batch, head, p); chunking does not change

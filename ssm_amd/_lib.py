@@ -157,6 +157,13 @@ class SsdChunkStateVarlenArgs(C.Structure):
                 ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32)]
 
 
+class Mamba2DecodeArgs(C.Structure):
+    _fields_ = [("zxbcdt", _vp), ("conv_state", _vp), ("conv_weight", _vp), ("conv_bias", _vp), ("xbc", _vp),
+                ("ssm_state", _vp), ("A", _vp), ("Dskip", _vp), ("dt_bias", _vp), ("y", _vp),
+                ("batch", _i32), ("heads", _i32), ("headdim", _i32), ("groups", _i32), ("nstate", _i32),
+                ("conv_width", _i32), ("io_dtype", _i32), ("d_per_p", _i32), ("dt_softplus", _i32), ("gate", _i32)]
+
+
 class SsdCombinedArgs(C.Structure):
     _fields_ = [("x", _vp), ("dt", _vp), ("A", _vp), ("dt_bias", _vp), ("Bm", _vp), ("Cm", _vp), ("Dskip", _vp),
                 ("z", _vp), ("initial_states", _vp), ("y", _vp), ("final_states", _vp), ("workspace", _vp),
@@ -212,6 +219,7 @@ ENTRY_POINTS = {
     "ssm_state_step": StateStepArgs,
     "ssm_state_step_bwd": StateStepBwdArgs,
     "ssm_decode_step": DecodeStepArgs,
+    "ssm_mamba2_decode_step": Mamba2DecodeArgs,
     "ssm_dscan_fwd": DscanFwdArgs,
     "ssm_dscan_bwd": DscanBwdArgs,
     "ssm_ssd_chunk_cumsum": SsdCumsumArgs,

@@ -1,0 +1,151 @@
+// One decoding step of a Mamba-2 (SSD) block on cached states, in two launches.
+//
+// The block's input projection yields one row per sequence, z | xBC | dt (d_inner, d_inner + 2 G N, H
+// columns).  Kernel 1 takes the xBC columns through the depthwise causal convolution on the cached window
+// of the last K inputs (rolled in place) and SiLU.  Kernel 2 is the state update per (sequence, head):
+//   dt = softplus(dt_raw + bias_h) (opt.),  a = exp(dt A_h)
+//   S[p][n] <- a S[p][n] + dt x_p B_n ,   y_p = sum_n S[p][n] C_n + D x_p ,   y_p *= silu(z_p)
+// with the state (B, H, P, N) in float32, updated in place.  The same arithmetic as the single-token
+// selective_state_step with per-head parameters spread over the head's channels, minus the tensor
+// operations that spreading, slicing and window rolling cost when the step is composed from the
+// general operators.
+#include "common.hpp"
+
+#include <type_traits>
+
+namespace ssm {
+
+constexpr int M2_THREADS = 256;
+constexpr int M2_MAX_K = 8;
+
+struct Mamba2StepParams {
+  const void *zxbcdt;        // (B, proj) io dtype, proj = 2 d_inner + 2 G N + H
+  void *conv_state;          // (B, conv_dim, K) io dtype: the last K inputs of every conv channel, oldest first
+  const float *conv_w;       // (conv_dim, K)
+  const float *conv_b;       // (conv_dim,) or null
+  float *xbc;                // (B, conv_dim) float32: activated conv output (workspace and by-product)
+  float *state;              // (B, H, P, N) float32, in place
+  const float *A, *Dk, *bias;  // (H,), (H,) or (H, P) or null, (H,) or null
+  void *y;                   // (B, d_inner) io dtype
+  int batch, heads, hdim, groups, nstate, width;
+  int d_per_p, softplus, gate;
+};
+
+template <typename io_t>
+__global__ __launch_bounds__(M2_THREADS) void mamba2_conv_kernel(const Mamba2StepParams p) {
+  const int di = p.heads * p.hdim, conv_dim = di + 2 * p.groups * p.nstate, proj = 2 * di + 2 * p.groups * p.nstate + p.heads;
+  const size_t e = (size_t)blockIdx.x * M2_THREADS + threadIdx.x;
+  if (e >= (size_t)p.batch * conv_dim) return;
+  const int c = (int)(e % conv_dim), b = (int)(e / conv_dim);
+  const int K = p.width;
+  io_t *win = reinterpret_cast<io_t *>(p.conv_state) + e * K;
+  const float xin = to_f32(reinterpret_cast<const io_t *>(p.zxbcdt)[(size_t)b * proj + di + c]);
+  float w[M2_MAX_K];
+#pragma unroll
+  for (int k = 0; k < M2_MAX_K; ++k) w[k] = k < K ? to_f32(win[k]) : 0.0f;
+  float acc = p.conv_b ? p.conv_b[c] : 0.0f;
+#pragma unroll
+  for (int k = 0; k < M2_MAX_K; ++k) {
+    if (k < K) {
+      const float v = k + 1 < K ? w[k + 1] : xin;          // the window after the roll
+      acc = __builtin_fmaf(p.conv_w[(size_t)c * K + k], v, acc);
+      win[k] = from_f32<io_t>(v);
+    }
+  }
+  p.xbc[e] = silu_f32(acc);
+}
+
+// One workgroup per (sequence, head); thread = (channel p, quarter of the states).
+template <typename io_t>
+__global__ __launch_bounds__(M2_THREADS) void mamba2_state_kernel(const Mamba2StepParams p) {
+  extern __shared__ __align__(16) float bc[];              // B[N] then C[N] of the head's group
+  const int H = p.heads, P = p.hdim, N = p.nstate, G = p.groups;
+  const int di = H * P, conv_dim = di + 2 * G * N, proj = 2 * di + 2 * G * N + H;
+  const int h = blockIdx.x % H, b = blockIdx.x / H;
+  const int g = h / (H / G);
+  const io_t *row = reinterpret_cast<const io_t *>(p.zxbcdt) + (size_t)b * proj;
+  const float *xb = p.xbc + (size_t)b * conv_dim;
+  for (int n = threadIdx.x; n < 2 * N; n += blockDim.x)
+    bc[n] = n < N ? xb[di + g * N + n] : xb[di + G * N + g * N + (n - N)];
+  float dt = to_f32(row[di + conv_dim + h]) + (p.bias ? p.bias[h] : 0.0f);
+  if (p.softplus) dt = softplus_f32(dt);
+  const float a = exp2_hw(dt * p.A[h] * LOG2E);
+  __syncthreads();
+  const int nq = N / 4;                                    // states per thread
+  for (int pp = threadIdx.x >> 2; pp < P; pp += blockDim.x >> 2) {
+    const int q = threadIdx.x & 3;
+    const float x = xb[h * P + pp];
+    const float dtx = dt * x;
+    float *S = p.state + (((size_t)b * H + h) * P + pp) * N + q * nq;
+    const float *Bq = bc + q * nq, *Cq = bc + N + q * nq;
+    float y = 0.0f;
+    for (int n = 0; n < nq; n += 4) {
+      float4 s = *reinterpret_cast<float4 *>(S + n);
+      const float4 bv = *reinterpret_cast<const float4 *>(Bq + n), cv = *reinterpret_cast<const float4 *>(Cq + n);
+      s.x = __builtin_fmaf(a, s.x, dtx * bv.x);
+      s.y = __builtin_fmaf(a, s.y, dtx * bv.y);
+      s.z = __builtin_fmaf(a, s.z, dtx * bv.z);
+      s.w = __builtin_fmaf(a, s.w, dtx * bv.w);
+      y = __builtin_fmaf(s.x, cv.x, y);
+      y = __builtin_fmaf(s.y, cv.y, y);
+      y = __builtin_fmaf(s.z, cv.z, y);
+      y = __builtin_fmaf(s.w, cv.w, y);
+      *reinterpret_cast<float4 *>(S + n) = s;
+    }
+    // the four quarters sit in neighbouring lanes
+    y += __shfl_xor(y, 1, WAVE);
+    y += __shfl_xor(y, 2, WAVE);
+    if (q == 0) {
+      if (p.Dk) y = __builtin_fmaf(p.Dk[p.d_per_p ? (size_t)h * P + pp : (size_t)h], x, y);
+      if (p.gate) y *= silu_f32(to_f32(row[h * P + pp]));
+      reinterpret_cast<io_t *>(p.y)[(size_t)b * di + h * P + pp] = from_f32<io_t>(y);
+    }
+  }
+}
+
+template <typename io_t>
+static int launch_mamba2(const Mamba2StepParams &p, hipStream_t s) {
+  const int conv_dim = p.heads * p.hdim + 2 * p.groups * p.nstate;
+  const size_t total = (size_t)p.batch * conv_dim;
+  hipLaunchKernelGGL(mamba2_conv_kernel<io_t>, dim3((unsigned)((total + M2_THREADS - 1) / M2_THREADS)), dim3(M2_THREADS), 0, s, p);
+  const int threads = p.hdim * 4 < M2_THREADS ? ((p.hdim * 4 + WAVE - 1) / WAVE) * WAVE : M2_THREADS;
+  hipLaunchKernelGGL(mamba2_state_kernel<io_t>, dim3((unsigned)(p.batch * p.heads)), dim3(threads),
+                     (size_t)2 * p.nstate * sizeof(float), s, p);
+  SSM_CHECK_LAUNCH("ssm_mamba2_decode_step");
+  return SSM_OK;
+}
+
+}  // namespace ssm
+
+extern "C" int ssm_mamba2_decode_step(const ssm_mamba2_decode_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_mamba2_decode_step: args is NULL");
+  SSM_REQUIRE(a->zxbcdt && a->conv_state && a->conv_weight && a->xbc && a->ssm_state && a->A && a->y,
+              SSM_ERR_NULL_POINTER,
+              "ssm_mamba2_decode_step: zxbcdt, conv_state, conv_weight, xbc, ssm_state, A and y are required");
+  SSM_REQUIRE(a->batch > 0 && a->heads > 0 && a->headdim > 0 && a->groups > 0 && a->nstate > 0 && a->conv_width > 0,
+              SSM_ERR_BAD_SHAPE, "ssm_mamba2_decode_step: batch, heads, headdim, groups, nstate and conv_width must be positive");
+  SSM_REQUIRE(a->heads % a->groups == 0, SSM_ERR_BAD_SHAPE, "ssm_mamba2_decode_step: groups=%d must divide heads=%d",
+              a->groups, a->heads);
+  SSM_REQUIRE(a->nstate % 16 == 0 && a->nstate <= 1024, SSM_ERR_BAD_SHAPE,
+              "ssm_mamba2_decode_step: nstate=%d must be a multiple of 16, at most 1024", a->nstate);
+  SSM_REQUIRE(a->conv_width <= M2_MAX_K, SSM_ERR_TOO_LARGE, "ssm_mamba2_decode_step: conv_width=%d exceeds %d",
+              a->conv_width, M2_MAX_K);
+  SSM_REQUIRE(valid_dtype(a->io_dtype), SSM_ERR_BAD_DTYPE, "ssm_mamba2_decode_step: io_dtype=%d", a->io_dtype);
+  SSM_REQUIRE((size_t)a->batch * a->heads < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_mamba2_decode_step: too many heads");
+  const int es = dtype_size(a->io_dtype);
+  SSM_REQUIRE(aligned_to(a->zxbcdt, es) && aligned_to(a->conv_state, es) && aligned_to(a->y, es) &&
+                  aligned_to(a->ssm_state, 16) && aligned_to(a->xbc, 16),
+              SSM_ERR_ALIGNMENT, "ssm_mamba2_decode_step: a pointer is not sufficiently aligned");
+  Mamba2StepParams p{};
+  p.zxbcdt = a->zxbcdt; p.conv_state = a->conv_state; p.conv_w = a->conv_weight; p.conv_b = a->conv_bias;
+  p.xbc = a->xbc; p.state = a->ssm_state; p.A = a->A; p.Dk = a->Dskip; p.bias = a->dt_bias; p.y = a->y;
+  p.batch = a->batch; p.heads = a->heads; p.hdim = a->headdim; p.groups = a->groups; p.nstate = a->nstate;
+  p.width = a->conv_width; p.d_per_p = a->d_per_p ? 1 : 0; p.softplus = a->dt_softplus ? 1 : 0; p.gate = a->gate ? 1 : 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  switch (a->io_dtype) {
+    case SSM_F32: return launch_mamba2<float>(p, s);
+    case SSM_BF16: return launch_mamba2<bf16_t>(p, s);
+    default: return launch_mamba2<f16_t>(p, s);
+  }
+}

@@ -402,6 +402,57 @@ def decode_step(conv_state, ssm_state, x, dt, A, B, C, conv_weight, conv_bias=No
     return y
 
 
+def mamba2_decode_step(zxbcdt, conv_state, ssm_state, conv_weight, conv_bias, A, D=None, dt_bias=None,
+                       ngroups=1, softplus=True, gate=True, return_conv_out=False):
+    """One decoding step of a Mamba-2 (SSD) block on cached states, consuming the row of the input
+    projection as it is (two launches: convolution on the cached windows, state update per head).
+
+    Args:
+        zxbcdt: ``(B, 2*d_inner + 2*G*N + H)`` row of the input projection, ``z | x B C | dt``.
+        conv_state: ``(B, d_inner + 2*G*N, K)`` last ``K`` inputs of every convolution channel (oldest
+            first), dtype of ``zxbcdt``; rolled in place.
+        ssm_state: ``(B, H, P, N)`` float32, updated in place.
+        conv_weight: ``(d_inner + 2*G*N, K)``; conv_bias: ``(d_inner + 2*G*N,)`` or ``None``.
+        A: ``(H,)``; D: ``(H,)`` or ``(H, P)`` or ``None``; dt_bias: ``(H,)`` or ``None``.
+        ngroups: ``G``, the number of B/C groups.
+        softplus: Apply softplus to ``dt + dt_bias``.
+        gate: Multiply ``y`` by ``silu(z)``.
+        return_conv_out: Also return the activated convolution output ``(B, d_inner + 2*G*N)`` (float32).
+
+    Returns:
+        ``y (B, d_inner)`` in ``zxbcdt.dtype``, or ``(y, conv_out)``.
+    """
+    if ssm_state.ndim != 4 or zxbcdt.ndim != 2 or conv_state.ndim != 3:
+        raise ValueError("zxbcdt must be (B, proj), conv_state (B, C, K) and ssm_state (B, H, P, N).")
+    batch, heads, hdim, nstate = (int(v) for v in ssm_state.shape)
+    G = int(ngroups)
+    di, conv_dim = heads * hdim, heads * hdim + 2 * G * nstate
+    K_ = int(conv_state.shape[2])
+    if tuple(zxbcdt.shape) != (batch, 2 * di + 2 * G * nstate + heads):
+        raise ValueError("zxbcdt must have 2*d_inner + 2*G*N + H columns.")
+    if tuple(conv_state.shape) != (batch, conv_dim, K_) or conv_state.dtype != zxbcdt.dtype:
+        raise ValueError("conv_state must be (B, d_inner + 2*G*N, K) in the dtype of zxbcdt.")
+    if ssm_state.dtype != torch.float32 or not ssm_state.is_contiguous() or not conv_state.is_contiguous():
+        raise ValueError("ssm_state must be contiguous float32 and conv_state contiguous (both are updated in place).")
+    if tuple(A.shape) != (heads,) or (D is not None and tuple(D.shape) not in ((heads,), (heads, hdim))):
+        raise ValueError("A must be (H,) and D (H,) or (H, P).")
+    dev = K.require_gpu(zxbcdt, conv_state, ssm_state, conv_weight, conv_bias, A, D, dt_bias)
+    K.check_float("zxbcdt", zxbcdt)
+    row = K.cast_c(zxbcdt, zxbcdt.dtype)
+    wf = K.as_f32_vec(conv_weight.reshape(conv_dim, K_))
+    bf, Af, Df, biasf = K.as_f32_vec(conv_bias), K.as_f32_vec(A), K.as_f32_vec(D), K.as_f32_vec(dt_bias)
+    xbc = torch.empty(batch, conv_dim, dtype=torch.float32, device=dev)
+    y = torch.empty(batch, di, dtype=zxbcdt.dtype, device=dev)
+    args = _lib.Mamba2DecodeArgs(
+        zxbcdt=_lib.ptr(row), conv_state=_lib.ptr(conv_state), conv_weight=_lib.ptr(wf), conv_bias=_lib.ptr(bf),
+        xbc=_lib.ptr(xbc), ssm_state=_lib.ptr(ssm_state), A=_lib.ptr(Af), Dskip=_lib.ptr(Df), dt_bias=_lib.ptr(biasf),
+        y=_lib.ptr(y), batch=batch, heads=heads, headdim=hdim, groups=G, nstate=nstate, conv_width=K_,
+        io_dtype=_lib.dtype_enum(row.dtype), d_per_p=int(D is not None and D.ndim == 2),
+        dt_softplus=int(bool(softplus)), gate=int(bool(gate)))
+    _lib.call("ssm_mamba2_decode_step", args, dev)
+    return (y, xbc) if return_conv_out else y
+
+
 # ---------------------------------------------------------------------------
 # diagonal chunk scan (the reference's ``ssd_chunk_scan``)
 # ---------------------------------------------------------------------------
@@ -684,6 +735,7 @@ __all__ = [
     "selective_scan",
     "selective_state_step",
     "decode_step",
+    "mamba2_decode_step",
     "ssd_chunk_scan",
     "dw_causal_conv",
     "fused_layer_norm",

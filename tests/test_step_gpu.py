@@ -199,6 +199,88 @@ def test_fused_decode_step_equals_conv_window_then_state_step(io, K):
     torch.testing.assert_close(st.cpu(), st_ref, **(FP32_TOL if io == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
 
 
+@pytest.mark.parametrize("io", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 4, 64, 1, 64, 4), (3, 6, 32, 2, 16, 4), (1, 3, 80, 3, 128, 2), (2, 8, 64, 8, 32, 7)],
+                         ids=lambda s: "B%d_H%d_P%d_G%d_N%d_K%d" % s)
+def test_mamba2_decode_step_equals_window_conv_then_per_head_state_step(io, shape):
+    """mamba2_decode_step over three consecutive tokens == splitting the projected row into z | xBC | dt,
+    rolling the convolution window, tap sum + bias + SiLU, and the oracle's single-token update with the
+    per-head dt, A, D spread over the head's channels (the tensor ops of the reference's Mamba2.step)."""
+    ops = _ops()
+    Bsz, H, P, G, N, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    di, conv_dim = H * P, H * P + 2 * G * N
+    A = -(torch.rand(H, generator=g) * 4.0 + 0.5)
+    D = torch.randn(H, generator=g)
+    bias = torch.randn(H, generator=g) - 2.0
+    w = torch.rand(conv_dim, K, generator=g) - 0.5
+    cb = torch.randn(conv_dim, generator=g) * 0.1
+    cs_ref = torch.randn(Bsz, conv_dim, K, generator=g).to(io).float()
+    st_ref = torch.randn(Bsz, H, P, N, generator=g)
+    cs, st = cs_ref.to(io).cuda(), st_ref.clone().cuda()
+    tol = FP32_TOL if io == torch.float32 else HALF_TOL
+    for step in range(3):
+        row = torch.randn(Bsz, 2 * di + 2 * G * N + H, generator=g).to(io)
+        z, xBC, dt = torch.split(row.float(), [di, conv_dim, H], dim=-1)
+        cs_ref = torch.roll(cs_ref, -1, dims=-1)
+        cs_ref[..., -1] = xBC
+        act = torch.nn.functional.silu((cs_ref * w).sum(-1) + cb)
+        x, Bm, Cm = torch.split(act, [di, G * N, G * N], dim=-1)
+        flat = st_ref.reshape(Bsz, di, N).clone()
+        y_ref = O.selective_state_step(flat, x, dt.repeat_interleave(P, dim=-1),
+                                       A.repeat_interleave(P)[:, None].expand(di, N), Bm.reshape(Bsz, G, N),
+                                       Cm.reshape(Bsz, G, N), D=D.repeat_interleave(P), z=z,
+                                       dt_bias=bias.repeat_interleave(P), softplus=True)
+        st_ref = flat.reshape(Bsz, H, P, N)
+        y, act_gpu = ops.mamba2_decode_step(row.cuda(), cs, st, w.cuda(), cb.cuda(), A.cuda(), D=D.cuda(),
+                                            dt_bias=bias.cuda(), ngroups=G, softplus=True, gate=True,
+                                            return_conv_out=True)
+        assert y.dtype == io
+        torch.testing.assert_close(cs.float().cpu(), cs_ref, rtol=0, atol=0)
+        torch.testing.assert_close(act_gpu.cpu(), act, **FP32_TOL)
+        torch.testing.assert_close(y.float().cpu(), y_ref.float(), **tol)
+        torch.testing.assert_close(st.cpu(), st_ref, **FP32_TOL)
+
+
+def test_mamba2_decode_step_options_and_errors():
+    ops = _ops()
+    g = torch.Generator().manual_seed(5)
+    Bsz, H, P, G, N, K = 2, 2, 64, 1, 16, 4
+    di, conv_dim = H * P, H * P + 2 * G * N
+    row = torch.randn(Bsz, 2 * di + 2 * G * N + H, generator=g)
+    cs0 = torch.randn(Bsz, conv_dim, K, generator=g)
+    st0 = torch.randn(Bsz, H, P, N, generator=g)
+    w = torch.rand(conv_dim, K, generator=g) - 0.5
+    A = -torch.rand(H, generator=g) - 0.5
+    Dhp = torch.randn(H, P, generator=g)
+    # no bias, no softplus, no gate, D per channel
+    z, xBC, dt = torch.split(row, [di, conv_dim, H], dim=-1)
+    win = torch.roll(cs0, -1, dims=-1)
+    win[..., -1] = xBC
+    act = torch.nn.functional.silu((win * w).sum(-1))
+    x, Bm, Cm = torch.split(act, [di, G * N, G * N], dim=-1)
+    flat = st0.reshape(Bsz, di, N).clone()
+    y_ref = O.selective_state_step(flat, x, dt.repeat_interleave(P, dim=-1), A.repeat_interleave(P)[:, None].expand(di, N),
+                                   Bm.reshape(Bsz, G, N), Cm.reshape(Bsz, G, N), D=Dhp.reshape(di), z=None,
+                                   dt_bias=None, softplus=False)
+    cs, st = cs0.clone().cuda(), st0.clone().cuda()
+    y = ops.mamba2_decode_step(row.cuda(), cs, st, w.cuda(), None, A.cuda(), D=Dhp.cuda(), dt_bias=None, ngroups=G,
+                               softplus=False, gate=False)
+    torch.testing.assert_close(y.cpu(), y_ref, **FP32_TOL)
+    torch.testing.assert_close(st.cpu(), flat.reshape(Bsz, H, P, N), **FP32_TOL)
+    with pytest.raises(ValueError):
+        ops.mamba2_decode_step(row[:, :-1].cuda(), cs, st, w.cuda(), None, A.cuda())
+    with pytest.raises(ValueError):
+        ops.mamba2_decode_step(row.cuda(), cs.to(torch.bfloat16), st, w.cuda(), None, A.cuda())
+    with pytest.raises(ValueError):
+        ops.mamba2_decode_step(row.cuda(), cs, st.to(torch.bfloat16), w.cuda(), None, A.cuda())
+    bad_n = torch.zeros(Bsz, H, P, 12, device="cuda")
+    with pytest.raises((ValueError, RuntimeError)):
+        ops.mamba2_decode_step(torch.zeros(Bsz, 2 * di + 24 + H, device="cuda"),
+                               torch.zeros(Bsz, di + 24, K, device="cuda"), bad_n, torch.zeros(di + 24, K, device="cuda"),
+                               None, A.cuda())
+
+
 # ---------------------------------------------------------------------------
 # backward: gradients of (y, new_state) against float64 autograd through the
 # CPU restatement of the step
