@@ -280,6 +280,10 @@ extern "C" int ssm_ssd_bmm_chunk(const ssm_ssd_bmm_args *a, void *hip_stream) {
     SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk(mfma)");
     return SSM_OK;
   }
+  if (!a->force_generic && ssd_bmm_tiled(p, s)) {
+    SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk(tiled)");
+    return SSM_OK;
+  }
   hipLaunchKernelGGL(ssd_bmm_kernel, dim3(grid_for(total)), dim3(SSD_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk");
   return SSM_OK;
@@ -309,6 +313,10 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   if (!a->force_generic && ssd_chunk_state_mfma(p, s)) {
     g_mfma_launches |= 2;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
+    return SSM_OK;
+  }
+  if (!a->force_generic && ssd_chunk_state_tiled(p, s)) {
+    SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(tiled)");
     return SSM_OK;
   }
   const size_t total = (size_t)p.d.batch * p.d.nchunks * p.d.heads * p.d.hdim * p.d.nstate;
@@ -361,6 +369,10 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
     g_mfma_launches |= 4;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
+    return SSM_OK;
+  }
+  if (!a->force_generic && ssd_chunk_scan_tiled(p, s)) {
+    SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(tiled)");
     return SSM_OK;
   }
   const size_t total = (size_t)p.d.batch * p.d.len * p.d.heads * p.d.hdim;

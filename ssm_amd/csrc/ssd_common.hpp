@@ -107,6 +107,11 @@ bool ssd_bmm_mfma(const SsdBmmParams &p, hipStream_t s);
 bool ssd_chunk_state_mfma(const SsdStateParams &p, hipStream_t s);
 size_t ssd_chunk_state_scratch_bytes(const SsdDims &d);
 bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s);
+// Float32 matrix-core variants for all other dtypes and shapes, defined in ssd_tiled.hip; false when the
+// chunk is too long for their LDS arrays.
+bool ssd_bmm_tiled(const SsdBmmParams &p, hipStream_t s);
+bool ssd_chunk_state_tiled(const SsdStateParams &p, hipStream_t s);
+bool ssd_chunk_scan_tiled(const SsdScanParams &p, hipStream_t s);
 void note_mfma_launch(int bits);   // recorded for ssm_ssd_mfma_launches()
 
 }  // namespace ssm
