@@ -242,7 +242,8 @@ def test_packed_arguments_are_checked():
 
 
 @pytest.mark.parametrize("shape,Q", [((1, 1, 1, 1, 1, 1), 1), ((2, 19, 4, 5, 2, 6), 8), ((2, 64, 4, 16, 1, 32), 16),
-                                     ((1, 300, 2, 64, 2, 128), 64), ((2, 130, 3, 7, 3, 9), 256)],
+                                     ((1, 300, 2, 64, 2, 128), 64), ((2, 130, 3, 7, 3, 9), 256),
+                                     ((1, 250, 2, 100, 1, 70), 96), ((1, 200, 1, 130, 1, 33), 200)],
                          ids=lambda v: str(v).replace(" ", ""))
 def test_fp32_combined_matches_float64_recurrence(shape, Q):
     b, l, h, p, g, n = shape
@@ -254,6 +255,25 @@ def test_fp32_combined_matches_float64_recurrence(shape, Q):
                                 return_final_states=True)
     torch.testing.assert_close(y.cpu().double(), y64, **FP32_TOL)
     torch.testing.assert_close(fin.cpu().double(), f64, **FP32_TOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_tiled_kernels_match_the_one_thread_per_output_kernels(dtype):
+    """Float32 / float16 calls run 64x64 tiles on the float32 matrix cores; ``force_generic`` keeps the
+    plain kernels (one thread per output element) as a second opinion: tiles with remainders in every
+    dimension, a ragged last chunk and packed sequences."""
+    b, l, h, p, g, n, Q = 2, 333, 4, 72, 2, 80, 160
+    inp = make(17, b, l, h, p, g, n, d_mat=True)
+    seq_idx = torch.zeros(b, l, dtype=torch.int32)
+    seq_idx[:, 120:] = 1
+    seq_idx[:, 170:] = 2
+    args = [cu(inp[k]).to(dtype) if k in ("x", "B", "C") else cu(inp[k]) for k in ("x", "dt", "A", "B", "C")]
+    kw = dict(D=cu(inp["D"]), z=cu(inp["z"]).to(dtype), seq_idx=seq_idx.cuda(), return_final_states=True)
+    y, fin = ssd().ssd_combined(*args, Q, **kw)
+    yg, fing = ssd().ssd_combined(*args, Q, force_generic=True, **kw)
+    tol = FP32_TOL if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(y.float(), yg.float(), **tol)
+    torch.testing.assert_close(fin, fing, **tol)
 
 
 def test_components_match_oracle_fp32():
