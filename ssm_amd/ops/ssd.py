@@ -317,9 +317,6 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
     return out
 
 
-_KEEP_WORKSPACE = []      # debugging aid: when non-empty, receives [workspace tensor, offset] of the last one-pass call
-
-
 def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
     """Whether the one-pass kernel covers this call (bf16 tensors on the GPU and a
     shape ``ssm_ssd_combined_supported`` accepts)."""
@@ -361,8 +358,6 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
         dt_softplus=int(bool(dt_softplus)), d_per_p=int(d_per_p),
         dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]))
     _lib.call("ssm_ssd_combined_fwd", args, dev)
-    if _KEEP_WORKSPACE:
-        _KEEP_WORKSPACE[:] = [work, off]
     if return_final_states:
         return y, final
     return y
