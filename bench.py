@@ -308,6 +308,28 @@ def bench_model(batch=16, prompt=2048, new_tokens=256):
                      "d_state 128, vocab 50280, bf16, random weights"}
 
 
+def bench_model1(batch=8, prompt=2048, new_tokens=256):
+    """Mamba-1-130M-style stack (24 layers, d_model 768, 1536 channels, 16 states, 4 taps: every mixer call has
+    the shape of the headline scan workload), bf16, random weights: prefill through selective_scan with the
+    state handed over, then greedy decoding on cached states with the step replayed as a HIP graph."""
+    from ssm_amd.harness import Mamba1Config, Mamba1LM
+    model = Mamba1LM(Mamba1Config(), seed=0)
+    gen = torch.Generator().manual_seed(0)
+    tokens = torch.randint(0, model.cfg.vocab_size, (batch, prompt), generator=gen).cuda()
+    model.generate(tokens, 4)
+    best = None
+    for _ in range(2):
+        _, t = model.generate(tokens, new_tokens)
+        if best is None or t["prefill_s"] + t["decode_s"] < best["prefill_s"] + best["decode_s"]:
+            best = t
+    return {"prefill_ms": round(best["prefill_s"] * 1e3, 2),
+            "prefill_tokens_per_s": round(batch * prompt / best["prefill_s"], 1),
+            "decode_ms_per_token": round(best["decode_s"] * 1e3 / (new_tokens - 1), 4),
+            "decode_tokens_per_s": round(batch * (new_tokens - 1) / best["decode_s"], 1),
+            "shape": f"batch {batch}, prompt {prompt}, {new_tokens} new tokens, 24 layers, d_model 768, "
+                     "d_state 16, vocab 50280, bf16, random weights"}
+
+
 def cpu_baseline_scan(dtype=torch.bfloat16, dim=1536, length=2048, nstate=16, budget_s=15.0):
     """Time the CPU restatement of the reference's Python loop on a batch slice
     of the headline workload; returns GB/s of the same algorithmic bytes."""
@@ -349,7 +371,7 @@ def main():
                     help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
-                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model"],
+                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
     args = ap.parse_args()
@@ -374,7 +396,8 @@ def main():
 
     if args.only:
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
-              "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model}[args.only]
+              "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model,
+              "model1": bench_model1}[args.only]
         print(json.dumps({args.only: fn()}))
         return
 
@@ -420,6 +443,7 @@ def main():
         extra["ssd_combined_config3"] = bench_ssd()
         extra["ssd_config3_backward_and_packed"] = bench_ssd_train()
         extra["mamba2_130m_style_model_config4"] = bench_model()
+        extra["mamba1_130m_style_model_config1_shape"] = bench_model1()
         line["extra"] = extra
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_scan()

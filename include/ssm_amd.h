@@ -232,6 +232,23 @@ typedef struct ssm_mamba2_decode_args {
 } ssm_mamba2_decode_args;
 int ssm_mamba2_decode_step(const ssm_mamba2_decode_args *args, void *hip_stream);
 
+/* The convolution part of a decoding step on its own: the new input x enters the cached window, which moves
+ * on by one, and out = act(bias + sum_k weight[:, k] * window[:, :, k]).  It replaces the window roll, tap sum
+ * and SiLU that `Mamba1.step` spells out with tensor ops at src/ssm/modules/mamba1.py:345-353, for blocks
+ * whose dt, B and C are projections of this very output (so that ssm_decode_step does not apply). */
+typedef struct ssm_conv1d_update_args {
+  const void *x;             /* (B, C) io dtype; row b starts x_row_stride * b elements in */
+  void *conv_state;          /* (B, C, K) io dtype: last K inputs per channel, oldest first; in place */
+  const float *weight;       /* (C, K) fp32 */
+  const float *bias;         /* (C,) fp32 or NULL */
+  void *out;                 /* (B, C) io dtype */
+  int64_t x_row_stride;      /* >= channels */
+  int32_t batch, channels, width;
+  int32_t io_dtype;          /* ssm_dtype */
+  int32_t activation;        /* ssm_activation */
+} ssm_conv1d_update_args;
+int ssm_conv1d_update(const ssm_conv1d_update_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * diagonal chunk scan: the operator the reference calls `ssd_chunk_scan`
  * (an element-wise recurrence per (batch, head, p); chunking does not change

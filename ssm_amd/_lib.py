@@ -164,6 +164,12 @@ class Mamba2DecodeArgs(C.Structure):
                 ("conv_width", _i32), ("io_dtype", _i32), ("d_per_p", _i32), ("dt_softplus", _i32), ("gate", _i32)]
 
 
+class Conv1dUpdateArgs(C.Structure):
+    _fields_ = [("x", _vp), ("conv_state", _vp), ("weight", _vp), ("bias", _vp), ("out", _vp),
+                ("x_row_stride", C.c_int64), ("batch", _i32), ("channels", _i32), ("width", _i32),
+                ("io_dtype", _i32), ("activation", _i32)]
+
+
 class SsdCombinedArgs(C.Structure):
     _fields_ = [("x", _vp), ("dt", _vp), ("A", _vp), ("dt_bias", _vp), ("Bm", _vp), ("Cm", _vp), ("Dskip", _vp),
                 ("z", _vp), ("initial_states", _vp), ("y", _vp), ("final_states", _vp), ("workspace", _vp),
@@ -231,6 +237,7 @@ ENTRY_POINTS = {
     "ssm_ssd_combined_fwd": SsdCombinedArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
+    "ssm_conv1d_update": Conv1dUpdateArgs,
     "ssm_norm_fwd": NormFwdArgs,
     "ssm_norm_bwd": NormBwdArgs,
 }

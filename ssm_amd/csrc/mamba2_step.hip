@@ -55,6 +55,47 @@ __global__ __launch_bounds__(M2_THREADS) void mamba2_conv_kernel(const Mamba2Ste
   p.xbc[e] = silu_f32(acc);
 }
 
+// The convolution step on its own: x (B, C) enters the window (B, C, K), out = act(bias + taps . window).
+struct ConvUpdateParams {
+  const void *x;
+  size_t x_stride;           // elements between the rows of x
+  void *conv_state;
+  const float *w, *b;
+  void *out;                 // (B, C) io dtype
+  int batch, chans, width, silu;
+};
+
+template <typename io_t>
+__global__ __launch_bounds__(M2_THREADS) void conv_update_kernel(const ConvUpdateParams p) {
+  const size_t e = (size_t)blockIdx.x * M2_THREADS + threadIdx.x;
+  if (e >= (size_t)p.batch * p.chans) return;
+  const int c = (int)(e % p.chans), b = (int)(e / p.chans);
+  const int K = p.width;
+  io_t *win = reinterpret_cast<io_t *>(p.conv_state) + e * K;
+  const float xin = to_f32(reinterpret_cast<const io_t *>(p.x)[(size_t)b * p.x_stride + c]);
+  float w[M2_MAX_K];
+#pragma unroll
+  for (int k = 0; k < M2_MAX_K; ++k) w[k] = k < K ? to_f32(win[k]) : 0.0f;
+  float acc = p.b ? p.b[c] : 0.0f;
+#pragma unroll
+  for (int k = 0; k < M2_MAX_K; ++k) {
+    if (k < K) {
+      const float v = k + 1 < K ? w[k + 1] : xin;
+      acc = __builtin_fmaf(p.w[(size_t)c * K + k], v, acc);
+      win[k] = from_f32<io_t>(v);
+    }
+  }
+  reinterpret_cast<io_t *>(p.out)[e] = from_f32<io_t>(p.silu ? silu_f32(acc) : acc);
+}
+
+template <typename io_t>
+static int launch_conv_update(const ConvUpdateParams &p, hipStream_t s) {
+  const size_t total = (size_t)p.batch * p.chans;
+  hipLaunchKernelGGL(conv_update_kernel<io_t>, dim3((unsigned)((total + M2_THREADS - 1) / M2_THREADS)), dim3(M2_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_conv1d_update");
+  return SSM_OK;
+}
+
 // One workgroup per (sequence, head); thread = (channel p, quarter of the states).
 template <typename io_t>
 __global__ __launch_bounds__(M2_THREADS) void mamba2_state_kernel(const Mamba2StepParams p) {
@@ -147,5 +188,32 @@ extern "C" int ssm_mamba2_decode_step(const ssm_mamba2_decode_args *a, void *hip
     case SSM_F32: return launch_mamba2<float>(p, s);
     case SSM_BF16: return launch_mamba2<bf16_t>(p, s);
     default: return launch_mamba2<f16_t>(p, s);
+  }
+}
+
+extern "C" int ssm_conv1d_update(const ssm_conv1d_update_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_conv1d_update: args is NULL");
+  SSM_REQUIRE(a->x && a->conv_state && a->weight && a->out, SSM_ERR_NULL_POINTER,
+              "ssm_conv1d_update: x, conv_state, weight and out are required");
+  SSM_REQUIRE(a->batch > 0 && a->channels > 0 && a->width > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_conv1d_update: batch, channels and width must be positive");
+  SSM_REQUIRE(a->width <= M2_MAX_K, SSM_ERR_TOO_LARGE, "ssm_conv1d_update: width=%d exceeds %d", a->width, M2_MAX_K);
+  SSM_REQUIRE(a->x_row_stride >= a->channels, SSM_ERR_BAD_SHAPE, "ssm_conv1d_update: x_row_stride=%lld is less than channels=%d",
+              (long long)a->x_row_stride, a->channels);
+  SSM_REQUIRE(valid_dtype(a->io_dtype), SSM_ERR_BAD_DTYPE, "ssm_conv1d_update: io_dtype=%d", a->io_dtype);
+  SSM_REQUIRE(a->activation == SSM_ACT_IDENTITY || a->activation == SSM_ACT_SILU, SSM_ERR_BAD_KIND,
+              "ssm_conv1d_update: activation=%d", a->activation);
+  const int es = dtype_size(a->io_dtype);
+  SSM_REQUIRE(aligned_to(a->x, es) && aligned_to(a->conv_state, es) && aligned_to(a->out, es), SSM_ERR_ALIGNMENT,
+              "ssm_conv1d_update: a pointer is not sufficiently aligned");
+  ConvUpdateParams p{};
+  p.x = a->x; p.x_stride = (size_t)a->x_row_stride; p.conv_state = a->conv_state; p.w = a->weight; p.b = a->bias;
+  p.out = a->out; p.batch = a->batch; p.chans = a->channels; p.width = a->width; p.silu = a->activation == SSM_ACT_SILU;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  switch (a->io_dtype) {
+    case SSM_F32: return launch_conv_update<float>(p, s);
+    case SSM_BF16: return launch_conv_update<bf16_t>(p, s);
+    default: return launch_conv_update<f16_t>(p, s);
   }
 }

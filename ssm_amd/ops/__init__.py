@@ -453,6 +453,51 @@ def mamba2_decode_step(zxbcdt, conv_state, ssm_state, conv_weight, conv_bias, A,
     return (y, xbc) if return_conv_out else y
 
 
+def conv_window_step(conv_state, x, weight, bias=None, activation="silu"):
+    """The depthwise causal convolution for one new token on a cached window.
+
+    ``conv_state`` moves on by one (its oldest column drops out, ``x`` becomes the newest) and the
+    result is ``act(bias + sum_k weight[:, k] * conv_state[:, :, k])``: what ``dw_causal_conv`` returns
+    at the last position of the sequence the window ends.
+
+    Args:
+        conv_state: ``(B, C, K)`` last ``K`` inputs of every channel, oldest first; updated in place.
+        x: ``(B, C)`` new input in the dtype of ``conv_state``; a column slice of a wider matrix is read
+            in place (unit stride along ``C``).
+        weight: ``(C, K)`` or ``(C, 1, K)``; bias: ``(C,)`` or ``None``.
+        activation: ``"silu"``/``"swish"`` or ``"identity"``/``"none"``.
+
+    Returns:
+        ``(B, C)`` tensor in ``x.dtype``.
+    """
+    if conv_state.ndim != 3 or x.ndim != 2 or tuple(conv_state.shape[:2]) != tuple(x.shape):
+        raise ValueError("conv_state must have shape (B, C, K) and x (B, C).")
+    batch, chans, width = (int(v) for v in conv_state.shape)
+    w = weight[:, 0, :] if weight.ndim == 3 else weight
+    if tuple(w.shape) != (chans, width):
+        raise ValueError("weight must have shape (C, K) matching conv_state.")
+    if bias is not None and tuple(bias.shape) != (chans,):
+        raise ValueError("bias must have shape (C,).")
+    act = str(activation).lower()
+    if act not in ("silu", "swish", "identity", "none"):
+        raise ValueError(f"Unsupported activation '{activation}'.")
+    dev = K.require_gpu(conv_state, x, weight, bias)
+    K.check_float("x", x)
+    if conv_state.dtype != x.dtype or not conv_state.is_contiguous():
+        raise ValueError("conv_state must be contiguous and share the dtype of x (it is updated in place).")
+    xs = x.detach()
+    if xs.stride(1) != 1 or xs.stride(0) < chans:
+        xs = xs.contiguous()
+    wf, bf = K.as_f32_vec(w), K.as_f32_vec(bias)
+    out = torch.empty(batch, chans, dtype=x.dtype, device=dev)
+    args = _lib.Conv1dUpdateArgs(
+        x=_lib.ptr(xs), conv_state=_lib.ptr(conv_state), weight=_lib.ptr(wf), bias=_lib.ptr(bf), out=_lib.ptr(out),
+        x_row_stride=int(xs.stride(0)), batch=batch, channels=chans, width=width,
+        io_dtype=_lib.dtype_enum(x.dtype), activation=_lib.ACT_SILU if act in ("silu", "swish") else _lib.ACT_IDENTITY)
+    _lib.call("ssm_conv1d_update", args, dev)
+    return out
+
+
 # ---------------------------------------------------------------------------
 # diagonal chunk scan (the reference's ``ssd_chunk_scan``)
 # ---------------------------------------------------------------------------
@@ -736,6 +781,7 @@ __all__ = [
     "selective_state_step",
     "decode_step",
     "mamba2_decode_step",
+    "conv_window_step",
     "ssd_chunk_scan",
     "dw_causal_conv",
     "fused_layer_norm",

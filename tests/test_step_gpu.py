@@ -281,6 +281,35 @@ def test_mamba2_decode_step_options_and_errors():
                                None, A.cuda())
 
 
+@pytest.mark.parametrize("io", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("K,act", [(4, "silu"), (2, "identity"), (7, "silu"), (1, "silu")])
+def test_conv_window_step_follows_the_full_convolution(io, K, act):
+    """Feeding a sequence token by token through conv_window_step (window starting at zero) gives the
+    columns of dw_causal_conv over the whole sequence; x is read in place from a wider matrix."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(K)
+    Bsz, Cn, L = 3, 70, 9
+    wide = torch.randn(Bsz, L, Cn + 5, generator=g).to(io)
+    w = torch.rand(Cn, K, generator=g) - 0.5
+    cb = torch.randn(Cn, generator=g) * 0.1
+    xs = wide[:, :, 2:2 + Cn]
+    x32 = torch.nn.functional.pad(xs.float().transpose(1, 2), (K - 1, 0))
+    full = torch.nn.functional.conv1d(x32, w[:, None], cb, groups=Cn)
+    if act == "silu":
+        full = torch.nn.functional.silu(full)
+    state = torch.zeros(Bsz, Cn, K, dtype=io).cuda()
+    wide_gpu = wide.cuda()
+    for t in range(L):
+        out = ops.conv_window_step(state, wide_gpu[:, t, 2:2 + Cn], w.cuda(), cb.cuda(), activation=act)
+        assert out.dtype == io
+        torch.testing.assert_close(out.float().cpu(), full[:, :, t], **(FP32_TOL if io == torch.float32 else HALF_TOL))
+    torch.testing.assert_close(state.float().cpu(), x32[:, :, -K:], rtol=0, atol=0)
+    with pytest.raises(ValueError):
+        ops.conv_window_step(state, wide_gpu[:, 0, :Cn - 1], w.cuda(), cb.cuda())
+    with pytest.raises(ValueError):
+        ops.conv_window_step(state, wide_gpu[:, 0, :Cn], w.cuda(), cb.cuda(), activation="relu")
+
+
 # ---------------------------------------------------------------------------
 # backward: gradients of (y, new_state) against float64 autograd through the
 # CPU restatement of the step
