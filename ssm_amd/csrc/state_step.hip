@@ -10,6 +10,8 @@
 // the partial dot products are combined with a butterfly inside the wave.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace ssm {
 
 struct StepParams {
@@ -48,6 +50,35 @@ __device__ __forceinline__ void load_vec_rt(const void *p, int dtype, size_t off
   if (dtype == SSM_F32) load_vec<float, VEC>(reinterpret_cast<const float *>(p) + off, v);
   else if (dtype == SSM_BF16) load_vec<bf16_t, VEC>(reinterpret_cast<const bf16_t *>(p) + off, v);
   else load_vec<f16_t, VEC>(reinterpret_cast<const f16_t *>(p) + off, v);
+}
+
+// Accesses of the activations and projections.  io_t = void: the element type is looked up at run time
+// (any mix of dtypes); otherwise x, dt, z, B, C, the conv window and the outputs all have type io_t and
+// the reads of a thread are straight-line code that the compiler issues together.
+template <typename io_t>
+__device__ __forceinline__ float ld_io(const void *p, int dtype, size_t i) {
+  if constexpr (std::is_void<io_t>::value) return load_as_f32(p, dtype, i);
+  else return to_f32(reinterpret_cast<const io_t *>(p)[i]);
+}
+template <typename io_t>
+__device__ __forceinline__ void st_io(void *p, int dtype, size_t i, float v) {
+  if constexpr (std::is_void<io_t>::value) store_from_f32(p, dtype, i, v);
+  else reinterpret_cast<io_t *>(p)[i] = from_f32<io_t>(v);
+}
+template <typename io_t, int VEC>
+__device__ __forceinline__ void ld_vec_io(const void *p, int dtype, size_t off, float (&v)[VEC]) {
+  if constexpr (std::is_void<io_t>::value) load_vec_rt<VEC>(p, dtype, off, v);
+  else load_vec<io_t, VEC>(reinterpret_cast<const io_t *>(p) + off, v);
+}
+template <typename io_t>
+__device__ __forceinline__ float round_io(float v, int dtype) {
+  if constexpr (std::is_void<io_t>::value) {
+    if (dtype == SSM_BF16) return to_f32(from_f32<bf16_t>(v));
+    if (dtype == SSM_F16) return to_f32(from_f32<f16_t>(v));
+    return v;
+  } else {
+    return to_f32(from_f32<io_t>(v));
+  }
 }
 
 template <typename state_t, int VEC>
@@ -150,7 +181,7 @@ __global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
 // third of the cache traffic (A is as large as the state) and most of the small reads.  The three
 // per-row scalars x, dt, z are fetched by lanes 0, 1, 2 of the row with one instruction and
 // shared through the wave.
-template <typename state_t, int RB>
+template <typename state_t, typename io_t, bool CONV, int RB>
 __global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) {
   constexpr int VEC = 4;
   const int tpr = 1 << p.tpr_log2;
@@ -159,8 +190,8 @@ __global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) 
   const int sub = (int)(gid & (tpr - 1));
   const size_t ncols = (size_t)p.dim * (p.batch / RB);
   const bool live = col < ncols;
-  const size_t cc = live ? col : 0;
-  const int d = (int)(cc % p.dim), bg = (int)(cc / p.dim);
+  const unsigned cc = live ? (unsigned)col : 0u;          // batch * dim < 2^27: 32-bit index arithmetic
+  const int d = (int)(cc % (unsigned)p.dim), bg = (int)(cc / (unsigned)p.dim);
   const int N = p.nstate, n0 = sub * VEC;
   const int lane = lane_id(), base = lane & ~(tpr - 1);
 
@@ -169,26 +200,32 @@ __global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) 
   const float bias = p.bias ? p.bias[d] : 0.0f;
   const float Dk = p.Dk ? p.Dk[d] : 0.0f;
   const int K = p.conv_k;
-  const float tap = (p.conv_state && sub < K) ? p.conv_w[(size_t)d * K + sub] : 0.0f;
-  const float cbias = (p.conv_state && p.conv_b) ? p.conv_b[d] : 0.0f;
-  const void *scal_ptr = sub == 0 ? p.x : (sub == 1 ? p.dt : p.z);
-  const bool scal_on = sub < 2 || (sub == 2 && p.z);
+  float tap = 0.0f;
+  if (CONV) {
+    tap = p.conv_w[(size_t)d * K + min(sub, K - 1)];
+    if (sub >= K) tap = 0.0f;
+  }
+  const float cbias = (CONV && p.conv_b) ? p.conv_b[d] : 0.0f;
+  // every lane reads one of the row's scalars (lanes past the third repeat x): no lane-dependent branch
+  const void *scal_ptr = sub == 1 ? p.dt : (sub == 2 && p.z ? p.z : p.x);
+  const int bgrp = p.b_kind == SSM_PROJ_BGNL ? d / (p.dim / p.b_groups) : 0;
+  const int cgrp = p.c_kind == SSM_PROJ_BGNL ? d / (p.dim / p.c_groups) : 0;
+  const int win_k = min(sub + 1, max(K - 1, 0));
 
   float h[RB][VEC], bv[RB][VEC], cv[RB][VEC], scal[RB], win[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int b = bg * RB + rb;
     const size_t r = (size_t)b * p.dim + d;
-    size_t b_off, c_off;
-    if (p.b_kind == SSM_PROJ_BGNL) b_off = ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * N;
-    else b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
-    if (p.c_kind == SSM_PROJ_BGNL) c_off = ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * N;
-    else c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+    const size_t b_off = p.b_kind == SSM_PROJ_BGNL ? ((size_t)b * p.b_groups + bgrp) * N
+                                                    : ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+    const size_t c_off = p.c_kind == SSM_PROJ_BGNL ? ((size_t)b * p.c_groups + cgrp) * N
+                                                    : ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
     load_vec<state_t, VEC>(reinterpret_cast<const state_t *>(p.state) + r * N + n0, h[rb]);
-    load_vec_rt<VEC>(p.Bp, p.bc_dtype, b_off + n0, bv[rb]);
-    load_vec_rt<VEC>(p.Cp, p.bc_dtype, c_off + n0, cv[rb]);
-    scal[rb] = scal_on ? load_as_f32(scal_ptr, p.io_dtype, r) : 0.0f;
-    win[rb] = (p.conv_state && sub + 1 < K) ? load_as_f32(p.conv_state, p.io_dtype, r * K + sub + 1) : 0.0f;
+    ld_vec_io<io_t, VEC>(p.Bp, p.bc_dtype, b_off + n0, bv[rb]);
+    ld_vec_io<io_t, VEC>(p.Cp, p.bc_dtype, c_off + n0, cv[rb]);
+    scal[rb] = ld_io<io_t>(scal_ptr, p.io_dtype, r);
+    win[rb] = CONV ? ld_io<io_t>(p.conv_state, p.io_dtype, r * K + win_k) : 0.0f;
   }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -198,17 +235,15 @@ __global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) 
     float dtv = __shfl(scal[rb], base + 1, WAVE) + bias;
     const float zv = __shfl(scal[rb], base + 2, WAVE);
     if (p.softplus) dtv = softplus_f32(dtv);
-    if (p.conv_state) {
+    if (CONV) {
       // window <- (window[1:], x); x <- act(bias + sum_k w[k] window[k]); lane k of the row owns tap k
       const float v = sub + 1 < K ? win[rb] : xv;
       float part = sub < K ? v * tap : 0.0f;
-      if (live && sub < K) store_from_f32(p.conv_state, p.io_dtype, r * K + sub, v);
+      if (live && sub < K) st_io<io_t>(p.conv_state, p.io_dtype, r * K + sub, v);
       for (int m = tpr >> 1; m >= 1; m >>= 1) part += __shfl_xor(part, m, WAVE);
       part += cbias;
-      xv = p.conv_silu ? silu_f32(part) : part;
-      if (p.io_dtype == SSM_BF16) xv = to_f32(from_f32<bf16_t>(xv));
-      else if (p.io_dtype == SSM_F16) xv = to_f32(from_f32<f16_t>(xv));
-      if (p.conv_out && live && sub == 0) store_from_f32(p.conv_out, p.io_dtype, r, xv);
+      xv = round_io<io_t>(p.conv_silu ? silu_f32(part) : part, p.io_dtype);
+      if (p.conv_out && live && sub == 0) st_io<io_t>(p.conv_out, p.io_dtype, r, xv);
     }
     const float dx = dtv * xv, dt2 = dtv * LOG2E;
     float acc = 0.0f;
@@ -224,9 +259,16 @@ __global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) 
     if (live && sub == 0) {
       float y = __builtin_fmaf(Dk, xv, acc);
       if (p.z) y *= silu_f32(zv);
-      store_from_f32(p.out, p.io_dtype, r, y);
+      st_io<io_t>(p.out, p.io_dtype, r, y);
     }
   }
+}
+
+template <typename state_t, typename io_t>
+static void launch_rb(const StepParams &p, unsigned grid, hipStream_t stream) {
+  constexpr int RB = 4;
+  if (p.conv_state) hipLaunchKernelGGL((state_step_rb_kernel<state_t, io_t, true, RB>), dim3(grid), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((state_step_rb_kernel<state_t, io_t, false, RB>), dim3(grid), dim3(256), 0, stream, p);
 }
 
 template <typename state_t>
@@ -240,8 +282,18 @@ static int launch_step(const StepParams &p0, bool vec4, hipStream_t stream) {
   constexpr int RB = 4;
   if (vec4 && p.nstate == (4 << lg) && lg >= 2 && p.batch % RB == 0 && (!p.conv_state || p.conv_k <= (1 << lg))) {
     const size_t threads_rb = ((size_t)p.dim * (p.batch / RB)) << lg;
-    hipLaunchKernelGGL((state_step_rb_kernel<state_t, RB>), dim3((unsigned)((threads_rb + 255) / 256)), dim3(256), 0,
-                       stream, p);
+    const unsigned grid_rb = (unsigned)((threads_rb + 255) / 256);
+    // float32 states with activations and projections of one type: element types known at compile time
+    bool done = false;
+    if constexpr (std::is_same<state_t, float>::value) {
+      if (p.io_dtype == p.bc_dtype) {
+        if (p.io_dtype == SSM_BF16) launch_rb<state_t, bf16_t>(p, grid_rb, stream);
+        else if (p.io_dtype == SSM_F16) launch_rb<state_t, f16_t>(p, grid_rb, stream);
+        else launch_rb<state_t, float>(p, grid_rb, stream);
+        done = true;
+      }
+    }
+    if (!done) launch_rb<state_t, void>(p, grid_rb, stream);
     SSM_CHECK_LAUNCH("ssm_state_step");
     return SSM_OK;
   }
