@@ -13,6 +13,8 @@
 // per-row partials and folded in a fixed order afterwards (no atomics).
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace ssm {
 
 struct StepBwdParams {
@@ -85,6 +87,89 @@ __global__ __launch_bounds__(256) void state_step_bwd_kernel(const StepBwdParams
   p.pbias[r] = ddt;
 }
 
+// The same with one lane per (row, state) for N = 2^k <= 64: every access of the state-sized tensors is
+// coalesced, the sums over a row's states are butterflies inside the wave.  io_t = void looks the element
+// types up at run time; otherwise x, dt, z, B, C and the gradients of the activations have type io_t and
+// the state tensors are float32, so that the reads are straight-line code issued together.
+template <typename io_t>
+__global__ __launch_bounds__(256) void state_step_bwd_lanes_kernel(const StepBwdParams p, const int lg) {
+  constexpr bool RT = std::is_void<io_t>::value;
+  using act_t = typename std::conditional<RT, float, io_t>::type;
+  const int N = 1 << lg;
+  const size_t rows = (size_t)p.batch * p.dim;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const bool live = gid < (rows << lg);
+  const size_t g = live ? gid : 0;
+  const unsigned r = (unsigned)(g >> lg);
+  const int n = (int)(g & (size_t)(N - 1));
+  const int b = (int)(r / (unsigned)p.dim), d = (int)(r % (unsigned)p.dim);
+  const size_t b_off = p.b_kind == SSM_PROJ_BGNL ? ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * N
+                                                  : ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+  const size_t c_off = p.c_kind == SSM_PROJ_BGNL ? ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * N
+                                                  : ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
+  auto act = [&](const void *q, size_t i) -> float {
+    if constexpr (RT) return load_as_f32(q, p.io_dtype, i);
+    else return to_f32(reinterpret_cast<const act_t *>(q)[i]);
+  };
+  auto proj = [&](const void *q, size_t i) -> float {
+    if constexpr (RT) return load_as_f32(q, p.bc_dtype, i);
+    else return to_f32(reinterpret_cast<const act_t *>(q)[i]);
+  };
+  auto st = [&](const void *q, size_t i) -> float {
+    if constexpr (RT) return load_as_f32(q, p.state_dtype, i);
+    else return reinterpret_cast<const float *>(q)[i];
+  };
+  // absent inputs read a present one and drop the value: no branch around a read
+  const float dt_raw = act(p.dt, r), xv = act(p.x, r);
+  const float gy_raw = act(p.gy ? p.gy : p.x, r), z_raw = act(p.z ? p.z : p.x, r);
+  const float h = st(p.state, g), gs_raw = st(p.gstate ? p.gstate : p.state, g);
+  const float A = p.A[(size_t)d * N + n], Bn = proj(p.Bp, b_off + n), Cn = proj(p.Cp, c_off + n);
+  const float bias = p.bias ? p.bias[d] : 0.0f, Dv = p.Dk ? p.Dk[d] : 0.0f;
+
+  const float pre = dt_raw + bias;
+  const float step = p.softplus ? softplus_f32(pre) : pre;
+  const float dstep_dpre = p.softplus ? (pre > 20.0f ? 1.0f : sigmoid_f32(pre)) : 1.0f;
+  const float gy = p.gy ? gy_raw : 0.0f;
+  float gate = 1.0f, dgate = 0.0f;
+  if (p.z) {
+    const float sg = sigmoid_f32(z_raw);
+    gate = z_raw * sg;
+    dgate = sg * (1.0f + z_raw * (1.0f - sg));
+  }
+  const float g0 = gy * gate;
+  const float a = exp2_hw(step * A * LOG2E);
+  const float hn = __builtin_fmaf(a, h, step * xv * Bn);
+  const float gn = (p.gstate ? gs_raw : 0.0f) + g0 * Cn;
+  float y0 = hn * Cn, dstep = gn * __builtin_fmaf(h * a, A, xv * Bn), sum_gb = gn * Bn;
+  for (int m = N >> 1; m >= 1; m >>= 1) {
+    y0 += __shfl_xor(y0, m, WAVE);
+    dstep += __shfl_xor(dstep, m, WAVE);
+    sum_gb += __shfl_xor(sum_gb, m, WAVE);
+  }
+  if (!live) return;
+  if constexpr (RT) store_rt(p.dstate, p.state_dtype, g, gn * a);
+  else reinterpret_cast<float *>(p.dstate)[g] = gn * a;
+  p.pA[g] = gn * h * a * step;
+  p.pB[g] = gn * step * xv;
+  p.pC[g] = g0 * hn;
+  if (n == 0) {
+    y0 = __builtin_fmaf(Dv, xv, y0);
+    const float ddt = dstep * dstep_dpre;
+    const float dxv = __builtin_fmaf(g0, Dv, step * sum_gb);
+    if constexpr (RT) {
+      store_rt(p.dx, p.io_dtype, r, dxv);
+      store_rt(p.ddt, p.io_dtype, r, ddt);
+      if (p.dz) store_rt(p.dz, p.io_dtype, r, gy * y0 * dgate);
+    } else {
+      reinterpret_cast<act_t *>(p.dx)[r] = from_f32<act_t>(dxv);
+      reinterpret_cast<act_t *>(p.ddt)[r] = from_f32<act_t>(ddt);
+      if (p.dz) reinterpret_cast<act_t *>(p.dz)[r] = from_f32<act_t>(gy * y0 * dgate);
+    }
+    p.pD[r] = g0 * xv;
+    p.pbias[r] = ddt;
+  }
+}
+
 }  // namespace ssm
 
 static size_t step_bwd_floats(int batch, int dim, int nstate) {
@@ -137,7 +222,18 @@ extern "C" int ssm_state_step_bwd(const ssm_state_step_bwd_args *a, void *hip_st
   p.c_groups = a->c_kind == SSM_PROJ_BGNL ? a->c_groups : 1;
   p.softplus = a->dt_softplus ? 1 : 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  hipLaunchKernelGGL(state_step_bwd_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, s, p);
+  int lg = 0;
+  while ((1 << lg) < a->nstate) ++lg;
+  if ((1 << lg) == a->nstate && lg <= 6) {
+    const dim3 grid((unsigned)(((rows << lg) + 255) / 256));
+    const bool typed = a->state_dtype == SSM_F32 && a->io_dtype == a->bc_dtype;
+    if (typed && a->io_dtype == SSM_BF16) hipLaunchKernelGGL(state_step_bwd_lanes_kernel<bf16_t>, grid, dim3(256), 0, s, p, lg);
+    else if (typed && a->io_dtype == SSM_F16) hipLaunchKernelGGL(state_step_bwd_lanes_kernel<f16_t>, grid, dim3(256), 0, s, p, lg);
+    else if (typed && a->io_dtype == SSM_F32) hipLaunchKernelGGL(state_step_bwd_lanes_kernel<float>, grid, dim3(256), 0, s, p, lg);
+    else hipLaunchKernelGGL(state_step_bwd_lanes_kernel<void>, grid, dim3(256), 0, s, p, lg);
+  } else {
+    hipLaunchKernelGGL(state_step_bwd_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, s, p);
+  }
   SSM_CHECK_LAUNCH("ssm_state_step_bwd");
 
   const int Bn = a->batch, D = a->dim, N = a->nstate;
