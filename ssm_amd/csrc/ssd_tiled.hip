@@ -8,8 +8,20 @@
 //                         + sum_{s<=l} CB[l][s] exp(cs_l - cs_s) dt_s x[s][p]  + D x[l][p],  times silu(z)
 #include "ssd_common.hpp"
 
+#include <type_traits>
+
 namespace ssm {
 namespace {
+
+// Element reads while staging.  T = void: the element type is looked up at run time (calls that mix
+// types); otherwise every streamed tensor of the call has type T.  Indices are clamped into the tensor
+// and the value dropped afterwards where a tile hangs over an edge, so that no read sits behind a
+// lane-dependent branch and a thread's reads of one slab are in flight together.
+template <typename T>
+__device__ __forceinline__ float tl_ld(const void *p, int dtype, size_t i) {
+  if constexpr (std::is_void<T>::value) return load_as_f32(p, dtype, i);
+  else return to_f32(reinterpret_cast<const T *>(p)[i]);
+}
 
 constexpr int TL_THREADS = 256;   // 4 waves, 2 x 2 blocks of 32 x 32
 constexpr int TL_MN = 64;         // tile edge of the output
@@ -34,6 +46,7 @@ __device__ __forceinline__ void slab_mma(const Slabs &t, int wr, int wc, int lan
 __device__ __forceinline__ void along_m(int e, int &k, int &m) { m = e & (TL_MN - 1); k = e >> 6; }
 __device__ __forceinline__ void along_k(int e, int &k, int &m) { k = e & (TL_K - 1); m = e >> 5; }
 
+template <typename T>
 __global__ __launch_bounds__(TL_THREADS) void ssd_chunk_state_tiled_kernel(const SsdStateParams p) {
   __shared__ Slabs t;
   extern __shared__ float wq[];                            // weight of every step of the chunk
@@ -66,13 +79,12 @@ __global__ __launch_bounds__(TL_THREADS) void ssd_chunk_state_tiled_kernel(const
     for (int j = 0; j < TL_K * TL_MN / TL_THREADS; ++j) {
       int k, m;
       along_m(tid + TL_THREADS * j, k, m);
-      const int l = k0 + k;
+      const int l = min(k0 + k, qlen - 1);
       const size_t row = (size_t)b * d.len + c * Q + l;
-      float xv = 0.0f, bv = 0.0f;
-      if (l < qlen) {
-        if (p0 + m < d.hdim) xv = load_as_f32(p.x, p.x_dtype, (row * d.heads + h) * d.hdim + p0 + m);
-        if (n0 + m < d.nstate) bv = load_as_f32(p.Bm, p.b_dtype, (row * d.groups + g) * d.nstate + n0 + m) * wq[l];
-      }
+      float xv = tl_ld<T>(p.x, p.x_dtype, (row * d.heads + h) * d.hdim + min(p0 + m, d.hdim - 1));
+      float bv = tl_ld<T>(p.Bm, p.b_dtype, (row * d.groups + g) * d.nstate + min(n0 + m, d.nstate - 1)) * wq[l];
+      if (k0 + k >= qlen || p0 + m >= d.hdim) xv = 0.0f;
+      if (k0 + k >= qlen || n0 + m >= d.nstate) bv = 0.0f;
       t.a[k][m] = xv;
       t.b[k][m] = bv;
     }
@@ -88,6 +100,7 @@ __global__ __launch_bounds__(TL_THREADS) void ssd_chunk_state_tiled_kernel(const
   }
 }
 
+template <typename T>
 __global__ __launch_bounds__(TL_THREADS) void ssd_chunk_scan_tiled_kernel(const SsdScanParams p) {
   __shared__ Slabs t;
   extern __shared__ float dyn[];                           // cs[Q], dt[Q] of the chunk
@@ -117,14 +130,12 @@ __global__ __launch_bounds__(TL_THREADS) void ssd_chunk_scan_tiled_kernel(const 
     for (int j = 0; j < TL_K * TL_MN / TL_THREADS; ++j) {
       int k, m;
       along_k(tid + TL_THREADS * j, k, m);
-      const int n = k0 + k;
-      float cv = 0.0f, sv = 0.0f;
-      if (n < d.nstate) {
-        if (l0 + m < qlen)
-          cv = load_as_f32(p.Cm, p.c_dtype, (((size_t)b * d.len + c * Q + l0 + m) * d.groups + g) * d.nstate + n);
-        if (p0 + m < d.hdim)
-          sv = load_as_f32(p.prev, p.states_dtype, ((((size_t)b * d.nchunks + c) * d.heads + h) * d.hdim + p0 + m) * d.nstate + n);
-      }
+      const int n = min(k0 + k, d.nstate - 1);
+      float cv = tl_ld<T>(p.Cm, p.c_dtype, (((size_t)b * d.len + c * Q + min(l0 + m, qlen - 1)) * d.groups + g) * d.nstate + n);
+      float sv = tl_ld<T>(p.prev, p.states_dtype,
+                          ((((size_t)b * d.nchunks + c) * d.heads + h) * d.hdim + min(p0 + m, d.hdim - 1)) * d.nstate + n);
+      if (k0 + k >= d.nstate || l0 + m >= qlen) cv = 0.0f;
+      if (k0 + k >= d.nstate || p0 + m >= d.hdim) sv = 0.0f;
       t.a[k][m] = cv;
       t.b[k][m] = sv;
     }
@@ -150,21 +161,19 @@ __global__ __launch_bounds__(TL_THREADS) void ssd_chunk_scan_tiled_kernel(const 
     for (int j = 0; j < TL_K * TL_MN / TL_THREADS; ++j) {
       int k, m;
       along_k(tid + TL_THREADS * j, k, m);
-      const int s = k0 + k, l = l0 + m;
-      float v = 0.0f;
-      if (s <= l && l < qlen)
-        v = load_as_f32(p.CB, p.cb_dtype, ((((size_t)b * d.nchunks + c) * d.groups + g) * Q + l) * Q + s) *
-            decay_exp(csq[l] - csq[s]) * dtq[s];
+      const int s = min(k0 + k, Q - 1), l = min(l0 + m, Q - 1);
+      float v = tl_ld<T>(p.CB, p.cb_dtype, ((((size_t)b * d.nchunks + c) * d.groups + g) * Q + l) * Q + s) *
+                decay_exp(csq[l] - csq[s]) * dtq[s];
+      if (k0 + k > l0 + m || l0 + m >= qlen) v = 0.0f;
       t.a[k][m] = v;
     }
 #pragma unroll
     for (int j = 0; j < TL_K * TL_MN / TL_THREADS; ++j) {
       int k, m;
       along_m(tid + TL_THREADS * j, k, m);
-      const int s = k0 + k;
-      float v = 0.0f;
-      if (s < send && p0 + m < d.hdim)
-        v = load_as_f32(p.x, p.x_dtype, (((size_t)b * d.len + c * Q + s) * d.heads + h) * d.hdim + p0 + m);
+      const int s = min(k0 + k, send - 1);
+      float v = tl_ld<T>(p.x, p.x_dtype, (((size_t)b * d.len + c * Q + s) * d.heads + h) * d.hdim + min(p0 + m, d.hdim - 1));
+      if (k0 + k >= send || p0 + m >= d.hdim) v = 0.0f;
       t.b[k][m] = v;
     }
     __syncthreads();
@@ -179,14 +188,15 @@ __global__ __launch_bounds__(TL_THREADS) void ssd_chunk_scan_tiled_kernel(const 
     if (l >= qlen) continue;
     const size_t at = (((size_t)b * d.len + c * Q + l) * d.heads + h) * d.hdim + pp;
     float v = acc[r];
-    if (p.Dk) v = __builtin_fmaf(Dv, load_as_f32(p.x, p.x_dtype, at), v);
-    if (p.z) v *= silu_f32(load_as_f32(p.z, p.z_dtype, at));
+    if (p.Dk) v = __builtin_fmaf(Dv, tl_ld<T>(p.x, p.x_dtype, at), v);
+    if (p.z) v *= silu_f32(tl_ld<T>(p.z, p.z_dtype, at));
     store_any(p.y, p.y_dtype, at, v);
   }
 }
 
 // CB[l][s] = <a_l, b_s> over the K columns of both, zero above the diagonal when causal or across
 // sequences of a packed batch.
+template <typename T>
 __global__ __launch_bounds__(TL_THREADS) void ssd_bmm_tiled_kernel(const SsdBmmParams p) {
   __shared__ Slabs t;
   const int Q = p.chunk, tiles = (Q + TL_MN - 1) / TL_MN;
@@ -205,11 +215,11 @@ __global__ __launch_bounds__(TL_THREADS) void ssd_bmm_tiled_kernel(const SsdBmmP
     for (int j = 0; j < TL_K * TL_MN / TL_THREADS; ++j) {
       int k, m;
       along_k(tid + TL_THREADS * j, k, m);
-      float av = 0.0f, bv = 0.0f;
-      if (k0 + k < p.kdim) {
-        if (l0 + m < qlen) av = load_as_f32(p.a, p.in_dtype, (((size_t)b * p.len + c * Q + l0 + m) * p.groups + g) * p.kdim + k0 + k);
-        if (s0 + m < qlen) bv = load_as_f32(p.b, p.in_dtype, (((size_t)b * p.len + c * Q + s0 + m) * p.groups + g) * p.kdim + k0 + k);
-      }
+      const int kk = min(k0 + k, p.kdim - 1);
+      float av = tl_ld<T>(p.a, p.in_dtype, (((size_t)b * p.len + c * Q + min(l0 + m, qlen - 1)) * p.groups + g) * p.kdim + kk);
+      float bv = tl_ld<T>(p.b, p.in_dtype, (((size_t)b * p.len + c * Q + min(s0 + m, qlen - 1)) * p.groups + g) * p.kdim + kk);
+      if (k0 + k >= p.kdim || l0 + m >= qlen) av = 0.0f;
+      if (k0 + k >= p.kdim || s0 + m >= qlen) bv = 0.0f;
       t.a[k][m] = av;
       t.b[k][m] = bv;
     }
@@ -237,7 +247,10 @@ bool ssd_bmm_tiled(const SsdBmmParams &p, hipStream_t s) {
   const size_t per = (size_t)((p.chunk + TL_MN - 1) / TL_MN);
   const size_t tiles = (size_t)p.batch * p.nchunks * p.groups * per * per;
   if (tiles >= ((size_t)1 << 31)) return false;
-  hipLaunchKernelGGL(ssd_bmm_tiled_kernel, dim3((unsigned)tiles), dim3(TL_THREADS), 0, s, p);
+  const dim3 grid((unsigned)tiles), block(TL_THREADS);
+  if (p.in_dtype == SSM_F32) hipLaunchKernelGGL(ssd_bmm_tiled_kernel<float>, grid, block, 0, s, p);
+  else if (p.in_dtype == SSM_BF16) hipLaunchKernelGGL(ssd_bmm_tiled_kernel<bf16_t>, grid, block, 0, s, p);
+  else hipLaunchKernelGGL(ssd_bmm_tiled_kernel<f16_t>, grid, block, 0, s, p);
   return true;
 }
 
@@ -245,7 +258,13 @@ bool ssd_chunk_state_tiled(const SsdStateParams &p, hipStream_t s) {
   const SsdDims &d = p.d;
   const size_t tiles = (size_t)d.batch * d.nchunks * d.heads * ((d.hdim + TL_MN - 1) / TL_MN) * ((d.nstate + TL_MN - 1) / TL_MN);
   if (d.chunk > TL_MAX_CHUNK || tiles >= ((size_t)1 << 31)) return false;
-  hipLaunchKernelGGL(ssd_chunk_state_tiled_kernel, dim3((unsigned)tiles), dim3(TL_THREADS), (size_t)d.chunk * sizeof(float), s, p);
+  const dim3 grid((unsigned)tiles), block(TL_THREADS);
+  const size_t lds = (size_t)d.chunk * sizeof(float);
+  const bool same = p.x_dtype == p.b_dtype;
+  if (same && p.x_dtype == SSM_F32) hipLaunchKernelGGL(ssd_chunk_state_tiled_kernel<float>, grid, block, lds, s, p);
+  else if (same && p.x_dtype == SSM_BF16) hipLaunchKernelGGL(ssd_chunk_state_tiled_kernel<bf16_t>, grid, block, lds, s, p);
+  else if (same && p.x_dtype == SSM_F16) hipLaunchKernelGGL(ssd_chunk_state_tiled_kernel<f16_t>, grid, block, lds, s, p);
+  else hipLaunchKernelGGL(ssd_chunk_state_tiled_kernel<void>, grid, block, lds, s, p);
   return true;
 }
 
@@ -253,7 +272,14 @@ bool ssd_chunk_scan_tiled(const SsdScanParams &p, hipStream_t s) {
   const SsdDims &d = p.d;
   const size_t tiles = (size_t)d.batch * d.nchunks * d.heads * ((d.hdim + TL_MN - 1) / TL_MN) * ((d.chunk + TL_MN - 1) / TL_MN);
   if (d.chunk > TL_MAX_CHUNK || tiles >= ((size_t)1 << 31)) return false;
-  hipLaunchKernelGGL(ssd_chunk_scan_tiled_kernel, dim3((unsigned)tiles), dim3(TL_THREADS), (size_t)2 * d.chunk * sizeof(float), s, p);
+  const dim3 grid((unsigned)tiles), block(TL_THREADS);
+  const size_t lds = (size_t)2 * d.chunk * sizeof(float);
+  const bool same = p.x_dtype == p.c_dtype && p.x_dtype == p.cb_dtype && p.x_dtype == p.states_dtype &&
+                    (!p.z || p.z_dtype == p.x_dtype);
+  if (same && p.x_dtype == SSM_F32) hipLaunchKernelGGL(ssd_chunk_scan_tiled_kernel<float>, grid, block, lds, s, p);
+  else if (same && p.x_dtype == SSM_BF16) hipLaunchKernelGGL(ssd_chunk_scan_tiled_kernel<bf16_t>, grid, block, lds, s, p);
+  else if (same && p.x_dtype == SSM_F16) hipLaunchKernelGGL(ssd_chunk_scan_tiled_kernel<f16_t>, grid, block, lds, s, p);
+  else hipLaunchKernelGGL(ssd_chunk_scan_tiled_kernel<void>, grid, block, lds, s, p);
   return true;
 }
 
