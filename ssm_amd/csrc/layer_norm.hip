@@ -174,6 +174,126 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_kernel(const NormParams p
   }
 }
 
+// The one-wavefront-per-row kernel with the element types known at compile time (XT: x and y; RT: residual
+// and residual_out) for rows of a multiple of four columns with 16-byte aligned tensors.  Every read is
+// unconditional - column indices are clamped into the row, an absent residual or bias reads a stand-in of
+// the same type whose value is dropped - so a wavefront's reads are in flight together instead of one
+// behind the other, which is what a call on a handful of rows (a decoding step) waits for.
+template <typename T, int VEC>
+__device__ __forceinline__ void ld_pack(const void *p, size_t i, float (&v)[VEC]) {
+  const Pack<T, VEC> raw = *reinterpret_cast<const Pack<T, VEC> *>(reinterpret_cast<const T *>(p) + i);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) v[j] = to_f32(raw.v[j]);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void st_pack(void *p, size_t i, const float (&v)[VEC]) {
+  Pack<T, VEC> raw;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) raw.v[j] = from_f32<T>(v[j]);
+  *reinterpret_cast<Pack<T, VEC> *>(reinterpret_cast<T *>(p) + i) = raw;
+}
+
+template <int TRIPS, typename XT, typename RT>
+__global__ __launch_bounds__(LN_THREADS) void norm_fwd_typed_kernel(const NormParams p) {
+  constexpr int VEC = 4;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row = (int)(blockIdx.x * LN_WAVES + wave);
+  if (row >= p.rows) return;
+  const int H = p.hidden;
+  const size_t base = (size_t)row * H;
+  const bool has_res = p.res != nullptr, has_b = p.b != nullptr;
+  // stand-ins of the right element type: residual_out (type RT) or, without one, x (then RT = XT)
+  const void *resp = has_res ? p.res : (p.res_out ? (const void *)p.res_out : p.x);
+  const float *bp = has_b ? p.b : p.w;
+  float v[TRIPS][VEC], r[TRIPS][VEC];
+  float sum = 0.0f;
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int colc = min((k * WAVE + lane) * VEC, H - VEC);
+    ld_pack<XT, VEC>(p.x, base + colc, v[k]);
+    ld_pack<RT, VEC>(resp, base + colc, r[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int col = (k * WAVE + lane) * VEC;
+    const bool live = col < H;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      if (!has_res) r[k][i] = 0.0f;
+      if (p.prenorm) v[k][i] += r[k][i];
+      if (!live) v[k][i] = 0.0f;
+      sum += v[k][i];
+    }
+    if (p.res_out && live) st_pack<RT, VEC>(p.res_out, base + col, v[k]);
+  }
+  float wv[TRIPS][VEC], bv[TRIPS][VEC];
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int colc = min((k * WAVE + lane) * VEC, H - VEC);
+    ld_pack<float, VEC>(p.w, colc, wv[k]);
+    ld_pack<float, VEC>(bp, colc, bv[k]);
+  }
+  const float inv_h = 1.0f / (float)H;
+  float mean = 0.0f;
+  if (!p.is_rms) mean = wave_sum(sum) * inv_h;
+  float sq = 0.0f;
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const bool live = (k * WAVE + lane) * VEC < H;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float c = live ? v[k][i] - mean : 0.0f;
+      sq = __builtin_fmaf(c, c, sq);
+    }
+  }
+  const float rstd = 1.0f / sqrtf(wave_sum(sq) * inv_h + p.eps);
+  if (lane == 0) {
+    if (p.mean) p.mean[row] = mean;
+    if (p.rstd) p.rstd[row] = rstd;
+  }
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int col = (k * WAVE + lane) * VEC;
+    float out[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float o = (v[k][i] - mean) * rstd * wv[k][i];
+      if (has_b) o += bv[k][i];
+      if (has_res && !p.prenorm) o += r[k][i];
+      out[i] = o;
+    }
+    if (col < H) st_pack<XT, VEC>(p.y, base + col, out);
+  }
+}
+
+template <typename XT, typename RT>
+static void launch_norm_fwd_typed(const NormParams &p, int per_lane, unsigned grid, hipStream_t s) {
+  if (per_lane <= 4) hipLaunchKernelGGL((norm_fwd_typed_kernel<1, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
+  else if (per_lane <= 8) hipLaunchKernelGGL((norm_fwd_typed_kernel<2, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
+  else if (per_lane <= 12) hipLaunchKernelGGL((norm_fwd_typed_kernel<3, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
+  else if (per_lane <= 16) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
+  else hipLaunchKernelGGL((norm_fwd_typed_kernel<8, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
+}
+
+// True when the call was taken by a typed kernel.
+static bool norm_fwd_typed(const NormParams &p, int per_lane, unsigned grid, hipStream_t s) {
+  if (per_lane > 32 || p.hidden < 4) return false;
+  // residual and residual_out must agree on one type, float32 or that of x
+  int rt = -1;
+  if (p.res) rt = p.res_dtype;
+  if (p.res_out) {
+    if (rt >= 0 && p.res_out_dtype != rt) return false;
+    rt = p.res_out_dtype;
+  }
+  if (rt < 0) rt = p.x_dtype;
+  if (rt != SSM_F32 && rt != p.x_dtype) return false;
+  const bool rf = rt == SSM_F32;
+  if (p.x_dtype == SSM_BF16) rf ? launch_norm_fwd_typed<bf16_t, float>(p, per_lane, grid, s) : launch_norm_fwd_typed<bf16_t, bf16_t>(p, per_lane, grid, s);
+  else if (p.x_dtype == SSM_F16) rf ? launch_norm_fwd_typed<f16_t, float>(p, per_lane, grid, s) : launch_norm_fwd_typed<f16_t, f16_t>(p, per_lane, grid, s);
+  else launch_norm_fwd_typed<float, float>(p, per_lane, grid, s);
+  return true;
+}
+
 // Any hidden size: three sweeps over the row from memory.
 __global__ __launch_bounds__(LN_THREADS) void norm_fwd_long_kernel(const NormParams p) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -429,6 +549,10 @@ extern "C" int ssm_norm_fwd(const ssm_norm_fwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const unsigned grid = (unsigned)((a->rows + LN_WAVES - 1) / LN_WAVES);
   const int per_lane = (a->hidden + WAVE - 1) / WAVE;
+  if (vec_ok && norm_fwd_typed(p, per_lane, grid, s)) {
+    SSM_CHECK_LAUNCH("ssm_norm_fwd");
+    return SSM_OK;
+  }
   if (per_lane <= 4) hipLaunchKernelGGL((norm_fwd_kernel<1, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
   else if (per_lane <= 8) hipLaunchKernelGGL((norm_fwd_kernel<2, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
   else if (per_lane <= 12) hipLaunchKernelGGL((norm_fwd_kernel<3, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);

@@ -40,15 +40,20 @@ __global__ __launch_bounds__(M2_THREADS) void mamba2_conv_kernel(const Mamba2Ste
   const int K = p.width;
   io_t *win = reinterpret_cast<io_t *>(p.conv_state) + e * K;
   const float xin = to_f32(reinterpret_cast<const io_t *>(p.zxbcdt)[(size_t)b * proj + di + c]);
-  float w[M2_MAX_K];
-#pragma unroll
-  for (int k = 0; k < M2_MAX_K; ++k) w[k] = k < K ? to_f32(win[k]) : 0.0f;
-  float acc = p.conv_b ? p.conv_b[c] : 0.0f;
+  // every read is unconditional (indices clamped to the window): all of them are in flight together
+  float w[M2_MAX_K], tap[M2_MAX_K];
 #pragma unroll
   for (int k = 0; k < M2_MAX_K; ++k) {
+    w[k] = to_f32(win[min(k, K - 1)]);
+    tap[k] = p.conv_w[(size_t)c * K + min(k, K - 1)];
+  }
+  float acc = (p.conv_b ? p.conv_b : p.conv_w)[c];
+  if (!p.conv_b) acc = 0.0f;
+#pragma unroll
+  for (int k = 0; k < M2_MAX_K; ++k) {
+    const float v = k + 1 < K ? w[min(k + 1, M2_MAX_K - 1)] : xin;          // the window after the roll
     if (k < K) {
-      const float v = k + 1 < K ? w[k + 1] : xin;          // the window after the roll
-      acc = __builtin_fmaf(p.conv_w[(size_t)c * K + k], v, acc);
+      acc = __builtin_fmaf(tap[k], v, acc);
       win[k] = from_f32<io_t>(v);
     }
   }
@@ -73,15 +78,19 @@ __global__ __launch_bounds__(M2_THREADS) void conv_update_kernel(const ConvUpdat
   const int K = p.width;
   io_t *win = reinterpret_cast<io_t *>(p.conv_state) + e * K;
   const float xin = to_f32(reinterpret_cast<const io_t *>(p.x)[(size_t)b * p.x_stride + c]);
-  float w[M2_MAX_K];
-#pragma unroll
-  for (int k = 0; k < M2_MAX_K; ++k) w[k] = k < K ? to_f32(win[k]) : 0.0f;
-  float acc = p.b ? p.b[c] : 0.0f;
+  float w[M2_MAX_K], tap[M2_MAX_K];
 #pragma unroll
   for (int k = 0; k < M2_MAX_K; ++k) {
+    w[k] = to_f32(win[min(k, K - 1)]);
+    tap[k] = p.w[(size_t)c * K + min(k, K - 1)];
+  }
+  float acc = (p.b ? p.b : p.w)[c];
+  if (!p.b) acc = 0.0f;
+#pragma unroll
+  for (int k = 0; k < M2_MAX_K; ++k) {
+    const float v = k + 1 < K ? w[min(k + 1, M2_MAX_K - 1)] : xin;
     if (k < K) {
-      const float v = k + 1 < K ? w[k + 1] : xin;
-      acc = __builtin_fmaf(p.w[(size_t)c * K + k], v, acc);
+      acc = __builtin_fmaf(tap[k], v, acc);
       win[k] = from_f32<io_t>(v);
     }
   }
@@ -144,11 +153,71 @@ __global__ __launch_bounds__(M2_THREADS) void mamba2_state_kernel(const Mamba2St
   }
 }
 
+// The same update with eight states per lane (N / 8 a power of two up to 64 lanes per channel): every lane
+// issues its reads - two 16-byte pieces each of the state, B and C - at once and unconditionally, the sum over
+// the states is a butterfly inside the wave, and there are B*H*P*N/8 lanes to fill the device (one workgroup
+// per (sequence, head) leaves most of it idle at decoding batch sizes).
+template <typename io_t>
+__global__ __launch_bounds__(M2_THREADS) void mamba2_state8_kernel(const Mamba2StepParams p, const int lg) {
+  const int H = p.heads, P = p.hdim, N = p.nstate, G = p.groups;
+  const int di = H * P, conv_dim = di + 2 * G * N, proj = 2 * di + 2 * G * N + H;
+  const size_t total = ((size_t)p.batch * di) << lg;
+  const size_t gid = (size_t)blockIdx.x * M2_THREADS + threadIdx.x;
+  const bool live = gid < total;
+  const size_t g_ = live ? gid : 0;
+  const int j = (int)(g_ & (size_t)((1 << lg) - 1));
+  const unsigned ch = (unsigned)(g_ >> lg);                  // b * di + h * P + p
+  const int b = (int)(ch / (unsigned)di), hp = (int)(ch % (unsigned)di);
+  const int h = hp / P, grp = h / (H / G);
+  const io_t *row = reinterpret_cast<const io_t *>(p.zxbcdt) + (size_t)b * proj;
+  const float *xb = p.xbc + (size_t)b * conv_dim;
+  float *S = p.state + ((size_t)ch << lg) * 8 + (size_t)j * 8;
+  const float4 s0 = *reinterpret_cast<const float4 *>(S), s1 = *reinterpret_cast<const float4 *>(S + 4);
+  const float *Bq = xb + di + grp * N + j * 8, *Cq = xb + di + G * N + grp * N + j * 8;
+  const float4 b0 = *reinterpret_cast<const float4 *>(Bq), b1 = *reinterpret_cast<const float4 *>(Bq + 4);
+  const float4 c0 = *reinterpret_cast<const float4 *>(Cq), c1 = *reinterpret_cast<const float4 *>(Cq + 4);
+  const float x = xb[hp];
+  const float zraw = to_f32(row[hp]);
+  float dt = to_f32(row[di + conv_dim + h]);
+  const float biasv = (p.bias ? p.bias : p.A)[h];
+  const float Av = p.A[h];
+  const float Dv = p.Dk ? p.Dk[p.d_per_p ? (size_t)hp : (size_t)h] : 0.0f;
+  if (p.bias) dt += biasv;
+  if (p.softplus) dt = softplus_f32(dt);
+  const float a = exp2_hw(dt * Av * LOG2E), dtx = dt * x;
+  float4 n0, n1;
+  n0.x = __builtin_fmaf(a, s0.x, dtx * b0.x); n0.y = __builtin_fmaf(a, s0.y, dtx * b0.y);
+  n0.z = __builtin_fmaf(a, s0.z, dtx * b0.z); n0.w = __builtin_fmaf(a, s0.w, dtx * b0.w);
+  n1.x = __builtin_fmaf(a, s1.x, dtx * b1.x); n1.y = __builtin_fmaf(a, s1.y, dtx * b1.y);
+  n1.z = __builtin_fmaf(a, s1.z, dtx * b1.z); n1.w = __builtin_fmaf(a, s1.w, dtx * b1.w);
+  float y = n0.x * c0.x;
+  y = __builtin_fmaf(n0.y, c0.y, y); y = __builtin_fmaf(n0.z, c0.z, y); y = __builtin_fmaf(n0.w, c0.w, y);
+  y = __builtin_fmaf(n1.x, c1.x, y); y = __builtin_fmaf(n1.y, c1.y, y);
+  y = __builtin_fmaf(n1.z, c1.z, y); y = __builtin_fmaf(n1.w, c1.w, y);
+  for (int m = (1 << lg) >> 1; m >= 1; m >>= 1) y += __shfl_xor(y, m, WAVE);
+  if (!live) return;
+  *reinterpret_cast<float4 *>(S) = n0;
+  *reinterpret_cast<float4 *>(S + 4) = n1;
+  if (j == 0) {
+    y = __builtin_fmaf(Dv, x, y);
+    if (p.gate) y *= silu_f32(zraw);
+    reinterpret_cast<io_t *>(p.y)[ch] = from_f32<io_t>(y);
+  }
+}
+
 template <typename io_t>
 static int launch_mamba2(const Mamba2StepParams &p, hipStream_t s) {
   const int conv_dim = p.heads * p.hdim + 2 * p.groups * p.nstate;
   const size_t total = (size_t)p.batch * conv_dim;
   hipLaunchKernelGGL(mamba2_conv_kernel<io_t>, dim3((unsigned)((total + M2_THREADS - 1) / M2_THREADS)), dim3(M2_THREADS), 0, s, p);
+  int lg = 0;
+  while ((8 << lg) < p.nstate) ++lg;
+  if ((8 << lg) == p.nstate && lg <= 6 && (p.heads * p.hdim) % 4 == 0) {       // float4 reads of B and C out of xbc
+    const size_t lanes = ((size_t)p.batch * p.heads * p.hdim) << lg;
+    hipLaunchKernelGGL(mamba2_state8_kernel<io_t>, dim3((unsigned)((lanes + M2_THREADS - 1) / M2_THREADS)), dim3(M2_THREADS), 0, s, p, lg);
+    SSM_CHECK_LAUNCH("ssm_mamba2_decode_step");
+    return SSM_OK;
+  }
   const int threads = p.hdim * 4 < M2_THREADS ? ((p.hdim * 4 + WAVE - 1) / WAVE) * WAVE : M2_THREADS;
   hipLaunchKernelGGL(mamba2_state_kernel<io_t>, dim3((unsigned)(p.batch * p.heads)), dim3(threads),
                      (size_t)2 * p.nstate * sizeof(float), s, p);
