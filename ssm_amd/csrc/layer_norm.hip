@@ -16,6 +16,8 @@
 // partials are written once and folded by a second kernel in a fixed order.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace ssm {
 
 constexpr int LN_THREADS = 256;
@@ -334,9 +336,15 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_long_kernel(const NormPar
 
 // Each wave handles rows wave_global, wave_global + nwaves, ...; columns are
 // owned by (lane, trip) exactly as in the forward kernel.
-template <int TRIPS, bool WG>
+// XT = void: element types looked up at run time.  Otherwise x, dy, dx have type XT, residual and dresidual
+// type RT, rows are a multiple of four columns long and aligned, and all reads of a row are unconditional
+// (clamped columns, a stand-in for an absent residual), i.e. in flight together.
+template <int TRIPS, bool WG, typename XT = void, typename RT = void>
 __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p, int vec_ok) {
   constexpr int VEC = 4;
+  constexpr bool TYPED = !std::is_void<XT>::value;
+  using xt = typename std::conditional<TYPED, XT, float>::type;
+  using rt = typename std::conditional<TYPED, RT, float>::type;
   constexpr int OWNERS = WG ? LN_THREADS : WAVE;       // threads that share a row
   __shared__ float red[LN_WAVES];
   const int wave = threadIdx.x >> 6, lane = WG ? (int)threadIdx.x : (int)(threadIdx.x & 63);
@@ -349,28 +357,49 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
     const int col = (k * OWNERS + lane) * VEC;
-    load_cols<VEC>(p.w, SSM_F32, 0, col, H, vok, wv[k]);
+    if constexpr (TYPED) ld_pack<float, VEC>(p.w, min(col, H - VEC), wv[k]);
+    else load_cols<VEC>(p.w, SSM_F32, 0, col, H, vok, wv[k]);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) dw[k][i] = db[k][i] = 0.0f;
   }
+  const bool has_add = p.res && p.prenorm;
+  // typed reads of an absent residual go to memory of the same element type and are dropped
+  const void *resp = has_add ? p.res : (p.dres ? (const void *)p.dres : p.x);
+  const float *meanp = p.is_rms ? p.rstd : p.mean;
   for (int row = gw; row < p.rows; row += nwaves) {
     const size_t base = (size_t)row * H;
-    const float mean = p.is_rms ? 0.0f : p.mean[row];
+    float mean = meanp[row];
+    if (p.is_rms) mean = 0.0f;
     const float rstd = p.rstd[row];
     float xh[TRIPS][VEC], g[TRIPS][VEC], dyv[TRIPS][VEC];
     float s1 = 0.0f, s2 = 0.0f;     // sum g*xhat, sum g
+    float vin[TRIPS][VEC], rin[TRIPS][VEC];
+    if constexpr (TYPED) {
+#pragma unroll
+      for (int k = 0; k < TRIPS; ++k) {
+        const int colc = min((k * OWNERS + lane) * VEC, H - VEC);
+        ld_pack<xt, VEC>(p.x, base + colc, vin[k]);
+        ld_pack<rt, VEC>(resp, base + colc, rin[k]);
+        ld_pack<xt, VEC>(p.dy, base + colc, dyv[k]);
+      }
+    }
 #pragma unroll
     for (int k = 0; k < TRIPS; ++k) {
       const int col = (k * OWNERS + lane) * VEC;
       float v[VEC];
-      load_cols<VEC>(p.x, p.x_dtype, base, col, H, vok, v);
-      if (p.res && p.prenorm) {
-        float r[VEC];
-        load_cols<VEC>(p.res, p.res_dtype, base, col, H, vok, r);
+      if constexpr (TYPED) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) v[i] += r[i];
+        for (int i = 0; i < VEC; ++i) v[i] = has_add ? vin[k][i] + rin[k][i] : vin[k][i];
+      } else {
+        load_cols<VEC>(p.x, p.x_dtype, base, col, H, vok, v);
+        if (has_add) {
+          float r[VEC];
+          load_cols<VEC>(p.res, p.res_dtype, base, col, H, vok, r);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) v[i] += r[i];
+        }
+        load_cols<VEC>(p.dy, p.x_dtype, base, col, H, vok, dyv[k]);
       }
-      load_cols<VEC>(p.dy, p.x_dtype, base, col, H, vok, dyv[k]);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         const bool in = col + i < H;
@@ -391,8 +420,13 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
       float dxv[VEC];
 #pragma unroll
       for (int i = 0; i < VEC; ++i) dxv[i] = (g[k][i] - c2 - xh[k][i] * c1) * rstd;
-      store_cols<VEC>(p.dx, p.x_dtype, base, col, H, vok, dxv);
-      if (p.dres) store_cols<VEC>(p.dres, p.res_dtype, base, col, H, vok, p.prenorm ? dxv : dyv[k]);
+      if constexpr (TYPED) {
+        st_pack<xt, VEC>(p.dx, base + col, dxv);
+        if (p.dres) st_pack<rt, VEC>(p.dres, base + col, p.prenorm ? dxv : dyv[k]);
+      } else {
+        store_cols<VEC>(p.dx, p.x_dtype, base, col, H, vok, dxv);
+        if (p.dres) store_cols<VEC>(p.dres, p.res_dtype, base, col, H, vok, p.prenorm ? dxv : dyv[k]);
+      }
     }
   }
   if constexpr (WG) {                                  // every thread owns its columns: the partial is complete
@@ -566,6 +600,21 @@ extern "C" int ssm_norm_fwd(const ssm_norm_fwd_args *a, void *hip_stream) {
   return SSM_OK;
 }
 
+namespace ssm {
+template <typename XT, typename RT>
+static void launch_norm_bwd_typed(const NormParams &p, int hidden, int grid, hipStream_t s) {
+  const int per_lane = (hidden + WAVE - 1) / WAVE;
+  const dim3 g(grid), b(LN_THREADS);
+  if (per_lane <= 4) hipLaunchKernelGGL((norm_bwd_kernel<1, false, XT, RT>), g, b, 0, s, p, 1);
+  else if (per_lane <= 8) hipLaunchKernelGGL((norm_bwd_kernel<2, false, XT, RT>), g, b, 0, s, p, 1);
+  else if (per_lane <= 12) hipLaunchKernelGGL((norm_bwd_kernel<3, false, XT, RT>), g, b, 0, s, p, 1);
+  else if (hidden <= 1024) hipLaunchKernelGGL((norm_bwd_kernel<1, true, XT, RT>), g, b, 0, s, p, 1);
+  else if (hidden <= 2048) hipLaunchKernelGGL((norm_bwd_kernel<2, true, XT, RT>), g, b, 0, s, p, 1);
+  else if (hidden <= 4096) hipLaunchKernelGGL((norm_bwd_kernel<4, true, XT, RT>), g, b, 0, s, p, 1);
+  else hipLaunchKernelGGL((norm_bwd_kernel<8, true, XT, RT>), g, b, 0, s, p, 1);
+}
+}  // namespace ssm
+
 extern "C" size_t ssm_norm_bwd_workspace_bytes(int rows, int hidden) {
   if (rows <= 0 || hidden <= 0) return 0;
   return (size_t)ssm::norm_bwd_grid(rows) * ssm::LN_WAVES * 2 * (size_t)hidden * sizeof(float);
@@ -596,7 +645,15 @@ extern "C" int ssm_norm_bwd(const ssm_norm_bwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const int grid = norm_bwd_grid(a->rows);
   const int per_lane = (a->hidden + WAVE - 1) / WAVE;
-  if (per_lane <= 4) hipLaunchKernelGGL((norm_bwd_kernel<1, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
+  // typed kernels: one element type RT (float32 or that of x) for residual and dresidual
+  const int rt = (a->residual || a->dresidual) ? a->residual_dtype : a->x_dtype;
+  if (vec_ok && a->hidden >= 4 && a->hidden <= 8192 && (rt == SSM_F32 || rt == a->x_dtype)) {
+    const bool rf = rt == SSM_F32;
+    if (a->x_dtype == SSM_BF16) rf ? launch_norm_bwd_typed<bf16_t, float>(p, a->hidden, grid, s) : launch_norm_bwd_typed<bf16_t, bf16_t>(p, a->hidden, grid, s);
+    else if (a->x_dtype == SSM_F16) rf ? launch_norm_bwd_typed<f16_t, float>(p, a->hidden, grid, s) : launch_norm_bwd_typed<f16_t, f16_t>(p, a->hidden, grid, s);
+    else launch_norm_bwd_typed<float, float>(p, a->hidden, grid, s);
+  }
+  else if (per_lane <= 4) hipLaunchKernelGGL((norm_bwd_kernel<1, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
   else if (per_lane <= 8) hipLaunchKernelGGL((norm_bwd_kernel<2, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
   else if (per_lane <= 12) hipLaunchKernelGGL((norm_bwd_kernel<3, false>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
   else if (a->hidden <= 1024) hipLaunchKernelGGL((norm_bwd_kernel<1, true>), dim3(grid), dim3(LN_THREADS), 0, s, p, vec_ok);
