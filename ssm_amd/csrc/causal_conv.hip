@@ -42,6 +42,26 @@ __device__ __forceinline__ float silu_grad(float pre) {
   return s * __builtin_fmaf(pre, 1.0f - s, 1.0f);
 }
 
+// A whole vector at element t of a row of `len` elements (a multiple of VEC, 16-byte aligned), zeros when
+// the vector lies before or past the row: the read itself is unconditional (the index is clamped into the
+// row), so several of them are in flight together instead of each waiting behind its own bounds check.
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec_or_zero(const T *row, int t, int len, float (&out)[VEC]) {
+  const int tc = min(max(t, 0), len - VEC);
+  const Pack<T, VEC> raw = *reinterpret_cast<const Pack<T, VEC> *>(row + tc);
+  const bool in = t >= 0 && t < len;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) out[i] = in ? to_f32(raw.v[i]) : 0.0f;
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_vec(T *row, int t, const float (&v)[VEC]) {
+  Pack<T, VEC> raw;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) raw.v[i] = from_f32<T>(v[i]);
+  *reinterpret_cast<Pack<T, VEC> *>(row + t) = raw;
+}
+
 // ---------------------------------------------------------------- forward, (B,C,L)
 
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
@@ -58,16 +78,25 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvPar
   const float bias = p.bias ? p.bias[c] : 0.0f;
   for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
     float win[2 * VEC];
-    if (t0 > 0) {
-      float prev[VEC];
-      load_run<T, VEC>(xr, t0 - VEC, p.len, AL, prev);
+    if constexpr (AL) {
+      float prev[VEC], cur[VEC];
+      load_vec_or_zero<T, VEC>(xr, t0 - VEC, p.len, prev);
+      load_vec_or_zero<T, VEC>(xr, t0, p.len, cur);
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) win[i] = prev[i];
+      for (int i = 0; i < VEC; ++i) {
+        win[i] = prev[i];
+        win[VEC + i] = cur[i];
+      }
     } else {
+      if (t0 > 0) {
+        float prev[VEC];
+        load_run<T, VEC>(xr, t0 - VEC, p.len, AL, prev);
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) win[i] = 0.0f;
-    }
-    {
+        for (int i = 0; i < VEC; ++i) win[i] = prev[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) win[i] = 0.0f;
+      }
       float cur[VEC];
       load_run<T, VEC>(xr, t0, p.len, AL, cur);
 #pragma unroll
@@ -81,7 +110,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvPar
       for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[m], win[VEC + i - m], acc);
       out[i] = p.silu ? silu_f32(acc) : acc;
     }
-    store_run<T, VEC>(yr, t0, p.len, AL, out);
+    if constexpr (AL) store_vec<T, VEC>(yr, t0, out);
+    else store_run<T, VEC>(yr, t0, p.len, AL, out);
   }
 }
 
@@ -193,7 +223,19 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
   for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
     // x over [t0-VEC, t0+2*VEC), dout over [t0, t0+2*VEC)
     float xw[3 * VEC], g[2 * VEC];
-    {
+    if constexpr (AL) {
+      float v0[VEC], v1[VEC], v2[VEC], g0[VEC], g1[VEC];
+      load_vec_or_zero<T, VEC>(xr, t0 - VEC, p.len, v0);
+      load_vec_or_zero<T, VEC>(xr, t0, p.len, v1);
+      load_vec_or_zero<T, VEC>(xr, t0 + VEC, p.len, v2);
+      load_vec_or_zero<T, VEC>(gr, t0, p.len, g0);
+      load_vec_or_zero<T, VEC>(gr, t0 + VEC, p.len, g1);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        xw[i] = v0[i]; xw[VEC + i] = v1[i]; xw[2 * VEC + i] = v2[i];
+        g[i] = g0[i]; g[VEC + i] = g1[i];
+      }
+    } else {
       float v[VEC];
       if (t0 > 0) load_run<T, VEC>(xr, t0 - VEC, p.len, AL, v);
       else {
@@ -238,7 +280,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
 #pragma unroll
       for (int m = 0; m < CONV_TAPS; ++m) dwrev[m] = __builtin_fmaf(g[i], xw[VEC + i - m], dwrev[m]);
     }
-    store_run<T, VEC>(dxr, t0, p.len, AL, dx);
+    if constexpr (AL) store_vec<T, VEC>(dxr, t0, dx);
+    else store_run<T, VEC>(dxr, t0, p.len, AL, dx);
   }
   // block reduction of dw[0..K) and db
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
