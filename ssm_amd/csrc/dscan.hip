@@ -119,7 +119,11 @@ __global__ __launch_bounds__(DS_THREADS) void dscan_kernel(const DscanParams p) 
       xv[j] = ds_load<io_t>(p.X, p.x_dtype, xi);
       bv[j] = ds_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
       cv[j] = ds_load<io_t>(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
-      zv[j] = p.z ? ds_load<io_t>(p.z, p.z_dtype, p.z_per_p ? xi : (x_row + t) * p.heads + h) : 0.0f;
+      {
+        // an absent gate reads X in its place (value dropped): no branch around the read
+        const float zraw = ds_load<io_t>(p.z ? p.z : p.X, p.z ? p.z_dtype : p.x_dtype, (p.z && !p.z_per_p) ? (x_row + t) * p.heads + h : xi);
+        zv[j] = p.z ? zraw : 0.0f;
+      }
     }
 #pragma unroll
     for (int j = 0; j < DS_UNROLL; ++j) {

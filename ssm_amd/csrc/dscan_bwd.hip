@@ -96,7 +96,11 @@ __global__ __launch_bounds__(DB_THREADS) void dscan_bwd_fold_kernel(const DscanB
       bv[j] = db_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
       cv[j] = db_load<io_t>(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
       gv[j] = db_load<io_t>(p.gy, p.x_dtype, xi);
-      zv[j] = p.z ? db_load<io_t>(p.z, p.z_dtype, p.z_per_p ? xi : (row0 + t) * p.heads + h) : 0.0f;
+      {
+        // an absent gate reads X in its place (value dropped): no branch around the read
+        const float zraw = db_load<io_t>(p.z ? p.z : p.X, p.z ? p.z_dtype : p.x_dtype, (p.z && !p.z_per_p) ? (row0 + t) * p.heads + h : xi);
+        zv[j] = p.z ? zraw : 0.0f;
+      }
     }
 #pragma unroll
     for (int j = 0; j < DB_UNROLL; ++j) {
@@ -191,12 +195,17 @@ __global__ __launch_bounds__(DB_THREADS) void dscan_bwd_kernel(const DscanBwdPar
       bv[j] = db_load<io_t>(p.Bp, p.bc_dtype, (size_t)(b * p.b_stride_b + t * p.b_stride_t) + hp);
       cv[j] = db_load<io_t>(p.Cp, p.bc_dtype, (size_t)(b * p.c_stride_b + t * p.c_stride_t) + hp);
       gv[j] = db_load<io_t>(p.gy, p.x_dtype, xi);
-      zv[j] = p.z ? db_load<io_t>(p.z, p.z_dtype, p.z_per_p ? xi : (row0 + t) * p.heads + h) : 0.0f;
+      {
+        // an absent gate reads X in its place (value dropped): no branch around the read
+        const float zraw = db_load<io_t>(p.z ? p.z : p.X, p.z ? p.z_dtype : p.x_dtype, (p.z && !p.z_per_p) ? (row0 + t) * p.heads + h : xi);
+        zv[j] = p.z ? zraw : 0.0f;
+      }
       st[j] = p.states[xi];
     }
     {
       const int t = t1 - DB_UNROLL;
-      st[DB_UNROLL] = t >= t_begin ? p.states[(row0 + t) * HP + hp] : s_in;
+      const float before = p.states[(row0 + max(t, t_begin)) * HP + hp];
+      st[DB_UNROLL] = t >= t_begin ? before : s_in;
     }
 #pragma unroll
     for (int j = 0; j < DB_UNROLL; ++j) {
