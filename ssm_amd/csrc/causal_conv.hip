@@ -165,6 +165,37 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
   T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
   const int t_begin = strip * CONV_CL_STRIP;
   const int t_end = min(p.len, t_begin + CONV_CL_STRIP);
+  if constexpr (AL) {
+    // all rows of the strip and the K-1 before it are requested at once, unconditionally (row index clamped
+    // into the sequence, rows before its start become zeros): one wait instead of one per step
+    Pack<T, VEC> raw[HIST + CONV_CL_STRIP];
+#pragma unroll
+    for (int j = 0; j < HIST + CONV_CL_STRIP; ++j) {
+      const int ts = t_begin - HIST + j;
+      raw[j] = *reinterpret_cast<const Pack<T, VEC> *>(xb + (size_t)min(max(ts, 0), p.len - 1) * p.chans);
+    }
+#pragma unroll
+    for (int j = 0; j < HIST; ++j) {
+      if (t_begin - HIST + j < 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) raw[j].v[i] = from_f32<T>(0.0f);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < CONV_CL_STRIP; ++s) {
+      if (t_begin + s >= t_end) break;
+      float out[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float acc = bias[i];
+#pragma unroll
+        for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + s - m].v[i]), acc);
+        out[i] = p.silu ? silu_f32(acc) : acc;
+      }
+      store_vec<T, VEC>(yb + (size_t)(t_begin + s) * p.chans, 0, out);
+    }
+    return;
+  }
   // hist[j] holds x at time (t - 1 - j); filled with the K-1 rows before the strip
   float hist[HIST][VEC];
 #pragma unroll
