@@ -399,12 +399,12 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
     for (int i = 0; i < VEC; ++i) gh[m][i] = 0.0f;
 
   const int t_last = t_end + HIST;                    // exclusive: dx of the last own step needs g three steps on
-  for (int t = t_begin; t < t_last; ++t) {
+  // one step, given x_t and dout_t (ignored past the end of the sequence)
+  auto step = [&](const int t, const float (&cur_in)[VEC], const float (&go)[VEC]) {
     float cur[VEC], g[VEC];
     if (t < p.len) {
-      float go[VEC];
-      load_run<T, VEC>(xb + (size_t)t * p.chans, 0, cw, AL, cur);
-      load_run<T, VEC>(gb + (size_t)t * p.chans, 0, cw, AL, go);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) cur[i] = cur_in[i];
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         g[i] = go[i];
@@ -453,6 +453,42 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
         out[i] = acc;
       }
       store_run<T, VEC>(dxb + (size_t)td * p.chans, 0, cw, AL, out);
+    }
+  };
+  if constexpr (AL) {
+    // rows of a group of steps are requested together, unconditionally (row index clamped into the sequence)
+    constexpr int GROUP = 8;
+    for (int tg = t_begin; tg < t_last; tg += GROUP) {
+      Pack<T, VEC> rx[GROUP], rg[GROUP];
+#pragma unroll
+      for (int j = 0; j < GROUP; ++j) {
+        const size_t at = (size_t)min(tg + j, p.len - 1) * p.chans;
+        rx[j] = *reinterpret_cast<const Pack<T, VEC> *>(xb + at);
+        rg[j] = *reinterpret_cast<const Pack<T, VEC> *>(gb + at);
+      }
+#pragma unroll
+      for (int j = 0; j < GROUP; ++j) {
+        if (tg + j >= t_last) break;
+        float cur[VEC], go[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          cur[i] = to_f32(rx[j].v[i]);
+          go[i] = to_f32(rg[j].v[i]);
+        }
+        step(tg + j, cur, go);
+      }
+    }
+  } else {
+    for (int t = t_begin; t < t_last; ++t) {
+      float cur[VEC], go[VEC];
+      if (t < p.len) {
+        load_run<T, VEC>(xb + (size_t)t * p.chans, 0, cw, AL, cur);
+        load_run<T, VEC>(gb + (size_t)t * p.chans, 0, cw, AL, go);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) cur[i] = go[i] = 0.0f;
+      }
+      step(t, cur, go);
     }
   }
   // partial[(b * nseg + seg)][c][K + 1]: taps in the order of w, then the bias sum
@@ -512,16 +548,32 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_generic_kernel(const Co
   }
 }
 
-// dw[c,k] = sum_b partial[b][c][k], dbias[c] = sum_b partial[b][c][K]; fixed order.
+// dw[c,k] = sum_b partial[b][c][k], dbias[c] = sum_b partial[b][c][K]; fixed order: a workgroup takes 16
+// neighbouring outputs, its 256 threads are those outputs x 16 slices of the partials (slice s adds partials
+// s, s + 16, ...), and the slices are added up in order.
+constexpr int CONV_FOLD_COLS = 16, CONV_FOLD_SLICES = CONV_THREADS / CONV_FOLD_COLS;
+
 __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_fold_kernel(const float *partial, float *dw, float *dbias,
                                                                       int batch, int chans, int K) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= chans * (K + 1)) return;
-  const int c = e / (K + 1), k = e % (K + 1);
+  __shared__ float part[CONV_FOLD_SLICES][CONV_FOLD_COLS];
+  const int n = chans * (K + 1);
+  const int col = threadIdx.x % CONV_FOLD_COLS, sl = threadIdx.x / CONV_FOLD_COLS;
+  const int e = blockIdx.x * CONV_FOLD_COLS + col;
   float s = 0.0f;
-  for (int b = 0; b < batch; ++b) s += partial[((size_t)b * chans + c) * (K + 1) + k];
-  if (k < K) dw[(size_t)c * K + k] = s;
-  else if (dbias) dbias[c] = s;
+  if (e < n) {
+#pragma unroll 4
+    for (int b = sl; b < batch; b += CONV_FOLD_SLICES) s += partial[(size_t)b * n + e];
+  }
+  part[sl][col] = s;
+  __syncthreads();
+  if (sl == 0 && e < n) {
+    float t = 0.0f;
+#pragma unroll
+    for (int k = 0; k < CONV_FOLD_SLICES; ++k) t += part[k][col];
+    const int c = e / (K + 1), k = e % (K + 1);
+    if (k < K) dw[(size_t)c * K + k] = t;
+    else if (dbias) dbias[c] = t;
+  }
 }
 
 template <typename T>
@@ -568,7 +620,7 @@ static int conv_bwd_typed(const ConvParams &p, int channels_last, bool vec_ok, f
   }
   SSM_CHECK_LAUNCH("ssm_conv1d_bwd");
   const int n = p.chans * (p.K + 1);
-  hipLaunchKernelGGL(conv_bwd_fold_kernel, dim3((n + CONV_THREADS - 1) / CONV_THREADS), dim3(CONV_THREADS), 0, s,
+  hipLaunchKernelGGL(conv_bwd_fold_kernel, dim3((n + CONV_FOLD_COLS - 1) / CONV_FOLD_COLS), dim3(CONV_THREADS), 0, s,
                      p.partial, dw, dbias, fold_count, p.chans, p.K);
   SSM_CHECK_LAUNCH("ssm_conv1d_bwd(fold)");
   return SSM_OK;
