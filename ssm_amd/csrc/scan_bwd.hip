@@ -588,15 +588,49 @@ __global__ __launch_bounds__(BW_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
 #undef BT
 }
 
-// out[o][i] = sum_{j < count} in[(o * count + j) * inner + i], fixed order.
+// out[o][i] = sum_{j < count} in[(o * count + j) * inner + i], fixed order.  The terms of an output are read
+// eight at a time (independent reads in flight together) and added in order.
 __global__ __launch_bounds__(256) void fold_sum_kernel(const float *in, float *out, size_t outer, int count,
                                                        size_t inner) {
   const size_t total = outer * inner;
   for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
     const size_t o = e / inner, i = e % inner;
+    const float *src = in + o * count * inner + i;
     float s = 0.0f;
-    for (int j = 0; j < count; ++j) s += in[(o * count + j) * inner + i];
+    int j = 0;
+    for (; j + 8 <= count; j += 8) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = src[(size_t)(j + k) * inner];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) s += v[k];
+    }
+    for (; j < count; ++j) s += src[(size_t)j * inner];
     out[e] = s;
+  }
+}
+
+// The same for four neighbouring outputs per thread (inner a multiple of four, 16-byte aligned tensors).
+__global__ __launch_bounds__(256) void fold_sum_vec4_kernel(const float *in, float *out, size_t outer, int count,
+                                                            size_t inner) {
+  const size_t inner4 = inner / 4, total = outer * inner4;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t o = e / inner4, i = (e % inner4) * 4;
+    const float *src = in + o * count * inner + i;
+    float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    int j = 0;
+    for (; j + 4 <= count; j += 4) {
+      float4 v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = *reinterpret_cast<const float4 *>(src + (size_t)(j + k) * inner);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
+    }
+    for (; j < count; ++j) {
+      const float4 v = *reinterpret_cast<const float4 *>(src + (size_t)j * inner);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    *reinterpret_cast<float4 *>(out + o * inner + i) = s;
   }
 }
 
@@ -646,6 +680,10 @@ void launch_fold_sum(const float *in, float *out, size_t outer, int count, size_
     const int bpo = (int)((inner + cols - 1) / cols);
     hipLaunchKernelGGL(fold_sum_wide_kernel, dim3((unsigned)(outer * bpo)), dim3(256), 0, s, in, out, count, inner, cols,
                        bpo);
+    return;
+  }
+  if (inner % 4 == 0 && aligned_to(in, 16) && aligned_to(out, 16)) {
+    hipLaunchKernelGGL(fold_sum_vec4_kernel, dim3(fold_grid(outer * inner / 4)), dim3(256), 0, s, in, out, outer, count, inner);
     return;
   }
   hipLaunchKernelGGL(fold_sum_kernel, dim3(fold_grid(outer * inner)), dim3(256), 0, s, in, out, outer, count, inner);
@@ -812,8 +850,7 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
     if (kind == SSM_PROJ_BGNL) {
       // (B, G, nblk/G, N*L) -> (B, G, N*L)
       const int per_group = pl.nblk / groups;
-      hipLaunchKernelGGL(fold_sum_kernel, dim3(fold_grid((size_t)Bn * groups * N * L)), dim3(256), 0, s, partial,
-                         out, (size_t)Bn * groups, per_group, (size_t)N * L);
+      launch_fold_sum(partial, out, (size_t)Bn * groups, per_group, (size_t)N * L, s);
     } else if (kind == SSM_PROJ_BDN) {
       hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)Bn * D * N)), dim3(256), 0, s, partial, out, 1,
                          (size_t)Bn * D * N);
