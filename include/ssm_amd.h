@@ -455,6 +455,58 @@ int ssm_ssd_combined_supported(const ssm_ssd_dims *dims, int io_dtype);   /* 1 /
 size_t ssm_ssd_combined_workspace_bytes(const ssm_ssd_dims *dims);
 int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *args, void *hip_stream);
 
+/* Element-wise stages of the gradient of the combined forward.  The reference holds no code for them: its
+ * fixture `ssd_combined.combined_full.gradients` (tests/mamba_reference_cases.json, written by
+ * scripts/refresh_mamba_goldens.py:677-705) fixes the nine gradients, which the Python side of this package
+ * forms from passes of the forward kernels with operands in other roles; these three launches replace the
+ * tensor operations between those passes.  Rows are (batch, step, head) vectors of `headdim` channels;
+ * `headdim` must be 4 * 2^k (at most 256).
+ *   gate: dy = dout silu(z) (dout without z), written in `dy_dtype` in time order and, when `dy_rev` is
+ *         given, reversed in time;  dz = dout (ypre + D x) silu'(z);  s2 = <dy as stored, ypre>;  dyx = <dy, x>
+ *   dx:   dx = dt u + D dy,  xu = <x, u>,  s1 = <dt x (rounded to bfloat16 if round_bf16), u>, with u given
+ *         reversed in time
+ *   db:   dB[b][l][g][n] = sum_{h in group g} dt[b][l][h] v_rev[b][L-1-l][h][n] */
+typedef struct ssm_ssd_bwd_gate_args {
+  const void *dout;          /* (B, L, H, P) io dtype */
+  const void *z;             /* (B, L, H, P) io dtype or NULL */
+  const void *x;             /* (B, L, H, P) io dtype */
+  const float *ypre;         /* (B, L, H, P) fp32: output before skip and gate */
+  const float *Dskip;        /* (H,) or (H, P) if d_per_p, or NULL */
+  void *dy;                  /* (B, L, H, P) dy_dtype */
+  void *dy_rev;              /* (B, L, H, P) dy_dtype, time reversed, or NULL */
+  float *dz;                 /* (B, L, H, P) fp32; NULL exactly when z is */
+  float *s2;                 /* (B, L, H) fp32 */
+  float *dyx;                /* (B, L, H) fp32 */
+  int32_t batch, seqlen, heads, headdim;
+  int32_t io_dtype;          /* ssm_dtype of dout, z, x */
+  int32_t dy_dtype;          /* SSM_F32 or SSM_BF16 */
+  int32_t d_per_p;
+} ssm_ssd_bwd_gate_args;
+int ssm_ssd_bwd_gate(const ssm_ssd_bwd_gate_args *args, void *hip_stream);
+
+typedef struct ssm_ssd_bwd_dx_args {
+  const void *dout;          /* (B, L, H, P) io dtype */
+  const void *z;             /* (B, L, H, P) io dtype or NULL */
+  const void *x;             /* (B, L, H, P) io dtype */
+  const float *u_rev;        /* (B, L, H, P) fp32, time reversed */
+  const float *dt;           /* (B, L, H) fp32: the step after bias, softplus and clamp */
+  const float *Dskip;        /* (H,) or (H, P) if d_per_p, or NULL */
+  float *dx;                 /* (B, L, H, P) fp32 */
+  float *xu;                 /* (B, L, H) fp32 */
+  float *s1;                 /* (B, L, H) fp32 */
+  int32_t batch, seqlen, heads, headdim;
+  int32_t io_dtype, d_per_p, round_bf16;
+} ssm_ssd_bwd_dx_args;
+int ssm_ssd_bwd_dx(const ssm_ssd_bwd_dx_args *args, void *hip_stream);
+
+typedef struct ssm_ssd_bwd_db_args {
+  const float *v_rev;        /* (B, L, H, N) fp32, time reversed */
+  const float *dt;           /* (B, L, H) fp32 */
+  float *dB;                 /* (B, L, G, N) fp32 */
+  int32_t batch, seqlen, heads, groups, nstate;
+} ssm_ssd_bwd_db_args;
+int ssm_ssd_bwd_db(const ssm_ssd_bwd_db_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).
  * Forward stands behind `dw_causal_conv(x, weight, bias, activation)`

@@ -177,6 +177,23 @@ class SsdCombinedArgs(C.Structure):
                 ("dt_softplus", _i32), ("d_per_p", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float)]
 
 
+class SsdBwdGateArgs(C.Structure):
+    _fields_ = [("dout", _vp), ("z", _vp), ("x", _vp), ("ypre", _vp), ("Dskip", _vp), ("dy", _vp), ("dy_rev", _vp),
+                ("dz", _vp), ("s2", _vp), ("dyx", _vp), ("batch", _i32), ("seqlen", _i32), ("heads", _i32),
+                ("headdim", _i32), ("io_dtype", _i32), ("dy_dtype", _i32), ("d_per_p", _i32)]
+
+
+class SsdBwdDxArgs(C.Structure):
+    _fields_ = [("dout", _vp), ("z", _vp), ("x", _vp), ("u_rev", _vp), ("dt", _vp), ("Dskip", _vp), ("dx", _vp),
+                ("xu", _vp), ("s1", _vp), ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("headdim", _i32),
+                ("io_dtype", _i32), ("d_per_p", _i32), ("round_bf16", _i32)]
+
+
+class SsdBwdDbArgs(C.Structure):
+    _fields_ = [("v_rev", _vp), ("dt", _vp), ("dB", _vp), ("batch", _i32), ("seqlen", _i32), ("heads", _i32),
+                ("groups", _i32), ("nstate", _i32)]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -235,6 +252,9 @@ ENTRY_POINTS = {
     "ssm_ssd_chunk_scan": SsdChunkScanArgs,
     "ssm_ssd_chunk_state_varlen": SsdChunkStateVarlenArgs,
     "ssm_ssd_combined_fwd": SsdCombinedArgs,
+    "ssm_ssd_bwd_gate": SsdBwdGateArgs,
+    "ssm_ssd_bwd_dx": SsdBwdDxArgs,
+    "ssm_ssd_bwd_db": SsdBwdDbArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_conv1d_update": Conv1dUpdateArgs,

@@ -1,0 +1,285 @@
+// Element-wise stages between the passes of the state-space-duality backward, one read of every tensor each:
+//
+//   gate   dy = dout silu(z);  dz = dout (ypre + D x) silu'(z);  s2 = <round(dy), ypre>;  dyx = <dy, x>
+//          (dy is written in the passes' operand type, in time order and reversed)
+//   dx     dx = dt u + D dy;  xu = <x, u>;  s1 = <round(dt x), u>      (u arrives reversed in time)
+//   db     dB[l][g][n] = sum_{h in g} dt[l][h] v[L-1-l][h][n]          (v arrives reversed in time)
+//
+// Rows are the (batch, step, head) vectors of P channels; a row is shared by P/4 lanes (a power of two up to
+// 64) that take four neighbouring channels each, row sums are butterflies inside the wave.  All reads are
+// unconditional (an absent gate reads dout in its place).
+#include "common.hpp"
+
+#include <type_traits>
+
+namespace ssm {
+namespace {
+
+constexpr int EB_THREADS = 256;
+
+struct ElemParams {
+  const void *dout, *z, *x;
+  const float *ypre, *u_rev, *dt, *Dk;
+  void *dy, *dy_rev;
+  float *dz, *dx, *s1, *s2, *dyx, *xu;
+  int batch, len, heads, hdim;
+  int d_per_p, round_bf16;
+  int lg;                       // lanes per row = 1 << lg
+};
+
+template <typename T>
+__device__ __forceinline__ void ld4(const void *p, size_t i, float (&v)[4]) {
+  const Pack<T, 4> raw = *reinterpret_cast<const Pack<T, 4> *>(reinterpret_cast<const T *>(p) + i);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = to_f32(raw.v[j]);
+}
+template <typename T>
+__device__ __forceinline__ void st4(void *p, size_t i, const float (&v)[4]) {
+  Pack<T, 4> raw;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) raw.v[j] = from_f32<T>(v[j]);
+  *reinterpret_cast<Pack<T, 4> *>(reinterpret_cast<T *>(p) + i) = raw;
+}
+
+__device__ __forceinline__ float row_sum(float v, int lg) {
+  for (int m = (1 << lg) >> 1; m >= 1; m >>= 1) v += __shfl_xor(v, m, WAVE);
+  return v;
+}
+
+struct RowAt {
+  bool live;
+  size_t row, rev;     // (b, l, h) and (b, L-1-l, h)
+  int h, c0;           // head, first of the lane's four channels
+};
+
+__device__ __forceinline__ RowAt locate(const ElemParams &p) {
+  const size_t rows = (size_t)p.batch * p.len * p.heads;
+  const size_t gid = (size_t)blockIdx.x * EB_THREADS + threadIdx.x;
+  RowAt a;
+  a.live = gid < (rows << p.lg);
+  const size_t g = a.live ? gid : 0;
+  a.row = g >> p.lg;
+  a.c0 = (int)(g & (size_t)((1 << p.lg) - 1)) * 4;
+  a.h = (int)(a.row % (size_t)p.heads);
+  const size_t bl = a.row / (size_t)p.heads;
+  const size_t b = bl / (size_t)p.len, l = bl % (size_t)p.len;
+  a.rev = (b * p.len + (p.len - 1 - l)) * p.heads + a.h;
+  return a;
+}
+
+// IO: type of dout, z, x.  OT: type of dy (the passes' operand type).
+template <typename IO, typename OT>
+__global__ __launch_bounds__(EB_THREADS) void ssd_bwd_gate_kernel(const ElemParams p) {
+  const RowAt a = locate(p);
+  const size_t at = a.row * p.hdim + a.c0;
+  float go[4], zv[4], xv[4], yp[4], Dv[4];
+  ld4<IO>(p.dout, at, go);
+  ld4<IO>(p.z ? p.z : p.dout, at, zv);
+  ld4<IO>(p.x, at, xv);
+  ld4<float>(p.ypre, at, yp);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) Dv[j] = p.Dk ? p.Dk[p.d_per_p ? a.h * p.hdim + a.c0 + j : a.h] : 0.0f;
+  float dy[4], dz[4], s2 = 0.0f, dyx = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (p.z) {
+      const float sg = sigmoid_f32(zv[j]);
+      dy[j] = go[j] * zv[j] * sg;
+      dz[j] = go[j] * __builtin_fmaf(Dv[j], xv[j], yp[j]) * (sg * __builtin_fmaf(zv[j], 1.0f - sg, 1.0f));
+    } else {
+      dy[j] = go[j];
+      dz[j] = 0.0f;
+    }
+    dyx = __builtin_fmaf(dy[j], xv[j], dyx);
+    s2 = __builtin_fmaf(to_f32(from_f32<OT>(dy[j])), yp[j], s2);
+  }
+  s2 = row_sum(s2, p.lg);
+  dyx = row_sum(dyx, p.lg);
+  if (!a.live) return;
+  st4<OT>(p.dy, at, dy);
+  if (p.dy_rev) st4<OT>(p.dy_rev, a.rev * p.hdim + a.c0, dy);
+  if (p.dz) st4<float>(p.dz, at, dz);
+  if (a.c0 == 0) {
+    p.s2[a.row] = s2;
+    p.dyx[a.row] = dyx;
+  }
+}
+
+template <typename IO>
+__global__ __launch_bounds__(EB_THREADS) void ssd_bwd_dx_kernel(const ElemParams p) {
+  const RowAt a = locate(p);
+  const size_t at = a.row * p.hdim + a.c0;
+  float go[4], zv[4], xv[4], uv[4], Dv[4];
+  ld4<IO>(p.dout, at, go);
+  ld4<IO>(p.z ? p.z : p.dout, at, zv);
+  ld4<IO>(p.x, at, xv);
+  ld4<float>(p.u_rev, a.rev * p.hdim + a.c0, uv);
+  const float dt = p.dt[a.row];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) Dv[j] = p.Dk ? p.Dk[p.d_per_p ? a.h * p.hdim + a.c0 + j : a.h] : 0.0f;
+  float dx[4], xu = 0.0f, s1 = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float dy = p.z ? go[j] * zv[j] * sigmoid_f32(zv[j]) : go[j];
+    dx[j] = __builtin_fmaf(dt, uv[j], Dv[j] * dy);
+    xu = __builtin_fmaf(xv[j], uv[j], xu);
+    const float xt = dt * xv[j];
+    s1 = __builtin_fmaf(p.round_bf16 ? to_f32(from_f32<bf16_t>(xt)) : xt, uv[j], s1);
+  }
+  xu = row_sum(xu, p.lg);
+  s1 = row_sum(s1, p.lg);
+  if (!a.live) return;
+  st4<float>(p.dx, at, dx);
+  if (a.c0 == 0) {
+    p.xu[a.row] = xu;
+    p.s1[a.row] = s1;
+  }
+}
+
+struct DbParams {
+  const float *v_rev, *dt;
+  float *dB;
+  int batch, len, heads, groups, nstate;
+};
+
+// One thread per four neighbouring states of a (batch, step, group); the heads of the group are added in order.
+__global__ __launch_bounds__(EB_THREADS) void ssd_bwd_db_kernel(const DbParams p) {
+  const int n4 = p.nstate / 4, per = p.heads / p.groups;
+  const size_t total = (size_t)p.batch * p.len * p.groups * n4;
+  const size_t gid = (size_t)blockIdx.x * EB_THREADS + threadIdx.x;
+  if (gid >= total) return;
+  const int n0 = (int)(gid % n4) * 4;
+  const int g = (int)((gid / n4) % p.groups);
+  const size_t bl = gid / ((size_t)n4 * p.groups);
+  const size_t b = bl / (size_t)p.len, l = bl % (size_t)p.len;
+  const size_t rev = b * p.len + (p.len - 1 - l);
+  float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  int h = 0;
+  for (; h + 4 <= per; h += 4) {
+    float4 v[4];
+    float w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int hh = g * per + h + k;
+      v[k] = *reinterpret_cast<const float4 *>(p.v_rev + (rev * p.heads + hh) * p.nstate + n0);
+      w[k] = p.dt[bl * p.heads + hh];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      s.x = __builtin_fmaf(w[k], v[k].x, s.x); s.y = __builtin_fmaf(w[k], v[k].y, s.y);
+      s.z = __builtin_fmaf(w[k], v[k].z, s.z); s.w = __builtin_fmaf(w[k], v[k].w, s.w);
+    }
+  }
+  for (; h < per; ++h) {
+    const int hh = g * per + h;
+    const float4 v = *reinterpret_cast<const float4 *>(p.v_rev + (rev * p.heads + hh) * p.nstate + n0);
+    const float w = p.dt[bl * p.heads + hh];
+    s.x = __builtin_fmaf(w, v.x, s.x); s.y = __builtin_fmaf(w, v.y, s.y);
+    s.z = __builtin_fmaf(w, v.z, s.z); s.w = __builtin_fmaf(w, v.w, s.w);
+  }
+  *reinterpret_cast<float4 *>(p.dB + (bl * p.groups + g) * p.nstate + n0) = s;
+}
+
+bool row_lanes(int hdim, int &lg) {
+  if (hdim % 4 != 0) return false;
+  lg = 0;
+  while ((4 << lg) < hdim) ++lg;
+  return (4 << lg) == hdim && lg <= 6;
+}
+
+unsigned elem_grid(const ElemParams &p) {
+  const size_t lanes = ((size_t)p.batch * p.len * p.heads) << p.lg;
+  return (unsigned)((lanes + EB_THREADS - 1) / EB_THREADS);
+}
+
+}  // namespace
+}  // namespace ssm
+
+extern "C" int ssm_ssd_bwd_gate(const ssm_ssd_bwd_gate_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_gate: args is NULL");
+  SSM_REQUIRE(a->dout && a->x && a->ypre && a->dy && a->s2 && a->dyx, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_bwd_gate: dout, x, ypre, dy, s2 and dyx are required");
+  SSM_REQUIRE((a->z != nullptr) == (a->dz != nullptr), SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_gate: dz must be given exactly when z is");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->headdim > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bwd_gate: batch, seqlen, heads and headdim must be positive");
+  ElemParams p{};
+  SSM_REQUIRE(row_lanes(a->headdim, p.lg), SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bwd_gate: headdim=%d must be 4 * 2^k, at most 256", a->headdim);
+  SSM_REQUIRE(valid_dtype(a->io_dtype) && (a->dy_dtype == SSM_F32 || a->dy_dtype == SSM_BF16), SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_bwd_gate: io_dtype=%d dy_dtype=%d (dy is float32 or bfloat16)", a->io_dtype, a->dy_dtype);
+  SSM_REQUIRE((size_t)a->batch * a->seqlen * a->heads < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_gate: too many rows");
+  SSM_REQUIRE(aligned_to(a->dout, 8) && aligned_to(a->x, 8) && (!a->z || aligned_to(a->z, 8)) && aligned_to(a->ypre, 16) &&
+                  aligned_to(a->dy, 8) && (!a->dy_rev || aligned_to(a->dy_rev, 8)) && (!a->dz || aligned_to(a->dz, 16)),
+              SSM_ERR_ALIGNMENT, "ssm_ssd_bwd_gate: a pointer is not sufficiently aligned");
+  p.dout = a->dout; p.z = a->z; p.x = a->x; p.ypre = a->ypre; p.Dk = a->Dskip; p.dy = a->dy; p.dy_rev = a->dy_rev;
+  p.dz = a->dz; p.s2 = a->s2; p.dyx = a->dyx;
+  p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.hdim = a->headdim; p.d_per_p = a->d_per_p ? 1 : 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  const dim3 grid(elem_grid(p)), block(EB_THREADS);
+  const bool of = a->dy_dtype == SSM_F32;
+  switch (a->io_dtype) {
+    case SSM_F32:
+      if (of) hipLaunchKernelGGL((ssd_bwd_gate_kernel<float, float>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((ssd_bwd_gate_kernel<float, bf16_t>), grid, block, 0, s, p);
+      break;
+    case SSM_BF16:
+      if (of) hipLaunchKernelGGL((ssd_bwd_gate_kernel<bf16_t, float>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((ssd_bwd_gate_kernel<bf16_t, bf16_t>), grid, block, 0, s, p);
+      break;
+    default:
+      if (of) hipLaunchKernelGGL((ssd_bwd_gate_kernel<f16_t, float>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((ssd_bwd_gate_kernel<f16_t, bf16_t>), grid, block, 0, s, p);
+  }
+  SSM_CHECK_LAUNCH("ssm_ssd_bwd_gate");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_bwd_dx(const ssm_ssd_bwd_dx_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_dx: args is NULL");
+  SSM_REQUIRE(a->dout && a->x && a->u_rev && a->dt && a->dx && a->xu && a->s1, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_bwd_dx: dout, x, u_rev, dt, dx, xu and s1 are required");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->headdim > 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bwd_dx: batch, seqlen, heads and headdim must be positive");
+  ElemParams p{};
+  SSM_REQUIRE(row_lanes(a->headdim, p.lg), SSM_ERR_BAD_SHAPE, "ssm_ssd_bwd_dx: headdim=%d must be 4 * 2^k, at most 256",
+              a->headdim);
+  SSM_REQUIRE(valid_dtype(a->io_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_bwd_dx: io_dtype=%d", a->io_dtype);
+  SSM_REQUIRE((size_t)a->batch * a->seqlen * a->heads < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_dx: too many rows");
+  SSM_REQUIRE(aligned_to(a->dout, 8) && aligned_to(a->x, 8) && (!a->z || aligned_to(a->z, 8)) && aligned_to(a->u_rev, 16) &&
+                  aligned_to(a->dx, 16),
+              SSM_ERR_ALIGNMENT, "ssm_ssd_bwd_dx: a pointer is not sufficiently aligned");
+  p.dout = a->dout; p.z = a->z; p.x = a->x; p.u_rev = a->u_rev; p.dt = a->dt; p.Dk = a->Dskip;
+  p.dx = a->dx; p.xu = a->xu; p.s1 = a->s1;
+  p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.hdim = a->headdim; p.d_per_p = a->d_per_p ? 1 : 0;
+  p.round_bf16 = a->round_bf16 ? 1 : 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  const dim3 grid(elem_grid(p)), block(EB_THREADS);
+  switch (a->io_dtype) {
+    case SSM_F32: hipLaunchKernelGGL(ssd_bwd_dx_kernel<float>, grid, block, 0, s, p); break;
+    case SSM_BF16: hipLaunchKernelGGL(ssd_bwd_dx_kernel<bf16_t>, grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL(ssd_bwd_dx_kernel<f16_t>, grid, block, 0, s, p);
+  }
+  SSM_CHECK_LAUNCH("ssm_ssd_bwd_dx");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_bwd_db(const ssm_ssd_bwd_db_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_db: args is NULL");
+  SSM_REQUIRE(a->v_rev && a->dt && a->dB, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_db: v_rev, dt and dB are required");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->groups > 0 && a->nstate > 0 && a->heads % a->groups == 0,
+              SSM_ERR_BAD_SHAPE, "ssm_ssd_bwd_db: sizes must be positive and groups must divide heads");
+  SSM_REQUIRE(a->nstate % 4 == 0, SSM_ERR_BAD_SHAPE, "ssm_ssd_bwd_db: nstate=%d must be a multiple of 4", a->nstate);
+  SSM_REQUIRE(aligned_to(a->v_rev, 16) && aligned_to(a->dB, 16), SSM_ERR_ALIGNMENT, "ssm_ssd_bwd_db: v_rev and dB must be 16-byte aligned");
+  DbParams p{};
+  p.v_rev = a->v_rev; p.dt = a->dt; p.dB = a->dB;
+  p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.groups = a->groups; p.nstate = a->nstate;
+  const size_t total = (size_t)p.batch * p.len * p.groups * (p.nstate / 4);
+  SSM_REQUIRE(total < ((size_t)1 << 40), SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_db: tensor too large");
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(ssd_bwd_db_kernel, dim3((unsigned)((total + EB_THREADS - 1) / EB_THREADS)), dim3(EB_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_bwd_db");
+  return SSM_OK;
+}

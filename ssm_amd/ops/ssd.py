@@ -519,6 +519,57 @@ def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None):
     return (y, final, entering) if want_entering else (y, final)
 
 
+def _elem_stages_ok(x, dout, z, hdim):
+    """Whether the fused element-wise stages of the backward take this call: one dtype for ``x``, ``dout``
+    and ``z``, and a head dimension of 4 * 2^k (at most 256)."""
+    q = hdim // 4
+    return (hdim % 4 == 0 and 1 <= q <= 64 and (q & (q - 1)) == 0 and dout.dtype == x.dtype
+            and (z is None or z.dtype == x.dtype))
+
+
+def _bwd_gate(dout, z, x, ypre, Df, cd, want_rev=True):
+    """``ssm_ssd_bwd_gate``: ``(dy, dy_rev, dz, s2, dyx)``."""
+    batch, seqlen, heads, hdim = (int(v) for v in x.shape)
+    dev = x.device
+    dy = torch.empty(batch, seqlen, heads, hdim, dtype=cd, device=dev)
+    dy_rev = torch.empty_like(dy) if want_rev else None
+    dz = torch.empty(batch, seqlen, heads, hdim, dtype=torch.float32, device=dev) if z is not None else None
+    s2 = torch.empty(batch, seqlen, heads, dtype=torch.float32, device=dev)
+    dyx = torch.empty_like(s2)
+    args = _lib.SsdBwdGateArgs(
+        dout=_lib.ptr(dout), z=_lib.ptr(z), x=_lib.ptr(x), ypre=_lib.ptr(ypre), Dskip=_lib.ptr(Df), dy=_lib.ptr(dy),
+        dy_rev=_lib.ptr(dy_rev), dz=_lib.ptr(dz), s2=_lib.ptr(s2), dyx=_lib.ptr(dyx), batch=batch, seqlen=seqlen,
+        heads=heads, headdim=hdim, io_dtype=_lib.dtype_enum(x.dtype), dy_dtype=_lib.dtype_enum(cd),
+        d_per_p=int(Df is not None and Df.ndim == 2))
+    _lib.call("ssm_ssd_bwd_gate", args, dev)
+    return dy, dy_rev, dz, s2, dyx
+
+
+def _bwd_dx(dout, z, x, u_rev, dte, Df, round_bf16):
+    """``ssm_ssd_bwd_dx``: ``(dx, xu, s1)``."""
+    batch, seqlen, heads, hdim = (int(v) for v in x.shape)
+    dev = x.device
+    dx = torch.empty(batch, seqlen, heads, hdim, dtype=torch.float32, device=dev)
+    xu = torch.empty(batch, seqlen, heads, dtype=torch.float32, device=dev)
+    s1 = torch.empty_like(xu)
+    args = _lib.SsdBwdDxArgs(
+        dout=_lib.ptr(dout), z=_lib.ptr(z), x=_lib.ptr(x), u_rev=_lib.ptr(u_rev), dt=_lib.ptr(dte), Dskip=_lib.ptr(Df),
+        dx=_lib.ptr(dx), xu=_lib.ptr(xu), s1=_lib.ptr(s1), batch=batch, seqlen=seqlen, heads=heads, headdim=hdim,
+        io_dtype=_lib.dtype_enum(x.dtype), d_per_p=int(Df is not None and Df.ndim == 2), round_bf16=int(bool(round_bf16)))
+    _lib.call("ssm_ssd_bwd_dx", args, dev)
+    return dx, xu, s1
+
+
+def _bwd_db(v_rev, dte, groups):
+    """``ssm_ssd_bwd_db``: ``dB (B, L, G, N)`` from the reversed pass output ``(B, L, H, N)``."""
+    batch, seqlen, heads, nstate = (int(v) for v in v_rev.shape)
+    dB = torch.empty(batch, seqlen, groups, nstate, dtype=torch.float32, device=v_rev.device)
+    args = _lib.SsdBwdDbArgs(v_rev=_lib.ptr(v_rev), dt=_lib.ptr(dte), dB=_lib.ptr(dB), batch=batch, seqlen=seqlen,
+                             heads=heads, groups=groups, nstate=nstate)
+    _lib.call("ssm_ssd_bwd_db", args, v_rev.device)
+    return dB
+
+
 def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
                           initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
     """Gradients of :func:`ssd_combined` (outputs ``y`` and ``final_states``).
@@ -551,14 +602,18 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     Q = int(chunk_size)
     per = heads // groups
     f32 = torch.float32
-    xf, Bf, Cf, Af = x.detach().to(f32), B.detach().to(f32), C.detach().to(f32), A.detach().to(f32)
-    dof = dout.detach().to(f32)
+    Af = A.detach().to(f32)
+    fused = _elem_stages_ok(x, dout, z, hdim)
+    xd, dod = x.detach().contiguous(), dout.detach().contiguous()
+    zd = None if z is None else z.detach().contiguous()
+    xf = None if fused else xd.to(f32)
+    dof = None if fused else dod.to(f32)
     # The passes take their operands in the inputs' precision when that is bfloat16 (matrix-core kernels,
     # float32 accumulation and states); everything between the passes is float32 either way.
     cd = torch.bfloat16 if (x.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and C.dtype == torch.bfloat16) else f32
-    xc, Bc, Cc = (x.detach(), B.detach(), C.detach()) if cd != f32 else (xf, Bf, Cf)
-    Df = None if D is None else D.detach().to(f32)
-    Dx = 0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * xf
+    xc, Bc, Cc = (xd, B.detach(), C.detach()) if cd != f32 else (xd.to(f32), B.detach().to(f32), C.detach().to(f32))
+    Df = None if D is None else D.detach().to(f32).contiguous()
+    Dx = 0.0 if (Df is None or fused) else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * xf
     init = None if initial_states is None else initial_states.detach().to(f32)
     dfin = None if dfinal is None else dfinal.detach().to(f32).contiguous()
 
@@ -573,39 +628,56 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     # C.B-times-decay blocks, and the running sum that gives q (a difference of their row and column sums)
     # sees each product twice with the same value instead of collecting the two passes' rounding noise.
     _, ones_c = chunk_cumsum(torch.ones_like(dte), torch.zeros_like(Af), Q)
-    xt = (dte[..., None] * xf).to(cd)
+    dte = dte.contiguous()
+    xt = (dte[..., None] * xd).to(cd)
     ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
-    if z is not None:
-        zf = z.detach().to(f32)
-        sg = torch.sigmoid(zf)
-        dy = dof * zf * sg
-        dz = dof * (ypre + Dx) * (sg * (1.0 + zf * (1.0 - sg)))
-    else:
-        dy, dz = dof, None
     dD = None
-    if Df is not None:
-        dD = (dy * xf).sum(dim=(0, 1, 3)) if Df.ndim == 1 else (dy * xf).sum(dim=(0, 1))
+    if fused:
+        dyc, dyr, dz, s2, dyx = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd)
+        if Df is not None and Df.ndim == 1:
+            dD = dyx.sum(dim=(0, 1))
+        elif Df is not None:
+            gate = 1.0 if zd is None else torch.nn.functional.silu(zd.to(f32))
+            dD = (dod.to(f32) * gate * xd.to(f32)).sum(dim=(0, 1))
+    else:
+        if z is not None:
+            zf = zd.to(f32)
+            sg = torch.sigmoid(zf)
+            dy = dof * zf * sg
+            dz = dof * (ypre + Dx) * (sg * (1.0 + zf * (1.0 - sg)))
+        else:
+            dy, dz = dof, None
+        if Df is not None:
+            dD = (dy * xf).sum(dim=(0, 1, 3)) if Df.ndim == 1 else (dy * xf).sum(dim=(0, 1))
     # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
     dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
     dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
-    dyc = dy.to(cd)
-    dyr = dyc.flip(1).contiguous()
+    if not fused:
+        dyc = dy.to(cd)
+        dyr = dyc.flip(1).contiguous()
     u_r, Gfin, ent_r = _lin_pass(dyr, ones_c, dA_r, Cc.flip(1).contiguous(), Bc.flip(1).contiguous(), dfin,
                                  want_entering=True)
-    u = u_r.flip(1)
     dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin
-    dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
+    if fused:
+        dx, xu, s1 = _bwd_dx(dod, zd, xd, u_r.contiguous(), dte, Df, cd == torch.bfloat16)
+    else:
+        u = u_r.flip(1)
+        dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
     Bh = Bc.repeat_interleave(per, dim=2) if per > 1 else Bc
     Ch = Cc.repeat_interleave(per, dim=2) if per > 1 else Cc
     v_r, _ = _lin_pass(Ch.flip(1).contiguous(), ones_c, dA_r, dyr, xc.flip(1).contiguous(),
                        None if dfin is None else dfin.transpose(2, 3).contiguous())
-    dB = (dte[..., None] * v_r.flip(1)).view(batch, seqlen, groups, per, nstate).sum(3)
+    if nstate % 4 == 0:
+        dB = _bwd_db(v_r.contiguous(), dte, groups)
+    else:
+        dB = (dte[..., None] * v_r.flip(1)).view(batch, seqlen, groups, per, nstate).sum(3)
     dCh, _ = _lin_pass(Bh.contiguous(), dt_c, dA_cs, xc, dyc.contiguous(),
                        None if init is None else init.transpose(2, 3).contiguous())
     dC = dCh.view(batch, seqlen, groups, per, nstate).sum(3)
-    xu = (xf * u).sum(-1)                                             # (B, L, H)
-    s1 = (xt.to(f32) * u).sum(-1)                  # with the rounded operand of the pass for y
-    s2 = (dyc.to(f32) * ypre).sum(-1)              # the same rounded dy that the pass for u saw
+    if not fused:
+        xu = (xf * u).sum(-1)                                             # (B, L, H)
+        s1 = (xt.to(f32) * u).sum(-1)                  # with the rounded operand of the pass for y
+        s2 = (dyc.to(f32) * ypre).sum(-1)              # the same rounded dy that the pass for u saw
     W0 = (dinit * init).sum(dim=(2, 3)) if init is not None else torch.zeros(batch, heads, dtype=f32, device=x.device)
     nc = (seqlen + Q - 1) // Q
     if seqlen % Q == 0 and nc > 1:
