@@ -195,12 +195,14 @@ __device__ __forceinline__ void st_pack(void *p, size_t i, const float (&v)[VEC]
   *reinterpret_cast<Pack<T, VEC> *>(reinterpret_cast<T *>(p) + i) = raw;
 }
 
-template <int TRIPS, typename XT, typename RT>
+template <int TRIPS, bool WG, typename XT, typename RT>
 __global__ __launch_bounds__(LN_THREADS) void norm_fwd_typed_kernel(const NormParams p) {
   constexpr int VEC = 4;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int row = (int)(blockIdx.x * LN_WAVES + wave);
-  if (row >= p.rows) return;
+  constexpr int OWNERS = WG ? LN_THREADS : WAVE;       // threads that share a row
+  __shared__ float red[LN_WAVES];
+  const int wave = threadIdx.x >> 6, lane = WG ? (int)threadIdx.x : (int)(threadIdx.x & 63);
+  const int row = WG ? (int)blockIdx.x : (int)(blockIdx.x * LN_WAVES + wave);
+  if (row >= p.rows) return;                           // whole workgroups in WG mode
   const int H = p.hidden;
   const size_t base = (size_t)row * H;
   const bool has_res = p.res != nullptr, has_b = p.b != nullptr;
@@ -211,13 +213,13 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_typed_kernel(const NormPa
   float sum = 0.0f;
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int colc = min((k * WAVE + lane) * VEC, H - VEC);
+    const int colc = min((k * OWNERS + lane) * VEC, H - VEC);
     ld_pack<XT, VEC>(p.x, base + colc, v[k]);
     ld_pack<RT, VEC>(resp, base + colc, r[k]);
   }
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int col = (k * WAVE + lane) * VEC;
+    const int col = (k * OWNERS + lane) * VEC;
     const bool live = col < H;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -231,31 +233,31 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_typed_kernel(const NormPa
   float wv[TRIPS][VEC], bv[TRIPS][VEC];
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int colc = min((k * WAVE + lane) * VEC, H - VEC);
+    const int colc = min((k * OWNERS + lane) * VEC, H - VEC);
     ld_pack<float, VEC>(p.w, colc, wv[k]);
     ld_pack<float, VEC>(bp, colc, bv[k]);
   }
   const float inv_h = 1.0f / (float)H;
   float mean = 0.0f;
-  if (!p.is_rms) mean = wave_sum(sum) * inv_h;
+  if (!p.is_rms) mean = row_sum<WG>(sum, red) * inv_h;
   float sq = 0.0f;
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const bool live = (k * WAVE + lane) * VEC < H;
+    const bool live = (k * OWNERS + lane) * VEC < H;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       const float c = live ? v[k][i] - mean : 0.0f;
       sq = __builtin_fmaf(c, c, sq);
     }
   }
-  const float rstd = 1.0f / sqrtf(wave_sum(sq) * inv_h + p.eps);
+  const float rstd = 1.0f / sqrtf(row_sum<WG>(sq, red) * inv_h + p.eps);
   if (lane == 0) {
     if (p.mean) p.mean[row] = mean;
     if (p.rstd) p.rstd[row] = rstd;
   }
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
-    const int col = (k * WAVE + lane) * VEC;
+    const int col = (k * OWNERS + lane) * VEC;
     float out[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -270,16 +272,20 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_typed_kernel(const NormPa
 
 template <typename XT, typename RT>
 static void launch_norm_fwd_typed(const NormParams &p, int per_lane, unsigned grid, hipStream_t s) {
-  if (per_lane <= 4) hipLaunchKernelGGL((norm_fwd_typed_kernel<1, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
-  else if (per_lane <= 8) hipLaunchKernelGGL((norm_fwd_typed_kernel<2, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
-  else if (per_lane <= 12) hipLaunchKernelGGL((norm_fwd_typed_kernel<3, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
-  else if (per_lane <= 16) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
-  else hipLaunchKernelGGL((norm_fwd_typed_kernel<8, XT, RT>), dim3(grid), dim3(LN_THREADS), 0, s, p);
+  const dim3 b(LN_THREADS);
+  if (per_lane <= 4) hipLaunchKernelGGL((norm_fwd_typed_kernel<1, false, XT, RT>), dim3(grid), b, 0, s, p);
+  else if (per_lane <= 8) hipLaunchKernelGGL((norm_fwd_typed_kernel<2, false, XT, RT>), dim3(grid), b, 0, s, p);
+  else if (per_lane <= 12) hipLaunchKernelGGL((norm_fwd_typed_kernel<3, false, XT, RT>), dim3(grid), b, 0, s, p);
+  else if (per_lane <= 16) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, false, XT, RT>), dim3(grid), b, 0, s, p);
+  else if (per_lane <= 32) hipLaunchKernelGGL((norm_fwd_typed_kernel<8, false, XT, RT>), dim3(grid), b, 0, s, p);
+  else if (p.hidden <= 4096) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, true, XT, RT>), dim3(p.rows), b, 0, s, p);
+  else if (p.hidden <= 8192) hipLaunchKernelGGL((norm_fwd_typed_kernel<8, true, XT, RT>), dim3(p.rows), b, 0, s, p);
+  else hipLaunchKernelGGL((norm_fwd_typed_kernel<16, true, XT, RT>), dim3(p.rows), b, 0, s, p);
 }
 
 // True when the call was taken by a typed kernel.
 static bool norm_fwd_typed(const NormParams &p, int per_lane, unsigned grid, hipStream_t s) {
-  if (per_lane > 32 || p.hidden < 4) return false;
+  if (p.hidden > 16384 || p.hidden < 4) return false;
   // residual and residual_out must agree on one type, float32 or that of x
   int rt = -1;
   if (p.res) rt = p.res_dtype;

@@ -264,9 +264,8 @@ __global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) 
   }
 }
 
-template <typename state_t, typename io_t>
+template <typename state_t, typename io_t, int RB>
 static void launch_rb(const StepParams &p, unsigned grid, hipStream_t stream) {
-  constexpr int RB = 4;
   if (p.conv_state) hipLaunchKernelGGL((state_step_rb_kernel<state_t, io_t, true, RB>), dim3(grid), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((state_step_rb_kernel<state_t, io_t, false, RB>), dim3(grid), dim3(256), 0, stream, p);
 }
@@ -279,21 +278,23 @@ static int launch_step(const StepParams &p0, bool vec4, hipStream_t stream) {
   int lg = 0;
   while ((1 << lg) < per_row && lg < 4) ++lg;    // at most 16 lanes per row
   p.tpr_log2 = lg;
-  constexpr int RB = 4;
-  if (vec4 && p.nstate == (4 << lg) && lg >= 2 && p.batch % RB == 0 && (!p.conv_state || p.conv_k <= (1 << lg))) {
-    const size_t threads_rb = ((size_t)p.dim * (p.batch / RB)) << lg;
+  if (vec4 && p.nstate == (4 << lg) && lg >= 2 && (!p.conv_state || p.conv_k <= (1 << lg))) {
+    // four batch rows per thread when the batch allows it (and is large enough to fill the device that way),
+    // one otherwise; float32 states with activations and projections of one type: element types known at
+    // compile time
+    const bool four = p.batch % 4 == 0 && (size_t)p.batch * p.dim >= 65536;
+    const size_t threads_rb = ((size_t)p.dim * (four ? p.batch / 4 : p.batch)) << lg;
     const unsigned grid_rb = (unsigned)((threads_rb + 255) / 256);
-    // float32 states with activations and projections of one type: element types known at compile time
     bool done = false;
     if constexpr (std::is_same<state_t, float>::value) {
       if (p.io_dtype == p.bc_dtype) {
-        if (p.io_dtype == SSM_BF16) launch_rb<state_t, bf16_t>(p, grid_rb, stream);
-        else if (p.io_dtype == SSM_F16) launch_rb<state_t, f16_t>(p, grid_rb, stream);
-        else launch_rb<state_t, float>(p, grid_rb, stream);
+        if (p.io_dtype == SSM_BF16) four ? launch_rb<state_t, bf16_t, 4>(p, grid_rb, stream) : launch_rb<state_t, bf16_t, 1>(p, grid_rb, stream);
+        else if (p.io_dtype == SSM_F16) four ? launch_rb<state_t, f16_t, 4>(p, grid_rb, stream) : launch_rb<state_t, f16_t, 1>(p, grid_rb, stream);
+        else four ? launch_rb<state_t, float, 4>(p, grid_rb, stream) : launch_rb<state_t, float, 1>(p, grid_rb, stream);
         done = true;
       }
     }
-    if (!done) launch_rb<state_t, void>(p, grid_rb, stream);
+    if (!done) four ? launch_rb<state_t, void, 4>(p, grid_rb, stream) : launch_rb<state_t, void, 1>(p, grid_rb, stream);
     SSM_CHECK_LAUNCH("ssm_state_step");
     return SSM_OK;
   }
