@@ -86,7 +86,7 @@ typedef struct ssm_scan_fwd_args {
   int32_t b_groups, c_groups; /* G for SSM_PROJ_BGNL (must divide D), else ignored */
   int32_t delta_softplus; /* 0 / 1 */
   int32_t tune_items;     /* 0 = automatic; else 100 * steps-per-lane + states-per-LDS-pass (408, 808, 816);
-                             1616 = 816 with two channels per wave */
+                             1616, 2416, 3216, 4816 = 816 with two, three, four, six channels per wave */
 } ssm_scan_fwd_args;
 
 int ssm_scan_fwd(const ssm_scan_fwd_args *args, void *hip_stream);

@@ -70,14 +70,33 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   int tune = a->tune_items;
   if (tune == 0) {
     if (a->seqlen <= 256 && !a->chunk_states) tune = 408;
-    else if (pair_ok && (size_t)a->batch * a->dim / 16 >= 512) tune = 1616;
     else tune = a->nstate > 8 ? 816 : 808;
+    if (tune != 408 && pair_ok) {
+      // Several channels per wave share one staged B/C slab.  Two workgroups of 8 waves are resident per CU;
+      // take the number of channels per wave whose grid leaves the fewest of those 512 places idle in its
+      // last round (at B=8, D=1536: 3 -> 512 workgroups, one full round; 2 -> 768, the second round half empty).
+      const int cand[4] = {3, 2, 4, 6};
+      double best = 0.0;
+      for (int i = 0; i < 4; ++i) {
+        const int per_wg = cand[i] * SCAN_MAX_WAVES;
+        if (per_b % per_wg != 0 || per_c % per_wg != 0) continue;
+        const size_t wgs = (size_t)a->batch * a->dim / per_wg;
+        if (wgs < 512) continue;
+        const size_t rounds = (wgs + 511) / 512;
+        const double fill = (double)wgs / (double)(rounds * 512);
+        if (fill > best + 1e-9) {
+          best = fill;
+          tune = cand[i] * 800 + 16;
+        }
+      }
+    }
   }
-  if (tune == 1616) {
-    if (pair_ok) rows = 2 * SCAN_MAX_WAVES;
+  if (tune == 1616 || tune == 2416 || tune == 3216 || tune == 4816) {        // 2, 3, 4, 6 channels per wave
+    const int r = tune / 100;
+    if (pair_ok && per_b % r == 0 && per_c % r == 0) rows = r;
     else tune = 816;
   }
-  const int steps_per_lane = tune == 1616 ? 8 : tune / 100;
+  const int steps_per_lane = tune >= 1616 ? 8 : tune / 100;
   if (a->chunk_states)
     SSM_REQUIRE(steps_per_lane * WAVE == ssm_scan_chunk_len(), SSM_ERR_BAD_KIND,
                 "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (tune_items 808, 816 or 1616)",

@@ -345,6 +345,9 @@ static int dispatch_flags(const ScanFwdParams &p, int rows, hipStream_t s) {
   const bool sn = p.nstate <= SCAN_LANE_STATES;
   // two rows per wave when a workgroup of 16 channels fits one group and all states fit one slab
   if (bv && cv && sn && rows == 2 * SCAN_MAX_WAVES) return launch_scan_fwd<io_t, K, NB, true, true, true, 2>(p, rows, s);
+  if (bv && cv && sn && rows == 3 * SCAN_MAX_WAVES) return launch_scan_fwd<io_t, K, NB, true, true, true, 3>(p, rows, s);
+  if (bv && cv && sn && rows == 4 * SCAN_MAX_WAVES) return launch_scan_fwd<io_t, K, NB, true, true, true, 4>(p, rows, s);
+  if (bv && cv && sn && rows == 6 * SCAN_MAX_WAVES) return launch_scan_fwd<io_t, K, NB, true, true, true, 6>(p, rows, s);
   const int key = (bv ? 4 : 0) | (cv ? 2 : 0) | (sn ? 1 : 0);
   switch (key) {
     case 0: return launch_scan_fwd<io_t, K, NB, false, false, false, 1>(p, rows, s);
@@ -366,8 +369,9 @@ int scan_fwd_dispatch(const ScanFwdParams &p, int tune, int rows, hipStream_t s)
     case 808: return dispatch_flags<io_t, 8, 8>(p, rows, s);
     case 816: return dispatch_flags<io_t, 8, 16>(p, rows, s);
     case 1616: return dispatch_flags<io_t, 8, 16>(p, rows, s);      // 816 with two rows per wave (see entry point)
+    case 2416: case 3216: case 4816: return dispatch_flags<io_t, 8, 16>(p, rows, s);   // 816 with 3, 4, 6 rows per wave
     default:
-      set_error("ssm_scan_fwd: unsupported tune_items %d (408, 808, 816, 1616)", tune);
+      set_error("ssm_scan_fwd: unsupported tune_items %d (408, 808, 816, 1616, 2416)", tune);
       return SSM_ERR_BAD_KIND;
   }
 }

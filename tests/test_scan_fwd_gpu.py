@@ -203,6 +203,19 @@ def test_every_tile_width_matches_oracle(items):
     torch.testing.assert_close(h.cpu(), hr, **FP32_TOL)
 
 
+@pytest.mark.parametrize("items,dim", [(1616, 48), (2416, 48), (3216, 64), (4816, 48)])
+def test_several_channels_per_wave_match_oracle(items, dim):
+    """2, 3, 4 or 6 channels of one B/C group share a wave (and one staged slab); ragged last chunk, bf16."""
+    from ssm_amd.ops import _scan_forward
+    inp = make_inputs(items, 2, dim, 1300, 16, dtype=torch.bfloat16)
+    yr, hr = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"],
+                              z=inp["z"], dt_bias=inp["dt_bias"], softplus=True, return_last_state=True)
+    y, h = _scan_forward(dev(inp["u"]), dev(inp["delta"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]),
+                         dev(inp["D"]), dev(inp["z"]), dev(inp["dt_bias"]), True, True, tune_items=items)
+    torch.testing.assert_close(y.float().cpu(), yr.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(h.float().cpu(), hr.float(), rtol=2e-2, atol=2e-2)
+
+
 # ---------------------------------------------- benchmark shapes and properties
 
 def test_config0_fp32_full_size_against_oracle():
