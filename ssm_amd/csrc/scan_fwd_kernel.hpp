@@ -148,6 +148,7 @@ __global__ __launch_bounds__(WAVE *SCAN_MAX_WAVES) void scan_fwd_kernel(const Sc
   const int d0 = ((int)blockIdx.x % blocks_per_batch) * rows;
   const int L = p.len, N = p.nstate;
   const bool vec_ok = p.vec_ok != 0;
+  const bool fast_rows = vec_ok && p.len % K == 0;       // aligned rows of whole runs
 
   constexpr bool bvary = BVARY, cvary = CVARY;
   float *Bs = tiles;
@@ -200,8 +201,21 @@ __global__ __launch_bounds__(WAVE *SCAN_MAX_WAVES) void scan_fwd_kernel(const Sc
           const float Dk = p.Dk ? p.Dk[d] : 0.0f;
           const float bias = p.bias ? p.bias[d] : 0.0f;
           float uu[K];
-          load_run<io_t, K>(reinterpret_cast<const io_t *>(p.u) + row * L, t, L, vec_ok, uu);
-          load_run<io_t, K>(reinterpret_cast<const io_t *>(p.delta) + row * L, t, L, vec_ok, dl);
+          if (fast_rows) {
+            // whole runs, read unconditionally and together (a lane past the end re-reads the last run; its
+            // steps become the identity below and nothing of it is stored)
+            const size_t at = row * L + min(t, L - K);
+            const Pack<io_t, K> ur = *reinterpret_cast<const Pack<io_t, K> *>(reinterpret_cast<const io_t *>(p.u) + at);
+            const Pack<io_t, K> dr = *reinterpret_cast<const Pack<io_t, K> *>(reinterpret_cast<const io_t *>(p.delta) + at);
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+              uu[i] = to_f32(ur.v[i]);
+              dl[i] = to_f32(dr.v[i]);
+            }
+          } else {
+            load_run<io_t, K>(reinterpret_cast<const io_t *>(p.u) + row * L, t, L, vec_ok, uu);
+            load_run<io_t, K>(reinterpret_cast<const io_t *>(p.delta) + row * L, t, L, vec_ok, dl);
+          }
           if (p.chunk_states) {
             float *cs = p.chunk_states + (row * nchunks + c) * (size_t)N;
             if (lane < N) cs[lane] = carry_lanes[rr];
