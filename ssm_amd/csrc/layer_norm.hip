@@ -530,7 +530,22 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_fold_kernel(const float *
   const int c = blockIdx.x * FOLD_COLS + cl;
   float sw = 0.0f, sb = 0.0f;
   if (c < hidden) {
-    for (int w = sl; w < nparts; w += FOLD_SLICES) {
+    // eight partials at a time: their reads are in flight together, the additions keep their order
+    int w = sl;
+    for (; w + 7 * FOLD_SLICES < nparts; w += 8 * FOLD_SLICES) {
+      float a[8], b[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        a[k] = partial[(size_t)(w + k * FOLD_SLICES) * 2 * hidden + c];
+        b[k] = partial[(size_t)(w + k * FOLD_SLICES) * 2 * hidden + hidden + c];
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        sw += a[k];
+        sb += b[k];
+      }
+    }
+    for (; w < nparts; w += FOLD_SLICES) {
       sw += partial[(size_t)w * 2 * hidden + c];
       sb += partial[(size_t)w * 2 * hidden + hidden + c];
     }
