@@ -638,7 +638,15 @@ __global__ __launch_bounds__(256) void fold_sum_vec4_kernel(const float *in, flo
 __global__ __launch_bounds__(256) void fold_rows_kernel(const float *in, float *out, int count, size_t inner) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < inner; i += (size_t)gridDim.x * blockDim.x) {
     float s = 0.0f;
-    for (int j = 0; j < count; ++j) s += in[(size_t)j * inner + i];
+    int j = 0;
+    for (; j + 8 <= count; j += 8) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = in[(size_t)(j + k) * inner + i];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) s += v[k];
+    }
+    for (; j < count; ++j) s += in[(size_t)j * inner + i];
     out[i] = s;
   }
 }
@@ -663,8 +671,18 @@ __global__ __launch_bounds__(256) void fold_sum_wide_kernel(const float *in, flo
   const size_t o = blockIdx.x / blocks_per_outer;
   const size_t i = (size_t)(blockIdx.x % blocks_per_outer) * cols + cl;
   float sum = 0.0f;
-  if (i < inner && sl < slices)
-    for (int j = sl; j < count; j += slices) sum += in[(o * count + j) * inner + i];
+  if (i < inner && sl < slices) {
+    // eight terms at a time: their reads are in flight together, the additions keep their order
+    int j = sl;
+    for (; j + 7 * slices < count; j += 8 * slices) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = in[(o * count + j + k * slices) * inner + i];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) sum += v[k];
+    }
+    for (; j < count; j += slices) sum += in[(o * count + j) * inner + i];
+  }
   part[threadIdx.x] = sum;
   __syncthreads();
   if (sl == 0 && i < inner) {
