@@ -450,6 +450,8 @@ typedef struct ssm_ssd_combined_args {
   int32_t io_dtype;           /* must be SSM_BF16 */
   int32_t dt_dtype, dt_softplus, d_per_p;
   float dt_min, dt_max;       /* clamp applied after softplus; use 0 and +inf for none */
+  const int32_t *seq_idx;     /* (B, L) sequence ids of a packed batch (first id 0), or NULL: no state and no
+                                 in-chunk term crosses from one sequence into the next */
 } ssm_ssd_combined_args;
 int ssm_ssd_combined_supported(const ssm_ssd_dims *dims, int io_dtype);   /* 1 / 0 */
 size_t ssm_ssd_combined_workspace_bytes(const ssm_ssd_dims *dims);

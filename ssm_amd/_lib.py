@@ -174,7 +174,8 @@ class SsdCombinedArgs(C.Structure):
     _fields_ = [("x", _vp), ("dt", _vp), ("A", _vp), ("dt_bias", _vp), ("Bm", _vp), ("Cm", _vp), ("Dskip", _vp),
                 ("z", _vp), ("initial_states", _vp), ("y", _vp), ("final_states", _vp), ("workspace", _vp),
                 ("workspace_bytes", C.c_size_t), ("dims", SsdDims), ("io_dtype", _i32), ("dt_dtype", _i32),
-                ("dt_softplus", _i32), ("d_per_p", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float)]
+                ("dt_softplus", _i32), ("d_per_p", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float),
+                ("seq_idx", _vp)]
 
 
 class SsdBwdGateArgs(C.Structure):

@@ -72,9 +72,17 @@ struct SsdPrepParams {
   const __bf16 *Cm, *Bm;
   __bf16 *Cblk, *Btblk, *CBblk;
   unsigned n_dt, n_pack;                 // workgroups of the first two roles
+  const int *seq_idx;                    // (B, L) sequence ids of a packed batch, or null
 };
 
-__device__ __forceinline__ void prep_dt_role(const SsdCumsumParams &p, float *dA2, int wg, float *lds) {
+// Packed sequences: the first step of a sequence gets an extra decay of 2^-64 (a jump in the running sum),
+// so that nothing of the sequences before it - state or in-chunk terms - reaches it or the steps after it:
+// exp2(cs_l - cs_s) then carries that factor whenever a boundary lies in (s, l].  The steps of one sequence
+// see the same jumps on both sides of the difference; with every step of a 256-step chunk a boundary the sum
+// reaches 2^14, where float32 still resolves 1e-3 of the exponent.
+constexpr float SEQ_JUMP_LN = -64.0f * 0.69314718056f;
+
+__device__ __forceinline__ void prep_dt_role(const SsdCumsumParams &p, float *dA2, const int *seq_idx, int wg, float *lds) {
   float (*tile)[256 + 1] = reinterpret_cast<float (*)[256 + 1]>(lds);
   const SsdDims &d = p.d;
   const int Q = d.chunk;
@@ -109,6 +117,11 @@ __device__ __forceinline__ void prep_dt_role(const SsdCumsumParams &p, float *dA
         v[i] = fminf(fmaxf(x, p.dt_min), p.dt_max);
       }
       tot = __builtin_fmaf(v[i], A, tot);
+      if (seq_idx && i < per && l < Q) {
+        const size_t t = (size_t)c * Q + l;
+        const int *sid = seq_idx + (size_t)b * d.len;
+        if (t == 0 ? sid[0] != 0 : sid[t] != sid[t - 1]) tot += SEQ_JUMP_LN;
+      }
       run[i] = tot;
     }
     float incl = tot;
@@ -202,7 +215,7 @@ __device__ __forceinline__ void prep_cb_role(const SsdPrepParams &pp, unsigned w
 __global__ __launch_bounds__(256) void ssd_fused_prep_kernel(const SsdPrepParams pp) {
   __shared__ float lds[4 * 32 * 33];
   const unsigned wg = blockIdx.x;
-  if (wg < pp.n_dt) prep_dt_role(pp.cs, pp.dA2, (int)wg, lds);
+  if (wg < pp.n_dt) prep_dt_role(pp.cs, pp.dA2, pp.seq_idx, (int)wg, lds);
   else if (wg < pp.n_dt + pp.n_pack) prep_pack_role(pp, wg - pp.n_dt);
   else prep_cb_role(pp, wg - pp.n_dt - pp.n_pack, lds);
 }
@@ -789,6 +802,7 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   const size_t n_cb = (bcg * (NLB * (NLB + 1) / 2) + 3) / 4;
   SSM_REQUIRE(n_dt + n_pack + n_cb < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_combined_fwd: too many workgroups");
   pp.n_dt = (unsigned)n_dt; pp.n_pack = (unsigned)n_pack;
+  pp.seq_idx = a->seq_idx;
   hipLaunchKernelGGL(ssd_fused_prep_kernel, dim3((unsigned)(n_dt + n_pack + n_cb)), dim3(256), 0, s, pp);
   SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(prep)");
 

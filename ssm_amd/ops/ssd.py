@@ -329,8 +329,10 @@ def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
     return bool(_lib.load().ssm_ssd_combined_supported(dims, _lib.dtype_enum(torch.bfloat16)))
 
 
-def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit, return_final_states, shape):
+def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit, return_final_states, shape,
+               seq_idx=None):
     batch, seqlen, heads, hdim, groups, nstate = shape
+    si = _seq_idx_i32(seq_idx, batch, seqlen)
     d_per_p = False
     if D is not None:
         _need(tuple(D.shape) in ((heads,), (heads, hdim)), "D must have shape (H,) or (H, P).")
@@ -356,7 +358,7 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
         final_states=_lib.ptr(final), workspace=work.data_ptr() + off, workspace_bytes=nbytes, dims=dims,
         io_dtype=_lib.dtype_enum(torch.bfloat16), dt_dtype=_lib.dtype_enum(dtc.dtype),
         dt_softplus=int(bool(dt_softplus)), d_per_p=int(d_per_p),
-        dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]))
+        dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]), seq_idx=_lib.ptr(si))
     _lib.call("ssm_ssd_combined_fwd", args, dev)
     if return_final_states:
         return y, final
@@ -455,7 +457,6 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
     Q = int(chunk_size)
     _need(not return_varlen_states or cu_seqlens is not None, "return_varlen_states needs cu_seqlens.")
     _need(cu_seqlens is None or batch == 1, "cu_seqlens describes one packed batch row: batch size must be 1.")
-    packed = seq_idx is not None or return_varlen_states
     if x.dtype == torch.bfloat16 and hdim > 64 and hdim % 64 == 0 and not force_generic:
         # Channels of a head do not interact: a head of 64k channels is k heads of 64 with the same step,
         # decay and group, which is the width the one-pass and matrix-core kernels are built for.  The
@@ -475,13 +476,13 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
         for i in range(1, len(outs)):                 # final states, per-sequence states: (.., H k, 64, N)
             outs[i] = outs[i].reshape(outs[i].shape[0], heads, hdim, nstate)
         return outs[0] if len(outs) == 1 else tuple(outs)
-    can_fuse = not force_generic and fused is not False and not packed and \
+    can_fuse = not force_generic and fused is not False and not return_varlen_states and \
         _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
     _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "
           "chunk in {64,128,256}, nstate in {64,128} and seqlen % chunk == 0.")
     if can_fuse:
         return _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit,
-                          return_final_states, (batch, seqlen, heads, hdim, groups, nstate))
+                          return_final_states, (batch, seqlen, heads, hdim, groups, nstate), seq_idx=seq_idx)
     sdt = states_dtype or x.dtype
     dA, dtc = chunk_cumsum(dt, A, Q, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit)
     states = chunk_state(B, x, dtc, dA, states_dtype=sdt, force_generic=force_generic, seq_idx=seq_idx)

@@ -228,6 +228,41 @@ def test_packed_sequences_match_the_oracle_and_separate_runs(Q, lens, dtype, P):
         torch.testing.assert_close(vs[k].cpu(), fk[0].cpu(), **stol)
 
 
+@pytest.mark.parametrize("Q,lens,N", [(64, [100, 28, 64, 64], 64), (128, [300, 1, 83, 128], 128), (64, [64, 64, 64, 64], 64)])
+def test_packed_sequences_on_the_one_pass_kernel(Q, lens, N):
+    """seq_idx alone (no per-sequence end states asked for) stays on the one-pass kernel, which separates the
+    sequences by an extra decay of 2^-64 at every first step: against the float64 oracle, and against the
+    five-kernel path with its explicit masks."""
+    g = torch.Generator().manual_seed(29)
+    H, G, P = 4, 2, 64
+    L = sum(lens)
+    bf = torch.bfloat16
+    x = torch.randn(2, L, H, P, generator=g).to(bf)
+    dt = torch.rand(2, L, H, generator=g) * 0.5
+    A = -torch.rand(H, generator=g) * 2
+    Bm = torch.randn(2, L, G, N, generator=g).to(bf)
+    Cm = torch.randn(2, L, G, N, generator=g).to(bf)
+    D = torch.randn(H, generator=g)
+    z = torch.randn(2, L, H, P, generator=g).to(bf)
+    init = torch.randn(2, H, P, N, generator=g)
+    row = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])
+    seq_idx = torch.stack([row, torch.zeros_like(row)])          # second batch row: one sequence
+    from ssm_amd import _lib
+    _lib.load().ssm_ssd_mfma_launches()
+    y, fin = ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
+                                return_final_states=True, seq_idx=cu(seq_idx))
+    assert _lib.load().ssm_ssd_mfma_launches() & 8
+    y5, fin5 = ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
+                                  return_final_states=True, seq_idx=cu(seq_idx), fused=False, states_dtype=torch.float32)
+    wy, wf = S.ssd_combined(x, dt, A, Bm, Cm, Q, D=D, z=z, initial_states=init, clamp_decay=False, seq_idx=seq_idx)[:2]
+    tol = dict(rtol=2e-2, atol=2e-2 * float(wy.abs().max()))
+    stol = dict(rtol=2e-2, atol=2e-2 * float(wf.abs().max()))
+    torch.testing.assert_close(y.float().cpu(), wy.float(), **tol)
+    torch.testing.assert_close(fin.cpu(), wf.float(), **stol)
+    torch.testing.assert_close(y.float(), y5.float(), **tol)
+    torch.testing.assert_close(fin, fin5, **stol)
+
+
 def test_packed_arguments_are_checked():
     x = torch.zeros(2, 8, 2, 4).cuda()
     dt = torch.zeros(2, 8, 2).cuda()
