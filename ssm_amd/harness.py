@@ -260,6 +260,7 @@ class _Layer1:
 
         self.norm_w = torch.ones(d, dtype=torch.float32, device=device)
         self.in_proj_x, self.in_proj_z = rnd(di, d), rnd(di, d)
+        self.in_proj_xz = torch.cat([self.in_proj_x, self.in_proj_z], dim=0)      # one GEMM per token when decoding
         self.conv_w = (torch.rand(di, cfg.d_conv, generator=gen) - 0.5).float().to(device)
         self.conv_b = (torch.randn(di, generator=gen) * 0.02).float().to(device)
         self.x_proj = rnd(R + 2 * N, di)
@@ -335,8 +336,8 @@ class Mamba1LM(_GreedyDecoding):
             hidden, residual = ops.fused_layer_norm_with_residual(hidden, layer.norm_w, None, residual=residual,
                                                                   is_rms=True, eps=cfg.eps)
             hrow = hidden[:, 0]
-            x = hrow @ layer.in_proj_x.t()
-            z = hrow @ layer.in_proj_z.t()
+            xz = hrow @ layer.in_proj_xz.t()                          # (B, 2 d_inner): x is read in place, z copied
+            x, z = xz[:, :cfg.d_inner], xz[:, cfg.d_inner:]
             u = ops.conv_window_step(cw, x, layer.conv_w, layer.conv_b, activation="silu")
             low = u @ layer.x_proj.t()                                # (B, R + 2N)
             dt = low[:, :R] @ layer.dt_proj.t()
