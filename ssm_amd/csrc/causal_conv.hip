@@ -140,9 +140,10 @@ constexpr int CONV_CL_STRIP = 16;   // time steps per thread
 
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
 // number of vectors; otherwise the same kernel reads and writes element by element.
+constexpr int CONV_CL_FWD_BYTES = 8;   // bytes of channels per thread
 template <typename T, bool AL>
 __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvParams p) {
-  constexpr int VEC = 16 / sizeof(T);
+  constexpr int VEC = CONV_CL_FWD_BYTES / sizeof(T);
   const int cvecs = (p.chans + VEC - 1) / VEC;
   const int strips = (p.len + CONV_CL_STRIP - 1) / CONV_CL_STRIP;
   const size_t total = (size_t)p.batch * strips * cvecs;
@@ -349,9 +350,10 @@ __host__ __device__ inline int conv_cl_seg_len(int len) {
 
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
 // number of vectors; otherwise the same kernel reads and writes element by element.
+constexpr int CONV_CL_BWD_BYTES = 4;   // bytes of channels per thread: the walk keeps ~20 values per channel in registers
 template <typename T, bool AL>
 __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvParams p) {
-  constexpr int VEC = 16 / sizeof(T);
+  constexpr int VEC = CONV_CL_BWD_BYTES / sizeof(T);
   constexpr int HIST = CONV_TAPS - 1;
   const int cvecs = (p.chans + VEC - 1) / VEC;
   const int seg_len = conv_cl_seg_len(p.len);
@@ -585,7 +587,8 @@ static int conv_fwd_typed(const ConvParams &p, int channels_last, bool vec_ok, h
     else hipLaunchKernelGGL((conv_fwd_cf_kernel<T, false>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
   } else if (p.K <= CONV_TAPS && channels_last) {
     const int strips = (p.len + CONV_CL_STRIP - 1) / CONV_CL_STRIP;
-    const size_t threads = (size_t)p.batch * strips * ((p.chans + VEC - 1) / VEC);
+    constexpr int VECF = CONV_CL_FWD_BYTES / sizeof(T);
+    const size_t threads = (size_t)p.batch * strips * ((p.chans + VECF - 1) / VECF);
     const dim3 grid((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS));
     if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_fwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
     else hipLaunchKernelGGL((conv_fwd_cl_kernel<T, false>), grid, dim3(CONV_THREADS), 0, s, p);
@@ -608,7 +611,8 @@ static int conv_bwd_typed(const ConvParams &p, int channels_last, bool vec_ok, f
   } else if (p.K <= CONV_TAPS && channels_last) {
     const int seg_len = conv_cl_seg_len(p.len);
     const int nseg = (p.len + seg_len - 1) / seg_len;
-    const size_t threads = (size_t)p.batch * nseg * ((p.chans + VEC - 1) / VEC);
+    constexpr int VECB = CONV_CL_BWD_BYTES / sizeof(T);
+    const size_t threads = (size_t)p.batch * nseg * ((p.chans + VECB - 1) / VECB);
     const dim3 grid((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS));
     if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_bwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
     else hipLaunchKernelGGL((conv_bwd_cl_kernel<T, false>), grid, dim3(CONV_THREADS), 0, s, p);
