@@ -194,7 +194,7 @@ class SsdCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, dt_softplus, dt_limit,
-                states_dtype, force_generic, fused):
+                states_dtype, force_generic, fused, seq_idx=None):
         from .ssd import _ssd_combined_forward
 
         y, final = _ssd_combined_forward(x.detach(), dt.detach(), A.detach(), B.detach(), C.detach(), chunk_size,
@@ -202,9 +202,11 @@ class SsdCombinedFn(torch.autograd.Function):
                                          dt_bias=None if dt_bias is None else dt_bias.detach(),
                                          initial_states=None if initial_states is None else initial_states.detach(),
                                          dt_softplus=dt_softplus, dt_limit=dt_limit, return_final_states=True,
-                                         states_dtype=states_dtype, force_generic=force_generic, fused=fused)
+                                         states_dtype=states_dtype, force_generic=force_generic, fused=fused,
+                                         seq_idx=seq_idx)
         ctx.save_for_backward(x, dt, A, B, C, D, z, dt_bias, initial_states)
         ctx.conf = (chunk_size, dt_softplus, dt_limit)
+        ctx.seq_idx = seq_idx
         return y, final
 
     @staticmethod
@@ -217,9 +219,9 @@ class SsdCombinedFn(torch.autograd.Function):
             grad_y = torch.zeros_like(x)
         dx, ddt, dA, dB, dC, dD, dz, dbias, dinit = ssd_combined_backward(
             grad_y, grad_final, x, dt, A, B, C, Q, D=D, z=z, dt_bias=dt_bias, initial_states=init,
-            dt_softplus=softplus, dt_limit=limit)
+            dt_softplus=softplus, dt_limit=limit, seq_idx=ctx.seq_idx)
         need = ctx.needs_input_grad
         pick = lambda i, g, r: _like(g, r) if (r is not None and g is not None and need[i]) else None
         return (pick(0, dx, x), pick(1, ddt, dt), pick(2, dA, A), pick(3, dB, B), pick(4, dC, C), None,
                 pick(6, dD, D), pick(7, dz, z), pick(8, dbias, dt_bias), pick(9, dinit, init),
-                None, None, None, None, None)
+                None, None, None, None, None, None)

@@ -430,12 +430,14 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         return out[:, :seqlen]
     tensors = (x, dt, A, B, C, D, z, dt_bias, initial_states)
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
-        _need(seq_idx is None and cu_seqlens is None and not return_varlen_states,
-              "gradients of packed sequences (seq_idx / cu_seqlens) are not implemented.")
+        _need(cu_seqlens is None and not return_varlen_states,
+              "gradients through the per-sequence end states (cu_seqlens / return_varlen_states) are not "
+              "implemented; seq_idx alone is differentiable.")
         from ._autograd import SsdCombinedFn
+        si = None if seq_idx is None else _seq_idx_i32(seq_idx, int(x.shape[0]), int(x.shape[1]))
         y, final = SsdCombinedFn.apply(x, dt, A, B, C, int(chunk_size), D, z, dt_bias, initial_states,
                                        bool(dt_softplus), (float(dt_limit[0]), float(dt_limit[1])),
-                                       states_dtype, bool(force_generic), fused)
+                                       states_dtype, bool(force_generic), fused, si)
         return (y, final) if return_final_states else y
     return _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias,
                                  initial_states=initial_states, dt_softplus=dt_softplus, dt_limit=dt_limit,
@@ -572,7 +574,7 @@ def _bwd_db(v_rev, dte, groups):
 
 
 def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
-                          initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
+                          initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")), seq_idx=None):
     """Gradients of :func:`ssd_combined` (outputs ``y`` and ``final_states``).
 
     With ``a_t = exp(dt_t A)``, ``H_t = a_t H_{t-1} + dt_t x_t (x) B_t`` and the adjoint state
@@ -589,7 +591,11 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     scalar ``q_t = a_t <G_t, H_{t-1}>`` that ``ddt`` and ``dA`` need follows from
     ``<G_t, H_t> = <G_{t-1}, H_{t-1}> - <dy_{t-1}, H_{t-1} C_{t-1}> + dt_t <x_t, u_t>``, a running sum of
     quantities the passes have already produced.  The element-wise steps between the passes are
-    ordinary tensor operations.
+    fused kernels where the shape allows, tensor operations otherwise.
+
+    Packed sequences (``seq_idx``) need no masks here: the first step of a sequence simply has decay zero
+    (a jump of ``-64 ln 2`` in the running sums handed to the passes, forward and reversed), and every
+    formula above holds for any decay.
 
     Args:
         dout: ``(B, L, H, P)`` gradient of ``y``.
@@ -629,6 +635,17 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     # C.B-times-decay blocks, and the running sum that gives q (a difference of their row and column sums)
     # sees each product twice with the same value instead of collecting the two passes' rounding noise.
     _, ones_c = chunk_cumsum(torch.ones_like(dte), torch.zeros_like(Af), Q)
+    bnd = None
+    if seq_idx is not None:
+        sid = seq_idx.to(torch.int64)
+        bnd = sid != torch.cat([torch.zeros_like(sid[:, :1]), sid[:, :-1]], dim=1)      # (B, L): first steps
+
+        def jumps(first_steps):               # (B, L) bool -> (B, 1, nc, Q) running sums of the jumps per chunk
+            nc_ = dA_cs.shape[2]
+            f = torch.nn.functional.pad(first_steps.to(f32), (0, nc_ * Q - seqlen))
+            return (f.view(batch, nc_, Q).cumsum(-1) * (-64.0 * math.log(2.0)))[:, None]
+
+        dA_cs = dA_cs + jumps(bnd)
     dte = dte.contiguous()
     xt = (dte[..., None] * xd).to(cd)
     ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
@@ -653,12 +670,16 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
     dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
     dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
+    if bnd is not None:                       # the reversed passes decay by the following step's factor
+        dA_r = dA_r + jumps(torch.cat([bnd[:, 1:], torch.zeros_like(bnd[:, :1])], dim=1).flip(1))
     if not fused:
         dyc = dy.to(cd)
         dyr = dyc.flip(1).contiguous()
     u_r, Gfin, ent_r = _lin_pass(dyr, ones_c, dA_r, Cc.flip(1).contiguous(), Bc.flip(1).contiguous(), dfin,
                                  want_entering=True)
     dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin
+    if bnd is not None:
+        dinit = dinit * (~bnd[:, 0]).to(f32)[:, None, None, None]
     if fused:
         dx, xu, s1 = _bwd_dx(dod, zd, xd, u_r.contiguous(), dte, Df, cd == torch.bfloat16)
     else:
@@ -686,6 +707,8 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         # (a_t <G_t, H_{t-1}>, float32), and from there the running sum inside the chunk only: what the
         # two passes round differently then adds up over one chunk instead of the whole sequence.
         a_first = torch.exp(dte[:, ::Q] * Af[None, None])                           # (B, nc, H)
+        if bnd is not None:
+            a_first = a_first * (~bnd[:, ::Q]).to(f32)[..., None]
         anchor = (ent_r.flip(1)[:, :-1] * ent_f[:, 1:]).sum(dim=(3, 4))             # (B, nc-1, H): chunks 1..
         anchor = torch.cat([W0[:, None], a_first[:, 1:] * anchor], dim=1)
         dq = (s1 - s2).view(batch, nc, Q, heads)

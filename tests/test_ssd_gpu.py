@@ -160,13 +160,68 @@ def test_combined_gradient_vector_on_the_decaying_head():
         torch.testing.assert_close(f(d[k].grad.cpu()), f(gr[k]), rtol=5e-2, atol=5e-2, msg=lambda m: f"{k}: {m}")
 
 
-def test_gradients_of_packed_sequences_are_refused():
+def test_gradients_through_per_sequence_end_states_are_refused():
     x = torch.zeros(1, 8, 2, 4).cuda().requires_grad_(True)
     dt = torch.zeros(1, 8, 2).cuda()
     A = -torch.ones(2).cuda()
     Bm = torch.zeros(1, 8, 1, 4).cuda()
     with pytest.raises(ValueError):
-        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, seq_idx=torch.zeros(1, 8, dtype=torch.int32).cuda())
+        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, seq_idx=torch.zeros(1, 8, dtype=torch.int32).cuda(),
+                           cu_seqlens=torch.tensor([0, 8], dtype=torch.int32).cuda(), return_varlen_states=True)
+
+
+@pytest.mark.parametrize("dtype,lens,Q,P,N", [(torch.float32, [40, 24, 64], 32, 16, 8),
+                                            (torch.float32, [64, 64], 64, 8, 4),
+                                            (torch.bfloat16, [100, 28, 128], 64, 64, 64)])
+def test_gradients_of_packed_sequences_equal_those_of_the_sequences_alone(dtype, lens, Q, P, N):
+    """A packed row with seq_idx gives every input the gradient it gets when each sequence runs alone (the
+    first one with the initial state): per-step gradients side by side, parameter gradients added up."""
+    g = torch.Generator().manual_seed(41)
+    H, G = 4, 2
+    L = sum(lens)
+    mk = lambda *shape: torch.randn(*shape, generator=g)
+    base = dict(x=mk(1, L, H, P).to(dtype), dt=torch.rand(1, L, H, generator=g) * 0.5 + 0.05,
+                A=-torch.rand(H, generator=g) * 2 - 0.1, B=mk(1, L, G, N).to(dtype), C=mk(1, L, G, N).to(dtype),
+                D=mk(H), z=mk(1, L, H, P).to(dtype), init=mk(1, H, P, N))
+    wy = mk(1, L, H, P)
+    cu_l = [0]
+    for n in lens:
+        cu_l.append(cu_l[-1] + n)
+    seq_idx = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])[None].cuda()
+
+    def leaves(sl=None, with_init=True):
+        out = {}
+        for k, v in base.items():
+            t = v if (sl is None or k in ("A", "D", "init")) else v[:, sl]
+            out[k] = t.clone().cuda().requires_grad_(True)
+        if not with_init:
+            out["init"] = None
+        return out
+
+    p = leaves()
+    y = ssd().ssd_combined(p["x"], p["dt"], p["A"], p["B"], p["C"], Q, D=p["D"], z=p["z"], initial_states=p["init"],
+                           seq_idx=seq_idx)
+    (y.float() * wy.cuda()).sum().backward()
+    acc = {k: torch.zeros_like(v, dtype=torch.float32) for k, v in base.items()}
+    for k_seq in range(len(lens)):
+        sl = slice(cu_l[k_seq], cu_l[k_seq + 1])
+        q = leaves(sl, with_init=(k_seq == 0))
+        yk = ssd().ssd_combined(q["x"], q["dt"], q["A"], q["B"], q["C"], Q, D=q["D"], z=q["z"],
+                                initial_states=q["init"])
+        (yk.float() * wy[:, sl].cuda()).sum().backward()
+        for k in base:
+            if q[k] is None or q[k].grad is None:
+                continue
+            gk = q[k].grad.float().cpu()
+            if k in ("A", "D", "init"):
+                acc[k] += gk
+            else:
+                acc[k][:, sl] = gk
+    for k in base:
+        got, want = p[k].grad.float().cpu(), acc[k]
+        scale = float(want.abs().max()) + 1e-6
+        tol = dict(rtol=1e-3, atol=1e-4 * scale) if dtype == torch.float32 else dict(rtol=5e-2, atol=3e-2 * scale)
+        torch.testing.assert_close(got, want, **tol, msg=lambda m, k=k: f"gradient of {k}: {m}")
 
 
 def test_combined_varlen_vector():
