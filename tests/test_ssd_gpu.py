@@ -283,7 +283,8 @@ def test_packed_sequences_match_the_oracle_and_separate_runs(Q, lens, dtype, P):
         torch.testing.assert_close(vs[k].cpu(), fk[0].cpu(), **stol)
 
 
-@pytest.mark.parametrize("Q,lens,N", [(64, [100, 28, 64, 64], 64), (128, [300, 1, 83, 128], 128), (64, [64, 64, 64, 64], 64)])
+@pytest.mark.parametrize("Q,lens,N", [(64, [100, 28, 64, 64], 64), (128, [300, 1, 83, 128], 128), (64, [64, 64, 64, 64], 64),
+                                      (64, [1] * 64 + [3] * 21 + [1, 64], 64), (256, [1] * 256 + [200, 56], 128)])
 def test_packed_sequences_on_the_one_pass_kernel(Q, lens, N):
     """seq_idx alone (no per-sequence end states asked for) stays on the one-pass kernel, which separates the
     sequences by an extra decay of 2^-64 at every first step: against the float64 oracle, and against the
