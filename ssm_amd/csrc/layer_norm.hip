@@ -369,8 +369,9 @@ __global__ __launch_bounds__(LN_THREADS) void norm_bwd_kernel(const NormParams p
     for (int i = 0; i < VEC; ++i) dw[k][i] = db[k][i] = 0.0f;
   }
   const bool has_add = p.res && p.prenorm;
-  // typed reads of an absent residual go to memory of the same element type and are dropped
-  const void *resp = has_add ? p.res : (p.dres ? (const void *)p.dres : p.x);
+  // typed reads of a residual that is absent (or not added: post-norm) go to memory of the same element type
+  // and extent and are dropped: the residual itself if there is one, else dresidual, else x (then RT = XT)
+  const void *resp = p.res ? p.res : (p.dres ? (const void *)p.dres : p.x);
   const float *meanp = p.is_rms ? p.rstd : p.mean;
   for (int row = gw; row < p.rows; row += nwaves) {
     const size_t base = (size_t)row * H;

@@ -134,3 +134,22 @@ def test_config4_layer_shape_bf16():
     yr, ror = O.fused_layer_norm_with_residual(x[:, sl], w, None, residual=r[:, sl], is_rms=True)
     torch.testing.assert_close(y[:, sl].float().cpu(), yr.float(), **HALF_TOL)
     torch.testing.assert_close(ro[:, sl].cpu(), ror, **FP32_TOL)
+
+
+@pytest.mark.parametrize("is_rms", [True, False])
+def test_postnorm_backward_with_a_residual_that_needs_no_gradient(is_rms):
+    """bf16 x, float32 residual added after the norm, gradient asked for x and the weight only: the typed
+    backward reads its stand-in for the unused residual from the residual itself (same type and extent)."""
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(3, 37, 768, generator=g).to(torch.bfloat16)
+    r = torch.randn(3, 37, 768, generator=g)
+    w = torch.randn(768, generator=g)
+    gy = torch.randn(3, 37, 768, generator=g).to(torch.bfloat16)
+    xg, wg = x.clone().cuda().requires_grad_(True), w.clone().cuda().requires_grad_(True)
+    y = _ops().fused_layer_norm(xg, wg, None, residual=r.cuda(), is_rms=is_rms, prenorm=False)
+    y.backward(gy.cuda())
+    xr, wr = x.clone().float().requires_grad_(True), w.clone().requires_grad_(True)
+    yr = O.fused_layer_norm(xr, wr, None, residual=r, is_rms=is_rms, prenorm=False)
+    yr.backward(gy.float())
+    torch.testing.assert_close(xg.grad.float().cpu(), xr.grad, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(wg.grad.cpu(), wr.grad, rtol=2e-2, atol=2e-2 * float(wr.grad.abs().max()))
