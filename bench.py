@@ -118,10 +118,18 @@ def bench_conv(dtype=torch.bfloat16, batch=8, chans=1536, length=2048, width=4):
     fwd_us = _time_us(lambda i: ops._conv_forward(xs[i % 3], w, b, "silu"))
     bwd_us = _time_us(lambda i: ops._conv_backward(go, xs[i % 3], w, b, "silu"))
     fb, bb = 2 * elt * batch * chans * length, 3 * elt * batch * chans * length
+    # the same tensor channels last, (B, L, C): the layout of the Mamba-2 block
+    xl = [x.transpose(1, 2).contiguous() for x in xs]
+    gl = go.transpose(1, 2).contiguous()
+    cl_fwd_us = _time_us(lambda i: ops._conv_forward(xl[i % 3], w, b, "silu"))
+    cl_bwd_us = _time_us(lambda i: ops._conv_backward(gl, xl[i % 3], w, b, "silu"))
     return {"fwd_us": round(fwd_us, 1), "fwd_GBps": round(fb / fwd_us / 1e3, 1),
             "fwd_frac_hbm": round(fb / fwd_us / 1e3 / HBM_PEAK_GBPS, 4),
             "bwd_us": round(bwd_us, 1), "bwd_GBps": round(bb / bwd_us / 1e3, 1),
-            "bwd_frac_hbm": round(bb / bwd_us / 1e3 / HBM_PEAK_GBPS, 4)}
+            "bwd_frac_hbm": round(bb / bwd_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "channels_last_fwd_us": round(cl_fwd_us, 1), "channels_last_bwd_us": round(cl_bwd_us, 1),
+            "channels_last_fwd_frac_hbm": round(fb / cl_fwd_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "channels_last_bwd_frac_hbm": round(bb / cl_bwd_us / 1e3 / HBM_PEAK_GBPS, 4)}
 
 
 def bench_norm(batch=16, length=2048, hidden=768):
