@@ -1,13 +1,19 @@
 // C-ABI entry point of the forward selective scan: argument validation and
 // kernel selection.  The kernels live in scan_fwd_kernel.hpp and are
 // instantiated per activation dtype in scan_fwd_{f32,bf16,f16}.hip.
-#include "scan_fwd_kernel.hpp"
+#include "scan_fwd_fast.hpp"
 
 namespace ssm {
 
 extern template int scan_fwd_dispatch<float>(const ScanFwdParams &, int, int, hipStream_t);
 extern template int scan_fwd_dispatch<bf16_t>(const ScanFwdParams &, int, int, hipStream_t);
 extern template int scan_fwd_dispatch<f16_t>(const ScanFwdParams &, int, int, hipStream_t);
+
+extern template int scan_fwd_fast_dispatch<float, float>(const ScanFwdParams &, int, hipStream_t);
+extern template int scan_fwd_fast_dispatch<bf16_t, bf16_t>(const ScanFwdParams &, int, hipStream_t);
+extern template int scan_fwd_fast_dispatch<bf16_t, float>(const ScanFwdParams &, int, hipStream_t);
+extern template int scan_fwd_fast_dispatch<f16_t, f16_t>(const ScanFwdParams &, int, hipStream_t);
+extern template int scan_fwd_fast_dispatch<f16_t, float>(const ScanFwdParams &, int, hipStream_t);
 
 static bool valid_kind(int k) { return k == SSM_PROJ_DN || k == SSM_PROJ_BDN || k == SSM_PROJ_BGNL; }
 
@@ -68,6 +74,40 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   // Two channels per wave (tune 1616) pay off once the grid still fills every CU twice.
   const bool pair_ok = bvary && cvary && a->nstate <= 16 && per_b % 16 == 0 && per_c % 16 == 0;
   int tune = a->tune_items;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+
+  // The specialised kernel: time-varying B and C of one element type (that of the activations, or fp32), at most
+  // 16 states, aligned rows of whole 16-step runs.  tune_items 100000 + v asks for its variant v.
+  const bool fast_ok = bvary && cvary && a->nstate <= FAST_N && p.vec_ok && a->seqlen % 16 == 0 &&
+                       aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs) &&
+                       (a->bc_dtype == a->io_dtype || a->bc_dtype == SSM_F32);
+  if (tune == 0 && fast_ok && a->seqlen > 256) {
+    // The variant whose workgroups (48, 24 or 8 channels of one group) still give every CU its share:
+    // two rows per wave with 16-step runs where 256 such workgroups exist, else 8-step runs at six waves
+    // per SIMD, else the smallest workgroup.
+    const size_t total = (size_t)a->batch * a->dim;
+    const int pref[3] = {22121, 12121, 11082};
+    int pick = 0;
+    for (int i = 0; i < 3 && !pick; ++i) {
+      const int per_wg = scan_fwd_fast_rows(pref[i]);
+      if (per_b % per_wg == 0 && per_c % per_wg == 0 && (total / per_wg >= 256 || i == 2)) pick = pref[i];
+    }
+    if (pick) tune = 100000 + pick;
+  }
+  if (tune >= 100000) {
+    SSM_REQUIRE(fast_ok, SSM_ERR_BAD_KIND, "ssm_scan_fwd: tune_items %d needs the shape of the specialised kernel", tune);
+    const int v = tune - 100000, per_wg = scan_fwd_fast_rows(v);
+    SSM_REQUIRE(per_wg > 0 && per_b % per_wg == 0 && per_c % per_wg == 0, SSM_ERR_BAD_KIND,
+                "ssm_scan_fwd: variant %d takes %d channels per workgroup, which must divide a group", v, per_wg);
+    const bool bc32 = a->bc_dtype == SSM_F32;
+    switch (a->io_dtype) {
+      case SSM_F32: return scan_fwd_fast_dispatch<float, float>(p, v, stream);
+      case SSM_BF16: return bc32 ? scan_fwd_fast_dispatch<bf16_t, float>(p, v, stream)
+                                 : scan_fwd_fast_dispatch<bf16_t, bf16_t>(p, v, stream);
+      default: return bc32 ? scan_fwd_fast_dispatch<f16_t, float>(p, v, stream)
+                           : scan_fwd_fast_dispatch<f16_t, f16_t>(p, v, stream);
+    }
+  }
   if (tune == 0) {
     if (a->seqlen <= 256 && !a->chunk_states) tune = 408;
     else tune = a->nstate > 8 ? 816 : 808;
@@ -101,7 +141,6 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
     SSM_REQUIRE(steps_per_lane * WAVE == ssm_scan_chunk_len(), SSM_ERR_BAD_KIND,
                 "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (tune_items 808, 816 or 1616)",
                 ssm_scan_chunk_len());
-  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   switch (a->io_dtype) {
     case SSM_F32: return scan_fwd_dispatch<float>(p, tune, rows, stream);
     case SSM_BF16: return scan_fwd_dispatch<bf16_t>(p, tune, rows, stream);

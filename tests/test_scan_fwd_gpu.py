@@ -216,6 +216,52 @@ def test_several_channels_per_wave_match_oracle(items, dim):
     torch.testing.assert_close(h.float().cpu(), hr.float(), rtol=2e-2, atol=2e-2)
 
 
+FAST_VARIANTS = [(13082, 24), (12121, 24), (11082, 8), (22121, 48), (21081, 16)]
+
+
+@pytest.mark.parametrize("variant,rows", FAST_VARIANTS)
+@pytest.mark.parametrize("length,nstate", [(1520, 16), (512, 16), (48, 5), (1040, 9)])
+def test_specialised_kernel_variants_match_oracle(variant, rows, length, nstate):
+    """Every variant of the kernel for time-varying grouped B/C with at most 16 states (8- or 16-step runs per
+    lane, one or two rows per wave at once): whole and ragged last chunks, fewer than 16 states, two groups,
+    state hand-over between chunks, last_state."""
+    from ssm_amd.ops import _scan_forward
+    inp = make_inputs(variant + length, 2, 2 * rows, length, nstate, groups=2)
+    yr, hr = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"],
+                              z=inp["z"], dt_bias=inp["dt_bias"], softplus=True, return_last_state=True)
+    y, h = _scan_forward(dev(inp["u"]), dev(inp["delta"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]),
+                         dev(inp["D"]), dev(inp["z"]), dev(inp["dt_bias"]), True, True,
+                         tune_items=100000 + variant)
+    torch.testing.assert_close(y.cpu(), yr, **FP32_TOL)
+    torch.testing.assert_close(h.cpu(), hr, **FP32_TOL)
+
+
+@pytest.mark.parametrize("variant,rows", FAST_VARIANTS)
+@pytest.mark.parametrize("dtype,bc_dtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                            (torch.float16, torch.float16)])
+def test_specialised_kernel_half_types_and_options(variant, rows, dtype, bc_dtype):
+    """16-bit activations with projections of the same type or fp32; no gate, no skip, no bias, no softplus."""
+    from ssm_amd.ops import _scan_forward
+    inp = make_inputs(variant, 1, rows, 1072, 16, dtype=dtype, bc_dtype=bc_dtype, use_D=False, use_z=False,
+                      use_bias=False)
+    inp["delta"] = (0.05 * torch.rand(1, rows, 1072)).to(dtype)
+    yr, hr = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], softplus=False,
+                              return_last_state=True)
+    y, h = _scan_forward(dev(inp["u"]), dev(inp["delta"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]),
+                         None, None, None, False, True, tune_items=100000 + variant)
+    torch.testing.assert_close(y.float().cpu(), yr.float(), **HALF_TOL)
+    torch.testing.assert_close(h.float().cpu(), hr.float(), **HALF_TOL)
+
+
+def test_specialised_kernel_refuses_other_shapes():
+    """Asking for a variant on a call it does not cover is an error, not a silent fall-back."""
+    from ssm_amd.ops import _scan_forward
+    inp = make_inputs(3, 1, 24, 1000, 16)       # 1000 is not a multiple of 16
+    with pytest.raises(Exception):
+        _scan_forward(dev(inp["u"]), dev(inp["delta"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]),
+                      dev(inp["D"]), dev(inp["z"]), dev(inp["dt_bias"]), True, True, tune_items=112121)
+
+
 # ---------------------------------------------- benchmark shapes and properties
 
 def test_config0_fp32_full_size_against_oracle():
