@@ -591,6 +591,18 @@ typedef struct ssm_norm_bwd_args {
 size_t ssm_norm_bwd_workspace_bytes(int rows, int hidden);
 int ssm_norm_bwd(const ssm_norm_bwd_args *args, void *hip_stream);
 
+/* ssm_norm_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving or
+ * training loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The partial column
+ * sums go to a buffer of SSM_NORM_BWD_STATIC_BYTES that is part of the library's code object (each GPU the
+ * library runs on holds one until the process ends) instead of `workspace`, whose two fields are ignored; the call
+ * allocates and frees nothing, and its results are bit-identical to ssm_norm_bwd's.  Calls whose partial sums
+ * do not fit -- min(1024, ceil(rows / 4)) x 2 x hidden floats for hidden <= 8192 -- return SSM_ERR_TOO_LARGE.
+ * All calls on one GPU share the buffer: calls that overlap there (two streams, two threads) race; calls on one
+ * stream are ordered and safe.  The first call on a device looks the buffer's address up and must not happen
+ * while a stream is being captured. */
+#define SSM_NORM_BWD_STATIC_BYTES (8u << 20)
+int ssm_norm_bwd_static(const ssm_norm_bwd_args *args, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

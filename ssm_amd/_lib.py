@@ -261,6 +261,7 @@ ENTRY_POINTS = {
     "ssm_conv1d_update": Conv1dUpdateArgs,
     "ssm_norm_fwd": NormFwdArgs,
     "ssm_norm_bwd": NormBwdArgs,
+    "ssm_norm_bwd_static": NormBwdArgs,
 }
 # name -> (restype, argtypes) of the remaining exported functions
 PLAIN_SYMBOLS = {

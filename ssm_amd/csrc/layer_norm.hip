@@ -16,6 +16,8 @@
 // partials are written once and folded by a second kernel in a fixed order.
 #include "common.hpp"
 
+#include <mutex>
+
 #include <type_traits>
 
 namespace ssm {
@@ -642,22 +644,31 @@ extern "C" size_t ssm_norm_bwd_workspace_bytes(int rows, int hidden) {
   return (size_t)ssm::norm_bwd_grid(rows) * ssm::LN_WAVES * 2 * (size_t)hidden * sizeof(float);
 }
 
-extern "C" int ssm_norm_bwd(const ssm_norm_bwd_args *a, void *hip_stream) {
-  using namespace ssm;
-  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_norm_bwd: args is NULL");
-  int rc = norm_check("ssm_norm_bwd", a->x, a->weight, a->dx, a->rows, a->hidden, a->x_dtype, a->residual,
-                      a->residual_dtype);
+namespace ssm {
+
+// Partial column sums one call writes before the fold reads them: one per workgroup, or one per wave for rows
+// beyond 8192 columns.
+static size_t norm_bwd_partials(int rows, int hidden) {
+  const size_t grid = (size_t)norm_bwd_grid(rows);
+  return hidden <= 8192 ? grid : grid * LN_WAVES;
+}
+
+static int norm_bwd_check(const char *who, const ssm_norm_bwd_args *a) {
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "%s: args is NULL", who);
+  int rc = norm_check(who, a->x, a->weight, a->dx, a->rows, a->hidden, a->x_dtype, a->residual, a->residual_dtype);
   if (rc != SSM_OK) return rc;
   SSM_REQUIRE(a->dy && a->rstd && a->dweight && (a->is_rms || a->mean), SSM_ERR_NULL_POINTER,
-              "ssm_norm_bwd: dy, rstd, dweight (and mean for LayerNorm) are required");
-  SSM_REQUIRE(!a->dresidual || a->residual, SSM_ERR_NULL_POINTER, "ssm_norm_bwd: dresidual needs residual");
-  SSM_REQUIRE(a->workspace && a->workspace_bytes >= ssm_norm_bwd_workspace_bytes(a->rows, a->hidden),
-              SSM_ERR_WORKSPACE, "ssm_norm_bwd: workspace of %zu bytes required",
-              ssm_norm_bwd_workspace_bytes(a->rows, a->hidden));
+              "%s: dy, rstd, dweight (and mean for LayerNorm) are required", who);
+  SSM_REQUIRE(!a->dresidual || a->residual, SSM_ERR_NULL_POINTER, "%s: dresidual needs residual", who);
+  return SSM_OK;
+}
+
+// The launches of the backward pass; `partial` holds norm_bwd_partials() x 2 x hidden floats.
+static int norm_bwd_launch(const ssm_norm_bwd_args *a, float *partial, void *hip_stream) {
   NormParams p{};
   p.x = a->x; p.res = a->residual; p.dy = a->dy; p.w = a->weight; p.dx = a->dx; p.dres = a->dresidual;
   p.mean = const_cast<float *>(a->mean); p.rstd = const_cast<float *>(a->rstd);
-  p.partial = reinterpret_cast<float *>(a->workspace);
+  p.partial = partial;
   p.rows = a->rows; p.hidden = a->hidden;
   p.x_dtype = a->x_dtype; p.res_dtype = a->residual_dtype;
   p.is_rms = a->is_rms ? 1 : 0; p.prenorm = a->prenorm ? 1 : 0;
@@ -689,4 +700,63 @@ extern "C" int ssm_norm_bwd(const ssm_norm_bwd_args *a, void *hip_stream) {
                      p.partial, a->dweight, a->dbias, nparts, a->hidden);
   SSM_CHECK_LAUNCH("ssm_norm_bwd(fold)");
   return SSM_OK;
+}
+
+// Device memory for the partial sums of ssm_norm_bwd_static: part of the code object, so every GPU that the
+// library runs on holds its own copy from load to process end.  The name is a host-side handle only; the
+// address on the current device comes from hipGetSymbolAddress and is kept per device.
+constexpr size_t NORM_BWD_STATIC_FLOATS = SSM_NORM_BWD_STATIC_BYTES / sizeof(float);
+static __device__ __align__(256) float scratch[NORM_BWD_STATIC_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+static std::mutex scratch_lock;
+static float *scratch_on_device[MAX_DEVICES];
+
+static int norm_bwd_scratch(float **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    set_error("ssm_norm_bwd_static: no usable current device (%s)", e == hipSuccess ? "index out of range" : hipGetErrorString(e));
+    return SSM_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (!scratch_on_device[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      set_error("ssm_norm_bwd_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return SSM_ERR_LAUNCH;
+    }
+    scratch_on_device[dev] = reinterpret_cast<float *>(ptr);
+  }
+  *out = scratch_on_device[dev];
+  return SSM_OK;
+}
+
+}  // namespace ssm
+
+extern "C" int ssm_norm_bwd(const ssm_norm_bwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  const int rc = norm_bwd_check("ssm_norm_bwd", a);
+  if (rc != SSM_OK) return rc;
+  SSM_REQUIRE(a->workspace && a->workspace_bytes >= ssm_norm_bwd_workspace_bytes(a->rows, a->hidden),
+              SSM_ERR_WORKSPACE, "ssm_norm_bwd: workspace of %zu bytes required",
+              ssm_norm_bwd_workspace_bytes(a->rows, a->hidden));
+  return norm_bwd_launch(a, reinterpret_cast<float *>(a->workspace), hip_stream);
+}
+
+extern "C" int ssm_norm_bwd_static(const ssm_norm_bwd_args *a, void *hip_stream) {
+  using namespace ssm;
+  int rc = norm_bwd_check("ssm_norm_bwd_static", a);
+  if (rc != SSM_OK) return rc;
+  const size_t need = norm_bwd_partials(a->rows, a->hidden) * 2 * (size_t)a->hidden;
+  SSM_REQUIRE(need <= NORM_BWD_STATIC_FLOATS, SSM_ERR_TOO_LARGE,
+              "ssm_norm_bwd_static: rows=%d hidden=%d need %zu bytes of partial sums, the built-in buffer holds %zu; "
+              "use ssm_norm_bwd with a workspace", a->rows, a->hidden, need * sizeof(float),
+              (size_t)SSM_NORM_BWD_STATIC_BYTES);
+  float *partial = nullptr;
+  rc = norm_bwd_scratch(&partial);
+  if (rc != SSM_OK) return rc;
+  return norm_bwd_launch(a, partial, hip_stream);
 }

@@ -702,8 +702,29 @@ def _norm_forward(x, weight, bias, residual, is_rms, eps, prenorm, residual_in_f
     return y, res_out, mean, rstd
 
 
-def _norm_backward(grad_out, x, weight, residual, mean, rstd, is_rms, prenorm, want_dbias, want_dres):
+def _norm_backward(grad_out, x, weight, residual, mean, rstd, is_rms, prenorm, want_dbias, want_dres,
+                   out=None):
+    """``ssm_norm_bwd``.  With ``out = (dx, dres, dw, db)`` (preallocated, contiguous; ``None`` where a
+    gradient is not wanted) the call goes to ``ssm_norm_bwd_static`` instead and allocates nothing on
+    the device: inputs must then already be contiguous and ``weight`` float32."""
     rows, hidden = K.check_norm(x, weight, None, residual)
+    if out is not None:
+        dev = K.require_gpu(x, weight, residual, grad_out)
+        dx, dres, dw, db = out
+        for t in (x, grad_out, residual, weight):
+            if t is not None and not t.is_contiguous():
+                raise ValueError("the allocation-free norm backward takes contiguous tensors")
+        if weight.dtype != torch.float32 or grad_out.dtype != x.dtype:
+            raise ValueError("the allocation-free norm backward takes a float32 weight and grad_out of x's dtype")
+        args = _lib.NormBwdArgs(
+            x=_lib.ptr(x), residual=_lib.ptr(residual), dy=_lib.ptr(grad_out), weight=_lib.ptr(weight),
+            mean=_lib.ptr(mean), rstd=_lib.ptr(rstd), dx=_lib.ptr(dx), dresidual=_lib.ptr(dres),
+            dweight=_lib.ptr(dw), dbias=_lib.ptr(db), workspace=None, workspace_bytes=0, rows=rows,
+            hidden=hidden, x_dtype=_lib.dtype_enum(x.dtype),
+            residual_dtype=_lib.dtype_enum(residual.dtype) if residual is not None else 0,
+            is_rms=int(bool(is_rms)), prenorm=int(bool(prenorm)))
+        _lib.call("ssm_norm_bwd_static", args, dev)
+        return dx, dres, dw, db
     dev = K.require_gpu(x, weight, residual, grad_out)
     xc, gc = K.cast_c(x, x.dtype), K.cast_c(grad_out, x.dtype)
     rc = K.cast_c(residual, residual.dtype) if residual is not None else None
