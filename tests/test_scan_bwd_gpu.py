@@ -100,6 +100,26 @@ def test_fp32_gradients_match_oracle(shape, kinds):
     compare(got, want, rtol=1e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("shape,with_last", [((2, 32, 1024, 16), False), ((3, 6, 513, 16), True), ((1, 48, 2048, 16), False)],
+                         ids=lambda v: str(v).replace(" ", ""))
+def test_fp32_gradient_error_is_that_of_fp32_arithmetic(shape, with_last):
+    """Which of two float32 results is right is settled by float64: for each of the eight gradients the kernel's
+    error against the float64 oracle must not exceed four times the float32 oracle's own error against it (plus
+    one part in a million of the gradient's size, for gradients the float32 oracle happens to hit exactly)."""
+    b, d, l, n = shape
+    inp = make_inputs(sum(shape) + 1, b, d, l, n)
+    got, want32 = grads_both(inp, with_last=with_last)
+    _, want64 = grads_both(inp, with_last=with_last, acc=torch.float64)
+    for k in NAMES:
+        if want64[k] is None:
+            continue
+        w64 = want64[k].double()
+        ours = float((got[k].double() - w64).abs().max())
+        theirs = float((want32[k].double() - w64).abs().max())
+        floor = 1e-6 * float(w64.abs().max())
+        assert ours <= 4.0 * theirs + floor, f"grad {k}: kernel error {ours:.3e}, float32 oracle error {theirs:.3e}"
+
+
 @pytest.mark.parametrize("groups,dim", [(1, 8), (2, 8), (8, 8), (3, 6), (2, 96)])
 def test_groups(groups, dim):
     inp = make_inputs(4, 2, dim, 200, 16, groups=groups)
