@@ -23,10 +23,6 @@
 
 #include <type_traits>
 #include <utility>
-#ifdef BW_TIMING
-#include <cstdio>
-#include <vector>
-#endif
 
 namespace ssm {
 
@@ -52,9 +48,6 @@ struct ScanBwdParams {
   int rows_per_wg;       // channels walked by one workgroup (all in one B group and one C group)
   int nblk;              // workgroups per batch row = dim / rows_per_wg
   int bc_vec_ok;
-#ifdef BW_TIMING
-  long long *times;      // [workgroup][wave][12] clock counts per phase (debug builds)
-#endif
 };
 
 // Stage one [BW_MAX_N][BW_T] slab of a time-varying projection (fp32, transposed
@@ -243,12 +236,7 @@ __global__ __launch_bounds__(BW_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
   const io_t *zsrc = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.u);
 
   const int rev_lane = WAVE - 1 - lane;
-#ifdef BW_TIMING
-  long long tacc[12] = {0}; long long tprev = __builtin_amdgcn_s_memtime();
-#define BT(i) { const long long tn = __builtin_amdgcn_s_memtime(); tacc[i] += tn - tprev; tprev = tn; }
-#else
 #define BT(i)
-#endif
 
   for (int c = nchunks - 1; c >= 0; --c) {
     const int t0 = c * T;
@@ -581,10 +569,6 @@ __global__ __launch_bounds__(BW_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
     p.dD_rows[row] = sumD[r];
     p.dbias_rows[row] = sumb[r];
   }
-#ifdef BW_TIMING
-  if (lane == 0)
-    for (int i = 0; i < 12; ++i) p.times[((size_t)blockIdx.x * BW_WAVES + wave) * 12 + i] = tacc[i];
-#endif
 #undef BT
 }
 
@@ -828,12 +812,6 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
   p.rows_per_wg = pl.rows_per_wg; p.nblk = pl.nblk;
   p.bc_vec_ok = a->seqlen % 4 == 0 && aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs);
 
-#ifdef BW_TIMING
-  static long long *tbuf = nullptr;
-  const size_t tcount = (size_t)a->batch * pl.nblk * BW_WAVES * 12;
-  if (!tbuf) (void)hipMalloc(&tbuf, (size_t)1 << 26);
-  p.times = tbuf;
-#endif
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   int rc;
   switch (a->io_dtype) {
@@ -842,19 +820,6 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
     default: rc = launch_bwd<f16_t>(p, s); break;
   }
   if (rc != SSM_OK) return rc;
-#ifdef BW_TIMING
-  {
-    (void)hipDeviceSynchronize();
-    std::vector<long long> host(tcount);
-    (void)hipMemcpy(host.data(), tbuf, tcount * 8, hipMemcpyDeviceToHost);
-    const char *names[12] = {"chunk tail", "chunk barrier", "tiles+finish prev", "elementwise", "barrier 1", "load+fold", "scan fwd", "F: LDS sums", "replay..gathers", "F: stores", "final+part+sums", "barrier 2"};
-    double tot = 0; double ph[12] = {0};
-    for (size_t i = 0; i < tcount; ++i) { ph[i % 12] += (double)host[i]; tot += (double)host[i]; }
-    const double nw = (double)tcount / 12;
-    fprintf(stderr, "scan_bwd timing: %.0f counts per wave\n", tot / nw);
-    for (int i = 0; i < 12; ++i) fprintf(stderr, "  %-18s %9.0f  %5.1f%%\n", names[i], ph[i] / nw, 100.0 * ph[i] / tot);
-  }
-#endif
 
   const int Bn = a->batch, D = a->dim, N = a->nstate, L = a->seqlen;
   // dA (D,N), dD (D,), dbias (D,): fold over batch

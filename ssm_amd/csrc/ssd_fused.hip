@@ -39,9 +39,6 @@ struct SsdFusedParams {
   const float *Dk, *init;
   float *final_states;
   int batch, len, heads, groups, nstate, chunk, nchunks, d_per_p;
-#ifdef FH_TIMING
-  long long *times;
-#endif
 };
 
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
@@ -448,12 +445,6 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     f2 = buf_load16(rf, st.vf, FH_C_OFF(0, lbF, 1));
     f3 = buf_load16(rf, st.vf, FH_C_OFF(0, lbS, 1));
   }
-#ifdef FH_TIMING
-  long long tacc[10] = {0}; long long tprev = __builtin_amdgcn_s_memtime();
-#define FH_T(i) { const long long tn = __builtin_amdgcn_s_memtime(); tacc[i] += tn - tprev; tprev = tn; }
-#else
-#define FH_T(i)
-#endif
 
   for (int c = 0; c < nc; ++c) {
     // LDS addresses are rebuilt from the lane number in every chunk: kept across chunks they would
@@ -478,7 +469,6 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     st.off_bt = f_bt + (((unit * KS) * NT + min(nt_s, NT - 1)) << 10);
 
     __syncthreads();                       // previous chunk: every read of the tiles and the output staging are over
-    FH_T(0)
     if (sact && carry) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -513,9 +503,7 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
         *reinterpret_cast<bf16x8_t *>(xr + at) = colr;
       }
     }
-    FH_T(1)
     __syncthreads();
-    FH_T(2)
 
     // ---- carried state: acc[p][l] = sum_n S[p][n] C[l][n] for both row blocks
     if (yact && carry) {
@@ -558,7 +546,6 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
       stream_pair(st, 2, f2, f3);
       stream_pair(st, 4, f0, f1);
     }
-    FH_T(3)
 
     // ---- the two row blocks.  Pair q of the stream lives in (f0, f1) if q is even, in (f2, f3) if odd:
     // the diagonal block of the first row block is pair lbF, that of the second pair NLB.
@@ -571,9 +558,7 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
         half_skip_term(accS, lbS, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
       }
     }
-    FH_T(4)
     __syncthreads();                       // every wave is past the carried state: its tile becomes the output staging
-    FH_T(5)
 
     // ---- state: S^T[n][p] <- S^T g_k + sum_{s in block k} B[s][n] x~[s][p], and the chunk's reads from
     // HBM: the gate operands of this wave's rows (in the row-major order of the output pass) and the next
@@ -640,7 +625,6 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
 #undef FH_REQUEST_HBM
 #undef FH_STEP_C
 #undef FH_SCALE_C
-    FH_T(6)
     // the gate operands are first looked at here: without this the scheduler starts converting them in
     // the middle of the state update, which then waits for the reads from HBM after all
     if (HAS_Z) asm volatile("" : "+v"(zF[0]), "+v"(zF[1]), "+v"(zS[0]), "+v"(zS[1]) : : "memory");
@@ -679,7 +663,6 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
         wave_lds_sync();
       }
     }
-    FH_T(7)
   }
 #undef FH_REQUEST_CHUNK
 #undef FH_C_OFF
@@ -690,11 +673,6 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     for (int q = 0; q < 4; ++q)
       *reinterpret_cast<float4 *>(fp + 8 * q + 4 * g2) = make_float4(S[4 * q], S[4 * q + 1], S[4 * q + 2], S[4 * q + 3]);
   }
-#ifdef FH_TIMING
-  if (lane == 0)
-    for (int i = 0; i < 10; ++i) p.times[((size_t)vid * 4 + wave) * 10 + i] = tacc[i];
-#endif
-#undef FH_T
 }
 
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -714,9 +692,6 @@ static FusedLayout fused_layout(const SsdDims &d) {
   f.Cblk = at; at += bc;
   f.Btblk = at; at += bc;
   f.CBblk = at; at += cb;
-#ifdef FH_TIMING
-  at += (size_t)d.batch * d.heads * 2 * 4 * 10 * sizeof(long long);   // per-wave phase clocks behind everything else
-#endif
   f.total = at;
   return f;
 }
@@ -814,9 +789,6 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   fp.Dk = a->Dskip; fp.init = a->initial_states; fp.final_states = a->final_states;
   fp.batch = d.batch; fp.len = d.len; fp.heads = d.heads; fp.groups = d.groups; fp.nstate = d.nstate; fp.chunk = d.chunk;
   fp.nchunks = d.nchunks; fp.d_per_p = a->d_per_p ? 1 : 0;
-#ifdef FH_TIMING
-  fp.times = reinterpret_cast<long long *>(ws + lay.CBblk + align_up((size_t)d.batch * d.nchunks * d.groups * d.chunk * d.chunk * 2));
-#endif
   const int dmode = !a->Dskip ? 0 : (a->d_per_p ? 2 : 1);
   const unsigned grid = (unsigned)(d.batch * d.heads) * 2;
 #define SSM_LAUNCH_FUSED(QQ, NN, DM, HZ)                                                           \
