@@ -317,6 +317,25 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
     return out
 
 
+_DECAYING = {}        # (data_ptr, version, numel) of an A tensor -> all(A <= 0), so that a persistent parameter is read once
+
+
+def _is_decaying(A):
+    """``all(A <= 0)``: what the one-pass kernel assumes (it bounds each factor of a decay by 1; with a growing
+    state its results are wrong, while the five kernels keep the upstream kernels' behaviour there).  Reading the
+    answer costs a device synchronisation, so it is remembered per tensor (address and version) and not looked up
+    at all while a stream is being captured, where the caller's word (``fused=True``) or the default is taken."""
+    if torch.cuda.is_current_stream_capturing():
+        return True
+    key = (A.data_ptr(), A._version, A.numel())
+    hit = _DECAYING.get(key)
+    if hit is None:
+        if len(_DECAYING) > 4096:
+            _DECAYING.clear()
+        hit = _DECAYING[key] = bool((A.detach() <= 0).all())
+    return hit
+
+
 def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
     """Whether the one-pass kernel covers this call (bf16 tensors on the GPU and a
     shape ``ssm_ssd_combined_supported`` accepts)."""
@@ -389,10 +408,16 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         return_final_states: Also return the state after the last token.
         states_dtype: dtype of the per-chunk states kept in HBM between the kernels
             (default: ``x.dtype``; the recurrence itself accumulates in float32).
-        fused: ``None`` picks the one-pass kernel when it applies, ``False`` never
-            uses it, ``True`` requires it (``ValueError`` if the call is not covered).
+        fused: ``None`` picks the one-pass kernel when it applies and ``A <= 0`` everywhere (looked up
+            once per ``A`` tensor: a device synchronisation the first time a tensor is seen), ``False``
+            never uses it, ``True`` requires it (``ValueError`` if the call is not covered) and takes
+            the caller's word that ``A <= 0``: with a growing state its results are wrong.
         seq_idx: Optional ``(B, L)`` int sequence ids of a packed batch (ids start at 0):
-            no state and no product crosses from one sequence into the next.
+            no state and no product crosses from one sequence into the next.  The five kernels
+            mask exactly.  The one-pass kernel (picked for bfloat16 calls it covers) and the
+            backward separate sequences by an extra decay of ``2**-64`` at every first step
+            instead: what crosses a boundary is scaled by 5e-20, which is exact in effect for
+            the decaying ``A <= 0`` both require.
         cu_seqlens: Optional ``(nseq + 1,)`` sequence boundaries of a packed batch row
             (batch size 1), only used for ``return_varlen_states``.
         return_varlen_states: Also return the state at the last step of every sequence,
@@ -414,7 +439,10 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         if dt_softplus:
             dt_fill = torch.full_like(dt[:, :1], float("-inf")).expand(-1, pad, -1)     # softplus(-inf) = 0
         elif dt_bias is not None:
-            dt_fill = (-dt_bias.detach().to(dt.dtype))[None, None].expand(dt.shape[0], pad, -1)
+            # raw step + bias must be exactly zero: in float32 (a 16-bit -bias would leave bias - round(bias), a
+            # small step that lets the state decay over the padding)
+            dt = dt.to(torch.float32)
+            dt_fill = (-dt_bias.detach().to(torch.float32))[None, None].expand(dt.shape[0], pad, -1)
         else:
             dt_fill = torch.zeros_like(dt[:, :1]).expand(-1, pad, -1)
         sp = None
@@ -480,6 +508,8 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
         return outs[0] if len(outs) == 1 else tuple(outs)
     can_fuse = not force_generic and fused is not False and not return_varlen_states and \
         _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
+    if can_fuse and fused is None and not _is_decaying(A):
+        can_fuse = False          # a growing state: only the five kernels follow the upstream kernels there
     _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "
           "chunk in {64,128,256}, nstate in {64,128} and seqlen % chunk == 0.")
     if can_fuse:

@@ -567,3 +567,48 @@ def test_config3_shape_bf16():
     assert float(excess.max()) < 8e-2, f"worst (batch, head) pair: {excess.max():.3e} of the rms at {excess.argmax()}"
     assert float(diff.mean()) < 3e-3 * rms
     half_close(fin, fin5, "final states, one pass against five kernels, all heads")
+
+
+def test_ragged_length_with_16_bit_steps_and_a_bias_keeps_the_final_state():
+    """bf16 raw steps, a bias, no softplus, a ragged length: the padded steps must have size exactly zero, or the
+    final state decays over the padding (A is large here so that even a step of 1e-3 would show)."""
+    b, l, h, p, g, n, Q = 1, 300, 2, 64, 1, 64, 256
+    inp = make(21, b, l, h, p, g, n, dtype=torch.bfloat16, use_init=True)
+    gen = torch.Generator().manual_seed(2)
+    bias = torch.rand(h, generator=gen) * 0.5 + 0.1234567
+    raw = (inp["dt"].float() * 0.2).to(torch.bfloat16)
+    A = -torch.full((h,), 40.0)
+    y, fin = ssd().ssd_combined(cu(inp["x"]), cu(raw), cu(A), cu(inp["B"]), cu(inp["C"]), Q, dt_bias=cu(bias),
+                                initial_states=cu(inp["init"]), dt_softplus=False, return_final_states=True)
+    y64, f64 = S.ssd_sequential(inp["x"], raw, A, inp["B"], inp["C"], dt_bias=bias, dt_softplus=False,
+                                initial_states=inp["init"])
+    half_close(y, y64, "y")
+    half_close(fin, f64, "final states")
+
+
+def test_growing_states_are_kept_off_the_one_pass_kernel():
+    """Positive A: the one-pass kernel bounds every factor of a decay by 1 and would be wrong, so the default
+    path must not pick it; the five kernels follow the upstream kernels (decay inside a chunk clamped to 1),
+    packed or not."""
+    b, l, h, p, g, n, Q = 1, 512, 2, 64, 1, 64, 128
+    inp = make(31, b, l, h, p, g, n, dtype=torch.bfloat16, use_init=True)
+    A = torch.full((h,), 0.25)
+    dt = torch.full((b, l, h), 0.03)
+    seq_idx = torch.zeros(b, l, dtype=torch.int32)
+    seq_idx[:, 200:] = 1
+    seq_idx[:, 333:] = 2
+    from ssm_amd import _lib
+    for sid in (None, seq_idx):
+        _lib.load().ssm_ssd_mfma_launches()
+        y, fin = ssd().ssd_combined(cu(inp["x"]), cu(dt), cu(A), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]), z=cu(inp["z"]),
+                                    initial_states=cu(inp["init"]), return_final_states=True, seq_idx=cu(sid),
+                                    states_dtype=torch.float32)
+        assert not (_lib.load().ssm_ssd_mfma_launches() & 8)
+        wy, wf = S.ssd_combined(inp["x"], dt, A, inp["B"], inp["C"], Q, D=inp["D"], z=inp["z"], initial_states=inp["init"],
+                                clamp_decay=True, seq_idx=sid)[:2]
+        half_close(y, wy, "y")
+        half_close(fin, wf, "final states")
+    # the same call with a decaying A does take the one-pass kernel
+    _lib.load().ssm_ssd_mfma_launches()
+    ssd().ssd_combined(cu(inp["x"]), cu(dt), cu(-A), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]), z=cu(inp["z"]))
+    assert _lib.load().ssm_ssd_mfma_launches() & 8
