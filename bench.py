@@ -34,6 +34,57 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 
 
+PROFILES = os.path.join(ROOT, "profiles")
+CLOCK_GHZ = 2.4            # MI355X peak engine clock
+SIMDS = 256 * 4
+
+
+def _profile_rows(name):
+    """Rows ``(kernel, counter, mean per dispatch)`` of a counter summary under profiles/ (the text
+    ``rocprofv3 --pmc`` runs of this file were condensed to), or [] when the file is missing."""
+    path = os.path.join(PROFILES, name)
+    rows = []
+    if not os.path.exists(path):
+        return rows
+    for line in open(path):
+        parts = line.rstrip("\n").rsplit(None, 3)
+        if len(parts) == 4 and parts[2].isdigit():
+            try:
+                rows.append((parts[0].strip(), parts[1], float(parts[3])))
+            except ValueError:
+                pass
+    return rows
+
+
+def headline_counters(kernel_substr="scan_fwd_fast_kernel"):
+    """HBM traffic and vector-ALU instruction count of one launch of the headline kernel, from the counter
+    summaries committed under profiles/ (``FETCH_SIZE`` and ``WRITE_SIZE`` in KiB, each scaled by what the same
+    counter read for the 256 MiB copy of ``--copy-calibration`` in the same run).  A summary taken with another
+    kernel than the one named here does not count: the figure is then ``None``."""
+    out = {"traffic": None, "valu_insts": None, "source": None}
+    fetch = _profile_rows("scan_fwd_bf16_headline_pmc_FETCH_SIZE.txt")
+    write = _profile_rows("scan_fwd_bf16_headline_pmc_WRITE_SIZE.txt")
+    sq = _profile_rows("scan_fwd_bf16_headline_pmc_SQ.txt")
+
+    def pick(rows, counter, sub):
+        for k, c, v in rows:
+            if c == counter and sub in k:
+                return k, v
+        return None, None
+
+    kf, f = pick(fetch, "FETCH_SIZE", kernel_substr)
+    kw, w = pick(write, "WRITE_SIZE", kernel_substr)
+    _, cf = pick(fetch, "FETCH_SIZE", "CUDAFunctorOnSelf_add")
+    _, cw = pick(write, "WRITE_SIZE", "CUDAFunctorOnSelf_add")
+    if None not in (f, w, cf, cw) and cf > 0 and cw > 0:
+        copy_kib = 256.0 * 1024.0
+        out["traffic"] = int(round((f * copy_kib / cf + w * copy_kib / cw) * 1024))
+        out["source"] = f"profiles/scan_fwd_bf16_headline_pmc_{{FETCH,WRITE}}_SIZE.txt ({kf})"
+    _, v = pick(sq, "SQ_INSTS_VALU", kernel_substr)
+    out["valu_insts"] = v
+    return out
+
+
 def _event_ms(fn, iters):
     """Average duration (ms) of ``fn``'s GPU work, one event pair per call, on the
     current stream (the stream the kernels are launched on)."""
@@ -50,8 +101,11 @@ def _event_ms(fn, iters):
     return sum(times) / len(times), times[len(times) // 2]
 
 
+SPIN_UP_LAUNCHES = 300
+
+
 def bench_scan_fwd(steps, warmup, dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nstate=16,
-                   nsets=4):
+                   nsets=4, spin_up=SPIN_UP_LAUNCHES):
     from ssm_amd import configs
     from ssm_amd.ops import ScanPlan
 
@@ -63,6 +117,11 @@ def bench_scan_fwd(steps, warmup, dtype=torch.bfloat16, batch=8, dim=1536, lengt
     elt = 2 if dtype != torch.float32 else 4
     nbytes = configs.scan_fwd_bytes(batch, dim, length, nstate, elt)
 
+    # The device takes some tens of milliseconds of work to reach its clocks after idling (the first hundred
+    # launches of a fresh process run up to 15 % slower): bring it there before the W warm-up steps.
+    for i in range(spin_up):
+        plans[i % nsets].run()
+    torch.cuda.synchronize()
     for i in range(warmup):
         plans[i % nsets].run()
     torch.cuda.synchronize()
@@ -338,6 +397,90 @@ def bench_model1(batch=8, prompt=2048, new_tokens=256):
                      "d_state 16, vocab 50280, bf16, random weights"}
 
 
+def bench_scan_facade(dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nstate=16):
+    """The headline call through the drop-in entry ``ops.selective_scan`` (validation, dtype normalisation and
+    output allocation inside the timed region) instead of a prepared plan: wall time per call over a queue of
+    calls, and the kernel's share of it."""
+    from ssm_amd import configs, ops
+    sets = [configs.to_device(configs.scan_inputs(batch, dim, length, nstate, dtype=dtype, seed=s)) for s in range(4)]
+
+    def call(i):
+        g = sets[i % 4]
+        return ops.selective_scan(g["u"], g["delta"], g["A"], g["B"], g["C"], D=g["D"], z=g["z"],
+                                  dt_bias=g["dt_bias"], softplus=True, return_last_state=True)
+    for i in range(5):
+        call(i)
+    torch.cuda.synchronize()
+    n = 50
+    t0 = time.perf_counter()
+    for i in range(n):
+        call(i)
+    host = (time.perf_counter() - t0) / n
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / n
+    return {"wall_us_per_call": round(wall * 1e6, 1), "host_us_per_call": round(host * 1e6, 1),
+            "note": "host time is what the Python entry costs per call; it overlaps the previous call's kernel"}
+
+
+def bench_scan_per_channel_bc(dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nstate=16):
+    """The shape the reference's Mamba1 module calls with (src/ssm/modules/mamba1.py:229-247): B and C as
+    (B, D, N, L), one group per channel, so the projections dominate the traffic."""
+    from ssm_amd import configs
+    from ssm_amd.ops import ScanPlan
+    g = configs.to_device(configs.scan_inputs(batch, dim, length, nstate, dtype=dtype, seed=0))
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    Bm = torch.randn(batch, dim, nstate, length, generator=gen, device="cuda", dtype=torch.float32).to(dtype)
+    Cm = torch.randn(batch, dim, nstate, length, generator=gen, device="cuda", dtype=torch.float32).to(dtype)
+    plan = ScanPlan(g["u"], g["delta"], g["A"], Bm, Cm, g["D"], g["z"], g["dt_bias"], True, True)
+    us = _time_us(lambda i: plan.run(), iters=10)
+    elt = 2 if dtype != torch.float32 else 4
+    nbytes = configs.scan_fwd_bytes(batch, dim, length, nstate, elt, groups=dim)
+    return {"kernel_us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
+            "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes,
+            "shape": "B, C (8, 1536, 16, 2048) bf16: one B/C group per channel"}
+
+
+VALU_KINDS = [
+    (0, "fp32 fma, 8 independent", 8), (1, "fp32 fma, dependent chain", 8), (2, "exp2", 8), (3, "log2", 8), (4, "rcp", 8),
+    (5, "exp2 and fma alternating", 8), (6, "scan state step: mul, exp2, mul, fma, fmac", 40),
+    (7, "the same with a move for exp2", 40), (8, "DPP multiply (quad broadcast)", 8),
+    (9, "DPP fmac / mul of a lane scan", 8), (10, "half-wave / row swaps", 8),
+    (11, "4 state steps + one fp32 16x16x4 matrix instruction", 21), (12, "8-byte LDS reads", 8),
+]
+
+
+def bench_valu(waves=(1, 2, 3, 4)):
+    """Issue rates of the vector ALU (``ssm_probe_valu``): shader clocks per wave instruction per SIMD, with one
+    workgroup per CU and 1 to 4 waves per SIMD."""
+    import ctypes
+    from ssm_amd import _lib
+    lib = _lib.load()
+    wgs, rounds = 256, 8
+    out = torch.empty(wgs * rounds * 1024, dtype=torch.float32, device="cuda")
+    clk = torch.zeros(2, dtype=torch.int64, device="cuda")
+    stream = _lib.stream_handle(out.device)
+    table = {}
+    for kind, name, per_iter in VALU_KINDS:
+        iters = 2048 if per_iter >= 20 else 4096
+        row = {}
+        for w in waves:
+            def go():
+                rc = lib.ssm_probe_valu(kind, w, wgs * rounds, iters, ctypes.c_void_p(out.data_ptr()),
+                                        ctypes.c_void_p(clk.data_ptr()), stream)
+                assert rc == 0, lib.ssm_amd_last_error()
+            go()
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record(); go(); e.record(); torch.cuda.synchronize()
+            ticks = clk.cpu()
+            mhz = float(ticks[0]) / (float(ticks[1]) / 100.0)
+            cycles = s.elapsed_time(e) * 1e3 * mhz
+            row[f"{w}_waves_per_simd"] = round(cycles / (rounds * w * iters * per_iter), 2)
+            row["clock_mhz"] = round(mhz)
+        table[name] = row
+    return table
+
+
 def cpu_baseline_scan(dtype=torch.bfloat16, dim=1536, length=2048, nstate=16, budget_s=15.0):
     """Time the CPU restatement of the reference's Python loop on a batch slice
     of the headline workload; returns GB/s of the same algorithmic bytes."""
@@ -360,7 +503,17 @@ def cpu_baseline_scan(dtype=torch.bfloat16, dim=1536, length=2048, nstate=16, bu
     times = [first] + [once() for _ in range(reps)]
     best = sorted(times)[len(times) // 2]
     nbytes = configs.scan_fwd_bytes(batch, dim, length, nstate, elt)
+    # configuration 0 at full size (B=1, D=512, L=2048, N=16, float32): the one case the reference publishes
+    # a time for (1012.9 ms on its authors' CPU, README.md:53 of the reference)
+    c0 = configs.scan_inputs(1, 512, 2048, 16, dtype=torch.float32, seed=0)
+    t0s = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ops_oracle.selective_scan(c0["u"], c0["delta"], c0["A"], c0["B"], c0["C"], D=c0["D"], z=c0["z"],
+                                  dt_bias=c0["dt_bias"], softplus=True, return_last_state=True)
+        t0s.append(time.perf_counter() - t0)
     return dict(value=nbytes / best / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                config0_ms=round(sorted(t0s)[1] * 1e3, 1), config0_reference_published_ms=1012.9,
                 sample=f"selective_scan fwd, batch slice B={batch} of the headline workload "
                        f"(D={dim}, L={length}, N={nstate}, {str(dtype).split('.')[-1]}), "
                        f"median of {len(times)} runs, {best * 1e3:.0f} ms each; "
@@ -379,7 +532,8 @@ def main():
                     help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
-                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1"],
+                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1", "valu",
+                             "scan_facade", "scan_per_channel_bc"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
     args = ap.parse_args()
@@ -405,13 +559,23 @@ def main():
     if args.only:
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
               "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model,
-              "model1": bench_model1}[args.only]
+              "model1": bench_model1, "valu": bench_valu, "scan_facade": bench_scan_facade,
+              "scan_per_channel_bc": bench_scan_per_channel_bc}[args.only]
         print(json.dumps({args.only: fn()}))
         return
 
     r = bench_scan_fwd(args.steps, args.warmup)
     value = r["bytes"] / r["wall_s"] / 1e9
     achieved = r["bytes"] / (r["kernel_ms"] * 1e-3) / 1e9
+    counters = headline_counters()
+    valu = None
+    if counters["valu_insts"]:
+        # vector-ALU instructions of one launch at the nominal 4 clocks each on 1024 SIMDs, against the kernel's time
+        busy_s = counters["valu_insts"] * 4.0 / (SIMDS * CLOCK_GHZ * 1e9)
+        valu = {"insts_per_launch": int(counters["valu_insts"]), "clocks_per_inst": 4, "clock_ghz": CLOCK_GHZ,
+                "simds": SIMDS, "frac": round(busy_s / (r["kernel_ms"] * 1e-3), 4),
+                "insts_per_state_step": round(counters["valu_insts"] * 64.0 / (8 * 1536 * 2048 * 16), 2),
+                "source": "profiles/scan_fwd_bf16_headline_pmc_SQ.txt"}
     line = {
         "metric": "selective_scan GB/s (%HBM peak)",
         "value": round(value, 2),
@@ -427,14 +591,16 @@ def main():
         "data": "synthetic",
         "config": {"workload": "selective_scan forward, B=8 D=1536 L=2048 N=16, bf16 activations, "
                                "fp32 state, G=1 time-varying B/C, D skip, z gate, dt_bias, softplus",
-                   "io_dtype": "bf16", "tokens_per_step": r["tokens"],
+                   "io_dtype": "bf16", "arithmetic": "fp32", "untimed_spin_up_launches": SPIN_UP_LAUNCHES,
+                   "tokens_per_step": r["tokens"],
                    "tokens_per_s": round(r["tokens"] / r["wall_s"], 1),
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": configs.scan_fwd_headline_traffic_bytes(),
-                     "kernel": "scan_fwd_kernel<bf16, 8>", "kernel_us": round(r["kernel_ms"] * 1e3, 2),
-                     "algorithmic_bytes": r["bytes"]},
+                     "traffic": counters["traffic"], "traffic_source": counters["source"],
+                     "kernel": "scan_fwd_fast_kernel<bf16, bf16, 32 lanes per row, 2 rows in turn, 12 waves>",
+                     "kernel_us": round(r["kernel_ms"] * 1e3, 2),
+                     "algorithmic_bytes": r["bytes"], "valu": valu},
     }
     if not args.no_extra:
         extra = {}
@@ -443,6 +609,8 @@ def main():
         extra["selective_scan_fwd_fp32_io"] = {
             "kernel_us": round(r32["kernel_ms"] * 1e3, 2), "GBps": round(a32, 1),
             "frac_hbm": round(a32 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": r32["bytes"]}
+        extra["selective_scan_fwd_through_ops_entry"] = bench_scan_facade()
+        extra["selective_scan_fwd_per_channel_bc"] = bench_scan_per_channel_bc()
         extra["selective_scan_bwd_bf16"] = bench_scan_bwd()
         extra["dw_causal_conv_bf16"] = bench_conv()
         extra["fused_add_rmsnorm"] = bench_norm()

@@ -603,6 +603,19 @@ int ssm_norm_bwd(const ssm_norm_bwd_args *args, void *hip_stream);
 #define SSM_NORM_BWD_STATIC_BYTES (8u << 20)
 int ssm_norm_bwd_static(const ssm_norm_bwd_args *args, void *hip_stream);
 
+/* ------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference): a loop of `iters` repetitions of one instruction
+ * pattern with no memory traffic on `workgroups` workgroups of 256 * waves_per_simd threads, one per CU at a
+ * time.  kind: 0 eight independent fp32 fma, 1 eight dependent fma, 2 / 3 / 4 eight exp2 / log2 / rcp,
+ * 5 exp2 and fma alternating (8), 6 the scan's state step for eight states (mul, exp2, mul, fma, fmac: 40),
+ * 7 the same with a move in place of exp2, 8 eight DPP multiplies (quad broadcast), 9 eight DPP fmac / mul of a
+ * lane scan, 10 eight half-wave / row swaps, 11 four state steps and one fp32 16x16x4 matrix instruction (21),
+ * 12 eight 8-byte LDS reads.  `out` takes workgroups * 1024 floats; clocks[0] / clocks[1] receive the shader
+ * and the 100 MHz wall clock ticks that the loop took on the first workgroup.
+ * ---------------------------------------------------------------------- */
+int ssm_probe_valu(int kind, int waves_per_simd, int workgroups, int iters, float *out, long long *clocks,
+                   void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -279,6 +279,7 @@ PLAIN_SYMBOLS = {
     "ssm_ssd_combined_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
     "ssm_conv1d_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "ssm_norm_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+    "ssm_probe_valu": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
 }
 
 _lock = threading.Lock()

@@ -48,19 +48,3 @@ def scan_fwd_bytes(batch: int, dim: int, length: int, nstate: int, elt: int, gro
 
 def to_device(d: dict, device="cuda") -> dict:
     return {k: (v.to(device) if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
-
-
-# HBM traffic of one launch of the headline scan-forward kernel (B=8, D=1536, L=2048, N=16,
-# bf16), from hardware counters: mean FETCH_SIZE / WRITE_SIZE per dispatch (rocprofv3 --pmc,
-# one counter per run; summaries in profiles/scan_fwd_bf16_headline_pmc_*.txt), each scaled by
-# what the same counter reads for a 256 MiB elementwise copy in the same run
-# (FETCH_SIZE: 131085.5 for 262144 KiB read -> x2.0; WRITE_SIZE: 262144.0 -> x1.0).
-SCAN_FWD_HEADLINE_TRAFFIC = {
-    "fetch_counter": 78044.6, "fetch_scale": 262144.0 / 131085.6,
-    "write_counter": 49536.0, "write_scale": 262144.0 / 262144.0,
-}
-
-
-def scan_fwd_headline_traffic_bytes():
-    t = SCAN_FWD_HEADLINE_TRAFFIC
-    return int(round((t["fetch_counter"] * t["fetch_scale"] + t["write_counter"] * t["write_scale"]) * 1024))

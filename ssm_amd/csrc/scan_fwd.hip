@@ -92,6 +92,8 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
       const int per_wg = scan_fwd_fast_rows(pref[i]);
       if (per_b % per_wg == 0 && per_c % per_wg == 0 && (total / per_wg >= 256 || i == 2)) pick = pref[i];
     }
+    // groups of fewer than 8 channels (down to one per channel): nothing to share, a row per wave
+    if (!pick && aligned_to(a->Bproj, 16) && aligned_to(a->Cproj, 16) && ((size_t)a->seqlen * bs) % 16 == 0) pick = 31041;
     if (pick) tune = 100000 + pick;
   }
   if (tune >= 100000) {

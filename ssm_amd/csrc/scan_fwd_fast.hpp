@@ -281,6 +281,120 @@ void scan_fwd_fast_kernel(const ScanFwdParams p) {
   }
 }
 
+// The same scan for projections that few channels share (down to one B/C group per channel, the layout
+// (B, D, N, L) a Mamba-1 block passes): nothing is staged.  A wave owns one row, a lane its 8-step run, and the
+// lane reads the 16 bytes of B and of C of its run for every state straight from memory (consecutive lanes,
+// consecutive bytes), one state ahead of the arithmetic.  No LDS, no barrier: the call is bound by those reads.
+template <typename io_t, typename bc_t, int WAVES, int OCC>
+__global__ __launch_bounds__(WAVE *WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
+  constexpr int K = 8, T = FAST_T;
+  const int wave = wave_id_uniform();
+  const int lane = lane_id();
+  const size_t row = (size_t)blockIdx.x * WAVES + wave;
+  if (row >= (size_t)p.batch * p.dim) return;                // no barrier below: a wave may leave alone
+  const int b = (int)(row / p.dim), d = (int)(row % p.dim);
+  const int L = p.len, N = p.nstate;
+  const bc_t *Bg = reinterpret_cast<const bc_t *>(p.Bp) + ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * (size_t)N * L;
+  const bc_t *Cg = reinterpret_cast<const bc_t *>(p.Cp) + ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * (size_t)N * L;
+  const io_t *U = reinterpret_cast<const io_t *>(p.u), *DT = reinterpret_cast<const io_t *>(p.delta);
+  const io_t *Z = reinterpret_cast<const io_t *>(p.z);
+  io_t *Y = reinterpret_cast<io_t *>(p.out);
+
+  const float A2_lanes = lane < N ? p.A[(size_t)d * N + lane] * LOG2E : 0.0f;
+  float carry_lanes = 0.0f;
+  const float Dk = p.Dk ? p.Dk[d] : 0.0f, bias = p.bias ? p.bias[d] : 0.0f;
+
+  const int nchunks = (L + T - 1) / T;
+  for (int c = 0; c < nchunks; ++c) {
+    const int t = c * T + lane * K;
+    const bool live = t < L;
+    const int tc = live ? t : 0;
+    const size_t at = row * L + tc;
+    float dl[K], du[K], y[K];
+    Pack<io_t, K> zr;
+    Pack<bc_t, K> braw = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + tc);
+    Pack<bc_t, K> craw = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + tc);
+    {
+      const Pack<io_t, K> ur = *reinterpret_cast<const Pack<io_t, K> *>(U + at);
+      const Pack<io_t, K> dr = *reinterpret_cast<const Pack<io_t, K> *>(DT + at);
+      if (p.z) zr = *reinterpret_cast<const Pack<io_t, K> *>(Z + at);
+      if (p.chunk_states && lane < N) p.chunk_states[(row * nchunks + c) * (size_t)N + lane] = carry_lanes;
+#pragma unroll
+      for (int i = 0; i < K; ++i) dl[i] = to_f32(dr.v[i]) + bias;
+      if (p.softplus) {
+#pragma unroll
+        for (int i = 0; i < K; ++i) dl[i] = fast_softplus(dl[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < K; ++i) {
+        const float uu = to_f32(ur.v[i]);
+        dl[i] = live ? dl[i] : 0.0f;
+        du[i] = dl[i] * uu;
+        y[i] = Dk * uu;
+      }
+    }
+    float dsum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < K; ++i) dsum += dl[i];
+
+    for (int n = 0; n < N; ++n) {
+      // the next state's projections are requested before this state's arithmetic
+      const int nn = n + 1 < N ? n + 1 : n;
+      const Pack<bc_t, K> bnext = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + (size_t)nn * L + tc);
+      const Pack<bc_t, K> cnext = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + (size_t)nn * L + tc);
+      const float A2 = wave_read_lane(A2_lanes, n);
+      const float H = wave_read_lane(carry_lanes, n);
+      float a[K], bx[K], P = dsum * A2, h;
+#pragma unroll
+      for (int i = 0; i < K; ++i) a[i] = dl[i] * A2;
+      exp2_run(a, P);
+#pragma unroll
+      for (int i = 0; i < K; ++i) {
+        bx[i] = du[i] * to_f32(braw.v[i]);
+        h = i == 0 ? bx[0] : __builtin_fmaf(a[i], h, bx[i]);
+      }
+      h = __builtin_fmaf(P, lane == 0 ? H : 0.0f, h);
+      wave_scan_affine_x1(P, h);
+      float hs = wave_prev(h, H);
+      const float hend = wave_read_lane(h, WAVE - 1);
+      carry_lanes = lane == n ? hend : carry_lanes;
+#pragma unroll
+      for (int i = 0; i < K; ++i) {
+        hs = __builtin_fmaf(a[i], hs, bx[i]);
+        y[i] = __builtin_fmaf(hs, to_f32(craw.v[i]), y[i]);
+      }
+      braw = bnext;
+      craw = cnext;
+    }
+
+    if (p.z) {
+#pragma unroll
+      for (int i = 0; i < K; ++i) {
+        const float zz = to_f32(zr.v[i]);
+        y[i] *= zz * rcp_hw(1.0f + exp2_hw(-LOG2E * zz));
+      }
+    }
+    if (live) {
+      Pack<io_t, K> o;
+#pragma unroll
+      for (int i = 0; i < K; ++i) o.v[i] = from_f32<io_t>(y[i]);
+      *reinterpret_cast<Pack<io_t, K> *>(Y + at) = o;
+    }
+  }
+  if (p.last && lane < N) reinterpret_cast<io_t *>(p.last)[row * N + lane] = from_f32<io_t>(carry_lanes);
+}
+
+template <typename io_t, typename bc_t>
+static int launch_scan_fwd_rowbc(const ScanFwdParams &p, hipStream_t stream) {
+  constexpr int WAVES = 4;
+  const size_t rows = (size_t)p.batch * p.dim;
+  hipLaunchKernelGGL((scan_fwd_rowbc_kernel<io_t, bc_t, WAVES, 6>), dim3((unsigned)((rows + WAVES - 1) / WAVES)),
+                     dim3(WAVE * WAVES), 0, stream, p);
+  SSM_CHECK_LAUNCH("ssm_scan_fwd");
+  return SSM_OK;
+}
+
 template <typename io_t, typename bc_t, int LPR, int RPW, int WAVES, int W, int OCC>
 static int launch_scan_fwd_fast(const ScanFwdParams &p, hipStream_t stream) {
   const size_t lds = (size_t)2 * FAST_N * FAST_T * sizeof(float);
@@ -304,6 +418,7 @@ inline int scan_fwd_fast_rows(int variant) {
     case 11082: return 8;
     case 22121: return 48;
     case 21081: return 16;
+    case 31041: return 1;       // a row per wave, projections read straight from memory
     default: return 0;
   }
 }
@@ -316,6 +431,7 @@ int scan_fwd_fast_dispatch(const ScanFwdParams &p, int variant, hipStream_t s) {
     case 11082: return launch_scan_fwd_fast<io_t, bc_t, 64, 1, 8, 2, 4>(p, s);
     case 22121: return launch_scan_fwd_fast<io_t, bc_t, 32, 2, 12, 1, 3>(p, s);    // 3 waves per SIMD, 16-step runs
     case 21081: return launch_scan_fwd_fast<io_t, bc_t, 32, 1, 8, 1, 4>(p, s);
+    case 31041: return launch_scan_fwd_rowbc<io_t, bc_t>(p, s);
     default:
       set_error("ssm_scan_fwd: unknown variant %d of the specialised kernel", variant);
       return SSM_ERR_BAD_KIND;

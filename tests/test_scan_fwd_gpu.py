@@ -216,7 +216,7 @@ def test_several_channels_per_wave_match_oracle(items, dim):
     torch.testing.assert_close(h.float().cpu(), hr.float(), rtol=2e-2, atol=2e-2)
 
 
-FAST_VARIANTS = [(13082, 24), (12121, 24), (11082, 8), (22121, 48), (21081, 16)]
+FAST_VARIANTS = [(13082, 24), (12121, 24), (11082, 8), (22121, 48), (21081, 16), (31041, 3)]
 
 
 @pytest.mark.parametrize("variant,rows", FAST_VARIANTS)
@@ -251,6 +251,17 @@ def test_specialised_kernel_half_types_and_options(variant, rows, dtype, bc_dtyp
                          None, None, None, False, True, tune_items=100000 + variant)
     torch.testing.assert_close(y.float().cpu(), yr.float(), **HALF_TOL)
     torch.testing.assert_close(h.float().cpu(), hr.float(), **HALF_TOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_one_projection_group_per_channel(dtype):
+    """B and C as (B, D, N, L), the layout the reference's Mamba-1 block passes (src/ssm/modules/mamba1.py:229-247
+    of the reference): picked automatically, a row per wave with the projections read straight from memory."""
+    inp = make_inputs(23, 2, 10, 1040, 16, dtype=dtype, groups=10)
+    (y, h), (yr, hr) = run_both(inp)
+    tol = FP32_TOL if dtype == torch.float32 else HALF_TOL
+    torch.testing.assert_close(y.float(), yr.float(), **tol)
+    torch.testing.assert_close(h.float(), hr.float(), **tol)
 
 
 def test_specialised_kernel_refuses_other_shapes():
