@@ -83,10 +83,10 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
                        (a->bc_dtype == a->io_dtype || a->bc_dtype == SSM_F32);
   if (tune == 0 && fast_ok && a->seqlen > 256) {
     // The variant whose workgroups (48, 24 or 8 channels of one group) still give every CU its share:
-    // two rows per wave with 16-step runs where 256 such workgroups exist, else 8-step runs at six waves
+    // two rows per wave with 16-step runs and two slabs where 256 such workgroups exist, else 8-step runs at six waves
     // per SIMD, else the smallest workgroup.
     const size_t total = (size_t)a->batch * a->dim;
-    const int pref[3] = {22121, 12121, 11082};
+    const int pref[3] = {22123, 12121, 11082};
     int pick = 0;
     for (int i = 0; i < 3 && !pick; ++i) {
       const int per_wg = scan_fwd_fast_rows(pref[i]);

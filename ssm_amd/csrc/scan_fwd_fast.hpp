@@ -104,11 +104,14 @@ __device__ __forceinline__ float group_read_lane(float v, int src, int lane) {
   else return __int_as_float(__builtin_amdgcn_ds_bpermute(((lane & ~(LPR - 1)) + src) * 4, __float_as_int(v)));
 }
 
-template <typename io_t, typename bc_t, int LPR, int RPW, int WAVES, int W, int OCC>
+// DB: two slabs in LDS (for variants of which one workgroup fills a CU): the slab of the next chunk is staged by
+// each wave as soon as it is done with its rows of this one, while slower waves still work, and a chunk costs
+// one barrier instead of two.
+template <typename io_t, typename bc_t, int LPR, int RPW, int WAVES, int W, int OCC, bool DB>
 __global__ __launch_bounds__(WAVE *WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void scan_fwd_fast_kernel(const ScanFwdParams p) {
   constexpr int T = FAST_T, K = T / LPR, SUBS = WAVE / LPR;
-  extern __shared__ __align__(16) float tiles[];           // B [16][T] then C [16][T]
+  extern __shared__ __align__(16) float tiles[];           // B [16][T] then C [16][T] (twice with DB)
   float *Bs = tiles, *Cs = tiles + FAST_N * T;
 
   constexpr int rows = WAVES * RPW * SUBS;
@@ -144,10 +147,20 @@ void scan_fwd_fast_kernel(const ScanFwdParams p) {
     const bool live = t < L;                 // L % K == 0: a lane's run is inside or outside as a whole
     const int tc = live ? t : 0;
 
-    __syncthreads();
-    fast_stage<bc_t, LPR>(Bs, Bg, L, t0, N, WAVE * WAVES);
-    fast_stage<bc_t, LPR>(Cs, Cg, L, t0, N, WAVE * WAVES);
-    __syncthreads();
+    if constexpr (DB) {
+      if (c == 0) {
+        fast_stage<bc_t, LPR>(Bs, Bg, L, 0, N, WAVE * WAVES);
+        fast_stage<bc_t, LPR>(Cs, Cg, L, 0, N, WAVE * WAVES);
+      }
+      __syncthreads();           // slab c is complete; every wave is done with slab c - 1 (staged over below)
+      Bs = tiles + (c & 1) * 2 * FAST_N * T;
+      Cs = Bs + FAST_N * T;
+    } else {
+      __syncthreads();
+      fast_stage<bc_t, LPR>(Bs, Bg, L, t0, N, WAVE * WAVES);
+      fast_stage<bc_t, LPR>(Cs, Cg, L, t0, N, WAVE * WAVES);
+      __syncthreads();
+    }
 
 #pragma unroll
     for (int rr = 0; rr < RPW; ++rr) {
@@ -268,6 +281,13 @@ void scan_fwd_fast_kernel(const ScanFwdParams p) {
 #pragma unroll
         for (int i = 0; i < K; ++i) o.v[i] = from_f32<io_t>(y[i]);
         *reinterpret_cast<Pack<io_t, K> *>(Y + at) = o;
+      }
+    }
+    if constexpr (DB) {
+      if (c + 1 < nchunks) {
+        float *nb = tiles + ((c + 1) & 1) * 2 * FAST_N * T;
+        fast_stage<bc_t, LPR>(nb, Bg, L, t0 + T, N, WAVE * WAVES);
+        fast_stage<bc_t, LPR>(nb + FAST_N * T, Cg, L, t0 + T, N, WAVE * WAVES);
       }
     }
   }
@@ -395,10 +415,10 @@ static int launch_scan_fwd_rowbc(const ScanFwdParams &p, hipStream_t stream) {
   return SSM_OK;
 }
 
-template <typename io_t, typename bc_t, int LPR, int RPW, int WAVES, int W, int OCC>
+template <typename io_t, typename bc_t, int LPR, int RPW, int WAVES, int W, int OCC, bool DB = false>
 static int launch_scan_fwd_fast(const ScanFwdParams &p, hipStream_t stream) {
-  const size_t lds = (size_t)2 * FAST_N * FAST_T * sizeof(float);
-  auto kernel = scan_fwd_fast_kernel<io_t, bc_t, LPR, RPW, WAVES, W, OCC>;
+  const size_t lds = (size_t)(DB ? 4 : 2) * FAST_N * FAST_T * sizeof(float);
+  auto kernel = scan_fwd_fast_kernel<io_t, bc_t, LPR, RPW, WAVES, W, OCC, DB>;
   if (allow_dynamic_lds(kernel, lds) != hipSuccess) {
     (void)hipGetLastError();
     set_error("ssm_scan_fwd: cannot reserve %zu bytes of LDS", lds);
@@ -416,7 +436,7 @@ inline int scan_fwd_fast_rows(int variant) {
   switch (variant) {
     case 13082: case 12121: return 24;
     case 11082: return 8;
-    case 22121: return 48;
+    case 22121: case 22123: return 48;
     case 21081: return 16;
     case 31041: return 1;       // a row per wave, projections read straight from memory
     default: return 0;
@@ -430,6 +450,7 @@ int scan_fwd_fast_dispatch(const ScanFwdParams &p, int variant, hipStream_t s) {
     case 12121: return launch_scan_fwd_fast<io_t, bc_t, 64, 2, 12, 1, 6>(p, s);    // 6 waves per SIMD
     case 11082: return launch_scan_fwd_fast<io_t, bc_t, 64, 1, 8, 2, 4>(p, s);
     case 22121: return launch_scan_fwd_fast<io_t, bc_t, 32, 2, 12, 1, 3>(p, s);    // 3 waves per SIMD, 16-step runs
+    case 22123: return launch_scan_fwd_fast<io_t, bc_t, 32, 2, 12, 1, 3, true>(p, s);   // the same with two slabs
     case 21081: return launch_scan_fwd_fast<io_t, bc_t, 32, 1, 8, 1, 4>(p, s);
     case 31041: return launch_scan_fwd_rowbc<io_t, bc_t>(p, s);
     default:

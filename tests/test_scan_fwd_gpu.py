@@ -216,7 +216,7 @@ def test_several_channels_per_wave_match_oracle(items, dim):
     torch.testing.assert_close(h.float().cpu(), hr.float(), rtol=2e-2, atol=2e-2)
 
 
-FAST_VARIANTS = [(13082, 24), (12121, 24), (11082, 8), (22121, 48), (21081, 16), (31041, 3)]
+FAST_VARIANTS = [(13082, 24), (12121, 24), (11082, 8), (22121, 48), (22123, 48), (21081, 16), (31041, 3)]
 
 
 @pytest.mark.parametrize("variant,rows", FAST_VARIANTS)
