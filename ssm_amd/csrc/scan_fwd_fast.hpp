@@ -180,10 +180,13 @@ void scan_fwd_fast_kernel(const ScanFwdParams p) {
 #pragma unroll
           for (int i = 0; i < K; ++i) dl[i] = fast_softplus(dl[i]);
         }
+        if (t0 + T > L) {                      // only the last chunk can have lanes past the end: the identity map there
+#pragma unroll
+          for (int i = 0; i < K; ++i) dl[i] = live ? dl[i] : 0.0f;
+        }
 #pragma unroll
         for (int i = 0; i < K; ++i) {
           const float uu = to_f32(ur.v[i]);
-          dl[i] = live ? dl[i] : 0.0f;        // steps past the end are the identity map
           du[i] = dl[i] * uu;
           y[i] = Dk[rr] * uu;
         }
