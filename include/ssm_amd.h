@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SSM_AMD_ABI_VERSION 1
+#define SSM_AMD_ABI_VERSION 2
 
 typedef enum ssm_status {
   SSM_OK = 0,
@@ -122,6 +122,7 @@ typedef struct ssm_scan_bwd_args {
   int32_t io_dtype, bc_dtype;
   int32_t b_kind, c_kind, b_groups, c_groups;
   int32_t delta_softplus;
+  int32_t tune_items;             /* 0 = automatic; 1 = the general kernel also where the specialised one applies */
 } ssm_scan_bwd_args;
 
 size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, int nstate, int b_kind, int c_kind,

@@ -19,7 +19,7 @@ import os
 # SSM_AMD_LIB points the binding at another build of the same C ABI.
 LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
                 Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
 PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
@@ -55,7 +55,7 @@ class ScanBwdArgs(C.Structure):
         ("ddt_bias", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
         ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32),
         ("io_dtype", _i32), ("bc_dtype", _i32), ("b_kind", _i32), ("c_kind", _i32),
-        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32),
+        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("tune_items", _i32),
     ]
 
 

@@ -748,6 +748,8 @@ static int launch_bwd(const ScanBwdParams &p, hipStream_t s) {
 
 }  // namespace ssm
 
+#include "scan_bwd_fast.hpp"
+
 extern "C" size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, int nstate, int b_kind, int c_kind,
                                                int b_groups, int c_groups) {
   using namespace ssm;
@@ -814,10 +816,30 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
 
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   int rc;
-  switch (a->io_dtype) {
-    case SSM_F32: rc = launch_bwd<float>(p, s); break;
-    case SSM_BF16: rc = launch_bwd<bf16_t>(p, s); break;
-    default: rc = launch_bwd<f16_t>(p, s); break;
+  // The specialised kernel: 16-bit activations in aligned rows of whole 8-step runs, time-varying B and C of the
+  // activations' type or float32, groups that workgroups of 16, 32 or 48 channels tile, and no more partial
+  // sums than the workspace was sized for.  tune_items 1 keeps the general kernel.
+  int fast_rpw = 0;
+  if (bv && cv && a->io_dtype != SSM_F32 && a->tune_items != 1 && a->seqlen % 8 == 0 &&
+      (a->bc_dtype == a->io_dtype || a->bc_dtype == SSM_F32) && aligned_to(a->u, 16) && aligned_to(a->delta, 16) &&
+      aligned_to(a->dout, 16) && aligned_to(a->du, 16) && aligned_to(a->ddelta, 16) &&
+      (!a->z || (aligned_to(a->z, 16) && aligned_to(a->dz, 16))) && aligned_to(a->Bproj, 4 * bs) &&
+      aligned_to(a->Cproj, 4 * bs)) {
+    fast_rpw = scan_bwd_fast_rpw(a->batch, a->dim, a->dim / p.b_groups, a->dim / p.c_groups);
+    if (fast_rpw && a->dim / (BF_WAVES * fast_rpw) > pl.nblk) fast_rpw = 0;
+  }
+  if (fast_rpw) {
+    p.rows_per_wg = BF_WAVES * fast_rpw;
+    p.nblk = a->dim / p.rows_per_wg;
+    const bool bc32 = a->bc_dtype == SSM_F32;
+    if (a->io_dtype == SSM_BF16) rc = bc32 ? launch_bwd_fast<bf16_t, float>(p, fast_rpw, s) : launch_bwd_fast<bf16_t, bf16_t>(p, fast_rpw, s);
+    else rc = bc32 ? launch_bwd_fast<f16_t, float>(p, fast_rpw, s) : launch_bwd_fast<f16_t, f16_t>(p, fast_rpw, s);
+  } else {
+    switch (a->io_dtype) {
+      case SSM_F32: rc = launch_bwd<float>(p, s); break;
+      case SSM_BF16: rc = launch_bwd<bf16_t>(p, s); break;
+      default: rc = launch_bwd<f16_t>(p, s); break;
+    }
   }
   if (rc != SSM_OK) return rc;
 
@@ -832,7 +854,7 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
   auto fold_proj = [&](int kind, int groups, const float *partial, float *out) {
     if (kind == SSM_PROJ_BGNL) {
       // (B, G, nblk/G, N*L) -> (B, G, N*L)
-      const int per_group = pl.nblk / groups;
+      const int per_group = p.nblk / groups;
       launch_fold_sum(partial, out, (size_t)Bn * groups, per_group, (size_t)N * L, s);
     } else if (kind == SSM_PROJ_BDN) {
       hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)Bn * D * N)), dim3(256), 0, s, partial, out, 1,

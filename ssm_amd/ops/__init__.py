@@ -109,7 +109,8 @@ def _slice_states(p, kind, lo, hi):
     return p[:, :, lo:hi, :]
 
 
-def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softplus, chunk_states=None):
+def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softplus, chunk_states=None,
+                   tune_items=0):
     """Run ``ssm_scan_bwd``; returns fp32/io-dtype gradients in input order
     ``(du, ddelta, dA, dB, dC, dD, dz, ddt_bias)``.  State sizes above 16 are
     processed in blocks of 16 states (the recurrence is independent per state and
@@ -169,7 +170,7 @@ def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softpl
             ddt_bias=_lib.ptr(dbias_b), workspace=ws_ptr, workspace_bytes=nbytes,
             batch=batch, dim=dim, seqlen=length, nstate=n_blk, io_dtype=_lib.dtype_enum(io),
             bc_dtype=_lib.dtype_enum(bc), b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
-            delta_softplus=int(bool(softplus)))
+            delta_softplus=int(bool(softplus)), tune_items=int(tune_items))
         _lib.call("ssm_scan_bwd", args, dev)
         if single:
             du, ddl, dz, dbias = du_b, ddl_b, dz_b, dbias_b

@@ -204,7 +204,11 @@ def test_config1_shape_bf16_slice():
     for k in ("B", "C"):
         s = lo[k].float() + hi[k].float()
         torch.testing.assert_close(full[k].float(), s, rtol=2e-2, atol=2e-2 * float(s.abs().max()))
-    torch.testing.assert_close(full["u"][:, :768].float(), lo["u"].float(), rtol=0, atol=0)
+    # a row's sums over the states run in an order that depends on the wave that owns the row, and the block shape
+    # follows the channel count: the same row in the two calls agrees to one rounding of the 16-bit result
+    a, b = full["u"][:, :768].float(), lo["u"].float()
+    torch.testing.assert_close(a, b, rtol=2 ** -7, atol=1e-6 * float(b.abs().max()))
+    assert float((a != b).float().mean()) < 1e-3
     # slice of 8 channels against the oracle
     idx = torch.arange(0, 1536, 192)
     sub = {k: (inp[k][:, idx] if k in ("u", "delta", "z") else inp[k][idx] if k in ("A", "D", "dt_bias") else inp[k])
@@ -219,3 +223,67 @@ def test_config1_shape_bf16_slice():
     for k in ("A", "D", "dt_bias"):
         w = lv[k].grad.float()
         torch.testing.assert_close(full[k][idx.cuda()].float().cpu(), w, rtol=3e-2, atol=3e-2 * float(w.abs().max()))
+
+
+# ------------------------------------------------------------------ the specialised kernel (16-bit activations)
+
+def _bwd_direct(inp, go, gl, tune_items):
+    from ssm_amd import ops
+    dev = {k: (v.cuda() if v is not None else None) for k, v in inp.items()}
+    return ops._scan_backward(go.cuda(), None if gl is None else gl.cuda(), dev["u"], dev["delta"], dev["A"], dev["B"],
+                              dev["C"], dev["D"], dev["z"], dev["dt_bias"], True, tune_items=tune_items)
+
+
+@pytest.mark.parametrize("shape,groups,use_z,with_last", [
+    ((2, 48, 1040, 16), 1, True, True), ((1, 96, 512, 16), 2, True, False), ((2, 32, 1536, 9), 1, False, True),
+    ((1, 16, 72, 16), 1, True, False), ((3, 48, 2048, 16), 3, True, False)], ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("dtype,bc_dtype", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32)])
+def test_specialised_backward_matches_general_kernel_and_oracle(shape, groups, use_z, with_last, dtype, bc_dtype):
+    """16-bit activations, time-varying grouped B/C, groups that 16-channel blocks tile: the wave-per-row kernel
+    (all states in turn, dB/dC summed in LDS under a skew) against the general kernel on the same inputs (both
+    compute in float32 from the same 16-bit values: they agree to float32 rounding where the outputs are float32 and
+    to one 16-bit rounding elsewhere) and against float64 autograd through the oracle."""
+    b, d, l, n = shape
+    inp = make_inputs(sum(shape), b, d, l, n, dtype=dtype, bc_dtype=bc_dtype, groups=groups, use_z=use_z)
+    g = torch.Generator().manual_seed(3)
+    go = torch.randn(b, d, l, generator=g).to(dtype)
+    gl = torch.randn(b, d, n, generator=g) if with_last else None
+    fast = _bwd_direct(inp, go, gl, 0)
+    gen = _bwd_direct(inp, go, gl, 1)
+    names = ("u", "delta", "A", "B", "C", "D", "z", "dt_bias")
+    for k, f, r in zip(names, fast, gen):
+        if r is None:
+            assert f is None, k
+            continue
+        f, r = f.float().cpu(), r.float().cpu()
+        scale = float(r.abs().max()) + 1e-30
+        if k in ("u", "delta", "z"):
+            torch.testing.assert_close(f, r, rtol=2e-2, atol=1e-3 * scale, msg=lambda m, k=k: f"grad {k} vs general kernel: {m}")
+        else:
+            torch.testing.assert_close(f, r, rtol=2e-4, atol=2e-5 * scale, msg=lambda m, k=k: f"grad {k} vs general kernel: {m}")
+    # float64 autograd through the oracle on the same 16-bit values
+    w = {k: (None if v is None else v.double().requires_grad_(True)) for k, v in inp.items()}
+    out = O.selective_scan(w["u"], w["delta"], w["A"], w["B"], w["C"], D=w["D"], z=w["z"], dt_bias=w["dt_bias"],
+                           softplus=True, return_last_state=with_last, acc=torch.float64)
+    if with_last:
+        ((out[0] * go.double()).sum() + (out[1] * gl.double()).sum()).backward()
+    else:
+        (out * go.double()).sum().backward()
+    for k, f in zip(names, fast):
+        if w[k] is None:
+            continue
+        want = w[k].grad
+        scale = float(want.abs().max()) + 1e-30
+        tol = dict(rtol=2e-2, atol=4e-3 * scale) if k in ("u", "delta", "z") else dict(rtol=1e-3, atol=1e-4 * scale)
+        torch.testing.assert_close(f.double().cpu(), want, **tol, msg=lambda m, k=k: f"grad {k} vs float64: {m}")
+
+
+def test_specialised_backward_is_bit_reproducible():
+    inp = make_inputs(11, 2, 48, 1040, 16, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(4)
+    go = torch.randn(2, 48, 1040, generator=g).to(torch.bfloat16)
+    first = _bwd_direct(inp, go, None, 0)
+    for _ in range(3):
+        again = _bwd_direct(inp, go, None, 0)
+        for a, b in zip(first, again):
+            assert (a is None and b is None) or torch.equal(a, b)
