@@ -9,10 +9,15 @@
 // with the same scan on lane-reversed operands, replay backwards with the true adjoint.  What
 // sums over states (pre-activation, <gh, B>, the A-term of d delta) never leaves the lane's
 // registers; what sums over the channels of a group (dB, dC) is added into an LDS tile by the
-// 16 wavefronts of the workgroup, which are kept on 16 different states by a skew (wave w works
-// on state (w + slot) mod 16) with a barrier between slots: every element of the tile is touched
-// by one wave per slot, in a fixed order, so results are bit-reproducible without atomics'
-// ordering mattering.  The tile goes to memory once per chunk as one partial per workgroup.
+// 16 wavefronts of the workgroup, which are kept on 16 different states by a skew: wave w works
+// on state (w + slot) mod 16, so a state's part of the tile passes from wave w + 1 to wave w from
+// one slot to the next.  A wave counts its finished slots in LDS and, before it touches the tile
+// (a plain read, add, write at the very end of the slot), waits for the count of the wave it
+// takes over from; the rest of a slot needs no agreement between waves, which may drift apart by
+// most of a slot.  (A workgroup barrier per slot costs 25 % of the kernel's time here, LDS float
+// atomics, which take the 64 lanes one by one on this chip, eight times the whole kernel.)
+// Every element is added to by one wave at a time in a fixed order, so results are the same bits
+// on every run.  The tile goes to memory once per chunk as one partial per workgroup.
 // 128 KB of LDS: one workgroup of 16 waves per CU, four waves per SIMD.
 #pragma once
 #include "scan_fwd_fast.hpp"
@@ -22,10 +27,7 @@ namespace ssm {
 constexpr int BF_WAVES = 16;
 constexpr int BF_THREADS = WAVE * BF_WAVES;
 constexpr int BF_K = 8;
-#ifndef BF_DEP_DIR
-#define BF_DEP_DIR 1
-#endif
-constexpr int BF_DEP = BF_DEP_DIR;             // wave w takes a state over from wave w + BF_DEP
+constexpr int BF_DEP = 1;             // wave w takes a state over from wave w + BF_DEP (-1 measured 2 % slower)
 
 __device__ __forceinline__ float lane_from(float v, int src_lane) {
   return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
