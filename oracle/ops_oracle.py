@@ -18,8 +18,7 @@ goldens (``selective_scan_case1``, ``selective_scan_grouped``,
 ``mamba_reference_cases.json`` (selective_scan fwd + gradients,
 selective_state_update, dw_causal_conv fwd + gradients, layer norms fwd +
 gradients), library special cases (``F.conv1d``, ``F.layer_norm``,
-``F.rms_norm``), closed forms (geometric series) and the independent C
-restatement in ``oracle/scan_oracle.c``.
+``F.rms_norm``) and closed forms (geometric series).
 
 Every function takes ``acc`` (default ``None``): ``None`` applies the
 reference's dtype policy (half/bfloat16 accumulate in float32, others in
