@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SSM_AMD_ABI_VERSION 2
+#define SSM_AMD_ABI_VERSION 3
 
 typedef enum ssm_status {
   SSM_OK = 0,
@@ -509,6 +509,21 @@ typedef struct ssm_ssd_bwd_db_args {
   int32_t batch, seqlen, heads, groups, nstate;
 } ssm_ssd_bwd_db_args;
 int ssm_ssd_bwd_db(const ssm_ssd_bwd_db_args *args, void *hip_stream);
+
+/* The matrix both dB and dC of a chunk's own steps follow from (the "dCB" of the published backward,
+ * state-spaces/mamba ssd_combined.py: _chunk_scan_bwd_dcb + _chunk_state_bwd_db folded over heads):
+ *   dCB[b,c,g,l,s] = sum_{h in g} dt[s,h] exp(cs[l,h] - cs[s,h]) <dy[b,cQ+l,h,:], x[b,cQ+s,h,:]>  (s <= l, else 0)
+ * so that dB[cQ+s] = sum_l dCB[l,s] C[cQ+l] and dC[cQ+l] = sum_s dCB[l,s] B[cQ+s] are plain matrix products.
+ * bf16 operands, float32 result; headdim 32 or 64, chunk a multiple of 32 that divides seqlen. */
+typedef struct ssm_ssd_bwd_dcb_args {
+  const void *dy;            /* (B, L, H, P) bf16: gradient at the output before skip and gate */
+  const void *x;             /* (B, L, H, P) bf16 */
+  const float *dt;           /* (B, H, nc, Q) fp32: the step after bias, softplus and clamp */
+  const float *dA_cumsum;    /* (B, H, nc, Q) fp32: running sums of dt * A inside each chunk */
+  float *dCB;                /* (B, nc, G, Q, Q) fp32 */
+  int32_t batch, seqlen, heads, headdim, groups, chunk;
+} ssm_ssd_bwd_dcb_args;
+int ssm_ssd_bwd_dcb(const ssm_ssd_bwd_dcb_args *args, void *hip_stream);
 
 /* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).

@@ -19,7 +19,7 @@ import os
 # SSM_AMD_LIB points the binding at another build of the same C ABI.
 LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
                 Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
 PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
@@ -195,6 +195,11 @@ class SsdBwdDbArgs(C.Structure):
                 ("groups", _i32), ("nstate", _i32)]
 
 
+class SsdBwdDcbArgs(C.Structure):
+    _fields_ = [("dy", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("dCB", _vp), ("batch", _i32),
+                ("seqlen", _i32), ("heads", _i32), ("headdim", _i32), ("groups", _i32), ("chunk", _i32)]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -256,6 +261,7 @@ ENTRY_POINTS = {
     "ssm_ssd_bwd_gate": SsdBwdGateArgs,
     "ssm_ssd_bwd_dx": SsdBwdDxArgs,
     "ssm_ssd_bwd_db": SsdBwdDbArgs,
+    "ssm_ssd_bwd_dcb": SsdBwdDcbArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_conv1d_update": Conv1dUpdateArgs,

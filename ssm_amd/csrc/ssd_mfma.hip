@@ -92,6 +92,94 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_bmm_mfma_kernel(const SsdBmmPa
   }
 }
 
+// ------------------------------------------------------------------ backward: dCB
+// dCB[b,c,g,l,s] = sum over the heads h of group g of  dt[s,h] exp(cs[l,h] - cs[s,h]) <dy[l,h,:], x[s,h,:]>  for s <= l,
+// zero above the diagonal: the matrix from which both dB (= dCB^T C) and dC (= dCB B) of a chunk's own steps follow,
+// so that the sum over heads is taken once, before the products with C and B.  One workgroup per 64x64 tile, a wave
+// per 32x32 block; per head the block of <dy, x> is formed on the matrix cores from operands read straight from
+// memory (rows of dy and x with the channel axis contiguous) and added with its per-element weight in float32.
+struct SsdDcbParams {
+  const __bf16 *dy, *x;        // (B, L, H, P)
+  const float *dt, *dA_cs;     // (B, H, nc, Q)
+  float *out;                  // (B, nc, G, Q, Q)
+  int batch, len, heads, hdim, groups, chunk, nchunks;
+};
+
+template <int KS>              // P = 16 * KS
+__global__ __launch_bounds__(MF_THREADS) void ssd_bwd_dcb_kernel(const SsdDcbParams p) {
+  // One workgroup per 32x32 block on or below the diagonal; its four waves take every fourth head of the group
+  // (a head is one round trip to memory and little arithmetic, so the heads must be spread over many waves), and
+  // their sums meet in LDS.
+  __shared__ float part[MF_WAVES - 1][16][WAVE];
+  const int Q = p.chunk, P = 16 * KS, H = p.heads;
+  const int nb = Q / 32, nblk = nb * (nb + 1) / 2;
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int unit = blockIdx.x / nblk;
+  int tri = blockIdx.x % nblk;                            // (lb, sb) with sb <= lb, row by row
+  int lb = 0;
+  while (tri > lb) tri -= ++lb;
+  const int sb = tri;
+  const int g = unit % p.groups;
+  const int c = (unit / p.groups) % p.nchunks;
+  const int b = unit / (p.groups * p.nchunks);
+  const int l0 = lb * 32, s0 = sb * 32;
+  float *out = p.out + (((size_t)b * p.nchunks + c) * p.groups + g) * (size_t)Q * Q;
+  const int g2 = lane >> 5, m = lane & 31;
+  f32x16_t acc = {0};
+  const int per = H / p.groups;
+  const bool diag = s0 == l0;
+  const size_t trow = (size_t)H * P;
+  const __bf16 *arow = p.dy + ((size_t)b * p.len + (size_t)c * Q + l0 + m) * trow + (size_t)g * per * P + 8 * g2;
+  const __bf16 *brow = p.x + ((size_t)b * p.len + (size_t)c * Q + s0 + m) * trow + (size_t)g * per * P + 8 * g2;
+  const size_t csb = (((size_t)b * H + (size_t)g * per) * p.nchunks + c) * Q;
+  bf16x8_t fa[KS], fb[KS];
+  if (wave < per) {
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      fa[k] = load_frag(arow + (size_t)wave * P + 16 * k);
+      fb[k] = load_frag(brow + (size_t)wave * P + 16 * k);
+    }
+  }
+  for (int hh = wave; hh < per; hh += MF_WAVES) {
+    const float *cs = p.dA_cs + csb + (size_t)hh * p.nchunks * Q;
+    const float *dts = p.dt + csb + (size_t)hh * p.nchunks * Q;
+    const float cs_s = cs[s0 + m], dt_s = dts[s0 + m];
+    float4 cl[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cl[j] = *reinterpret_cast<const float4 *>(cs + l0 + 8 * j + 4 * g2);
+    f32x16_t t = {0};
+#pragma unroll
+    for (int k = 0; k < KS; ++k) t = mma(fa[k], fb[k], t);
+    if (hh + MF_WAVES < per) {                           // the wave's next head, requested before this head's weights
+#pragma unroll
+      for (int k = 0; k < KS; ++k) {
+        fa[k] = load_frag(arow + (size_t)(hh + MF_WAVES) * P + 16 * k);
+        fb[k] = load_frag(brow + (size_t)(hh + MF_WAVES) * P + 16 * k);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float cs_l = r % 4 == 0 ? cl[r / 4].x : r % 4 == 1 ? cl[r / 4].y : r % 4 == 2 ? cl[r / 4].z : cl[r / 4].w;
+      float w = dt_s * exp2_hw(fminf(cs_l - cs_s, 0.0f) * LOG2E);
+      if (diag && s0 + m > l0 + crow(r, g2)) w = 0.0f;
+      acc[r] = __builtin_fmaf(w, t[r], acc[r]);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[wave - 1][r][lane] = acc[r];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float v = ((acc[r] + part[0][r][lane]) + part[1][r][lane]) + part[2][r][lane];
+      out[(size_t)(l0 + crow(r, g2)) * Q + s0 + m] = v;
+      if (!diag) out[(size_t)(s0 + crow(r, g2)) * Q + l0 + m] = 0.0f;      // the mirrored block above the diagonal
+    }
+  }
+}
+
 // ---------------------------------------------------------------- transpose B
 // Bt[b,g,n,t] = Bm[b,t,g,n]   (bf16), tiles of 64 x 64 through LDS.
 __global__ __launch_bounds__(MF_THREADS) void ssd_transpose_kernel(const uint16_t *src, uint16_t *dst, int len, int groups,
@@ -359,3 +447,33 @@ bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s) {
 }
 
 }  // namespace ssm
+
+extern "C" int ssm_ssd_bwd_dcb(const ssm_ssd_bwd_dcb_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_dcb: args is NULL");
+  SSM_REQUIRE(a->dy && a->x && a->dt && a->dA_cumsum && a->dCB, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_bwd_dcb: dy, x, dt, dA_cumsum and dCB are required");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->groups > 0 && a->chunk > 0 && a->heads % a->groups == 0,
+              SSM_ERR_BAD_SHAPE, "ssm_ssd_bwd_dcb: sizes must be positive and groups must divide heads");
+  SSM_REQUIRE(a->headdim == 32 || a->headdim == 64, SSM_ERR_BAD_SHAPE, "ssm_ssd_bwd_dcb: headdim=%d, supported: 32, 64",
+              a->headdim);
+  SSM_REQUIRE(a->chunk % 32 == 0 && a->seqlen % a->chunk == 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bwd_dcb: chunk=%d must be a multiple of 32 and divide seqlen=%d", a->chunk, a->seqlen);
+  SSM_REQUIRE(aligned_to(a->dy, 16) && aligned_to(a->x, 16) && aligned_to(a->dA_cumsum, 16) && aligned_to(a->dt, 4) &&
+                  aligned_to(a->dCB, 4),
+              SSM_ERR_ALIGNMENT, "ssm_ssd_bwd_dcb: dy, x and dA_cumsum must be 16-byte aligned");
+  SsdDcbParams p{};
+  p.dy = reinterpret_cast<const __bf16 *>(a->dy);
+  p.x = reinterpret_cast<const __bf16 *>(a->x);
+  p.dt = a->dt; p.dA_cs = a->dA_cumsum; p.out = a->dCB;
+  p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.hdim = a->headdim; p.groups = a->groups;
+  p.chunk = a->chunk; p.nchunks = a->seqlen / a->chunk;
+  const int nb = p.chunk / 32;
+  const size_t grid = (size_t)p.batch * p.nchunks * p.groups * (nb * (nb + 1) / 2);
+  SSM_REQUIRE(grid < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_dcb: too many blocks");
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  if (p.hdim == 64) hipLaunchKernelGGL(ssd_bwd_dcb_kernel<4>, dim3((unsigned)grid), dim3(MF_THREADS), 0, s, p);
+  else hipLaunchKernelGGL(ssd_bwd_dcb_kernel<2>, dim3((unsigned)grid), dim3(MF_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_bwd_dcb");
+  return SSM_OK;
+}

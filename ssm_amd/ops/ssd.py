@@ -603,6 +603,63 @@ def _bwd_db(v_rev, dte, groups):
     return dB
 
 
+def _bwd_dcb(dy, x, dt_c, dA_cs, groups):
+    """``ssm_ssd_bwd_dcb``: ``(B, nc, G, Q, Q)`` float32, the head-summed weighted ``<dy_l, x_s>`` of every chunk."""
+    batch, seqlen, heads, hdim = (int(v) for v in x.shape)
+    nc, Q = int(dA_cs.shape[2]), int(dA_cs.shape[3])
+    out = torch.empty(batch, nc, groups, Q, Q, dtype=torch.float32, device=x.device)
+    args = _lib.SsdBwdDcbArgs(dy=_lib.ptr(dy), x=_lib.ptr(x), dt=_lib.ptr(dt_c), dA_cumsum=_lib.ptr(dA_cs),
+                              dCB=_lib.ptr(out), batch=batch, seqlen=seqlen, heads=heads, headdim=hdim, groups=groups,
+                              chunk=Q)
+    _lib.call("ssm_ssd_bwd_dcb", args, x.device)
+    return out
+
+
+def _mm_f32(a, b):
+    """Batched product of bfloat16 matrices with a float32 result."""
+    try:
+        return torch.bmm(a.reshape(-1, *a.shape[-2:]), b.reshape(-1, *b.shape[-2:]),
+                         out_dtype=torch.float32).view(*a.shape[:-1], b.shape[-1])
+    except (TypeError, RuntimeError):
+        return torch.matmul(a, b).float()
+
+
+def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, ent_f, entr_fwd, groups):
+    """``dB`` and ``dC`` ``(B, L, G, N)`` with the sum over a group's heads taken before the products with ``C`` and
+    ``B`` (state-spaces/mamba ssd_combined.py, ``_chunk_scan_bwd_dcb`` / ``_chunk_state_bwd_db`` /
+    ``_chunk_scan_bwd_dC``): inside a chunk both follow from one ``Q x Q`` matrix per group, ``dCB``; what crosses
+    chunk boundaries is a product of the weighted ``x`` (``dy``) rows, all heads of the group side by side, with
+    the adjoint (forward) states entering the chunk."""
+    batch, seqlen, heads, hdim = (int(v) for v in xc.shape)
+    nc, Q = int(dA_cs.shape[2]), int(dA_cs.shape[3])
+    nstate = int(Bc.shape[-1])
+    per = heads // groups
+    f32, bf = torch.float32, torch.bfloat16
+    dCB = _bwd_dcb(dyc, xc, dt_c, dA_cs, groups)                                    # (B, nc, G, Q, Q)
+    Bg = Bc.view(batch, nc, Q, groups, nstate).permute(0, 1, 3, 2, 4).to(f32)       # (B, nc, G, Q, N)
+    Cg = Cc.view(batch, nc, Q, groups, nstate).permute(0, 1, 3, 2, 4).to(f32)
+    dB = torch.matmul(dCB.transpose(-1, -2), Cg)
+    dC = torch.matmul(dCB, Bg)
+
+    def blh(t_c):
+        return t_c.permute(0, 2, 3, 1).reshape(batch, seqlen, heads)
+
+    def rows(t, w):        # (B, L, H, P) bf16 scaled per (step, head) -> (B, nc, G, Q, per * P)
+        r = t * w.to(bf)[..., None]
+        return r.view(batch, nc, Q, groups, per * hdim).permute(0, 1, 3, 2, 4)
+
+    def states(e):         # (B, nc, H, P, N) float32 -> (B, nc, G, per * P, N) bf16
+        return e.to(bf).view(batch, nc, groups, per * hdim, nstate)
+
+    # dC_l += sum_{h,p} exp(cs_l) dy_l[h,p] H_in[h,p,:];  dB_s += sum_{h,p} dt_s exp(cs'_s) x_s[h,p] G_in[h,p,:]
+    # with cs' the running sum of the reversed pass at that step (the decay from s to the end of its chunk and
+    # over the step that follows)
+    dC = dC + _mm_f32(rows(dyc, torch.exp(blh(dA_cs))), states(ent_f))
+    dB = dB + _mm_f32(rows(xc, dte * torch.exp(blh(dA_r)).flip(1)), states(entr_fwd))
+    back = lambda t: t.permute(0, 1, 3, 2, 4).reshape(batch, seqlen, groups, nstate)
+    return back(dB), back(dC)
+
+
 def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
                           initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")), seq_idx=None):
     """Gradients of :func:`ssd_combined` (outputs ``y`` and ``final_states``).
@@ -715,17 +772,24 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     else:
         u = u_r.flip(1)
         dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
-    Bh = Bc.repeat_interleave(per, dim=2) if per > 1 else Bc
-    Ch = Cc.repeat_interleave(per, dim=2) if per > 1 else Cc
-    v_r, _ = _lin_pass(Ch.flip(1).contiguous(), ones_c, dA_r, dyr, xc.flip(1).contiguous(),
-                       None if dfin is None else dfin.transpose(2, 3).contiguous())
-    if nstate % 4 == 0:
-        dB = _bwd_db(v_r.contiguous(), dte, groups)
+    entr_fwd = None
+    if (fused and cd == torch.bfloat16 and hdim in (32, 64) and Q % 32 == 0 and seqlen % Q == 0
+            and xc.is_contiguous() and Bc.is_contiguous() and Cc.is_contiguous()):
+        # the sum over a group's heads first, then two small products per chunk
+        entr_fwd = ent_r.flip(1)
+        dB, dC = _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, ent_f, entr_fwd, groups)
     else:
-        dB = (dte[..., None] * v_r.flip(1)).view(batch, seqlen, groups, per, nstate).sum(3)
-    dCh, _ = _lin_pass(Bh.contiguous(), dt_c, dA_cs, xc, dyc.contiguous(),
-                       None if init is None else init.transpose(2, 3).contiguous())
-    dC = dCh.view(batch, seqlen, groups, per, nstate).sum(3)
+        Bh = Bc.repeat_interleave(per, dim=2) if per > 1 else Bc
+        Ch = Cc.repeat_interleave(per, dim=2) if per > 1 else Cc
+        v_r, _ = _lin_pass(Ch.flip(1).contiguous(), ones_c, dA_r, dyr, xc.flip(1).contiguous(),
+                           None if dfin is None else dfin.transpose(2, 3).contiguous())
+        if nstate % 4 == 0:
+            dB = _bwd_db(v_r.contiguous(), dte, groups)
+        else:
+            dB = (dte[..., None] * v_r.flip(1)).view(batch, seqlen, groups, per, nstate).sum(3)
+        dCh, _ = _lin_pass(Bh.contiguous(), dt_c, dA_cs, xc, dyc.contiguous(),
+                           None if init is None else init.transpose(2, 3).contiguous())
+        dC = dCh.view(batch, seqlen, groups, per, nstate).sum(3)
     if not fused:
         xu = (xf * u).sum(-1)                                             # (B, L, H)
         s1 = (xt.to(f32) * u).sum(-1)                  # with the rounded operand of the pass for y
@@ -739,7 +803,9 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         a_first = torch.exp(dte[:, ::Q] * Af[None, None])                           # (B, nc, H)
         if bnd is not None:
             a_first = a_first * (~bnd[:, ::Q]).to(f32)[..., None]
-        anchor = (ent_r.flip(1)[:, :-1] * ent_f[:, 1:]).sum(dim=(3, 4))             # (B, nc-1, H): chunks 1..
+        if entr_fwd is None:
+            entr_fwd = ent_r.flip(1)
+        anchor = (entr_fwd[:, :-1] * ent_f[:, 1:]).sum(dim=(3, 4))               # (B, nc-1, H): chunks 1..
         anchor = torch.cat([W0[:, None], a_first[:, 1:] * anchor], dim=1)
         dq = (s1 - s2).view(batch, nc, Q, heads)
         q = (anchor[:, :, None] + dq.cumsum(2) - dq).reshape(batch, seqlen, heads)

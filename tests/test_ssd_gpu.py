@@ -612,3 +612,33 @@ def test_growing_states_are_kept_off_the_one_pass_kernel():
     _lib.load().ssm_ssd_mfma_launches()
     ssd().ssd_combined(cu(inp["x"]), cu(dt), cu(-A), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]), z=cu(inp["z"]))
     assert _lib.load().ssm_ssd_mfma_launches() & 8
+
+
+# ------------------------------------------------------------------ backward: the head-summed matrix of a chunk
+
+@pytest.mark.parametrize("b,l,h,p,g,Q", [(2, 256, 4, 64, 1, 64), (1, 512, 6, 32, 2, 256), (1, 96, 3, 64, 3, 32)],
+                         ids=lambda v: str(v))
+def test_bwd_dcb_kernel_matches_the_sum_over_heads_in_float64(b, l, h, p, g, Q):
+    """``ssm_ssd_bwd_dcb`` against ``sum_h dt_s exp(cs_l - cs_s) <dy_l, x_s>`` (lower triangle) formed in float64
+    from the same bf16 operands."""
+    from ssm_amd.ops import ssd as ops_ssd
+    gen = torch.Generator().manual_seed(5 + l)
+    dy = torch.randn(b, l, h, p, generator=gen).to(torch.bfloat16)
+    x = torch.randn(b, l, h, p, generator=gen).to(torch.bfloat16)
+    dt = torch.nn.functional.softplus(torch.randn(b, l, h, generator=gen) - 2.0)
+    A = -(torch.rand(h, generator=gen) * 4 + 0.5)
+    dA_cs, dt_c = ops_ssd.chunk_cumsum(dt.cuda(), A.cuda(), Q)
+    got = ops_ssd._bwd_dcb(dy.cuda(), x.cuda(), dt_c, dA_cs, g).cpu().double()
+    nc, per = l // Q, h // g
+    cs = dA_cs.cpu().double()                                    # (B, H, nc, Q)
+    dtc = dt_c.cpu().double()
+    dyc = dy.double().view(b, nc, Q, g, per, p)
+    xc = x.double().view(b, nc, Q, g, per, p)
+    m = torch.einsum("bclgrp,bcsgrp->bcgrls", dyc, xc)           # per head
+    csh = cs.view(b, g, per, nc, Q).permute(0, 3, 1, 2, 4)       # (B, nc, G, per, Q)
+    dth = dtc.view(b, g, per, nc, Q).permute(0, 3, 1, 2, 4)
+    w = torch.exp(csh[..., :, None] - csh[..., None, :]) * dth[..., None, :]
+    w = w * torch.tril(torch.ones(Q, Q, dtype=torch.float64))
+    want = (m * w).sum(3)
+    assert got.shape == want.shape
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5 * float(want.abs().max()))
