@@ -138,6 +138,14 @@ void scan_bwd_fast_kernel(const ScanBwdParams p) {
 
       for (int slot = 0; slot < NS; ++slot) {
         const int n = (BF_DEP * wave + slot) & (NS - 1);
+        // the SIMD serves its oldest wave first; turn the order round slot by slot so that its four waves keep pace
+        {
+          const int pr = (slot + (wave >> 2)) & 3;
+          if (pr == 0) __builtin_amdgcn_s_setprio(0);
+          else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+          else if (pr == 2) __builtin_amdgcn_s_setprio(2);
+          else __builtin_amdgcn_s_setprio(3);
+        }
         if (n < N) {
           float bq[K], cq[K];
 #pragma unroll
