@@ -267,10 +267,29 @@ void scan_fwd_fast_kernel(const ScanFwdParams p) {
         }
       };
 
+      // The SIMD serves its oldest wave first.  Turning the order of the workgroup's waves on a SIMD round from
+      // state to state keeps them out of step with each other (one in its exponentials while another replays),
+      // which is worth 7 % of the kernel's time with three waves per SIMD.
+      auto turn = [&](int k) {
+        constexpr int RANKS = WAVES / 4;
+        if constexpr (RANKS >= 3) {
+          const int pr = (k + (wave >> 2)) % RANKS;
+          if (pr == 0) __builtin_amdgcn_s_setprio(0);
+          else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+          else if (pr == 2) __builtin_amdgcn_s_setprio(2);
+          else __builtin_amdgcn_s_setprio(3);
+        }
+      };
       int n0 = 0;
       if constexpr (W == 2)
-        for (; n0 + 2 <= N; n0 += 2) process(std::integral_constant<int, 2>{}, n0);
-      for (; n0 < N; ++n0) process(std::integral_constant<int, 1>{}, n0);
+        for (; n0 + 2 <= N; n0 += 2) {
+          turn(n0 >> 1);
+          process(std::integral_constant<int, 2>{}, n0);
+        }
+      for (; n0 < N; ++n0) {
+        turn(n0);
+        process(std::integral_constant<int, 1>{}, n0);
+      }
 
       if (p.z) {
 #pragma unroll
