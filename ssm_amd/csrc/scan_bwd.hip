@@ -816,11 +816,11 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
 
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   int rc;
-  // The specialised kernel: 16-bit activations in aligned rows of whole 8-step runs, time-varying B and C of the
+  // The specialised kernel: activations in aligned rows of whole 8-step runs, time-varying B and C of the
   // activations' type or float32, groups that workgroups of 16, 32 or 48 channels tile, and no more partial
   // sums than the workspace was sized for.  tune_items 1 keeps the general kernel.
   int fast_rpw = 0;
-  if (bv && cv && a->io_dtype != SSM_F32 && a->tune_items != 1 && a->seqlen % 8 == 0 &&
+  if (bv && cv && a->tune_items != 1 && a->seqlen % 8 == 0 &&
       (a->bc_dtype == a->io_dtype || a->bc_dtype == SSM_F32) && aligned_to(a->u, 16) && aligned_to(a->delta, 16) &&
       aligned_to(a->dout, 16) && aligned_to(a->du, 16) && aligned_to(a->ddelta, 16) &&
       (!a->z || (aligned_to(a->z, 16) && aligned_to(a->dz, 16))) && aligned_to(a->Bproj, 4 * bs) &&
@@ -832,7 +832,8 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
     p.rows_per_wg = BF_WAVES * fast_rpw;
     p.nblk = a->dim / p.rows_per_wg;
     const bool bc32 = a->bc_dtype == SSM_F32;
-    if (a->io_dtype == SSM_BF16) rc = bc32 ? launch_bwd_fast<bf16_t, float>(p, fast_rpw, s) : launch_bwd_fast<bf16_t, bf16_t>(p, fast_rpw, s);
+    if (a->io_dtype == SSM_F32) rc = launch_bwd_fast<float, float>(p, fast_rpw, s);
+    else if (a->io_dtype == SSM_BF16) rc = bc32 ? launch_bwd_fast<bf16_t, float>(p, fast_rpw, s) : launch_bwd_fast<bf16_t, bf16_t>(p, fast_rpw, s);
     else rc = bc32 ? launch_bwd_fast<f16_t, float>(p, fast_rpw, s) : launch_bwd_fast<f16_t, f16_t>(p, fast_rpw, s);
   } else {
     switch (a->io_dtype) {

@@ -1,5 +1,5 @@
 // Selective scan, backward: the kernel for the common call shape (time-varying grouped B and C,
-// at most 16 states, 16-bit activations in aligned rows of whole 8-step runs).  Included by
+// at most 16 states, activations of any supported type in aligned rows of whole 8-step runs).  Included by
 // scan_bwd.hip after ScanBwdParams.
 //
 // A wavefront owns one row at a time and walks its states one after the other, lanes split
