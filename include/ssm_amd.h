@@ -525,6 +525,22 @@ typedef struct ssm_ssd_bwd_dcb_args {
 } ssm_ssd_bwd_dcb_args;
 int ssm_ssd_bwd_dcb(const ssm_ssd_bwd_dcb_args *args, void *hip_stream);
 
+/* The states at the chunk boundaries, as the two products above want them, and the anchors of the running sum
+ * behind ddt and dA: `entering_fwd[b,c]` is the state before chunk c (first pass), `entering_rev[b,r]` the adjoint
+ * state before reversed chunk r (second pass), i.e. behind chunk nc-1-r in time order.  Writes both as bfloat16
+ * with chunks in time order (rev_bf16[b,c] = entering_rev[b,nc-1-c]) and
+ *   anchor[b,c-1,h] = <entering_rev[b,nc-c,h], entering_fwd[b,c,h]>   for c = 1..nc-1,
+ * every input read once.  `dim` = headdim * nstate.  No counterpart in the reference (see ssm_ssd_bwd_gate). */
+typedef struct ssm_ssd_bwd_states_args {
+  const float *entering_fwd;   /* (B, nc, H, dim) fp32 */
+  const float *entering_rev;   /* (B, nc, H, dim) fp32 */
+  void *fwd_bf16;              /* (B, nc, H, dim) bf16 */
+  void *rev_bf16;              /* (B, nc, H, dim) bf16 */
+  float *anchor;               /* (B, nc-1, H) fp32; may be NULL when nc == 1 */
+  int32_t batch, nchunks, heads, dim;
+} ssm_ssd_bwd_states_args;
+int ssm_ssd_bwd_states(const ssm_ssd_bwd_states_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).
  * Forward stands behind `dw_causal_conv(x, weight, bias, activation)`

@@ -200,6 +200,11 @@ class SsdBwdDcbArgs(C.Structure):
                 ("seqlen", _i32), ("heads", _i32), ("headdim", _i32), ("groups", _i32), ("chunk", _i32)]
 
 
+class SsdBwdStatesArgs(C.Structure):
+    _fields_ = [("entering_fwd", _vp), ("entering_rev", _vp), ("fwd_bf16", _vp), ("rev_bf16", _vp), ("anchor", _vp),
+                ("batch", _i32), ("nchunks", _i32), ("heads", _i32), ("dim", _i32)]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -262,6 +267,7 @@ ENTRY_POINTS = {
     "ssm_ssd_bwd_dx": SsdBwdDxArgs,
     "ssm_ssd_bwd_db": SsdBwdDbArgs,
     "ssm_ssd_bwd_dcb": SsdBwdDcbArgs,
+    "ssm_ssd_bwd_states": SsdBwdStatesArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_conv1d_update": Conv1dUpdateArgs,

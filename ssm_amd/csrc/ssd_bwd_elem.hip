@@ -192,6 +192,51 @@ unsigned elem_grid(const ElemParams &p) {
   return (unsigned)((lanes + EB_THREADS - 1) / EB_THREADS);
 }
 
+// Chunk-boundary states of the two passes for the products that give dB and dC, and the anchors of the running
+// sum behind ddt and dA.  One workgroup per (batch, chunk c, head): the forward state entering chunk c and the
+// adjoint state entering reversed chunk nc - c (the one that sits in front of chunk c - 1 in time order) are read
+// once, written as bfloat16 in time order, and their inner product is the anchor of chunk c.
+struct StatesParams {
+  const float *ent_f, *ent_r;     // (B, nc, H, dim)
+  bf16_t *f16, *r16;              // (B, nc, H, dim)
+  float *anchor;                  // (B, nc - 1, H)
+  int batch, nchunks, heads, dim;
+};
+
+__global__ __launch_bounds__(EB_THREADS) void ssd_bwd_states_kernel(const StatesParams p) {
+  __shared__ float part[EB_THREADS / WAVE];
+  const int h = blockIdx.x % p.heads;
+  const int c = (blockIdx.x / p.heads) % p.nchunks;
+  const int b = blockIdx.x / (p.heads * p.nchunks);
+  const int nc = p.nchunks;
+  const size_t at = (((size_t)b * nc + c) * p.heads + h) * (size_t)p.dim;
+  const float *F = p.ent_f + at;
+  bf16_t *F16 = p.f16 + at;
+  // c >= 1: the adjoint state whose place in time order is c - 1; c == 0: the one whose place is nc - 1 (no anchor)
+  const int rsrc = c >= 1 ? nc - c : 0, rdst = c >= 1 ? c - 1 : nc - 1;
+  const float *R = p.ent_r + (((size_t)b * nc + rsrc) * p.heads + h) * (size_t)p.dim;
+  bf16_t *R16 = p.r16 + (((size_t)b * nc + rdst) * p.heads + h) * (size_t)p.dim;
+  float acc = 0.0f;
+  for (int i = threadIdx.x * 4; i < p.dim; i += EB_THREADS * 4) {
+    const float4 f = *reinterpret_cast<const float4 *>(F + i), r = *reinterpret_cast<const float4 *>(R + i);
+    acc = __builtin_fmaf(f.x, r.x, acc);
+    acc = __builtin_fmaf(f.y, r.y, acc);
+    acc = __builtin_fmaf(f.z, r.z, acc);
+    acc = __builtin_fmaf(f.w, r.w, acc);
+    const float fv[4] = {f.x, f.y, f.z, f.w}, rv[4] = {r.x, r.y, r.z, r.w};
+    st4<bf16_t>(F16, i, fv);
+    st4<bf16_t>(R16, i, rv);
+  }
+  acc = wave_sum(acc);
+  if (lane_id() == 0) part[wave_id_uniform()] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0 && c >= 1) {
+    float t = 0.0f;
+    for (int w = 0; w < EB_THREADS / WAVE; ++w) t += part[w];
+    p.anchor[((size_t)b * (nc - 1) + (c - 1)) * p.heads + h] = t;
+  }
+}
+
 }  // namespace
 }  // namespace ssm
 
@@ -281,5 +326,29 @@ extern "C" int ssm_ssd_bwd_db(const ssm_ssd_bwd_db_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   hipLaunchKernelGGL(ssd_bwd_db_kernel, dim3((unsigned)((total + EB_THREADS - 1) / EB_THREADS)), dim3(EB_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_bwd_db");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_bwd_states(const ssm_ssd_bwd_states_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_states: args is NULL");
+  SSM_REQUIRE(a->entering_fwd && a->entering_rev && a->fwd_bf16 && a->rev_bf16, SSM_ERR_NULL_POINTER,
+              "ssm_ssd_bwd_states: the two state tensors and their bfloat16 copies are required");
+  SSM_REQUIRE(a->batch > 0 && a->nchunks > 0 && a->heads > 0 && a->dim > 0 && a->dim % 4 == 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bwd_states: sizes must be positive and dim=%d a multiple of 4", a->dim);
+  SSM_REQUIRE(a->anchor || a->nchunks == 1, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_states: anchor is required with more than one chunk");
+  SSM_REQUIRE(aligned_to(a->entering_fwd, 16) && aligned_to(a->entering_rev, 16) && aligned_to(a->fwd_bf16, 8) &&
+                  aligned_to(a->rev_bf16, 8),
+              SSM_ERR_ALIGNMENT, "ssm_ssd_bwd_states: state tensors must be 16-byte aligned, their copies 8-byte");
+  const size_t grid = (size_t)a->batch * a->nchunks * a->heads;
+  SSM_REQUIRE(grid < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_states: too many (batch, chunk, head) triples");
+  StatesParams p{};
+  p.ent_f = a->entering_fwd; p.ent_r = a->entering_rev;
+  p.f16 = reinterpret_cast<bf16_t *>(a->fwd_bf16); p.r16 = reinterpret_cast<bf16_t *>(a->rev_bf16);
+  p.anchor = a->anchor;
+  p.batch = a->batch; p.nchunks = a->nchunks; p.heads = a->heads; p.dim = a->dim;
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(ssd_bwd_states_kernel, dim3((unsigned)grid), dim3(EB_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_bwd_states");
   return SSM_OK;
 }

@@ -615,6 +615,21 @@ def _bwd_dcb(dy, x, dt_c, dA_cs, groups):
     return out
 
 
+def _bwd_states(ent_f, ent_r):
+    """``ssm_ssd_bwd_states``: both stacks of chunk-boundary states as bfloat16 with chunks in time order, and the
+    anchors ``<adjoint state, forward state>`` at the boundaries ``1..nc-1`` ``(B, nc-1, H)``."""
+    batch, nc, heads, hdim, nstate = (int(v) for v in ent_f.shape)
+    dev = ent_f.device
+    f16 = torch.empty(ent_f.shape, dtype=torch.bfloat16, device=dev)
+    r16 = torch.empty_like(f16)
+    anchor = torch.empty(batch, max(nc - 1, 0), heads, dtype=torch.float32, device=dev)
+    args = _lib.SsdBwdStatesArgs(entering_fwd=_lib.ptr(ent_f), entering_rev=_lib.ptr(ent_r), fwd_bf16=_lib.ptr(f16),
+                                 rev_bf16=_lib.ptr(r16), anchor=_lib.ptr(anchor) if nc > 1 else None, batch=batch,
+                                 nchunks=nc, heads=heads, dim=hdim * nstate)
+    _lib.call("ssm_ssd_bwd_states", args, dev)
+    return f16, r16, anchor
+
+
 def _mm_f32(a, b):
     """Batched product of bfloat16 matrices with a float32 result."""
     try:
@@ -624,7 +639,7 @@ def _mm_f32(a, b):
         return torch.matmul(a, b).float()
 
 
-def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, ent_f, entr_fwd, groups):
+def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, f16, r16, groups):
     """``dB`` and ``dC`` ``(B, L, G, N)`` with the sum over a group's heads taken before the products with ``C`` and
     ``B`` (state-spaces/mamba ssd_combined.py, ``_chunk_scan_bwd_dcb`` / ``_chunk_state_bwd_db`` /
     ``_chunk_scan_bwd_dC``): inside a chunk both follow from one ``Q x Q`` matrix per group, ``dCB``; what crosses
@@ -648,14 +663,14 @@ def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, ent_f, entr_fwd,
         r = t * w.to(bf)[..., None]
         return r.view(batch, nc, Q, groups, per * hdim).permute(0, 1, 3, 2, 4)
 
-    def states(e):         # (B, nc, H, P, N) float32 -> (B, nc, G, per * P, N) bf16
-        return e.to(bf).view(batch, nc, groups, per * hdim, nstate)
+    def states(e):         # (B, nc, H, P, N) bf16, chunks in time order -> (B, nc, G, per * P, N)
+        return e.view(batch, nc, groups, per * hdim, nstate)
 
     # dC_l += sum_{h,p} exp(cs_l) dy_l[h,p] H_in[h,p,:];  dB_s += sum_{h,p} dt_s exp(cs'_s) x_s[h,p] G_in[h,p,:]
     # with cs' the running sum of the reversed pass at that step (the decay from s to the end of its chunk and
     # over the step that follows)
-    dC = dC + _mm_f32(rows(dyc, torch.exp(blh(dA_cs))), states(ent_f))
-    dB = dB + _mm_f32(rows(xc, dte * torch.exp(blh(dA_r)).flip(1)), states(entr_fwd))
+    dC = dC + _mm_f32(rows(dyc, torch.exp(blh(dA_cs))), states(f16))
+    dB = dB + _mm_f32(rows(xc, dte * torch.exp(blh(dA_r)).flip(1)), states(r16))
     back = lambda t: t.permute(0, 1, 3, 2, 4).reshape(batch, seqlen, groups, nstate)
     return back(dB), back(dC)
 
@@ -772,12 +787,12 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     else:
         u = u_r.flip(1)
         dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
-    entr_fwd = None
+    anchor_in = None
     if (fused and cd == torch.bfloat16 and hdim in (32, 64) and Q % 32 == 0 and seqlen % Q == 0
-            and xc.is_contiguous() and Bc.is_contiguous() and Cc.is_contiguous()):
+            and (hdim * nstate) % 4 == 0 and xc.is_contiguous() and Bc.is_contiguous() and Cc.is_contiguous()):
         # the sum over a group's heads first, then two small products per chunk
-        entr_fwd = ent_r.flip(1)
-        dB, dC = _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, ent_f, entr_fwd, groups)
+        f16, r16, anchor_in = _bwd_states(ent_f.contiguous(), ent_r.contiguous())
+        dB, dC = _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, f16, r16, groups)
     else:
         Bh = Bc.repeat_interleave(per, dim=2) if per > 1 else Bc
         Ch = Cc.repeat_interleave(per, dim=2) if per > 1 else Cc
@@ -803,9 +818,10 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         a_first = torch.exp(dte[:, ::Q] * Af[None, None])                           # (B, nc, H)
         if bnd is not None:
             a_first = a_first * (~bnd[:, ::Q]).to(f32)[..., None]
-        if entr_fwd is None:
-            entr_fwd = ent_r.flip(1)
-        anchor = (entr_fwd[:, :-1] * ent_f[:, 1:]).sum(dim=(3, 4))               # (B, nc-1, H): chunks 1..
+        if anchor_in is not None:
+            anchor = anchor_in                                                     # (B, nc-1, H): chunks 1..
+        else:
+            anchor = (ent_r.flip(1)[:, :-1] * ent_f[:, 1:]).sum(dim=(3, 4))
         anchor = torch.cat([W0[:, None], a_first[:, 1:] * anchor], dim=1)
         dq = (s1 - s2).view(batch, nc, Q, heads)
         q = (anchor[:, :, None] + dq.cumsum(2) - dq).reshape(batch, seqlen, heads)

@@ -642,3 +642,17 @@ def test_bwd_dcb_kernel_matches_the_sum_over_heads_in_float64(b, l, h, p, g, Q):
     want = (m * w).sum(3)
     assert got.shape == want.shape
     torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5 * float(want.abs().max()))
+
+
+def test_bwd_states_kernel_casts_reverses_and_anchors():
+    from ssm_amd.ops import ssd as ops_ssd
+    gen = torch.Generator().manual_seed(9)
+    ent_f = torch.randn(2, 5, 3, 8, 12, generator=gen).cuda()
+    ent_r = torch.randn(2, 5, 3, 8, 12, generator=gen).cuda()
+    f16, r16, anchor = ops_ssd._bwd_states(ent_f, ent_r)
+    assert torch.equal(f16, ent_f.to(torch.bfloat16))
+    assert torch.equal(r16, ent_r.flip(1).to(torch.bfloat16))
+    want = (ent_r.flip(1)[:, :-1].double() * ent_f[:, 1:].double()).sum(dim=(3, 4))
+    torch.testing.assert_close(anchor.double(), want, rtol=1e-5, atol=1e-5)
+    f1, r1, a1 = ops_ssd._bwd_states(ent_f[:, :1].contiguous(), ent_r[:, :1].contiguous())      # a single chunk
+    assert a1.shape == (2, 0, 3) and torch.equal(r1, ent_r[:, :1].to(torch.bfloat16))
