@@ -484,6 +484,10 @@ typedef struct ssm_ssd_bwd_gate_args {
   int32_t io_dtype;          /* ssm_dtype of dout, z, x */
   int32_t dy_dtype;          /* SSM_F32 or SSM_BF16 */
   int32_t d_per_p;
+  const float *w_dy;         /* (B, L, H) fp32 or NULL: per-row weight of dy_w */
+  const float *w_x;          /* (B, L, H) fp32 or NULL: per-row weight of x_w */
+  void *dy_w;                /* (B, L, H, P) dy_dtype or NULL: dy as stored times w_dy (rows of the product for dC) */
+  void *x_w;                 /* (B, L, H, P) dy_dtype or NULL: x times w_x (rows of the product for dB) */
 } ssm_ssd_bwd_gate_args;
 int ssm_ssd_bwd_gate(const ssm_ssd_bwd_gate_args *args, void *hip_stream);
 

@@ -22,6 +22,8 @@ struct ElemParams {
   const float *ypre, *u_rev, *dt, *Dk;
   void *dy, *dy_rev;
   float *dz, *dx, *s1, *s2, *dyx, *xu;
+  const float *w_dy, *w_x;      // (B, L, H) weights of the extra row-scaled copies, or null
+  void *dy_w, *x_w;             // (B, L, H, P) dy as stored times w_dy, x times w_x, in dy's type; or null
   int batch, len, heads, hdim;
   int d_per_p, round_bf16;
   int lg;                       // lanes per row = 1 << lg
@@ -99,6 +101,20 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_gate_kernel(const ElemPara
   st4<OT>(p.dy, at, dy);
   if (p.dy_rev) st4<OT>(p.dy_rev, a.rev * p.hdim + a.c0, dy);
   if (p.dz) st4<float>(p.dz, at, dz);
+  if (p.dy_w) {
+    const float w = p.w_dy[a.row];
+    float t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = to_f32(from_f32<OT>(dy[j])) * w;
+    st4<OT>(p.dy_w, at, t);
+  }
+  if (p.x_w) {
+    const float w = p.w_x[a.row];
+    float t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = xv[j] * w;
+    st4<OT>(p.x_w, at, t);
+  }
   if (a.c0 == 0) {
     p.s2[a.row] = s2;
     p.dyx[a.row] = dyx;
@@ -259,6 +275,11 @@ extern "C" int ssm_ssd_bwd_gate(const ssm_ssd_bwd_gate_args *a, void *hip_stream
               SSM_ERR_ALIGNMENT, "ssm_ssd_bwd_gate: a pointer is not sufficiently aligned");
   p.dout = a->dout; p.z = a->z; p.x = a->x; p.ypre = a->ypre; p.Dk = a->Dskip; p.dy = a->dy; p.dy_rev = a->dy_rev;
   p.dz = a->dz; p.s2 = a->s2; p.dyx = a->dyx;
+  SSM_REQUIRE((a->dy_w == nullptr || a->w_dy != nullptr) && (a->x_w == nullptr || a->w_x != nullptr), SSM_ERR_NULL_POINTER,
+              "ssm_ssd_bwd_gate: dy_w needs w_dy and x_w needs w_x");
+  SSM_REQUIRE((!a->dy_w || aligned_to(a->dy_w, 8)) && (!a->x_w || aligned_to(a->x_w, 8)), SSM_ERR_ALIGNMENT,
+              "ssm_ssd_bwd_gate: dy_w and x_w must be 8-byte aligned");
+  p.w_dy = a->w_dy; p.w_x = a->w_x; p.dy_w = a->dy_w; p.x_w = a->x_w;
   p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.hdim = a->headdim; p.d_per_p = a->d_per_p ? 1 : 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid(elem_grid(p)), block(EB_THREADS);

@@ -560,8 +560,9 @@ def _elem_stages_ok(x, dout, z, hdim):
             and (z is None or z.dtype == x.dtype))
 
 
-def _bwd_gate(dout, z, x, ypre, Df, cd, want_rev=True):
-    """``ssm_ssd_bwd_gate``: ``(dy, dy_rev, dz, s2, dyx)``."""
+def _bwd_gate(dout, z, x, ypre, Df, cd, want_rev=True, w_dy=None, w_x=None):
+    """``ssm_ssd_bwd_gate``: ``(dy, dy_rev, dz, s2, dyx)``; with the per-row weights ``w_dy``, ``w_x (B, L, H)``
+    also ``dy * w_dy`` and ``x * w_x`` in ``dy``'s type, as the sixth and seventh result."""
     batch, seqlen, heads, hdim = (int(v) for v in x.shape)
     dev = x.device
     dy = torch.empty(batch, seqlen, heads, hdim, dtype=cd, device=dev)
@@ -569,12 +570,17 @@ def _bwd_gate(dout, z, x, ypre, Df, cd, want_rev=True):
     dz = torch.empty(batch, seqlen, heads, hdim, dtype=torch.float32, device=dev) if z is not None else None
     s2 = torch.empty(batch, seqlen, heads, dtype=torch.float32, device=dev)
     dyx = torch.empty_like(s2)
+    dy_w = torch.empty_like(dy) if w_dy is not None else None
+    x_w = torch.empty_like(dy) if w_x is not None else None
     args = _lib.SsdBwdGateArgs(
         dout=_lib.ptr(dout), z=_lib.ptr(z), x=_lib.ptr(x), ypre=_lib.ptr(ypre), Dskip=_lib.ptr(Df), dy=_lib.ptr(dy),
         dy_rev=_lib.ptr(dy_rev), dz=_lib.ptr(dz), s2=_lib.ptr(s2), dyx=_lib.ptr(dyx), batch=batch, seqlen=seqlen,
         heads=heads, headdim=hdim, io_dtype=_lib.dtype_enum(x.dtype), dy_dtype=_lib.dtype_enum(cd),
-        d_per_p=int(Df is not None and Df.ndim == 2))
+        d_per_p=int(Df is not None and Df.ndim == 2), w_dy=_lib.ptr(w_dy), w_x=_lib.ptr(w_x), dy_w=_lib.ptr(dy_w),
+        x_w=_lib.ptr(x_w))
     _lib.call("ssm_ssd_bwd_gate", args, dev)
+    if w_dy is not None or w_x is not None:
+        return dy, dy_rev, dz, s2, dyx, dy_w, x_w
     return dy, dy_rev, dz, s2, dyx
 
 
@@ -639,12 +645,12 @@ def _mm_f32(a, b):
         return torch.matmul(a, b).float()
 
 
-def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, f16, r16, groups):
+def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dA_cs, wdy, xw, f16, r16, groups):
     """``dB`` and ``dC`` ``(B, L, G, N)`` with the sum over a group's heads taken before the products with ``C`` and
     ``B`` (state-spaces/mamba ssd_combined.py, ``_chunk_scan_bwd_dcb`` / ``_chunk_state_bwd_db`` /
     ``_chunk_scan_bwd_dC``): inside a chunk both follow from one ``Q x Q`` matrix per group, ``dCB``; what crosses
-    chunk boundaries is a product of the weighted ``x`` (``dy``) rows, all heads of the group side by side, with
-    the adjoint (forward) states entering the chunk."""
+    chunk boundaries is a product of the weighted ``x`` (``dy``) rows ``xw`` (``wdy``), all heads of the group side by
+    side, with the adjoint (forward) states entering the chunk, ``r16`` (``f16``)."""
     batch, seqlen, heads, hdim = (int(v) for v in xc.shape)
     nc, Q = int(dA_cs.shape[2]), int(dA_cs.shape[3])
     nstate = int(Bc.shape[-1])
@@ -656,21 +662,15 @@ def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, f16, r16, groups
     dB = torch.matmul(dCB.transpose(-1, -2), Cg)
     dC = torch.matmul(dCB, Bg)
 
-    def blh(t_c):
-        return t_c.permute(0, 2, 3, 1).reshape(batch, seqlen, heads)
-
-    def rows(t, w):        # (B, L, H, P) bf16 scaled per (step, head) -> (B, nc, G, Q, per * P)
-        r = t * w.to(bf)[..., None]
-        return r.view(batch, nc, Q, groups, per * hdim).permute(0, 1, 3, 2, 4)
+    def rows(t):           # (B, L, H, P) -> (B, nc, G, Q, per * P)
+        return t.view(batch, nc, Q, groups, per * hdim).permute(0, 1, 3, 2, 4)
 
     def states(e):         # (B, nc, H, P, N) bf16, chunks in time order -> (B, nc, G, per * P, N)
         return e.view(batch, nc, groups, per * hdim, nstate)
 
-    # dC_l += sum_{h,p} exp(cs_l) dy_l[h,p] H_in[h,p,:];  dB_s += sum_{h,p} dt_s exp(cs'_s) x_s[h,p] G_in[h,p,:]
-    # with cs' the running sum of the reversed pass at that step (the decay from s to the end of its chunk and
-    # over the step that follows)
-    dC = dC + _mm_f32(rows(dyc, torch.exp(blh(dA_cs))), states(f16))
-    dB = dB + _mm_f32(rows(xc, dte * torch.exp(blh(dA_r)).flip(1)), states(r16))
+    # dC_l += sum_{h,p} (exp(cs_l) dy_l)[h,p] H_in[h,p,:];  dB_s += sum_{h,p} (dt_s exp(cs'_s) x_s)[h,p] G_in[h,p,:]
+    dC = dC + _mm_f32(rows(wdy), states(f16))
+    dB = dB + _mm_f32(rows(xw), states(r16))
     back = lambda t: t.permute(0, 1, 3, 2, 4).reshape(batch, seqlen, groups, nstate)
     return back(dB), back(dC)
 
@@ -751,9 +751,26 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     dte = dte.contiguous()
     xt = (dte[..., None] * xd).to(cd)
     ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
+    # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
+    dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
+    dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
+    if bnd is not None:                       # the reversed passes decay by the following step's factor
+        dA_r = dA_r + jumps(torch.cat([bnd[:, 1:], torch.zeros_like(bnd[:, :1])], dim=1).flip(1))
+    # dB and dC with the sum over a group's heads taken first (two small products per chunk)?
+    chunked = (fused and cd == torch.bfloat16 and hdim in (32, 64) and Q % 32 == 0 and seqlen % Q == 0
+               and (hdim * nstate) % 4 == 0 and xc.is_contiguous() and Bc.is_contiguous() and Cc.is_contiguous())
     dD = None
-    if fused:
+    wdy = xw = None
+    if fused and chunked:
+        # the rows of the two products across chunk boundaries leave the gate kernel with their weights on:
+        # dy_l exp(cs_l) for dC, x_s dt_s exp(cs'_s) for dB, cs' the running sum of the reversed pass at that step
+        # (the decay from s to the end of its chunk and over the step that follows)
+        w_dy = torch.exp(blh(dA_cs)).contiguous()
+        w_x = (dte * torch.exp(blh(dA_r)).flip(1)).contiguous()
+        dyc, dyr, dz, s2, dyx, wdy, xw = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, w_dy=w_dy, w_x=w_x)
+    elif fused:
         dyc, dyr, dz, s2, dyx = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd)
+    if fused:
         if Df is not None and Df.ndim == 1:
             dD = dyx.sum(dim=(0, 1))
         elif Df is not None:
@@ -769,11 +786,6 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
             dy, dz = dof, None
         if Df is not None:
             dD = (dy * xf).sum(dim=(0, 1, 3)) if Df.ndim == 1 else (dy * xf).sum(dim=(0, 1))
-    # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
-    dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
-    dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
-    if bnd is not None:                       # the reversed passes decay by the following step's factor
-        dA_r = dA_r + jumps(torch.cat([bnd[:, 1:], torch.zeros_like(bnd[:, :1])], dim=1).flip(1))
     if not fused:
         dyc = dy.to(cd)
         dyr = dyc.flip(1).contiguous()
@@ -788,11 +800,9 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         u = u_r.flip(1)
         dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
     anchor_in = None
-    if (fused and cd == torch.bfloat16 and hdim in (32, 64) and Q % 32 == 0 and seqlen % Q == 0
-            and (hdim * nstate) % 4 == 0 and xc.is_contiguous() and Bc.is_contiguous() and Cc.is_contiguous()):
-        # the sum over a group's heads first, then two small products per chunk
+    if chunked:
         f16, r16, anchor_in = _bwd_states(ent_f.contiguous(), ent_r.contiguous())
-        dB, dC = _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dte, dA_cs, dA_r, f16, r16, groups)
+        dB, dC = _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dA_cs, wdy, xw, f16, r16, groups)
     else:
         Bh = Bc.repeat_interleave(per, dim=2) if per > 1 else Bc
         Ch = Cc.repeat_interleave(per, dim=2) if per > 1 else Cc
