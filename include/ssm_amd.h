@@ -477,7 +477,7 @@ typedef struct ssm_ssd_bwd_gate_args {
   const float *Dskip;        /* (H,) or (H, P) if d_per_p, or NULL */
   void *dy;                  /* (B, L, H, P) dy_dtype */
   void *dy_rev;              /* (B, L, H, P) dy_dtype, time reversed, or NULL */
-  float *dz;                 /* (B, L, H, P) fp32; NULL exactly when z is */
+  void *dz;                  /* (B, L, H, P) fp32 (io_dtype with dz_in_io_dtype); NULL exactly when z is */
   float *s2;                 /* (B, L, H) fp32 */
   float *dyx;                /* (B, L, H) fp32 */
   int32_t batch, seqlen, heads, headdim;
@@ -488,6 +488,7 @@ typedef struct ssm_ssd_bwd_gate_args {
   const float *w_x;          /* (B, L, H) fp32 or NULL: per-row weight of x_w */
   void *dy_w;                /* (B, L, H, P) dy_dtype or NULL: dy as stored times w_dy (rows of the product for dC) */
   void *x_w;                 /* (B, L, H, P) dy_dtype or NULL: x times w_x (rows of the product for dB) */
+  int32_t dz_in_io_dtype;    /* nonzero: dz is written in io_dtype instead of fp32 */
 } ssm_ssd_bwd_gate_args;
 int ssm_ssd_bwd_gate(const ssm_ssd_bwd_gate_args *args, void *hip_stream);
 
@@ -498,11 +499,12 @@ typedef struct ssm_ssd_bwd_dx_args {
   const float *u_rev;        /* (B, L, H, P) fp32, time reversed */
   const float *dt;           /* (B, L, H) fp32: the step after bias, softplus and clamp */
   const float *Dskip;        /* (H,) or (H, P) if d_per_p, or NULL */
-  float *dx;                 /* (B, L, H, P) fp32 */
+  void *dx;                  /* (B, L, H, P) fp32 (io_dtype with dx_in_io_dtype) */
   float *xu;                 /* (B, L, H) fp32 */
   float *s1;                 /* (B, L, H) fp32 */
   int32_t batch, seqlen, heads, headdim;
   int32_t io_dtype, d_per_p, round_bf16;
+  int32_t dx_in_io_dtype;    /* nonzero: dx is written in io_dtype instead of fp32 */
 } ssm_ssd_bwd_dx_args;
 int ssm_ssd_bwd_dx(const ssm_ssd_bwd_dx_args *args, void *hip_stream);
 

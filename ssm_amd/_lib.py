@@ -182,13 +182,13 @@ class SsdBwdGateArgs(C.Structure):
     _fields_ = [("dout", _vp), ("z", _vp), ("x", _vp), ("ypre", _vp), ("Dskip", _vp), ("dy", _vp), ("dy_rev", _vp),
                 ("dz", _vp), ("s2", _vp), ("dyx", _vp), ("batch", _i32), ("seqlen", _i32), ("heads", _i32),
                 ("headdim", _i32), ("io_dtype", _i32), ("dy_dtype", _i32), ("d_per_p", _i32), ("w_dy", _vp),
-                ("w_x", _vp), ("dy_w", _vp), ("x_w", _vp)]
+                ("w_x", _vp), ("dy_w", _vp), ("x_w", _vp), ("dz_in_io_dtype", _i32)]
 
 
 class SsdBwdDxArgs(C.Structure):
     _fields_ = [("dout", _vp), ("z", _vp), ("x", _vp), ("u_rev", _vp), ("dt", _vp), ("Dskip", _vp), ("dx", _vp),
                 ("xu", _vp), ("s1", _vp), ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("headdim", _i32),
-                ("io_dtype", _i32), ("d_per_p", _i32), ("round_bf16", _i32)]
+                ("io_dtype", _i32), ("d_per_p", _i32), ("round_bf16", _i32), ("dx_in_io_dtype", _i32)]
 
 
 class SsdBwdDbArgs(C.Structure):

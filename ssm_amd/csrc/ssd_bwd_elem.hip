@@ -21,7 +21,9 @@ struct ElemParams {
   const void *dout, *z, *x;
   const float *ypre, *u_rev, *dt, *Dk;
   void *dy, *dy_rev;
-  float *dz, *dx, *s1, *s2, *dyx, *xu;
+  void *dz, *dx;                // float32, or the type of dout / x with grads_io
+  float *s1, *s2, *dyx, *xu;
+  int grads_io;
   const float *w_dy, *w_x;      // (B, L, H) weights of the extra row-scaled copies, or null
   void *dy_w, *x_w;             // (B, L, H, P) dy as stored times w_dy, x times w_x, in dy's type; or null
   int batch, len, heads, hdim;
@@ -100,7 +102,10 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_gate_kernel(const ElemPara
   if (!a.live) return;
   st4<OT>(p.dy, at, dy);
   if (p.dy_rev) st4<OT>(p.dy_rev, a.rev * p.hdim + a.c0, dy);
-  if (p.dz) st4<float>(p.dz, at, dz);
+  if (p.dz) {
+    if (p.grads_io) st4<IO>(p.dz, at, dz);
+    else st4<float>(p.dz, at, dz);
+  }
   if (p.dy_w) {
     const float w = p.w_dy[a.row];
     float t[4];
@@ -145,7 +150,8 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_dx_kernel(const ElemParams
   xu = row_sum(xu, p.lg);
   s1 = row_sum(s1, p.lg);
   if (!a.live) return;
-  st4<float>(p.dx, at, dx);
+  if (p.grads_io) st4<IO>(p.dx, at, dx);
+  else st4<float>(p.dx, at, dx);
   if (a.c0 == 0) {
     p.xu[a.row] = xu;
     p.s1[a.row] = s1;
@@ -280,6 +286,7 @@ extern "C" int ssm_ssd_bwd_gate(const ssm_ssd_bwd_gate_args *a, void *hip_stream
   SSM_REQUIRE((!a->dy_w || aligned_to(a->dy_w, 8)) && (!a->x_w || aligned_to(a->x_w, 8)), SSM_ERR_ALIGNMENT,
               "ssm_ssd_bwd_gate: dy_w and x_w must be 8-byte aligned");
   p.w_dy = a->w_dy; p.w_x = a->w_x; p.dy_w = a->dy_w; p.x_w = a->x_w;
+  p.grads_io = a->dz_in_io_dtype ? 1 : 0;
   p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.hdim = a->headdim; p.d_per_p = a->d_per_p ? 1 : 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid(elem_grid(p)), block(EB_THREADS);
@@ -320,6 +327,7 @@ extern "C" int ssm_ssd_bwd_dx(const ssm_ssd_bwd_dx_args *a, void *hip_stream) {
   p.dx = a->dx; p.xu = a->xu; p.s1 = a->s1;
   p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.hdim = a->headdim; p.d_per_p = a->d_per_p ? 1 : 0;
   p.round_bf16 = a->round_bf16 ? 1 : 0;
+  p.grads_io = a->dx_in_io_dtype ? 1 : 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid(elem_grid(p)), block(EB_THREADS);
   switch (a->io_dtype) {

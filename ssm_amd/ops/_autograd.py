@@ -219,7 +219,7 @@ class SsdCombinedFn(torch.autograd.Function):
             grad_y = torch.zeros_like(x)
         dx, ddt, dA, dB, dC, dD, dz, dbias, dinit = ssd_combined_backward(
             grad_y, grad_final, x, dt, A, B, C, Q, D=D, z=z, dt_bias=dt_bias, initial_states=init,
-            dt_softplus=softplus, dt_limit=limit, seq_idx=ctx.seq_idx)
+            dt_softplus=softplus, dt_limit=limit, seq_idx=ctx.seq_idx, grads_in_input_dtype=True)
         need = ctx.needs_input_grad
         pick = lambda i, g, r: _like(g, r) if (r is not None and g is not None and need[i]) else None
         return (pick(0, dx, x), pick(1, ddt, dt), pick(2, dA, A), pick(3, dB, B), pick(4, dC, C), None,

@@ -560,14 +560,15 @@ def _elem_stages_ok(x, dout, z, hdim):
             and (z is None or z.dtype == x.dtype))
 
 
-def _bwd_gate(dout, z, x, ypre, Df, cd, want_rev=True, w_dy=None, w_x=None):
+def _bwd_gate(dout, z, x, ypre, Df, cd, want_rev=True, w_dy=None, w_x=None, grads_io=False):
     """``ssm_ssd_bwd_gate``: ``(dy, dy_rev, dz, s2, dyx)``; with the per-row weights ``w_dy``, ``w_x (B, L, H)``
     also ``dy * w_dy`` and ``x * w_x`` in ``dy``'s type, as the sixth and seventh result."""
     batch, seqlen, heads, hdim = (int(v) for v in x.shape)
     dev = x.device
     dy = torch.empty(batch, seqlen, heads, hdim, dtype=cd, device=dev)
     dy_rev = torch.empty_like(dy) if want_rev else None
-    dz = torch.empty(batch, seqlen, heads, hdim, dtype=torch.float32, device=dev) if z is not None else None
+    dz = (torch.empty(batch, seqlen, heads, hdim, dtype=x.dtype if grads_io else torch.float32, device=dev)
+          if z is not None else None)
     s2 = torch.empty(batch, seqlen, heads, dtype=torch.float32, device=dev)
     dyx = torch.empty_like(s2)
     dy_w = torch.empty_like(dy) if w_dy is not None else None
@@ -577,24 +578,25 @@ def _bwd_gate(dout, z, x, ypre, Df, cd, want_rev=True, w_dy=None, w_x=None):
         dy_rev=_lib.ptr(dy_rev), dz=_lib.ptr(dz), s2=_lib.ptr(s2), dyx=_lib.ptr(dyx), batch=batch, seqlen=seqlen,
         heads=heads, headdim=hdim, io_dtype=_lib.dtype_enum(x.dtype), dy_dtype=_lib.dtype_enum(cd),
         d_per_p=int(Df is not None and Df.ndim == 2), w_dy=_lib.ptr(w_dy), w_x=_lib.ptr(w_x), dy_w=_lib.ptr(dy_w),
-        x_w=_lib.ptr(x_w))
+        x_w=_lib.ptr(x_w), dz_in_io_dtype=int(bool(grads_io)))
     _lib.call("ssm_ssd_bwd_gate", args, dev)
     if w_dy is not None or w_x is not None:
         return dy, dy_rev, dz, s2, dyx, dy_w, x_w
     return dy, dy_rev, dz, s2, dyx
 
 
-def _bwd_dx(dout, z, x, u_rev, dte, Df, round_bf16):
+def _bwd_dx(dout, z, x, u_rev, dte, Df, round_bf16, grads_io=False):
     """``ssm_ssd_bwd_dx``: ``(dx, xu, s1)``."""
     batch, seqlen, heads, hdim = (int(v) for v in x.shape)
     dev = x.device
-    dx = torch.empty(batch, seqlen, heads, hdim, dtype=torch.float32, device=dev)
+    dx = torch.empty(batch, seqlen, heads, hdim, dtype=x.dtype if grads_io else torch.float32, device=dev)
     xu = torch.empty(batch, seqlen, heads, dtype=torch.float32, device=dev)
     s1 = torch.empty_like(xu)
     args = _lib.SsdBwdDxArgs(
         dout=_lib.ptr(dout), z=_lib.ptr(z), x=_lib.ptr(x), u_rev=_lib.ptr(u_rev), dt=_lib.ptr(dte), Dskip=_lib.ptr(Df),
         dx=_lib.ptr(dx), xu=_lib.ptr(xu), s1=_lib.ptr(s1), batch=batch, seqlen=seqlen, heads=heads, headdim=hdim,
-        io_dtype=_lib.dtype_enum(x.dtype), d_per_p=int(Df is not None and Df.ndim == 2), round_bf16=int(bool(round_bf16)))
+        io_dtype=_lib.dtype_enum(x.dtype), d_per_p=int(Df is not None and Df.ndim == 2), round_bf16=int(bool(round_bf16)),
+        dx_in_io_dtype=int(bool(grads_io)))
     _lib.call("ssm_ssd_bwd_dx", args, dev)
     return dx, xu, s1
 
@@ -676,7 +678,8 @@ def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dA_cs, wdy, xw, f16, r16, groups):
 
 
 def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
-                          initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")), seq_idx=None):
+                          initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")), seq_idx=None,
+                          grads_in_input_dtype=False):
     """Gradients of :func:`ssd_combined` (outputs ``y`` and ``final_states``).
 
     With ``a_t = exp(dt_t A)``, ``H_t = a_t H_{t-1} + dt_t x_t (x) B_t`` and the adjoint state
@@ -705,7 +708,9 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         (others): the arguments of the forward.
 
     Returns:
-        ``(dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)`` in float32 (``None`` for absent inputs).
+        ``(dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)`` in float32 (``None`` for absent inputs); with
+        ``grads_in_input_dtype`` the two large ones, ``dx`` and ``dz``, come back in ``x.dtype`` where the fused
+        element-wise stages write them (one rounding, as a cast afterwards would give).
     """
     batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
     Q = int(chunk_size)
@@ -767,9 +772,10 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         # (the decay from s to the end of its chunk and over the step that follows)
         w_dy = torch.exp(blh(dA_cs)).contiguous()
         w_x = (dte * torch.exp(blh(dA_r)).flip(1)).contiguous()
-        dyc, dyr, dz, s2, dyx, wdy, xw = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, w_dy=w_dy, w_x=w_x)
+        dyc, dyr, dz, s2, dyx, wdy, xw = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, w_dy=w_dy, w_x=w_x,
+                                                     grads_io=grads_in_input_dtype)
     elif fused:
-        dyc, dyr, dz, s2, dyx = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd)
+        dyc, dyr, dz, s2, dyx = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, grads_io=grads_in_input_dtype)
     if fused:
         if Df is not None and Df.ndim == 1:
             dD = dyx.sum(dim=(0, 1))
@@ -795,7 +801,8 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     if bnd is not None:
         dinit = dinit * (~bnd[:, 0]).to(f32)[:, None, None, None]
     if fused:
-        dx, xu, s1 = _bwd_dx(dod, zd, xd, u_r.contiguous(), dte, Df, cd == torch.bfloat16)
+        dx, xu, s1 = _bwd_dx(dod, zd, xd, u_r.contiguous(), dte, Df, cd == torch.bfloat16,
+                             grads_io=grads_in_input_dtype)
     else:
         u = u_r.flip(1)
         dx = dte[..., None] * u + (0.0 if Df is None else (Df[None, None, :, None] if Df.ndim == 1 else Df[None, None]) * dy)
