@@ -547,6 +547,18 @@ typedef struct ssm_ssd_bwd_states_args {
 } ssm_ssd_bwd_states_args;
 int ssm_ssd_bwd_states(const ssm_ssd_bwd_states_args *args, void *hip_stream);
 
+/* out[row][:] = x[row][:] * w[row], the product formed in float32 and rounded once to `out_dtype`: the operand
+ * dt x of the backward's first pass.  `cols` a multiple of 4.  No counterpart in the reference. */
+typedef struct ssm_ssd_scale_rows_args {
+  const void *x;             /* (rows, cols) x_dtype */
+  const float *w;            /* (rows,) fp32 */
+  void *out;                 /* (rows, cols) out_dtype */
+  int64_t rows;
+  int32_t cols;
+  int32_t x_dtype, out_dtype;   /* out_dtype: SSM_F32 or SSM_BF16 */
+} ssm_ssd_scale_rows_args;
+int ssm_ssd_scale_rows(const ssm_ssd_scale_rows_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).
  * Forward stands behind `dw_causal_conv(x, weight, bias, activation)`

@@ -206,6 +206,11 @@ class SsdBwdStatesArgs(C.Structure):
                 ("batch", _i32), ("nchunks", _i32), ("heads", _i32), ("dim", _i32)]
 
 
+class SsdScaleRowsArgs(C.Structure):
+    _fields_ = [("x", _vp), ("w", _vp), ("out", _vp), ("rows", C.c_int64), ("cols", _i32), ("x_dtype", _i32),
+                ("out_dtype", _i32)]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -269,6 +274,7 @@ ENTRY_POINTS = {
     "ssm_ssd_bwd_db": SsdBwdDbArgs,
     "ssm_ssd_bwd_dcb": SsdBwdDcbArgs,
     "ssm_ssd_bwd_states": SsdBwdStatesArgs,
+    "ssm_ssd_scale_rows": SsdScaleRowsArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_conv1d_update": Conv1dUpdateArgs,

@@ -259,6 +259,29 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_states_kernel(const States
   }
 }
 
+// out[row][:] = x[row][:] * w[row], formed in float32 and rounded once: the step-weighted operand of the first pass.
+struct ScaleParams {
+  const void *x;
+  const float *w;
+  void *out;
+  size_t rows;
+  int cols;
+};
+
+template <typename IO, typename OT>
+__global__ __launch_bounds__(EB_THREADS) void ssd_scale_rows_kernel(const ScaleParams p) {
+  const size_t quads = p.rows * (size_t)(p.cols / 4);
+  const size_t gid = (size_t)blockIdx.x * EB_THREADS + threadIdx.x;
+  if (gid >= quads) return;
+  const size_t row = gid / (size_t)(p.cols / 4);
+  const float w = p.w[row];
+  float v[4];
+  ld4<IO>(p.x, gid * 4, v);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] *= w;
+  st4<OT>(p.out, gid * 4, v);
+}
+
 }  // namespace
 }  // namespace ssm
 
@@ -379,5 +402,32 @@ extern "C" int ssm_ssd_bwd_states(const ssm_ssd_bwd_states_args *a, void *hip_st
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   hipLaunchKernelGGL(ssd_bwd_states_kernel, dim3((unsigned)grid), dim3(EB_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_bwd_states");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_scale_rows(const ssm_ssd_scale_rows_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_scale_rows: args is NULL");
+  SSM_REQUIRE(a->x && a->w && a->out, SSM_ERR_NULL_POINTER, "ssm_ssd_scale_rows: x, w and out are required");
+  SSM_REQUIRE(a->rows > 0 && a->cols > 0 && a->cols % 4 == 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_scale_rows: rows must be positive and cols=%d a positive multiple of 4", a->cols);
+  SSM_REQUIRE(valid_dtype(a->x_dtype) && (a->out_dtype == SSM_F32 || a->out_dtype == SSM_BF16), SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_scale_rows: x_dtype=%d, out_dtype=%d (float32 or bfloat16)", a->x_dtype, a->out_dtype);
+  SSM_REQUIRE(aligned_to(a->x, 4 * dtype_size(a->x_dtype)) && aligned_to(a->out, 4 * dtype_size(a->out_dtype)),
+              SSM_ERR_ALIGNMENT, "ssm_ssd_scale_rows: x and out must be aligned to four elements");
+  ScaleParams p{};
+  p.x = a->x; p.w = a->w; p.out = a->out; p.rows = (size_t)a->rows; p.cols = a->cols;
+  const size_t quads = p.rows * (size_t)(p.cols / 4);
+  SSM_REQUIRE(quads < ((size_t)1 << 39), SSM_ERR_TOO_LARGE, "ssm_ssd_scale_rows: tensor too large");
+  const dim3 grid((unsigned)((quads + EB_THREADS - 1) / EB_THREADS)), block(EB_THREADS);
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+#define SSM_SCALE(IO)                                                                                          \
+  {                                                                                                            \
+    if (a->out_dtype == SSM_F32) hipLaunchKernelGGL((ssd_scale_rows_kernel<IO, float>), grid, block, 0, s, p);  \
+    else hipLaunchKernelGGL((ssd_scale_rows_kernel<IO, bf16_t>), grid, block, 0, s, p);                         \
+  }
+  if (a->x_dtype == SSM_F32) SSM_SCALE(float) else if (a->x_dtype == SSM_BF16) SSM_SCALE(bf16_t) else SSM_SCALE(f16_t)
+#undef SSM_SCALE
+  SSM_CHECK_LAUNCH("ssm_ssd_scale_rows");
   return SSM_OK;
 }

@@ -623,6 +623,16 @@ def _bwd_dcb(dy, x, dt_c, dA_cs, groups):
     return out
 
 
+def _scale_rows(x, w, out_dtype):
+    """``ssm_ssd_scale_rows``: ``x * w[..., None]`` formed in float32 and rounded once to ``out_dtype``."""
+    cols = int(x.shape[-1])
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    args = _lib.SsdScaleRowsArgs(x=_lib.ptr(x), w=_lib.ptr(w), out=_lib.ptr(out), rows=x.numel() // cols, cols=cols,
+                                 x_dtype=_lib.dtype_enum(x.dtype), out_dtype=_lib.dtype_enum(out_dtype))
+    _lib.call("ssm_ssd_scale_rows", args, x.device)
+    return out
+
+
 def _bwd_states(ent_f, ent_r):
     """``ssm_ssd_bwd_states``: both stacks of chunk-boundary states as bfloat16 with chunks in time order, and the
     anchors ``<adjoint state, forward state>`` at the boundaries ``1..nc-1`` ``(B, nc-1, H)``."""
@@ -754,7 +764,7 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
 
         dA_cs = dA_cs + jumps(bnd)
     dte = dte.contiguous()
-    xt = (dte[..., None] * xd).to(cd)
+    xt = _scale_rows(xd, dte, cd) if (fused and cd in (torch.float32, torch.bfloat16)) else (dte[..., None] * xd).to(cd)
     ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
     # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
     dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()

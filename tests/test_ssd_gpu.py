@@ -656,3 +656,14 @@ def test_bwd_states_kernel_casts_reverses_and_anchors():
     torch.testing.assert_close(anchor.double(), want, rtol=1e-5, atol=1e-5)
     f1, r1, a1 = ops_ssd._bwd_states(ent_f[:, :1].contiguous(), ent_r[:, :1].contiguous())      # a single chunk
     assert a1.shape == (2, 0, 3) and torch.equal(r1, ent_r[:, :1].to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_scale_rows_kernel_rounds_once(dtype):
+    from ssm_amd.ops import ssd as ops_ssd
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 37, 5, 12, generator=gen).to(dtype).cuda()
+    w = torch.rand(3, 37, 5, generator=gen).cuda()
+    got = ops_ssd._scale_rows(x, w, torch.bfloat16)
+    assert torch.equal(got, (w[..., None] * x.float()).to(torch.bfloat16))
+    assert torch.equal(ops_ssd._scale_rows(x, w, torch.float32), w[..., None] * x.float())
