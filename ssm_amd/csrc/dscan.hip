@@ -141,6 +141,122 @@ __global__ __launch_bounds__(DS_THREADS) void dscan_kernel(const DscanParams p) 
   }
 }
 
+// ---------------------------------------------------------------- one pass
+// The common call (per-token B and C of X's shape and type, per-head A and D, gate of X's shape or none) with
+// every input read once.  A workgroup of eight waves owns 64 * VEC neighbouring channels of one batch row (a
+// lane VEC of them, so that a wave's access is 128 * VEC bytes of 16-bit elements) and walks time in rounds of
+// 64 steps, wave w taking steps 8w..8w+7 of the round: it folds its steps from zero into (decay product, state),
+// the eight folds meet in LDS (one barrier per round, two buffers), every wave chains them from the state carried
+// into the round -- which gives it the state entering its own steps and, in the same sweep, the state carried
+// into the next round -- and replays its steps from the values it still holds in registers.  The reads of the
+// next round are requested before the arithmetic of this one.  All workgroups are resident at once and the call
+// is bound by memory, so it does not matter that they are fewer than the CUs can hold.
+constexpr int DO_WAVES = 16, DO_SEG = 8, DO_ROUND = DO_WAVES * DO_SEG;
+
+template <typename io_t, int VEC>
+struct DoRegs {
+  float dt[DO_SEG];
+  Pack<io_t, VEC> x[DO_SEG], bq[DO_SEG], cq[DO_SEG], zq[DO_SEG];
+};
+
+template <typename io_t, int VEC, bool HAS_Z>
+__global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const DscanParams p) {
+  __shared__ float4 segs[2][DO_WAVES][WAVE];
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int HP = p.heads * p.proj;
+  const int ch = ((int)blockIdx.x * WAVE + lane) * VEC;
+  const int b = blockIdx.y;
+  const int h = ch / p.proj;
+  const int L = p.len;
+  const int valid = p.lengths ? min(max(p.lengths[b], 0), L) : L;
+  const float A2 = p.A[h] * LOG2E;
+  const float Dk = p.Dk ? p.Dk[h] : 0.0f;
+  const io_t *X = reinterpret_cast<const io_t *>(p.X), *Bp = reinterpret_cast<const io_t *>(p.Bp);
+  const io_t *Cp = reinterpret_cast<const io_t *>(p.Cp), *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.X);
+  const float *DT = reinterpret_cast<const float *>(p.dt);
+  io_t *Y = reinterpret_cast<io_t *>(p.Y);
+  const size_t row0 = (size_t)b * L;
+  float carry[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) carry[v] = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + ch + v) : 0.0f;
+
+  auto request = [&](DoRegs<io_t, VEC> &r, int round) {
+    const int t0 = round * DO_ROUND + wave * DO_SEG;
+#pragma unroll
+    for (int j = 0; j < DO_SEG; ++j) {
+      const size_t row = row0 + min(t0 + j, L - 1);            // steps past the end read the last row, unused
+      const size_t at = row * HP + ch;
+      r.dt[j] = DT[row * p.heads + h];
+      r.x[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(X + at);
+      r.bq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Bp + at);
+      r.cq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Cp + at);
+      if (HAS_Z) r.zq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Z + at);
+    }
+  };
+
+  const int rounds = (L + DO_ROUND - 1) / DO_ROUND;
+  DoRegs<io_t, VEC> cur, nxt;
+  request(cur, 0);
+  for (int r = 0; r < rounds; ++r) {
+    if (r + 1 < rounds) request(nxt, r + 1);
+    const int t0 = r * DO_ROUND + wave * DO_SEG;
+    float a[DO_SEG], inc[VEC][DO_SEG], s[VEC], prod = 1.0f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) s[v] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < DO_SEG; ++j) {
+      const bool live = t0 + j < valid;                        // past the row's length: the identity, nothing added
+      a[j] = live ? exp2_hw(cur.dt[j] * A2) : 1.0f;
+      prod *= a[j];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        inc[v][j] = live ? cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]) : 0.0f;
+        s[v] = __builtin_fmaf(a[j], s[v], inc[v][j]);
+      }
+    }
+    segs[r & 1][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
+    __syncthreads();
+    float e[VEC], enter[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) e[v] = enter[v] = carry[v];
+#pragma unroll
+    for (int w = 0; w < DO_WAVES; ++w) {
+      const float4 f = segs[r & 1][w][lane];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        enter[v] = w == wave ? e[v] : enter[v];
+        e[v] = __builtin_fmaf(f.x, e[v], v == 0 ? f.y : f.z);
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      carry[v] = e[v];
+      s[v] = enter[v];
+    }
+#pragma unroll
+    for (int j = 0; j < DO_SEG; ++j) {
+      const int t = t0 + j;
+      Pack<io_t, VEC> o;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        s[v] = __builtin_fmaf(a[j], s[v], inc[v][j]);
+        float y = __builtin_fmaf(s[v], to_f32(cur.cq[j].v[v]), Dk * to_f32(cur.x[j].v[v]));
+        if (HAS_Z) y *= silu_f32(to_f32(cur.zq[j].v[v]));
+        o.v[v] = from_f32<io_t>(t < valid ? y : 0.0f);
+      }
+      if (t < L) *reinterpret_cast<Pack<io_t, VEC> *>(Y + (row0 + t) * HP + ch) = o;
+    }
+    cur = nxt;
+  }
+}
+
+template <typename io_t, int VEC>
+static void launch_onepass(const DscanParams &p, hipStream_t s) {
+  const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
+  if (p.z) hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, true>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
+  else hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, false>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
+}
+
 int dscan_segments(int batch, int len, int hp) {
   // enough (segment, channel-block) workgroups to cover ~4 per CU, segments of >= 32 steps
   const int blocks = (hp + DS_THREADS - 1) / DS_THREADS;
@@ -204,6 +320,21 @@ extern "C" int ssm_dscan_fwd(const ssm_dscan_fwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid((unsigned)((HP + DS_THREADS - 1) / DS_THREADS), (unsigned)p.nseg, (unsigned)a->batch);
   const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
+  // one pass: per-token B and C, per-head A and D, a gate of X's shape or none, channels in whole waves
+  {
+    const int vec = a->x_dtype == SSM_F32 ? 1 : 2;
+    const size_t bytes = (size_t)vec * dtype_size(a->x_dtype);
+    if (typed && a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP && !a->a_per_p && !a->d_per_p &&
+        (!a->z || a->z_per_p) && HP % (WAVE * vec) == 0 && a->proj % vec == 0 && aligned_to(a->X, bytes) &&
+        aligned_to(a->Bproj, bytes) && aligned_to(a->Cproj, bytes) && aligned_to(a->Y, bytes) &&
+        (!a->z || aligned_to(a->z, bytes)) && a->batch < 65536) {
+      if (a->x_dtype == SSM_BF16) launch_onepass<bf16_t, 2>(p, s);
+      else if (a->x_dtype == SSM_F16) launch_onepass<f16_t, 2>(p, s);
+      else launch_onepass<float, 1>(p, s);
+      SSM_CHECK_LAUNCH("ssm_dscan_fwd");
+      return SSM_OK;
+    }
+  }
 #define SSM_DS_LAUNCH(T)                                                                   \
   {                                                                                        \
     if (p.nseg > 1) hipLaunchKernelGGL((dscan_kernel<1, T>), grid, dim3(DS_THREADS), 0, s, p); \

@@ -177,3 +177,25 @@ def test_backward_bf16_activations():
         scale = float(want[k].abs().max()) + 1e-6
         torch.testing.assert_close(got[k].float().cpu().double(), want[k], rtol=3e-2, atol=3e-2 * scale,
                                    msg=lambda m, n=k: f"grad {n}: {m}")
+
+
+# ------------------------------------------------------------------ the one-pass kernel's call shape
+
+@pytest.mark.parametrize("dtype,hp", [(torch.bfloat16, (4, 64)), (torch.float16, (2, 64)), (torch.float32, (3, 64)),
+                                      (torch.bfloat16, (8, 32))], ids=lambda v: str(v).replace("torch.", ""))
+@pytest.mark.parametrize("length,z_mode,d_mode,init,ragged", [(333, 4, "vec", True, False), (128, 0, "none", False, False),
+                                                               (1000, 4, "vec", False, True), (7, 4, "none", True, True)])
+def test_one_pass_call_shape(dtype, hp, length, z_mode, d_mode, init, ragged):
+    """Per-token B and C of X's type, float32 dt, per-head A and D, a gate of X's shape or none, channels in whole
+    waves: the kernel that reads every input once (rounds of 128 steps over 16 waves), over lengths that are not a
+    multiple of a round, with an entering state and with rows that end early."""
+    h, p = hp
+    b = 3
+    inp = make(length + h, b, length, h, p, dtype=dtype, d_mode=d_mode, z_mode=z_mode, init=init)
+    inp["dt"] = inp["dt"].float()
+    meta = {"seq_lens": [length, max(length // 3, 0), 0]} if ragged else None
+    y, yr = both(inp, meta=meta)
+    assert y.dtype == dtype
+    torch.testing.assert_close(y.float(), yr.float(), **(FP32_TOL if dtype == torch.float32 else HALF_TOL))
+    if ragged:
+        assert torch.count_nonzero(y[2]) == 0 and torch.count_nonzero(y[1, length // 3:]) == 0
