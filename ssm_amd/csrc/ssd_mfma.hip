@@ -114,8 +114,19 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_bwd_dcb_kernel(const SsdDcbPar
   const int Q = p.chunk, P = 16 * KS, H = p.heads;
   const int nb = Q / 32, nblk = nb * (nb + 1) / 2;
   const int wave = wave_id_uniform(), lane = lane_id();
-  const int unit = blockIdx.x / nblk;
-  int tri = blockIdx.x % nblk;                            // (lb, sb) with sb <= lb, row by row
+  // Consecutive workgroup numbers go to different XCDs (eight, each with its own L2).  All blocks of a (batch,
+  // chunk, group) unit read the same rows of dy and x, so a unit's blocks are given numbers that are equal mod 8:
+  // they run on one XCD and its L2 fetches the unit's operands once.
+  const int units = p.batch * p.nchunks * p.groups;
+  int unit, tri;
+  if (units % 8 == 0) {
+    const int k = (int)blockIdx.x >> 3;
+    unit = (k / nblk) * 8 + ((int)blockIdx.x & 7);
+    tri = k % nblk;                                       // (lb, sb) with sb <= lb, row by row
+  } else {
+    unit = blockIdx.x / nblk;
+    tri = blockIdx.x % nblk;
+  }
   int lb = 0;
   while (tri > lb) tri -= ++lb;
   const int sb = tri;
@@ -129,17 +140,25 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_bwd_dcb_kernel(const SsdDcbPar
   const int per = H / p.groups;
   const bool diag = s0 == l0;
   const size_t trow = (size_t)H * P;
-  const __bf16 *arow = p.dy + ((size_t)b * p.len + (size_t)c * Q + l0 + m) * trow + (size_t)g * per * P + 8 * g2;
-  const __bf16 *brow = p.x + ((size_t)b * p.len + (size_t)c * Q + s0 + m) * trow + (size_t)g * per * P + 8 * g2;
   const size_t csb = (((size_t)b * H + (size_t)g * per) * p.nchunks + c) * Q;
-  bf16x8_t fa[KS], fb[KS];
-  if (wave < per) {
+  // Rows of dy and x are 10 KB apart in memory, so a fragment read straight from them (lane = row) touches 32
+  // cache lines for 32 bytes each.  A wave reads its head's 2 x 32 rows with consecutive lanes on consecutive
+  // 16-byte pieces instead (every line whole, once) and turns them into fragments through a tile of its own in LDS.
+  constexpr int PIECES = 2 * KS;                  // 16-byte pieces per row
+  constexpr int RS = 16 * KS + 8;                 // elements between rows of the tile: conflict-free 16-byte reads
+  __shared__ __align__(16) __bf16 tile[MF_WAVES][2][32 * RS];
+  const __bf16 *abase = p.dy + ((size_t)b * p.len + (size_t)c * Q + l0) * trow + (size_t)g * per * P;
+  const __bf16 *bbase = p.x + ((size_t)b * p.len + (size_t)c * Q + s0) * trow + (size_t)g * per * P;
+  bf16x8_t ra[KS], rb[KS];
+  auto request = [&](int head) {
 #pragma unroll
-    for (int k = 0; k < KS; ++k) {
-      fa[k] = load_frag(arow + (size_t)wave * P + 16 * k);
-      fb[k] = load_frag(brow + (size_t)wave * P + 16 * k);
+    for (int j = 0; j < KS; ++j) {
+      const int idx = j * WAVE + lane, row = idx / PIECES, piece = idx % PIECES;
+      ra[j] = load_frag(abase + (size_t)row * trow + (size_t)head * P + 8 * piece);
+      rb[j] = load_frag(bbase + (size_t)row * trow + (size_t)head * P + 8 * piece);
     }
-  }
+  };
+  if (wave < per) request(wave);
   for (int hh = wave; hh < per; hh += MF_WAVES) {
     const float *cs = p.dA_cs + csb + (size_t)hh * p.nchunks * Q;
     const float *dts = p.dt + csb + (size_t)hh * p.nchunks * Q;
@@ -147,16 +166,22 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_bwd_dcb_kernel(const SsdDcbPar
     float4 cl[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) cl[j] = *reinterpret_cast<const float4 *>(cs + l0 + 8 * j + 4 * g2);
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+      const int idx = j * WAVE + lane, row = idx / PIECES, piece = idx % PIECES;
+      *reinterpret_cast<bf16x8_t *>(&tile[wave][0][row * RS + 8 * piece]) = ra[j];
+      *reinterpret_cast<bf16x8_t *>(&tile[wave][1][row * RS + 8 * piece]) = rb[j];
+    }
+    bf16x8_t fa[KS], fb[KS];
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      fa[k] = load_frag(&tile[wave][0][m * RS + 16 * k + 8 * g2]);
+      fb[k] = load_frag(&tile[wave][1][m * RS + 16 * k + 8 * g2]);
+    }
+    if (hh + MF_WAVES < per) request(hh + MF_WAVES);     // the wave's next head, requested before this head's arithmetic
     f32x16_t t = {0};
 #pragma unroll
     for (int k = 0; k < KS; ++k) t = mma(fa[k], fb[k], t);
-    if (hh + MF_WAVES < per) {                           // the wave's next head, requested before this head's weights
-#pragma unroll
-      for (int k = 0; k < KS; ++k) {
-        fa[k] = load_frag(arow + (size_t)(hh + MF_WAVES) * P + 16 * k);
-        fb[k] = load_frag(brow + (size_t)(hh + MF_WAVES) * P + 16 * k);
-      }
-    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const float cs_l = r % 4 == 0 ? cl[r / 4].x : r % 4 == 1 ? cl[r / 4].y : r % 4 == 2 ? cl[r / 4].z : cl[r / 4].w;
