@@ -135,6 +135,52 @@ __global__ __launch_bounds__(SSD_THREADS) void ssd_state_passing_kernel(const Ss
   p.final_states[gid] = cur;
 }
 
+// The same with float32 states in 16-byte pieces: four neighbouring elements per thread, and the reads of eight
+// chunks requested before the first is used (they do not depend on the running state).
+__global__ __launch_bounds__(SSD_THREADS) void ssd_state_passing_f32x4_kernel(const SsdPassParams p) {
+  constexpr int GROUP = 8;
+  const size_t quads = (size_t)p.batch * p.heads * (p.dim / 4);
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= quads) return;
+  const int i = (int)(gid % (p.dim / 4)) * 4;
+  const int h = (int)((gid / (p.dim / 4)) % p.heads);
+  const int b = (int)(gid / ((size_t)(p.dim / 4) * p.heads));
+  const size_t el = ((size_t)b * p.heads + h) * p.dim + i;
+  float4 cur = p.init ? *reinterpret_cast<const float4 *>(p.init + el) : make_float4(0.f, 0.f, 0.f, 0.f);
+  const float *src = reinterpret_cast<const float *>(p.states);
+  float *dst = reinterpret_cast<float *>(p.out);
+  const size_t cstride = (size_t)p.heads * p.dim;
+  const size_t at0 = ((size_t)b * p.nchunks * p.heads + h) * p.dim + i;
+  const float *dal = p.dA_last + ((size_t)b * p.heads + h) * p.nchunks;
+  int sid_prev = 0;
+  for (int c0 = 0; c0 < p.nchunks; c0 += GROUP) {
+    float4 contrib[GROUP];
+    float scale[GROUP];
+#pragma unroll
+    for (int k = 0; k < GROUP; ++k) {
+      const int c = min(c0 + k, p.nchunks - 1);
+      contrib[k] = *reinterpret_cast<const float4 *>(src + at0 + (size_t)c * cstride);
+      scale[k] = exp2_hw(dal[c] * LOG2E);
+      if (p.seq_idx) {
+        const int sid_new = p.seq_idx[(size_t)b * p.len + min((c + 1) * p.chunk, p.len) - 1];
+        if (sid_new != sid_prev) scale[k] = 0.0f;
+        sid_prev = sid_new;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < GROUP; ++k) {
+      if (c0 + k < p.nchunks) {
+        *reinterpret_cast<float4 *>(dst + at0 + (size_t)(c0 + k) * cstride) = cur;
+        cur.x = __builtin_fmaf(scale[k], cur.x, contrib[k].x);
+        cur.y = __builtin_fmaf(scale[k], cur.y, contrib[k].y);
+        cur.z = __builtin_fmaf(scale[k], cur.z, contrib[k].z);
+        cur.w = __builtin_fmaf(scale[k], cur.w, contrib[k].w);
+      }
+    }
+  }
+  *reinterpret_cast<float4 *>(p.final_states + el) = cur;
+}
+
 // One thread per (b, t, h, p).
 __global__ __launch_bounds__(SSD_THREADS) void ssd_chunk_scan_kernel(const SsdScanParams p) {
   const SsdDims &d = p.d;
@@ -343,8 +389,13 @@ extern "C" int ssm_ssd_state_passing(const ssm_ssd_state_passing_args *a, void *
                 "ssm_ssd_state_passing: with seq_idx, seqlen=%d and chunk=%d must give nchunks=%d", a->seqlen, a->chunk,
                 a->nchunks);
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  hipLaunchKernelGGL(ssd_state_passing_kernel, dim3(grid_for((size_t)p.batch * p.heads * p.dim)), dim3(SSD_THREADS),
-                     0, s, p);
+  if (p.states_dtype == SSM_F32 && p.dim % 4 == 0 && aligned_to(p.states, 16) && aligned_to(p.out, 16) &&
+      aligned_to(p.final_states, 16) && (!p.init || aligned_to(p.init, 16)))
+    hipLaunchKernelGGL(ssd_state_passing_f32x4_kernel, dim3(grid_for((size_t)p.batch * p.heads * (p.dim / 4))),
+                       dim3(SSD_THREADS), 0, s, p);
+  else
+    hipLaunchKernelGGL(ssd_state_passing_kernel, dim3(grid_for((size_t)p.batch * p.heads * p.dim)), dim3(SSD_THREADS),
+                       0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_state_passing");
   return SSM_OK;
 }
