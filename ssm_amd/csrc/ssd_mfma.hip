@@ -310,13 +310,33 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   const size_t xbase = (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
   const __bf16 *xg = reinterpret_cast<const __bf16 *>(p.x) + xbase;
   stage_xT<false>(xT, xg, xrow, Q, P, nullptr, stride);
+  // The state entering the chunk, [P][N], as bfloat16 in LDS: read once by the workgroup in whole lines (a fragment
+  // read straight from memory, lane = row, touches 32 lines for 32 bytes each, and every row block would read it again).
+  __bf16 *Sb = reinterpret_cast<__bf16 *>(ent + Q);                       // [P][N + 8]
+  const int SR = N + 8;
+  {
+    const st_t *Sg0 = reinterpret_cast<const st_t *>(p.prev) + ((((size_t)b * d.nchunks + c) * d.heads + h) * P) * (size_t)N;
+    const int pieces = N / 8;
+    for (int e = threadIdx.x; e < P * pieces; e += MF_THREADS) {
+      const int row = e / pieces, piece = e % pieces;
+      const st_t *sp = Sg0 + (size_t)row * N + 8 * piece;
+      bf16x8_t v;
+      if constexpr (sizeof(st_t) == 2) {
+        v = load_frag(sp);
+      } else {
+        const float4 lo = *reinterpret_cast<const float4 *>(sp), hi = *reinterpret_cast<const float4 *>(sp + 4);
+        const float t8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        v = pack8(t8);
+      }
+      *reinterpret_cast<bf16x8_t *>(Sb + row * SR + 8 * piece) = v;
+    }
+  }
   __syncthreads();
 
   const int g2 = lane >> 5, m = lane & 31;
   const int nlb = Q / 32;
   const __bf16 *Cg = reinterpret_cast<const __bf16 *>(p.Cm) + (((size_t)b * d.len + (size_t)c * Q) * d.groups + g) * N;
   const size_t c_stride = (size_t)d.groups * N;
-  const st_t *Sg = reinterpret_cast<const st_t *>(p.prev) + ((((size_t)b * d.nchunks + c) * d.heads + h) * P) * (size_t)N;
   const __bf16 *CBg = reinterpret_cast<const __bf16 *>(p.CB) + (((size_t)b * d.nchunks + c) * d.groups + g) * (size_t)Q * Q;
   const __bf16 *zg = p.z ? reinterpret_cast<const __bf16 *>(p.z) + xbase : nullptr;
   __bf16 *yg = reinterpret_cast<__bf16 *>(p.y) + xbase;
@@ -337,19 +357,7 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
       for (int n0 = 0; n0 < N; n0 += 16) {
         const bf16x8_t af = load_frag(crow_p + n0);
 #pragma unroll
-        for (int i = 0; i < PT; ++i) {
-          bf16x8_t bf;
-          const st_t *sp = Sg + (size_t)(32 * i + m) * N + n0 + 8 * g2;
-          if constexpr (sizeof(st_t) == 2) {
-            bf = load_frag(sp);
-          } else {
-            float t8[8];
-            const float4 lo = *reinterpret_cast<const float4 *>(sp), hi = *reinterpret_cast<const float4 *>(sp + 4);
-            t8[0] = lo.x; t8[1] = lo.y; t8[2] = lo.z; t8[3] = lo.w; t8[4] = hi.x; t8[5] = hi.y; t8[6] = hi.z; t8[7] = hi.w;
-            bf = pack8(t8);
-          }
-          acc[i] = mma(af, bf, acc[i]);
-        }
+        for (int i = 0; i < PT; ++i) acc[i] = mma(af, load_frag(Sb + (32 * i + m) * SR + n0 + 8 * g2), acc[i]);
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -454,7 +462,7 @@ bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s) {
   if (!mfma_shape_ok(d) || p.x_dtype != SSM_BF16 || p.c_dtype != SSM_BF16 || p.cb_dtype != SSM_BF16) return false;
   if (p.states_dtype == SSM_F16 || (p.z && p.z_dtype != SSM_BF16)) return false;
   if (!aligned_to(p.x, 16) || !aligned_to(p.Cm, 16) || !aligned_to(p.CB, 16) || !aligned_to(p.prev, 16)) return false;
-  const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 12;
+  const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 12 + (size_t)d.hdim * (d.nstate + 8) * 2;
   const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);
 #define SSM_LAUNCH_SC(ST, PT)                                                                              \
   {                                                                                                        \
