@@ -559,6 +559,29 @@ typedef struct ssm_ssd_scale_rows_args {
 } ssm_ssd_scale_rows_args;
 int ssm_ssd_scale_rows(const ssm_ssd_scale_rows_args *args, void *hip_stream);
 
+/* The per-step scalars of the gradient of the combined forward (see ssm_ssd_bwd_gate), chunk by chunk:
+ *   q[l]   = q_c + sum_{j<l in chunk} (s1[j] - s2[j]),  q_c = q0 for the first chunk and
+ *            exp(dt A) at the chunk's first step (0 at the first step of a packed sequence) times anchor[c-1] after it
+ *   ddt[l] = (A q[l] + xu[l]) * slope,  slope = sigmoid(raw) under softplus (else 1), 0 outside [dt_min, dt_max]
+ *   dA_part[b,c,h] = sum_l dt[l] q[l],   dbias_part[b,c,h] = sum_l ddt[l]      (raw = dt_raw + dt_bias)
+ * seqlen must be a multiple of chunk. */
+typedef struct ssm_ssd_bwd_dt_args {
+  const float *s1, *s2, *xu;       /* (B, L, H) fp32: outputs of ssm_ssd_bwd_dx / ssm_ssd_bwd_gate */
+  const float *dt;                 /* (B, L, H) fp32: the step after bias, softplus and clamp */
+  const void *dt_raw;              /* (B, L, H) dt_dtype: the step as given to the forward */
+  const float *A;                  /* (H,) */
+  const float *dt_bias;            /* (H,) or NULL */
+  const float *q0;                 /* (B, H) or NULL (zero) */
+  const float *anchor;             /* (B, nc-1, H); may be NULL with a single chunk */
+  const uint8_t *first_step;       /* (B, L) nonzero at the first step of a packed sequence, or NULL */
+  float *ddt;                      /* (B, L, H) fp32 */
+  float *dA_part, *dbias_part;     /* (B, nc, H) fp32 */
+  int32_t batch, seqlen, heads, chunk;
+  int32_t dt_dtype, dt_softplus;
+  float dt_min, dt_max;
+} ssm_ssd_bwd_dt_args;
+int ssm_ssd_bwd_dt(const ssm_ssd_bwd_dt_args *args, void *hip_stream);
+
 /* ------------------------------------------------------------------------
  * depthwise causal conv1d (+ optional SiLU).
  * Forward stands behind `dw_causal_conv(x, weight, bias, activation)`

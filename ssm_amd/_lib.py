@@ -211,6 +211,13 @@ class SsdScaleRowsArgs(C.Structure):
                 ("out_dtype", _i32)]
 
 
+class SsdBwdDtArgs(C.Structure):
+    _fields_ = [("s1", _vp), ("s2", _vp), ("xu", _vp), ("dt", _vp), ("dt_raw", _vp), ("A", _vp), ("dt_bias", _vp),
+                ("q0", _vp), ("anchor", _vp), ("first_step", _vp), ("ddt", _vp), ("dA_part", _vp), ("dbias_part", _vp),
+                ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("chunk", _i32), ("dt_dtype", _i32),
+                ("dt_softplus", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float)]
+
+
 LAYOUT_BCL, LAYOUT_BLC = 0, 1
 ACT_IDENTITY, ACT_SILU = 0, 1
 
@@ -275,6 +282,7 @@ ENTRY_POINTS = {
     "ssm_ssd_bwd_dcb": SsdBwdDcbArgs,
     "ssm_ssd_bwd_states": SsdBwdStatesArgs,
     "ssm_ssd_scale_rows": SsdScaleRowsArgs,
+    "ssm_ssd_bwd_dt": SsdBwdDtArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_conv1d_update": Conv1dUpdateArgs,

@@ -282,6 +282,68 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_scale_rows_kernel(const ScaleP
   st4<OT>(p.out, gid * 4, v);
 }
 
+// The per-step scalars of the backward, one thread per (batch, chunk, head) walking its chunk:
+//   q_l    = anchor + sum_{j<l} (s1_j - s2_j),  anchor = W0 for the first chunk, a_first <G, H> at a later boundary
+//   ddt_l  = (A q_l + xu_l) * d(step)/d(raw dt)      (softplus' = sigmoid, and 0 outside the clamp)
+//   dA    += dt_l q_l,   dbias += ddt_l              (one partial per thread, summed afterwards in a fixed order)
+struct DtParams {
+  const float *s1, *s2, *xu, *dte, *A, *bias, *W0, *anchor;
+  const void *dt_raw;
+  const unsigned char *first;     // (B, L) 1 at the first step of a packed sequence, or null
+  float *ddt, *dA_part, *db_part;
+  int batch, len, heads, chunk, nchunks, dt_dtype, softplus;
+  float lo, hi;
+};
+
+__global__ __launch_bounds__(EB_THREADS) void ssd_bwd_dt_kernel(const DtParams p) {
+  constexpr int G = 8;
+  const size_t gid = (size_t)blockIdx.x * EB_THREADS + threadIdx.x;
+  if (gid >= (size_t)p.batch * p.nchunks * p.heads) return;
+  const int h = (int)(gid % p.heads);
+  const int c = (int)((gid / p.heads) % p.nchunks);
+  const int b = (int)(gid / ((size_t)p.heads * p.nchunks));
+  const float Ah = p.A[h], bias = p.bias ? p.bias[h] : 0.0f;
+  const size_t row0 = ((size_t)b * p.len + (size_t)c * p.chunk) * p.heads + h;
+  float q;
+  if (c == 0) {
+    q = p.W0 ? p.W0[(size_t)b * p.heads + h] : 0.0f;
+  } else {
+    float a_first = exp2_hw(p.dte[row0] * Ah * LOG2E);
+    if (p.first && p.first[(size_t)b * p.len + (size_t)c * p.chunk]) a_first = 0.0f;
+    q = a_first * p.anchor[((size_t)b * (p.nchunks - 1) + (c - 1)) * p.heads + h];
+  }
+  float dA = 0.0f, db = 0.0f;
+  for (int l0 = 0; l0 < p.chunk; l0 += G) {
+    float d[G], xu[G], dte[G], raw[G];
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+      const size_t at = row0 + (size_t)min(l0 + k, p.chunk - 1) * p.heads;
+      d[k] = p.s1[at] - p.s2[at];
+      xu[k] = p.xu[at];
+      dte[k] = p.dte[at];
+      raw[k] = load_as_f32(p.dt_raw, p.dt_dtype, at) + bias;
+    }
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+      if (l0 + k < p.chunk) {
+        const float ddte = __builtin_fmaf(Ah, q, xu[k]);
+        dA = __builtin_fmaf(dte[k], q, dA);
+        q += d[k];
+        float v = raw[k], slope = 1.0f;
+        if (p.softplus) {
+          v = raw[k] > 20.0f ? raw[k] : log2_hw(1.0f + exp2_hw(raw[k] * LOG2E)) * LN2;
+          slope = sigmoid_f32(raw[k]);
+        }
+        const float g = (v >= p.lo && v <= p.hi) ? ddte * slope : 0.0f;
+        p.ddt[row0 + (size_t)(l0 + k) * p.heads] = g;
+        db += g;
+      }
+    }
+  }
+  p.dA_part[gid] = dA;
+  p.db_part[gid] = db;
+}
+
 }  // namespace
 }  // namespace ssm
 
@@ -429,5 +491,27 @@ extern "C" int ssm_ssd_scale_rows(const ssm_ssd_scale_rows_args *a, void *hip_st
   if (a->x_dtype == SSM_F32) SSM_SCALE(float) else if (a->x_dtype == SSM_BF16) SSM_SCALE(bf16_t) else SSM_SCALE(f16_t)
 #undef SSM_SCALE
   SSM_CHECK_LAUNCH("ssm_ssd_scale_rows");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_bwd_dt(const ssm_ssd_bwd_dt_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_dt: args is NULL");
+  SSM_REQUIRE(a->s1 && a->s2 && a->xu && a->dt && a->dt_raw && a->A && a->ddt && a->dA_part && a->dbias_part,
+              SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_dt: s1, s2, xu, dt, dt_raw, A, ddt, dA_part and dbias_part are required");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->chunk > 0 && a->seqlen % a->chunk == 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bwd_dt: sizes must be positive and chunk=%d must divide seqlen=%d", a->chunk, a->seqlen);
+  SSM_REQUIRE(a->anchor || a->seqlen == a->chunk, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_dt: anchor is required with more than one chunk");
+  SSM_REQUIRE(valid_dtype(a->dt_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_bwd_dt: dt_dtype=%d", a->dt_dtype);
+  DtParams p{};
+  p.s1 = a->s1; p.s2 = a->s2; p.xu = a->xu; p.dte = a->dt; p.A = a->A; p.bias = a->dt_bias; p.W0 = a->q0; p.anchor = a->anchor;
+  p.dt_raw = a->dt_raw; p.first = a->first_step; p.ddt = a->ddt; p.dA_part = a->dA_part; p.db_part = a->dbias_part;
+  p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.chunk = a->chunk; p.nchunks = a->seqlen / a->chunk;
+  p.dt_dtype = a->dt_dtype; p.softplus = a->dt_softplus ? 1 : 0; p.lo = a->dt_min; p.hi = a->dt_max;
+  const size_t total = (size_t)p.batch * p.nchunks * p.heads;
+  SSM_REQUIRE(total < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_dt: too many (batch, chunk, head) triples");
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(ssd_bwd_dt_kernel, dim3((unsigned)((total + EB_THREADS - 1) / EB_THREADS)), dim3(EB_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_bwd_dt");
   return SSM_OK;
 }

@@ -623,6 +623,26 @@ def _bwd_dcb(dy, x, dt_c, dA_cs, groups):
     return out
 
 
+def _bwd_dt(s1, s2, xu, dte, dt_raw, Af, dt_bias, W0, anchor, first, Q, dt_softplus, dt_limit):
+    """``ssm_ssd_bwd_dt``: ``(ddt (B, L, H), dA (H,), dbias (H,))``."""
+    batch, seqlen, heads = (int(v) for v in dte.shape)
+    nc = seqlen // Q
+    dev = dte.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    ddt = torch.empty(batch, seqlen, heads, **f32)
+    dA_p = torch.empty(batch, nc, heads, **f32)
+    db_p = torch.empty_like(dA_p)
+    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    args = _lib.SsdBwdDtArgs(
+        s1=_lib.ptr(s1), s2=_lib.ptr(s2), xu=_lib.ptr(xu), dt=_lib.ptr(dte), dt_raw=_lib.ptr(dt_raw), A=_lib.ptr(Af),
+        dt_bias=_lib.ptr(dt_bias), q0=_lib.ptr(W0), anchor=_lib.ptr(anchor) if nc > 1 else None, first_step=_lib.ptr(first),
+        ddt=_lib.ptr(ddt), dA_part=_lib.ptr(dA_p), dbias_part=_lib.ptr(db_p), batch=batch, seqlen=seqlen, heads=heads,
+        chunk=Q, dt_dtype=_lib.dtype_enum(dt_raw.dtype), dt_softplus=int(bool(dt_softplus)),
+        dt_min=lo if lo > -math.inf else -3.0e38, dt_max=hi if hi < math.inf else 3.0e38)
+    _lib.call("ssm_ssd_bwd_dt", args, dev)
+    return ddt, dA_p.sum(dim=(0, 1)), db_p.sum(dim=(0, 1))
+
+
 def _scale_rows(x, w, out_dtype):
     """``ssm_ssd_scale_rows``: ``x * w[..., None]`` formed in float32 and rounded once to ``out_dtype``."""
     cols = int(x.shape[-1])
@@ -838,6 +858,14 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         s2 = (dyc.to(f32) * ypre).sum(-1)              # the same rounded dy that the pass for u saw
     W0 = (dinit * init).sum(dim=(2, 3)) if init is not None else torch.zeros(batch, heads, dtype=f32, device=x.device)
     nc = (seqlen + Q - 1) // Q
+    if anchor_in is not None and s1.is_contiguous() and s2.is_contiguous() and xu.is_contiguous():
+        # the running sum behind ddt and dA, anchored at every chunk boundary on the two passes' float32 states
+        # there (see below), the chain through softplus and clamp, and the sums for dA and the bias: one launch
+        first = None if bnd is None else bnd.to(torch.uint8).contiguous()
+        ddt, dA, dbias = _bwd_dt(s1, s2, xu, dte, dt.detach().contiguous(), Af.contiguous(),
+                                 None if dt_bias is None else dt_bias.detach().to(f32).contiguous(),
+                                 W0.contiguous() if init is not None else None, anchor_in, first, Q, dt_softplus, dt_limit)
+        return dx, ddt, dA, dB, dC, dD, dz, (dbias if dt_bias is not None else None), (dinit if init is not None else None)
     if seqlen % Q == 0 and nc > 1:
         # q at the first step of every chunk straight from the two passes' states at the chunk boundary
         # (a_t <G_t, H_{t-1}>, float32), and from there the running sum inside the chunk only: what the

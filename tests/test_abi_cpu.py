@@ -62,7 +62,8 @@ def test_ctypes_struct_sizes_match_the_header(tmp_path):
              "Mamba2DecodeArgs": "ssm_mamba2_decode_args", "Conv1dUpdateArgs": "ssm_conv1d_update_args",
              "SsdBwdGateArgs": "ssm_ssd_bwd_gate_args", "SsdBwdDxArgs": "ssm_ssd_bwd_dx_args",
              "SsdBwdDbArgs": "ssm_ssd_bwd_db_args", "SsdBwdDcbArgs": "ssm_ssd_bwd_dcb_args",
-             "SsdBwdStatesArgs": "ssm_ssd_bwd_states_args", "SsdScaleRowsArgs": "ssm_ssd_scale_rows_args"}
+             "SsdBwdStatesArgs": "ssm_ssd_bwd_states_args", "SsdScaleRowsArgs": "ssm_ssd_scale_rows_args",
+             "SsdBwdDtArgs": "ssm_ssd_bwd_dt_args"}
     assert set(structs) <= set(cname), set(structs) - set(cname)
     src = tmp_path / "sizes.c"
     lines = ['#include <stdio.h>', f'#include "{HEADER}"', "int main(void) {"]
