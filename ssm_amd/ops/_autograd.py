@@ -225,3 +225,38 @@ class SsdCombinedFn(torch.autograd.Function):
         return (pick(0, dx, x), pick(1, ddt, dt), pick(2, dA, A), pick(3, dB, B), pick(4, dC, C), None,
                 pick(6, dD, D), pick(7, dz, z), pick(8, dbias, dt_bias), pick(9, dinit, init),
                 None, None, None, None, None, None)
+
+
+class SsdVarlenStatesFn(torch.autograd.Function):
+    """The state at the last step of every sequence of a packed batch row, ``(nseq, H, P, N)``: the
+    ``return_varlen_states`` output of the call at scripts/refresh_mamba_goldens.py:618-632 (the reference
+    ships its values, ``ssd_combined.combined_varlen``; no gradients of it)."""
+
+    @staticmethod
+    def forward(ctx, x, dt, A, B, chunk_size, dt_bias, initial_states, dt_softplus, dt_limit, states_dtype,
+                force_generic, seq_idx, cu_seqlens):
+        from .ssd import _check_boundaries, _need, _ssd_shapes, _varlen_states_forward
+
+        _need(_ssd_shapes(x, B)[0] == 1, "cu_seqlens describes one packed batch row: batch size must be 1.")
+        _check_boundaries(seq_idx, [int(v) for v in cu_seqlens.tolist()], int(x.shape[1]))
+        det = lambda t: None if t is None else t.detach()
+        out = _varlen_states_forward(det(x), det(dt), det(A), det(B), chunk_size, det(dt_bias), det(initial_states),
+                                     dt_softplus, dt_limit, states_dtype, force_generic, seq_idx, cu_seqlens)
+        ctx.save_for_backward(x, dt, A, B, dt_bias, initial_states, cu_seqlens)
+        ctx.conf = (dt_softplus, dt_limit)
+        ctx.seq_idx = seq_idx
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_states):
+        from .ssd import varlen_states_backward
+
+        x, dt, A, B, dt_bias, init, cu = ctx.saved_tensors
+        softplus, limit = ctx.conf
+        dx, ddt, dA, dB, dbias, dinit = varlen_states_backward(
+            grad_states, x, dt, A, B, cu, dt_bias=dt_bias, initial_states=init, dt_softplus=softplus,
+            dt_limit=limit, seq_idx=ctx.seq_idx)
+        need = ctx.needs_input_grad
+        pick = lambda i, g, r: _like(g, r) if (r is not None and g is not None and need[i]) else None
+        return (pick(0, dx, x), pick(1, ddt, dt), pick(2, dA, A), pick(3, dB, B), None, pick(5, dbias, dt_bias),
+                pick(6, dinit, init), None, None, None, None, None, None)

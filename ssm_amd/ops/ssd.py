@@ -421,7 +421,9 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         cu_seqlens: Optional ``(nseq + 1,)`` sequence boundaries of a packed batch row
             (batch size 1), only used for ``return_varlen_states``.
         return_varlen_states: Also return the state at the last step of every sequence,
-            ``(nseq, H, P, N)`` float32 (needs ``cu_seqlens``).
+            ``(nseq, H, P, N)`` float32 (needs ``cu_seqlens``).  Differentiable in ``x, dt, A, B,
+            dt_bias, initial_states`` when ``seq_idx`` changes exactly at the inner entries of
+            ``cu_seqlens`` (:func:`varlen_states_backward`).
 
     Returns:
         ``y (B, L, H, P)`` in ``x.dtype``; with ``return_final_states`` and / or
@@ -458,15 +460,19 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         return out[:, :seqlen]
     tensors = (x, dt, A, B, C, D, z, dt_bias, initial_states)
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
-        _need(cu_seqlens is None and not return_varlen_states,
-              "gradients through the per-sequence end states (cu_seqlens / return_varlen_states) are not "
-              "implemented; seq_idx alone is differentiable.")
-        from ._autograd import SsdCombinedFn
+        from ._autograd import SsdCombinedFn, SsdVarlenStatesFn
+        _need(not return_varlen_states or cu_seqlens is not None, "return_varlen_states needs cu_seqlens.")
         si = None if seq_idx is None else _seq_idx_i32(seq_idx, int(x.shape[0]), int(x.shape[1]))
+        limit = (float(dt_limit[0]), float(dt_limit[1]))
         y, final = SsdCombinedFn.apply(x, dt, A, B, C, int(chunk_size), D, z, dt_bias, initial_states,
-                                       bool(dt_softplus), (float(dt_limit[0]), float(dt_limit[1])),
-                                       states_dtype, bool(force_generic), fused, si)
-        return (y, final) if return_final_states else y
+                                       bool(dt_softplus), limit, states_dtype, bool(force_generic), fused, si)
+        outs = (y, final) if return_final_states else (y,)
+        if return_varlen_states:
+            # a second node of the graph: its gradients add to those of y and the final state
+            outs += (SsdVarlenStatesFn.apply(x, dt, A, B, int(chunk_size), dt_bias, initial_states,
+                                             bool(dt_softplus), limit, states_dtype, bool(force_generic), si,
+                                             cu_seqlens),)
+        return outs[0] if len(outs) == 1 else outs
     return _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias,
                                  initial_states=initial_states, dt_softplus=dt_softplus, dt_limit=dt_limit,
                                  return_final_states=return_final_states, states_dtype=states_dtype,
@@ -527,6 +533,105 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
     if return_varlen_states:
         outs.append(chunk_state_varlen(B, x, dtc, dA, cu_seqlens, entering))
     return outs[0] if len(outs) == 1 else tuple(outs)
+
+
+def _varlen_states_forward(x, dt, A, B, chunk_size, dt_bias, initial_states, dt_softplus, dt_limit, states_dtype,
+                           force_generic, seq_idx, cu_seqlens):
+    """The per-sequence end states alone: ``chunk_cumsum -> chunk_state -> state_passing ->
+    chunk_state_varlen``, the same kernels and the same dtype of the states between them as in
+    :func:`_ssd_combined_forward`, so the values agree with its ``return_varlen_states`` output."""
+    Q = int(chunk_size)
+    dA, dtc = chunk_cumsum(dt, A, Q, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit)
+    states = chunk_state(B, x, dtc, dA, states_dtype=states_dtype or x.dtype, force_generic=force_generic,
+                         seq_idx=seq_idx)
+    entering, _ = state_passing(states, dA[:, :, :, -1].contiguous(), initial_states=initial_states,
+                                seq_idx=seq_idx, chunk_size=Q)
+    return chunk_state_varlen(B, x, dtc, dA, cu_seqlens, entering)
+
+
+def _check_boundaries(seq_idx, cu, seqlen):
+    """Gradients of the per-sequence end states are formed from ``cu_seqlens`` alone, so the sequences that
+    ``seq_idx`` separates in the forward must be the same ones."""
+    inner = sorted({v for v in cu[1:-1] if 0 < v < seqlen})
+    if seq_idx is None:
+        have = []
+    else:
+        row = seq_idx.reshape(-1, seqlen)[0]
+        have = (torch.nonzero(row[1:] != row[:-1]).flatten() + 1).tolist()
+    _need(have == inner, "gradients through the per-sequence end states need seq_idx to change exactly at the "
+          "inner entries of cu_seqlens.")
+
+
+def varlen_states_backward(dstates, x, dt, A, B, cu_seqlens, dt_bias=None, initial_states=None,
+                           dt_softplus=False, dt_limit=(0.0, float("inf")), seq_idx=None):
+    """Gradients of the per-sequence end states of a packed batch row (``return_varlen_states`` of
+    :func:`ssd_combined`, the call at /root/reference/scripts/refresh_mamba_goldens.py:618-632).
+
+    With ``w_t = exp(sum_{t < r < end} dt_r A)`` the end state of a sequence is
+    ``sum_t w_t dt_t x_t (x) B_t`` over its steps, plus ``exp(sum_r dt_r A) * initial_states`` for the
+    sequence that begins at step 0; this differentiates that sum sequence by sequence with float32
+    tensor operations (a side output of packed batches: a few small products per sequence).
+
+    Args:
+        dstates: ``(nseq, H, P, N)`` gradient of the end states.
+        x, dt, A, B, dt_bias, initial_states, dt_softplus, dt_limit, seq_idx: As given to the forward.
+        cu_seqlens: ``(nseq + 1,)`` sequence boundaries.
+
+    Returns:
+        ``(dx, ddt, dA, dB, ddt_bias, dinitial_states)`` in float32 (the last two ``None`` without the input).
+    """
+    batch, seqlen, heads, hdim, groups, nstate = _ssd_shapes(x, B)
+    _need(batch == 1, "cu_seqlens describes one packed batch row: batch size must be 1.")
+    cu = [int(v) for v in cu_seqlens.tolist()]
+    nseq = len(cu) - 1
+    _need(tuple(dstates.shape) == (nseq, heads, hdim, nstate), "dstates must have shape (nseq, H, P, N).")
+    _check_boundaries(seq_idx, cu, seqlen)
+    per = heads // groups
+    f32 = torch.float32
+    Af = A.detach().to(f32)
+    u = dt.detach().to(f32)[0]                                  # (L, H)
+    if dt_bias is not None:
+        u = u + dt_bias.detach().to(f32)
+    sp = torch.nn.functional.softplus(u, threshold=20.0) if dt_softplus else u
+    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    dtp = sp.clamp(lo, hi)
+    chain = ((sp >= lo) & (sp <= hi)).to(f32)                   # d dtp / d u
+    if dt_softplus:
+        chain = chain * torch.sigmoid(u)
+    xf, Bf, G_all = x.detach()[0], B.detach()[0], dstates.detach().to(f32)
+    dx = torch.zeros(1, seqlen, heads, hdim, device=x.device, dtype=f32)
+    dB = torch.zeros(1, seqlen, groups, nstate, device=x.device, dtype=f32)
+    ddtp = torch.zeros(seqlen, heads, device=x.device, dtype=f32)
+    dA = torch.zeros(heads, device=x.device, dtype=f32)
+    dinit = None if initial_states is None else torch.zeros_like(initial_states, dtype=f32)
+    for i in range(nseq):
+        a, e = cu[i], min(cu[i + 1], seqlen)
+        if e <= a:
+            continue
+        G = G_all[i]                                            # (H, P, N)
+        dts = dtp[a:e]
+        cum = torch.cumsum(dts * Af, dim=0)
+        w = torch.exp((cum[-1:] - cum).clamp(max=0.0))          # decay from after step t to the end
+        xs = xf[a:e].to(f32)
+        Bh = Bf[a:e].to(f32).repeat_interleave(per, dim=1)      # (l, H, N)
+        GB = torch.einsum("hpn,lhn->lhp", G, Bh)
+        xG = torch.einsum("lhp,hpn->lhn", xs, G)
+        coef = dts * w
+        dx[0, a:e] = coef[..., None] * GB
+        dB[0, a:e] = (coef[..., None] * xG).reshape(e - a, groups, per, nstate).sum(dim=2)
+        sdot = (xs * GB).sum(dim=-1)                            # x_t' G B_t
+        contrib = coef * sdot
+        # dt_r A enters every term of an earlier step: the sum of those terms
+        ddA = torch.cumsum(contrib, dim=0) - contrib
+        if a == 0 and initial_states is not None:
+            tot = torch.exp(cum[-1].clamp(max=0.0))             # (H,)
+            dinit[0] = tot[:, None, None] * G
+            ddA = ddA + (tot * (G * initial_states.detach()[0].to(f32)).sum(dim=(1, 2)))[None]
+        ddtp[a:e] = w * sdot + ddA * Af
+        dA += (ddA * dts).sum(dim=0)
+    ddt = (ddtp * chain)[None]
+    dbias = None if dt_bias is None else ddt.sum(dim=(0, 1))
+    return dx, ddt, dA, dB, dbias, dinit
 
 
 def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None):

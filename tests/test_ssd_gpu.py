@@ -177,14 +177,84 @@ def test_combined_gradient_vector_on_the_decaying_head():
         torch.testing.assert_close(f(d[k].grad.cpu()), f(gr[k]), rtol=5e-2, atol=5e-2, msg=lambda m: f"{k}: {m}")
 
 
-def test_gradients_through_per_sequence_end_states_are_refused():
+@pytest.mark.parametrize("dtype,lens,Q,P,N,softplus", [(torch.float32, [40, 24, 64], 32, 16, 8, True),
+                                                     (torch.float32, [5, 70, 1, 20], 16, 8, 4, False),
+                                                     (torch.bfloat16, [100, 28, 128], 64, 64, 64, True),
+                                                     (torch.bfloat16, [100, 30, 70], 64, 128, 32, False)])
+def test_gradients_through_per_sequence_end_states_match_the_oracle(dtype, lens, Q, P, N, softplus):
+    """A loss on y, the final state and the per-sequence end states together: every gradient against float64
+    autograd through the oracle (the end states add their own terms to x, dt, A, B, the bias and the initial
+    state).  Some raw steps fall outside the clamp, where the gradient of the step is zero."""
+    g = torch.Generator().manual_seed(77)
+    H, G = 4, 2
+    L = sum(lens)
+    mk = lambda *shape: torch.randn(*shape, generator=g)
+    base = dict(x=mk(1, L, H, P).to(dtype), dt=torch.rand(1, L, H, generator=g) * 0.6 - (0.3 if softplus else 0.0),
+                A=-torch.rand(H, generator=g) * 1.5 - 0.1, B=(mk(1, L, G, N) * 0.5).to(dtype),
+                C=(mk(1, L, G, N) * 0.5).to(dtype), D=mk(H), z=mk(1, L, H, P).to(dtype), bias=mk(H) * 0.2,
+                init=mk(1, H, P, N))
+    limit = (0.3, 0.9) if softplus else (0.05, 0.5)
+    cu_l = [0]
+    for n in lens:
+        cu_l.append(cu_l[-1] + n)
+    seq_idx = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])[None]
+    wy, wf, wv = mk(1, L, H, P), mk(1, H, P, N), mk(len(lens), H, P, N)
+
+    d = {k: cu(v).clone().requires_grad_(True) for k, v in base.items()}
+    y, fin, vs = ssd().ssd_combined(d["x"], d["dt"], d["A"], d["B"], d["C"], Q, D=d["D"], z=d["z"], dt_bias=d["bias"],
+                                    initial_states=d["init"], dt_softplus=softplus, dt_limit=limit,
+                                    return_final_states=True, seq_idx=cu(seq_idx),
+                                    cu_seqlens=torch.tensor(cu_l, dtype=torch.int32).cuda(),
+                                    return_varlen_states=True, states_dtype=torch.float32)
+    ((y.float() * cu(wy)).sum() + (fin * cu(wf)).sum() + (vs * cu(wv)).sum()).backward()
+
+    r = {k: v.detach().double().requires_grad_(True) for k, v in base.items()}
+    oy, of, ov = S.ssd_combined(r["x"], r["dt"], r["A"], r["B"], r["C"], Q, D=r["D"], z=r["z"], dt_bias=r["bias"],
+                                initial_states=r["init"], dt_softplus=softplus, dt_limit=limit, seq_idx=seq_idx,
+                                cu_seqlens=cu_l)
+    torch.testing.assert_close(vs.cpu().double(), ov.detach(), rtol=2e-2 if dtype != torch.float32 else 1e-4,
+                               atol=(2e-2 if dtype != torch.float32 else 1e-5) * float(ov.detach().abs().max()))
+    ((oy * wy).sum() + (of * wf).sum() + (ov * wv).sum()).backward()
+    for k in base:
+        got, want = d[k].grad.cpu().double(), r[k].grad
+        assert got.shape == want.shape and d[k].grad.dtype == base[k].dtype, k
+        scale = float(want.pow(2).mean().sqrt())
+        if dtype == torch.float32:
+            torch.testing.assert_close(got, want, rtol=1e-3, atol=2e-4 * scale, msg=lambda m: f"{k}: {m}")
+        else:
+            err = (got - want).abs()
+            assert float(err.max()) <= 0.08 * scale + 0.05 * float(want.abs().max()), (k, float(err.max()), scale)
+            assert float(err.mean()) <= 0.02 * scale, (k, float(err.mean()), scale)
+
+    # the end states alone: only their own node of the graph runs
+    d2 = {k: cu(v).clone().requires_grad_(True) for k, v in base.items()}
+    vs2 = ssd().ssd_combined(d2["x"], d2["dt"], d2["A"], d2["B"], d2["C"], Q, D=d2["D"], z=d2["z"], dt_bias=d2["bias"],
+                             initial_states=d2["init"], dt_softplus=softplus, dt_limit=limit, seq_idx=cu(seq_idx),
+                             cu_seqlens=torch.tensor(cu_l, dtype=torch.int32).cuda(), return_varlen_states=True,
+                             states_dtype=torch.float32)[1]
+    (vs2 * cu(wv)).sum().backward()
+    r2 = {k: v.detach().double().requires_grad_(True) for k, v in base.items()}
+    ov2 = S.ssd_combined(r2["x"], r2["dt"], r2["A"], r2["B"], r2["C"], Q, D=r2["D"], z=r2["z"], dt_bias=r2["bias"],
+                         initial_states=r2["init"], dt_softplus=softplus, dt_limit=limit, seq_idx=seq_idx,
+                         cu_seqlens=cu_l)[2]
+    (ov2 * wv).sum().backward()
+    for k in ("x", "dt", "A", "B", "bias", "init"):
+        got, want = d2[k].grad.cpu().double(), r2[k].grad
+        scale = float(want.pow(2).mean().sqrt())
+        tol = dict(rtol=1e-3, atol=2e-4 * scale) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2 * scale)
+        torch.testing.assert_close(got, want, msg=lambda m: f"end states alone, {k}: {m}", **tol)
+    assert d2["C"].grad is None or float(d2["C"].grad.abs().max()) == 0.0
+
+
+def test_gradients_through_end_states_need_matching_boundaries():
     x = torch.zeros(1, 8, 2, 4).cuda().requires_grad_(True)
     dt = torch.zeros(1, 8, 2).cuda()
     A = -torch.ones(2).cuda()
     Bm = torch.zeros(1, 8, 1, 4).cuda()
+    seq_idx = torch.tensor([[0, 0, 0, 1, 1, 1, 1, 1]], dtype=torch.int32).cuda()
     with pytest.raises(ValueError):
-        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, seq_idx=torch.zeros(1, 8, dtype=torch.int32).cuda(),
-                           cu_seqlens=torch.tensor([0, 8], dtype=torch.int32).cuda(), return_varlen_states=True)
+        ssd().ssd_combined(x, dt, A, Bm, Bm, 4, seq_idx=seq_idx,
+                           cu_seqlens=torch.tensor([0, 4, 8], dtype=torch.int32).cuda(), return_varlen_states=True)
 
 
 @pytest.mark.parametrize("dtype,lens,Q,P,N", [(torch.float32, [40, 24, 64], 32, 16, 8),
