@@ -451,6 +451,25 @@ VALU_KINDS = [
 ]
 
 
+def bench_stream():
+    """What plain element-wise kernels of the framework reach on this GPU, as the yardstick for the streaming
+    kernels: ``dst = 2 * src`` and ``dst.copy_(src)`` on float32 buffers of 64 MiB (source and destination fit the
+    256 MB memory-side cache together) and of 1 GiB (they do not)."""
+    out = {}
+    for mib in (64, 1024):
+        n = mib * 1024 * 1024 // 4
+        src = torch.empty(n, device="cuda", dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        moved = 2.0 * n * 4
+        us = _time_us(lambda i: torch.mul(src, 2.0, out=dst), iters=30, warmup=10)
+        out[f"scale_{mib}MiB_GBps"] = round(moved / us / 1e3, 1)
+        us = _time_us(lambda i: dst.copy_(src), iters=30, warmup=10)
+        out[f"copy_{mib}MiB_GBps"] = round(moved / us / 1e3, 1)
+        del src, dst
+    out["frac_hbm_peak_scale_1GiB"] = round(out["scale_1024MiB_GBps"] / HBM_PEAK_GBPS, 4)
+    return out
+
+
 def bench_valu(waves=(1, 2, 3, 4)):
     """Issue rates of the vector ALU (``ssm_probe_valu``): shader clocks per wave instruction per SIMD, with one
     workgroup per CU and 1 to 4 waves per SIMD."""
@@ -535,7 +554,7 @@ def main():
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
                     choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1", "valu",
-                             "scan_facade", "scan_per_channel_bc"],
+                             "scan_facade", "scan_per_channel_bc", "stream"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
     args = ap.parse_args()
@@ -562,7 +581,7 @@ def main():
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
               "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model,
               "model1": bench_model1, "valu": bench_valu, "scan_facade": bench_scan_facade,
-              "scan_per_channel_bc": bench_scan_per_channel_bc}[args.only]
+              "scan_per_channel_bc": bench_scan_per_channel_bc, "stream": bench_stream}[args.only]
         if args.only != "valu":
             bench_scan_fwd(1, 0)        # the untimed spin-up of the default run, so that figures compare
         print(json.dumps({args.only: fn()}))
@@ -624,6 +643,7 @@ def main():
         extra["ssd_config3_backward_and_packed"] = bench_ssd_train()
         extra["mamba2_130m_style_model_config4"] = bench_model()
         extra["mamba1_130m_style_model_config1_shape"] = bench_model1()
+        extra["elementwise_streaming_yardstick"] = bench_stream()
         line["extra"] = extra
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_scan()
