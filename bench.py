@@ -230,14 +230,22 @@ def bench_dscan(batch=4, length=4096, heads=80, proj=64, chunk=256):
     z = torch.randn(batch, length, heads, proj, generator=g).to(torch.bfloat16).cuda()
     gy = torch.randn(batch, length, heads, proj, generator=g).to(torch.bfloat16).cuda()
     fus = _time_us(lambda i: ops._dscan_forward(X, dt, A, Bm, Cm, chunk, D, z, None, None), iters=10)
-    bus = _time_us(lambda i: ops._dscan_backward(gy, X, dt, A, Bm, Cm, chunk, D, z, None, None), iters=10)
+    # the backward as autograd runs it: the forward left the state entering every 64 steps, and the gradients of
+    # X's shape come back in X's type
+    _, table = ops._dscan_forward(X, dt, A, Bm, Cm, chunk, D, z, None, None, want_round_states=True)
+    bus = _time_us(lambda i: ops._dscan_backward(gy, X, dt, A, Bm, Cm, chunk, D, z, None, None,
+                                                 grads_in_input_dtype=True, round_states=table), iters=10)
+    # and called on its own with float32 gradients (its own forward sweep first)
+    sus = _time_us(lambda i: ops._dscan_backward(gy, X, dt, A, Bm, Cm, chunk, D, z, None, None), iters=10)
     el = batch * length * heads * proj
     fbytes = el * 2 * 5 + batch * length * heads * 4               # X, B, C, z in; Y out; dt
-    bbytes = el * 2 * 5 + el * 2 + el * 4 * 3 + batch * length * heads * 8   # + grad_y in; dX out; dB, dC, dz fp32 out
+    bbytes = el * 2 * 6 + el * 2 * 4 + batch * length * heads * 8  # X, B, C, z, grad_y in; dX, dB, dC, dz out; dt, ddt
+    sbytes = el * 2 * 6 + el * 2 + el * 4 * 3 + batch * length * heads * 8   # dB, dC, dz in float32
     return {"fwd_us": round(fus, 1), "fwd_GBps": round(fbytes / fus / 1e3, 1),
             "fwd_frac_hbm": round(fbytes / fus / 1e3 / HBM_PEAK_GBPS, 4),
             "bwd_us": round(bus, 1), "bwd_GBps": round(bbytes / bus / 1e3, 1),
             "bwd_frac_hbm": round(bbytes / bus / 1e3 / HBM_PEAK_GBPS, 4),
+            "bwd_alone_fp32_grads_us": round(sus, 1), "bwd_alone_fp32_grads_GBps": round(sbytes / sus / 1e3, 1),
             "shape": f"X (B={batch}, L={length}, H={heads}, P={proj}) bf16, chunk {chunk}"}
 
 

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SSM_AMD_ABI_VERSION 3
+#define SSM_AMD_ABI_VERSION 4
 
 typedef enum ssm_status {
   SSM_OK = 0,
@@ -279,10 +279,16 @@ typedef struct ssm_dscan_fwd_args {
   int32_t x_dtype, dt_dtype, bc_dtype, z_dtype, init_dtype;
   int32_t b_kind, c_kind;     /* ssm_chunk_kind */
   int32_t a_per_p, d_per_p, z_per_p;
+  float *round_states;        /* optional output (B, ceil(L/64), H*P) fp32: the state entering every 64 steps, which
+                                 ssm_dscan_bwd_args.round_states takes; only for calls for which
+                                 ssm_dscan_fwd_one_pass() is non-zero (an error otherwise); or NULL */
 } ssm_dscan_fwd_args;
 
 size_t ssm_dscan_fwd_workspace_bytes(int batch, int seqlen, int heads, int proj);
 int ssm_dscan_fwd(const ssm_dscan_fwd_args *args, void *hip_stream);
+/* Non-zero when the call described (pointers included: alignment counts) runs the kernel that reads every input
+ * once; only that kernel can fill round_states.  No counterpart in the reference. */
+int ssm_dscan_fwd_one_pass(const ssm_dscan_fwd_args *args);
 
 /* Backward of the diagonal chunk scan.  Stands behind the backend call
  * `ssd_chunk_scan_backward(grad_out, X, dt, A, B, C, D, z, seq_lens, cu_seqlens,
@@ -301,9 +307,9 @@ typedef struct ssm_dscan_bwd_args {
   void *dX;                   /* (B, L, H, P) x dtype */
   float *ddt;                 /* (B, L, H) */
   float *dA;                  /* (H, P) if a_per_p else (H,) */
-  float *dB, *dC;             /* fp32, shaped like Bproj / Cproj */
+  void *dB, *dC;              /* shaped like Bproj / Cproj; fp32 (see grads_in_io_dtype) */
   float *dD;                  /* (H, P) if d_per_p else (H,), or NULL */
-  float *dz;                  /* fp32, shaped like z; given exactly when z is */
+  void *dz;                   /* shaped like z; fp32 (see grads_in_io_dtype); given exactly when z is */
   float *dinitial_states;     /* (B, H, P) fp32 or NULL */
   void *workspace;            /* ssm_dscan_bwd_workspace_bytes() bytes */
   size_t workspace_bytes;
@@ -311,6 +317,12 @@ typedef struct ssm_dscan_bwd_args {
   int32_t x_dtype, dt_dtype, bc_dtype, z_dtype, init_dtype;
   int32_t b_kind, c_kind;
   int32_t a_per_p, d_per_p, z_per_p;
+  int32_t grads_in_io_dtype;  /* non-zero: the gradients that have X's shape are written in their tensors' element
+                                 types instead of fp32: dB / dC when the projection is per token (bc dtype), dz when
+                                 the gate is per channel (z dtype); every other gradient stays fp32 */
+  int32_t tune_two_kernels;   /* non-zero keeps the general two-kernel path (for measurements and cross-checks) */
+  const float *round_states;  /* optional: what ssm_dscan_fwd wrote for the same inputs; spares the backward its own
+                                 forward sweep when it takes the one-pass kernels (ignored otherwise); or NULL */
 } ssm_dscan_bwd_args;
 
 size_t ssm_dscan_bwd_workspace_bytes(int batch, int seqlen, int heads, int proj);

@@ -19,7 +19,7 @@ import os
 # SSM_AMD_LIB points the binding at another build of the same C ABI.
 LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
                 Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
 PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
@@ -99,6 +99,7 @@ class DscanFwdArgs(C.Structure):
         ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("proj", _i32),
         ("x_dtype", _i32), ("dt_dtype", _i32), ("bc_dtype", _i32), ("z_dtype", _i32), ("init_dtype", _i32),
         ("b_kind", _i32), ("c_kind", _i32), ("a_per_p", _i32), ("d_per_p", _i32), ("z_per_p", _i32),
+        ("round_states", _vp),
     ]
 
 
@@ -111,6 +112,7 @@ class DscanBwdArgs(C.Structure):
         ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("proj", _i32),
         ("x_dtype", _i32), ("dt_dtype", _i32), ("bc_dtype", _i32), ("z_dtype", _i32), ("init_dtype", _i32),
         ("b_kind", _i32), ("c_kind", _i32), ("a_per_p", _i32), ("d_per_p", _i32), ("z_per_p", _i32),
+        ("grads_in_io_dtype", _i32), ("tune_two_kernels", _i32), ("round_states", _vp),
     ]
 
 
@@ -300,6 +302,7 @@ PLAIN_SYMBOLS = {
     "ssm_state_step_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 3),
     "ssm_dscan_fwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ssm_dscan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
+    "ssm_dscan_fwd_one_pass": (C.c_int, [C.POINTER(DscanFwdArgs)]),
     "ssm_ssd_chunk_state_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
     "ssm_ssd_mfma_launches": (C.c_int, []),
     "ssm_ssd_combined_supported": (C.c_int, [C.POINTER(SsdDims), C.c_int]),

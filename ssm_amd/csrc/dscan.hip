@@ -33,6 +33,7 @@ struct DscanParams {
   long long b_stride_b, b_stride_t, c_stride_b, c_stride_t;   // element strides of B / C (0 = broadcast)
   int z_per_p;                  // 1 for z (B,L,H,P), 0 for z (B,L,H)
   int seg_len, nseg;
+  float *round_states;          // (B, ceil(L/64), HP): the state entering every 64 steps, or null (one-pass kernel)
 };
 
 __device__ __forceinline__ void ds_store(void *p, int dtype, size_t i, float v) {
@@ -228,6 +229,16 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
         e[v] = __builtin_fmaf(f.x, e[v], v == 0 ? f.y : f.z);
       }
     }
+    if (p.round_states && (wave & (DO_WAVES / 2 - 1)) == 0) {
+      // what the backward starts its rounds of 64 steps from: the states entering wave 0's and wave 8's steps
+      const int rounds64 = (L + DO_ROUND / 2 - 1) / (DO_ROUND / 2);
+      const int k = 2 * r + wave / (DO_WAVES / 2);
+      if (k < rounds64) {
+        float *table = p.round_states + ((size_t)b * rounds64 + k) * HP + ch;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) table[v] = enter[v];
+      }
+    }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       carry[v] = e[v];
@@ -275,6 +286,25 @@ extern "C" size_t ssm_dscan_fwd_workspace_bytes(int batch, int seqlen, int heads
   return (size_t)batch * nseg * heads * proj * 2 * sizeof(float);
 }
 
+// One pass: per-token B and C of X's type, float32 dt, per-head A and D, a gate of X's shape or none, channels in
+// whole waves, vectors aligned.
+static bool dscan_fwd_takes_one_pass(const ssm_dscan_fwd_args *a) {
+  using namespace ssm;
+  if (!valid_dtype(a->x_dtype)) return false;
+  const long long HP = (long long)a->heads * a->proj;
+  const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
+  const int vec = a->x_dtype == SSM_F32 ? 1 : 2;
+  const size_t bytes = (size_t)vec * dtype_size(a->x_dtype);
+  return typed && a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP && !a->a_per_p && !a->d_per_p &&
+         (!a->z || a->z_per_p) && HP % (WAVE * vec) == 0 && a->proj % vec == 0 && aligned_to(a->X, bytes) &&
+         aligned_to(a->Bproj, bytes) && aligned_to(a->Cproj, bytes) && aligned_to(a->Y, bytes) &&
+         (!a->z || aligned_to(a->z, bytes)) && a->batch < 65536;
+}
+
+extern "C" int ssm_dscan_fwd_one_pass(const ssm_dscan_fwd_args *a) {
+  return a != nullptr && a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->proj > 0 && dscan_fwd_takes_one_pass(a);
+}
+
 extern "C" int ssm_dscan_fwd(const ssm_dscan_fwd_args *a, void *hip_stream) {
   using namespace ssm;
   SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_dscan_fwd: args is NULL");
@@ -320,20 +350,16 @@ extern "C" int ssm_dscan_fwd(const ssm_dscan_fwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid((unsigned)((HP + DS_THREADS - 1) / DS_THREADS), (unsigned)p.nseg, (unsigned)a->batch);
   const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
-  // one pass: per-token B and C, per-head A and D, a gate of X's shape or none, channels in whole waves
-  {
-    const int vec = a->x_dtype == SSM_F32 ? 1 : 2;
-    const size_t bytes = (size_t)vec * dtype_size(a->x_dtype);
-    if (typed && a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP && !a->a_per_p && !a->d_per_p &&
-        (!a->z || a->z_per_p) && HP % (WAVE * vec) == 0 && a->proj % vec == 0 && aligned_to(a->X, bytes) &&
-        aligned_to(a->Bproj, bytes) && aligned_to(a->Cproj, bytes) && aligned_to(a->Y, bytes) &&
-        (!a->z || aligned_to(a->z, bytes)) && a->batch < 65536) {
-      if (a->x_dtype == SSM_BF16) launch_onepass<bf16_t, 2>(p, s);
-      else if (a->x_dtype == SSM_F16) launch_onepass<f16_t, 2>(p, s);
-      else launch_onepass<float, 1>(p, s);
-      SSM_CHECK_LAUNCH("ssm_dscan_fwd");
-      return SSM_OK;
-    }
+  const bool one_pass = dscan_fwd_takes_one_pass(a);
+  SSM_REQUIRE(!a->round_states || (one_pass && aligned_to(a->round_states, 4)), SSM_ERR_BAD_SHAPE,
+              "ssm_dscan_fwd: round_states is only written by the one-pass kernel (ask ssm_dscan_fwd_one_pass first)");
+  if (one_pass) {
+    p.round_states = a->round_states;
+    if (a->x_dtype == SSM_BF16) launch_onepass<bf16_t, 2>(p, s);
+    else if (a->x_dtype == SSM_F16) launch_onepass<f16_t, 2>(p, s);
+    else launch_onepass<float, 1>(p, s);
+    SSM_CHECK_LAUNCH("ssm_dscan_fwd");
+    return SSM_OK;
   }
 #define SSM_DS_LAUNCH(T)                                                                   \
   {                                                                                        \

@@ -34,9 +34,11 @@ struct DscanBwdParams {
   float *states;                  // (B,L,HP) scratch
   float *ddt_p;                   // (B,L,HP) partial of ddt (summed over p afterwards); unused with ddt_direct
   float *ddt_direct;              // (B,L,H): written by the kernel when a head is exactly one wavefront
-  float *dz_p;                    // (B,L,HP): dz itself when z is per channel, else a partial
+  void *dz_p;                     // (B,L,HP): dz itself when z is per channel (element type g_z_dtype), else a float32 partial
   float *dz_direct;               // (B,L,H): per-head gate and a head is one wavefront
-  float *dB_t, *dC_t;             // (B,L,HP) when the projection is time-varying, else null
+  void *dB_t, *dC_t;              // (B,L,HP) when the projection is time-varying (element type g_bc_dtype), else null
+  int g_bc_dtype, g_z_dtype;      // float32 unless the caller asked for gradients in the tensors' own types
+  float *round_states;            // (B, ceil(L/64), HP): the state entering every 64 steps (one-pass kernels)
   float *fold;                    // (B, nseg, HP, 3): decay product, local state, local adjoint
   float *pA, *pD, *pB, *pC;       // (B, nseg, HP) sums over the segment's steps
   float *dinit;                   // (B,HP) or null
@@ -175,9 +177,9 @@ __global__ __launch_bounds__(DB_THREADS) void dscan_bwd_kernel(const DscanBwdPar
     if (p.ddt_direct) { if (pp == 0) p.ddt_direct[(row0 + t) * p.heads + h] = 0.0f; }
     else p.ddt_p[xi] = 0.0f;
     if (p.dz_direct) { if (pp == 0) p.dz_direct[(row0 + t) * p.heads + h] = 0.0f; }
-    else if (p.dz_p) p.dz_p[xi] = 0.0f;
-    if (p.dB_t) p.dB_t[xi] = 0.0f;
-    if (p.dC_t) p.dC_t[xi] = 0.0f;
+    else if (p.dz_p) db_store(p.dz_p, p.g_z_dtype, xi, 0.0f);
+    if (p.dB_t) db_store(p.dB_t, p.g_bc_dtype, xi, 0.0f);
+    if (p.dC_t) db_store(p.dC_t, p.g_bc_dtype, xi, 0.0f);
   }
 
   // reverse sweep
@@ -223,7 +225,7 @@ __global__ __launch_bounds__(DB_THREADS) void dscan_bwd_kernel(const DscanBwdPar
             const float tot = wave_sum(dzv);
             if (lane == 0) p.dz_direct[(row0 + t) * p.heads + h] = tot;
           } else {
-            p.dz_p[xi] = dzv;
+            db_store(p.dz_p, p.g_z_dtype, xi, dzv);
           }
           g0 = gv[j] * zv[j] * sg;
         }
@@ -237,8 +239,8 @@ __global__ __launch_bounds__(DB_THREADS) void dscan_bwd_kernel(const DscanBwdPar
           p.ddt_p[xi] = ddtv;
         }
         const float gB = lam * dtv[j] * xv[j], gC = g0 * st[j];
-        if (p.dB_t) p.dB_t[xi] = gB; else accB += gB;
-        if (p.dC_t) p.dC_t[xi] = gC; else accC += gC;
+        if (p.dB_t) db_store(p.dB_t, p.g_bc_dtype, xi, gB); else accB += gB;
+        if (p.dC_t) db_store(p.dC_t, p.g_bc_dtype, xi, gC); else accC += gC;
         accA = __builtin_fmaf(lam * sprev, a * dtv[j], accA);
         accD = __builtin_fmaf(g0, xv[j], accD);
         lam_next_a = lam * a;
@@ -254,6 +256,8 @@ __global__ __launch_bounds__(DB_THREADS) void dscan_bwd_kernel(const DscanBwdPar
 }
 
 }  // namespace ssm
+
+#include "dscan_bwd_onepass.hpp"
 
 // Workspace (floats): states, ddt partial, dz partial (dB/dC time-varying copies are outputs
 // themselves); then per (batch, segment, channel) the three folds and four partial sums.
@@ -309,9 +313,12 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   p.A = a->A; p.Dk = a->Dskip; p.lengths = a->seq_lens; p.dX = a->dX;
   p.states = ws; p.ddt_p = ws + blhp;
   const bool dz_direct = a->z && a->z_per_p;
-  p.dz_p = !a->z ? nullptr : (dz_direct ? a->dz : ws + 2 * blhp);
+  p.dz_p = !a->z ? nullptr : (dz_direct ? a->dz : (void *)(ws + 2 * blhp));
   p.dB_t = a->b_kind == SSM_CHUNK_BLHP ? a->dB : nullptr;
   p.dC_t = a->c_kind == SSM_CHUNK_BLHP ? a->dC : nullptr;
+  const bool grads_io = a->grads_in_io_dtype != 0;
+  p.g_bc_dtype = grads_io ? a->bc_dtype : SSM_F32;
+  p.g_z_dtype = (grads_io && dz_direct) ? a->z_dtype : SSM_F32;
   p.fold = ws + 3 * blhp;
   p.pA = p.fold + 3 * bshp; p.pD = p.pA + bshp; p.pB = p.pD + bshp; p.pC = p.pB + bshp;
   p.dinit = a->dinitial_states;
@@ -319,7 +326,7 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   // a head of 64 channels is one wavefront: the sums over p are taken in the kernel
   const bool wave_heads = P == WAVE;
   p.ddt_direct = wave_heads ? a->ddt : nullptr;
-  p.dz_direct = (wave_heads && a->z && !a->z_per_p) ? a->dz : nullptr;
+  p.dz_direct = (wave_heads && a->z && !a->z_per_p) ? reinterpret_cast<float *>(a->dz) : nullptr;
   p.batch = Bn; p.len = L; p.heads = H; p.proj = P;
   p.x_dtype = a->x_dtype; p.dt_dtype = a->dt_dtype; p.bc_dtype = a->bc_dtype; p.z_dtype = a->z_dtype;
   p.init_dtype = a->init_dtype;
@@ -336,6 +343,30 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid((unsigned)((HP + DB_THREADS - 1) / DB_THREADS), (unsigned)nseg, (unsigned)Bn);
   const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
+  // one pass: per-token B and C, per-head A and D, a gate of X's shape or none, a head's channels in 16, 32 or 64 lanes
+  const int vec = a->x_dtype == SSM_F32 ? 1 : 2;
+  const size_t vbytes = (size_t)vec * dtype_size(a->x_dtype);
+  const size_t gbytes = grads_io ? vbytes : (size_t)vec * 4;
+  const int lph = P % vec == 0 ? P / vec : 0;
+  const bool onepass = a->tune_two_kernels == 0 && typed && a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP &&
+                       !a->a_per_p && !a->d_per_p && (!a->z || a->z_per_p) && (lph == 16 || lph == 32 || lph == 64) &&
+                       HP % (WAVE * vec) == 0 && (size_t)L * HP < ((size_t)1 << 30) && aligned_to(a->X, vbytes) && aligned_to(a->grad_y, vbytes) &&
+                       aligned_to(a->Bproj, vbytes) && aligned_to(a->Cproj, vbytes) && aligned_to(a->dX, vbytes) &&
+                       (!a->z || aligned_to(a->z, vbytes)) && aligned_to(a->dB, gbytes) && aligned_to(a->dC, gbytes) &&
+                       (!a->z || aligned_to(a->dz, gbytes));
+  if (onepass) {
+    const int rounds = (L + DBO_ROUND - 1) / DBO_ROUND;
+    p.round_states = a->round_states ? const_cast<float *>(a->round_states) : ws;
+    p.pA = ws + (size_t)Bn * rounds * HP;
+    p.pD = p.pA + bhp;
+    p.ddt_direct = a->ddt;
+    nseg = 1;
+    const bool sweep = a->round_states == nullptr;      // no table from the forward: make it
+    if (a->x_dtype == SSM_BF16) launch_bwd_onepass<bf16_t, 2>(p, grads_io, sweep, s);
+    else if (a->x_dtype == SSM_F16) launch_bwd_onepass<f16_t, 2>(p, grads_io, sweep, s);
+    else launch_bwd_onepass<float, 1>(p, grads_io, sweep, s);
+    SSM_CHECK_LAUNCH("ssm_dscan_bwd");
+  } else {
 #define SSM_DB_LAUNCH(T)                                                                       \
   {                                                                                            \
     if (nseg > 1) hipLaunchKernelGGL(dscan_bwd_fold_kernel<T>, grid, dim3(DB_THREADS), 0, s, p); \
@@ -347,10 +378,11 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   else SSM_DB_LAUNCH(void)
 #undef SSM_DB_LAUNCH
   SSM_CHECK_LAUNCH("ssm_dscan_bwd");
+  }
 
   // ddt (B,L,H) and, for a per-head gate, dz (B,L,H): sums over p, unless the kernel took them itself
   if (!p.ddt_direct) launch_fold_sum(p.ddt_p, a->ddt, (size_t)Bn * L * H, P, 1, s);
-  if (a->z && !dz_direct && !p.dz_direct) launch_fold_sum(p.dz_p, a->dz, (size_t)Bn * L * H, P, 1, s);
+  if (a->z && !dz_direct && !p.dz_direct) launch_fold_sum(reinterpret_cast<const float *>(p.dz_p), reinterpret_cast<float *>(a->dz), (size_t)Bn * L * H, P, 1, s);
   // sums over batch and segments, then over p when the parameter is per head; `states` is free again
   // and serves as the (H,P) intermediate
   float *tmp = p.states;
@@ -367,8 +399,8 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
     if (kind == SSM_CHUNK_HP) launch_fold_rows(partial, out, Bn * nseg, (size_t)HP, s);
     else if (kind == SSM_CHUNK_BHP) launch_fold_sum(partial, out, (size_t)Bn, nseg, (size_t)HP, s);
   };
-  fold_proj(a->b_kind, p.pB, a->dB);
-  fold_proj(a->c_kind, p.pC, a->dC);
+  fold_proj(a->b_kind, p.pB, reinterpret_cast<float *>(a->dB));
+  fold_proj(a->c_kind, p.pC, reinterpret_cast<float *>(a->dC));
   SSM_CHECK_LAUNCH("ssm_dscan_bwd(fold)");
   return SSM_OK;
 }

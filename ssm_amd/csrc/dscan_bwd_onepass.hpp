@@ -1,0 +1,398 @@
+// Backward of the diagonal chunked scan for the common call (per-token B and C of X's shape and type,
+// float32 dt, per-head A and D, a gate of X's shape or none, a head's channels in 16, 32 or 64 lanes):
+// every input is read once by the kernel that forms the gradients, no state goes through memory.
+//
+// A workgroup of 16 waves owns 64 * VEC neighbouring channels of one batch row and walks time backwards in
+// rounds of 64 steps, wave w taking steps 4w..4w+3 of the round.  In a round every wave folds its steps twice
+// from zero: forwards into (decay product, state) and backwards into the adjoint it would hand to the steps
+// before it (mu_t = lambda_t a_t obeys mu_t = a_t (mu_{t+1} + g0_t C_t): the same decays).  The 16 pairs of
+// folds meet in LDS (one barrier per round, two buffers); wave w chains the folds of the waves before it from
+// the state entering the round on the left, and those of the waves after it from the adjoint entering the round
+// on the right (15 links in all, whatever w), which gives it what enters its own steps from both sides, then
+// replays its steps forwards (states, kept in registers) and backwards (gradients).  Wave 0's chain ends at the
+// round's left edge: it leaves the adjoint there in LDS for everyone's next round.  The state entering a round
+// comes from a table written beforehand by dscan_round_states_kernel, a forward sweep of the same shape that
+// reads only X, B and dt.  The reads of the next round are requested before the arithmetic of this one.
+#pragma once
+
+namespace ssm {
+
+constexpr int DBO_WAVES = 16, DBO_SEG = 4, DBO_ROUND = DBO_WAVES * DBO_SEG;
+
+// Sum over each group of LPH neighbouring lanes (16, 32 or 64), valid in the group's last lane.
+template <int LPH>
+__device__ __forceinline__ float lane_group_sum_last(float v) {
+  v += dpp_move<DPP_ROW_SHR1, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR2, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR4, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR8, 0xf>(0.0f, v);
+  if (LPH >= 32) v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.0f, v);
+  if (LPH >= 64) v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.0f, v);
+  return v;
+}
+
+// ---- the state entering every round of 64 steps: (B, rounds, HP) float32
+// Same walk as the forward's one-pass kernel (16 waves, 8 steps each, rounds of 128 steps) without C, the gate
+// and the output; the state in the middle of a round is the chain's value in front of wave 8.
+constexpr int DRS_WAVES = 16, DRS_SEG = 8, DRS_ROUND = DRS_WAVES * DRS_SEG;
+static_assert(DRS_ROUND == 2 * DBO_ROUND, "two rounds of the backward per round of the table's sweep");
+
+template <typename io_t, int VEC>
+struct DrsRegs {
+  float dt[DRS_SEG];
+  Pack<io_t, VEC> x[DRS_SEG], bq[DRS_SEG];
+};
+
+template <typename io_t, int VEC>
+__global__ __launch_bounds__(WAVE *DRS_WAVES) void dscan_round_states_kernel(const DscanBwdParams p) {
+  __shared__ float4 segs[2][DRS_WAVES][WAVE];
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int HP = p.heads * p.proj;
+  const int ch = ((int)blockIdx.x * WAVE + lane) * VEC;
+  const int b = blockIdx.y;
+  const int h = ch / p.proj;
+  const int L = p.len;
+  const int valid = p.lengths ? min(max(p.lengths[b], 0), L) : L;
+  const float A2 = p.A[h] * LOG2E;
+  const io_t *X = reinterpret_cast<const io_t *>(p.X), *Bp = reinterpret_cast<const io_t *>(p.Bp);
+  const float *DT = reinterpret_cast<const float *>(p.dt);
+  const size_t row0 = (size_t)b * L;
+  const int rounds64 = (L + DBO_ROUND - 1) / DBO_ROUND;
+  float *table = p.round_states + (size_t)b * rounds64 * HP + ch;
+  float carry[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) carry[v] = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + ch + v) : 0.0f;
+
+  auto request = [&](DrsRegs<io_t, VEC> &r, int round) {
+    const int t0 = round * DRS_ROUND + wave * DRS_SEG;
+#pragma unroll
+    for (int j = 0; j < DRS_SEG; ++j) {
+      const size_t row = row0 + min(t0 + j, L - 1);            // steps past the end read the last row, unused
+      const size_t at = row * HP + ch;
+      r.dt[j] = DT[row * p.heads + h];
+      r.x[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(X + at);
+      r.bq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Bp + at);
+    }
+  };
+
+  const int rounds = (L + DRS_ROUND - 1) / DRS_ROUND;
+  DrsRegs<io_t, VEC> cur, nxt;
+  request(cur, 0);
+  for (int r = 0; r < rounds; ++r) {
+    if (r + 1 < rounds) request(nxt, r + 1);
+    const int t0 = r * DRS_ROUND + wave * DRS_SEG;
+    float s[VEC], prod = 1.0f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) s[v] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < DRS_SEG; ++j) {
+      const bool live = t0 + j < valid;
+      const float a = live ? exp2_hw(cur.dt[j] * A2) : 1.0f;
+      prod *= a;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v)
+        s[v] = __builtin_fmaf(a, s[v], live ? cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]) : 0.0f);
+    }
+    segs[r & 1][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
+    __syncthreads();
+    float e[VEC], mid[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) e[v] = mid[v] = carry[v];
+#pragma unroll
+    for (int w = 0; w < DRS_WAVES; ++w) {
+      const float4 f = segs[r & 1][w][lane];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        mid[v] = w == DRS_WAVES / 2 ? e[v] : mid[v];
+        e[v] = __builtin_fmaf(f.x, e[v], v == 0 ? f.y : f.z);
+      }
+    }
+    if (wave == 0) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        table[(size_t)(2 * r) * HP + v] = carry[v];
+        if (2 * r + 1 < rounds64) table[(size_t)(2 * r + 1) * HP + v] = mid[v];
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) carry[v] = e[v];
+    cur = nxt;
+  }
+}
+
+// ---- the gradients
+template <typename io_t, int VEC, bool HAS_Z>
+struct DboRegs {
+  float dt[DBO_SEG];
+  Pack<io_t, VEC> x[DBO_SEG], bq[DBO_SEG], cq[DBO_SEG], gq[DBO_SEG], zq[DBO_SEG];
+  float enter[VEC];                 // the state entering the round
+};
+
+// The bits of a vector of elements as they sit in registers, and back.
+template <typename io_t, int VEC>
+struct DboBits {
+  using type = typename std::conditional<sizeof(Pack<io_t, VEC>) == 4, unsigned, unsigned long long>::type;
+};
+
+// Zero when the step is past the row's length (every tensor of a dead step reads as zero: the step is the
+// identity, adds nothing and receives nothing), and opaque to the compiler: the float32 values of a vector are
+// formed again where they are used instead of being kept from one phase of a round to the next.
+template <typename io_t, int VEC>
+__device__ __forceinline__ void dbo_mask(Pack<io_t, VEC> &v, bool live) {
+  using bits_t = typename DboBits<io_t, VEC>::type;
+  static_assert(sizeof(bits_t) == sizeof(Pack<io_t, VEC>), "one or two registers");
+  bits_t raw = __builtin_bit_cast(bits_t, v);
+  raw = live ? raw : bits_t(0);
+  v = __builtin_bit_cast(Pack<io_t, VEC>, raw);
+}
+template <typename io_t, int VEC>
+__device__ __forceinline__ void dbo_launder(Pack<io_t, VEC> &v) {
+  using bits_t = typename DboBits<io_t, VEC>::type;
+  bits_t raw = __builtin_bit_cast(bits_t, v);
+  __asm__ volatile("" : "+v"(raw));
+  v = __builtin_bit_cast(Pack<io_t, VEC>, raw);
+}
+
+// A wave-uniform base plus a 32-bit byte offset per lane: the form of address the memory instructions take as
+// it is (a base in scalar registers, an offset in one vector register), with no 64-bit arithmetic per access.
+template <typename T, typename B>
+__device__ __forceinline__ T *at_bytes(B *base, unsigned bytes) {
+  using C = typename std::conditional<std::is_const<B>::value, const char, char>::type;
+  return reinterpret_cast<T *>(reinterpret_cast<C *>(base) + bytes);
+}
+
+// g_t: element type of dB, dC and dz (io_t, or float).  LPH: lanes that hold one head's channels.
+template <typename io_t, typename g_t, int VEC, bool HAS_Z, int LPH>
+__global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
+  static_assert(sizeof(Pack<io_t, VEC>) == 4 || sizeof(Pack<io_t, VEC>) == 8, "a lane's vector is one or two registers");
+  __shared__ float4 fwd[2][DBO_WAVES][WAVE];     // a wave's four steps per lane: decay product, state from zero (per channel)
+  __shared__ float2 rev[2][DBO_WAVES][WAVE];     // ... and the adjoint (times its decay) from zero
+  __shared__ float2 left[2][WAVE];               // the adjoint leaving the round, from wave 0 to everyone's next round
+  const int wave = wave_id_uniform(), lane = lane_id();
+  const int HP = p.heads * p.proj;
+  const unsigned ch = ((unsigned)blockIdx.x * WAVE + lane) * VEC;
+  const int b = blockIdx.y;
+  const int h = (int)ch / p.proj;
+  const int L = p.len;
+  const int valid = p.lengths ? min(max(p.lengths[b], 0), L) : L;
+  const float A = p.A[h], A2 = A * LOG2E;
+  const float Dk = p.Dk ? p.Dk[h] : 0.0f;
+  // the batch row's part of every tensor: offsets inside it fit 32 bits (checked by the host)
+  const size_t row0 = (size_t)b * L;
+  const io_t *X = reinterpret_cast<const io_t *>(p.X) + row0 * HP, *Bp = reinterpret_cast<const io_t *>(p.Bp) + row0 * HP;
+  const io_t *Cp = reinterpret_cast<const io_t *>(p.Cp) + row0 * HP, *G = reinterpret_cast<const io_t *>(p.gy) + row0 * HP;
+  const io_t *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.X) + row0 * HP;
+  const float *DT = reinterpret_cast<const float *>(p.dt) + row0 * p.heads;
+  io_t *dX = reinterpret_cast<io_t *>(p.dX) + row0 * HP;
+  g_t *dB = reinterpret_cast<g_t *>(p.dB_t) + row0 * HP, *dC = reinterpret_cast<g_t *>(p.dC_t) + row0 * HP;
+  g_t *dZ = reinterpret_cast<g_t *>(HAS_Z ? p.dz_p : p.dB_t) + row0 * HP;
+  float *DDT = p.ddt_direct + row0 * p.heads;
+  const int rounds = (L + DBO_ROUND - 1) / DBO_ROUND;
+  const float *table = p.round_states + (size_t)b * rounds * HP;
+
+  auto request = [&](DboRegs<io_t, VEC, HAS_Z> &r, int round) {
+    const int t0 = round * DBO_ROUND + wave * DBO_SEG;
+#pragma unroll
+    for (int j = 0; j < DBO_SEG; ++j) {
+      const unsigned row = (unsigned)min(t0 + j, L - 1);       // steps past the end read the last row, unused
+      const unsigned at = (row * (unsigned)HP + ch) * (unsigned)sizeof(io_t);
+      r.dt[j] = *at_bytes<const float>(DT, (row * (unsigned)p.heads + (unsigned)h) * 4u);
+      r.x[j] = *at_bytes<const Pack<io_t, VEC>>(X, at);
+      r.bq[j] = *at_bytes<const Pack<io_t, VEC>>(Bp, at);
+      r.cq[j] = *at_bytes<const Pack<io_t, VEC>>(Cp, at);
+      r.gq[j] = *at_bytes<const Pack<io_t, VEC>>(G, at);
+      if (HAS_Z) r.zq[j] = *at_bytes<const Pack<io_t, VEC>>(Z, at);
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) r.enter[v] = *at_bytes<const float>(table, ((unsigned)round * (unsigned)HP + ch + v) * 4u);
+  };
+
+  float accA[VEC], accD[VEC], mu_left[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) accA[v] = accD[v] = mu_left[v] = 0.0f;
+
+  auto round_of = [&](DboRegs<io_t, VEC, HAS_Z> &cur, int r) {
+    const int q = r & 1;
+    const int t0 = r * DBO_ROUND + wave * DBO_SEG;
+    float a[DBO_SEG], sg[VEC][DBO_SEG];
+    float s[VEC], M[VEC], prod = 1.0f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) s[v] = M[v] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < DBO_SEG; ++j) {
+      const bool live = t0 + j < valid;
+      cur.dt[j] = live ? cur.dt[j] : 0.0f;
+      dbo_mask<io_t, VEC>(cur.x[j], live);
+      dbo_mask<io_t, VEC>(cur.bq[j], live);
+      dbo_mask<io_t, VEC>(cur.cq[j], live);
+      dbo_mask<io_t, VEC>(cur.gq[j], live);
+      if (HAS_Z) dbo_mask<io_t, VEC>(cur.zq[j], live);
+      a[j] = exp2_hw(cur.dt[j] * A2);
+      prod *= a[j];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v)
+        s[v] = __builtin_fmaf(a[j], s[v], cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]));
+    }
+#pragma unroll
+    for (int j = DBO_SEG - 1; j >= 0; --j) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        float g0 = to_f32(cur.gq[j].v[v]);
+        if (HAS_Z) {
+          const float zz = to_f32(cur.zq[j].v[v]);
+          sg[v][j] = sigmoid_f32(zz);
+          g0 *= zz * sg[v][j];
+        }
+        M[v] = a[j] * __builtin_fmaf(g0, to_f32(cur.cq[j].v[v]), M[v]);
+      }
+    }
+    fwd[q][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
+    rev[q][wave][lane] = make_float2(M[0], M[VEC - 1]);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < DBO_SEG; ++j) {
+      dbo_launder<io_t, VEC>(cur.x[j]);
+      dbo_launder<io_t, VEC>(cur.bq[j]);
+      dbo_launder<io_t, VEC>(cur.cq[j]);
+      dbo_launder<io_t, VEC>(cur.gq[j]);
+      if (HAS_Z) dbo_launder<io_t, VEC>(cur.zq[j]);
+    }
+    // the state entering this wave's steps: the folds of the waves before it, from the state entering the round
+    float st[VEC][DBO_SEG + 1];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) st[v][0] = cur.enter[v];
+    for (int w = 0; w < wave; ++w) {
+      const float4 f = fwd[q][w][lane];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) st[v][0] = __builtin_fmaf(f.x, st[v][0], v == 0 ? f.y : f.z);
+    }
+    // the adjoint entering them: the folds of the waves after it, from the adjoint that left the round before
+    float mu[VEC];
+    if (r < rounds - 1) {
+      const float2 c = left[q ^ 1][lane];
+      mu_left[0] = c.x;
+      mu_left[VEC - 1] = c.y;
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) mu[v] = mu_left[v];
+    for (int w = DBO_WAVES - 1; w > wave; --w) {
+      const float pr = fwd[q][w][lane].x;
+      const float2 f = rev[q][w][lane];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) mu[v] = __builtin_fmaf(pr, mu[v], v == 0 ? f.x : f.y);
+    }
+    if (wave == 0) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) mu_left[v] = __builtin_fmaf(prod, mu[v], M[v]);
+      left[q][lane] = make_float2(mu_left[0], mu_left[VEC - 1]);
+    }
+    // forward replay: st[v][j + 1] = the state after step j
+#pragma unroll
+    for (int j = 0; j < DBO_SEG; ++j) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v)
+        st[v][j + 1] = __builtin_fmaf(a[j], st[v][j], cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]));
+    }
+    // backward replay; mu[v] is lambda_{t+1} a_{t+1}
+#pragma unroll
+    for (int j = DBO_SEG - 1; j >= 0; --j) {
+      const int t = t0 + j;
+      Pack<io_t, VEC> ox;
+      Pack<g_t, VEC> ob, oc, oz;
+      float ddt = 0.0f;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        const float xv = to_f32(cur.x[j].v[v]), bv = to_f32(cur.bq[j].v[v]), cv = to_f32(cur.cq[j].v[v]);
+        float g0 = to_f32(cur.gq[j].v[v]);
+        if (HAS_Z) {
+          const float zz = to_f32(cur.zq[j].v[v]);
+          const float y0 = __builtin_fmaf(st[v][j + 1], cv, Dk * xv);
+          oz.v[v] = from_f32<g_t>(g0 * y0 * sg[v][j] * __builtin_fmaf(zz, 1.0f - sg[v][j], 1.0f));
+          g0 *= zz * sg[v][j];
+        }
+        const float lam = __builtin_fmaf(g0, cv, mu[v]);
+        const float ld = lam * cur.dt[j];
+        ox.v[v] = from_f32<io_t>(__builtin_fmaf(g0, Dk, ld * bv));
+        ob.v[v] = from_f32<g_t>(ld * xv);
+        oc.v[v] = from_f32<g_t>(g0 * st[v][j + 1]);
+        const float sa = st[v][j] * a[j];
+        ddt = __builtin_fmaf(lam, __builtin_fmaf(sa, A, bv * xv), ddt);
+        accA[v] = __builtin_fmaf(lam * sa, cur.dt[j], accA[v]);
+        accD[v] = __builtin_fmaf(g0, xv, accD[v]);
+        mu[v] = lam * a[j];
+      }
+      const float head = lane_group_sum_last<LPH>(ddt);
+      if (t < L) {
+        const unsigned at = (unsigned)t * (unsigned)HP + ch;
+        *at_bytes<Pack<io_t, VEC>>(dX, at * (unsigned)sizeof(io_t)) = ox;
+        *at_bytes<Pack<g_t, VEC>>(dB, at * (unsigned)sizeof(g_t)) = ob;
+        *at_bytes<Pack<g_t, VEC>>(dC, at * (unsigned)sizeof(g_t)) = oc;
+        if (HAS_Z) *at_bytes<Pack<g_t, VEC>>(dZ, at * (unsigned)sizeof(g_t)) = oz;
+        if ((lane & (LPH - 1)) == LPH - 1) *at_bytes<float>(DDT, ((unsigned)t * (unsigned)p.heads + (unsigned)h) * 4u) = head;
+      }
+    }
+  };
+
+  // two sets of registers take turns: one is worked on while the other's reads are in flight
+  DboRegs<io_t, VEC, HAS_Z> ra, rb;
+  request(ra, rounds - 1);
+  for (int r = rounds - 1; r >= 0; r -= 2) {
+    if (r > 0) request(rb, r - 1);
+    round_of(ra, r);
+    if (r > 0) {
+      if (r > 1) request(ra, r - 2);
+      round_of(rb, r - 1);
+    }
+  }
+
+  // sums over time of the whole walk: the 16 waves' shares meet in LDS (after everyone has left the last round)
+  __syncthreads();
+  float *red = reinterpret_cast<float *>(&fwd[0][0][0]);        // [2 VEC][16][64] floats fit the first buffer
+  static_assert(2 * VEC <= 4, "the sums fit the buffer of one round's folds");
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    red[((2 * v) * DBO_WAVES + wave) * WAVE + lane] = accA[v];
+    red[((2 * v + 1) * DBO_WAVES + wave) * WAVE + lane] = accD[v];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      float sa = 0.0f, sd = 0.0f;
+#pragma unroll
+      for (int w = 0; w < DBO_WAVES; ++w) {
+        sa += red[((2 * v) * DBO_WAVES + w) * WAVE + lane];
+        sd += red[((2 * v + 1) * DBO_WAVES + w) * WAVE + lane];
+      }
+      p.pA[(size_t)b * HP + ch + v] = sa;
+      p.pD[(size_t)b * HP + ch + v] = sd;
+      if (p.dinit) p.dinit[(size_t)b * HP + ch + v] = mu_left[v];     // lambda_0 a_0
+    }
+  }
+}
+
+template <typename io_t, typename g_t, int VEC, bool HAS_Z>
+static void launch_dbo_lph(const DscanBwdParams &p, int lph, hipStream_t s) {
+  const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
+  const dim3 block(WAVE * DBO_WAVES);
+  if (lph == 16) hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 16>), grid, block, 0, s, p);
+  else if (lph == 32) hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 32>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 64>), grid, block, 0, s, p);
+}
+
+// The kernels of the one-pass backward for one element type (`sweep`: the table of round states is made here).
+template <typename io_t, int VEC>
+static void launch_bwd_onepass(const DscanBwdParams &p, bool grads_io, bool sweep, hipStream_t s) {
+  const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
+  if (sweep) hipLaunchKernelGGL((dscan_round_states_kernel<io_t, VEC>), grid, dim3(WAVE * DRS_WAVES), 0, s, p);
+  const int lph = p.proj / VEC;
+  if (grads_io) {
+    if (p.z) launch_dbo_lph<io_t, io_t, VEC, true>(p, lph, s);
+    else launch_dbo_lph<io_t, io_t, VEC, false>(p, lph, s);
+  } else {
+    if (p.z) launch_dbo_lph<io_t, float, VEC, true>(p, lph, s);
+    else launch_dbo_lph<io_t, float, VEC, false>(p, lph, s);
+  }
+}
+
+}  // namespace ssm

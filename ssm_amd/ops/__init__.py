@@ -503,9 +503,12 @@ def conv_window_step(conv_state, x, weight, bias=None, activation="silu"):
 # diagonal chunk scan (the reference's ``ssd_chunk_scan``)
 # ---------------------------------------------------------------------------
 
-def _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states):
+def _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states, want_round_states=False):
     """Validate, normalise dtypes/layout, and run ``ssm_dscan_fwd``; ``lengths`` is the
-    int32 device tensor of valid steps per batch row (or ``None``)."""
+    int32 device tensor of valid steps per batch row (or ``None``).  With ``want_round_states``
+    returns ``(Y, round_states)``: the state entering every 64 steps, ``(B, ceil(L/64), H*P)`` float32, which
+    :func:`_dscan_backward` takes instead of sweeping forward itself -- or ``None`` when the call does not run the
+    kernel that can write it."""
     batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p = \
         K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
     dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states)
@@ -527,13 +530,22 @@ def _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states):
         z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
         init_dtype=_lib.dtype_enum(ic.dtype) if ic is not None else 0,
         b_kind=bk, c_kind=ck, a_per_p=int(a_per_p), d_per_p=int(d_per_p), z_per_p=int(z_per_p))
+    table = None
+    if want_round_states and _lib.load().ssm_dscan_fwd_one_pass(args):
+        table = torch.empty(batch, (seqlen + 63) // 64, heads * proj, dtype=torch.float32, device=dev)
+        args.round_states = _lib.ptr(table)
     _lib.call("ssm_dscan_fwd", args, dev)
-    return Y
+    return (Y, table) if want_round_states else Y
 
 
-def _dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_states):
+def _dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_states, grads_in_input_dtype=False,
+                    two_kernels=False, round_states=None):
     """Run ``ssm_dscan_bwd``: gradients ``(dX, ddt, dA, dB, dC, dD, dz, dinitial_states)``.
-    ``dX`` comes back in ``X.dtype``, the rest in float32 with the shape of its tensor."""
+    ``dX`` comes back in ``X.dtype``, the rest in float32 with the shape of its tensor; with
+    ``grads_in_input_dtype`` the kernel writes a per-token ``dB`` / ``dC`` and a per-channel ``dz`` in their
+    tensors' own types (no float32 copy of a tensor of ``X``'s size is made and converted afterwards).
+    ``two_kernels`` keeps the general path for a call the one-pass kernels cover; ``round_states`` is what
+    :func:`_dscan_forward` returned for the same inputs (or ``None``)."""
     batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p = \
         K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
     dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states, grad_y)
@@ -548,9 +560,13 @@ def _dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_s
     dX = torch.empty_like(Xc)
     ddt = torch.empty(batch, seqlen, heads, **f32)
     dA = torch.empty(A.shape, **f32)
-    dB, dC = torch.empty(Bc.shape, **f32), torch.empty(Cc.shape, **f32)
+    io = bool(grads_in_input_dtype)
+    dB = torch.empty(Bc.shape, dtype=bc if (io and bk == _lib.CHUNK_BLHP) else torch.float32, device=dev)
+    dC = torch.empty(Cc.shape, dtype=bc if (io and ck == _lib.CHUNK_BLHP) else torch.float32, device=dev)
     dD = torch.empty(D.shape, **f32) if D is not None else None
-    dz = torch.empty(zc.shape, **f32) if zc is not None else None
+    dz = None
+    if zc is not None:
+        dz = torch.empty(zc.shape, dtype=zc.dtype if (io and z_per_p) else torch.float32, device=dev)
     dinit = torch.empty(batch, heads, proj, **f32) if ic is not None else None
     nbytes = int(_lib.load().ssm_dscan_bwd_workspace_bytes(batch, seqlen, heads, proj))
     ws = torch.empty(nbytes // 4, **f32)
@@ -563,7 +579,13 @@ def _dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_s
         x_dtype=_lib.dtype_enum(Xc.dtype), dt_dtype=_lib.dtype_enum(dtc.dtype), bc_dtype=_lib.dtype_enum(bc),
         z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
         init_dtype=_lib.dtype_enum(ic.dtype) if ic is not None else 0,
-        b_kind=bk, c_kind=ck, a_per_p=int(a_per_p), d_per_p=int(d_per_p), z_per_p=int(z_per_p))
+        b_kind=bk, c_kind=ck, a_per_p=int(a_per_p), d_per_p=int(d_per_p), z_per_p=int(z_per_p),
+        grads_in_io_dtype=int(io), tune_two_kernels=int(bool(two_kernels)))
+    if round_states is not None:
+        want = (batch, (seqlen + 63) // 64, heads * proj)
+        if tuple(round_states.shape) != want or round_states.dtype != torch.float32 or not round_states.is_contiguous():
+            raise ValueError(f"round_states must be a contiguous float32 tensor of shape {want}.")
+        args.round_states = _lib.ptr(round_states)
     _lib.call("ssm_dscan_bwd", args, dev)
     return dX, ddt, dA, dB, dC, dD, dz, dinit
 

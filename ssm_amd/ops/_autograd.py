@@ -127,8 +127,9 @@ class DiagScanFn(torch.autograd.Function):
     def forward(ctx, X, dt, A, B, C, chunk_size, D, z, lengths, initial_states):
         from . import _dscan_forward
 
-        Y = _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states)
-        ctx.save_for_backward(X, dt, A, B, C, D, z, lengths, initial_states)
+        # the forward leaves the state entering every 64 steps for the backward when its kernel can
+        Y, table = _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states, want_round_states=True)
+        ctx.save_for_backward(X, dt, A, B, C, D, z, lengths, initial_states, table)
         ctx.chunk_size = chunk_size
         return Y
 
@@ -136,9 +137,9 @@ class DiagScanFn(torch.autograd.Function):
     def backward(ctx, grad_y):
         from . import _dscan_backward
 
-        X, dt, A, B, C, D, z, lengths, init = ctx.saved_tensors
+        X, dt, A, B, C, D, z, lengths, init, table = ctx.saved_tensors
         dX, ddt, dA, dB, dC, dD, dz, dinit = _dscan_backward(grad_y, X, dt, A, B, C, ctx.chunk_size, D, z, lengths,
-                                                             init)
+                                                             init, grads_in_input_dtype=True, round_states=table)
         need = ctx.needs_input_grad
         pick = lambda i, g, r: _like(g, r) if (r is not None and need[i]) else None
         return (pick(0, dX, X), pick(1, ddt, dt), pick(2, dA, A), pick(3, dB, B), pick(4, dC, C), None,

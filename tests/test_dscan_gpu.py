@@ -191,7 +191,7 @@ def test_one_pass_call_shape(dtype, hp, length, z_mode, d_mode, init, ragged):
     multiple of a round, with an entering state and with rows that end early."""
     h, p = hp
     b = 3
-    inp = make(length + h, b, length, h, p, dtype=dtype, d_mode=d_mode, z_mode=z_mode, init=init)
+    inp = make(length + h, b, length, h, p, dtype=dtype, a_vec=True, d_mode=d_mode, z_mode=z_mode, init=init)
     inp["dt"] = inp["dt"].float()
     meta = {"seq_lens": [length, max(length // 3, 0), 0]} if ragged else None
     y, yr = both(inp, meta=meta)
@@ -199,3 +199,73 @@ def test_one_pass_call_shape(dtype, hp, length, z_mode, d_mode, init, ragged):
     torch.testing.assert_close(y.float(), yr.float(), **(FP32_TOL if dtype == torch.float32 else HALF_TOL))
     if ragged:
         assert torch.count_nonzero(y[2]) == 0 and torch.count_nonzero(y[1, length // 3:]) == 0
+
+
+@pytest.mark.parametrize("dtype,hp", [(torch.bfloat16, (4, 64)), (torch.float16, (2, 128)), (torch.float32, (3, 64)),
+                                      (torch.bfloat16, (8, 32)), (torch.float32, (8, 16))],
+                         ids=lambda v: str(v).replace("torch.", ""))
+@pytest.mark.parametrize("length,z_mode,d_mode,init,ragged", [(333, 4, "vec", True, False), (128, 0, "none", False, False),
+                                                               (200, 4, "vec", False, True), (7, 4, "none", True, True)])
+def test_one_pass_backward_call_shape(dtype, hp, length, z_mode, d_mode, init, ragged):
+    """The same call shape backwards (a table of the states entering every 64 steps, then one walk from the end that
+    reads every input once): all eight gradients against float64 autograd through the oracle and against the general
+    two-kernel path, with float32 gradients and with dB, dC, dz written in the tensors' own types."""
+    ops = _ops()
+    h, p = hp
+    b = 3
+    inp = make(2 * length + h, b, length, h, p, dtype=dtype, a_vec=True, d_mode=d_mode, z_mode=z_mode, init=init)
+    inp["dt"] = inp["dt"].float()
+    lens = [length, max(length // 3, 0), 0] if ragged else None
+    meta = {"seq_lens": lens} if ragged else None
+    gy = torch.randn(b, length, h, p, generator=torch.Generator().manual_seed(length)).to(dtype)
+    want = _grads_oracle({k: (v.float() if v is not None else None) for k, v in inp.items()}, meta, gy.float())
+    d = {k: dev(v) for k, v in inp.items()}
+    lengths = torch.tensor(lens, dtype=torch.int32).cuda() if ragged else None
+    run = lambda **kw: ops._dscan_backward(dev(gy), d["X"], d["dt"], d["A"], d["B"], d["C"], 64, d["D"], d["z"], lengths,
+                                           d["init"], **kw)
+    one = run()
+    two = run(two_kernels=True)
+    own = run(grads_in_input_dtype=True)
+    names = ["X", "dt", "A", "B", "C", "D", "z", "init"]
+    half = dtype != torch.float32
+    for k, g1, g2, g3 in zip(names, one, two, own):
+        if want[k] is None:
+            assert g1 is None and g3 is None
+            continue
+        w = want[k]
+        scale = float(w.abs().max()) + 1e-6
+        tol = dict(rtol=3e-2, atol=3e-2 * scale) if half else dict(rtol=2e-4, atol=2e-5 * max(scale, 1.0))
+        assert g1.dtype == (dtype if k == "X" else torch.float32) and g1.shape == w.shape, k
+        torch.testing.assert_close(g1.float().cpu().double(), w, msg=lambda m, n=k: f"grad {n} against the oracle: {m}", **tol)
+        # the two paths sum in different orders; both are float32 sums of the same terms
+        torch.testing.assert_close(g1.float(), g2.float(), rtol=1e-2 if half else 1e-4,
+                                   atol=(1e-2 if half else 1e-5) * max(scale, 1.0),
+                                   msg=lambda m, n=k: f"grad {n} against the two-kernel path: {m}")
+        # the same arithmetic compiled a second time (fused differently here and there): one rounding of the type apart
+        ulp = {torch.float32: 2.0 ** -20, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}
+        if k in ("B", "C", "z"):
+            assert g3.dtype == dtype, k
+            torch.testing.assert_close(g3.float(), g1.float(), rtol=ulp[dtype], atol=ulp[dtype] * 1e-2 * max(scale, 1.0),
+                                       msg=lambda m, n=k: f"grad {n} in its own type: {m}")
+        else:
+            assert g3.dtype == g1.dtype, k
+            torch.testing.assert_close(g3.float(), g1.float(), rtol=ulp[dtype] if k == "X" else 1e-5,
+                                       atol=1e-5 * max(scale, 1.0), msg=lambda m, n=k: f"grad {n}: {m}")
+    if ragged:
+        assert float(one[0][2].abs().max()) == 0.0 and float(one[3][1, length // 3:].abs().max()) == 0.0
+    # the forward can leave the table of round states for the backward: the same gradients without the extra sweep
+    y, table = ops._dscan_forward(d["X"], d["dt"], d["A"], d["B"], d["C"], 64, d["D"], d["z"], lengths, d["init"],
+                                  want_round_states=True)
+    assert table is not None and tuple(table.shape) == (b, (length + 63) // 64, h * p)
+    for k, g1, g4 in zip(names, one, run(round_states=table)):
+        if g1 is not None:
+            torch.testing.assert_close(g4, g1, rtol=1e-6, atol=0, msg=lambda m, n=k: f"grad {n} with the forward's table: {m}")
+    # and through autograd, which does exactly that and returns every gradient in its tensor's type
+    auto = _grads_gpu(inp, meta, gy)
+    for k, g3 in zip(names, own):
+        if g3 is None:
+            continue
+        key = "init" if k == "init" else k
+        assert auto[key].dtype == inp[key].dtype and auto[key].shape == inp[key].shape, k
+        torch.testing.assert_close(auto[key].float(), g3.to(inp[key].dtype).float().reshape(inp[key].shape), rtol=1e-6, atol=0,
+                                   msg=lambda m, n=k: f"grad {n} through autograd: {m}")
