@@ -366,6 +366,9 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
     else if (a->x_dtype == SSM_F16) launch_bwd_onepass<f16_t, 2>(p, grads_io, sweep, s);
     else launch_bwd_onepass<float, 1>(p, grads_io, sweep, s);
     SSM_CHECK_LAUNCH("ssm_dscan_bwd");
+    hipLaunchKernelGGL(dscan_bwd_head_sums_kernel, dim3(H), dim3(WAVE), 0, s, p.pA, p.pD, a->dA, a->dD, Bn, H, P);
+    SSM_CHECK_LAUNCH("ssm_dscan_bwd(sums)");
+    return SSM_OK;
   } else {
 #define SSM_DB_LAUNCH(T)                                                                       \
   {                                                                                            \

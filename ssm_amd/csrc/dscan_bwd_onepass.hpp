@@ -371,6 +371,27 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
   }
 }
 
+// dA and dD per head: the workgroups' per-channel sums added over batch rows and the head's channels, one wave
+// per head, in a fixed order.
+__global__ __launch_bounds__(WAVE) void dscan_bwd_head_sums_kernel(const float *pA, const float *pD, float *dA, float *dD,
+                                                                   int batch, int heads, int proj) {
+  const int h = blockIdx.x, lane = lane_id();
+  float sa = 0.0f, sd = 0.0f;
+  for (int b = 0; b < batch; ++b) {
+    for (int pp = lane; pp < proj; pp += WAVE) {
+      const size_t at = ((size_t)b * heads + h) * proj + pp;
+      sa += pA[at];
+      sd += pD[at];
+    }
+  }
+  sa = wave_sum(sa);
+  sd = wave_sum(sd);
+  if (lane == 0) {
+    dA[h] = sa;
+    if (dD) dD[h] = sd;
+  }
+}
+
 template <typename io_t, typename g_t, int VEC, bool HAS_Z>
 static void launch_dbo_lph(const DscanBwdParams &p, int lph, hipStream_t s) {
   const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
