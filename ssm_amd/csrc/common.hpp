@@ -1,6 +1,7 @@
 // Shared device/host helpers for the gfx950 kernels: dtype conversion, vector
 // loads, fp32 transcendental helpers, wave64 DPP scans, error reporting.
 #pragma once
+#include <type_traits>
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -219,6 +220,38 @@ __device__ __forceinline__ float wave_inclusive_sum(float v) {
   v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.0f, v);
   v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.0f, v);
   return v;
+}
+
+// One 32-bit register of elements as loaded (two 16-bit elements, or one float), kept as bits until an element is
+// used: a register per vector whatever the element type, and the float32 values are formed where they are needed
+// instead of being kept.
+template <typename io_t>
+struct Word {
+  unsigned w;
+  __device__ __forceinline__ float elem(int v) const;
+  // zero when the step is past the row's length: every tensor of a dead step reads as zero, which makes the step
+  // the identity that adds nothing and receives nothing
+  __device__ __forceinline__ void mask(bool live) { w = live ? w : 0u; }
+  // opaque to the compiler from here on: values formed from the bits before are not carried across
+  __device__ __forceinline__ void launder() { __asm__ volatile("" : "+v"(w)); }
+  // ... and not before `after` has been computed: keeps the conversions of one step of an unrolled loop from
+  // being moved in front of the steps before it (where they would all be live at once)
+  __device__ __forceinline__ void launder_after(float after) { __asm__ volatile("" : "+v"(w) : "v"(after)); }
+};
+template <> __device__ __forceinline__ float Word<float>::elem(int) const { return __uint_as_float(w); }
+template <> __device__ __forceinline__ float Word<bf16_t>::elem(int v) const {
+  return __uint_as_float(v ? (w & 0xffff0000u) : (w << 16));
+}
+template <> __device__ __forceinline__ float Word<f16_t>::elem(int v) const {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)(v ? (w >> 16) : (w & 0xffffu)));
+}
+
+// A wave-uniform base plus a 32-bit byte offset per lane: the form of address the memory instructions take as
+// it is (a base in scalar registers, an offset in one vector register), with no 64-bit arithmetic per access.
+template <typename T, typename B>
+__device__ __forceinline__ T *at_bytes(B *base, unsigned bytes) {
+  using C = typename std::conditional<std::is_const<B>::value, const char, char>::type;
+  return reinterpret_cast<T *>(reinterpret_cast<C *>(base) + bytes);
 }
 
 __device__ __forceinline__ int wave_id_uniform() {

@@ -144,90 +144,108 @@ __global__ __launch_bounds__(DS_THREADS) void dscan_kernel(const DscanParams p) 
 
 // ---------------------------------------------------------------- one pass
 // The common call (per-token B and C of X's shape and type, per-head A and D, gate of X's shape or none) with
-// every input read once.  A workgroup of eight waves owns 64 * VEC neighbouring channels of one batch row (a
+// every input read once.  A workgroup of 16 waves owns 64 * VEC neighbouring channels of one batch row (a
 // lane VEC of them, so that a wave's access is 128 * VEC bytes of 16-bit elements) and walks time in rounds of
-// 64 steps, wave w taking steps 8w..8w+7 of the round: it folds its steps from zero into (decay product, state),
-// the eight folds meet in LDS (one barrier per round, two buffers), every wave chains them from the state carried
-// into the round -- which gives it the state entering its own steps and, in the same sweep, the state carried
-// into the next round -- and replays its steps from the values it still holds in registers.  The reads of the
-// next round are requested before the arithmetic of this one.  All workgroups are resident at once and the call
-// is bound by memory, so it does not matter that they are fewer than the CUs can hold.
+// 128 steps, wave w taking steps 8w..8w+7 of the round: it folds its steps from zero into (decay product, state),
+// the 16 folds meet in LDS (one barrier per round, two buffers), wave w chains the folds of the waves before it
+// from the state entering the round -- which gives it the state entering its own steps -- and replays its steps
+// from the values it still holds in registers.  The last wave's chain ends at the round's right edge: it leaves
+// the state there in LDS for everyone's next round.  The reads of the next round are requested before the
+// arithmetic of this one.  A workgroup fills a CU's registers (one per CU), so the call is as fast as one
+// workgroup's instruction stream: addresses are a uniform base plus a 32-bit offset per lane, steps past a row's
+// length are masked only in the rounds that contain any, and two sets of registers take turns without copies.
 constexpr int DO_WAVES = 16, DO_SEG = 8, DO_ROUND = DO_WAVES * DO_SEG;
 
 template <typename io_t, int VEC>
 struct DoRegs {
   float dt[DO_SEG];
-  Pack<io_t, VEC> x[DO_SEG], bq[DO_SEG], cq[DO_SEG], zq[DO_SEG];
+  Word<io_t> x[DO_SEG], bq[DO_SEG], cq[DO_SEG], zq[DO_SEG];
 };
 
 template <typename io_t, int VEC, bool HAS_Z>
 __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const DscanParams p) {
+  static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
   __shared__ float4 segs[2][DO_WAVES][WAVE];
+  __shared__ float2 right[2][WAVE];
   const int wave = wave_id_uniform(), lane = lane_id();
   const int HP = p.heads * p.proj;
-  const int ch = ((int)blockIdx.x * WAVE + lane) * VEC;
+  const unsigned ch = ((unsigned)blockIdx.x * WAVE + lane) * VEC;
   const int b = blockIdx.y;
-  const int h = ch / p.proj;
+  const int h = (int)ch / p.proj;
   const int L = p.len;
   const int valid = p.lengths ? min(max(p.lengths[b], 0), L) : L;
   const float A2 = p.A[h] * LOG2E;
   const float Dk = p.Dk ? p.Dk[h] : 0.0f;
-  const io_t *X = reinterpret_cast<const io_t *>(p.X), *Bp = reinterpret_cast<const io_t *>(p.Bp);
-  const io_t *Cp = reinterpret_cast<const io_t *>(p.Cp), *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.X);
-  const float *DT = reinterpret_cast<const float *>(p.dt);
-  io_t *Y = reinterpret_cast<io_t *>(p.Y);
+  // the batch row's part of every tensor: offsets inside it fit 32 bits (checked by the host)
   const size_t row0 = (size_t)b * L;
-  float carry[VEC];
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) carry[v] = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + ch + v) : 0.0f;
+  const io_t *X = reinterpret_cast<const io_t *>(p.X) + row0 * HP, *Bp = reinterpret_cast<const io_t *>(p.Bp) + row0 * HP;
+  const io_t *Cp = reinterpret_cast<const io_t *>(p.Cp) + row0 * HP, *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.X) + row0 * HP;
+  const float *DT = reinterpret_cast<const float *>(p.dt) + row0 * p.heads;
+  io_t *Y = reinterpret_cast<io_t *>(p.Y) + row0 * HP;
 
   auto request = [&](DoRegs<io_t, VEC> &r, int round) {
     const int t0 = round * DO_ROUND + wave * DO_SEG;
 #pragma unroll
     for (int j = 0; j < DO_SEG; ++j) {
-      const size_t row = row0 + min(t0 + j, L - 1);            // steps past the end read the last row, unused
-      const size_t at = row * HP + ch;
-      r.dt[j] = DT[row * p.heads + h];
-      r.x[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(X + at);
-      r.bq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Bp + at);
-      r.cq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Cp + at);
-      if (HAS_Z) r.zq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Z + at);
+      const unsigned row = (unsigned)min(t0 + j, L - 1);       // steps past the end read the last row, unused
+      const unsigned at = (row * (unsigned)HP + ch) * (unsigned)sizeof(io_t);
+      r.dt[j] = *at_bytes<const float>(DT, (row * (unsigned)p.heads + (unsigned)h) * 4u);
+      r.x[j] = Word<io_t>{*at_bytes<const unsigned>(X, at)};
+      r.bq[j] = Word<io_t>{*at_bytes<const unsigned>(Bp, at)};
+      r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
+      if (HAS_Z) r.zq[j] = Word<io_t>{*at_bytes<const unsigned>(Z, at)};
     }
   };
 
   const int rounds = (L + DO_ROUND - 1) / DO_ROUND;
-  DoRegs<io_t, VEC> cur, nxt;
-  request(cur, 0);
-  for (int r = 0; r < rounds; ++r) {
-    if (r + 1 < rounds) request(nxt, r + 1);
+  auto round_of = [&](DoRegs<io_t, VEC> &cur, int r) {
+    const int q = r & 1;
     const int t0 = r * DO_ROUND + wave * DO_SEG;
-    float a[DO_SEG], inc[VEC][DO_SEG], s[VEC], prod = 1.0f;
+    if (t0 + DO_SEG > valid) {
+      // the row ends inside these steps (uniform, rare): a dead step reads as zero everywhere -- the identity,
+      // nothing added, a zero output
+#pragma unroll
+      for (int j = 0; j < DO_SEG; ++j) {
+        const bool live = t0 + j < valid;
+        cur.dt[j] = live ? cur.dt[j] : 0.0f;
+        cur.x[j].mask(live);
+        cur.bq[j].mask(live);
+        cur.cq[j].mask(live);
+      }
+    }
+    float a[DO_SEG], s[VEC], prod = 1.0f;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) s[v] = 0.0f;
 #pragma unroll
     for (int j = 0; j < DO_SEG; ++j) {
-      const bool live = t0 + j < valid;                        // past the row's length: the identity, nothing added
-      a[j] = live ? exp2_hw(cur.dt[j] * A2) : 1.0f;
+      a[j] = exp2_hw(cur.dt[j] * A2);
       prod *= a[j];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        inc[v][j] = live ? cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]) : 0.0f;
-        s[v] = __builtin_fmaf(a[j], s[v], inc[v][j]);
-      }
+      for (int v = 0; v < VEC; ++v)
+        s[v] = __builtin_fmaf(a[j], s[v], cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v));
     }
-    segs[r & 1][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
+    segs[q][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
     __syncthreads();
-    float e[VEC], enter[VEC];
+    // the state entering this wave's steps: the folds of the waves before it, from the state entering the round
+    float enter[VEC];
+    if (r == 0) {
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) e[v] = enter[v] = carry[v];
+      for (int v = 0; v < VEC; ++v) enter[v] = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + ch + v) : 0.0f;
+    } else {
+      const float2 c = right[q ^ 1][lane];
+      enter[0] = c.x;
+      enter[VEC - 1] = c.y;
+    }
+    for (int w = 0; w < wave; ++w) {
+      const float4 f = segs[q][w][lane];
 #pragma unroll
-    for (int w = 0; w < DO_WAVES; ++w) {
-      const float4 f = segs[r & 1][w][lane];
+      for (int v = 0; v < VEC; ++v) enter[v] = __builtin_fmaf(f.x, enter[v], v == 0 ? f.y : f.z);
+    }
+    if (wave == DO_WAVES - 1) {
+      float leave[VEC];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        enter[v] = w == wave ? e[v] : enter[v];
-        e[v] = __builtin_fmaf(f.x, e[v], v == 0 ? f.y : f.z);
-      }
+      for (int v = 0; v < VEC; ++v) leave[v] = __builtin_fmaf(prod, enter[v], s[v]);
+      right[q][lane] = make_float2(leave[0], leave[VEC - 1]);
     }
     if (p.round_states && (wave & (DO_WAVES / 2 - 1)) == 0) {
       // what the backward starts its rounds of 64 steps from: the states entering wave 0's and wave 8's steps
@@ -240,24 +258,37 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
       }
     }
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      carry[v] = e[v];
-      s[v] = enter[v];
-    }
-#pragma unroll
     for (int j = 0; j < DO_SEG; ++j) {
       const int t = t0 + j;
+      // the float32 values of a step's elements are formed here, step by step, not kept from the fold above
+      // and not all in front of the first step
+      cur.x[j].launder_after(enter[0]);
+      cur.bq[j].launder_after(enter[0]);
+      cur.cq[j].launder_after(enter[0]);
+      if (HAS_Z) cur.zq[j].launder_after(enter[0]);
       Pack<io_t, VEC> o;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        s[v] = __builtin_fmaf(a[j], s[v], inc[v][j]);
-        float y = __builtin_fmaf(s[v], to_f32(cur.cq[j].v[v]), Dk * to_f32(cur.x[j].v[v]));
-        if (HAS_Z) y *= silu_f32(to_f32(cur.zq[j].v[v]));
-        o.v[v] = from_f32<io_t>(t < valid ? y : 0.0f);
+        const float xv = cur.x[j].elem(v);
+        enter[v] = __builtin_fmaf(a[j], enter[v], cur.dt[j] * cur.bq[j].elem(v) * xv);
+        float y = __builtin_fmaf(enter[v], cur.cq[j].elem(v), Dk * xv);
+        if (HAS_Z) y *= silu_f32(cur.zq[j].elem(v));
+        o.v[v] = from_f32<io_t>(y);
       }
-      if (t < L) *reinterpret_cast<Pack<io_t, VEC> *>(Y + (row0 + t) * HP + ch) = o;
+      if (t < L) *at_bytes<Pack<io_t, VEC>>(Y, ((unsigned)t * (unsigned)HP + ch) * (unsigned)sizeof(io_t)) = o;
     }
-    cur = nxt;
+  };
+
+  // two sets of registers take turns: one is worked on while the other's reads are in flight
+  DoRegs<io_t, VEC> ra, rb;
+  request(ra, 0);
+  for (int r = 0; r < rounds; r += 2) {
+    if (r + 1 < rounds) request(rb, r + 1);
+    round_of(ra, r);
+    if (r + 1 < rounds) {
+      if (r + 2 < rounds) request(ra, r + 2);
+      round_of(rb, r + 1);
+    }
   }
 }
 
@@ -296,7 +327,8 @@ static bool dscan_fwd_takes_one_pass(const ssm_dscan_fwd_args *a) {
   const int vec = a->x_dtype == SSM_F32 ? 1 : 2;
   const size_t bytes = (size_t)vec * dtype_size(a->x_dtype);
   return typed && a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP && !a->a_per_p && !a->d_per_p &&
-         (!a->z || a->z_per_p) && HP % (WAVE * vec) == 0 && a->proj % vec == 0 && aligned_to(a->X, bytes) &&
+         (!a->z || a->z_per_p) && HP % (WAVE * vec) == 0 && a->proj % vec == 0 &&
+         (long long)a->seqlen * HP < (1ll << 30) && aligned_to(a->X, bytes) &&
          aligned_to(a->Bproj, bytes) && aligned_to(a->Cproj, bytes) && aligned_to(a->Y, bytes) &&
          (!a->z || aligned_to(a->z, bytes)) && a->batch < 65536;
 }

@@ -40,7 +40,7 @@ static_assert(DRS_ROUND == 2 * DBO_ROUND, "two rounds of the backward per round 
 template <typename io_t, int VEC>
 struct DrsRegs {
   float dt[DRS_SEG];
-  Pack<io_t, VEC> x[DRS_SEG], bq[DRS_SEG];
+  Word<io_t> x[DRS_SEG], bq[DRS_SEG];
 };
 
 template <typename io_t, int VEC>
@@ -70,8 +70,8 @@ __global__ __launch_bounds__(WAVE *DRS_WAVES) void dscan_round_states_kernel(con
       const size_t row = row0 + min(t0 + j, L - 1);            // steps past the end read the last row, unused
       const size_t at = row * HP + ch;
       r.dt[j] = DT[row * p.heads + h];
-      r.x[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(X + at);
-      r.bq[j] = *reinterpret_cast<const Pack<io_t, VEC> *>(Bp + at);
+      r.x[j] = Word<io_t>{*reinterpret_cast<const unsigned *>(X + at)};
+      r.bq[j] = Word<io_t>{*reinterpret_cast<const unsigned *>(Bp + at)};
     }
   };
 
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(WAVE *DRS_WAVES) void dscan_round_states_kernel(con
       prod *= a;
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
-        s[v] = __builtin_fmaf(a, s[v], live ? cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]) : 0.0f);
+        s[v] = __builtin_fmaf(a, s[v], live ? cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v) : 0.0f);
     }
     segs[r & 1][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
     __syncthreads();
@@ -124,47 +124,14 @@ __global__ __launch_bounds__(WAVE *DRS_WAVES) void dscan_round_states_kernel(con
 template <typename io_t, int VEC, bool HAS_Z>
 struct DboRegs {
   float dt[DBO_SEG];
-  Pack<io_t, VEC> x[DBO_SEG], bq[DBO_SEG], cq[DBO_SEG], gq[DBO_SEG], zq[DBO_SEG];
+  Word<io_t> x[DBO_SEG], bq[DBO_SEG], cq[DBO_SEG], gq[DBO_SEG], zq[DBO_SEG];
   float enter[VEC];                 // the state entering the round
 };
-
-// The bits of a vector of elements as they sit in registers, and back.
-template <typename io_t, int VEC>
-struct DboBits {
-  using type = typename std::conditional<sizeof(Pack<io_t, VEC>) == 4, unsigned, unsigned long long>::type;
-};
-
-// Zero when the step is past the row's length (every tensor of a dead step reads as zero: the step is the
-// identity, adds nothing and receives nothing), and opaque to the compiler: the float32 values of a vector are
-// formed again where they are used instead of being kept from one phase of a round to the next.
-template <typename io_t, int VEC>
-__device__ __forceinline__ void dbo_mask(Pack<io_t, VEC> &v, bool live) {
-  using bits_t = typename DboBits<io_t, VEC>::type;
-  static_assert(sizeof(bits_t) == sizeof(Pack<io_t, VEC>), "one or two registers");
-  bits_t raw = __builtin_bit_cast(bits_t, v);
-  raw = live ? raw : bits_t(0);
-  v = __builtin_bit_cast(Pack<io_t, VEC>, raw);
-}
-template <typename io_t, int VEC>
-__device__ __forceinline__ void dbo_launder(Pack<io_t, VEC> &v) {
-  using bits_t = typename DboBits<io_t, VEC>::type;
-  bits_t raw = __builtin_bit_cast(bits_t, v);
-  __asm__ volatile("" : "+v"(raw));
-  v = __builtin_bit_cast(Pack<io_t, VEC>, raw);
-}
-
-// A wave-uniform base plus a 32-bit byte offset per lane: the form of address the memory instructions take as
-// it is (a base in scalar registers, an offset in one vector register), with no 64-bit arithmetic per access.
-template <typename T, typename B>
-__device__ __forceinline__ T *at_bytes(B *base, unsigned bytes) {
-  using C = typename std::conditional<std::is_const<B>::value, const char, char>::type;
-  return reinterpret_cast<T *>(reinterpret_cast<C *>(base) + bytes);
-}
 
 // g_t: element type of dB, dC and dz (io_t, or float).  LPH: lanes that hold one head's channels.
 template <typename io_t, typename g_t, int VEC, bool HAS_Z, int LPH>
 __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
-  static_assert(sizeof(Pack<io_t, VEC>) == 4 || sizeof(Pack<io_t, VEC>) == 8, "a lane's vector is one or two registers");
+  static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
   __shared__ float4 fwd[2][DBO_WAVES][WAVE];     // a wave's four steps per lane: decay product, state from zero (per channel)
   __shared__ float2 rev[2][DBO_WAVES][WAVE];     // ... and the adjoint (times its decay) from zero
   __shared__ float2 left[2][WAVE];               // the adjoint leaving the round, from wave 0 to everyone's next round
@@ -197,11 +164,11 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
       const unsigned row = (unsigned)min(t0 + j, L - 1);       // steps past the end read the last row, unused
       const unsigned at = (row * (unsigned)HP + ch) * (unsigned)sizeof(io_t);
       r.dt[j] = *at_bytes<const float>(DT, (row * (unsigned)p.heads + (unsigned)h) * 4u);
-      r.x[j] = *at_bytes<const Pack<io_t, VEC>>(X, at);
-      r.bq[j] = *at_bytes<const Pack<io_t, VEC>>(Bp, at);
-      r.cq[j] = *at_bytes<const Pack<io_t, VEC>>(Cp, at);
-      r.gq[j] = *at_bytes<const Pack<io_t, VEC>>(G, at);
-      if (HAS_Z) r.zq[j] = *at_bytes<const Pack<io_t, VEC>>(Z, at);
+      r.x[j] = Word<io_t>{*at_bytes<const unsigned>(X, at)};
+      r.bq[j] = Word<io_t>{*at_bytes<const unsigned>(Bp, at)};
+      r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
+      r.gq[j] = Word<io_t>{*at_bytes<const unsigned>(G, at)};
+      if (HAS_Z) r.zq[j] = Word<io_t>{*at_bytes<const unsigned>(Z, at)};
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) r.enter[v] = *at_bytes<const float>(table, ((unsigned)round * (unsigned)HP + ch + v) * 4u);
@@ -222,28 +189,28 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
     for (int j = 0; j < DBO_SEG; ++j) {
       const bool live = t0 + j < valid;
       cur.dt[j] = live ? cur.dt[j] : 0.0f;
-      dbo_mask<io_t, VEC>(cur.x[j], live);
-      dbo_mask<io_t, VEC>(cur.bq[j], live);
-      dbo_mask<io_t, VEC>(cur.cq[j], live);
-      dbo_mask<io_t, VEC>(cur.gq[j], live);
-      if (HAS_Z) dbo_mask<io_t, VEC>(cur.zq[j], live);
+      cur.x[j].mask(live);
+      cur.bq[j].mask(live);
+      cur.cq[j].mask(live);
+      cur.gq[j].mask(live);
+      if (HAS_Z) cur.zq[j].mask(live);
       a[j] = exp2_hw(cur.dt[j] * A2);
       prod *= a[j];
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
-        s[v] = __builtin_fmaf(a[j], s[v], cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]));
+        s[v] = __builtin_fmaf(a[j], s[v], cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v));
     }
 #pragma unroll
     for (int j = DBO_SEG - 1; j >= 0; --j) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        float g0 = to_f32(cur.gq[j].v[v]);
+        float g0 = cur.gq[j].elem(v);
         if (HAS_Z) {
-          const float zz = to_f32(cur.zq[j].v[v]);
+          const float zz = cur.zq[j].elem(v);
           sg[v][j] = sigmoid_f32(zz);
           g0 *= zz * sg[v][j];
         }
-        M[v] = a[j] * __builtin_fmaf(g0, to_f32(cur.cq[j].v[v]), M[v]);
+        M[v] = a[j] * __builtin_fmaf(g0, cur.cq[j].elem(v), M[v]);
       }
     }
     fwd[q][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
@@ -251,11 +218,11 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < DBO_SEG; ++j) {
-      dbo_launder<io_t, VEC>(cur.x[j]);
-      dbo_launder<io_t, VEC>(cur.bq[j]);
-      dbo_launder<io_t, VEC>(cur.cq[j]);
-      dbo_launder<io_t, VEC>(cur.gq[j]);
-      if (HAS_Z) dbo_launder<io_t, VEC>(cur.zq[j]);
+      cur.x[j].launder();
+      cur.bq[j].launder();
+      cur.cq[j].launder();
+      cur.gq[j].launder();
+      if (HAS_Z) cur.zq[j].launder();
     }
     // the state entering this wave's steps: the folds of the waves before it, from the state entering the round
     float st[VEC][DBO_SEG + 1];
@@ -291,21 +258,27 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
     for (int j = 0; j < DBO_SEG; ++j) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
-        st[v][j + 1] = __builtin_fmaf(a[j], st[v][j], cur.dt[j] * to_f32(cur.bq[j].v[v]) * to_f32(cur.x[j].v[v]));
+        st[v][j + 1] = __builtin_fmaf(a[j], st[v][j], cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v));
     }
     // backward replay; mu[v] is lambda_{t+1} a_{t+1}
 #pragma unroll
     for (int j = DBO_SEG - 1; j >= 0; --j) {
       const int t = t0 + j;
+      // a step's float32 values are formed at the step, not all in front of the loop
+      cur.x[j].launder_after(mu[0]);
+      cur.bq[j].launder_after(mu[0]);
+      cur.cq[j].launder_after(mu[0]);
+      cur.gq[j].launder_after(mu[0]);
+      if (HAS_Z) cur.zq[j].launder_after(mu[0]);
       Pack<io_t, VEC> ox;
       Pack<g_t, VEC> ob, oc, oz;
       float ddt = 0.0f;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        const float xv = to_f32(cur.x[j].v[v]), bv = to_f32(cur.bq[j].v[v]), cv = to_f32(cur.cq[j].v[v]);
-        float g0 = to_f32(cur.gq[j].v[v]);
+        const float xv = cur.x[j].elem(v), bv = cur.bq[j].elem(v), cv = cur.cq[j].elem(v);
+        float g0 = cur.gq[j].elem(v);
         if (HAS_Z) {
-          const float zz = to_f32(cur.zq[j].v[v]);
+          const float zz = cur.zq[j].elem(v);
           const float y0 = __builtin_fmaf(st[v][j + 1], cv, Dk * xv);
           oz.v[v] = from_f32<g_t>(g0 * y0 * sg[v][j] * __builtin_fmaf(zz, 1.0f - sg[v][j], 1.0f));
           g0 *= zz * sg[v][j];
