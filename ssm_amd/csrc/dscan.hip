@@ -162,7 +162,9 @@ struct DoRegs {
   Word<io_t> x[DO_SEG], bq[DO_SEG], cq[DO_SEG], zq[DO_SEG];
 };
 
-template <typename io_t, int VEC, bool HAS_Z>
+// STATES_ONLY: the walk without C, the gate and the output -- only the table of round states is written (the
+// backward's own forward sweep when it is called without one).
+template <typename io_t, int VEC, bool HAS_Z, bool STATES_ONLY>
 __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const DscanParams p) {
   static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
   __shared__ float4 segs[2][DO_WAVES][WAVE];
@@ -192,8 +194,8 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
       r.dt[j] = *at_bytes<const float>(DT, (row * (unsigned)p.heads + (unsigned)h) * 4u);
       r.x[j] = Word<io_t>{*at_bytes<const unsigned>(X, at)};
       r.bq[j] = Word<io_t>{*at_bytes<const unsigned>(Bp, at)};
-      r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
-      if (HAS_Z) r.zq[j] = Word<io_t>{*at_bytes<const unsigned>(Z, at)};
+      if (!STATES_ONLY) r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
+      if (HAS_Z && !STATES_ONLY) r.zq[j] = Word<io_t>{*at_bytes<const unsigned>(Z, at)};
     }
   };
 
@@ -210,7 +212,7 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
         cur.dt[j] = live ? cur.dt[j] : 0.0f;
         cur.x[j].mask(live);
         cur.bq[j].mask(live);
-        cur.cq[j].mask(live);
+        if (!STATES_ONLY) cur.cq[j].mask(live);
       }
     }
     float a[DO_SEG], s[VEC], prod = 1.0f;
@@ -257,6 +259,7 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
         for (int v = 0; v < VEC; ++v) table[v] = enter[v];
       }
     }
+    if (STATES_ONLY) return;
 #pragma unroll
     for (int j = 0; j < DO_SEG; ++j) {
       const int t = t0 + j;
@@ -295,8 +298,23 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
 template <typename io_t, int VEC>
 static void launch_onepass(const DscanParams &p, hipStream_t s) {
   const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
-  if (p.z) hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, true>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
-  else hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, false>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
+  if (p.z) hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, true, false>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
+  else hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, false, false>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
+}
+
+// The table of round states alone, for a call shape the one-pass kernels cover (the caller has checked).
+void launch_dscan_round_states(const void *X, const void *dt, const void *Bproj, const float *A, const void *init,
+                               int init_dtype, const int *lengths, float *round_states, int batch, int len, int heads,
+                               int proj, int x_dtype, hipStream_t s) {
+  DscanParams p{};
+  p.X = X; p.dt = dt; p.Bp = Bproj; p.Cp = Bproj; p.A = A; p.init = init; p.init_dtype = init_dtype;
+  p.lengths = lengths; p.round_states = round_states;
+  p.batch = batch; p.len = len; p.heads = heads; p.proj = proj;
+  const int vec = x_dtype == SSM_F32 ? 1 : 2;
+  const dim3 grid((unsigned)((size_t)heads * proj / (WAVE * vec)), (unsigned)batch), block(WAVE * DO_WAVES);
+  if (x_dtype == SSM_BF16) hipLaunchKernelGGL((dscan_onepass_kernel<bf16_t, 2, false, true>), grid, block, 0, s, p);
+  else if (x_dtype == SSM_F16) hipLaunchKernelGGL((dscan_onepass_kernel<f16_t, 2, false, true>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((dscan_onepass_kernel<float, 1, false, true>), grid, block, 0, s, p);
 }
 
 int dscan_segments(int batch, int len, int hp) {

@@ -25,6 +25,10 @@ constexpr int DB_THREADS = 256;
 constexpr int DB_UNROLL = 8;          // time steps whose reads are in flight together
 
 int dscan_segments(int batch, int len, int hp);   // dscan.hip: the forward's choice, reused here
+// dscan.hip: the forward's one-pass walk reduced to the table of the states entering every 64 steps
+void launch_dscan_round_states(const void *X, const void *dt, const void *Bproj, const float *A, const void *init,
+                               int init_dtype, const int *lengths, float *round_states, int batch, int len, int heads,
+                               int proj, int x_dtype, hipStream_t s);
 
 struct DscanBwdParams {
   const void *gy, *X, *dt, *Bp, *Cp, *z, *init;
@@ -361,10 +365,12 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
     p.pD = p.pA + bhp;
     p.ddt_direct = a->ddt;
     nseg = 1;
-    const bool sweep = a->round_states == nullptr;      // no table from the forward: make it
-    if (a->x_dtype == SSM_BF16) launch_bwd_onepass<bf16_t, 2>(p, grads_io, sweep, s);
-    else if (a->x_dtype == SSM_F16) launch_bwd_onepass<f16_t, 2>(p, grads_io, sweep, s);
-    else launch_bwd_onepass<float, 1>(p, grads_io, sweep, s);
+    if (a->round_states == nullptr)                      // no table from the forward: make it
+      launch_dscan_round_states(a->X, a->dt, a->Bproj, a->A, a->initial_states, a->init_dtype, a->seq_lens, ws, Bn, L, H,
+                                P, a->x_dtype, s);
+    if (a->x_dtype == SSM_BF16) launch_bwd_onepass<bf16_t, 2>(p, grads_io, s);
+    else if (a->x_dtype == SSM_F16) launch_bwd_onepass<f16_t, 2>(p, grads_io, s);
+    else launch_bwd_onepass<float, 1>(p, grads_io, s);
     SSM_CHECK_LAUNCH("ssm_dscan_bwd");
     hipLaunchKernelGGL(dscan_bwd_head_sums_kernel, dim3(H), dim3(WAVE), 0, s, p.pA, p.pD, a->dA, a->dD, Bn, H, P);
     SSM_CHECK_LAUNCH("ssm_dscan_bwd(sums)");

@@ -11,8 +11,8 @@
 // on the right (15 links in all, whatever w), which gives it what enters its own steps from both sides, then
 // replays its steps forwards (states, kept in registers) and backwards (gradients).  Wave 0's chain ends at the
 // round's left edge: it leaves the adjoint there in LDS for everyone's next round.  The state entering a round
-// comes from a table written beforehand by dscan_round_states_kernel, a forward sweep of the same shape that
-// reads only X, B and dt.  The reads of the next round are requested before the arithmetic of this one.
+// comes from a table written beforehand: by the forward's one-pass kernel, or by that kernel's walk reduced to
+// X, B and dt (launch_dscan_round_states).  The reads of the next round are requested before the arithmetic of this one.
 #pragma once
 
 namespace ssm {
@@ -29,95 +29,6 @@ __device__ __forceinline__ float lane_group_sum_last(float v) {
   if (LPH >= 32) v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.0f, v);
   if (LPH >= 64) v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.0f, v);
   return v;
-}
-
-// ---- the state entering every round of 64 steps: (B, rounds, HP) float32
-// Same walk as the forward's one-pass kernel (16 waves, 8 steps each, rounds of 128 steps) without C, the gate
-// and the output; the state in the middle of a round is the chain's value in front of wave 8.
-constexpr int DRS_WAVES = 16, DRS_SEG = 8, DRS_ROUND = DRS_WAVES * DRS_SEG;
-static_assert(DRS_ROUND == 2 * DBO_ROUND, "two rounds of the backward per round of the table's sweep");
-
-template <typename io_t, int VEC>
-struct DrsRegs {
-  float dt[DRS_SEG];
-  Word<io_t> x[DRS_SEG], bq[DRS_SEG];
-};
-
-template <typename io_t, int VEC>
-__global__ __launch_bounds__(WAVE *DRS_WAVES) void dscan_round_states_kernel(const DscanBwdParams p) {
-  __shared__ float4 segs[2][DRS_WAVES][WAVE];
-  const int wave = wave_id_uniform(), lane = lane_id();
-  const int HP = p.heads * p.proj;
-  const int ch = ((int)blockIdx.x * WAVE + lane) * VEC;
-  const int b = blockIdx.y;
-  const int h = ch / p.proj;
-  const int L = p.len;
-  const int valid = p.lengths ? min(max(p.lengths[b], 0), L) : L;
-  const float A2 = p.A[h] * LOG2E;
-  const io_t *X = reinterpret_cast<const io_t *>(p.X), *Bp = reinterpret_cast<const io_t *>(p.Bp);
-  const float *DT = reinterpret_cast<const float *>(p.dt);
-  const size_t row0 = (size_t)b * L;
-  const int rounds64 = (L + DBO_ROUND - 1) / DBO_ROUND;
-  float *table = p.round_states + (size_t)b * rounds64 * HP + ch;
-  float carry[VEC];
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) carry[v] = p.init ? load_as_f32(p.init, p.init_dtype, (size_t)b * HP + ch + v) : 0.0f;
-
-  auto request = [&](DrsRegs<io_t, VEC> &r, int round) {
-    const int t0 = round * DRS_ROUND + wave * DRS_SEG;
-#pragma unroll
-    for (int j = 0; j < DRS_SEG; ++j) {
-      const size_t row = row0 + min(t0 + j, L - 1);            // steps past the end read the last row, unused
-      const size_t at = row * HP + ch;
-      r.dt[j] = DT[row * p.heads + h];
-      r.x[j] = Word<io_t>{*reinterpret_cast<const unsigned *>(X + at)};
-      r.bq[j] = Word<io_t>{*reinterpret_cast<const unsigned *>(Bp + at)};
-    }
-  };
-
-  const int rounds = (L + DRS_ROUND - 1) / DRS_ROUND;
-  DrsRegs<io_t, VEC> cur, nxt;
-  request(cur, 0);
-  for (int r = 0; r < rounds; ++r) {
-    if (r + 1 < rounds) request(nxt, r + 1);
-    const int t0 = r * DRS_ROUND + wave * DRS_SEG;
-    float s[VEC], prod = 1.0f;
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) s[v] = 0.0f;
-#pragma unroll
-    for (int j = 0; j < DRS_SEG; ++j) {
-      const bool live = t0 + j < valid;
-      const float a = live ? exp2_hw(cur.dt[j] * A2) : 1.0f;
-      prod *= a;
-#pragma unroll
-      for (int v = 0; v < VEC; ++v)
-        s[v] = __builtin_fmaf(a, s[v], live ? cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v) : 0.0f);
-    }
-    segs[r & 1][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
-    __syncthreads();
-    float e[VEC], mid[VEC];
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) e[v] = mid[v] = carry[v];
-#pragma unroll
-    for (int w = 0; w < DRS_WAVES; ++w) {
-      const float4 f = segs[r & 1][w][lane];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        mid[v] = w == DRS_WAVES / 2 ? e[v] : mid[v];
-        e[v] = __builtin_fmaf(f.x, e[v], v == 0 ? f.y : f.z);
-      }
-    }
-    if (wave == 0) {
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        table[(size_t)(2 * r) * HP + v] = carry[v];
-        if (2 * r + 1 < rounds64) table[(size_t)(2 * r + 1) * HP + v] = mid[v];
-      }
-    }
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) carry[v] = e[v];
-    cur = nxt;
-  }
 }
 
 // ---- the gradients
@@ -374,11 +285,9 @@ static void launch_dbo_lph(const DscanBwdParams &p, int lph, hipStream_t s) {
   else hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 64>), grid, block, 0, s, p);
 }
 
-// The kernels of the one-pass backward for one element type (`sweep`: the table of round states is made here).
+// The one-pass backward for one element type.
 template <typename io_t, int VEC>
-static void launch_bwd_onepass(const DscanBwdParams &p, bool grads_io, bool sweep, hipStream_t s) {
-  const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
-  if (sweep) hipLaunchKernelGGL((dscan_round_states_kernel<io_t, VEC>), grid, dim3(WAVE * DRS_WAVES), 0, s, p);
+static void launch_bwd_onepass(const DscanBwdParams &p, bool grads_io, hipStream_t s) {
   const int lph = p.proj / VEC;
   if (grads_io) {
     if (p.z) launch_dbo_lph<io_t, io_t, VEC, true>(p, lph, s);
