@@ -8,8 +8,8 @@ benchmark configuration describes (``d_state = 128``, one B/C group, gated
 RMSNorm before the output projection), as published with Mamba-2:
 
     residual, h = add + RMSNorm                        fused_layer_norm_with_residual
-    z | xBC | dt = in_proj(h)                          GEMM (torch)
-    xBC = silu(conv1d(xBC))                            dw_causal_conv (channels last)
+    z | xBC | dt = in_proj(h)                          GEMMs (torch), one per part of the row
+    xBC = silu(conv1d(xBC))                            dw_causal_conv_channels_last, x and B|C apart
     y = SSD(x, dt, A, B, C, D, gate z)                 ssm_amd.ops.ssd.ssd_combined
     out = out_proj(RMSNorm(y))                         fused_layer_norm, GEMM (torch)
 
@@ -99,6 +99,14 @@ class _Layer:
         # float32 copies of the convolution parameters for the single-token step
         self.conv_w_f32 = self.conv_w.float().contiguous()
         self.conv_b_f32 = self.conv_b.float().contiguous()
+        # The rows of the input projection by what they produce (views, no copies): over a whole sequence each
+        # part is projected on its own, so that z, the conv inputs and dt come out as dense tensors the kernels
+        # take as they are -- slicing one projected row of 2 d_inner + 2 G N + H columns would cost a strided
+        # copy of z, x|B|C and x again per layer (0.67 GB at 16 x 2048 tokens).
+        gn2 = cfg.conv_dim - di
+        self.in_proj_z, self.in_proj_x, self.in_proj_bc, self.in_proj_dt = torch.split(self.in_proj, [di, di, gn2, H], dim=0)
+        self.conv_w_x, self.conv_w_bc = torch.split(self.conv_w, [di, gn2], dim=0)
+        self.conv_b_x, self.conv_b_bc = torch.split(self.conv_b, [di, gn2], dim=0)
 
 
 @dataclass
@@ -165,12 +173,15 @@ class Mamba2LM(_GreedyDecoding):
         cfg = self.cfg
         Bsz, L, _ = h.shape
         di, H, P, G, N = cfg.d_inner, cfg.nheads, cfg.headdim, cfg.ngroups, cfg.d_state
-        zxbcdt = h @ layer.in_proj.t()
-        z, xBC, dt = torch.split(zxbcdt, [di, cfg.conv_dim, H], dim=-1)
-        xBC_in = xBC.contiguous()
-        xBC = ops.dw_causal_conv(xBC_in, layer.conv_w, layer.conv_b, activation="silu")      # (B, L, C) channels last
-        x, Bm, Cm = torch.split(xBC, [di, G * N, G * N], dim=-1)
-        out = ssd_ops.ssd_combined(x.reshape(Bsz, L, H, P), dt.contiguous(), layer.A, Bm.reshape(Bsz, L, G, N),
+        z = h @ layer.in_proj_z.t()
+        x_in = h @ layer.in_proj_x.t()
+        bc_in = h @ layer.in_proj_bc.t()
+        dt = h @ layer.in_proj_dt.t()
+        # (B, L, C) channels last; the taps are per channel, so x and B|C convolve separately
+        x = ops.dw_causal_conv_channels_last(x_in, layer.conv_w_x, layer.conv_b_x, activation="silu")
+        bc = ops.dw_causal_conv_channels_last(bc_in, layer.conv_w_bc, layer.conv_b_bc, activation="silu")
+        Bm, Cm = torch.split(bc, [G * N, G * N], dim=-1)
+        out = ssd_ops.ssd_combined(x.reshape(Bsz, L, H, P), dt, layer.A, Bm.reshape(Bsz, L, G, N),
                                    Cm.reshape(Bsz, L, G, N), cfg.chunk_size, D=layer.D,
                                    z=z.reshape(Bsz, L, H, P), dt_bias=layer.dt_bias, dt_softplus=True,
                                    return_final_states=want_state)
@@ -180,8 +191,9 @@ class Mamba2LM(_GreedyDecoding):
         if not want_state:
             return res, None, None
         K = cfg.d_conv
-        window = xBC_in[:, -K:] if L >= K else torch.cat(
-            [torch.zeros(Bsz, K - L, cfg.conv_dim, dtype=xBC_in.dtype, device=h.device), xBC_in], dim=1)
+        window = torch.cat([x_in[:, -K:], bc_in[:, -K:]], dim=-1)              # the conv inputs of the last K tokens
+        if L < K:
+            window = torch.cat([torch.zeros(Bsz, K - L, cfg.conv_dim, dtype=window.dtype, device=h.device), window], dim=1)
         return res, window.transpose(1, 2).contiguous(), final.contiguous()
 
     def forward(self, tokens: torch.Tensor, return_cache: bool = False, last_only: bool = False):

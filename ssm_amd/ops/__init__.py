@@ -635,8 +635,8 @@ def _conv_weight_f32(weight):
     return w.to(torch.float32).contiguous()
 
 
-def _conv_forward(x, weight, bias, activation):
-    batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation)
+def _conv_forward(x, weight, bias, activation, channels_last=None):
+    batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation, channels_last)
     dev = K.require_gpu(x, weight, bias)
     xc = K.cast_c(x, x.dtype)
     wf, bf = _conv_weight_f32(weight), K.as_f32_vec(bias)
@@ -650,9 +650,9 @@ def _conv_forward(x, weight, bias, activation):
     return y
 
 
-def _conv_backward(grad_out, x, weight, bias, activation):
+def _conv_backward(grad_out, x, weight, bias, activation, channels_last=None):
     """-> (dx, dweight (C,K) fp32, dbias (C,) fp32 or None)."""
-    batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation)
+    batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation, channels_last)
     dev = K.require_gpu(x, weight, bias, grad_out)
     xc, gc = K.cast_c(x, x.dtype), K.cast_c(grad_out, x.dtype)
     wf, bf = _conv_weight_f32(weight), K.as_f32_vec(bias)
@@ -684,11 +684,21 @@ def dw_causal_conv(x, weight, bias=None, activation="silu"):
     Returns:
         Tensor with the layout and dtype of ``x``.
     """
+    return _dw_causal_conv(x, weight, bias, activation, None)
+
+
+def dw_causal_conv_channels_last(x, weight, bias=None, activation="silu"):
+    """:func:`dw_causal_conv` on ``x (B, L, C)`` whatever ``L`` is.  Not in the reference, whose layout rule
+    (src/ssm/ops/python/reference.py:483-533) reads a sequence as long as there are channels as ``(B, C, L)``."""
+    return _dw_causal_conv(x, weight, bias, activation, True)
+
+
+def _dw_causal_conv(x, weight, bias, activation, channels_last):
     tensors = (x, weight, bias)
     if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
         from ._autograd import CausalConvFn
-        return CausalConvFn.apply(x, weight, bias, activation)
-    return _conv_forward(x, weight, bias, activation)
+        return CausalConvFn.apply(x, weight, bias, activation, channels_last)
+    return _conv_forward(x, weight, bias, activation, channels_last)
 
 
 # ---------------------------------------------------------------------------
@@ -828,6 +838,7 @@ __all__ = [
     "conv_window_step",
     "ssd_chunk_scan",
     "dw_causal_conv",
+    "dw_causal_conv_channels_last",
     "fused_layer_norm",
     "fused_layer_norm_with_residual",
     "_cpu_backend_status",

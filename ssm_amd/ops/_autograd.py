@@ -26,12 +26,13 @@ def _like(grad, ref):
 
 class CausalConvFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, activation):
+    def forward(ctx, x, weight, bias, activation, channels_last=None):
         from . import _conv_forward
 
-        y = _conv_forward(x, weight, bias, activation)
+        y = _conv_forward(x, weight, bias, activation, channels_last)
         ctx.save_for_backward(x, weight, bias)
         ctx.activation = activation
+        ctx.channels_last = channels_last
         return y
 
     @staticmethod
@@ -39,12 +40,12 @@ class CausalConvFn(torch.autograd.Function):
         from . import _conv_backward
 
         x, weight, bias = ctx.saved_tensors
-        dx, dw, db = _conv_backward(grad_out, x, weight, bias, ctx.activation)
+        dx, dw, db = _conv_backward(grad_out, x, weight, bias, ctx.activation, ctx.channels_last)
         need = ctx.needs_input_grad
         return (_like(dx, x) if need[0] else None,
                 _like(dw, weight) if need[1] else None,
                 _like(db, bias) if (bias is not None and need[2]) else None,
-                None)
+                None, None)
 
 
 class FusedNormFn(torch.autograd.Function):

@@ -188,13 +188,19 @@ def check_state_step(state, x, dt, A, B, C, D, z, dt_bias):
 
 # ------------------------------------------------------------ depthwise conv
 
-def check_conv(x, weight, bias, activation):
+def check_conv(x, weight, bias, activation, channels_last=None):
     """Layout detection and shape contract of ``dw_causal_conv``
-    (reference.py:483-533): channels-first is tested first."""
+    (reference.py:483-533): channels-first is tested first.  ``channels_last`` (not in the
+    reference) names the layout instead, for callers whose sequence length may equal the
+    channel count."""
     if x.ndim != 3:
         raise ValueError("x must have shape (B, C, L) or (B, L, C).")
     chans = int(weight.shape[0]) if weight.ndim >= 1 else -1
-    if x.shape[1] == chans:
+    if channels_last is not None:
+        channels_first = not channels_last
+        if x.shape[1 if channels_first else 2] != chans:
+            raise ValueError("weight channel dimension must match x in the layout named.")
+    elif x.shape[1] == chans:
         channels_first = True
     elif x.shape[2] == chans:
         channels_first = False

@@ -139,3 +139,29 @@ def test_config1_shape_bf16():
     # weight/bias gradients sum 16384 bf16 products: compare against an fp32 evaluation of the slice
     torch.testing.assert_close(wg.grad[idx.cuda()].cpu(), wr.grad, rtol=2e-2, atol=1.0)
     torch.testing.assert_close(bg.grad[idx.cuda()].cpu(), br.grad, rtol=2e-2, atol=1.0)
+
+
+def test_channels_last_entry_when_length_equals_channels():
+    """A sequence as long as there are channels: the reference's rule reads it channels-first; the entry that names
+    the layout convolves along dim 1, forward and backward, like the oracle on the transposed tensor."""
+    from ssm_amd import ops
+    from oracle import ops_oracle as O
+    g = torch.Generator().manual_seed(5)
+    n = 24
+    x = torch.randn(2, n, n, generator=g)
+    w = torch.randn(n, 4, generator=g) * 0.5
+    b = torch.randn(n, generator=g) * 0.1
+    want = O.dw_causal_conv(x.transpose(1, 2).contiguous(), w, b, activation="silu").transpose(1, 2)
+    xg = x.cuda().requires_grad_(True)
+    wg, bg = w.cuda().requires_grad_(True), b.cuda().requires_grad_(True)
+    y = ops.dw_causal_conv_channels_last(xg, wg, bg, activation="silu")
+    torch.testing.assert_close(y.detach().cpu(), want, rtol=1e-5, atol=1e-5)
+    assert not torch.allclose(ops.dw_causal_conv(x.cuda(), w.cuda(), b.cuda()).cpu(), want, atol=1e-3)   # channels-first there
+    go = torch.randn(2, n, n, generator=g)
+    y.backward(go.cuda())
+    xr = x.clone().requires_grad_(True)
+    wr, br = w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    O.dw_causal_conv(xr.transpose(1, 2), wr, br, activation="silu").transpose(1, 2).backward(go)
+    torch.testing.assert_close(xg.grad.cpu(), xr.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(wg.grad.cpu(), wr.grad, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(bg.grad.cpu(), br.grad, rtol=1e-4, atol=1e-4)
