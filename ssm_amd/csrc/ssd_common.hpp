@@ -99,6 +99,30 @@ __device__ __forceinline__ void unpack8(bf16x8_t r, float (&v)[8]) {
   for (int j = 0; j < 8; ++j) v[j] = (float)r[j];
 }
 
+// ---- the same for float16 operands (v_mfma_f32_32x32x16_f16), and the element type as a parameter ----
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+
+__device__ __forceinline__ f32x16_t mma(f16x8_t a, f16x8_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ void unpack8(f16x8_t r, float (&v)[8]) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (float)r[j];
+}
+template <typename E> struct Vec8;
+template <> struct Vec8<__bf16> { using type = bf16x8_t; };
+template <> struct Vec8<_Float16> { using type = f16x8_t; };
+template <typename E> using V8 = typename Vec8<E>::type;
+template <typename E>
+__device__ __forceinline__ V8<E> load_frag_e(const void *p) { return *reinterpret_cast<const V8<E> *>(p); }
+template <typename E>
+__device__ __forceinline__ V8<E> pack8_e(const float (&v)[8]) {
+  V8<E> r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = (E)v[j];
+  return r;
+}
+
 // Row of C-layout register r for a lane in half g = lane / 32.
 __device__ __forceinline__ int crow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
 

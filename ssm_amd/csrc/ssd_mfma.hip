@@ -32,8 +32,8 @@ __device__ __forceinline__ int xt_off(int p, int l, int stride) {
 // Transpose the [Q][P] bf16 slab x[b, t0.., h, :] into LDS as [P][Q] (optionally
 // scaling row l by w[l]).  A thread moves 8x8 blocks: eight 16-byte global reads
 // along p, eight 16-byte LDS writes along l.
-template <bool WEIGHTED>
-__device__ __forceinline__ void stage_xT(__bf16 *xT, const __bf16 *x, size_t row_stride, int Q, int P,
+template <bool WEIGHTED, typename E>
+__device__ __forceinline__ void stage_xT(E *xT, const E *x, size_t row_stride, int Q, int P,
                                          const float *w_lds, int stride) {
   const int pblocks = P >> 3;
   const int nblocks = (Q >> 3) * pblocks;
@@ -42,24 +42,24 @@ __device__ __forceinline__ void stage_xT(__bf16 *xT, const __bf16 *x, size_t row
     float v[8][8];
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const bf16x8_t raw = load_frag(x + (size_t)(lb * 8 + r) * row_stride + pb * 8);
+      const V8<E> raw = load_frag_e<E>(x + (size_t)(lb * 8 + r) * row_stride + pb * 8);
       const float w = WEIGHTED ? w_lds[lb * 8 + r] : 1.0f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[r][i] = WEIGHTED ? (float)raw[i] * w : (float)raw[i];
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      bf16x8_t col;
+      V8<E> col;
 #pragma unroll
-      for (int r = 0; r < 8; ++r) col[r] = (__bf16)v[r][i];
-      *reinterpret_cast<bf16x8_t *>(xT + xt_off(pb * 8 + i, lb * 8, stride)) = col;
+      for (int r = 0; r < 8; ++r) col[r] = (E)v[r][i];
+      *reinterpret_cast<V8<E> *>(xT + xt_off(pb * 8 + i, lb * 8, stride)) = col;
     }
   }
 }
 
 // ------------------------------------------------------------------ bmm_chunk
 // out[b,c,g,l,s] = <a[b,cQ+l,g,:], b[b,cQ+s,g,:]>; one workgroup per 64x64 tile.
-template <typename out_t>
+template <typename E, typename out_t>
 __global__ __launch_bounds__(MF_THREADS) void ssd_bmm_mfma_kernel(const SsdBmmParams p) {
   const int Q = p.chunk, K = p.kdim;
   const int tiles = Q / 64 + (Q % 64 ? 1 : 0);          // 64-wide tiles per side (Q % 32 == 0)
@@ -77,9 +77,9 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_bmm_mfma_kernel(const SsdBmmPa
   f32x16_t acc = {0};
   const bool skip = p.causal && s0 > l0 + 31;
   if (!skip) {
-    const __bf16 *arow = reinterpret_cast<const __bf16 *>(p.a) + (((size_t)b * p.len + c * Q + l0 + m) * p.groups + g) * K + 8 * g2;
-    const __bf16 *brow = reinterpret_cast<const __bf16 *>(p.b) + (((size_t)b * p.len + c * Q + s0 + m) * p.groups + g) * K + 8 * g2;
-    for (int k0 = 0; k0 < K; k0 += 16) acc = mma(load_frag(arow + k0), load_frag(brow + k0), acc);
+    const E *arow = reinterpret_cast<const E *>(p.a) + (((size_t)b * p.len + c * Q + l0 + m) * p.groups + g) * K + 8 * g2;
+    const E *brow = reinterpret_cast<const E *>(p.b) + (((size_t)b * p.len + c * Q + s0 + m) * p.groups + g) * K + 8 * g2;
+    for (int k0 = 0; k0 < K; k0 += 16) acc = mma(load_frag_e<E>(arow + k0), load_frag_e<E>(brow + k0), acc);
   }
   const int *sid = p.seq_idx ? p.seq_idx + (size_t)b * p.len + c * Q : nullptr;
 #pragma unroll
@@ -228,13 +228,13 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_transpose_kernel(const uint16_
 
 // ---------------------------------------------------------------- chunk_state
 // states[b,c,h,p,n] = sum_l xw[l][p] * B[l][n];  one workgroup per (b, c, h).
-template <typename st_t, int PT>
-__global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const SsdStateParams p, const __bf16 *Bt) {
+template <typename E, typename st_t, int PT>
+__global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const SsdStateParams p, const E *Bt) {
   const SsdDims &d = p.d;
   const int Q = d.chunk, P = 32 * PT, N = d.nstate;
   const int stride = Q + XT_PAD;
   extern __shared__ __align__(16) unsigned char smem[];
-  __bf16 *xT = reinterpret_cast<__bf16 *>(smem);                         // [P][Q + pad]
+  E *xT = reinterpret_cast<E *>(smem);                         // [P][Q + pad]
   float *w = reinterpret_cast<float *>(smem + (size_t)P * stride * 2);   // [Q]
   const int wave = wave_id_uniform(), lane = lane_id();
   const int h = blockIdx.x % d.heads;
@@ -249,8 +249,8 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const 
   for (int l = threadIdx.x; l < Q; l += MF_THREADS)
     w[l] = (sid && sid[l] != sid_last) ? 0.0f : decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
   __syncthreads();
-  const __bf16 *xg = reinterpret_cast<const __bf16 *>(p.x) + (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
-  stage_xT<true>(xT, xg, (size_t)d.heads * P, Q, P, w, stride);
+  const E *xg = reinterpret_cast<const E *>(p.x) + (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
+  stage_xT<true, E>(xT, xg, (size_t)d.heads * P, Q, P, w, stride);
   __syncthreads();
 
   const int g2 = lane >> 5, m = lane & 31;
@@ -260,13 +260,13 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const 
 #pragma unroll
     for (int i = 0; i < PT; ++i) acc[i] = (f32x16_t){0};
     const bool ncol_ok = n0 + m < N;
-    const __bf16 *bt = Bt + (((size_t)b * d.groups + g) * N + (ncol_ok ? n0 + m : 0)) * (size_t)d.len + (size_t)c * Q + 8 * g2;
+    const E *bt = Bt + (((size_t)b * d.groups + g) * N + (ncol_ok ? n0 + m : 0)) * (size_t)d.len + (size_t)c * Q + 8 * g2;
     for (int k0 = 0; k0 < Q; k0 += 16) {
-      bf16x8_t bf = load_frag(bt + k0);
-      if (!ncol_ok) bf = (bf16x8_t){0};
+      V8<E> bf = load_frag_e<E>(bt + k0);
+      if (!ncol_ok) bf = (V8<E>){0};
 #pragma unroll
       for (int i = 0; i < PT; ++i) {
-        const bf16x8_t af = load_frag(xT + xt_off(32 * i + m, k0 + 8 * g2, stride));
+        const V8<E> af = load_frag_e<E>(xT + xt_off(32 * i + m, k0 + 8 * g2, stride));
         acc[i] = mma(af, bf, acc[i]);
       }
     }
@@ -281,13 +281,13 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const 
 
 // ----------------------------------------------------------------- chunk_scan
 // One workgroup per (b, c, h); wave w owns row blocks w, nlb-1-w, w+4, ... of 32 rows.
-template <typename st_t, int PT>
+template <typename E, typename st_t, int PT>
 __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const SsdScanParams p) {
   const SsdDims &d = p.d;
   const int Q = d.chunk, P = 32 * PT, N = d.nstate;
   const int stride = Q + XT_PAD;
   extern __shared__ __align__(16) unsigned char smem[];
-  __bf16 *xT = reinterpret_cast<__bf16 *>(smem);                          // [P][Q + pad], unweighted
+  E *xT = reinterpret_cast<E *>(smem);                          // [P][Q + pad], unweighted
   float *dAs = reinterpret_cast<float *>(smem + (size_t)P * stride * 2);  // [Q]
   float *dts = dAs + Q;                                                   // [Q]
   float *ent = dts + Q;                                                   // [Q] 1 where the entering state reaches the step
@@ -308,11 +308,11 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   }
   const size_t xrow = (size_t)d.heads * P;                                 // elements between time steps
   const size_t xbase = (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
-  const __bf16 *xg = reinterpret_cast<const __bf16 *>(p.x) + xbase;
-  stage_xT<false>(xT, xg, xrow, Q, P, nullptr, stride);
+  const E *xg = reinterpret_cast<const E *>(p.x) + xbase;
+  stage_xT<false, E>(xT, xg, xrow, Q, P, nullptr, stride);
   // The state entering the chunk, [P][N], as bfloat16 in LDS: read once by the workgroup in whole lines (a fragment
   // read straight from memory, lane = row, touches 32 lines for 32 bytes each, and every row block would read it again).
-  __bf16 *Sb = reinterpret_cast<__bf16 *>(ent + Q);                       // [P][N + 8]
+  E *Sb = reinterpret_cast<E *>(ent + Q);                       // [P][N + 8]
   const int SR = N + 8;
   {
     const st_t *Sg0 = reinterpret_cast<const st_t *>(p.prev) + ((((size_t)b * d.nchunks + c) * d.heads + h) * P) * (size_t)N;
@@ -320,26 +320,26 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
     for (int e = threadIdx.x; e < P * pieces; e += MF_THREADS) {
       const int row = e / pieces, piece = e % pieces;
       const st_t *sp = Sg0 + (size_t)row * N + 8 * piece;
-      bf16x8_t v;
+      V8<E> v;
       if constexpr (sizeof(st_t) == 2) {
-        v = load_frag(sp);
+        v = load_frag_e<E>(sp);
       } else {
         const float4 lo = *reinterpret_cast<const float4 *>(sp), hi = *reinterpret_cast<const float4 *>(sp + 4);
         const float t8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        v = pack8(t8);
+        v = pack8_e<E>(t8);
       }
-      *reinterpret_cast<bf16x8_t *>(Sb + row * SR + 8 * piece) = v;
+      *reinterpret_cast<V8<E> *>(Sb + row * SR + 8 * piece) = v;
     }
   }
   __syncthreads();
 
   const int g2 = lane >> 5, m = lane & 31;
   const int nlb = Q / 32;
-  const __bf16 *Cg = reinterpret_cast<const __bf16 *>(p.Cm) + (((size_t)b * d.len + (size_t)c * Q) * d.groups + g) * N;
+  const E *Cg = reinterpret_cast<const E *>(p.Cm) + (((size_t)b * d.len + (size_t)c * Q) * d.groups + g) * N;
   const size_t c_stride = (size_t)d.groups * N;
-  const __bf16 *CBg = reinterpret_cast<const __bf16 *>(p.CB) + (((size_t)b * d.nchunks + c) * d.groups + g) * (size_t)Q * Q;
-  const __bf16 *zg = p.z ? reinterpret_cast<const __bf16 *>(p.z) + xbase : nullptr;
-  __bf16 *yg = reinterpret_cast<__bf16 *>(p.y) + xbase;
+  const E *CBg = reinterpret_cast<const E *>(p.CB) + (((size_t)b * d.nchunks + c) * d.groups + g) * (size_t)Q * Q;
+  const E *zg = p.z ? reinterpret_cast<const E *>(p.z) + xbase : nullptr;
+  E *yg = reinterpret_cast<E *>(p.y) + xbase;
   float *yf = reinterpret_cast<float *>(p.y) + xbase;
   const bool y_f32 = p.y_dtype == SSM_F32;
 
@@ -353,11 +353,11 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
       for (int i = 0; i < PT; ++i) acc[i] = (f32x16_t){0};
 
       // carried-in state: C[l][:] . S[p][:]
-      const __bf16 *crow_p = Cg + (size_t)(l0 + m) * c_stride + 8 * g2;
+      const E *crow_p = Cg + (size_t)(l0 + m) * c_stride + 8 * g2;
       for (int n0 = 0; n0 < N; n0 += 16) {
-        const bf16x8_t af = load_frag(crow_p + n0);
+        const V8<E> af = load_frag_e<E>(crow_p + n0);
 #pragma unroll
-        for (int i = 0; i < PT; ++i) acc[i] = mma(af, load_frag(Sb + (32 * i + m) * SR + n0 + 8 * g2), acc[i]);
+        for (int i = 0; i < PT; ++i) acc[i] = mma(af, load_frag_e<E>(Sb + (32 * i + m) * SR + n0 + 8 * g2), acc[i]);
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -369,10 +369,10 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
       // within the chunk: M[l][s] = CB[l][s] exp(dA_l - dA_s) dt_s for s <= l
       const int lrow = l0 + m;                       // this lane's row as an A operand
       const float dal = dAs[lrow];
-      const __bf16 *cbrow = CBg + (size_t)lrow * Q + 8 * g2;
+      const E *cbrow = CBg + (size_t)lrow * Q + 8 * g2;
       for (int s0 = 0; s0 < l0 + 32; s0 += 16) {
         float cb[8];
-        unpack8(load_frag(cbrow + s0), cb);
+        unpack8(load_frag_e<E>(cbrow + s0), cb);
         const int sbase = s0 + 8 * g2;
         const float4 a0 = *reinterpret_cast<const float4 *>(dAs + sbase), a1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
         const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
@@ -384,10 +384,10 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
           const float v = cb[j] * decay_exp(dal - das[j]) * dtv[j];
           mv[j] = (sbase + j <= lrow) ? v : 0.0f;
         }
-        const bf16x8_t af = pack8(mv);
+        const V8<E> af = pack8_e<E>(mv);
 #pragma unroll
         for (int i = 0; i < PT; ++i) {
-          const bf16x8_t bf = load_frag(xT + xt_off(32 * i + m, sbase, stride));
+          const V8<E> bf = load_frag_e<E>(xT + xt_off(32 * i + m, sbase, stride));
           acc[i] = mma(af, bf, acc[i]);
         }
       }
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
           if (p.Dk) v = __builtin_fmaf(Dv, (float)xg[at], v);
           if (zg) v *= silu_f32((float)zg[at]);
           if (y_f32) yf[at] = v;
-          else yg[at] = (__bf16)v;
+          else yg[at] = (E)v;
         }
       }
     }
@@ -417,13 +417,20 @@ static bool mfma_shape_ok(const SsdDims &d) {
 }
 
 bool ssd_bmm_mfma(const SsdBmmParams &p, hipStream_t s) {
-  if (p.in_dtype != SSM_BF16 || p.out_dtype == SSM_F16) return false;
+  // 16-bit operands of one type; the product in float32 or in the operands' type
+  if (p.in_dtype != SSM_BF16 && p.in_dtype != SSM_F16) return false;
+  if (p.out_dtype != SSM_F32 && p.out_dtype != p.in_dtype) return false;
   if (p.len % p.chunk != 0 || p.chunk % 32 != 0 || p.kdim % 16 != 0) return false;
   if (!aligned_to(p.a, 16) || !aligned_to(p.b, 16)) return false;
   const int tiles = (p.chunk + 63) / 64;
-  const unsigned grid = (unsigned)((size_t)p.batch * p.nchunks * p.groups * tiles * tiles);
-  if (p.out_dtype == SSM_F32) hipLaunchKernelGGL(ssd_bmm_mfma_kernel<float>, dim3(grid), dim3(MF_THREADS), 0, s, p);
-  else hipLaunchKernelGGL(ssd_bmm_mfma_kernel<bf16_t>, dim3(grid), dim3(MF_THREADS), 0, s, p);
+  const dim3 grid((unsigned)((size_t)p.batch * p.nchunks * p.groups * tiles * tiles)), block(MF_THREADS);
+  if (p.in_dtype == SSM_BF16) {
+    if (p.out_dtype == SSM_F32) hipLaunchKernelGGL((ssd_bmm_mfma_kernel<__bf16, float>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((ssd_bmm_mfma_kernel<__bf16, bf16_t>), grid, block, 0, s, p);
+  } else {
+    if (p.out_dtype == SSM_F32) hipLaunchKernelGGL((ssd_bmm_mfma_kernel<_Float16, float>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((ssd_bmm_mfma_kernel<_Float16, f16_t>), grid, block, 0, s, p);
+  }
   return true;
 }
 
@@ -433,48 +440,63 @@ size_t ssd_chunk_state_scratch_bytes(const SsdDims &d) {
 
 bool ssd_chunk_state_mfma(const SsdStateParams &p, hipStream_t s) {
   const SsdDims &d = p.d;
-  if (!mfma_shape_ok(d) || p.x_dtype != SSM_BF16 || p.b_dtype != SSM_BF16 || p.states_dtype == SSM_F16) return false;
+  const bool half = p.x_dtype == SSM_BF16 || p.x_dtype == SSM_F16;
+  if (!mfma_shape_ok(d) || !half || p.b_dtype != p.x_dtype) return false;
+  if (p.states_dtype != SSM_F32 && p.states_dtype != p.x_dtype) return false;
   if (!p.scratch || p.scratch_bytes < ssd_chunk_state_scratch_bytes(d)) return false;
   if (!aligned_to(p.x, 16) || !aligned_to(p.scratch, 16) || d.len % 8 != 0) return false;
-  __bf16 *Bt = reinterpret_cast<__bf16 *>(p.scratch);
   hipLaunchKernelGGL(ssd_transpose_kernel, dim3((d.len + 63) / 64, (d.nstate + 63) / 64, d.batch * d.groups),
-                     dim3(MF_THREADS), 0, s, reinterpret_cast<const uint16_t *>(p.Bm), reinterpret_cast<uint16_t *>(Bt),
+                     dim3(MF_THREADS), 0, s, reinterpret_cast<const uint16_t *>(p.Bm), reinterpret_cast<uint16_t *>(p.scratch),
                      d.len, d.groups, d.nstate);
   const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 4;
   const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);
-#define SSM_LAUNCH_CS(ST, PT)                                                                              \
+#define SSM_LAUNCH_CS(E, ST, PT)                                                                           \
   {                                                                                                        \
-    auto kernel = ssd_chunk_state_mfma_kernel<ST, PT>;                                                     \
+    auto kernel = ssd_chunk_state_mfma_kernel<E, ST, PT>;                                                  \
     if (allow_dynamic_lds(kernel, lds) != hipSuccess) { (void)hipGetLastError(); return false; }           \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(MF_THREADS), lds, s, p, Bt);                               \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(MF_THREADS), lds, s, p, reinterpret_cast<const E *>(p.scratch)); \
   }
-  if (p.states_dtype == SSM_F32) {
-    if (d.hdim == 64) SSM_LAUNCH_CS(float, 2) else SSM_LAUNCH_CS(float, 1)
-  } else {
-    if (d.hdim == 64) SSM_LAUNCH_CS(bf16_t, 2) else SSM_LAUNCH_CS(bf16_t, 1)
+#define SSM_LAUNCH_CS_E(E, ST16)                                                                           \
+  {                                                                                                        \
+    if (p.states_dtype == SSM_F32) {                                                                       \
+      if (d.hdim == 64) SSM_LAUNCH_CS(E, float, 2) else SSM_LAUNCH_CS(E, float, 1)                         \
+    } else {                                                                                               \
+      if (d.hdim == 64) SSM_LAUNCH_CS(E, ST16, 2) else SSM_LAUNCH_CS(E, ST16, 1)                           \
+    }                                                                                                      \
   }
+  if (p.x_dtype == SSM_BF16) SSM_LAUNCH_CS_E(__bf16, bf16_t)
+  else SSM_LAUNCH_CS_E(_Float16, f16_t)
+#undef SSM_LAUNCH_CS_E
 #undef SSM_LAUNCH_CS
   return true;
 }
 
 bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s) {
   const SsdDims &d = p.d;
-  if (!mfma_shape_ok(d) || p.x_dtype != SSM_BF16 || p.c_dtype != SSM_BF16 || p.cb_dtype != SSM_BF16) return false;
-  if (p.states_dtype == SSM_F16 || (p.z && p.z_dtype != SSM_BF16)) return false;
+  const bool half = p.x_dtype == SSM_BF16 || p.x_dtype == SSM_F16;
+  if (!mfma_shape_ok(d) || !half || p.c_dtype != p.x_dtype || p.cb_dtype != p.x_dtype) return false;
+  if ((p.states_dtype != SSM_F32 && p.states_dtype != p.x_dtype) || (p.z && p.z_dtype != p.x_dtype)) return false;
+  if (p.y_dtype != SSM_F32 && p.y_dtype != p.x_dtype) return false;
   if (!aligned_to(p.x, 16) || !aligned_to(p.Cm, 16) || !aligned_to(p.CB, 16) || !aligned_to(p.prev, 16)) return false;
   const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 12 + (size_t)d.hdim * (d.nstate + 8) * 2;
   const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);
-#define SSM_LAUNCH_SC(ST, PT)                                                                              \
+#define SSM_LAUNCH_SC(E, ST, PT)                                                                           \
   {                                                                                                        \
-    auto kernel = ssd_chunk_scan_mfma_kernel<ST, PT>;                                                      \
+    auto kernel = ssd_chunk_scan_mfma_kernel<E, ST, PT>;                                                   \
     if (allow_dynamic_lds(kernel, lds) != hipSuccess) { (void)hipGetLastError(); return false; }           \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(MF_THREADS), lds, s, p);                                   \
   }
-  if (p.states_dtype == SSM_F32) {
-    if (d.hdim == 64) SSM_LAUNCH_SC(float, 2) else SSM_LAUNCH_SC(float, 1)
-  } else {
-    if (d.hdim == 64) SSM_LAUNCH_SC(bf16_t, 2) else SSM_LAUNCH_SC(bf16_t, 1)
+#define SSM_LAUNCH_SC_E(E, ST16)                                                                           \
+  {                                                                                                        \
+    if (p.states_dtype == SSM_F32) {                                                                       \
+      if (d.hdim == 64) SSM_LAUNCH_SC(E, float, 2) else SSM_LAUNCH_SC(E, float, 1)                         \
+    } else {                                                                                               \
+      if (d.hdim == 64) SSM_LAUNCH_SC(E, ST16, 2) else SSM_LAUNCH_SC(E, ST16, 1)                           \
+    }                                                                                                      \
   }
+  if (p.x_dtype == SSM_BF16) SSM_LAUNCH_SC_E(__bf16, bf16_t)
+  else SSM_LAUNCH_SC_E(_Float16, f16_t)
+#undef SSM_LAUNCH_SC_E
 #undef SSM_LAUNCH_SC
   return true;
 }

@@ -431,7 +431,7 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
     """
     Q = int(chunk_size)
     seqlen = int(x.shape[1]) if x.ndim == 4 else 0
-    if (x.ndim == 4 and x.dtype == torch.bfloat16 and Q > 0 and seqlen % Q != 0 and not force_generic
+    if (x.ndim == 4 and x.dtype in (torch.bfloat16, torch.float16) and Q > 0 and seqlen % Q != 0 and not force_generic
             and float(dt_limit[0]) <= 0.0 and dt.ndim == 3):
         # The matrix-core kernels take whole chunks.  Steps of size zero neither decay the state nor add to
         # it, so a ragged end is filled up with them (zeros for x, B, C, z) and the extra rows of y dropped;
@@ -493,7 +493,7 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
     Q = int(chunk_size)
     _need(not return_varlen_states or cu_seqlens is not None, "return_varlen_states needs cu_seqlens.")
     _need(cu_seqlens is None or batch == 1, "cu_seqlens describes one packed batch row: batch size must be 1.")
-    if x.dtype == torch.bfloat16 and hdim > 64 and hdim % 64 == 0 and not force_generic:
+    if x.dtype in (torch.bfloat16, torch.float16) and hdim > 64 and hdim % 64 == 0 and not force_generic:
         # Channels of a head do not interact: a head of 64k channels is k heads of 64 with the same step,
         # decay and group, which is the width the one-pass and matrix-core kernels are built for.  The
         # channel axis is innermost, so this is a view of x, z and the states.

@@ -484,9 +484,11 @@ def test_components_match_oracle_fp32():
 @pytest.mark.parametrize("shape,Q", [((2, 512, 4, 64, 1, 128), 256), ((1, 256, 2, 64, 2, 64), 64),
                                      ((2, 384, 8, 32, 1, 128), 128), ((1, 700, 2, 64, 1, 128), 256)],
                          ids=lambda v: str(v).replace(" ", ""))
-def test_bf16_mfma_matches_generic_and_oracle(shape, Q):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda v: str(v).replace("torch.", ""))
+def test_bf16_mfma_matches_generic_and_oracle(shape, Q, dtype):
+    """The five matrix-core kernels, for both 16-bit element types (v_mfma_f32_32x32x16_bf16 / _f16)."""
     b, l, h, p, g, n = shape
-    inp = make(11, b, l, h, p, g, n, dtype=torch.bfloat16)
+    inp = make(11, b, l, h, p, g, n, dtype=dtype)
     args = (cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
     kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
     from ssm_amd import _lib
