@@ -281,6 +281,8 @@ static void launch_norm_fwd_typed(const NormParams &p, int per_lane, unsigned gr
   else if (per_lane <= 16) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, false, XT, RT>), dim3(grid), b, 0, s, p);
   else if (per_lane <= 32) hipLaunchKernelGGL((norm_fwd_typed_kernel<8, false, XT, RT>), dim3(grid), b, 0, s, p);
   else if (p.hidden <= 4096) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, true, XT, RT>), dim3(p.rows), b, 0, s, p);
+  else if (p.hidden <= 5120) hipLaunchKernelGGL((norm_fwd_typed_kernel<5, true, XT, RT>), dim3(p.rows), b, 0, s, p);
+  else if (p.hidden <= 6144) hipLaunchKernelGGL((norm_fwd_typed_kernel<6, true, XT, RT>), dim3(p.rows), b, 0, s, p);
   else if (p.hidden <= 8192) hipLaunchKernelGGL((norm_fwd_typed_kernel<8, true, XT, RT>), dim3(p.rows), b, 0, s, p);
   else hipLaunchKernelGGL((norm_fwd_typed_kernel<16, true, XT, RT>), dim3(p.rows), b, 0, s, p);
 }
@@ -634,7 +636,12 @@ static void launch_norm_bwd_typed(const NormParams &p, int hidden, int grid, hip
   else if (per_lane <= 12) hipLaunchKernelGGL((norm_bwd_kernel<3, false, XT, RT>), g, b, 0, s, p, 1);
   else if (hidden <= 1024) hipLaunchKernelGGL((norm_bwd_kernel<1, true, XT, RT>), g, b, 0, s, p, 1);
   else if (hidden <= 2048) hipLaunchKernelGGL((norm_bwd_kernel<2, true, XT, RT>), g, b, 0, s, p, 1);
+  // a thread's registers grow with the trips it is compiled for: the widths of common models (2560, 5120) get
+  // their own count rather than the next power of two
+  else if (hidden <= 3072) hipLaunchKernelGGL((norm_bwd_kernel<3, true, XT, RT>), g, b, 0, s, p, 1);
   else if (hidden <= 4096) hipLaunchKernelGGL((norm_bwd_kernel<4, true, XT, RT>), g, b, 0, s, p, 1);
+  else if (hidden <= 5120) hipLaunchKernelGGL((norm_bwd_kernel<5, true, XT, RT>), g, b, 0, s, p, 1);
+  else if (hidden <= 6144) hipLaunchKernelGGL((norm_bwd_kernel<6, true, XT, RT>), g, b, 0, s, p, 1);
   else hipLaunchKernelGGL((norm_bwd_kernel<8, true, XT, RT>), g, b, 0, s, p, 1);
 }
 }  // namespace ssm
