@@ -151,6 +151,9 @@ typedef struct ssm_state_step_args {
   int32_t state_dtype, io_dtype, bc_dtype;
   int32_t b_kind, c_kind, b_groups, c_groups;
   int32_t dt_softplus;
+  /* Elements between consecutive batch rows of z and of grouped (B,G,N) projections, for rows that are slices of
+   * wider rows (a decoding block's projected row); 0 = dense.  The rows themselves are contiguous. */
+  int64_t z_batch_stride, b_batch_stride, c_batch_stride;
 } ssm_state_step_args;
 
 int ssm_state_step(const ssm_state_step_args *args, void *hip_stream);

@@ -67,6 +67,7 @@ class StateStepArgs(C.Structure):
         ("state_dtype", _i32), ("io_dtype", _i32), ("bc_dtype", _i32),
         ("b_kind", _i32), ("c_kind", _i32), ("b_groups", _i32), ("c_groups", _i32),
         ("dt_softplus", _i32),
+        ("z_batch_stride", C.c_int64), ("b_batch_stride", C.c_int64), ("c_batch_stride", C.c_int64),
     ]
 
 

@@ -24,6 +24,7 @@ struct StepParams {
   int b_kind, c_kind, b_groups, c_groups;
   int softplus;
   int tpr_log2;   // lanes per row = 1 << tpr_log2
+  long long z_bs, b_bs, c_bs;   // elements between batch rows of z and of grouped B / C (dense: dim, groups * nstate)
   // fused causal-conv front end (decode): x is the raw input, the conv window is rolled in place
   void *conv_state;          // (B, D, K) io dtype or null
   const float *conv_w;       // (D, K)
@@ -94,9 +95,9 @@ __global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
   const int N = p.nstate;
 
   size_t b_off, c_off;
-  if (p.b_kind == SSM_PROJ_BGNL) b_off = ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * N;
+  if (p.b_kind == SSM_PROJ_BGNL) b_off = (size_t)b * p.b_bs + (size_t)(d / (p.dim / p.b_groups)) * N;
   else b_off = ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
-  if (p.c_kind == SSM_PROJ_BGNL) c_off = ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * N;
+  if (p.c_kind == SSM_PROJ_BGNL) c_off = (size_t)b * p.c_bs + (size_t)(d / (p.dim / p.c_groups)) * N;
   else c_off = ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
   state_t *srow = reinterpret_cast<state_t *>(p.state) + r * N;
   const float *arow = p.A + (size_t)d * N;
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(256) void state_step_kernel(const StepParams p) {
   float dtv = load_as_f32(p.dt, p.io_dtype, r);
   if (p.bias) dtv += p.bias[d];
   float xv = load_as_f32(p.x, p.io_dtype, r);
-  const float zv = p.z ? load_as_f32(p.z, p.io_dtype, r) : 0.0f;
+  const float zv = p.z ? load_as_f32(p.z, p.io_dtype, (size_t)b * p.z_bs + d) : 0.0f;
   if (p.softplus) dtv = softplus_f32(dtv);
   if (p.conv_state) {
     // window <- (window[1:], x); x <- act(bias + sum_k w[k] window[k]).  The row's lanes
@@ -217,14 +218,14 @@ __global__ __launch_bounds__(256) void state_step_rb_kernel(const StepParams p) 
   for (int rb = 0; rb < RB; ++rb) {
     const int b = bg * RB + rb;
     const size_t r = (size_t)b * p.dim + d;
-    const size_t b_off = p.b_kind == SSM_PROJ_BGNL ? ((size_t)b * p.b_groups + bgrp) * N
+    const size_t b_off = p.b_kind == SSM_PROJ_BGNL ? (size_t)b * p.b_bs + (size_t)bgrp * N
                                                     : ((p.b_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
-    const size_t c_off = p.c_kind == SSM_PROJ_BGNL ? ((size_t)b * p.c_groups + cgrp) * N
+    const size_t c_off = p.c_kind == SSM_PROJ_BGNL ? (size_t)b * p.c_bs + (size_t)cgrp * N
                                                     : ((p.c_kind == SSM_PROJ_BDN ? (size_t)b * p.dim : 0) + d) * (size_t)N;
     load_vec<state_t, VEC>(reinterpret_cast<const state_t *>(p.state) + r * N + n0, h[rb]);
     ld_vec_io<io_t, VEC>(p.Bp, p.bc_dtype, b_off + n0, bv[rb]);
     ld_vec_io<io_t, VEC>(p.Cp, p.bc_dtype, c_off + n0, cv[rb]);
-    scal[rb] = ld_io<io_t>(scal_ptr, p.io_dtype, r);
+    scal[rb] = ld_io<io_t>(scal_ptr, p.io_dtype, (sub == 2 && p.z) ? (size_t)b * p.z_bs + d : r);
     win[rb] = CONV ? ld_io<io_t>(p.conv_state, p.io_dtype, r * K + win_k) : 0.0f;
   }
 #pragma unroll
@@ -361,6 +362,15 @@ static int run_state_step(const ssm_state_step_args *a, const ssm_decode_step_ar
   p.b_groups = a->b_kind == SSM_PROJ_BGNL ? a->b_groups : 1;
   p.c_groups = a->c_kind == SSM_PROJ_BGNL ? a->c_groups : 1;
   p.softplus = a->dt_softplus ? 1 : 0;
+  SSM_REQUIRE(a->z_batch_stride >= 0 && a->b_batch_stride >= 0 && a->c_batch_stride >= 0 &&
+                  (a->z_batch_stride == 0 || a->z_batch_stride >= a->dim) &&
+                  (a->b_batch_stride == 0 || (a->b_kind == SSM_PROJ_BGNL && a->b_batch_stride >= (long long)a->b_groups * a->nstate)) &&
+                  (a->c_batch_stride == 0 || (a->c_kind == SSM_PROJ_BGNL && a->c_batch_stride >= (long long)a->c_groups * a->nstate)),
+              SSM_ERR_BAD_SHAPE,
+              "ssm_state_step: batch strides must hold a row (z: dim; B, C: groups * nstate, grouped projections only)");
+  p.z_bs = a->z_batch_stride ? a->z_batch_stride : a->dim;
+  p.b_bs = a->b_batch_stride ? a->b_batch_stride : (long long)p.b_groups * a->nstate;
+  p.c_bs = a->c_batch_stride ? a->c_batch_stride : (long long)p.c_groups * a->nstate;
   p.tpr_log2 = 0;
   p.conv_state = nullptr; p.conv_w = nullptr; p.conv_b = nullptr; p.conv_out = nullptr; p.conv_k = 0; p.conv_silu = 0;
   if (dec) {
@@ -370,7 +380,7 @@ static int run_state_step(const ssm_state_step_args *a, const ssm_decode_step_ar
     p.conv_out = dec->conv_out; p.conv_k = dec->conv_width; p.conv_silu = dec->conv_activation == SSM_ACT_SILU;
   }
   const bool vec4 = a->nstate % 4 == 0 && aligned_to(a->state, 4 * ss) && aligned_to(a->A, 16) &&
-                    aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs);
+                    aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs) && p.b_bs % 4 == 0 && p.c_bs % 4 == 0;
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   switch (a->state_dtype) {
     case SSM_F32: return launch_step<float>(p, vec4, stream);

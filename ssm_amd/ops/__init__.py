@@ -245,8 +245,13 @@ class StepPlan:
         io = K.common_io_dtype([x, dt, z])
         bc = K.common_io_dtype([B, C])
         self.result_dtype = x.dtype
-        self.keep = dict(x=K.cast_c(x, io), dt=K.cast_c(dt, io), z=K.cast_c(z, io), B=K.cast_c(B, bc),
-                         C=K.cast_c(C, bc), A=K.as_f32_vec(A), D=K.as_f32_vec(D), bias=K.as_f32_vec(dt_bias))
+        # z and grouped B / C may be slices of wider rows (a block's projected row): taken as they are, with the
+        # distance between batch rows, instead of being copied
+        zk, z_bs = _rows_as_given(z, io)
+        Bk, b_bs = _rows_as_given(B, bc) if bkind == _lib.PROJ_BGNL else (K.cast_c(B, bc), 0)
+        Ck, c_bs = _rows_as_given(C, bc) if ckind == _lib.PROJ_BGNL else (K.cast_c(C, bc), 0)
+        self.keep = dict(x=K.cast_c(x, io), dt=K.cast_c(dt, io), z=zk, B=Bk, C=Ck, A=K.as_f32_vec(A),
+                         D=K.as_f32_vec(D), bias=K.as_f32_vec(dt_bias))
         k = self.keep
         self.state = state.detach()
         self.out = out if out is not None else torch.empty(batch, dim, dtype=io, device=self.device)
@@ -257,11 +262,25 @@ class StepPlan:
             batch=batch, dim=dim, nstate=nstate,
             state_dtype=_lib.dtype_enum(state.dtype), io_dtype=_lib.dtype_enum(io),
             bc_dtype=_lib.dtype_enum(bc), b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
-            dt_softplus=int(bool(softplus)))
+            dt_softplus=int(bool(softplus)), z_batch_stride=z_bs, b_batch_stride=b_bs, c_batch_stride=c_bs)
 
     def run(self):
         _lib.call("ssm_state_step", self.args, self.device)
         return self.out
+
+
+def _rows_as_given(t, dtype):
+    """``(tensor, batch stride)`` for ``ssm_state_step``: a tensor of the right dtype whose batch rows are
+    contiguous but apart from each other (a slice of wider rows) is passed as it is with its batch stride;
+    anything else as a dense copy with stride 0 (= dense)."""
+    if t is None:
+        return None, 0
+    if t.dtype == dtype and t.ndim >= 2 and t.shape[0] > 1 and not t.is_contiguous():
+        row = t[0]
+        if row.is_contiguous() and t.stride(0) >= row.numel() and (t.stride(0) * t.element_size()) % 8 == 0 \
+                and t.data_ptr() % 8 == 0:
+            return t, int(t.stride(0))
+    return K.cast_c(t, dtype), 0
 
 
 def _state_step_backward(grad_out, grad_state, state, x, dt, A, B, C, D, z, dt_bias, softplus):

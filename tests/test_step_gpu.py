@@ -119,6 +119,37 @@ def test_optional_arguments(use_D, use_z, use_bias, softplus):
     torch.testing.assert_close(st, sr, **FP32_TOL)
 
 
+@pytest.mark.parametrize("io,batch,dim,nstate,groups", [(torch.bfloat16, 8, 1536, 16, 1), (torch.float32, 3, 96, 8, 2),
+                                                         (torch.float16, 5, 64, 12, 1), (torch.bfloat16, 2, 40, 6, 1)])
+def test_rows_cut_out_of_wider_rows_are_taken_as_they_are(io, batch, dim, nstate, groups):
+    """z, B and C as slices of one projected row per batch entry (what a decoding block has): the kernel reads them
+    in place through their batch strides; same result as dense copies, and the wrapper makes no copy when the
+    slices are 8-byte aligned (an odd offset falls back to one)."""
+    inp = make(21, batch, dim, nstate, io=io, st=torch.float32, groups=groups)
+    gn = groups * nstate
+    for lead in (8, 3):
+        wide = torch.cat([torch.zeros(batch, lead).to(io), inp["z"], inp["B"].reshape(batch, gn),
+                          inp["C"].reshape(batch, gn), torch.zeros(batch, 5).to(io)], dim=1).cuda()
+        z = wide[:, lead:lead + dim]
+        Bm = wide[:, lead + dim:lead + dim + gn].reshape(batch, groups, nstate)
+        Cm = wide[:, lead + dim + gn:lead + dim + 2 * gn].reshape(batch, groups, nstate)
+        assert not z.is_contiguous() and Bm.data_ptr() == wide.data_ptr() + (lead + dim) * wide.element_size()
+        st = dev(inp["state"].clone())
+        plan = _ops().StepPlan(st, dev(inp["x"]), dev(inp["dt"]), dev(inp["A"]), Bm, Cm, dev(inp["D"]), z,
+                               dev(inp["dt_bias"]), True)
+        in_place = plan.keep["z"].data_ptr() == z.data_ptr() and plan.keep["B"].data_ptr() == Bm.data_ptr()
+        y = plan.run()
+        st2 = dev(inp["state"].clone())
+        y2 = _ops().selective_state_step(st2, dev(inp["x"]), dev(inp["dt"]), dev(inp["A"]), dev(inp["B"]), dev(inp["C"]),
+                                         D=dev(inp["D"]), z=dev(inp["z"]), dt_bias=dev(inp["dt_bias"]), softplus=True)
+        torch.testing.assert_close(y, y2, rtol=0, atol=0)
+        torch.testing.assert_close(st, st2, rtol=0, atol=0)
+        row_bytes_ok = (wide.stride(0) * wide.element_size()) % 8 == 0
+        offsets_ok = all(t.data_ptr() % 8 == 0 for t in (z, Bm, Cm))
+        if row_bytes_ok and offsets_ok:
+            assert in_place, "aligned slices should be read in place"
+
+
 def test_repeated_steps_equal_scan_last_state():
     """L steps from a zero state reproduce selective_scan and its last_state."""
     from tests.test_scan_fwd_gpu import make_inputs
