@@ -241,12 +241,31 @@ def bench_dscan(batch=4, length=4096, heads=80, proj=64, chunk=256):
     fbytes = el * 2 * 5 + batch * length * heads * 4               # X, B, C, z in; Y out; dt
     bbytes = el * 2 * 6 + el * 2 * 4 + batch * length * heads * 8  # X, B, C, z, grad_y in; dX, dB, dC, dz out; dt, ddt
     sbytes = el * 2 * 6 + el * 2 + el * 4 * 3 + batch * length * heads * 8   # dB, dC, dz in float32
-    return {"fwd_us": round(fus, 1), "fwd_GBps": round(fbytes / fus / 1e3, 1),
-            "fwd_frac_hbm": round(fbytes / fus / 1e3 / HBM_PEAK_GBPS, 4),
-            "bwd_us": round(bus, 1), "bwd_GBps": round(bbytes / bus / 1e3, 1),
-            "bwd_frac_hbm": round(bbytes / bus / 1e3 / HBM_PEAK_GBPS, 4),
-            "bwd_alone_fp32_grads_us": round(sus, 1), "bwd_alone_fp32_grads_GBps": round(sbytes / sus / 1e3, 1),
-            "shape": f"X (B={batch}, L={length}, H={heads}, P={proj}) bf16, chunk {chunk}"}
+    out = {"fwd_us": round(fus, 1), "fwd_GBps": round(fbytes / fus / 1e3, 1),
+           "fwd_frac_hbm": round(fbytes / fus / 1e3 / HBM_PEAK_GBPS, 4),
+           "bwd_us": round(bus, 1), "bwd_GBps": round(bbytes / bus / 1e3, 1),
+           "bwd_frac_hbm": round(bbytes / bus / 1e3 / HBM_PEAK_GBPS, 4),
+           "bwd_alone_fp32_grads_us": round(sus, 1), "bwd_alone_fp32_grads_GBps": round(sbytes / sus / 1e3, 1),
+           "shape": f"X (B={batch}, L={length}, H={heads}, P={proj}) bf16, chunk {chunk}"}
+    del Bm, Cm, z, table
+    # the call of the reference's own Mamba2 module (src/ssm/modules/mamba2.py:189-199): B, C, A, D are (H, P)
+    # parameters, no gate, float32 activations (the module promotes half to float32); bf16 activations beside it
+    Ap = -(torch.rand(heads, proj, generator=g) * 15 + 1).cuda()
+    Bp, Cp = torch.randn(heads, proj, generator=g).cuda(), torch.randn(heads, proj, generator=g).cuda()
+    Dp = torch.ones(heads, proj).cuda()
+    for name, dtype in (("module_call_fp32", torch.float32), ("module_call_bf16", torch.bfloat16)):
+        Xm, gm = X.to(dtype), gy.to(dtype)
+        f = _time_us(lambda i: ops._dscan_forward(Xm, dt, Ap, Bp, Cp, chunk, Dp, None, None, None, want_round_states=True),
+                     iters=10)
+        _, table = ops._dscan_forward(Xm, dt, Ap, Bp, Cp, chunk, Dp, None, None, None, want_round_states=True)
+        b = _time_us(lambda i: ops._dscan_backward(gm, Xm, dt, Ap, Bp, Cp, chunk, Dp, None, None, None,
+                                                   grads_in_input_dtype=True, round_states=table), iters=10)
+        e = Xm.element_size()
+        fb = el * e * 2 + batch * length * heads * 4 + table.numel() * 4       # X in, Y out; dt; the table out
+        bb = el * e * 3 + batch * length * heads * 8 + table.numel() * 4       # X, grad_y in, dX out; dt, ddt; the table in
+        out[name] = {"fwd_us": round(f, 1), "fwd_frac_hbm": round(fb / f / 1e3 / HBM_PEAK_GBPS, 4),
+                     "bwd_us": round(b, 1), "bwd_frac_hbm": round(bb / b / 1e3 / HBM_PEAK_GBPS, 4)}
+    return out
 
 
 def bench_decode(batch=64, dim=5120, nstate=16, width=4, steps=512):

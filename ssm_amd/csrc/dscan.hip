@@ -164,10 +164,14 @@ struct DoRegs {
 
 // STATES_ONLY: the walk without C, the gate and the output -- only the table of round states is written (the
 // backward's own forward sweep when it is called without one).
-template <typename io_t, int VEC, bool HAS_Z, bool STATES_ONLY>
+// PARAMS: the call of the reference's own Mamba2 module (src/ssm/modules/mamba2.py:189-199): B and C are
+// parameters, one value per channel ((H,P), or (B,H,P)), kept in registers instead of streamed, and A and D may be
+// per channel, so every channel of a lane has its own decay (one per lane otherwise).
+template <typename io_t, int VEC, bool HAS_Z, bool STATES_ONLY, bool PARAMS>
 __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const DscanParams p) {
   static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
-  __shared__ float4 segs[2][DO_WAVES][WAVE];
+  constexpr int AV = PARAMS ? VEC : 1;            // decays per lane
+  __shared__ float4 segs[2][DO_WAVES][WAVE];     // a wave's fold per lane: decay product(s), state(s) from zero
   __shared__ float2 right[2][WAVE];
   const int wave = wave_id_uniform(), lane = lane_id();
   const int HP = p.heads * p.proj;
@@ -176,12 +180,22 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
   const int h = (int)ch / p.proj;
   const int L = p.len;
   const int valid = p.lengths ? min(max(p.lengths[b], 0), L) : L;
-  const float A2 = p.A[h] * LOG2E;
-  const float Dk = p.Dk ? p.Dk[h] : 0.0f;
+  float A2[AV], Dk[AV], Bc[VEC], Cc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    if (v < AV) {     // per channel (index h*P + p = ch + v) or per head
+      A2[v] = p.A[p.a_stride_p ? (size_t)ch + v : (size_t)h] * LOG2E;
+      Dk[v] = p.Dk ? p.Dk[p.d_stride_p ? (size_t)ch + v : (size_t)h] : 0.0f;
+    }
+    // constant projections: element strides b_stride_b / c_stride_b are 0 for (H,P) and H*P for (B,H,P)
+    Bc[v] = PARAMS ? load_as_f32(p.Bp, p.bc_dtype, (size_t)b * p.b_stride_b + ch + v) : 0.0f;
+    Cc[v] = PARAMS ? load_as_f32(p.Cp, p.bc_dtype, (size_t)b * p.c_stride_b + ch + v) : 0.0f;
+  }
   // the batch row's part of every tensor: offsets inside it fit 32 bits (checked by the host)
   const size_t row0 = (size_t)b * L;
-  const io_t *X = reinterpret_cast<const io_t *>(p.X) + row0 * HP, *Bp = reinterpret_cast<const io_t *>(p.Bp) + row0 * HP;
-  const io_t *Cp = reinterpret_cast<const io_t *>(p.Cp) + row0 * HP, *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.X) + row0 * HP;
+  const io_t *X = reinterpret_cast<const io_t *>(p.X) + row0 * HP;
+  const io_t *Bp = reinterpret_cast<const io_t *>(PARAMS ? p.X : p.Bp) + row0 * HP, *Cp = reinterpret_cast<const io_t *>(PARAMS ? p.X : p.Cp) + row0 * HP;
+  const io_t *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.X) + row0 * HP;
   const float *DT = reinterpret_cast<const float *>(p.dt) + row0 * p.heads;
   io_t *Y = reinterpret_cast<io_t *>(p.Y) + row0 * HP;
 
@@ -193,8 +207,8 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
       const unsigned at = (row * (unsigned)HP + ch) * (unsigned)sizeof(io_t);
       r.dt[j] = *at_bytes<const float>(DT, (row * (unsigned)p.heads + (unsigned)h) * 4u);
       r.x[j] = Word<io_t>{*at_bytes<const unsigned>(X, at)};
-      r.bq[j] = Word<io_t>{*at_bytes<const unsigned>(Bp, at)};
-      if (!STATES_ONLY) r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
+      if (!PARAMS) r.bq[j] = Word<io_t>{*at_bytes<const unsigned>(Bp, at)};
+      if (!STATES_ONLY && !PARAMS) r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
       if (HAS_Z && !STATES_ONLY) r.zq[j] = Word<io_t>{*at_bytes<const unsigned>(Z, at)};
     }
   };
@@ -211,22 +225,27 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
         const bool live = t0 + j < valid;
         cur.dt[j] = live ? cur.dt[j] : 0.0f;
         cur.x[j].mask(live);
-        cur.bq[j].mask(live);
-        if (!STATES_ONLY) cur.cq[j].mask(live);
+        if (!PARAMS) cur.bq[j].mask(live);
+        if (!STATES_ONLY && !PARAMS) cur.cq[j].mask(live);
       }
     }
-    float a[DO_SEG], s[VEC], prod = 1.0f;
+    float a[AV][DO_SEG], s[VEC], prod[AV];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) s[v] = 0.0f;
 #pragma unroll
+    for (int v = 0; v < AV; ++v) prod[v] = 1.0f;
+#pragma unroll
     for (int j = 0; j < DO_SEG; ++j) {
-      a[j] = exp2_hw(cur.dt[j] * A2);
-      prod *= a[j];
+#pragma unroll
+      for (int v = 0; v < AV; ++v) {
+        a[v][j] = exp2_hw(cur.dt[j] * A2[v]);
+        prod[v] *= a[v][j];
+      }
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
-        s[v] = __builtin_fmaf(a[j], s[v], cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v));
+        s[v] = __builtin_fmaf(a[v % AV][j], s[v], cur.dt[j] * (PARAMS ? Bc[v] : cur.bq[j].elem(v)) * cur.x[j].elem(v));
     }
-    segs[q][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
+    segs[q][wave][lane] = make_float4(prod[0], prod[AV - 1], s[0], s[VEC - 1]);
     __syncthreads();
     // the state entering this wave's steps: the folds of the waves before it, from the state entering the round
     float enter[VEC];
@@ -241,12 +260,12 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
     for (int w = 0; w < wave; ++w) {
       const float4 f = segs[q][w][lane];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) enter[v] = __builtin_fmaf(f.x, enter[v], v == 0 ? f.y : f.z);
+      for (int v = 0; v < VEC; ++v) enter[v] = __builtin_fmaf(v % AV == 0 ? f.x : f.y, enter[v], v == 0 ? f.z : f.w);
     }
     if (wave == DO_WAVES - 1) {
       float leave[VEC];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) leave[v] = __builtin_fmaf(prod, enter[v], s[v]);
+      for (int v = 0; v < VEC; ++v) leave[v] = __builtin_fmaf(prod[v % AV], enter[v], s[v]);
       right[q][lane] = make_float2(leave[0], leave[VEC - 1]);
     }
     if (p.round_states && (wave & (DO_WAVES / 2 - 1)) == 0) {
@@ -266,16 +285,17 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
       // the float32 values of a step's elements are formed here, step by step, not kept from the fold above
       // and not all in front of the first step
       cur.x[j].launder_after(enter[0]);
-      cur.bq[j].launder_after(enter[0]);
-      cur.cq[j].launder_after(enter[0]);
+      if (!PARAMS) cur.bq[j].launder_after(enter[0]);
+      if (!PARAMS) cur.cq[j].launder_after(enter[0]);
       if (HAS_Z) cur.zq[j].launder_after(enter[0]);
       Pack<io_t, VEC> o;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         const float xv = cur.x[j].elem(v);
-        enter[v] = __builtin_fmaf(a[j], enter[v], cur.dt[j] * cur.bq[j].elem(v) * xv);
-        float y = __builtin_fmaf(enter[v], cur.cq[j].elem(v), Dk * xv);
+        enter[v] = __builtin_fmaf(a[v % AV][j], enter[v], cur.dt[j] * (PARAMS ? Bc[v] : cur.bq[j].elem(v)) * xv);
+        float y = __builtin_fmaf(enter[v], PARAMS ? Cc[v] : cur.cq[j].elem(v), Dk[v % AV] * xv);
         if (HAS_Z) y *= silu_f32(cur.zq[j].elem(v));
+        if (PARAMS && t >= valid) y = 0.0f;      // nothing streamed carries the zero of a dead step here
         o.v[v] = from_f32<io_t>(y);
       }
       if (t < L) *at_bytes<Pack<io_t, VEC>>(Y, ((unsigned)t * (unsigned)HP + ch) * (unsigned)sizeof(io_t)) = o;
@@ -296,25 +316,40 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
 }
 
 template <typename io_t, int VEC>
-static void launch_onepass(const DscanParams &p, hipStream_t s) {
+static void launch_onepass(const DscanParams &p, bool params, hipStream_t s) {
   const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
-  if (p.z) hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, true, false>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
-  else hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, false, false>), grid, dim3(WAVE * DO_WAVES), 0, s, p);
+  const dim3 block(WAVE * DO_WAVES);
+  if (params) {
+    if (p.z) hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, true, false, true>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, false, false, true>), grid, block, 0, s, p);
+  } else {
+    if (p.z) hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, true, false, false>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((dscan_onepass_kernel<io_t, VEC, false, false, false>), grid, block, 0, s, p);
+  }
 }
 
 // The table of round states alone, for a call shape the one-pass kernels cover (the caller has checked).
+// b_const: B is one value per channel, (H,P) (b_stride_b 0) or (B,H,P) (b_stride_b H*P), of type bc_dtype.
 void launch_dscan_round_states(const void *X, const void *dt, const void *Bproj, const float *A, const void *init,
                                int init_dtype, const int *lengths, float *round_states, int batch, int len, int heads,
-                               int proj, int x_dtype, hipStream_t s) {
+                               int proj, int x_dtype, bool b_const, int bc_dtype, long long b_stride_b, bool a_per_p,
+                               hipStream_t s) {
   DscanParams p{};
   p.X = X; p.dt = dt; p.Bp = Bproj; p.Cp = Bproj; p.A = A; p.init = init; p.init_dtype = init_dtype;
   p.lengths = lengths; p.round_states = round_states;
   p.batch = batch; p.len = len; p.heads = heads; p.proj = proj;
+  p.bc_dtype = bc_dtype; p.b_stride_b = p.c_stride_b = b_stride_b; p.a_stride_p = a_per_p ? 1 : 0;
   const int vec = x_dtype == SSM_F32 ? 1 : 2;
   const dim3 grid((unsigned)((size_t)heads * proj / (WAVE * vec)), (unsigned)batch), block(WAVE * DO_WAVES);
-  if (x_dtype == SSM_BF16) hipLaunchKernelGGL((dscan_onepass_kernel<bf16_t, 2, false, true>), grid, block, 0, s, p);
-  else if (x_dtype == SSM_F16) hipLaunchKernelGGL((dscan_onepass_kernel<f16_t, 2, false, true>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((dscan_onepass_kernel<float, 1, false, true>), grid, block, 0, s, p);
+#define SSM_STATES(T, V)                                                                                    \
+  {                                                                                                         \
+    if (b_const) hipLaunchKernelGGL((dscan_onepass_kernel<T, V, false, true, true>), grid, block, 0, s, p); \
+    else hipLaunchKernelGGL((dscan_onepass_kernel<T, V, false, true, false>), grid, block, 0, s, p);        \
+  }
+  if (x_dtype == SSM_BF16) SSM_STATES(bf16_t, 2)
+  else if (x_dtype == SSM_F16) SSM_STATES(f16_t, 2)
+  else SSM_STATES(float, 1)
+#undef SSM_STATES
 }
 
 int dscan_segments(int batch, int len, int hp) {
@@ -335,20 +370,24 @@ extern "C" size_t ssm_dscan_fwd_workspace_bytes(int batch, int seqlen, int heads
   return (size_t)batch * nseg * heads * proj * 2 * sizeof(float);
 }
 
-// One pass: per-token B and C of X's type, float32 dt, per-head A and D, a gate of X's shape or none, channels in
-// whole waves, vectors aligned.
-static bool dscan_fwd_takes_one_pass(const ssm_dscan_fwd_args *a) {
+// One pass: float32 dt, a gate of X's shape and type or none, channels in whole waves, vectors aligned, and either
+// per-token B and C of X's type with per-head A and D (*params = false), or B and C one value per channel -- (H,P)
+// or (B,H,P), any type -- with A and D per head or per channel (*params = true).
+static bool dscan_fwd_takes_one_pass(const ssm_dscan_fwd_args *a, bool *params = nullptr) {
   using namespace ssm;
-  if (!valid_dtype(a->x_dtype)) return false;
+  if (!valid_dtype(a->x_dtype) || !valid_dtype(a->bc_dtype)) return false;
   const long long HP = (long long)a->heads * a->proj;
-  const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
   const int vec = a->x_dtype == SSM_F32 ? 1 : 2;
   const size_t bytes = (size_t)vec * dtype_size(a->x_dtype);
-  return typed && a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP && !a->a_per_p && !a->d_per_p &&
-         (!a->z || a->z_per_p) && HP % (WAVE * vec) == 0 && a->proj % vec == 0 &&
-         (long long)a->seqlen * HP < (1ll << 30) && aligned_to(a->X, bytes) &&
-         aligned_to(a->Bproj, bytes) && aligned_to(a->Cproj, bytes) && aligned_to(a->Y, bytes) &&
-         (!a->z || aligned_to(a->z, bytes)) && a->batch < 65536;
+  const bool streamed = a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP && a->bc_dtype == a->x_dtype &&
+                        !a->a_per_p && !a->d_per_p && aligned_to(a->Bproj, bytes) && aligned_to(a->Cproj, bytes);
+  auto per_channel = [](int kind) { return kind == SSM_CHUNK_HP || kind == SSM_CHUNK_BHP; };
+  const bool constant = per_channel(a->b_kind) && per_channel(a->c_kind) &&
+                        aligned_to(a->Bproj, dtype_size(a->bc_dtype)) && aligned_to(a->Cproj, dtype_size(a->bc_dtype));
+  if (params) *params = constant;
+  return (streamed || constant) && a->dt_dtype == SSM_F32 && (!a->z || (a->z_dtype == a->x_dtype && a->z_per_p)) &&
+         HP % (WAVE * vec) == 0 && a->proj % vec == 0 && (long long)a->seqlen * HP < (1ll << 30) &&
+         aligned_to(a->X, bytes) && aligned_to(a->Y, bytes) && (!a->z || aligned_to(a->z, bytes)) && a->batch < 65536;
 }
 
 extern "C" int ssm_dscan_fwd_one_pass(const ssm_dscan_fwd_args *a) {
@@ -400,14 +439,15 @@ extern "C" int ssm_dscan_fwd(const ssm_dscan_fwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid((unsigned)((HP + DS_THREADS - 1) / DS_THREADS), (unsigned)p.nseg, (unsigned)a->batch);
   const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
-  const bool one_pass = dscan_fwd_takes_one_pass(a);
+  bool params = false;
+  const bool one_pass = dscan_fwd_takes_one_pass(a, &params);
   SSM_REQUIRE(!a->round_states || (one_pass && aligned_to(a->round_states, 4)), SSM_ERR_BAD_SHAPE,
               "ssm_dscan_fwd: round_states is only written by the one-pass kernel (ask ssm_dscan_fwd_one_pass first)");
   if (one_pass) {
     p.round_states = a->round_states;
-    if (a->x_dtype == SSM_BF16) launch_onepass<bf16_t, 2>(p, s);
-    else if (a->x_dtype == SSM_F16) launch_onepass<f16_t, 2>(p, s);
-    else launch_onepass<float, 1>(p, s);
+    if (a->x_dtype == SSM_BF16) launch_onepass<bf16_t, 2>(p, params, s);
+    else if (a->x_dtype == SSM_F16) launch_onepass<f16_t, 2>(p, params, s);
+    else launch_onepass<float, 1>(p, params, s);
     SSM_CHECK_LAUNCH("ssm_dscan_fwd");
     return SSM_OK;
   }

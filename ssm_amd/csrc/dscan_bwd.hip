@@ -28,7 +28,8 @@ int dscan_segments(int batch, int len, int hp);   // dscan.hip: the forward's ch
 // dscan.hip: the forward's one-pass walk reduced to the table of the states entering every 64 steps
 void launch_dscan_round_states(const void *X, const void *dt, const void *Bproj, const float *A, const void *init,
                                int init_dtype, const int *lengths, float *round_states, int batch, int len, int heads,
-                               int proj, int x_dtype, hipStream_t s);
+                               int proj, int x_dtype, bool b_const, int bc_dtype, long long b_stride_b, bool a_per_p,
+                               hipStream_t s);
 
 struct DscanBwdParams {
   const void *gy, *X, *dt, *Bp, *Cp, *z, *init;
@@ -347,32 +348,57 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   const dim3 grid((unsigned)((HP + DB_THREADS - 1) / DB_THREADS), (unsigned)nseg, (unsigned)Bn);
   const bool typed = a->dt_dtype == SSM_F32 && a->bc_dtype == a->x_dtype && (!a->z || a->z_dtype == a->x_dtype);
-  // one pass: per-token B and C, per-head A and D, a gate of X's shape or none, a head's channels in 16, 32 or 64 lanes
+  // one pass: float32 dt, a gate of X's shape and type or none, a head's channels in 16, 32 or 64 lanes, and either
+  // per-token B and C of X's type with per-head A and D, or B and C one value per channel (any type, gradients in
+  // float32) with A and D per head or per channel
   const int vec = a->x_dtype == SSM_F32 ? 1 : 2;
   const size_t vbytes = (size_t)vec * dtype_size(a->x_dtype);
   const size_t gbytes = grads_io ? vbytes : (size_t)vec * 4;
   const int lph = P % vec == 0 ? P / vec : 0;
-  const bool onepass = a->tune_two_kernels == 0 && typed && a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP &&
-                       !a->a_per_p && !a->d_per_p && (!a->z || a->z_per_p) && (lph == 16 || lph == 32 || lph == 64) &&
-                       HP % (WAVE * vec) == 0 && (size_t)L * HP < ((size_t)1 << 30) && aligned_to(a->X, vbytes) && aligned_to(a->grad_y, vbytes) &&
-                       aligned_to(a->Bproj, vbytes) && aligned_to(a->Cproj, vbytes) && aligned_to(a->dX, vbytes) &&
-                       (!a->z || aligned_to(a->z, vbytes)) && aligned_to(a->dB, gbytes) && aligned_to(a->dC, gbytes) &&
-                       (!a->z || aligned_to(a->dz, gbytes));
+  const bool streamed = a->b_kind == SSM_CHUNK_BLHP && a->c_kind == SSM_CHUNK_BLHP && a->bc_dtype == a->x_dtype &&
+                        !a->a_per_p && !a->d_per_p && aligned_to(a->Bproj, vbytes) && aligned_to(a->Cproj, vbytes) &&
+                        aligned_to(a->dB, gbytes) && aligned_to(a->dC, gbytes);
+  const bool constant = a->b_kind != SSM_CHUNK_BLHP && a->c_kind != SSM_CHUNK_BLHP &&
+                        aligned_to(a->Bproj, dtype_size(a->bc_dtype)) && aligned_to(a->Cproj, dtype_size(a->bc_dtype)) &&
+                        aligned_to(a->dB, 4) && aligned_to(a->dC, 4);
+  const bool onepass = a->tune_two_kernels == 0 && (streamed || constant) && a->dt_dtype == SSM_F32 &&
+                       (!a->z || (a->z_dtype == a->x_dtype && a->z_per_p)) && (lph == 16 || lph == 32 || lph == 64) &&
+                       HP % (WAVE * vec) == 0 && (size_t)L * HP < ((size_t)1 << 30) && aligned_to(a->X, vbytes) &&
+                       aligned_to(a->grad_y, vbytes) && aligned_to(a->dX, vbytes) &&
+                       (!a->z || (aligned_to(a->z, vbytes) && aligned_to(a->dz, gbytes)));
   if (onepass) {
     const int rounds = (L + DBO_ROUND - 1) / DBO_ROUND;
     p.round_states = a->round_states ? const_cast<float *>(a->round_states) : ws;
-    p.pA = ws + (size_t)Bn * rounds * HP;
-    p.pD = p.pA + bhp;
+    // per-channel sums of a batch row, (B, HP) each; those that are the caller's gradient already go there
+    float *sums = ws + (size_t)Bn * rounds * HP;
+    p.pA = sums;
+    p.pD = sums + bhp;
+    p.pB = (constant && a->b_kind == SSM_CHUNK_BHP) ? reinterpret_cast<float *>(a->dB) : sums + 2 * bhp;
+    p.pC = (constant && a->c_kind == SSM_CHUNK_BHP) ? reinterpret_cast<float *>(a->dC) : sums + 3 * bhp;
+    float *head_tmp = sums + 4 * bhp;                      // (HP) on the way to a per-head sum
     p.ddt_direct = a->ddt;
-    nseg = 1;
     if (a->round_states == nullptr)                      // no table from the forward: make it
       launch_dscan_round_states(a->X, a->dt, a->Bproj, a->A, a->initial_states, a->init_dtype, a->seq_lens, ws, Bn, L, H,
-                                P, a->x_dtype, s);
-    if (a->x_dtype == SSM_BF16) launch_bwd_onepass<bf16_t, 2>(p, grads_io, s);
-    else if (a->x_dtype == SSM_F16) launch_bwd_onepass<f16_t, 2>(p, grads_io, s);
-    else launch_bwd_onepass<float, 1>(p, grads_io, s);
+                                P, a->x_dtype, constant, a->bc_dtype, p.b_stride_b, a->a_per_p != 0, s);
+    if (a->x_dtype == SSM_BF16) launch_bwd_onepass<bf16_t, 2>(p, grads_io, constant, s);
+    else if (a->x_dtype == SSM_F16) launch_bwd_onepass<f16_t, 2>(p, grads_io, constant, s);
+    else launch_bwd_onepass<float, 1>(p, grads_io, constant, s);
     SSM_CHECK_LAUNCH("ssm_dscan_bwd");
-    hipLaunchKernelGGL(dscan_bwd_head_sums_kernel, dim3(H), dim3(WAVE), 0, s, p.pA, p.pD, a->dA, a->dD, Bn, H, P);
+    if (!a->a_per_p && !a->d_per_p) {
+      hipLaunchKernelGGL(dscan_bwd_head_sums_kernel, dim3(H), dim3(WAVE), 0, s, p.pA, p.pD, a->dA, a->dD, Bn, H, P);
+    } else {
+      auto param_sum = [&](const float *partial, float *out, bool per_p) {
+        if (per_p) launch_fold_rows(partial, out, Bn, (size_t)HP, s);
+        else {
+          launch_fold_rows(partial, head_tmp, Bn, (size_t)HP, s);
+          launch_fold_sum(head_tmp, out, (size_t)H, P, 1, s);
+        }
+      };
+      param_sum(p.pA, a->dA, a->a_per_p != 0);
+      if (a->dD) param_sum(p.pD, a->dD, a->d_per_p != 0);
+    }
+    if (constant && a->b_kind == SSM_CHUNK_HP) launch_fold_rows(p.pB, reinterpret_cast<float *>(a->dB), Bn, (size_t)HP, s);
+    if (constant && a->c_kind == SSM_CHUNK_HP) launch_fold_rows(p.pC, reinterpret_cast<float *>(a->dC), Bn, (size_t)HP, s);
     SSM_CHECK_LAUNCH("ssm_dscan_bwd(sums)");
     return SSM_OK;
   } else {

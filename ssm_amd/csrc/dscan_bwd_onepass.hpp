@@ -1,6 +1,8 @@
-// Backward of the diagonal chunked scan for the common call (per-token B and C of X's shape and type,
-// float32 dt, per-head A and D, a gate of X's shape or none, a head's channels in 16, 32 or 64 lanes):
-// every input is read once by the kernel that forms the gradients, no state goes through memory.
+// Backward of the diagonal chunked scan for the two common calls (float32 dt, a gate of X's shape or none, a
+// head's channels in 16, 32 or 64 lanes): per-token B and C of X's shape and type with per-head A and D, or
+// (PARAMS) B and C one value per channel -- parameters, as the reference's Mamba2 module passes them,
+// src/ssm/modules/mamba2.py:189-199 -- with A and D per head or per channel.
+// Every input is read once by the kernel that forms the gradients, no state goes through memory.
 //
 // A workgroup of 16 waves owns 64 * VEC neighbouring channels of one batch row and walks time backwards in
 // rounds of 64 steps, wave w taking steps 4w..4w+3 of the round.  In a round every wave folds its steps twice
@@ -40,10 +42,13 @@ struct DboRegs {
 };
 
 // g_t: element type of dB, dC and dz (io_t, or float).  LPH: lanes that hold one head's channels.
-template <typename io_t, typename g_t, int VEC, bool HAS_Z, int LPH>
-__global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
+// PARAMS: B and C are held in registers, one value per channel, and their gradients are sums over time like dA's
+// and dD's; each channel of a lane has its own decay.
+template <typename io_t, typename g_t, int VEC, bool HAS_Z, int LPH, bool PARAMS>
+__global__ __launch_bounds__(WAVE *DBO_WAVES, (PARAMS && !HAS_Z && VEC == 1) ? 8 : 4) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
   static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
-  __shared__ float4 fwd[2][DBO_WAVES][WAVE];     // a wave's four steps per lane: decay product, state from zero (per channel)
+  constexpr int AV = PARAMS ? VEC : 1;            // decays per lane
+  __shared__ float4 fwd[2][DBO_WAVES][WAVE];     // a wave's four steps per lane: decay product(s), state(s) from zero
   __shared__ float2 rev[2][DBO_WAVES][WAVE];     // ... and the adjoint (times its decay) from zero
   __shared__ float2 left[2][WAVE];               // the adjoint leaving the round, from wave 0 to everyone's next round
   const int wave = wave_id_uniform(), lane = lane_id();
@@ -53,17 +58,28 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
   const int h = (int)ch / p.proj;
   const int L = p.len;
   const int valid = p.lengths ? min(max(p.lengths[b], 0), L) : L;
-  const float A = p.A[h], A2 = A * LOG2E;
-  const float Dk = p.Dk ? p.Dk[h] : 0.0f;
+  float A[AV], A2[AV], Dk[AV], Bc[VEC], Cc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    if (v < AV) {     // per channel (index h*P + p = ch + v) or per head
+      A[v] = p.A[p.a_stride_p ? (size_t)ch + v : (size_t)h];
+      A2[v] = A[v] * LOG2E;
+      Dk[v] = p.Dk ? p.Dk[p.d_stride_p ? (size_t)ch + v : (size_t)h] : 0.0f;
+    }
+    // constant projections: element strides b_stride_b / c_stride_b are 0 for (H,P) and H*P for (B,H,P)
+    Bc[v] = PARAMS ? load_as_f32(p.Bp, p.bc_dtype, (size_t)b * p.b_stride_b + ch + v) : 0.0f;
+    Cc[v] = PARAMS ? load_as_f32(p.Cp, p.bc_dtype, (size_t)b * p.c_stride_b + ch + v) : 0.0f;
+  }
   // the batch row's part of every tensor: offsets inside it fit 32 bits (checked by the host)
   const size_t row0 = (size_t)b * L;
-  const io_t *X = reinterpret_cast<const io_t *>(p.X) + row0 * HP, *Bp = reinterpret_cast<const io_t *>(p.Bp) + row0 * HP;
-  const io_t *Cp = reinterpret_cast<const io_t *>(p.Cp) + row0 * HP, *G = reinterpret_cast<const io_t *>(p.gy) + row0 * HP;
+  const io_t *X = reinterpret_cast<const io_t *>(p.X) + row0 * HP, *G = reinterpret_cast<const io_t *>(p.gy) + row0 * HP;
+  const io_t *Bp = reinterpret_cast<const io_t *>(PARAMS ? p.X : p.Bp) + row0 * HP;
+  const io_t *Cp = reinterpret_cast<const io_t *>(PARAMS ? p.X : p.Cp) + row0 * HP;
   const io_t *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.X) + row0 * HP;
   const float *DT = reinterpret_cast<const float *>(p.dt) + row0 * p.heads;
   io_t *dX = reinterpret_cast<io_t *>(p.dX) + row0 * HP;
-  g_t *dB = reinterpret_cast<g_t *>(p.dB_t) + row0 * HP, *dC = reinterpret_cast<g_t *>(p.dC_t) + row0 * HP;
-  g_t *dZ = reinterpret_cast<g_t *>(HAS_Z ? p.dz_p : p.dB_t) + row0 * HP;
+  g_t *dB = reinterpret_cast<g_t *>(PARAMS ? p.dX : p.dB_t) + row0 * HP, *dC = reinterpret_cast<g_t *>(PARAMS ? p.dX : p.dC_t) + row0 * HP;
+  g_t *dZ = reinterpret_cast<g_t *>(HAS_Z ? p.dz_p : p.dX) + row0 * HP;
   float *DDT = p.ddt_direct + row0 * p.heads;
   const int rounds = (L + DBO_ROUND - 1) / DBO_ROUND;
   const float *table = p.round_states + (size_t)b * rounds * HP;
@@ -76,8 +92,8 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
       const unsigned at = (row * (unsigned)HP + ch) * (unsigned)sizeof(io_t);
       r.dt[j] = *at_bytes<const float>(DT, (row * (unsigned)p.heads + (unsigned)h) * 4u);
       r.x[j] = Word<io_t>{*at_bytes<const unsigned>(X, at)};
-      r.bq[j] = Word<io_t>{*at_bytes<const unsigned>(Bp, at)};
-      r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
+      if (!PARAMS) r.bq[j] = Word<io_t>{*at_bytes<const unsigned>(Bp, at)};
+      if (!PARAMS) r.cq[j] = Word<io_t>{*at_bytes<const unsigned>(Cp, at)};
       r.gq[j] = Word<io_t>{*at_bytes<const unsigned>(G, at)};
       if (HAS_Z) r.zq[j] = Word<io_t>{*at_bytes<const unsigned>(Z, at)};
     }
@@ -85,31 +101,36 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
     for (int v = 0; v < VEC; ++v) r.enter[v] = *at_bytes<const float>(table, ((unsigned)round * (unsigned)HP + ch + v) * 4u);
   };
 
-  float accA[VEC], accD[VEC], mu_left[VEC];
+  float accA[VEC], accD[VEC], accB[VEC], accC[VEC], mu_left[VEC];
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) accA[v] = accD[v] = mu_left[v] = 0.0f;
+  for (int v = 0; v < VEC; ++v) accA[v] = accD[v] = accB[v] = accC[v] = mu_left[v] = 0.0f;
 
   auto round_of = [&](DboRegs<io_t, VEC, HAS_Z> &cur, int r) {
     const int q = r & 1;
     const int t0 = r * DBO_ROUND + wave * DBO_SEG;
-    float a[DBO_SEG], sg[VEC][DBO_SEG];
-    float s[VEC], M[VEC], prod = 1.0f;
+    float a[AV][DBO_SEG], sg[VEC][DBO_SEG];
+    float s[VEC], M[VEC], prod[AV];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) s[v] = M[v] = 0.0f;
+#pragma unroll
+    for (int v = 0; v < AV; ++v) prod[v] = 1.0f;
 #pragma unroll
     for (int j = 0; j < DBO_SEG; ++j) {
       const bool live = t0 + j < valid;
       cur.dt[j] = live ? cur.dt[j] : 0.0f;
       cur.x[j].mask(live);
-      cur.bq[j].mask(live);
-      cur.cq[j].mask(live);
+      if (!PARAMS) cur.bq[j].mask(live);
+      if (!PARAMS) cur.cq[j].mask(live);
       cur.gq[j].mask(live);
       if (HAS_Z) cur.zq[j].mask(live);
-      a[j] = exp2_hw(cur.dt[j] * A2);
-      prod *= a[j];
+#pragma unroll
+      for (int v = 0; v < AV; ++v) {
+        a[v][j] = exp2_hw(cur.dt[j] * A2[v]);
+        prod[v] *= a[v][j];
+      }
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
-        s[v] = __builtin_fmaf(a[j], s[v], cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v));
+        s[v] = __builtin_fmaf(a[v % AV][j], s[v], cur.dt[j] * (PARAMS ? Bc[v] : cur.bq[j].elem(v)) * cur.x[j].elem(v));
     }
 #pragma unroll
     for (int j = DBO_SEG - 1; j >= 0; --j) {
@@ -121,17 +142,17 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
           sg[v][j] = sigmoid_f32(zz);
           g0 *= zz * sg[v][j];
         }
-        M[v] = a[j] * __builtin_fmaf(g0, cur.cq[j].elem(v), M[v]);
+        M[v] = a[v % AV][j] * __builtin_fmaf(g0, PARAMS ? Cc[v] : cur.cq[j].elem(v), M[v]);
       }
     }
-    fwd[q][wave][lane] = make_float4(prod, s[0], s[VEC - 1], 0.0f);
+    fwd[q][wave][lane] = make_float4(prod[0], prod[AV - 1], s[0], s[VEC - 1]);
     rev[q][wave][lane] = make_float2(M[0], M[VEC - 1]);
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < DBO_SEG; ++j) {
       cur.x[j].launder();
-      cur.bq[j].launder();
-      cur.cq[j].launder();
+      if (!PARAMS) cur.bq[j].launder();
+      if (!PARAMS) cur.cq[j].launder();
       cur.gq[j].launder();
       if (HAS_Z) cur.zq[j].launder();
     }
@@ -142,7 +163,7 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
     for (int w = 0; w < wave; ++w) {
       const float4 f = fwd[q][w][lane];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) st[v][0] = __builtin_fmaf(f.x, st[v][0], v == 0 ? f.y : f.z);
+      for (int v = 0; v < VEC; ++v) st[v][0] = __builtin_fmaf(v % AV == 0 ? f.x : f.y, st[v][0], v == 0 ? f.z : f.w);
     }
     // the adjoint entering them: the folds of the waves after it, from the adjoint that left the round before
     float mu[VEC];
@@ -154,14 +175,14 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
 #pragma unroll
     for (int v = 0; v < VEC; ++v) mu[v] = mu_left[v];
     for (int w = DBO_WAVES - 1; w > wave; --w) {
-      const float pr = fwd[q][w][lane].x;
+      const float2 pr = *reinterpret_cast<const float2 *>(&fwd[q][w][lane]);      // the decay products
       const float2 f = rev[q][w][lane];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) mu[v] = __builtin_fmaf(pr, mu[v], v == 0 ? f.x : f.y);
+      for (int v = 0; v < VEC; ++v) mu[v] = __builtin_fmaf(v % AV == 0 ? pr.x : pr.y, mu[v], v == 0 ? f.x : f.y);
     }
     if (wave == 0) {
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) mu_left[v] = __builtin_fmaf(prod, mu[v], M[v]);
+      for (int v = 0; v < VEC; ++v) mu_left[v] = __builtin_fmaf(prod[v % AV], mu[v], M[v]);
       left[q][lane] = make_float2(mu_left[0], mu_left[VEC - 1]);
     }
     // forward replay: st[v][j + 1] = the state after step j
@@ -169,7 +190,7 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
     for (int j = 0; j < DBO_SEG; ++j) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
-        st[v][j + 1] = __builtin_fmaf(a[j], st[v][j], cur.dt[j] * cur.bq[j].elem(v) * cur.x[j].elem(v));
+        st[v][j + 1] = __builtin_fmaf(a[v % AV][j], st[v][j], cur.dt[j] * (PARAMS ? Bc[v] : cur.bq[j].elem(v)) * cur.x[j].elem(v));
     }
     // backward replay; mu[v] is lambda_{t+1} a_{t+1}
 #pragma unroll
@@ -177,8 +198,8 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
       const int t = t0 + j;
       // a step's float32 values are formed at the step, not all in front of the loop
       cur.x[j].launder_after(mu[0]);
-      cur.bq[j].launder_after(mu[0]);
-      cur.cq[j].launder_after(mu[0]);
+      if (!PARAMS) cur.bq[j].launder_after(mu[0]);
+      if (!PARAMS) cur.cq[j].launder_after(mu[0]);
       cur.gq[j].launder_after(mu[0]);
       if (HAS_Z) cur.zq[j].launder_after(mu[0]);
       Pack<io_t, VEC> ox;
@@ -186,31 +207,37 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
       float ddt = 0.0f;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        const float xv = cur.x[j].elem(v), bv = cur.bq[j].elem(v), cv = cur.cq[j].elem(v);
+        const float xv = cur.x[j].elem(v), bv = PARAMS ? Bc[v] : cur.bq[j].elem(v), cv = PARAMS ? Cc[v] : cur.cq[j].elem(v);
+        const float Av = A[v % AV], Dv = Dk[v % AV], av = a[v % AV][j];
         float g0 = cur.gq[j].elem(v);
         if (HAS_Z) {
           const float zz = cur.zq[j].elem(v);
-          const float y0 = __builtin_fmaf(st[v][j + 1], cv, Dk * xv);
+          const float y0 = __builtin_fmaf(st[v][j + 1], cv, Dv * xv);
           oz.v[v] = from_f32<g_t>(g0 * y0 * sg[v][j] * __builtin_fmaf(zz, 1.0f - sg[v][j], 1.0f));
           g0 *= zz * sg[v][j];
         }
         const float lam = __builtin_fmaf(g0, cv, mu[v]);
         const float ld = lam * cur.dt[j];
-        ox.v[v] = from_f32<io_t>(__builtin_fmaf(g0, Dk, ld * bv));
-        ob.v[v] = from_f32<g_t>(ld * xv);
-        oc.v[v] = from_f32<g_t>(g0 * st[v][j + 1]);
-        const float sa = st[v][j] * a[j];
-        ddt = __builtin_fmaf(lam, __builtin_fmaf(sa, A, bv * xv), ddt);
+        ox.v[v] = from_f32<io_t>(__builtin_fmaf(g0, Dv, ld * bv));
+        if (PARAMS) {
+          accB[v] = __builtin_fmaf(ld, xv, accB[v]);
+          accC[v] = __builtin_fmaf(g0, st[v][j + 1], accC[v]);
+        } else {
+          ob.v[v] = from_f32<g_t>(ld * xv);
+          oc.v[v] = from_f32<g_t>(g0 * st[v][j + 1]);
+        }
+        const float sa = st[v][j] * av;
+        ddt = __builtin_fmaf(lam, __builtin_fmaf(sa, Av, bv * xv), ddt);
         accA[v] = __builtin_fmaf(lam * sa, cur.dt[j], accA[v]);
         accD[v] = __builtin_fmaf(g0, xv, accD[v]);
-        mu[v] = lam * a[j];
+        mu[v] = lam * av;
       }
       const float head = lane_group_sum_last<LPH>(ddt);
       if (t < L) {
         const unsigned at = (unsigned)t * (unsigned)HP + ch;
         *at_bytes<Pack<io_t, VEC>>(dX, at * (unsigned)sizeof(io_t)) = ox;
-        *at_bytes<Pack<g_t, VEC>>(dB, at * (unsigned)sizeof(g_t)) = ob;
-        *at_bytes<Pack<g_t, VEC>>(dC, at * (unsigned)sizeof(g_t)) = oc;
+        if (!PARAMS) *at_bytes<Pack<g_t, VEC>>(dB, at * (unsigned)sizeof(g_t)) = ob;
+        if (!PARAMS) *at_bytes<Pack<g_t, VEC>>(dC, at * (unsigned)sizeof(g_t)) = oc;
         if (HAS_Z) *at_bytes<Pack<g_t, VEC>>(dZ, at * (unsigned)sizeof(g_t)) = oz;
         if ((lane & (LPH - 1)) == LPH - 1) *at_bytes<float>(DDT, ((unsigned)t * (unsigned)p.heads + (unsigned)h) * 4u) = head;
       }
@@ -231,26 +258,25 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(cons
 
   // sums over time of the whole walk: the 16 waves' shares meet in LDS (after everyone has left the last round)
   __syncthreads();
-  float *red = reinterpret_cast<float *>(&fwd[0][0][0]);        // [2 VEC][16][64] floats fit the first buffer
-  static_assert(2 * VEC <= 4, "the sums fit the buffer of one round's folds");
+  constexpr int SUMS = PARAMS ? 4 : 2;                          // per channel: A, D (and B, C)
+  float *red = reinterpret_cast<float *>(&fwd[0][0][0]);        // [SUMS VEC][16][64] floats
+  static_assert(SUMS * VEC * DBO_WAVES * WAVE * sizeof(float) <= sizeof(fwd), "the sums fit the buffers of the folds");
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
-    red[((2 * v) * DBO_WAVES + wave) * WAVE + lane] = accA[v];
-    red[((2 * v + 1) * DBO_WAVES + wave) * WAVE + lane] = accD[v];
+    const float mine[4] = {accA[v], accD[v], accB[v], accC[v]};
+#pragma unroll
+    for (int k = 0; k < SUMS; ++k) red[((SUMS * v + k) * DBO_WAVES + wave) * WAVE + lane] = mine[k];
   }
   __syncthreads();
-  if (wave == 0) {
+  if (wave < SUMS) {                                             // wave k adds the k-th sum
+    float *const out[4] = {p.pA, p.pD, p.pB, p.pC};
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      float sa = 0.0f, sd = 0.0f;
+      float sum = 0.0f;
 #pragma unroll
-      for (int w = 0; w < DBO_WAVES; ++w) {
-        sa += red[((2 * v) * DBO_WAVES + w) * WAVE + lane];
-        sd += red[((2 * v + 1) * DBO_WAVES + w) * WAVE + lane];
-      }
-      p.pA[(size_t)b * HP + ch + v] = sa;
-      p.pD[(size_t)b * HP + ch + v] = sd;
-      if (p.dinit) p.dinit[(size_t)b * HP + ch + v] = mu_left[v];     // lambda_0 a_0
+      for (int w = 0; w < DBO_WAVES; ++w) sum += red[((SUMS * v + wave) * DBO_WAVES + w) * WAVE + lane];
+      out[wave][(size_t)b * HP + ch + v] = sum;
+      if (wave == 0 && p.dinit) p.dinit[(size_t)b * HP + ch + v] = mu_left[v];     // lambda_0 a_0
     }
   }
 }
@@ -276,25 +302,30 @@ __global__ __launch_bounds__(WAVE) void dscan_bwd_head_sums_kernel(const float *
   }
 }
 
-template <typename io_t, typename g_t, int VEC, bool HAS_Z>
+template <typename io_t, typename g_t, int VEC, bool HAS_Z, bool PARAMS>
 static void launch_dbo_lph(const DscanBwdParams &p, int lph, hipStream_t s) {
   const dim3 grid((unsigned)((size_t)p.heads * p.proj / (WAVE * VEC)), (unsigned)p.batch);
   const dim3 block(WAVE * DBO_WAVES);
-  if (lph == 16) hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 16>), grid, block, 0, s, p);
-  else if (lph == 32) hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 32>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 64>), grid, block, 0, s, p);
+  if (lph == 16) hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 16, PARAMS>), grid, block, 0, s, p);
+  else if (lph == 32) hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 32, PARAMS>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((dscan_bwd_onepass_kernel<io_t, g_t, VEC, HAS_Z, 64, PARAMS>), grid, block, 0, s, p);
 }
 
-// The one-pass backward for one element type.
+// The one-pass backward for one element type.  params: B and C are per-channel constants (their gradients and dz
+// then are the only ones whose type grads_io chooses, and without a gate none is).
 template <typename io_t, int VEC>
-static void launch_bwd_onepass(const DscanBwdParams &p, bool grads_io, hipStream_t s) {
+static void launch_bwd_onepass(const DscanBwdParams &p, bool grads_io, bool params, hipStream_t s) {
   const int lph = p.proj / VEC;
-  if (grads_io) {
-    if (p.z) launch_dbo_lph<io_t, io_t, VEC, true>(p, lph, s);
-    else launch_dbo_lph<io_t, io_t, VEC, false>(p, lph, s);
+  if (params) {
+    if (!p.z) launch_dbo_lph<io_t, io_t, VEC, false, true>(p, lph, s);
+    else if (grads_io) launch_dbo_lph<io_t, io_t, VEC, true, true>(p, lph, s);
+    else launch_dbo_lph<io_t, float, VEC, true, true>(p, lph, s);
+  } else if (grads_io) {
+    if (p.z) launch_dbo_lph<io_t, io_t, VEC, true, false>(p, lph, s);
+    else launch_dbo_lph<io_t, io_t, VEC, false, false>(p, lph, s);
   } else {
-    if (p.z) launch_dbo_lph<io_t, float, VEC, true>(p, lph, s);
-    else launch_dbo_lph<io_t, float, VEC, false>(p, lph, s);
+    if (p.z) launch_dbo_lph<io_t, float, VEC, true, false>(p, lph, s);
+    else launch_dbo_lph<io_t, float, VEC, false, false>(p, lph, s);
   }
 }
 

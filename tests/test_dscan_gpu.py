@@ -269,3 +269,72 @@ def test_one_pass_backward_call_shape(dtype, hp, length, z_mode, d_mode, init, r
         assert auto[key].dtype == inp[key].dtype and auto[key].shape == inp[key].shape, k
         torch.testing.assert_close(auto[key].float(), g3.to(inp[key].dtype).float().reshape(inp[key].shape), rtol=1e-6, atol=0,
                                    msg=lambda m, n=k: f"grad {n} through autograd: {m}")
+
+
+# ------------------------------------------------------------------ B and C as parameters: the reference module's call
+
+@pytest.mark.parametrize("dtype,hp,kinds", [(torch.float32, (3, 64), (2, 2)), (torch.bfloat16, (4, 64), (2, 3)),
+                                            (torch.float16, (2, 128), (3, 2)), (torch.float32, (8, 16), (3, 3)),
+                                            (torch.bfloat16, (8, 32), (2, 2))],
+                         ids=lambda v: str(v).replace("torch.", "").replace(" ", ""))
+@pytest.mark.parametrize("length,a_vec,z_mode,d_mode,init,ragged",
+                         [(333, False, 0, "mat", False, False), (128, True, 4, "vec", True, False),
+                          (200, False, 0, "mat", False, True), (7, False, 4, "none", True, True),
+                          (130, True, 0, "none", False, False)])
+def test_one_pass_with_parameter_projections(dtype, hp, kinds, length, a_vec, z_mode, d_mode, init, ragged):
+    """``B`` and ``C`` of shape ``(H, P)`` or ``(B, H, P)`` -- float32 parameters beside activations of any type -- with
+    ``A`` and ``D`` per channel or per head, no gate (or one of X's shape) and ``seq_lens``: what the reference's Mamba2
+    module passes (src/ssm/modules/mamba2.py:189-199).  The one-pass kernels keep the two projections in registers and
+    sum their gradients over time.  Forward against the oracle; every gradient against float64 autograd through the
+    oracle and against the general two-kernel path; the forward's table of round states in place of the sweep."""
+    ops = _ops()
+    h, p = hp
+    b = 3
+    inp = make(3 * length + h, b, length, h, p, dtype=dtype, bkind=kinds[0], ckind=kinds[1], a_vec=a_vec, d_mode=d_mode,
+               z_mode=z_mode, init=init)
+    inp["dt"] = inp["dt"].float()
+    inp["B"], inp["C"] = inp["B"].float(), inp["C"].float()
+    lens = [length, max(length // 3, 0), 0] if ragged else None
+    meta = {"seq_lens": lens} if ragged else None
+    half = dtype != torch.float32
+    y, yr = both(inp, meta=meta)
+    assert y.dtype == dtype
+    torch.testing.assert_close(y.float(), yr.float(), **(HALF_TOL if half else FP32_TOL))
+    if ragged:
+        assert torch.count_nonzero(y[2]) == 0 and torch.count_nonzero(y[1, length // 3:]) == 0
+
+    gy = torch.randn(b, length, h, p, generator=torch.Generator().manual_seed(length)).to(dtype)
+    want = _grads_oracle({k: (v.float() if v is not None else None) for k, v in inp.items()}, meta, gy.float())
+    d = {k: dev(v) for k, v in inp.items()}
+    lengths = torch.tensor(lens, dtype=torch.int32).cuda() if ragged else None
+    run = lambda **kw: ops._dscan_backward(dev(gy), d["X"], d["dt"], d["A"], d["B"], d["C"], 64, d["D"], d["z"], lengths,
+                                           d["init"], **kw)
+    one = run()
+    two = run(two_kernels=True)
+    for k, g1, g2 in zip(GRAD_NAMES, one, two):
+        if want[k] is None:
+            assert g1 is None
+            continue
+        w = want[k]
+        scale = float(w.abs().max()) + 1e-6
+        tol = dict(rtol=3e-2, atol=3e-2 * scale) if half else dict(rtol=2e-4, atol=2e-5 * max(scale, 1.0))
+        assert g1.dtype == (dtype if k == "X" else torch.float32) and g1.shape == w.shape, k
+        torch.testing.assert_close(g1.float().cpu().double(), w, msg=lambda m, n=k: f"grad {n} against the oracle: {m}", **tol)
+        torch.testing.assert_close(g1.float(), g2.float(), rtol=1e-2 if half else 1e-4,
+                                   atol=(1e-2 if half else 1e-5) * max(scale, 1.0),
+                                   msg=lambda m, n=k: f"grad {n} against the two-kernel path: {m}")
+    if ragged:
+        assert float(one[0][2].abs().max()) == 0.0 and float(one[1][1, length // 3:].abs().max()) == 0.0
+    y2, table = ops._dscan_forward(d["X"], d["dt"], d["A"], d["B"], d["C"], 64, d["D"], d["z"], lengths, d["init"],
+                                   want_round_states=True)
+    assert table is not None and tuple(table.shape) == (b, (length + 63) // 64, h * p)
+    for k, g1, g4 in zip(GRAD_NAMES, one, run(round_states=table)):
+        if g1 is not None:
+            torch.testing.assert_close(g4, g1, rtol=1e-6, atol=0, msg=lambda m, n=k: f"grad {n} with the forward's table: {m}")
+    auto = _grads_gpu(inp, meta, gy)
+    for k, g1 in zip(GRAD_NAMES, run(grads_in_input_dtype=True)):
+        if g1 is None:
+            continue
+        assert auto[k].dtype == inp[k].dtype and auto[k].shape == inp[k].shape, k
+        torch.testing.assert_close(auto[k].float(), g1.to(inp[k].dtype).float().reshape(inp[k].shape), rtol=1e-6, atol=0,
+                                   msg=lambda m, n=k: f"grad {n} through autograd: {m}")
