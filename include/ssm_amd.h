@@ -574,6 +574,30 @@ typedef struct ssm_ssd_scale_rows_args {
 } ssm_ssd_scale_rows_args;
 int ssm_ssd_scale_rows(const ssm_ssd_scale_rows_args *args, void *hip_stream);
 
+/* What the gradient of the combined forward derives from the raw steps alone, in one launch (whole chunks):
+ *   dt_out / dt_rows  the effective step (bias, softplus, clamp), chunked (B, H, nc, Q) and by rows (B, L, H)
+ *   dA_cumsum         its running sum times A inside the chunk, as ssm_ssd_chunk_cumsum gives it
+ *   dA_cumsum_rev     the same for the time-reversed sequence in which a step decays by the factor of the step that
+ *                     follows it in time (position i of reversed chunk nc-1-c is step cQ + Q-1-i)
+ *   w_dy[t] = exp(dA_cumsum at t),  w_x[t] = dt[t] * exp(dA_cumsum_rev at t's reversed position)
+ * The published backward takes these inside its kernels (_chunk_scan_bwd_* of the mamba_ssm package the reference's
+ * goldens come from, scripts/refresh_mamba_goldens.py:591-604); no single counterpart in the reference. */
+typedef struct ssm_ssd_bwd_prep_args {
+  const void *dt;            /* (B, L, H) dt_dtype: raw steps */
+  const float *A;            /* (H,) */
+  const float *dt_bias;      /* (H,) or NULL */
+  float *dA_cumsum;          /* (B, H, nc, Q) */
+  float *dt_out;             /* (B, H, nc, Q) */
+  float *dA_cumsum_rev;      /* (B, H, nc, Q) */
+  float *dt_rows;            /* (B, L, H) */
+  float *w_dy;               /* (B, L, H) */
+  float *w_x;                /* (B, L, H) */
+  int32_t batch, seqlen, heads, chunk;
+  int32_t dt_dtype, dt_softplus;
+  float dt_min, dt_max;
+} ssm_ssd_bwd_prep_args;
+int ssm_ssd_bwd_prep(const ssm_ssd_bwd_prep_args *args, void *hip_stream);
+
 /* The per-step scalars of the gradient of the combined forward (see ssm_ssd_bwd_gate), chunk by chunk:
  *   q[l]   = q_c + sum_{j<l in chunk} (s1[j] - s2[j]),  q_c = q0 for the first chunk and
  *            exp(dt A) at the chunk's first step (0 at the first step of a packed sequence) times anchor[c-1] after it

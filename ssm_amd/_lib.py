@@ -214,6 +214,12 @@ class SsdScaleRowsArgs(C.Structure):
                 ("out_dtype", _i32)]
 
 
+class SsdBwdPrepArgs(C.Structure):
+    _fields_ = [("dt", _vp), ("A", _vp), ("dt_bias", _vp), ("dA_cumsum", _vp), ("dt_out", _vp), ("dA_cumsum_rev", _vp),
+                ("dt_rows", _vp), ("w_dy", _vp), ("w_x", _vp), ("batch", _i32), ("seqlen", _i32), ("heads", _i32),
+                ("chunk", _i32), ("dt_dtype", _i32), ("dt_softplus", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float)]
+
+
 class SsdBwdDtArgs(C.Structure):
     _fields_ = [("s1", _vp), ("s2", _vp), ("xu", _vp), ("dt", _vp), ("dt_raw", _vp), ("A", _vp), ("dt_bias", _vp),
                 ("q0", _vp), ("anchor", _vp), ("first_step", _vp), ("ddt", _vp), ("dA_part", _vp), ("dbias_part", _vp),
@@ -286,6 +292,7 @@ ENTRY_POINTS = {
     "ssm_ssd_bwd_states": SsdBwdStatesArgs,
     "ssm_ssd_scale_rows": SsdScaleRowsArgs,
     "ssm_ssd_bwd_dt": SsdBwdDtArgs,
+    "ssm_ssd_bwd_prep": SsdBwdPrepArgs,
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_conv1d_update": Conv1dUpdateArgs,

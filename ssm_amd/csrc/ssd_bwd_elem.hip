@@ -344,6 +344,71 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_dt_kernel(const DtParams p
   p.db_part[gid] = db;
 }
 
+// Everything the backward derives from the raw steps alone, one wavefront per (b, h, chunk): the effective step
+// (bias, softplus, clamp) in both layouts, its running sum times A inside the chunk, the same for the time-reversed
+// sequence whose decay at a step is that of the step that follows it, and the two per-row weights
+// exp(running sum) and step * exp(reversed running sum).  Whole chunks only.
+struct PrepParams {
+  const void *dt;
+  const float *A, *bias;
+  float *dA_cs, *dt_c, *dA_rev;     // (B, H, nc, Q)
+  float *dte, *w_dy, *w_x;          // (B, L, H)
+  int batch, len, heads, chunk, nchunks;
+  int dt_dtype, softplus;
+  float lo, hi;
+};
+
+__global__ __launch_bounds__(EB_THREADS) void ssd_bwd_prep_kernel(const PrepParams p) {
+  const size_t gw = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int lane = lane_id();
+  if (gw >= (size_t)p.batch * p.heads * p.nchunks) return;      // whole wavefronts
+  const int c = (int)(gw % p.nchunks);
+  const int h = (int)((gw / p.nchunks) % p.heads);
+  const int b = (int)(gw / ((size_t)p.nchunks * p.heads));
+  const float A = p.A[h];
+  const float bias = p.bias ? p.bias[h] : 0.0f;
+  const int Q = p.chunk;
+  auto step_at = [&](int t) {              // the effective step; 0 past the end of the sequence
+    if (t >= p.len) return 0.0f;
+    float v = load_as_f32(p.dt, p.dt_dtype, ((size_t)b * p.len + t) * p.heads + h) + bias;
+    if (p.softplus) v = softplus_f32(v);
+    return fminf(fmaxf(v, p.lo), p.hi);
+  };
+  const size_t out = (((size_t)b * p.heads + h) * p.nchunks + c) * Q;
+  float carry = 0.0f;
+  for (int l0 = 0; l0 < Q; l0 += WAVE) {
+    const int l = l0 + lane;
+    const bool in = l < Q;
+    const int t = c * Q + l;
+    const float v = in ? step_at(t) : 0.0f;
+    const float run = carry + wave_inclusive_sum(v * A);
+    if (in) {
+      const size_t row = ((size_t)b * p.len + t) * p.heads + h;
+      p.dt_c[out + l] = v;
+      p.dA_cs[out + l] = run;
+      p.dte[row] = v;
+      p.w_dy[row] = expf(run);
+    }
+    carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(run), WAVE - 1));
+  }
+  // reversed time: position i of reversed chunk nc-1-c is step t = cQ + Q-1-i, decaying by the step after it
+  const size_t out_r = (((size_t)b * p.heads + h) * p.nchunks + (p.nchunks - 1 - c)) * Q;
+  carry = 0.0f;
+  for (int i0 = 0; i0 < Q; i0 += WAVE) {
+    const int i = i0 + lane;
+    const bool in = i < Q;
+    const int t = c * Q + Q - 1 - i;
+    const float next = in ? step_at(t + 1) : 0.0f;
+    const float run = carry + wave_inclusive_sum(next * A);
+    if (in) {
+      p.dA_rev[out_r + i] = run;
+      p.w_x[((size_t)b * p.len + t) * p.heads + h] = step_at(t) * expf(run);
+    }
+    carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(run), WAVE - 1));
+  }
+}
+
+
 }  // namespace
 }  // namespace ssm
 
@@ -513,5 +578,26 @@ extern "C" int ssm_ssd_bwd_dt(const ssm_ssd_bwd_dt_args *a, void *hip_stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   hipLaunchKernelGGL(ssd_bwd_dt_kernel, dim3((unsigned)((total + EB_THREADS - 1) / EB_THREADS)), dim3(EB_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_bwd_dt");
+  return SSM_OK;
+}
+
+extern "C" int ssm_ssd_bwd_prep(const ssm_ssd_bwd_prep_args *a, void *hip_stream) {
+  using namespace ssm;
+  SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_prep: args is NULL");
+  SSM_REQUIRE(a->dt && a->A && a->dA_cumsum && a->dt_out && a->dA_cumsum_rev && a->dt_rows && a->w_dy && a->w_x,
+              SSM_ERR_NULL_POINTER, "ssm_ssd_bwd_prep: dt, A and the six outputs are required");
+  SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->heads > 0 && a->chunk > 0 && a->seqlen % a->chunk == 0, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_bwd_prep: sizes must be positive and chunk=%d must divide seqlen=%d", a->chunk, a->seqlen);
+  SSM_REQUIRE(valid_dtype(a->dt_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_bwd_prep: dt_dtype=%d", a->dt_dtype);
+  PrepParams p{};
+  p.dt = a->dt; p.A = a->A; p.bias = a->dt_bias; p.dA_cs = a->dA_cumsum; p.dt_c = a->dt_out; p.dA_rev = a->dA_cumsum_rev;
+  p.dte = a->dt_rows; p.w_dy = a->w_dy; p.w_x = a->w_x;
+  p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.chunk = a->chunk; p.nchunks = a->seqlen / a->chunk;
+  p.dt_dtype = a->dt_dtype; p.softplus = a->dt_softplus ? 1 : 0; p.lo = a->dt_min; p.hi = a->dt_max;
+  const size_t waves = (size_t)p.batch * p.heads * p.nchunks;
+  SSM_REQUIRE(waves < ((size_t)1 << 31) / WAVE, SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_prep: too many (batch, head, chunk) triples");
+  hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(ssd_bwd_prep_kernel, dim3((unsigned)((waves * WAVE + EB_THREADS - 1) / EB_THREADS)), dim3(EB_THREADS), 0, s, p);
+  SSM_CHECK_LAUNCH("ssm_ssd_bwd_prep");
   return SSM_OK;
 }

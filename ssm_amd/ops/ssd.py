@@ -758,6 +758,41 @@ def _scale_rows(x, w, out_dtype):
     return out
 
 
+def _bwd_prep(dt, A, chunk_size, dt_bias, dt_softplus, dt_limit):
+    """``ssm_ssd_bwd_prep``: ``(dA_cumsum, dt_out, dA_cumsum_rev)`` as ``(B, H, nc, Q)`` and ``(dt_rows, w_dy, w_x)``
+    as ``(B, L, H)``, float32, for a sequence of whole chunks."""
+    batch, seqlen, heads = (int(v) for v in dt.shape)
+    Q = int(chunk_size)
+    dev = dt.device
+    dtc = K.cast_c(dt, dt.dtype)
+    Af, bf = K.as_f32_vec(A), K.as_f32_vec(dt_bias)
+    chunked = [torch.empty(batch, heads, seqlen // Q, Q, dtype=torch.float32, device=dev) for _ in range(3)]
+    rows = [torch.empty(batch, seqlen, heads, dtype=torch.float32, device=dev) for _ in range(3)]
+    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    args = _lib.SsdBwdPrepArgs(
+        dt=_lib.ptr(dtc), A=_lib.ptr(Af), dt_bias=_lib.ptr(bf), dA_cumsum=_lib.ptr(chunked[0]), dt_out=_lib.ptr(chunked[1]),
+        dA_cumsum_rev=_lib.ptr(chunked[2]), dt_rows=_lib.ptr(rows[0]), w_dy=_lib.ptr(rows[1]), w_x=_lib.ptr(rows[2]),
+        batch=batch, seqlen=seqlen, heads=heads, chunk=Q, dt_dtype=_lib.dtype_enum(dtc.dtype),
+        dt_softplus=int(bool(dt_softplus)), dt_min=lo if lo > -math.inf else -3.0e38, dt_max=hi if hi < math.inf else 3.0e38)
+    _lib.call("ssm_ssd_bwd_prep", args, dev)
+    return (*chunked, *rows)
+
+
+_ONES = {}
+
+
+def _ones_like_cached(t):
+    """A float32 tensor of ones with ``t``'s shape on its device, kept between calls (a read-only operand: the passes'
+    step weights when the step is already in the operand)."""
+    key = (tuple(t.shape), t.device)
+    ones = _ONES.get(key)
+    if ones is None:
+        if len(_ONES) >= 8:
+            _ONES.clear()
+        ones = _ONES[key] = torch.ones(t.shape, dtype=torch.float32, device=t.device)
+    return ones
+
+
 def _bwd_states(ent_f, ent_r):
     """``ssm_ssd_bwd_states``: both stacks of chunk-boundary states as bfloat16 with chunks in time order, and the
     anchors ``<adjoint state, forward state>`` at the boundaries ``1..nc-1`` ``(B, nc-1, H)``."""
@@ -869,14 +904,23 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     def blh(t_c):                         # (B, H, nc, Q) -> (B, L, H)
         return t_c.permute(0, 2, 3, 1).reshape(batch, -1, heads)[:, :seqlen]
 
-    dA_cs, dt_c = chunk_cumsum(dt.detach(), Af, Q, dt_bias=None if dt_bias is None else dt_bias.detach(),
-                               dt_softplus=dt_softplus, dt_limit=dt_limit)
-    dte = blh(dt_c)                                                   # effective step
+    # everything that follows from the raw steps alone: one launch for whole chunks without packed sequences
+    prepared = seq_idx is None and seqlen % Q == 0
+    if prepared:
+        dA_cs, dt_c, dA_r, dte, w_dy, w_x = _bwd_prep(dt.detach(), Af, Q, None if dt_bias is None else dt_bias.detach(),
+                                                      dt_softplus, dt_limit)
+    else:
+        dA_cs, dt_c = chunk_cumsum(dt.detach(), Af, Q, dt_bias=None if dt_bias is None else dt_bias.detach(),
+                                   dt_softplus=dt_softplus, dt_limit=dt_limit)
+        dte = blh(dt_c)                                               # effective step
     # y before skip and gate.  The step enters through the operand (x~ = dt x, rounded once) rather than as a
     # weight inside the kernels: then this pass and the reversed one below multiply the same rounded
     # C.B-times-decay blocks, and the running sum that gives q (a difference of their row and column sums)
     # sees each product twice with the same value instead of collecting the two passes' rounding noise.
-    _, ones_c = chunk_cumsum(torch.ones_like(dte), torch.zeros_like(Af), Q)
+    if prepared:
+        ones_c = _ones_like_cached(dt_c)
+    else:
+        _, ones_c = chunk_cumsum(torch.ones_like(dte), torch.zeros_like(Af), Q)
     bnd = None
     if seq_idx is not None:
         sid = seq_idx.to(torch.int64)
@@ -892,8 +936,9 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     xt = _scale_rows(xd, dte, cd) if (fused and cd in (torch.float32, torch.bfloat16)) else (dte[..., None] * xd).to(cd)
     ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
     # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
-    dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
-    dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
+    if not prepared:
+        dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()
+        dA_r, _ = chunk_cumsum(dts, Af, Q, dt_limit=(-math.inf, math.inf))
     if bnd is not None:                       # the reversed passes decay by the following step's factor
         dA_r = dA_r + jumps(torch.cat([bnd[:, 1:], torch.zeros_like(bnd[:, :1])], dim=1).flip(1))
     # dB and dC with the sum over a group's heads taken first (two small products per chunk)?
@@ -905,8 +950,9 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         # the rows of the two products across chunk boundaries leave the gate kernel with their weights on:
         # dy_l exp(cs_l) for dC, x_s dt_s exp(cs'_s) for dB, cs' the running sum of the reversed pass at that step
         # (the decay from s to the end of its chunk and over the step that follows)
-        w_dy = torch.exp(blh(dA_cs)).contiguous()
-        w_x = (dte * torch.exp(blh(dA_r)).flip(1)).contiguous()
+        if not prepared:
+            w_dy = torch.exp(blh(dA_cs)).contiguous()
+            w_x = (dte * torch.exp(blh(dA_r)).flip(1)).contiguous()
         dyc, dyr, dz, s2, dyx, wdy, xw = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, w_dy=w_dy, w_x=w_x,
                                                      grads_io=grads_in_input_dtype)
     elif fused:
@@ -932,9 +978,11 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         dyr = dyc.flip(1).contiguous()
     u_r, Gfin, ent_r = _lin_pass(dyr, ones_c, dA_r, Cc.flip(1).contiguous(), Bc.flip(1).contiguous(), dfin,
                                  want_entering=True)
-    dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin
-    if bnd is not None:
-        dinit = dinit * (~bnd[:, 0]).to(f32)[:, None, None, None]
+    dinit = None
+    if init is not None:
+        dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin
+        if bnd is not None:
+            dinit = dinit * (~bnd[:, 0]).to(f32)[:, None, None, None]
     if fused:
         dx, xu, s1 = _bwd_dx(dod, zd, xd, u_r.contiguous(), dte, Df, cd == torch.bfloat16,
                              grads_io=grads_in_input_dtype)

@@ -739,3 +739,32 @@ def test_scale_rows_kernel_rounds_once(dtype):
     got = ops_ssd._scale_rows(x, w, torch.bfloat16)
     assert torch.equal(got, (w[..., None] * x.float()).to(torch.bfloat16))
     assert torch.equal(ops_ssd._scale_rows(x, w, torch.float32), w[..., None] * x.float())
+
+
+@pytest.mark.parametrize("Q,L,softplus,limit", [(64, 256, True, (0.001, 0.1)), (96, 288, False, (0.0, float("inf"))),
+                                                 (256, 256, True, (0.0, float("inf"))), (32, 160, True, (0.01, 1.0))])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_bwd_prep_kernel_matches_the_steps_taken_one_by_one(Q, L, softplus, limit, dtype):
+    """One launch for what the backward derives from the raw steps: the chunked running sums are those of
+    ``chunk_cumsum`` (forward, and over the time-reversed steps that decay by the step after them) to the bit, and the
+    two row weights are their exponentials in float64 to a few ulps."""
+    import math
+    from ssm_amd.ops import ssd as ops_ssd
+    gen = torch.Generator().manual_seed(Q + L)
+    b, h = 2, 5
+    dt = (torch.randn(b, L, h, generator=gen) * (1.0 if softplus else 0.05)).to(dtype).cuda()
+    if not softplus:
+        dt = dt.abs()
+    A = -(torch.rand(h, generator=gen) * 8 + 0.1).cuda()
+    bias = torch.randn(h, generator=gen).cuda() * 0.1 if softplus else None
+    dA_cs, dt_c, dA_r, dte, w_dy, w_x = ops_ssd._bwd_prep(dt, A, Q, bias, softplus, limit)
+    want_cs, want_dt = ops_ssd.chunk_cumsum(dt, A, Q, dt_bias=bias, dt_softplus=softplus, dt_limit=limit)
+    assert torch.equal(dA_cs, want_cs) and torch.equal(dt_c, want_dt)
+    rows = want_dt.permute(0, 2, 3, 1).reshape(b, L, h)
+    assert torch.equal(dte, rows)
+    shifted = torch.cat([rows[:, 1:], torch.zeros_like(rows[:, :1])], dim=1).flip(1).contiguous()
+    want_r, _ = ops_ssd.chunk_cumsum(shifted, A, Q, dt_limit=(-math.inf, math.inf))
+    assert torch.equal(dA_r, want_r)
+    by_rows = lambda t: t.permute(0, 2, 3, 1).reshape(b, L, h)
+    torch.testing.assert_close(w_dy.double(), torch.exp(by_rows(want_cs).double()), rtol=2e-6, atol=1e-30)
+    torch.testing.assert_close(w_x.double(), rows.double() * torch.exp(by_rows(want_r).double()).flip(1), rtol=2e-6, atol=1e-30)
