@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SSM_AMD_ABI_VERSION 4
+#define SSM_AMD_ABI_VERSION 5
 
 typedef enum ssm_status {
   SSM_OK = 0,
@@ -384,6 +384,9 @@ typedef struct ssm_ssd_chunk_state_args {
   ssm_ssd_dims dims;
   int32_t x_dtype, b_dtype, states_dtype, force_generic;
   const int32_t *seq_idx;   /* (B,L) or NULL: steps of another sequence than the chunk's last step add nothing */
+  const float *x_row_scale; /* (B,H,nc,Q) or NULL: x stands for x * scale rounded to x's dtype, as if that tensor had
+                               been written first (the backward puts the step into the operand this way); only the
+                               matrix-core kernel takes it, and only for bfloat16 x: an error otherwise */
 } ssm_ssd_chunk_state_args;
 size_t ssm_ssd_chunk_state_workspace_bytes(const ssm_ssd_dims *dims);
 int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *args, void *hip_stream);
@@ -418,6 +421,7 @@ typedef struct ssm_ssd_chunk_scan_args {
                                formed with the same seq_idx */
   int32_t y_f32;            /* nonzero: y is float32 whatever x's dtype is (the backward's running sums need the
                                passes' results unrounded); 0: y has x's dtype */
+  const float *x_row_scale; /* (B,H,nc,Q) or NULL: as in ssm_ssd_chunk_state_args (the skip term D x is not scaled) */
 } ssm_ssd_chunk_scan_args;
 int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
 

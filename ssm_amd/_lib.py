@@ -19,7 +19,7 @@ import os
 # SSM_AMD_LIB points the binding at another build of the same C ABI.
 LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
                 Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
 PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
@@ -137,7 +137,7 @@ class SsdChunkStateArgs(C.Structure):
     _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("states", _vp),
                 ("workspace", _vp), ("workspace_bytes", C.c_size_t), ("dims", SsdDims),
                 ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("force_generic", _i32),
-                ("seq_idx", _vp)]
+                ("seq_idx", _vp), ("x_row_scale", _vp)]
 
 
 class SsdStatePassingArgs(C.Structure):
@@ -151,7 +151,7 @@ class SsdChunkScanArgs(C.Structure):
                 ("dA_cumsum", _vp), ("Dskip", _vp), ("y", _vp), ("dims", SsdDims),
                 ("x_dtype", _i32), ("c_dtype", _i32), ("cb_dtype", _i32), ("states_dtype", _i32),
                 ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32), ("seq_idx", _vp),
-                ("y_f32", _i32)]
+                ("y_f32", _i32), ("x_row_scale", _vp)]
 
 
 class SsdChunkStateVarlenArgs(C.Structure):

@@ -355,12 +355,20 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   p.scratch = a->workspace; p.scratch_bytes = a->workspace_bytes;
   p.x_dtype = a->x_dtype; p.b_dtype = a->b_dtype; p.states_dtype = a->states_dtype;
   p.seq_idx = a->seq_idx;
+  p.x_scale = a->x_row_scale;
+  // (float16 is left out: the conversion that rounds the product does not keep float16 subnormals, which a tensor
+  // written beforehand would hold)
+  SSM_REQUIRE(a->x_row_scale == nullptr || a->x_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_chunk_state: x_row_scale needs bfloat16 x (x_dtype=%d)", a->x_dtype);
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   if (!a->force_generic && ssd_chunk_state_mfma(p, s)) {
     g_mfma_launches |= 2;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
     return SSM_OK;
   }
+  SSM_REQUIRE(a->x_row_scale == nullptr, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_chunk_state: x_row_scale is taken by the matrix-core kernel only (bfloat16 x and B, whole "
+              "chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64, a workspace)");
   if (!a->force_generic && ssd_chunk_state_tiled(p, s)) {
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(tiled)");
     return SSM_OK;
@@ -416,12 +424,18 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   p.z_dtype = a->z_dtype; p.d_per_p = a->d_per_p ? 1 : 0;
   p.seq_idx = a->seq_idx;
   p.y_dtype = a->y_f32 ? SSM_F32 : a->x_dtype;
+  p.x_scale = a->x_row_scale;
+  SSM_REQUIRE(a->x_row_scale == nullptr || a->x_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_chunk_scan: x_row_scale needs bfloat16 x (x_dtype=%d)", a->x_dtype);
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
     g_mfma_launches |= 4;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
     return SSM_OK;
   }
+  SSM_REQUIRE(a->x_row_scale == nullptr, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_chunk_scan: x_row_scale is taken by the matrix-core kernel only (bfloat16 x, C and CB, "
+              "whole chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64)");
   if (!a->force_generic && ssd_chunk_scan_tiled(p, s)) {
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(tiled)");
     return SSM_OK;

@@ -42,6 +42,7 @@ struct SsdStateParams {
   SsdDims d;
   int x_dtype, b_dtype, states_dtype;
   const int *seq_idx;         // (B, L) or null
+  const float *x_scale;       // (B, H, nc, Q) or null: x stands for x * scale rounded to x's type (matrix-core kernels only)
 };
 
 struct SsdPassParams {
@@ -65,6 +66,7 @@ struct SsdScanParams {
   int d_per_p;                // D is (H, P) instead of (H,)
   const int *seq_idx;         // (B, L) or null
   int y_dtype;                // x_dtype, or SSM_F32 on request
+  const float *x_scale;       // (B, H, nc, Q) or null: x stands for x * scale rounded to x's type (matrix-core kernels only)
 };
 
 __device__ __forceinline__ void store_any(void *p, int dtype, size_t i, float v) {

@@ -32,9 +32,11 @@ __device__ __forceinline__ int xt_off(int p, int l, int stride) {
 // Transpose the [Q][P] bf16 slab x[b, t0.., h, :] into LDS as [P][Q] (optionally
 // scaling row l by w[l]).  A thread moves 8x8 blocks: eight 16-byte global reads
 // along p, eight 16-byte LDS writes along l.
-template <bool WEIGHTED, typename E>
+// PRE: row l is first multiplied by pre[l] (global memory, the chunk's Q values) and rounded to E -- the operand
+// then is exactly the tensor round(x * pre) that a separate launch would have written.
+template <bool WEIGHTED, bool PRE, typename E>
 __device__ __forceinline__ void stage_xT(E *xT, const E *x, size_t row_stride, int Q, int P,
-                                         const float *w_lds, int stride) {
+                                         const float *w_lds, int stride, const float *pre = nullptr) {
   const int pblocks = P >> 3;
   const int nblocks = (Q >> 3) * pblocks;
   for (int blk = threadIdx.x; blk < nblocks; blk += MF_THREADS) {
@@ -44,8 +46,13 @@ __device__ __forceinline__ void stage_xT(E *xT, const E *x, size_t row_stride, i
     for (int r = 0; r < 8; ++r) {
       const V8<E> raw = load_frag_e<E>(x + (size_t)(lb * 8 + r) * row_stride + pb * 8);
       const float w = WEIGHTED ? w_lds[lb * 8 + r] : 1.0f;
+      const float pr = PRE ? pre[lb * 8 + r] : 1.0f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[r][i] = WEIGHTED ? (float)raw[i] * w : (float)raw[i];
+      for (int i = 0; i < 8; ++i) {
+        float e = (float)raw[i];
+        if (PRE) e = (float)(E)(e * pr);
+        v[r][i] = WEIGHTED ? e * w : e;
+      }
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -250,7 +257,8 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const 
     w[l] = (sid && sid[l] != sid_last) ? 0.0f : decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
   __syncthreads();
   const E *xg = reinterpret_cast<const E *>(p.x) + (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
-  stage_xT<true, E>(xT, xg, (size_t)d.heads * P, Q, P, w, stride);
+  if (p.x_scale) stage_xT<true, true, E>(xT, xg, (size_t)d.heads * P, Q, P, w, stride, p.x_scale + cs);
+  else stage_xT<true, false, E>(xT, xg, (size_t)d.heads * P, Q, P, w, stride);
   __syncthreads();
 
   const int g2 = lane >> 5, m = lane & 31;
@@ -309,7 +317,8 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   const size_t xrow = (size_t)d.heads * P;                                 // elements between time steps
   const size_t xbase = (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
   const E *xg = reinterpret_cast<const E *>(p.x) + xbase;
-  stage_xT<false, E>(xT, xg, xrow, Q, P, nullptr, stride);
+  if (p.x_scale) stage_xT<false, true, E>(xT, xg, xrow, Q, P, nullptr, stride, p.x_scale + cs);
+  else stage_xT<false, false, E>(xT, xg, xrow, Q, P, nullptr, stride);
   // The state entering the chunk, [P][N], as bfloat16 in LDS: read once by the workgroup in whole lines (a fragment
   // read straight from memory, lane = row, touches 32 lines for 32 bytes each, and every row block would read it again).
   E *Sb = reinterpret_cast<E *>(ent + Q);                       // [P][N + 8]

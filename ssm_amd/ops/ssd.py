@@ -130,7 +130,25 @@ def _seq_idx_i32(seq_idx, batch, seqlen):
     return seq_idx.to(torch.int32).contiguous()
 
 
-def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=False, seq_idx=None):
+def _scale_arg(x_scale, dt):
+    if x_scale is None:
+        return None
+    _need(x_scale.shape == dt.shape and x_scale.dtype == torch.float32 and x_scale.device == dt.device,
+          "x_scale must be a float32 tensor of dt's shape (B, H, nc, Q).")
+    return x_scale.contiguous()
+
+
+def _row_scale_ok(x, Bm, Cm, chunk_size):
+    """Whether ``chunk_state`` / ``chunk_scan`` take ``x_scale`` for these operands: the matrix-core kernels' shapes
+    (bfloat16 tensors, whole chunks of a multiple of 32 up to 256 steps, a state size that is a multiple of 16, heads
+    of 32 channels or a multiple of 64, which :func:`_lin_pass` cuts into pieces of 64)."""
+    Q, seqlen, hdim, nstate = int(chunk_size), int(x.shape[1]), int(x.shape[-1]), int(Bm.shape[-1])
+    return (x.dtype == torch.bfloat16 and Bm.dtype == x.dtype and Cm.dtype == x.dtype
+            and seqlen % Q == 0 and Q % 32 == 0 and Q <= 256 and nstate % 16 == 0 and seqlen % 8 == 0
+            and (hdim == 32 or hdim % 64 == 0))
+
+
+def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=False, seq_idx=None, x_scale=None):
     """Contribution of each chunk to the state at its end.
 
     Args:
@@ -141,6 +159,8 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
         states_dtype: dtype of the result.
         seq_idx: Optional ``(B, L)`` int sequence ids of a packed batch: steps of another
             sequence than the chunk's last step add nothing.
+        x_scale: Optional ``(B, H, nc, Q)`` float32: ``x`` stands for ``x * x_scale`` rounded to ``x.dtype`` (only
+            for calls :func:`_row_scale_ok` accepts).
 
     Returns:
         ``states (B, nc, H, P, N)``.
@@ -166,7 +186,7 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
         workspace=_lib.ptr(ws), workspace_bytes=nbytes,
         dims=dims, x_dtype=_lib.dtype_enum(xc.dtype),
         b_dtype=_lib.dtype_enum(Bc.dtype), states_dtype=_lib.dtype_enum(states_dtype),
-        force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si))
+        force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)))
     _lib.call("ssm_ssd_chunk_state", args, dev)
     return states
 
@@ -221,7 +241,7 @@ def state_passing(states, dA_chunk_cumsum, initial_states=None, seq_idx=None, ch
 
 
 def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False, seq_idx=None,
-               out_f32=False):
+               out_f32=False, x_scale=None):
     """Outputs of every chunk from the state entering it.
 
     Args:
@@ -236,6 +256,7 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
             whose id equals that of the last step of the chunk before (id 0 for the first
             chunk), and products across sequences inside a chunk are dropped.
         out_f32: Return ``y`` in float32 (the accumulators as they are) instead of ``x.dtype``.
+        x_scale: As in :func:`chunk_state` (the skip term ``D x`` takes ``x`` as it is).
 
     Returns:
         ``y (B, L, H, P)`` in ``x.dtype`` (float32 with ``out_f32``).
@@ -271,7 +292,8 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         dims=_dims(batch, seqlen, heads, hdim, groups, nstate, Q), x_dtype=_lib.dtype_enum(xc.dtype),
         c_dtype=_lib.dtype_enum(Cc.dtype), cb_dtype=_lib.dtype_enum(cb.dtype),
         states_dtype=_lib.dtype_enum(ps.dtype), z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
-        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), y_f32=int(bool(out_f32)))
+        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), y_f32=int(bool(out_f32)),
+        x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)))
     _lib.call("ssm_ssd_chunk_scan", args, dev)
     return y
 
@@ -634,26 +656,28 @@ def varlen_states_backward(dstates, x, dt, A, B, cu_seqlens, dt_bias=None, initi
     return dx, ddt, dA, dB, dbias, dinit
 
 
-def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None):
+def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_scale=None):
     """``y_t = sum_{s<=t} exp(cs_t - cs_s) <C_t, B_s> w_s x_s + exp(cs_t) C_t . init`` and the state
     after the last step, through chunk_state -> state_passing -> chunk_scan (states in float32).
 
     Channels are independent of each other, so with bfloat16 operands a head dimension beyond 64 (the
     backward's passes that put the state axis in the channel role) is cut into pieces of 64, the width
     the matrix-core kernels are built for.  With ``want_entering`` the states entering the chunks
-    ``(B, nc, H, P, N)`` come back as a third result."""
+    ``(B, nc, H, P, N)`` come back as a third result.  ``x_scale (B, H, nc, Q)``: ``x`` stands for ``x * x_scale``
+    rounded to its type (for calls :func:`_row_scale_ok` accepts)."""
     hd = int(x.shape[-1])
     if x.dtype == torch.bfloat16 and hd > 64 and hd % 64 == 0:
         Q = int(dA_cs.shape[3])
         CB = bmm_chunk(Cm, Bm, Q, causal=True, output_dtype=x.dtype)          # the same for every piece
         parts = [_lin_pass(x[..., k:k + 64].contiguous(), w_c, dA_cs, Bm, Cm,
-                           None if init is None else init[:, :, k:k + 64].contiguous(), want_entering, CB=CB)
+                           None if init is None else init[:, :, k:k + 64].contiguous(), want_entering, CB=CB,
+                           x_scale=x_scale)
                  for k in range(0, hd, 64)]
         out = (torch.cat([q[0] for q in parts], dim=-1), torch.cat([q[1] for q in parts], dim=2))
         return out + (torch.cat([q[2] for q in parts], dim=3),) if want_entering else out
-    states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32)
+    states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32, x_scale=x_scale)
     entering, final = state_passing(states, dA_cs[:, :, :, -1].contiguous(), initial_states=init)
-    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, CB=CB, out_f32=True)
+    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, CB=CB, out_f32=True, x_scale=x_scale)
     return (y, final, entering) if want_entering else (y, final)
 
 
@@ -933,8 +957,12 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
 
         dA_cs = dA_cs + jumps(bnd)
     dte = dte.contiguous()
-    xt = _scale_rows(xd, dte, cd) if (fused and cd in (torch.float32, torch.bfloat16)) else (dte[..., None] * xd).to(cd)
-    ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
+    if fused and cd == torch.bfloat16 and xd.dtype == cd and _row_scale_ok(xd, Bc, Cc, Q):
+        # the kernels round dt x as they stage it: the same operand without a tensor of x's size written and read
+        ypre, _, ent_f = _lin_pass(xd, ones_c, dA_cs, Bc, Cc, init, want_entering=True, x_scale=dt_c)
+    else:
+        xt = _scale_rows(xd, dte, cd) if (fused and cd in (torch.float32, torch.bfloat16)) else (dte[..., None] * xd).to(cd)
+        ypre, _, ent_f = _lin_pass(xt, ones_c, dA_cs, Bc, Cc, init, want_entering=True)
     # decay of the reversed passes: a'_tau = a_{t+1} with t = L - 1 - tau; weights 1 on real steps
     if not prepared:
         dts = torch.cat([dte[:, 1:], torch.zeros_like(dte[:, :1])], dim=1).flip(1).contiguous()

@@ -768,3 +768,32 @@ def test_bwd_prep_kernel_matches_the_steps_taken_one_by_one(Q, L, softplus, limi
     by_rows = lambda t: t.permute(0, 2, 3, 1).reshape(b, L, h)
     torch.testing.assert_close(w_dy.double(), torch.exp(by_rows(want_cs).double()), rtol=2e-6, atol=1e-30)
     torch.testing.assert_close(w_x.double(), rows.double() * torch.exp(by_rows(want_r).double()).flip(1), rtol=2e-6, atol=1e-30)
+
+
+@pytest.mark.parametrize("shape,Q", [((2, 256, 3, 64, 1, 32), 64), ((1, 512, 4, 32, 2, 16), 256), ((2, 192, 2, 128, 1, 64), 96)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_operand_scaled_while_staged_equals_the_scaled_tensor(shape, Q, dtype=torch.bfloat16):
+    """``x_scale``: the matrix-core ``chunk_state`` and ``chunk_scan`` round ``x * scale`` as they stage ``x`` -- the
+    bits of a pass over the tensor ``round(x * scale)`` written beforehand, entering states included."""
+    from ssm_amd.ops import ssd as ops_ssd
+    b, l, h, p, g, n = shape
+    gen = torch.Generator().manual_seed(l + h)
+    x = torch.randn(b, l, h, p, generator=gen).to(dtype).cuda()
+    Bm = torch.randn(b, l, g, n, generator=gen).to(dtype).cuda()
+    Cm = torch.randn(b, l, g, n, generator=gen).to(dtype).cuda()
+    dt = (torch.rand(b, l, h, generator=gen) * 0.2).cuda()
+    A = -(torch.rand(h, generator=gen) * 4 + 0.1).cuda()
+    init = torch.randn(b, h, p, n, generator=gen).cuda()
+    dA_cs, dt_c = ops_ssd.chunk_cumsum(dt, A, Q)
+    ones = torch.ones_like(dt_c)
+    assert ops_ssd._row_scale_ok(x, Bm, Cm, Q)
+    scaled = (dt[..., None] * x.float()).to(dtype)
+    want = ops_ssd._lin_pass(scaled, ones, dA_cs, Bm, Cm, init, want_entering=True)
+    got = ops_ssd._lin_pass(x, ones, dA_cs, Bm, Cm, init, want_entering=True, x_scale=dt_c)
+    for a, w, name in zip(got, want, ("y", "final state", "entering states")):
+        assert torch.equal(a, w), name
+    # a call the matrix-core kernels do not take refuses the scale instead of dropping it
+    for other in (torch.float32, torch.float16):
+        with pytest.raises(Exception, match="x_row_scale"):
+            ops_ssd.chunk_state(Bm.to(other), x.to(other), ones, dA_cs, x_scale=dt_c)
+        assert not ops_ssd._row_scale_ok(x.to(other), Bm.to(other), Cm.to(other), Q)
