@@ -422,6 +422,18 @@ typedef struct ssm_ssd_chunk_scan_args {
   int32_t y_f32;            /* nonzero: y is float32 whatever x's dtype is (the backward's running sums need the
                                passes' results unrounded); 0: y has x's dtype */
   const float *x_row_scale; /* (B,H,nc,Q) or NULL: as in ssm_ssd_chunk_state_args (the skip term D x is not scaled) */
+  /* The gradient's time-reversed pass (x = dy reversed, B and C in each other's place) can finish dx in this kernel
+   * instead of writing its result u (y may then be NULL): with t = L-1-tau the forward step of reversed row tau,
+   *   dx_out[t] = dx_dt[t] u[tau] + dx_Dskip dy[t],  dx_xu[t] = sum_p dx_x[t] u[tau],
+   *   dx_s1[t] = sum_p round(dx_dt[t] dx_x[t]) u[tau]      (rounded to x's dtype if dx_round_dtx)
+   * -- what ssm_ssd_bwd_dx computes from u (there dy is taken before its rounding to the operand's type, here after).
+   * Matrix-core kernel only: bfloat16 operands, float32 states, no z / Dskip / seq_idx; an error otherwise. */
+  const void *dx_x;         /* (B,L,H,P) x dtype, forward time */
+  const float *dx_dt;       /* (B,L,H) */
+  const float *dx_Dskip;    /* (H,P) if dx_d_per_p else (H,), or NULL */
+  void *dx_out;             /* (B,L,H,P) float32 if dx_out_f32 else x dtype; NULL: the ordinary call */
+  float *dx_xu, *dx_s1;     /* (B,L,H) */
+  int32_t dx_d_per_p, dx_out_f32, dx_round_dtx;
 } ssm_ssd_chunk_scan_args;
 int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
 

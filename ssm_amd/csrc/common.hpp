@@ -165,6 +165,29 @@ constexpr int DPP_ROW_BCAST15 = 0x142, DPP_ROW_BCAST31 = 0x143, DPP_WAVE_SHR1 = 
 constexpr int DPP_ROW_SHL1 = 0x101, DPP_ROW_SHL2 = 0x102, DPP_ROW_SHL4 = 0x104, DPP_ROW_SHL8 = 0x108;
 constexpr int DPP_WAVE_SHL1 = 0x130;
 
+// Sum over each group of LPH neighbouring lanes (16, 32 or 64), valid in the group's last lane.
+template <int LPH>
+__device__ __forceinline__ float lane_group_sum_last(float v) {
+  v += dpp_move<DPP_ROW_SHR1, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR2, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR4, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR8, 0xf>(0.0f, v);
+  if (LPH >= 32) v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.0f, v);
+  if (LPH >= 64) v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.0f, v);
+  return v;
+}
+
+// Sum over each run of N neighbouring lanes (8 or 16, aligned), valid in the run's last lane.
+template <int N>
+__device__ __forceinline__ float lane_run_sum_last(float v) {
+  static_assert(N == 8 || N == 16, "runs inside a row of 16 lanes");
+  v += dpp_move<DPP_ROW_SHR1, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR2, 0xf>(0.0f, v);
+  v += dpp_move<DPP_ROW_SHR4, 0xf>(0.0f, v);
+  if (N == 16) v += dpp_move<DPP_ROW_SHR8, 0xf>(0.0f, v);
+  return v;
+}
+
 // Inclusive scan across the 64 lanes of the pair (a, b) under
 //   (a1, b1) then (a2, b2)  ->  (a1 a2, a2 b1 + b2)
 // i.e. the composition of the affine maps h -> a h + b, earlier lanes first.

@@ -21,18 +21,6 @@ namespace ssm {
 
 constexpr int DBO_WAVES = 16, DBO_SEG = 4, DBO_ROUND = DBO_WAVES * DBO_SEG;
 
-// Sum over each group of LPH neighbouring lanes (16, 32 or 64), valid in the group's last lane.
-template <int LPH>
-__device__ __forceinline__ float lane_group_sum_last(float v) {
-  v += dpp_move<DPP_ROW_SHR1, 0xf>(0.0f, v);
-  v += dpp_move<DPP_ROW_SHR2, 0xf>(0.0f, v);
-  v += dpp_move<DPP_ROW_SHR4, 0xf>(0.0f, v);
-  v += dpp_move<DPP_ROW_SHR8, 0xf>(0.0f, v);
-  if (LPH >= 32) v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.0f, v);
-  if (LPH >= 64) v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.0f, v);
-  return v;
-}
-
 // ---- the gradients
 template <typename io_t, int VEC, bool HAS_Z>
 struct DboRegs {

@@ -410,8 +410,8 @@ extern "C" int ssm_ssd_state_passing(const ssm_ssd_state_passing_args *a, void *
 
 extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_stream) {
   using namespace ssm;
-  SSM_REQUIRE(a && a->CB && a->Cm && a->x && a->dt && a->dA_cumsum && a->prev_states && a->y, SSM_ERR_NULL_POINTER,
-              "ssm_ssd_chunk_scan: CB, Cm, x, dt, dA_cumsum, prev_states and y are required");
+  SSM_REQUIRE(a && a->CB && a->Cm && a->x && a->dt && a->dA_cumsum && a->prev_states && (a->y || a->dx_out),
+              SSM_ERR_NULL_POINTER, "ssm_ssd_chunk_scan: CB, Cm, x, dt, dA_cumsum, prev_states and y (or dx_out) are required");
   SsdScanParams p{};
   int rc = dims_check("ssm_ssd_chunk_scan", a->dims, p.d);
   if (rc != SSM_OK) return rc;
@@ -427,12 +427,24 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   p.x_scale = a->x_row_scale;
   SSM_REQUIRE(a->x_row_scale == nullptr || a->x_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE,
               "ssm_ssd_chunk_scan: x_row_scale needs bfloat16 x (x_dtype=%d)", a->x_dtype);
+  if (a->dx_out) {
+    SSM_REQUIRE(a->dx_x && a->dx_dt && a->dx_xu && a->dx_s1, SSM_ERR_NULL_POINTER,
+                "ssm_ssd_chunk_scan: dx_out needs dx_x, dx_dt, dx_xu and dx_s1");
+    SSM_REQUIRE(aligned_to(a->dx_x, 2) && aligned_to(a->dx_out, a->dx_out_f32 ? 4 : 2) && aligned_to(a->dx_dt, 4) &&
+                    aligned_to(a->dx_xu, 4) && aligned_to(a->dx_s1, 4),
+                SSM_ERR_ALIGNMENT, "ssm_ssd_chunk_scan: a dx_* pointer is not aligned to its element");
+    p.dx.x = a->dx_x; p.dx.dt = a->dx_dt; p.dx.Dk = a->dx_Dskip; p.dx.dx = a->dx_out; p.dx.xu = a->dx_xu; p.dx.s1 = a->dx_s1;
+    p.dx.d_per_p = a->dx_d_per_p ? 1 : 0; p.dx.dx_f32 = a->dx_out_f32 ? 1 : 0; p.dx.round_dtx = a->dx_round_dtx ? 1 : 0;
+  }
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
     g_mfma_launches |= 4;
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
     return SSM_OK;
   }
+  SSM_REQUIRE(a->dx_out == nullptr, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_chunk_scan: dx_out is written by the matrix-core kernel only (bfloat16 x, C and CB, float32 states, "
+              "no z, Dskip or seq_idx, whole chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64)");
   SSM_REQUIRE(a->x_row_scale == nullptr, SSM_ERR_BAD_SHAPE,
               "ssm_ssd_chunk_scan: x_row_scale is taken by the matrix-core kernel only (bfloat16 x, C and CB, "
               "whole chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64)");

@@ -57,6 +57,19 @@ struct SsdPassParams {
   const int *seq_idx;         // (B, L) or null
 };
 
+// In place of y, the matrix-core chunk_scan of the backward's time-reversed pass can finish dx itself: with u its
+// own result at reversed step tau (forward step t = L-1-tau) and dy its operand x,
+//   dx_t = dt_t u + D dy,   xu_t = sum_p x_t u,   s1_t = sum_p round(dt_t x_t) u
+// (what ssm_ssd_bwd_dx computes from u written out in float32).
+struct SsdDxEpilogue {
+  const void *x;              // (B, L, H, P) of the pass's element type, forward time
+  const float *dt;            // (B, L, H)
+  const float *Dk;            // (H,) / (H, P) or null
+  void *dx;                   // (B, L, H, P) float32 or the element type; null: no such epilogue
+  float *xu, *s1;             // (B, L, H)
+  int d_per_p, dx_f32, round_dtx;
+};
+
 struct SsdScanParams {
   const void *CB, *Cm, *x, *z, *prev;
   const float *dt, *dA_cs, *Dk;
@@ -67,6 +80,7 @@ struct SsdScanParams {
   const int *seq_idx;         // (B, L) or null
   int y_dtype;                // x_dtype, or SSM_F32 on request
   const float *x_scale;       // (B, H, nc, Q) or null: x stands for x * scale rounded to x's type (matrix-core kernels only)
+  SsdDxEpilogue dx;
 };
 
 __device__ __forceinline__ void store_any(void *p, int dtype, size_t i, float v) {
@@ -117,6 +131,22 @@ template <> struct Vec8<_Float16> { using type = f16x8_t; };
 template <typename E> using V8 = typename Vec8<E>::type;
 template <typename E>
 __device__ __forceinline__ V8<E> load_frag_e(const void *p) { return *reinterpret_cast<const V8<E> *>(p); }
+// Four neighbouring 16-bit elements (8 bytes, 8-byte aligned) to and from float32.
+template <typename E>
+__device__ __forceinline__ void load4_e(const E *p, float (&v)[4]) {
+  typedef __attribute__((__vector_size__(4 * sizeof(E)))) E vec4_t;
+  const vec4_t r = *reinterpret_cast<const vec4_t *>(p);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = (float)r[j];
+}
+template <typename E>
+__device__ __forceinline__ void store4_e(E *p, const float (&v)[4]) {
+  typedef __attribute__((__vector_size__(4 * sizeof(E)))) E vec4_t;
+  vec4_t r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) r[j] = (E)v[j];
+  *reinterpret_cast<vec4_t *>(p) = r;
+}
 template <typename E>
 __device__ __forceinline__ V8<E> pack8_e(const float (&v)[8]) {
   V8<E> r;

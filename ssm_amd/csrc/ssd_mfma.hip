@@ -289,7 +289,9 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const 
 
 // ----------------------------------------------------------------- chunk_scan
 // One workgroup per (b, c, h); wave w owns row blocks w, nlb-1-w, w+4, ... of 32 rows.
-template <typename E, typename st_t, int PT>
+// DX (1: dx in the element type, 2: in float32): the result is not written; it is the u of the backward's reversed
+// pass and goes straight into dx and the two row sums that need it (SsdDxEpilogue).
+template <typename E, typename st_t, int PT, int DX = 0>
 __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const SsdScanParams p) {
   const SsdDims &d = p.d;
   const int Q = d.chunk, P = 32 * PT, N = d.nstate;
@@ -317,6 +319,18 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   const size_t xrow = (size_t)d.heads * P;                                 // elements between time steps
   const size_t xbase = (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
   const E *xg = reinterpret_cast<const E *>(p.x) + xbase;
+  // The epilogue's reads (x and dt at the chunk's steps in forward time) come at the very end of the workgroup's life
+  // with nothing left to hide them behind: one early read per row and half line brings them near, its value unused.
+  unsigned near0 = 0, near1 = 0;
+  float near2 = 0.0f;
+  if constexpr (DX) {
+    const int rl = threadIdx.x % Q;
+    const size_t row = ((size_t)b * d.len + (d.len - 1 - (c * Q + rl))) * d.heads + h;
+    const unsigned *xr = reinterpret_cast<const unsigned *>(reinterpret_cast<const E *>(p.dx.x) + row * P);
+    near0 = xr[0];
+    near1 = xr[P / 4];
+    near2 = p.dx.dt[row];
+  }
   if (p.x_scale) stage_xT<false, true, E>(xT, xg, xrow, Q, P, nullptr, stride, p.x_scale + cs);
   else stage_xT<false, false, E>(xT, xg, xrow, Q, P, nullptr, stride);
   // The state entering the chunk, [P][N], as bfloat16 in LDS: read once by the workgroup in whole lines (a fragment
@@ -352,70 +366,186 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   float *yf = reinterpret_cast<float *>(p.y) + xbase;
   const bool y_f32 = p.y_dtype == SSM_F32;
 
-  for (int pair = wave; pair < (nlb + 1) / 2; pair += MF_WAVES) {
-    for (int side = 0; side < 2; ++side) {
-      const int lb = side == 0 ? pair : nlb - 1 - pair;
-      if (side == 1 && lb == pair) break;             // odd count: middle block once
-      const int l0 = 32 * lb;
-      f32x16_t acc[PT];
+  // The products are formed transposed (the x / state fragment as the first operand): a lane then holds, for its row
+  // l0 + m of the chunk, channels 32 i + 8 q + 4 g2 + (0..3) in acc[i][4 q + (0..3)], and a row's factors are one
+  // value per lane.  A wave owns at most two row blocks (Q <= 256): it forms both, and once every wave is through
+  // (the staged tiles are free then) turns each into rows through a tile of its own in LDS, so that the epilogue's
+  // reads and writes are whole runs of a row's channels on neighbouring lanes.
+  auto block_of = [&](int lb, f32x16_t (&acc)[PT]) {
+    const int l0 = 32 * lb;
+    const int lrow = l0 + m;                        // this lane's row: as an operand and in the result
 #pragma unroll
-      for (int i = 0; i < PT; ++i) acc[i] = (f32x16_t){0};
-
-      // carried-in state: C[l][:] . S[p][:]
-      const E *crow_p = Cg + (size_t)(l0 + m) * c_stride + 8 * g2;
-      for (int n0 = 0; n0 < N; n0 += 16) {
-        const V8<E> af = load_frag_e<E>(crow_p + n0);
+    for (int i = 0; i < PT; ++i) acc[i] = (f32x16_t){0};
+    // carried-in state: S[p][:] . C[l][:]
+    const E *crow_p = Cg + (size_t)lrow * c_stride + 8 * g2;
+    for (int n0 = 0; n0 < N; n0 += 16) {
+      const V8<E> af = load_frag_e<E>(crow_p + n0);
 #pragma unroll
-        for (int i = 0; i < PT; ++i) acc[i] = mma(af, load_frag_e<E>(Sb + (32 * i + m) * SR + n0 + 8 * g2), acc[i]);
+      for (int i = 0; i < PT; ++i) acc[i] = mma(load_frag_e<E>(Sb + (32 * i + m) * SR + n0 + 8 * g2), af, acc[i]);
+    }
+    const float dal = dAs[lrow];
+    {
+      const float sc = exp2_hw(dal * LOG2E) * ent[lrow];
+#pragma unroll
+      for (int i = 0; i < PT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] *= sc;
+    }
+    // within the chunk: M[l][s] = CB[l][s] exp(dA_l - dA_s) dt_s for s <= l
+    const E *cbrow = CBg + (size_t)lrow * Q + 8 * g2;
+    for (int s0 = 0; s0 < l0 + 32; s0 += 16) {
+      float cb[8];
+      unpack8(load_frag_e<E>(cbrow + s0), cb);
+      const int sbase = s0 + 8 * g2;
+      const float4 a0 = *reinterpret_cast<const float4 *>(dAs + sbase), a1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
+      const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
+      const float das[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+      const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+      float mv[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float v = cb[j] * decay_exp(dal - das[j]) * dtv[j];
+        mv[j] = (sbase + j <= lrow) ? v : 0.0f;
       }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float sc = exp2_hw(dAs[l0 + crow(r, g2)] * LOG2E) * ent[l0 + crow(r, g2)];
-#pragma unroll
-        for (int i = 0; i < PT; ++i) acc[i][r] *= sc;
-      }
-
-      // within the chunk: M[l][s] = CB[l][s] exp(dA_l - dA_s) dt_s for s <= l
-      const int lrow = l0 + m;                       // this lane's row as an A operand
-      const float dal = dAs[lrow];
-      const E *cbrow = CBg + (size_t)lrow * Q + 8 * g2;
-      for (int s0 = 0; s0 < l0 + 32; s0 += 16) {
-        float cb[8];
-        unpack8(load_frag_e<E>(cbrow + s0), cb);
-        const int sbase = s0 + 8 * g2;
-        const float4 a0 = *reinterpret_cast<const float4 *>(dAs + sbase), a1 = *reinterpret_cast<const float4 *>(dAs + sbase + 4);
-        const float4 t0 = *reinterpret_cast<const float4 *>(dts + sbase), t1 = *reinterpret_cast<const float4 *>(dts + sbase + 4);
-        const float das[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        const float dtv[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
-        float mv[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float v = cb[j] * decay_exp(dal - das[j]) * dtv[j];
-          mv[j] = (sbase + j <= lrow) ? v : 0.0f;
-        }
-        const V8<E> af = pack8_e<E>(mv);
-#pragma unroll
-        for (int i = 0; i < PT; ++i) {
-          const V8<E> bf = load_frag_e<E>(xT + xt_off(32 * i + m, sbase, stride));
-          acc[i] = mma(af, bf, acc[i]);
-        }
-      }
-      // epilogue: + D x, gate, store
+      const V8<E> af = pack8_e<E>(mv);
 #pragma unroll
       for (int i = 0; i < PT; ++i) {
-        const int pcol = 32 * i + m;
-        const float Dv = p.Dk ? p.Dk[p.d_per_p ? (size_t)h * P + pcol : (size_t)h] : 0.0f;
+        const V8<E> bf = load_frag_e<E>(xT + xt_off(32 * i + m, sbase, stride));
+        acc[i] = mma(bf, af, acc[i]);
+      }
+    }
+  };
+
+  const int npairs = (nlb + 1) / 2;                  // <= MF_WAVES (checked by the host)
+  const bool has0 = wave < npairs, has1 = has0 && (nlb - 1 - wave) != wave;
+  f32x16_t acc0[PT], acc1[PT];
+  if (has0) block_of(wave, acc0);
+  if (has1) block_of(nlb - 1 - wave, acc1);
+  __syncthreads();                                   // nobody reads the staged tiles any more
+
+  constexpr int SCR = 32 * PT + 4;                   // floats per row of a wave's tile (the pad spreads the banks)
+  constexpr int LPR = 8 * PT, RPI = WAVE / LPR;      // lanes per row, rows per instruction
+  float *scr = reinterpret_cast<float *>(smem) + (size_t)wave * (32 * SCR);
+  const int rsub = lane / LPR, c4 = (lane % LPR) * 4;
+  // Nothing inside the loops over a tile's rows is decided at run time (the options are template arguments of the
+  // lambdas below) and every address is a base the workgroup shares plus a 32-bit byte offset: the reads of all of
+  // a tile's rows are then issued together.
+  using Yes = std::true_type;
+  using No = std::false_type;
+
+  auto to_rows = [&](const f32x16_t (&acc)[PT]) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int l = l0 + crow(r, g2);
-          const size_t at = (size_t)l * xrow + pcol;
-          float v = acc[i][r];
-          if (p.Dk) v = __builtin_fmaf(Dv, (float)xg[at], v);
-          if (zg) v *= silu_f32((float)zg[at]);
-          if (y_f32) yf[at] = v;
-          else yg[at] = (E)v;
+    for (int i = 0; i < PT; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<float4 *>(scr + m * SCR + 32 * i + 8 * q + 4 * g2) =
+            make_float4(acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the wave's own tile: written, now read by other lanes
+  };
+  auto tile_row = [&](int it, float (&v)[4]) {
+    const float4 t4 = *reinterpret_cast<const float4 *>(scr + (it * RPI + rsub) * SCR + c4);
+    v[0] = t4.x; v[1] = t4.y; v[2] = t4.z; v[3] = t4.w;
+  };
+
+  if constexpr (DX) {
+    // dx = dt u + D dy and the two row sums, at the forward-time step of every row.  Row l of the chunk is forward
+    // step t0 + (Q-1-l), t0 the chunk's earliest.
+    const SsdDxEpilogue &e = p.dx;
+    const size_t row0 = ((size_t)b * d.len + (d.len - (size_t)(c + 1) * Q)) * d.heads + h;
+    const E *xf = reinterpret_cast<const E *>(e.x) + row0 * P;
+    const float *dtf = e.dt + row0;
+    float *xuf = e.xu + row0, *s1f = e.s1 + row0;
+    float4 Dp = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (e.Dk) {
+      if (e.d_per_p) Dp = *reinterpret_cast<const float4 *>(e.Dk + (size_t)h * P + c4);
+      else Dp.x = Dp.y = Dp.z = Dp.w = e.Dk[h];
+    }
+    const float Dv4[4] = {Dp.x, Dp.y, Dp.z, Dp.w};
+    const bool rnd = e.round_dtx != 0;
+    auto rows_dx = [&](int lb, const f32x16_t (&acc)[PT]) {
+      to_rows(acc);
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int l = 32 * lb + it * RPI + rsub;
+        const unsigned rowoff = (unsigned)(Q - 1 - l) * (unsigned)d.heads;                    // rows of (B, L, H)
+        const unsigned at = rowoff * (unsigned)P + (unsigned)c4;                             // elements of (B, L, H, P)
+        float v[4], xv[4], dyv[4], dxv[4];
+        tile_row(it, v);
+        const float dtv = *at_bytes<const float>(dtf, rowoff * 4u);
+        load4_e<E>(at_bytes<const E>(xf, at * (unsigned)sizeof(E)), xv);
+        // the pass's own operand is dy (read even without a skip term, whose factor is zero then)
+        load4_e<E>(at_bytes<const E>(xg, ((unsigned)l * (unsigned)xrow + (unsigned)c4) * (unsigned)sizeof(E)), dyv);
+        float xu = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          dxv[j] = __builtin_fmaf(Dv4[j], dyv[j], dtv * v[j]);
+          xu = __builtin_fmaf(xv[j], v[j], xu);
+          const float xt = dtv * xv[j];
+          s1 = __builtin_fmaf(rnd ? (float)(E)xt : xt, v[j], s1);
+        }
+        if constexpr (DX == 2)
+          *at_bytes<float4>(reinterpret_cast<float *>(e.dx) + row0 * P, at * 4u) = make_float4(dxv[0], dxv[1], dxv[2], dxv[3]);
+        else
+          store4_e<E>(at_bytes<E>(reinterpret_cast<E *>(e.dx) + row0 * P, at * (unsigned)sizeof(E)), dxv);
+        xu = lane_run_sum_last<LPR>(xu);
+        s1 = lane_run_sum_last<LPR>(s1);
+        if (lane % LPR == LPR - 1) {
+          *at_bytes<float>(xuf, rowoff * 4u) = xu;
+          *at_bytes<float>(s1f, rowoff * 4u) = s1;
         }
       }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // read before the next tile is written over it
+    };
+    if (has0) rows_dx(wave, acc0);
+    if (has1) rows_dx(nlb - 1 - wave, acc1);
+    asm volatile("" ::"v"(near0), "v"(near1), "v"(near2));      // (the early reads end here)
+  } else {
+    // + D x, gate, store
+    float4 Dp = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (p.Dk) {
+      if (p.d_per_p) Dp = *reinterpret_cast<const float4 *>(p.Dk + (size_t)h * P + c4);
+      else Dp.x = Dp.y = Dp.z = Dp.w = p.Dk[h];
+    }
+    const float Dv4[4] = {Dp.x, Dp.y, Dp.z, Dp.w};
+    auto rows_y = [&](int lb, const f32x16_t (&acc)[PT], auto has_d, auto has_z, auto out_f32) {
+      to_rows(acc);
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int l = 32 * lb + it * RPI + rsub;
+        const unsigned at = (unsigned)l * (unsigned)xrow + (unsigned)c4;
+        float v[4];
+        tile_row(it, v);
+        if constexpr (decltype(has_d)::value) {
+          float xv[4];
+          load4_e<E>(at_bytes<const E>(xg, at * (unsigned)sizeof(E)), xv);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = __builtin_fmaf(Dv4[j], xv[j], v[j]);
+        }
+        if constexpr (decltype(has_z)::value) {
+          float zv[4];
+          load4_e<E>(at_bytes<const E>(zg, at * (unsigned)sizeof(E)), zv);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] *= silu_f32(zv[j]);
+        }
+        if constexpr (decltype(out_f32)::value) *at_bytes<float4>(yf, at * 4u) = make_float4(v[0], v[1], v[2], v[3]);
+        else store4_e<E>(at_bytes<E>(yg, at * (unsigned)sizeof(E)), v);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // read before the next tile is written over it
+    };
+    auto both = [&](auto has_d, auto has_z, auto out_f32) {
+      if (has0) rows_y(wave, acc0, has_d, has_z, out_f32);
+      if (has1) rows_y(nlb - 1 - wave, acc1, has_d, has_z, out_f32);
+    };
+    const int opts = (p.Dk ? 4 : 0) | (zg ? 2 : 0) | (y_f32 ? 1 : 0);
+    switch (opts) {
+      case 0: both(No{}, No{}, No{}); break;
+      case 1: both(No{}, No{}, Yes{}); break;
+      case 2: both(No{}, Yes{}, No{}); break;
+      case 3: both(No{}, Yes{}, Yes{}); break;
+      case 4: both(Yes{}, No{}, No{}); break;
+      case 5: both(Yes{}, No{}, Yes{}); break;
+      case 6: both(Yes{}, Yes{}, No{}); break;
+      default: both(Yes{}, Yes{}, Yes{}); break;
     }
   }
 }
@@ -487,8 +617,31 @@ bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s) {
   if ((p.states_dtype != SSM_F32 && p.states_dtype != p.x_dtype) || (p.z && p.z_dtype != p.x_dtype)) return false;
   if (p.y_dtype != SSM_F32 && p.y_dtype != p.x_dtype) return false;
   if (!aligned_to(p.x, 16) || !aligned_to(p.Cm, 16) || !aligned_to(p.CB, 16) || !aligned_to(p.prev, 16)) return false;
-  const size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 12 + (size_t)d.hdim * (d.nstate + 8) * 2;
+  // the epilogue moves four channels at a time
+  if ((p.y && !aligned_to(p.y, 16)) || (p.z && !aligned_to(p.z, 8))) return false;
+  if (p.dx.dx && (!aligned_to(p.dx.dx, 16) || !aligned_to(p.dx.x, 8))) return false;
+  if ((p.Dk && p.d_per_p && !aligned_to(p.Dk, 16)) || (p.dx.dx && p.dx.Dk && p.dx.d_per_p && !aligned_to(p.dx.Dk, 16))) return false;
+  size_t lds = (size_t)d.hdim * (d.chunk + XT_PAD) * 2 + (size_t)d.chunk * 12 + (size_t)d.hdim * (d.nstate + 8) * 2;
+  // afterwards the same memory holds a tile of 32 rows per wave that has row blocks (two each: chunk <= 256)
+  const size_t tiles = (size_t)((d.chunk / 32 + 1) / 2) * 32 * (d.hdim + 4) * 4;
+  if ((d.chunk / 32 + 1) / 2 > MF_WAVES) return false;
+  if ((size_t)d.chunk * d.heads * d.hdim * 4 >= ((size_t)1 << 31)) return false;     // a chunk's rows in 32-bit byte offsets
+  if (lds < tiles) lds = tiles;
   const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);
+  if (p.dx.dx) {
+    // the backward's own call: bfloat16 operands, float32 states, nothing of the forward's epilogue
+    if (p.x_dtype != SSM_BF16 || p.states_dtype != SSM_F32 || p.z || p.Dk || p.seq_idx) return false;
+#define SSM_LAUNCH_DX(PT, MODE)                                                                            \
+  {                                                                                                        \
+    auto kernel = ssd_chunk_scan_mfma_kernel<__bf16, float, PT, MODE>;                                     \
+    if (allow_dynamic_lds(kernel, lds) != hipSuccess) { (void)hipGetLastError(); return false; }           \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(MF_THREADS), lds, s, p);                                   \
+  }
+    if (d.hdim == 64) { if (p.dx.dx_f32) SSM_LAUNCH_DX(2, 2) else SSM_LAUNCH_DX(2, 1) }
+    else { if (p.dx.dx_f32) SSM_LAUNCH_DX(1, 2) else SSM_LAUNCH_DX(1, 1) }
+#undef SSM_LAUNCH_DX
+    return true;
+  }
 #define SSM_LAUNCH_SC(E, ST, PT)                                                                           \
   {                                                                                                        \
     auto kernel = ssd_chunk_scan_mfma_kernel<E, ST, PT>;                                                   \

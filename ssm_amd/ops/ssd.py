@@ -15,6 +15,7 @@ Shapes: ``x, z, y (B, L, H, P)``; ``dt (B, L, H)``; ``A (H,)``; ``B, C (B, L, G,
 from __future__ import annotations
 
 import math
+import weakref
 from typing import Optional
 
 import torch
@@ -241,7 +242,7 @@ def state_passing(states, dA_chunk_cumsum, initial_states=None, seq_idx=None, ch
 
 
 def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False, seq_idx=None,
-               out_f32=False, x_scale=None):
+               out_f32=False, x_scale=None, dx_epilogue=None):
     """Outputs of every chunk from the state entering it.
 
     Args:
@@ -257,6 +258,10 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
             chunk), and products across sequences inside a chunk are dropped.
         out_f32: Return ``y`` in float32 (the accumulators as they are) instead of ``x.dtype``.
         x_scale: As in :func:`chunk_state` (the skip term ``D x`` takes ``x`` as it is).
+        dx_epilogue: ``(x, dt_rows, D, out_dtype, round_dtx)`` -- the call is the gradient's time-reversed pass
+            (``x`` here is ``dy`` reversed) and finishes ``dx`` itself instead of returning its result ``u``:
+            returns ``(dx, xu, s1)`` as :func:`_bwd_dx` would from ``u`` (for calls :func:`_row_scale_ok` accepts
+            with a head of 32 or 64 channels).
 
     Returns:
         ``y (B, L, H, P)`` in ``x.dtype`` (float32 with ``out_f32``).
@@ -285,7 +290,19 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
             K.check_float(name, t)
     ps, cb = K.cast_c(prev_states, prev_states.dtype), K.cast_c(CB, CB.dtype)
     dtf, daf, Df = K.as_f32_vec(dt), K.as_f32_vec(dA_cumsum), K.as_f32_vec(D)
-    y = torch.empty_like(xc, dtype=torch.float32) if out_f32 else torch.empty_like(xc)
+    y = dxo = None
+    if dx_epilogue is None:
+        y = torch.empty_like(xc, dtype=torch.float32) if out_f32 else torch.empty_like(xc)
+    else:
+        ex, edt, eD, eout, eround = dx_epilogue
+        _need(ex.shape == xc.shape and ex.dtype == xc.dtype and ex.is_contiguous(), "dx_epilogue: x must match the operand.")
+        _need(tuple(edt.shape) == (batch, seqlen, heads) and edt.dtype == torch.float32 and edt.is_contiguous(),
+              "dx_epilogue: dt_rows must be a contiguous float32 (B, L, H) tensor.")
+        _need(eout in (torch.float32, xc.dtype), "dx_epilogue: out_dtype is float32 or the operand's type.")
+        eDf = K.as_f32_vec(eD)
+        dxo = torch.empty(xc.shape, dtype=eout, device=dev)
+        exu = torch.empty(batch, seqlen, heads, dtype=torch.float32, device=dev)
+        es1 = torch.empty_like(exu)
     args = _lib.SsdChunkScanArgs(
         CB=_lib.ptr(cb), Cm=_lib.ptr(Cc), x=_lib.ptr(xc), z=_lib.ptr(zc), prev_states=_lib.ptr(ps),
         dt=_lib.ptr(dtf), dA_cumsum=_lib.ptr(daf), Dskip=_lib.ptr(Df), y=_lib.ptr(y),
@@ -294,8 +311,14 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         states_dtype=_lib.dtype_enum(ps.dtype), z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
         d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), y_f32=int(bool(out_f32)),
         x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)))
+    if dx_epilogue is not None:
+        args.dx_x, args.dx_dt, args.dx_Dskip = _lib.ptr(ex), _lib.ptr(edt), _lib.ptr(eDf)
+        args.dx_out, args.dx_xu, args.dx_s1 = _lib.ptr(dxo), _lib.ptr(exu), _lib.ptr(es1)
+        args.dx_d_per_p = int(eD is not None and eD.ndim == 2)
+        args.dx_out_f32 = int(eout == torch.float32)
+        args.dx_round_dtx = int(bool(eround))
     _lib.call("ssm_ssd_chunk_scan", args, dev)
-    return y
+    return y if dx_epilogue is None else (dxo, exu, es1)
 
 
 def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
@@ -339,23 +362,28 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
     return out
 
 
-_DECAYING = {}        # (data_ptr, version, numel) of an A tensor -> all(A <= 0), so that a persistent parameter is read once
+_DECAYING = {}        # id of an A tensor -> (weak reference, version, all(A <= 0)), so that a persistent parameter is read once
 
 
 def _is_decaying(A):
     """``all(A <= 0)``: what the one-pass kernel assumes (it bounds each factor of a decay by 1; with a growing
     state its results are wrong, while the five kernels keep the upstream kernels' behaviour there).  Reading the
-    answer costs a device synchronisation, so it is remembered per tensor (address and version) and not looked up
-    at all while a stream is being captured, where the caller's word (``fused=True``) or the default is taken."""
+    answer costs a device synchronisation, so it is remembered per tensor object (while that object lives and its
+    version counter stands: an address alone may pass to another tensor) and not looked up at all while a stream is
+    being captured, where the caller's word (``fused=True``) or the default is taken."""
     if torch.cuda.is_current_stream_capturing():
         return True
-    key = (A.data_ptr(), A._version, A.numel())
-    hit = _DECAYING.get(key)
-    if hit is None:
-        if len(_DECAYING) > 4096:
-            _DECAYING.clear()
-        hit = _DECAYING[key] = bool((A.detach() <= 0).all())
-    return hit
+    hit = _DECAYING.get(id(A))
+    if hit is not None and hit[0]() is A and hit[1] == A._version:
+        return hit[2]
+    if len(_DECAYING) > 4096:
+        _DECAYING.clear()
+    answer = bool((A.detach() <= 0).all())
+    try:
+        _DECAYING[id(A)] = (weakref.ref(A), A._version, answer)
+    except TypeError:              # an object that cannot be weakly referenced: not remembered
+        pass
+    return answer
 
 
 def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
@@ -656,7 +684,7 @@ def varlen_states_backward(dstates, x, dt, A, B, cu_seqlens, dt_bias=None, initi
     return dx, ddt, dA, dB, dbias, dinit
 
 
-def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_scale=None):
+def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_scale=None, dx_epilogue=None):
     """``y_t = sum_{s<=t} exp(cs_t - cs_s) <C_t, B_s> w_s x_s + exp(cs_t) C_t . init`` and the state
     after the last step, through chunk_state -> state_passing -> chunk_scan (states in float32).
 
@@ -664,7 +692,8 @@ def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_
     backward's passes that put the state axis in the channel role) is cut into pieces of 64, the width
     the matrix-core kernels are built for.  With ``want_entering`` the states entering the chunks
     ``(B, nc, H, P, N)`` come back as a third result.  ``x_scale (B, H, nc, Q)``: ``x`` stands for ``x * x_scale``
-    rounded to its type (for calls :func:`_row_scale_ok` accepts)."""
+    rounded to its type (for calls :func:`_row_scale_ok` accepts).  ``dx_epilogue``: see :func:`chunk_scan`; the first
+    result then is ``(dx, xu, s1)`` (heads of at most 64 channels)."""
     hd = int(x.shape[-1])
     if x.dtype == torch.bfloat16 and hd > 64 and hd % 64 == 0:
         Q = int(dA_cs.shape[3])
@@ -677,7 +706,7 @@ def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_
         return out + (torch.cat([q[2] for q in parts], dim=3),) if want_entering else out
     states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32, x_scale=x_scale)
     entering, final = state_passing(states, dA_cs[:, :, :, -1].contiguous(), initial_states=init)
-    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, CB=CB, out_f32=True, x_scale=x_scale)
+    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, CB=CB, out_f32=True, x_scale=x_scale, dx_epilogue=dx_epilogue)
     return (y, final, entering) if want_entering else (y, final)
 
 
@@ -1004,14 +1033,19 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     if not fused:
         dyc = dy.to(cd)
         dyr = dyc.flip(1).contiguous()
+    # the reversed pass finishes dx itself where its matrix-core kernel runs: u never goes through memory
+    dx_in_pass = (fused and cd == torch.bfloat16 and xd.dtype == cd and hdim in (32, 64) and _row_scale_ok(xd, Bc, Cc, Q))
+    epilogue = (xd, dte, Df, xd.dtype if grads_in_input_dtype else f32, True) if dx_in_pass else None
     u_r, Gfin, ent_r = _lin_pass(dyr, ones_c, dA_r, Cc.flip(1).contiguous(), Bc.flip(1).contiguous(), dfin,
-                                 want_entering=True)
+                                 want_entering=True, dx_epilogue=epilogue)
     dinit = None
     if init is not None:
         dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin
         if bnd is not None:
             dinit = dinit * (~bnd[:, 0]).to(f32)[:, None, None, None]
-    if fused:
+    if dx_in_pass:
+        dx, xu, s1 = u_r
+    elif fused:
         dx, xu, s1 = _bwd_dx(dod, zd, xd, u_r.contiguous(), dte, Df, cd == torch.bfloat16,
                              grads_io=grads_in_input_dtype)
     else:
