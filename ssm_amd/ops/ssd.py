@@ -881,11 +881,13 @@ def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dA_cs, wdy, xw, f16, r16, groups):
     nstate = int(Bc.shape[-1])
     per = heads // groups
     f32, bf = torch.float32, torch.bfloat16
-    dCB = _bwd_dcb(dyc, xc, dt_c, dA_cs, groups)                                    # (B, nc, G, Q, Q)
-    Bg = Bc.view(batch, nc, Q, groups, nstate).permute(0, 1, 3, 2, 4).to(f32)       # (B, nc, G, Q, N)
-    Cg = Cc.view(batch, nc, Q, groups, nstate).permute(0, 1, 3, 2, 4).to(f32)
-    dB = torch.matmul(dCB.transpose(-1, -2), Cg)
-    dC = torch.matmul(dCB, Bg)
+    # the head-summed matrix is formed in float32 and rounded once: both products then run on the matrix cores with
+    # float32 accumulation (a sum of Q terms whose roundings are independent)
+    dCB = _bwd_dcb(dyc, xc, dt_c, dA_cs, groups).to(bf)                             # (B, nc, G, Q, Q)
+    Bg = Bc.view(batch, nc, Q, groups, nstate).permute(0, 1, 3, 2, 4)               # (B, nc, G, Q, N)
+    Cg = Cc.view(batch, nc, Q, groups, nstate).permute(0, 1, 3, 2, 4)
+    dB = _mm_f32(dCB.transpose(-1, -2), Cg)
+    dC = _mm_f32(dCB, Bg)
 
     def rows(t):           # (B, L, H, P) -> (B, nc, G, Q, per * P)
         return t.view(batch, nc, Q, groups, per * hdim).permute(0, 1, 3, 2, 4)
