@@ -312,7 +312,7 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
   const int *sid = p.seq_idx ? p.seq_idx + (size_t)b * d.len : nullptr;
   const int sid_prev = (sid && c > 0) ? sid[(size_t)c * Q - 1] : 0;
   for (int l = threadIdx.x; l < Q; l += MF_THREADS) {
-    dAs[l] = p.dA_cs[cs + l];
+    dAs[l] = p.dA_cs[cs + l] * LOG2E;              // in units of log 2: the factors below are exp2 of differences
     dts[l] = p.dt[cs + l];
     ent[l] = (sid && sid[(size_t)c * Q + l] != sid_prev) ? 0.0f : 1.0f;
   }
@@ -385,15 +385,16 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
     }
     const float dal = dAs[lrow];
     {
-      const float sc = exp2_hw(dal * LOG2E) * ent[lrow];
+      const float sc = exp2_hw(dal) * ent[lrow];
 #pragma unroll
       for (int i = 0; i < PT; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][r] *= sc;
     }
-    // within the chunk: M[l][s] = CB[l][s] exp(dA_l - dA_s) dt_s for s <= l
+    // within the chunk: M[l][s] = CB[l][s] exp(dA_l - dA_s) dt_s for s <= l (the difference clamped at 0, as the
+    // published kernels do); only the row block's own 32 columns hold any s > l
     const E *cbrow = CBg + (size_t)lrow * Q + 8 * g2;
-    for (int s0 = 0; s0 < l0 + 32; s0 += 16) {
+    auto columns = [&](int s0, auto diagonal) {
       float cb[8];
       unpack8(load_frag_e<E>(cbrow + s0), cb);
       const int sbase = s0 + 8 * g2;
@@ -404,8 +405,8 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
       float mv[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float v = cb[j] * decay_exp(dal - das[j]) * dtv[j];
-        mv[j] = (sbase + j <= lrow) ? v : 0.0f;
+        const float v = cb[j] * exp2_hw(fminf(dal - das[j], 0.0f)) * dtv[j];
+        mv[j] = (!decltype(diagonal)::value || sbase + j <= lrow) ? v : 0.0f;
       }
       const V8<E> af = pack8_e<E>(mv);
 #pragma unroll
@@ -413,7 +414,10 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
         const V8<E> bf = load_frag_e<E>(xT + xt_off(32 * i + m, sbase, stride));
         acc[i] = mma(bf, af, acc[i]);
       }
-    }
+    };
+    for (int s0 = 0; s0 < l0; s0 += 16) columns(s0, std::false_type{});
+    columns(l0, std::true_type{});
+    columns(l0 + 16, std::true_type{});
   };
 
   const int npairs = (nlb + 1) / 2;                  // <= MF_WAVES (checked by the host)
