@@ -171,7 +171,7 @@ template <typename io_t, int VEC, bool HAS_Z, bool STATES_ONLY, bool PARAMS>
 __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const DscanParams p) {
   static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
   constexpr int AV = PARAMS ? VEC : 1;            // decays per lane
-  __shared__ float4 segs[2][DO_WAVES][WAVE];     // a wave's fold per lane: decay product(s), state(s) from zero
+  __shared__ float4 segs[2][DO_WAVES][WAVE];     // a wave's fold per lane: decay product(s), states from zero
   __shared__ float2 right[2][WAVE];
   const int wave = wave_id_uniform(), lane = lane_id();
   const int HP = p.heads * p.proj;
@@ -245,7 +245,8 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
       for (int v = 0; v < VEC; ++v)
         s[v] = __builtin_fmaf(a[v % AV][j], s[v], cur.dt[j] * (PARAMS ? Bc[v] : cur.bq[j].elem(v)) * cur.x[j].elem(v));
     }
-    segs[q][wave][lane] = make_float4(prod[0], prod[AV - 1], s[0], s[VEC - 1]);
+    // (one decay per lane: three words to read per link; two: four)
+    segs[q][wave][lane] = AV == 1 ? make_float4(prod[0], s[0], s[VEC - 1], 0.0f) : make_float4(prod[0], prod[AV - 1], s[0], s[VEC - 1]);
     __syncthreads();
     // the state entering this wave's steps: the folds of the waves before it, from the state entering the round
     float enter[VEC];
@@ -260,7 +261,8 @@ __global__ __launch_bounds__(WAVE *DO_WAVES) void dscan_onepass_kernel(const Dsc
     for (int w = 0; w < wave; ++w) {
       const float4 f = segs[q][w][lane];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) enter[v] = __builtin_fmaf(v % AV == 0 ? f.x : f.y, enter[v], v == 0 ? f.z : f.w);
+      for (int v = 0; v < VEC; ++v)
+        enter[v] = AV == 1 ? __builtin_fmaf(f.x, enter[v], v == 0 ? f.y : f.z) : __builtin_fmaf(v == 0 ? f.x : f.y, enter[v], v == 0 ? f.z : f.w);
     }
     if (wave == DO_WAVES - 1) {
       float leave[VEC];

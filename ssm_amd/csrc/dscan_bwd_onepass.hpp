@@ -33,10 +33,10 @@ struct DboRegs {
 // PARAMS: B and C are held in registers, one value per channel, and their gradients are sums over time like dA's
 // and dD's; each channel of a lane has its own decay.
 template <typename io_t, typename g_t, int VEC, bool HAS_Z, int LPH, bool PARAMS>
-__global__ __launch_bounds__(WAVE *DBO_WAVES, (PARAMS && !HAS_Z && VEC == 1) ? 8 : 4) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
+__global__ __launch_bounds__(WAVE *DBO_WAVES, (PARAMS && !HAS_Z && VEC == 1) ? 8 : 1) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
   static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
   constexpr int AV = PARAMS ? VEC : 1;            // decays per lane
-  __shared__ float4 fwd[2][DBO_WAVES][WAVE];     // a wave's four steps per lane: decay product(s), state(s) from zero
+  __shared__ float4 fwd[2][DBO_WAVES][WAVE];     // a wave's four steps per lane: decay product(s), states from zero
   __shared__ float2 rev[2][DBO_WAVES][WAVE];     // ... and the adjoint (times its decay) from zero
   __shared__ float2 left[2][WAVE];               // the adjoint leaving the round, from wave 0 to everyone's next round
   const int wave = wave_id_uniform(), lane = lane_id();
@@ -133,7 +133,8 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES, (PARAMS && !HAS_Z && VEC == 1) ? 8
         M[v] = a[v % AV][j] * __builtin_fmaf(g0, PARAMS ? Cc[v] : cur.cq[j].elem(v), M[v]);
       }
     }
-    fwd[q][wave][lane] = make_float4(prod[0], prod[AV - 1], s[0], s[VEC - 1]);
+    // (one decay per lane: three words to read per link of the forward chain, one per link of the other; two: four, two)
+    fwd[q][wave][lane] = AV == 1 ? make_float4(prod[0], s[0], s[VEC - 1], 0.0f) : make_float4(prod[0], prod[AV - 1], s[0], s[VEC - 1]);
     rev[q][wave][lane] = make_float2(M[0], M[VEC - 1]);
     __syncthreads();
 #pragma unroll
@@ -151,7 +152,8 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES, (PARAMS && !HAS_Z && VEC == 1) ? 8
     for (int w = 0; w < wave; ++w) {
       const float4 f = fwd[q][w][lane];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) st[v][0] = __builtin_fmaf(v % AV == 0 ? f.x : f.y, st[v][0], v == 0 ? f.z : f.w);
+      for (int v = 0; v < VEC; ++v)
+        st[v][0] = AV == 1 ? __builtin_fmaf(f.x, st[v][0], v == 0 ? f.y : f.z) : __builtin_fmaf(v == 0 ? f.x : f.y, st[v][0], v == 0 ? f.z : f.w);
     }
     // the adjoint entering them: the folds of the waves after it, from the adjoint that left the round before
     float mu[VEC];
@@ -163,10 +165,17 @@ __global__ __launch_bounds__(WAVE *DBO_WAVES, (PARAMS && !HAS_Z && VEC == 1) ? 8
 #pragma unroll
     for (int v = 0; v < VEC; ++v) mu[v] = mu_left[v];
     for (int w = DBO_WAVES - 1; w > wave; --w) {
-      const float2 pr = *reinterpret_cast<const float2 *>(&fwd[q][w][lane]);      // the decay products
+      float pr0, pr1;                                                                 // the decay products
+      if constexpr (AV == 1) {
+        pr0 = pr1 = fwd[q][w][lane].x;
+      } else {
+        const float2 pr = *reinterpret_cast<const float2 *>(&fwd[q][w][lane]);
+        pr0 = pr.x;
+        pr1 = pr.y;
+      }
       const float2 f = rev[q][w][lane];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) mu[v] = __builtin_fmaf(v % AV == 0 ? pr.x : pr.y, mu[v], v == 0 ? f.x : f.y);
+      for (int v = 0; v < VEC; ++v) mu[v] = __builtin_fmaf(v % AV == 0 ? pr0 : pr1, mu[v], v == 0 ? f.x : f.y);
     }
     if (wave == 0) {
 #pragma unroll
