@@ -33,7 +33,7 @@ struct DboRegs {
 // PARAMS: B and C are held in registers, one value per channel, and their gradients are sums over time like dA's
 // and dD's; each channel of a lane has its own decay.
 template <typename io_t, typename g_t, int VEC, bool HAS_Z, int LPH, bool PARAMS>
-__global__ __launch_bounds__(WAVE *DBO_WAVES, (PARAMS && !HAS_Z && VEC == 1) ? 8 : 1) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
+__global__ __launch_bounds__(WAVE *DBO_WAVES) void dscan_bwd_onepass_kernel(const DscanBwdParams p) {
   static_assert(sizeof(io_t) * VEC == 4, "a lane's vector is one register");
   constexpr int AV = PARAMS ? VEC : 1;            // decays per lane
   __shared__ float4 fwd[2][DBO_WAVES][WAVE];     // a wave's four steps per lane: decay product(s), states from zero
