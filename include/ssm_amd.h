@@ -387,6 +387,9 @@ typedef struct ssm_ssd_chunk_state_args {
   const float *x_row_scale; /* (B,H,nc,Q) or NULL: x stands for x * scale rounded to x's dtype, as if that tensor had
                                been written first (the backward puts the step into the operand this way); only the
                                matrix-core kernel takes it, and only for bfloat16 x: an error otherwise */
+  int32_t x_time_reversed;  /* nonzero: the call walks the sequence backwards in time (B, dt, dA_cumsum given reversed)
+                               while x is given in forward time: step tau reads x's row L-1-tau, and no reversed copy
+                               of x is needed.  Matrix-core kernel only: an error otherwise */
 } ssm_ssd_chunk_state_args;
 size_t ssm_ssd_chunk_state_workspace_bytes(const ssm_ssd_dims *dims);
 int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *args, void *hip_stream);
@@ -434,6 +437,8 @@ typedef struct ssm_ssd_chunk_scan_args {
   void *dx_out;             /* (B,L,H,P) float32 if dx_out_f32 else x dtype; NULL: the ordinary call */
   float *dx_xu, *dx_s1;     /* (B,L,H) */
   int32_t dx_d_per_p, dx_out_f32, dx_round_dtx;
+  int32_t x_time_reversed;  /* as in ssm_ssd_chunk_state_args (C, CB, prev_states, dt, dA_cumsum given reversed, y or dx_*
+                               as without it); not together with Dskip */
 } ssm_ssd_chunk_scan_args;
 int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *args, void *hip_stream);
 

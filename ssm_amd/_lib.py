@@ -137,7 +137,7 @@ class SsdChunkStateArgs(C.Structure):
     _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("states", _vp),
                 ("workspace", _vp), ("workspace_bytes", C.c_size_t), ("dims", SsdDims),
                 ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("force_generic", _i32),
-                ("seq_idx", _vp), ("x_row_scale", _vp)]
+                ("seq_idx", _vp), ("x_row_scale", _vp), ("x_time_reversed", _i32)]
 
 
 class SsdStatePassingArgs(C.Structure):
@@ -152,7 +152,8 @@ class SsdChunkScanArgs(C.Structure):
                 ("x_dtype", _i32), ("c_dtype", _i32), ("cb_dtype", _i32), ("states_dtype", _i32),
                 ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32), ("seq_idx", _vp),
                 ("y_f32", _i32), ("x_row_scale", _vp), ("dx_x", _vp), ("dx_dt", _vp), ("dx_Dskip", _vp), ("dx_out", _vp),
-                ("dx_xu", _vp), ("dx_s1", _vp), ("dx_d_per_p", _i32), ("dx_out_f32", _i32), ("dx_round_dtx", _i32)]
+                ("dx_xu", _vp), ("dx_s1", _vp), ("dx_d_per_p", _i32), ("dx_out_f32", _i32), ("dx_round_dtx", _i32),
+                ("x_time_reversed", _i32)]
 
 
 class SsdChunkStateVarlenArgs(C.Structure):

@@ -356,6 +356,7 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   p.x_dtype = a->x_dtype; p.b_dtype = a->b_dtype; p.states_dtype = a->states_dtype;
   p.seq_idx = a->seq_idx;
   p.x_scale = a->x_row_scale;
+  p.x_reversed = a->x_time_reversed ? 1 : 0;
   // (float16 is left out: the conversion that rounds the product does not keep float16 subnormals, which a tensor
   // written beforehand would hold)
   SSM_REQUIRE(a->x_row_scale == nullptr || a->x_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE,
@@ -366,6 +367,7 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
     return SSM_OK;
   }
+  SSM_REQUIRE(!a->x_time_reversed, SSM_ERR_BAD_SHAPE, "ssm_ssd_chunk_state: x_time_reversed is taken by the matrix-core kernel only");
   SSM_REQUIRE(a->x_row_scale == nullptr, SSM_ERR_BAD_SHAPE,
               "ssm_ssd_chunk_state: x_row_scale is taken by the matrix-core kernel only (bfloat16 x and B, whole "
               "chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64, a workspace)");
@@ -425,6 +427,7 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   p.seq_idx = a->seq_idx;
   p.y_dtype = a->y_f32 ? SSM_F32 : a->x_dtype;
   p.x_scale = a->x_row_scale;
+  p.x_reversed = a->x_time_reversed ? 1 : 0;
   SSM_REQUIRE(a->x_row_scale == nullptr || a->x_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE,
               "ssm_ssd_chunk_scan: x_row_scale needs bfloat16 x (x_dtype=%d)", a->x_dtype);
   if (a->dx_out) {
@@ -442,6 +445,8 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
     return SSM_OK;
   }
+  SSM_REQUIRE(!a->x_time_reversed, SSM_ERR_BAD_SHAPE,
+              "ssm_ssd_chunk_scan: x_time_reversed is taken by the matrix-core kernel only, and not together with Dskip");
   SSM_REQUIRE(a->dx_out == nullptr, SSM_ERR_BAD_SHAPE,
               "ssm_ssd_chunk_scan: dx_out is written by the matrix-core kernel only (bfloat16 x, C and CB, float32 states, "
               "no z, Dskip or seq_idx, whole chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64)");

@@ -43,6 +43,7 @@ struct SsdStateParams {
   int x_dtype, b_dtype, states_dtype;
   const int *seq_idx;         // (B, L) or null
   const float *x_scale;       // (B, H, nc, Q) or null: x stands for x * scale rounded to x's type (matrix-core kernels only)
+  int x_reversed;             // x is given in forward time while the call walks reversed time: step tau reads row L-1-tau
 };
 
 struct SsdPassParams {
@@ -81,6 +82,7 @@ struct SsdScanParams {
   int y_dtype;                // x_dtype, or SSM_F32 on request
   const float *x_scale;       // (B, H, nc, Q) or null: x stands for x * scale rounded to x's type (matrix-core kernels only)
   SsdDxEpilogue dx;
+  int x_reversed;             // as in SsdStateParams
 };
 
 __device__ __forceinline__ void store_any(void *p, int dtype, size_t i, float v) {

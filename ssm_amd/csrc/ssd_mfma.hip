@@ -35,7 +35,7 @@ __device__ __forceinline__ int xt_off(int p, int l, int stride) {
 // PRE: row l is first multiplied by pre[l] (global memory, the chunk's Q values) and rounded to E -- the operand
 // then is exactly the tensor round(x * pre) that a separate launch would have written.
 template <bool WEIGHTED, bool PRE, typename E>
-__device__ __forceinline__ void stage_xT(E *xT, const E *x, size_t row_stride, int Q, int P,
+__device__ __forceinline__ void stage_xT(E *xT, const E *x, long row_stride, int Q, int P,
                                          const float *w_lds, int stride, const float *pre = nullptr) {
   const int pblocks = P >> 3;
   const int nblocks = (Q >> 3) * pblocks;
@@ -44,7 +44,7 @@ __device__ __forceinline__ void stage_xT(E *xT, const E *x, size_t row_stride, i
     float v[8][8];
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const V8<E> raw = load_frag_e<E>(x + (size_t)(lb * 8 + r) * row_stride + pb * 8);
+      const V8<E> raw = load_frag_e<E>(x + (long)(lb * 8 + r) * row_stride + pb * 8);
       const float w = WEIGHTED ? w_lds[lb * 8 + r] : 1.0f;
       const float pr = PRE ? pre[lb * 8 + r] : 1.0f;
 #pragma unroll
@@ -256,9 +256,13 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_state_mfma_kernel(const 
   for (int l = threadIdx.x; l < Q; l += MF_THREADS)
     w[l] = (sid && sid[l] != sid_last) ? 0.0f : decay_exp(last - p.dA_cs[cs + l]) * p.dt[cs + l];
   __syncthreads();
-  const E *xg = reinterpret_cast<const E *>(p.x) + (((size_t)b * d.len + (size_t)c * Q) * d.heads + h) * P;
-  if (p.x_scale) stage_xT<true, true, E>(xT, xg, (size_t)d.heads * P, Q, P, w, stride, p.x_scale + cs);
-  else stage_xT<true, false, E>(xT, xg, (size_t)d.heads * P, Q, P, w, stride);
+  // the chunk's first row and the step from row to row (backwards from the mirrored row when x is in forward time
+  // and the call in reversed time)
+  const size_t first = p.x_reversed ? (size_t)d.len - 1 - (size_t)c * Q : (size_t)c * Q;
+  const long xstep = p.x_reversed ? -(long)d.heads * P : (long)d.heads * P;
+  const E *xg = reinterpret_cast<const E *>(p.x) + (((size_t)b * d.len + first) * d.heads + h) * P;
+  if (p.x_scale) stage_xT<true, true, E>(xT, xg, xstep, Q, P, w, stride, p.x_scale + cs);
+  else stage_xT<true, false, E>(xT, xg, xstep, Q, P, w, stride);
   __syncthreads();
 
   const int g2 = lane >> 5, m = lane & 31;
@@ -331,8 +335,13 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
     near1 = xr[P / 4];
     near2 = p.dx.dt[row];
   }
-  if (p.x_scale) stage_xT<false, true, E>(xT, xg, xrow, Q, P, nullptr, stride, p.x_scale + cs);
-  else stage_xT<false, false, E>(xT, xg, xrow, Q, P, nullptr, stride);
+  {
+    // (the rows of the mirrored chunk, backwards, when x is in forward time and the call in reversed time)
+    const E *xs = p.x_reversed ? reinterpret_cast<const E *>(p.x) + (((size_t)b * d.len + (d.len - 1 - (size_t)c * Q)) * d.heads + h) * P : xg;
+    const long xstep = p.x_reversed ? -(long)xrow : (long)xrow;
+    if (p.x_scale) stage_xT<false, true, E>(xT, xs, xstep, Q, P, nullptr, stride, p.x_scale + cs);
+    else stage_xT<false, false, E>(xT, xs, xstep, Q, P, nullptr, stride);
+  }
   // The state entering the chunk, [P][N], as bfloat16 in LDS: read once by the workgroup in whole lines (a fragment
   // read straight from memory, lane = row, touches 32 lines for 32 bytes each, and every row block would read it again).
   E *Sb = reinterpret_cast<E *>(ent + Q);                       // [P][N + 8]
@@ -457,6 +466,7 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
     const SsdDxEpilogue &e = p.dx;
     const size_t row0 = ((size_t)b * d.len + (d.len - (size_t)(c + 1) * Q)) * d.heads + h;
     const E *xf = reinterpret_cast<const E *>(e.x) + row0 * P;
+    const E *dyg = p.x_reversed ? reinterpret_cast<const E *>(p.x) + row0 * P : xg;      // dy in forward time: x's rows
     const float *dtf = e.dt + row0;
     float *xuf = e.xu + row0, *s1f = e.s1 + row0;
     float4 Dp = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -478,7 +488,7 @@ __global__ __launch_bounds__(MF_THREADS) void ssd_chunk_scan_mfma_kernel(const S
         const float dtv = *at_bytes<const float>(dtf, rowoff * 4u);
         load4_e<E>(at_bytes<const E>(xf, at * (unsigned)sizeof(E)), xv);
         // the pass's own operand is dy (read even without a skip term, whose factor is zero then)
-        load4_e<E>(at_bytes<const E>(xg, ((unsigned)l * (unsigned)xrow + (unsigned)c4) * (unsigned)sizeof(E)), dyv);
+        load4_e<E>(at_bytes<const E>(dyg, (p.x_reversed ? at : (unsigned)l * (unsigned)xrow + (unsigned)c4) * (unsigned)sizeof(E)), dyv);
         float xu = 0.0f, s1 = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -629,6 +639,7 @@ bool ssd_chunk_scan_mfma(const SsdScanParams &p, hipStream_t s) {
   // afterwards the same memory holds a tile of 32 rows per wave that has row blocks (two each: chunk <= 256)
   const size_t tiles = (size_t)((d.chunk / 32 + 1) / 2) * 32 * (d.hdim + 4) * 4;
   if ((d.chunk / 32 + 1) / 2 > MF_WAVES) return false;
+  if (p.x_reversed && p.Dk) return false;            // the skip term reads x at the call's own rows
   if ((size_t)d.chunk * d.heads * d.hdim * 4 >= ((size_t)1 << 31)) return false;     // a chunk's rows in 32-bit byte offsets
   if (lds < tiles) lds = tiles;
   const unsigned grid = (unsigned)((size_t)d.batch * d.nchunks * d.heads);

@@ -149,7 +149,8 @@ def _row_scale_ok(x, Bm, Cm, chunk_size):
             and (hdim == 32 or hdim % 64 == 0))
 
 
-def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=False, seq_idx=None, x_scale=None):
+def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=False, seq_idx=None, x_scale=None,
+                x_reversed=False):
     """Contribution of each chunk to the state at its end.
 
     Args:
@@ -162,6 +163,8 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
             sequence than the chunk's last step add nothing.
         x_scale: Optional ``(B, H, nc, Q)`` float32: ``x`` stands for ``x * x_scale`` rounded to ``x.dtype`` (only
             for calls :func:`_row_scale_ok` accepts).
+        x_reversed: The call walks the sequence backwards in time (``B``, ``dt``, ``dA_cumsum`` given reversed) while
+            ``x`` is given in forward time (same calls).
 
     Returns:
         ``states (B, nc, H, P, N)``.
@@ -187,7 +190,8 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
         workspace=_lib.ptr(ws), workspace_bytes=nbytes,
         dims=dims, x_dtype=_lib.dtype_enum(xc.dtype),
         b_dtype=_lib.dtype_enum(Bc.dtype), states_dtype=_lib.dtype_enum(states_dtype),
-        force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)))
+        force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)),
+        x_time_reversed=int(bool(x_reversed)))
     _lib.call("ssm_ssd_chunk_state", args, dev)
     return states
 
@@ -242,7 +246,7 @@ def state_passing(states, dA_chunk_cumsum, initial_states=None, seq_idx=None, ch
 
 
 def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, force_generic=False, seq_idx=None,
-               out_f32=False, x_scale=None, dx_epilogue=None):
+               out_f32=False, x_scale=None, dx_epilogue=None, x_reversed=False):
     """Outputs of every chunk from the state entering it.
 
     Args:
@@ -258,6 +262,7 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
             chunk), and products across sequences inside a chunk are dropped.
         out_f32: Return ``y`` in float32 (the accumulators as they are) instead of ``x.dtype``.
         x_scale: As in :func:`chunk_state` (the skip term ``D x`` takes ``x`` as it is).
+        x_reversed: As in :func:`chunk_state` (``C``, ``CB``, ``prev_states`` given reversed as well; not with ``D``).
         dx_epilogue: ``(x, dt_rows, D, out_dtype, round_dtx)`` -- the call is the gradient's time-reversed pass
             (``x`` here is ``dy`` reversed) and finishes ``dx`` itself instead of returning its result ``u``:
             returns ``(dx, xu, s1)`` as :func:`_bwd_dx` would from ``u`` (for calls :func:`_row_scale_ok` accepts
@@ -310,7 +315,7 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         c_dtype=_lib.dtype_enum(Cc.dtype), cb_dtype=_lib.dtype_enum(cb.dtype),
         states_dtype=_lib.dtype_enum(ps.dtype), z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
         d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), y_f32=int(bool(out_f32)),
-        x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)))
+        x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)), x_time_reversed=int(bool(x_reversed)))
     if dx_epilogue is not None:
         args.dx_x, args.dx_dt, args.dx_Dskip = _lib.ptr(ex), _lib.ptr(edt), _lib.ptr(eDf)
         args.dx_out, args.dx_xu, args.dx_s1 = _lib.ptr(dxo), _lib.ptr(exu), _lib.ptr(es1)
@@ -684,7 +689,8 @@ def varlen_states_backward(dstates, x, dt, A, B, cu_seqlens, dt_bias=None, initi
     return dx, ddt, dA, dB, dbias, dinit
 
 
-def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_scale=None, dx_epilogue=None):
+def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_scale=None, dx_epilogue=None,
+              x_reversed=False):
     """``y_t = sum_{s<=t} exp(cs_t - cs_s) <C_t, B_s> w_s x_s + exp(cs_t) C_t . init`` and the state
     after the last step, through chunk_state -> state_passing -> chunk_scan (states in float32).
 
@@ -693,20 +699,22 @@ def _lin_pass(x, w_c, dA_cs, Bm, Cm, init=None, want_entering=False, CB=None, x_
     the matrix-core kernels are built for.  With ``want_entering`` the states entering the chunks
     ``(B, nc, H, P, N)`` come back as a third result.  ``x_scale (B, H, nc, Q)``: ``x`` stands for ``x * x_scale``
     rounded to its type (for calls :func:`_row_scale_ok` accepts).  ``dx_epilogue``: see :func:`chunk_scan`; the first
-    result then is ``(dx, xu, s1)`` (heads of at most 64 channels)."""
+    result then is ``(dx, xu, s1)`` (heads of at most 64 channels).  ``x_reversed``: everything but ``x`` is given
+    reversed in time, ``x`` in forward time (same calls)."""
     hd = int(x.shape[-1])
     if x.dtype == torch.bfloat16 and hd > 64 and hd % 64 == 0:
         Q = int(dA_cs.shape[3])
         CB = bmm_chunk(Cm, Bm, Q, causal=True, output_dtype=x.dtype)          # the same for every piece
         parts = [_lin_pass(x[..., k:k + 64].contiguous(), w_c, dA_cs, Bm, Cm,
                            None if init is None else init[:, :, k:k + 64].contiguous(), want_entering, CB=CB,
-                           x_scale=x_scale)
+                           x_scale=x_scale, x_reversed=x_reversed)
                  for k in range(0, hd, 64)]
         out = (torch.cat([q[0] for q in parts], dim=-1), torch.cat([q[1] for q in parts], dim=2))
         return out + (torch.cat([q[2] for q in parts], dim=3),) if want_entering else out
-    states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32, x_scale=x_scale)
+    states = chunk_state(Bm, x, w_c, dA_cs, states_dtype=torch.float32, x_scale=x_scale, x_reversed=x_reversed)
     entering, final = state_passing(states, dA_cs[:, :, :, -1].contiguous(), initial_states=init)
-    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, CB=CB, out_f32=True, x_scale=x_scale, dx_epilogue=dx_epilogue)
+    y = chunk_scan(Bm, Cm, x, w_c, dA_cs, entering, CB=CB, out_f32=True, x_scale=x_scale, dx_epilogue=dx_epilogue,
+                   x_reversed=x_reversed)
     return (y, final, entering) if want_entering else (y, final)
 
 
@@ -1005,6 +1013,8 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
                and (hdim * nstate) % 4 == 0 and xc.is_contiguous() and Bc.is_contiguous() and Cc.is_contiguous())
     dD = None
     wdy = xw = None
+    # the reversed pass reads dy in forward time where its matrix-core kernels run: no reversed copy is written
+    rev_in_place = fused and chunked and xd.dtype == cd and _row_scale_ok(xd, Bc, Cc, Q)
     if fused and chunked:
         # the rows of the two products across chunk boundaries leave the gate kernel with their weights on:
         # dy_l exp(cs_l) for dC, x_s dt_s exp(cs'_s) for dB, cs' the running sum of the reversed pass at that step
@@ -1012,8 +1022,8 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
         if not prepared:
             w_dy = torch.exp(blh(dA_cs)).contiguous()
             w_x = (dte * torch.exp(blh(dA_r)).flip(1)).contiguous()
-        dyc, dyr, dz, s2, dyx, wdy, xw = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, w_dy=w_dy, w_x=w_x,
-                                                     grads_io=grads_in_input_dtype)
+        dyc, dyr, dz, s2, dyx, wdy, xw = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, want_rev=not rev_in_place,
+                                                     w_dy=w_dy, w_x=w_x, grads_io=grads_in_input_dtype)
     elif fused:
         dyc, dyr, dz, s2, dyx = _bwd_gate(dod, zd, xd, ypre.contiguous(), Df, cd, grads_io=grads_in_input_dtype)
     if fused:
@@ -1038,8 +1048,9 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     # the reversed pass finishes dx itself where its matrix-core kernel runs: u never goes through memory
     dx_in_pass = (fused and cd == torch.bfloat16 and xd.dtype == cd and hdim in (32, 64) and _row_scale_ok(xd, Bc, Cc, Q))
     epilogue = (xd, dte, Df, xd.dtype if grads_in_input_dtype else f32, True) if dx_in_pass else None
-    u_r, Gfin, ent_r = _lin_pass(dyr, ones_c, dA_r, Cc.flip(1).contiguous(), Bc.flip(1).contiguous(), dfin,
-                                 want_entering=True, dx_epilogue=epilogue)
+    u_r, Gfin, ent_r = _lin_pass(dyc if rev_in_place else dyr, ones_c, dA_r, Cc.flip(1).contiguous(),
+                                 Bc.flip(1).contiguous(), dfin, want_entering=True, dx_epilogue=epilogue,
+                                 x_reversed=rev_in_place)
     dinit = None
     if init is not None:
         dinit = torch.exp(dte[:, 0] * Af[None])[:, :, None, None] * Gfin

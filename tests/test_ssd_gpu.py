@@ -850,3 +850,36 @@ def test_sign_of_A_is_remembered_per_tensor_not_per_address():
     assert ops_ssd._is_decaying(decay)            # from the cache
     decay.neg_()                                  # the same object, changed in place
     assert not ops_ssd._is_decaying(decay)
+
+
+@pytest.mark.parametrize("shape,Q", [((2, 256, 3, 64, 1, 32), 64), ((1, 512, 4, 32, 2, 16), 256), ((2, 192, 2, 128, 1, 64), 96)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_reversed_pass_reads_its_operand_in_forward_time(shape, Q):
+    """``x_reversed``: a pass over reversed time given ``x`` in forward time equals, to the bit, the pass given the
+    reversed copy -- its result, the states, and ``dx`` with its row sums when the kernel finishes those."""
+    from ssm_amd.ops import ssd as ops_ssd
+    b, l, h, p, g, n = shape
+    gen = torch.Generator().manual_seed(l + h + 2)
+    bf = torch.bfloat16
+    x = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
+    dy = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
+    Br = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
+    Cr = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
+    dt = (torch.rand(b, l, h, generator=gen) * 0.2).cuda()
+    A = -(torch.rand(h, generator=gen) * 4 + 0.1).cuda()
+    D = torch.randn(h, generator=gen).cuda()
+    dfin = torch.randn(b, h, p, n, generator=gen).cuda()
+    dA_cs, dt_c = ops_ssd.chunk_cumsum(dt, A, Q)
+    ones = torch.ones_like(dt_c)
+    want = ops_ssd._lin_pass(dy.flip(1).contiguous(), ones, dA_cs, Br, Cr, dfin, want_entering=True)
+    got = ops_ssd._lin_pass(dy, ones, dA_cs, Br, Cr, dfin, want_entering=True, x_reversed=True)
+    for a, w, name in zip(got, want, ("result", "final state", "entering states")):
+        assert torch.equal(a, w), name
+    if p <= 64:
+        ep = (x, dt, D, bf, True)
+        want = ops_ssd._lin_pass(dy.flip(1).contiguous(), ones, dA_cs, Br, Cr, dfin, want_entering=True, dx_epilogue=ep)
+        got = ops_ssd._lin_pass(dy, ones, dA_cs, Br, Cr, dfin, want_entering=True, dx_epilogue=ep, x_reversed=True)
+        for a, w, name in zip(got[0], want[0], ("dx", "xu", "s1")):
+            assert torch.equal(a, w), name
+    with pytest.raises(Exception, match="x_time_reversed"):
+        ops_ssd.chunk_state(Br.float(), dy.float(), ones, dA_cs, x_reversed=True)
