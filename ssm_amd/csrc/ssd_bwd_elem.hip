@@ -295,29 +295,49 @@ struct DtParams {
   float lo, hi;
 };
 
+// A workgroup takes 16 neighbouring heads of one (batch, chunk) and cuts the chunk into 16 segments: thread
+// (head, segment) first adds up its segment's differences s1 - s2, the segments' sums meet in LDS, and from the
+// running sum at its segment's start the thread walks its steps.  (One thread per chunk walked 256 dependent steps
+// while 20 workgroups were all the launch had.)
+constexpr int DT_HEADS = 16, DT_SEGS = EB_THREADS / DT_HEADS;
+
 __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_dt_kernel(const DtParams p) {
-  constexpr int G = 8;
-  const size_t gid = (size_t)blockIdx.x * EB_THREADS + threadIdx.x;
-  if (gid >= (size_t)p.batch * p.nchunks * p.heads) return;
-  const int h = (int)(gid % p.heads);
-  const int c = (int)((gid / p.heads) % p.nchunks);
-  const int b = (int)(gid / ((size_t)p.heads * p.nchunks));
-  const float Ah = p.A[h], bias = p.bias ? p.bias[h] : 0.0f;
-  const size_t row0 = ((size_t)b * p.len + (size_t)c * p.chunk) * p.heads + h;
+  __shared__ float seg_sum[DT_SEGS][DT_HEADS], seg_dA[DT_SEGS][DT_HEADS], seg_db[DT_SEGS][DT_HEADS];
+  const int hh = threadIdx.x % DT_HEADS, sg = threadIdx.x / DT_HEADS;
+  const int hblocks = (p.heads + DT_HEADS - 1) / DT_HEADS;
+  const int hb = blockIdx.x % hblocks;
+  const int c = (blockIdx.x / hblocks) % p.nchunks;
+  const int b = blockIdx.x / (hblocks * p.nchunks);
+  const int h = hb * DT_HEADS + hh;
+  const bool live = h < p.heads;
+  const int hc = live ? h : p.heads - 1;                       // (a lane past the last head reads the last head's values)
+  const int seg_len = (p.chunk + DT_SEGS - 1) / DT_SEGS;
+  const int l_begin = min(sg * seg_len, p.chunk), l_end = min(l_begin + seg_len, p.chunk);
+  const float Ah = p.A[hc], bias = p.bias ? p.bias[hc] : 0.0f;
+  const size_t row0 = ((size_t)b * p.len + (size_t)c * p.chunk) * p.heads + hc;
+  float mine = 0.0f;
+  for (int l = l_begin; l < l_end; ++l) {
+    const size_t at = row0 + (size_t)l * p.heads;
+    mine += p.s1[at] - p.s2[at];
+  }
+  seg_sum[sg][hh] = mine;
   float q;
   if (c == 0) {
-    q = p.W0 ? p.W0[(size_t)b * p.heads + h] : 0.0f;
+    q = p.W0 ? p.W0[(size_t)b * p.heads + hc] : 0.0f;
   } else {
     float a_first = exp2_hw(p.dte[row0] * Ah * LOG2E);
     if (p.first && p.first[(size_t)b * p.len + (size_t)c * p.chunk]) a_first = 0.0f;
-    q = a_first * p.anchor[((size_t)b * (p.nchunks - 1) + (c - 1)) * p.heads + h];
+    q = a_first * p.anchor[((size_t)b * (p.nchunks - 1) + (c - 1)) * p.heads + hc];
   }
+  __syncthreads();
+  for (int k = 0; k < sg; ++k) q += seg_sum[k][hh];
   float dA = 0.0f, db = 0.0f;
-  for (int l0 = 0; l0 < p.chunk; l0 += G) {
+  constexpr int G = 4;
+  for (int l0 = l_begin; l0 < l_end; l0 += G) {
     float d[G], xu[G], dte[G], raw[G];
 #pragma unroll
     for (int k = 0; k < G; ++k) {
-      const size_t at = row0 + (size_t)min(l0 + k, p.chunk - 1) * p.heads;
+      const size_t at = row0 + (size_t)min(l0 + k, l_end - 1) * p.heads;
       d[k] = p.s1[at] - p.s2[at];
       xu[k] = p.xu[at];
       dte[k] = p.dte[at];
@@ -325,7 +345,7 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_dt_kernel(const DtParams p
     }
 #pragma unroll
     for (int k = 0; k < G; ++k) {
-      if (l0 + k < p.chunk) {
+      if (l0 + k < l_end) {
         const float ddte = __builtin_fmaf(Ah, q, xu[k]);
         dA = __builtin_fmaf(dte[k], q, dA);
         q += d[k];
@@ -335,13 +355,25 @@ __global__ __launch_bounds__(EB_THREADS) void ssd_bwd_dt_kernel(const DtParams p
           slope = sigmoid_f32(raw[k]);
         }
         const float g = (v >= p.lo && v <= p.hi) ? ddte * slope : 0.0f;
-        p.ddt[row0 + (size_t)(l0 + k) * p.heads] = g;
+        if (live) p.ddt[row0 + (size_t)(l0 + k) * p.heads] = g;
         db += g;
       }
     }
   }
-  p.dA_part[gid] = dA;
-  p.db_part[gid] = db;
+  seg_dA[sg][hh] = dA;
+  seg_db[sg][hh] = db;
+  __syncthreads();
+  if (sg == 0 && live) {
+    float sa = 0.0f, sb = 0.0f;
+#pragma unroll
+    for (int k = 0; k < DT_SEGS; ++k) {
+      sa += seg_dA[k][hh];
+      sb += seg_db[k][hh];
+    }
+    const size_t gid = ((size_t)b * p.nchunks + c) * p.heads + h;
+    p.dA_part[gid] = sa;
+    p.db_part[gid] = sb;
+  }
 }
 
 // Everything the backward derives from the raw steps alone, one wavefront per (b, h, chunk): the effective step
@@ -573,10 +605,10 @@ extern "C" int ssm_ssd_bwd_dt(const ssm_ssd_bwd_dt_args *a, void *hip_stream) {
   p.dt_raw = a->dt_raw; p.first = a->first_step; p.ddt = a->ddt; p.dA_part = a->dA_part; p.db_part = a->dbias_part;
   p.batch = a->batch; p.len = a->seqlen; p.heads = a->heads; p.chunk = a->chunk; p.nchunks = a->seqlen / a->chunk;
   p.dt_dtype = a->dt_dtype; p.softplus = a->dt_softplus ? 1 : 0; p.lo = a->dt_min; p.hi = a->dt_max;
-  const size_t total = (size_t)p.batch * p.nchunks * p.heads;
+  const size_t total = (size_t)p.batch * p.nchunks * ((p.heads + DT_HEADS - 1) / DT_HEADS);
   SSM_REQUIRE(total < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_bwd_dt: too many (batch, chunk, head) triples");
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  hipLaunchKernelGGL(ssd_bwd_dt_kernel, dim3((unsigned)((total + EB_THREADS - 1) / EB_THREADS)), dim3(EB_THREADS), 0, s, p);
+  hipLaunchKernelGGL(ssd_bwd_dt_kernel, dim3((unsigned)total), dim3(EB_THREADS), 0, s, p);
   SSM_CHECK_LAUNCH("ssm_ssd_bwd_dt");
   return SSM_OK;
 }
