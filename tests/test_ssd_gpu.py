@@ -883,3 +883,33 @@ def test_reversed_pass_reads_its_operand_in_forward_time(shape, Q):
             assert torch.equal(a, w), name
     with pytest.raises(Exception, match="x_time_reversed"):
         ops_ssd.chunk_state(Br.float(), dy.float(), ones, dA_cs, x_reversed=True)
+
+
+def test_backward_helpers_refuse_calls_they_do_not_cover():
+    """The entry points added for the gradient say so when a call is outside what they cover, instead of computing
+    something else: whole chunks for the preparation, the matrix-core kernel's own call for a finished ``dx``."""
+    from ssm_amd.ops import ssd as ops_ssd
+    gen = torch.Generator().manual_seed(0)
+    bf = torch.bfloat16
+    dt = torch.rand(1, 100, 2, generator=gen).cuda()
+    A = -torch.rand(2, generator=gen).cuda()
+    with pytest.raises(Exception, match="chunk"):
+        ops_ssd._bwd_prep(dt, A, 64, None, False, (0.0, float("inf")))
+    b, l, h, p, g, n, Q = 1, 128, 2, 64, 1, 32, 64
+    x = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
+    Bm = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
+    Cm = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
+    dtc = torch.rand(b, l, h, generator=gen).cuda()
+    dA_cs, dt_c = ops_ssd.chunk_cumsum(dtc, -torch.rand(h, generator=gen).cuda(), Q)
+    ent = torch.zeros(b, l // Q, h, p, n).cuda()
+    ep = (x, dtc, None, bf, True)
+    # a gate of the call's own, or the shape-generic kernels, cannot finish dx
+    with pytest.raises(Exception, match="dx_out"):
+        ops_ssd.chunk_scan(Bm, Cm, x, dt_c, dA_cs, ent, z=x, dx_epilogue=ep)
+    with pytest.raises(Exception, match="dx_out"):
+        ops_ssd.chunk_scan(Bm, Cm, x, dt_c, dA_cs, ent, dx_epilogue=ep, force_generic=True)
+    with pytest.raises(Exception, match="x_time_reversed"):
+        ops_ssd.chunk_scan(Bm, Cm, x, dt_c, dA_cs, ent, D=torch.ones(h).cuda(), x_reversed=True)
+    # and the ordinary call is untouched by all of it
+    y = ops_ssd.chunk_scan(Bm, Cm, x, dt_c, dA_cs, ent)
+    assert y.shape == x.shape and torch.isfinite(y.float()).all()
