@@ -105,8 +105,9 @@ class _Layer:
         # copy of z, x|B|C and x again per layer (0.67 GB at 16 x 2048 tokens).
         gn2 = cfg.conv_dim - di
         self.in_proj_z, self.in_proj_x, self.in_proj_bc, self.in_proj_dt = torch.split(self.in_proj, [di, di, gn2, H], dim=0)
-        self.conv_w_x, self.conv_w_bc = torch.split(self.conv_w, [di, gn2], dim=0)
-        self.conv_b_x, self.conv_b_bc = torch.split(self.conv_b, [di, gn2], dim=0)
+        # taps and bias as the kernels take them (float32, the same values): cut once, not converted on every call
+        self.conv_w_x, self.conv_w_bc = (t.contiguous() for t in torch.split(self.conv_w_f32, [di, gn2], dim=0))
+        self.conv_b_x, self.conv_b_bc = (t.contiguous() for t in torch.split(self.conv_b_f32, [di, gn2], dim=0))
 
 
 @dataclass
