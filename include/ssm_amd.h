@@ -489,6 +489,9 @@ typedef struct ssm_ssd_combined_args {
   float dt_min, dt_max;       /* clamp applied after softplus; use 0 and +inf for none */
   const int32_t *seq_idx;     /* (B, L) sequence ids of a packed batch (first id 0), or NULL: no state and no
                                  in-chunk term crosses from one sequence into the next */
+  int64_t b_row_stride, c_row_stride;  /* elements from one step's (G, N) block of Bm / Cm to the next step's; 0: dense
+                                 (G * N).  Lets B and C be the two halves of one projected row, read in place; rows
+                                 stay 16-byte aligned (a multiple of 8 elements) */
 } ssm_ssd_combined_args;
 int ssm_ssd_combined_supported(const ssm_ssd_dims *dims, int io_dtype);   /* 1 / 0 */
 size_t ssm_ssd_combined_workspace_bytes(const ssm_ssd_dims *dims);

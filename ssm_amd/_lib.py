@@ -180,7 +180,7 @@ class SsdCombinedArgs(C.Structure):
                 ("z", _vp), ("initial_states", _vp), ("y", _vp), ("final_states", _vp), ("workspace", _vp),
                 ("workspace_bytes", C.c_size_t), ("dims", SsdDims), ("io_dtype", _i32), ("dt_dtype", _i32),
                 ("dt_softplus", _i32), ("d_per_p", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float),
-                ("seq_idx", _vp)]
+                ("seq_idx", _vp), ("b_row_stride", _i64), ("c_row_stride", _i64)]
 
 
 class SsdBwdGateArgs(C.Structure):

@@ -70,6 +70,7 @@ struct SsdPrepParams {
   __bf16 *Cblk, *Btblk, *CBblk;
   unsigned n_dt, n_pack;                 // workgroups of the first two roles
   const int *seq_idx;                    // (B, L) sequence ids of a packed batch, or null
+  size_t b_row, c_row;                   // elements between the (G, N) blocks of consecutive steps in Bm / Cm
 };
 
 // Packed sequences: the first step of a sequence gets an extra decay of 2^-64 (a jump in the running sum),
@@ -161,12 +162,12 @@ __device__ __forceinline__ void prep_pack_role(const SsdPrepParams &pp, unsigned
   bf16x8_t v;
   if (is_c) {
     const int lb = inner / KN, kn = inner % KN;
-    v = load_frag(pp.Cm + (((size_t)b * len + (size_t)c * Q + 32 * lb + m) * groups + g) * N + 16 * kn + 8 * g2);
+    v = load_frag(pp.Cm + ((size_t)b * len + (size_t)c * Q + 32 * lb + m) * pp.c_row + (size_t)g * N + 16 * kn + 8 * g2);
   } else {
     const int ks = inner / NT, nt = inner % NT;
-    const __bf16 *col = pp.Bm + (((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * groups + g) * N + 32 * nt + m;
+    const __bf16 *col = pp.Bm + ((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * pp.b_row + (size_t)g * N + 32 * nt + m;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = col[(size_t)j * groups * N];
+    for (int j = 0; j < 8; ++j) v[j] = col[(size_t)j * pp.b_row];
   }
   *reinterpret_cast<bf16x8_t *>((is_c ? pp.Cblk : pp.Btblk) + f * FRAG + lane * 8) = v;
 }
@@ -188,8 +189,8 @@ __device__ __forceinline__ void prep_cb_role(const SsdPrepParams &pp, unsigned w
   const int g = (int)(unit % groups);
   const size_t bc = unit / groups;                        // b * nchunks + c: the chunk's first row is bc * Q
   const int m = lane & 31, g2 = lane >> 5;
-  const __bf16 *crow_p = pp.Cm + ((bc * Q + 32 * lb + m) * groups + g) * N + 8 * g2;
-  const __bf16 *brow_p = pp.Bm + ((bc * Q + 32 * sb + m) * groups + g) * N + 8 * g2;
+  const __bf16 *crow_p = pp.Cm + (bc * Q + 32 * lb + m) * pp.c_row + (size_t)g * N + 8 * g2;
+  const __bf16 *brow_p = pp.Bm + (bc * Q + 32 * sb + m) * pp.b_row + (size_t)g * N + 8 * g2;
   f32x16_t acc = {0};
   for (int k0 = 0; k0 < N; k0 += 16) acc = mma(load_frag(crow_p + k0), load_frag(brow_p + k0), acc);
   float (*tile)[33] = reinterpret_cast<float (*)[33]>(lds + wave * 32 * 33);
@@ -770,6 +771,13 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   cp.d = d; cp.dt_dtype = a->dt_dtype; cp.softplus = a->dt_softplus ? 1 : 0; cp.dt_min = a->dt_min; cp.dt_max = a->dt_max;
   pp.dA2 = reinterpret_cast<float *>(ws + lay.dA2);
   pp.Cm = reinterpret_cast<const __bf16 *>(a->Cm); pp.Bm = reinterpret_cast<const __bf16 *>(a->Bm);
+  const size_t dense_row = (size_t)d.groups * d.nstate;
+  SSM_REQUIRE(a->b_row_stride >= 0 && a->c_row_stride >= 0 && (a->b_row_stride == 0 || (size_t)a->b_row_stride >= dense_row) &&
+                  (a->c_row_stride == 0 || (size_t)a->c_row_stride >= dense_row) && a->b_row_stride % 8 == 0 && a->c_row_stride % 8 == 0,
+              SSM_ERR_BAD_SHAPE, "ssm_ssd_combined_fwd: b_row_stride=%lld c_row_stride=%lld must be 0 or at least groups * nstate=%zu, in multiples of 8",
+              (long long)a->b_row_stride, (long long)a->c_row_stride, dense_row);
+  pp.b_row = a->b_row_stride ? (size_t)a->b_row_stride : dense_row;
+  pp.c_row = a->c_row_stride ? (size_t)a->c_row_stride : dense_row;
   __bf16 *Cblk = reinterpret_cast<__bf16 *>(ws + lay.Cblk), *Btblk = reinterpret_cast<__bf16 *>(ws + lay.Btblk);
   pp.Cblk = Cblk; pp.Btblk = Btblk; pp.CBblk = reinterpret_cast<__bf16 *>(ws + lay.CBblk);
   const size_t n_dt = (size_t)d.batch * d.nchunks * ((d.heads + PD_HEADS - 1) / PD_HEADS);

@@ -403,6 +403,17 @@ def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
     return bool(_lib.load().ssm_ssd_combined_supported(dims, _lib.dtype_enum(torch.bfloat16)))
 
 
+def _rows_in_place(t):
+    """``(tensor, row stride)`` for a ``(B, L, G, N)`` operand of the one-pass kernel: the tensor itself with the
+    distance in elements between consecutive steps when its ``(G, N)`` blocks are dense, follow each other at one
+    stride through batch and time, and start 16-byte aligned (a slice of wider rows); else a dense copy and 0."""
+    b, l, g, n = t.shape
+    sb, sl, sg, sn = t.stride()
+    ok = (sn == 1 and (g == 1 or sg == n) and sl >= g * n and sl % 8 == 0 and (b == 1 or sb == l * sl)
+          and t.data_ptr() % 16 == 0)
+    return (t, int(sl)) if ok and not t.is_contiguous() else (K.cast_c(t, t.dtype), 0)
+
+
 def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit, return_final_states, shape,
                seq_idx=None):
     batch, seqlen, heads, hdim, groups, nstate = shape
@@ -415,7 +426,9 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
     _need(tuple(A.shape) == (heads,), "A must have shape (H,).")
     _need(dt_bias is None or tuple(dt_bias.shape) == (heads,), "dt_bias must have shape (H,).")
     dev = K.require_gpu(x, dt, A, B, C, D, z, dt_bias, initial_states)
-    xc, Bc, Cc = K.cast_c(x, x.dtype), K.cast_c(B, B.dtype), K.cast_c(C, C.dtype)
+    xc = K.cast_c(x, x.dtype)
+    # B and C cut out of wider rows (the two halves of one projection) are read where they are
+    (Bc, b_row), (Cc, c_row) = _rows_in_place(B), _rows_in_place(C)
     zc = K.cast_c(z, z.dtype) if z is not None else None
     dtc = K.cast_c(dt, dt.dtype)
     K.check_float("dt", dtc)
@@ -432,7 +445,8 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
         final_states=_lib.ptr(final), workspace=work.data_ptr() + off, workspace_bytes=nbytes, dims=dims,
         io_dtype=_lib.dtype_enum(torch.bfloat16), dt_dtype=_lib.dtype_enum(dtc.dtype),
         dt_softplus=int(bool(dt_softplus)), d_per_p=int(d_per_p),
-        dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]), seq_idx=_lib.ptr(si))
+        dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]), seq_idx=_lib.ptr(si), b_row_stride=b_row,
+        c_row_stride=c_row)
     _lib.call("ssm_ssd_combined_fwd", args, dev)
     if return_final_states:
         return y, final

@@ -913,3 +913,24 @@ def test_backward_helpers_refuse_calls_they_do_not_cover():
     # and the ordinary call is untouched by all of it
     y = ops_ssd.chunk_scan(Bm, Cm, x, dt_c, dA_cs, ent)
     assert y.shape == x.shape and torch.isfinite(y.float()).all()
+
+
+def test_one_pass_reads_b_and_c_cut_out_of_wider_rows_in_place():
+    """``B`` and ``C`` as the two halves of one projected row (views with a row stride of ``2 G N``) give the bits of
+    the call with dense copies, and no copy is made."""
+    b, l, h, p, g, n, Q = 2, 512, 4, 64, 2, 64, 128
+    gen = torch.Generator().manual_seed(17)
+    bf = torch.bfloat16
+    x = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
+    z = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
+    bc = (torch.randn(b, l, 2 * g * n, generator=gen) * 0.5).to(bf).cuda()
+    dt = (torch.rand(b, l, h, generator=gen) * 0.2).cuda()
+    A = -(torch.rand(h, generator=gen) * 2 + 0.1).cuda()
+    D = torch.randn(h, generator=gen).cuda()
+    Bv, Cv = (t.reshape(b, l, g, n) for t in torch.split(bc, [g * n, g * n], dim=-1))
+    assert not Bv.is_contiguous() and Bv.data_ptr() == bc.data_ptr()
+    from ssm_amd.ops import ssd as ops_ssd
+    assert ops_ssd._rows_in_place(Cv)[0] is Cv and ops_ssd._rows_in_place(Cv)[1] == 2 * g * n
+    y, fin = ssd().ssd_combined(x, dt, A, Bv, Cv, Q, D=D, z=z, return_final_states=True, fused=True)
+    y2, fin2 = ssd().ssd_combined(x, dt, A, Bv.contiguous(), Cv.contiguous(), Q, D=D, z=z, return_final_states=True, fused=True)
+    assert torch.equal(y, y2) and torch.equal(fin, fin2)
