@@ -217,7 +217,15 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_typed_kernel(const NormPa
   for (int k = 0; k < TRIPS; ++k) {
     const int colc = min((k * OWNERS + lane) * VEC, H - VEC);
     ld_pack<XT, VEC>(p.x, base + colc, v[k]);
-    ld_pack<RT, VEC>(resp, base + colc, r[k]);
+  }
+  if (has_res) {                 // one test in front of all of a row's residual reads, none between them
+#pragma unroll
+    for (int k = 0; k < TRIPS; ++k) ld_pack<RT, VEC>(resp, base + min((k * OWNERS + lane) * VEC, H - VEC), r[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < TRIPS; ++k)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) r[k][i] = 0.0f;
   }
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
@@ -225,7 +233,6 @@ __global__ __launch_bounds__(LN_THREADS) void norm_fwd_typed_kernel(const NormPa
     const bool live = col < H;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
-      if (!has_res) r[k][i] = 0.0f;
       if (p.prenorm) v[k][i] += r[k][i];
       if (!live) v[k][i] = 0.0f;
       sum += v[k][i];
@@ -279,6 +286,10 @@ static void launch_norm_fwd_typed(const NormParams &p, int per_lane, unsigned gr
   else if (per_lane <= 8) hipLaunchKernelGGL((norm_fwd_typed_kernel<2, false, XT, RT>), dim3(grid), b, 0, s, p);
   else if (per_lane <= 12) hipLaunchKernelGGL((norm_fwd_typed_kernel<3, false, XT, RT>), dim3(grid), b, 0, s, p);
   else if (per_lane <= 16) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, false, XT, RT>), dim3(grid), b, 0, s, p);
+  // (a trip that holds no column still reads one: rows of 1280, 1536 and 1792 columns get trip counts of their own)
+  else if (per_lane <= 20) hipLaunchKernelGGL((norm_fwd_typed_kernel<5, false, XT, RT>), dim3(grid), b, 0, s, p);
+  else if (per_lane <= 24) hipLaunchKernelGGL((norm_fwd_typed_kernel<6, false, XT, RT>), dim3(grid), b, 0, s, p);
+  else if (per_lane <= 28) hipLaunchKernelGGL((norm_fwd_typed_kernel<7, false, XT, RT>), dim3(grid), b, 0, s, p);
   else if (per_lane <= 32) hipLaunchKernelGGL((norm_fwd_typed_kernel<8, false, XT, RT>), dim3(grid), b, 0, s, p);
   else if (p.hidden <= 4096) hipLaunchKernelGGL((norm_fwd_typed_kernel<4, true, XT, RT>), dim3(p.rows), b, 0, s, p);
   else if (p.hidden <= 5120) hipLaunchKernelGGL((norm_fwd_typed_kernel<5, true, XT, RT>), dim3(p.rows), b, 0, s, p);
