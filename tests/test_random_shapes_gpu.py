@@ -168,8 +168,114 @@ def _norm_case(rng, seed):
                           [x, w, bias, res], desc, 2e-2 if half else 2e-4, 3e-2 if half else 5e-4)
 
 
+def _decode_case(rng, seed):
+    """Three tokens through the fused decode step against window roll + tap sum + activation + oracle step."""
+    g = torch.Generator().manual_seed(seed)
+    io = rng.choice([torch.float32, torch.bfloat16, torch.float16])
+    b, d, n, K = rng.randint(1, 9), rng.choice([4, 16, 40, 64, 100, 256, 1024]), rng.choice([1, 4, 16, 16, 32, 64, 5]), rng.choice([2, 3, 4, 4, 7])
+    grp = rng.choice([gg for gg in (1, 2, 4) if d % gg == 0 and gg != d])
+    A = -(torch.rand(d, n, generator=g) * 3 + 0.1)
+    D = torch.randn(d, generator=g) if rng.random() < 0.6 else None
+    bias = torch.randn(d, generator=g) * 0.5 if rng.random() < 0.6 else None
+    use_z, use_cb = rng.random() < 0.6, rng.random() < 0.7
+    act = rng.choice(["silu", "silu", "identity"])
+    w = torch.rand(d, K, generator=g) - 0.5
+    cb = torch.randn(d, generator=g) * 0.1 if use_cb else None
+    cs_ref = torch.randn(b, d, K, generator=g).to(io).float()
+    st_ref = torch.randn(b, d, n, generator=g)
+    cs, st = cs_ref.to(io).cuda(), st_ref.clone().cuda()
+    desc = ("decode", seed, (b, d, n, K), grp, str(io), D is not None, use_z, bias is not None, use_cb, act)
+    tol = 2e-4 if io == torch.float32 else 2e-2
+    dev = lambda t: None if t is None else t.cuda()
+    for _ in range(3):
+        x, dt = torch.randn(b, d, generator=g).to(io), torch.randn(b, d, generator=g).to(io)
+        Bm, Cm = torch.randn(b, grp, n, generator=g).to(io), torch.randn(b, grp, n, generator=g).to(io)
+        z = torch.randn(b, d, generator=g).to(io) if use_z else None
+        cs_ref = torch.roll(cs_ref, -1, dims=-1)
+        cs_ref[..., -1] = x.float()
+        pre = (cs_ref * w).sum(-1) + (0.0 if cb is None else cb)
+        xc = (torch.nn.functional.silu(pre) if act == "silu" else pre).to(io)
+        y_ref, st_ref = O.selective_state_step_functional(st_ref.double(), xc, dt, A, Bm, Cm, D, z, bias, softplus=True,
+                                                          acc=torch.float64)
+        y = _ops().decode_step(cs, st, x.cuda(), dt.cuda(), A.cuda(), Bm.cuda(), Cm.cuda(), w.cuda(), conv_bias=dev(cb),
+                               D=dev(D), z=dev(z), dt_bias=dev(bias), softplus=True, activation=act)
+        assert torch.equal(cs.float().cpu(), cs_ref), desc
+        assert _rel(y, y_ref) < tol, desc
+        assert _rel(st, st_ref) < tol, desc          # half inputs: the convolution output is rounded to them first
+        st_ref = st_ref.float()
+
+
+def _mamba2_decode_case(rng, seed):
+    """Three tokens through the Mamba-2 decode step against split + window conv + per-head oracle step."""
+    g = torch.Generator().manual_seed(seed)
+    io = rng.choice([torch.float32, torch.bfloat16, torch.float16])
+    b, G = rng.randint(1, 5), rng.choice([1, 1, 2, 4])
+    H, P = G * rng.choice([1, 2, 3, 6]), rng.choice([16, 32, 64, 64, 80, 128])
+    N, K = rng.choice([16, 32, 64, 128, 128]), rng.choice([2, 3, 4, 4, 7])
+    di, conv_dim = H * P, H * P + 2 * G * N
+    A = -(torch.rand(H, generator=g) * 4.0 + 0.5)
+    D = rng.choice([None, torch.randn(H, generator=g), torch.randn(H, P, generator=g)])
+    bias = torch.randn(H, generator=g) - 2.0 if rng.random() < 0.7 else None
+    gate = rng.random() < 0.7
+    w = torch.rand(conv_dim, K, generator=g) - 0.5
+    cb = torch.randn(conv_dim, generator=g) * 0.1 if rng.random() < 0.7 else None
+    cs_ref = torch.randn(b, conv_dim, K, generator=g).to(io).float()
+    st_ref = torch.randn(b, H, P, N, generator=g)
+    cs, st = cs_ref.to(io).cuda(), st_ref.clone().cuda()
+    desc = ("mamba2 decode", seed, (b, H, P, G, N, K), str(io), None if D is None else tuple(D.shape), bias is not None, gate, cb is not None)
+    tol = 2e-4 if io == torch.float32 else 2e-2
+    dev = lambda t: None if t is None else t.cuda()
+    Dflat = None if D is None else (D.repeat_interleave(P) if D.ndim == 1 else D.reshape(di))
+    for _ in range(3):
+        row = torch.randn(b, 2 * di + 2 * G * N + H, generator=g).to(io)
+        z, xBC, dt = torch.split(row.float(), [di, conv_dim, H], dim=-1)
+        cs_ref = torch.roll(cs_ref, -1, dims=-1)
+        cs_ref[..., -1] = xBC
+        act = torch.nn.functional.silu((cs_ref * w).sum(-1) + (0.0 if cb is None else cb))
+        x, Bm, Cm = torch.split(act, [di, G * N, G * N], dim=-1)
+        y_ref, flat = O.selective_state_step_functional(
+            st_ref.reshape(b, di, N).double(), x.double(), dt.repeat_interleave(P, dim=-1).double(),
+            A.repeat_interleave(P)[:, None].expand(di, N), Bm.reshape(b, G, N).double(), Cm.reshape(b, G, N).double(), Dflat,
+            z.double() if gate else None, None if bias is None else bias.repeat_interleave(P), softplus=True, acc=torch.float64)
+        st_ref = flat.reshape(b, H, P, N).float()
+        y = _ops().mamba2_decode_step(row.cuda(), cs, st, w.cuda(), dev(cb), A.cuda(), D=dev(D), dt_bias=dev(bias), ngroups=G,
+                                      softplus=True, gate=gate)
+        assert torch.equal(cs.float().cpu(), cs_ref), desc
+        assert _rel(y, y_ref) < tol, desc
+        assert _rel(st, flat.reshape(b, H, P, N)) < 2e-4, desc
+
+
+def _dscan_case(rng, seed):
+    """The reference's diagonal ``ssd_chunk_scan`` with its optional arguments, values and gradients."""
+    g = torch.Generator().manual_seed(seed)
+    dtype = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+    b, l, h, p = rng.choice([1, 2, 3]), rng.randint(1, 700), rng.choice([1, 2, 4, 5]), rng.choice([8, 64, 128, 192, 20])
+    chunk = rng.choice([16, 64, 256])
+    X = torch.randn(b, l, h, p, generator=g).to(dtype)
+    dt = torch.rand(b, l, h, generator=g) * 0.2
+    per_p = rng.random() < 0.3
+    A = -(torch.rand(*((h, p) if per_p else (h,)), generator=g) * 4 + 0.1)
+    kind = rng.choice(["blhp", "blhp", "hp", "bhp"])
+    shape = {"blhp": (b, l, h, p), "hp": (h, p), "bhp": (b, h, p)}[kind]
+    pt = dtype if kind == "blhp" else rng.choice([dtype, torch.float32])
+    Bm, Cm = torch.randn(*shape, generator=g).to(pt), torch.randn(*shape, generator=g).to(pt)
+    D = torch.randn(*((h, p) if per_p else (h,)), generator=g) if rng.random() < 0.5 else None
+    z = torch.randn(b, l, h, p, generator=g).to(dtype) if rng.random() < 0.6 else None
+    init = torch.randn(b, h, p, generator=g) if rng.random() < 0.5 else None
+    lens = [rng.randint(0, l) for _ in range(b)] if rng.random() < 0.4 else None
+    meta = {"seq_lens": lens} if lens else None
+    desc = ("dscan", seed, (b, l, h, p), chunk, str(dtype), kind, str(pt), per_p, D is not None, z is not None, init is not None, lens)
+    half = dtype in HALF
+    _values_and_gradients(
+        lambda X, dt, A, Bm, Cm, D, z, init: _ops().ssd_chunk_scan(X, dt, A, Bm, Cm, chunk, D=D, z=z, seq_meta=meta, initial_states=init),
+        lambda X, dt, A, Bm, Cm, D, z, init: O.ssd_chunk_scan(X, dt, A, Bm, Cm, chunk, D=D, z=z, seq_meta=meta, initial_states=init,
+                                                              acc=torch.float64),
+        [X, dt, A, Bm, Cm, D, z, init], desc, 2e-2 if half else 2e-4, 3e-2 if half else 5e-4)
+
+
 @pytest.mark.parametrize("block", range(4))
-@pytest.mark.parametrize("case", [_scan_case, _step_case, _conv_case, _norm_case], ids=["scan", "step", "conv", "norm"])
+@pytest.mark.parametrize("case", [_scan_case, _step_case, _conv_case, _norm_case, _decode_case, _mamba2_decode_case, _dscan_case],
+                         ids=["scan", "step", "conv", "norm", "decode", "mamba2_decode", "dscan"])
 def test_operator_over_random_shapes_matches_the_float64_oracle(case, block):
     for i in range(CASES_PER_BLOCK):
         seed = 10_000 * (block + 1) + i
