@@ -351,6 +351,76 @@ def _ssd_case(rng, seed):
             assert float(err.mean()) / rms < mean_bar and float(err.max()) / rms < max_bar, (desc, k)
 
 
+def _ssd_stages_case(rng, seed):
+    """Each stage of the SSD on its own, fed with the float64 oracle's result of the stage before, so that no
+    stage's error hides behind another's: running sums, chunk products, chunk states, state passing, chunk
+    outputs, and the per-sequence end states of a packed row."""
+    from ssm_amd.ops import ssd as S
+    gen = torch.Generator().manual_seed(seed)
+    dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+    b, Q = rng.choice([1, 1, 2, 3]), rng.choice([16, 32, 64, 128, 256])
+    l = rng.choice([Q * rng.randint(1, 4), rng.randint(1, 3 * Q)])
+    g, per = rng.choice([1, 2]), rng.choice([1, 2, 3])
+    h = g * per
+    p, n = rng.choice([16, 32, 64, 64, 24]), rng.choice([16, 32, 64, 128, 48])
+    softplus, use_z, use_init = rng.random() < 0.7, rng.random() < 0.6, rng.random() < 0.5
+    use_D = rng.choice([None, "h", "hp"])
+    cuts = sorted(rng.sample(range(1, l), min(l - 1, rng.randint(1, 3)))) if (rng.random() < 0.4 and l >= 4) else None
+    x = torch.randn(b, l, h, p, generator=gen).to(dtype)
+    dt = torch.randn(b, l, h, generator=gen) * 0.5 if softplus else torch.rand(b, l, h, generator=gen) * 0.3
+    A = -(torch.rand(h, generator=gen) + 0.2)
+    Bm = (torch.randn(b, l, g, n, generator=gen) * 0.5).to(dtype)
+    Cm = (torch.randn(b, l, g, n, generator=gen) * 0.5).to(dtype)
+    D = None if use_D is None else (torch.randn(h, generator=gen) if use_D == "h" else torch.randn(h, p, generator=gen))
+    z = torch.randn(b, l, h, p, generator=gen).to(dtype) if use_z else None
+    bias = torch.randn(h, generator=gen) * 0.3 if softplus else None
+    init = torch.randn(b, h, p, n, generator=gen) if use_init else None
+    seq_idx = None
+    if cuts:
+        seq_idx = torch.zeros(b, l, dtype=torch.int32)
+        for c in cuts:
+            seq_idx[:, c:] += 1
+    desc = ("ssd stages", seed, str(dtype), (b, l, h, p, g, n), Q, softplus, use_z, use_init, use_D, cuts)
+    dev = lambda t: None if t is None else t.cuda()
+    tol = 2e-4 if dtype == torch.float32 else 2e-2
+    sid = dev(seq_idx)
+
+    cs64, dtc64 = SO.chunk_cumsum(dt, A, Q, dt_bias=bias, dt_softplus=softplus)
+    cs, dtc = S.chunk_cumsum(dev(dt), dev(A), Q, dt_bias=dev(bias), dt_softplus=softplus)
+    assert _rel(cs, cs64) < 1e-5 and _rel(dtc, dtc64) < 1e-5, (desc, "chunk_cumsum")
+    cs32, dtc32 = cs64.float().cuda(), dtc64.float().cuda()
+
+    causal = rng.random() < 0.5
+    cb64 = SO.bmm_chunk(Cm, Bm, Q, seq_idx=seq_idx, causal=causal)
+    cb = S.bmm_chunk(dev(Cm), dev(Bm), Q, seq_idx=sid, causal=causal, output_dtype=torch.float32)
+    assert _rel(cb, cb64) < (1e-5 if dtype == torch.float32 else 1e-3), (desc, "bmm_chunk")
+
+    st64 = SO.chunk_state(Bm, x, dtc64, cs64, seq_idx=seq_idx)
+    st = S.chunk_state(dev(Bm), dev(x), dtc32, cs32, seq_idx=sid)
+    assert _rel(st, st64) < tol, (desc, "chunk_state")
+
+    ent64, fin64 = SO.state_passing(st64, cs64[..., -1], initial_states=init, seq_idx=seq_idx, chunk_size=Q)
+    ent, fin = S.state_passing(st64.float().cuda(), cs32[..., -1].contiguous(), initial_states=dev(init), seq_idx=sid, chunk_size=Q)
+    assert _rel(ent, ent64) < 2e-5 and _rel(fin, fin64) < 2e-5, (desc, "state_passing")
+
+    y64 = SO.chunk_scan(Bm, Cm, x, dtc64, cs64, ent64, D=D, z=z, seq_idx=seq_idx)
+    y = S.chunk_scan(dev(Bm), dev(Cm), dev(x), dtc32, cs32, ent64.float().cuda(), D=dev(D), z=dev(z), seq_idx=sid)
+    assert _rel(y, y64) < (2e-4 if dtype == torch.float32 else 2.5e-2), (desc, "chunk_scan")
+
+    if cuts and b == 1:
+        cu = torch.tensor([0] + cuts + [l], dtype=torch.int32)
+        ends64 = SO.chunk_state_varlen(Bm, x, dtc64, cs64, cu, ent64)
+        ends = S.chunk_state_varlen(dev(Bm), dev(x), dtc32, cs32, cu.cuda(), ent64.float().cuda())
+        assert _rel(ends, ends64) < tol, (desc, "chunk_state_varlen")
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_ssd_stages_over_random_shapes_match_the_float64_oracle_stage_by_stage(block):
+    for i in range(CASES_PER_BLOCK):
+        seed = 30_000 * (block + 1) + i
+        _ssd_stages_case(random.Random(seed), seed)
+
+
 @pytest.mark.parametrize("block", range(4))
 def test_ssd_combined_over_random_shapes_matches_the_float64_recurrence(block):
     for i in range(CASES_PER_BLOCK):
