@@ -351,6 +351,61 @@ def _ssd_case(rng, seed):
             assert float(err.mean()) / rms < mean_bar and float(err.max()) / rms < max_bar, (desc, k)
 
 
+def _scan_wide_case(rng, seed):
+    """Shapes of the size the specialised scan kernels are picked for (hundreds of channels per group, long rows,
+    whole grids of workgroups).  Forward against the float64 oracle; backward -- the oracle's autograd takes
+    minutes at these sizes -- against the general backward kernel on the same inputs, which the small shapes
+    above pin against the oracle."""
+    g = torch.Generator().manual_seed(seed)
+    dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+    groups = rng.choice([1, 1, 2, 4])
+    d = groups * rng.choice([48, 96, 192, 384, 768, 1536, 40, 200])
+    b, n = rng.randint(1, 8), rng.choice([16, 16, 16, 8, 4])
+    l = rng.choice([16 * rng.randint(17, 160), 8 * rng.randint(33, 300), rng.randint(257, 2500)])
+    while b * d * l > 6_000_000:
+        if b > 1:
+            b //= 2
+        else:
+            l //= 2
+    u = torch.randn(b, d, l, generator=g).to(dtype)
+    delta = torch.randn(b, d, l, generator=g).to(dtype)
+    A = -(torch.rand(d, n, generator=g) * 3 + 0.1)
+    bc = rng.choice([dtype, dtype, torch.float32])
+    Bm, Cm = torch.randn(b, groups, n, l, generator=g).to(bc), torch.randn(b, groups, n, l, generator=g).to(bc)
+    D = torch.randn(d, generator=g) if rng.random() < 0.7 else None
+    z = torch.randn(b, d, l, generator=g).to(dtype) if rng.random() < 0.7 else None
+    bias = torch.randn(d, generator=g) * 0.5 if rng.random() < 0.7 else None
+    with_last = rng.random() < 0.5
+    half = dtype in HALF
+    desc = ("scan wide", seed, (b, d, l, n), groups, str(dtype), str(bc), D is not None, z is not None, bias is not None, with_last)
+    dev = lambda t: None if t is None else t.cuda()
+    with torch.no_grad():
+        y64, last64 = O.selective_scan(u, delta, A, Bm, Cm, D, z, bias, softplus=True, return_last_state=True, acc=torch.float64)
+        y, last = _ops().selective_scan(dev(u), dev(delta), dev(A), dev(Bm), dev(Cm), dev(D), dev(z), dev(bias), softplus=True,
+                                        return_last_state=True)
+    assert _rel(y, y64) < (2e-2 if half else 2e-4), (desc, "y")
+    assert _rel(last, last64) < (5e-3 if half else 2e-4), (desc, "last state")      # returned in the type of u
+    go = torch.randn(b, d, l, generator=g).to(dtype).cuda()
+    gl = torch.randn(b, d, n, generator=g).cuda() if with_last else None
+    args = (go, gl, dev(u), dev(delta), dev(A), dev(Bm), dev(Cm), dev(D), dev(z), dev(bias), True)
+    fast = _ops()._scan_backward(*args, tune_items=0)
+    general = _ops()._scan_backward(*args, tune_items=1)
+    for name, f, r in zip("u delta A B C D z dt_bias".split(), fast, general):
+        assert (f is None) == (r is None), (desc, name)
+        if r is None:
+            continue
+        # per-token gradients come back in the element type: one last place of a 16-bit value apart at most
+        bar = 2e-2 if (half and name in ("u", "delta", "z")) else 3e-4
+        assert _rel(f.float(), r.float()) < bar, (desc, name)
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_scan_at_the_sizes_of_its_specialised_kernels_matches_the_float64_oracle(block):
+    for i in range(4):
+        seed = 50_000 * (block + 1) + i
+        _scan_wide_case(random.Random(seed), seed)
+
+
 def _model_case(rng, seed):
     """A small Mamba-2 or Mamba-1 stack of random block shape: dense forward over a prompt of random length,
     then cached steps, against the CPU oracle stack on the same weights (bars of tests/test_harness_gpu.py)."""
