@@ -348,7 +348,9 @@ def _ssd_case(rng, seed):
             assert float(err.max()) <= bar * float(want.abs().max()) + 1e-6, (desc, k)
         else:
             rms = float(want.pow(2).mean().sqrt()) + 1e-30
-            assert float(err.mean()) / rms < mean_bar and float(err.max()) / rms < max_bar, (desc, k)
+            # a single element tens of times the rms carries the rounding of its own 16-bit value
+            assert float(err.mean()) / rms < mean_bar, (desc, k, float(err.mean()) / rms)
+            assert bool((err <= max_bar * rms + (0.0 if dtype == torch.float32 else 2e-2) * want.abs()).all()), (desc, k)
 
 
 def _scan_wide_case(rng, seed):
