@@ -469,15 +469,6 @@ def bench_scan_per_channel_bc(dtype=torch.bfloat16, batch=8, dim=1536, length=20
             "shape": "B, C (8, 1536, 16, 2048) bf16: one B/C group per channel"}
 
 
-VALU_KINDS = [
-    (0, "fp32 fma, 8 independent", 8), (1, "fp32 fma, dependent chain", 8), (2, "exp2", 8), (3, "log2", 8), (4, "rcp", 8),
-    (5, "exp2 and fma alternating", 8), (6, "scan state step: mul, exp2, mul, fma, fmac", 40),
-    (7, "the same with a move for exp2", 40), (8, "DPP multiply (quad broadcast)", 8),
-    (9, "DPP fmac / mul of a lane scan", 8), (10, "half-wave / row swaps", 8),
-    (11, "4 state steps + one fp32 16x16x4 matrix instruction", 21), (12, "8-byte LDS reads", 8),
-]
-
-
 def bench_stream():
     """What plain element-wise kernels of the framework reach on this GPU, as the yardstick for the streaming
     kernels: ``dst = 2 * src`` and ``dst.copy_(src)`` on float32 buffers of 64 MiB (source and destination fit the
@@ -495,38 +486,6 @@ def bench_stream():
         del src, dst
     out["frac_hbm_peak_scale_1GiB"] = round(out["scale_1024MiB_GBps"] / HBM_PEAK_GBPS, 4)
     return out
-
-
-def bench_valu(waves=(1, 2, 3, 4)):
-    """Issue rates of the vector ALU (``ssm_probe_valu``): shader clocks per wave instruction per SIMD, with one
-    workgroup per CU and 1 to 4 waves per SIMD."""
-    import ctypes
-    from ssm_amd import _lib
-    lib = _lib.load()
-    wgs, rounds = 256, 8
-    out = torch.empty(wgs * rounds * 1024, dtype=torch.float32, device="cuda")
-    clk = torch.zeros(2, dtype=torch.int64, device="cuda")
-    stream = _lib.stream_handle(out.device)
-    table = {}
-    for kind, name, per_iter in VALU_KINDS:
-        iters = 2048 if per_iter >= 20 else 4096
-        row = {}
-        for w in waves:
-            def go():
-                rc = lib.ssm_probe_valu(kind, w, wgs * rounds, iters, ctypes.c_void_p(out.data_ptr()),
-                                        ctypes.c_void_p(clk.data_ptr()), stream)
-                assert rc == 0, lib.ssm_amd_last_error()
-            go()
-            torch.cuda.synchronize()
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record(); go(); e.record(); torch.cuda.synchronize()
-            ticks = clk.cpu()
-            mhz = float(ticks[0]) / (float(ticks[1]) / 100.0)
-            cycles = s.elapsed_time(e) * 1e3 * mhz
-            row[f"{w}_waves_per_simd"] = round(cycles / (rounds * w * iters * per_iter), 2)
-            row["clock_mhz"] = round(mhz)
-        table[name] = row
-    return table
 
 
 def cpu_baseline_scan(dtype=torch.bfloat16, dim=1536, length=2048, nstate=16, budget_s=15.0):
@@ -580,7 +539,7 @@ def main():
                     help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
-                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1", "valu",
+                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1",
                              "scan_facade", "scan_per_channel_bc", "stream"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
@@ -607,10 +566,9 @@ def main():
     if args.only:
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
               "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model,
-              "model1": bench_model1, "valu": bench_valu, "scan_facade": bench_scan_facade,
+              "model1": bench_model1, "scan_facade": bench_scan_facade,
               "scan_per_channel_bc": bench_scan_per_channel_bc, "stream": bench_stream}[args.only]
-        if args.only != "valu":
-            bench_scan_fwd(1, 0)        # the untimed spin-up of the default run, so that figures compare
+        bench_scan_fwd(1, 0)            # the untimed spin-up of the default run, so that figures compare
         print(json.dumps({args.only: fn()}))
         return
 

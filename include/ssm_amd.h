@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SSM_AMD_ABI_VERSION 5
+#define SSM_AMD_ABI_VERSION 6
 
 typedef enum ssm_status {
   SSM_OK = 0,
@@ -85,8 +85,7 @@ typedef struct ssm_scan_fwd_args {
   int32_t b_kind, c_kind; /* ssm_proj_kind */
   int32_t b_groups, c_groups; /* G for SSM_PROJ_BGNL (must divide D), else ignored */
   int32_t delta_softplus; /* 0 / 1 */
-  int32_t tune_items;     /* 0 = automatic; else 100 * steps-per-lane + states-per-LDS-pass (408, 808, 816);
-                             1616, 2416, 3216, 4816 = 816 with two, three, four, six channels per wave */
+  int32_t reserved;       /* must be 0 */
 } ssm_scan_fwd_args;
 
 int ssm_scan_fwd(const ssm_scan_fwd_args *args, void *hip_stream);
@@ -122,7 +121,7 @@ typedef struct ssm_scan_bwd_args {
   int32_t io_dtype, bc_dtype;
   int32_t b_kind, c_kind, b_groups, c_groups;
   int32_t delta_softplus;
-  int32_t tune_items;             /* 0 = automatic; 1 = the general kernel also where the specialised one applies */
+  int32_t reserved;               /* must be 0 */
 } ssm_scan_bwd_args;
 
 size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, int nstate, int b_kind, int c_kind,
@@ -323,7 +322,7 @@ typedef struct ssm_dscan_bwd_args {
   int32_t grads_in_io_dtype;  /* non-zero: the gradients that have X's shape are written in their tensors' element
                                  types instead of fp32: dB / dC when the projection is per token (bc dtype), dz when
                                  the gate is per channel (z dtype); every other gradient stays fp32 */
-  int32_t tune_two_kernels;   /* non-zero keeps the general two-kernel path (for measurements and cross-checks) */
+  int32_t reserved;           /* must be 0 */
   const float *round_states;  /* optional: what ssm_dscan_fwd wrote for the same inputs; spares the backward its own
                                  forward sweep when it takes the one-pass kernels (ignored otherwise); or NULL */
 } ssm_dscan_bwd_args;
@@ -339,13 +338,9 @@ int ssm_dscan_bwd(const ssm_dscan_bwd_args *args, void *hip_stream);
  * state_passing, chunk_scan), :591-604 (combined) and :680-705 (bmm_chunk).
  * Layouts: x, z, y (B,L,H,P); dt (B,L,H); A (H,); Bm, Cm (B,L,G,N);
  * dt_out, dA_cumsum (B,H,nc,Q) fp32; CB (B,nc,G,Q,Q); states (B,nc,H,P,N);
- * final_states (B,H,P,N) fp32; nc = ceil(L/Q).  `force_generic` skips the
- * bf16 MFMA kernels (used by the tests to cross-check them).
+ * final_states (B,H,P,N) fp32; nc = ceil(L/Q).  Fields named `reserved`
+ * must be 0.
  * ---------------------------------------------------------------------- */
-/* Which of the calls made by this thread since the last query ran a bf16 MFMA
- * kernel: bit 0 bmm_chunk, bit 1 chunk_state, bit 2 chunk_scan, bit 3 the one-pass
- * ssm_ssd_combined_fwd.  Resets on read. */
-int ssm_ssd_mfma_launches(void);
 
 typedef struct ssm_ssd_dims {
   int32_t batch, seqlen, heads, headdim, groups, nstate, chunk;
@@ -368,7 +363,7 @@ typedef struct ssm_ssd_bmm_args {
   const int32_t *seq_idx;   /* (B,L) or NULL: entries across sequences are zeroed */
   void *out;                /* (B,nc,G,Q,Q) out dtype: out[l][s] = <a_l, b_s> */
   int32_t batch, seqlen, groups, kdim, chunk;
-  int32_t in_dtype, out_dtype, causal, force_generic;
+  int32_t in_dtype, out_dtype, causal, reserved;
 } ssm_ssd_bmm_args;
 int ssm_ssd_bmm_chunk(const ssm_ssd_bmm_args *args, void *hip_stream);
 
@@ -382,7 +377,7 @@ typedef struct ssm_ssd_chunk_state_args {
                                without it the MFMA kernel is not used */
   size_t workspace_bytes;
   ssm_ssd_dims dims;
-  int32_t x_dtype, b_dtype, states_dtype, force_generic;
+  int32_t x_dtype, b_dtype, states_dtype, reserved;
   const int32_t *seq_idx;   /* (B,L) or NULL: steps of another sequence than the chunk's last step add nothing */
   const float *x_row_scale; /* (B,H,nc,Q) or NULL: x stands for x * scale rounded to x's dtype, as if that tensor had
                                been written first (the backward puts the step into the operand this way); only the
@@ -418,7 +413,7 @@ typedef struct ssm_ssd_chunk_scan_args {
   const float *Dskip;       /* (H,P) if d_per_p else (H,), or NULL */
   void *y;                  /* (B,L,H,P) x dtype (float32 if y_f32) */
   ssm_ssd_dims dims;
-  int32_t x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype, d_per_p, force_generic;
+  int32_t x_dtype, c_dtype, cb_dtype, states_dtype, z_dtype, d_per_p, reserved;
   const int32_t *seq_idx;   /* (B,L) or NULL: the entering state only reaches steps whose sequence id equals that of
                                the last step of the chunk before (id 0 for the first chunk); CB must have been
                                formed with the same seq_idx */
@@ -738,19 +733,6 @@ int ssm_norm_bwd(const ssm_norm_bwd_args *args, void *hip_stream);
  * while a stream is being captured. */
 #define SSM_NORM_BWD_STATIC_BYTES (8u << 20)
 int ssm_norm_bwd_static(const ssm_norm_bwd_args *args, void *hip_stream);
-
-/* ------------------------------------------------------------------------
- * Measurement aid (no counterpart in the reference): a loop of `iters` repetitions of one instruction
- * pattern with no memory traffic on `workgroups` workgroups of 256 * waves_per_simd threads, one per CU at a
- * time.  kind: 0 eight independent fp32 fma, 1 eight dependent fma, 2 / 3 / 4 eight exp2 / log2 / rcp,
- * 5 exp2 and fma alternating (8), 6 the scan's state step for eight states (mul, exp2, mul, fma, fmac: 40),
- * 7 the same with a move in place of exp2, 8 eight DPP multiplies (quad broadcast), 9 eight DPP fmac / mul of a
- * lane scan, 10 eight half-wave / row swaps, 11 four state steps and one fp32 16x16x4 matrix instruction (21),
- * 12 eight 8-byte LDS reads.  `out` takes workgroups * 1024 floats; clocks[0] / clocks[1] receive the shader
- * and the 100 MHz wall clock ticks that the loop took on the first workgroup.
- * ---------------------------------------------------------------------- */
-int ssm_probe_valu(int kind, int waves_per_simd, int workgroups, int iters, float *out, long long *clocks,
-                   void *hip_stream);
 
 #ifdef __cplusplus
 }

@@ -312,15 +312,19 @@ def ssd_chunk_scan(X, dt, A, B, C, chunk_size, D=None, z=None, seq_meta=None,
     XX = X.to(ct)
     dd = dt.to(ct)
     rows = []
+    # one view per step, split off up front: autograd then assembles each input's gradient once
+    # instead of writing a tensor of the input's size per step
+    X_t, dt_t, B_t, C_t = XX.unbind(1), dd.unbind(1), Bf.unbind(1), Cf.unbind(1)
+    z_t = zz.unbind(1) if zz is not None else None
     for t in range(seqlen):
         live = (valid > t).to(ct)[:, None, None]          # (B,1,1)
-        step = dd[:, t, :, None]                           # (B,H,1)
-        s_new = torch.exp(step * AA[None]) * s + step * (Bf[:, t] * XX[:, t])
-        y = s_new * Cf[:, t]
+        step = dt_t[t][:, :, None]                         # (B,H,1)
+        s_new = torch.exp(step * AA[None]) * s + step * (B_t[t] * X_t[t])
+        y = s_new * C_t[t]
         if Dv is not None:
-            y = y + Dv[None] * XX[:, t]
+            y = y + Dv[None] * X_t[t]
         if zz is not None:
-            y = y * F.silu(zz[:, t])
+            y = y * F.silu(z_t[t])
         # finished sequences neither advance their state nor emit output
         s = torch.where(live.bool(), s_new, s)
         rows.append(torch.where(live.bool(), y, torch.zeros_like(y)))

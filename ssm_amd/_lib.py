@@ -19,7 +19,7 @@ import os
 # SSM_AMD_LIB points the binding at another build of the same C ABI.
 LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
                 Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
 PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
@@ -43,7 +43,7 @@ class ScanFwdArgs(C.Structure):
         ("Dskip", _vp), ("dt_bias", _vp), ("out", _vp), ("last_state", _vp), ("chunk_states", _vp),
         ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32),
         ("io_dtype", _i32), ("bc_dtype", _i32), ("b_kind", _i32), ("c_kind", _i32),
-        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("tune_items", _i32),
+        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("reserved", _i32),
     ]
 
 
@@ -55,7 +55,7 @@ class ScanBwdArgs(C.Structure):
         ("ddt_bias", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
         ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32),
         ("io_dtype", _i32), ("bc_dtype", _i32), ("b_kind", _i32), ("c_kind", _i32),
-        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("tune_items", _i32),
+        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("reserved", _i32),
     ]
 
 
@@ -113,7 +113,7 @@ class DscanBwdArgs(C.Structure):
         ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("proj", _i32),
         ("x_dtype", _i32), ("dt_dtype", _i32), ("bc_dtype", _i32), ("z_dtype", _i32), ("init_dtype", _i32),
         ("b_kind", _i32), ("c_kind", _i32), ("a_per_p", _i32), ("d_per_p", _i32), ("z_per_p", _i32),
-        ("grads_in_io_dtype", _i32), ("tune_two_kernels", _i32), ("round_states", _vp),
+        ("grads_in_io_dtype", _i32), ("reserved", _i32), ("round_states", _vp),
     ]
 
 
@@ -130,13 +130,13 @@ class SsdCumsumArgs(C.Structure):
 class SsdBmmArgs(C.Structure):
     _fields_ = [("a", _vp), ("b", _vp), ("seq_idx", _vp), ("out", _vp),
                 ("batch", _i32), ("seqlen", _i32), ("groups", _i32), ("kdim", _i32), ("chunk", _i32),
-                ("in_dtype", _i32), ("out_dtype", _i32), ("causal", _i32), ("force_generic", _i32)]
+                ("in_dtype", _i32), ("out_dtype", _i32), ("causal", _i32), ("reserved", _i32)]
 
 
 class SsdChunkStateArgs(C.Structure):
     _fields_ = [("Bm", _vp), ("x", _vp), ("dt", _vp), ("dA_cumsum", _vp), ("states", _vp),
                 ("workspace", _vp), ("workspace_bytes", C.c_size_t), ("dims", SsdDims),
-                ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("force_generic", _i32),
+                ("x_dtype", _i32), ("b_dtype", _i32), ("states_dtype", _i32), ("reserved", _i32),
                 ("seq_idx", _vp), ("x_row_scale", _vp), ("x_time_reversed", _i32)]
 
 
@@ -150,7 +150,7 @@ class SsdChunkScanArgs(C.Structure):
     _fields_ = [("CB", _vp), ("Cm", _vp), ("x", _vp), ("z", _vp), ("prev_states", _vp), ("dt", _vp),
                 ("dA_cumsum", _vp), ("Dskip", _vp), ("y", _vp), ("dims", SsdDims),
                 ("x_dtype", _i32), ("c_dtype", _i32), ("cb_dtype", _i32), ("states_dtype", _i32),
-                ("z_dtype", _i32), ("d_per_p", _i32), ("force_generic", _i32), ("seq_idx", _vp),
+                ("z_dtype", _i32), ("d_per_p", _i32), ("reserved", _i32), ("seq_idx", _vp),
                 ("y_f32", _i32), ("x_row_scale", _vp), ("dx_x", _vp), ("dx_dt", _vp), ("dx_Dskip", _vp), ("dx_out", _vp),
                 ("dx_xu", _vp), ("dx_s1", _vp), ("dx_d_per_p", _i32), ("dx_out_f32", _i32), ("dx_round_dtx", _i32),
                 ("x_time_reversed", _i32)]
@@ -314,50 +314,87 @@ PLAIN_SYMBOLS = {
     "ssm_dscan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ssm_dscan_fwd_one_pass": (C.c_int, [C.POINTER(DscanFwdArgs)]),
     "ssm_ssd_chunk_state_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
-    "ssm_ssd_mfma_launches": (C.c_int, []),
     "ssm_ssd_combined_supported": (C.c_int, [C.POINTER(SsdDims), C.c_int]),
     "ssm_ssd_combined_workspace_bytes": (C.c_size_t, [C.POINTER(SsdDims)]),
     "ssm_conv1d_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "ssm_norm_bwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
-    "ssm_probe_valu": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
 }
 
+# exported by the test-hooks build only (include/ssm_amd_testing.h)
+HOOKS_SYMBOLS = {
+    "ssm_ssd_mfma_launches": (C.c_int, []),
+}
+HOOKS_LIB_PATH = LIB_PATH.with_name("libssm_amd_testhooks.so")
+
 _lock = threading.Lock()
-_lib: Optional[C.CDLL] = None
-_load_error: Optional[Exception] = None
+_libs: dict = {}                     # hooks? -> CDLL
+_load_errors: dict = {}              # hooks? -> Exception
+_hooks_active = 0                    # depth of test_hooks_build() contexts
+
+
+def _bind(path: Path, hooks: bool) -> C.CDLL:
+    if not path.exists():
+        raise FileNotFoundError(f"{path} not found: build it with `python -m ssm_amd.build`")
+    lib = C.CDLL(str(path))
+    plain = dict(PLAIN_SYMBOLS, **HOOKS_SYMBOLS) if hooks else PLAIN_SYMBOLS
+    for name, (res, argt) in plain.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = argt
+    got = lib.ssm_amd_abi_version()
+    if got != ABI_VERSION:
+        raise RuntimeError(f"{path.name} ABI {got}, binding expects {ABI_VERSION}")
+    for name, struct in ENTRY_POINTS.items():
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.POINTER(struct), _vp]
+    return lib
+
+
+def _load(hooks: bool) -> C.CDLL:
+    lib = _libs.get(hooks)
+    if lib is not None:
+        return lib
+    with _lock:
+        if hooks in _libs:
+            return _libs[hooks]
+        if hooks in _load_errors:
+            raise BackendUnavailable(str(_load_errors[hooks]))
+        try:
+            _libs[hooks] = _bind(HOOKS_LIB_PATH if hooks else LIB_PATH, hooks)
+        except Exception as exc:  # remembered: a broken install stays broken
+            _load_errors[hooks] = exc
+            raise BackendUnavailable(str(exc)) from exc
+    return _libs[hooks]
 
 
 def load() -> C.CDLL:
-    """Load the library once; raise :class:`BackendUnavailable` if impossible."""
-    global _lib, _load_error
-    if _lib is not None:
-        return _lib
-    with _lock:
-        if _lib is not None:
-            return _lib
-        if _load_error is not None:
-            raise BackendUnavailable(str(_load_error))
-        try:
-            if not LIB_PATH.exists():
-                raise FileNotFoundError(
-                    f"{LIB_PATH} not found: build it with `python -m ssm_amd.build`")
-            lib = C.CDLL(str(LIB_PATH))
-            for name, (res, argt) in PLAIN_SYMBOLS.items():
-                fn = getattr(lib, name)
-                fn.restype = res
-                fn.argtypes = argt
-            got = lib.ssm_amd_abi_version()
-            if got != ABI_VERSION:
-                raise RuntimeError(f"libssm_amd ABI {got}, binding expects {ABI_VERSION}")
-            for name, struct in ENTRY_POINTS.items():
-                fn = getattr(lib, name)
-                fn.restype = C.c_int
-                fn.argtypes = [C.POINTER(struct), _vp]
-            _lib = lib
-        except Exception as exc:  # remembered: a broken install stays broken
-            _load_error = exc
-            raise BackendUnavailable(str(exc)) from exc
-    return _lib
+    """The shipped library, loaded once; raises :class:`BackendUnavailable` if impossible.  Inside
+    :func:`test_hooks_build` the test-hooks build stands in for it."""
+    return _load(_hooks_active > 0)
+
+
+def load_test_hooks() -> C.CDLL:
+    """The ``-DSSM_TEST_HOOKS`` build of the same sources (``include/ssm_amd_testing.h``): reads the argument
+    structs' ``reserved`` fields as kernel selectors and exports ``ssm_ssd_mfma_launches``."""
+    return _load(True)
+
+
+class test_hooks_build:
+    """Context manager for the test suite: every call inside goes to the test-hooks build, so that
+    ``load().ssm_ssd_mfma_launches()`` reports the kernels those calls took."""
+    __test__ = False
+
+    def __enter__(self):
+        global _hooks_active
+        load_test_hooks()
+        _hooks_active += 1
+        return _libs[True]
+
+    def __exit__(self, *exc):
+        global _hooks_active
+        _hooks_active -= 1
+        return False
 
 
 def available() -> bool:
@@ -387,7 +424,8 @@ def call(name: str, args: C.Structure, device: torch.device) -> None:
     """Invoke an entry point on the current stream of ``device``; a contract
     violation reported by the library surfaces as ``ValueError`` (as the
     reference's compiled backends do, src/ssm/ops/__init__.py:1244-1252)."""
-    lib = load()
+    # a kernel selector in the struct only means something to the test-hooks build
+    lib = load_test_hooks() if getattr(args, "reserved", 0) else load()
     with torch.cuda.device(device):
         status = getattr(lib, name)(C.byref(args), stream_handle(device))
     if status != 0:

@@ -33,6 +33,18 @@ void set_error(const char *fmt, ...);   // defined in status.hip
     }                                                                           \
   } while (0)
 
+// Kernel-route selectors travel in the argument structs' `reserved` fields and exist only in a build with
+// -DSSM_TEST_HOOKS (include/ssm_amd_testing.h): the shipped library picks kernels by shape and dtype alone and
+// rejects a non-zero value.
+#ifdef SSM_TEST_HOOKS
+#define SSM_RESERVED(a) ((a)->reserved)
+#define SSM_CHECK_RESERVED(who, a) do { } while (0)
+#else
+#define SSM_RESERVED(a) 0
+#define SSM_CHECK_RESERVED(who, a) \
+  SSM_REQUIRE((a)->reserved == 0, SSM_ERR_BAD_KIND, "%s: reserved must be 0 (kernel selectors need a -DSSM_TEST_HOOKS build)", who)
+#endif
+
 inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 inline bool valid_dtype(int d) { return d == SSM_F32 || d == SSM_BF16 || d == SSM_F16; }
 inline int dtype_size(int d) { return d == SSM_F32 ? 4 : 2; }

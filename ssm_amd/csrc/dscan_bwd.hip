@@ -286,6 +286,7 @@ extern "C" size_t ssm_dscan_bwd_workspace_bytes(int batch, int seqlen, int heads
 extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   using namespace ssm;
   SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_dscan_bwd: args is NULL");
+  SSM_CHECK_RESERVED("ssm_dscan_bwd", a);
   SSM_REQUIRE(a->grad_y && a->X && a->dt && a->A && a->Bproj && a->Cproj && a->dX && a->ddt && a->dA && a->dB && a->dC,
               SSM_ERR_NULL_POINTER,
               "ssm_dscan_bwd: grad_y, X, dt, A, Bproj, Cproj, dX, ddt, dA, dB and dC are required");
@@ -361,7 +362,7 @@ extern "C" int ssm_dscan_bwd(const ssm_dscan_bwd_args *a, void *hip_stream) {
   const bool constant = a->b_kind != SSM_CHUNK_BLHP && a->c_kind != SSM_CHUNK_BLHP &&
                         aligned_to(a->Bproj, dtype_size(a->bc_dtype)) && aligned_to(a->Cproj, dtype_size(a->bc_dtype)) &&
                         aligned_to(a->dB, 4) && aligned_to(a->dC, 4);
-  const bool onepass = a->tune_two_kernels == 0 && (streamed || constant) && a->dt_dtype == SSM_F32 &&
+  const bool onepass = SSM_RESERVED(a) == 0 && a->batch < 65536 && (streamed || constant) && a->dt_dtype == SSM_F32 &&
                        (!a->z || (a->z_dtype == a->x_dtype && a->z_per_p)) && (lph == 16 || lph == 32 || lph == 64) &&
                        HP % (WAVE * vec) == 0 && (size_t)L * HP < ((size_t)1 << 30) && aligned_to(a->X, vbytes) &&
                        aligned_to(a->grad_y, vbytes) && aligned_to(a->dX, vbytes) &&

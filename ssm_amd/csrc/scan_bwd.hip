@@ -48,6 +48,7 @@ struct ScanBwdParams {
   int rows_per_wg;       // channels walked by one workgroup (all in one B group and one C group)
   int nblk;              // workgroups per batch row = dim / rows_per_wg
   int bc_vec_ok;
+  int spin_limit;        // wave-per-row kernel: looks at a neighbour's slot count before a wave gives up (scan_bwd_fast.hpp)
 };
 
 // Stage one [BW_MAX_N][BW_T] slab of a time-varying projection (fp32, transposed
@@ -762,6 +763,7 @@ extern "C" size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, i
 extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
   using namespace ssm;
   SSM_REQUIRE(a != nullptr, SSM_ERR_NULL_POINTER, "ssm_scan_bwd: args is NULL");
+  SSM_CHECK_RESERVED("ssm_scan_bwd", a);
   SSM_REQUIRE(a->u && a->delta && a->A && a->Bproj && a->Cproj && a->dout && a->chunk_states &&
                   a->du && a->ddelta && a->dA && a->dB && a->dC,
               SSM_ERR_NULL_POINTER,
@@ -813,14 +815,17 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
   p.softplus = a->delta_softplus ? 1 : 0;
   p.rows_per_wg = pl.rows_per_wg; p.nblk = pl.nblk;
   p.bc_vec_ok = a->seqlen % 4 == 0 && aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs);
+  // A selector of 2 (test-hooks build) lets no wave wait for its neighbour at all, so that the give-up path of
+  // the wave-per-row kernel runs: every wave goes on at once and poisons dB and dC.
+  p.spin_limit = SSM_RESERVED(a) == 2 ? 0 : (1 << 16);
 
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   int rc;
   // The specialised kernel: activations in aligned rows of whole 8-step runs, time-varying B and C of the
   // activations' type or float32, groups that workgroups of 16, 32 or 48 channels tile, and no more partial
-  // sums than the workspace was sized for.  tune_items 1 keeps the general kernel.
+  // sums than the workspace was sized for.  A selector of 1 keeps the general kernel.
   int fast_rpw = 0;
-  if (bv && cv && a->tune_items != 1 && a->seqlen % 8 == 0 &&
+  if (bv && cv && SSM_RESERVED(a) != 1 && a->seqlen % 8 == 0 &&
       (a->bc_dtype == a->io_dtype || a->bc_dtype == SSM_F32) && aligned_to(a->u, 16) && aligned_to(a->delta, 16) &&
       aligned_to(a->dout, 16) && aligned_to(a->du, 16) && aligned_to(a->ddelta, 16) &&
       (!a->z || (aligned_to(a->z, 16) && aligned_to(a->dz, 16))) && aligned_to(a->Bproj, 4 * bs) &&

@@ -34,15 +34,15 @@ __device__ __forceinline__ float lane_from(float v, int src_lane) {
 }
 
 // Wait until the count at `flag` (LDS, written by one other wave of the workgroup, only ever growing) has reached
-// `want`; false if it has not after about three milliseconds.  Every wave of a workgroup is resident and the
+// `want`; false if it has not after `spin_limit` looks (2^16 in every call of the library: about three milliseconds).  Every wave of a workgroup is resident and the
 // waves' waits form no cycle (a wave in slot k waits for slot k - 1 of its neighbour), so the wait ends; the bound
 // is there so that a mistake elsewhere ends as NaN in dB and dC (the caller poisons its sums), not as waves that
 // never finish or as sums that are silently wrong.
 typedef __attribute__((address_space(3))) int lds_int;
 
-__device__ __forceinline__ bool wait_for_slots(lds_int *flag, int want) {
+__device__ __forceinline__ bool wait_for_slots(lds_int *flag, int want, int spin_limit) {
   bool reached = false;
-  for (int spin = 0; spin < (1 << 16); ++spin) {
+  for (int spin = 0; spin < spin_limit; ++spin) {
     const int seen = __builtin_amdgcn_readfirstlane(*(volatile lds_int *)flag);
     if (seen >= want) {
       reached = true;
@@ -210,7 +210,7 @@ void scan_bwd_fast_kernel(const ScanBwdParams p) {
           // The skew gives this wave the state's part of both tiles to itself for the slot (plain read, add,
           // write), once the wave that had it in the slot before is through with it.
           float4 *aB = reinterpret_cast<float4 *>(accB + n * T + lane * 4), *aC = reinterpret_cast<float4 *>(accC + n * T + lane * 4);
-          if (!wait_for_slots(done + ((wave + BF_DEP) & (BF_WAVES - 1)), nslots)) sb[0] = sc[0] = __builtin_nanf("");
+          if (!wait_for_slots(done + ((wave + BF_DEP) & (BF_WAVES - 1)), nslots, p.spin_limit)) sb[0] = sc[0] = __builtin_nanf("");
 #pragma unroll
           for (int q = 0; q < K / 4; ++q) {
             float4 vb = aB[q * WAVE], vc = aC[q * WAVE];

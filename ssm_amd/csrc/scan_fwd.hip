@@ -73,11 +73,12 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
 
   // Two channels per wave (tune 1616) pay off once the grid still fills every CU twice.
   const bool pair_ok = bvary && cvary && a->nstate <= 16 && per_b % 16 == 0 && per_c % 16 == 0;
-  int tune = a->tune_items;
+  SSM_CHECK_RESERVED("ssm_scan_fwd", a);
+  int tune = SSM_RESERVED(a);               // 0 = automatic
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
 
   // The specialised kernel: time-varying B and C of one element type (that of the activations, or fp32), at most
-  // 16 states, aligned rows of whole 16-step runs.  tune_items 100000 + v asks for its variant v.
+  // 16 states, aligned rows of whole 16-step runs.  A selector of 100000 + v asks for its variant v.
   const bool fast_ok = bvary && cvary && a->nstate <= FAST_N && p.vec_ok && a->seqlen % 16 == 0 &&
                        aligned_to(a->Bproj, 4 * bs) && aligned_to(a->Cproj, 4 * bs) &&
                        (a->bc_dtype == a->io_dtype || a->bc_dtype == SSM_F32);
@@ -97,7 +98,7 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
     if (pick) tune = 100000 + pick;
   }
   if (tune >= 100000) {
-    SSM_REQUIRE(fast_ok, SSM_ERR_BAD_KIND, "ssm_scan_fwd: tune_items %d needs the shape of the specialised kernel", tune);
+    SSM_REQUIRE(fast_ok, SSM_ERR_BAD_KIND, "ssm_scan_fwd: selector %d needs the shape of the specialised kernel", tune);
     const int v = tune - 100000, per_wg = scan_fwd_fast_rows(v);
     SSM_REQUIRE(per_wg > 0 && per_b % per_wg == 0 && per_c % per_wg == 0, SSM_ERR_BAD_KIND,
                 "ssm_scan_fwd: variant %d takes %d channels per workgroup, which must divide a group", v, per_wg);
@@ -141,7 +142,7 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
   const int steps_per_lane = tune >= 1616 ? 8 : tune / 100;
   if (a->chunk_states)
     SSM_REQUIRE(steps_per_lane * WAVE == ssm_scan_chunk_len(), SSM_ERR_BAD_KIND,
-                "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (tune_items 808, 816 or 1616)",
+                "ssm_scan_fwd: chunk_states needs a tiling of %d steps per chunk (selectors 808, 816 or 1616)",
                 ssm_scan_chunk_len());
   switch (a->io_dtype) {
     case SSM_F32: return scan_fwd_dispatch<float>(p, tune, rows, stream);

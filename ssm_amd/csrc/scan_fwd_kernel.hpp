@@ -385,7 +385,7 @@ int scan_fwd_dispatch(const ScanFwdParams &p, int tune, int rows, hipStream_t s)
     case 1616: return dispatch_flags<io_t, 8, 16>(p, rows, s);      // 816 with two rows per wave (see entry point)
     case 2416: case 3216: case 4816: return dispatch_flags<io_t, 8, 16>(p, rows, s);   // 816 with 3, 4, 6 rows per wave
     default:
-      set_error("ssm_scan_fwd: unsupported tune_items %d (408, 808, 816, 1616, 2416)", tune);
+      set_error("ssm_scan_fwd: unsupported selector %d (408, 808, 816, 1616, 2416)", tune);
       return SSM_ERR_BAD_KIND;
   }
 }

@@ -17,9 +17,12 @@ namespace ssm {
 
 constexpr int SSD_THREADS = 256;
 
+#ifdef SSM_TEST_HOOKS
 static thread_local int g_mfma_launches = 0;   // bit0 bmm_chunk, bit1 chunk_state, bit2 chunk_scan, bit3 one-pass forward
-
 void note_mfma_launch(int bits) { g_mfma_launches |= bits; }
+#else
+void note_mfma_launch(int) {}
+#endif
 
 static unsigned grid_for(size_t n) {
   const size_t g = (n + SSD_THREADS - 1) / SSD_THREADS;
@@ -279,11 +282,13 @@ static int dims_check(const char *who, const ssm_ssd_dims &s, SsdDims &d) {
 
 }  // namespace ssm
 
-extern "C" int ssm_ssd_mfma_launches(void) {
+#ifdef SSM_TEST_HOOKS
+extern "C" int ssm_ssd_mfma_launches(void) {   // include/ssm_amd_testing.h
   const int v = ssm::g_mfma_launches;
   ssm::g_mfma_launches = 0;
   return v;
 }
+#endif
 
 extern "C" int ssm_ssd_chunk_cumsum(const ssm_ssd_cumsum_args *a, void *hip_stream) {
   using namespace ssm;
@@ -309,6 +314,7 @@ extern "C" int ssm_ssd_chunk_cumsum(const ssm_ssd_cumsum_args *a, void *hip_stre
 extern "C" int ssm_ssd_bmm_chunk(const ssm_ssd_bmm_args *a, void *hip_stream) {
   using namespace ssm;
   SSM_REQUIRE(a && a->a && a->b && a->out, SSM_ERR_NULL_POINTER, "ssm_ssd_bmm_chunk: a, b and out are required");
+  SSM_CHECK_RESERVED("ssm_ssd_bmm_chunk", a);
   SSM_REQUIRE(a->batch > 0 && a->seqlen > 0 && a->groups > 0 && a->kdim > 0 && a->chunk > 0, SSM_ERR_BAD_SHAPE,
               "ssm_ssd_bmm_chunk: batch, seqlen, groups, kdim and chunk must be positive");
   SSM_REQUIRE(valid_dtype(a->in_dtype) && valid_dtype(a->out_dtype), SSM_ERR_BAD_DTYPE,
@@ -321,12 +327,12 @@ extern "C" int ssm_ssd_bmm_chunk(const ssm_ssd_bmm_args *a, void *hip_stream) {
   const size_t total = (size_t)p.batch * p.nchunks * p.groups * p.chunk * p.chunk;
   SSM_REQUIRE(total < ((size_t)1 << 40), SSM_ERR_TOO_LARGE, "ssm_ssd_bmm_chunk: tensor too large");
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  if (!a->force_generic && ssd_bmm_mfma(p, s)) {
-    g_mfma_launches |= 1;
+  if (!SSM_RESERVED(a) && ssd_bmm_mfma(p, s)) {
+    note_mfma_launch(1);
     SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk(mfma)");
     return SSM_OK;
   }
-  if (!a->force_generic && ssd_bmm_tiled(p, s)) {
+  if (!SSM_RESERVED(a) && ssd_bmm_tiled(p, s)) {
     SSM_CHECK_LAUNCH("ssm_ssd_bmm_chunk(tiled)");
     return SSM_OK;
   }
@@ -346,6 +352,7 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   using namespace ssm;
   SSM_REQUIRE(a && a->Bm && a->x && a->dt && a->dA_cumsum && a->states, SSM_ERR_NULL_POINTER,
               "ssm_ssd_chunk_state: Bm, x, dt, dA_cumsum and states are required");
+  SSM_CHECK_RESERVED("ssm_ssd_chunk_state", a);
   SsdStateParams p{};
   int rc = dims_check("ssm_ssd_chunk_state", a->dims, p.d);
   if (rc != SSM_OK) return rc;
@@ -362,8 +369,8 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   SSM_REQUIRE(a->x_row_scale == nullptr || a->x_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE,
               "ssm_ssd_chunk_state: x_row_scale needs bfloat16 x (x_dtype=%d)", a->x_dtype);
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  if (!a->force_generic && ssd_chunk_state_mfma(p, s)) {
-    g_mfma_launches |= 2;
+  if (!SSM_RESERVED(a) && ssd_chunk_state_mfma(p, s)) {
+    note_mfma_launch(2);
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(mfma)");
     return SSM_OK;
   }
@@ -371,7 +378,7 @@ extern "C" int ssm_ssd_chunk_state(const ssm_ssd_chunk_state_args *a, void *hip_
   SSM_REQUIRE(a->x_row_scale == nullptr, SSM_ERR_BAD_SHAPE,
               "ssm_ssd_chunk_state: x_row_scale is taken by the matrix-core kernel only (bfloat16 x and B, whole "
               "chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64, a workspace)");
-  if (!a->force_generic && ssd_chunk_state_tiled(p, s)) {
+  if (!SSM_RESERVED(a) && ssd_chunk_state_tiled(p, s)) {
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_state(tiled)");
     return SSM_OK;
   }
@@ -414,6 +421,7 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   using namespace ssm;
   SSM_REQUIRE(a && a->CB && a->Cm && a->x && a->dt && a->dA_cumsum && a->prev_states && (a->y || a->dx_out),
               SSM_ERR_NULL_POINTER, "ssm_ssd_chunk_scan: CB, Cm, x, dt, dA_cumsum, prev_states and y (or dx_out) are required");
+  SSM_CHECK_RESERVED("ssm_ssd_chunk_scan", a);
   SsdScanParams p{};
   int rc = dims_check("ssm_ssd_chunk_scan", a->dims, p.d);
   if (rc != SSM_OK) return rc;
@@ -440,8 +448,8 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
     p.dx.d_per_p = a->dx_d_per_p ? 1 : 0; p.dx.dx_f32 = a->dx_out_f32 ? 1 : 0; p.dx.round_dtx = a->dx_round_dtx ? 1 : 0;
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  if (!a->force_generic && ssd_chunk_scan_mfma(p, s)) {
-    g_mfma_launches |= 4;
+  if (!SSM_RESERVED(a) && ssd_chunk_scan_mfma(p, s)) {
+    note_mfma_launch(4);
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(mfma)");
     return SSM_OK;
   }
@@ -453,7 +461,7 @@ extern "C" int ssm_ssd_chunk_scan(const ssm_ssd_chunk_scan_args *a, void *hip_st
   SSM_REQUIRE(a->x_row_scale == nullptr, SSM_ERR_BAD_SHAPE,
               "ssm_ssd_chunk_scan: x_row_scale is taken by the matrix-core kernel only (bfloat16 x, C and CB, "
               "whole chunks of a multiple of 32 up to 256 steps, nstate a multiple of 16, headdim 32 or 64)");
-  if (!a->force_generic && ssd_chunk_scan_tiled(p, s)) {
+  if (!SSM_RESERVED(a) && ssd_chunk_scan_tiled(p, s)) {
     SSM_CHECK_LAUNCH("ssm_ssd_chunk_scan(tiled)");
     return SSM_OK;
   }

@@ -22,8 +22,15 @@
 // B, C and CB are re-laid once per call so that every MFMA operand fragment is
 // one contiguous KiB (64 lanes x 8 bf16).
 //
-// Requires bf16 tensors, P = 64, Q in {64, 128, 256}, N in {64, 128},
-// L % Q == 0 and A <= 0 (the factors above are clamped to 1 individually).
+// Requires bf16 tensors, P = 64, Q in {64, 128, 256}, N in {64, 128} and L % Q == 0.
+//
+// A head with A > 0 (a growing state): the published kernels evaluate the decays inside a chunk as
+// exp(min(x, 0)) - chunk_state's weights and chunk_scan's in-chunk factors - and leave the two factors on the
+// carried state alone (exp(cs_l) on C_l.S, exp(cs[Q-1]) in state passing).  Steps are not negative, so all
+// running-sum differences of such a head are >= 0 and every factor of the split above, bounded by 1 one by
+// one, is exactly 1, as the clamp wants; what remains is to apply the unclamped growth to the carried state,
+// once per chunk in front of the state update and once per row on the carried term.  The sign of A is read
+// per head inside the kernel: no call depends on the host having looked at the values of A.
 #include "ssd_common.hpp"
 
 namespace ssm {
@@ -36,7 +43,7 @@ struct SsdFusedParams {
   __bf16 *y;
   const float *dA2, *dtv;               // (B,H,nc,Q): log2-scaled running sum, step
   const __bf16 *Cblk, *Btblk, *CBblk;   // fragment-blocked copies
-  const float *Dk, *init;
+  const float *Dk, *init, *A;
   float *final_states;
   int batch, len, heads, groups, nstate, chunk, nchunks, d_per_p;
 };
@@ -237,7 +244,7 @@ __global__ __launch_bounds__(256) void ssd_fused_prep_kernel(const SsdPrepParams
 // offset that does not change, the rest is scalar.
 constexpr int FH_THREADS = 256;
 constexpr int FH_TILE_BYTES = 16384;                       // [32][256] bf16
-constexpr int FH_LDS_BYTES = 3 * FH_TILE_BYTES + 3 * 256 * 4;
+constexpr int FH_LDS_BYTES = 3 * FH_TILE_BYTES + 4 * 256 * 4;
 
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
@@ -289,8 +296,8 @@ __device__ __forceinline__ void stream_pair(const HalfStream &st, int i, bf16x8_
 template <bool SKIP>
 __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16x8_t &a1, bf16x8_t &b0, bf16x8_t &b1,
                                                int lb, int pos0, const HalfStream &st, const __bf16 *xw, const __bf16 *xr,
-                                               const float *dAs, const float *dqs, int Q, int qmask, int m, int g2,
-                                               float dskip) {
+                                               const float *dAs, const float *dqs, const float *l2s, int Q, int qmask,
+                                               int m, int g2, float dskip) {
   float prev_end = 0.0f;
   const int lrow = 32 * lb + m;
   const float dal = dAs[lrow];
@@ -323,12 +330,16 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
     const bf16x8_t f = kk == 0 ? a0 : a1;
     const int sbase = 32 * lb + 16 * kk + 8 * g2;
     const float4 q0 = *reinterpret_cast<const float4 *>(dqs + sbase), q1 = *reinterpret_cast<const float4 *>(dqs + sbase + 4);
+    const float4 c0 = *reinterpret_cast<const float4 *>(l2s + sbase), c1 = *reinterpret_cast<const float4 *>(l2s + sbase + 4);
     const float dq[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const float cap[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
     float mv[8];
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
-      // dt_s exp(cs_l - cs_s) as one exponential; the bound keeps the (zeroed) places above the diagonal finite
-      const float e = exp2_hw(fminf(dal + dq[jj], 126.0f));
+      // dt_s exp(min(cs_l - cs_s, 0)) as one exponential: min(a, 0) + b = min(a + b, b) with b = log2 dt_s.  The
+      // bound is inactive on and below the diagonal of a decaying head, is the clamp of a growing one, and keeps
+      // the (zeroed) places above the diagonal finite.
+      const float e = exp2_hw(fminf(dal + dq[jj], cap[jj]));
       if (SKIP) {
         // element jj of fragment kk lies on the diagonal in lane 16 kk + jj (g2 = 0) and lane 32 + 16 kk + 8 + jj (g2 = 1)
         const unsigned long long on_diag = (1ull << (16 * kk + jj)) | (1ull << (40 + 16 * kk + jj));
@@ -373,6 +384,7 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
   float *dAs = reinterpret_cast<float *>(smem + 3 * FH_TILE_BYTES);     // [Q] log2-scaled running sum
   float *dqs = dAs + 256;                                               // [Q] log2(dt) - running sum: exponent offset of a step as a source
   float *wss = dqs + 256;                                               // [Q] staging weight dt exp(cs[l | 31] - cs[l])
+  float *l2s = wss + 256;                                               // [Q] log2(dt): the bound of a source step's exponent
 
   const int H = p.heads, G = p.groups, nc = p.nchunks;
   constexpr int NLB = Q >> 5, NT = N >> 5, KS = Q >> 4, KN = N >> 4;
@@ -396,6 +408,7 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
   const bool has_init = p.init != nullptr;
   const int xrow_b = H * FU_P * 2;                     // bytes between rows of x, z and y
   const float dhead = DMODE == 1 ? p.Dk[h] : 0.0f;
+  const bool grow = p.A[h] > 0.0f;                     // a growing state: see the head of this file
   const int tid = wave * WAVE + lane;
 
   // ---- buffers and the lanes' constant offsets
@@ -483,8 +496,10 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     if (tid < Q) {                         // whole waves: Q is a multiple of 64
       // weight of a step towards the end of its block of 32: the running sum there is in lane | 31
       const float w_t = dt_t * exp2_hw(fminf(__shfl(dA_t, lane | 31, WAVE) - dA_t, 0.0f));
+      const float l2_t = log2_hw(dt_t);    // dt = 0: -inf, a weight of zero
       dAs[tid] = dA_t;
-      dqs[tid] = log2_hw(dt_t) - dA_t;     // dt = 0: -inf, a weight of zero
+      dqs[tid] = l2_t - dA_t;
+      l2s[tid] = l2_t;
       wss[tid] = w_t;
       wave_lds_sync();                     // the eight weights this thread needs come from its own wave
       const float4 wa = *reinterpret_cast<const float4 *>(wss + slb8 * 8), wb = *reinterpret_cast<const float4 *>(wss + slb8 * 8 + 4);
@@ -538,6 +553,14 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
       FH_STEP_A(f2, f3, KN - 1)
       stream_pair(st, 2, f2, f3);
 #undef FH_STEP_A
+      if (grow) {                          // the carried term of a growing head takes exp(cs_l), unclamped
+        const float gF = exp2_hw(fmaxf(dAs[32 * lbF + m], 0.0f)), gS = exp2_hw(fmaxf(dAs[32 * lbS + m], 0.0f));
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          accF[r] *= gF;
+          accS[r] *= gS;
+        }
+      }
     } else if (yact) {                     // first chunk without an initial state
       accF = (f32x16_t){0};
       accS = (f32x16_t){0};
@@ -551,9 +574,9 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     // ---- the two row blocks.  Pair q of the stream lives in (f0, f1) if q is even, in (f2, f3) if odd:
     // the diagonal block of the first row block is pair lbF, that of the second pair NLB.
     if (yact) {
-      if (lbF & 1) half_row_block<DMODE == 1>(accF, f2, f3, f0, f1, lbF, 0, st, xw, xr, dAs, dqs, Q, qmask, m, g2, dhead);
-      else half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dqs, Q, qmask, m, g2, dhead);
-      half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dqs, Q, qmask, m, g2, dhead);
+      if (lbF & 1) half_row_block<DMODE == 1>(accF, f2, f3, f0, f1, lbF, 0, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
+      else half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
+      half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
       if constexpr (DMODE == 2) {
         half_skip_term(accF, lbF, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
         half_skip_term(accS, lbS, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
@@ -594,6 +617,11 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
         /* the requests go out here: the scheduler must not sink them into the update */        \
         asm volatile("" ::: "memory");                                                          \
       }
+    if (sact && grow) {                    // the carried state of a growing head takes exp(cs[Q-1]), unclamped
+      const float gt = exp2_hw(fmaxf(dAs[Q - 1], 0.0f));
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[r] *= gt;
+    }
     if (sact) {
 #pragma unroll
       for (int k0 = 0; k0 < KS; k0 += 4) {
@@ -794,7 +822,7 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   fp.y = reinterpret_cast<__bf16 *>(a->y);
   fp.dA2 = reinterpret_cast<const float *>(ws + lay.dA2); fp.dtv = cp.dt_out;
   fp.Cblk = Cblk; fp.CBblk = reinterpret_cast<const __bf16 *>(ws + lay.CBblk); fp.Btblk = Btblk;
-  fp.Dk = a->Dskip; fp.init = a->initial_states; fp.final_states = a->final_states;
+  fp.Dk = a->Dskip; fp.init = a->initial_states; fp.A = a->A; fp.final_states = a->final_states;
   fp.batch = d.batch; fp.len = d.len; fp.heads = d.heads; fp.groups = d.groups; fp.nstate = d.nstate; fp.chunk = d.chunk;
   fp.nchunks = d.nchunks; fp.d_per_p = a->d_per_p ? 1 : 0;
   const int dmode = !a->Dskip ? 0 : (a->d_per_p ? 2 : 1);

@@ -81,7 +81,7 @@ class ScanPlan:
             batch=batch, dim=dim, seqlen=length, nstate=nstate,
             io_dtype=_lib.dtype_enum(io), bc_dtype=_lib.dtype_enum(bc),
             b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
-            delta_softplus=int(bool(softplus)), tune_items=int(tune_items))
+            delta_softplus=int(bool(softplus)), reserved=int(tune_items))
 
     def run(self):
         _lib.call("ssm_scan_fwd", self.args, self.device)
@@ -170,7 +170,7 @@ def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softpl
             ddt_bias=_lib.ptr(dbias_b), workspace=ws_ptr, workspace_bytes=nbytes,
             batch=batch, dim=dim, seqlen=length, nstate=n_blk, io_dtype=_lib.dtype_enum(io),
             bc_dtype=_lib.dtype_enum(bc), b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
-            delta_softplus=int(bool(softplus)), tune_items=int(tune_items))
+            delta_softplus=int(bool(softplus)), reserved=int(tune_items))
         _lib.call("ssm_scan_bwd", args, dev)
         if single:
             du, ddl, dz, dbias = du_b, ddl_b, dz_b, dbias_b
@@ -599,7 +599,7 @@ def _dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_s
         z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
         init_dtype=_lib.dtype_enum(ic.dtype) if ic is not None else 0,
         b_kind=bk, c_kind=ck, a_per_p=int(a_per_p), d_per_p=int(d_per_p), z_per_p=int(z_per_p),
-        grads_in_io_dtype=int(io), tune_two_kernels=int(bool(two_kernels)))
+        grads_in_io_dtype=int(io), reserved=int(bool(two_kernels)))
     if round_states is not None:
         want = (batch, (seqlen + 63) // 64, heads * proj)
         if tuple(round_states.shape) != want or round_states.dtype != torch.float32 or not round_states.is_contiguous():

@@ -15,7 +15,6 @@ Shapes: ``x, z, y (B, L, H, P)``; ``dt (B, L, H)``; ``A (H,)``; ``B, C (B, L, G,
 from __future__ import annotations
 
 import math
-import weakref
 from typing import Optional
 
 import torch
@@ -107,7 +106,7 @@ def bmm_chunk(a, b, chunk_size, seq_idx=None, causal=False, output_dtype=None, f
     args = _lib.SsdBmmArgs(a=_lib.ptr(ac), b=_lib.ptr(bc), seq_idx=_lib.ptr(si), out=_lib.ptr(out),
                            batch=batch, seqlen=seqlen, groups=groups, kdim=kdim, chunk=Q,
                            in_dtype=_lib.dtype_enum(io), out_dtype=_lib.dtype_enum(out_dt),
-                           causal=int(bool(causal)), force_generic=int(bool(force_generic)))
+                           causal=int(bool(causal)), reserved=int(bool(force_generic)))
     _lib.call("ssm_ssd_bmm_chunk", args, dev)
     return out if grouped else out[:, :, 0]
 
@@ -190,7 +189,7 @@ def chunk_state(B, x, dt, dA_cumsum, states_dtype=torch.float32, force_generic=F
         workspace=_lib.ptr(ws), workspace_bytes=nbytes,
         dims=dims, x_dtype=_lib.dtype_enum(xc.dtype),
         b_dtype=_lib.dtype_enum(Bc.dtype), states_dtype=_lib.dtype_enum(states_dtype),
-        force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)),
+        reserved=int(bool(force_generic)), seq_idx=_lib.ptr(si), x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)),
         x_time_reversed=int(bool(x_reversed)))
     _lib.call("ssm_ssd_chunk_state", args, dev)
     return states
@@ -314,7 +313,7 @@ def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None, CB=None, for
         dims=_dims(batch, seqlen, heads, hdim, groups, nstate, Q), x_dtype=_lib.dtype_enum(xc.dtype),
         c_dtype=_lib.dtype_enum(Cc.dtype), cb_dtype=_lib.dtype_enum(cb.dtype),
         states_dtype=_lib.dtype_enum(ps.dtype), z_dtype=_lib.dtype_enum(zc.dtype) if zc is not None else 0,
-        d_per_p=int(d_per_p), force_generic=int(bool(force_generic)), seq_idx=_lib.ptr(si), y_f32=int(bool(out_f32)),
+        d_per_p=int(d_per_p), reserved=int(bool(force_generic)), seq_idx=_lib.ptr(si), y_f32=int(bool(out_f32)),
         x_row_scale=_lib.ptr(_scale_arg(x_scale, dt)), x_time_reversed=int(bool(x_reversed)))
     if dx_epilogue is not None:
         args.dx_x, args.dx_dt, args.dx_Dskip = _lib.ptr(ex), _lib.ptr(edt), _lib.ptr(eDf)
@@ -365,30 +364,6 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
         states_dtype=_lib.dtype_enum(cs.dtype))
     _lib.call("ssm_ssd_chunk_state_varlen", args, dev)
     return out
-
-
-_DECAYING = {}        # id of an A tensor -> (weak reference, version, all(A <= 0)), so that a persistent parameter is read once
-
-
-def _is_decaying(A):
-    """``all(A <= 0)``: what the one-pass kernel assumes (it bounds each factor of a decay by 1; with a growing
-    state its results are wrong, while the five kernels keep the upstream kernels' behaviour there).  Reading the
-    answer costs a device synchronisation, so it is remembered per tensor object (while that object lives and its
-    version counter stands: an address alone may pass to another tensor) and not looked up at all while a stream is
-    being captured, where the caller's word (``fused=True``) or the default is taken."""
-    if torch.cuda.is_current_stream_capturing():
-        return True
-    hit = _DECAYING.get(id(A))
-    if hit is not None and hit[0]() is A and hit[1] == A._version:
-        return hit[2]
-    if len(_DECAYING) > 4096:
-        _DECAYING.clear()
-    answer = bool((A.detach() <= 0).all())
-    try:
-        _DECAYING[id(A)] = (weakref.ref(A), A._version, answer)
-    except TypeError:              # an object that cannot be weakly referenced: not remembered
-        pass
-    return answer
 
 
 def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
@@ -477,16 +452,16 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
         return_final_states: Also return the state after the last token.
         states_dtype: dtype of the per-chunk states kept in HBM between the kernels
             (default: ``x.dtype``; the recurrence itself accumulates in float32).
-        fused: ``None`` picks the one-pass kernel when it applies and ``A <= 0`` everywhere (looked up
-            once per ``A`` tensor: a device synchronisation the first time a tensor is seen), ``False``
-            never uses it, ``True`` requires it (``ValueError`` if the call is not covered) and takes
-            the caller's word that ``A <= 0``: with a growing state its results are wrong.
+        fused: ``None`` picks the one-pass kernel when it covers the call, ``False`` never uses it,
+            ``True`` requires it (``ValueError`` if the call is not covered).  The values of ``A`` play no
+            part in the choice and are never read on the host: the kernel looks at the sign of a head's
+            ``A`` itself and treats a growing state as the five kernels do (decays inside a chunk bounded
+            by 1, the carried state growing freely).
         seq_idx: Optional ``(B, L)`` int sequence ids of a packed batch (ids start at 0):
             no state and no product crosses from one sequence into the next.  The five kernels
             mask exactly.  The one-pass kernel (picked for bfloat16 calls it covers) and the
             backward separate sequences by an extra decay of ``2**-64`` at every first step
-            instead: what crosses a boundary is scaled by 5e-20, which is exact in effect for
-            the decaying ``A <= 0`` both require.
+            instead: what crosses a boundary is scaled by 5e-20.
         cu_seqlens: Optional ``(nseq + 1,)`` sequence boundaries of a packed batch row
             (batch size 1), only used for ``return_varlen_states``.
         return_varlen_states: Also return the state at the last step of every sequence,
@@ -583,8 +558,6 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
         return outs[0] if len(outs) == 1 else tuple(outs)
     can_fuse = not force_generic and fused is not False and not return_varlen_states and \
         _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
-    if can_fuse and fused is None and not _is_decaying(A):
-        can_fuse = False          # a growing state: only the five kernels follow the upstream kernels there
     _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "
           "chunk in {64,128,256}, nstate in {64,128} and seqlen % chunk == 0.")
     if can_fuse:
@@ -658,6 +631,10 @@ def varlen_states_backward(dstates, x, dt, A, B, cu_seqlens, dt_bias=None, initi
     per = heads // groups
     f32 = torch.float32
     Af = A.detach().to(f32)
+    # The forward bounds the decays inside a chunk by 1 and lets the carried state grow across chunks, which is
+    # not the plain sum this function differentiates; the two agree for a decaying system only.  (This path
+    # already reads cu_seqlens on the host, so the look at A costs no further synchronisation.)
+    _need(bool((Af <= 0).all()), "gradients through the per-sequence end states need A <= 0 on every head.")
     u = dt.detach().to(f32)[0]                                  # (L, H)
     if dt_bias is not None:
         u = u + dt_bias.detach().to(f32)
@@ -680,7 +657,7 @@ def varlen_states_backward(dstates, x, dt, A, B, cu_seqlens, dt_bias=None, initi
         G = G_all[i]                                            # (H, P, N)
         dts = dtp[a:e]
         cum = torch.cumsum(dts * Af, dim=0)
-        w = torch.exp((cum[-1:] - cum).clamp(max=0.0))          # decay from after step t to the end
+        w = torch.exp(cum[-1:] - cum)                           # decay from after step t to the end
         xs = xf[a:e].to(f32)
         Bh = Bf[a:e].to(f32).repeat_interleave(per, dim=1)      # (l, H, N)
         GB = torch.einsum("hpn,lhn->lhp", G, Bh)
@@ -693,7 +670,7 @@ def varlen_states_backward(dstates, x, dt, A, B, cu_seqlens, dt_bias=None, initi
         # dt_r A enters every term of an earlier step: the sum of those terms
         ddA = torch.cumsum(contrib, dim=0) - contrib
         if a == 0 and initial_states is not None:
-            tot = torch.exp(cum[-1].clamp(max=0.0))             # (H,)
+            tot = torch.exp(cum[-1])                            # (H,)
             dinit[0] = tot[:, None, None] * G
             ddA = ddA + (tot * (G * initial_states.detach()[0].to(f32)).sum(dim=(1, 2)))[None]
         ddtp[a:e] = w * sdot + ddA * Af
@@ -883,13 +860,30 @@ def _bwd_states(ent_f, ent_r):
     return f16, r16, anchor
 
 
+_BMM_F32_OUT = None       # whether this torch build's bmm forms float32 results from bfloat16 operands (probed once)
+
+
+def _bmm_has_f32_out(device):
+    global _BMM_F32_OUT
+    if _BMM_F32_OUT is None:
+        probe = torch.ones(1, 16, 16, dtype=torch.bfloat16, device=device)
+        try:
+            _BMM_F32_OUT = torch.bmm(probe, probe, out_dtype=torch.float32).dtype == torch.float32
+        except (TypeError, RuntimeError, NotImplementedError):
+            _BMM_F32_OUT = False
+    return _BMM_F32_OUT
+
+
 def _mm_f32(a, b):
-    """Batched product of bfloat16 matrices with a float32 result."""
-    try:
-        return torch.bmm(a.reshape(-1, *a.shape[-2:]), b.reshape(-1, *b.shape[-2:]),
-                         out_dtype=torch.float32).view(*a.shape[:-1], b.shape[-1])
-    except (TypeError, RuntimeError):
-        return torch.matmul(a, b).float()
+    """Batched product of bfloat16 matrices with float32 accumulation and a float32 result.  Where the torch
+    build has no ``out_dtype`` for ``bmm`` the operands are raised to float32 first, so the accuracy does not
+    depend on the build; an error of the product itself (shapes, memory) surfaces as it is."""
+    a3, b3 = a.reshape(-1, *a.shape[-2:]), b.reshape(-1, *b.shape[-2:])
+    if _bmm_has_f32_out(a.device):
+        out = torch.bmm(a3, b3, out_dtype=torch.float32)
+    else:
+        out = torch.bmm(a3.float(), b3.float())
+    return out.view(*a.shape[:-1], b.shape[-1])
 
 
 def _dB_dC_from_chunks(dyc, xc, Bc, Cc, dt_c, dA_cs, wdy, xw, f16, r16, groups):

@@ -138,6 +138,34 @@ def test_shape_and_dtype_errors_come_back_as_status_codes():
     assert lib.ssm_scan_bwd_workspace_bytes(8, 1536, 2048, 16, 2, 2, 7, 1) == 0
 
 
+def test_shipped_library_has_no_test_hooks_and_the_hooks_build_does():
+    """Kernel selectors and the record of kernels taken exist in the -DSSM_TEST_HOOKS build only
+    (include/ssm_amd_testing.h): the shipped library rejects a non-zero ``reserved`` field and does not export
+    ``ssm_ssd_mfma_launches``; the hooks build exports everything the header declares plus that."""
+    L = _lib()
+    lib, hooks = L.load(), L.load_test_hooks()
+    assert not hasattr(lib, "ssm_ssd_mfma_launches")
+    assert hooks.ssm_ssd_mfma_launches() == 0
+    missing = [n for n in declared_functions() if not hasattr(hooks, n)]
+    assert not missing, missing
+    buf = (ctypes.c_float * 64)()
+    p = ctypes.addressof(buf)
+    a = L.ScanFwdArgs(u=p, delta=p, A=p, Bproj=p, Cproj=p, out=p, batch=1, dim=2, seqlen=4, nstate=2, reserved=808)
+    assert lib.ssm_scan_fwd(ctypes.byref(a), None) == -4
+    assert b"reserved" in lib.ssm_amd_last_error()
+    for name in ("ssm_scan_bwd", "ssm_dscan_bwd", "ssm_ssd_bmm_chunk", "ssm_ssd_chunk_state", "ssm_ssd_chunk_scan"):
+        args = L.ENTRY_POINTS[name]()
+        for field, ctype in args._fields_:
+            if ctype is ctypes.c_void_p:
+                setattr(args, field, p)            # past the NULL checks; the reserved check comes before any use
+        args.reserved = 1
+        assert getattr(lib, name)(ctypes.byref(args), None) == -4, name
+        assert b"reserved" in lib.ssm_amd_last_error(), name
+    with L.test_hooks_build() as inside:
+        assert inside is hooks and L.load() is hooks
+    assert L.load() is lib
+
+
 def test_missing_library_fails_loudly(tmp_path):
     code = ("import os, sys; os.environ['SSM_AMD_LIB'] = r'%s'; sys.path.insert(0, r'%s');\n"
             "from ssm_amd import _lib\n"

@@ -113,6 +113,90 @@ def test_config3_outer_shape_bf16_slice():
     torch.testing.assert_close(y[:, :, hs].float().cpu(), yr.float(), **HALF_TOL)
 
 
+def _full_size_heads_oracle(inp, hs, gy, chunk):
+    """Forward in float32 and all gradients in float64 of the heads ``hs`` alone (heads are independent)."""
+    def cut(k, v):
+        if v is None:
+            return None
+        if k in ("X", "z", "dt") or v.ndim == 4:
+            return v[:, :, hs]
+        return v[hs]
+    sub = {k: cut(k, v) for k, v in inp.items()}
+    y32 = O.ssd_chunk_scan(sub["X"], sub["dt"], sub["A"], sub["B"], sub["C"], chunk, D=sub["D"], z=sub["z"])
+    leaves = {k: (v.double().clone().requires_grad_(True) if v is not None else None) for k, v in sub.items()}
+    y = O.ssd_chunk_scan(leaves["X"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], chunk, D=leaves["D"],
+                         z=leaves["z"], acc=torch.float64)
+    (y.double() * gy[:, :, hs].double()).sum().backward()
+    return y32, {k: (v.grad if v is not None else None) for k, v in leaves.items()}, cut
+
+
+def test_config3_outer_shape_one_pass_per_token_projections():
+    """(B, L, H, P) = (4, 4096, 80, 64), bf16 X, z and per-token B, C of X's shape, **float32 dt**, per-head A and
+    D: the call whose forward and backward ``bench.py`` times, which runs the one-pass kernels on a grid of
+    320 workgroups.  Forward and, through autograd (which hands the forward's table of round states over), all
+    seven gradients of two heads against the oracle on those heads alone (float64 autograd for the gradients)."""
+    from tests.closeness import half_close
+    g = torch.Generator().manual_seed(43)
+    b, l, h, p = 4, 4096, 80, 64
+    inp = dict(X=torch.randn(b, l, h, p, generator=g).to(torch.bfloat16),
+               dt=torch.rand(b, l, h, generator=g) * 0.1,
+               A=-(torch.rand(h, generator=g) * 15 + 1),
+               B=torch.randn(b, l, h, p, generator=g).to(torch.bfloat16),
+               C=torch.randn(b, l, h, p, generator=g).to(torch.bfloat16),
+               D=torch.ones(h), z=torch.randn(b, l, h, p, generator=g).to(torch.bfloat16))
+    gy = torch.randn(b, l, h, p, generator=g).to(torch.bfloat16)
+    hs = [0, 41, 79]
+    as_f32 = {k: v.float() for k, v in inp.items()}
+    yr, want, cut = _full_size_heads_oracle(as_f32, hs, gy.float(), 256)
+    leaves = {k: dev(v).requires_grad_(True) for k, v in inp.items()}
+    y = _ops().ssd_chunk_scan(leaves["X"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], 256, D=leaves["D"],
+                              z=leaves["z"])
+    assert y.dtype == torch.bfloat16
+    torch.testing.assert_close(y[:, :, hs].float().cpu(), yr.float(), **HALF_TOL)
+    (y * dev(gy)).sum().backward()
+    for k, v in leaves.items():
+        assert v.grad.dtype == inp[k].dtype and v.grad.shape == inp[k].shape, k
+        half_close(cut(k, v.grad), want[k], what=f"grad {k}", atol_rms=4e-2, mean_rms=5e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+def test_config3_outer_shape_one_pass_module_call(dtype):
+    """The call of the reference's Mamba2 module at (4, 4096, 80, 64): B, C, A, D as (H, P) float32 parameters, no
+    gate, float32 dt (``/root/reference/src/ssm/modules/mamba2.py:189-199``), activations in float32 as the module
+    promotes them and in bf16.  Forward and, through autograd, all gradients of three heads against the oracle
+    (float64 autograd for the gradients; the float32 oracle arbitrates float32 values)."""
+    from tests.closeness import fp32_close, half_close
+    g = torch.Generator().manual_seed(44)
+    b, l, h, p = 4, 4096, 80, 64
+    inp = dict(X=torch.randn(b, l, h, p, generator=g).to(dtype),
+               dt=torch.rand(b, l, h, generator=g) * 0.1,
+               A=-(torch.rand(h, p, generator=g) * 15 + 1),
+               B=torch.randn(h, p, generator=g), C=torch.randn(h, p, generator=g),
+               D=torch.ones(h, p), z=None)
+    gy = torch.randn(b, l, h, p, generator=g).to(dtype)
+    hs = [1, 40, 78]
+    as_f32 = {k: (v.float() if v is not None else None) for k, v in inp.items()}
+    yr, want, cut = _full_size_heads_oracle(as_f32, hs, gy.float(), 256)
+    leaves = {k: (dev(v).requires_grad_(True) if v is not None else None) for k, v in inp.items()}
+    y = _ops().ssd_chunk_scan(leaves["X"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], 256, D=leaves["D"])
+    assert y.dtype == dtype
+    half = dtype != torch.float32
+    torch.testing.assert_close(y[:, :, hs].float().cpu(), yr.float(), **(HALF_TOL if half else FP32_TOL))
+    (y * dev(gy)).sum().backward()
+    # float32 autograd through the oracle: what float32 sums over 16384 steps are worth
+    l32 = {k: (cut(k, v).clone().requires_grad_(True) if v is not None else None) for k, v in as_f32.items()}
+    y32 = O.ssd_chunk_scan(l32["X"], l32["dt"], l32["A"], l32["B"], l32["C"], 256, D=l32["D"])
+    (y32 * gy[:, :, hs].float()).sum().backward()
+    for k, v in leaves.items():
+        if v is None:
+            continue
+        assert v.grad.dtype == inp[k].dtype and v.grad.shape == inp[k].shape, k
+        if half:
+            half_close(cut(k, v.grad), want[k], what=f"grad {k}", atol_rms=4e-2, mean_rms=5e-3)
+        else:
+            fp32_close(cut(k, v.grad), want[k], oracle32=l32[k].grad, what=f"grad {k}", rtol=1e-4, atol_rms=1e-5)
+
+
 # ---------------------------------------------------------------------------
 # backward: all eight gradients against float64 autograd through the CPU restatement
 # ---------------------------------------------------------------------------

@@ -2,12 +2,14 @@
 one: every operator's values and gradients against the CPU oracle evaluated in float64.
 
 Each case draws its shape and options from ``random.Random(seed)`` and its data from a torch generator, so a
-failure names a case that can be rebuilt from the seed alone.  Bars: float32 tensors 2e-4 (values) / 5e-4
-(gradients), 16-bit tensors 2e-2 / 3e-2, of the largest magnitude of the expected tensor — the float64 oracle
+failure names a case that can be rebuilt from the seed alone.  Bars (``_close``): every element within a relative
+bound of itself plus a fraction of the root mean square of the expected tensor -- float32 tensors 1e-5 (values) /
+1e-4 + 1e-5 (gradients), with the float32 oracle arbitrating elements beyond that (the kernel may be at most four
+times as far from the float64 value as the float32 oracle is at its worst); 16-bit tensors 2e-2 + 4e-2 of the
+rms (values) / 3e-2 + 6e-2 (gradients) and a mean error of at most 5e-3 / 1e-2 of the rms -- the float64 oracle
 does not round its result to the element type, so a 16-bit output carries its own last-place rounding on top
 of the accumulated error.  For the SSD the two gradients that are sums over the whole sequence with cancelling
-terms (``dA``, the bias of the step) are measured against the sum of the magnitudes of their terms where those
-are available (the bias: the step's own gradient), and ``dA`` against the largest head."""
+terms (``dA``, the bias of the step) are measured against the sum of the magnitudes of their terms."""
 
 import random
 
@@ -28,11 +30,35 @@ def _ops():
     return ops
 
 
-def _rel(a, r):
+def _close(a, r64, what, half=False, grad=False, r32=None, rtol=None, atol_rms=None, mean_rms=None):
+    """``a`` (from the GPU) against the float64 oracle's ``r64``, element by element: within ``rtol`` of the element
+    itself plus ``atol_rms`` of the root mean square of the expected tensor (not of its largest element).
+    16-bit calls (``half``): one rounding of the result plus the float32 arithmetic behind it, with a bound on
+    the mean error an order of magnitude lower.  float32 calls: 1e-5 for values and 1e-4 for gradients; an element
+    outside that still passes when the float32 oracle ``r32`` is itself that far from the float64 value somewhere
+    (at most four times its largest error): two float32 sums of the same terms in different orders."""
     a = a.detach().double().cpu()
-    r = r.detach().double().cpu()
-    assert torch.isfinite(a).all()
-    return float((a - r).abs().max()) / (float(r.abs().max()) + 1e-30)
+    r = r64.detach().double().cpu()
+    assert a.shape == r.shape, (what, tuple(a.shape), tuple(r.shape))
+    assert torch.isfinite(a).all(), what
+    if r.numel() == 0:
+        return
+    rms = float(r.pow(2).mean().sqrt()) + 1e-30
+    err = (a - r).abs()
+    if half:
+        rt, at, mt = (3e-2, 6e-2, 1e-2) if grad else (2e-2, 4e-2, 5e-3)
+    else:
+        rt, at, mt = (1e-4, 1e-5, None) if grad else (1e-5, 1e-5, None)
+    rt = rt if rtol is None else rtol
+    at = at if atol_rms is None else atol_rms
+    mt = mt if mean_rms is None else mean_rms
+    bar = rt * r.abs() + at * rms
+    if r32 is not None:
+        bar = torch.clamp(bar, min=4.0 * float((r32.detach().double().cpu() - r).abs().max()))
+    worst = float((err / (bar + 1e-300)).max())
+    assert worst <= 1.0, (what, "max err / rms %.3e" % (float(err.max()) / rms), "err / bar %.2f" % worst)
+    if mt is not None:
+        assert float(err.mean()) <= mt * rms, (what, "mean err / rms %.3e" % (float(err.mean()) / rms))
 
 
 def _leaf(t, grad=True):
@@ -41,26 +67,38 @@ def _leaf(t, grad=True):
     return (t.cuda().detach().requires_grad_(grad), t.double().detach().requires_grad_(grad))
 
 
-def _values_and_gradients(fn_dev, fn_ref, ins, desc, tol, gtol):
+def _values_and_gradients(fn_dev, fn_ref, ins, desc, half):
+    """``fn_ref(acc, *tensors)`` is the oracle: float64 arithmetic with ``acc=torch.float64``, the reference's own
+    float32 with ``acc=None`` (run for float32 calls only, to arbitrate)."""
     devs, refs = zip(*[_leaf(t) for t in ins])
-    out_d, out_r = fn_dev(*devs), fn_ref(*refs)
+    out_d, out_r = fn_dev(*devs), fn_ref(torch.float64, *refs)
+    refs32 = out_32 = None
+    if not half:
+        refs32 = [None if t is None else t.detach().clone().requires_grad_(True) for t in ins]
+        out_32 = fn_ref(None, *refs32)
     if not isinstance(out_d, tuple):
         out_d, out_r = (out_d,), (out_r,)
+        out_32 = None if out_32 is None else (out_32,)
     for i, (a, r) in enumerate(zip(out_d, out_r)):
-        assert _rel(a, r) < tol, (desc, "output", i)
+        _close(a, r, (desc, "output", i), half=half, r32=None if out_32 is None else out_32[i])
     g = torch.Generator().manual_seed(7)
-    loss_d = loss_r = 0
-    for a, r in zip(out_d, out_r):
+    loss_d = loss_r = loss_32 = 0
+    for i, (a, r) in enumerate(zip(out_d, out_r)):
         w = torch.randn(r.shape, generator=g, dtype=torch.float64).to(a.dtype).double()
         loss_d = loss_d + (a.double() * w.cuda()).sum()
         loss_r = loss_r + (r * w).sum()
+        if out_32 is not None:
+            loss_32 = loss_32 + (out_32[i] * w.float()).sum()
     loss_d.backward()
     loss_r.backward()
+    if out_32 is not None:
+        loss_32.backward()
     for i, (d, r) in enumerate(zip(devs, refs)):
         if d is None:
             continue
         assert d.grad is not None and r.grad is not None, (desc, "gradient", i)
-        assert _rel(d.grad, r.grad) < gtol, (desc, "gradient", i)
+        _close(d.grad, r.grad, (desc, "gradient", i), half=half, grad=True,
+               r32=None if refs32 is None else refs32[i].grad)
 
 
 def _scan_case(rng, seed):
@@ -86,8 +124,8 @@ def _scan_case(rng, seed):
     half = dtype in HALF
     desc = ("scan", seed, (b, d, l, n), kind, groups, str(dtype), D is not None, z is not None, bias is not None, sp)
     _values_and_gradients(lambda *a: _ops().selective_scan(*a, softplus=sp, return_last_state=True),
-                          lambda *a: O.selective_scan(*a, softplus=sp, return_last_state=True, acc=torch.float64),
-                          [u, delta, A, Bm, Cm, D, z, bias], desc, 2e-2 if half else 2e-4, 3e-2 if half else 5e-4)
+                          lambda acc, *a: O.selective_scan(*a, softplus=sp, return_last_state=True, acc=acc),
+                          [u, delta, A, Bm, Cm, D, z, bias], desc, half)
 
 
 def _step_case(rng, seed):
@@ -115,9 +153,11 @@ def _step_case(rng, seed):
     new_state = devs[0].clone()
     y = _ops().selective_state_step(new_state, *devs[1:], softplus=sp)
     y_ref, state_ref = O.selective_state_step_functional(*refs, softplus=sp, acc=torch.float64)
-    tol = 2e-2 if half else 2e-4
-    assert _rel(y, y_ref) < tol, desc
-    assert _rel(new_state, state_ref) < tol, desc
+    y_32 = s_32 = None
+    if not half:
+        y_32, s_32 = O.selective_state_step_functional(state, x, dt, A, Bm, Cm, D, z, bias, softplus=sp)
+    _close(y, y_ref, (desc, "y"), half=half, r32=y_32)
+    _close(new_state, state_ref, (desc, "state"), half=half, r32=s_32)
 
 
 def _conv_case(rng, seed):
@@ -137,13 +177,12 @@ def _conv_case(rng, seed):
     half = dtype in HALF
     fn = _ops().dw_causal_conv_channels_last if channels_last else _ops().dw_causal_conv
 
-    def ref(x, w, bias):
+    def ref(acc, x, w, bias):
         if channels_last:
-            return O.dw_causal_conv(x.transpose(1, 2), w, bias, activation=act, acc=torch.float64).transpose(1, 2)
-        return O.dw_causal_conv(x, w, bias, activation=act, acc=torch.float64)
+            return O.dw_causal_conv(x.transpose(1, 2), w, bias, activation=act, acc=acc).transpose(1, 2)
+        return O.dw_causal_conv(x, w, bias, activation=act, acc=acc)
 
-    _values_and_gradients(lambda x, w, bias: fn(x, w, bias, activation=act), ref, [x, w, bias], desc,
-                          2e-2 if half else 2e-4, 3e-2 if half else 5e-4)
+    _values_and_gradients(lambda x, w, bias: fn(x, w, bias, activation=act), ref, [x, w, bias], desc, half)
 
 
 def _norm_case(rng, seed):
@@ -164,8 +203,8 @@ def _norm_case(rng, seed):
     half = dtype in HALF
     kw = dict(is_rms=rms, prenorm=prenorm, residual_in_fp32=res_fp32)
     _values_and_gradients(lambda x, w, bias, res: _ops().fused_layer_norm_with_residual(x, w, bias, residual=res, **kw),
-                          lambda x, w, bias, res: O.fused_layer_norm_with_residual(x, w, bias, residual=res, acc=torch.float64, **kw),
-                          [x, w, bias, res], desc, 2e-2 if half else 2e-4, 3e-2 if half else 5e-4)
+                          lambda acc, x, w, bias, res: O.fused_layer_norm_with_residual(x, w, bias, residual=res, acc=acc, **kw),
+                          [x, w, bias, res], desc, half)
 
 
 def _decode_case(rng, seed):
@@ -185,7 +224,7 @@ def _decode_case(rng, seed):
     st_ref = torch.randn(b, d, n, generator=g)
     cs, st = cs_ref.to(io).cuda(), st_ref.clone().cuda()
     desc = ("decode", seed, (b, d, n, K), grp, str(io), D is not None, use_z, bias is not None, use_cb, act)
-    tol = 2e-4 if io == torch.float32 else 2e-2
+    half = io != torch.float32
     dev = lambda t: None if t is None else t.cuda()
     for _ in range(3):
         x, dt = torch.randn(b, d, generator=g).to(io), torch.randn(b, d, generator=g).to(io)
@@ -200,8 +239,10 @@ def _decode_case(rng, seed):
         y = _ops().decode_step(cs, st, x.cuda(), dt.cuda(), A.cuda(), Bm.cuda(), Cm.cuda(), w.cuda(), conv_bias=dev(cb),
                                D=dev(D), z=dev(z), dt_bias=dev(bias), softplus=True, activation=act)
         assert torch.equal(cs.float().cpu(), cs_ref), desc
-        assert _rel(y, y_ref) < tol, desc
-        assert _rel(st, st_ref) < tol, desc          # half inputs: the convolution output is rounded to them first
+        # the convolution output is rounded to the element type before the update on both sides; float32: it is a
+        # float32 tap sum on the GPU against a float32 tap sum here, so the update's input agrees to a rounding
+        _close(y, y_ref, (desc, "y"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
+        _close(st, st_ref, (desc, "state"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
         st_ref = st_ref.float()
 
 
@@ -223,7 +264,7 @@ def _mamba2_decode_case(rng, seed):
     st_ref = torch.randn(b, H, P, N, generator=g)
     cs, st = cs_ref.to(io).cuda(), st_ref.clone().cuda()
     desc = ("mamba2 decode", seed, (b, H, P, G, N, K), str(io), None if D is None else tuple(D.shape), bias is not None, gate, cb is not None)
-    tol = 2e-4 if io == torch.float32 else 2e-2
+    half = io != torch.float32
     dev = lambda t: None if t is None else t.cuda()
     Dflat = None if D is None else (D.repeat_interleave(P) if D.ndim == 1 else D.reshape(di))
     for _ in range(3):
@@ -241,8 +282,8 @@ def _mamba2_decode_case(rng, seed):
         y = _ops().mamba2_decode_step(row.cuda(), cs, st, w.cuda(), dev(cb), A.cuda(), D=dev(D), dt_bias=dev(bias), ngroups=G,
                                       softplus=True, gate=gate)
         assert torch.equal(cs.float().cpu(), cs_ref), desc
-        assert _rel(y, y_ref) < tol, desc
-        assert _rel(st, flat.reshape(b, H, P, N)) < 2e-4, desc
+        _close(y, y_ref, (desc, "y"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
+        _close(st, flat.reshape(b, H, P, N), (desc, "state"), rtol=1e-4, atol_rms=2e-5)
 
 
 def _dscan_case(rng, seed):
@@ -268,9 +309,9 @@ def _dscan_case(rng, seed):
     half = dtype in HALF
     _values_and_gradients(
         lambda X, dt, A, Bm, Cm, D, z, init: _ops().ssd_chunk_scan(X, dt, A, Bm, Cm, chunk, D=D, z=z, seq_meta=meta, initial_states=init),
-        lambda X, dt, A, Bm, Cm, D, z, init: O.ssd_chunk_scan(X, dt, A, Bm, Cm, chunk, D=D, z=z, seq_meta=meta, initial_states=init,
-                                                              acc=torch.float64),
-        [X, dt, A, Bm, Cm, D, z, init], desc, 2e-2 if half else 2e-4, 3e-2 if half else 5e-4)
+        lambda acc, X, dt, A, Bm, Cm, D, z, init: O.ssd_chunk_scan(X, dt, A, Bm, Cm, chunk, D=D, z=z, seq_meta=meta,
+                                                                   initial_states=init, acc=acc),
+        [X, dt, A, Bm, Cm, D, z, init], desc, half)
 
 
 @pytest.mark.parametrize("block", range(4))
@@ -325,9 +366,11 @@ def _ssd_case(rng, seed):
     d = {k: (None if v is None else v.cuda().clone().requires_grad_(True)) for k, v in vals.items()}
     y, fin = S.ssd_combined(d["x"], d["dt"], d["A"], d["B"], d["C"], Q, D=d["D"], z=d["z"], dt_bias=d["dt_bias"],
                             initial_states=d["init"], dt_softplus=softplus, return_final_states=True, seq_idx=seq_idx)
-    tol = 2e-4 if dtype == torch.float32 else 2.5e-2
-    assert _rel(y, y64) < tol, (desc, "y")
-    assert _rel(fin, fin64) < tol, (desc, "final state")
+    # float32 calls: the chunked form (differences of running sums under one exponential) against the step-by-step
+    # recurrence; the running sum's own float32 rounding, times its size, is the floor
+    half = dtype != torch.float32
+    _close(y, y64, (desc, "y"), half=half, rtol=None if half else 2e-4, atol_rms=None if half else 2e-4)
+    _close(fin, fin64, (desc, "final state"), half=half, rtol=None if half else 2e-4, atol_rms=None if half else 2e-4)
     ((y64 * dout.double()).sum() + (fin64 * dfin.double()).sum()).backward()
     ((y.float() * dout.cuda().float()).sum() + (fin.float() * dfin.cuda()).sum()).backward()
     mean_bar, max_bar = (2e-4, 2e-3) if dtype == torch.float32 else (2e-2, 0.3)
@@ -385,8 +428,8 @@ def _scan_wide_case(rng, seed):
         y64, last64 = O.selective_scan(u, delta, A, Bm, Cm, D, z, bias, softplus=True, return_last_state=True, acc=torch.float64)
         y, last = _ops().selective_scan(dev(u), dev(delta), dev(A), dev(Bm), dev(Cm), dev(D), dev(z), dev(bias), softplus=True,
                                         return_last_state=True)
-    assert _rel(y, y64) < (2e-2 if half else 2e-4), (desc, "y")
-    assert _rel(last, last64) < (5e-3 if half else 2e-4), (desc, "last state")      # returned in the type of u
+    _close(y, y64, (desc, "y"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
+    _close(last, last64, (desc, "last state"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
     go = torch.randn(b, d, l, generator=g).to(dtype).cuda()
     gl = torch.randn(b, d, n, generator=g).cuda() if with_last else None
     args = (go, gl, dev(u), dev(delta), dev(A), dev(Bm), dev(Cm), dev(D), dev(z), dev(bias), True)
@@ -397,8 +440,10 @@ def _scan_wide_case(rng, seed):
         if r is None:
             continue
         # per-token gradients come back in the element type: one last place of a 16-bit value apart at most
-        bar = 2e-2 if (half and name in ("u", "delta", "z")) else 3e-4
-        assert _rel(f.float(), r.float()) < bar, (desc, name)
+        if half and name in ("u", "delta", "z"):
+            _close(f.float(), r.float(), (desc, name), rtol=2.0 ** -7, atol_rms=1e-3)
+        else:
+            _close(f.float(), r.float(), (desc, name), rtol=3e-4, atol_rms=3e-4)
 
 
 @pytest.mark.parametrize("block", range(3))
@@ -497,36 +542,38 @@ def _ssd_stages_case(rng, seed):
             seq_idx[:, c:] += 1
     desc = ("ssd stages", seed, str(dtype), (b, l, h, p, g, n), Q, softplus, use_z, use_init, use_D, cuts)
     dev = lambda t: None if t is None else t.cuda()
-    tol = 2e-4 if dtype == torch.float32 else 2e-2
+    half = dtype != torch.float32
     sid = dev(seq_idx)
 
     cs64, dtc64 = SO.chunk_cumsum(dt, A, Q, dt_bias=bias, dt_softplus=softplus)
     cs, dtc = S.chunk_cumsum(dev(dt), dev(A), Q, dt_bias=dev(bias), dt_softplus=softplus)
-    assert _rel(cs, cs64) < 1e-5 and _rel(dtc, dtc64) < 1e-5, (desc, "chunk_cumsum")
+    _close(cs, cs64, (desc, "chunk_cumsum"), rtol=1e-5, atol_rms=1e-5)
+    _close(dtc, dtc64, (desc, "chunk_cumsum dt"), rtol=1e-5, atol_rms=1e-5)
     cs32, dtc32 = cs64.float().cuda(), dtc64.float().cuda()
 
     causal = rng.random() < 0.5
     cb64 = SO.bmm_chunk(Cm, Bm, Q, seq_idx=seq_idx, causal=causal)
     cb = S.bmm_chunk(dev(Cm), dev(Bm), Q, seq_idx=sid, causal=causal, output_dtype=torch.float32)
-    assert _rel(cb, cb64) < (1e-5 if dtype == torch.float32 else 1e-3), (desc, "bmm_chunk")
+    _close(cb, cb64, (desc, "bmm_chunk"), rtol=1e-5, atol_rms=1e-5)      # exact products of 16-bit values, float32 sums
 
     st64 = SO.chunk_state(Bm, x, dtc64, cs64, seq_idx=seq_idx)
     st = S.chunk_state(dev(Bm), dev(x), dtc32, cs32, seq_idx=sid)
-    assert _rel(st, st64) < tol, (desc, "chunk_state")
+    _close(st, st64, (desc, "chunk_state"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
 
     ent64, fin64 = SO.state_passing(st64, cs64[..., -1], initial_states=init, seq_idx=seq_idx, chunk_size=Q)
     ent, fin = S.state_passing(st64.float().cuda(), cs32[..., -1].contiguous(), initial_states=dev(init), seq_idx=sid, chunk_size=Q)
-    assert _rel(ent, ent64) < 2e-5 and _rel(fin, fin64) < 2e-5, (desc, "state_passing")
+    _close(ent, ent64, (desc, "state_passing"), rtol=2e-5, atol_rms=2e-5)
+    _close(fin, fin64, (desc, "state_passing final"), rtol=2e-5, atol_rms=2e-5)
 
     y64 = SO.chunk_scan(Bm, Cm, x, dtc64, cs64, ent64, D=D, z=z, seq_idx=seq_idx)
     y = S.chunk_scan(dev(Bm), dev(Cm), dev(x), dtc32, cs32, ent64.float().cuda(), D=dev(D), z=dev(z), seq_idx=sid)
-    assert _rel(y, y64) < (2e-4 if dtype == torch.float32 else 2.5e-2), (desc, "chunk_scan")
+    _close(y, y64, (desc, "chunk_scan"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 1e-4)
 
     if cuts and b == 1:
         cu = torch.tensor([0] + cuts + [l], dtype=torch.int32)
         ends64 = SO.chunk_state_varlen(Bm, x, dtc64, cs64, cu, ent64)
         ends = S.chunk_state_varlen(dev(Bm), dev(x), dtc32, cs32, cu.cuda(), ent64.float().cuda())
-        assert _rel(ends, ends64) < tol, (desc, "chunk_state_varlen")
+        _close(ends, ends64, (desc, "chunk_state_varlen"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
 
 
 @pytest.mark.parametrize("block", range(4))

@@ -171,8 +171,10 @@ def test_half_inputs(dtype):
         assert got[k].dtype == dtype
     for k in ("A", "D", "dt_bias"):
         assert got[k].dtype == torch.float32
-    # the oracle differentiates the same bf16-rounded inputs in fp32; outputs are rounded once
-    compare(got, want, rtol=3e-2, atol=3e-2)
+    # the oracle differentiates the same 16-bit inputs in fp32; outputs are rounded once
+    from tests.closeness import half_close
+    for k in NAMES:
+        half_close(got[k], want[k], what=f"grad {k}", atol_rms=4e-2, mean_rms=5e-3)
 
 
 def test_config1_shape_bf16_slice():
@@ -201,9 +203,10 @@ def test_config1_shape_bf16_slice():
 
     full = run(slice(0, 1536))
     lo, hi = run(slice(0, 768)), run(slice(768, 1536))
+    from tests.closeness import half_close
     for k in ("B", "C"):
-        s = lo[k].float() + hi[k].float()
-        torch.testing.assert_close(full[k].float(), s, rtol=2e-2, atol=2e-2 * float(s.abs().max()))
+        s = lo[k].float() + hi[k].float()          # three roundings to bf16 against one
+        half_close(full[k], s, what=f"grad {k}: whole call against the sum of two halves", atol_rms=4e-2, mean_rms=8e-3)
     # a row's sums over the states run in an order that depends on the wave that owns the row, and the block shape
     # follows the channel count: the same row in the two calls agrees to one rounding of the 16-bit result
     a, b = full["u"][:, :768].float(), lo["u"].float()
@@ -218,11 +221,9 @@ def test_config1_shape_bf16_slice():
                          dt_bias=lv["dt_bias"], softplus=True)
     y.backward(go[:, idx])
     for k in ("u", "delta", "z"):
-        w = lv[k].grad.float()
-        torch.testing.assert_close(full[k][:, idx.cuda()].float().cpu(), w, rtol=3e-2, atol=3e-2 * float(w.abs().max()))
+        half_close(full[k][:, idx.cuda()], lv[k].grad, what=f"grad {k}", atol_rms=4e-2, mean_rms=5e-3)
     for k in ("A", "D", "dt_bias"):
-        w = lv[k].grad.float()
-        torch.testing.assert_close(full[k][idx.cuda()].float().cpu(), w, rtol=3e-2, atol=3e-2 * float(w.abs().max()))
+        half_close(full[k][idx.cuda()], lv[k].grad, what=f"grad {k}", atol_rms=4e-2, mean_rms=5e-3)
 
 
 # ------------------------------------------------------------------ the specialised kernel (16-bit activations)
@@ -289,3 +290,26 @@ def test_specialised_backward_is_bit_reproducible():
         again = _bwd_direct(inp, go, None, 0)
         for a, b in zip(first, again):
             assert (a is None and b is None) or torch.equal(a, b)
+
+
+def test_a_wave_that_gives_up_its_wait_poisons_dB_and_dC():
+    """The wave-per-row kernel bounds its wait for the neighbouring wave's slot count; a wave that gives up
+    writes NaN into its sums so that the caller cannot take them for gradients.  The test-hooks build cuts the
+    bound to nothing (selector 2, include/ssm_amd_testing.h), so every wave gives up at once: the kernel still ends
+    normally, dB and dC come back NaN, and the gradients that do not pass through the shared tiles are those of
+    an ordinary call."""
+    inp = make_inputs(12, 2, 48, 1040, 16, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(5)
+    go = torch.randn(2, 48, 1040, generator=g).to(torch.bfloat16)
+    good = _bwd_direct(inp, go, None, 0)
+    bad = _bwd_direct(inp, go, None, 2)
+    torch.cuda.synchronize()
+    names = ("u", "delta", "A", "B", "C", "D", "z", "dt_bias")
+    for k, a, b in zip(names, good, bad):
+        if a is None:
+            continue
+        if k in ("B", "C"):
+            assert bool(torch.isnan(b).any()), f"grad {k} must be poisoned"
+            assert not bool(torch.isnan(a).any())
+        else:
+            assert torch.equal(a, b), k

@@ -39,6 +39,18 @@ def cu(t):
     return None if t is None else t.cuda()
 
 
+def kernels_taken(fn):
+    """Run ``fn()`` once more on the test-hooks build of the library (the same sources compiled with
+    ``-DSSM_TEST_HOOKS``, include/ssm_amd_testing.h) and return which matrix-core kernels its calls launched:
+    bit 0 bmm_chunk, bit 1 chunk_state, bit 2 chunk_scan, bit 3 the one-pass forward.  The shipped library
+    picks its kernels by the same code but keeps no record."""
+    from ssm_amd import _lib
+    with _lib.test_hooks_build() as lib:
+        lib.ssm_ssd_mfma_launches()
+        fn()
+        return lib.ssm_ssd_mfma_launches()
+
+
 def test_chunk_cumsum_vectors():
     rec = fx.upstream("ssd_components", "chunk_cumsum"); i = rec["inputs"]
     dA, dt_c = ssd().chunk_cumsum(cu(i["dt"]), cu(i["A"]), 3, dt_bias=cu(i["dt_bias"]), dt_softplus=True)
@@ -348,13 +360,12 @@ def test_packed_sequences_match_the_oracle_and_separate_runs(Q, lens, dtype, P):
     for n in lens:
         cu_l.append(cu_l[-1] + n)
     seq_idx = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])[None]
-    from ssm_amd import _lib
-    _lib.load().ssm_ssd_mfma_launches()
-    y, fin, vs = ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
-                                    return_final_states=True, seq_idx=cu(seq_idx),
-                                    cu_seqlens=torch.tensor(cu_l, dtype=torch.int32).cuda(),
-                                    return_varlen_states=True, states_dtype=torch.float32)
-    used = _lib.load().ssm_ssd_mfma_launches()
+    call = lambda: ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
+                                      return_final_states=True, seq_idx=cu(seq_idx),
+                                      cu_seqlens=torch.tensor(cu_l, dtype=torch.int32).cuda(),
+                                      return_varlen_states=True, states_dtype=torch.float32)
+    y, fin, vs = call()
+    used = kernels_taken(call)
     assert (used & 6) == (6 if (dtype == torch.bfloat16 and P in (32, 64)) else 0)
     wy, wf, wv = S.ssd_combined(x, dt, A, Bm, Cm, Q, D=D, z=z, initial_states=init, clamp_decay=False,
                                 seq_idx=seq_idx, cu_seqlens=cu_l)
@@ -399,11 +410,10 @@ def test_packed_sequences_on_the_one_pass_kernel(Q, lens, N):
     init = torch.randn(2, H, P, N, generator=g)
     row = torch.cat([torch.full((n,), k, dtype=torch.int32) for k, n in enumerate(lens)])
     seq_idx = torch.stack([row, torch.zeros_like(row)])          # second batch row: one sequence
-    from ssm_amd import _lib
-    _lib.load().ssm_ssd_mfma_launches()
-    y, fin = ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
-                                return_final_states=True, seq_idx=cu(seq_idx))
-    assert _lib.load().ssm_ssd_mfma_launches() & 8
+    call = lambda: ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
+                                      return_final_states=True, seq_idx=cu(seq_idx))
+    y, fin = call()
+    assert kernels_taken(call) & 8
     y5, fin5 = ssd().ssd_combined(cu(x), cu(dt), cu(A), cu(Bm), cu(Cm), Q, D=cu(D), z=cu(z), initial_states=cu(init),
                                   return_final_states=True, seq_idx=cu(seq_idx), fused=False, states_dtype=torch.float32)
     wy, wf = S.ssd_combined(x, dt, A, Bm, Cm, Q, D=D, z=z, initial_states=init, clamp_decay=False, seq_idx=seq_idx)[:2]
@@ -491,13 +501,12 @@ def test_bf16_mfma_matches_generic_and_oracle(shape, Q, dtype):
     inp = make(11, b, l, h, p, g, n, dtype=dtype)
     args = (cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
     kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
-    from ssm_amd import _lib
-    _lib.load().ssm_ssd_mfma_launches()
     y, fin = ssd().ssd_combined(*args, fused=False, **kw)
-    used = _lib.load().ssm_ssd_mfma_launches()
+    used = kernels_taken(lambda: ssd().ssd_combined(*args, fused=False, **kw))
     assert used == 7, f"MFMA kernels used: {used:03b}"      # a ragged end is filled up to whole chunks
-    yg, fing = ssd().ssd_combined(*args, force_generic=True, states_dtype=torch.float32, **kw)
-    assert _lib.load().ssm_ssd_mfma_launches() == 0
+    generic = lambda: ssd().ssd_combined(*args, force_generic=True, states_dtype=torch.float32, **kw)
+    yg, fing = generic()                                    # the selector routes this call to the test-hooks build
+    assert kernels_taken(generic) == 0
     y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
                                 initial_states=inp["init"])
     half_close(yg, y64, "y, plain kernels")
@@ -523,10 +532,8 @@ def test_bf16_one_pass_matches_oracle_and_five_kernel_path(shape, Q, d_mat, use_
     inp = make(17 + l + Q, b, l, h, p, g, n, dtype=torch.bfloat16, d_mat=d_mat, use_z=use_z, use_init=use_init)
     args = (cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
     kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
-    from ssm_amd import _lib
-    _lib.load().ssm_ssd_mfma_launches()
     y, fin = ssd().ssd_combined(*args, fused=True, **kw)
-    assert _lib.load().ssm_ssd_mfma_launches() == 8
+    assert kernels_taken(lambda: ssd().ssd_combined(*args, fused=True, **kw)) == 8
     y5, fin5 = ssd().ssd_combined(*args, fused=False, **kw)
     y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
                                 initial_states=inp["init"])
@@ -559,11 +566,11 @@ def test_wide_heads_run_as_heads_of_64_channels(shape, Q, d_mat):
     kernel (a head of 64k channels is k heads of 64); packed sequences through the five kernels."""
     b, l, h, p, g, n = shape
     inp = make(5 + p, b, l, h, p, g, n, dtype=torch.bfloat16, d_mat=d_mat, use_z=True, use_init=True)
-    from ssm_amd import _lib
-    _lib.load().ssm_ssd_mfma_launches()
-    y, fin = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]),
-                                z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
-    assert _lib.load().ssm_ssd_mfma_launches() == 8
+    call = lambda: ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q,
+                                      D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]),
+                                      return_final_states=True)
+    y, fin = call()
+    assert kernels_taken(call) == 8
     y64, f64 = S.ssd_sequential(inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
                                 initial_states=inp["init"])
     assert tuple(y.shape) == (b, l, h, p) and tuple(fin.shape) == (b, h, p, n)
@@ -589,13 +596,13 @@ def test_ragged_length_is_filled_up_with_steps_of_size_zero(shape, Q, softplus):
     gen = torch.Generator().manual_seed(l)
     dt = torch.randn(b, l, h, generator=gen) if softplus else inp["dt"]
     bias = torch.randn(h, generator=gen) * 0.3 if softplus else None
-    from ssm_amd import _lib
-    _lib.load().ssm_ssd_mfma_launches()
     xg = cu(inp["x"]).requires_grad_(True)
-    y, fin = ssd().ssd_combined(xg, cu(dt), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]), z=cu(inp["z"]),
-                                initial_states=cu(inp["init"]), dt_bias=None if bias is None else cu(bias),
-                                dt_softplus=softplus, return_final_states=True)
-    assert _lib.load().ssm_ssd_mfma_launches() != 0 and tuple(y.shape) == (b, l, h, p)
+    call = lambda: ssd().ssd_combined(xg, cu(dt), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]),
+                                      z=cu(inp["z"]), initial_states=cu(inp["init"]),
+                                      dt_bias=None if bias is None else cu(bias), dt_softplus=softplus,
+                                      return_final_states=True)
+    y, fin = call()
+    assert kernels_taken(call) != 0 and tuple(y.shape) == (b, l, h, p)
     x64 = inp["x"].double().requires_grad_(True)
     y64, f64 = S.ssd_sequential(x64, dt, inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
                                 initial_states=inp["init"], dt_bias=bias, dt_softplus=softplus)
@@ -617,11 +624,11 @@ def test_config3_shape_bf16():
     """BASELINE config 3: B=4, L=4096, H=80, P=64, N=128, G=1, Q=256, bf16.  Full size on the
     GPU; two heads of one batch row are replayed by the float64 sequential recurrence."""
     inp = make(3, 4, 4096, 80, 64, 1, 128, dtype=torch.bfloat16, use_init=False)
-    from ssm_amd import _lib
-    _lib.load().ssm_ssd_mfma_launches()
-    y, fin = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), 256,
-                                D=cu(inp["D"]), z=cu(inp["z"]), return_final_states=True)
-    assert _lib.load().ssm_ssd_mfma_launches() == 8
+    g3 = {k: cu(v) for k, v in inp.items()}
+    call = lambda: ssd().ssd_combined(g3["x"], g3["dt"], g3["A"], g3["B"], g3["C"], 256, D=g3["D"], z=g3["z"],
+                                      return_final_states=True)
+    y, fin = call()
+    assert kernels_taken(call) == 8
     assert y.dtype == torch.bfloat16 and fin.dtype == torch.float32 and tuple(fin.shape) == (4, 80, 64, 128)
     hs = [5, 71]
     y64, f64 = S.ssd_sequential(inp["x"][1:2, :, hs], inp["dt"][1:2, :, hs], inp["A"][hs], inp["B"][1:2],
@@ -658,32 +665,66 @@ def test_ragged_length_with_16_bit_steps_and_a_bias_keeps_the_final_state():
     half_close(fin, f64, "final states")
 
 
-def test_growing_states_are_kept_off_the_one_pass_kernel():
-    """Positive A: the one-pass kernel bounds every factor of a decay by 1 and would be wrong, so the default
-    path must not pick it; the five kernels follow the upstream kernels (decay inside a chunk clamped to 1),
-    packed or not."""
-    b, l, h, p, g, n, Q = 1, 512, 2, 64, 1, 64, 128
+def test_growing_states_on_the_one_pass_kernel():
+    """Positive A on some heads: the one-pass kernel looks at the sign of a head's A itself and follows the
+    upstream kernels there (decays inside a chunk clamped to 1, the carried state growing freely), packed or
+    not, so the default path picks it whatever the values of A are and agrees with the five kernels and with
+    the oracle's restatement of the clamps."""
+    b, l, h, p, g, n, Q = 2, 512, 4, 64, 1, 64, 128
     inp = make(31, b, l, h, p, g, n, dtype=torch.bfloat16, use_init=True)
-    A = torch.full((h,), 0.25)
-    dt = torch.full((b, l, h), 0.03)
+    A = torch.tensor([0.25, -0.5, 0.04, -3.0])
+    dt = torch.rand(b, l, h, generator=torch.Generator().manual_seed(4)) * 0.05 + 0.005
     seq_idx = torch.zeros(b, l, dtype=torch.int32)
     seq_idx[:, 200:] = 1
     seq_idx[:, 333:] = 2
-    from ssm_amd import _lib
     for sid in (None, seq_idx):
-        _lib.load().ssm_ssd_mfma_launches()
-        y, fin = ssd().ssd_combined(cu(inp["x"]), cu(dt), cu(A), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]), z=cu(inp["z"]),
-                                    initial_states=cu(inp["init"]), return_final_states=True, seq_idx=cu(sid),
-                                    states_dtype=torch.float32)
-        assert not (_lib.load().ssm_ssd_mfma_launches() & 8)
+        call = lambda **kw: ssd().ssd_combined(cu(inp["x"]), cu(dt), cu(A), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]),
+                                               z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True,
+                                               seq_idx=cu(sid), **kw)
+        y, fin = call()
+        assert kernels_taken(call) == 8
+        y5, fin5 = call(fused=False, states_dtype=torch.float32)
         wy, wf = S.ssd_combined(inp["x"], dt, A, inp["B"], inp["C"], Q, D=inp["D"], z=inp["z"], initial_states=inp["init"],
                                 clamp_decay=True, seq_idx=sid)[:2]
         half_close(y, wy, "y")
         half_close(fin, wf, "final states")
-    # the same call with a decaying A does take the one-pass kernel
-    _lib.load().ssm_ssd_mfma_launches()
-    ssd().ssd_combined(cu(inp["x"]), cu(dt), cu(-A), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]), z=cu(inp["z"]))
-    assert _lib.load().ssm_ssd_mfma_launches() & 8
+        half_close(y5, wy, "y, five kernels")
+        half_close(fin5, wf, "final states, five kernels")
+
+
+def test_one_pass_choice_never_reads_A_on_the_host():
+    """``ssd_combined`` under stream capture with ``A`` written anew before every replay, growing on one head:
+    the captured call is the eager call (no host read of ``A`` decides anything), and every replay agrees with
+    the oracle for the values of ``A`` it was replayed with."""
+    b, l, h, p, g, n, Q = 1, 256, 3, 64, 1, 128, 64
+    inp = make(77, b, l, h, p, g, n, dtype=torch.bfloat16, use_init=False)
+    dev = {k: cu(v) for k, v in inp.items()}
+    dt = (torch.rand(b, l, h, generator=torch.Generator().manual_seed(5)) * 0.05 + 0.005)
+    dt_g = cu(dt)
+    A_log = torch.zeros(h, device="cuda")
+    sign = torch.tensor([-1.0, 1.0, -1.0], device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run = lambda: ssd().ssd_combined(dev["x"], dt_g, sign * torch.exp(A_log), dev["B"], dev["C"], Q, D=dev["D"],
+                                         z=dev["z"], return_final_states=True)
+        run()                                              # warm-up outside the capture
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            y_g, fin_g = run()
+    torch.cuda.current_stream().wait_stream(side)
+    for k, values in enumerate(([0.0, -1.5, 1.0], [-2.0, -3.0, 0.5], [1.0, -0.7, -4.0])):
+        A_log.copy_(torch.tensor(values))
+        graph.replay()
+        torch.cuda.synchronize()
+        A = (sign * torch.exp(A_log)).cpu()
+        y_e, fin_e = ssd().ssd_combined(dev["x"], dt_g, cu(A), dev["B"], dev["C"], Q, D=dev["D"], z=dev["z"],
+                                        return_final_states=True)
+        assert torch.equal(y_g, y_e) and torch.equal(fin_g, fin_e), f"replay {k} differs from the eager call"
+        wy, wf = S.ssd_combined(inp["x"], dt, A, inp["B"], inp["C"], Q, D=inp["D"], z=inp["z"], clamp_decay=True)[:2]
+        half_close(y_g, wy, f"y, replay {k}")
+        half_close(fin_g, wf, f"final states, replay {k}")
 
 
 # ------------------------------------------------------------------ backward: the head-summed matrix of a chunk
@@ -768,6 +809,71 @@ def test_bwd_prep_kernel_matches_the_steps_taken_one_by_one(Q, L, softplus, limi
     by_rows = lambda t: t.permute(0, 2, 3, 1).reshape(b, L, h)
     torch.testing.assert_close(w_dy.double(), torch.exp(by_rows(want_cs).double()), rtol=2e-6, atol=1e-30)
     torch.testing.assert_close(w_x.double(), rows.double() * torch.exp(by_rows(want_r).double()).flip(1), rtol=2e-6, atol=1e-30)
+
+
+@pytest.mark.parametrize("shape,Q", [((2, 256, 3, 64, 1, 32), 64), ((1, 512, 4, 32, 2, 16), 256), ((2, 192, 2, 128, 1, 64), 96)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_operand_scaled_while_staged_equals_the_scaled_tensor(shape, Q, dtype=torch.bfloat16):
+    """``x_scale``: the matrix-core ``chunk_state`` and ``chunk_scan`` round ``x * scale`` as they stage ``x`` -- the
+    bits of a pass over the tensor ``round(x * scale)`` written beforehand, entering states included."""
+    from ssm_amd.ops import ssd as ops_ssd
+    b, l, h, p, g, n = shape
+    gen = torch.Generator().manual_seed(l + h)
+    x = torch.randn(b, l, h, p, generator=gen).to(dtype).cuda()
+    Bm = torch.randn(b, l, g, n, generator=gen).to(dtype).cuda()
+    Cm = torch.randn(b, l, g, n, generator=gen).to(dtype).cuda()
+    dt = (torch.rand(b, l, h, generator=gen) * 0.2).cuda()
+    A = -(torch.rand(h, generator=gen) * 4 + 0.1).cuda()
+    init = torch.randn(b, h, p, n, generator=gen).cuda()
+    dA_cs, dt_c = ops_ssd.chunk_cumsum(dt, A, Q)
+    ones = torch.ones_like(dt_c)
+    assert ops_ssd._row_scale_ok(x, Bm, Cm, Q)
+    scaled = (dt[..., None] * x.float()).to(dtype)
+    want = ops_ssd._lin_pass(scaled, ones, dA_cs, Bm, Cm, init, want_entering=True)
+    got = ops_ssd._lin_pass(x, ones, dA_cs, Bm, Cm, init, want_entering=True, x_scale=dt_c)
+    for a, w, name in zip(got, want, ("y", "final state", "entering states")):
+        assert torch.equal(a, w), name
+    # a call the matrix-core kernels do not take refuses the scale instead of dropping it
+    for other in (torch.float32, torch.float16):
+        with pytest.raises(Exception, match="x_row_scale"):
+            ops_ssd.chunk_state(Bm.to(other), x.to(other), ones, dA_cs, x_scale=dt_c)
+        assert not ops_ssd._row_scale_ok(x.to(other), Bm.to(other), Cm.to(other), Q)
+
+
+@pytest.mark.parametrize("shape,Q,d_mode,out", [((2, 256, 3, 64, 1, 32), 64, "vec", torch.float32),
+                                                 ((1, 512, 4, 32, 2, 16), 256, "mat", torch.bfloat16),
+                                                 ((2, 192, 2, 64, 1, 64), 96, "none", torch.bfloat16)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v).replace("torch.", ""))
+def test_reversed_pass_finishes_dx_in_its_own_kernel(shape, Q, d_mode, out):
+    """``dx_epilogue``: the matrix-core ``chunk_scan`` of the gradient's time-reversed pass writes ``dx`` and the row
+    sums ``xu``, ``s1`` instead of its result ``u``; against ``ssm_ssd_bwd_dx`` fed with ``u`` from the same pass
+    (equal up to the float32 order of the row sums; the skip term sees ``dy`` after its rounding to bfloat16)."""
+    from ssm_amd.ops import ssd as ops_ssd
+    b, l, h, p, g, n = shape
+    gen = torch.Generator().manual_seed(l + h + p)
+    bf = torch.bfloat16
+    x = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
+    dy = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
+    Bm = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
+    Cm = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
+    dt = (torch.rand(b, l, h, generator=gen) * 0.2).cuda()
+    A = -(torch.rand(h, generator=gen) * 4 + 0.1).cuda()
+    D = {"none": None, "vec": torch.randn(h, generator=gen).cuda(), "mat": torch.randn(h, p, generator=gen).cuda()}[d_mode]
+    dfin = torch.randn(b, h, p, n, generator=gen).cuda()
+    dA_cs, dt_c = ops_ssd.chunk_cumsum(dt, A, Q)
+    ones = torch.ones_like(dt_c)
+    dyr = dy.flip(1).contiguous()
+    Cr, Br = Cm.flip(1).contiguous(), Bm.flip(1).contiguous()
+    u_r, fin, ent = ops_ssd._lin_pass(dyr, ones, dA_cs, Cr, Br, dfin, want_entering=True)
+    want = ops_ssd._bwd_dx(dy, None, x, u_r.contiguous(), dt, D, True, grads_io=(out == bf))
+    (dx, xu, s1), fin2, ent2 = ops_ssd._lin_pass(dyr, ones, dA_cs, Cr, Br, dfin, want_entering=True,
+                                                  dx_epilogue=(x, dt, D, out, True))
+    assert torch.equal(fin, fin2) and torch.equal(ent, ent2)
+    assert dx.dtype == out and want[0].dtype == out
+    scale = float(want[0].float().abs().max())
+    torch.testing.assert_close(dx.float(), want[0].float(), rtol=2.0 ** -7 if out == bf else 1e-6, atol=1e-6 * scale)
+    for got, w, name in ((xu, want[1], "xu"), (s1, want[2], "s1")):
+        torch.testing.assert_close(got, w, rtol=1e-5, atol=1e-5 * float(w.abs().max()), msg=lambda m_, n_=name: f"{n_}: {m_}")
 
 
 @pytest.mark.parametrize("shape,Q", [((2, 256, 3, 64, 1, 32), 64), ((1, 512, 4, 32, 2, 16), 256), ((2, 192, 2, 128, 1, 64), 96)],

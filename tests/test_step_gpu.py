@@ -199,6 +199,54 @@ def test_config2_shape_512_steps():
     torch.testing.assert_close(st_gpu[:, idx.cuda()].cpu(), st_ref, rtol=1e-4, atol=1e-4)
 
 
+def test_config2_fused_decode_step_512_steps():
+    """BASELINE config 2 with both of its states: B=64, D=5120, N=16, conv width 4, bf16 activations and
+    window, fp32 SSM state, grouped B/C (64,1,16), 512 in-place fused decode steps (the call ``bench.py``
+    times).  A channel slice is replayed on the CPU the way the reference's ``Mamba1.step`` does
+    (``/root/reference/src/ssm/modules/mamba1.py:345-381``): roll the window, tap sum + bias, SiLU, then the
+    oracle's state step.  The window holds copies of the inputs, so it is compared bit for bit."""
+    ops = _ops()
+    from ssm_amd.configs import inverse_softplus_dt
+    g = torch.Generator().manual_seed(22)
+    Bsz, D, N, K, steps = 64, 5120, 16, 4, 512
+    state = torch.randn(Bsz, D, N, generator=g)
+    window = torch.randn(Bsz, D, K, generator=g).to(torch.bfloat16)
+    A = -torch.arange(1, N + 1, dtype=torch.float32).repeat(D, 1)
+    Dk = torch.ones(D)
+    bias = inverse_softplus_dt(D, g)
+    w = torch.rand(D, K, generator=g) - 0.5
+    cb = torch.randn(D, generator=g) * 0.02
+    idx = torch.cat([torch.arange(0, D, 320), torch.tensor([1, 2, 3, D - 1])])
+    idx_g = idx.cuda()
+    st_gpu, win_gpu = state.cuda(), window.cuda()
+    st_ref, win_ref = state[:, idx].clone(), window[:, idx].float()
+    A_g, D_g, b_g, w_g, cb_g = A.cuda(), Dk.cuda(), bias.cuda(), w.cuda(), cb.cuda()
+    check_at = {0, 1, 2, 3, 4, 17, 255, 511}
+    for s in range(steps):
+        x = torch.randn(Bsz, D, generator=g).to(torch.bfloat16)
+        z = torch.randn(Bsz, D, generator=g).to(torch.bfloat16)
+        dt = torch.randn(Bsz, D, generator=g).to(torch.bfloat16)
+        Bm = torch.randn(Bsz, 1, N, generator=g).to(torch.bfloat16)
+        Cm = torch.randn(Bsz, 1, N, generator=g).to(torch.bfloat16)
+        y, xc = ops.decode_step(win_gpu, st_gpu, x.cuda(), dt.cuda(), A_g, Bm.cuda(), Cm.cuda(), w_g, conv_bias=cb_g,
+                                D=D_g, z=z.cuda(), dt_bias=b_g, softplus=True, return_conv_out=True)
+        win_ref = torch.roll(win_ref, -1, dims=-1)
+        win_ref[..., -1] = x[:, idx].float()
+        xc_ref = torch.nn.functional.silu((win_ref * w[idx]).sum(-1) + cb[idx]).to(torch.bfloat16)
+        yr = O.selective_state_step(st_ref, xc_ref, dt[:, idx], A[idx], Bm, Cm, D=Dk[idx], z=z[:, idx],
+                                    dt_bias=bias[idx], softplus=True)
+        if s in check_at:
+            torch.testing.assert_close(win_gpu[:, idx_g].float().cpu(), win_ref, rtol=0, atol=0)
+            torch.testing.assert_close(xc[:, idx_g].float().cpu(), xc_ref.float(), **HALF_TOL)
+            torch.testing.assert_close(y[:, idx_g].float().cpu(), yr.float(), **HALF_TOL)
+    torch.testing.assert_close(win_gpu[:, idx_g].float().cpu(), win_ref, rtol=0, atol=0)
+    # the convolution output is rounded to bf16 on both sides; where the two roundings fall on different
+    # sides the state sees one bf16 ulp of xc times dt.B, which decays like the state itself
+    torch.testing.assert_close(st_gpu[:, idx_g].cpu(), st_ref, rtol=2e-2, atol=2e-2)
+    err = (st_gpu[:, idx_g].cpu() - st_ref).abs().mean() / st_ref.abs().mean()
+    assert float(err) < 2e-3, float(err)
+
+
 @pytest.mark.parametrize("io", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("K", [2, 4, 7])
 def test_fused_decode_step_equals_conv_window_then_state_step(io, K):
