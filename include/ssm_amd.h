@@ -462,9 +462,10 @@ int ssm_ssd_chunk_state_varlen(const ssm_ssd_chunk_state_varlen_args *args, void
  * chunk_scan; combined call recorded at scripts/refresh_mamba_goldens.py:591-604)
  * as one pass over the sequence that keeps the running state on chip: the
  * per-chunk states never reach device memory.  Covers bf16 tensors with
- * headdim 64, chunk in {64, 128, 256}, nstate in {64, 128},
- * seqlen % chunk == 0 and A <= 0; ssm_ssd_combined_supported() tells, other
- * shapes go through the five calls above. */
+ * headdim 64, chunk in {64, 128, 256}, nstate in {64, 128} and
+ * seqlen % chunk == 0; ssm_ssd_combined_supported() tells, other shapes go
+ * through the five calls above.  A head with A > 0 is treated as those calls
+ * treat it (decays inside a chunk bounded by 1, the carried state growing). */
 typedef struct ssm_ssd_combined_args {
   const void *x;              /* (B,L,H,P) io dtype */
   const void *dt;             /* (B,L,H) dt dtype, before bias / softplus / clamp */

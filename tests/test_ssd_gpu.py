@@ -686,10 +686,11 @@ def test_growing_states_on_the_one_pass_kernel():
         y5, fin5 = call(fused=False, states_dtype=torch.float32)
         wy, wf = S.ssd_combined(inp["x"], dt, A, inp["B"], inp["C"], Q, D=inp["D"], z=inp["z"], initial_states=inp["init"],
                                 clamp_decay=True, seq_idx=sid)[:2]
-        half_close(y, wy, "y")
-        half_close(fin, wf, "final states")
-        half_close(y5, wy, "y, five kernels")
-        half_close(fin5, wf, "final states, five kernels")
+        for hh in range(h):                # head by head: a growing head is orders of magnitude larger than a decaying one
+            half_close(y[:, :, hh], wy[:, :, hh], f"y, head {hh}")
+            half_close(fin[:, hh], wf[:, hh], f"final states, head {hh}")
+            half_close(y5[:, :, hh], wy[:, :, hh], f"y, five kernels, head {hh}")
+            half_close(fin5[:, hh], wf[:, hh], f"final states, five kernels, head {hh}")
 
 
 def test_one_pass_choice_never_reads_A_on_the_host():
@@ -723,8 +724,9 @@ def test_one_pass_choice_never_reads_A_on_the_host():
                                         return_final_states=True)
         assert torch.equal(y_g, y_e) and torch.equal(fin_g, fin_e), f"replay {k} differs from the eager call"
         wy, wf = S.ssd_combined(inp["x"], dt, A, inp["B"], inp["C"], Q, D=inp["D"], z=inp["z"], clamp_decay=True)[:2]
-        half_close(y_g, wy, f"y, replay {k}")
-        half_close(fin_g, wf, f"final states, replay {k}")
+        for hh in range(h):
+            half_close(y_g[:, :, hh], wy[:, :, hh], f"y, replay {k}, head {hh}")
+            half_close(fin_g[:, hh], wf[:, hh], f"final states, replay {k}, head {hh}")
 
 
 # ------------------------------------------------------------------ backward: the head-summed matrix of a chunk
@@ -874,88 +876,6 @@ def test_reversed_pass_finishes_dx_in_its_own_kernel(shape, Q, d_mode, out):
     torch.testing.assert_close(dx.float(), want[0].float(), rtol=2.0 ** -7 if out == bf else 1e-6, atol=1e-6 * scale)
     for got, w, name in ((xu, want[1], "xu"), (s1, want[2], "s1")):
         torch.testing.assert_close(got, w, rtol=1e-5, atol=1e-5 * float(w.abs().max()), msg=lambda m_, n_=name: f"{n_}: {m_}")
-
-
-@pytest.mark.parametrize("shape,Q", [((2, 256, 3, 64, 1, 32), 64), ((1, 512, 4, 32, 2, 16), 256), ((2, 192, 2, 128, 1, 64), 96)],
-                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
-def test_operand_scaled_while_staged_equals_the_scaled_tensor(shape, Q, dtype=torch.bfloat16):
-    """``x_scale``: the matrix-core ``chunk_state`` and ``chunk_scan`` round ``x * scale`` as they stage ``x`` -- the
-    bits of a pass over the tensor ``round(x * scale)`` written beforehand, entering states included."""
-    from ssm_amd.ops import ssd as ops_ssd
-    b, l, h, p, g, n = shape
-    gen = torch.Generator().manual_seed(l + h)
-    x = torch.randn(b, l, h, p, generator=gen).to(dtype).cuda()
-    Bm = torch.randn(b, l, g, n, generator=gen).to(dtype).cuda()
-    Cm = torch.randn(b, l, g, n, generator=gen).to(dtype).cuda()
-    dt = (torch.rand(b, l, h, generator=gen) * 0.2).cuda()
-    A = -(torch.rand(h, generator=gen) * 4 + 0.1).cuda()
-    init = torch.randn(b, h, p, n, generator=gen).cuda()
-    dA_cs, dt_c = ops_ssd.chunk_cumsum(dt, A, Q)
-    ones = torch.ones_like(dt_c)
-    assert ops_ssd._row_scale_ok(x, Bm, Cm, Q)
-    scaled = (dt[..., None] * x.float()).to(dtype)
-    want = ops_ssd._lin_pass(scaled, ones, dA_cs, Bm, Cm, init, want_entering=True)
-    got = ops_ssd._lin_pass(x, ones, dA_cs, Bm, Cm, init, want_entering=True, x_scale=dt_c)
-    for a, w, name in zip(got, want, ("y", "final state", "entering states")):
-        assert torch.equal(a, w), name
-    # a call the matrix-core kernels do not take refuses the scale instead of dropping it
-    for other in (torch.float32, torch.float16):
-        with pytest.raises(Exception, match="x_row_scale"):
-            ops_ssd.chunk_state(Bm.to(other), x.to(other), ones, dA_cs, x_scale=dt_c)
-        assert not ops_ssd._row_scale_ok(x.to(other), Bm.to(other), Cm.to(other), Q)
-
-
-@pytest.mark.parametrize("shape,Q,d_mode,out", [((2, 256, 3, 64, 1, 32), 64, "vec", torch.float32),
-                                                 ((1, 512, 4, 32, 2, 16), 256, "mat", torch.bfloat16),
-                                                 ((2, 192, 2, 64, 1, 64), 96, "none", torch.bfloat16)],
-                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v).replace("torch.", ""))
-def test_reversed_pass_finishes_dx_in_its_own_kernel(shape, Q, d_mode, out):
-    """``dx_epilogue``: the matrix-core ``chunk_scan`` of the gradient's time-reversed pass writes ``dx`` and the row
-    sums ``xu``, ``s1`` instead of its result ``u``; against ``ssm_ssd_bwd_dx`` fed with ``u`` from the same pass
-    (equal up to the float32 order of the row sums; the skip term sees ``dy`` after its rounding to bfloat16)."""
-    from ssm_amd.ops import ssd as ops_ssd
-    b, l, h, p, g, n = shape
-    gen = torch.Generator().manual_seed(l + h + p)
-    bf = torch.bfloat16
-    x = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
-    dy = torch.randn(b, l, h, p, generator=gen).to(bf).cuda()
-    Bm = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
-    Cm = torch.randn(b, l, g, n, generator=gen).to(bf).cuda()
-    dt = (torch.rand(b, l, h, generator=gen) * 0.2).cuda()
-    A = -(torch.rand(h, generator=gen) * 4 + 0.1).cuda()
-    D = {"none": None, "vec": torch.randn(h, generator=gen).cuda(), "mat": torch.randn(h, p, generator=gen).cuda()}[d_mode]
-    dfin = torch.randn(b, h, p, n, generator=gen).cuda()
-    dA_cs, dt_c = ops_ssd.chunk_cumsum(dt, A, Q)
-    ones = torch.ones_like(dt_c)
-    dyr = dy.flip(1).contiguous()
-    Cr, Br = Cm.flip(1).contiguous(), Bm.flip(1).contiguous()
-    u_r, fin, ent = ops_ssd._lin_pass(dyr, ones, dA_cs, Cr, Br, dfin, want_entering=True)
-    want = ops_ssd._bwd_dx(dy, None, x, u_r.contiguous(), dt, D, True, grads_io=(out == bf))
-    (dx, xu, s1), fin2, ent2 = ops_ssd._lin_pass(dyr, ones, dA_cs, Cr, Br, dfin, want_entering=True,
-                                                  dx_epilogue=(x, dt, D, out, True))
-    assert torch.equal(fin, fin2) and torch.equal(ent, ent2)
-    assert dx.dtype == out and want[0].dtype == out
-    scale = float(want[0].float().abs().max())
-    torch.testing.assert_close(dx.float(), want[0].float(), rtol=2.0 ** -7 if out == bf else 1e-6, atol=1e-6 * scale)
-    for got, w, name in ((xu, want[1], "xu"), (s1, want[2], "s1")):
-        torch.testing.assert_close(got, w, rtol=1e-5, atol=1e-5 * float(w.abs().max()), msg=lambda m_, n_=name: f"{n_}: {m_}")
-
-
-def test_sign_of_A_is_remembered_per_tensor_not_per_address():
-    """The check of ``all(A <= 0)`` is cached; a new tensor that the allocator places at a freed tensor's address
-    must be looked at again."""
-    from ssm_amd.ops import ssd as ops_ssd
-    grow = torch.full((8,), 0.25).cuda()
-    addr = grow.data_ptr()
-    assert not ops_ssd._is_decaying(grow)
-    del grow
-    decay = torch.full((8,), -0.25).cuda()
-    if decay.data_ptr() != addr:
-        pytest.skip("the allocator did not hand the address out again")
-    assert ops_ssd._is_decaying(decay)
-    assert ops_ssd._is_decaying(decay)            # from the cache
-    decay.neg_()                                  # the same object, changed in place
-    assert not ops_ssd._is_decaying(decay)
 
 
 @pytest.mark.parametrize("shape,Q", [((2, 256, 3, 64, 1, 32), 64), ((1, 512, 4, 32, 2, 16), 256), ((2, 192, 2, 128, 1, 64), 96)],
