@@ -437,7 +437,9 @@ def bench_scan_facade(dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nsta
         g = sets[i % 4]
         return ops.selective_scan(g["u"], g["delta"], g["A"], g["B"], g["C"], D=g["D"], z=g["z"],
                                   dt_bias=g["dt_bias"], softplus=True, return_last_state=True)
-    for i in range(5):
+    # the input sets above were made on the host while the device idled: bring it back to its clocks first, as
+    # the headline does (the first hundred launches after idling run up to 15 % slower)
+    for i in range(SPIN_UP_LAUNCHES):
         call(i)
     torch.cuda.synchronize()
     n = 50
@@ -521,11 +523,64 @@ def cpu_baseline_scan(dtype=torch.bfloat16, dim=1536, length=2048, nstate=16, bu
         t0s.append(time.perf_counter() - t0)
     return dict(value=nbytes / best / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
                 config0_ms=round(sorted(t0s)[1] * 1e3, 1), config0_reference_published_ms=1012.9,
+                config2_decode=cpu_baseline_decode(), config3_ssd=cpu_baseline_ssd(),
                 sample=f"selective_scan fwd, batch slice B={batch} of the headline workload "
                        f"(D={dim}, L={length}, N={nstate}, {str(dtype).split('.')[-1]}), "
                        f"median of {len(times)} runs, {best * 1e3:.0f} ms each; "
                        f"host has {os.cpu_count()} logical cpus",
                 seconds_per_call=best)
+
+
+def cpu_baseline_decode(batch=64, dim=5120, nstate=16, width=4, steps=32):
+    """Config 2 on the host: the tensor operations of the reference's ``Mamba1.step`` (window roll, tap sum,
+    SiLU: src/ssm/modules/mamba1.py:345-381) followed by the oracle's state step, at full width, for a bounded
+    number of the 512 steps (every step costs the same)."""
+    from oracle import ops_oracle
+    from ssm_amd import configs
+
+    g = torch.Generator().manual_seed(2)
+    state = torch.randn(batch, dim, nstate, generator=g)
+    window = torch.randn(batch, dim, width, generator=g).to(torch.bfloat16)
+    A = -torch.arange(1, nstate + 1, dtype=torch.float32).repeat(dim, 1)
+    D, bias = torch.ones(dim), configs.inverse_softplus_dt(dim, g)
+    w, cb = torch.rand(dim, width, generator=g) - 0.5, torch.randn(dim, generator=g) * 0.02
+    x, z, dt = (torch.randn(batch, dim, generator=g).to(torch.bfloat16) for _ in range(3))
+    Bm, Cm = (torch.randn(batch, 1, nstate, generator=g).to(torch.bfloat16) for _ in range(2))
+
+    def step():
+        nonlocal window
+        window = torch.roll(window, -1, dims=-1)
+        window[..., -1] = x
+        xc = torch.nn.functional.silu((window.float() * w).sum(-1) + cb).to(torch.bfloat16)
+        ops_oracle.selective_state_step(state, xc, dt, A, Bm, Cm, D=D, z=z, dt_bias=bias, softplus=True)
+
+    step()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    per = (time.perf_counter() - t0) / steps
+    return {"us_per_step": round(per * 1e6, 1), "steps_timed": steps, "of_steps": 512,
+            "shape": f"B={batch}, D={dim}, N={nstate}, K={width}, bf16 activations, fp32 state"}
+
+
+def cpu_baseline_ssd(length=4096, heads=2, hdim=64, nstate=128):
+    """Config 3 on the host: the token-by-token recurrence that fixes the SSD's semantics (float32, two of the
+    320 (batch, head) pairs over the whole sequence; pairs are independent, so the whole call costs 160 times
+    this with the same threads)."""
+    from oracle import ssd_oracle
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, length, heads, hdim, generator=g)
+    dt = torch.rand(1, length, heads, generator=g) * 0.1
+    A = -(torch.rand(heads, generator=g) * 15 + 1)
+    Bm, Cm = torch.randn(1, length, 1, nstate, generator=g), torch.randn(1, length, 1, nstate, generator=g)
+    z = torch.randn(1, length, heads, hdim, generator=g)
+    t0 = time.perf_counter()
+    ssd_oracle.ssd_sequential(x, dt, A, Bm, Cm, D=torch.ones(heads), z=z, acc=torch.float32)
+    sec = time.perf_counter() - t0
+    pairs = 4 * 80
+    return {"ms_for_sample": round(sec * 1e3, 1), "sample": f"{heads} of {pairs} (batch, head) pairs, L={length}, P={hdim}, N={nstate}",
+            "ms_whole_call_extrapolated": round(sec * 1e3 * pairs / heads, 1)}
 
 
 def main():

@@ -417,7 +417,11 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def stream_handle(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """The raw HIP stream that torch currently launches on for ``device``."""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(index)
 
 
 def call(name: str, args: C.Structure, device: torch.device) -> None:
@@ -426,8 +430,13 @@ def call(name: str, args: C.Structure, device: torch.device) -> None:
     reference's compiled backends do, src/ssm/ops/__init__.py:1244-1252)."""
     # a kernel selector in the struct only means something to the test-hooks build
     lib = load_test_hooks() if getattr(args, "reserved", 0) else load()
-    with torch.cuda.device(device):
-        status = getattr(lib, name)(C.byref(args), stream_handle(device))
+    fn = getattr(lib, name)
+    index = device.index
+    if index is None or index == torch.cuda.current_device():
+        status = fn(C.byref(args), stream_handle(device))        # the usual case: no device switch to pay for
+    else:
+        with torch.cuda.device(device):
+            status = fn(C.byref(args), stream_handle(device))
     if status != 0:
         detail = lib.ssm_amd_last_error().decode() or lib.ssm_amd_status_string(status).decode()
         if status == -7:

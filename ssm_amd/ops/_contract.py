@@ -19,6 +19,10 @@ class DeviceError(RuntimeError):
     """Inputs are not all on one ROCm device (this backend has no CPU path)."""
 
 
+def on_gpu(t) -> bool:
+    return t.is_cuda
+
+
 def require_gpu(*tensors: Optional[torch.Tensor]) -> torch.device:
     """All tensor arguments must live on the same ``cuda`` (ROCm) device.
 

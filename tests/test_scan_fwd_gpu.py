@@ -320,3 +320,34 @@ def test_config1_shape_bf16_properties():
                             gpu["B"][..., :half], gpu["C"][..., :half], D=gpu["D"],
                             z=gpu["z"][:, :, :half], dt_bias=gpu["dt_bias"], softplus=True)
     assert torch.equal(y2, y[:, :, :half])
+
+
+def test_repeated_call_of_one_form_goes_through_the_remembered_struct():
+    """The second call of a form (same shapes, element types, optional arguments) skips the validation and fills
+    a remembered argument struct: same bits as the first call and as a prepared plan; a call of the same form
+    whose tensors need a copy first (non-contiguous) still goes the long way and agrees."""
+    from ssm_amd import ops
+    inp = make_inputs(5, 2, 48, 1040, 16, dtype=torch.bfloat16)
+    g = {k: dev(v) for k, v in inp.items()}
+    call = lambda t: ops.selective_scan(t["u"], t["delta"], t["A"], t["B"], t["C"], D=t["D"], z=t["z"],
+                                        dt_bias=t["dt_bias"], softplus=True, return_last_state=True)
+    ops._SCAN_FORMS.clear()
+    y1, h1 = call(g)
+    assert len(ops._SCAN_FORMS) == 1
+    y2, h2 = call(g)
+    assert torch.equal(y1, y2) and torch.equal(h1, h2)
+    other = {k: (v.clone() if v is not None else None) for k, v in g.items()}
+    other["u"] = torch.randn_like(other["u"].float()).to(torch.bfloat16)
+    y3, h3 = call(other)                               # same form, other tensors: other pointers, own result
+    plan = ops.ScanPlan(other["u"], other["delta"], other["A"], other["B"], other["C"], other["D"], other["z"],
+                        other["dt_bias"], True, True)
+    y4, h4 = plan.run()
+    assert torch.equal(y3, y4) and torch.equal(h3, h4) and not torch.equal(y3, y1)
+    strided = dict(other)
+    strided["u"] = other["u"].transpose(0, 1).contiguous().transpose(0, 1)       # same values, not contiguous
+    y5, h5 = call(strided)
+    assert torch.equal(y5, y3) and torch.equal(h5, h3)
+    with pytest.raises(ValueError):
+        bad = dict(other)
+        bad["A"] = other["A"][:, :8].contiguous()      # a form never seen, and inconsistent: the long way refuses it
+        call(bad)
