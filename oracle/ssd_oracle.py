@@ -61,7 +61,10 @@ def ssd_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=Fal
     """Token-by-token recurrence; returns ``(y (B,L,H,P), final_states (B,H,P,N))``.
 
     Shapes: x (B,L,H,P); dt (B,L,H); A (H,); B,C (B,L,G,N); D (H,)|(H,P);
-    z (B,L,H,P); initial_states (B,H,P,N)."""
+    z (B,L,H,P); initial_states (B,H,P,N).  ``A`` may also be given per step,
+    ``(B,L,H)`` (the same value repeated): autograd then returns the terms
+    ``dt_t q_t`` whose sum over batch and time is the gradient of ``A``, which
+    lets a test measure an error in that sum against the size of its terms."""
     batch, seqlen, heads, hdim = x.shape
     groups, nstate = B.shape[2], B.shape[3]
     per = heads // groups
@@ -75,7 +78,7 @@ def ssd_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=Fal
     ys = []
     for t in range(seqlen):
         step = dtv[:, t]                                           # (B,H)
-        decay = torch.exp(step * AA[None])                         # (B,H)
+        decay = torch.exp(step * (AA[None] if AA.ndim == 1 else AA[:, t]))   # (B,H)
         h = decay[:, :, None, None] * h \
             + (step[:, :, None] * xx[:, t])[:, :, :, None] * Bh[:, t][:, :, None, :]
         y = (h * Ch[:, t][:, :, None, :]).sum(-1)                  # (B,H,P)

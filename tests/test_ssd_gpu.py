@@ -20,6 +20,9 @@ def ssd():
 
 # gradients of 16-bit calls: sums of many rounded products
 GRAD_ATOL_RMS, GRAD_MEAN_RMS = 6e-2, 2e-2
+# dA, per head, against the sum over batch and time of the magnitudes of its terms dt_t q_t (seen over some two hundred
+# random cases: 1.4e-2 at worst with 16-bit operands, median 5e-4; 1.1e-4 and 3e-6 in float32)
+DA_TERM_BAR_HALF, DA_TERM_BAR_F32 = 2e-2, 2e-4
 
 
 def half_close(got, want, what="", atol_rms=4e-2, mean_rms=3e-3, rtol=2e-2):
@@ -153,9 +156,13 @@ def test_combined_gradients_match_float64_autograd(shape, Q, dtype, d_mat, use_z
     vals = dict(x=x, dt=dt, A=A, B=Bm, C=Cm, D=D, z=z, dt_bias=bias, init=init)
     # float64 reference
     w = {k: (None if v is None else v.double().clone().requires_grad_(True)) for k, v in vals.items()}
-    y64, f64 = S.ssd_sequential(w["x"], w["dt"], w["A"], w["B"], w["C"], D=w["D"], z=w["z"], dt_bias=w["dt_bias"],
+    # A given per step (the same value at every step): its gradient holds the terms dt_t q_t whose sum is dA
+    A_steps = A.double()[None, None, :].expand(b, l, h).clone().requires_grad_(True)
+    y64, f64 = S.ssd_sequential(w["x"], w["dt"], A_steps, w["B"], w["C"], D=w["D"], z=w["z"], dt_bias=w["dt_bias"],
                                 dt_softplus=softplus, initial_states=w["init"])
     ((y64 * dout.double()).sum() + (f64 * dfin.double()).sum()).backward()
+    w["A"].grad = A_steps.grad.sum(dim=(0, 1))
+    dA_terms = A_steps.grad.abs().sum(dim=(0, 1))
     # device
     d = {k: (None if v is None else v.cuda().clone().requires_grad_(True)) for k, v in vals.items()}
     y, fin = ssd().ssd_combined(d["x"], d["dt"], d["A"], d["B"], d["C"], Q, D=d["D"], z=d["z"], dt_bias=d["dt_bias"],
@@ -167,7 +174,13 @@ def test_combined_gradients_match_float64_autograd(shape, Q, dtype, d_mat, use_z
         want = w[k].grad
         got = d[k].grad.float().cpu().double()
         assert got.shape == want.shape and d[k].grad.dtype == vals[k].dtype
-        if dtype == torch.float32:
+        if k == "A":
+            # a sum over the sequence whose terms cancel: every head against the sum of the magnitudes of its own
+            # terms (a head's own value, or the largest head's, says little about what the sum may be off by)
+            bar = DA_TERM_BAR_F32 if dtype == torch.float32 else DA_TERM_BAR_HALF
+            ratio = (got - want).abs() / (dA_terms + 1e-30)
+            assert bool((ratio <= bar).all()), f"gradient of A: error / sum |dt_t q_t| per head {ratio.tolist()}"
+        elif dtype == torch.float32:
             scale = float(want.abs().max())
             torch.testing.assert_close(got, want, rtol=2e-3, atol=2e-4 * scale, msg=lambda m: f"{k}: {m}")
         else:

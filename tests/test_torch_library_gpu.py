@@ -1,0 +1,119 @@
+"""``torch.ops.ssm_amd.*`` on the device: the registered operators run the HIP kernels (same values as the Python
+façade), differentiate through their registered backward operators (same gradients as the façade's autograd
+functions), and pass PyTorch's own consistency checks of a registration (schema, fake tensors, autograd)."""
+
+import pytest
+import torch
+
+from ssm_amd import ops
+from ssm_amd import torch_library  # noqa: F401  (registers the operators)
+from tests.test_scan_fwd_gpu import make_inputs
+
+pytestmark = pytest.mark.gpu
+
+CHECKS = ("test_schema", "test_faketensor", "test_autograd_registration")
+
+
+def _dev(t):
+    return None if t is None else t.cuda()
+
+
+def _scan_args(dtype, grad):
+    inp = make_inputs(7, 2, 16, 272, 16, dtype=dtype)
+    g = {k: _dev(v) for k, v in inp.items()}
+    if grad:
+        for v in g.values():
+            v.requires_grad_(True)
+    return g
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_selective_scan_through_the_dispatcher(dtype):
+    g, h = _scan_args(dtype, True), _scan_args(dtype, True)
+    y, last = torch.ops.ssm_amd.selective_scan(g["u"], g["delta"], g["A"], g["B"], g["C"], g["D"], g["z"], g["dt_bias"],
+                                               True, True)
+    yr, lr = ops.selective_scan(h["u"], h["delta"], h["A"], h["B"], h["C"], D=h["D"], z=h["z"], dt_bias=h["dt_bias"],
+                                softplus=True, return_last_state=True)
+    assert torch.equal(y, yr) and torch.equal(last, lr)
+    w = torch.randn_like(y.float()).to(dtype)
+    wl = torch.randn_like(last.float()).to(dtype)
+    ((y.float() * w.float()).sum() + (last.float() * wl.float()).sum()).backward()
+    ((yr.float() * w.float()).sum() + (lr.float() * wl.float()).sum()).backward()
+    for k in g:
+        assert g[k].grad is not None and g[k].grad.dtype == g[k].dtype, k
+        torch.testing.assert_close(g[k].grad, h[k].grad, rtol=1e-6, atol=0, msg=lambda m, k=k: f"grad {k}: {m}")
+    y2, none = torch.ops.ssm_amd.selective_scan(g["u"].detach(), g["delta"].detach(), g["A"].detach(), g["B"].detach(),
+                                                g["C"].detach())
+    assert none.numel() == 0 and y2.shape == y.shape
+
+
+def test_state_step_updates_the_state_in_place():
+    g = torch.Generator().manual_seed(3)
+    state = torch.randn(3, 40, 16, generator=g).cuda()
+    x, dt, z = (torch.randn(3, 40, generator=g).cuda() for _ in range(3))
+    A = -(torch.rand(40, 16, generator=g) + 0.5).cuda()
+    Bm, Cm = torch.randn(3, 1, 16, generator=g).cuda(), torch.randn(3, 1, 16, generator=g).cuda()
+    s1, s2 = state.clone(), state.clone()
+    y1 = torch.ops.ssm_amd.selective_state_step(s1, x, dt, A, Bm, Cm, None, z, None, True)
+    y2 = ops.selective_state_step(s2, x, dt, A, Bm, Cm, z=z, softplus=True)
+    assert torch.equal(y1, y2) and torch.equal(s1, s2) and not torch.equal(s1, state)
+
+
+def test_chunk_scan_conv_and_norm_differentiate_through_the_dispatcher():
+    g = torch.Generator().manual_seed(5)
+    leaf = lambda *s: torch.randn(*s, generator=g).cuda().requires_grad_(True)
+    # diagonal chunk scan
+    X, Bm, Cm = leaf(2, 70, 2, 64), leaf(2, 70, 2, 64), leaf(2, 70, 2, 64)
+    dt = (torch.rand(2, 70, 2, generator=g) * 0.2).cuda().requires_grad_(True)
+    A = (-(torch.rand(2, generator=g) + 0.3)).cuda().requires_grad_(True)
+    args = (X, dt, A, Bm, Cm)
+    twins = tuple(t.detach().clone().requires_grad_(True) for t in args)
+    Y = torch.ops.ssm_amd.ssd_chunk_scan(*args, 32)
+    Yr = ops.ssd_chunk_scan(*twins, 32)
+    assert torch.equal(Y, Yr)
+    w = torch.randn_like(Y)
+    (Y * w).sum().backward()
+    (Yr * w).sum().backward()
+    for a, b in zip(args, twins):
+        torch.testing.assert_close(a.grad, b.grad, rtol=1e-6, atol=0)
+    # convolution
+    x, wt, bias = leaf(2, 24, 100), leaf(24, 4), leaf(24)
+    tw = tuple(t.detach().clone().requires_grad_(True) for t in (x, wt, bias))
+    y = torch.ops.ssm_amd.dw_causal_conv(x, wt, bias, "silu")
+    yr = ops.dw_causal_conv(*tw, activation="silu")
+    assert torch.equal(y, yr)
+    y.square().sum().backward()
+    yr.square().sum().backward()
+    for a, b in zip((x, wt, bias), tw):
+        torch.testing.assert_close(a.grad, b.grad, rtol=1e-6, atol=0)
+    # residual add + RMSNorm
+    x, wt, res = leaf(3, 5, 96), leaf(96), leaf(3, 5, 96)
+    tw = tuple(t.detach().clone().requires_grad_(True) for t in (x, wt, res))
+    y = torch.ops.ssm_amd.fused_layer_norm(x, wt, None, res, True, 1e-5, True, True)
+    yr = ops.fused_layer_norm(tw[0], tw[1], None, residual=tw[2], is_rms=True, eps=1e-5, prenorm=True,
+                              residual_in_fp32=True)
+    assert torch.equal(y, yr)
+    y.square().sum().backward()
+    yr.square().sum().backward()
+    for a, b in zip((x, wt, res), tw):
+        torch.testing.assert_close(a.grad, b.grad, rtol=1e-5, atol=1e-6)
+
+
+def test_registrations_pass_opcheck():
+    g = _scan_args(torch.float32, True)
+    torch.library.opcheck(torch.ops.ssm_amd.selective_scan.default,
+                          (g["u"], g["delta"], g["A"], g["B"], g["C"], g["D"], g["z"], g["dt_bias"], True, True),
+                          test_utils=CHECKS)
+    gen = torch.Generator().manual_seed(1)
+    x = torch.randn(2, 24, 100, generator=gen).cuda().requires_grad_(True)
+    wt = torch.randn(24, 4, generator=gen).cuda().requires_grad_(True)
+    torch.library.opcheck(torch.ops.ssm_amd.dw_causal_conv.default, (x, wt, None, "silu"), test_utils=CHECKS)
+    state = torch.randn(3, 40, 16, generator=gen).cuda()
+    v = lambda: torch.randn(3, 40, generator=gen).cuda()
+    A = -(torch.rand(40, 16, generator=gen) + 0.5).cuda()
+    Bm, Cm = torch.randn(3, 1, 16, generator=gen).cuda(), torch.randn(3, 1, 16, generator=gen).cuda()
+    torch.library.opcheck(torch.ops.ssm_amd.selective_state_step.default, (state, v(), v(), A, Bm, Cm),
+                          test_utils=("test_schema", "test_faketensor"))
+    xn = torch.randn(3, 5, 96, generator=gen).cuda().requires_grad_(True)
+    wn = torch.randn(96, generator=gen).cuda().requires_grad_(True)
+    torch.library.opcheck(torch.ops.ssm_amd.fused_layer_norm.default, (xn, wn, None, None, True), test_utils=CHECKS)
