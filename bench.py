@@ -341,8 +341,12 @@ def bench_ssd(batch=4, length=4096, heads=80, hdim=64, nstate=128, chunk=256):
     nc = length // chunk
     flops = (2 * chunk * chunk * nstate * batch * nc + 2 * chunk * chunk * hdim * batch * nc * heads
              + 2 * 2 * chunk * nstate * hdim * batch * nc * heads)
+    # the same call on float16 tensors (the one-pass kernel is compiled for both 16-bit types)
+    x16, B16, C16, z16 = (t.to(torch.float16) for t in (x, Bm, Cm, z))
+    us16 = _time_us(lambda i: ssd.ssd_combined(x16, dt, A, B16, C16, chunk, D=D, z=z16, return_final_states=True), iters=10)
     return {"us": round(us, 1), "TFLOPs": round(flops / us / 1e6, 1),
-            "frac_mfma_bf16_peak": round(flops / us / 1e6 / 2500.0, 4), "dense_tile_flops": flops}
+            "frac_mfma_bf16_peak": round(flops / us / 1e6 / 2500.0, 4), "dense_tile_flops": flops,
+            "float16_us": round(us16, 1)}
 
 
 def bench_ssd_train(batch=4, length=4096, heads=80, hdim=64, nstate=128, chunk=256):

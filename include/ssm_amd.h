@@ -461,7 +461,7 @@ int ssm_ssd_chunk_state_varlen(const ssm_ssd_chunk_state_varlen_args *args, void
 /* The whole forward (chunk_cumsum, bmm_chunk, chunk_state, state_passing,
  * chunk_scan; combined call recorded at scripts/refresh_mamba_goldens.py:591-604)
  * as one pass over the sequence that keeps the running state on chip: the
- * per-chunk states never reach device memory.  Covers bf16 tensors with
+ * per-chunk states never reach device memory.  Covers bf16 and fp16 tensors with
  * headdim 64, chunk in {64, 128, 256}, nstate in {64, 128} and
  * seqlen % chunk == 0; ssm_ssd_combined_supported() tells, other shapes go
  * through the five calls above.  A head with A > 0 is treated as those calls
@@ -480,7 +480,7 @@ typedef struct ssm_ssd_combined_args {
   void *workspace;            /* ssm_ssd_combined_workspace_bytes() bytes, 256-byte aligned */
   size_t workspace_bytes;
   ssm_ssd_dims dims;
-  int32_t io_dtype;           /* must be SSM_BF16 */
+  int32_t io_dtype;           /* SSM_BF16 or SSM_F16 */
   int32_t dt_dtype, dt_softplus, d_per_p;
   float dt_min, dt_max;       /* clamp applied after softplus; use 0 and +inf for none */
   const int32_t *seq_idx;     /* (B, L) sequence ids of a packed batch (first id 0), or NULL: no state and no

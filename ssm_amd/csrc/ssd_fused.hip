@@ -22,7 +22,7 @@
 // B, C and CB are re-laid once per call so that every MFMA operand fragment is
 // one contiguous KiB (64 lanes x 8 bf16).
 //
-// Requires bf16 tensors, P = 64, Q in {64, 128, 256}, N in {64, 128} and L % Q == 0.
+// Requires bf16 or fp16 tensors (the kernels are compiled per element type), P = 64, Q in {64, 128, 256}, N in {64, 128} and L % Q == 0.
 //
 // A head with A > 0 (a growing state): the published kernels evaluate the decays inside a chunk as
 // exp(min(x, 0)) - chunk_state's weights and chunk_scan's in-chunk factors - and leave the two factors on the
@@ -38,17 +38,20 @@ namespace ssm {
 constexpr int FU_P = 64;
 constexpr int FRAG = 512;                                  // bf16 elements per operand fragment
 
-struct SsdFusedParams {
-  const __bf16 *x, *z;
-  __bf16 *y;
+struct SsdFusedParams {                 // x, z, y and the fragment copies hold the call's 16-bit element type
+  const void *x, *z;
+  void *y;
   const float *dA2, *dtv;               // (B,H,nc,Q): log2-scaled running sum, step
-  const __bf16 *Cblk, *Btblk, *CBblk;   // fragment-blocked copies
+  const void *Cblk, *Btblk, *CBblk;     // fragment-blocked copies
   const float *Dk, *init, *A;
   float *final_states;
   int batch, len, heads, groups, nstate, chunk, nchunks, d_per_p;
 };
 
-typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+template <typename E> struct Vec4;
+template <> struct Vec4<__bf16> { typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 type; };
+template <> struct Vec4<_Float16> { typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 type; };
+template <typename E> using V4 = typename Vec4<E>::type;
 
 __device__ __forceinline__ void wave_lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
@@ -73,8 +76,8 @@ constexpr int PD_HEADS = 4;
 struct SsdPrepParams {
   SsdCumsumParams cs;
   float *dA2;
-  const __bf16 *Cm, *Bm;
-  __bf16 *Cblk, *Btblk, *CBblk;
+  const void *Cm, *Bm;                   // element type of the call
+  void *Cblk, *Btblk, *CBblk;
   unsigned n_dt, n_pack;                 // workgroups of the first two roles
   const int *seq_idx;                    // (B, L) sequence ids of a packed batch, or null
   size_t b_row, c_row;                   // elements between the (G, N) blocks of consecutive steps in Bm / Cm
@@ -148,7 +151,9 @@ __device__ __forceinline__ void prep_dt_role(const SsdCumsumParams &p, float *dA
   }
 }
 
+template <typename E>
 __device__ __forceinline__ void prep_pack_role(const SsdPrepParams &pp, unsigned wg) {
+  const E *Cm = reinterpret_cast<const E *>(pp.Cm), *Bm = reinterpret_cast<const E *>(pp.Bm);
   const SsdDims &d = pp.cs.d;
   const int wave = wave_id_uniform(), lane = lane_id();
   const int Q = d.chunk, N = d.nstate, nc = d.nchunks, groups = d.groups, len = d.len;
@@ -166,19 +171,20 @@ __device__ __forceinline__ void prep_pack_role(const SsdPrepParams &pp, unsigned
   const int c = (int)((unit / groups) % nc);
   const int b = (int)(unit / ((size_t)groups * nc));
   const int m = lane & 31, g2 = lane >> 5;
-  bf16x8_t v;
+  V8<E> v;
   if (is_c) {
     const int lb = inner / KN, kn = inner % KN;
-    v = load_frag(pp.Cm + ((size_t)b * len + (size_t)c * Q + 32 * lb + m) * pp.c_row + (size_t)g * N + 16 * kn + 8 * g2);
+    v = load_frag_e<E>(Cm + ((size_t)b * len + (size_t)c * Q + 32 * lb + m) * pp.c_row + (size_t)g * N + 16 * kn + 8 * g2);
   } else {
     const int ks = inner / NT, nt = inner % NT;
-    const __bf16 *col = pp.Bm + ((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * pp.b_row + (size_t)g * N + 32 * nt + m;
+    const E *col = Bm + ((size_t)b * len + (size_t)c * Q + 16 * ks + 8 * g2) * pp.b_row + (size_t)g * N + 32 * nt + m;
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = col[(size_t)j * pp.b_row];
   }
-  *reinterpret_cast<bf16x8_t *>((is_c ? pp.Cblk : pp.Btblk) + f * FRAG + lane * 8) = v;
+  *reinterpret_cast<V8<E> *>(reinterpret_cast<E *>(is_c ? pp.Cblk : pp.Btblk) + f * FRAG + lane * 8) = v;
 }
 
+template <typename E>
 __device__ __forceinline__ void prep_cb_role(const SsdPrepParams &pp, unsigned wg, float *lds) {
   const SsdDims &d = pp.cs.d;
   const int wave = wave_id_uniform(), lane = lane_id();
@@ -196,15 +202,15 @@ __device__ __forceinline__ void prep_cb_role(const SsdPrepParams &pp, unsigned w
   const int g = (int)(unit % groups);
   const size_t bc = unit / groups;                        // b * nchunks + c: the chunk's first row is bc * Q
   const int m = lane & 31, g2 = lane >> 5;
-  const __bf16 *crow_p = pp.Cm + (bc * Q + 32 * lb + m) * pp.c_row + (size_t)g * N + 8 * g2;
-  const __bf16 *brow_p = pp.Bm + (bc * Q + 32 * sb + m) * pp.b_row + (size_t)g * N + 8 * g2;
+  const E *crow_p = reinterpret_cast<const E *>(pp.Cm) + (bc * Q + 32 * lb + m) * pp.c_row + (size_t)g * N + 8 * g2;
+  const E *brow_p = reinterpret_cast<const E *>(pp.Bm) + (bc * Q + 32 * sb + m) * pp.b_row + (size_t)g * N + 8 * g2;
   f32x16_t acc = {0};
-  for (int k0 = 0; k0 < N; k0 += 16) acc = mma(load_frag(crow_p + k0), load_frag(brow_p + k0), acc);
+  for (int k0 = 0; k0 < N; k0 += 16) acc = mma(load_frag_e<E>(crow_p + k0), load_frag_e<E>(brow_p + k0), acc);
   float (*tile)[33] = reinterpret_cast<float (*)[33]>(lds + wave * 32 * 33);
 #pragma unroll
   for (int r = 0; r < 16; ++r) tile[crow(r, g2)][m] = acc[r];
   wave_lds_sync();
-  __bf16 *out = pp.CBblk + ((unit * NLB + lb) * KS + 2 * sb) * FRAG + lane * 8;
+  E *out = reinterpret_cast<E *>(pp.CBblk) + ((unit * NLB + lb) * KS + 2 * sb) * FRAG + lane * 8;
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) {
     float v[8];
@@ -213,16 +219,17 @@ __device__ __forceinline__ void prep_cb_role(const SsdPrepParams &pp, unsigned w
       const int sl = 16 * kk + 8 * g2 + j;
       v[j] = (sb < lb || sl <= m) ? tile[m][sl] : 0.0f;
     }
-    *reinterpret_cast<bf16x8_t *>(out + kk * FRAG) = pack8(v);
+    *reinterpret_cast<V8<E> *>(out + kk * FRAG) = pack8_e<E>(v);
   }
 }
 
+template <typename E>
 __global__ __launch_bounds__(256) void ssd_fused_prep_kernel(const SsdPrepParams pp) {
   __shared__ float lds[4 * 32 * 33];
   const unsigned wg = blockIdx.x;
   if (wg < pp.n_dt) prep_dt_role(pp.cs, pp.dA2, pp.seq_idx, (int)wg, lds);
-  else if (wg < pp.n_dt + pp.n_pack) prep_pack_role(pp, wg - pp.n_dt);
-  else prep_cb_role(pp, wg - pp.n_dt - pp.n_pack, lds);
+  else if (wg < pp.n_dt + pp.n_pack) prep_pack_role<E>(pp, wg - pp.n_dt);
+  else prep_cb_role<E>(pp, wg - pp.n_dt - pp.n_pack, lds);
 }
 
 // ------------------------------------------------- fused kernel, half a head
@@ -254,11 +261,13 @@ typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2_t;
 __device__ __forceinline__ rsrc_t make_rsrc(const void *p) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0x7fffffff, 0x00020000);
 }
-__device__ __forceinline__ bf16x8_t buf_load16(rsrc_t r, int voff, int soff) {
-  return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+template <typename E>
+__device__ __forceinline__ V8<E> buf_load16(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(V8<E>, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
-__device__ __forceinline__ bf16x4_t buf_load8(rsrc_t r, int voff, int soff) {
-  return __builtin_bit_cast(bf16x4_t, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+template <typename E>
+__device__ __forceinline__ V4<E> buf_load8(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(V4<E>, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
 }
 __device__ __forceinline__ float4 buf_load_f4(rsrc_t r, int voff, int soff) {
   return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
@@ -275,7 +284,8 @@ struct HalfStream {
   int off_first, off_second, off_bt, bt_step;
 };
 // Places i (even) and i + 1 of the stream; both lie in the same part of it.
-__device__ __forceinline__ void stream_pair(const HalfStream &st, int i, bf16x8_t &fa, bf16x8_t &fb) {
+template <typename E>
+__device__ __forceinline__ void stream_pair(const HalfStream &st, int i, V8<E> &fa, V8<E> &fb) {
   const int o1 = st.off_first + (i << 10);
   const int o2 = st.off_second + ((i - st.n_first) << 10);
   const int o3 = st.off_bt + (i - st.n_both) * st.bt_step;
@@ -283,8 +293,8 @@ __device__ __forceinline__ void stream_pair(const HalfStream &st, int i, bf16x8_
   const int o12 = in1 ? o1 : o2;
   const int off = in2 ? o12 : o3;
   const int step = in2 ? 1024 : st.bt_step;
-  fa = buf_load16(st.r, st.vf, off);
-  fb = buf_load16(st.r, st.vf, off + step);
+  fa = buf_load16<E>(st.r, st.vf, off);
+  fb = buf_load16<E>(st.r, st.vf, off + step);
 }
 
 // Blocks below the diagonal and the diagonal block of row block `lb` into `acc` (one 32 x 32
@@ -293,9 +303,9 @@ __device__ __forceinline__ void stream_pair(const HalfStream &st, int i, bf16x8_
 // every second block before it, (b0, b1) the other pair.
 // With SKIP, the per-head skip factor dskip joins the diagonal of the last operand (CB dt + D at
 // s = l, rounded to bf16 as one number), so that the product with the plain x adds D x.
-template <bool SKIP>
-__device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16x8_t &a1, bf16x8_t &b0, bf16x8_t &b1,
-                                               int lb, int pos0, const HalfStream &st, const __bf16 *xw, const __bf16 *xr,
+template <typename E, bool SKIP>
+__device__ __forceinline__ void half_row_block(f32x16_t &acc, V8<E> &a0, V8<E> &a1, V8<E> &b0, V8<E> &b1,
+                                               int lb, int pos0, const HalfStream &st, const E *xw, const E *xr,
                                                const float *dAs, const float *dqs, const float *l2s, int Q, int qmask,
                                                int m, int g2, float dskip) {
   float prev_end = 0.0f;
@@ -307,11 +317,11 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
     const float gs = exp2_hw(fminf(endv - prev_end, 0.0f));                                     \
     prev_end = endv;                                                                            \
     _Pragma("unroll") for (int r = 0; r < 16; ++r) acc[r] *= gs;                                \
-    const bf16x8_t x0 = load_frag(xw + m * Q + (((4 * (SB) + g2) ^ (m & qmask)) << 3));         \
-    const bf16x8_t x1 = load_frag(xw + m * Q + (((4 * (SB) + 2 + g2) ^ (m & qmask)) << 3));     \
+    const V8<E> x0 = load_frag_e<E>(xw + m * Q + (((4 * (SB) + g2) ^ (m & qmask)) << 3));       \
+    const V8<E> x1 = load_frag_e<E>(xw + m * Q + (((4 * (SB) + 2 + g2) ^ (m & qmask)) << 3));   \
     acc = mma(x0, FA, acc);                                                                     \
     acc = mma(x1, FB, acc);                                                                     \
-    stream_pair(st, pos0 + 2 * (SB) + 4, FA, FB);                                               \
+    stream_pair<E>(st, pos0 + 2 * (SB) + 4, FA, FB);                                            \
   }
   const int odd = lb & 1;
   if (odd) FH_BLOCK(b0, b1, 0)
@@ -327,7 +337,7 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
   // only needs a bound there
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) {
-    const bf16x8_t f = kk == 0 ? a0 : a1;
+    const V8<E> f = kk == 0 ? a0 : a1;
     const int sbase = 32 * lb + 16 * kk + 8 * g2;
     const float4 q0 = *reinterpret_cast<const float4 *>(dqs + sbase), q1 = *reinterpret_cast<const float4 *>(dqs + sbase + 4);
     const float4 c0 = *reinterpret_cast<const float4 *>(l2s + sbase), c1 = *reinterpret_cast<const float4 *>(l2s + sbase + 4);
@@ -341,6 +351,7 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
       // the (zeroed) places above the diagonal finite.
       const float e = exp2_hw(fminf(dal + dq[jj], cap[jj]));
       if (SKIP) {
+        // (CB dt + D at s = l, rounded to the element type as one number)
         // element jj of fragment kk lies on the diagonal in lane 16 kk + jj (g2 = 0) and lane 32 + 16 kk + 8 + jj (g2 = 1)
         const unsigned long long on_diag = (1ull << (16 * kk + jj)) | (1ull << (40 + 16 * kk + jj));
         float sel;
@@ -350,14 +361,15 @@ __device__ __forceinline__ void half_row_block(f32x16_t &acc, bf16x8_t &a0, bf16
         mv[jj] = (float)f[jj] * e;
       }
     }
-    const bf16x8_t a = load_frag(xr + m * Q + (((4 * lb + 2 * kk + g2) ^ (m & qmask)) << 3));
-    acc = mma(a, pack8(mv), acc);
+    const V8<E> a = load_frag_e<E>(xr + m * Q + (((4 * lb + 2 * kk + g2) ^ (m & qmask)) << 3));
+    acc = mma(a, pack8_e<E>(mv), acc);
   }
-  stream_pair(st, pos0 + 2 * lb + 4, a0, a1);
+  stream_pair<E>(st, pos0 + 2 * lb + 4, a0, a1);
 }
 
 // acc[p][l] += D[p] x[l][p] for row block lb, x read from the plain tile (per-channel skip factors).
-__device__ __forceinline__ void half_skip_term(f32x16_t &acc, int lb, const __bf16 *xr, int Q, int qmask, int m, int g2,
+template <typename E>
+__device__ __forceinline__ void half_skip_term(f32x16_t &acc, int lb, const E *xr, int Q, int qmask, int m, int g2,
                                                const float *Dp) {
   const int lrow = 32 * lb + m;
   const int xcol = lrow & 7, xchunk = lrow >> 3;
@@ -374,13 +386,13 @@ __device__ __forceinline__ void half_skip_term(f32x16_t &acc, int lb, const __bf
   }
 }
 
-template <int Q, int N, int DMODE, bool HAS_Z>
+template <typename E, int Q, int N, int DMODE, bool HAS_Z>
 __global__ __launch_bounds__(FH_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void ssd_fused_half_kernel(const SsdFusedParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  __bf16 *xw = reinterpret_cast<__bf16 *>(smem);                        // x~ [32][Q]
-  __bf16 *xr = reinterpret_cast<__bf16 *>(smem + FH_TILE_BYTES);        // x  [32][Q]
-  __bf16 *sbf = reinterpret_cast<__bf16 *>(smem + 2 * FH_TILE_BYTES);   // S as bf16 [32][N]; later the output staging
+  E *xw = reinterpret_cast<E *>(smem);                                  // x~ [32][Q]
+  E *xr = reinterpret_cast<E *>(smem + FH_TILE_BYTES);                  // x  [32][Q]
+  E *sbf = reinterpret_cast<E *>(smem + 2 * FH_TILE_BYTES);             // S in 16 bits [32][N]; later the output staging
   float *dAs = reinterpret_cast<float *>(smem + 3 * FH_TILE_BYTES);     // [Q] log2-scaled running sum
   float *dqs = dAs + 256;                                               // [Q] log2(dt) - running sum: exponent offset of a step as a source
   float *wss = dqs + 256;                                               // [Q] staging weight dt exp(cs[l | 31] - cs[l])
@@ -413,8 +425,9 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
 
   // ---- buffers and the lanes' constant offsets
   const size_t xbase = ((size_t)b * p.len * H + h) * FU_P + p0;
-  const rsrc_t rx = make_rsrc(p.x + xbase), ry = make_rsrc(p.y + xbase);
-  const rsrc_t rz = make_rsrc(HAS_Z ? p.z + xbase : p.x + xbase);
+  const E *px = reinterpret_cast<const E *>(p.x);
+  const rsrc_t rx = make_rsrc(px + xbase), ry = make_rsrc(reinterpret_cast<E *>(p.y) + xbase);
+  const rsrc_t rz = make_rsrc(HAS_Z ? reinterpret_cast<const E *>(p.z) + xbase : px + xbase);
   const size_t tbase = ((size_t)b * H + h) * nc * Q;   // dA2 and dtv are laid out alike
   const rsrc_t rt = make_rsrc(p.dtv + tbase);
   const int t_dA = (int)((const char *)p.dA2 - (const char *)p.dtv);
@@ -439,14 +452,14 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     for (int r = 0; r < 16; ++r) S[r] = ip[crow(r, g2)];
   }
   f32x16_t accF, accS;
-  bf16x8_t f0, f1, f2, f3;
+  V8<E> f0, f1, f2, f3;
   // what a chunk reads from HBM, requested one chunk ahead: x, dt and the running sums
-  bf16x4_t raw[8];
+  V4<E> raw[8];
   float dA_t, dt_t;
 #define FH_REQUEST_CHUNK(CC)                                                                              \
   {                                                                                                       \
     const int xo_ = (CC) * Q * xrow_b, to_ = (CC) * Q * 4;                                                \
-    _Pragma("unroll") for (int r = 0; r < 8; ++r) raw[r] = buf_load8(rx, v_raw, xo_ + r * xrow_b);        \
+    _Pragma("unroll") for (int r = 0; r < 8; ++r) raw[r] = buf_load8<E>(rx, v_raw, xo_ + r * xrow_b);        \
     dA_t = buf_load_f1(rt, v_t, t_dA + to_);                                                              \
     dt_t = buf_load_f1(rt, v_t, to_);                                                                     \
   }
@@ -454,10 +467,10 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
 #define FH_C_OFF(CC, LB, KNI) ((((((b * nc + (CC)) * G + g) * NLB + (LB)) * KN + (KNI))) << 10)
   FH_REQUEST_CHUNK(0)
   if (yact && has_init) {
-    f0 = buf_load16(rf, st.vf, FH_C_OFF(0, lbF, 0));
-    f1 = buf_load16(rf, st.vf, FH_C_OFF(0, lbS, 0));
-    f2 = buf_load16(rf, st.vf, FH_C_OFF(0, lbF, 1));
-    f3 = buf_load16(rf, st.vf, FH_C_OFF(0, lbS, 1));
+    f0 = buf_load16<E>(rf, st.vf, FH_C_OFF(0, lbF, 0));
+    f1 = buf_load16<E>(rf, st.vf, FH_C_OFF(0, lbS, 0));
+    f2 = buf_load16<E>(rf, st.vf, FH_C_OFF(0, lbF, 1));
+    f3 = buf_load16<E>(rf, st.vf, FH_C_OFF(0, lbS, 1));
   }
 
   for (int c = 0; c < nc; ++c) {
@@ -486,11 +499,11 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     if (sact && carry) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        bf16x4_t v;
+        V4<E> v;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = (__bf16)S[4 * q + j];
+        for (int j = 0; j < 4; ++j) v[j] = (E)S[4 * q + j];
         const int chunk16 = 4 * nt_s + q;
-        *reinterpret_cast<bf16x4_t *>(sbf + m * N + ((chunk16 ^ (m & nmask)) << 3) + 4 * g2) = v;
+        *reinterpret_cast<V4<E> *>(sbf + m * N + ((chunk16 ^ (m & nmask)) << 3) + 4 * g2) = v;
       }
     }
     if (tid < Q) {                         // whole waves: Q is a multiple of 64
@@ -507,16 +520,16 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
       // ---- stage x~ and x, transposed to [p][s]
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        bf16x8_t colw, colr;
+        V8<E> colw, colr;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
           colr[r] = raw[r][i];
-          colw[r] = (__bf16)((float)raw[r][i] * w8[r]);
+          colw[r] = (E)((float)raw[r][i] * w8[r]);
         }
         const int prow = spb * 4 + i;
         const int at = prow * Q + ((slb8 ^ (prow & qmask)) << 3);
-        *reinterpret_cast<bf16x8_t *>(xw + at) = colw;
-        *reinterpret_cast<bf16x8_t *>(xr + at) = colr;
+        *reinterpret_cast<V8<E> *>(xw + at) = colw;
+        *reinterpret_cast<V8<E> *>(xr + at) = colr;
       }
     }
     __syncthreads();
@@ -526,32 +539,32 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
       const int cF = FH_C_OFF(c, lbF, 0), cS = FH_C_OFF(c, lbS, 0);
 #define FH_STEP_A(FF, FS, KK)                                                                     \
       {                                                                                           \
-        const bf16x8_t a = load_frag(sbf + m * N + (((2 * (KK) + g2) ^ (m & nmask)) << 3));       \
+        const V8<E> a = load_frag_e<E>(sbf + m * N + (((2 * (KK) + g2) ^ (m & nmask)) << 3));     \
         accF = mma(a, FF, accF);                                                                  \
         accS = mma(a, FS, accS);                                                                  \
       }
       {                                    // the first step starts the accumulators
-        const bf16x8_t a = load_frag(sbf + m * N + ((g2 ^ (m & nmask)) << 3));
+        const V8<E> a = load_frag_e<E>(sbf + m * N + ((g2 ^ (m & nmask)) << 3));
         accF = mma(a, f0, (f32x16_t){0});
         accS = mma(a, f1, (f32x16_t){0});
-        f0 = buf_load16(rf, st.vf, cF + (2 << 10));
-        f1 = buf_load16(rf, st.vf, cS + (2 << 10));
+        f0 = buf_load16<E>(rf, st.vf, cF + (2 << 10));
+        f1 = buf_load16<E>(rf, st.vf, cS + (2 << 10));
         FH_STEP_A(f2, f3, 1)
-        f2 = buf_load16(rf, st.vf, cF + (3 << 10));
-        f3 = buf_load16(rf, st.vf, cS + (3 << 10));
+        f2 = buf_load16<E>(rf, st.vf, cF + (3 << 10));
+        f3 = buf_load16<E>(rf, st.vf, cS + (3 << 10));
       }
       for (int kn0 = 2; kn0 < KN - 2; kn0 += 2) {
         FH_STEP_A(f0, f1, kn0)
-        f0 = buf_load16(rf, st.vf, cF + ((kn0 + 2) << 10));
-        f1 = buf_load16(rf, st.vf, cS + ((kn0 + 2) << 10));
+        f0 = buf_load16<E>(rf, st.vf, cF + ((kn0 + 2) << 10));
+        f1 = buf_load16<E>(rf, st.vf, cS + ((kn0 + 2) << 10));
         FH_STEP_A(f2, f3, kn0 + 1)
-        f2 = buf_load16(rf, st.vf, cF + ((kn0 + 3) << 10));
-        f3 = buf_load16(rf, st.vf, cS + ((kn0 + 3) << 10));
+        f2 = buf_load16<E>(rf, st.vf, cF + ((kn0 + 3) << 10));
+        f3 = buf_load16<E>(rf, st.vf, cS + ((kn0 + 3) << 10));
       }
       FH_STEP_A(f0, f1, KN - 2)
-      stream_pair(st, 0, f0, f1);
+      stream_pair<E>(st, 0, f0, f1);
       FH_STEP_A(f2, f3, KN - 1)
-      stream_pair(st, 2, f2, f3);
+      stream_pair<E>(st, 2, f2, f3);
 #undef FH_STEP_A
       if (grow) {                          // the carried term of a growing head takes exp(cs_l), unclamped
         const float gF = exp2_hw(fmaxf(dAs[32 * lbF + m], 0.0f)), gS = exp2_hw(fmaxf(dAs[32 * lbS + m], 0.0f));
@@ -564,22 +577,22 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     } else if (yact) {                     // first chunk without an initial state
       accF = (f32x16_t){0};
       accS = (f32x16_t){0};
-      stream_pair(st, 0, f0, f1);
-      stream_pair(st, 2, f2, f3);
+      stream_pair<E>(st, 0, f0, f1);
+      stream_pair<E>(st, 2, f2, f3);
     } else {                               // no row blocks: straight to where the state update expects the ring
-      stream_pair(st, 2, f2, f3);
-      stream_pair(st, 4, f0, f1);
+      stream_pair<E>(st, 2, f2, f3);
+      stream_pair<E>(st, 4, f0, f1);
     }
 
     // ---- the two row blocks.  Pair q of the stream lives in (f0, f1) if q is even, in (f2, f3) if odd:
     // the diagonal block of the first row block is pair lbF, that of the second pair NLB.
     if (yact) {
-      if (lbF & 1) half_row_block<DMODE == 1>(accF, f2, f3, f0, f1, lbF, 0, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
-      else half_row_block<DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
-      half_row_block<DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
+      if (lbF & 1) half_row_block<E, DMODE == 1>(accF, f2, f3, f0, f1, lbF, 0, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
+      else half_row_block<E, DMODE == 1>(accF, f0, f1, f2, f3, lbF, 0, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
+      half_row_block<E, DMODE == 1>(accS, f0, f1, f2, f3, lbS, st.n_first, st, xw, xr, dAs, dqs, l2s, Q, qmask, m, g2, dhead);
       if constexpr (DMODE == 2) {
-        half_skip_term(accF, lbF, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
-        half_skip_term(accS, lbS, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
+        half_skip_term<E>(accF, lbF, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
+        half_skip_term<E>(accS, lbS, xr, Q, qmask, m, g2, p.Dk + h * FU_P + p0);
       }
     }
     __syncthreads();                       // every wave is past the carried state: its tile becomes the output staging
@@ -590,12 +603,12 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
     // read from HBM waits for it: the requests go out after the first four steps, behind the ring's first
     // refills.  The ring stands one pair on; its last refills are the next chunk's first fragments of C.
     const int cn = min(c + 1, nc - 1);
-    bf16x8_t zF[2], zS[2];
+    V8<E> zF[2], zS[2];
     const int row_o = c * Q * xrow_b;
     float prev_end = 0.0f;
 #define FH_STEP_C(F, KK)                                                                        \
       {                                                                                         \
-        const bf16x8_t xf = load_frag(xw + m * Q + (((2 * (KK) + g2) ^ (m & qmask)) << 3));     \
+        const V8<E> xf = load_frag_e<E>(xw + m * Q + (((2 * (KK) + g2) ^ (m & qmask)) << 3));   \
         S = mma(F, xf, S);                                                                      \
       }
 #define FH_SCALE_C(KK)                                                                          \
@@ -609,8 +622,8 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
       {                                                                                         \
         if (yact && HAS_Z) {                                                                    \
           _Pragma("unroll") for (int pass = 0; pass < 2; ++pass) {                              \
-            zF[pass] = buf_load16(rz, v_row, row_o + (32 * lbF + 16 * pass) * xrow_b);          \
-            zS[pass] = buf_load16(rz, v_row, row_o + (32 * lbS + 16 * pass) * xrow_b);          \
+            zF[pass] = buf_load16<E>(rz, v_row, row_o + (32 * lbF + 16 * pass) * xrow_b);          \
+            zS[pass] = buf_load16<E>(rz, v_row, row_o + (32 * lbS + 16 * pass) * xrow_b);          \
           }                                                                                     \
         }                                                                                       \
         FH_REQUEST_CHUNK(cn)                                                                    \
@@ -628,27 +641,27 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
         const bool more = k0 + 4 < KS;
         FH_SCALE_C(k0)
         FH_STEP_C(f2, k0)
-        if (more) f2 = buf_load16(rf, st.vf, st.off_bt + (k0 + 4) * st.bt_step);
-        else if (yact) f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
+        if (more) f2 = buf_load16<E>(rf, st.vf, st.off_bt + (k0 + 4) * st.bt_step);
+        else if (yact) f2 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbF, 1));
         FH_STEP_C(f3, k0 + 1)
-        if (more) f3 = buf_load16(rf, st.vf, st.off_bt + (k0 + 5) * st.bt_step);
-        else if (yact) f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
+        if (more) f3 = buf_load16<E>(rf, st.vf, st.off_bt + (k0 + 5) * st.bt_step);
+        else if (yact) f3 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbS, 1));
         FH_SCALE_C(k0 + 2)
         FH_STEP_C(f0, k0 + 2)
-        if (more) f0 = buf_load16(rf, st.vf, st.off_bt + (k0 + 6) * st.bt_step);
-        else if (yact) f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
+        if (more) f0 = buf_load16<E>(rf, st.vf, st.off_bt + (k0 + 6) * st.bt_step);
+        else if (yact) f0 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbF, 0));
         FH_STEP_C(f1, k0 + 3)
-        if (more) f1 = buf_load16(rf, st.vf, st.off_bt + (k0 + 7) * st.bt_step);
-        else if (yact) f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
+        if (more) f1 = buf_load16<E>(rf, st.vf, st.off_bt + (k0 + 7) * st.bt_step);
+        else if (yact) f1 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbS, 0));
         if (k0 == 0) FH_REQUEST_HBM
       }
     } else {
       FH_REQUEST_HBM
       if (yact) {
-        f0 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 0));
-        f1 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 0));
-        f2 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbF, 1));
-        f3 = buf_load16(rf, st.vf, FH_C_OFF(cn, lbS, 1));
+        f0 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbF, 0));
+        f1 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbS, 0));
+        f2 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbF, 1));
+        f3 = buf_load16<E>(rf, st.vf, FH_C_OFF(cn, lbS, 1));
       }
     }
 #undef FH_REQUEST_HBM
@@ -685,7 +698,7 @@ void ssd_fused_half_kernel(const SsdFusedParams p) {
           // instruction that rewrites the registers in the next two slots has been seen to get ahead of the
           // read under load (wrong dwords in the last quarter of each 16 lanes).  So the data stays live, and
           // idle slots follow the store.
-          const u32x4_t packed = __builtin_bit_cast(u32x4_t, pack8(v));
+          const u32x4_t packed = __builtin_bit_cast(u32x4_t, pack8_e<E>(v));
           __builtin_amdgcn_raw_buffer_store_b128(packed, ry, v_row, row_o + (32 * lb + 16 * pass) * xrow_b, 0);
           asm volatile("s_nop 3" : : "v"(packed) : "memory");
         }
@@ -756,7 +769,7 @@ static int fused_dims(const char *who, const ssm_ssd_dims *s, ssm::SsdDims &d) {
 extern "C" int ssm_ssd_combined_supported(const ssm_ssd_dims *dims, int io_dtype) {
   ssm::SsdDims d;
   if (fused_dims("ssm_ssd_combined_supported", dims, d) != SSM_OK) return 0;
-  return io_dtype == SSM_BF16 && ssm::fused_shape_ok(d) ? 1 : 0;
+  return (io_dtype == SSM_BF16 || io_dtype == SSM_F16) && ssm::fused_shape_ok(d) ? 1 : 0;
 }
 
 extern "C" size_t ssm_ssd_combined_workspace_bytes(const ssm_ssd_dims *dims) {
@@ -772,7 +785,8 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   SsdDims d;
   int rc = fused_dims("ssm_ssd_combined_fwd", &a->dims, d);
   if (rc != SSM_OK) return rc;
-  SSM_REQUIRE(a->io_dtype == SSM_BF16, SSM_ERR_BAD_DTYPE, "ssm_ssd_combined_fwd: x, z, y, Bm and Cm must be bf16");
+  SSM_REQUIRE(a->io_dtype == SSM_BF16 || a->io_dtype == SSM_F16, SSM_ERR_BAD_DTYPE,
+              "ssm_ssd_combined_fwd: x, z, y, Bm and Cm must be bf16 or fp16 (one type for all)");
   SSM_REQUIRE(valid_dtype(a->dt_dtype), SSM_ERR_BAD_DTYPE, "ssm_ssd_combined_fwd: dt_dtype=%d", a->dt_dtype);
   SSM_REQUIRE(fused_shape_ok(d), SSM_ERR_BAD_SHAPE,
               "ssm_ssd_combined_fwd: needs headdim 64, chunk in {64,128,256}, nstate in {64,128} and "
@@ -798,7 +812,7 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   cp.dt_out = reinterpret_cast<float *>(ws + lay.dt_out);
   cp.d = d; cp.dt_dtype = a->dt_dtype; cp.softplus = a->dt_softplus ? 1 : 0; cp.dt_min = a->dt_min; cp.dt_max = a->dt_max;
   pp.dA2 = reinterpret_cast<float *>(ws + lay.dA2);
-  pp.Cm = reinterpret_cast<const __bf16 *>(a->Cm); pp.Bm = reinterpret_cast<const __bf16 *>(a->Bm);
+  pp.Cm = a->Cm; pp.Bm = a->Bm;
   const size_t dense_row = (size_t)d.groups * d.nstate;
   SSM_REQUIRE(a->b_row_stride >= 0 && a->c_row_stride >= 0 && (a->b_row_stride == 0 || (size_t)a->b_row_stride >= dense_row) &&
                   (a->c_row_stride == 0 || (size_t)a->c_row_stride >= dense_row) && a->b_row_stride % 8 == 0 && a->c_row_stride % 8 == 0,
@@ -806,22 +820,24 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
               (long long)a->b_row_stride, (long long)a->c_row_stride, dense_row);
   pp.b_row = a->b_row_stride ? (size_t)a->b_row_stride : dense_row;
   pp.c_row = a->c_row_stride ? (size_t)a->c_row_stride : dense_row;
-  __bf16 *Cblk = reinterpret_cast<__bf16 *>(ws + lay.Cblk), *Btblk = reinterpret_cast<__bf16 *>(ws + lay.Btblk);
-  pp.Cblk = Cblk; pp.Btblk = Btblk; pp.CBblk = reinterpret_cast<__bf16 *>(ws + lay.CBblk);
+  void *Cblk = ws + lay.Cblk, *Btblk = ws + lay.Btblk;
+  pp.Cblk = Cblk; pp.Btblk = Btblk; pp.CBblk = ws + lay.CBblk;
   const size_t n_dt = (size_t)d.batch * d.nchunks * ((d.heads + PD_HEADS - 1) / PD_HEADS);
   const size_t n_pack = (bcg * NLB * KN + bcg * KS * NT + 3) / 4;
   const size_t n_cb = (bcg * (NLB * (NLB + 1) / 2) + 3) / 4;
   SSM_REQUIRE(n_dt + n_pack + n_cb < ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "ssm_ssd_combined_fwd: too many workgroups");
   pp.n_dt = (unsigned)n_dt; pp.n_pack = (unsigned)n_pack;
   pp.seq_idx = a->seq_idx;
-  hipLaunchKernelGGL(ssd_fused_prep_kernel, dim3((unsigned)(n_dt + n_pack + n_cb)), dim3(256), 0, s, pp);
+  const bool f16 = a->io_dtype == SSM_F16;
+  if (f16) hipLaunchKernelGGL(ssd_fused_prep_kernel<_Float16>, dim3((unsigned)(n_dt + n_pack + n_cb)), dim3(256), 0, s, pp);
+  else hipLaunchKernelGGL(ssd_fused_prep_kernel<__bf16>, dim3((unsigned)(n_dt + n_pack + n_cb)), dim3(256), 0, s, pp);
   SSM_CHECK_LAUNCH("ssm_ssd_combined_fwd(prep)");
 
   SsdFusedParams fp{};
-  fp.x = reinterpret_cast<const __bf16 *>(a->x); fp.z = reinterpret_cast<const __bf16 *>(a->z);
-  fp.y = reinterpret_cast<__bf16 *>(a->y);
+  fp.x = a->x; fp.z = a->z;
+  fp.y = a->y;
   fp.dA2 = reinterpret_cast<const float *>(ws + lay.dA2); fp.dtv = cp.dt_out;
-  fp.Cblk = Cblk; fp.CBblk = reinterpret_cast<const __bf16 *>(ws + lay.CBblk); fp.Btblk = Btblk;
+  fp.Cblk = Cblk; fp.CBblk = ws + lay.CBblk; fp.Btblk = Btblk;
   fp.Dk = a->Dskip; fp.init = a->initial_states; fp.A = a->A; fp.final_states = a->final_states;
   fp.batch = d.batch; fp.len = d.len; fp.heads = d.heads; fp.groups = d.groups; fp.nstate = d.nstate; fp.chunk = d.chunk;
   fp.nchunks = d.nchunks; fp.d_per_p = a->d_per_p ? 1 : 0;
@@ -829,7 +845,7 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
   const unsigned grid = (unsigned)(d.batch * d.heads) * 2;
 #define SSM_LAUNCH_FUSED(QQ, NN, DM, HZ)                                                           \
   {                                                                                                \
-    auto kernel = ssd_fused_half_kernel<QQ, NN, DM, HZ>;                                           \
+    auto kernel = f16 ? ssd_fused_half_kernel<_Float16, QQ, NN, DM, HZ> : ssd_fused_half_kernel<__bf16, QQ, NN, DM, HZ>; \
     if (allow_dynamic_lds(kernel, FH_LDS_BYTES) != hipSuccess) {                                   \
       set_error("ssm_ssd_combined_fwd: cannot reserve %d bytes of LDS", FH_LDS_BYTES);             \
       return SSM_ERR_LAUNCH;                                                                       \

@@ -367,15 +367,15 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
 
 
 def _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q):
-    """Whether the one-pass kernel covers this call (bf16 tensors on the GPU and a
+    """Whether the one-pass kernel covers this call (bf16 or fp16 tensors of one type on the GPU and a
     shape ``ssm_ssd_combined_supported`` accepts)."""
     if Q <= 0 or seqlen % Q != 0:
         return False
     tensors = [x, B, C] + ([z] if z is not None else [])
-    if any(t.dtype != torch.bfloat16 for t in tensors) or not x.is_cuda:
+    if x.dtype not in (torch.bfloat16, torch.float16) or any(t.dtype != x.dtype for t in tensors) or not x.is_cuda:
         return False
     dims = _dims(batch, seqlen, heads, hdim, groups, nstate, Q)
-    return bool(_lib.load().ssm_ssd_combined_supported(dims, _lib.dtype_enum(torch.bfloat16)))
+    return bool(_lib.load().ssm_ssd_combined_supported(dims, _lib.dtype_enum(x.dtype)))
 
 
 def _rows_in_place(t):
@@ -418,7 +418,7 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
         x=_lib.ptr(xc), dt=_lib.ptr(dtc), A=_lib.ptr(Af), dt_bias=_lib.ptr(bf), Bm=_lib.ptr(Bc), Cm=_lib.ptr(Cc),
         Dskip=_lib.ptr(Df), z=_lib.ptr(zc), initial_states=_lib.ptr(init), y=_lib.ptr(y),
         final_states=_lib.ptr(final), workspace=work.data_ptr() + off, workspace_bytes=nbytes, dims=dims,
-        io_dtype=_lib.dtype_enum(torch.bfloat16), dt_dtype=_lib.dtype_enum(dtc.dtype),
+        io_dtype=_lib.dtype_enum(xc.dtype), dt_dtype=_lib.dtype_enum(dtc.dtype),
         dt_softplus=int(bool(dt_softplus)), d_per_p=int(d_per_p),
         dt_min=float(dt_limit[0]), dt_max=float(dt_limit[1]), seq_idx=_lib.ptr(si), b_row_stride=b_row,
         c_row_stride=c_row)
@@ -433,7 +433,7 @@ def ssd_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initi
                  states_dtype=None, force_generic=False, fused=None, seq_idx=None, cu_seqlens=None,
                  return_varlen_states=False):
     """Mamba-2 SSD, differentiable in ``x, dt, A, B, C, D, z, dt_bias, initial_states`` (gradients:
-    :func:`ssd_combined_backward`).  bf16 calls whose shape the one-pass kernel covers run
+    :func:`ssd_combined_backward`).  bf16 and fp16 calls whose shape the one-pass kernel covers run
     ``ssm_ssd_combined_fwd``; everything else runs
     ``chunk_cumsum -> bmm_chunk, chunk_state -> state_passing -> chunk_scan``.
 
@@ -558,7 +558,7 @@ def _ssd_combined_forward(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=No
         return outs[0] if len(outs) == 1 else tuple(outs)
     can_fuse = not force_generic and fused is not False and not return_varlen_states and \
         _fused_ok(x, dt, B, C, z, D, batch, seqlen, heads, hdim, groups, nstate, Q)
-    _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 x/B/C/z, headdim 64, "
+    _need(can_fuse or not fused, "fused=True, but the one-pass kernel needs bf16 or fp16 x/B/C/z, headdim 64, "
           "chunk in {64,128,256}, nstate in {64,128} and seqlen % chunk == 0.")
     if can_fuse:
         return _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt_limit,

@@ -539,10 +539,12 @@ FUSED_CASES = [
 ]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
 @pytest.mark.parametrize("shape,Q,d_mat,use_z,use_init", FUSED_CASES, ids=lambda v: str(v).replace(" ", ""))
-def test_bf16_one_pass_matches_oracle_and_five_kernel_path(shape, Q, d_mat, use_z, use_init):
+def test_one_pass_matches_oracle_and_five_kernel_path(shape, Q, d_mat, use_z, use_init, dtype):
+    """The one-pass kernel in both 16-bit element types (it is compiled per type: v_mfma_f32_32x32x16_bf16 / _f16)."""
     b, l, h, p, g, n = shape
-    inp = make(17 + l + Q, b, l, h, p, g, n, dtype=torch.bfloat16, d_mat=d_mat, use_z=use_z, use_init=use_init)
+    inp = make(17 + l + Q, b, l, h, p, g, n, dtype=dtype, d_mat=d_mat, use_z=use_z, use_init=use_init)
     args = (cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
     kw = dict(D=cu(inp["D"]), z=cu(inp["z"]), initial_states=cu(inp["init"]), return_final_states=True)
     y, fin = ssd().ssd_combined(*args, fused=True, **kw)
@@ -552,7 +554,8 @@ def test_bf16_one_pass_matches_oracle_and_five_kernel_path(shape, Q, d_mat, use_
                                 initial_states=inp["init"])
     half_close(y, y64, "y, one pass")
     half_close(fin, f64, "final states, one pass")
-    # the two GPU paths round at different places; they agree to bf16 resolution
+    assert y.dtype == dtype
+    # the two GPU paths round at different places; they agree to the resolution of the element type
     half_close(y, y5.float(), "y, one pass against five kernels")
     half_close(fin, fin5, "final states, one pass against five kernels")
 
