@@ -231,6 +231,78 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
   }
 }
 
+// The same forward for aligned rows of sequences of at least a few strips: a thread walks CONV_CL_WALK strips in
+// turn.  A launch of one strip per thread runs as a single round of waves that all read, then all compute, then
+// all write.  Walking, a thread requests the rows of its next strip before it computes the present one and keeps
+// the present strip's last K-1 rows as the next one's history (no row is read twice): 25.4 -> 24.1 us at
+// 8 x 2048 x 1536 bf16, whatever the number of strips walked (2 to 16).  What remains is not the shape of the
+// walk: the channels-first kernel does the same arithmetic per element in 19.5 us on rows that are contiguous
+// in time.
+constexpr int CONV_CL_WALK = 4, CONV_CL_WALK_STRIP = 8;   // strips of 8 steps: 24.1 us against 25.4 with 16 and 27.9 with 32
+constexpr int CONV_CL_WALK_THREADS = 64;
+template <typename T>
+__global__ __launch_bounds__(CONV_CL_WALK_THREADS) void conv_fwd_cl_walk_kernel(const ConvParams p) {
+  constexpr int VEC = CONV_CL_FWD_BYTES / sizeof(T);
+  constexpr int HIST = CONV_TAPS - 1, S = CONV_CL_WALK_STRIP, SPAN = CONV_CL_WALK_STRIP * CONV_CL_WALK;
+  const int cvecs = p.chans / VEC;
+  const int spans = (p.len + SPAN - 1) / SPAN;
+  const size_t total = (size_t)p.batch * spans * cvecs;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int cv = (int)(gid % cvecs);
+  const int span = (int)((gid / cvecs) % spans);
+  const int b = (int)(gid / ((size_t)cvecs * spans));
+  const int c0 = cv * VEC;
+  float wrev[VEC][CONV_TAPS], bias[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    bias[i] = p.bias ? p.bias[c0 + i] : 0.0f;
+    load_taps(p.w, c0 + i, p.K, wrev[i]);
+  }
+  const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
+  T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
+  const int t_first = span * SPAN;
+  Pack<T, VEC> raw[HIST + S];
+#pragma unroll
+  for (int j = 0; j < HIST + S; ++j)
+    raw[j] = *reinterpret_cast<const Pack<T, VEC> *>(xb + (size_t)min(max(t_first - HIST + j, 0), p.len - 1) * p.chans);
+#pragma unroll
+  for (int j = 0; j < HIST; ++j) {
+    if (t_first - HIST + j < 0) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) raw[j].v[i] = from_f32<T>(0.0f);
+    }
+  }
+#pragma unroll
+  for (int w = 0; w < CONV_CL_WALK; ++w) {
+    const int t_begin = t_first + w * S;
+    Pack<T, VEC> nxt[S];
+    if (w + 1 < CONV_CL_WALK) {
+#pragma unroll
+      for (int j = 0; j < S; ++j)
+        nxt[j] = *reinterpret_cast<const Pack<T, VEC> *>(xb + (size_t)min(t_begin + S + j, p.len - 1) * p.chans);
+    }
+#pragma unroll
+    for (int sidx = 0; sidx < S; ++sidx) {
+      float out[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float acc = bias[i];
+#pragma unroll
+        for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + sidx - m].v[i]), acc);
+        out[i] = p.silu ? silu_f32(acc) : acc;
+      }
+      if (t_begin + sidx < p.len) store_vec<T, VEC>(yb + (size_t)(t_begin + sidx) * p.chans, 0, out);
+    }
+    if (w + 1 < CONV_CL_WALK) {
+#pragma unroll
+      for (int j = 0; j < HIST; ++j) raw[j] = raw[S + j];
+#pragma unroll
+      for (int j = 0; j < S; ++j) raw[HIST + j] = nxt[j];
+    }
+  }
+}
+
 // --------------------------------------------------------------- backward, (B,C,L)
 
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
@@ -590,7 +662,12 @@ static int conv_fwd_typed(const ConvParams &p, int channels_last, bool vec_ok, h
     constexpr int VECF = CONV_CL_FWD_BYTES / sizeof(T);
     const size_t threads = (size_t)p.batch * strips * ((p.chans + VECF - 1) / VECF);
     const dim3 grid((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS));
-    if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_fwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
+    if (vec_ok && p.chans % VEC == 0 && p.len >= 2 * CONV_CL_WALK_STRIP * CONV_CL_WALK) {
+      const int spans = (p.len + CONV_CL_WALK_STRIP * CONV_CL_WALK - 1) / (CONV_CL_WALK_STRIP * CONV_CL_WALK);
+      const size_t walkers = (size_t)p.batch * spans * (p.chans / VECF);
+      const dim3 wgrid((unsigned)((walkers + CONV_CL_WALK_THREADS - 1) / CONV_CL_WALK_THREADS));
+      hipLaunchKernelGGL(conv_fwd_cl_walk_kernel<T>, wgrid, dim3(CONV_CL_WALK_THREADS), 0, s, p);
+    } else if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_fwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
     else hipLaunchKernelGGL((conv_fwd_cl_kernel<T, false>), grid, dim3(CONV_THREADS), 0, s, p);
   } else {
     const unsigned grid = (unsigned)min((size_t)65535 * 16, (total + CONV_THREADS - 1) / CONV_THREADS);
