@@ -87,7 +87,10 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
     // two rows per wave with 16-step runs and two slabs where 256 such workgroups exist, else 8-step runs at six waves
     // per SIMD, else the smallest workgroup.
     const size_t total = (size_t)a->batch * a->dim;
-    const int pref[3] = {22123, 12121, 11082};
+    // float32 activations: the 8-step runs at six waves per SIMD come out ahead (142.9 against 149.6 us at the
+    // headline shape, where twice the bytes per step leave more to wait for); 16-bit: the 16-step runs (120.5 / 133.3)
+    const int pref16[3] = {22123, 12121, 11082}, pref32[3] = {12121, 22123, 11082};
+    const int *pref = a->io_dtype == SSM_F32 ? pref32 : pref16;
     int pick = 0;
     for (int i = 0; i < 3 && !pick; ++i) {
       const int per_wg = scan_fwd_fast_rows(pref[i]);
