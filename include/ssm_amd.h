@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SSM_AMD_ABI_VERSION 6
+#define SSM_AMD_ABI_VERSION 7
 
 typedef enum ssm_status {
   SSM_OK = 0,
@@ -734,6 +734,132 @@ int ssm_norm_bwd(const ssm_norm_bwd_args *args, void *hip_stream);
  * while a stream is being captured. */
 #define SSM_NORM_BWD_STATIC_BYTES (8u << 20)
 int ssm_norm_bwd_static(const ssm_norm_bwd_args *args, void *hip_stream);
+
+/* -------------------------------------------------------------------------
+ * The five operators in double precision.
+ *
+ * The reference computes in the promoted type of its inputs (src/ssm/ops/python/reference.py:9-19, :135-137:
+ * float64 tensors, or a float64 `A`, make float64 the compute type) and runs torch.autograd.gradcheck in float64
+ * on the device against every operator of a compiled backend (tests/ops/test_backend_gradients.py:1172-1201
+ * selective_scan, :1291-1321 selective_state_step, :1416-1447 ssd_chunk_scan, :1497-1517 dw_causal_conv,
+ * :1578-1612 fused_layer_norm).  These entry points serve such calls: every tensor is `double`, all arithmetic is
+ * double, nothing is allocated, results are the same bits on every run.  They are plain kernels (one thread per
+ * independent recurrence), not tuned ones.
+ *
+ * Projections that the reference broadcasts are passed as views: a base pointer and element strides over the
+ * full index space, 0 on a broadcast axis.  Gradients of such operands are written dense over the full index
+ * space and summed over the broadcast axes by the caller; gradients of per-channel parameters are written as one
+ * row per batch entry (`*_rows`) and summed over the batch by the caller.  Each struct serves the forward and
+ * the backward entry; a forward call ignores the backward's fields.
+ * ---------------------------------------------------------------------- */
+typedef struct ssm_f64_scan_args {   /* reference.py:88-197 */
+  const double *u, *delta;           /* (B, D, L) */
+  const double *z;                   /* (B, D, L) or NULL */
+  const double *A;                   /* (D, N) */
+  const double *Bproj, *Cproj;       /* views over (B, D, N, L) */
+  const double *Dskip, *dt_bias;     /* (D,) or NULL */
+  double *out;                       /* (B, D, L) */
+  double *last_state;                /* (B, D, N): the final state; required (it is the running state); the backward
+                                        entry uses it as scratch */
+  int64_t b_stride[4], c_stride[4];  /* element strides of Bproj / Cproj over (B, D, N, L) */
+  /* backward */
+  const double *dout;                /* (B, D, L) */
+  const double *dlast_state;         /* (B, D, N) or NULL */
+  double *states;                    /* scratch (B, D, L, N) */
+  double *ypre;                      /* scratch (B, D, L) */
+  double *du, *ddelta;               /* (B, D, L) */
+  double *dz;                        /* (B, D, L); required with z */
+  double *dA_rows;                   /* (B, D, N) */
+  double *dB, *dC;                   /* dense (B, D, N, L) */
+  double *dD_rows, *dbias_rows;      /* (B, D) or NULL */
+  int32_t batch, dim, seqlen, nstate, delta_softplus;
+} ssm_f64_scan_args;
+int ssm_f64_scan_fwd(const ssm_f64_scan_args *args, void *hip_stream);
+int ssm_f64_scan_bwd(const ssm_f64_scan_args *args, void *hip_stream);
+
+typedef struct ssm_f64_step_args {   /* reference.py:200-312 */
+  double *state;                     /* (B, D, N): updated in place by the forward; the state before the step for the backward */
+  const double *x, *dt;              /* (B, D) */
+  const double *z;                   /* (B, D) or NULL */
+  const double *A;                   /* (D, N) */
+  const double *Bproj, *Cproj;       /* views over (B, D, N) */
+  const double *Dskip, *dt_bias;     /* (D,) or NULL */
+  double *out;                       /* (B, D) */
+  int64_t b_stride[3], c_stride[3];
+  /* backward */
+  const double *dout;                /* (B, D) or NULL */
+  const double *dstate_new;          /* (B, D, N) gradient of the updated state, or NULL */
+  double *dstate;                    /* (B, D, N) */
+  double *dx, *ddt;                  /* (B, D); ddt is also the bias gradient's rows */
+  double *dz;                        /* (B, D); required with z */
+  double *dA_rows, *dB, *dC;         /* (B, D, N) */
+  double *dD_rows;                   /* (B, D) or NULL */
+  int32_t batch, dim, nstate, dt_softplus;
+} ssm_f64_step_args;
+int ssm_f64_state_step(const ssm_f64_step_args *args, void *hip_stream);
+int ssm_f64_state_step_bwd(const ssm_f64_step_args *args, void *hip_stream);
+
+typedef struct ssm_f64_dscan_args {  /* reference.py:315-480 */
+  const double *X;                   /* (B, L, H, P) */
+  const double *dt;                  /* (B, L, H) */
+  const double *A;                   /* (H, P) */
+  const double *Bproj, *Cproj;       /* views over (B, L, H, P) */
+  const double *Dskip;               /* (H, P) or NULL */
+  const double *z;                   /* view over (B, L, H, P), or NULL */
+  const double *init;                /* (B, H, P) or NULL */
+  const int32_t *lengths;            /* (B,) valid steps per row, or NULL */
+  double *Y;                         /* (B, L, H, P) */
+  int64_t b_stride[4], c_stride[4], z_stride[4];
+  /* backward */
+  const double *dY;                  /* (B, L, H, P) */
+  double *states;                    /* scratch (B, L, H, P) */
+  double *dX, *ddt_rows, *dB, *dC;   /* dense (B, L, H, P); ddt_rows is summed over P by the caller */
+  double *dz;                        /* dense (B, L, H, P); required with z */
+  double *dA_rows;                   /* (B, H, P) */
+  double *dD_rows, *dinit;           /* (B, H, P) or NULL */
+  int32_t batch, seqlen, heads, hdim;
+} ssm_f64_dscan_args;
+int ssm_f64_dscan_fwd(const ssm_f64_dscan_args *args, void *hip_stream);
+int ssm_f64_dscan_bwd(const ssm_f64_dscan_args *args, void *hip_stream);
+
+typedef struct ssm_f64_conv_args {   /* reference.py:483-533 */
+  const double *x;                   /* view over (B, C, L): either layout */
+  const double *weight;              /* (C, K) */
+  const double *bias;                /* (C,) or NULL */
+  double *y;                         /* view over (B, C, L) */
+  int64_t x_stride[3], y_stride[3];
+  /* backward */
+  const double *dy;                  /* view over (B, C, L) */
+  double *dx;                        /* view over (B, C, L) */
+  int64_t dy_stride[3], dx_stride[3];
+  double *dpre;                      /* scratch, dense (B, C, L) */
+  double *dw;                        /* (C, K) */
+  double *db;                        /* (C,) or NULL */
+  int32_t batch, channels, seqlen, width, activation;   /* ssm_activation */
+} ssm_f64_conv_args;
+int ssm_f64_conv_fwd(const ssm_f64_conv_args *args, void *hip_stream);
+int ssm_f64_conv_bwd(const ssm_f64_conv_args *args, void *hip_stream);
+
+typedef struct ssm_f64_norm_args {   /* reference.py:536-609 */
+  const double *x;                   /* (rows, hidden) */
+  const double *residual;            /* (rows, hidden) or NULL */
+  const double *weight;              /* (hidden,) */
+  const double *bias;                /* (hidden,) or NULL */
+  double *y;                         /* (rows, hidden) */
+  double *residual_out;              /* (rows, hidden) or NULL: x (+ residual if prenorm) */
+  double *mean, *rstd;               /* (rows,): written by the forward, read by the backward */
+  /* backward */
+  const double *dy;                  /* (rows, hidden) */
+  double *dx;                        /* (rows, hidden) */
+  double *dresidual;                 /* (rows, hidden) or NULL */
+  double *dw;                        /* (hidden,) */
+  double *db;                        /* (hidden,) or NULL */
+  int64_t rows;
+  int32_t hidden, is_rms, prenorm;
+  double eps;
+} ssm_f64_norm_args;
+int ssm_f64_norm_fwd(const ssm_f64_norm_args *args, void *hip_stream);
+int ssm_f64_norm_bwd(const ssm_f64_norm_args *args, void *hip_stream);
 
 #ifdef __cplusplus
 }

@@ -19,7 +19,7 @@ import os
 # SSM_AMD_LIB points the binding at another build of the same C ABI.
 LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
                 Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
 PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
@@ -271,6 +271,57 @@ class NormBwdArgs(C.Structure):
 
 
 # name -> argument struct (every entry point is ``int f(const args*, void* stream)``)
+_pd, _f64 = C.c_void_p, C.c_double
+
+
+class F64ScanArgs(C.Structure):
+    _fields_ = [
+        ("u", _pd), ("delta", _pd), ("z", _pd), ("A", _pd), ("Bproj", _pd), ("Cproj", _pd), ("Dskip", _pd),
+        ("dt_bias", _pd), ("out", _pd), ("last_state", _pd), ("b_stride", _i64 * 4), ("c_stride", _i64 * 4),
+        ("dout", _pd), ("dlast_state", _pd), ("states", _pd), ("ypre", _pd), ("du", _pd), ("ddelta", _pd),
+        ("dz", _pd), ("dA_rows", _pd), ("dB", _pd), ("dC", _pd), ("dD_rows", _pd), ("dbias_rows", _pd),
+        ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32), ("delta_softplus", _i32),
+    ]
+
+
+class F64StepArgs(C.Structure):
+    _fields_ = [
+        ("state", _pd), ("x", _pd), ("dt", _pd), ("z", _pd), ("A", _pd), ("Bproj", _pd), ("Cproj", _pd),
+        ("Dskip", _pd), ("dt_bias", _pd), ("out", _pd), ("b_stride", _i64 * 3), ("c_stride", _i64 * 3),
+        ("dout", _pd), ("dstate_new", _pd), ("dstate", _pd), ("dx", _pd), ("ddt", _pd), ("dz", _pd),
+        ("dA_rows", _pd), ("dB", _pd), ("dC", _pd), ("dD_rows", _pd),
+        ("batch", _i32), ("dim", _i32), ("nstate", _i32), ("dt_softplus", _i32),
+    ]
+
+
+class F64DscanArgs(C.Structure):
+    _fields_ = [
+        ("X", _pd), ("dt", _pd), ("A", _pd), ("Bproj", _pd), ("Cproj", _pd), ("Dskip", _pd), ("z", _pd),
+        ("init", _pd), ("lengths", _pd), ("Y", _pd),
+        ("b_stride", _i64 * 4), ("c_stride", _i64 * 4), ("z_stride", _i64 * 4),
+        ("dY", _pd), ("states", _pd), ("dX", _pd), ("ddt_rows", _pd), ("dB", _pd), ("dC", _pd), ("dz", _pd),
+        ("dA_rows", _pd), ("dD_rows", _pd), ("dinit", _pd),
+        ("batch", _i32), ("seqlen", _i32), ("heads", _i32), ("hdim", _i32),
+    ]
+
+
+class F64ConvArgs(C.Structure):
+    _fields_ = [
+        ("x", _pd), ("weight", _pd), ("bias", _pd), ("y", _pd), ("x_stride", _i64 * 3), ("y_stride", _i64 * 3),
+        ("dy", _pd), ("dx", _pd), ("dy_stride", _i64 * 3), ("dx_stride", _i64 * 3), ("dpre", _pd), ("dw", _pd),
+        ("db", _pd),
+        ("batch", _i32), ("channels", _i32), ("seqlen", _i32), ("width", _i32), ("activation", _i32),
+    ]
+
+
+class F64NormArgs(C.Structure):
+    _fields_ = [
+        ("x", _pd), ("residual", _pd), ("weight", _pd), ("bias", _pd), ("y", _pd), ("residual_out", _pd),
+        ("mean", _pd), ("rstd", _pd), ("dy", _pd), ("dx", _pd), ("dresidual", _pd), ("dw", _pd), ("db", _pd),
+        ("rows", _i64), ("hidden", _i32), ("is_rms", _i32), ("prenorm", _i32), ("eps", _f64),
+    ]
+
+
 ENTRY_POINTS = {
     "ssm_scan_fwd": ScanFwdArgs,
     "ssm_scan_bwd": ScanBwdArgs,
@@ -301,6 +352,16 @@ ENTRY_POINTS = {
     "ssm_norm_fwd": NormFwdArgs,
     "ssm_norm_bwd": NormBwdArgs,
     "ssm_norm_bwd_static": NormBwdArgs,
+    "ssm_f64_scan_fwd": F64ScanArgs,
+    "ssm_f64_scan_bwd": F64ScanArgs,
+    "ssm_f64_state_step": F64StepArgs,
+    "ssm_f64_state_step_bwd": F64StepArgs,
+    "ssm_f64_dscan_fwd": F64DscanArgs,
+    "ssm_f64_dscan_bwd": F64DscanArgs,
+    "ssm_f64_conv_fwd": F64ConvArgs,
+    "ssm_f64_conv_bwd": F64ConvArgs,
+    "ssm_f64_norm_fwd": F64NormArgs,
+    "ssm_f64_norm_bwd": F64NormArgs,
 }
 # name -> (restype, argtypes) of the remaining exported functions
 PLAIN_SYMBOLS = {

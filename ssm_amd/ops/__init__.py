@@ -56,6 +56,13 @@ class ScanPlan:
         batch, dim, length, nstate, (bkind, bgroups), (ckind, cgroups) = \
             K.check_selective_scan(u, delta, A, B, C, D, z, dt_bias)
         self.device = K.require_gpu(u, delta, A, B, C, D, z, dt_bias)
+        self.result_dtype = u.dtype
+        self.chunk_states = None
+        self.f64 = None
+        if K.f64_compute(u, A):           # computed in double precision by kernels of their own
+            self.f64 = (u, delta, A, B, C, D, z, dt_bias, softplus, want_state)
+            return
+        u, delta, A, B, C, D, z, dt_bias = K.narrow(u, delta, A, B, C, D, z, dt_bias)
         io = K.common_io_dtype([u, delta, z])
         bc = K.common_io_dtype([B, C])
         self.result_dtype = u.dtype
@@ -84,6 +91,9 @@ class ScanPlan:
             delta_softplus=int(bool(softplus)), reserved=int(tune_items))
 
     def run(self):
+        if self.f64 is not None:
+            from . import _f64
+            return _f64.scan_forward(*self.f64)
         _lib.call("ssm_scan_fwd", self.args, self.device)
         return self.out, self.last
 
@@ -135,6 +145,8 @@ def _scan_forward(u, delta, A, B, C, D, z, dt_bias, softplus, want_state, tune_i
             return again[0], again[1]
     plan = ScanPlan(u, delta, A, B, C, D, z, dt_bias, softplus, want_state, tune_items)
     out, last = plan.run()
+    if plan.f64 is not None:
+        return out, last
     if not tune_items and plan.chunk_states is None and len(_SCAN_FORMS) < 256:
         # remembered under the key that _scan_forward_again forms from the caller's tensors: only a call whose
         # tensors went in as they were (no cast, no copy) can be repeated through it
@@ -170,6 +182,10 @@ def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softpl
     ``(du, ddelta, dA, dB, dC, dD, dz, ddt_bias)``.  State sizes above 16 are
     processed in blocks of 16 states (the recurrence is independent per state and
     every gradient is additive over states)."""
+    if K.f64_compute(u, A):
+        from . import _f64
+        return _f64.scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softplus)
+    u, delta, A, B, C, D, z, dt_bias = K.narrow(u, delta, A, B, C, D, z, dt_bias)
     batch, dim, length, nstate, (bkind, bgroups), (ckind, cgroups) = \
         K.check_selective_scan(u, delta, A, B, C, D, z, dt_bias)
     dev = K.require_gpu(u, delta, A, B, C, D, z, dt_bias, grad_out)
@@ -295,6 +311,12 @@ class StepPlan:
         batch, dim, nstate, (bkind, bgroups), (ckind, cgroups) = \
             K.check_state_step(state, x, dt, A, B, C, D, z, dt_bias)
         self.device = K.require_gpu(state, x, dt, A, B, C, D, z, dt_bias)
+        self.result_dtype = x.dtype
+        self.f64 = None
+        if K.f64_compute(state, A):       # computed in double precision by kernels of their own
+            self.f64 = (state, x, dt, A, B, C, D, z, dt_bias, softplus)
+            return
+        x, dt, A, B, C, D, z, dt_bias = K.narrow(x, dt, A, B, C, D, z, dt_bias)
         if not state.is_contiguous():
             raise ValueError("state must be contiguous to be updated in place")
         io = K.common_io_dtype([x, dt, z])
@@ -320,6 +342,9 @@ class StepPlan:
             dt_softplus=int(bool(softplus)), z_batch_stride=z_bs, b_batch_stride=b_bs, c_batch_stride=c_bs)
 
     def run(self):
+        if self.f64 is not None:
+            from . import _f64
+            return _f64.state_step(*self.f64)
         _lib.call("ssm_state_step", self.args, self.device)
         return self.out
 
@@ -343,6 +368,10 @@ def _state_step_backward(grad_out, grad_state, state, x, dt, A, B, C, D, z, dt_b
     ``(state, x, dt, A, B, C, D, z, dt_bias)``.  ``state`` is the state before the step;
     ``grad_out`` / ``grad_state`` (gradient of the updated state) may be ``None``.
     Parameter gradients come back in float32, the others in the dtype of their tensor."""
+    if K.f64_compute(state, A):
+        from . import _f64
+        return _f64.state_step_backward(grad_out, grad_state, state, x, dt, A, B, C, D, z, dt_bias, softplus)
+    x, dt, A, B, C, D, z, dt_bias = K.narrow(x, dt, A, B, C, D, z, dt_bias)
     batch, dim, nstate, (bkind, bgroups), (ckind, cgroups) = \
         K.check_state_step(state, x, dt, A, B, C, D, z, dt_bias)
     dev = K.require_gpu(state, x, dt, A, B, C, D, z, dt_bias, grad_out, grad_state)
@@ -583,6 +612,11 @@ def _dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states, wa
     returns ``(Y, round_states)``: the state entering every 64 steps, ``(B, ceil(L/64), H*P)`` float32, which
     :func:`_dscan_backward` takes instead of sweeping forward itself -- or ``None`` when the call does not run the
     kernel that can write it."""
+    if K.f64_compute(X, A):
+        from . import _f64
+        Y = _f64.dscan_forward(X, dt, A, B, C, chunk_size, D, z, lengths, initial_states)
+        return (Y, None) if want_round_states else Y
+    dt, A, B, C, D, z, initial_states = K.narrow(dt, A, B, C, D, z, initial_states)
     batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p = \
         K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
     dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states)
@@ -620,6 +654,10 @@ def _dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_s
     tensors' own types (no float32 copy of a tensor of ``X``'s size is made and converted afterwards).
     ``two_kernels`` keeps the general path for a call the one-pass kernels cover; ``round_states`` is what
     :func:`_dscan_forward` returned for the same inputs (or ``None``)."""
+    if K.f64_compute(X, A):
+        from . import _f64
+        return _f64.dscan_backward(grad_y, X, dt, A, B, C, chunk_size, D, z, lengths, initial_states)
+    dt, A, B, C, D, z, initial_states = K.narrow(dt, A, B, C, D, z, initial_states)
     batch, seqlen, heads, proj, a_per_p, bk, ck, d_per_p, z_per_p = \
         K.check_chunk_scan(X, dt, A, B, C, chunk_size, D, z, initial_states)
     dev = K.require_gpu(X, dt, A, B, C, D, z, initial_states, grad_y)
@@ -710,6 +748,10 @@ def _conv_weight_f32(weight):
 
 
 def _conv_forward(x, weight, bias, activation, channels_last=None):
+    if K.f64_compute(x):
+        from . import _f64
+        return _f64.conv_forward(x, weight, bias, activation, channels_last)
+    weight, bias = K.narrow(weight, bias)
     batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation, channels_last)
     dev = K.require_gpu(x, weight, bias)
     xc = K.cast_c(x, x.dtype)
@@ -726,6 +768,10 @@ def _conv_forward(x, weight, bias, activation, channels_last=None):
 
 def _conv_backward(grad_out, x, weight, bias, activation, channels_last=None):
     """-> (dx, dweight (C,K) fp32, dbias (C,) fp32 or None)."""
+    if K.f64_compute(x):
+        from . import _f64
+        return _f64.conv_backward(grad_out, x, weight, bias, activation, channels_last)
+    weight, bias = K.narrow(weight, bias)
     batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation, channels_last)
     dev = K.require_gpu(x, weight, bias, grad_out)
     xc, gc = K.cast_c(x, x.dtype), K.cast_c(grad_out, x.dtype)
@@ -781,6 +827,10 @@ def _dw_causal_conv(x, weight, bias, activation, channels_last):
 
 def _norm_forward(x, weight, bias, residual, is_rms, eps, prenorm, residual_in_fp32,
                   want_residual_out=False, want_stats=False):
+    if K.f64_compute(x):
+        from . import _f64
+        return _f64.norm_forward(x, weight, bias, residual, is_rms, eps, prenorm, want_residual_out)
+    weight, bias, residual = K.narrow(weight, bias, residual)
     rows, hidden = K.check_norm(x, weight, bias, residual)
     dev = K.require_gpu(x, weight, bias, residual)
     xc = K.cast_c(x, x.dtype)
@@ -814,6 +864,12 @@ def _norm_backward(grad_out, x, weight, residual, mean, rstd, is_rms, prenorm, w
     """``ssm_norm_bwd``.  With ``out = (dx, dres, dw, db)`` (preallocated, contiguous; ``None`` where a
     gradient is not wanted) the call goes to ``ssm_norm_bwd_static`` instead and allocates nothing on
     the device: inputs must then already be contiguous and ``weight`` float32."""
+    if K.f64_compute(x):
+        if out is not None:
+            raise ValueError("the allocation-free norm backward takes float32, bfloat16 or float16 tensors")
+        from . import _f64
+        return _f64.norm_backward(grad_out, x, weight, residual, mean, rstd, is_rms, prenorm, want_dbias, want_dres)
+    weight, residual = K.narrow(weight, residual)
     rows, hidden = K.check_norm(x, weight, None, residual)
     if out is not None:
         dev = K.require_gpu(x, weight, residual, grad_out)

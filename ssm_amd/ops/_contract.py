@@ -12,7 +12,7 @@ from typing import Iterable, Optional
 
 import torch
 
-SUPPORTED = (torch.float32, torch.bfloat16, torch.float16)
+SUPPORTED = (torch.float32, torch.bfloat16, torch.float16, torch.float64)
 
 
 class DeviceError(RuntimeError):
@@ -45,8 +45,27 @@ def require_gpu(*tensors: Optional[torch.Tensor]) -> torch.device:
 def check_float(name: str, t: torch.Tensor) -> None:
     if t.dtype not in SUPPORTED:
         raise ValueError(
-            f"{name} has dtype {t.dtype}; the HIP backend supports float32, bfloat16 and float16 "
-            "(accumulation is always float32).")
+            f"{name} has dtype {t.dtype}; the HIP backend supports float32, bfloat16, float16 "
+            "(accumulated in float32) and float64 (computed in float64).")
+
+
+def f64_compute(primary: torch.Tensor, A: Optional[torch.Tensor] = None) -> bool:
+    """Whether the reference would compute this call in float64: the compute type is the primary tensor's
+    (16-bit types widen to float32), promoted with ``A``'s when ``A`` is not float32
+    (src/ssm/ops/python/reference.py:9-19, :135-137).  Complex tensors are not supported."""
+    for t in (primary, A):
+        if t is not None and t.is_complex():
+            raise ValueError("complex tensors are not supported by the HIP backend.")
+    ct = torch.float32 if primary.dtype in (torch.float16, torch.bfloat16) else primary.dtype
+    if A is not None and A.dtype != torch.float32 and A.dtype != ct:
+        ct = torch.promote_types(torch.float32 if A.dtype in (torch.float16, torch.bfloat16) else A.dtype, ct)
+    return ct == torch.float64
+
+
+def narrow(*tensors: Optional[torch.Tensor]):
+    """Float64 tensors of a call that computes in float32 (the reference casts every operand to the compute
+    type, reference.py:139-160), as float32."""
+    return tuple(t.to(torch.float32) if (t is not None and t.dtype == torch.float64) else t for t in tensors)
 
 
 def common_io_dtype(tensors: Iterable[Optional[torch.Tensor]]) -> torch.dtype:

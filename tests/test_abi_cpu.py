@@ -63,7 +63,10 @@ def test_ctypes_struct_sizes_match_the_header(tmp_path):
              "SsdBwdGateArgs": "ssm_ssd_bwd_gate_args", "SsdBwdDxArgs": "ssm_ssd_bwd_dx_args",
              "SsdBwdDbArgs": "ssm_ssd_bwd_db_args", "SsdBwdDcbArgs": "ssm_ssd_bwd_dcb_args",
              "SsdBwdStatesArgs": "ssm_ssd_bwd_states_args", "SsdScaleRowsArgs": "ssm_ssd_scale_rows_args",
-             "SsdBwdDtArgs": "ssm_ssd_bwd_dt_args", "SsdBwdPrepArgs": "ssm_ssd_bwd_prep_args"}
+             "SsdBwdDtArgs": "ssm_ssd_bwd_dt_args", "SsdBwdPrepArgs": "ssm_ssd_bwd_prep_args",
+             "F64ScanArgs": "ssm_f64_scan_args", "F64StepArgs": "ssm_f64_step_args",
+             "F64DscanArgs": "ssm_f64_dscan_args", "F64ConvArgs": "ssm_f64_conv_args",
+             "F64NormArgs": "ssm_f64_norm_args"}
     assert set(structs) <= set(cname), set(structs) - set(cname)
     src = tmp_path / "sizes.c"
     lines = ['#include <stdio.h>', f'#include "{HEADER}"', "int main(void) {"]

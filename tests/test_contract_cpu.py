@@ -89,7 +89,22 @@ def test_selective_scan_contract_errors():
     with pytest.raises(ValueError):
         ops.selective_scan(u, u, A, Bm, Bm, dt_bias=torch.ones(5))
     with pytest.raises(ValueError):
-        ops.selective_scan(u.double(), u.double(), A, Bm, Bm)          # unsupported dtype
+        ops.selective_scan(u, u, torch.complex(A, A), Bm, Bm)         # complex tensors: not supported
+    with pytest.raises(ValueError):
+        ops.selective_scan(u.to(torch.int32), u, A, Bm, Bm)           # not a floating type
+
+
+def test_compute_type_follows_the_reference():
+    """reference.py:9-19, :135-137: the primary tensor's type, 16-bit widened to float32, promoted with A's when
+    A is not float32; every other operand is cast to it."""
+    from ssm_amd.ops import _contract as K
+    f16, bf, f32, f64 = torch.float16, torch.bfloat16, torch.float32, torch.float64
+    t = lambda dt: torch.zeros(1, dtype=dt)
+    assert not K.f64_compute(t(f32)) and not K.f64_compute(t(bf), t(f32)) and not K.f64_compute(t(f16), t(f16))
+    assert K.f64_compute(t(f64)) and K.f64_compute(t(f64), t(f32))
+    assert K.f64_compute(t(f32), t(f64)) and K.f64_compute(t(bf), t(f64))
+    a, b, c = K.narrow(t(f64), None, t(bf))
+    assert a.dtype == f32 and b is None and c.dtype == bf
 
 
 def test_state_step_contract_errors():
