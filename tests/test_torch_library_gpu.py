@@ -117,3 +117,39 @@ def test_registrations_pass_opcheck():
     xn = torch.randn(3, 5, 96, generator=gen).cuda().requires_grad_(True)
     wn = torch.randn(96, generator=gen).cuda().requires_grad_(True)
     torch.library.opcheck(torch.ops.ssm_amd.fused_layer_norm.default, (xn, wn, None, None, True), test_utils=CHECKS)
+
+
+def test_a_traced_graph_holds_one_node_per_operator_call():
+    """What the registration is for (the reference's ``TORCH_LIBRARY`` block, src/ssm/ops/cpu/bindings.cpp:151-189):
+    a function that calls the operators traces into a graph with one opaque node per call, forward and backward,
+    and the compiled function gives the eager results."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 24, 100, generator=gen).cuda().requires_grad_(True)
+    wt = torch.randn(24, 4, generator=gen).cuda().requires_grad_(True)
+    delta = torch.randn(2, 24, 100, generator=gen).cuda().requires_grad_(True)
+    A = (-(torch.rand(24, 8, generator=gen) + 0.5)).cuda().requires_grad_(True)
+    Bm = torch.randn(2, 1, 8, 100, generator=gen).cuda().requires_grad_(True)
+    Cm = torch.randn(2, 1, 8, 100, generator=gen).cuda().requires_grad_(True)
+    wn = torch.randn(24, generator=gen).cuda().requires_grad_(True)
+
+    def block(x, wt, delta, A, Bm, Cm, wn):
+        h = torch.ops.ssm_amd.dw_causal_conv(x, wt, None, "silu")
+        y, _ = torch.ops.ssm_amd.selective_scan(h, delta, A, Bm, Cm, None, None, None, True, False)
+        return torch.ops.ssm_amd.fused_layer_norm(y.transpose(1, 2), wn, None, None, True)
+
+    args = (x, wt, delta, A, Bm, Cm, wn)
+    graph = make_fx(block, tracing_mode="fake")(*args)
+    targets = [n.target for n in graph.graph.nodes if n.op == "call_function"]
+    for op in (torch.ops.ssm_amd.dw_causal_conv.default, torch.ops.ssm_amd.selective_scan.default,
+               torch.ops.ssm_amd.fused_layer_norm.default):
+        assert targets.count(op) == 1, targets
+
+    eager = block(*args)
+    grads = torch.autograd.grad(eager.square().sum(), args)
+    compiled = torch.compile(block, backend="aot_eager", fullgraph=True)
+    out = compiled(*args)
+    assert torch.equal(out, eager)
+    for a, b in zip(torch.autograd.grad(out.square().sum(), args), grads):
+        assert torch.equal(a, b)
