@@ -167,6 +167,34 @@ def bench_scan_bwd(dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nstate=
             "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes}
 
 
+def bench_mixer_config1(dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nstate=16, width=4):
+    """BASELINE configuration 1 as one step: depthwise causal conv (width 4, SiLU) -> selective scan (per-token
+    B/C, z gate, D skip, bias + softplus), forward and backward through autograd with a random upstream gradient,
+    gradients for x, the conv weights, delta, A, B, C, D and the bias."""
+    from ssm_amd import configs, ops
+
+    inp = configs.to_device(configs.scan_inputs(batch, dim, length, nstate, dtype=dtype, seed=0))
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(batch, dim, length, generator=g).to(dtype).cuda().requires_grad_()
+    w = (torch.rand(dim, width, generator=g) - 0.5).cuda().requires_grad_()
+    b = (torch.randn(dim, generator=g) * 0.02).cuda().requires_grad_()
+    go = torch.randn(batch, dim, length, generator=g).to(dtype).cuda()
+    leaves = [x, w, b] + [inp[k].requires_grad_() for k in ("delta", "A", "B", "C", "D", "dt_bias")]
+
+    def step(_):
+        u = ops.dw_causal_conv(x, w, b, activation="silu")
+        y = ops.selective_scan(u, inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                               dt_bias=inp["dt_bias"], softplus=True)
+        y.backward(go)
+        for t in leaves:
+            t.grad = None
+
+    us = _time_us(step, iters=20, warmup=30)
+    return {"fwd_bwd_us": round(us, 1), "tokens_per_s": round(batch * length / us * 1e6, 1),
+            "shape": f"B={batch} D={dim} L={length} N={nstate} K={width} {str(dtype).split('.')[-1]}: conv + scan, "
+                     "forward + backward through autograd"}
+
+
 def bench_conv(dtype=torch.bfloat16, batch=8, chans=1536, length=2048, width=4):
     from ssm_amd import ops
 
@@ -598,7 +626,7 @@ def main():
                     help="also run a plain 256 MiB elementwise copy (dst = src + 0) three times: "
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
-                    choices=["scan_bwd", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1",
+                    choices=["scan_bwd", "mixer", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1",
                              "scan_facade", "scan_per_channel_bc", "stream"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
@@ -624,7 +652,7 @@ def main():
 
     if args.only:
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
-              "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model,
+              "mixer": bench_mixer_config1, "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model,
               "model1": bench_model1, "scan_facade": bench_scan_facade,
               "scan_per_channel_bc": bench_scan_per_channel_bc, "stream": bench_stream}[args.only]
         bench_scan_fwd(1, 0)            # the untimed spin-up of the default run, so that figures compare
@@ -679,6 +707,7 @@ def main():
         extra["selective_scan_fwd_through_ops_entry"] = bench_scan_facade()
         extra["selective_scan_fwd_per_channel_bc"] = bench_scan_per_channel_bc()
         extra["selective_scan_bwd_bf16"] = bench_scan_bwd()
+        extra["mamba1_mixer_config1_fwd_bwd"] = bench_mixer_config1()
         extra["dw_causal_conv_bf16"] = bench_conv()
         extra["fused_add_rmsnorm"] = bench_norm()
         extra["decode_step_config2"] = bench_decode()

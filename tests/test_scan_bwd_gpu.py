@@ -313,3 +313,48 @@ def test_a_wave_that_gives_up_its_wait_poisons_dB_and_dC():
             assert not bool(torch.isnan(a).any())
         else:
             assert torch.equal(a, b), k
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_conv_then_scan_forward_and_backward(dtype):
+    """The step that configuration 1 times (conv, SiLU, scan with gate, skip and softplus; forward and backward
+    through autograd) on a shape the oracle differentiates in seconds: gradients reach the conv's input, taps
+    and bias through the scan's gradient of ``u``."""
+    ops = _ops()
+    inp = make_inputs(21, 2, 32, 300, 16, dtype=dtype)
+    g = torch.Generator().manual_seed(22)
+    x = torch.randn(2, 32, 300, generator=g).to(dtype)
+    w, b = torch.rand(32, 4, generator=g) - 0.5, torch.randn(32, generator=g) * 0.02
+    go = torch.randn(2, 32, 300, generator=g).to(dtype)
+    names = ("x", "w", "b") + tuple(k for k in NAMES if k != "u")
+
+    def run(where, acc):
+        # the float64 value of the chain: the same inputs widened, so that nothing in between is rounded to float32
+        put = (lambda t: t.cuda()) if where == "gpu" else ((lambda t: t.double()) if acc is not None else (lambda t: t))
+        lv = dict(x=x, w=w, b=b, **{k: inp[k] for k in NAMES if k != "u"})
+        lv = {k: put(v.detach().clone()).requires_grad_(True) for k, v in lv.items()}
+        if where == "gpu":
+            u = ops.dw_causal_conv(lv["x"], lv["w"], lv["b"], activation="silu")
+            y = ops.selective_scan(u, lv["delta"], lv["A"], lv["B"], lv["C"], D=lv["D"], z=lv["z"],
+                                   dt_bias=lv["dt_bias"], softplus=True)
+        else:
+            u = O.dw_causal_conv(lv["x"], lv["w"], lv["b"], activation="silu")
+            y = O.selective_scan(u, lv["delta"], lv["A"], lv["B"], lv["C"], D=lv["D"], z=lv["z"],
+                                 dt_bias=lv["dt_bias"], softplus=True)
+        y.backward(put(go).to(y.dtype))
+        return y.detach().cpu(), {k: lv[k].grad.detach().cpu() for k in names}
+
+    y, got = run("gpu", None)
+    from tests.closeness import fp32_close, half_close
+    if dtype == torch.float32:
+        y64, want64 = run("cpu", torch.float64)
+        y32, want32 = run("cpu", None)
+        fp32_close(y, y64, y32, what="y")
+        for k in names:
+            fp32_close(got[k], want64[k], want32[k], what=f"grad {k}")
+    else:
+        # the 16-bit path rounds the conv's output once before the scan reads it, as the oracle's chain does
+        yr, want = run("cpu", None)
+        half_close(y, yr, what="y")
+        for k in names:
+            half_close(got[k], want[k], what=f"grad {k}", atol_rms=4e-2, mean_rms=5e-3)
