@@ -797,9 +797,9 @@ extern "C" int ssm_ssd_combined_fwd(const ssm_ssd_combined_args *a, void *hip_st
               "ssm_ssd_combined_fwd: workspace of %zu bytes required", lay.total);
   SSM_REQUIRE(aligned_to(a->x, 16) && aligned_to(a->y, 16) && (!a->z || aligned_to(a->z, 16)) && aligned_to(a->Bm, 16) &&
                   aligned_to(a->Cm, 16) && aligned_to(a->workspace, 256) &&
-                  (!a->Dskip || aligned_to(a->Dskip, 16)) && (!a->final_states || aligned_to(a->final_states, 16)) &&
+                  (!a->Dskip || aligned_to(a->Dskip, a->d_per_p ? 16 : 4)) && (!a->final_states || aligned_to(a->final_states, 16)) &&
                   (!a->initial_states || aligned_to(a->initial_states, 4)),
-              SSM_ERR_ALIGNMENT, "ssm_ssd_combined_fwd: tensors must be 16-byte aligned (workspace 256)");
+              SSM_ERR_ALIGNMENT, "ssm_ssd_combined_fwd: tensors must be 16-byte aligned (workspace 256; a per-head Dskip 4)");
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
   unsigned char *ws = reinterpret_cast<unsigned char *>(a->workspace);
 

@@ -408,6 +408,8 @@ def _ssd_fused(x, dt, A, B, C, Q, D, z, dt_bias, initial_states, dt_softplus, dt
     dtc = K.cast_c(dt, dt.dtype)
     K.check_float("dt", dtc)
     Af, Df, bf, init = K.as_f32_vec(A), K.as_f32_vec(D), K.as_f32_vec(dt_bias), K.as_f32_vec(initial_states)
+    if d_per_p and Df.data_ptr() % 16:          # a view into a larger buffer: the kernel reads (H, P) factors as 16-byte vectors
+        Df = Df.clone()
     dims = _dims(batch, seqlen, heads, hdim, groups, nstate, Q)
     nbytes = int(_lib.load().ssm_ssd_combined_workspace_bytes(dims))
     work = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)

@@ -560,6 +560,26 @@ def test_one_pass_matches_oracle_and_five_kernel_path(shape, Q, d_mat, use_z, us
     half_close(fin, fin5, "final states, one pass against five kernels")
 
 
+@pytest.mark.parametrize("d_mat", [False, True], ids=["per-head", "per-channel"])
+def test_one_pass_takes_parameters_that_are_views_into_larger_buffers(d_mat):
+    """``A``, ``D`` and the bias of a few heads cut out of a model's parameter vectors start at any 4-byte offset."""
+    b, l, h, p, g, n, Q = 1, 256, 3, 64, 1, 64, 128
+    inp = make(41, b, l, h, p, g, n, dtype=torch.bfloat16, d_mat=d_mat, use_z=True, use_init=False)
+
+    def view(t):                      # the same values one float32 into a larger buffer: not 16-byte aligned
+        buf = torch.zeros(t.numel() + 1, device="cuda")
+        buf[1:] = cu(t).reshape(-1)
+        v = buf[1:].view(t.shape)
+        assert v.data_ptr() % 16 == 4
+        return v
+
+    args = (cu(inp["x"]), cu(inp["dt"]), view(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q)
+    y = ssd().ssd_combined(*args, D=view(inp["D"]), z=cu(inp["z"]), fused=True)
+    want = ssd().ssd_combined(cu(inp["x"]), cu(inp["dt"]), cu(inp["A"]), cu(inp["B"]), cu(inp["C"]), Q, D=cu(inp["D"]),
+                              z=cu(inp["z"]), fused=True)
+    assert torch.equal(y, want)
+
+
 def test_one_pass_dt_bias_softplus_and_clamp():
     b, l, h, p, g, n, Q = 2, 256, 4, 64, 1, 64, 128
     inp = make(5, b, l, h, p, g, n, dtype=torch.bfloat16, use_init=False)
