@@ -114,6 +114,8 @@ def _scan_forward_again(u, delta, A, B, C, D, z, dt_bias, softplus, want_state):
     for t, want in ((D, _F32), (z, dt), (dt_bias, _F32)):
         if t is not None and not (t.dtype == want and t.is_contiguous()):
             return None
+    if (u.data_ptr() | delta.data_ptr() | B.data_ptr() | C.data_ptr() | (0 if z is None else z.data_ptr())) & 15:
+        return None                      # a view off the 16-byte grid: the long way copies it
     dev = u.device
     key = (u.shape, dt, delta.shape, A.shape, B.shape, B.dtype, C.shape, None if D is None else D.shape,
            None if z is None else z.shape, None if dt_bias is None else dt_bias.shape, bool(softplus),

@@ -82,12 +82,17 @@ def as_f32_vec(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
 
 
 def cast_c(t: Optional[torch.Tensor], dt: torch.dtype) -> Optional[torch.Tensor]:
+    """``t`` as the kernels take an input: detached, of type ``dt``, contiguous and starting on a 16-byte boundary
+    (a contiguous view that starts elsewhere in a larger buffer is copied: the vector accesses of the fast kernels
+    need the boundary, and a copy costs less than the element-wise kernels would)."""
     if t is None:
         return None
     t = t.detach()
     if t.dtype != dt:
         t = t.to(dt)
-    return t if t.is_contiguous() else t.contiguous()
+    if not t.is_contiguous():
+        t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
 # ----------------------------------------------------------- selective scan

@@ -961,8 +961,10 @@ def ssd_combined_backward(dout, dfinal, x, dt, A, B, C, chunk_size, D=None, z=No
     f32 = torch.float32
     Af = A.detach().to(f32)
     fused = _elem_stages_ok(x, dout, z, hdim)
-    xd, dod = x.detach().contiguous(), dout.detach().contiguous()
-    zd = None if z is None else z.detach().contiguous()
+    # (dense, 16-byte aligned: a view that starts elsewhere in a larger buffer is copied once, here)
+    xd, dod = K.cast_c(x, x.dtype), K.cast_c(dout, dout.dtype)
+    zd = None if z is None else K.cast_c(z, z.dtype)
+    B, C = K.cast_c(B, B.dtype), K.cast_c(C, C.dtype)
     xf = None if fused else xd.to(f32)
     dof = None if fused else dod.to(f32)
     # The passes take their operands in the inputs' precision when that is bfloat16 (matrix-core kernels,
