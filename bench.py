@@ -498,8 +498,18 @@ def bench_scan_per_channel_bc(dtype=torch.bfloat16, batch=8, dim=1536, length=20
     us = _time_us(lambda i: plan.run(), iters=10)
     elt = 2 if dtype != torch.float32 else 4
     nbytes = configs.scan_fwd_bytes(batch, dim, length, nstate, elt, groups=dim)
+    # backward of the same call (a wave per row; dB and dC written straight to their place in B's own type)
+    from ssm_amd.ops import _scan_backward
+    cs_plan = ScanPlan(g["u"], g["delta"], g["A"], Bm, Cm, g["D"], g["z"], g["dt_bias"], True, False, want_chunk_states=True)
+    cs_plan.run()
+    go = torch.randn(batch, dim, length, generator=gen, device="cuda", dtype=torch.float32).to(dtype)
+    bus = _time_us(lambda i: _scan_backward(go, None, g["u"], g["delta"], g["A"], Bm, Cm, g["D"], g["z"], g["dt_bias"], True,
+                                            chunk_states=cs_plan.chunk_states, grads_in_input_dtype=True), iters=10)
+    bbytes = 7 * elt * batch * dim * length + 4 * elt * batch * dim * nstate * length
     return {"kernel_us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
             "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes,
+            "bwd_us": round(bus, 1), "bwd_GBps": round(bbytes / bus / 1e3, 1),
+            "bwd_frac_hbm": round(bbytes / bus / 1e3 / HBM_PEAK_GBPS, 4), "bwd_algorithmic_bytes": bbytes,
             "shape": "B, C (8, 1536, 16, 2048) bf16: one B/C group per channel"}
 
 

@@ -113,7 +113,7 @@ typedef struct ssm_scan_bwd_args {
   const float *chunk_states;      /* from ssm_scan_fwd */
   void *du, *ddelta, *dz;         /* (B, D, L) io dtype; dz NULL iff z NULL */
   float *dA;                      /* (D, N) */
-  float *dB, *dC;                 /* fp32, shape of Bproj / Cproj */
+  void *dB, *dC;                  /* shape of Bproj / Cproj, float32 unless dbc_dtype says otherwise */
   float *dD, *ddt_bias;           /* (D,) or NULL */
   void *workspace;                /* ssm_scan_bwd_workspace_bytes(), 256-byte aligned */
   size_t workspace_bytes;
@@ -122,10 +122,18 @@ typedef struct ssm_scan_bwd_args {
   int32_t b_kind, c_kind, b_groups, c_groups;
   int32_t delta_softplus;
   int32_t reserved;               /* must be 0 */
+  int32_t dbc_dtype;              /* element type of dB and dC: SSM_F32 (= 0), or bc_dtype in a call that
+                                     ssm_scan_bwd_per_row_workspace_bytes() accepts */
 } ssm_scan_bwd_args;
 
 size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, int nstate, int b_kind, int c_kind,
                                     int b_groups, int c_groups);
+/* Projections of their own per channel -- B and C of shape (B, D, N, L), i.e. b_groups == c_groups == dim, the form
+ * of the reference's own Mamba1 module (src/ssm/modules/mamba1.py:229-246) -- in aligned rows of whole 8-step
+ * runs: nothing sums over channels, dB and dC are written straight to their place (in float32 or, on request, in
+ * the projections' type) and the call needs only this much workspace.  0: not such a call; it then needs
+ * ssm_scan_bwd_workspace_bytes() and writes dB and dC in float32. */
+size_t ssm_scan_bwd_per_row_workspace_bytes(const ssm_scan_bwd_args *args);
 int ssm_scan_bwd(const ssm_scan_bwd_args *args, void *hip_stream);
 
 /* ------------------------------------------------------------------------

@@ -55,7 +55,7 @@ class ScanBwdArgs(C.Structure):
         ("ddt_bias", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
         ("batch", _i32), ("dim", _i32), ("seqlen", _i32), ("nstate", _i32),
         ("io_dtype", _i32), ("bc_dtype", _i32), ("b_kind", _i32), ("c_kind", _i32),
-        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("reserved", _i32),
+        ("b_groups", _i32), ("c_groups", _i32), ("delta_softplus", _i32), ("reserved", _i32), ("dbc_dtype", _i32),
     ]
 
 
@@ -370,6 +370,7 @@ PLAIN_SYMBOLS = {
     "ssm_amd_last_error": (C.c_char_p, []),
     "ssm_scan_chunk_len": (C.c_int, []),
     "ssm_scan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 8),
+    "ssm_scan_bwd_per_row_workspace_bytes": (C.c_size_t, [C.POINTER(ScanBwdArgs)]),
     "ssm_state_step_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 3),
     "ssm_dscan_fwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),
     "ssm_dscan_bwd_workspace_bytes": (C.c_size_t, [C.c_int] * 4),

@@ -750,6 +750,7 @@ static int launch_bwd(const ScanBwdParams &p, hipStream_t s) {
 }  // namespace ssm
 
 #include "scan_bwd_fast.hpp"
+#include "scan_bwd_rowbc.hpp"
 
 extern "C" size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, int nstate, int b_kind, int c_kind,
                                                int b_groups, int c_groups) {
@@ -758,6 +759,26 @@ extern "C" size_t ssm_scan_bwd_workspace_bytes(int batch, int dim, int seqlen, i
   if (b_kind == SSM_PROJ_BGNL && (b_groups <= 0 || dim % b_groups)) return 0;
   if (c_kind == SSM_PROJ_BGNL && (c_groups <= 0 || dim % c_groups)) return 0;
   return plan_bwd(batch, dim, seqlen, nstate, b_kind, c_kind, b_groups, c_groups).total;
+}
+
+// Whether a call takes the kernel for projections of their own per channel (scan_bwd_rowbc.hpp): B and C of shape
+// (B, D, N, L), activations in aligned rows of whole 8-step runs.  A selector of 1 (test-hooks build) keeps the
+// general kernel.
+static bool scan_bwd_is_per_row(const ssm_scan_bwd_args *a) {
+  using namespace ssm;
+  if (!a || SSM_RESERVED(a) == 1) return false;
+  if (a->b_kind != SSM_PROJ_BGNL || a->c_kind != SSM_PROJ_BGNL || a->b_groups != a->dim || a->c_groups != a->dim) return false;
+  if (a->seqlen <= 0 || a->seqlen % 8 != 0 || a->nstate <= 0 || a->nstate > BW_MAX_N) return false;
+  if (!valid_dtype(a->io_dtype) || !(a->bc_dtype == a->io_dtype || a->bc_dtype == SSM_F32)) return false;
+  const int bs = dtype_size(a->bc_dtype);
+  return aligned_to(a->u, 16) && aligned_to(a->delta, 16) && aligned_to(a->dout, 16) && aligned_to(a->du, 16) &&
+         aligned_to(a->ddelta, 16) && (!a->z || (aligned_to(a->z, 16) && aligned_to(a->dz, 16))) &&
+         aligned_to(a->Bproj, 8 * bs) && aligned_to(a->Cproj, 8 * bs) && aligned_to(a->dB, 16) && aligned_to(a->dC, 16);
+}
+
+extern "C" size_t ssm_scan_bwd_per_row_workspace_bytes(const ssm_scan_bwd_args *a) {
+  if (!scan_bwd_is_per_row(a)) return 0;
+  return ssm::plan_bwd(a->batch, a->dim, a->seqlen, a->nstate, a->b_kind, a->c_kind, a->b_groups, a->c_groups).off_dB;
 }
 
 extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
@@ -790,8 +811,13 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
               SSM_ERR_TOO_LARGE, "ssm_scan_bwd: tensor too large");
   const BwdPlan pl = plan_bwd(a->batch, a->dim, a->seqlen, a->nstate, a->b_kind, a->c_kind,
                               bv ? a->b_groups : 1, cv ? a->c_groups : 1);
-  SSM_REQUIRE(a->workspace && a->workspace_bytes >= pl.total && aligned_to(a->workspace, 256), SSM_ERR_WORKSPACE,
-              "ssm_scan_bwd: a 256-byte aligned workspace of %zu bytes is required", pl.total);
+  const bool per_row = scan_bwd_is_per_row(a);
+  SSM_REQUIRE(a->dbc_dtype == SSM_F32 || (per_row && a->dbc_dtype == a->bc_dtype), SSM_ERR_BAD_DTYPE,
+              "ssm_scan_bwd: dbc_dtype=%d: dB and dC are float32, or of the projections' type in a call for which "
+              "ssm_scan_bwd_per_row_workspace_bytes() is not 0", a->dbc_dtype);
+  const size_t ws_need = per_row ? pl.off_dB : pl.total;     // per row: no partial sums of dB and dC
+  SSM_REQUIRE(a->workspace && a->workspace_bytes >= ws_need && aligned_to(a->workspace, 256), SSM_ERR_WORKSPACE,
+              "ssm_scan_bwd: a 256-byte aligned workspace of %zu bytes is required", ws_need);
   const int es = dtype_size(a->io_dtype), bs = dtype_size(a->bc_dtype);
   SSM_REQUIRE(aligned_to(a->u, es) && aligned_to(a->delta, es) && aligned_to(a->dout, es) && aligned_to(a->du, es) &&
                   aligned_to(a->ddelta, es) && (!a->z || (aligned_to(a->z, es) && aligned_to(a->dz, es))) &&
@@ -833,7 +859,16 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
     fast_rpw = scan_bwd_fast_rpw(a->batch, a->dim, a->dim / p.b_groups, a->dim / p.c_groups);
     if (fast_rpw && a->dim / (BF_WAVES * fast_rpw) > pl.nblk) fast_rpw = 0;
   }
-  if (fast_rpw) {
+  if (per_row) {
+    const bool bc32 = a->bc_dtype == SSM_F32, o32 = a->dbc_dtype == SSM_F32;
+    if (a->io_dtype == SSM_F32) rc = launch_bwd_rowbc<float, float, float>(p, a->dB, a->dC, s);
+    else if (a->io_dtype == SSM_BF16)
+      rc = bc32 ? launch_bwd_rowbc<bf16_t, float, float>(p, a->dB, a->dC, s)
+                : (o32 ? launch_bwd_rowbc<bf16_t, bf16_t, float>(p, a->dB, a->dC, s) : launch_bwd_rowbc<bf16_t, bf16_t, bf16_t>(p, a->dB, a->dC, s));
+    else
+      rc = bc32 ? launch_bwd_rowbc<f16_t, float, float>(p, a->dB, a->dC, s)
+                : (o32 ? launch_bwd_rowbc<f16_t, f16_t, float>(p, a->dB, a->dC, s) : launch_bwd_rowbc<f16_t, f16_t, f16_t>(p, a->dB, a->dC, s));
+  } else if (fast_rpw) {
     p.rows_per_wg = BF_WAVES * fast_rpw;
     p.nblk = a->dim / p.rows_per_wg;
     const bool bc32 = a->bc_dtype == SSM_F32;
@@ -870,8 +905,10 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
                          (size_t)D * N);
     }
   };
-  fold_proj(a->b_kind, p.b_groups, p.dB_part, a->dB);
-  fold_proj(a->c_kind, p.c_groups, p.dC_part, a->dC);
+  if (!per_row) {
+    fold_proj(a->b_kind, p.b_groups, p.dB_part, reinterpret_cast<float *>(a->dB));
+    fold_proj(a->c_kind, p.c_groups, p.dC_part, reinterpret_cast<float *>(a->dC));
+  }
   SSM_CHECK_LAUNCH("ssm_scan_bwd(fold)");
   return SSM_OK;
 }

@@ -179,11 +179,13 @@ def _slice_states(p, kind, lo, hi):
 
 
 def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softplus, chunk_states=None,
-                   tune_items=0):
+                   tune_items=0, grads_in_input_dtype=False):
     """Run ``ssm_scan_bwd``; returns fp32/io-dtype gradients in input order
     ``(du, ddelta, dA, dB, dC, dD, dz, ddt_bias)``.  State sizes above 16 are
     processed in blocks of 16 states (the recurrence is independent per state and
-    every gradient is additive over states)."""
+    every gradient is additive over states).  With ``grads_in_input_dtype``, ``dB`` and ``dC`` of projections that
+    every channel has for itself, ``(B, D, N, L)``, come back in the projections' own type where the kernel for
+    that form writes them (no float32 tensors of that size, and no cast of them afterwards)."""
     if K.f64_compute(u, A):
         from . import _f64
         return _f64.scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softplus)
@@ -201,8 +203,7 @@ def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softpl
     lib = _lib.load()
 
     dA = torch.empty(dim, nstate, dtype=torch.float32, device=dev)
-    dB = torch.empty(B_c.shape, dtype=torch.float32, device=dev)
-    dC = torch.empty(C_c.shape, dtype=torch.float32, device=dev)
+    dB = dC = None                    # allocated once the element type is known (first block of states)
     dD = torch.empty(dim, dtype=torch.float32, device=dev) if D is not None else None
     dbias = torch.empty(dim, dtype=torch.float32, device=dev) if dt_bias is not None else None
     blocks = [(lo, min(nstate, lo + _BWD_MAX_STATES)) for lo in range(0, nstate, _BWD_MAX_STATES)]
@@ -228,22 +229,32 @@ def _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, softpl
         du_b, ddl_b = torch.empty_like(u_c), torch.empty_like(u_c)
         dz_b = torch.empty_like(u_c) if z_c is not None else None
         dA_b = dA if single else torch.empty(dim, n_blk, dtype=torch.float32, device=dev)
-        dB_b = dB if single else torch.empty(B_b.shape, dtype=torch.float32, device=dev)
-        dC_b = dC if single else torch.empty(C_b.shape, dtype=torch.float32, device=dev)
+        dB_b = dC_b = None
         dD_b = dD if bi == 0 else None
         dbias_b = torch.empty(dim, dtype=torch.float32, device=dev) if dt_bias is not None else None
-        nbytes = lib.ssm_scan_bwd_workspace_bytes(batch, dim, length, n_blk, bkind, ckind, bgroups, cgroups)
-        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
-        ws_ptr = (ws.data_ptr() + 255) // 256 * 256
         args = _lib.ScanBwdArgs(
             u=_lib.ptr(u_c), delta=_lib.ptr(dl_c), z=_lib.ptr(z_c), dout=_lib.ptr(go_c), A=_lib.ptr(A_b),
             Bproj=_lib.ptr(B_b), Cproj=_lib.ptr(C_b), Dskip=_lib.ptr(D_b), dt_bias=_lib.ptr(bias_f),
             dlast_state=_lib.ptr(gl_b), chunk_states=_lib.ptr(cs), du=_lib.ptr(du_b), ddelta=_lib.ptr(ddl_b),
-            dz=_lib.ptr(dz_b), dA=_lib.ptr(dA_b), dB=_lib.ptr(dB_b), dC=_lib.ptr(dC_b), dD=_lib.ptr(dD_b),
-            ddt_bias=_lib.ptr(dbias_b), workspace=ws_ptr, workspace_bytes=nbytes,
+            dz=_lib.ptr(dz_b), dA=_lib.ptr(dA_b), dB=256, dC=256, dD=_lib.ptr(dD_b),       # (dB, dC: set below)
+            ddt_bias=_lib.ptr(dbias_b), workspace=None, workspace_bytes=0,
             batch=batch, dim=dim, seqlen=length, nstate=n_blk, io_dtype=_lib.dtype_enum(io),
             bc_dtype=_lib.dtype_enum(bc), b_kind=bkind, c_kind=ckind, b_groups=bgroups, c_groups=cgroups,
             delta_softplus=int(bool(softplus)), reserved=int(tune_items))
+        # projections of their own per channel: no partial sums of dB and dC, and their own type on request
+        nbytes = int((_lib.load_test_hooks() if tune_items else lib).ssm_scan_bwd_per_row_workspace_bytes(args))
+        g_dtype = bc if (nbytes and grads_in_input_dtype and single) else torch.float32
+        dB_b, dC_b = (torch.empty(B_b.shape, dtype=g_dtype, device=dev), torch.empty(C_b.shape, dtype=g_dtype, device=dev))
+        args.dB, args.dC, args.dbc_dtype = _lib.ptr(dB_b), _lib.ptr(dC_b), _lib.dtype_enum(g_dtype)
+        if single:
+            dB, dC = dB_b, dC_b
+        elif dB is None:
+            dB = torch.empty(B_c.shape, dtype=torch.float32, device=dev)
+            dC = torch.empty(C_c.shape, dtype=torch.float32, device=dev)
+        if not nbytes:
+            nbytes = lib.ssm_scan_bwd_workspace_bytes(batch, dim, length, n_blk, bkind, ckind, bgroups, cgroups)
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
+        args.workspace, args.workspace_bytes = (ws.data_ptr() + 255) // 256 * 256, nbytes
         _lib.call("ssm_scan_bwd", args, dev)
         if single:
             du, ddl, dz, dbias = du_b, ddl_b, dz_b, dbias_b

@@ -112,7 +112,7 @@ class SelectiveScanFn(torch.autograd.Function):
         if grad_last is not None and grad_last.numel() == 0:
             grad_last = None
         grads = _scan_backward(grad_out, grad_last, u, delta, A, B, C, D, z, dt_bias, ctx.softplus,
-                               chunk_states=chunk_states)
+                               chunk_states=chunk_states, grads_in_input_dtype=True)
         need = ctx.needs_input_grad
         refs = (u, delta, A, B, C, D, z, dt_bias)
         out = tuple(_like(g, r) if (r is not None and need[i]) else None

@@ -281,6 +281,84 @@ def test_specialised_backward_matches_general_kernel_and_oracle(shape, groups, u
         torch.testing.assert_close(f.double().cpu(), want, **tol, msg=lambda m, k=k: f"grad {k} vs float64: {m}")
 
 
+@pytest.mark.parametrize("shape,use_z,with_last", [((2, 24, 1040, 16), True, True), ((1, 7, 512, 16), True, False),
+                                                   ((2, 5, 1536, 9), False, True), ((3, 10, 72, 4), True, False)],
+                         ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("dtype,bc_dtype", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32),
+                                            (torch.float32, torch.float32)])
+def test_per_channel_projections_backward(shape, use_z, with_last, dtype, bc_dtype):
+    """``B`` and ``C`` of shape ``(B, D, N, L)``, the reference Mamba1 module's own call
+    (/root/reference/src/ssm/modules/mamba1.py:229-246): the wave-per-row kernel that writes ``dB`` and ``dC`` straight
+    to their place, against the general kernel (test-hooks selector 1) and float64 autograd through the oracle, and
+    through autograd with ``dB`` / ``dC`` written in the projections' own type."""
+    b, d, l, n = shape
+    inp = make_inputs(sum(shape) + 1, b, d, l, n, dtype=dtype, bc_dtype=bc_dtype, groups=d, use_z=use_z)
+    g = torch.Generator().manual_seed(5)
+    go = torch.randn(b, d, l, generator=g).to(dtype)
+    gl = torch.randn(b, d, n, generator=g) if with_last else None
+    fast = _bwd_direct(inp, go, gl, 0)
+    gen = _bwd_direct(inp, go, gl, 1)
+    names = ("u", "delta", "A", "B", "C", "D", "z", "dt_bias")
+    for k, f, r in zip(names, fast, gen):
+        if r is None:
+            assert f is None, k
+            continue
+        assert f.dtype == r.dtype and f.shape == r.shape, k
+        f, r = f.float().cpu(), r.float().cpu()
+        scale = float(r.abs().max()) + 1e-30
+        if k in ("u", "delta", "z") and dtype != torch.float32:
+            torch.testing.assert_close(f, r, rtol=2e-2, atol=1e-3 * scale, msg=lambda m, k=k: f"grad {k} vs general kernel: {m}")
+        else:
+            torch.testing.assert_close(f, r, rtol=2e-4, atol=2e-5 * scale, msg=lambda m, k=k: f"grad {k} vs general kernel: {m}")
+    w = {k: (None if v is None else v.double().requires_grad_(True)) for k, v in inp.items()}
+    out = O.selective_scan(w["u"], w["delta"], w["A"], w["B"], w["C"], D=w["D"], z=w["z"], dt_bias=w["dt_bias"],
+                           softplus=True, return_last_state=with_last, acc=torch.float64)
+    if with_last:
+        ((out[0] * go.double()).sum() + (out[1] * gl.double()).sum()).backward()
+    else:
+        (out * go.double()).sum().backward()
+    # through autograd: dB and dC arrive in the projections' type, written so by the kernel
+    lv = {k: (None if v is None else v.cuda().requires_grad_(True)) for k, v in inp.items()}
+    res = _ops().selective_scan(lv["u"], lv["delta"], lv["A"], lv["B"], lv["C"], D=lv["D"], z=lv["z"],
+                                dt_bias=lv["dt_bias"], softplus=True, return_last_state=with_last)
+    if with_last:
+        ((res[0].float() * go.cuda().float()).sum() + (res[1].float() * gl.cuda()).sum()).backward()
+    else:
+        (res.float() * go.cuda().float()).sum().backward()
+    for k, f in zip(names, fast):
+        if w[k] is None:
+            continue
+        want = w[k].grad
+        scale = float(want.abs().max()) + 1e-30
+        half = k in ("u", "delta", "z") and dtype != torch.float32
+        tol = dict(rtol=2e-2, atol=4e-3 * scale) if half else dict(rtol=1e-3, atol=1e-4 * scale)
+        torch.testing.assert_close(f.double().cpu(), want, **tol, msg=lambda m, k=k: f"grad {k} vs float64: {m}")
+        ga = lv[k].grad
+        assert ga.dtype == lv[k].dtype and ga.shape == lv[k].shape, k
+        half_a = half or (k in ("B", "C") and bc_dtype != torch.float32)
+        tol = dict(rtol=2e-2, atol=4e-3 * scale) if half_a else dict(rtol=1e-3, atol=1e-4 * scale)
+        torch.testing.assert_close(ga.double().cpu(), want, **tol, msg=lambda m, k=k: f"autograd grad {k} vs float64: {m}")
+
+
+def test_per_channel_projections_backward_needs_no_partial_sums():
+    """The call's workspace holds the per-row sums of dA, dD and the bias only (the general kernel would need a
+    float32 copy of dB and dC on top)."""
+    from ssm_amd import _lib
+    b, d, l, n = 2, 24, 1024, 16
+    lib = _lib.load()
+    general = lib.ssm_scan_bwd_workspace_bytes(b, d, l, n, _lib.PROJ_BGNL, _lib.PROJ_BGNL, d, d)
+    x = torch.zeros(b, d, l, device="cuda")
+    p = torch.zeros(b, d, n, l, device="cuda")
+    args = _lib.ScanBwdArgs(u=x.data_ptr(), delta=x.data_ptr(), dout=x.data_ptr(), du=x.data_ptr(), ddelta=x.data_ptr(),
+                            Bproj=p.data_ptr(), Cproj=p.data_ptr(), dB=p.data_ptr(), dC=p.data_ptr(), batch=b, dim=d, seqlen=l,
+                            nstate=n, io_dtype=_lib.SSM_F32, bc_dtype=_lib.SSM_F32, b_kind=_lib.PROJ_BGNL, c_kind=_lib.PROJ_BGNL,
+                            b_groups=d, c_groups=d)
+    direct = lib.ssm_scan_bwd_per_row_workspace_bytes(args)
+    assert 0 < direct <= 4 * b * d * (n + 2) + 3 * 256 and general >= 2 * 4 * b * d * n * l
+    args.b_groups = args.c_groups = 1            # one group for all channels: not such a call
+    assert lib.ssm_scan_bwd_per_row_workspace_bytes(args) == 0
+
+
 def test_specialised_backward_is_bit_reproducible():
     inp = make_inputs(11, 2, 48, 1040, 16, dtype=torch.bfloat16)
     g = torch.Generator().manual_seed(4)
