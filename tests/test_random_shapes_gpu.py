@@ -324,7 +324,7 @@ def test_operator_over_random_shapes_matches_the_float64_oracle(case, block):
 
 
 # dA of the SSD, per head, against the sum of the magnitudes of its terms dt_t q_t
-DA_TERM_BAR_HALF, DA_TERM_BAR_F32 = 2e-2, 2e-4     # seen over 190 cases: 1.4e-2 and 1.1e-4 at worst, medians 5e-4 and 3e-6
+DA_TERM_BAR_HALF, DA_TERM_BAR_F32 = 2e-2, 5e-4     # seen over 1 260 cases: 1.4e-2 and 3.0e-4 at worst, medians 5e-4 and 3e-6
 
 
 def _ssd_case(rng, seed):
@@ -571,7 +571,9 @@ def _ssd_stages_case(rng, seed):
 
     st64 = SO.chunk_state(Bm, x, dtc64, cs64, seq_idx=seq_idx)
     st = S.chunk_state(dev(Bm), dev(x), dtc32, cs32, seq_idx=sid)
-    _close(st, st64, (desc, "chunk_state"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 2e-5)
+    # (float32: the running sums arrive rounded to float32, which the exponentials of their differences magnify;
+    #  worst of 1 070 cases 5.4e-5 of the rms)
+    _close(st, st64, (desc, "chunk_state"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 1e-4)
 
     ent64, fin64 = SO.state_passing(st64, cs64[..., -1], initial_states=init, seq_idx=seq_idx, chunk_size=Q)
     ent, fin = S.state_passing(st64.float().cuda(), cs32[..., -1].contiguous(), initial_states=dev(init), seq_idx=sid, chunk_size=Q)
@@ -580,7 +582,9 @@ def _ssd_stages_case(rng, seed):
 
     y64 = SO.chunk_scan(Bm, Cm, x, dtc64, cs64, ent64, D=D, z=z, seq_idx=seq_idx)
     y = S.chunk_scan(dev(Bm), dev(Cm), dev(x), dtc32, cs32, ent64.float().cuda(), D=dev(D), z=dev(z), seq_idx=sid)
-    _close(y, y64, (desc, "chunk_scan"), half=half, rtol=None if half else 1e-4, atol_rms=None if half else 1e-4)
+    # (16-bit: two roundings of operands ahead of the output's own, as in the gradients: their bar on single elements;
+    #  worst of 1 070 cases 7.6e-2 of the rms in one element, the mean error stays under 5e-3)
+    _close(y, y64, (desc, "chunk_scan"), half=half, rtol=None if half else 1e-4, atol_rms=8e-2 if half else 1e-4)
 
     if cuts and b == 1:
         cu = torch.tensor([0] + cuts + [l], dtype=torch.int32)
