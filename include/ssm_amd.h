@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SSM_AMD_ABI_VERSION 7
+#define SSM_AMD_ABI_VERSION 8
 
 typedef enum ssm_status {
   SSM_OK = 0,
@@ -48,7 +48,11 @@ typedef enum ssm_proj_kind {
   SSM_PROJ_BGNL = 2   /* (B, G, N, L) grouped and time-varying; channel d reads group d / (D/G) */
 } ssm_proj_kind;
 
-typedef enum ssm_layout { SSM_LAYOUT_BCL = 0, SSM_LAYOUT_BLC = 1 } ssm_layout;
+/* SSM_LAYOUT_ROWS_TO_BCL (the convolution only): x is a (B,C,L)-shaped view of memory laid out as rows of
+ * channels, one row per time step (`x_row_stride` elements apart, `x_batch_stride` between batch rows) -- what the
+ * reference's blocks pass (src/ssm/modules/mamba1.py:209-215, mamba2.py:159-165: `projected.permute(0, 2, 1)`);
+ * y and dout are dense (B,C,L), dx is written as dense (B,L,C) rows. */
+typedef enum ssm_layout { SSM_LAYOUT_BCL = 0, SSM_LAYOUT_BLC = 1, SSM_LAYOUT_ROWS_TO_BCL = 2 } ssm_layout;
 typedef enum ssm_activation { SSM_ACT_IDENTITY = 0, SSM_ACT_SILU = 1 } ssm_activation;
 
 int ssm_amd_abi_version(void);
@@ -661,25 +665,29 @@ typedef struct ssm_conv1d_fwd_args {
   const void *x;          /* (B,C,L) or (B,L,C), io dtype */
   const float *weight;    /* (C, K) fp32 */
   const float *bias;      /* (C,) fp32 or NULL */
-  void *y;                /* same layout and dtype as x */
+  void *y;                /* same layout and dtype as x (SSM_LAYOUT_ROWS_TO_BCL: dense (B,C,L)) */
   int32_t batch, channels, seqlen, width;
   int32_t io_dtype, layout, activation;
+  int32_t pad0;
+  int64_t x_batch_stride, x_row_stride;   /* elements; SSM_LAYOUT_ROWS_TO_BCL only, zero otherwise */
 } ssm_conv1d_fwd_args;
 
 int ssm_conv1d_fwd(const ssm_conv1d_fwd_args *args, void *hip_stream);
 
 typedef struct ssm_conv1d_bwd_args {
   const void *x;          /* forward input */
-  const void *dout;       /* gradient of y, same layout/dtype as x */
+  const void *dout;       /* gradient of y, same layout/dtype as x (SSM_LAYOUT_ROWS_TO_BCL: dense (B,C,L)) */
   const float *weight;
   const float *bias;      /* or NULL (needed to rebuild the pre-activation) */
-  void *dx;               /* same layout/dtype as x */
+  void *dx;               /* same layout/dtype as x (SSM_LAYOUT_ROWS_TO_BCL: dense (B,L,C) rows) */
   float *dweight;         /* (C, K) fp32 */
   float *dbias;           /* (C,) fp32 or NULL */
   void *workspace;        /* ssm_conv1d_bwd_workspace_bytes() bytes of device memory */
   size_t workspace_bytes;
   int32_t batch, channels, seqlen, width;
   int32_t io_dtype, layout, activation;
+  int32_t pad0;
+  int64_t x_batch_stride, x_row_stride;   /* elements; SSM_LAYOUT_ROWS_TO_BCL only, zero otherwise */
 } ssm_conv1d_bwd_args;
 
 size_t ssm_conv1d_bwd_workspace_bytes(int batch, int channels, int width);

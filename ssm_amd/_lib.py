@@ -19,7 +19,7 @@ import os
 # SSM_AMD_LIB points the binding at another build of the same C ABI.
 LIB_PATH = Path(os.environ.get("SSM_AMD_LIB") or
                 Path(__file__).resolve().parent / "lib" / "libssm_amd.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 SSM_F32, SSM_BF16, SSM_F16 = 0, 1, 2
 PROJ_DN, PROJ_BDN, PROJ_BGNL = 0, 1, 2
@@ -229,7 +229,7 @@ class SsdBwdDtArgs(C.Structure):
                 ("dt_softplus", _i32), ("dt_min", C.c_float), ("dt_max", C.c_float)]
 
 
-LAYOUT_BCL, LAYOUT_BLC = 0, 1
+LAYOUT_BCL, LAYOUT_BLC, LAYOUT_ROWS_TO_BCL = 0, 1, 2
 ACT_IDENTITY, ACT_SILU = 0, 1
 
 
@@ -237,7 +237,8 @@ class Conv1dFwdArgs(C.Structure):
     _fields_ = [
         ("x", _vp), ("weight", _vp), ("bias", _vp), ("y", _vp),
         ("batch", _i32), ("channels", _i32), ("seqlen", _i32), ("width", _i32),
-        ("io_dtype", _i32), ("layout", _i32), ("activation", _i32),
+        ("io_dtype", _i32), ("layout", _i32), ("activation", _i32), ("pad0", _i32),
+        ("x_batch_stride", C.c_int64), ("x_row_stride", C.c_int64),
     ]
 
 
@@ -246,7 +247,8 @@ class Conv1dBwdArgs(C.Structure):
         ("x", _vp), ("dout", _vp), ("weight", _vp), ("bias", _vp), ("dx", _vp), ("dweight", _vp),
         ("dbias", _vp), ("workspace", _vp), ("workspace_bytes", C.c_size_t),
         ("batch", _i32), ("channels", _i32), ("seqlen", _i32), ("width", _i32),
-        ("io_dtype", _i32), ("layout", _i32), ("activation", _i32),
+        ("io_dtype", _i32), ("layout", _i32), ("activation", _i32), ("pad0", _i32),
+        ("x_batch_stride", C.c_int64), ("x_row_stride", C.c_int64),
     ]
 
 

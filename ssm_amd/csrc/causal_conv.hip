@@ -28,6 +28,38 @@ __device__ __forceinline__ void load_taps(const float *w, int c, int K, float (&
   for (int m = 0; m < CONV_TAPS; ++m) wrev[m] = m < K ? w[(size_t)c * K + (K - 1 - m)] : 0.0f;
 }
 
+// The taps and the bias of VEC neighbouring channels from channel c0 on.  `wide`: the kernel is 4 wide and weight and
+// bias start on 16-byte boundaries, c0 is a multiple of VEC: one 16-byte read per channel and one read for the
+// biases instead of five 4-byte reads per channel (a thread that owns 8 steps of 4 channels otherwise issues more
+// reads for its taps than for its rows).
+template <int VEC>
+__device__ __forceinline__ void load_taps_of(const float *w, const float *b, int c0, int K, bool wide,
+                                             float (&wrev)[VEC][CONV_TAPS], float (&bias)[VEC]) {
+  if (wide) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const Pack<float, 4> q = *reinterpret_cast<const Pack<float, 4> *>(w + (size_t)(c0 + i) * 4);
+      wrev[i][0] = q.v[3]; wrev[i][1] = q.v[2]; wrev[i][2] = q.v[1]; wrev[i][3] = q.v[0];
+#pragma unroll
+      for (int m = 4; m < CONV_TAPS; ++m) wrev[i][m] = 0.0f;
+    }
+    if (b) {
+      const Pack<float, VEC> q = *reinterpret_cast<const Pack<float, VEC> *>(b + c0);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) bias[i] = q.v[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) bias[i] = 0.0f;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      bias[i] = b ? b[c0 + i] : 0.0f;
+      load_taps(w, c0 + i, K, wrev[i]);
+    }
+  }
+}
+
 struct ConvParams {
   const void *x, *dout;
   const float *w, *bias;     // (C,K) fp32, (C,) fp32 or null
@@ -35,6 +67,8 @@ struct ConvParams {
   float *partial;            // bwd: [B][C][K+1] partial sums (dw..., dbias)
   int batch, chans, len, K;
   int silu;
+  long long x_bs, x_rs;      // rows-in kernels: elements between batch rows and between time steps of x
+  int wide_taps;             // K == 4, weight and bias on 16-byte boundaries (see load_taps_of)
 };
 
 __device__ __forceinline__ float silu_grad(float pre) {
@@ -73,9 +107,10 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvPar
   const int c = row % p.chans;
   const T *xr = reinterpret_cast<const T *>(p.x) + (size_t)row * p.len;
   T *yr = reinterpret_cast<T *>(p.y) + (size_t)row * p.len;
-  float wrev[CONV_TAPS];
-  load_taps(p.w, c, p.K, wrev);
-  const float bias = p.bias ? p.bias[c] : 0.0f;
+  float wrev1[1][CONV_TAPS], bias1[1];
+  load_taps_of<1>(p.w, p.bias, c, p.K, p.wide_taps, wrev1, bias1);
+  const float (&wrev)[CONV_TAPS] = wrev1[0];
+  const float bias = bias1[0];
   for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
     float win[2 * VEC];
     if constexpr (AL) {
@@ -157,10 +192,13 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
   const int K = p.K;
   constexpr int HIST = CONV_TAPS - 1;
   float wrev[VEC][CONV_TAPS], bias[VEC];
+  if constexpr (AL) load_taps_of<VEC>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
+  else {
 #pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    bias[i] = (p.bias && i < cw) ? p.bias[c0 + i] : 0.0f;
-    load_taps(p.w, i < cw ? c0 + i : c0, K, wrev[i]);
+    for (int i = 0; i < VEC; ++i) {
+      bias[i] = (p.bias && i < cw) ? p.bias[c0 + i] : 0.0f;
+      load_taps(p.w, i < cw ? c0 + i : c0, K, wrev[i]);
+    }
   }
   const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
   T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
@@ -254,11 +292,7 @@ __global__ __launch_bounds__(CONV_CL_WALK_THREADS) void conv_fwd_cl_walk_kernel(
   const int b = (int)(gid / ((size_t)cvecs * spans));
   const int c0 = cv * VEC;
   float wrev[VEC][CONV_TAPS], bias[VEC];
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    bias[i] = p.bias ? p.bias[c0 + i] : 0.0f;
-    load_taps(p.w, c0 + i, p.K, wrev[i]);
-  }
+  load_taps_of<VEC>(p.w, p.bias, c0, p.K, p.wide_taps, wrev, bias);
   const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
   T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
   const int t_first = span * SPAN;
@@ -317,9 +351,10 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
   const T *xr = reinterpret_cast<const T *>(p.x) + (size_t)row * p.len;
   const T *gr = reinterpret_cast<const T *>(p.dout) + (size_t)row * p.len;
   T *dxr = reinterpret_cast<T *>(p.y) + (size_t)row * p.len;
-  float wrev[CONV_TAPS];
-  load_taps(p.w, c, K, wrev);
-  const float bias = p.bias ? p.bias[c] : 0.0f;
+  float wrev1[1][CONV_TAPS], bias1[1];
+  load_taps_of<1>(p.w, p.bias, c, K, p.wide_taps, wrev1, bias1);
+  const float (&wrev)[CONV_TAPS] = wrev1[0];
+  const float bias = bias1[0];
   float dwrev[CONV_TAPS], db = 0.0f;
 #pragma unroll
   for (int m = 0; m < CONV_TAPS; ++m) dwrev[m] = 0.0f;
@@ -440,10 +475,16 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
   const int cw = min(VEC, p.chans - c0);          // channels of this vector that exist
   const int K = p.K;
   float wrev[VEC][CONV_TAPS], bias[VEC], dwr[VEC][CONV_TAPS], db[VEC];
+  if constexpr (AL) load_taps_of<VEC>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
+  else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      bias[i] = (p.bias && i < cw) ? p.bias[c0 + i] : 0.0f;
+      load_taps(p.w, i < cw ? c0 + i : c0, K, wrev[i]);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
-    bias[i] = (p.bias && i < cw) ? p.bias[c0 + i] : 0.0f;
-    load_taps(p.w, i < cw ? c0 + i : c0, K, wrev[i]);
     db[i] = 0.0f;
 #pragma unroll
     for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = 0.0f;
@@ -577,6 +618,232 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
   }
 }
 
+// ------------------------------------------- rows of (B,L,C) in, (B,C,L) out (forward and backward)
+// The reference's blocks hand the convolution a (B,C,L)-shaped view of a projection whose memory is (B,L,C') rows
+// (src/ssm/modules/mamba1.py:209-215, mamba2.py:159-165: `projected.permute(0, 2, 1)`, in the first a half of a
+// wider projection, so with gaps between the rows) and use the result as (B,C,L).  These kernels take that view
+// as it lies instead of a transposed copy: a workgroup owns a tile of 64 channels x TT steps; its threads work
+// with channels innermost (a thread: VEC neighbouring channels over 8 steps, the rows read straight from global
+// memory, the lanes of a row on 128 or 256 contiguous bytes), and the turn to time innermost goes through LDS in
+// 16-byte units of steps of one channel.  Unit u of the tile row of channel group g (the VEC channels of one thread)
+// lies at unit (u ^ (g mod units per row)): the 16 lanes that hold one unit each for 16 channel groups, and the
+// 16 lanes that move 16 neighbouring units of one row, both land on different bank groups (all 16, or 8 of them
+// twice where a row has 8 units).
+constexpr int CONV_TR_CH = 64, CONV_TR_STRIP = 8;
+constexpr int CONV_TR_FWD_VEC = 4, CONV_TR_FWD_STEPS = 64;    // forward: 16 lanes x 8 strips
+constexpr int CONV_TR_BWD_VEC = 2, CONV_TR_BWD_STEPS = 64;     // backward: 32 lanes x 8 strips (registers)
+constexpr int CONV_TR_THREADS = 256;
+constexpr int CONV_TR_ALIGN = 4;                                // channels: count, strides and start of x are multiples
+constexpr int CONV_TR_FWD_THREADS = (CONV_TR_CH / CONV_TR_FWD_VEC) * (CONV_TR_FWD_STEPS / CONV_TR_STRIP);
+static_assert((CONV_TR_CH / CONV_TR_BWD_VEC) * (CONV_TR_BWD_STEPS / CONV_TR_STRIP) == CONV_TR_THREADS, "backward tile");
+
+// AL: the rows of y (L elements each) start on 16-byte boundaries and L is a whole number of 16-byte units.
+template <typename T, bool AL>
+__global__ __launch_bounds__(CONV_TR_FWD_THREADS) void conv_fwd_tr_kernel(const ConvParams p) {
+  constexpr int CH = CONV_TR_CH, TT = CONV_TR_FWD_STEPS, S = CONV_TR_STRIP, VEC = CONV_TR_FWD_VEC, HIST = CONV_TAPS - 1;
+  constexpr int UNIT = 16 / sizeof(T), UPR = TT / UNIT, UPS = S / UNIT;   // elements per unit, units per row / strip
+  constexpr int GROUPS = CH / VEC;
+  __shared__ __attribute__((aligned(16))) T tile[CH * TT];
+  const int ttiles = (p.len + TT - 1) / TT, ctiles = (p.chans + CH - 1) / CH;
+  int bid = blockIdx.x;
+  const int ct = bid % ctiles; bid /= ctiles;
+  const int tt = bid % ttiles;
+  const int b = bid / ttiles;
+  const int cg = threadIdx.x % GROUPS, ts = threadIdx.x / GROUPS;
+  const int c_own = ct * CH + cg * VEC;
+  const int c0 = c_own < p.chans ? c_own : 0;        // the channel count is a multiple of VEC: a group is all in or all out
+  const int t0 = tt * TT + ts * S;
+  float wrev[VEC][CONV_TAPS], bias[VEC];
+  load_taps_of<VEC>(p.w, p.bias, c0, p.K, p.wide_taps, wrev, bias);
+  const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.x_bs + c0;
+  Pack<T, VEC> raw[HIST + S];
+#pragma unroll
+  for (int j = 0; j < HIST + S; ++j)
+    raw[j] = *reinterpret_cast<const Pack<T, VEC> *>(xb + (size_t)min(max(t0 - HIST + j, 0), p.len - 1) * p.x_rs);
+#pragma unroll
+  for (int j = 0; j < HIST; ++j) {
+    if (t0 - HIST + j < 0) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) raw[j].v[i] = from_f32<T>(0.0f);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    Pack<T, UNIT> col[UPS];
+#pragma unroll
+    for (int sidx = 0; sidx < S; ++sidx) {
+      float acc = bias[i];
+#pragma unroll
+      for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + sidx - m].v[i]), acc);
+      col[sidx / UNIT].v[sidx % UNIT] = from_f32<T>(p.silu ? silu_f32(acc) : acc);
+    }
+    const int r = cg * VEC + i;
+#pragma unroll
+    for (int h = 0; h < UPS; ++h)
+      *reinterpret_cast<Pack<T, UNIT> *>(tile + r * TT + ((ts * UPS + h) ^ (cg % UPR)) * UNIT) = col[h];
+  }
+  __syncthreads();
+  T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.chans * p.len;
+  for (int v = threadIdx.x; v < CH * UPR; v += CONV_TR_FWD_THREADS) {
+    const int r = v / UPR, u = v % UPR;
+    const int c = ct * CH + r, t = tt * TT + u * UNIT;
+    if (c >= p.chans || t >= p.len) continue;
+    const Pack<T, UNIT> val = *reinterpret_cast<const Pack<T, UNIT> *>(tile + r * TT + (u ^ ((r / VEC) % UPR)) * UNIT);
+    T *dst = yb + (size_t)c * p.len + t;
+    if constexpr (AL) *reinterpret_cast<Pack<T, UNIT> *>(dst) = val;
+    else {
+#pragma unroll
+      for (int e = 0; e < UNIT; ++e)
+        if (t + e < p.len) dst[e] = val.v[e];
+    }
+  }
+}
+
+// Backward on the same kind of tile: dout (B,C,L) comes in through LDS (a tile's steps and one unit beyond them,
+// zeros past the end of the sequence), x is read as rows, dx goes out as dense (B,L,C) rows.  A thread rebuilds the
+// pre-activation at its 8 steps and the 4 after them (dx of a step takes g of the 4 steps that follow), so the
+// transcendental work is 1.5 times the forward's; the kernel stays bound by its three streams.  A workgroup walks
+// the tiles of one time segment (CONV_CL_SEGS segments per batch row at most) and leaves one partial sum of dw
+// and dbias per segment.
+__host__ __device__ inline int conv_tr_seg_tiles(int len) {
+  const int tiles = (len + CONV_TR_BWD_STEPS - 1) / CONV_TR_BWD_STEPS;
+  return (tiles + CONV_CL_SEGS - 1) / CONV_CL_SEGS;
+}
+
+template <typename T, bool AL>
+__global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const ConvParams p) {
+  constexpr int CH = CONV_TR_CH, TT = CONV_TR_BWD_STEPS, S = CONV_TR_STRIP, VEC = CONV_TR_BWD_VEC, HIST = CONV_TAPS - 1;
+  constexpr int UNIT = 16 / sizeof(T), UPR = TT / UNIT, UPS = S / UNIT;
+  constexpr int GU = (S + HIST + UNIT - 1) / UNIT;      // units of dout a thread takes: its strip and 4 steps on
+  constexpr int GROUPS = CH / VEC, GROUPS_PER_WAVE = GROUPS < WAVE ? GROUPS : WAVE;
+  __shared__ __attribute__((aligned(16))) T gt[CH * TT];       // the tile's units, swizzled
+  __shared__ __attribute__((aligned(16))) T gnext[CH * UNIT];  // per channel, the unit beyond the tile
+  __shared__ float red[CONV_TR_THREADS / WAVE][CH][CONV_TAPS + 1];
+  const int ttiles = (p.len + TT - 1) / TT, ctiles = (p.chans + CH - 1) / CH;
+  const int seg_tiles = conv_tr_seg_tiles(p.len);
+  const int nseg = (ttiles + seg_tiles - 1) / seg_tiles;
+  int bid = blockIdx.x;
+  const int seg = bid % nseg; bid /= nseg;
+  const int ct = bid % ctiles;
+  const int b = bid / ctiles;
+  const int cg = threadIdx.x % GROUPS, ts = threadIdx.x / GROUPS;
+  const int c_own = ct * CH + cg * VEC;
+  const bool c_in = c_own < p.chans;
+  const int c0 = c_in ? c_own : 0;
+  const int K = p.K;
+  float wrev[VEC][CONV_TAPS], bias[VEC], dwr[VEC][CONV_TAPS], db[VEC];
+  load_taps_of<VEC>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    db[i] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = 0.0f;
+  }
+  const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.x_bs + c0;
+  const T *gb = reinterpret_cast<const T *>(p.dout) + (size_t)b * p.chans * p.len;
+  T *dxb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
+
+  const int tt_end = min(ttiles, (seg + 1) * seg_tiles);
+  for (int tt = seg * seg_tiles; tt < tt_end; ++tt) {
+    const int t0 = tt * TT + ts * S;
+    // this thread's rows of x: 4 before the strip, the strip, 4 after it
+    Pack<T, VEC> raw[HIST + S + HIST];
+#pragma unroll
+    for (int j = 0; j < HIST + S + HIST; ++j)
+      raw[j] = *reinterpret_cast<const Pack<T, VEC> *>(xb + (size_t)min(max(t0 - HIST + j, 0), p.len - 1) * p.x_rs);
+    // dout of the tile into LDS
+    for (int v = threadIdx.x; v < CH * (UPR + 1); v += CONV_TR_THREADS) {
+      const bool beyond = v >= CH * UPR;
+      const int r = beyond ? v - CH * UPR : v / UPR, u = beyond ? UPR : v % UPR;
+      const int c = ct * CH + r, t = tt * TT + u * UNIT;
+      Pack<T, UNIT> val;
+      if (c < p.chans && t < p.len) {
+        const T *src = gb + (size_t)c * p.len + t;
+        if constexpr (AL) val = *reinterpret_cast<const Pack<T, UNIT> *>(src);
+        else {
+#pragma unroll
+          for (int e = 0; e < UNIT; ++e) val.v[e] = t + e < p.len ? src[e] : from_f32<T>(0.0f);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < UNIT; ++e) val.v[e] = from_f32<T>(0.0f);
+      }
+      if (!beyond) *reinterpret_cast<Pack<T, UNIT> *>(gt + r * TT + (u ^ ((r / VEC) % UPR)) * UNIT) = val;
+      else *reinterpret_cast<Pack<T, UNIT> *>(gnext + r * UNIT) = val;
+    }
+#pragma unroll
+    for (int j = 0; j < HIST; ++j) {
+      if (t0 - HIST + j < 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) raw[j].v[i] = from_f32<T>(0.0f);
+      }
+    }
+    __syncthreads();
+    Pack<T, VEC> out[S];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const int r = cg * VEC + i;
+      Pack<T, UNIT> gu[GU];
+#pragma unroll
+      for (int h = 0; h < GU; ++h) {
+        const int u = ts * UPS + h;
+        gu[h] = u < UPR ? *reinterpret_cast<const Pack<T, UNIT> *>(gt + r * TT + (u ^ (cg % UPR)) * UNIT)
+                        : *reinterpret_cast<const Pack<T, UNIT> *>(gnext + r * UNIT);
+      }
+      float g[S + HIST];
+#pragma unroll
+      for (int j = 0; j < S + HIST; ++j) {
+        g[j] = t0 + j < p.len ? to_f32(gu[j / UNIT].v[j % UNIT]) : 0.0f;
+        if (p.silu && t0 + j < p.len) {
+          float pre = bias[i];
+#pragma unroll
+          for (int m = 0; m < CONV_TAPS; ++m) pre = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + j - m].v[i]), pre);
+          g[j] *= silu_grad(pre);
+        }
+      }
+#pragma unroll
+      for (int sidx = 0; sidx < S; ++sidx) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(g[sidx + m], wrev[i][m], acc);
+        out[sidx].v[i] = from_f32<T>(acc);
+        db[i] += g[sidx];
+#pragma unroll
+        for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = __builtin_fmaf(g[sidx], to_f32(raw[HIST + sidx - m].v[i]), dwr[i][m]);
+      }
+    }
+    if (c_in) {
+#pragma unroll
+      for (int sidx = 0; sidx < S; ++sidx)
+        if (t0 + sidx < p.len) *reinterpret_cast<Pack<T, VEC> *>(dxb + (size_t)(t0 + sidx) * p.chans) = out[sidx];
+    }
+    __syncthreads();                                      // the next tile's dout overwrites gt
+  }
+  // sums over the workgroup's strips: those of one wave through lane exchanges, the waves through LDS
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+#pragma unroll
+    for (int m = 0; m <= CONV_TAPS; ++m) {
+      float s = m < CONV_TAPS ? dwr[i][m] : db[i];
+#pragma unroll
+      for (int d = GROUPS_PER_WAVE; d < WAVE; d *= 2) s += __shfl_xor(s, d);
+      if (lane < GROUPS_PER_WAVE) red[wave][cg * VEC + i][m] = s;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < CH * (K + 1); e += CONV_TR_THREADS) {
+    const int r = e / (K + 1), k = e % (K + 1);
+    const int c = ct * CH + r;
+    if (c >= p.chans) continue;
+    const int src = k < K ? K - 1 - k : CONV_TAPS;        // slot k < K holds dw[k] = dwrev[K-1-k]; slot K the bias sum
+    float s = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < CONV_TR_THREADS / WAVE; ++wv) s += red[wv][r][src];
+    p.partial[(((size_t)b * nseg + seg) * p.chans + c) * (K + 1) + k] = s;
+  }
+}
+
 // Element-wise backward (any K / alignment, either layout): one thread per
 // (b, c) row walks the row sequentially.  Slow path, correctness only.
 template <typename T>
@@ -651,10 +918,15 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_fold_kernel(const float
 }
 
 template <typename T>
-static int conv_fwd_typed(const ConvParams &p, int channels_last, bool vec_ok, hipStream_t s) {
+static int conv_fwd_typed(const ConvParams &p, int layout, bool vec_ok, hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
   const size_t total = (size_t)p.batch * p.chans * p.len;
-  if (p.K <= CONV_TAPS && !channels_last) {
+  const int channels_last = layout == SSM_LAYOUT_BLC;
+  if (layout == SSM_LAYOUT_ROWS_TO_BCL) {
+    const size_t blocks = (size_t)p.batch * ((p.chans + CONV_TR_CH - 1) / CONV_TR_CH) * ((p.len + CONV_TR_FWD_STEPS - 1) / CONV_TR_FWD_STEPS);
+    if (p.len % VEC == 0) hipLaunchKernelGGL((conv_fwd_tr_kernel<T, true>), dim3((unsigned)blocks), dim3(CONV_TR_FWD_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((conv_fwd_tr_kernel<T, false>), dim3((unsigned)blocks), dim3(CONV_TR_FWD_THREADS), 0, s, p);
+  } else if (p.K <= CONV_TAPS && !channels_last) {
     if (vec_ok && p.len % VEC == 0) hipLaunchKernelGGL((conv_fwd_cf_kernel<T, true>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
     else hipLaunchKernelGGL((conv_fwd_cf_kernel<T, false>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
   } else if (p.K <= CONV_TAPS && channels_last) {
@@ -678,11 +950,19 @@ static int conv_fwd_typed(const ConvParams &p, int channels_last, bool vec_ok, h
 }
 
 template <typename T>
-static int conv_bwd_typed(const ConvParams &p, int channels_last, bool vec_ok, float *dw, float *dbias,
+static int conv_bwd_typed(const ConvParams &p, int layout, bool vec_ok, float *dw, float *dbias,
                           hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
   int fold_count = p.batch;
-  if (p.K <= CONV_TAPS && !channels_last) {
+  const int channels_last = layout == SSM_LAYOUT_BLC;
+  if (layout == SSM_LAYOUT_ROWS_TO_BCL) {
+    const int ttiles = (p.len + CONV_TR_BWD_STEPS - 1) / CONV_TR_BWD_STEPS, seg_tiles = conv_tr_seg_tiles(p.len);
+    const int nseg = (ttiles + seg_tiles - 1) / seg_tiles;
+    const size_t blocks = (size_t)p.batch * ((p.chans + CONV_TR_CH - 1) / CONV_TR_CH) * nseg;
+    if (p.len % VEC == 0) hipLaunchKernelGGL((conv_bwd_tr_kernel<T, true>), dim3((unsigned)blocks), dim3(CONV_TR_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((conv_bwd_tr_kernel<T, false>), dim3((unsigned)blocks), dim3(CONV_TR_THREADS), 0, s, p);
+    fold_count = p.batch * nseg;
+  } else if (p.K <= CONV_TAPS && !channels_last) {
     if (vec_ok && p.len % VEC == 0) hipLaunchKernelGGL((conv_bwd_cf_kernel<T, true>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
     else hipLaunchKernelGGL((conv_bwd_cf_kernel<T, false>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
   } else if (p.K <= CONV_TAPS && channels_last) {
@@ -713,13 +993,33 @@ static int conv_check(const char *who, const void *x, const void *w, const void 
   SSM_REQUIRE(batch > 0 && chans > 0 && len > 0 && K > 0, SSM_ERR_BAD_SHAPE,
               "%s: batch=%d channels=%d seqlen=%d width=%d must all be positive", who, batch, chans, len, K);
   SSM_REQUIRE(valid_dtype(dtype), SSM_ERR_BAD_DTYPE, "%s: dtype=%d", who, dtype);
-  SSM_REQUIRE(layout == SSM_LAYOUT_BCL || layout == SSM_LAYOUT_BLC, SSM_ERR_BAD_KIND, "%s: layout=%d", who, layout);
+  SSM_REQUIRE(layout == SSM_LAYOUT_BCL || layout == SSM_LAYOUT_BLC || layout == SSM_LAYOUT_ROWS_TO_BCL, SSM_ERR_BAD_KIND,
+              "%s: layout=%d", who, layout);
   SSM_REQUIRE(act == SSM_ACT_IDENTITY || act == SSM_ACT_SILU, SSM_ERR_BAD_KIND, "%s: activation=%d", who, act);
   SSM_REQUIRE((size_t)batch * chans < ((size_t)1 << 31) && (size_t)batch * chans * len < ((size_t)1 << 40),
               SSM_ERR_TOO_LARGE, "%s: tensor too large", who);
   const int es = dtype_size(dtype);
   SSM_REQUIRE(aligned_to(x, es) && aligned_to(y, es) && aligned_to(w, 4), SSM_ERR_ALIGNMENT,
               "%s: a pointer is not aligned to its element size", who);
+  return SSM_OK;
+}
+
+// SSM_LAYOUT_ROWS_TO_BCL: what the rows-in kernels assume of x and of the tensors written or read as (B,C,L).
+static int conv_rows_check(const char *who, const void *x, long long x_bs, long long x_rs, const void *bcl_a,
+                           const void *bcl_b, const void *rows_out, int batch, int chans, int len, int K, int dtype) {
+  const int es = dtype_size(dtype);
+  SSM_REQUIRE(K <= CONV_TAPS && chans % CONV_TR_ALIGN == 0, SSM_ERR_BAD_SHAPE,
+              "%s: rows of (B,L,C) in, (B,C,L) out takes width <= %d and a multiple of %d channels (got width=%d "
+              "channels=%d): hand over a (B,C,L) copy", who, CONV_TAPS, CONV_TR_ALIGN, K, chans);
+  SSM_REQUIRE(x_rs >= chans && x_rs % CONV_TR_ALIGN == 0 && x_bs % CONV_TR_ALIGN == 0 &&
+              (batch == 1 || x_bs >= (long long)(len - 1) * x_rs + chans), SSM_ERR_BAD_SHAPE,
+              "%s: x_row_stride=%lld, x_batch_stride=%lld must be multiples of %d, rows must not overlap", who,
+              x_rs, x_bs, CONV_TR_ALIGN);
+  SSM_REQUIRE((size_t)batch * ((chans + CONV_TR_CH - 1) / CONV_TR_CH) * ((len + CONV_TR_BWD_STEPS - 1) / CONV_TR_BWD_STEPS) <
+                  ((size_t)1 << 31), SSM_ERR_TOO_LARGE, "%s: too many tiles", who);
+  SSM_REQUIRE(aligned_to(x, CONV_TR_ALIGN * es) && aligned_to(bcl_a, 16) && (!bcl_b || aligned_to(bcl_b, 16)) &&
+              (!rows_out || aligned_to(rows_out, 16)), SSM_ERR_ALIGNMENT,
+              "%s: x must start on a %d-byte boundary, the dense tensors on 16-byte ones", who, CONV_TR_ALIGN * es);
   return SSM_OK;
 }
 
@@ -735,13 +1035,22 @@ extern "C" int ssm_conv1d_fwd(const ssm_conv1d_fwd_args *a, void *hip_stream) {
   p.x = a->x; p.w = a->weight; p.bias = a->bias; p.y = a->y;
   p.batch = a->batch; p.chans = a->channels; p.len = a->seqlen; p.K = a->width;
   p.silu = a->activation == SSM_ACT_SILU;
+  p.wide_taps = a->width == 4 && aligned_to(a->weight, 16) && (!a->bias || aligned_to(a->bias, 16));
   const bool vec_ok = aligned_to(a->x, 16) && aligned_to(a->y, 16);
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  const int cl = a->layout == SSM_LAYOUT_BLC;
+  if (a->layout == SSM_LAYOUT_ROWS_TO_BCL) {
+    p.x_bs = a->x_batch_stride; p.x_rs = a->x_row_stride;
+    rc = conv_rows_check("ssm_conv1d_fwd", a->x, p.x_bs, p.x_rs, a->y, nullptr, nullptr, a->batch, a->channels,
+                         a->seqlen, a->width, a->io_dtype);
+    if (rc != SSM_OK) return rc;
+  } else {
+    SSM_REQUIRE(a->x_batch_stride == 0 && a->x_row_stride == 0, SSM_ERR_BAD_KIND,
+                "ssm_conv1d_fwd: strides of x go with SSM_LAYOUT_ROWS_TO_BCL only");
+  }
   switch (a->io_dtype) {
-    case SSM_F32: return conv_fwd_typed<float>(p, cl, vec_ok, s);
-    case SSM_BF16: return conv_fwd_typed<bf16_t>(p, cl, vec_ok, s);
-    default: return conv_fwd_typed<f16_t>(p, cl, vec_ok, s);
+    case SSM_F32: return conv_fwd_typed<float>(p, a->layout, vec_ok, s);
+    case SSM_BF16: return conv_fwd_typed<bf16_t>(p, a->layout, vec_ok, s);
+    default: return conv_fwd_typed<f16_t>(p, a->layout, vec_ok, s);
   }
 }
 
@@ -768,12 +1077,21 @@ extern "C" int ssm_conv1d_bwd(const ssm_conv1d_bwd_args *a, void *hip_stream) {
   p.partial = reinterpret_cast<float *>(a->workspace);
   p.batch = a->batch; p.chans = a->channels; p.len = a->seqlen; p.K = a->width;
   p.silu = a->activation == SSM_ACT_SILU;
+  p.wide_taps = a->width == 4 && aligned_to(a->weight, 16) && (!a->bias || aligned_to(a->bias, 16));
   const bool vec_ok = aligned_to(a->x, 16) && aligned_to(a->dx, 16) && aligned_to(a->dout, 16);
   hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
-  const int cl = a->layout == SSM_LAYOUT_BLC;
+  if (a->layout == SSM_LAYOUT_ROWS_TO_BCL) {
+    p.x_bs = a->x_batch_stride; p.x_rs = a->x_row_stride;
+    rc = conv_rows_check("ssm_conv1d_bwd", a->x, p.x_bs, p.x_rs, a->dout, nullptr, a->dx, a->batch, a->channels,
+                         a->seqlen, a->width, a->io_dtype);
+    if (rc != SSM_OK) return rc;
+  } else {
+    SSM_REQUIRE(a->x_batch_stride == 0 && a->x_row_stride == 0, SSM_ERR_BAD_KIND,
+                "ssm_conv1d_bwd: strides of x go with SSM_LAYOUT_ROWS_TO_BCL only");
+  }
   switch (a->io_dtype) {
-    case SSM_F32: return conv_bwd_typed<float>(p, cl, vec_ok, a->dweight, a->dbias, s);
-    case SSM_BF16: return conv_bwd_typed<bf16_t>(p, cl, vec_ok, a->dweight, a->dbias, s);
-    default: return conv_bwd_typed<f16_t>(p, cl, vec_ok, a->dweight, a->dbias, s);
+    case SSM_F32: return conv_bwd_typed<float>(p, a->layout, vec_ok, a->dweight, a->dbias, s);
+    case SSM_BF16: return conv_bwd_typed<bf16_t>(p, a->layout, vec_ok, a->dweight, a->dbias, s);
+    default: return conv_bwd_typed<f16_t>(p, a->layout, vec_ok, a->dweight, a->dbias, s);
   }
 }

@@ -760,6 +760,22 @@ def _conv_weight_f32(weight):
     return w.to(torch.float32).contiguous()
 
 
+def _conv_rows_view(x, channels_first, width):
+    """Whether ``x (B, C, L)`` is a view whose memory runs channels innermost -- what the reference's blocks pass
+    (src/ssm/modules/mamba1.py:209-215, mamba2.py:159-165: ``projected.permute(0, 2, 1)``, in the first one half of
+    a wider projection) -- in a form the kernels read as it lies: -> (batch stride, row stride) in elements, or
+    None (the caller then takes a dense copy)."""
+    if not channels_first or x.is_contiguous() or x.dtype == torch.float64:
+        return None
+    batch, chans, length = x.shape
+    sb, sc, sl = x.stride()
+    quad = 4 * x.element_size()
+    if (sc != 1 or chans % 4 or width > 5 or sl < chans or sl % 4 or sb % 4 or x.data_ptr() % quad
+            or (batch > 1 and sb < (length - 1) * sl + chans)):
+        return None
+    return int(sb), int(sl)
+
+
 def _conv_forward(x, weight, bias, activation, channels_last=None):
     if K.f64_compute(x):
         from . import _f64
@@ -767,39 +783,56 @@ def _conv_forward(x, weight, bias, activation, channels_last=None):
     weight, bias = K.narrow(weight, bias)
     batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation, channels_last)
     dev = K.require_gpu(x, weight, bias)
-    xc = K.cast_c(x, x.dtype)
     wf, bf = _conv_weight_f32(weight), K.as_f32_vec(bias)
-    y = torch.empty_like(xc)
+    rows = _conv_rows_view(x, channels_first, width)
+    if rows is not None:
+        xc = x.detach()
+        y = torch.empty(x.shape, dtype=x.dtype, device=dev)
+        layout, strides = _lib.LAYOUT_ROWS_TO_BCL, rows
+    else:
+        xc = K.cast_c(x, x.dtype)
+        y = torch.empty_like(xc)
+        layout, strides = (_lib.LAYOUT_BCL if channels_first else _lib.LAYOUT_BLC), (0, 0)
     args = _lib.Conv1dFwdArgs(
         x=_lib.ptr(xc), weight=_lib.ptr(wf), bias=_lib.ptr(bf), y=_lib.ptr(y),
         batch=batch, channels=chans, seqlen=length, width=width, io_dtype=_lib.dtype_enum(xc.dtype),
-        layout=_lib.LAYOUT_BCL if channels_first else _lib.LAYOUT_BLC,
-        activation=_lib.ACT_SILU if silu else _lib.ACT_IDENTITY)
+        layout=layout, activation=_lib.ACT_SILU if silu else _lib.ACT_IDENTITY,
+        x_batch_stride=strides[0], x_row_stride=strides[1])
     _lib.call("ssm_conv1d_fwd", args, dev)
     return y
 
 
 def _conv_backward(grad_out, x, weight, bias, activation, channels_last=None):
-    """-> (dx, dweight (C,K) fp32, dbias (C,) fp32 or None)."""
+    """-> (dx, dweight (C,K) fp32, dbias (C,) fp32 or None).  ``dx`` has the shape of ``x``; for an ``x`` whose
+    memory runs channels innermost (see :func:`_conv_rows_view`) so does the memory of ``dx``."""
     if K.f64_compute(x):
         from . import _f64
         return _f64.conv_backward(grad_out, x, weight, bias, activation, channels_last)
     weight, bias = K.narrow(weight, bias)
     batch, chans, length, width, channels_first, silu = K.check_conv(x, weight, bias, activation, channels_last)
     dev = K.require_gpu(x, weight, bias, grad_out)
-    xc, gc = K.cast_c(x, x.dtype), K.cast_c(grad_out, x.dtype)
     wf, bf = _conv_weight_f32(weight), K.as_f32_vec(bias)
-    dx = torch.empty_like(xc)
+    gc = K.cast_c(grad_out, x.dtype)
+    rows = _conv_rows_view(x, channels_first, width)
+    if rows is not None:
+        xc = x.detach()
+        dx_rows = torch.empty(batch, length, chans, dtype=x.dtype, device=dev)
+        dx, dx_mem = dx_rows.permute(0, 2, 1), dx_rows
+        layout, strides = _lib.LAYOUT_ROWS_TO_BCL, rows
+    else:
+        xc = K.cast_c(x, x.dtype)
+        dx = dx_mem = torch.empty_like(xc)
+        layout, strides = (_lib.LAYOUT_BCL if channels_first else _lib.LAYOUT_BLC), (0, 0)
     dw = torch.empty(chans, width, dtype=torch.float32, device=dev)
     db = torch.empty(chans, dtype=torch.float32, device=dev) if bias is not None else None
     nbytes = _lib.load().ssm_conv1d_bwd_workspace_bytes(batch, chans, width)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     args = _lib.Conv1dBwdArgs(
-        x=_lib.ptr(xc), dout=_lib.ptr(gc), weight=_lib.ptr(wf), bias=_lib.ptr(bf), dx=_lib.ptr(dx),
+        x=_lib.ptr(xc), dout=_lib.ptr(gc), weight=_lib.ptr(wf), bias=_lib.ptr(bf), dx=_lib.ptr(dx_mem),
         dweight=_lib.ptr(dw), dbias=_lib.ptr(db), workspace=_lib.ptr(ws), workspace_bytes=nbytes,
         batch=batch, channels=chans, seqlen=length, width=width, io_dtype=_lib.dtype_enum(xc.dtype),
-        layout=_lib.LAYOUT_BCL if channels_first else _lib.LAYOUT_BLC,
-        activation=_lib.ACT_SILU if silu else _lib.ACT_IDENTITY)
+        layout=layout, activation=_lib.ACT_SILU if silu else _lib.ACT_IDENTITY,
+        x_batch_stride=strides[0], x_row_stride=strides[1])
     _lib.call("ssm_conv1d_bwd", args, dev)
     return dx, dw, db
 

@@ -165,3 +165,70 @@ def test_channels_last_entry_when_length_equals_channels():
     torch.testing.assert_close(xg.grad.cpu(), xr.grad, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(wg.grad.cpu(), wr.grad, rtol=1e-4, atol=1e-4)
     torch.testing.assert_close(bg.grad.cpu(), br.grad, rtol=1e-4, atol=1e-4)
+
+
+# ------------------------------------------------------------------ a (B,C,L) view of (B,L,C') rows, as it lies
+# The reference's blocks convolve `projected.permute(0, 2, 1)` (src/ssm/modules/mamba1.py:209-215, where `projected`
+# is one half of a wider projection; mamba2.py:159-165): a view whose memory runs channels innermost.
+
+def _rows_case(batch, length, chans, wide, K, seed, dtype=torch.float32, offset=0):
+    g = torch.Generator().manual_seed(seed)
+    proj = torch.randn(batch, length, wide, generator=g).to(dtype)
+    w = torch.rand(chans, K, generator=g) - 0.5
+    b = torch.randn(chans, generator=g) * 0.1
+    go = torch.randn(batch, chans, length, generator=g).to(dtype)
+    return proj, w, b, go, (lambda p: p[:, :, offset:offset + chans].permute(0, 2, 1))
+
+
+@pytest.mark.parametrize("K", [1, 2, 4, 5, 7])
+@pytest.mark.parametrize("act,with_bias", [("silu", True), ("identity", False)])
+@pytest.mark.parametrize("shape", [(2, 11, 8, 8, 0), (1, 300, 64, 128, 64), (3, 1000, 12, 40, 4), (2, 130, 68, 68, 0),
+                                   (1, 5000, 4, 8, 4), (2, 257, 132, 264, 132), (2, 64, 6, 6, 0)],
+                         ids=lambda s: "B{}L{}C{}of{}at{}".format(*s))
+def test_view_of_rows_fp32(K, act, with_bias, shape):
+    """Forward and backward on the view against the oracle on the same view (channel counts that are and are not
+    multiples of the tile's 64, lengths that cross tiles and segments, a width the vector kernels do not take, and
+    6 channels, which go through a copy)."""
+    from ssm_amd import ops
+    batch, length, chans, wide, offset = shape
+    proj, w, b, go, view = _rows_case(batch, length, chans, wide, K, seed=length + K, offset=offset)
+    if not with_bias:
+        b = None
+    res = []
+    for where in ("gpu", "cpu"):
+        to = (lambda t: None if t is None else t.cuda()) if where == "gpu" else (lambda t: None if t is None else t.clone())
+        p_, w_, b_ = to(proj).requires_grad_(), to(w).requires_grad_(), (to(b).requires_grad_() if b is not None else None)
+        fn = ops.dw_causal_conv if where == "gpu" else O.dw_causal_conv
+        y = fn(view(p_), w_, b_, activation=act)
+        assert y.shape == (batch, chans, length)
+        y.backward(to(go))
+        res.append((y.detach().cpu(), p_.grad.cpu(), w_.grad.cpu(), b_.grad.cpu() if b is not None else None))
+    check(res, FP32_TOL, dict(rtol=1e-4, atol=1e-4))
+    taken = ops._conv_rows_view(view(proj.cuda()), True, K)
+    assert (taken is not None) == (chans % 4 == 0 and K <= 5 and not view(proj).is_contiguous())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(2, 256, 64, 128, 0), (2, 1001, 72, 144, 72), (8, 2048, 1536, 3072, 0)],
+                         ids=lambda s: "B{}L{}C{}of{}at{}".format(*s))
+def test_view_of_rows_equals_the_dense_copy(dtype, shape):
+    """The kernels that read the view do the arithmetic of the (B,C,L) kernels in the same order: y and dx equal
+    those of a dense copy of the view bit for bit; the sums for dweight and dbias are taken in another order."""
+    from ssm_amd import ops
+    batch, length, chans, wide, offset = shape
+    proj, w, b, go, view = _rows_case(batch, length, chans, wide, 4, seed=7, dtype=dtype, offset=offset)
+    proj, w, b, go = proj.cuda(), w.cuda(), b.cuda(), go.cuda()
+    x = view(proj)
+    assert ops._conv_rows_view(x, True, 4) is not None
+    y = ops._conv_forward(x, w, b, "silu")
+    dx, dw, db = ops._conv_backward(go, x, w, b, "silu")
+    xd = x.contiguous()
+    yd = ops._conv_forward(xd, w, b, "silu")
+    dxd, dwd, dbd = ops._conv_backward(go, xd, w, b, "silu")
+    assert y.is_contiguous() and dx.shape == x.shape and dx.stride() == (length * chans, 1, chans)
+    assert torch.equal(y, yd)
+    assert torch.equal(dx, dxd)
+    scale = float(length * batch) ** 0.5
+    tol = 1e-5 if dtype == torch.float32 else 1e-4      # two orders of summing the same fp32 terms
+    torch.testing.assert_close(dw, dwd, rtol=1e-4, atol=tol * scale)
+    torch.testing.assert_close(db, dbd, rtol=1e-4, atol=tol * scale)
