@@ -23,25 +23,26 @@ constexpr int CONV_TAPS = 5;           // widest kernel the vector paths take (K
 constexpr int CONV_THREADS = 256;
 
 // Taps in reverse order: wrev[m] multiplies x[t - m]; zero beyond the kernel width.
-__device__ __forceinline__ void load_taps(const float *w, int c, int K, float (&wrev)[CONV_TAPS]) {
+template <int TAPS>
+__device__ __forceinline__ void load_taps(const float *w, int c, int K, float (&wrev)[TAPS]) {
 #pragma unroll
-  for (int m = 0; m < CONV_TAPS; ++m) wrev[m] = m < K ? w[(size_t)c * K + (K - 1 - m)] : 0.0f;
+  for (int m = 0; m < TAPS; ++m) wrev[m] = m < K ? w[(size_t)c * K + (K - 1 - m)] : 0.0f;
 }
 
 // The taps and the bias of VEC neighbouring channels from channel c0 on.  `wide`: the kernel is 4 wide and weight and
 // bias start on 16-byte boundaries, c0 is a multiple of VEC: one 16-byte read per channel and one read for the
 // biases instead of five 4-byte reads per channel (a thread that owns 8 steps of 4 channels otherwise issues more
 // reads for its taps than for its rows).
-template <int VEC>
+template <int VEC, int TAPS>
 __device__ __forceinline__ void load_taps_of(const float *w, const float *b, int c0, int K, bool wide,
-                                             float (&wrev)[VEC][CONV_TAPS], float (&bias)[VEC]) {
+                                             float (&wrev)[VEC][TAPS], float (&bias)[VEC]) {
   if (wide) {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       const Pack<float, 4> q = *reinterpret_cast<const Pack<float, 4> *>(w + (size_t)(c0 + i) * 4);
       wrev[i][0] = q.v[3]; wrev[i][1] = q.v[2]; wrev[i][2] = q.v[1]; wrev[i][3] = q.v[0];
 #pragma unroll
-      for (int m = 4; m < CONV_TAPS; ++m) wrev[i][m] = 0.0f;
+      for (int m = 4; m < TAPS; ++m) wrev[i][m] = 0.0f;
     }
     if (b) {
       const Pack<float, VEC> q = *reinterpret_cast<const Pack<float, VEC> *>(b + c0);
@@ -100,16 +101,16 @@ __device__ __forceinline__ void store_vec(T *row, int t, const float (&v)[VEC]) 
 
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
 // number of vectors; otherwise the same kernel reads and writes element by element.
-template <typename T, bool AL>
+template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvParams p) {
   constexpr int VEC = 16 / sizeof(T);
   const int row = blockIdx.x;                       // b * C + c
   const int c = row % p.chans;
   const T *xr = reinterpret_cast<const T *>(p.x) + (size_t)row * p.len;
   T *yr = reinterpret_cast<T *>(p.y) + (size_t)row * p.len;
-  float wrev1[1][CONV_TAPS], bias1[1];
-  load_taps_of<1>(p.w, p.bias, c, p.K, p.wide_taps, wrev1, bias1);
-  const float (&wrev)[CONV_TAPS] = wrev1[0];
+  float wrev1[1][TAPS], bias1[1];
+  load_taps_of<1, TAPS>(p.w, p.bias, c, p.K, p.wide_taps, wrev1, bias1);
+  const float (&wrev)[TAPS] = wrev1[0];
   const float bias = bias1[0];
   for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
     float win[2 * VEC];
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cf_kernel(const ConvPar
     for (int i = 0; i < VEC; ++i) {
       float acc = bias;
 #pragma unroll
-      for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[m], win[VEC + i - m], acc);
+      for (int m = 0; m < TAPS; ++m) acc = __builtin_fmaf(wrev[m], win[VEC + i - m], acc);
       out[i] = p.silu ? silu_f32(acc) : acc;
     }
     if constexpr (AL) store_vec<T, VEC>(yr, t0, out);
@@ -176,7 +177,7 @@ constexpr int CONV_CL_STRIP = 16;   // time steps per thread
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
 // number of vectors; otherwise the same kernel reads and writes element by element.
 constexpr int CONV_CL_FWD_BYTES = 8;   // bytes of channels per thread
-template <typename T, bool AL>
+template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvParams p) {
   constexpr int VEC = CONV_CL_FWD_BYTES / sizeof(T);
   const int cvecs = (p.chans + VEC - 1) / VEC;
@@ -190,9 +191,9 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
   const int c0 = cv * VEC;
   const int cw = min(VEC, p.chans - c0);          // channels of this vector that exist
   const int K = p.K;
-  constexpr int HIST = CONV_TAPS - 1;
-  float wrev[VEC][CONV_TAPS], bias[VEC];
-  if constexpr (AL) load_taps_of<VEC>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
+  constexpr int HIST = TAPS - 1;
+  float wrev[VEC][TAPS], bias[VEC];
+  if constexpr (AL) load_taps_of<VEC, TAPS>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
   else {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -228,7 +229,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
       for (int i = 0; i < VEC; ++i) {
         float acc = bias[i];
 #pragma unroll
-        for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + s - m].v[i]), acc);
+        for (int m = 0; m < TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + s - m].v[i]), acc);
         out[i] = p.silu ? silu_f32(acc) : acc;
       }
       store_vec<T, VEC>(yb + (size_t)(t_begin + s) * p.chans, 0, out);
@@ -278,10 +279,10 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_fwd_cl_kernel(const ConvPar
 // in time.
 constexpr int CONV_CL_WALK = 4, CONV_CL_WALK_STRIP = 8;   // strips of 8 steps: 24.1 us against 25.4 with 16 and 27.9 with 32
 constexpr int CONV_CL_WALK_THREADS = 64;
-template <typename T>
+template <typename T, int TAPS>
 __global__ __launch_bounds__(CONV_CL_WALK_THREADS) void conv_fwd_cl_walk_kernel(const ConvParams p) {
   constexpr int VEC = CONV_CL_FWD_BYTES / sizeof(T);
-  constexpr int HIST = CONV_TAPS - 1, S = CONV_CL_WALK_STRIP, SPAN = CONV_CL_WALK_STRIP * CONV_CL_WALK;
+  constexpr int HIST = TAPS - 1, S = CONV_CL_WALK_STRIP, SPAN = CONV_CL_WALK_STRIP * CONV_CL_WALK;
   const int cvecs = p.chans / VEC;
   const int spans = (p.len + SPAN - 1) / SPAN;
   const size_t total = (size_t)p.batch * spans * cvecs;
@@ -291,8 +292,8 @@ __global__ __launch_bounds__(CONV_CL_WALK_THREADS) void conv_fwd_cl_walk_kernel(
   const int span = (int)((gid / cvecs) % spans);
   const int b = (int)(gid / ((size_t)cvecs * spans));
   const int c0 = cv * VEC;
-  float wrev[VEC][CONV_TAPS], bias[VEC];
-  load_taps_of<VEC>(p.w, p.bias, c0, p.K, p.wide_taps, wrev, bias);
+  float wrev[VEC][TAPS], bias[VEC];
+  load_taps_of<VEC, TAPS>(p.w, p.bias, c0, p.K, p.wide_taps, wrev, bias);
   const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
   T *yb = reinterpret_cast<T *>(p.y) + (size_t)b * p.len * p.chans + c0;
   const int t_first = span * SPAN;
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(CONV_CL_WALK_THREADS) void conv_fwd_cl_walk_kernel(
       for (int i = 0; i < VEC; ++i) {
         float acc = bias[i];
 #pragma unroll
-        for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + sidx - m].v[i]), acc);
+        for (int m = 0; m < TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + sidx - m].v[i]), acc);
         out[i] = p.silu ? silu_f32(acc) : acc;
       }
       if (t_begin + sidx < p.len) store_vec<T, VEC>(yb + (size_t)(t_begin + sidx) * p.chans, 0, out);
@@ -341,23 +342,23 @@ __global__ __launch_bounds__(CONV_CL_WALK_THREADS) void conv_fwd_cl_walk_kernel(
 
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
 // number of vectors; otherwise the same kernel reads and writes element by element.
-template <typename T, bool AL>
+template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvParams p) {
   constexpr int VEC = 16 / sizeof(T);
-  __shared__ float red[CONV_THREADS / WAVE][CONV_TAPS + 1];
+  __shared__ float red[CONV_THREADS / WAVE][TAPS + 1];
   const int row = blockIdx.x;
   const int c = row % p.chans;
   const int K = p.K;
   const T *xr = reinterpret_cast<const T *>(p.x) + (size_t)row * p.len;
   const T *gr = reinterpret_cast<const T *>(p.dout) + (size_t)row * p.len;
   T *dxr = reinterpret_cast<T *>(p.y) + (size_t)row * p.len;
-  float wrev1[1][CONV_TAPS], bias1[1];
-  load_taps_of<1>(p.w, p.bias, c, K, p.wide_taps, wrev1, bias1);
-  const float (&wrev)[CONV_TAPS] = wrev1[0];
+  float wrev1[1][TAPS], bias1[1];
+  load_taps_of<1, TAPS>(p.w, p.bias, c, K, p.wide_taps, wrev1, bias1);
+  const float (&wrev)[TAPS] = wrev1[0];
   const float bias = bias1[0];
-  float dwrev[CONV_TAPS], db = 0.0f;
+  float dwrev[TAPS], db = 0.0f;
 #pragma unroll
-  for (int m = 0; m < CONV_TAPS; ++m) dwrev[m] = 0.0f;
+  for (int m = 0; m < TAPS; ++m) dwrev[m] = 0.0f;
 
   for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
     // x over [t0-VEC, t0+2*VEC), dout over [t0, t0+2*VEC)
@@ -403,7 +404,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
         if (i < VEC + K - 1) {
           float pre = bias;
 #pragma unroll
-          for (int m = 0; m < CONV_TAPS; ++m) pre = __builtin_fmaf(wrev[m], xw[VEC + i - m], pre);
+          for (int m = 0; m < TAPS; ++m) pre = __builtin_fmaf(wrev[m], xw[VEC + i - m], pre);
           g[i] *= silu_grad(pre);
         }
       }
@@ -413,11 +414,11 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
     for (int i = 0; i < VEC; ++i) {
       float acc = 0.0f;
 #pragma unroll
-      for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(g[i + m], wrev[m], acc);
+      for (int m = 0; m < TAPS; ++m) acc = __builtin_fmaf(g[i + m], wrev[m], acc);
       dx[i] = acc;
       db += g[i];
 #pragma unroll
-      for (int m = 0; m < CONV_TAPS; ++m) dwrev[m] = __builtin_fmaf(g[i], xw[VEC + i - m], dwrev[m]);
+      for (int m = 0; m < TAPS; ++m) dwrev[m] = __builtin_fmaf(g[i], xw[VEC + i - m], dwrev[m]);
     }
     if constexpr (AL) store_vec<T, VEC>(dxr, t0, dx);
     else store_run<T, VEC>(dxr, t0, p.len, AL, dx);
@@ -425,18 +426,18 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
   // block reduction of dw[0..K) and db
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 #pragma unroll
-  for (int m = 0; m < CONV_TAPS; ++m) {
+  for (int m = 0; m < TAPS; ++m) {
     const float s = wave_sum(dwrev[m]);
     if (lane == 0) red[wave][m] = s;
   }
   {
     const float s = wave_sum(db);
-    if (lane == 0) red[wave][CONV_TAPS] = s;
+    if (lane == 0) red[wave][TAPS] = s;
   }
   __syncthreads();
   if (threadIdx.x <= K) {
     // slot k < K holds dw[k] = dwrev[K-1-k]; slot K holds dbias
-    const int src = threadIdx.x < K ? (K - 1 - (int)threadIdx.x) : CONV_TAPS;
+    const int src = threadIdx.x < K ? (K - 1 - (int)threadIdx.x) : TAPS;
     float s = 0.0f;
     for (int wv = 0; wv < CONV_THREADS / WAVE; ++wv) s += red[wv][src];
     p.partial[(size_t)row * (K + 1) + threadIdx.x] = s;
@@ -458,10 +459,10 @@ __host__ __device__ inline int conv_cl_seg_len(int len) {
 // AL: rows (channel vectors) start on 16-byte boundaries and the row length (channel count) is a whole
 // number of vectors; otherwise the same kernel reads and writes element by element.
 constexpr int CONV_CL_BWD_BYTES = 4;   // bytes of channels per thread: the walk keeps ~20 values per channel in registers
-template <typename T, bool AL>
+template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvParams p) {
   constexpr int VEC = CONV_CL_BWD_BYTES / sizeof(T);
-  constexpr int HIST = CONV_TAPS - 1;
+  constexpr int HIST = TAPS - 1;
   const int cvecs = (p.chans + VEC - 1) / VEC;
   const int seg_len = conv_cl_seg_len(p.len);
   const int nseg = (p.len + seg_len - 1) / seg_len;
@@ -474,8 +475,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
   const int c0 = cv * VEC;
   const int cw = min(VEC, p.chans - c0);          // channels of this vector that exist
   const int K = p.K;
-  float wrev[VEC][CONV_TAPS], bias[VEC], dwr[VEC][CONV_TAPS], db[VEC];
-  if constexpr (AL) load_taps_of<VEC>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
+  float wrev[VEC][TAPS], bias[VEC], dwr[VEC][TAPS], db[VEC];
+  if constexpr (AL) load_taps_of<VEC, TAPS>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
   else {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -487,7 +488,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
   for (int i = 0; i < VEC; ++i) {
     db[i] = 0.0f;
 #pragma unroll
-    for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = 0.0f;
+    for (int m = 0; m < TAPS; ++m) dwr[i][m] = 0.0f;
   }
   const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.len * p.chans + c0;
   const T *gb = reinterpret_cast<const T *>(p.dout) + (size_t)b * p.len * p.chans + c0;
@@ -495,7 +496,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
   const int t_begin = seg * seg_len;
   const int t_end = min(p.len, t_begin + seg_len);
   // xh[j] = x at time (t - 1 - j), gh[m] = g at time (t - 1 - m) once the step's own values are pushed
-  float xh[HIST][VEC], gh[CONV_TAPS][VEC];
+  float xh[HIST][VEC], gh[TAPS][VEC];
 #pragma unroll
   for (int j = 0; j < HIST; ++j) {
     const int ts = t_begin - 1 - j;
@@ -509,7 +510,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
     for (int i = 0; i < VEC; ++i) xh[j][i] = v[i];
   }
 #pragma unroll
-  for (int m = 0; m < CONV_TAPS; ++m)
+  for (int m = 0; m < TAPS; ++m)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) gh[m][i] = 0.0f;
 
@@ -545,7 +546,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
     }
     // push: gh[0] = g_t ... gh[3] = g_{t-3};  xh[0] = x_t ...
 #pragma unroll
-    for (int m = CONV_TAPS - 1; m > 0; --m)
+    for (int m = TAPS - 1; m > 0; --m)
 #pragma unroll
       for (int i = 0; i < VEC; ++i) gh[m][i] = gh[m - 1][i];
 #pragma unroll
@@ -564,7 +565,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
       for (int i = 0; i < VEC; ++i) {
         float acc = 0.0f;
 #pragma unroll
-        for (int j = 0; j < CONV_TAPS; ++j) acc = __builtin_fmaf(gh[HIST - j][i], wrev[i][j], acc);
+        for (int j = 0; j < TAPS; ++j) acc = __builtin_fmaf(gh[HIST - j][i], wrev[i][j], acc);
         out[i] = acc;
       }
       store_run<T, VEC>(dxb + (size_t)td * p.chans, 0, cw, AL, out);
@@ -612,7 +613,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
     if (i >= cw) break;
     float *part = p.partial + (((size_t)b * nseg + seg) * p.chans + c0 + i) * (K + 1);
 #pragma unroll
-    for (int m = 0; m < CONV_TAPS; ++m)
+    for (int m = 0; m < TAPS; ++m)
       if (m < K) part[K - 1 - m] = dwr[i][m];
     part[K] = db[i];
   }
@@ -638,9 +639,9 @@ constexpr int CONV_TR_FWD_THREADS = (CONV_TR_CH / CONV_TR_FWD_VEC) * (CONV_TR_FW
 static_assert((CONV_TR_CH / CONV_TR_BWD_VEC) * (CONV_TR_BWD_STEPS / CONV_TR_STRIP) == CONV_TR_THREADS, "backward tile");
 
 // AL: the rows of y (L elements each) start on 16-byte boundaries and L is a whole number of 16-byte units.
-template <typename T, bool AL>
+template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_TR_FWD_THREADS) void conv_fwd_tr_kernel(const ConvParams p) {
-  constexpr int CH = CONV_TR_CH, TT = CONV_TR_FWD_STEPS, S = CONV_TR_STRIP, VEC = CONV_TR_FWD_VEC, HIST = CONV_TAPS - 1;
+  constexpr int CH = CONV_TR_CH, TT = CONV_TR_FWD_STEPS, S = CONV_TR_STRIP, VEC = CONV_TR_FWD_VEC, HIST = TAPS - 1;
   constexpr int UNIT = 16 / sizeof(T), UPR = TT / UNIT, UPS = S / UNIT;   // elements per unit, units per row / strip
   constexpr int GROUPS = CH / VEC;
   __shared__ __attribute__((aligned(16))) T tile[CH * TT];
@@ -653,8 +654,8 @@ __global__ __launch_bounds__(CONV_TR_FWD_THREADS) void conv_fwd_tr_kernel(const 
   const int c_own = ct * CH + cg * VEC;
   const int c0 = c_own < p.chans ? c_own : 0;        // the channel count is a multiple of VEC: a group is all in or all out
   const int t0 = tt * TT + ts * S;
-  float wrev[VEC][CONV_TAPS], bias[VEC];
-  load_taps_of<VEC>(p.w, p.bias, c0, p.K, p.wide_taps, wrev, bias);
+  float wrev[VEC][TAPS], bias[VEC];
+  load_taps_of<VEC, TAPS>(p.w, p.bias, c0, p.K, p.wide_taps, wrev, bias);
   const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.x_bs + c0;
   Pack<T, VEC> raw[HIST + S];
 #pragma unroll
@@ -674,7 +675,7 @@ __global__ __launch_bounds__(CONV_TR_FWD_THREADS) void conv_fwd_tr_kernel(const 
     for (int sidx = 0; sidx < S; ++sidx) {
       float acc = bias[i];
 #pragma unroll
-      for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + sidx - m].v[i]), acc);
+      for (int m = 0; m < TAPS; ++m) acc = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + sidx - m].v[i]), acc);
       col[sidx / UNIT].v[sidx % UNIT] = from_f32<T>(p.silu ? silu_f32(acc) : acc);
     }
     const int r = cg * VEC + i;
@@ -710,15 +711,15 @@ __host__ __device__ inline int conv_tr_seg_tiles(int len) {
   return (tiles + CONV_CL_SEGS - 1) / CONV_CL_SEGS;
 }
 
-template <typename T, bool AL>
+template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const ConvParams p) {
-  constexpr int CH = CONV_TR_CH, TT = CONV_TR_BWD_STEPS, S = CONV_TR_STRIP, VEC = CONV_TR_BWD_VEC, HIST = CONV_TAPS - 1;
+  constexpr int CH = CONV_TR_CH, TT = CONV_TR_BWD_STEPS, S = CONV_TR_STRIP, VEC = CONV_TR_BWD_VEC, HIST = TAPS - 1;
   constexpr int UNIT = 16 / sizeof(T), UPR = TT / UNIT, UPS = S / UNIT;
   constexpr int GU = (S + HIST + UNIT - 1) / UNIT;      // units of dout a thread takes: its strip and 4 steps on
   constexpr int GROUPS = CH / VEC, GROUPS_PER_WAVE = GROUPS < WAVE ? GROUPS : WAVE;
   __shared__ __attribute__((aligned(16))) T gt[CH * TT];       // the tile's units, swizzled
   __shared__ __attribute__((aligned(16))) T gnext[CH * UNIT];  // per channel, the unit beyond the tile
-  __shared__ float red[CONV_TR_THREADS / WAVE][CH][CONV_TAPS + 1];
+  __shared__ float red[CONV_TR_THREADS / WAVE][CH][TAPS + 1];
   const int ttiles = (p.len + TT - 1) / TT, ctiles = (p.chans + CH - 1) / CH;
   const int seg_tiles = conv_tr_seg_tiles(p.len);
   const int nseg = (ttiles + seg_tiles - 1) / seg_tiles;
@@ -731,13 +732,13 @@ __global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const Conv
   const bool c_in = c_own < p.chans;
   const int c0 = c_in ? c_own : 0;
   const int K = p.K;
-  float wrev[VEC][CONV_TAPS], bias[VEC], dwr[VEC][CONV_TAPS], db[VEC];
-  load_taps_of<VEC>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
+  float wrev[VEC][TAPS], bias[VEC], dwr[VEC][TAPS], db[VEC];
+  load_taps_of<VEC, TAPS>(p.w, p.bias, c0, K, p.wide_taps, wrev, bias);
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
     db[i] = 0.0f;
 #pragma unroll
-    for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = 0.0f;
+    for (int m = 0; m < TAPS; ++m) dwr[i][m] = 0.0f;
   }
   const T *xb = reinterpret_cast<const T *>(p.x) + (size_t)b * p.x_bs + c0;
   const T *gb = reinterpret_cast<const T *>(p.dout) + (size_t)b * p.chans * p.len;
@@ -797,7 +798,7 @@ __global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const Conv
         if (p.silu && t0 + j < p.len) {
           float pre = bias[i];
 #pragma unroll
-          for (int m = 0; m < CONV_TAPS; ++m) pre = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + j - m].v[i]), pre);
+          for (int m = 0; m < TAPS; ++m) pre = __builtin_fmaf(wrev[i][m], to_f32(raw[HIST + j - m].v[i]), pre);
           g[j] *= silu_grad(pre);
         }
       }
@@ -805,11 +806,11 @@ __global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const Conv
       for (int sidx = 0; sidx < S; ++sidx) {
         float acc = 0.0f;
 #pragma unroll
-        for (int m = 0; m < CONV_TAPS; ++m) acc = __builtin_fmaf(g[sidx + m], wrev[i][m], acc);
+        for (int m = 0; m < TAPS; ++m) acc = __builtin_fmaf(g[sidx + m], wrev[i][m], acc);
         out[sidx].v[i] = from_f32<T>(acc);
         db[i] += g[sidx];
 #pragma unroll
-        for (int m = 0; m < CONV_TAPS; ++m) dwr[i][m] = __builtin_fmaf(g[sidx], to_f32(raw[HIST + sidx - m].v[i]), dwr[i][m]);
+        for (int m = 0; m < TAPS; ++m) dwr[i][m] = __builtin_fmaf(g[sidx], to_f32(raw[HIST + sidx - m].v[i]), dwr[i][m]);
       }
     }
     if (c_in) {
@@ -824,8 +825,8 @@ __global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const Conv
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
 #pragma unroll
-    for (int m = 0; m <= CONV_TAPS; ++m) {
-      float s = m < CONV_TAPS ? dwr[i][m] : db[i];
+    for (int m = 0; m <= TAPS; ++m) {
+      float s = m < TAPS ? dwr[i][m] : db[i];
 #pragma unroll
       for (int d = GROUPS_PER_WAVE; d < WAVE; d *= 2) s += __shfl_xor(s, d);
       if (lane < GROUPS_PER_WAVE) red[wave][cg * VEC + i][m] = s;
@@ -836,7 +837,7 @@ __global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const Conv
     const int r = e / (K + 1), k = e % (K + 1);
     const int c = ct * CH + r;
     if (c >= p.chans) continue;
-    const int src = k < K ? K - 1 - k : CONV_TAPS;        // slot k < K holds dw[k] = dwrev[K-1-k]; slot K the bias sum
+    const int src = k < K ? K - 1 - k : TAPS;        // slot k < K holds dw[k] = dwrev[K-1-k]; slot K the bias sum
     float s = 0.0f;
 #pragma unroll
     for (int wv = 0; wv < CONV_TR_THREADS / WAVE; ++wv) s += red[wv][r][src];
@@ -917,6 +918,15 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_fold_kernel(const float
   }
 }
 
+// Every vector kernel exists for 4 and for 5 taps: the widths up to 4 (4 is what the models use) skip the fifth
+// multiply-add of each sum and, backward, the fourth step of look-ahead.
+#define CONV_LAUNCH(kernel, targs, grid, block)                                                        \
+  do {                                                                                                 \
+    if (p.K <= 4) hipLaunchKernelGGL((kernel<targs, 4>), grid, block, 0, s, p);                        \
+    else hipLaunchKernelGGL((kernel<targs, 5>), grid, block, 0, s, p);                                 \
+  } while (0)
+#define CONV_T_AL(al) T, al
+
 template <typename T>
 static int conv_fwd_typed(const ConvParams &p, int layout, bool vec_ok, hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
@@ -924,11 +934,11 @@ static int conv_fwd_typed(const ConvParams &p, int layout, bool vec_ok, hipStrea
   const int channels_last = layout == SSM_LAYOUT_BLC;
   if (layout == SSM_LAYOUT_ROWS_TO_BCL) {
     const size_t blocks = (size_t)p.batch * ((p.chans + CONV_TR_CH - 1) / CONV_TR_CH) * ((p.len + CONV_TR_FWD_STEPS - 1) / CONV_TR_FWD_STEPS);
-    if (p.len % VEC == 0) hipLaunchKernelGGL((conv_fwd_tr_kernel<T, true>), dim3((unsigned)blocks), dim3(CONV_TR_FWD_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((conv_fwd_tr_kernel<T, false>), dim3((unsigned)blocks), dim3(CONV_TR_FWD_THREADS), 0, s, p);
+    if (p.len % VEC == 0) CONV_LAUNCH(conv_fwd_tr_kernel, CONV_T_AL(true), dim3((unsigned)blocks), dim3(CONV_TR_FWD_THREADS));
+    else CONV_LAUNCH(conv_fwd_tr_kernel, CONV_T_AL(false), dim3((unsigned)blocks), dim3(CONV_TR_FWD_THREADS));
   } else if (p.K <= CONV_TAPS && !channels_last) {
-    if (vec_ok && p.len % VEC == 0) hipLaunchKernelGGL((conv_fwd_cf_kernel<T, true>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((conv_fwd_cf_kernel<T, false>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+    if (vec_ok && p.len % VEC == 0) CONV_LAUNCH(conv_fwd_cf_kernel, CONV_T_AL(true), dim3(p.batch * p.chans), dim3(CONV_THREADS));
+    else CONV_LAUNCH(conv_fwd_cf_kernel, CONV_T_AL(false), dim3(p.batch * p.chans), dim3(CONV_THREADS));
   } else if (p.K <= CONV_TAPS && channels_last) {
     const int strips = (p.len + CONV_CL_STRIP - 1) / CONV_CL_STRIP;
     constexpr int VECF = CONV_CL_FWD_BYTES / sizeof(T);
@@ -938,9 +948,9 @@ static int conv_fwd_typed(const ConvParams &p, int layout, bool vec_ok, hipStrea
       const int spans = (p.len + CONV_CL_WALK_STRIP * CONV_CL_WALK - 1) / (CONV_CL_WALK_STRIP * CONV_CL_WALK);
       const size_t walkers = (size_t)p.batch * spans * (p.chans / VECF);
       const dim3 wgrid((unsigned)((walkers + CONV_CL_WALK_THREADS - 1) / CONV_CL_WALK_THREADS));
-      hipLaunchKernelGGL(conv_fwd_cl_walk_kernel<T>, wgrid, dim3(CONV_CL_WALK_THREADS), 0, s, p);
-    } else if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_fwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((conv_fwd_cl_kernel<T, false>), grid, dim3(CONV_THREADS), 0, s, p);
+      CONV_LAUNCH(conv_fwd_cl_walk_kernel, T, wgrid, dim3(CONV_CL_WALK_THREADS));
+    } else if (vec_ok && p.chans % VEC == 0) CONV_LAUNCH(conv_fwd_cl_kernel, CONV_T_AL(true), grid, dim3(CONV_THREADS));
+    else CONV_LAUNCH(conv_fwd_cl_kernel, CONV_T_AL(false), grid, dim3(CONV_THREADS));
   } else {
     const unsigned grid = (unsigned)min((size_t)65535 * 16, (total + CONV_THREADS - 1) / CONV_THREADS);
     hipLaunchKernelGGL(conv_fwd_generic_kernel<T>, dim3(grid), dim3(CONV_THREADS), 0, s, p, channels_last);
@@ -959,20 +969,20 @@ static int conv_bwd_typed(const ConvParams &p, int layout, bool vec_ok, float *d
     const int ttiles = (p.len + CONV_TR_BWD_STEPS - 1) / CONV_TR_BWD_STEPS, seg_tiles = conv_tr_seg_tiles(p.len);
     const int nseg = (ttiles + seg_tiles - 1) / seg_tiles;
     const size_t blocks = (size_t)p.batch * ((p.chans + CONV_TR_CH - 1) / CONV_TR_CH) * nseg;
-    if (p.len % VEC == 0) hipLaunchKernelGGL((conv_bwd_tr_kernel<T, true>), dim3((unsigned)blocks), dim3(CONV_TR_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((conv_bwd_tr_kernel<T, false>), dim3((unsigned)blocks), dim3(CONV_TR_THREADS), 0, s, p);
+    if (p.len % VEC == 0) CONV_LAUNCH(conv_bwd_tr_kernel, CONV_T_AL(true), dim3((unsigned)blocks), dim3(CONV_TR_THREADS));
+    else CONV_LAUNCH(conv_bwd_tr_kernel, CONV_T_AL(false), dim3((unsigned)blocks), dim3(CONV_TR_THREADS));
     fold_count = p.batch * nseg;
   } else if (p.K <= CONV_TAPS && !channels_last) {
-    if (vec_ok && p.len % VEC == 0) hipLaunchKernelGGL((conv_bwd_cf_kernel<T, true>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((conv_bwd_cf_kernel<T, false>), dim3(p.batch * p.chans), dim3(CONV_THREADS), 0, s, p);
+    if (vec_ok && p.len % VEC == 0) CONV_LAUNCH(conv_bwd_cf_kernel, CONV_T_AL(true), dim3(p.batch * p.chans), dim3(CONV_THREADS));
+    else CONV_LAUNCH(conv_bwd_cf_kernel, CONV_T_AL(false), dim3(p.batch * p.chans), dim3(CONV_THREADS));
   } else if (p.K <= CONV_TAPS && channels_last) {
     const int seg_len = conv_cl_seg_len(p.len);
     const int nseg = (p.len + seg_len - 1) / seg_len;
     constexpr int VECB = CONV_CL_BWD_BYTES / sizeof(T);
     const size_t threads = (size_t)p.batch * nseg * ((p.chans + VECB - 1) / VECB);
     const dim3 grid((unsigned)((threads + CONV_THREADS - 1) / CONV_THREADS));
-    if (vec_ok && p.chans % VEC == 0) hipLaunchKernelGGL((conv_bwd_cl_kernel<T, true>), grid, dim3(CONV_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((conv_bwd_cl_kernel<T, false>), grid, dim3(CONV_THREADS), 0, s, p);
+    if (vec_ok && p.chans % VEC == 0) CONV_LAUNCH(conv_bwd_cl_kernel, CONV_T_AL(true), grid, dim3(CONV_THREADS));
+    else CONV_LAUNCH(conv_bwd_cl_kernel, CONV_T_AL(false), grid, dim3(CONV_THREADS));
     fold_count = p.batch * nseg;
   } else {
     const int rows = p.batch * p.chans;
@@ -986,6 +996,8 @@ static int conv_bwd_typed(const ConvParams &p, int layout, bool vec_ok, float *d
   SSM_CHECK_LAUNCH("ssm_conv1d_bwd(fold)");
   return SSM_OK;
 }
+#undef CONV_LAUNCH
+#undef CONV_T_AL
 
 static int conv_check(const char *who, const void *x, const void *w, const void *y, int batch, int chans, int len,
                       int K, int dtype, int layout, int act) {

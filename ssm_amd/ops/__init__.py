@@ -764,16 +764,26 @@ def _conv_rows_view(x, channels_first, width):
     """Whether ``x (B, C, L)`` is a view whose memory runs channels innermost -- what the reference's blocks pass
     (src/ssm/modules/mamba1.py:209-215, mamba2.py:159-165: ``projected.permute(0, 2, 1)``, in the first one half of
     a wider projection) -- in a form the kernels read as it lies: -> (batch stride, row stride) in elements, or
-    None (the caller then takes a dense copy)."""
-    if not channels_first or x.is_contiguous() or x.dtype == torch.float64:
+    None (the caller then takes a dense copy).  A rule on shapes and strides only, so that the layout of the
+    results can be told without the data (fake tensors)."""
+    if not channels_first or x.dtype == torch.float64 or x.ndim != 3:
         return None
     batch, chans, length = x.shape
     sb, sc, sl = x.stride()
-    quad = 4 * x.element_size()
-    if (sc != 1 or chans % 4 or width > 5 or sl < chans or sl % 4 or sb % 4 or x.data_ptr() % quad
+    if (x.is_contiguous() or sc != 1 or chans % 4 or width > 5 or sl < chans or sl % 4 or sb % 4
             or (batch > 1 and sb < (length - 1) * sl + chans)):
         return None
     return int(sb), int(sl)
+
+
+def _conv_rows_input(x, rows):
+    """``x`` as the rows-in kernels take it: detached, and starting on a boundary of 4 elements (a view that starts
+    elsewhere is copied into rows of its own)."""
+    x = x.detach()
+    if x.data_ptr() % (4 * x.element_size()):
+        x = x.permute(0, 2, 1).contiguous().permute(0, 2, 1)
+        rows = (int(x.stride(0)), int(x.stride(2)))
+    return x, rows
 
 
 def _conv_forward(x, weight, bias, activation, channels_last=None):
@@ -786,7 +796,7 @@ def _conv_forward(x, weight, bias, activation, channels_last=None):
     wf, bf = _conv_weight_f32(weight), K.as_f32_vec(bias)
     rows = _conv_rows_view(x, channels_first, width)
     if rows is not None:
-        xc = x.detach()
+        xc, rows = _conv_rows_input(x, rows)
         y = torch.empty(x.shape, dtype=x.dtype, device=dev)
         layout, strides = _lib.LAYOUT_ROWS_TO_BCL, rows
     else:
@@ -815,7 +825,7 @@ def _conv_backward(grad_out, x, weight, bias, activation, channels_last=None):
     gc = K.cast_c(grad_out, x.dtype)
     rows = _conv_rows_view(x, channels_first, width)
     if rows is not None:
-        xc = x.detach()
+        xc, rows = _conv_rows_input(x, rows)
         dx_rows = torch.empty(batch, length, chans, dtype=x.dtype, device=dev)
         dx, dx_mem = dx_rows.permute(0, 2, 1), dx_rows
         layout, strides = _lib.LAYOUT_ROWS_TO_BCL, rows

@@ -72,7 +72,9 @@ for _name, _schema in _SCHEMAS.items():
 
 
 def _like(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
-    return None if t is None else torch.empty_like(t)
+    """A dense tensor of the shape and type of ``t``: what the operators return whatever the strides of ``t`` are
+    (a compiler plans the consumers of an output on the strides its fake promises)."""
+    return None if t is None else torch.empty_like(t, memory_format=torch.contiguous_format)
 
 
 # ------------------------------------------------------------------ implementations on the device
@@ -104,7 +106,7 @@ _IMPLS = {
 
 def _scan_meta(u, delta, A, B, C, D=None, z=None, dt_bias=None, softplus=False, return_last_state=False):
     last = u.new_empty((u.shape[0], u.shape[1], A.shape[1])) if return_last_state else u.new_empty(0)
-    return torch.empty_like(u), last
+    return _like(u), last
 
 
 def _scan_bwd_meta(grad_output, grad_last_state, u, delta, A, B, C, D=None, z=None, dt_bias=None, softplus=False):
@@ -112,7 +114,7 @@ def _scan_bwd_meta(grad_output, grad_last_state, u, delta, A, B, C, D=None, z=No
 
 
 def _step_meta(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, softplus=True):
-    return torch.empty_like(x)
+    return _like(x)
 
 
 def _step_bwd_meta(grad_output, grad_state, state, x, dt, A, B, C, D=None, z=None, dt_bias=None, softplus=True):
@@ -120,7 +122,7 @@ def _step_bwd_meta(grad_output, grad_state, state, x, dt, A, B, C, D=None, z=Non
 
 
 def _chunk_meta(X, dt, A, B, C, chunk_size, D=None, z=None, seq_lens=None, cu_seqlens=None, initial_states=None):
-    return torch.empty_like(X)
+    return _like(X)
 
 
 def _chunk_bwd_meta(grad_output, X, dt, A, B, C, chunk_size, D=None, z=None, seq_lens=None, cu_seqlens=None,
@@ -129,15 +131,23 @@ def _chunk_bwd_meta(grad_output, X, dt, A, B, C, chunk_size, D=None, z=None, seq
 
 
 def _conv_meta(x, weight, bias=None, activation="silu"):
-    return torch.empty_like(x)
+    return _like(x)
 
 
 def _conv_bwd_meta(grad_output, x, weight, bias=None, activation="silu"):
-    return _like(x), _like(weight), _like(bias)
+    # the gradient of a (B, C, L) view of rows of channels lies in rows of channels itself (ops._conv_backward)
+    w = weight[:, 0, :] if weight.ndim == 3 else weight
+    channels_first = x.ndim == 3 and x.shape[1] == w.shape[0]
+    from .ops import _conv_rows_view
+    if _conv_rows_view(x, channels_first, int(w.shape[-1])) is not None:
+        dx = x.new_empty((x.shape[0], x.shape[2], x.shape[1])).permute(0, 2, 1)
+    else:
+        dx = _like(x)
+    return dx, _like(weight), _like(bias)
 
 
 def _norm_meta(x, weight, bias=None, residual=None, is_rms=False, eps=1e-5, prenorm=True, residual_in_fp32=True):
-    return torch.empty_like(x)
+    return _like(x)
 
 
 def _norm_bwd_meta(grad_output, x, weight, bias=None, residual=None, is_rms=False, eps=1e-5, prenorm=True,

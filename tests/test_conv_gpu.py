@@ -232,3 +232,21 @@ def test_view_of_rows_equals_the_dense_copy(dtype, shape):
     tol = 1e-5 if dtype == torch.float32 else 1e-4      # two orders of summing the same fp32 terms
     torch.testing.assert_close(dw, dwd, rtol=1e-4, atol=tol * scale)
     torch.testing.assert_close(db, dbd, rtol=1e-4, atol=tol * scale)
+
+
+def test_view_of_rows_that_starts_off_a_boundary_of_four_channels():
+    """Channels 2..65 of a projection: the strides are what the kernels take, the start is not; the call copies the
+    view into rows of its own and still returns dx in rows."""
+    from ssm_amd import ops
+    proj, w, b, go, view = _rows_case(2, 200, 64, 128, 4, seed=3, dtype=torch.bfloat16, offset=2)
+    proj, w, b, go = proj.cuda(), w.cuda(), b.cuda(), go.cuda()
+    x = view(proj)
+    assert ops._conv_rows_view(x, True, 4) is not None and x.data_ptr() % 8 != 0
+    y = ops._conv_forward(x, w, b, "silu")
+    dx, dw, db = ops._conv_backward(go, x, w, b, "silu")
+    xd = x.contiguous()
+    assert torch.equal(y, ops._conv_forward(xd, w, b, "silu"))
+    dxd, dwd, dbd = ops._conv_backward(go, xd, w, b, "silu")
+    assert torch.equal(dx, dxd) and dx.stride() == (200 * 64, 1, 64)
+    torch.testing.assert_close(dw, dwd, rtol=1e-4, atol=1e-2)
+    torch.testing.assert_close(db, dbd, rtol=1e-4, atol=1e-2)

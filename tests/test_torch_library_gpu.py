@@ -153,3 +153,33 @@ def test_a_traced_graph_holds_one_node_per_operator_call():
     assert torch.equal(out, eager)
     for a, b in zip(torch.autograd.grad(out.square().sum(), args), grads):
         assert torch.equal(a, b)
+
+
+def test_fake_outputs_promise_the_strides_the_kernels_produce():
+    """A compiler plans the consumers of an operator's output on the strides of its fake: for inputs that are views
+    (a permuted projection, a half of a wider one, an expanded parameter) the fakes must still describe what comes
+    back -- dense tensors, except the convolution's gradient of a view of rows, which lies in rows itself."""
+    g = torch.Generator().manual_seed(11)
+    wide = torch.randn(2, 96, 128, generator=g).to(torch.bfloat16).cuda()
+    w, b = torch.randn(64, 4, generator=g).cuda(), torch.randn(64, generator=g).cuda()
+    views = {"permuted half": wide[:, :, :64].permute(0, 2, 1), "permuted": wide.permute(0, 2, 1)[:, :64],
+             "6 channels (copied)": wide[:, :, :6].permute(0, 2, 1), "dense": wide[:, :, :64].permute(0, 2, 1).contiguous()}
+    for name, x in views.items():
+        ww, bb = (w, b) if x.shape[1] == 64 else (w[:6].contiguous(), b[:6].contiguous())
+        meta = lambda t: torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device="meta")
+        y = torch.ops.ssm_amd.dw_causal_conv(x, ww, bb, "silu")
+        ym = torch.ops.ssm_amd.dw_causal_conv(meta(x), meta(ww), meta(bb), "silu")
+        assert y.stride() == ym.stride() and y.shape == ym.shape, name
+        go = torch.randn_like(y)
+        real = torch.ops.ssm_amd.dw_causal_conv_backward(go, x, ww, bb, "silu")
+        fake = torch.ops.ssm_amd.dw_causal_conv_backward(meta(go), meta(x), meta(ww), meta(bb), "silu")
+        for r, f in zip(real, fake):
+            assert r.shape == f.shape and r.stride() == f.stride() and r.dtype == f.dtype, name
+    # the scan on views: outputs and gradients are dense whatever the inputs' strides
+    inp = make_inputs(7, 2, 16, 272, 16, dtype=torch.bfloat16)
+    u = inp["u"].cuda().transpose(1, 2).contiguous().transpose(1, 2)          # (B, D, L) view of (B, L, D) memory
+    rest = [inp[k].cuda() for k in ("delta", "A", "B", "C", "D", "z", "dt_bias")]
+    meta = lambda t: torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device="meta")
+    y, _ = torch.ops.ssm_amd.selective_scan(u, *rest, True, False)
+    ym, _ = torch.ops.ssm_amd.selective_scan(meta(u), *[meta(t) for t in rest], True, False)
+    assert y.stride() == ym.stride() and y.is_contiguous()
