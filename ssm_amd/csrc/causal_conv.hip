@@ -21,6 +21,7 @@ namespace ssm {
 
 constexpr int CONV_TAPS = 5;           // widest kernel the vector paths take (K <= 5)
 constexpr int CONV_THREADS = 256;
+constexpr int CONV_WHOLE_BATCH_MIN_CHANNELS = 1024;   // (B,C,L) backward: from here on a workgroup per channel
 
 // Taps in reverse order: wrev[m] multiplies x[t - m]; zero beyond the kernel width.
 template <int TAPS>
@@ -70,6 +71,8 @@ struct ConvParams {
   int silu;
   long long x_bs, x_rs;      // rows-in kernels: elements between batch rows and between time steps of x
   int wide_taps;             // K == 4, weight and bias on 16-byte boundaries (see load_taps_of)
+  float *dw, *dbias;         // (B,C,L) backward with `whole_batch`: the sums themselves instead of partials
+  int whole_batch;           // (B,C,L) backward: a workgroup takes a channel's rows of every batch entry in turn
 };
 
 __device__ __forceinline__ float silu_grad(float pre) {
@@ -346,12 +349,8 @@ template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvParams p) {
   constexpr int VEC = 16 / sizeof(T);
   __shared__ float red[CONV_THREADS / WAVE][TAPS + 1];
-  const int row = blockIdx.x;
-  const int c = row % p.chans;
+  const int c = blockIdx.x % p.chans;
   const int K = p.K;
-  const T *xr = reinterpret_cast<const T *>(p.x) + (size_t)row * p.len;
-  const T *gr = reinterpret_cast<const T *>(p.dout) + (size_t)row * p.len;
-  T *dxr = reinterpret_cast<T *>(p.y) + (size_t)row * p.len;
   float wrev1[1][TAPS], bias1[1];
   load_taps_of<1, TAPS>(p.w, p.bias, c, K, p.wide_taps, wrev1, bias1);
   const float (&wrev)[TAPS] = wrev1[0];
@@ -360,6 +359,14 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
 #pragma unroll
   for (int m = 0; m < TAPS; ++m) dwrev[m] = 0.0f;
 
+  // the rows of this workgroup: one (b, c) row, or with `whole_batch` channel c of every batch entry
+  const int b_first = p.whole_batch ? 0 : (int)(blockIdx.x / p.chans);
+  const int b_end = p.whole_batch ? p.batch : b_first + 1;
+  for (int b = b_first; b < b_end; ++b) {
+  const size_t row = (size_t)b * p.chans + c;
+  const T *xr = reinterpret_cast<const T *>(p.x) + row * p.len;
+  const T *gr = reinterpret_cast<const T *>(p.dout) + row * p.len;
+  T *dxr = reinterpret_cast<T *>(p.y) + row * p.len;
   for (int t0 = threadIdx.x * VEC; t0 < p.len; t0 += CONV_THREADS * VEC) {
     // x over [t0-VEC, t0+2*VEC), dout over [t0, t0+2*VEC)
     float xw[3 * VEC], g[2 * VEC];
@@ -423,6 +430,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
     if constexpr (AL) store_vec<T, VEC>(dxr, t0, dx);
     else store_run<T, VEC>(dxr, t0, p.len, AL, dx);
   }
+  }
   // block reduction of dw[0..K) and db
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 #pragma unroll
@@ -440,7 +448,9 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cf_kernel(const ConvPar
     const int src = threadIdx.x < K ? (K - 1 - (int)threadIdx.x) : TAPS;
     float s = 0.0f;
     for (int wv = 0; wv < CONV_THREADS / WAVE; ++wv) s += red[wv][src];
-    p.partial[(size_t)row * (K + 1) + threadIdx.x] = s;
+    if (!p.whole_batch) p.partial[(size_t)blockIdx.x * (K + 1) + threadIdx.x] = s;
+    else if ((int)threadIdx.x < K) p.dw[(size_t)c * K + threadIdx.x] = s;
+    else if (p.dbias) p.dbias[c] = s;
   }
 }
 
@@ -973,8 +983,21 @@ static int conv_bwd_typed(const ConvParams &p, int layout, bool vec_ok, float *d
     else CONV_LAUNCH(conv_bwd_tr_kernel, CONV_T_AL(false), dim3((unsigned)blocks), dim3(CONV_TR_THREADS));
     fold_count = p.batch * nseg;
   } else if (p.K <= CONV_TAPS && !channels_last) {
-    if (vec_ok && p.len % VEC == 0) CONV_LAUNCH(conv_bwd_cf_kernel, CONV_T_AL(true), dim3(p.batch * p.chans), dim3(CONV_THREADS));
-    else CONV_LAUNCH(conv_bwd_cf_kernel, CONV_T_AL(false), dim3(p.batch * p.chans), dim3(CONV_THREADS));
+    // enough channels to fill the GPU with one workgroup each: a workgroup sums over the batch itself and the
+    // fold of partials (a second launch of ~4 us) falls away
+    ConvParams q = p;
+    q.whole_batch = p.chans >= CONV_WHOLE_BATCH_MIN_CHANNELS && p.batch > 1;
+    q.dw = dw; q.dbias = dbias;
+    const dim3 grid(q.whole_batch ? p.chans : p.batch * p.chans);
+    {
+      const ConvParams &p = q;
+      if (vec_ok && p.len % VEC == 0) CONV_LAUNCH(conv_bwd_cf_kernel, CONV_T_AL(true), grid, dim3(CONV_THREADS));
+      else CONV_LAUNCH(conv_bwd_cf_kernel, CONV_T_AL(false), grid, dim3(CONV_THREADS));
+    }
+    if (q.whole_batch) {
+      SSM_CHECK_LAUNCH("ssm_conv1d_bwd");
+      return SSM_OK;
+    }
   } else if (p.K <= CONV_TAPS && channels_last) {
     const int seg_len = conv_cl_seg_len(p.len);
     const int nseg = (p.len + seg_len - 1) / seg_len;
