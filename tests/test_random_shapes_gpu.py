@@ -182,6 +182,18 @@ def _conv_case(rng, seed):
             return O.dw_causal_conv(x.transpose(1, 2), w, bias, activation=act, acc=acc).transpose(1, 2)
         return O.dw_causal_conv(x, w, bias, activation=act, acc=acc)
 
+    # a draw of its own (the cases above stay what they were): the (B, C, L) input as the reference's blocks pass
+    # it, a permuted view of (B, L, C') rows, C' = C or wider with the channels somewhere inside
+    own = random.Random(seed ^ 0x2F6B)
+    if not channels_last and own.random() < 0.3:
+        wide = c + own.choice([0, 0, 4, c, 3])
+        off = own.choice([o for o in (0, 4, wide - c, 1) if 0 <= o <= wide - c])
+        rows = torch.randn(b, l, wide, generator=g).to(dtype)
+        view = lambda t: t[:, :, off:off + c].permute(0, 2, 1)
+        desc = desc + ("view of rows", wide, off)
+        _values_and_gradients(lambda x, w, bias: fn(view(x), w, bias, activation=act),
+                              lambda acc, x, w, bias: ref(acc, view(x), w, bias), [rows, w, bias], desc, half)
+        return
     _values_and_gradients(lambda x, w, bias: fn(x, w, bias, activation=act), ref, [x, w, bias], desc, half)
 
 
