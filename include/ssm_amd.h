@@ -694,6 +694,22 @@ size_t ssm_conv1d_bwd_workspace_bytes(int batch, int channels, int width);
 int ssm_conv1d_bwd(const ssm_conv1d_bwd_args *args, void *hip_stream);
 
 /* ------------------------------------------------------------------------
+ * A dense (B,C,L) copy of a (B,C,L)-shaped view whose memory runs channels innermost (rows of channels, one row per
+ * time step): what `tensor.contiguous()` does in the reference's Python path (src/ssm/ops/python/reference.py has no
+ * layout demands, its kernels' wrappers call `.contiguous()`), and what the reference's blocks hand the scan --
+ * `delta = F.linear(...).permute(0, 2, 1)`, `z = gate.permute(0, 2, 1)` (src/ssm/modules/mamba1.py:223-228).  The
+ * scan walks time, so those views are copied; this entry point is that copy at the speed of the memory.
+ * ---------------------------------------------------------------------- */
+typedef struct ssm_rows_to_bcl_args {
+  const void *src;          /* element (b, c, t) at src[b * src_batch_stride + t * src_row_stride + c] */
+  void *dst;                /* (B, C, L) dense, same element size */
+  int64_t src_batch_stride, src_row_stride;   /* elements; multiples of 4, rows do not overlap */
+  int32_t batch, channels, seqlen;            /* channels a multiple of 4 */
+  int32_t element_size;                       /* 2 or 4 bytes */
+} ssm_rows_to_bcl_args;
+int ssm_rows_to_bcl(const ssm_rows_to_bcl_args *args, void *hip_stream);
+
+/* ------------------------------------------------------------------------
  * residual-add + LayerNorm / RMSNorm over the last axis of (rows, hidden).
  * Forward stands behind `fused_layer_norm(x, weight, bias, residual, is_rms,
  * eps, prenorm, residual_in_fp32)` (src/ssm/ops/__init__.py:1640-1652;

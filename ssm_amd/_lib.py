@@ -252,6 +252,13 @@ class Conv1dBwdArgs(C.Structure):
     ]
 
 
+class RowsToBclArgs(C.Structure):
+    _fields_ = [
+        ("src", _vp), ("dst", _vp), ("src_batch_stride", C.c_int64), ("src_row_stride", C.c_int64),
+        ("batch", _i32), ("channels", _i32), ("seqlen", _i32), ("element_size", _i32),
+    ]
+
+
 class NormFwdArgs(C.Structure):
     _fields_ = [
         ("x", _vp), ("residual", _vp), ("weight", _vp), ("bias", _vp), ("y", _vp), ("residual_out", _vp),
@@ -351,6 +358,7 @@ ENTRY_POINTS = {
     "ssm_conv1d_fwd": Conv1dFwdArgs,
     "ssm_conv1d_bwd": Conv1dBwdArgs,
     "ssm_conv1d_update": Conv1dUpdateArgs,
+    "ssm_rows_to_bcl": RowsToBclArgs,
     "ssm_norm_fwd": NormFwdArgs,
     "ssm_norm_bwd": NormBwdArgs,
     "ssm_norm_bwd_static": NormBwdArgs,

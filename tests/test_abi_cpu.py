@@ -66,7 +66,7 @@ def test_ctypes_struct_sizes_match_the_header(tmp_path):
              "SsdBwdDtArgs": "ssm_ssd_bwd_dt_args", "SsdBwdPrepArgs": "ssm_ssd_bwd_prep_args",
              "F64ScanArgs": "ssm_f64_scan_args", "F64StepArgs": "ssm_f64_step_args",
              "F64DscanArgs": "ssm_f64_dscan_args", "F64ConvArgs": "ssm_f64_conv_args",
-             "F64NormArgs": "ssm_f64_norm_args"}
+             "F64NormArgs": "ssm_f64_norm_args", "RowsToBclArgs": "ssm_rows_to_bcl_args"}
     assert set(structs) <= set(cname), set(structs) - set(cname)
     src = tmp_path / "sizes.c"
     lines = ['#include <stdio.h>', f'#include "{HEADER}"', "int main(void) {"]

@@ -109,3 +109,50 @@ def test_ssd_combined(fused):
     fn = lambda x, dt, A, B, C, D, z, b: ssd.ssd_combined(x, dt, A, B, C, Q, D=D, z=z, dt_bias=b, dt_softplus=True, fused=fused)
     ts = (xs, dts, As, Bs, Cs, Ds, zs, bs)
     same(grads_of(fn, ts, view), grads_of(fn, ts, own), dtype, "ssd_combined")
+
+
+# ------------------------------------------------------------- (B, C, L) views of memory that runs channels innermost
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.int32, torch.int16])
+@pytest.mark.parametrize("shape", [(2, 11, 8, 8, 0), (1, 300, 64, 128, 64), (3, 1000, 12, 40, 4), (2, 130, 68, 68, 0),
+                                   (2, 257, 132, 264, 132), (2, 64, 6, 6, 0), (2, 129, 8, 16, 2), (8, 2048, 1536, 3072, 1536)],
+                         ids=lambda s: "B{}L{}C{}of{}at{}".format(*s))
+def test_dense_copy_of_a_view_of_rows(dtype, shape):
+    """``dense_copy`` equals ``contiguous()`` bit for bit on every view: the tiled copy takes the ones whose channel
+    count, strides and start are multiples of 4 elements, torch the others (6 channels; a start 2 elements in)."""
+    from ssm_amd.ops import _contract as K
+    batch, length, chans, wide, offset = shape
+    g = torch.Generator(device="cuda").manual_seed(length)
+    rows = torch.randint(-30000, 30000, (batch, length, wide), device="cuda", generator=g).to(dtype)
+    v = rows[:, :, offset:offset + chans].permute(0, 2, 1)
+    out = K.dense_copy(v)
+    assert out.is_contiguous() and out.shape == v.shape and out.dtype == v.dtype
+    assert torch.equal(out, v.contiguous())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+def test_scan_on_permuted_views_equals_the_scan_on_dense_copies(dtype):
+    """What the reference's block passes (src/ssm/modules/mamba1.py:223-247): ``delta`` and ``z`` as permuted views of
+    (B, L, D) projections, ``z`` one half of a wider one.  Forward and backward equal the call on dense copies."""
+    from tests.test_scan_fwd_gpu import make_inputs
+    ops = _ops()
+    batch, dim, length, nstate = 2, 48, 520, 16
+    inp = {k: v.cuda() for k, v in make_inputs(5, batch, dim, length, nstate, dtype=dtype).items()}
+    g = torch.Generator(device="cuda").manual_seed(2)
+    delta_rows = torch.randn(batch, length, dim, device="cuda", generator=g).to(dtype)
+    xz = torch.randn(batch, length, 2 * dim, device="cuda", generator=g).to(dtype)
+    go = torch.randn(batch, dim, length, device="cuda", generator=g).to(dtype)
+    res = []
+    for dense in (False, True):
+        d_leaf, z_leaf = delta_rows.clone().requires_grad_(), xz.clone().requires_grad_()
+        delta, z = d_leaf.permute(0, 2, 1), z_leaf.chunk(2, dim=-1)[1].permute(0, 2, 1)
+        if dense:
+            delta, z = delta.contiguous(), z.contiguous()
+        else:
+            assert not delta.is_contiguous() and not z.is_contiguous()
+        u = inp["u"].clone().requires_grad_()
+        y = ops.selective_scan(u, delta, inp["A"], inp["B"], inp["C"], D=inp["D"], z=z, dt_bias=inp["dt_bias"], softplus=True)
+        y.backward(go)
+        res.append((y.detach(), u.grad, d_leaf.grad, z_leaf.grad))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
