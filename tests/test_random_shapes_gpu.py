@@ -123,8 +123,26 @@ def _scan_case(rng, seed):
         delta, bias = delta.abs() * 0.3, None
     half = dtype in HALF
     desc = ("scan", seed, (b, d, l, n), kind, groups, str(dtype), D is not None, z is not None, bias is not None, sp)
-    _values_and_gradients(lambda *a: _ops().selective_scan(*a, softplus=sp, return_last_state=True),
-                          lambda acc, *a: O.selective_scan(*a, softplus=sp, return_last_state=True, acc=acc),
+    # a draw of its own (the cases above stay what they were): u, delta, z as the reference's block passes the last
+    # two, (B, D, L)-shaped views of (B, L, D') rows (src/ssm/modules/mamba1.py:223-228)
+    own = random.Random(seed ^ 0x6C1D)
+    turned = [name for name in ("u", "delta", "z") if own.random() < 0.25]
+    if turned:
+        desc = desc + ("views of rows", tuple(turned))
+
+    def as_given(name, t):
+        """The leaf to differentiate and the view of it that the operator gets."""
+        if t is None or name not in turned:
+            return t, (lambda leaf: leaf)
+        pad = own.choice([0, 0, 4, d])
+        rows = torch.zeros(b, l, d + pad).to(t.dtype)
+        rows[:, :, :d] = t.transpose(1, 2)
+        return rows, (lambda leaf: leaf[:, :, :d].permute(0, 2, 1))
+
+    (u, vu), (delta, vd), (z, vz) = as_given("u", u), as_given("delta", delta), as_given("z", z)
+    look = lambda a: (vu(a[0]), vd(a[1]), *a[2:6], None if a[6] is None else vz(a[6]), a[7])
+    _values_and_gradients(lambda *a: _ops().selective_scan(*look(a), softplus=sp, return_last_state=True),
+                          lambda acc, *a: O.selective_scan(*look(a), softplus=sp, return_last_state=True, acc=acc),
                           [u, delta, A, Bm, Cm, D, z, bias], desc, half)
 
 
