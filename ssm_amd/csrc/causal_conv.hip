@@ -642,11 +642,11 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_bwd_cl_kernel(const ConvPar
 // twice where a row has 8 units).
 constexpr int CONV_TR_CH = 64, CONV_TR_STRIP = 8;
 constexpr int CONV_TR_FWD_VEC = 4, CONV_TR_FWD_STEPS = 64;    // forward: 16 lanes x 8 strips
-constexpr int CONV_TR_BWD_VEC = 2, CONV_TR_BWD_STEPS = 64;     // backward: 32 lanes x 8 strips (registers)
+constexpr int CONV_TR_BWD_VEC = 2, CONV_TR_BWD_STEPS = 128, CONV_TR_BWD_STRIP = 16;   // backward: 32 lanes x 8 strips of 16 steps
 constexpr int CONV_TR_THREADS = 256;
 constexpr int CONV_TR_ALIGN = 4;                                // channels: count, strides and start of x are multiples
 constexpr int CONV_TR_FWD_THREADS = (CONV_TR_CH / CONV_TR_FWD_VEC) * (CONV_TR_FWD_STEPS / CONV_TR_STRIP);
-static_assert((CONV_TR_CH / CONV_TR_BWD_VEC) * (CONV_TR_BWD_STEPS / CONV_TR_STRIP) == CONV_TR_THREADS, "backward tile");
+static_assert((CONV_TR_CH / CONV_TR_BWD_VEC) * (CONV_TR_BWD_STEPS / CONV_TR_BWD_STRIP) == CONV_TR_THREADS, "backward tile");
 
 // AL: the rows of y (L elements each) start on 16-byte boundaries and L is a whole number of 16-byte units.
 template <typename T, bool AL, int TAPS>
@@ -723,7 +723,7 @@ __host__ __device__ inline int conv_tr_seg_tiles(int len) {
 
 template <typename T, bool AL, int TAPS>
 __global__ __launch_bounds__(CONV_TR_THREADS) void conv_bwd_tr_kernel(const ConvParams p) {
-  constexpr int CH = CONV_TR_CH, TT = CONV_TR_BWD_STEPS, S = CONV_TR_STRIP, VEC = CONV_TR_BWD_VEC, HIST = TAPS - 1;
+  constexpr int CH = CONV_TR_CH, TT = CONV_TR_BWD_STEPS, S = CONV_TR_BWD_STRIP, VEC = CONV_TR_BWD_VEC, HIST = TAPS - 1;
   constexpr int UNIT = 16 / sizeof(T), UPR = TT / UNIT, UPS = S / UNIT;
   constexpr int GU = (S + HIST + UNIT - 1) / UNIT;      // units of dout a thread takes: its strip and 4 steps on
   constexpr int GROUPS = CH / VEC, GROUPS_PER_WAVE = GROUPS < WAVE ? GROUPS : WAVE;
