@@ -88,6 +88,38 @@ def test_causal_conv_beyond_2_31_elements():
                    what=f"channels last dx ({b0}, {c0}..)")
 
 
+def test_view_of_rows_beyond_2_31_elements():
+    """The permuted view of (B, L, C) rows that the reference's blocks pass: the convolution reads it as it lies
+    (forward and backward) and ``dense_copy`` turns it, at more than 2**31 elements."""
+    ops = _ops()
+    from ssm_amd.ops import _contract as K
+    batch, length, chans, width = 3, 387072, 2048, 4
+    assert batch * length * chans > 2 ** 31
+    g = _gen(6)
+    rows = torch.empty(batch, length, chans, device="cuda", dtype=BF).normal_(generator=g)
+    w = torch.rand(chans, width, device="cuda", generator=g) - 0.5
+    b = torch.randn(chans, device="cuda", generator=g) * 0.02
+    x = rows.permute(0, 2, 1)
+    assert ops._conv_rows_view(x, True, width) is not None
+    y = ops._conv_forward(x, w, b, "silu")
+    for (b0, c0) in ((batch - 1, chans - 8), (0, 0)):
+        xs = x[b0:b0 + 1, c0:c0 + 8].contiguous()
+        ws, bs = w[c0:c0 + 8].contiguous(), b[c0:c0 + 8].contiguous()
+        assert torch.equal(y[b0:b0 + 1, c0:c0 + 8], ops._conv_forward(xs, ws, bs, "silu")), (b0, c0)
+    go = y                                   # any (B, C, L) tensor of the type serves as the incoming gradient
+    dx, _, _ = ops._conv_backward(go, x, w, b, "silu")
+    assert dx.shape == x.shape and dx.stride() == (length * chans, 1, chans)
+    for (b0, c0) in ((batch - 1, chans - 8), (0, 0)):
+        xs, gs = x[b0:b0 + 1, c0:c0 + 8].contiguous(), go[b0:b0 + 1, c0:c0 + 8].contiguous()
+        ws, bs = w[c0:c0 + 8].contiguous(), b[c0:c0 + 8].contiguous()
+        assert torch.equal(dx[b0:b0 + 1, c0:c0 + 8], ops._conv_backward(gs, xs, ws, bs, "silu")[0]), (b0, c0)
+    del dx, go
+    dense = K.dense_copy(x)
+    assert dense.is_contiguous()
+    for (b0, c0) in ((batch - 1, chans - 8), (1, 1000), (0, 0)):
+        assert torch.equal(dense[b0, c0:c0 + 8], x[b0, c0:c0 + 8]), (b0, c0)
+
+
 def test_fused_norm_beyond_2_31_elements():
     ops = _ops()
     rows, hidden = 2_900_000, 768
