@@ -128,3 +128,41 @@ def test_mamba2_forward_calls(dtype):
         fp32_close(got, want.double(), want, what="Y", rtol=1e-4, atol_rms=1e-4)
     else:
         half_close(got, want, what="Y")            # the two chains round the conv output to bfloat16 separately
+
+
+def test_mamba1_projections_factor_into_a_scan_with_constant_projections():
+    """``Mamba1.forward`` (src/ssm/modules/mamba1.py:229-247) materialises ``B = base_B (1 + B_gates)`` and ``C`` likewise
+    as ``(B, D, N, L)`` tensors, 16 times the activations.  The time-varying factor does not depend on the state
+    index, so it moves out of the recurrence: the same output is the scan with the constant ``(D, N)`` projections
+    on ``u (1 + B_gates)``, its result scaled by ``(1 + C_gates)``, plus the skip term and the gate outside.  Checked
+    here for values and every gradient through the operators of this package (float32, 1e-4)."""
+    ops = _ops()
+    batch, seqlen, inner, nstate = 2, 300, 48, 8
+    g = torch.Generator().manual_seed(41)
+    leaves = dict(
+        u=torch.randn(batch, inner, seqlen, generator=g), delta=torch.randn(batch, inner, seqlen, generator=g),
+        A=-torch.exp(torch.rand(inner, nstate, generator=g)), base_B=torch.randn(inner, nstate, generator=g),
+        base_C=torch.randn(inner, nstate, generator=g), gB=torch.randn(batch, inner, seqlen, generator=g) * 0.5,
+        gC=torch.randn(batch, inner, seqlen, generator=g) * 0.5, D=torch.randn(inner, generator=g),
+        z=torch.randn(batch, inner, seqlen, generator=g), dt_bias=torch.randn(inner, generator=g))
+    go = torch.randn(batch, inner, seqlen, generator=g).cuda()
+
+    def run(factored):
+        t = {k: v.clone().cuda().requires_grad_() for k, v in leaves.items()}
+        if factored:
+            core = ops.selective_scan(t["u"] * (1 + t["gB"]), t["delta"], t["A"], t["base_B"], t["base_C"],
+                                      dt_bias=t["dt_bias"], softplus=True)
+            y = (core * (1 + t["gC"]) + t["D"].view(1, -1, 1) * t["u"]) * torch.nn.functional.silu(t["z"])
+        else:
+            Bm = t["base_B"].view(1, inner, nstate, 1) * (1 + t["gB"].unsqueeze(2))
+            Cm = t["base_C"].view(1, inner, nstate, 1) * (1 + t["gC"].unsqueeze(2))
+            y = ops.selective_scan(t["u"], t["delta"], t["A"], Bm, Cm, D=t["D"], z=t["z"], dt_bias=t["dt_bias"], softplus=True)
+        y.backward(go)
+        return y.detach(), {k: v.grad for k, v in t.items()}
+
+    y_m, g_m = run(False)
+    y_f, g_f = run(True)
+    scale = lambda t: float(t.double().pow(2).mean().sqrt()) + 1e-30
+    assert float((y_m - y_f).abs().max()) <= 1e-4 * scale(y_m)
+    for k in leaves:
+        assert float((g_m[k] - g_f[k]).abs().max()) <= 1e-4 * scale(g_m[k]) + 1e-6, k
