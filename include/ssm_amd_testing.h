@@ -12,7 +12,8 @@
  *                                     1616, 2416, 3216, 4816 = 816 with two, three, four, six channels per wave;
  *                                     100000 + v = variant v of the kernel for grouped time-varying projections
  *   ssm_scan_bwd_args.reserved        1 = the general kernel also where a wave-per-row kernel applies (grouped
- *                                     projections, or projections of their own per channel);
+ *                                     projections, projections of their own per channel, or projections that are
+ *                                     constant in time);
  *                                     2 = the wave-per-row kernel with its bounded wait for a neighbouring wave
  *                                     cut to nothing, so that every wave takes the give-up path (dB and dC
  *                                     come back as NaN; the kernel ends normally)

@@ -776,6 +776,17 @@ static bool scan_bwd_is_per_row(const ssm_scan_bwd_args *a) {
          aligned_to(a->Bproj, 8 * bs) && aligned_to(a->Cproj, 8 * bs) && aligned_to(a->dB, 16) && aligned_to(a->dC, 16);
 }
 
+// Whether a call takes the wave-per-row kernel for projections that are constant in time, (D, N) or (B, D, N).
+static bool scan_bwd_is_const_row(const ssm_scan_bwd_args *a) {
+  using namespace ssm;
+  if (!a || SSM_RESERVED(a) == 1) return false;
+  if (a->b_kind == SSM_PROJ_BGNL || a->c_kind == SSM_PROJ_BGNL) return false;
+  if (a->seqlen <= 0 || a->seqlen % 8 != 0 || a->nstate <= 0 || a->nstate > BW_MAX_N) return false;
+  if (!valid_dtype(a->io_dtype) || !valid_dtype(a->bc_dtype)) return false;
+  return aligned_to(a->u, 16) && aligned_to(a->delta, 16) && aligned_to(a->dout, 16) && aligned_to(a->du, 16) &&
+         aligned_to(a->ddelta, 16) && (!a->z || (aligned_to(a->z, 16) && aligned_to(a->dz, 16)));
+}
+
 extern "C" size_t ssm_scan_bwd_per_row_workspace_bytes(const ssm_scan_bwd_args *a) {
   if (!scan_bwd_is_per_row(a)) return 0;
   return ssm::plan_bwd(a->batch, a->dim, a->seqlen, a->nstate, a->b_kind, a->c_kind, a->b_groups, a->c_groups).off_dB;
@@ -859,7 +870,13 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
     fast_rpw = scan_bwd_fast_rpw(a->batch, a->dim, a->dim / p.b_groups, a->dim / p.c_groups);
     if (fast_rpw && a->dim / (BF_WAVES * fast_rpw) > pl.nblk) fast_rpw = 0;
   }
-  if (per_row) {
+  if (scan_bwd_is_const_row(a)) {
+    switch (a->io_dtype) {
+      case SSM_F32: rc = launch_bwd_row_const<float>(p, s); break;
+      case SSM_BF16: rc = launch_bwd_row_const<bf16_t>(p, s); break;
+      default: rc = launch_bwd_row_const<f16_t>(p, s); break;
+    }
+  } else if (per_row) {
     const bool bc32 = a->bc_dtype == SSM_F32, o32 = a->dbc_dtype == SSM_F32;
     if (a->io_dtype == SSM_F32) rc = launch_bwd_rowbc<float, float, float>(p, a->dB, a->dC, s);
     else if (a->io_dtype == SSM_BF16)

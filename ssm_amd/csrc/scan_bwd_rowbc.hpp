@@ -12,6 +12,12 @@
 // against 4 x 16 bytes per lane for the whole row).  Two waves per SIMD: a state's four vectors in flight and the
 // row's sums take more than 128 registers, and at 168 the kernel with the gate still spills (config 1's shape in bf16:
 // 0.95 ms at four waves per SIMD with 47-64 registers spilled, 0.75 ms at three, 0.70 ms at two).
+//
+// CONST_BC: the same walk for projections that do not vary in time, (D, N) or (B, D, N) -- the reference's other
+// accepted forms (src/ssm/ops/python/reference.py:22-56), and what its Mamba1 block's per-channel projections
+// reduce to once the per-token gate is taken out of the recurrence.  A row's N values of B and of C sit in lanes like
+// A; dB and dC are sums over time, kept in lanes like dA and left per row for the folds over the batch.  Nothing
+// of the size of the projections moves, so the kernel is bound by its arithmetic and runs four waves per SIMD.
 #pragma once
 #include "scan_bwd_fast.hpp"
 
@@ -19,8 +25,8 @@ namespace ssm {
 
 constexpr int BR_WAVES = 4;
 
-template <typename io_t, typename bc_t, typename out_t, bool HAS_Z>
-__global__ __launch_bounds__(WAVE *BR_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <typename io_t, typename bc_t, typename out_t, bool HAS_Z, bool CONST_BC = false>
+__global__ __launch_bounds__(WAVE *BR_WAVES) __attribute__((amdgpu_waves_per_eu(CONST_BC ? 4 : 2, CONST_BC ? 4 : 2)))
 void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
   constexpr int K = BF_K, T = FAST_T;
   const int wave = wave_id_uniform();
@@ -31,9 +37,15 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
   const int L = p.len, N = p.nstate;
   const int nchunks = (L + T - 1) / T;
   const int rev_lane = WAVE - 1 - lane;
-  const size_t proj0 = row * (size_t)N * L;                   // the row's own (N, L) block of B, C, dB and dC
+  const size_t proj0 = CONST_BC ? 0 : row * (size_t)N * L;    // the row's own (N, L) block of B, C, dB and dC
   const bc_t *Bg = reinterpret_cast<const bc_t *>(p.Bp) + proj0, *Cg = reinterpret_cast<const bc_t *>(p.Cp) + proj0;
   out_t *dBg = dBo + proj0, *dCg = dCo + proj0;
+  // CONST_BC: lane n holds B[n] and C[n] of the row ((D, N), or (B, D, N) with the batch entry's own) and their sums
+  float B_lanes = 0.0f, C_lanes = 0.0f, dB_lanes = 0.0f, dC_lanes = 0.0f;
+  if (CONST_BC && lane < N) {
+    B_lanes = load_as_f32(p.Bp, p.bc_dtype, (p.b_kind == SSM_PROJ_BDN ? row : (size_t)d) * N + lane);
+    C_lanes = load_as_f32(p.Cp, p.bc_dtype, (p.c_kind == SSM_PROJ_BDN ? row : (size_t)d) * N + lane);
+  }
   const io_t *U = reinterpret_cast<const io_t *>(p.u), *DT = reinterpret_cast<const io_t *>(p.delta);
   const io_t *GO = reinterpret_cast<const io_t *>(p.dout), *Z = reinterpret_cast<const io_t *>(HAS_Z ? p.z : p.u);
   io_t *DU = reinterpret_cast<io_t *>(p.du), *DDL = reinterpret_cast<io_t *>(p.ddelta), *DZ = reinterpret_cast<io_t *>(p.dz);
@@ -50,8 +62,11 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
     const bool live = t < L;
     const int tc = live ? t : 0;
     const size_t at = row * L + tc;
-    Pack<bc_t, K> braw = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + tc);
-    Pack<bc_t, K> craw = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + tc);
+    Pack<bc_t, K> braw, craw;
+    if (!CONST_BC) {
+      braw = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + tc);
+      craw = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + tc);
+    }
     const Pack<io_t, K> ur = *reinterpret_cast<const Pack<io_t, K> *>(U + at);
     const Pack<io_t, K> dr = *reinterpret_cast<const Pack<io_t, K> *>(DT + at);
     const Pack<io_t, K> gr = *reinterpret_cast<const Pack<io_t, K> *>(GO + at);
@@ -80,13 +95,23 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
     for (int n = 0; n < N; ++n) {
       // the next state's projections are requested before this state's arithmetic
       const int nn = n + 1 < N ? n + 1 : n;
-      const Pack<bc_t, K> bnext = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + (size_t)nn * L + tc);
-      const Pack<bc_t, K> cnext = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + (size_t)nn * L + tc);
+      Pack<bc_t, K> bnext, cnext;
       float bq[K], cq[K];
+      if (!CONST_BC) {
+        bnext = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + (size_t)nn * L + tc);
+        cnext = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + (size_t)nn * L + tc);
 #pragma unroll
-      for (int i = 0; i < K; ++i) {
-        bq[i] = to_f32(braw.v[i]);
-        cq[i] = to_f32(craw.v[i]);
+        for (int i = 0; i < K; ++i) {
+          bq[i] = to_f32(braw.v[i]);
+          cq[i] = to_f32(craw.v[i]);
+        }
+      } else {
+        const float bn = wave_read_lane(B_lanes, n), cn = wave_read_lane(C_lanes, n);
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+          bq[i] = bn;
+          cq[i] = cn;
+        }
       }
       const float A2 = wave_read_lane(A2_lanes, n);
       const float Hin = wave_read_lane(Hin_lanes, n);
@@ -119,13 +144,18 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
       const float qnew = wave_read_lane(qr, WAVE - 1);         // adjoint leaving the chunk towards earlier steps
       qcarry = lane == n ? qnew : qcarry;
       float qn = lane_from(wave_prev(qr, qc), rev_lane);       // adjoint entering this lane's run from the right
-      float sA = 0.0f;
+      float sA = 0.0f, sB = 0.0f, sC = 0.0f;
       Pack<out_t, K> ob, oc;
 #pragma unroll
       for (int i = K - 1; i >= 0; --i) {
         const float gh = __builtin_fmaf(g[i], cq[i], qn);
-        oc.v[i] = from_f32<out_t>(g[i] * hv[i + 1]);
-        ob.v[i] = from_f32<out_t>(gh * du[i]);
+        if (!CONST_BC) {
+          oc.v[i] = from_f32<out_t>(g[i] * hv[i + 1]);
+          ob.v[i] = from_f32<out_t>(gh * du[i]);
+        } else {
+          sC = __builtin_fmaf(g[i], hv[i + 1], sC);
+          sB = __builtin_fmaf(gh, du[i], sB);
+        }
         ghB[i] = __builtin_fmaf(gh, bq[i], ghB[i]);
         qn = a[i] * gh;
         const float qh = qn * hv[i];
@@ -134,12 +164,18 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
       }
       const float tot = wave_sum(sA);
       dA_lanes += lane == n ? tot : 0.0f;
-      if (live) {
-        *reinterpret_cast<Pack<out_t, K> *>(dBg + (size_t)n * L + tc) = ob;
-        *reinterpret_cast<Pack<out_t, K> *>(dCg + (size_t)n * L + tc) = oc;
+      if (!CONST_BC) {
+        if (live) {
+          *reinterpret_cast<Pack<out_t, K> *>(dBg + (size_t)n * L + tc) = ob;
+          *reinterpret_cast<Pack<out_t, K> *>(dCg + (size_t)n * L + tc) = oc;
+        }
+        braw = bnext;
+        craw = cnext;
+      } else {
+        const float totB = wave_sum(sB), totC = wave_sum(sC);
+        dB_lanes += lane == n ? totB : 0.0f;
+        dC_lanes += lane == n ? totC : 0.0f;
       }
-      braw = bnext;
-      craw = cnext;
     }
 
     // ---- what the row's elements receive
@@ -182,10 +218,25 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
 
   const float sd = wave_sum(dD_part), sb = wave_sum(db_part);
   if (lane < N) p.dA_rows[row * N + lane] = dA_lanes;
+  if (CONST_BC && lane < N) {
+    p.dB_part[row * N + lane] = dB_lanes;
+    p.dC_part[row * N + lane] = dC_lanes;
+  }
   if (lane == 0) {
     p.dD_rows[row] = sd;
     p.dbias_rows[row] = sb;
   }
+}
+
+// Projections constant in time: the partial sums per row go to p.dB_part / p.dC_part, (B, D, N) float32.
+template <typename io_t>
+static int launch_bwd_row_const(const ScanBwdParams &p, hipStream_t s) {
+  const size_t rows = (size_t)p.batch * p.dim;
+  const dim3 grid((unsigned)((rows + BR_WAVES - 1) / BR_WAVES)), block(WAVE * BR_WAVES);
+  if (p.z) hipLaunchKernelGGL((scan_bwd_rowbc_kernel<io_t, float, float, true, true>), grid, block, 0, s, p, nullptr, nullptr);
+  else hipLaunchKernelGGL((scan_bwd_rowbc_kernel<io_t, float, float, false, true>), grid, block, 0, s, p, nullptr, nullptr);
+  SSM_CHECK_LAUNCH("ssm_scan_bwd");
+  return SSM_OK;
 }
 
 template <typename io_t, typename bc_t, typename out_t>

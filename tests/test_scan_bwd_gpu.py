@@ -436,3 +436,50 @@ def test_conv_then_scan_forward_and_backward(dtype):
         half_close(y, yr, what="y")
         for k in names:
             half_close(got[k], want[k], what=f"grad {k}", atol_rms=4e-2, mean_rms=5e-3)
+
+
+@pytest.mark.parametrize("shape,bkind,ckind,use_z,with_last", [
+    ((2, 48, 1040, 16), "dn", "dn", True, True), ((1, 96, 512, 16), "bdn", "bdn", True, False),
+    ((2, 32, 1536, 9), "dn", "bdn", False, True), ((1, 16, 72, 16), "bdn", "dn", True, False),
+    ((3, 40, 2048, 16), "dn", "dn", True, False)], ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("dtype,bc_dtype", [(torch.bfloat16, torch.float32), (torch.float16, torch.float16),
+                                            (torch.float32, torch.float32)])
+def test_constant_projections_backward(shape, bkind, ckind, use_z, with_last, dtype, bc_dtype):
+    """``B`` and ``C`` of shape ``(D, N)`` or ``(B, D, N)`` (the reference's other accepted forms,
+    /root/reference/src/ssm/ops/python/reference.py:22-56): the wave-per-row kernel with the projections and their
+    sums in lanes, against the general kernel on the same inputs (test-hooks selector 1) and against float64 autograd
+    through the oracle."""
+    b, d, l, n = shape
+    inp = make_inputs(sum(shape) + 2, b, d, l, n, dtype=dtype, bc_dtype=bc_dtype, bkind=bkind, ckind=ckind, use_z=use_z)
+    g = torch.Generator().manual_seed(6)
+    go = torch.randn(b, d, l, generator=g).to(dtype)
+    gl = torch.randn(b, d, n, generator=g) if with_last else None
+    fast = _bwd_direct(inp, go, gl, 0)
+    gen = _bwd_direct(inp, go, gl, 1)
+    names = ("u", "delta", "A", "B", "C", "D", "z", "dt_bias")
+    for k, f, r in zip(names, fast, gen):
+        if r is None:
+            assert f is None, k
+            continue
+        assert f.dtype == r.dtype and f.shape == r.shape, k
+        f, r = f.float().cpu(), r.float().cpu()
+        scale = float(r.abs().max()) + 1e-30
+        if k in ("u", "delta", "z") and dtype != torch.float32:
+            torch.testing.assert_close(f, r, rtol=2e-2, atol=1e-3 * scale, msg=lambda m, k=k: f"grad {k} vs general kernel: {m}")
+        else:
+            torch.testing.assert_close(f, r, rtol=2e-4, atol=2e-5 * scale, msg=lambda m, k=k: f"grad {k} vs general kernel: {m}")
+    w = {k: (None if v is None else v.double().requires_grad_(True)) for k, v in inp.items()}
+    out = O.selective_scan(w["u"], w["delta"], w["A"], w["B"], w["C"], D=w["D"], z=w["z"], dt_bias=w["dt_bias"],
+                           softplus=True, return_last_state=with_last, acc=torch.float64)
+    if with_last:
+        ((out[0] * go.double()).sum() + (out[1] * gl.double()).sum()).backward()
+    else:
+        (out * go.double()).sum().backward()
+    for k, f in zip(names, fast):
+        if w[k] is None:
+            continue
+        want = w[k].grad
+        scale = float(want.abs().max()) + 1e-30
+        half = k in ("u", "delta", "z") and dtype != torch.float32
+        tol = dict(rtol=2e-2, atol=4e-3 * scale) if half else dict(rtol=1e-3, atol=1e-4 * scale)
+        torch.testing.assert_close(f.double().cpu(), want, **tol, msg=lambda m, k=k: f"grad {k} vs float64: {m}")
