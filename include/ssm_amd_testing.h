@@ -11,6 +11,7 @@
  *   ssm_scan_fwd_args.reserved        0 = automatic; 100 * steps-per-lane + states-per-LDS-pass (408, 808, 816);
  *                                     1616, 2416, 3216, 4816 = 816 with two, three, four, six channels per wave;
  *                                     100000 + v = variant v of the kernel for grouped time-varying projections
+ *                                     (131042: the row-per-wave kernel for projections constant in time)
  *   ssm_scan_bwd_args.reserved        1 = the general kernel also where a wave-per-row kernel applies (grouped
  *                                     projections, projections of their own per channel, or projections that are
  *                                     constant in time);

@@ -100,6 +100,17 @@ extern "C" int ssm_scan_fwd(const ssm_scan_fwd_args *a, void *hip_stream) {
     if (!pick && aligned_to(a->Bproj, 16) && aligned_to(a->Cproj, 16) && ((size_t)a->seqlen * bs) % 16 == 0) pick = 31041;
     if (pick) tune = 100000 + pick;
   }
+  // Projections constant in time, (D, N) or (B, D, N): a row per wave with B and C in lanes (variant 31042).
+  const bool const_ok = !bvary && !cvary && a->nstate <= FAST_N && p.vec_ok && a->seqlen % 8 == 0;
+  if ((tune == 0 && const_ok && a->seqlen > 256) || tune == 100000 + 31042) {
+    SSM_REQUIRE(const_ok, SSM_ERR_BAD_KIND, "ssm_scan_fwd: selector %d needs constant projections, at most %d states "
+                "and aligned rows of whole 8-step runs", tune, FAST_N);
+    switch (a->io_dtype) {
+      case SSM_F32: return scan_fwd_fast_dispatch<float, float>(p, 31042, stream);
+      case SSM_BF16: return scan_fwd_fast_dispatch<bf16_t, float>(p, 31042, stream);
+      default: return scan_fwd_fast_dispatch<f16_t, float>(p, 31042, stream);
+    }
+  }
   if (tune >= 100000) {
     SSM_REQUIRE(fast_ok, SSM_ERR_BAD_KIND, "ssm_scan_fwd: selector %d needs the shape of the specialised kernel", tune);
     const int v = tune - 100000, per_wg = scan_fwd_fast_rows(v);

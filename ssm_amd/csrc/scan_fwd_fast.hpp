@@ -327,7 +327,10 @@ void scan_fwd_fast_kernel(const ScanFwdParams p) {
 // (B, D, N, L) a Mamba-1 block passes): nothing is staged.  A wave owns one row, a lane its 8-step run, and the
 // lane reads the 16 bytes of B and of C of its run for every state straight from memory (consecutive lanes,
 // consecutive bytes), one state ahead of the arithmetic.  No LDS, no barrier: the call is bound by those reads.
-template <typename io_t, typename bc_t, int WAVES, int OCC>
+// CONST_BC: the same walk for projections that do not vary in time, (D, N) or (B, D, N) (the reference's other
+// accepted forms, src/ssm/ops/python/reference.py:22-56): a row's N values of B and of C sit in lanes like A, nothing
+// of the projections is read inside the loop.
+template <typename io_t, typename bc_t, int WAVES, int OCC, bool CONST_BC = false>
 __global__ __launch_bounds__(WAVE *WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
   constexpr int K = 8, T = FAST_T;
@@ -337,8 +340,17 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
   if (row >= (size_t)p.batch * p.dim) return;                // no barrier below: a wave may leave alone
   const int b = (int)(row / p.dim), d = (int)(row % p.dim);
   const int L = p.len, N = p.nstate;
-  const bc_t *Bg = reinterpret_cast<const bc_t *>(p.Bp) + ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * (size_t)N * L;
-  const bc_t *Cg = reinterpret_cast<const bc_t *>(p.Cp) + ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * (size_t)N * L;
+  const bc_t *Bg = reinterpret_cast<const bc_t *>(p.Bp), *Cg = reinterpret_cast<const bc_t *>(p.Cp);
+  float B_lanes = 0.0f, C_lanes = 0.0f;
+  if constexpr (CONST_BC) {
+    if (lane < N) {
+      B_lanes = load_as_f32(p.Bp, p.bc_dtype, (p.b_kind == SSM_PROJ_BDN ? row : (size_t)d) * N + lane);
+      C_lanes = load_as_f32(p.Cp, p.bc_dtype, (p.c_kind == SSM_PROJ_BDN ? row : (size_t)d) * N + lane);
+    }
+  } else {
+    Bg += ((size_t)b * p.b_groups + d / (p.dim / p.b_groups)) * (size_t)N * L;
+    Cg += ((size_t)b * p.c_groups + d / (p.dim / p.c_groups)) * (size_t)N * L;
+  }
   const io_t *U = reinterpret_cast<const io_t *>(p.u), *DT = reinterpret_cast<const io_t *>(p.delta);
   const io_t *Z = reinterpret_cast<const io_t *>(p.z);
   io_t *Y = reinterpret_cast<io_t *>(p.out);
@@ -355,8 +367,11 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
     const size_t at = row * L + tc;
     float dl[K], du[K], y[K];
     Pack<io_t, K> zr;
-    Pack<bc_t, K> braw = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + tc);
-    Pack<bc_t, K> craw = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + tc);
+    Pack<bc_t, K> braw, craw;
+    if constexpr (!CONST_BC) {
+      braw = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + tc);
+      craw = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + tc);
+    }
     {
       const Pack<io_t, K> ur = *reinterpret_cast<const Pack<io_t, K> *>(U + at);
       const Pack<io_t, K> dr = *reinterpret_cast<const Pack<io_t, K> *>(DT + at);
@@ -383,8 +398,24 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
     for (int n = 0; n < N; ++n) {
       // the next state's projections are requested before this state's arithmetic
       const int nn = n + 1 < N ? n + 1 : n;
-      const Pack<bc_t, K> bnext = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + (size_t)nn * L + tc);
-      const Pack<bc_t, K> cnext = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + (size_t)nn * L + tc);
+      Pack<bc_t, K> bnext, cnext;
+      float bq[K], cq[K];
+      if constexpr (!CONST_BC) {
+        bnext = *reinterpret_cast<const Pack<bc_t, K> *>(Bg + (size_t)nn * L + tc);
+        cnext = *reinterpret_cast<const Pack<bc_t, K> *>(Cg + (size_t)nn * L + tc);
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+          bq[i] = to_f32(braw.v[i]);
+          cq[i] = to_f32(craw.v[i]);
+        }
+      } else {
+        const float bn = wave_read_lane(B_lanes, n), cn = wave_read_lane(C_lanes, n);
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+          bq[i] = bn;
+          cq[i] = cn;
+        }
+      }
       const float A2 = wave_read_lane(A2_lanes, n);
       const float H = wave_read_lane(carry_lanes, n);
       float a[K], bx[K], P = dsum * A2, h;
@@ -393,7 +424,7 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
       exp2_run(a, P);
 #pragma unroll
       for (int i = 0; i < K; ++i) {
-        bx[i] = du[i] * to_f32(braw.v[i]);
+        bx[i] = du[i] * bq[i];
         h = i == 0 ? bx[0] : __builtin_fmaf(a[i], h, bx[i]);
       }
       h = __builtin_fmaf(P, lane == 0 ? H : 0.0f, h);
@@ -404,10 +435,12 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
 #pragma unroll
       for (int i = 0; i < K; ++i) {
         hs = __builtin_fmaf(a[i], hs, bx[i]);
-        y[i] = __builtin_fmaf(hs, to_f32(craw.v[i]), y[i]);
+        y[i] = __builtin_fmaf(hs, cq[i], y[i]);
       }
-      braw = bnext;
-      craw = cnext;
+      if constexpr (!CONST_BC) {
+        braw = bnext;
+        craw = cnext;
+      }
     }
 
     if (p.z) {
@@ -452,6 +485,16 @@ static int launch_scan_fwd_fast(const ScanFwdParams &p, hipStream_t stream) {
   return SSM_OK;
 }
 
+template <typename io_t>
+static int launch_scan_fwd_row_const(const ScanFwdParams &p, hipStream_t stream) {
+  constexpr int WAVES = 4;
+  const size_t rows = (size_t)p.batch * p.dim;
+  hipLaunchKernelGGL((scan_fwd_rowbc_kernel<io_t, float, WAVES, 6, true>), dim3((unsigned)((rows + WAVES - 1) / WAVES)),
+                     dim3(WAVE * WAVES), 0, stream, p);
+  SSM_CHECK_LAUNCH("ssm_scan_fwd");
+  return SSM_OK;
+}
+
 // Channels per workgroup of a variant; 0 for an unknown one.
 // variant = 10000 * (rows a wave walks at once) + 1000 * (rows a wave walks in turn) + 10 * waves + states in flight
 inline int scan_fwd_fast_rows(int variant) {
@@ -461,6 +504,7 @@ inline int scan_fwd_fast_rows(int variant) {
     case 22121: case 22123: return 48;
     case 21081: return 16;
     case 31041: return 1;       // a row per wave, projections read straight from memory
+    case 31042: return 1;       // a row per wave, projections constant in time
     default: return 0;
   }
 }
@@ -475,6 +519,7 @@ int scan_fwd_fast_dispatch(const ScanFwdParams &p, int variant, hipStream_t s) {
     case 22123: return launch_scan_fwd_fast<io_t, bc_t, 32, 2, 12, 1, 3, true>(p, s);   // the same with two slabs
     case 21081: return launch_scan_fwd_fast<io_t, bc_t, 32, 1, 8, 1, 4>(p, s);
     case 31041: return launch_scan_fwd_rowbc<io_t, bc_t>(p, s);
+    case 31042: return launch_scan_fwd_row_const<io_t>(p, s);
     default:
       set_error("ssm_scan_fwd: unknown variant %d of the specialised kernel", variant);
       return SSM_ERR_BAD_KIND;

@@ -351,3 +351,34 @@ def test_repeated_call_of_one_form_goes_through_the_remembered_struct():
         bad = dict(other)
         bad["A"] = other["A"][:, :8].contiguous()      # a form never seen, and inconsistent: the long way refuses it
         call(bad)
+
+
+@pytest.mark.parametrize("bkind,ckind", [("dn", "dn"), ("bdn", "bdn"), ("dn", "bdn"), ("bdn", "dn")])
+@pytest.mark.parametrize("dtype,bc_dtype,length,nstate", [
+    (torch.float32, torch.float32, 1520, 16), (torch.float32, torch.float32, 48, 5), (torch.bfloat16, torch.float32, 1040, 9),
+    (torch.float16, torch.float16, 512, 16), (torch.bfloat16, torch.bfloat16, 2048, 16)])
+def test_constant_projections_row_per_wave(bkind, ckind, dtype, bc_dtype, length, nstate):
+    """``B`` and ``C`` of shape ``(D, N)`` or ``(B, D, N)`` (/root/reference/src/ssm/ops/python/reference.py:22-56): the
+    kernel with a row per wave and the projections in lanes (variant 31042; what sequences beyond 256 steps take
+    unasked) against the oracle and against the general kernel (selector 816) on the same inputs -- values, the last
+    state, and the chunk states that the backward starts from."""
+    from ssm_amd import ops
+    inp = make_inputs(length + nstate, 2, 24, length, nstate, dtype=dtype, bc_dtype=bc_dtype, bkind=bkind, ckind=ckind)
+    yr, hr = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"],
+                              z=inp["z"], dt_bias=inp["dt_bias"], softplus=True, return_last_state=True)
+    args = [dev(inp[k]) for k in ("u", "delta", "A", "B", "C", "D", "z", "dt_bias")]
+    got = {}
+    for name, sel in (("row per wave", 100000 + 31042), ("general", 816)):
+        plan = ops.ScanPlan(*args, True, True, want_chunk_states=True, tune_items=sel)
+        y, h = plan.run()
+        got[name] = (y.float().cpu(), h.float().cpu(), plan.chunk_states.cpu())
+    tol = FP32_TOL if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got["row per wave"][0], yr.float(), **tol)
+    torch.testing.assert_close(got["row per wave"][1], hr.float(), **tol)
+    for a, b, what in zip(got["row per wave"], got["general"], ("y", "last state", "chunk states")):
+        scale = float(b.abs().max()) + 1e-30
+        torch.testing.assert_close(a, b, rtol=tol["rtol"], atol=(1e-5 if what == "chunk states" or dtype == torch.float32 else 1e-2) * scale,
+                                   msg=lambda m, what=what: f"{what} vs the general kernel: {m}")
+    if length > 256:      # the automatic choice is this kernel: the same bits as when asked for
+        y0, h0 = ops._scan_forward(*args, True, True)
+        assert torch.equal(y0.float().cpu(), got["row per wave"][0]) and torch.equal(h0.float().cpu(), got["row per wave"][1])
