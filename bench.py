@@ -547,6 +547,30 @@ def bench_scan_per_channel_bc(dtype=torch.bfloat16, batch=8, dim=1536, length=20
             "shape": "B, C (8, 1536, 16, 2048) bf16: one B/C group per channel"}
 
 
+def bench_scan_const_bc(dtype=torch.bfloat16, batch=8, dim=1536, length=2048, nstate=16):
+    """Config 1's shape with projections constant in time, ``B`` and ``C`` of shape ``(D, N)`` (the reference's other
+    accepted form, src/ssm/ops/python/reference.py:22-56; what its Mamba1 block's projections reduce to with the
+    per-token gate outside the recurrence): forward, and backward from the forward's chunk states."""
+    from ssm_amd import configs
+    from ssm_amd.ops import ScanPlan, _scan_backward
+    g = configs.to_device(configs.scan_inputs(batch, dim, length, nstate, dtype=dtype, seed=0))
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    Bm = torch.randn(dim, nstate, generator=gen, device="cuda")
+    Cm = torch.randn(dim, nstate, generator=gen, device="cuda")
+    plan = ScanPlan(g["u"], g["delta"], g["A"], Bm, Cm, g["D"], g["z"], g["dt_bias"], True, True)
+    us = _time_us(lambda i: plan.run(), iters=20, warmup=20)
+    cs_plan = ScanPlan(g["u"], g["delta"], g["A"], Bm, Cm, g["D"], g["z"], g["dt_bias"], True, False, want_chunk_states=True)
+    cs_plan.run()
+    go = torch.randn(batch, dim, length, generator=gen, device="cuda", dtype=torch.float32).to(dtype)
+    bus = _time_us(lambda i: _scan_backward(go, None, g["u"], g["delta"], g["A"], Bm, Cm, g["D"], g["z"], g["dt_bias"], True,
+                                            chunk_states=cs_plan.chunk_states), iters=20, warmup=30)
+    elt = 2 if dtype != torch.float32 else 4
+    fbytes, bbytes = 4 * elt * batch * dim * length, 7 * elt * batch * dim * length
+    return {"fwd_us": round(us, 1), "fwd_frac_hbm": round(fbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bwd_us": round(bus, 1), "bwd_frac_hbm": round(bbytes / bus / 1e3 / HBM_PEAK_GBPS, 4),
+            "shape": "B=8 D=1536 L=2048 N=16 bf16 activations, B and C (1536, 16) float32"}
+
+
 def bench_stream():
     """What plain element-wise kernels of the framework reach on this GPU, as the yardstick for the streaming
     kernels: ``dst = 2 * src`` and ``dst.copy_(src)`` on float32 buffers of 64 MiB (source and destination fit the
@@ -671,7 +695,7 @@ def main():
                          "the reference for hardware byte counters")
     ap.add_argument("--only", default=None,
                     choices=["scan_bwd", "mixer", "conv", "norm", "decode", "ssd", "ssd_train", "dscan", "model", "model1",
-                             "scan_facade", "scan_per_channel_bc", "stream"],
+                             "scan_facade", "scan_per_channel_bc", "scan_const_bc", "stream"],
                     help="run one of the secondary workloads alone and print its figures "
                          "(for profiling that kernel; not the benchmark line)")
     args = ap.parse_args()
@@ -698,7 +722,8 @@ def main():
         fn = {"scan_bwd": bench_scan_bwd, "conv": bench_conv, "norm": bench_norm, "decode": bench_decode,
               "mixer": bench_mixer_config1, "ssd": bench_ssd, "ssd_train": bench_ssd_train, "dscan": bench_dscan, "model": bench_model,
               "model1": bench_model1, "scan_facade": bench_scan_facade,
-              "scan_per_channel_bc": bench_scan_per_channel_bc, "stream": bench_stream}[args.only]
+              "scan_per_channel_bc": bench_scan_per_channel_bc, "scan_const_bc": bench_scan_const_bc,
+              "stream": bench_stream}[args.only]
         bench_scan_fwd(1, 0)            # the untimed spin-up of the default run, so that figures compare
         print(json.dumps({args.only: fn()}))
         return
@@ -750,6 +775,7 @@ def main():
             "frac_hbm": round(a32 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": r32["bytes"]}
         extra["selective_scan_fwd_through_ops_entry"] = bench_scan_facade()
         extra["selective_scan_fwd_per_channel_bc"] = bench_scan_per_channel_bc()
+        extra["selective_scan_constant_bc"] = bench_scan_const_bc()
         extra["selective_scan_bwd_bf16"] = bench_scan_bwd()
         extra["mamba1_mixer_config1_fwd_bwd"] = bench_mixer_config1()
         extra["dw_causal_conv_bf16"] = bench_conv()
