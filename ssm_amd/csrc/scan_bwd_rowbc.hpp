@@ -25,10 +25,13 @@ namespace ssm {
 
 constexpr int BR_WAVES = 4;
 
-template <typename io_t, typename bc_t, typename out_t, bool HAS_Z, bool CONST_BC = false>
-__global__ __launch_bounds__(WAVE *BR_WAVES) __attribute__((amdgpu_waves_per_eu(CONST_BC ? 4 : 2, CONST_BC ? 4 : 2)))
+// K: steps per lane, 8 or 16 (a lane's run; 64 runs make a chunk of the walk).  The states that enter chunks come
+// from the forward in steps of FAST_T = 512, so a walk in chunks of 1024 takes every second one.
+template <typename io_t, typename bc_t, typename out_t, bool HAS_Z, bool CONST_BC = false, int K = BF_K, int OCC = (CONST_BC ? 4 : 2)>
+__global__ __launch_bounds__(WAVE *BR_WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
-  constexpr int K = BF_K, T = FAST_T;
+  constexpr int T = WAVE * K;
+  static_assert(T % FAST_T == 0, "chunks of the walk are whole chunks of the forward");
   const int wave = wave_id_uniform();
   const int lane = lane_id();
   const size_t row = (size_t)blockIdx.x * BR_WAVES + wave;
@@ -36,6 +39,7 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
   const int d = (int)(row % p.dim);
   const int L = p.len, N = p.nstate;
   const int nchunks = (L + T - 1) / T;
+  const int fwd_chunks = (L + FAST_T - 1) / FAST_T;           // rows of chunk_states per (batch, channel)
   const int rev_lane = WAVE - 1 - lane;
   const size_t proj0 = CONST_BC ? 0 : row * (size_t)N * L;    // the row's own (N, L) block of B, C, dB and dC
   const bc_t *Bg = reinterpret_cast<const bc_t *>(p.Bp) + proj0, *Cg = reinterpret_cast<const bc_t *>(p.Cp) + proj0;
@@ -72,7 +76,7 @@ void scan_bwd_rowbc_kernel(const ScanBwdParams p, out_t *dBo, out_t *dCo) {
     const Pack<io_t, K> gr = *reinterpret_cast<const Pack<io_t, K> *>(GO + at);
     Pack<io_t, K> zr;
     if (HAS_Z) zr = *reinterpret_cast<const Pack<io_t, K> *>(Z + at);
-    const float Hin_lanes = lane < N ? p.chunk_states[(row * nchunks + c) * (size_t)N + lane] : 0.0f;
+    const float Hin_lanes = lane < N ? p.chunk_states[(row * fwd_chunks + c * (T / FAST_T)) * (size_t)N + lane] : 0.0f;
 
     float dl[K], du[K], g[K], ghB[K], At[K], pre[K];
     float dsum = 0.0f;
@@ -233,7 +237,13 @@ template <typename io_t>
 static int launch_bwd_row_const(const ScanBwdParams &p, hipStream_t s) {
   const size_t rows = (size_t)p.batch * p.dim;
   const dim3 grid((unsigned)((rows + BR_WAVES - 1) / BR_WAVES)), block(WAVE * BR_WAVES);
-  if (p.z) hipLaunchKernelGGL((scan_bwd_rowbc_kernel<io_t, float, float, true, true>), grid, block, 0, s, p, nullptr, nullptr);
+  // 16-step runs halve the lane scans and wave sums per step; their 243 registers leave two waves per SIMD (at three,
+  // 66 spill): 303 against 323 us at 8 x 1536 x 2048.  For sequences that fill chunks of 1024 steps.
+  const int tail = p.len % 1024;
+  if (p.len % 16 == 0 && p.len >= 1024 && (tail == 0 || tail > 512)) {
+    if (p.z) hipLaunchKernelGGL((scan_bwd_rowbc_kernel<io_t, float, float, true, true, 16, 2>), grid, block, 0, s, p, nullptr, nullptr);
+    else hipLaunchKernelGGL((scan_bwd_rowbc_kernel<io_t, float, float, false, true, 16, 2>), grid, block, 0, s, p, nullptr, nullptr);
+  } else if (p.z) hipLaunchKernelGGL((scan_bwd_rowbc_kernel<io_t, float, float, true, true>), grid, block, 0, s, p, nullptr, nullptr);
   else hipLaunchKernelGGL((scan_bwd_rowbc_kernel<io_t, float, float, false, true>), grid, block, 0, s, p, nullptr, nullptr);
   SSM_CHECK_LAUNCH("ssm_scan_bwd");
   return SSM_OK;

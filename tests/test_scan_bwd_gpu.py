@@ -441,14 +441,16 @@ def test_conv_then_scan_forward_and_backward(dtype):
 @pytest.mark.parametrize("shape,bkind,ckind,use_z,with_last", [
     ((2, 48, 1040, 16), "dn", "dn", True, True), ((1, 96, 512, 16), "bdn", "bdn", True, False),
     ((2, 32, 1536, 9), "dn", "bdn", False, True), ((1, 16, 72, 16), "bdn", "dn", True, False),
-    ((3, 40, 2048, 16), "dn", "dn", True, False)], ids=lambda v: str(v).replace(" ", ""))
+    ((3, 40, 2048, 16), "dn", "dn", True, False), ((1, 16, 1600, 16), "bdn", "dn", True, True),
+    ((1, 8, 3712, 5), "dn", "dn", False, False)], ids=lambda v: str(v).replace(" ", ""))
 @pytest.mark.parametrize("dtype,bc_dtype", [(torch.bfloat16, torch.float32), (torch.float16, torch.float16),
                                             (torch.float32, torch.float32)])
 def test_constant_projections_backward(shape, bkind, ckind, use_z, with_last, dtype, bc_dtype):
     """``B`` and ``C`` of shape ``(D, N)`` or ``(B, D, N)`` (the reference's other accepted forms,
     /root/reference/src/ssm/ops/python/reference.py:22-56): the wave-per-row kernel with the projections and their
     sums in lanes, against the general kernel on the same inputs (test-hooks selector 1) and against float64 autograd
-    through the oracle."""
+    through the oracle.  Sequences that fill chunks of 1024 steps (2048; 1600 and 3712 with a ragged last chunk) take
+    the 16-steps-per-lane form, the others 8."""
     b, d, l, n = shape
     inp = make_inputs(sum(shape) + 2, b, d, l, n, dtype=dtype, bc_dtype=bc_dtype, bkind=bkind, ckind=ckind, use_z=use_z)
     g = torch.Generator().manual_seed(6)
