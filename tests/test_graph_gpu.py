@@ -148,3 +148,36 @@ def test_ssd_combined_forward_and_backward():
         return (y, final) + tuple(g for g in grads if g is not None)
 
     _check_replays(inputs, fn, "ssd_combined")
+
+
+def test_the_reference_blocks_views_in_a_graph():
+    """The calls of ``Mamba1.forward`` (/root/reference/src/ssm/modules/mamba1.py:203-247) on its views -- the
+    convolution on a permuted half of a projection, read as it lies, and the scan on a permuted ``delta`` and ``z``,
+    turned by the library's own copy kernel, with projections constant in time -- forward and backward inside one
+    captured graph."""
+    ops = _ops()
+    B, L, D, N, dtype = 2, 1024, 96, 16, torch.bfloat16
+
+    def inputs(seed):
+        g = torch.Generator().manual_seed(seed)
+        xz = torch.randn(B, L, 2 * D, generator=g).to(dtype).cuda()
+        delta_rows = torch.randn(B, L, D, generator=g).to(dtype).cuda()
+        w, cb = (torch.rand(D, 4, generator=g) - 0.5).cuda(), (torch.randn(D, generator=g) * 0.1).cuda()
+        A = (-(torch.rand(D, N, generator=g) + 0.5)).cuda()
+        Bm, Cm = torch.randn(D, N, generator=g).cuda(), torch.randn(D, N, generator=g).cuda()
+        Dk, bias = torch.randn(D, generator=g).cuda(), torch.randn(D, generator=g).cuda()
+        go = torch.randn(B, D, L, generator=g).to(dtype).cuda()
+        return [xz, delta_rows, w, cb, A, Bm, Cm, Dk, bias, go]
+
+    def fn(xz, delta_rows, w, cb, A, Bm, Cm, Dk, bias, go):
+        projected, gate = xz.chunk(2, dim=-1)
+        x = projected.permute(0, 2, 1)
+        assert ops._conv_rows_view(x, True, 4) is not None
+        u = ops._conv_forward(x, w, cb, "silu")
+        delta, z = delta_rows.permute(0, 2, 1), gate.permute(0, 2, 1)
+        y, last = ops._scan_forward(u, delta, A, Bm, Cm, Dk, z, bias, True, True)
+        grads = ops._scan_backward(go, None, u, delta, A, Bm, Cm, Dk, z, bias, True)
+        dx, dw, db = ops._conv_backward(grads[0], x, w, cb, "silu")
+        return (u, y, last, dx, dw, db) + tuple(grads)
+
+    _check_replays(inputs, fn, "the reference block's calls on views")
