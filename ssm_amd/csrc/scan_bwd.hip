@@ -636,6 +636,41 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(const float *in, float *
   }
 }
 
+// Up to five such sums in one launch (dA, dD, the bias and, for projections constant in time, dB and dC: launches
+// of a few microseconds each, of which the gaps between them were as long as the work): workgroup ranges per job.
+constexpr int FOLD_JOBS = 5;
+struct FoldJobs {
+  const float *in[FOLD_JOBS];
+  float *out[FOLD_JOBS];
+  size_t inner[FOLD_JOBS];
+  int count[FOLD_JOBS];
+  unsigned first_block[FOLD_JOBS + 1];
+  int n;
+};
+
+__global__ __launch_bounds__(256) void fold_rows_multi_kernel(const FoldJobs jobs) {
+  int j = 0;
+  while (j + 1 < jobs.n && blockIdx.x >= jobs.first_block[j + 1]) ++j;
+  const float *in = jobs.in[j];
+  float *out = jobs.out[j];
+  const size_t inner = jobs.inner[j];
+  const int count = jobs.count[j];
+  const size_t blocks = jobs.first_block[j + 1] - jobs.first_block[j];
+  for (size_t i = (size_t)(blockIdx.x - jobs.first_block[j]) * blockDim.x + threadIdx.x; i < inner; i += blocks * blockDim.x) {
+    float s = 0.0f;
+    int k0 = 0;
+    for (; k0 + 8 <= count; k0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = in[(size_t)(k0 + k) * inner + i];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) s += v[k];
+    }
+    for (; k0 < count; ++k0) s += in[(size_t)k0 * inner + i];
+    out[i] = s;
+  }
+}
+
 static unsigned fold_grid(size_t n) {
   const size_t g = (n + 255) / 256;
   return (unsigned)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
@@ -902,30 +937,33 @@ extern "C" int ssm_scan_bwd(const ssm_scan_bwd_args *a, void *hip_stream) {
   if (rc != SSM_OK) return rc;
 
   const int Bn = a->batch, D = a->dim, N = a->nstate, L = a->seqlen;
-  // dA (D,N), dD (D,), dbias (D,): fold over batch
-  hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)D * N)), dim3(256), 0, s, p.dA_rows, a->dA, Bn,
-                     (size_t)D * N);
-  if (a->dD) hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid(D)), dim3(256), 0, s, p.dD_rows, a->dD, Bn, (size_t)D);
-  if (a->ddt_bias)
-    hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid(D)), dim3(256), 0, s, p.dbias_rows, a->ddt_bias, Bn, (size_t)D);
-  // dB / dC in the shape of the given projection
+  // dA (D,N), dD (D,), dbias (D,): sums over the batch; dB / dC in the shape of the given projection.  The sums
+  // over rows share one launch.
+  FoldJobs jobs{};
+  auto add_job = [&](const float *in, float *out, int count, size_t inner) {
+    const int j = jobs.n++;
+    jobs.in[j] = in; jobs.out[j] = out; jobs.count[j] = count; jobs.inner[j] = inner;
+    jobs.first_block[j + 1] = jobs.first_block[j] + fold_grid(inner);
+  };
+  add_job(p.dA_rows, a->dA, Bn, (size_t)D * N);
+  if (a->dD) add_job(p.dD_rows, a->dD, Bn, (size_t)D);
+  if (a->ddt_bias) add_job(p.dbias_rows, a->ddt_bias, Bn, (size_t)D);
   auto fold_proj = [&](int kind, int groups, const float *partial, float *out) {
     if (kind == SSM_PROJ_BGNL) {
       // (B, G, nblk/G, N*L) -> (B, G, N*L)
       const int per_group = p.nblk / groups;
       launch_fold_sum(partial, out, (size_t)Bn * groups, per_group, (size_t)N * L, s);
     } else if (kind == SSM_PROJ_BDN) {
-      hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)Bn * D * N)), dim3(256), 0, s, partial, out, 1,
-                         (size_t)Bn * D * N);
+      add_job(partial, out, 1, (size_t)Bn * D * N);
     } else {
-      hipLaunchKernelGGL(fold_rows_kernel, dim3(fold_grid((size_t)D * N)), dim3(256), 0, s, partial, out, Bn,
-                         (size_t)D * N);
+      add_job(partial, out, Bn, (size_t)D * N);
     }
   };
   if (!per_row) {
     fold_proj(a->b_kind, p.b_groups, p.dB_part, reinterpret_cast<float *>(a->dB));
     fold_proj(a->c_kind, p.c_groups, p.dC_part, reinterpret_cast<float *>(a->dC));
   }
+  hipLaunchKernelGGL(fold_rows_multi_kernel, dim3(jobs.first_block[jobs.n]), dim3(256), 0, s, jobs);
   SSM_CHECK_LAUNCH("ssm_scan_bwd(fold)");
   return SSM_OK;
 }
