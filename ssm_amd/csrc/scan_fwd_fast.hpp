@@ -330,10 +330,13 @@ void scan_fwd_fast_kernel(const ScanFwdParams p) {
 // CONST_BC: the same walk for projections that do not vary in time, (D, N) or (B, D, N) (the reference's other
 // accepted forms, src/ssm/ops/python/reference.py:22-56): a row's N values of B and of C sit in lanes like A, nothing
 // of the projections is read inside the loop.
-template <typename io_t, typename bc_t, int WAVES, int OCC, bool CONST_BC = false>
+// K: steps per lane, 8 or 16; with 16 a chunk of the walk is two chunks of FAST_T steps and the state that enters
+// the second one (what lane 32 starts from) is written to chunk_states as well.
+template <typename io_t, typename bc_t, int WAVES, int OCC, bool CONST_BC = false, int K = 8>
 __global__ __launch_bounds__(WAVE *WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
-  constexpr int K = 8, T = FAST_T;
+  constexpr int T = WAVE * K;
+  static_assert(T == FAST_T || T == 2 * FAST_T, "chunks of the walk are one or two chunks of the forward's states");
   const int wave = wave_id_uniform();
   const int lane = lane_id();
   const size_t row = (size_t)blockIdx.x * WAVES + wave;
@@ -360,6 +363,7 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
   const float Dk = p.Dk ? p.Dk[d] : 0.0f, bias = p.bias ? p.bias[d] : 0.0f;
 
   const int nchunks = (L + T - 1) / T;
+  const int state_chunks = (L + FAST_T - 1) / FAST_T;         // rows of chunk_states per (batch, channel)
   for (int c = 0; c < nchunks; ++c) {
     const int t = c * T + lane * K;
     const bool live = t < L;
@@ -376,7 +380,7 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
       const Pack<io_t, K> ur = *reinterpret_cast<const Pack<io_t, K> *>(U + at);
       const Pack<io_t, K> dr = *reinterpret_cast<const Pack<io_t, K> *>(DT + at);
       if (p.z) zr = *reinterpret_cast<const Pack<io_t, K> *>(Z + at);
-      if (p.chunk_states && lane < N) p.chunk_states[(row * nchunks + c) * (size_t)N + lane] = carry_lanes;
+      if (p.chunk_states && lane < N) p.chunk_states[(row * state_chunks + c * (T / FAST_T)) * (size_t)N + lane] = carry_lanes;
 #pragma unroll
       for (int i = 0; i < K; ++i) dl[i] = to_f32(dr.v[i]) + bias;
       if (p.softplus) {
@@ -432,6 +436,12 @@ void scan_fwd_rowbc_kernel(const ScanFwdParams p) {
       float hs = wave_prev(h, H);
       const float hend = wave_read_lane(h, WAVE - 1);
       carry_lanes = lane == n ? hend : carry_lanes;
+      if constexpr (T == 2 * FAST_T) {
+        // the state entering the second half of the chunk: what lane 32 starts from
+        const float hmid = wave_read_lane(hs, WAVE / 2);
+        if (p.chunk_states && lane == n && c * 2 + 1 < state_chunks)
+          p.chunk_states[(row * state_chunks + c * 2 + 1) * (size_t)N + n] = hmid;
+      }
 #pragma unroll
       for (int i = 0; i < K; ++i) {
         hs = __builtin_fmaf(a[i], hs, bx[i]);
@@ -489,8 +499,12 @@ template <typename io_t>
 static int launch_scan_fwd_row_const(const ScanFwdParams &p, hipStream_t stream) {
   constexpr int WAVES = 4;
   const size_t rows = (size_t)p.batch * p.dim;
-  hipLaunchKernelGGL((scan_fwd_rowbc_kernel<io_t, float, WAVES, 6, true>), dim3((unsigned)((rows + WAVES - 1) / WAVES)),
-                     dim3(WAVE * WAVES), 0, stream, p);
+  const dim3 grid((unsigned)((rows + WAVES - 1) / WAVES)), block(WAVE * WAVES);
+  const int tail = p.len % (2 * FAST_T);
+  if (p.len % 16 == 0 && p.len >= 2 * FAST_T && (tail == 0 || tail > FAST_T))
+    hipLaunchKernelGGL((scan_fwd_rowbc_kernel<io_t, float, WAVES, 4, true, 16>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((scan_fwd_rowbc_kernel<io_t, float, WAVES, 6, true>), grid, block, 0, stream, p);
   SSM_CHECK_LAUNCH("ssm_scan_fwd");
   return SSM_OK;
 }

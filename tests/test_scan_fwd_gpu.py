@@ -356,12 +356,14 @@ def test_repeated_call_of_one_form_goes_through_the_remembered_struct():
 @pytest.mark.parametrize("bkind,ckind", [("dn", "dn"), ("bdn", "bdn"), ("dn", "bdn"), ("bdn", "dn")])
 @pytest.mark.parametrize("dtype,bc_dtype,length,nstate", [
     (torch.float32, torch.float32, 1520, 16), (torch.float32, torch.float32, 48, 5), (torch.bfloat16, torch.float32, 1040, 9),
-    (torch.float16, torch.float16, 512, 16), (torch.bfloat16, torch.bfloat16, 2048, 16)])
+    (torch.float16, torch.float16, 512, 16), (torch.bfloat16, torch.bfloat16, 2048, 16), (torch.float32, torch.float32, 1600, 16),
+    (torch.float32, torch.float32, 3712, 7)])
 def test_constant_projections_row_per_wave(bkind, ckind, dtype, bc_dtype, length, nstate):
     """``B`` and ``C`` of shape ``(D, N)`` or ``(B, D, N)`` (/root/reference/src/ssm/ops/python/reference.py:22-56): the
     kernel with a row per wave and the projections in lanes (variant 31042; what sequences beyond 256 steps take
     unasked) against the oracle and against the general kernel (selector 816) on the same inputs -- values, the last
-    state, and the chunk states that the backward starts from."""
+    state, and the chunk states that the backward starts from.  Sequences that fill chunks of 1024 steps (2048; 1600
+    and 3712 with a ragged last chunk) walk 16 steps per lane and write the state in the middle of a chunk too."""
     from ssm_amd import ops
     inp = make_inputs(length + nstate, 2, 24, length, nstate, dtype=dtype, bc_dtype=bc_dtype, bkind=bkind, ckind=ckind)
     yr, hr = O.selective_scan(inp["u"], inp["delta"], inp["A"], inp["B"], inp["C"], D=inp["D"],
