@@ -141,6 +141,38 @@ def test_shape_and_dtype_errors_come_back_as_status_codes():
     assert lib.ssm_scan_bwd_workspace_bytes(8, 1536, 2048, 16, 2, 2, 7, 1) == 0
 
 
+def test_views_of_rows_are_checked_before_anything_is_launched():
+    """The convolution's rows-in layout and the transposing copy say what they do not take, as status codes."""
+    L = _lib()
+    lib = L.load()
+    buf = (ctypes.c_float * 4096)()
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    conv = dict(x=p, weight=p, y=p, batch=2, channels=8, seqlen=16, width=4, io_dtype=0, layout=L.LAYOUT_ROWS_TO_BCL,
+                activation=1, x_batch_stride=16 * 8, x_row_stride=8)
+    a = L.Conv1dFwdArgs(**conv)
+    a.channels = 6
+    assert lib.ssm_conv1d_fwd(ctypes.byref(a), None) == -2          # channels not a multiple of 4
+    assert b"(B,C,L) copy" in lib.ssm_amd_last_error()
+    a = L.Conv1dFwdArgs(**dict(conv, width=7))
+    assert lib.ssm_conv1d_fwd(ctypes.byref(a), None) == -2          # wider than the vector kernels take
+    a = L.Conv1dFwdArgs(**dict(conv, x_row_stride=6))
+    assert lib.ssm_conv1d_fwd(ctypes.byref(a), None) == -2          # rows overlap
+    a = L.Conv1dFwdArgs(**dict(conv, x_batch_stride=8))
+    assert lib.ssm_conv1d_fwd(ctypes.byref(a), None) == -2          # batch entries overlap
+    a = L.Conv1dFwdArgs(**dict(conv, x=p + 4))
+    assert lib.ssm_conv1d_fwd(ctypes.byref(a), None) == -5          # x off a boundary of four elements
+    a = L.Conv1dFwdArgs(**dict(conv, layout=L.LAYOUT_BCL))
+    assert lib.ssm_conv1d_fwd(ctypes.byref(a), None) == -4          # strides with another layout
+    assert lib.ssm_conv1d_fwd(ctypes.byref(L.Conv1dFwdArgs(**dict(conv, layout=3))), None) == -4
+    t = dict(src=p, dst=p + 8192, src_batch_stride=16 * 8, src_row_stride=8, batch=2, channels=8, seqlen=16, element_size=4)
+    assert lib.ssm_rows_to_bcl(ctypes.byref(L.RowsToBclArgs(**dict(t, element_size=8))), None) == -3
+    assert lib.ssm_rows_to_bcl(ctypes.byref(L.RowsToBclArgs(**dict(t, channels=6))), None) == -2
+    assert lib.ssm_rows_to_bcl(ctypes.byref(L.RowsToBclArgs(**dict(t, src_row_stride=4))), None) == -2
+    assert lib.ssm_rows_to_bcl(ctypes.byref(L.RowsToBclArgs(**dict(t, src=p + 4))), None) == -5
+    assert lib.ssm_rows_to_bcl(ctypes.byref(L.RowsToBclArgs(**dict(t, dst=None))), None) == -1
+
+
 def test_shipped_library_has_no_test_hooks_and_the_hooks_build_does():
     """Kernel selectors and the record of kernels taken exist in the -DSSM_TEST_HOOKS build only
     (include/ssm_amd_testing.h): the shipped library rejects a non-zero ``reserved`` field and does not export
