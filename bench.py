@@ -246,7 +246,13 @@ def bench_conv(dtype=torch.bfloat16, batch=8, chans=1536, length=2048, width=4):
     rv_fwd_us = _graph_us(lambda i: ops._conv_forward(views[i % 3], w, b, "silu"))
     rv_bwd_us = _graph_us(lambda i: ops._conv_backward(go, views[i % 3], w, b, "silu"))
     frac = lambda nbytes, us: round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)
+    # the dense (B,C,L) copy of such a view that the scan asks for (delta and z of the reference's Mamba1 block)
+    from ssm_amd.ops import _contract
+    copy_us = _graph_us(lambda i: _contract.dense_copy(views[i % 3]))
+    torch_copy_us = _graph_us(lambda i: views[i % 3].contiguous(), calls=6, replays=2)
     return {"fwd_us": round(fwd_us, 1), "fwd_GBps": round(fb / fwd_us / 1e3, 1), "fwd_frac_hbm": frac(fb, fwd_us),
+            "view_of_rows_dense_copy_us": round(copy_us, 1), "view_of_rows_dense_copy_frac_hbm": frac(fb, copy_us),
+            "view_of_rows_dense_copy_by_torch_us": round(torch_copy_us, 1),
             "bwd_us": round(bwd_us, 1), "bwd_GBps": round(bb / bwd_us / 1e3, 1), "bwd_frac_hbm": frac(bb, bwd_us),
             "channels_last_fwd_us": round(cl_fwd_us, 1), "channels_last_bwd_us": round(cl_bwd_us, 1),
             "channels_last_fwd_frac_hbm": frac(fb, cl_fwd_us), "channels_last_bwd_frac_hbm": frac(bb, cl_bwd_us),
