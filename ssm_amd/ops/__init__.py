@@ -418,6 +418,45 @@ def _state_step_backward(grad_out, grad_state, state, x, dt, A, B, C, D, z, dt_b
     return dstate, dx, ddt, dA, dB, dC, dD, dz, dbias
 
 
+# Argument structs of state steps that were validated before, keyed by everything the validation looks at (as
+# _SCAN_FORMS for the scan): a decoding loop calls with one form for its whole life, a new token's tensors each time.
+_STEP_FORMS = {}
+
+
+def _state_step_again(state, x, dt, A, B, C, D, z, dt_bias, softplus):
+    """The step through a struct remembered from an earlier call of the same form, or ``None`` if the form is new or
+    a tensor would need a cast, a copy or a batch stride first (those go the long way)."""
+    io = x.dtype
+    if not (K.on_gpu(state) and dt.dtype == io and A.dtype == _F32 and B.dtype == C.dtype and state.is_contiguous()
+            and x.is_contiguous() and dt.is_contiguous() and A.is_contiguous() and B.is_contiguous() and C.is_contiguous()):
+        return None
+    for t, want in ((D, _F32), (z, io), (dt_bias, _F32)):
+        if t is not None and not (t.dtype == want and t.is_contiguous()):
+            return None
+    if (state.data_ptr() | x.data_ptr() | dt.data_ptr() | A.data_ptr() | B.data_ptr() | C.data_ptr()
+            | (0 if z is None else z.data_ptr()) | (0 if D is None else D.data_ptr())
+            | (0 if dt_bias is None else dt_bias.data_ptr())) & 15:
+        return None
+    dev = state.device
+    key = (state.shape, state.dtype, x.shape, io, A.shape, B.shape, B.dtype, C.shape, D is None or D.shape,
+           z is None or z.shape, dt_bias is None or dt_bias.shape, bool(softplus), dev.index)
+    form = _STEP_FORMS.get(key)
+    if form is None:
+        return None
+    for t in (x, dt, A, B, C, D, z, dt_bias):
+        if t is not None and t.device != dev:
+            return None
+    args = _lib.StateStepArgs.from_buffer_copy(form)
+    out = torch.empty_like(x)
+    args.state, args.x, args.dt, args.A, args.Bproj, args.Cproj, args.out = (
+        state.data_ptr(), x.data_ptr(), dt.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr(), out.data_ptr())
+    args.z = None if z is None else z.data_ptr()
+    args.Dskip = None if D is None else D.data_ptr()
+    args.dt_bias = None if dt_bias is None else dt_bias.data_ptr()
+    _lib.call("ssm_state_step", args, dev)
+    return out
+
+
 def selective_state_step(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, softplus=True):
     """Advance the selective state by one token on the GPU; ``state`` is updated in place.
 
@@ -440,9 +479,24 @@ def selective_state_step(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, so
     if any(t is not None and t.requires_grad for t in tensors) and torch.is_grad_enabled():
         from ._autograd import state_step_with_grad
         return state_step_with_grad(state, x, dt, A, B, C, D, z, dt_bias, bool(softplus))
+    again = _state_step_again(state, x, dt, A, B, C, D, z, dt_bias, softplus)
+    if again is not None:
+        return again
     if state.is_contiguous():
         plan = StepPlan(state, x, dt, A, B, C, D, z, dt_bias, softplus)
         out = plan.run()
+        if plan.f64 is None and len(_STEP_FORMS) < 256 and out.dtype == x.dtype:
+            # remembered only when every tensor went in as it was (no cast, no copy, no batch stride): that is what
+            # _state_step_again can repeat
+            k, a = plan.keep, plan.args
+            same = all(p is None or q is None or p.data_ptr() == q.data_ptr()
+                       for p, q in ((x, k["x"]), (dt, k["dt"]), (z, k["z"]), (B, k["B"]), (C, k["C"]), (A, k["A"]),
+                                    (D, k["D"]), (dt_bias, k["bias"])))
+            if same and not (a.z_batch_stride or a.b_batch_stride or a.c_batch_stride) and K.on_gpu(state):
+                key = (state.shape, state.dtype, x.shape, x.dtype, A.shape, B.shape, B.dtype, C.shape,
+                       D is None or D.shape, z is None or z.shape, dt_bias is None or dt_bias.shape, bool(softplus),
+                       state.device.index)
+                _STEP_FORMS[key] = bytes(a)
     else:
         work = state.contiguous()
         plan = StepPlan(work, x, dt, A, B, C, D, z, dt_bias, softplus)

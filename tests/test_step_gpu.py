@@ -469,3 +469,33 @@ def test_autograd_through_two_steps_matches_oracle():
     for k in lw:
         torch.testing.assert_close(lg[k].grad.cpu().double(), lw[k].grad, rtol=1e-4, atol=1e-5,
                                    msg=lambda m, n=k: f"grad {n}: {m}")
+
+
+def test_repeated_step_of_one_form_goes_through_the_remembered_struct():
+    """The second step of a form (same shapes, element types, optional arguments) skips the validation and fills a
+    remembered argument struct: the same bits as a prepared plan on the same values, new tensors each time; a call
+    whose tensors need a copy first, and a form never seen, still go the long way."""
+    from ssm_amd import ops
+    g = torch.Generator().manual_seed(8)
+    batch, dim, nstate = 4, 96, 16
+    A = (-(torch.rand(dim, nstate, generator=g) + 0.5)).cuda()
+    D, bias = torch.randn(dim, generator=g).cuda(), torch.randn(dim, generator=g).cuda()
+    def token(seed):
+        h = torch.Generator().manual_seed(seed)
+        x, dt, z = (torch.randn(batch, dim, generator=h).to(torch.bfloat16).cuda() for _ in range(3))
+        Bm, Cm = (torch.randn(batch, 1, nstate, generator=h).to(torch.bfloat16).cuda() for _ in range(2))
+        return x, dt, z, Bm, Cm
+    ops._STEP_FORMS.clear()
+    state, ref_state = torch.zeros(batch, dim, nstate).cuda(), torch.zeros(batch, dim, nstate).cuda()
+    for step in range(4):
+        x, dt, z, Bm, Cm = token(step)
+        y = ops.selective_state_step(state, x, dt, A, Bm, Cm, D, z=z, dt_bias=bias, softplus=True)
+        assert len(ops._STEP_FORMS) == 1
+        want = ops.StepPlan(ref_state, x, dt, A, Bm, Cm, D, z, bias, True).run()
+        assert torch.equal(y, want) and torch.equal(state, ref_state), step
+    x, dt, z, Bm, Cm = token(9)
+    y = ops.selective_state_step(state, x.t().contiguous().t(), dt, A, Bm, Cm, D, z=z, dt_bias=bias, softplus=True)
+    want = ops.StepPlan(ref_state, x, dt, A, Bm, Cm, D, z, bias, True).run()
+    assert torch.equal(y, want) and torch.equal(state, ref_state)
+    with pytest.raises(ValueError):
+        ops.selective_state_step(state, x, dt, A[:, :8].contiguous(), Bm, Cm, D, z=z, dt_bias=bias, softplus=True)
