@@ -466,12 +466,18 @@ def _scan_wide_case(rng, seed):
     A = -(torch.rand(d, n, generator=g) * 3 + 0.1)
     bc = rng.choice([dtype, dtype, torch.float32])
     Bm, Cm = torch.randn(b, groups, n, l, generator=g).to(bc), torch.randn(b, groups, n, l, generator=g).to(bc)
+    const = random.Random(seed ^ 0x7A3F)                   # (drawn apart again)
+    kinds = None
+    if const.random() < 0.15:                              # projections constant in time: (D, N) or (B, D, N)
+        kinds = const.choice([("dn", "dn"), ("bdn", "bdn"), ("dn", "bdn"), ("bdn", "dn")])
+        shape = {"dn": (d, n), "bdn": (b, d, n)}
+        Bm, Cm = (torch.randn(*shape[k], generator=g).to(const.choice([torch.float32, bc])) for k in kinds)
     D = torch.randn(d, generator=g) if rng.random() < 0.7 else None
     z = torch.randn(b, d, l, generator=g).to(dtype) if rng.random() < 0.7 else None
     bias = torch.randn(d, generator=g) * 0.5 if rng.random() < 0.7 else None
     with_last = rng.random() < 0.5
     half = dtype in HALF
-    desc = ("scan wide", seed, (b, d, l, n), groups, str(dtype), str(bc), D is not None, z is not None, bias is not None, with_last)
+    desc = ("scan wide", seed, (b, d, l, n), groups, str(dtype), str(bc), D is not None, z is not None, bias is not None, with_last, kinds)
     dev = lambda t: None if t is None else t.cuda()
     with torch.no_grad():
         y64, last64 = O.selective_scan(u, delta, A, Bm, Cm, D, z, bias, softplus=True, return_last_state=True, acc=torch.float64)
